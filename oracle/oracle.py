@@ -1,0 +1,297 @@
+"""numpy front end of the CPU oracle (TEST INFRASTRUCTURE, not product code).
+
+Loads ``liboracle.so`` (built from ``ref_oracle.c`` by ``make -C oracle``) and
+exposes the ref-target arithmetic on numpy arrays.  Only tests, the smoke
+check and the benchmark's cpu_baseline leg import this module; the shipped
+library never does.
+
+Low-precision element types have no numpy dtype, so they travel as raw bits:
+half and bf16 as ``uint16``, fp8 e4m3fn as ``uint8``; the ``*_type`` argument
+says how the bits are to be read.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+I8, U8, I32, F32, F16, BF16, FP8, F64 = range(8)
+_NP = {I8: np.int8, U8: np.uint8, I32: np.int32, F32: np.float32,
+       F16: np.uint16, BF16: np.uint16, FP8: np.uint8, F64: np.float64}
+
+
+def build():
+    """Compile the oracle (used by __graft_entry__.build and by tests when the
+    library is missing)."""
+    subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"],
+                          stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+    lib.orc_gemm.argtypes = [vp, ci, vp, vp, ci] + [i64] * 10
+    lib.orc_gemm.restype = None
+    lib.orc_quantizelinear.argtypes = [vp, ci, vp, ci, vp, i64, i64, vp, i64, i64, i64, i64]
+    lib.orc_quantizelinear.restype = None
+    lib.orc_dequantizelinear.argtypes = [vp, vp, ci, vp, ci, i64, i64, vp, i64, i64, i64, i64]
+    lib.orc_dequantizelinear.restype = None
+    lib.orc_unpack_int4.argtypes = [vp, vp, ci, i64, i64, i64]
+    lib.orc_unpack_int4.restype = None
+    lib.orc_pack_int4.argtypes = [vp, vp, ci, i64, i64, i64]
+    lib.orc_pack_int4.restype = None
+    lib.orc_convert.argtypes = [vp, ci, vp, ci, ctypes.c_size_t]
+    lib.orc_convert.restype = None
+    lib.orc_mul_f32.argtypes = [vp, vp, i64, i64, vp, i64, i64, i64, i64]
+    lib.orc_mul_f32.restype = None
+    for name in ("half", "bf16", "fp8e4m3fn"):
+        getattr(lib, f"orc_{name}_from_f32_n").argtypes = [vp, vp, ctypes.c_size_t]
+        getattr(lib, f"orc_{name}_from_f32_n").restype = None
+        getattr(lib, f"orc_{name}_to_f32_n").argtypes = [vp, vp, ctypes.c_size_t]
+        getattr(lib, f"orc_{name}_to_f32_n").restype = None
+    return lib
+
+
+_lib = _load()
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+# --- scalar formats --------------------------------------------------------
+
+def _conv(name, x, src, dst):
+    x = _c(x, src)
+    y = np.empty(x.shape, dst)
+    getattr(_lib, name)(_p(x), _p(y), x.size)
+    return y
+
+
+def half_from_f32(x):
+    return _conv("orc_half_from_f32_n", x, np.float32, np.uint16)
+
+
+def half_to_f32(x):
+    return _conv("orc_half_to_f32_n", x, np.uint16, np.float32)
+
+
+def bf16_from_f32(x):
+    return _conv("orc_bf16_from_f32_n", x, np.float32, np.uint16)
+
+
+def bf16_to_f32(x):
+    return _conv("orc_bf16_to_f32_n", x, np.uint16, np.float32)
+
+
+def fp8_from_f32(x):
+    return _conv("orc_fp8e4m3fn_from_f32_n", x, np.float32, np.uint8)
+
+
+def fp8_to_f32(x):
+    return _conv("orc_fp8e4m3fn_to_f32_n", x, np.uint8, np.float32)
+
+
+# --- ops ---------------------------------------------------------------------
+
+def _elem_strides(a):
+    return [s // a.itemsize for s in a.strides]
+
+
+def gemm(a, b, ab_type, c_type):
+    """C[..., M, N] = A[..., M, K] . B[..., K, N] as gemm_naive does it.
+
+    ``a`` and ``b`` may be arbitrary strided views (transposes); all leading
+    dimensions are batch dimensions and must match."""
+    assert a.ndim == b.ndim and a.ndim >= 2
+    assert a.shape[:-2] == b.shape[:-2] and a.shape[-1] == b.shape[-2]
+    m, k = a.shape[-2:]
+    n = b.shape[-1]
+    batch_shape = a.shape[:-2]
+    out = np.empty(batch_shape + (m, n), _NP[c_type])
+    if a.ndim > 2:
+        # collapse batch dims: copy only if they do not collapse to one stride
+        a3 = a.reshape((-1, m, k))
+        b3 = b.reshape((-1, k, n))
+    else:
+        a3, b3 = a[None], b[None]
+    nb = a3.shape[0]
+    sa, sb = _elem_strides(a3), _elem_strides(b3)
+    _lib.orc_gemm(_p(out), c_type, ctypes.c_void_p(a3.ctypes.data), ctypes.c_void_p(b3.ctypes.data),
+                  ab_type, m, n, k, sa[1], sa[2], sb[1], sb[2], nb, sa[0], sb[0])
+    return out
+
+
+def quant_dot(a, b, ab_type=I8):
+    """quant_dot: int8/uint8 -> int32, fp8 -> float (op/quant_dot.hpp:76-77)."""
+    return gemm(a, b, ab_type, I32 if ab_type in (I8, U8) else F32)
+
+
+def dot(a, b, ab_type):
+    return gemm(a, b, ab_type, ab_type)
+
+
+def _bcast2d(p, rows, cols, dtype):
+    """Return (array, row_stride, col_stride) addressing a q-param as [r, c]."""
+    p = np.asarray(p, dtype=dtype)
+    if p.ndim == 0 or p.size == 1:
+        return np.ascontiguousarray(p.reshape(1)), 0, 0
+    if p.ndim == 1:
+        if p.shape[0] == cols:
+            return np.ascontiguousarray(p), 0, 1
+        if p.shape[0] == rows:
+            return np.ascontiguousarray(p), 1, 0
+        raise ValueError("1-D parameter matches neither axis")
+    p = np.ascontiguousarray(np.broadcast_to(p, (rows, cols)))
+    return p, cols, 1
+
+
+def quantizelinear(x, scale, zp, x_type, out_type):
+    x = _c(x, _NP[x_type])
+    shp = x.shape
+    x2 = x.reshape(-1, shp[-1]) if x.ndim > 1 else x.reshape(1, -1)
+    rows, cols = x2.shape
+    s, ssr, ssc = _bcast2d(np.asarray(scale).reshape(-1, cols) if np.ndim(scale) > 2 else scale,
+                           rows, cols, _NP[x_type])
+    out = np.empty((rows, cols), _NP[out_type])
+    if zp is None:
+        _lib.orc_quantizelinear(_p(out), out_type, _p(x2), x_type, _p(s), ssr, ssc,
+                                None, 0, 0, rows, cols)
+    else:
+        z, zsr, zsc = _bcast2d(np.asarray(zp).reshape(-1, cols) if np.ndim(zp) > 2 else zp,
+                               rows, cols, _NP[out_type])
+        _lib.orc_quantizelinear(_p(out), out_type, _p(x2), x_type, _p(s), ssr, ssc,
+                                _p(z), zsr, zsc, rows, cols)
+    return out.reshape(shp)
+
+
+def dequantizelinear(x, scale, zp, x_type, s_type):
+    x = _c(x, _NP[x_type])
+    shp = x.shape
+    x2 = x.reshape(-1, shp[-1]) if x.ndim > 1 else x.reshape(1, -1)
+    rows, cols = x2.shape
+    s, ssr, ssc = _bcast2d(np.asarray(scale).reshape(-1, cols) if np.ndim(scale) > 2 else scale,
+                           rows, cols, _NP[s_type])
+    out = np.empty((rows, cols), _NP[s_type])
+    if zp is None:
+        _lib.orc_dequantizelinear(_p(out), _p(x2), x_type, _p(s), s_type, ssr, ssc,
+                                  None, 0, 0, rows, cols)
+    else:
+        z, zsr, zsc = _bcast2d(np.asarray(zp).reshape(-1, cols) if np.ndim(zp) > 2 else zp,
+                               rows, cols, _NP[x_type])
+        _lib.orc_dequantizelinear(_p(out), _p(x2), x_type, _p(s), s_type, ssr, ssc,
+                                  _p(z), zsr, zsc, rows, cols)
+    return out.reshape(shp)
+
+
+def _axis_split(shape, axis):
+    axis = axis % len(shape)
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return axis, outer, shape[axis], inner
+
+
+def unpack_int4(x, axis=-1):
+    signed = x.dtype == np.int8
+    xc = np.ascontiguousarray(x)
+    axis, outer, alen, inner = _axis_split(xc.shape, axis)
+    shp = list(xc.shape)
+    shp[axis] *= 2
+    out = np.empty(shp, xc.dtype)
+    _lib.orc_unpack_int4(_p(out), _p(xc), int(signed), outer, alen, inner)
+    return out
+
+
+def pack_int4(x, axis=-1):
+    signed = x.dtype == np.int8
+    xc = np.ascontiguousarray(x)
+    axis, outer, alen, inner = _axis_split(xc.shape, axis)
+    if alen % 2:
+        raise ValueError("PACK_INT4: Can not pack axis that has odd lengths")
+    shp = list(xc.shape)
+    shp[axis] //= 2
+    out = np.empty(shp, xc.dtype)
+    _lib.orc_pack_int4(_p(out), _p(xc), int(signed), outer, alen // 2, inner)
+    return out
+
+
+def convert(x, x_type, out_type):
+    x = _c(x, _NP[x_type])
+    out = np.empty(x.shape, _NP[out_type])
+    _lib.orc_convert(_p(out), out_type, _p(x), x_type, x.size)
+    return out
+
+
+def mul_f32(a, b, rows, cols):
+    a, asr, asc = _bcast2d(a, rows, cols, np.float32)
+    b, bsr, bsc = _bcast2d(b, rows, cols, np.float32)
+    out = np.empty((rows, cols), np.float32)
+    _lib.orc_mul_f32(_p(out), _p(a), asr, asc, _p(b), bsr, bsc, rows, cols)
+    return out
+
+
+# --- the composite paths of the benchmark configs ------------------------------
+
+def qdq_matmul_int8(x_q, w_q, s_x, s_w, zp_x=0, zp_w=0, out_type=F32):
+    """What simplify_qdq leaves for DQ(x_q) . DQ(w_q) (simplify_qdq.cpp:225-289):
+    quant_dot -> int32, out_scale = mul(s_x, s_w) in fp32, zero-point terms as
+    three extra quant_dots, dequantizelinear, optional convert."""
+    m, k = x_q.shape
+    n = w_q.shape[1]
+    acc = quant_dot(x_q, w_q, I8)
+    scale = mul_f32(np.asarray(s_x, np.float32), np.asarray(s_w, np.float32), m, n)
+    zp = None
+    if zp_x != 0 or zp_w != 0:
+        zp = np.zeros((m, n), np.int32)
+        zx = np.full((m, k), zp_x, np.int8)
+        zw = np.full((k, n), zp_w, np.int8)
+        if zp_x != 0:
+            zp = zp + quant_dot(zx, w_q, I8)
+        if zp_w != 0:
+            zp = zp + quant_dot(x_q, zw, I8)
+        if zp_x != 0 and zp_w != 0:
+            zp = zp - quant_dot(zx, zw, I8)
+        zp = zp.astype(np.int32)
+    out = dequantizelinear(acc, scale, zp, I32, F32)
+    if out_type != F32:
+        out = convert(out, F32, out_type)
+    return out
+
+
+def qdq_matmul_fp8(x_q, w_q, s_x, s_w, out_type=F32):
+    m = x_q.shape[0]
+    n = w_q.shape[1]
+    acc = quant_dot(x_q, w_q, FP8)
+    scale = mul_f32(np.asarray(s_x, np.float32), np.asarray(s_w, np.float32), m, n)
+    out = dequantizelinear(acc, scale, None, F32, F32)
+    if out_type != F32:
+        out = convert(out, F32, out_type)
+    return out
+
+
+def w4a16_matmul(a_h, w_packed, scales_h, zp, group):
+    """unpack_int4 -> dequantizelinear(scales, zp) -> transpose -> dot, the
+    graph of parse_matmulnbits.cpp:85-159 with fp16 activations and scales.
+
+    a_h       [M, K] half bits, w_packed [N, K/2] uint8 (low nibble = even k),
+    scales_h  [N, K/group] half bits, zp scalar or [N, K/group] uint8."""
+    n, kh = w_packed.shape
+    k = kh * 2
+    q = unpack_int4(w_packed)                               # [N, K] u8
+    s_full = np.repeat(scales_h, group, axis=1)[:, :k]
+    if np.ndim(zp) == 0:
+        z_full = np.full((n, k), zp, np.uint8)
+    else:
+        z_full = np.repeat(np.asarray(zp, np.uint8), group, axis=1)[:, :k]
+    w = dequantizelinear(q, s_full, z_full, U8, F16)        # [N, K] half bits
+    return dot(a_h, w.T, F16)

@@ -1,0 +1,646 @@
+/*
+ * ref_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C CPU restatement of the arithmetic that MIGraphX's `ref` target
+ * performs on the quantized-GEMM path.  It exists only so that tests, the
+ * smoke check and the benchmark's cpu_baseline leg have something to compare
+ * the HIP kernels against.  Nothing in the shipped library links, loads or
+ * calls this file.
+ *
+ * Every function names the reference source it follows (paths relative to
+ * the reference tree).  How each function is pinned (which of the reference's
+ * own known-answer vectors or which closed form checks it) is listed next to
+ * it; the checks themselves live in tests/test_oracle_*.py.
+ *
+ *   function                      pinned by
+ *   ---------------------------   -------------------------------------------
+ *   orc_fp8e4m3fn_to_f32          256-entry table of test/fp8e4m3fn.cpp:34-105
+ *   orc_fp8e4m3fn_from_f32        samples test/fp8e4m3fn.cpp:121-140 + brute
+ *                                 force "nearest table entry, ties to even
+ *                                 mantissa, saturate to 448" over random and
+ *                                 adversarial floats
+ *   orc_half_* / orc_bf16_*       tables test/half.cpp, test/bf16.cpp + closed
+ *                                 form (mantissa shift == round toward zero,
+ *                                 compared with numpy bit arithmetic)
+ *   orc_quant_dot                 16 quant_dot cases test/ref/dot_op.cpp:1391-
+ *                                 1865 + numpy int64 matmul + exact fixed point
+ *                                 closed form for fp8
+ *   orc_quantizelinear            test/ref/quantizelinear.cpp:33-168
+ *   orc_dequantizelinear          test/ref/dequantizelinear.cpp:32-83
+ *   orc_unpack_int4/orc_pack_int4 test/ref/unpack_int4.cpp, pack_int4.cpp,
+ *                                 pack_unpack_int4.cpp
+ *   orc_dot                       test/onnx/verify/matmulnbits_tests.cpp golds
+ *                                 (whole unpack -> dequantize -> dot chain)
+ *   orc_convert                   test/ref/convert.cpp + closed form
+ */
+#include <fenv.h>
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+/* element type codes shared with oracle.py */
+enum {
+    ORC_I8   = 0,
+    ORC_U8   = 1,
+    ORC_I32  = 2,
+    ORC_F32  = 3,
+    ORC_F16  = 4,
+    ORC_BF16 = 5,
+    ORC_FP8  = 6, /* OCP e4m3fn */
+    ORC_F64  = 7
+};
+
+static inline uint32_t f32_bits(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static inline float bits_f32(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* ------------------------------------------------------------------------
+ * generic_float<M,E>::from_float / to_float
+ * src/include/migraphx/generic_float.hpp:172-222 (from_float), :129-170
+ * (to_float).  half = generic_float<10,5> (half.hpp:34), bf16 =
+ * generic_float<7,8> (bf16.hpp:34).  The mantissa is shifted right, i.e. the
+ * conversion rounds toward zero; exponent overflow gives infinity.
+ * ---------------------------------------------------------------------- */
+static uint32_t gf_from_f32(float x, int msize, int esize)
+{
+    uint32_t u        = f32_bits(x);
+    uint32_t fsign    = u >> 31;
+    uint32_t fexp     = (u >> 23) & 0xffu;
+    uint32_t fman     = u & 0x7fffffu;
+    uint32_t all_ones = (1u << esize) - 1u;
+    int bias          = (1 << (esize - 1)) - 1;
+    int diff          = 127 - bias;
+    uint32_t e, m;
+    if(fexp == 0)
+    {
+        e = 0;
+        m = fman >> (23 - msize);
+    }
+    else if(fexp == 0xffu)
+    {
+        e = all_ones;
+        m = fman >> (23 - msize);
+    }
+    else
+    {
+        int ee = (int)fexp - diff;
+        if(ee >= (int)all_ones)
+        {
+            e = all_ones;
+            m = 0;
+        }
+        else if(ee < 1)
+        {
+            int shift        = diff - (int)fexp;
+            int shift_amount = shift + (23 - msize) + 1;
+            e                = 0;
+            if(shift_amount < 32)
+                m = (fman | (1u << 23)) >> shift_amount;
+            else
+                m = 0;
+        }
+        else
+        {
+            e = (uint32_t)ee;
+            m = fman >> (23 - msize);
+        }
+    }
+    if(e > all_ones)
+        e = all_ones;
+    m &= (1u << msize) - 1u;
+    return (fsign << (msize + esize)) | (e << msize) | m;
+}
+
+static float gf_to_f32(uint32_t bits, int msize, int esize)
+{
+    uint32_t all_ones = (1u << esize) - 1u;
+    uint32_t sign     = (bits >> (msize + esize)) & 1u;
+    uint32_t e        = (bits >> msize) & all_ones;
+    uint32_t m        = bits & ((1u << msize) - 1u);
+    int bias          = (1 << (esize - 1)) - 1;
+    uint32_t fe, fm;
+    if(e == 0 && esize != 8)
+    {
+        if(m == 0)
+        {
+            fe = 0;
+            fm = 0;
+        }
+        else
+        {
+            /* normalise the subnormal: shift so the leading one is dropped */
+            int top = 31 - __builtin_clz(m); /* index of leading one */
+            int shift = msize - (top + 1);
+            fm        = (m << (shift + 1)) & ((1u << msize) - 1u);
+            fe        = (uint32_t)(127 - bias - shift);
+            fm <<= (23 - msize);
+        }
+    }
+    else if(e == all_ones)
+    {
+        fm = m << (23 - msize);
+        fe = 0xffu;
+    }
+    else
+    {
+        fm = m << (23 - msize);
+        fe = (uint32_t)((int)e + (127 - bias));
+    }
+    return bits_f32((sign << 31) | (fe << 23) | fm);
+}
+
+uint16_t orc_half_from_f32(float x) { return (uint16_t)gf_from_f32(x, 10, 5); }
+float orc_half_to_f32(uint16_t h) { return gf_to_f32(h, 10, 5); }
+uint16_t orc_bf16_from_f32(float x) { return (uint16_t)gf_from_f32(x, 7, 8); }
+float orc_bf16_to_f32(uint16_t h) { return gf_to_f32(h, 7, 8); }
+
+/* ------------------------------------------------------------------------
+ * fp8 e4m3fn (OCP, "fn": no infinities, 0x7f/0xff are NaN, max 448)
+ * cast_from_f8<3,4,float,false>  src/include/migraphx/float8_impl.hpp:249-325
+ * cast_to_f8<3,4,float,false,true(clip)> float8_impl.hpp:38-247, selected by
+ * float8.hpp:87-101 with MIGRAPHX_F8_DOWNCAST_CLIPPING (float8.hpp:32).
+ * Round to nearest even, saturate to +-448 (0x7e/0xfe), +-inf -> +-448,
+ * NaN -> 0x7f / 0xff.
+ * ---------------------------------------------------------------------- */
+float orc_fp8e4m3fn_to_f32(uint8_t x)
+{
+    const int wm = 3, we = 4;
+    if(x == 0)
+        return 0.0f;
+    if(x == 0x80)
+        return bits_f32(0x80000000u);
+    if(x == 0x7f || x == 0xff)
+        return bits_f32(0x7f800001u);
+    uint32_t sign     = x >> 7;
+    uint32_t mantissa = x & ((1u << wm) - 1u);
+    int exponent      = (x & 0x7f) >> wm;
+    const int exp_low_cutoff = (1 << (8 - 1)) - (1 << (we - 1)) + 1; /* 121 */
+    if(exponent == 0)
+    {
+        int sh = 1 + __builtin_clz(mantissa) - (32 - wm);
+        mantissa <<= sh;
+        exponent += 1 - sh;
+        mantissa &= (1u << wm) - 1u;
+    }
+    exponent += exp_low_cutoff - 1;
+    mantissa <<= 23 - wm;
+    return bits_f32((sign << 31) | ((uint32_t)exponent << 23) | mantissa);
+}
+
+uint8_t orc_fp8e4m3fn_from_f32(float fx)
+{
+    const uint32_t wm = 3, we = 4, mfmt = 23;
+    uint32_t x        = f32_bits(fx);
+    uint32_t head     = x & 0xFF800000u;
+    uint32_t mantissa = x & 0x7FFFFFu;
+    int exponent      = (int)((head >> 23) & 0xFF);
+    uint32_t sign     = head >> 31;
+    const int bias    = 127;
+
+    uint32_t signed_inf      = (sign << 7) + (((1u << we) - 1u) << wm);
+    uint32_t signed_all_ones = (sign << 7) + ((((1u << we) - 1u) << wm) + ((1u << wm) - 1u));
+    uint32_t signed_max      = signed_all_ones - 1u; /* wm == 3 */
+
+    if((x & 0x7F800000u) == 0x7F800000u)
+    {
+        if(mantissa == 0)
+            return sign == 0 ? 0x7E : 0xFE;
+        return (uint8_t)(signed_inf + 7u); /* all-ones mantissa NaN */
+    }
+    if(x == 0)
+        return 0;
+    if(x == 0x80000000u)
+        return 0x80;
+
+    const int f8_bias                  = (1 << (we - 1u)) - 1; /* 7 */
+    const int f8_denormal_act_exponent = 1 - f8_bias;          /* -6 */
+    int act_exponent, f8_exponent, exponent_diff;
+
+    if(exponent == 0 && mantissa != 0)
+    {
+        act_exponent  = 1 - bias;
+        exponent_diff = f8_denormal_act_exponent - act_exponent;
+    }
+    else
+    {
+        act_exponent = exponent - bias;
+        if(act_exponent <= f8_denormal_act_exponent)
+            exponent_diff = f8_denormal_act_exponent - act_exponent;
+        else
+            exponent_diff = 0;
+        mantissa += (1u << mfmt);
+    }
+
+    uint32_t sh1 = mfmt - wm + (uint32_t)exponent_diff;
+    if(sh1 > 31u)
+        sh1 = 31u;
+    uint32_t sh2 = mfmt - wm + (uint32_t)exponent_diff - 1u;
+    if(sh2 > 31u)
+        sh2 = 31u;
+    int midpoint = (mantissa & ((1u << sh1) - 1u)) == (1u << sh2);
+
+    if(exponent_diff > 0)
+    {
+        uint32_t s = (uint32_t)exponent_diff;
+        if(s > 31u)
+            s = 31u;
+        mantissa >>= s;
+    }
+    else if(exponent_diff == -1)
+        mantissa <<= 1;
+    int implicit_one = (mantissa & (1u << mfmt)) != 0;
+    f8_exponent      = (act_exponent + exponent_diff) + f8_bias - (implicit_one ? 0 : 1);
+
+    uint32_t drop_mask = (1u << (mfmt - wm)) - 1u;
+    int odd            = (mantissa & (1u << (mfmt - wm))) != 0;
+    mantissa += (midpoint ? (odd ? mantissa : mantissa - 1u) : mantissa) & drop_mask;
+
+    if(f8_exponent == 0 && ((1u << mfmt) & mantissa))
+        f8_exponent = 1;
+    else if((1u << (mfmt + 1)) & mantissa)
+    {
+        mantissa >>= 1;
+        f8_exponent++;
+    }
+    mantissa >>= (mfmt - wm);
+
+    const int max_exp = (1 << we) - 1; /* wm == 3 */
+    if(f8_exponent > max_exp)
+        return (uint8_t)signed_max;
+    if(f8_exponent == 0 && mantissa == 0)
+        return (uint8_t)(sign << 7);
+    mantissa &= (1u << wm) - 1u;
+    uint8_t r = (uint8_t)((sign << 7) | ((uint32_t)f8_exponent << wm) | mantissa);
+    /* exponent 15 with mantissa 7 is the NaN code: the clip branch above is
+       reached only for f8_exponent > 15, so 0x7f can come out of the rounding
+       carry; the reference returns it unchanged (float8_impl.hpp:243-246). */
+    return r;
+}
+
+/* vector forms for the Python side */
+void orc_half_from_f32_n(const float* x, uint16_t* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_half_from_f32(x[i]);
+}
+void orc_half_to_f32_n(const uint16_t* x, float* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_half_to_f32(x[i]);
+}
+void orc_bf16_from_f32_n(const float* x, uint16_t* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_bf16_from_f32(x[i]);
+}
+void orc_bf16_to_f32_n(const uint16_t* x, float* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_bf16_to_f32(x[i]);
+}
+void orc_fp8e4m3fn_from_f32_n(const float* x, uint8_t* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_fp8e4m3fn_from_f32(x[i]);
+}
+void orc_fp8e4m3fn_to_f32_n(const uint8_t* x, float* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_fp8e4m3fn_to_f32(x[i]);
+}
+
+/* ------------------------------------------------------------------------
+ * typed element access: what `static_cast<double>(view[i])` and
+ * `view[i] = double_value` do for each element type on the ref target.
+ * ---------------------------------------------------------------------- */
+static inline double load_f64(const void* p, int type, size_t i)
+{
+    switch(type)
+    {
+    case ORC_I8: return (double)((const int8_t*)p)[i];
+    case ORC_U8: return (double)((const uint8_t*)p)[i];
+    case ORC_I32: return (double)((const int32_t*)p)[i];
+    case ORC_F32: return (double)((const float*)p)[i];
+    case ORC_F16: return (double)orc_half_to_f32(((const uint16_t*)p)[i]);
+    case ORC_BF16: return (double)orc_bf16_to_f32(((const uint16_t*)p)[i]);
+    case ORC_FP8: return (double)orc_fp8e4m3fn_to_f32(((const uint8_t*)p)[i]);
+    case ORC_F64: return ((const double*)p)[i];
+    default: return NAN;
+    }
+}
+
+/* double -> T as C++ does it for `T x = d` / `static_cast<T>(d)`:
+ * integers truncate, float rounds to nearest even, half/bf16/fp8 go through
+ * float first (their constructors take a float) and then apply their own
+ * conversion. */
+static inline void store_f64(void* p, int type, size_t i, double d)
+{
+    switch(type)
+    {
+    case ORC_I8: ((int8_t*)p)[i] = (int8_t)d; break;
+    case ORC_U8: ((uint8_t*)p)[i] = (uint8_t)d; break;
+    case ORC_I32: ((int32_t*)p)[i] = (int32_t)d; break;
+    case ORC_F32: ((float*)p)[i] = (float)d; break;
+    case ORC_F16: ((uint16_t*)p)[i] = orc_half_from_f32((float)d); break;
+    case ORC_BF16: ((uint16_t*)p)[i] = orc_bf16_from_f32((float)d); break;
+    case ORC_FP8: ((uint8_t*)p)[i] = orc_fp8e4m3fn_from_f32((float)d); break;
+    case ORC_F64: ((double*)p)[i] = d; break;
+    default: break;
+    }
+}
+
+static inline double type_max(int type)
+{
+    switch(type)
+    {
+    case ORC_I8: return 127.0;
+    case ORC_U8: return 255.0;
+    case ORC_I32: return 2147483647.0;
+    case ORC_F32: return 3.40282346638528859811704183484516925e+38;
+    case ORC_F16: return 65504.0;
+    case ORC_BF16: return 3.38953138925153547590470800371487867e+38;
+    case ORC_FP8: return 448.0;
+    default: return INFINITY;
+    }
+}
+static inline double type_lowest(int type)
+{
+    if(type == ORC_U8)
+        return 0.0;
+    if(type == ORC_I8)
+        return -128.0;
+    if(type == ORC_I32)
+        return -2147483648.0;
+    return -type_max(type);
+}
+
+/* ------------------------------------------------------------------------
+ * gemm_naive  src/gemm.cpp:42-63, reached from
+ *   ref_quant_gemm::compute  src/targets/ref/lowering.cpp:218-248 (quant_dot)
+ *   op::dot::compute         src/include/migraphx/op/dot.hpp:102-107
+ * One output element at a time: s (double) += double(a) * double(b) for k
+ * ascending, then C = static_cast<T>(s).  Strides are element strides so that
+ * transposed views (simplify_qdq.cpp:49-82 re-applies transposes to the
+ * quantized tensor) need no copy.  C is written row-major, batch outermost.
+ * ---------------------------------------------------------------------- */
+void orc_gemm(void* c,
+              int c_type,
+              const void* a,
+              const void* b,
+              int ab_type,
+              int64_t m,
+              int64_t n,
+              int64_t k,
+              int64_t a_sm,
+              int64_t a_sk,
+              int64_t b_sk,
+              int64_t b_sn,
+              int64_t batch,
+              int64_t a_sb,
+              int64_t b_sb)
+{
+    int64_t total = batch * m * n;
+#pragma omp parallel for schedule(static)
+    for(int64_t idx = 0; idx < total; idx++)
+    {
+        int64_t bi = idx / (m * n);
+        int64_t r  = idx % (m * n);
+        int64_t i  = r / n;
+        int64_t j  = r % n;
+        double s   = 0.0;
+        if(ab_type == ORC_I8)
+        {
+            const int8_t* ap = (const int8_t*)a + bi * a_sb + i * a_sm;
+            const int8_t* bp = (const int8_t*)b + bi * b_sb + j * b_sn;
+            for(int64_t kk = 0; kk < k; kk++)
+                s += (double)ap[kk * a_sk] * (double)bp[kk * b_sk];
+        }
+        else
+        {
+            size_t a0 = (size_t)(bi * a_sb + i * a_sm);
+            size_t b0 = (size_t)(bi * b_sb + j * b_sn);
+            for(int64_t kk = 0; kk < k; kk++)
+                s += load_f64(a, ab_type, a0 + (size_t)(kk * a_sk)) *
+                     load_f64(b, ab_type, b0 + (size_t)(kk * b_sk));
+        }
+        store_f64(c, c_type, (size_t)idx, s);
+    }
+}
+
+/* ------------------------------------------------------------------------
+ * quantizelinear::compute  src/include/migraphx/op/quantizelinear.hpp:71-108
+ * integral output:  clamp(double(nearbyint(x / s)) + double(zp)) where x / s
+ *   is evaluated in the input's own type (float division for float; for half
+ *   and bf16 the quotient is converted back to that type, generic_float.hpp
+ *   :318-326) under FE_TONEAREST.
+ * fp8 output: clamp(double(x) / double(s) + double(zp), -448, 448), then
+ *   double -> float -> fp8.
+ * x is a dense [rows, cols] array; scale and zero point are addressed with
+ * element strides (0 = broadcast) the way the broadcast views of the graph
+ * address them.  zp == NULL means the all-zero default.
+ * ---------------------------------------------------------------------- */
+void orc_quantizelinear(void* out,
+                        int out_type,
+                        const void* x,
+                        int x_type,
+                        const void* scale,
+                        int64_t s_sr,
+                        int64_t s_sc,
+                        const void* zp,
+                        int64_t z_sr,
+                        int64_t z_sc,
+                        int64_t rows,
+                        int64_t cols)
+{
+    int old = fegetround();
+    fesetround(FE_TONEAREST);
+    double lo    = type_lowest(out_type);
+    double hi    = type_max(out_type);
+    int integral = (out_type == ORC_I8 || out_type == ORC_U8 || out_type == ORC_I32);
+#pragma omp parallel for schedule(static)
+    for(int64_t r = 0; r < rows; r++)
+    {
+        fesetround(FE_TONEAREST);
+        for(int64_t c = 0; c < cols; c++)
+        {
+            size_t i  = (size_t)(r * cols + c);
+            size_t si = (size_t)(r * s_sr + c * s_sc);
+            double z  = zp ? load_f64(zp, out_type, (size_t)(r * z_sr + c * z_sc)) : 0.0;
+            double q;
+            if(integral)
+            {
+                float xv = (float)load_f64(x, x_type, i);
+                float sv = (float)load_f64(scale, x_type, si);
+                float d  = xv / sv;
+                if(x_type == ORC_F16)
+                    d = orc_half_to_f32(orc_half_from_f32(d));
+                else if(x_type == ORC_BF16)
+                    d = orc_bf16_to_f32(orc_bf16_from_f32(d));
+                q = (double)nearbyintf(d) + z;
+            }
+            else
+            {
+                q = load_f64(x, x_type, i) / load_f64(scale, x_type, si) + z;
+            }
+            double v = fmax(lo, fmin(hi, q));
+            store_f64(out, out_type, i, v);
+        }
+    }
+    fesetround(old);
+}
+
+/* ------------------------------------------------------------------------
+ * dequantizelinear::compute src/include/migraphx/op/dequantizelinear.hpp:60-83
+ * out = (double(x) - double(zp)) * scale, product in double (the scale is
+ * promoted), stored to the scale's type.
+ * ---------------------------------------------------------------------- */
+void orc_dequantizelinear(void* out,
+                          const void* x,
+                          int x_type,
+                          const void* scale,
+                          int s_type,
+                          int64_t s_sr,
+                          int64_t s_sc,
+                          const void* zp,
+                          int64_t z_sr,
+                          int64_t z_sc,
+                          int64_t rows,
+                          int64_t cols)
+{
+#pragma omp parallel for schedule(static)
+    for(int64_t r = 0; r < rows; r++)
+    {
+        for(int64_t c = 0; c < cols; c++)
+        {
+            size_t i = (size_t)(r * cols + c);
+            double z = zp ? load_f64(zp, x_type, (size_t)(r * z_sr + c * z_sc)) : 0.0;
+            double s = load_f64(scale, s_type, (size_t)(r * s_sr + c * s_sc));
+            store_f64(out, s_type, i, (load_f64(x, x_type, i) - z) * s);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------
+ * unpack_int4::compute  src/include/migraphx/op/unpack_int4.hpp:75-121
+ * pack_int4::compute    src/include/migraphx/op/pack_int4.hpp:79-124
+ * Dense tensor seen as [outer, axis_len, inner]; the axis doubles (unpack) or
+ * halves (pack).  Low nibble is the even element.
+ * ---------------------------------------------------------------------- */
+void orc_unpack_int4(
+    uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t a = 0; a < axis_len; a++)
+            for(int64_t i = 0; i < inner; i++)
+            {
+                uint8_t v   = in[(o * axis_len + a) * inner + i];
+                size_t lo_i = (size_t)((o * 2 * axis_len + 2 * a) * inner + i);
+                size_t hi_i = lo_i + (size_t)inner;
+                if(is_signed)
+                {
+                    int8_t v1   = (int8_t)(uint8_t)(v << 4);
+                    v1          = (int8_t)(v1 >> 4);
+                    int8_t v2   = (int8_t)((int8_t)v >> 4);
+                    out[lo_i]   = (uint8_t)v1;
+                    out[hi_i]   = (uint8_t)v2;
+                }
+                else
+                {
+                    out[lo_i] = v & 0xf;
+                    out[hi_i] = v >> 4;
+                }
+            }
+}
+
+void orc_pack_int4(
+    uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    /* axis_len is the OUTPUT axis length; the input axis is 2*axis_len */
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t a = 0; a < axis_len; a++)
+            for(int64_t i = 0; i < inner; i++)
+            {
+                size_t i1 = (size_t)((o * 2 * axis_len + 2 * a) * inner + i);
+                size_t i2 = i1 + (size_t)inner;
+                uint8_t u1, u2;
+                if(is_signed)
+                {
+                    int8_t v1 = (int8_t)in[i1], v2 = (int8_t)in[i2];
+                    v1 = v1 < -8 ? -8 : (v1 > 7 ? 7 : v1);
+                    v2 = v2 < -8 ? -8 : (v2 > 7 ? 7 : v2);
+                    u1 = (uint8_t)v1;
+                    u2 = (uint8_t)v2;
+                }
+                else
+                {
+                    u1 = in[i1] > 15 ? 15 : in[i1];
+                    u2 = in[i2] > 15 ? 15 : in[i2];
+                }
+                out[(o * axis_len + a) * inner + i] = (uint8_t)((u2 << 4) | (u1 & 0xf));
+            }
+}
+
+/* ------------------------------------------------------------------------
+ * convert::compute  src/include/migraphx/op/convert.hpp:64-87
+ * NaN -> quiet NaN of the target, +-inf kept for float targets, values at or
+ * beyond the finite range saturate to max/lowest, otherwise T(double(x)).
+ * ---------------------------------------------------------------------- */
+void orc_convert(void* out, int out_type, const void* x, int x_type, size_t n)
+{
+    int integral = (out_type == ORC_I8 || out_type == ORC_U8 || out_type == ORC_I32);
+#pragma omp parallel for schedule(static)
+    for(size_t i = 0; i < n; i++)
+    {
+        double dx = load_f64(x, x_type, i);
+        if(isnan(dx))
+        {
+            switch(out_type)
+            {
+            case ORC_F32: ((float*)out)[i] = bits_f32(0x7fc00000u); break;
+            case ORC_F16: ((uint16_t*)out)[i] = 0x7e00; break;
+            case ORC_BF16: ((uint16_t*)out)[i] = 0x7fc0; break;
+            case ORC_FP8: ((uint8_t*)out)[i] = 0x7f; break;
+            default: store_f64(out, out_type, i, 0.0); break;
+            }
+            continue;
+        }
+        if(!integral && isinf(dx))
+        {
+            store_f64(out, out_type, i, dx);
+            continue;
+        }
+        if(dx >= type_max(out_type))
+            dx = type_max(out_type);
+        else if(dx <= type_lowest(out_type))
+            dx = type_lowest(out_type);
+        store_f64(out, out_type, i, dx);
+    }
+}
+
+/* mul of two float tensors (op/mul.hpp via op/binary.hpp): plain IEEE float
+ * product, used by simplify_qdq.cpp:243-248 to combine the two input scales.
+ * a is addressed [r*a_sr + c*a_sc], same for b; out is dense. */
+void orc_mul_f32(float* out,
+                 const float* a,
+                 int64_t a_sr,
+                 int64_t a_sc,
+                 const float* b,
+                 int64_t b_sr,
+                 int64_t b_sc,
+                 int64_t rows,
+                 int64_t cols)
+{
+    for(int64_t r = 0; r < rows; r++)
+        for(int64_t c = 0; c < cols; c++)
+            out[r * cols + c] = a[r * a_sr + c * a_sc] * b[r * b_sr + c * b_sc];
+}

@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Collect the known-answer vectors that the reference's own tests hold for the
+quantized-GEMM path and write them to ``reference_vectors.json``.
+
+Run in the build container only (it reads the reference tree as text):
+
+    python tests/golden/extract_reference_vectors.py [/root/reference]
+
+The output holds DATA only: literal inputs, shapes, attributes and expected
+outputs of the reference's test cases, each tagged with the file it was read
+from.  No reference code is executed, imported or stored.
+"""
+import json
+import os
+import re
+import sys
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_vectors.json")
+
+
+def read(rel):
+    with open(os.path.join(REF, rel)) as f:
+        return f.read()
+
+
+def num(tok):
+    t = tok.strip().replace("'", "")
+    t = re.sub(r"/\*.*?\*/", "", t).strip()
+    if not t:
+        return None
+    if "quiet_NaN" in t:
+        return "nan"
+    if "infinity" in t:
+        return "-inf" if t.startswith("-") else "inf"
+    neg = t.startswith("-")
+    if neg:
+        t = t[1:]
+    if t.lower().startswith("0x"):
+        v = int(t, 16)
+    elif t.lower().startswith("0b"):
+        v = int(t, 2)
+    else:
+        t = t.rstrip("fF")
+        v = float(t) if any(c in t for c in ".eE") else int(t)
+    return -v if neg else v
+
+
+def num_list(s):
+    s = re.sub(r"/\*.*?\*/", "", s, flags=re.S)
+    s = re.sub(r"//[^\n]*", "", s)
+    return [v for v in (num(t) for t in s.split(",")) if v is not None]
+
+
+def test_cases(text):
+    """name -> body for every TEST_CASE(name) { ... } (bodies end at the next
+    TEST_CASE / template / EOF, which is enough for vector scraping)."""
+    out = {}
+    marks = [(m.start(), m.group(1)) for m in re.finditer(r"TEST_CASE\((\w+)\)", text)]
+    cuts = sorted([p for p, _ in marks] +
+                  [m.start() for m in re.finditer(r"\ntemplate <", text)] + [len(text)])
+    for pos, name in marks:
+        end = min(c for c in cuts if c > pos)
+        out[name] = text[pos:end]
+    return out
+
+
+def vec(body, name):
+    m = re.search(r"\b" + re.escape(name) + r"\s*(?:=\s*)?\{(.*?)\};", body, re.S)
+    if not m:
+        return None
+    return num_list(m.group(1))
+
+
+def shape(body, name):
+    m = re.search(r"(?:migraphx::shape\s+" + re.escape(name) + r"|auto " + re.escape(name) +
+                  r"\s*=\s*migraphx::shape)"
+                  r"\{migraphx::shape::(\w+)_type,\s*\{([^}]*)\}(?:,\s*\{([^}]*)\})?\}", body)
+    if not m:
+        return None
+    d = {"type": m.group(1), "lens": num_list(m.group(2))}
+    if m.group(3):
+        d["strides"] = num_list(m.group(3))
+    return d
+
+
+out = {"_provenance": "literal inputs and expected outputs read from the reference's test sources"}
+
+# ---- fp8 e4m3fn table and cast samples (test/fp8e4m3fn.cpp) ------------------
+t = read("test/fp8e4m3fn.cpp")
+m = re.search(r"e4m3fnuz_lut = \{(.*?)\};", t, re.S)
+out["fp8e4m3fn_lut"] = {"source": "test/fp8e4m3fn.cpp:34-105", "values": num_list(m.group(1))}
+m = re.search(r"test_vals = \{\s*\{(.*?)\}\};", t, re.S)
+pairs = re.findall(r"\{\s*([-+0-9.eE]+)\s*,\s*(0x[0-9a-fA-F]+)\s*\}", m.group(1))
+out["fp8e4m3fn_from_float"] = {"source": "test/fp8e4m3fn.cpp:121-140",
+                               "pairs": [[float(a), int(b, 16)] for a, b in pairs]}
+
+# ---- half / bf16 tables ------------------------------------------------------
+for nm, rel in (("half", "test/half.cpp"), ("bf16", "test/bf16.cpp")):
+    t = read(rel)
+    m = re.search(nm + r"_lut\(\).*?result = \{(.*?)\n    \};", t, re.S)
+    pairs = re.findall(r"\{\s*(0x[0-9a-fA-F]+)\s*,\s*([^}]+)\}", m.group(1))
+    out[nm + "_lut"] = {"source": rel, "pairs": [[int(a, 16), num(b)] for a, b in pairs]}
+
+# ---- quant_dot known answers (test/ref/dot_op.cpp) -----------------------------
+t = read("test/ref/dot_op.cpp")
+cases = test_cases(t)
+qd = []
+for name, body in cases.items():
+    if not name.startswith("quant_dot_") or "4args" in name:
+        continue
+    c = {"name": name, "source": "test/ref/dot_op.cpp"}
+    c["a"] = shape(body, "m1_shape")
+    c["b"] = shape(body, "m2_shape")
+    c["c"] = shape(body, "m3_shape")
+    c["a_perm"] = None
+    c["b_perm"] = None
+    m1 = re.search(r"auto tl1\s*=\s*mm->add_instruction\(\s*migraphx::make_op\(\"transpose\", "
+                   r"\{\{\"permutation\", \{([^}]*)\}\}\}\),\s*l1\)", body, re.S)
+    m2 = re.search(r"auto tl2\s*=\s*mm->add_instruction\(\s*migraphx::make_op\(\"transpose\", "
+                   r"\{\{\"permutation\", \{([^}]*)\}\}\}\),\s*l2\)", body, re.S)
+    if m1:
+        c["a_perm"] = num_list(m1.group(1))
+    if m2:
+        c["b_perm"] = num_list(m2.group(1))
+    ab = re.search(r"add_apply_alpha_beta\(\s*\*mm,\s*\{([^}]*)\},\s*migraphx::make_op\(\"quant_dot\"\)"
+                   r"(?:,\s*([-0-9.]+))?(?:,\s*([-0-9.]+))?\)", body, re.S)
+    c["alpha"], c["beta"], c["uses_c"] = 1, 0, False
+    if ab:
+        args = [a.strip() for a in ab.group(1).split(",")]
+        c["uses_c"] = len(args) == 3
+        if ab.group(2):
+            c["alpha"] = num(ab.group(2))
+        if ab.group(3):
+            c["beta"] = num(ab.group(3))
+    c["iota_start"] = {"a": 0, "b": 0}
+    m3 = re.search(r"std::iota\(data3\.begin\(\), data3\.end\(\), (\d+)\)", body)
+    if m3:
+        c["iota_start"]["c"] = int(m3.group(1))
+    c["gold"] = vec(body, "gold")
+    qd.append(c)
+out["quant_dot"] = qd
+
+body = cases["quant_dot_4args_scales"]
+out["quant_dot_4args_scales"] = {
+    "source": "test/ref/dot_op.cpp", "a": vec(body, "a_data"), "b": vec(body, "b_data"),
+    "scale_a": vec(body, "scale_a_data"), "scale_b": vec(body, "scale_b_data"),
+    "a_lens": [2, 3], "b_lens": [3, 2], "gold": vec(body, "gold")}
+
+# ---- quantizelinear / dequantizelinear -----------------------------------------
+t = read("test/ref/quantizelinear.cpp")
+cases = test_cases(t)
+ql = []
+for name in ("quantizelinear_1", "quantizelinear_2"):
+    body = cases[name]
+    ql.append({"name": name, "source": "test/ref/quantizelinear.cpp", "x": vec(body, "xv"),
+               "scale": vec(body, "sv"), "zp": vec(body, "zv"),
+               "zp_type": (shape(body, "zs") or {}).get("type"),
+               "lens": shape(body, "xs")["lens"], "gold": vec(body, "gold")})
+out["quantizelinear"] = ql
+m = re.search(r"static void quantizelinear_fp8e4m3\(\)(.*?)TEST_CASE_REGISTER", t, re.S)
+body = m.group(1)
+out["quantizelinear_fp8e4m3"] = {
+    "source": "test/ref/quantizelinear.cpp:86-127 (gold is computed there as "
+              "fp8(clamp(x/s + fp8(zp))) in double)",
+    "x": vec(body, "xv"), "scale": vec(body, "sv"), "zp_float": vec(body, "tmp"), "lens": [2, 2, 2]}
+
+t = read("test/ref/dequantizelinear.cpp")
+cases = test_cases(t)
+dq = []
+for name, body in cases.items():
+    dq.append({"name": name, "source": "test/ref/dequantizelinear.cpp", "x": vec(body, "xv"),
+               "x_type": shape(body, "xs")["type"], "scale": vec(body, "sv"), "zp": vec(body, "zv"),
+               "lens": shape(body, "xs")["lens"], "gold": vec(body, "gold")})
+out["dequantizelinear"] = dq
+
+# ---- unpack_int4 / pack_int4 -----------------------------------------------------
+def int4_cases(rel, opname):
+    t = read(rel)
+    res = []
+    for name, body in test_cases(t).items():
+        s = shape(body, "s")
+        lit = re.search(r"migraphx::literal\{\s*s,\s*\{(.*?)\}\}", body, re.S)
+        if not s or not lit:
+            continue
+        c = {"name": name, "source": rel, "shape": s, "data": num_list(lit.group(1)),
+             "gold": vec(body, "gold")}
+        ax = re.search(r"make_op\(\"" + opname + r"\", \{\{\"axis\", (-?\d+)\}\}\)", body)
+        c["axis"] = int(ax.group(1)) if ax else -1
+        mb = re.search(r"multibroadcast\", \{\{\"out_lens\", \{([^}]*)\}\}\}", body)
+        c["multibroadcast"] = num_list(mb.group(1)) if mb else None
+        res.append(c)
+    return res
+
+
+out["unpack_int4"] = int4_cases("test/ref/unpack_int4.cpp", "unpack_int4")
+out["pack_int4"] = int4_cases("test/ref/pack_int4.cpp", "pack_int4")
+
+# ---- MatMulNBits end-to-end golds (test/onnx/verify/matmulnbits_tests.cpp) -------
+# N, K and block size are fixed by the tensor shapes: b is [N, ceil(K/blk), blk/2]
+# (src/onnx/parse_matmulnbits.cpp:60-66) and K is a's last dimension.
+t = read("test/onnx/verify/matmulnbits_tests.cpp")
+mn = []
+for name, body in test_cases(t).items():
+    c = {"name": name, "source": "test/onnx/verify/matmulnbits_tests.cpp",
+         "a_lens": shape(body, "a_shape")["lens"], "b_lens": shape(body, "b_shape")["lens"]}
+    m = re.search(r"std::vector<float> a\{(.*?)\};", body, re.S)
+    c["a"] = num_list(m.group(1)) if m else "iota"
+    c["b"] = vec(body, "b")
+    c["scales"] = vec(body, "scales")
+    c["zp"] = vec(body, "zp") if "zp_shape" in body else None
+    c["gold"] = vec(body, "gold")
+    mn.append(c)
+out["matmulnbits"] = mn
+
+with open(OUT, "w") as f:
+    json.dump(out, f, indent=0, separators=(",", ":"))
+print("wrote", OUT, os.path.getsize(OUT), "bytes")
+for k, v in out.items():
+    if isinstance(v, list):
+        print(" ", k, len(v), "cases")
