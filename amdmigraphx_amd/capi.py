@@ -1,0 +1,102 @@
+"""ctypes binding of ``libmi355_qgemm.so`` (see ``include/mi355_qgemm.h``).
+
+There is no fallback: if the library cannot be loaded every use raises
+``Mi355Error``.  Pointers are raw device addresses (``tensor.data_ptr()``)."""
+import ctypes
+import os
+import subprocess
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_PKG, "lib", "libmi355_qgemm.so")
+
+
+class Mi355Error(RuntimeError):
+    pass
+
+
+class DT:
+    I8, U8, I32, F32, F16, BF16, FP8 = range(7)
+
+
+class QP:
+    NONE, PER_TENSOR, PER_ROW, PER_COL = range(4)
+
+
+class W4ZP:
+    SCALAR, GROUP, PACKED = range(3)
+
+
+class QuantDotDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in
+                ("m", "n", "k", "lda", "ldb", "ldc", "batch", "stride_a", "stride_b", "stride_c")] + \
+               [(n, ctypes.c_int32) for n in
+                ("trans_a", "trans_b", "in_type", "out_type", "dequant", "scale_a_mode",
+                 "scale_b_mode", "zp_a", "zp_b")]
+
+
+EXPORTS = {
+    "mi355_quant_dot": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 8,
+    "mi355_colsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                        ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p],
+    "mi355_rowsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                        ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p],
+    "mi355_quantizelinear": [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int64,
+                             ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                             ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
+                             ctypes.c_void_p],
+    "mi355_dequantizelinear": [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32,
+                               ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64,
+                               ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                               ctypes.c_void_p],
+    "mi355_unpack_int4": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64,
+                          ctypes.c_int64, ctypes.c_void_p],
+    "mi355_pack_int4": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64,
+                        ctypes.c_int64, ctypes.c_void_p],
+    "mi355_convert": [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32,
+                      ctypes.c_int64, ctypes.c_void_p],
+    "mi355_w4a16_gemm": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+                         ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
+                         ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                         ctypes.c_int64, ctypes.c_void_p],
+    "mi355_status_string": [ctypes.c_int],
+    "mi355_version": [],
+}
+
+
+def lib_path():
+    return _LIB
+
+
+def build_library(force=True):
+    """Compile every HIP source for gfx950 into lib/libmi355_qgemm.so."""
+    cmd = ["make", "-C", os.path.join(_PKG, "csrc"), "-j8"]
+    if force:
+        cmd.append("-B")
+    subprocess.check_call(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+
+
+_handle = None
+
+
+def lib():
+    """The loaded library with argument types set; raises if it is missing."""
+    global _handle
+    if _handle is None:
+        if not os.path.exists(_LIB):
+            raise Mi355Error(f"{_LIB} is not built: run __graft_entry__.build() "
+                             "(make -C amdmigraphx_amd/csrc)")
+        try:
+            h = ctypes.CDLL(_LIB)
+        except OSError as e:
+            raise Mi355Error(f"cannot load {_LIB}: {e}") from e
+        for name, argtypes in EXPORTS.items():
+            fn = getattr(h, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_char_p if name == "mi355_status_string" else ctypes.c_int
+        _handle = h
+    return _handle
+
+
+def check(status, what):
+    if status != 0:
+        raise Mi355Error(f"{what}: {lib().mi355_status_string(status).decode()} ({status})")

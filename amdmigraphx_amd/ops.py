@@ -1,0 +1,220 @@
+"""Torch-tensor front end over the C ABI, used by the tests, the smoke check
+and the benchmark.  torch supplies device memory and streams only; every
+computation goes through ``libmi355_qgemm.so``.
+
+Operator names and argument meaning follow the MIGraphX operators they stand
+for (quant_dot, quantizelinear, dequantizelinear, unpack_int4, pack_int4,
+convert); low-precision tensors without a torch dtype contract travel as raw
+bits (uint8 for fp8 e4m3fn, int16/uint16 views for half and bf16 are taken from
+torch.float16 / torch.bfloat16 tensors directly)."""
+import ctypes
+
+import torch
+
+from .capi import DT, QP, W4ZP, QuantDotDesc, Mi355Error, check, lib
+
+_TORCH2DT = {torch.int8: DT.I8, torch.uint8: DT.U8, torch.int32: DT.I32, torch.float32: DT.F32,
+             torch.float16: DT.F16, torch.bfloat16: DT.BF16}
+_DT2TORCH = {DT.I8: torch.int8, DT.U8: torch.uint8, DT.I32: torch.int32, DT.F32: torch.float32,
+             DT.F16: torch.float16, DT.BF16: torch.bfloat16, DT.FP8: torch.uint8}
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _require_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise Mi355Error("operands must be device tensors")
+
+
+def _mat_layout(t):
+    """(trans, ld, batch_stride) of a [..., R, C] view that is row-major or a
+    transpose of row-major storage in its last two dims."""
+    r, c = t.shape[-2:]
+    sr, sc = t.stride()[-2:]
+    if sc == 1 or c == 1:
+        return 0, max(sr if r > 1 else c, c, 1)
+    if sr == 1 or r == 1:
+        return 1, max(sc if c > 1 else r, r, 1)
+    raise Mi355Error("matrix is neither row-major nor a transpose view")
+
+
+def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
+              colsum_b=None, rowsum_a=None, out_dtype=None, out=None):
+    """quant_dot, optionally with the fused dequantizelinear epilogue.
+
+    a [..., M, K], b [..., K, N] int8 (or uint8 carrying fp8 e4m3fn bits with
+    fp8=True); transposed views are passed as they are.  Without scales the
+    bare accumulators come back (int32 / float32).  With ``scale_a`` (scalar
+    or [M]) / ``scale_b`` (scalar or [N]) float32 tensors the epilogue
+    (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied."""
+    _require_cuda(a, b, scale_a, scale_b)
+    if a.dim() != b.dim() or a.dim() < 2:
+        raise Mi355Error("QUANT_DOT: dot only accepts >= 2D operands of equal rank")
+    if a.shape[:-2] != b.shape[:-2]:
+        raise Mi355Error("QUANT_DOT: outer dimensions of A and B mismatch")
+    if a.shape[-1] != b.shape[-2]:
+        raise Mi355Error("QUANT_DOT: inner dimensions are not compatible")
+    if a.dtype != b.dtype:
+        raise Mi355Error("QUANT_DOT: operands must have the same type")
+    batch_shape = a.shape[:-2]
+    m, k = a.shape[-2:]
+    n = b.shape[-1]
+    nb = 1
+    for s in batch_shape:
+        nb *= s
+    if a.dim() > 2:
+        a3 = a.reshape((nb, m, k)) if a.dim() > 3 else a
+        b3 = b.reshape((nb, k, n)) if b.dim() > 3 else b
+        sa, sb = a3.stride(0), b3.stride(0)
+    else:
+        a3, b3, sa, sb = a, b, 0, 0
+    ta, lda = _mat_layout(a3)
+    tb, ldb = _mat_layout(b3)
+    dequant = scale_a is not None or scale_b is not None or out_dtype is not None
+    in_type = DT.FP8 if fp8 else DT.I8
+    if dequant:
+        odt = out_dtype or torch.float32
+    else:
+        odt = torch.float32 if fp8 else torch.int32
+    if out is None:
+        out = torch.empty(batch_shape + (m, n), dtype=odt, device=a.device)
+    d = QuantDotDesc(m=m, n=n, k=k, lda=lda, ldb=ldb, ldc=n, batch=nb, stride_a=sa, stride_b=sb,
+                     stride_c=m * n, trans_a=ta, trans_b=tb, in_type=in_type,
+                     out_type=_TORCH2DT[odt], dequant=int(dequant),
+                     scale_a_mode=QP.NONE if scale_a is None else
+                     (QP.PER_TENSOR if scale_a.numel() == 1 else QP.PER_ROW),
+                     scale_b_mode=QP.NONE if scale_b is None else
+                     (QP.PER_TENSOR if scale_b.numel() == 1 else QP.PER_COL),
+                     zp_a=int(zp_a), zp_b=int(zp_b))
+    if scale_a is not None and scale_a.numel() not in (1, m):
+        raise Mi355Error("scale_a must be a scalar or have M elements")
+    if scale_b is not None and scale_b.numel() not in (1, n):
+        raise Mi355Error("scale_b must be a scalar or have N elements")
+    st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
+                               _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
+    check(st, "mi355_quant_dot")
+    return out
+
+
+def colsum_i8(b):
+    k, n = b.shape
+    tb, ldb = _mat_layout(b)
+    out = torch.empty(n, dtype=torch.int32, device=b.device)
+    check(lib().mi355_colsum_i8(_ptr(b), k, n, ldb, tb, _ptr(out), _stream()), "mi355_colsum_i8")
+    return out
+
+
+def rowsum_i8(a):
+    m, k = a.shape
+    ta, lda = _mat_layout(a)
+    out = torch.empty(m, dtype=torch.int32, device=a.device)
+    check(lib().mi355_rowsum_i8(_ptr(a), m, k, lda, ta, _ptr(out), _stream()), "mi355_rowsum_i8")
+    return out
+
+
+def _qparam_strides(p, rows, cols):
+    if p is None:
+        return 0, 0
+    if p.numel() == 1:
+        return 0, 0
+    if p.dim() == 1 and p.numel() == cols:
+        return 0, 1
+    if p.dim() == 1 and p.numel() == rows:
+        return 1, 0
+    if p.numel() == rows * cols:
+        return cols, 1
+    raise Mi355Error("quantization parameter does not broadcast to the input")
+
+
+def quantizelinear(x, scale, zp=None, out_type=DT.I8):
+    """quantizelinear of a dense tensor (last dim = columns).  ``scale`` has
+    x's dtype; ``zp`` the output's (uint8 bits for fp8)."""
+    _require_cuda(x, scale, zp)
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    if scale.dtype != x.dtype:
+        raise Mi355Error("QUANTIZELINEAR: Scales and input must be the same type")
+    out = torch.empty(x.shape, dtype=_DT2TORCH[out_type], device=x.device)
+    ssr, ssc = _qparam_strides(scale, rows, cols)
+    zsr, zsc = _qparam_strides(zp, rows, cols)
+    st = lib().mi355_quantizelinear(_ptr(x), _TORCH2DT[x.dtype], _ptr(scale.contiguous()), ssr, ssc,
+                                    _ptr(None if zp is None else zp.contiguous()), zsr, zsc,
+                                    _ptr(out), out_type, rows, cols, _stream())
+    check(st, "mi355_quantizelinear")
+    return out
+
+
+def dequantizelinear(x, scale, zp=None, x_type=None):
+    _require_cuda(x, scale, zp)
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    xt = x_type if x_type is not None else _TORCH2DT[x.dtype]
+    out = torch.empty(x.shape, dtype=scale.dtype, device=x.device)
+    ssr, ssc = _qparam_strides(scale, rows, cols)
+    zsr, zsc = _qparam_strides(zp, rows, cols)
+    st = lib().mi355_dequantizelinear(_ptr(x), xt, _ptr(scale.contiguous()), _TORCH2DT[scale.dtype],
+                                      ssr, ssc, _ptr(None if zp is None else zp.contiguous()),
+                                      zsr, zsc, _ptr(out), rows, cols, _stream())
+    check(st, "mi355_dequantizelinear")
+    return out
+
+
+def unpack_int4(x):
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    out = torch.empty(x.shape[:-1] + (cols * 2,), dtype=x.dtype, device=x.device)
+    check(lib().mi355_unpack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
+                                  _stream()), "mi355_unpack_int4")
+    return out
+
+
+def pack_int4(x):
+    x = x.contiguous()
+    cols = x.shape[-1]
+    if cols % 2:
+        raise Mi355Error("PACK_INT4: Can not pack axis that has odd lengths")
+    rows = x.numel() // max(cols, 1)
+    out = torch.empty(x.shape[:-1] + (cols // 2,), dtype=x.dtype, device=x.device)
+    check(lib().mi355_pack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
+                                _stream()), "mi355_pack_int4")
+    return out
+
+
+def convert(x, out_type, in_type=None):
+    x = x.contiguous()
+    it = in_type if in_type is not None else _TORCH2DT[x.dtype]
+    out = torch.empty(x.shape, dtype=_DT2TORCH[out_type], device=x.device)
+    check(lib().mi355_convert(_ptr(x), it, _ptr(out), out_type, x.numel(), _stream()),
+          "mi355_convert")
+    return out
+
+
+def w4a16_gemm(a, w_packed, scales, group, zp=8, zp_mode=None, out=None):
+    """fp16 activations [M, K] times int4 weights packed [N, K/2] with fp16
+    group scales [N, K/group]; zp is an int (per tensor) or a uint8 tensor."""
+    _require_cuda(a, w_packed, scales)
+    m, k = a.shape
+    n = w_packed.shape[0]
+    if w_packed.shape[1] * 2 != k:
+        raise Mi355Error("packed weight does not match K")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    if isinstance(zp, int):
+        zptr, mode, zs = None, W4ZP.SCALAR, zp
+    else:
+        zptr, zs = _ptr(zp), 0
+        mode = zp_mode if zp_mode is not None else W4ZP.GROUP
+    st = lib().mi355_w4a16_gemm(_ptr(a), a.stride(0), _ptr(w_packed), _ptr(scales), zptr, mode, zs,
+                                _ptr(out), out.stride(0), m, n, k, group, _stream())
+    check(st, "mi355_w4a16_gemm")
+    return out

@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one int8 quant_dot (A[8192,8192] . B[8192,8192] -> int32, row-major,
+uniform int8 operands: BASELINE config 2 at its largest size) launched through
+the C ABI with both operands resident in HBM.  One JSON line is printed with
+the whole-job throughput in TOPS (2*M*N*K operations per step), the MFMA
+roofline fraction of the kernel (HIP events around the launches, on the stream
+they run on), and the CPU oracle's rate on a bounded slab of the same problem.
+The other shape classes of the metric (fp8 quant_dot, int4 weight-only GEMV)
+are reported in the same line under "also".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TOPS_INT8 = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_TFLOPS_FP8 = 5000.0  # dense fp8 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def _time_launches(fn, steps, warmup):
+    """Average device time of one call of fn, from events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return e0.elapsed_time(e1) / steps * 1e-3, wall
+
+
+def cpu_baseline(rows=16, n=8192, k=8192):
+    """The oracle (a port of the ref target's gemm_naive) on a slab of `rows`
+    output rows of the 8192^3 problem, all host threads."""
+    import numpy as np
+    from oracle import oracle as orc
+    rng = np.random.default_rng(0)
+    a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    t0 = time.perf_counter()
+    orc.quant_dot(a, b, orc.I8)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": 2.0 * rows * n * k / dt / 1e12, "unit": "TOPS", "cores": cores, "kind": "port",
+            "sample": f"{rows} of 8192 output rows of the 8192^3 int8 quant_dot, {dt:.1f} s, "
+                      "one repetition (rate extrapolates linearly in rows)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=256)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+    from amdmigraphx_amd import ops
+    torch.cuda.set_device(0)
+    dev = "cuda:0"
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+
+    # ---- headline: int8 quant_dot 8192^3 -> int32 --------------------------------
+    M = N = K = 8192
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+    b = torch.randint(-128, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+    c = torch.empty((M, N), dtype=torch.int32, device=dev)
+
+    def step():
+        ops.quant_dot(a, b, out=c)
+
+    kern_s, wall_s = _time_launches(step, args.steps, args.warmup)
+    ops_per_step = 2.0 * M * N * K
+    tops = ops_per_step / wall_s / 1e12
+    kern_tops = ops_per_step / kern_s / 1e12
+
+    also = {}
+    # ---- fp8 quant_dot with dequant epilogue, Llama-3-8B shape (config 3) ----------
+    try:
+        m3, k3, n3 = 4096, 4096, 14336 * 2
+        a8 = torch.randint(0, 0x7e, (m3, k3), dtype=torch.uint8, device=dev, generator=g)
+        b8 = torch.randint(0, 0x7e, (k3, n3), dtype=torch.uint8, device=dev, generator=g)
+        s1 = torch.full((1,), 0.01, dtype=torch.float32, device=dev)
+        s2 = torch.full((1,), 0.02, dtype=torch.float32, device=dev)
+        o8 = torch.empty((m3, n3), dtype=torch.bfloat16, device=dev)
+        t8, _ = _time_launches(lambda: ops.quant_dot(a8, b8, fp8=True, scale_a=s1, scale_b=s2,
+                                                     out_dtype=torch.bfloat16, out=o8),
+                               max(3, args.steps // 2), 2)
+        f8 = 2.0 * m3 * k3 * n3 / t8 / 1e12
+        also["fp8_quant_dot_bf16_out_M4096_K4096_N28672"] = {
+            "TFLOPS": round(f8, 1), "frac_mfma_peak": round(f8 / PEAK_TFLOPS_FP8, 4)}
+        del a8, b8, o8
+    except Exception as e:  # report, never hide the headline
+        also["fp8_quant_dot_error"] = str(e)
+
+    # ---- int4 weight-only GEMV, M = 1 (config 4) -------------------------------------
+    try:
+        for (k4, n4) in ((4096, 4096), (4096, 14336), (14336, 4096)):
+            grp = 128
+            bytes_per = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * k4 + 2 * n4
+            # rotate through enough weight copies to exceed the 256 MB last-level cache
+            copies = max(2, int(640e6 // bytes_per) + 1)
+            ws = [torch.randint(0, 256, (n4, k4 // 2), dtype=torch.uint8, device=dev, generator=g)
+                  for _ in range(copies)]
+            sc = [(torch.rand((n4, k4 // grp), device=dev, generator=g) * 0.015 + 0.005).half()
+                  for _ in range(copies)]
+            x = torch.randn((1, k4), device=dev, generator=g).half()
+            y = torch.empty((1, n4), dtype=torch.float16, device=dev)
+            it = [0]
+
+            def gemv():
+                i = it[0] % copies
+                it[0] += 1
+                ops.w4a16_gemm(x, ws[i], sc[i], grp, zp=8, out=y)
+
+            tg, _ = _time_launches(gemv, copies * 3, copies)
+            gbs = bytes_per / tg / 1e9
+            also[f"w4a16_gemv_M1_K{k4}_N{n4}"] = {"GB/s": round(gbs, 1),
+                                                 "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                                                 "us": round(tg * 1e6, 2)}
+            del ws, sc
+    except Exception as e:
+        also["w4a16_gemv_error"] = str(e)
+
+    line = {
+        "metric": "quant_dot TOPS & % MFMA peak (int8/fp8); int4 W-only GEMV GB/s & % HBM",
+        "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_s * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "int8 quant_dot A[8192,8192] x B[8192,8192] -> int32, row-major, "
+                               "uniform int8 (BASELINE config 2, M=N=K=8192)",
+                   "m": M, "n": N, "k": K},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_TOPS_INT8,
+                     "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
+                     "traffic": None},
+        "also": also,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(rows=args.cpu_rows)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,219 @@
+/*
+ * mi355_qgemm.h -- C ABI of the MI355X (gfx950) quantized-GEMM kernels.
+ *
+ * This is the boundary a MIGraphX target's lowered operators call from their
+ * `compute(context&, shape, args)`: plain device pointers and sizes in, a
+ * status code out.  Every entry point
+ *   - takes DEVICE pointers only (HBM resident operands),
+ *   - launches on the hipStream_t passed as `stream` (a void*; NULL = the
+ *     default stream) and returns without synchronising,
+ *   - allocates nothing and keeps no state between calls (re-entrant across
+ *     streams),
+ *   - returns MI355_OK or a negative mi355_status; it never throws.
+ *
+ * Each function names the reference operator whose `ref` target arithmetic it
+ * reproduces (paths relative to the MIGraphX source tree).
+ */
+#ifndef MI355_QGEMM_H
+#define MI355_QGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mi355_status {
+    MI355_OK              = 0,
+    MI355_ERR_BAD_ARG     = -1, /* null pointer, negative size, bad enum */
+    MI355_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+    MI355_ERR_LAUNCH      = -3  /* HIP reported an error at launch */
+} mi355_status;
+
+/* Element types.  half / bf16 / fp8 are passed as their raw bits. */
+typedef enum mi355_dtype {
+    MI355_I8   = 0,
+    MI355_U8   = 1,
+    MI355_I32  = 2,
+    MI355_F32  = 3,
+    MI355_F16  = 4, /* IEEE binary16 */
+    MI355_BF16 = 5,
+    MI355_FP8  = 6  /* OCP e4m3fn */
+} mi355_dtype;
+
+/* How a quantization parameter is broadcast over an [M, N] result. */
+typedef enum mi355_qparam_mode {
+    MI355_QP_NONE       = 0, /* absent: scale 1, zero point 0 */
+    MI355_QP_PER_TENSOR = 1, /* one element */
+    MI355_QP_PER_ROW    = 2, /* [M] */
+    MI355_QP_PER_COL    = 3  /* [N] */
+} mi355_qparam_mode;
+
+/*
+ * Problem description of one (batched) quant_dot, optionally with the
+ * dequantizelinear epilogue that simplify_qdq puts behind it.
+ *
+ * A is [batch, M, K]; element (b, m, k) lives at  a + b*stride_a + m*lda + k
+ *   (trans_a = 0) or a + b*stride_a + k*lda + m (trans_a = 1, a transpose
+ *   view of [K, M] storage).
+ * B is [batch, K, N]; element (b, k, n) lives at  b + b*stride_b + k*ldb + n
+ *   (trans_b = 0) or b + b*stride_b + n*ldb + k (trans_b = 1, the transpose
+ *   view of [N, K] storage that simplify_qdq.cpp:49-82 produces when the
+ *   weight's transpose sat between dequantizelinear and dot).
+ * C is [batch, M, N] row-major with leading dimension ldc.
+ * All strides are in elements.
+ */
+typedef struct mi355_quant_dot_desc {
+    int64_t m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t batch;
+    int64_t stride_a, stride_b, stride_c;
+    int32_t trans_a, trans_b;
+    int32_t in_type;  /* MI355_I8 or MI355_FP8 */
+    int32_t out_type; /* MI355_I32 / MI355_F32: bare quant_dot result (int8 / fp8).
+                         With an epilogue: MI355_F32, MI355_F16 or MI355_BF16. */
+    /* ---- fused dequantizelinear epilogue (all zero = bare quant_dot) ---- */
+    int32_t dequant;      /* 0: store accumulators, 1: apply the epilogue     */
+    int32_t scale_a_mode; /* MI355_QP_NONE / PER_TENSOR / PER_ROW             */
+    int32_t scale_b_mode; /* MI355_QP_NONE / PER_TENSOR / PER_COL             */
+    int32_t zp_a, zp_b;   /* zero points of the quantized A and B (int8 only) */
+} mi355_quant_dot_desc;
+
+/*
+ * quant_dot (+ fused dequantizelinear).
+ *
+ * Replaces: ref_quant_gemm::compute (src/targets/ref/lowering.cpp:218-248) ->
+ * gemm_naive (src/gemm.cpp:42-63) with the shape rules of
+ * op::quant_dot::compute_shape (src/include/migraphx/op/quant_dot.hpp:51-121):
+ * int8 x int8 -> int32 (exact), fp8 e4m3fn x fp8 e4m3fn -> float.
+ *
+ * With desc->dequant it also replaces the instructions simplify_qdq.cpp:225-289
+ * emits behind the quant_dot and that the ref target evaluates one by one:
+ *   scale[m,n] = scale_a[m or 0] * scale_b[n or 0]            (fp32 `mul`)
+ *   zp[m,n]    = zp_a*colsum_b[n] + zp_b*rowsum_a[m] - K*zp_a*zp_b
+ *                (what the three extra quant_dots of :250-279 add up to)
+ *   out        = float((double(acc) - double(zp)) * double(scale))
+ *                (op/dequantizelinear.hpp:71-78)
+ *   then `convert` to half / bf16 (op/convert.hpp:64-87: round toward zero,
+ *   saturating, NaN kept) when out_type asks for it.
+ * colsum_b [batch? no: N] / rowsum_a [M] are int32 sums over K of B's columns /
+ * A's rows (see mi355_colsum_i8 / mi355_rowsum_i8); they are read only when
+ * the matching zero point is non-zero and may be NULL otherwise.
+ */
+int mi355_quant_dot(const mi355_quant_dot_desc* desc,
+                    const void* a,
+                    const void* b,
+                    void* c,
+                    const float* scale_a,
+                    const float* scale_b,
+                    const int32_t* colsum_b,
+                    const int32_t* rowsum_a,
+                    void* stream);
+
+/* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
+ * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the
+ * zero-point term of simplify_qdq.cpp:260-266 divided by the zero point. */
+int mi355_colsum_i8(const void* b, int64_t k, int64_t n, int64_t ldb, int32_t trans_b,
+                    int32_t* out, void* stream);
+
+/* int32 row sums of an int8 [M, K] matrix: out[m] = sum_k A[m, k]
+ * (simplify_qdq.cpp:267-273). */
+int mi355_rowsum_i8(const void* a, int64_t m, int64_t k, int64_t lda, int32_t trans_a,
+                    int32_t* out, void* stream);
+
+/*
+ * quantizelinear on a dense [rows, cols] tensor.
+ *
+ * Replaces: op::quantizelinear::compute
+ * (src/include/migraphx/op/quantizelinear.hpp:71-108).
+ *   integral out: clamp(double(nearbyint(x / s)) + double(zp)), x / s divided
+ *                 in x's own type, ties to even;
+ *   fp8 out:      clamp(double(x)/double(s) + double(zp), -448, 448) -> fp8.
+ * scale has x's element type, zp (may be NULL = 0) has the output's.  Both are
+ * addressed as p[r*stride_r + c*stride_c] so a per-tensor parameter uses
+ * strides (0,0), a per-column one (0,1), a per-row one (1,0), a full one
+ * (cols,1) -- the strides the broadcast views of the graph carry.
+ */
+int mi355_quantizelinear(const void* x, int32_t x_type,
+                         const void* scale, int64_t scale_stride_r, int64_t scale_stride_c,
+                         const void* zp, int64_t zp_stride_r, int64_t zp_stride_c,
+                         void* out, int32_t out_type,
+                         int64_t rows, int64_t cols, void* stream);
+
+/*
+ * dequantizelinear on a dense [rows, cols] tensor.
+ *
+ * Replaces: op::dequantizelinear::compute
+ * (src/include/migraphx/op/dequantizelinear.hpp:60-83):
+ * out = (double(x) - double(zp)) * scale, stored in the scale's type.
+ * x_type in {I8, U8, I32, F32, FP8}; scale_type in {F32, F16, BF16}.
+ */
+int mi355_dequantizelinear(const void* x, int32_t x_type,
+                           const void* scale, int32_t scale_type,
+                           int64_t scale_stride_r, int64_t scale_stride_c,
+                           const void* zp, int64_t zp_stride_r, int64_t zp_stride_c,
+                           void* out, int64_t rows, int64_t cols, void* stream);
+
+/*
+ * unpack_int4 / pack_int4 along the last axis of a dense [rows, cols] byte
+ * tensor (cols = packed length for unpack, unpacked length for pack).
+ *
+ * Replaces: op::unpack_int4::compute (src/include/migraphx/op/unpack_int4.hpp:75-121)
+ * and op::pack_int4::compute (src/include/migraphx/op/pack_int4.hpp:79-124).
+ * Low nibble = even element; is_signed selects sign extension / [-8,7] clip.
+ */
+int mi355_unpack_int4(const void* in, void* out, int32_t is_signed,
+                      int64_t rows, int64_t cols, void* stream);
+int mi355_pack_int4(const void* in, void* out, int32_t is_signed,
+                    int64_t rows, int64_t cols, void* stream);
+
+/*
+ * convert float -> half / bf16 / fp8 and back on n dense elements.
+ *
+ * Replaces: op::convert::compute (src/include/migraphx/op/convert.hpp:64-87)
+ * with the software-float conversions of generic_float.hpp:172-222 (half and
+ * bf16: round toward zero) and float8_impl.hpp:38-247 (fp8: nearest even).
+ */
+int mi355_convert(const void* in, int32_t in_type, void* out, int32_t out_type,
+                  int64_t n, void* stream);
+
+/* Zero-point forms of the int4 weight-only GEMM. */
+typedef enum mi355_w4_zp_mode {
+    MI355_W4_ZP_SCALAR = 0, /* one value for the whole tensor (MatMulNBits default 8) */
+    MI355_W4_ZP_GROUP  = 1, /* uint8 [N, K/group], already unpacked */
+    MI355_W4_ZP_PACKED = 2  /* 4-bit pairs, uint8 [N, ceil(K/group/2)], low nibble first */
+} mi355_w4_zp_mode;
+
+/*
+ * int4 weight-only GEMM / GEMV with group-wise scales:
+ *   out[m, n] = half( sum_k a[m,k] * w[n,k] ),  w[n,k] = half((q[n,k] - zp) * scale[n, k/group])
+ *
+ * Replaces the chain the ref target runs op by op for the graph of
+ * src/onnx/parse_matmulnbits.cpp:85-159:
+ *   unpack_int4 (op/unpack_int4.hpp:75-121) ->
+ *   dequantizelinear with block-broadcast scales / zero points
+ *     (op/dequantizelinear.hpp:60-83, op/builder/.../quantize_dequantize_linear.hpp:84-152) ->
+ *   transpose -> dot (op/dot.hpp:102-107, gemm_naive src/gemm.cpp:42-63).
+ * a      fp16 [M, K] (lda), w_packed uint8 [N, K/2] (two nibbles per byte along K,
+ * low nibble = even k), scales fp16 [N, K/group], out fp16 [M, N] (ldc).
+ * K must be a multiple of `group`, group a multiple of 32.
+ */
+int mi355_w4a16_gemm(const void* a, int64_t lda,
+                     const void* w_packed,
+                     const void* scales,
+                     const void* zp, int32_t zp_mode, int32_t zp_scalar,
+                     void* out, int64_t ldc,
+                     int64_t m, int64_t n, int64_t k, int64_t group,
+                     void* stream);
+
+/* Human-readable text for a status code (static storage). */
+const char* mi355_status_string(int status);
+
+/* Library version, major*10000 + minor*100 + patch. */
+int mi355_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_QGEMM_H */

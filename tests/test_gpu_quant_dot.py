@@ -1,0 +1,249 @@
+"""GPU parity of quant_dot (+ fused dequantizelinear) against the CPU oracle,
+through the C ABI.  int32 accumulators and every int8-path output are required
+bit-exact; fp8 outputs within the stated floating-point tolerance."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.gpu_util import dev, bf16_bits, half_bits, ulp_distance_16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from amdmigraphx_amd import ops
+    return ops
+
+
+def _iota(lens, dtype, start=0):
+    n = int(np.prod(lens))
+    return (np.arange(n, dtype=np.int64) + start).astype(dtype).reshape(lens)
+
+
+def test_reference_known_answers_on_gpu(ops, golden):
+    """The 15 quant_dot cases of test/ref/dot_op.cpp run through the library
+    (transposed views and batches exercise the any-stride kernel)."""
+    for c in golden["quant_dot"]:
+        a = _iota(c["a"]["lens"], np.int8)
+        b = _iota(c["b"]["lens"], np.int8)
+        ta, tb = dev(a), dev(b)
+        if c["alpha"] != 1:
+            af = (np.float32(c["alpha"]) * a.astype(np.float32))
+            ta = dev(orc.convert(af, orc.F32, orc.I8).reshape(a.shape))
+        if c["a_perm"]:
+            ta = ta.permute(c["a_perm"])
+        if c["b_perm"]:
+            tb = tb.permute(c["b_perm"])
+        out = ops.quant_dot(ta, tb).cpu().numpy().astype(np.int64)
+        if c["uses_c"] and c["beta"] != 0:
+            cm = _iota(c["c"]["lens"], np.int32, c["iota_start"]["c"])
+            out = out + orc.convert(cm.astype(np.float32) * np.float32(c["beta"]),
+                                    orc.F32, orc.I32).reshape(out.shape)
+        assert out.flatten().tolist() == c["gold"], c["name"]
+
+
+SHAPES = [(256, 256, 128), (256, 1024, 1024), (512, 768, 384), (300, 260, 144),
+          (1, 4, 16), (16, 512, 2048), (128, 256, 4096), (257, 516, 272), (64, 100, 80),
+          (33, 7, 50)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_int8_accumulators_bit_exact(ops, m, n, k, trans_b):
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    want = orc.quant_dot(a, b, orc.I8)
+    tb = dev(np.ascontiguousarray(b.T)).t() if trans_b else dev(b)
+    got = ops.quant_dot(dev(a), tb).cpu().numpy()
+    assert got.dtype == np.int32
+    assert np.array_equal(got, want)
+
+
+def test_int8_extremes_and_batch(ops):
+    a = np.full((2, 256, 512), -128, np.int8)
+    b = np.full((2, 512, 256), -128, np.int8)
+    a[1] = 127
+    got = ops.quant_dot(dev(a), dev(b)).cpu().numpy()
+    assert np.all(got[0] == 128 * 128 * 512) and np.all(got[1] == -127 * 128 * 512)
+    rng = np.random.default_rng(1)
+    a = rng.integers(-128, 128, (3, 70, 96), dtype=np.int8)
+    b = rng.integers(-128, 128, (3, 96, 52), dtype=np.int8)
+    assert np.array_equal(ops.quant_dot(dev(a), dev(b)).cpu().numpy(), orc.quant_dot(a, b, orc.I8))
+
+
+def test_config1_qdq_matmul_bit_exact(ops):
+    """BASELINE config 1: X fp32 [256,1024] ~N(0,1) -> quantizelinear(1/32, 0) ->
+    quant_dot with W int8 U[-127,127] -> per-channel dequantizelinear, seed 0."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((256, 1024)).astype(np.float32)
+    w = rng.integers(-127, 128, (1024, 1024), dtype=np.int8)
+    sw = rng.uniform(0.001, 0.01, 1024).astype(np.float32)
+    sx = np.float32(1.0 / 32)
+    xq_ref = orc.quantizelinear(x, sx, np.int8(0), orc.F32, orc.I8)
+    want = orc.qdq_matmul_int8(xq_ref, w, sx, sw)
+    xq = ops.quantizelinear(dev(x), dev(np.float32([sx])), dev(np.int8([0])))
+    assert np.array_equal(xq.cpu().numpy(), xq_ref)
+    got = ops.quant_dot(xq, dev(w), scale_a=dev(np.float32([sx])), scale_b=dev(sw))
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("zp_a,zp_b", [(5, 0), (0, -3), (7, -9)])
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_int8_dequant_epilogue_bit_exact(ops, zp_a, zp_b, out):
+    """Asymmetric zero points (simplify_qdq.cpp:250-279), large accumulators
+    (|acc| > 2^24 so a float product would differ) and the truncating converts."""
+    rng = np.random.default_rng(11 + zp_a * 3 + zp_b)
+    m, n, k = 192, 320, 2048
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    a[:8] = 127
+    b[:, :8] = 127
+    sa = np.float32(0.0371)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    ot = {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[out]
+    want = orc.qdq_matmul_int8(a, b, sa, sb, zp_a, zp_b, ot)
+    ta, tb = dev(a), dev(b)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_dot(ta, tb, scale_a=dev(np.float32([sa])), scale_b=dev(sb), zp_a=zp_a, zp_b=zp_b,
+                        colsum_b=ops.colsum_i8(tb) if zp_a else None,
+                        rowsum_a=ops.rowsum_i8(ta) if zp_b else None, out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), want)
+
+
+def test_rowsum_colsum(ops):
+    rng = np.random.default_rng(5)
+    a = rng.integers(-128, 128, (130, 1000), dtype=np.int8)
+    ta = dev(a)
+    assert np.array_equal(ops.rowsum_i8(ta).cpu().numpy(), a.astype(np.int32).sum(1))
+    assert np.array_equal(ops.colsum_i8(ta).cpu().numpy(), a.astype(np.int32).sum(0))
+    assert np.array_equal(ops.colsum_i8(ta.t()).cpu().numpy(), a.astype(np.int32).sum(1))
+    assert np.array_equal(ops.rowsum_i8(ta.t()).cpu().numpy(), a.astype(np.int32).sum(0))
+
+
+def _fp8_codes(rng, shape, sigma):
+    x = rng.normal(0, sigma, shape).astype(np.float32)
+    return orc.fp8_from_f32(np.clip(x, -448, 448))
+
+
+def _fp8_bound(a, b):
+    """sum_k |a||b| per output: the scale of the fp32 accumulation error."""
+    fa = np.abs(orc.fp8_to_f32(a)).astype(np.float64)
+    fb = np.abs(orc.fp8_to_f32(b)).astype(np.float64)
+    return fa @ fb
+
+
+# Tolerance of the fp8 path.  The reference's double accumulator holds the
+# exact dot product and rounds once.  v_mfma_f32_16x16x128_f8f6f4 adds each
+# group of 128 exact products with a fixed-point window of about 20 bits below
+# the largest product of the group (measured: errors up to 2^-16 of sum|a||b|
+# for K = 128, truncating), then accumulates groups in fp32.  An output passes
+# when it is within 1e-3 relative of the reference, or (bf16/half outputs)
+# within 1 ulp of the output type, or -- where the exact sum cancels far below
+# its terms -- within 2^-14 of sum|a||b| (times the scale).
+FP8_ABS_FLOOR = 2.0**-14
+
+
+def _fp8_close(got, want, bound):
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    return (diff <= 1e-3 * np.abs(want)) | (diff <= bound * FP8_ABS_FLOOR)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (256, 512, 1024), (512, 384, 4096), (96, 132, 272)])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_fp8_accumulators(ops, m, n, k, trans_b):
+    rng = np.random.default_rng(m + n + k)
+    a = _fp8_codes(rng, (m, k), 1.0 * 100)
+    b = _fp8_codes(rng, (k, n), 0.02 * 5000)
+    want = orc.quant_dot(a, b, orc.FP8)
+    tb = dev(np.ascontiguousarray(b.T)).t() if trans_b else dev(b)
+    got = ops.quant_dot(dev(a), tb, fp8=True).cpu().numpy()
+    assert got.dtype == np.float32
+    ok = _fp8_close(got, want, _fp8_bound(a, b))
+    assert ok.all(), (np.abs(got - want).max(), (~ok).sum())
+    # the bulk is far tighter than the tolerance
+    rel = np.abs(got - want) / np.maximum(np.abs(want), 1e-30)
+    print("fp8 rel err median %.2e max %.2e; max |diff|/sum|a||b| %.2e" %
+          (np.median(rel), rel.max(), (np.abs(got - want) / _fp8_bound(a, b)).max()))
+    assert np.median(rel) < 1e-4
+
+
+def test_fp8_small_integers_are_exact(ops):
+    """Operands that are small integers give sums the fp32 accumulator holds
+    exactly, so the result must equal the reference bit for bit."""
+    rng = np.random.default_rng(2)
+    m, n, k = 256, 256, 512
+    a = orc.fp8_from_f32(rng.integers(-8, 9, (m, k)).astype(np.float32))
+    b = orc.fp8_from_f32(rng.integers(-8, 9, (k, n)).astype(np.float32))
+    want = orc.quant_dot(a, b, orc.FP8)
+    got = ops.quant_dot(dev(a), dev(b), fp8=True).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_fp8_dequant_epilogue(ops, out):
+    """BASELINE config 3 at reduced size: amax-scaled fp8 operands, per-tensor
+    scales, fp32 accumulate, truncating bf16 output."""
+    rng = np.random.default_rng(3)
+    m, n, k = 256, 384, 2048
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    sx = np.float32(np.abs(x).max() / 448)
+    sw = np.float32(np.abs(w).max() / 448)
+    xq = orc.quantizelinear(x, sx, None, orc.F32, orc.FP8)
+    wq = orc.quantizelinear(w, sw, None, orc.F32, orc.FP8)
+    ot = orc.F32 if out == "f32" else orc.BF16
+    want = orc.qdq_matmul_fp8(xq, wq, sx, sw, ot)
+    td = torch.float32 if out == "f32" else torch.bfloat16
+    got = ops.quant_dot(dev(xq), dev(wq), fp8=True, scale_a=dev(np.float32([sx])),
+                        scale_b=dev(np.float32([sw])), out_dtype=td)
+    bound = _fp8_bound(xq, wq) * float(sx) * float(sw)
+    if out == "f32":
+        ok = _fp8_close(got.cpu().numpy(), want, bound)
+    else:
+        gb = bf16_bits(got)
+        gf = orc.bf16_to_f32(gb)
+        wf = orc.bf16_to_f32(want)
+        ok = (ulp_distance_16(gb, want) <= 1) | _fp8_close(gf, wf, bound)
+        # most outputs are identical to the reference's bits
+        assert (gb == want).mean() > 0.98
+    assert ok.all(), (~ok).sum()
+
+
+def test_argument_errors(ops):
+    from amdmigraphx_amd import Mi355Error
+    a = torch.zeros((4, 8), dtype=torch.int8, device="cuda")
+    b = torch.zeros((9, 4), dtype=torch.int8, device="cuda")
+    with pytest.raises(Mi355Error):
+        ops.quant_dot(a, b)                       # inner dimensions differ
+    with pytest.raises(Mi355Error):
+        ops.quant_dot(a, torch.zeros((8, 4), dtype=torch.uint8, device="cuda"))
+    out = ops.quant_dot(torch.zeros((0, 8), dtype=torch.int8, device="cuda"),
+                        torch.zeros((8, 4), dtype=torch.int8, device="cuda"))
+    assert out.shape == (0, 4)
+
+
+def test_full_size_int8_properties(ops):
+    """BASELINE config 2 at 8192^3: sampled rows against the oracle and a
+    row-checksum identity over the whole result."""
+    torch.manual_seed(0)
+    n = 8192
+    a = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda")
+    b = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda")
+    c = ops.quant_dot(a, b)
+    rows = [0, 1, 255, 256, 4095, 4096, 8190, 8191]
+    want = orc.quant_dot(a[rows].cpu().numpy(), b.cpu().numpy(), orc.I8)
+    assert np.array_equal(c[rows].cpu().numpy(), want)
+    # sum_n C[m, n] == sum_k A[m, k] * (sum_n B[k, n]); all values < 2^53
+    lhs = c.double().sum(1)
+    rhs = a.double() @ b.double().sum(1)
+    assert torch.equal(lhs, rhs)
+    # column checksum as well
+    lhs = c.double().sum(0)
+    rhs = a.double().sum(0) @ b.double()
+    assert torch.equal(lhs, rhs)
