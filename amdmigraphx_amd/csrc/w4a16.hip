@@ -119,6 +119,276 @@ __global__ __launch_bounds__(W4_THREADS) void w4a16_gemv_kernel(w4_params p)
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// M = 1 streaming GEMV.
+//
+// A workgroup of 8 waves keeps the activation vector in LDS; each wave owns
+// one weight row at a time.  Lane l reads the 16-byte runs (c*64 + l) of the
+// packed row, c = 0..NCH-1, so one load instruction covers 1 KiB of contiguous
+// weights and the whole row (NCH KiB) is in flight at once; the loads of the
+// wave's next row are issued before the current row is consumed.
+//
+// Dequantization runs on packed halves, one fused multiply-add per pair of
+// weights.  The nibbles k and k+4 of a dword are masked in place at bits 4..7
+// of the two halves of a register: read as half-precision subnormals they are
+// q * 2^-20 exactly.  fma(q * 2^-20, scale * 2^20, -zp * scale) then forms
+// (q - zp) * scale exactly inside the FMA and rounds it once -- the one rounding
+// of the reference's float -> half store -- with the half-precision rounding
+// mode of the wave set to round-toward-zero so that it matches that truncation
+// bit for bit.  This needs scale * 2^20 and zp * scale to be exact halves: zp
+// in {0, 1, 2, 4, 8} and |scale| below 2^-5; a lane whose scale is outside
+// that range (or is not finite) takes the three-instruction form instead
+// (1024 + q built in the mantissa, minus 1024 + zp, times scale).
+// v_dot2_f32_f16 then multiplies by the matching activation pair and
+// accumulates in fp32.
+// The activations sit in LDS already paired (k, k+4) and laid out
+// [chunk][dword][lane] so a wave's 16-byte reads are conflict free.
+// Each row's 64 partial sums are reduced with DPP row operations.
+// ---------------------------------------------------------------------------
+constexpr int GV_THREADS = 512;
+constexpr int GV_WAVES   = GV_THREADS / 64;
+
+MI355_DEVINL float dpp_row_sum(float v)
+{
+    // 16-lane sums in every lane of each DPP row
+    int x = __builtin_bit_cast(int, v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, false));
+    x = __builtin_bit_cast(int, v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, false));
+    x = __builtin_bit_cast(int, v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, false));
+    x = __builtin_bit_cast(int, v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, false));
+    return v;
+}
+
+MI355_DEVINL float wave_sum_dpp(float v)
+{
+    v        = dpp_row_sum(v);
+    int x    = __builtin_bit_cast(int, v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+MI355_DEVINL uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits)
+{
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask), "v"(bits));
+    return r;
+}
+
+constexpr int GV_DEPTH = 4; // 16-byte runs per lane kept in flight
+
+__global__ __launch_bounds__(GV_THREADS) void w4a16_gemv_m1_kernel(w4_params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t gv_lds[];
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    // wave-uniform values are pinned to scalar registers so that the loop
+    // control around the pipeline below is scalar branches, not exec masking
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kbytes = p.k >> 1;
+    const int groups = p.k / p.group;
+    const int nch    = p.k >> 11; // 1 KiB runs per packed row
+    // scale index of this lane inside a run: the group size divides 2048
+    const int gshift = __builtin_ctz(p.group);
+    const int lane_g = (lane * 32) >> gshift;
+    const int run_g  = 2048 >> gshift;
+
+    // Half-precision arithmetic of this wave rounds toward zero from here on
+    // (MODE.fp_round bits 3:2); fp32 rounding is untouched.  Written as inline
+    // assembly: the compiler tracks s_setreg it emits itself and would put the
+    // default mode back in front of the first packed-half instruction.  All
+    // half arithmetic below sits behind the workgroup barrier, which this
+    // statement cannot move across.
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 2, 2), 3" ::: "memory");
+
+    // The activation loads go out first so that they are not queued behind the
+    // weight stream.  Slot s = (c*4 + d)*64 + l of the LDS copy holds the 8
+    // halves a[k0 .. k0+7], k0 = (c*64 + l)*32 + 8*d, reordered to
+    // (0,4,1,5,2,6,3,7).
+    const int a_slots = p.k >> 3;
+    uint4 areg[4];
+#pragma unroll
+    for(int it = 0; it < 4; it++)
+    {
+        const int s  = tid + it * GV_THREADS;
+        const int l  = s & 63;
+        const int cd = s >> 6;
+        const int k0 = ((cd >> 2) * 64 + l) * 32 + 8 * (cd & 3);
+        if(s < a_slots)
+            areg[it] = *reinterpret_cast<const uint4*>(p.a + k0);
+    }
+
+    // this wave's rows: row0, row0 + stride, ...; its work items are the 1 KiB
+    // runs of those rows in order
+    const int stride = gridDim.x * GV_WAVES;
+    const int row0   = blockIdx.x * GV_WAVES + wave;
+    const int nrows  = row0 < p.n ? (p.n - 1 - row0) / stride + 1 : 0;
+    const int total  = __builtin_amdgcn_readfirstlane(nrows * nch);
+
+    v4u wbuf[GV_DEPTH];
+    uint16_t sbuf[GV_DEPTH];
+    int ld_row = row0, ld_c = 0; // item the next issue() fetches
+    auto issue = [&](int slot) {
+        const uint8_t* q = p.w + (int64_t)ld_row * kbytes + ld_c * 1024 + lane * 16;
+        wbuf[slot]       = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(q));
+        sbuf[slot]       = p.scales[(int64_t)ld_row * groups + ld_c * run_g + lane_g];
+        if(++ld_c == nch)
+        {
+            ld_c = 0;
+            ld_row += stride;
+        }
+    };
+#pragma unroll
+    for(int u = 0; u < GV_DEPTH; u++)
+        if(u < total)
+            issue(u);
+
+#pragma unroll
+    for(int it = 0; it < 4; it++)
+    {
+        const int s = tid + it * GV_THREADS;
+        if(s < a_slots)
+        {
+            const uint4 v = areg[it];
+            uint4 o;
+            o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+            o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+            o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+            o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+            *reinterpret_cast<uint4*>(gv_lds + s * 16) = o;
+        }
+    }
+    __syncthreads();
+
+    // 1024 + zp as half bits (zp in 0..15 sits in the low mantissa bits); built
+    // from integers so that no float -> half conversion instruction appears in
+    // this kernel: the compiler resets the rounding mode in front of those.
+    const uint32_t zbits = 0x6400u | (uint32_t)p.zp_scalar;
+    const h2 zoff2       = __builtin_bit_cast(h2, zbits | (zbits << 16));
+    // mask and magic live in registers so that (w & mask) | magic is one
+    // v_and_or_b32 (the three-operand form takes no literal constants here)
+    uint32_t nib_mask = 0x000F000Fu, magic = 0x64006400u;
+    asm volatile("" : "+v"(nib_mask), "+v"(magic));
+    const int zpv      = p.zp_scalar;
+    const bool zp_pow2 = (zpv & (zpv - 1)) == 0; // 0, 1, 2, 4, 8
+    const int zp_log2  = zpv <= 1 ? 0 : (zpv == 2 ? 1 : (zpv == 4 ? 2 : 3));
+
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}; // independent chains for the dot units
+    int cs_row = row0, cs_c = 0;         // item being consumed
+
+    auto consume = [&](int slot) {
+        const uint16_t sb    = sbuf[slot];
+        const _Float16 sc    = __builtin_bit_cast(_Float16, sb);
+        const h2 scv         = {sc, sc};
+        const uint32_t wa[4] = {wbuf[slot].x, wbuf[slot].y, wbuf[slot].z, wbuf[slot].w};
+        // scale * 2^20 by adding 20 to the exponent field; exact for normal
+        // scales below 2^-5 (exponent field 1..10)
+        const uint32_t sexp = (sb >> 10) & 0x1fu;
+        // taken by the whole wave or not at all: the general form is right for
+        // every lane, so one out-of-range scale just costs the wave speed
+        const bool fast =
+            __builtin_amdgcn_ballot_w64(zp_pow2 && sexp >= 1 && sexp <= 10) == ~0ull;
+        const uint8_t* abase = gv_lds + (cs_c * 256 + lane) * 16;
+        if(fast)
+        {
+            const uint32_t sup = (uint32_t)sb + (20u << 10);
+            const h2 scv_up    = __builtin_bit_cast(h2, sup | (sup << 16));
+            // -zp * scale: exponent raised by log2(zp), sign flipped (zp == 0: +0)
+            const uint32_t zsb =
+                zpv == 0 ? 0u : (((uint32_t)sb + ((uint32_t)zp_log2 << 10)) ^ 0x8000u);
+            const h2 zs = __builtin_bit_cast(h2, zsb | (zsb << 16));
+#pragma unroll
+            for(int d = 0; d < 4; d++)
+            {
+                const uint4 av       = *reinterpret_cast<const uint4*>(abase + d * 1024);
+                const uint32_t ap[4] = {av.x, av.y, av.z, av.w};
+                // the four nibble pairs of the dword advance in lock step so that
+                // dependent packed-half instructions are never back to back
+                h2 x[4];
+                x[0] = __builtin_bit_cast(h2, (wa[d] << 4) & 0x00F000F0u);
+                x[1] = __builtin_bit_cast(h2, wa[d] & 0x00F000F0u);
+                x[2] = __builtin_bit_cast(h2, (wa[d] >> 4) & 0x00F000F0u);
+                x[3] = __builtin_bit_cast(h2, (wa[d] >> 8) & 0x00F000F0u);
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    x[j] = __builtin_elementwise_fma(x[j], scv_up, zs);
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    acc[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, ap[j]), x[j], acc[j],
+                                                    false);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for(int d = 0; d < 4; d++)
+            {
+                const uint4 av       = *reinterpret_cast<const uint4*>(abase + d * 1024);
+                const uint32_t ap[4] = {av.x, av.y, av.z, av.w};
+                h2 x[4];
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    x[j] = __builtin_bit_cast(h2, and_or(wa[d] >> (4 * j), nib_mask, magic));
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    x[j] = x[j] - zoff2;
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    x[j] = x[j] * scv;
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                    acc[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, ap[j]), x[j], acc[j],
+                                                    false);
+            }
+        }
+        if(++cs_c == nch)
+        {
+            const float t = wave_sum_dpp((acc[0] + acc[1]) + (acc[2] + acc[3]));
+            if(lane == 0)
+                p.out[cs_row] = f32_to_half_rtz(t);
+            acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
+            cs_c                              = 0;
+            cs_row += stride;
+        }
+    };
+
+    // GV_DEPTH register slots rotate: a slot is refilled with the item
+    // GV_DEPTH ahead as soon as it has been consumed
+    for(int base = 0; base < total; base += GV_DEPTH)
+    {
+#pragma unroll
+        for(int u = 0; u < GV_DEPTH; u++)
+        {
+            if(base + u < total)
+            {
+                consume(u);
+                if(base + u + GV_DEPTH < total)
+                    issue(u);
+            }
+        }
+    }
+}
+
+constexpr int GV_MAX_K = 32768; // activations staged in LDS: 64 KiB; 4 slots per thread
+
+int launch_gemv_m1(const w4_params& p, hipStream_t s)
+{
+    const int lds    = p.k * 2;
+    const int blocks = (p.n + GV_WAVES - 1) / GV_WAVES;
+    // one resident set of workgroups: every wave walks several rows with its
+    // next runs in flight, instead of a second round of workgroups starting cold
+    const int per_cu = lds <= 16384 ? 4 : 2;
+    const int grid   = min(blocks, 256 * per_cu);
+    hipLaunchKernelGGL(w4a16_gemv_m1_kernel, dim3(grid), dim3(GV_THREADS), lds, s, p);
+    return mi355_launch_status();
+}
+
 } // namespace
 
 extern "C" int mi355_w4a16_gemm(const void* a,
@@ -173,6 +443,9 @@ extern "C" int mi355_w4a16_gemm(const void* a,
     p.k         = (int)k;
     p.group     = (int)group;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if(m == 1 && zp_mode == MI355_W4_ZP_SCALAR && k % 2048 == 0 && k <= GV_MAX_K &&
+       (group & (group - 1)) == 0 && group <= 2048)
+        return launch_gemv_m1(p, s);
     dim3 grid((unsigned)((n + 3) / 4));
     if(m == 1)
         hipLaunchKernelGGL(w4a16_gemv_kernel<1>, grid, dim3(W4_THREADS), 0, s, p);
