@@ -1,0 +1,601 @@
+// quant_dot on the gfx950 matrix cores, main kernel: int8 x int8 -> int32
+// with v_mfma_i32_32x32x32_i8 and e4m3fn x e4m3fn -> fp32 with
+// v_mfma_f32_32x32x64_f8f6f4, dequantizelinear / convert epilogue in registers.
+//
+// Data path: global memory -> LDS directly (global_load_lds_dwordx4, no
+// register staging, no LDS store instructions), LDS -> MFMA operands.
+//
+// Tiling: a workgroup of 8 waves computes a 256 x 256 tile of C and walks K in
+// slabs of 64 bytes.  Waves are arranged 2 (M) x 4 (N), each owning 128 x 64
+// of the tile as 4 x 2 MFMA tiles of 32 x 32 (128 accumulator registers).
+// LDS holds a ring of 4 slab stages (32 KiB each): the loads of slab kt+3 are
+// issued while slab kt is multiplied, so a global load has about three slab
+// times to land.  One barrier per slab, placed between the two halves of the
+// slab's MFMAs so that the first operand reads of the next slab overlap the
+// second half.
+//
+// LDS layouts (16-byte chunks, XOR swizzled so that operand reads are bank
+// conflict free; a direct-to-LDS load writes lane l at base + 16*l, so the
+// swizzle is applied to the global address each lane fetches):
+//   K-contiguous operand (A, or B given as [N, K]): row r holds its 64 K bytes
+//     as 4 chunks; logical chunk c sits at position c ^ ((r >> 2) & 3).
+//   row-major B ([K, N]): row k holds 256 N bytes as 16 chunks; logical chunk c
+//     sits at position c ^ (k & 7).  MFMA wants K-contiguous bytes per column:
+//     ds_read_b64_tr_b8 does that transposition on the way out of LDS (a group
+//     of 16 lanes reads an 8 (k) x 16 (n) byte block and each lane receives one
+//     column).
+#include "common.h"
+#include <type_traits>
+
+namespace {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int BM          = 256;
+constexpr int BN          = 256;
+constexpr int BK          = 64;
+constexpr int STAGES      = 4;
+constexpr int NTHREADS    = 512;
+constexpr int A_BYTES     = BM * BK;
+constexpr int STAGE_BYTES = (BM + BN) * BK;
+constexpr int LDS_BYTES   = STAGES * STAGE_BYTES;
+
+struct dma_params
+{
+    const uint8_t* a;
+    const uint8_t* b;
+    void* c;
+    int m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;
+    int tiles_m, tiles_n;
+    const float* scale_a;
+    const float* scale_b;
+    const int32_t* colsum_b;
+    const int32_t* rowsum_a;
+    int scale_a_mode, scale_b_mode;
+    int zp_a, zp_b;
+};
+
+// s_waitcnt with only the vector-memory counter constrained
+template <int N>
+MI355_DEVINL void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64);
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// s_barrier alone: __syncthreads() would also drain the vector-memory counter
+// and with it the slabs that are meant to stay in flight.  The empty asm
+// statements keep the compiler from moving LDS accesses across it.
+MI355_DEVINL void block_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+MI355_DEVINL void load_to_lds(const uint8_t* g, uint8_t* l)
+{
+    // generic -> global / LDS address-space pointers need C-style casts
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g),
+                                     (__attribute__((address_space(3))) void*)(l),
+                                     16,
+                                     0,
+                                     0);
+}
+
+MI355_DEVINL v2i read_tr8(const uint8_t* l)
+{
+    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i __attribute__((address_space(3)))*)(l));
+}
+
+// XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs,
+// each with its own L2.  Give every XCD a contiguous run of the tile order, and
+// walk that order in column-major bands of 8 tile rows, so the ~32 tiles an
+// XCD works on at one time share A row panels and B column panels in its L2.
+MI355_DEVINL void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+    const int total = tiles_m * tiles_n;
+    int v           = wg;
+    if(total % 8 == 0)
+        v = (wg % 8) * (total / 8) + wg / 8;
+    constexpr int band = 8;
+    int per_band       = band * tiles_n;
+    int b              = v / per_band;
+    int first_m        = b * band;
+    int rows           = min(band, tiles_m - first_m);
+    int r              = v - b * per_band;
+    tm                 = first_m + r % rows;
+    tn                 = r / rows;
+}
+
+template <bool FP8>
+struct types
+{
+    using acc  = v16i;
+    using frag = v4i;
+};
+template <>
+struct types<true>
+{
+    using acc  = v16f;
+    using frag = v8i;
+};
+
+template <int OUT>
+MI355_DEVINL void store1(void* c, int64_t idx, float v)
+{
+    if constexpr(OUT == MI355_F32)
+        static_cast<float*>(c)[idx] = v;
+    else if constexpr(OUT == MI355_F16)
+        static_cast<uint16_t*>(c)[idx] = convert_f32_to_half(v);
+    else
+        static_cast<uint16_t*>(c)[idx] = convert_f32_to_bf16(v);
+}
+
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+__global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    using acc_t  = typename types<FP8>::acc;
+    using frag_t = typename types<FP8>::frag;
+
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 2; // 0..1
+    const int wave_n = wave & 3;  // 0..3
+
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
+    const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+
+    // ---- global -> LDS ----------------------------------------------------------
+    // Each wave issues 4 loads of 1 KiB per slab: A row blocks {wave, wave+8}
+    // (16 rows x 64 bytes each) and B blocks {wave, wave+8} (16 rows x 64 bytes
+    // of [N, K] storage, or 4 rows x 256 bytes of [K, N] storage).
+    uint32_t a_off[2], b_off[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+    {
+        const int blk = wave + 8 * h;
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int row   = min(m0 + r, p.m - 1);
+            a_off[h]        = (uint32_t)row * (uint32_t)p.lda + chunk * 16;
+        }
+        if constexpr(TRANS_B)
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int col   = min(n0 + r, p.n - 1);
+            b_off[h]        = (uint32_t)col * (uint32_t)p.ldb + chunk * 16;
+        }
+        else
+        {
+            const int k     = 4 * blk + (lane >> 4);
+            const int chunk = (lane & 15) ^ (k & 7);
+            const int col   = min(n0 + chunk * 16, p.n - 16);
+            b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
+        }
+    }
+    auto issue_slab = [&](int kt) {
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
+        const uint8_t* a_base = ga + (int64_t)kt * BK;
+        const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+            load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+            load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+    };
+
+    // ---- LDS -> operand fragments --------------------------------------------
+    // A 32-row operand tile: lane l supplies row l % 32 and the K bytes of lane
+    // group l / 32 (16 bytes per group for the K = 32 int8 instruction, 32 for
+    // the K = 64 fp8 one).  A and B use the same K assignment.
+    //
+    // A slab is multiplied in two steps.  int8: step s is K bytes 32s..32s+31
+    // against all 4 A tiles.  fp8: step s is all 64 K bytes against A tiles
+    // 2s, 2s+1.
+    //
+    // The reads are inline assembly on purpose.  The compiler keeps no alias
+    // information for direct-to-LDS loads, so in front of every LDS read it can
+    // see it waits for ALL outstanding ones (vmcnt(0)), which would serialise
+    // the slab pipeline; reads it cannot see leave the counters to the explicit
+    // waits below.  Each fragment is tied ("+v") into the s_waitcnt statement
+    // that must precede its first use, which is what orders the MFMAs.
+    constexpr int A_TILES = FP8 ? 2 : 4;
+    constexpr int A_PARTS = FP8 ? 2 : 1; // 16-byte reads per K-contiguous fragment
+    const int lrow        = lane & 31;
+    const int lgrp        = lane >> 5;
+    const int tr_i        = lane & 15;
+    const int tr_g        = lane >> 4;
+    const uint32_t lds0   = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+
+    // per-lane byte offsets inside a stage, [step or part]
+    uint32_t a_lane[2], b_lane[2];
+    {
+        const int sw = (lrow >> 2) & 3;
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+        {
+            // int8: x = step (chunk 2x + lgrp); fp8: x = part (chunk 2*lgrp + x)
+            const int chunk = FP8 ? 2 * lgrp + x : 2 * x + lgrp;
+            a_lane[x]       = (wave_m * 128 + lrow) * BK + ((chunk ^ sw) << 4);
+            if constexpr(TRANS_B)
+                b_lane[x] = A_BYTES + (wave_n * 64 + lrow) * BK + ((chunk ^ sw) << 4);
+        }
+        if constexpr(!TRANS_B)
+        {
+            // lane 16g + i supplies the address of row k = kbase + (i >> 1), byte
+            // half (i & 1) of the 16-byte chunk holding columns 16*(g & 1).. of
+            // the tile, and receives column 16*(g & 1) + i with 8 consecutive k
+            const int krow = (tr_g >> 1) * (FP8 ? 32 : 16) + (tr_i >> 1);
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+            {
+                const int chunk = wave_n * 4 + j * 2 + (tr_g & 1);
+                b_lane[j] = A_BYTES + krow * BN + ((chunk ^ (krow & 7)) << 4) + 8 * (tr_i & 1);
+            }
+        }
+    }
+
+    frag_t fa[2][A_TILES];
+    frag_t fb[2][2];
+
+    auto rd128 = [](uint32_t addr, auto imm) -> v4i {
+        v4i r;
+        asm volatile("ds_read_b128 %0, %1 offset:%2"
+                     : "=v"(r)
+                     : "v"(addr), "n"(decltype(imm)::value)
+                     : "memory");
+        return r;
+    };
+    auto rdtr8 = [](uint32_t addr, auto imm) -> v2i {
+        v2i r;
+        asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2"
+                     : "=v"(r)
+                     : "v"(addr), "n"(decltype(imm)::value)
+                     : "memory");
+        return r;
+    };
+#define IMM(x) std::integral_constant<int, (x)>{}
+
+    // Issues the LDS reads of step S of the slab in `stage` into fa[S], fb[S].
+    auto read_step = [&](int stage, auto step) {
+        constexpr int S     = decltype(step)::value;
+        const uint32_t base = lds0 + stage * STAGE_BYTES;
+        if constexpr(FP8)
+        {
+            const uint32_t a0 = base + a_lane[0], a1 = base + a_lane[1];
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+            {
+                v4i lo, hi;
+                if(i == 0)
+                {
+                    lo = rd128(a0, IMM((2 * S) * 32 * BK));
+                    hi = rd128(a1, IMM((2 * S) * 32 * BK));
+                }
+                else
+                {
+                    lo = rd128(a0, IMM((2 * S + 1) * 32 * BK));
+                    hi = rd128(a1, IMM((2 * S + 1) * 32 * BK));
+                }
+                fa[S][i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+            if constexpr(TRANS_B)
+            {
+                const uint32_t b0 = base + b_lane[0], b1 = base + b_lane[1];
+                v4i lo0 = rd128(b0, IMM(0)), hi0 = rd128(b1, IMM(0));
+                v4i lo1 = rd128(b0, IMM(32 * BK)), hi1 = rd128(b1, IMM(32 * BK));
+                fb[S][0] = v8i{lo0.x, lo0.y, lo0.z, lo0.w, hi0.x, hi0.y, hi0.z, hi0.w};
+                fb[S][1] = v8i{lo1.x, lo1.y, lo1.z, lo1.w, hi1.x, hi1.y, hi1.z, hi1.w};
+            }
+            else
+            {
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                {
+                    const uint32_t bj = base + b_lane[j];
+                    v2i p0 = rdtr8(bj, IMM(0)), p1 = rdtr8(bj, IMM(8 * BN));
+                    v2i p2 = rdtr8(bj, IMM(16 * BN)), p3 = rdtr8(bj, IMM(24 * BN));
+                    fb[S][j] = v8i{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+                }
+            }
+        }
+        else
+        {
+            const uint32_t as = base + a_lane[S];
+            fa[S][0]          = rd128(as, IMM(0));
+            fa[S][1]          = rd128(as, IMM(32 * BK));
+            fa[S][2]          = rd128(as, IMM(64 * BK));
+            fa[S][3]          = rd128(as, IMM(96 * BK));
+            if constexpr(TRANS_B)
+            {
+                const uint32_t bs = base + b_lane[S];
+                fb[S][0]          = rd128(bs, IMM(0));
+                fb[S][1]          = rd128(bs, IMM(32 * BK));
+            }
+            else
+            {
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                {
+                    const uint32_t bj = base + b_lane[j];
+                    v2i p0 = rdtr8(bj, IMM(S * 32 * BN)), p1 = rdtr8(bj, IMM(S * 32 * BN + 8 * BN));
+                    fb[S][j] = v4i{p0.x, p0.y, p1.x, p1.y};
+                }
+            }
+        }
+    };
+    // s_waitcnt lgkmcnt(0) that "produces" the fragments of step S: everything
+    // that uses them is ordered behind it.  (A macro: asm operands that name
+    // captured arrays do not compile inside a generic lambda.)
+#define WAIT_STEP(S)                                                                            \
+    do                                                                                          \
+    {                                                                                           \
+        if constexpr(FP8)                                                                       \
+            asm volatile("s_waitcnt lgkmcnt(0)"                                                 \
+                         : "+v"(fa[S][0]), "+v"(fa[S][1]), "+v"(fb[S][0]), "+v"(fb[S][1])       \
+                         :                                                                      \
+                         : "memory");                                                           \
+        else                                                                                    \
+            asm volatile("s_waitcnt lgkmcnt(0)"                                                 \
+                         : "+v"(fa[S][0]), "+v"(fa[S][1]), "+v"(fa[S][A_TILES - 2]),            \
+                           "+v"(fa[S][A_TILES - 1]), "+v"(fb[S][0]), "+v"(fb[S][1])             \
+                         :                                                                      \
+                         : "memory");                                                           \
+    } while(0)
+    auto mfma = [&](const frag_t& a, const frag_t& b, acc_t c) -> acc_t {
+        if constexpr(FP8)
+            // zero scale operands select the unscaled v_mfma_f32_32x32x64_f8f6f4;
+            // cbsz = blgp = 0 means e4m3 for both operands
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    };
+
+    acc_t acc[4][2];
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++)
+#pragma unroll
+            for(int e = 0; e < 16; e++)
+                acc[i][j][e] = 0;
+
+    auto mfma_step = [&](auto step) {
+        constexpr int S = decltype(step)::value;
+#pragma unroll
+        for(int i = 0; i < A_TILES; i++)
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+            {
+                const int tile = FP8 ? 2 * S + i : i;
+                acc[tile][j]   = mfma(fa[S][i], fb[S][j], acc[tile][j]);
+            }
+    };
+
+    // ---- main loop ---------------------------------------------------------------
+    // Per slab: issue the loads of slab kt+3, multiply step 0 while the step-1
+    // fragments are read, barrier, multiply step 1 while the first fragments of
+    // slab kt+1 are read.  The barrier sits between the two steps so that the
+    // LDS latency of the next slab's first reads is covered by MFMAs.
+    //
+    // Slab kt+1 must be complete and visible to every wave, and every wave must
+    // have its last fragments of slab kt in registers, before that barrier: the
+    // loads issued at the top of the next iteration (slab kt+4) overwrite the
+    // stage slab kt sits in.
+    const int nk = p.k / BK;
+#pragma unroll
+    for(int s = 0; s < STAGES - 1; s++)
+        if(s < nk)
+            issue_slab(s);
+    // slab 0 has landed when at most the loads of slabs 1 and 2 are outstanding
+    if(nk >= 3)
+        wait_vmcnt<8>();
+    else if(nk == 2)
+        wait_vmcnt<4>();
+    else
+        wait_vmcnt<0>();
+    block_barrier();
+    read_step(0, IMM(0));
+
+    for(int kt = 0; kt < nk; kt++)
+    {
+        const int stage = kt & (STAGES - 1);
+        if(kt + STAGES - 1 < nk)
+            issue_slab(kt + STAGES - 1);
+        // lgkmcnt counts every outstanding LDS read, so the wait for step 0
+        // comes before the step-1 reads are issued, not after
+        WAIT_STEP(0);
+        read_step(stage, IMM(1));
+        mfma_step(IMM(0));
+        if(kt + 3 < nk)
+            wait_vmcnt<8>();
+        else if(kt + 2 < nk)
+            wait_vmcnt<4>();
+        else
+            wait_vmcnt<0>();
+        WAIT_STEP(1);
+        block_barrier();
+        if(kt + 1 < nk)
+            read_step((kt + 1) & (STAGES - 1), IMM(0));
+        mfma_step(IMM(1));
+    }
+#undef IMM
+#undef WAIT_STEP
+
+    // ---- epilogue ------------------------------------------------------------------
+    // 32 x 32 accumulator: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4,
+    // column l % 32.
+#pragma unroll
+    for(int j = 0; j < 2; j++)
+    {
+        const int col = n0 + wave_n * 64 + j * 32 + lrow;
+        if(col >= p.n)
+            continue;
+        float sb    = 1.f;
+        int32_t csb = 0;
+        if constexpr(DEQ)
+        {
+            if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                sb = p.scale_b[0];
+            else if(p.scale_b_mode == MI355_QP_PER_COL)
+                sb = p.scale_b[col];
+            if(p.zp_a != 0)
+                csb = p.colsum_b[col];
+        }
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+#pragma unroll
+            for(int e = 0; e < 16; e++)
+            {
+                const int row = m0 + wave_m * 128 + i * 32 + 8 * (e >> 2) + 4 * lgrp + (e & 3);
+                if(row >= p.m)
+                    continue;
+                const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                if constexpr(!DEQ)
+                {
+                    if constexpr(FP8)
+                        static_cast<float*>(p.c)[idx] = acc[i][j][e];
+                    else
+                        static_cast<int32_t*>(p.c)[idx] = acc[i][j][e];
+                }
+                else
+                {
+                    float sa = 1.f;
+                    if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                        sa = p.scale_a[0];
+                    else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                        sa = p.scale_a[row];
+                    // scale = fp32 product of the two scales (the graph's `mul`),
+                    // then (double(acc) - double(zp)) * scale in double, one
+                    // rounding to float (dequantizelinear)
+                    const float s = sa * sb;
+                    double d;
+                    if constexpr(FP8)
+                    {
+                        d = (double)acc[i][j][e];
+                    }
+                    else
+                    {
+                        int64_t zp = (int64_t)p.zp_a * csb;
+                        if(p.zp_b != 0)
+                            zp += (int64_t)p.zp_b * p.rowsum_a[row] -
+                                  (int64_t)p.k * p.zp_a * p.zp_b;
+                        d = (double)acc[i][j][e] - (double)(int32_t)zp;
+                    }
+                    store1<OUT>(p.c, idx, (float)(d * (double)s));
+                }
+            }
+        }
+    }
+}
+
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+int launch_one(const dma_params& p, int batch, hipStream_t stream)
+{
+    auto kern = qgemm_dma_kernel<FP8, TRANS_B, DEQ, OUT>;
+    // above the 64 KiB default: opt in once per kernel instantiation
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if(attr != hipSuccess)
+        return MI355_ERR_LAUNCH;
+    dim3 grid(p.tiles_m * p.tiles_n, batch);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+    return mi355_launch_status();
+}
+
+template <bool FP8, bool TRANS_B>
+int launch_out(const dma_params& p, int batch, bool deq, int out, hipStream_t s)
+{
+    if(!deq)
+        return launch_one<FP8, TRANS_B, false, MI355_F32>(p, batch, s);
+    switch(out)
+    {
+    case MI355_F32: return launch_one<FP8, TRANS_B, true, MI355_F32>(p, batch, s);
+    case MI355_F16: return launch_one<FP8, TRANS_B, true, MI355_F16>(p, batch, s);
+    case MI355_BF16: return launch_one<FP8, TRANS_B, true, MI355_BF16>(p, batch, s);
+    default: return MI355_ERR_UNSUPPORTED;
+    }
+}
+
+} // namespace
+
+// The direct-to-LDS kernel moves whole 16-byte chunks and cannot zero-fill a
+// partial one: K must be a multiple of the 64-byte slab, row-major B needs N a
+// multiple of 16, and every chunk must be 16-byte aligned in memory.
+bool mi355_dma_gemm_supported(const mi355_quant_dot_desc* d, const void* a, const void* b)
+{
+    if(d->trans_a)
+        return false;
+    if(d->k % BK != 0 || d->k < BK)
+        return false;
+    if(d->lda % 16 != 0 || d->stride_a % 16 != 0 || reinterpret_cast<uintptr_t>(a) % 16 != 0)
+        return false;
+    if(d->ldb % 16 != 0 || d->stride_b % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0)
+        return false;
+    if(!d->trans_b && (d->n % 16 != 0 || d->n < 16))
+        return false;
+    if(d->m > (1 << 30) || d->n > (1 << 30) || d->k > (1 << 30))
+        return false;
+    // per-lane byte offsets inside one matrix are kept in 32 bits
+    const int64_t lim = (int64_t)1 << 31;
+    if(d->m * d->lda >= lim || (d->trans_b ? d->n * d->ldb : d->k * d->ldb) >= lim)
+        return false;
+    return true;
+}
+
+int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
+                          const void* a,
+                          const void* b,
+                          void* c,
+                          const float* scale_a,
+                          const float* scale_b,
+                          const int32_t* colsum_b,
+                          const int32_t* rowsum_a,
+                          hipStream_t stream)
+{
+    dma_params p;
+    p.a            = static_cast<const uint8_t*>(a);
+    p.b            = static_cast<const uint8_t*>(b);
+    p.c            = c;
+    p.m            = (int)d->m;
+    p.n            = (int)d->n;
+    p.k            = (int)d->k;
+    p.lda          = d->lda;
+    p.ldb          = d->ldb;
+    p.ldc          = d->ldc;
+    p.stride_a     = d->stride_a;
+    p.stride_b     = d->stride_b;
+    p.stride_c     = d->stride_c;
+    p.tiles_m      = (p.m + BM - 1) / BM;
+    p.tiles_n      = (p.n + BN - 1) / BN;
+    p.scale_a      = scale_a;
+    p.scale_b      = scale_b;
+    p.colsum_b     = colsum_b;
+    p.rowsum_a     = rowsum_a;
+    p.scale_a_mode = d->scale_a_mode;
+    p.scale_b_mode = d->scale_b_mode;
+    p.zp_a         = d->zp_a;
+    p.zp_b         = d->zp_b;
+    const bool fp8 = d->in_type == MI355_FP8;
+    const bool deq = d->dequant != 0;
+    if(fp8)
+        return d->trans_b ? launch_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_out<true, false>(p, (int)d->batch, deq, d->out_type, stream);
+    return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
+                      : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+}

@@ -102,6 +102,17 @@ struct acc_traits<true>
     using type = v4f;
 };
 
+template <bool FP8>
+struct frag_traits
+{
+    using type = v4i;
+};
+template <>
+struct frag_traits<true>
+{
+    using type = v8i;
+};
+
 template <int OUT>
 MI355_DEVINL void store4(void* c, int64_t idx, const float v[4])
 {
@@ -127,16 +138,20 @@ MI355_DEVINL void store4(void* c, int64_t idx, const float v[4])
 }
 
 // FP8: element type; TRANS_B: B stored [N, K]; DEQ: apply the epilogue;
-// OUT: output element type.
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+// OUT: output element type; KFULL: K is a multiple of the 128-byte slab, so no
+// load needs a bounds predicate (a predicate per load costs a branch each).
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
 __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    using acc_t = typename acc_traits<FP8>::type;
+    using acc_t  = typename acc_traits<FP8>::type;
+    using frag_t = typename frag_traits<FP8>::type;
 
-    const int tid    = threadIdx.x;
-    const int lane   = tid & 63;
-    const int wave   = tid >> 6;
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    // wave-uniform values live in scalar registers: addresses built from them
+    // use the scalar-base form of the global loads
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave >> 2; // 0..1
     const int wave_n = wave & 3;  // 0..3
 
@@ -150,32 +165,31 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
 
     // ---- global -> register staging -------------------------------------
     // A (and K-contiguous B): 4 passes of 64 rows, 8 lanes x 16 bytes per row.
+    // Per-lane byte offsets are 32-bit (the launcher checks the extents);
+    // the slab offset k0 goes into the uniform base.
     const int ld_row = tid >> 3;
     const int ld_kc  = (tid & 7) * 16;
-    const uint8_t* a_ptr[4];
+    uint32_t a_off[4];
 #pragma unroll
     for(int s = 0; s < 4; s++)
     {
         int row  = min(m0 + ld_row + 64 * s, p.m - 1);
-        a_ptr[s] = ga + (int64_t)row * p.lda + ld_kc;
+        a_off[s] = (uint32_t)row * (uint32_t)p.lda + ld_kc;
     }
-    // K-contiguous B: same pattern over n.
-    const uint8_t* bt_ptr[4];
-    // row-major B: wave w reads k rows 16w..16w+15, lane l the dword at n = 4l.
-    const uint8_t* b_ptr = nullptr;
+    uint32_t bt_off[4]; // K-contiguous B: same pattern over n
+    uint32_t b_off = 0; // row-major B: lane l reads the dword at column 4l
     if constexpr(TRANS_B)
     {
 #pragma unroll
         for(int s = 0; s < 4; s++)
         {
             int col   = min(n0 + ld_row + 64 * s, p.n - 1);
-            bt_ptr[s] = gb + (int64_t)col * p.ldb + ld_kc;
+            bt_off[s] = (uint32_t)col * (uint32_t)p.ldb + ld_kc;
         }
     }
     else
     {
-        int col = min(n0 + 4 * lane, p.n - 4);
-        b_ptr   = gb + (int64_t)(16 * wave) * p.ldb + col;
+        b_off = (uint32_t)min(n0 + 4 * lane, p.n - 4);
     }
 
     uint4 ra[4];
@@ -183,29 +197,31 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
     uint32_t rb[16];
 
     auto load_slab = [&](int k0) {
-        const bool kin = (k0 + ld_kc) < p.k;
+        const bool kin        = KFULL || (k0 + ld_kc) < p.k;
+        const uint8_t* a_base = ga + k0;
 #pragma unroll
         for(int s = 0; s < 4; s++)
-        {
-            ra[s] = kin ? *reinterpret_cast<const uint4*>(a_ptr[s] + k0) : make_uint4(0, 0, 0, 0);
-        }
+            ra[s] = kin ? *reinterpret_cast<const uint4*>(a_base + a_off[s])
+                        : make_uint4(0, 0, 0, 0);
         if constexpr(TRANS_B)
         {
+            const uint8_t* b_base = gb + k0;
 #pragma unroll
             for(int s = 0; s < 4; s++)
-            {
-                rbt[s] =
-                    kin ? *reinterpret_cast<const uint4*>(bt_ptr[s] + k0) : make_uint4(0, 0, 0, 0);
-            }
+                rbt[s] = kin ? *reinterpret_cast<const uint4*>(b_base + bt_off[s])
+                             : make_uint4(0, 0, 0, 0);
         }
         else
         {
+            // wave w reads k rows 16w..16w+15 of the slab
+            const uint8_t* b_base = gb + (int64_t)(k0 + 16 * wave) * p.ldb;
 #pragma unroll
             for(int i = 0; i < 16; i++)
             {
-                int kk = k0 + 16 * wave + i;
-                rb[i]  = kk < p.k ? *reinterpret_cast<const uint32_t*>(b_ptr + (int64_t)(k0 + i) * p.ldb)
-                                  : 0u;
+                const int kk = k0 + 16 * wave + i;
+                rb[i]        = (KFULL || kk < p.k)
+                                   ? *reinterpret_cast<const uint32_t*>(b_base + (int64_t)i * p.ldb + b_off)
+                                   : 0u;
             }
         }
     };
@@ -215,15 +231,13 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
         uint8_t* bs = as + BM * LDS_ROW;
 #pragma unroll
         for(int s = 0; s < 4; s++)
-        {
             *reinterpret_cast<uint4*>(as + (ld_row + 64 * s) * LDS_ROW + ld_kc) = ra[s];
-        }
         if constexpr(TRANS_B)
         {
 #pragma unroll
             for(int s = 0; s < 4; s++)
             {
-                int nl  = ld_row + 64 * s;        // column within the tile
+                int nl  = ld_row + 64 * s;           // column within the tile
                 int row = (nl & 3) * 64 + (nl >> 2); // permuted LDS row
                 *reinterpret_cast<uint4*>(bs + row * LDS_ROW + ld_kc) = rbt[s];
             }
@@ -252,78 +266,113 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
         for(int j = 0; j < 4; j++)
             acc[i][j] = acc_t{0, 0, 0, 0};
 
-    const int frag_row = lane & 15;
-    const int frag_kg  = lane >> 4;
-
-    auto compute = [&](int stage) {
-        const uint8_t* as = lds + stage * STAGE_BYTES + (wave_m * 128 + frag_row) * LDS_ROW;
-        const uint8_t* bs =
-            lds + stage * STAGE_BYTES + BM * LDS_ROW + (wave_n * 16 + frag_row) * LDS_ROW;
+    // ---- LDS -> MFMA operand fragments ------------------------------------
+    // Lane l supplies row (l % 16) of a 16-row operand tile and the K bytes of
+    // lane group l / 16: 16 bytes per group for the K = 64 int8 instruction,
+    // 32 for the K = 128 fp8 one.  A and B use the same K assignment, which is
+    // all the dot product needs.
+    constexpr int FRAG_BYTES = FP8 ? 32 : 16;
+    const int frag_off = (lane & 15) * LDS_ROW + (lane >> 4) * FRAG_BYTES;
+    auto read_frag = [&](const uint8_t* q) -> frag_t {
         if constexpr(FP8)
         {
-            // one K = 128 step: lane group g supplies k bytes 32g..32g+31
-            v8i bf[4];
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-            {
-                const uint8_t* q = bs + j * 64 * LDS_ROW + frag_kg * 32;
-                v4i lo           = *reinterpret_cast<const v4i*>(q);
-                v4i hi           = *reinterpret_cast<const v4i*>(q + 16);
-                bf[j]            = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            }
-#pragma unroll
-            for(int i = 0; i < 8; i++)
-            {
-                const uint8_t* q = as + i * 16 * LDS_ROW + frag_kg * 32;
-                v4i lo           = *reinterpret_cast<const v4i*>(q);
-                v4i hi           = *reinterpret_cast<const v4i*>(q + 16);
-                v8i af           = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-                for(int j = 0; j < 4; j++)
-                    // zero scale operands select the unscaled
-                    // v_mfma_f32_16x16x128_f8f6f4; cbsz = blgp = 0 means e4m3
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        af, bf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
-            }
+            v4i lo = *reinterpret_cast<const v4i*>(q);
+            v4i hi = *reinterpret_cast<const v4i*>(q + 16);
+            return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         }
         else
         {
+            return *reinterpret_cast<const v4i*>(q);
+        }
+    };
+    // half h of a slab: int8 -> K bytes 64h..64h+63 with all 8 A tiles;
+    //                   fp8  -> all 128 K bytes with A tiles 4h..4h+3.
+    auto a_frag = [&](int stage, int h, int i) -> frag_t {
+        const uint8_t* q = lds + stage * STAGE_BYTES + frag_off;
+        if constexpr(FP8)
+            return read_frag(q + (wave_m * 128 + (4 * h + i) * 16) * LDS_ROW);
+        else
+            return read_frag(q + (wave_m * 128 + i * 16) * LDS_ROW + h * 64);
+    };
+    auto b_frag = [&](int stage, int h, int j) -> frag_t {
+        const uint8_t* q =
+            lds + stage * STAGE_BYTES + BM * LDS_ROW + frag_off + (j * 64 + wave_n * 16) * LDS_ROW;
+        if constexpr(FP8)
+            return read_frag(q);
+        else
+            return read_frag(q + h * 64);
+    };
+    auto mfma = [&](const frag_t& a, const frag_t& b, acc_t c) -> acc_t {
+        if constexpr(FP8)
+            // zero scale operands select the unscaled v_mfma_f32_16x16x128_f8f6f4;
+            // cbsz = blgp = 0 means e4m3 for both operands
+            return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+    };
+
+    constexpr int A_STEPS = FP8 ? 4 : 8; // A tiles per half slab
+    frag_t af[2];                        // A fragments, double buffered
+    frag_t bf[FP8 ? 1 : 2][4];           // B fragments (int8: one set per half)
+
+    // The fragments a half starts with are read ahead of it; inside a half the
+    // next A fragment is requested before the four MFMAs of the current one
+    // issue, so the matrix pipe does not wait on LDS latency.
+    auto first_frags = [&](int stage) {
 #pragma unroll
-            for(int ks = 0; ks < 2; ks++)
+        for(int j = 0; j < 4; j++)
+            bf[0][j] = b_frag(stage, 0, j);
+        af[0] = a_frag(stage, 0, 0);
+    };
+    auto compute_half = [&](int stage, int h) {
+#pragma unroll
+        for(int i = 0; i < A_STEPS; i++)
+        {
+            const int cur = i & 1;
+            if(i + 1 < A_STEPS)
+                af[cur ^ 1] = a_frag(stage, h, i + 1);
+            else if(h == 0)
+                af[cur ^ 1] = a_frag(stage, 1, 0);
+            if constexpr(!FP8)
             {
-                v4i bf[4];
-#pragma unroll
-                for(int j = 0; j < 4; j++)
-                    bf[j] = *reinterpret_cast<const v4i*>(bs + j * 64 * LDS_ROW + ks * 64 +
-                                                          frag_kg * 16);
-#pragma unroll
-                for(int i = 0; i < 8; i++)
-                {
-                    v4i af = *reinterpret_cast<const v4i*>(as + i * 16 * LDS_ROW + ks * 64 +
-                                                           frag_kg * 16);
-#pragma unroll
-                    for(int j = 0; j < 4; j++)
-                        acc[i][j] =
-                            __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf[j], acc[i][j], 0, 0, 0);
-                }
+                if(h == 0 && i >= A_STEPS - 4)
+                    bf[1][i - (A_STEPS - 4)] = b_frag(stage, 1, i - (A_STEPS - 4));
             }
+            const int row = FP8 ? 4 * h + i : i;
+            const int bh  = FP8 ? 0 : h;
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+                acc[row][j] = mfma(af[cur], bf[bh][j], acc[row][j]);
+            // keep "LDS reads of the next step, then this step's MFMAs" as the
+            // issue order instead of letting the reads sink to their first use
+            __builtin_amdgcn_sched_group_barrier(0x100, FP8 ? 2 : 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         }
     };
 
     // ---- main loop ------------------------------------------------------------
+    // Slab kt+1 is fetched into registers at the top of iteration kt, written to
+    // the other LDS stage between the two halves of slab kt (that stage was last
+    // read before the previous barrier), and is visible after the barrier that
+    // ends the iteration.
     const int nk = (p.k + BK - 1) / BK;
     load_slab(0);
     store_slab(0);
     __syncthreads();
+    first_frags(0);
     for(int kt = 0; kt < nk; kt++)
     {
         const bool more = kt + 1 < nk;
+        const int stage = kt & 1;
         if(more)
             load_slab((kt + 1) * BK);
-        compute(kt & 1);
+        compute_half(stage, 0);
         if(more)
-            store_slab((kt + 1) & 1);
+            store_slab(stage ^ 1);
+        compute_half(stage, 1);
         __syncthreads();
+        if(more)
+            first_frags(stage ^ 1);
     }
 
     // ---- epilogue -------------------------------------------------------------
@@ -407,10 +456,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
     }
 }
 
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
-int launch_one(const gemm_params& p, int batch, hipStream_t stream)
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
+int launch_k(const gemm_params& p, int batch, hipStream_t stream)
 {
-    auto kern = qgemm_mfma_kernel<FP8, TRANS_B, DEQ, OUT>;
+    auto kern = qgemm_mfma_kernel<FP8, TRANS_B, DEQ, OUT, KFULL>;
     // above the 64 KiB default: opt in once per kernel instantiation
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -419,6 +468,13 @@ int launch_one(const gemm_params& p, int batch, hipStream_t stream)
     dim3 grid(p.tiles_m * p.tiles_n, batch);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
     return mi355_launch_status();
+}
+
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+int launch_one(const gemm_params& p, int batch, hipStream_t stream)
+{
+    return p.k % BK == 0 ? launch_k<FP8, TRANS_B, DEQ, OUT, true>(p, batch, stream)
+                         : launch_k<FP8, TRANS_B, DEQ, OUT, false>(p, batch, stream);
 }
 
 template <bool FP8, bool TRANS_B>
@@ -470,6 +526,10 @@ bool mi355_mfma_gemm_supported(const mi355_quant_dot_desc* d,
        reinterpret_cast<uintptr_t>(c) % (4 * osz) != 0)
         return false;
     if(d->m > (1 << 30) || d->n > (1 << 30) || d->k > (1 << 30))
+        return false;
+    // per-lane byte offsets inside one matrix are kept in 32 bits
+    const int64_t lim = (int64_t)1 << 31;
+    if(d->m * d->lda >= lim || (d->trans_b ? d->n * d->ldb : d->k * d->ldb) >= lim)
         return false;
     return true;
 }
