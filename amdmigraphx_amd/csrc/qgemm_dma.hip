@@ -504,6 +504,347 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     }
 }
 
+// ---------------------------------------------------------------------------
+// int8 with v_mfma_i32_16x16x64_i8.  Same data path, LDS layouts and slab ring
+// as the kernel above; the wave's 128 x 64 block is 8 x 4 tiles of 16 x 16 and
+// one MFMA covers the whole 64-byte slab.  Under uniformly random operands the
+// chip is power limited and the 16 x 16 instruction sustains a higher rate than
+// the 32 x 32 one, which is why int8 has its own kernel.
+//
+// The operands are passed swapped (B tile as the instruction's first operand):
+// the accumulator then holds C transposed, lane l owning row (l % 16) of the A
+// tile and 4 consecutive columns 4*(l / 16).. of the B tile, so C goes out in
+// 16-byte stores.
+//
+// A slab is multiplied in two steps of 16 MFMAs (A tiles 0-3, then 4-7) with
+// the barrier between them; the slab's four B fragments are shared by both
+// steps and double buffered across slabs, so the loop body exists for both
+// slab parities.
+// ---------------------------------------------------------------------------
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE>
+__global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 2; // 0..1
+    const int wave_n = wave & 3;  // 0..3
+
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
+    const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+
+    // ---- global -> LDS (identical to the kernel above) ------------------------
+    uint32_t a_off[2], b_off[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+    {
+        const int blk = wave + 8 * h;
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int row   = min(m0 + r, p.m - 1);
+            a_off[h]        = (uint32_t)row * (uint32_t)p.lda + chunk * 16;
+        }
+        if constexpr(TRANS_B)
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int col   = min(n0 + r, p.n - 1);
+            b_off[h]        = (uint32_t)col * (uint32_t)p.ldb + chunk * 16;
+        }
+        else
+        {
+            const int k     = 4 * blk + (lane >> 4);
+            const int chunk = (lane & 15) ^ (k & 7);
+            const int col   = min(n0 + chunk * 16, p.n - 16);
+            b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
+        }
+    }
+    auto issue_slab = [&](int kt) {
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
+        const uint8_t* a_base = ga + (int64_t)kt * BK;
+        const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+            load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+            load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+    };
+
+    // ---- LDS -> operand fragments ----------------------------------------------
+    // 16-row operand tile: lane l supplies row l % 16 and K bytes 16*(l / 16)..
+    const int lrow      = lane & 15;
+    const int lgrp      = lane >> 4;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    const int sw        = (lrow >> 2) & 3;
+    const uint32_t a_lane = (wave_m * 128 + lrow) * BK + ((lgrp ^ sw) << 4);
+    uint32_t b_lane[2]; // K-contiguous B: one offset; row-major B: one per 8-row k block
+    if constexpr(TRANS_B)
+    {
+        b_lane[0] = A_BYTES + (wave_n * 64 + lrow) * BK + ((lgrp ^ sw) << 4);
+        b_lane[1] = 0;
+    }
+    else
+    {
+        // transposing read: lane 16g + i supplies row k = 16g + 8r + (i >> 1), byte
+        // half (i & 1) of the 16-byte chunk with the tile's 16 columns, and
+        // receives column i with 8 consecutive k (r = 0, 1)
+#pragma unroll
+        for(int r = 0; r < 2; r++)
+        {
+            const int k = lgrp * 16 + 8 * r + (lrow >> 1);
+            // chunk index of tile j is wave_n*4 + j; its low bits are XORed with
+            // k & 7, which for j in 0..3 only needs (j ^ x) on the low two bits
+            b_lane[r] = A_BYTES + k * BN + 8 * (lrow & 1);
+        }
+    }
+    const int bsw = (lrow >> 1) & 7; // k & 7 of this lane's row in the transposing read
+
+    v4i fa[2][4];
+    v4i fb[2][4];
+    v4i acc[8][4];
+#pragma unroll
+    for(int i = 0; i < 8; i++)
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            acc[i][j] = v4i{0, 0, 0, 0};
+
+#define RD128(dst, addr, imm) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define RDTR8(dst, addr, imm) \
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+
+    // A tiles 4*S .. 4*S+3 of the slab in `stage` -> fa[S]
+#define READ_A(stage, S)                                              \
+    do                                                                \
+    {                                                                 \
+        const uint32_t q_ = lds0 + (stage) * STAGE_BYTES + a_lane;    \
+        RD128(fa[S][0], q_, (4 * (S) + 0) * 16 * BK);                 \
+        RD128(fa[S][1], q_, (4 * (S) + 1) * 16 * BK);                 \
+        RD128(fa[S][2], q_, (4 * (S) + 2) * 16 * BK);                 \
+        RD128(fa[S][3], q_, (4 * (S) + 3) * 16 * BK);                 \
+    } while(0)
+    // the four B tiles of the slab in `stage` -> fb[P]
+#define READ_B(stage, P)                                                                   \
+    do                                                                                     \
+    {                                                                                      \
+        const uint32_t s_ = lds0 + (stage) * STAGE_BYTES;                                  \
+        if constexpr(TRANS_B)                                                              \
+        {                                                                                  \
+            const uint32_t q_ = s_ + b_lane[0];                                            \
+            RD128(fb[P][0], q_, 0 * 16 * BK);                                              \
+            RD128(fb[P][1], q_, 1 * 16 * BK);                                              \
+            RD128(fb[P][2], q_, 2 * 16 * BK);                                              \
+            RD128(fb[P][3], q_, 3 * 16 * BK);                                              \
+        }                                                                                  \
+        else                                                                               \
+        {                                                                                  \
+            _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++)                                \
+            {                                                                              \
+                const uint32_t c_ = (uint32_t)(((wave_n * 4 + j_) ^ bsw) << 4);            \
+                v2i lo_, hi_;                                                              \
+                RDTR8(lo_, s_ + b_lane[0] + c_, 0);                                        \
+                RDTR8(hi_, s_ + b_lane[1] + c_, 0);                                        \
+                fb[P][j_] = v4i{lo_.x, lo_.y, hi_.x, hi_.y};                               \
+            }                                                                              \
+        }                                                                                  \
+    } while(0)
+#define WAIT4(x) \
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3])::"memory")
+    // 16 MFMAs: A tiles 4*S.. against the four B tiles in fb[P]
+#define MFMA_STEP(S, P)                                                                     \
+    do                                                                                      \
+    {                                                                                       \
+        _Pragma("unroll") for(int i_ = 0; i_ < 4; i_++)                                     \
+        {                                                                                   \
+            _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++) acc[4 * (S) + i_][j_] =         \
+                __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[P][j_], fa[S][i_],                \
+                                                      acc[4 * (S) + i_][j_], 0, 0, 0);      \
+        }                                                                                   \
+    } while(0)
+    // one slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P]
+#define SLAB(kt, P)                                                     \
+    do                                                                  \
+    {                                                                   \
+        const int stage_ = (kt) & (STAGES - 1);                         \
+        if((kt) + STAGES - 1 < nk)                                      \
+            issue_slab((kt) + STAGES - 1);                              \
+        WAIT4(fa[0]);                                                   \
+        WAIT4(fb[P]);                                                   \
+        READ_A(stage_, 1);                                              \
+        MFMA_STEP(0, P);                                                \
+        if((kt) + 3 < nk)                                               \
+            wait_vmcnt<8>();                                            \
+        else if((kt) + 2 < nk)                                          \
+            wait_vmcnt<4>();                                            \
+        else                                                            \
+            wait_vmcnt<0>();                                            \
+        WAIT4(fa[1]);                                                   \
+        block_barrier();                                                \
+        if((kt) + 1 < nk)                                               \
+        {                                                               \
+            READ_A(((kt) + 1) & (STAGES - 1), 0);                       \
+            READ_B(((kt) + 1) & (STAGES - 1), 1 - (P));                 \
+        }                                                               \
+        MFMA_STEP(1, P);                                                \
+    } while(0)
+
+    // ---- main loop (see the kernel above for the ordering argument) ----------
+    const int nk = p.k / BK;
+#pragma unroll
+    for(int s = 0; s < STAGES - 1; s++)
+        if(s < nk)
+            issue_slab(s);
+    if(nk >= 3)
+        wait_vmcnt<8>();
+    else if(nk == 2)
+        wait_vmcnt<4>();
+    else
+        wait_vmcnt<0>();
+    block_barrier();
+    READ_A(0, 0);
+    READ_B(0, 0);
+    int kt = 0;
+    for(; kt + 1 < nk; kt += 2)
+    {
+        SLAB(kt, 0);
+        SLAB(kt + 1, 1);
+    }
+    if(kt < nk)
+        SLAB(kt, 0);
+#undef SLAB
+#undef MFMA_STEP
+#undef WAIT4
+#undef READ_B
+#undef READ_A
+#undef RDTR8
+#undef RD128
+
+    // ---- epilogue ----------------------------------------------------------------
+    // acc[i][j][e]: row 16*i + (l % 16) of the wave's A block, column
+    // 16*j + 4*(l / 16) + e of its B block.
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+    {
+        const int col = n0 + wave_n * 64 + j * 16 + 4 * lgrp;
+        if(col >= p.n)
+            continue; // N is a multiple of 4 on this path, so the 4 columns are in or out together
+        float sb[4]   = {1.f, 1.f, 1.f, 1.f};
+        int32_t cs[4] = {0, 0, 0, 0};
+        if constexpr(DEQ)
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                    sb[e] = p.scale_b[0];
+                else if(p.scale_b_mode == MI355_QP_PER_COL)
+                    sb[e] = p.scale_b[col + e];
+                if(p.zp_a != 0)
+                    cs[e] = p.colsum_b[col + e];
+            }
+        }
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+        {
+            const int row = m0 + wave_m * 128 + i * 16 + lrow;
+            if(row >= p.m)
+                continue;
+            const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+            if constexpr(!DEQ)
+            {
+                int32_t* o = static_cast<int32_t*>(p.c) + idx;
+                if constexpr(VEC_STORE)
+                    *reinterpret_cast<v4i*>(o) = acc[i][j];
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        o[e] = acc[i][j][e];
+                }
+            }
+            else
+            {
+                float sa = 1.f;
+                if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                    sa = p.scale_a[0];
+                else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                    sa = p.scale_a[row];
+                int64_t zrow = 0;
+                if(p.zp_b != 0)
+                    zrow = (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b;
+                float v[4];
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    // scale = fp32 product of the two scales (the graph's `mul`),
+                    // then (double(acc) - double(zp)) * scale in double, one
+                    // rounding to float (dequantizelinear)
+                    const float s  = sa * sb[e];
+                    const double d = (double)acc[i][j][e] -
+                                     (double)(int32_t)(zrow + (int64_t)p.zp_a * cs[e]);
+                    v[e] = (float)(d * (double)s);
+                }
+                if constexpr(VEC_STORE)
+                {
+                    if constexpr(OUT == MI355_F32)
+                        *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) =
+                            v4f{v[0], v[1], v[2], v[3]};
+                    else if constexpr(OUT == MI355_F16)
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                            convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+                    else
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
+                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                }
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        store1<OUT>(p.c, idx + e, v[e]);
+                }
+            }
+        }
+    }
+}
+
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC>
+int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
+{
+    auto kern = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if(attr != hipSuccess)
+        return MI355_ERR_LAUNCH;
+    dim3 grid(p.tiles_m * p.tiles_n, batch);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+    return mi355_launch_status();
+}
+
+template <bool TRANS_B, bool VEC>
+int launch_i8_out(const dma_params& p, int batch, bool deq, int out, hipStream_t s)
+{
+    if(!deq)
+        return launch_i8_one<TRANS_B, false, MI355_F32, VEC>(p, batch, s);
+    switch(out)
+    {
+    case MI355_F32: return launch_i8_one<TRANS_B, true, MI355_F32, VEC>(p, batch, s);
+    case MI355_F16: return launch_i8_one<TRANS_B, true, MI355_F16, VEC>(p, batch, s);
+    case MI355_BF16: return launch_i8_one<TRANS_B, true, MI355_BF16, VEC>(p, batch, s);
+    default: return MI355_ERR_UNSUPPORTED;
+    }
+}
+
 template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
 int launch_one(const dma_params& p, int batch, hipStream_t stream)
 {
@@ -596,6 +937,19 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     if(fp8)
         return d->trans_b ? launch_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_out<true, false>(p, (int)d->batch, deq, d->out_type, stream);
-    return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
-                      : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+    // int8: 4 consecutive outputs of a row go out in one store when every row of
+    // C keeps them aligned (N % 4 == 0 holds whenever this path is taken for
+    // row-major B; for [N, K] B it is checked here)
+    const size_t osz = deq ? mi355_dtype_size(d->out_type) : 4;
+    const bool vec   = d->n % 4 == 0 && d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(c) % (4 * osz) == 0;
+    if(d->n % 4 != 0)
+        // the 16 x 16 kernel drops or keeps 4 columns together
+        return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+    if(vec)
+        return d->trans_b ? launch_i8_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_i8_out<false, true>(p, (int)d->batch, deq, d->out_type, stream);
+    return d->trans_b ? launch_i8_out<true, false>(p, (int)d->batch, deq, d->out_type, stream)
+                      : launch_i8_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
 }
