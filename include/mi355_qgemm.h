@@ -207,6 +207,33 @@ int mi355_w4a16_gemm(const void* a, int64_t lda,
                      int64_t m, int64_t n, int64_t k, int64_t group,
                      void* stream);
 
+/*
+ * Float dot: C[b, m, n] = T( sum_k double(A[b, m, k]) * double(B[b, k, n]) ), k ascending,
+ * T in {F32, F16, BF16} for all three tensors (16-bit results truncate, as the software
+ * floats do).
+ *
+ * Replaces: op::dot::compute (src/include/migraphx/op/dot.hpp:102-107) -> gemm_naive
+ * (src/gemm.cpp:42-63).  Bit-exact with it; meant for calibration runs of the unquantized
+ * graph and for the dot behind a dequantizelinear that the int4 kernel does not cover, not
+ * for throughput.  A and B are addressed by element strides, so transposed and broadcast views
+ * need no copy; C is row-major with leading dimension ldc.
+ */
+int mi355_dot(const void* a, const void* b, void* c, int32_t type,
+              int64_t m, int64_t n, int64_t k,
+              int64_t a_stride_m, int64_t a_stride_k, int64_t b_stride_k, int64_t b_stride_n,
+              int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+              void* stream);
+
+/*
+ * contiguous: gather a strided view (ndim <= MI355_MAX_DIMS, element strides, zero = broadcast)
+ * into a dense row-major tensor.  lens / strides are HOST arrays.
+ *
+ * Replaces: op::contiguous::compute (src/include/migraphx/op/contiguous.hpp:43-83).
+ */
+#define MI355_MAX_DIMS 8
+int mi355_contiguous(const void* in, void* out, int32_t elem_size, int32_t ndim,
+                     const int64_t* lens, const int64_t* strides, void* stream);
+
 /* Human-readable text for a status code (static storage). */
 const char* mi355_status_string(int status);
 
