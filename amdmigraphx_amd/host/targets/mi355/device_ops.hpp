@@ -1,0 +1,213 @@
+// Operators of the mi355 target.  Each compute() fills the C-ABI arguments from the shapes of the
+// arguments it was handed, launches on the context's stream and returns its output buffer (the
+// last argument), following the device-operator convention of
+// src/targets/gpu/include/migraphx/gpu/gemm.hpp:109-128.
+#ifndef MIGRAPHX_GUARD_MI355_DEVICE_OPS_HPP
+#define MIGRAPHX_GUARD_MI355_DEVICE_OPS_HPP
+
+#include <migraphx/mi355/target.hpp>
+#include <migraphx/operation.hpp>
+#include <mi355_qgemm.h>
+
+namespace migraphx {
+namespace mi355 {
+
+int to_mi355_type(shape::type_t t); // throws for a type the kernels do not take
+
+// How a [..., R, C] tensor maps onto the (pointer, leading dimension, transpose flag, batch
+// stride) form the GEMM entry points take.
+struct matrix_view
+{
+    bool ok           = false;
+    bool trans        = false; // element (r, c) at c*ld + r instead of r*ld + c
+    int64_t rows      = 0;
+    int64_t cols      = 0;
+    int64_t ld        = 0;
+    int64_t batch     = 1;
+    int64_t batch_stride = 0;
+    int64_t stride_r  = 0; // plain element strides, for entry points that take them
+    int64_t stride_c  = 0;
+};
+matrix_view view_as_matrix(const shape& s);
+
+// strides (row, column) of a tensor seen as [prod(leading dims), last dim]; false when the
+// leading dimensions do not collapse into one stride
+bool collapse_2d(const shape& s, int64_t& stride_r, int64_t& stride_c);
+
+struct allocate
+{
+    shape s;
+    argument buffer; // set by finalize
+    std::string name() const { return "mi355::allocate"; }
+    shape compute_shape(const std::vector<shape>&) const { return s; }
+    void finalize(migraphx::context&, const shape&, const std::vector<shape>&)
+    {
+        if(buffer.empty())
+            buffer = allocate_device(s);
+    }
+    argument compute(migraphx::context&, const shape&, const std::vector<argument>&) const;
+};
+
+struct device_literal
+{
+    argument data;
+    std::string name() const { return "mi355::literal"; }
+    shape compute_shape(const std::vector<shape>&) const { return data.get_shape(); }
+    argument compute(migraphx::context&, const shape&, const std::vector<argument>&) const
+    {
+        return data;
+    }
+};
+
+struct copy_to_device
+{
+    std::string name() const { return "mi355::copy_to_device"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+struct copy_from_device
+{
+    std::string name() const { return "mi355::copy_from_device"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const;
+};
+
+// inputs: a, b, [scale_a, scale_b] (dequant), [colsum_b] (zp_a != 0), [rowsum_a] (zp_b != 0), out
+struct quant_dot
+{
+    bool dequant           = false;
+    int64_t zp_a           = 0;
+    int64_t zp_b           = 0;
+    int64_t scale_a_mode   = MI355_QP_NONE;
+    int64_t scale_b_mode   = MI355_QP_NONE;
+    shape::type_t out_type = shape::int32_type;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.dequant, "dequant");
+        f(self.zp_a, "zp_a");
+        f(self.zp_b, "zp_b");
+        f(self.scale_a_mode, "scale_a_mode");
+        f(self.scale_b_mode, "scale_b_mode");
+        f(self.out_type, "out_type");
+    }
+    std::string name() const { return "mi355::quant_dot"; }
+    std::size_t expected_inputs() const
+    {
+        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0);
+    }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: int8 matrix, out (int32 [cols] or [rows])
+struct colsum
+{
+    std::string name() const { return "mi355::colsum"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+struct rowsum
+{
+    std::string name() const { return "mi355::rowsum"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: a, b, out
+struct dot
+{
+    std::string name() const { return "mi355::dot"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: a fp16 [M, K], packed weights uint8 [N, K/2], scales fp16 [N, K/group], [zero points], out
+struct w4a16_gemm
+{
+    int64_t group     = 128;
+    int64_t zp_mode   = MI355_W4_ZP_SCALAR;
+    int64_t zp_scalar = 8;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.group, "group");
+        f(self.zp_mode, "zp_mode");
+        f(self.zp_scalar, "zp_scalar");
+    }
+    std::string name() const { return "mi355::w4a16_gemm"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: x, scale view, [zero point view], out
+struct quantizelinear
+{
+    shape::type_t out_type = shape::uint8_type;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.out_type, "out_type");
+    }
+    std::string name() const { return "mi355::quantizelinear"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+struct dequantizelinear
+{
+    std::string name() const { return "mi355::dequantizelinear"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: x, out.  The packed axis is the last one.
+struct unpack_int4
+{
+    std::string name() const { return "mi355::unpack_int4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+struct pack_int4
+{
+    std::string name() const { return "mi355::pack_int4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+struct convert
+{
+    shape::type_t target_type = shape::half_type;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.target_type, "target_type");
+    }
+    std::string name() const { return "mi355::convert"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+struct contiguous
+{
+    std::string name() const { return "mi355::contiguous"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+} // namespace mi355
+} // namespace migraphx
+#endif

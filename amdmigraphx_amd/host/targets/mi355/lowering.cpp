@@ -1,0 +1,579 @@
+#include "device_ops.hpp"
+#include <migraphx/ops.hpp>
+#include <migraphx/passes.hpp>
+#include <migraphx/register_op.hpp>
+#include <algorithm>
+#include <set>
+#include <unordered_map>
+#include <unordered_set>
+
+namespace migraphx {
+namespace mi355 {
+
+namespace {
+
+std::vector<instruction_ref> all_instructions(const module& m)
+{
+    std::vector<instruction_ref> r;
+    for(auto it = m.begin(); it != m.end(); ++it)
+        r.push_back(it);
+    return r;
+}
+
+instruction_ref skip_broadcasts(instruction_ref i)
+{
+    while(i->name() == "broadcast" or i->name() == "multibroadcast")
+        i = i->inputs().front();
+    return i;
+}
+
+instruction_ref insert_allocation(module& m, instruction_ref ins, const shape& s)
+{
+    allocate a;
+    a.s = s;
+    return m.insert_instruction(ins, operation{a});
+}
+
+// a dense copy of `x` placed before `ins` when x is not in standard layout
+instruction_ref make_standard(module& m, instruction_ref ins, instruction_ref x)
+{
+    if(x->get_shape().standard())
+        return x;
+    auto out = insert_allocation(m, ins, shape{x->get_shape().type(), x->get_shape().lens()});
+    return m.insert_instruction(ins, operation{contiguous{}}, x, out);
+}
+
+// a quantization parameter the pointwise kernels can address with (row, column) strides
+instruction_ref make_param(module& m, instruction_ref ins, instruction_ref p)
+{
+    int64_t sr = 0;
+    int64_t sc = 0;
+    if(collapse_2d(p->get_shape(), sr, sc))
+        return p;
+    auto out = insert_allocation(m, ins, shape{p->get_shape().type(), p->get_shape().lens()});
+    return m.insert_instruction(ins, operation{contiguous{}}, p, out);
+}
+
+// value of a constant that is one element behind its broadcasts
+bool scalar_constant(instruction_ref i, int64_t& v)
+{
+    auto base = skip_broadcasts(i);
+    if(not base->can_eval() or base->get_shape().elements() != 1)
+        return false;
+    v = base->eval().to_vector<int64_t>().front();
+    return true;
+}
+
+bool all_zero_constant(instruction_ref i)
+{
+    auto base = skip_broadcasts(i);
+    if(not base->can_eval())
+        return false;
+    auto v = base->eval().to_vector<double>();
+    return std::all_of(v.begin(), v.end(), [](double x) { return x == 0; });
+}
+
+// ---- quant_dot -> dequantizelinear [-> convert] --------------------------------------------
+
+// the zero-point expression simplify_qdq builds (src/simplify_qdq.cpp:250-279):
+//   0 [+ quant_dot(zp_a, B)] [+ quant_dot(A, zp_b)] [- quant_dot(zp_a, zp_b)]
+struct zp_terms
+{
+    bool ok      = true;
+    int64_t zp_a = 0;
+    int64_t zp_b = 0;
+    bool seen_a = false, seen_b = false, seen_ab = false;
+};
+
+void parse_zp(instruction_ref e, instruction_ref a, instruction_ref b, bool negated, zp_terms& t)
+{
+    if(not t.ok)
+        return;
+    if(e->name() == "add")
+    {
+        parse_zp(e->inputs()[0], a, b, negated, t);
+        parse_zp(e->inputs()[1], a, b, negated, t);
+        return;
+    }
+    if(e->name() == "sub")
+    {
+        parse_zp(e->inputs()[0], a, b, negated, t);
+        parse_zp(e->inputs()[1], a, b, not negated, t);
+        return;
+    }
+    if(e->name() == "multibroadcast" or e->name() == "broadcast" or e->name() == "@literal")
+    {
+        t.ok = t.ok and not negated and all_zero_constant(e);
+        return;
+    }
+    if(e->name() != "quant_dot" or e->inputs().size() != 2)
+    {
+        t.ok = false;
+        return;
+    }
+    auto l = e->inputs()[0];
+    auto r = e->inputs()[1];
+    int64_t vl = 0;
+    int64_t vr = 0;
+    const bool cl = l != a and scalar_constant(l, vl);
+    const bool cr = r != b and scalar_constant(r, vr);
+    if(cl and r == b and not negated and not t.seen_a)
+    {
+        t.zp_a   = vl;
+        t.seen_a = true;
+    }
+    else if(l == a and cr and not negated and not t.seen_b)
+    {
+        t.zp_b   = vr;
+        t.seen_b = true;
+    }
+    else if(cl and cr and negated and not t.seen_ab)
+    {
+        t.seen_ab = true;
+        // checked against the two single terms once all are known
+        if((t.seen_a and t.zp_a != vl) or (t.seen_b and t.zp_b != vr))
+            t.ok = false;
+        t.zp_a = vl;
+        t.zp_b = vr;
+    }
+    else
+    {
+        t.ok = false;
+    }
+}
+
+// how a scale broadcast to the [.., M, N] result varies: per tensor, per row or per column
+int scale_mode(const shape& s)
+{
+    const std::size_t nd = s.ndim();
+    bool row = false;
+    bool col = false;
+    for(std::size_t i = 0; i < nd; i++)
+    {
+        if(s.lens()[i] == 1 or s.strides()[i] == 0)
+            continue;
+        if(i == nd - 2 and s.strides()[i] == 1)
+            row = true;
+        else if(i == nd - 1 and s.strides()[i] == 1)
+            col = true;
+        else
+            return -1;
+    }
+    if(row and col)
+        return -1;
+    return row ? MI355_QP_PER_ROW : (col ? MI355_QP_PER_COL : MI355_QP_PER_TENSOR);
+}
+
+bool fuse_quant_dot_dq(module& m, instruction_ref dq)
+{
+    if(dq->name() != "dequantizelinear")
+        return false;
+    auto qd = dq->inputs()[0];
+    if(qd->name() != "quant_dot" or qd->inputs().size() != 2 or qd->outputs().size() != 1)
+        return false;
+    auto a = qd->inputs()[0];
+    auto b = qd->inputs()[1];
+    if(not view_as_matrix(a->get_shape()).ok or not view_as_matrix(b->get_shape()).ok)
+        return false;
+    auto scale = dq->inputs()[1];
+    if(scale->get_shape().type() != shape::float_type)
+        return false;
+
+    // scale: mul(bcast(s1), bcast(s2)) or one broadcast tensor
+    instruction_ref sa = scale;
+    instruction_ref sb = scale;
+    int mode_a         = MI355_QP_NONE;
+    int mode_b         = MI355_QP_NONE;
+    if(scale->name() == "mul")
+    {
+        sa     = scale->inputs()[0];
+        sb     = scale->inputs()[1];
+        mode_a = scale_mode(sa->get_shape());
+        mode_b = scale_mode(sb->get_shape());
+        if(mode_a == MI355_QP_PER_COL and mode_b != MI355_QP_PER_COL)
+        {
+            std::swap(sa, sb);
+            std::swap(mode_a, mode_b);
+        }
+        else if(mode_b == MI355_QP_PER_ROW and mode_a != MI355_QP_PER_ROW)
+        {
+            std::swap(sa, sb);
+            std::swap(mode_a, mode_b);
+        }
+        if(mode_a < 0 or mode_b < 0 or mode_a == MI355_QP_PER_COL or mode_b == MI355_QP_PER_ROW)
+            return false;
+    }
+    else
+    {
+        const int mode = scale_mode(scale->get_shape());
+        if(mode < 0)
+            return false;
+        if(mode == MI355_QP_PER_COL)
+            mode_b = mode;
+        else
+            mode_a = mode;
+    }
+
+    zp_terms t;
+    if(dq->inputs().size() == 3)
+    {
+        parse_zp(dq->inputs()[2], a, b, false, t);
+        if(not t.ok)
+            return false;
+        // both zero points set needs the cross term, one alone must not have it
+        if(t.seen_ab != (t.seen_a and t.seen_b))
+            return false;
+        if(not t.seen_a)
+            t.zp_a = 0;
+        if(not t.seen_b)
+            t.zp_b = 0;
+        if((t.zp_a != 0 or t.zp_b != 0) and
+           (a->get_shape().type() != shape::int8_type or view_as_matrix(a->get_shape()).batch != 1))
+            return false;
+    }
+
+    // an only user that converts to a 16-bit float joins the epilogue
+    instruction_ref last   = dq;
+    shape::type_t out_type = shape::float_type;
+    if(dq->outputs().size() == 1 and dq->outputs().front()->name() == "convert")
+    {
+        auto cv = dq->outputs().front();
+        auto tt = any_cast<op::convert>(cv->get_operator()).target_type;
+        if(tt == shape::half_type or tt == shape::bf16_type)
+        {
+            last     = cv;
+            out_type = tt;
+        }
+    }
+
+    quant_dot op;
+    op.dequant      = true;
+    op.zp_a         = t.zp_a;
+    op.zp_b         = t.zp_b;
+    op.scale_a_mode = mode_a;
+    op.scale_b_mode = mode_b;
+    op.out_type     = out_type;
+    // an absent scale still needs a pointer-sized argument: pass the other one, its mode is NONE
+    std::vector<instruction_ref> args = {a, b, sa, sb};
+    if(t.zp_a != 0)
+    {
+        const auto n = b->get_shape().lens().back();
+        auto buf     = insert_allocation(m, last, shape{shape::int32_type, {n}});
+        args.push_back(m.insert_instruction(last, operation{colsum{}}, b, buf));
+    }
+    if(t.zp_b != 0)
+    {
+        const auto rows = a->get_shape().lens()[a->get_shape().ndim() - 2];
+        auto buf        = insert_allocation(m, last, shape{shape::int32_type, {rows}});
+        args.push_back(m.insert_instruction(last, operation{rowsum{}}, a, buf));
+    }
+    args.push_back(insert_allocation(m, last, shape{out_type, qd->get_shape().lens()}));
+    m.replace_instruction(last, operation{op}, args);
+    return true;
+}
+
+// ---- dot(x, transpose(dequantizelinear(unpack_int4(w), blockwise scales, zero points))) -------
+
+instruction_ref skip_full_slice(instruction_ref x, bool& sliced)
+{
+    sliced = false;
+    if(x->name() == "slice")
+    {
+        sliced = true;
+        return x->inputs().front();
+    }
+    return x;
+}
+
+// x = reshape{n,-1}(multibroadcast{[n, nblk, blk]}(unsqueeze{2}(base [n, nblk]))): every element
+// of base repeated blk times along the last axis (src/onnx/parse_matmulnbits.cpp:140-158)
+bool match_blockwise(instruction_ref x, std::size_t n, instruction_ref& base, std::size_t& blk)
+{
+    bool sliced = false;
+    x           = skip_full_slice(x, sliced);
+    if(sliced)
+        return false; // a runt block: K is not a multiple of the block size
+    if(x->name() != "reshape")
+        return false;
+    auto mb = x->inputs().front();
+    if(mb->name() != "multibroadcast" or mb->get_shape().ndim() != 3 or mb->get_shape().lens()[0] != n)
+        return false;
+    auto us = mb->inputs().front();
+    if(us->name() != "unsqueeze" or us->get_shape().ndim() != 3 or us->get_shape().lens()[2] != 1)
+        return false;
+    base = us->inputs().front();
+    if(base->get_shape().ndim() != 2 or not base->get_shape().standard())
+        return false;
+    blk = mb->get_shape().lens()[2];
+    return true;
+}
+
+bool lower_w4a16(module& m, instruction_ref ins)
+{
+    auto a  = ins->inputs()[0];
+    auto bt = ins->inputs()[1];
+    if(a->get_shape().type() != shape::half_type or a->get_shape().ndim() != 2)
+        return false;
+    if(bt->name() != "transpose")
+        return false;
+    auto dq = bt->inputs().front();
+    if(dq->name() != "dequantizelinear" or dq->get_shape().ndim() != 2 or
+       dq->get_shape().type() != shape::half_type)
+        return false;
+    const auto n = dq->get_shape().lens()[0];
+    const auto k = dq->get_shape().lens()[1];
+    bool sliced  = false;
+    auto unpk    = skip_full_slice(dq->inputs()[0], sliced);
+    if(sliced or unpk->name() != "unpack_int4" or unpk->get_shape().type() != shape::uint8_type)
+        return false;
+    auto packed = unpk->inputs().front();
+    if(not packed->get_shape().standard() or packed->get_shape().ndim() != 2)
+        return false;
+
+    instruction_ref scales;
+    std::size_t blk = 0;
+    if(not match_blockwise(dq->inputs()[1], n, scales, blk))
+        return false;
+    if(blk % 32 != 0 or k % blk != 0 or scales->get_shape().lens()[1] != k / blk)
+        return false;
+
+    w4a16_gemm op;
+    op.group = static_cast<int64_t>(blk);
+    std::vector<instruction_ref> args = {a, packed, scales};
+    if(dq->inputs().size() == 2)
+    {
+        op.zp_mode   = MI355_W4_ZP_SCALAR;
+        op.zp_scalar = 0;
+    }
+    else
+    {
+        auto z    = dq->inputs()[2];
+        int64_t v = 0;
+        instruction_ref zbase;
+        std::size_t zblk = 0;
+        if(scalar_constant(z, v))
+        {
+            op.zp_mode   = MI355_W4_ZP_SCALAR;
+            op.zp_scalar = v;
+        }
+        else if(match_blockwise(z, n, zbase, zblk) and zblk == blk)
+        {
+            bool zsliced = false;
+            auto zu      = skip_full_slice(zbase, zsliced);
+            if(zu->name() == "unpack_int4" and zu->inputs().front()->get_shape().standard())
+            {
+                op.zp_mode = MI355_W4_ZP_PACKED;
+                args.push_back(zu->inputs().front());
+            }
+            else if(not zsliced and zbase->get_shape().type() == shape::uint8_type)
+            {
+                op.zp_mode = MI355_W4_ZP_GROUP;
+                args.push_back(zbase);
+            }
+            else
+                return false;
+        }
+        else
+            return false;
+    }
+    if(a->get_shape().strides()[1] != 1 and a->get_shape().lens()[1] != 1)
+        args[0] = make_standard(m, ins, a);
+    args.push_back(insert_allocation(m, ins, shape{shape::half_type, {a->get_shape().lens()[0], n}}));
+    m.replace_instruction(ins, operation{op}, args);
+    return true;
+}
+
+// ---- one operator at a time ------------------------------------------------------------------
+
+void lower_instruction(module& m, instruction_ref ins)
+{
+    const auto name = ins->name();
+    auto out        = [&](const shape& s) { return insert_allocation(m, ins, s); };
+    auto standard_out = [&] { return out(shape{ins->get_shape().type(), ins->get_shape().lens()}); };
+    if(name == "quant_dot")
+    {
+        if(ins->inputs().size() != 2)
+            MIGRAPHX_THROW("mi355: quant_dot with block scales has no kernel");
+        auto a = ins->inputs()[0];
+        auto b = ins->inputs()[1];
+        if(not view_as_matrix(a->get_shape()).ok)
+            a = make_standard(m, ins, a);
+        if(not view_as_matrix(b->get_shape()).ok)
+            b = make_standard(m, ins, b);
+        quant_dot op;
+        op.out_type = ins->get_shape().type();
+        m.replace_instruction(ins, operation{op}, a, b, standard_out());
+    }
+    else if(name == "dot")
+    {
+        if(lower_w4a16(m, ins))
+            return;
+        m.replace_instruction(ins, operation{dot{}}, ins->inputs()[0], ins->inputs()[1], standard_out());
+    }
+    else if(name == "quantizelinear" or name == "dequantizelinear")
+    {
+        std::vector<instruction_ref> args;
+        args.push_back(make_standard(m, ins, ins->inputs()[0]));
+        for(std::size_t i = 1; i < ins->inputs().size(); i++)
+            args.push_back(make_param(m, ins, ins->inputs()[i]));
+        args.push_back(standard_out());
+        if(name == "quantizelinear")
+        {
+            quantizelinear op;
+            op.out_type = ins->get_shape().type();
+            m.replace_instruction(ins, operation{op}, args);
+        }
+        else
+        {
+            m.replace_instruction(ins, operation{dequantizelinear{}}, args);
+        }
+    }
+    else if(name == "unpack_int4" or name == "pack_int4")
+    {
+        const auto nd   = static_cast<int64_t>(ins->inputs()[0]->get_shape().ndim());
+        const auto axis = name == "unpack_int4" ? any_cast<op::unpack_int4>(ins->get_operator()).axis
+                                                : any_cast<op::pack_int4>(ins->get_operator()).axis;
+        if(axis != -1 and axis != nd - 1)
+            MIGRAPHX_THROW("mi355: " + name + " along an axis other than the last has no kernel");
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        if(name == "unpack_int4")
+            m.replace_instruction(ins, operation{unpack_int4{}}, x, standard_out());
+        else
+            m.replace_instruction(ins, operation{pack_int4{}}, x, standard_out());
+    }
+    else if(name == "convert")
+    {
+        convert op;
+        op.target_type = any_cast<op::convert>(ins->get_operator()).target_type;
+        auto x         = make_standard(m, ins, ins->inputs()[0]);
+        m.replace_instruction(ins, operation{op}, x, standard_out());
+    }
+    else if(name == "contiguous")
+    {
+        m.replace_instruction(ins, operation{contiguous{}}, ins->inputs()[0], standard_out());
+    }
+    else if(name == "reshape")
+    {
+        // the view operator only re-labels standard memory
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        if(x != ins->inputs()[0])
+            m.replace_instruction(ins, ins->get_operator(), x);
+    }
+    else if(name[0] == '@' or name == "capture" or name.rfind("mi355::", 0) == 0 or
+            (ins->get_operator().is_context_free() and ins->get_operator().output_alias({}) == 0))
+    {
+        // builtins, calibration taps, already lowered operators and views stay
+    }
+    else
+    {
+        MIGRAPHX_THROW("mi355: no kernel for operator '" + name + "'");
+    }
+}
+
+// ---- compile-time evaluation of constant subgraphs, on the device -----------------------------
+
+void fold_constants(module& m, context& ctx)
+{
+    migraphx::context gctx{ctx};
+    std::unordered_map<const instruction*, argument> known;
+    for(auto ins : all_instructions(m))
+    {
+        const auto name = ins->name();
+        if(name == "mi355::literal")
+        {
+            known[&*ins] = any_cast<device_literal>(ins->get_operator()).data;
+            continue;
+        }
+        if(name[0] == '@' or name == "capture" or name == "mi355::allocate" or
+           name == "mi355::copy_to_device" or name == "mi355::copy_from_device")
+            continue;
+        const bool kernel_op = name.rfind("mi355::", 0) == 0;
+        const auto& inputs   = ins->inputs();
+        const std::size_t n  = kernel_op ? inputs.size() - 1 : inputs.size();
+        if(inputs.empty())
+            continue;
+        bool all_known = true;
+        for(std::size_t i = 0; i < n; i++)
+            all_known = all_known and known.count(&*inputs[i]) > 0;
+        if(not all_known)
+            continue;
+        std::vector<argument> args;
+        for(std::size_t i = 0; i < n; i++)
+            args.push_back(known.at(&*inputs[i]));
+        if(not kernel_op)
+        {
+            // a view of a constant
+            if(ins->get_operator().is_context_free())
+                known[&*ins] = ins->get_operator().compute(ins->get_shape(), args);
+            continue;
+        }
+        if(inputs.back()->name() != "mi355::allocate")
+            continue;
+        args.push_back(allocate_device(inputs.back()->get_shape()));
+        argument result = ins->get_operator().compute(gctx, ins->get_shape(), args);
+        ctx.finish();
+        device_literal lit;
+        lit.data     = result;
+        known[&*ins] = result;
+        m.replace_instruction(ins, operation{lit}, std::vector<instruction_ref>{});
+    }
+}
+
+} // namespace
+
+void lowering::apply(module& m) const
+{
+    if(ctx == nullptr)
+        MIGRAPHX_THROW("mi355::lowering: no context");
+    // 1. fused patterns; what they absorb dies
+    for(auto ins : all_instructions(m))
+        fuse_quant_dot_dq(m, ins);
+    dead_code_elimination{}.apply(m);
+    // 2. everything else, one operator at a time
+    for(auto ins : all_instructions(m))
+        lower_instruction(m, ins);
+    dead_code_elimination{}.apply(m);
+    // 3. literals live in device memory
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "@literal")
+            continue;
+        device_literal lit;
+        lit.data = to_device(ins->get_literal().get_argument());
+        m.replace_instruction(ins, operation{lit}, std::vector<instruction_ref>{});
+    }
+    // 4. parameters and results cross the bus inside eval when asked to
+    if(offload_copy)
+    {
+        for(auto ins : all_instructions(m))
+        {
+            if(ins->name() != "@param" or ins->outputs().empty())
+                continue;
+            auto users = ins->outputs();
+            auto pos   = std::next(ins);
+            auto buf   = insert_allocation(m, pos, ins->get_shape());
+            auto dev   = m.insert_instruction(pos, operation{copy_to_device{}}, ins, buf);
+            for(auto u : users)
+                instruction::replace_argument(u, ins, dev);
+        }
+        auto last = std::prev(m.end());
+        if(last->name() == "@return")
+        {
+            auto rets = last->inputs();
+            for(auto r : rets)
+            {
+                auto h = m.insert_instruction(last, operation{copy_from_device{}}, r);
+                instruction::replace_argument(last, r, h);
+            }
+        }
+        else
+        {
+            m.add_instruction(operation{copy_from_device{}}, last);
+        }
+    }
+    // 5. constant subgraphs (weight quantization, column sums) run once, now
+    fold_constants(m, *ctx);
+}
+
+} // namespace mi355
+} // namespace migraphx

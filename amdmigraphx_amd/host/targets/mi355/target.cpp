@@ -1,0 +1,705 @@
+#include "device_ops.hpp"
+#include <migraphx/ops.hpp>
+#include <migraphx/passes.hpp>
+#include <migraphx/register_op.hpp>
+#include <migraphx/register_target.hpp>
+#include <hip/hip_runtime_api.h>
+#include <algorithm>
+
+namespace migraphx {
+namespace mi355 {
+
+namespace {
+
+void hip_check(hipError_t e, const char* what)
+{
+    if(e != hipSuccess)
+        MIGRAPHX_THROW(std::string("mi355: ") + what + " failed: " + hipGetErrorString(e));
+}
+
+void status_check(int st, const std::string& what)
+{
+    if(st != MI355_OK)
+        MIGRAPHX_THROW(what + ": " + mi355_status_string(st));
+}
+
+void* stream_of(migraphx::context& ctx) { return any_cast<context>(ctx).get_stream(); }
+
+void check_inputs(const std::vector<shape>& inputs, std::size_t n, const std::string& name)
+{
+    if(inputs.size() != n)
+        MIGRAPHX_THROW(name + ": expected " + std::to_string(n) + " arguments, got " +
+                       std::to_string(inputs.size()));
+}
+
+void check_standard(const shape& s, const std::string& name)
+{
+    if(not s.standard())
+        MIGRAPHX_THROW(name + ": tensor must be in standard layout");
+}
+
+} // namespace
+
+// ----------------------------------------------------------------- context, memory
+
+struct context::stream_holder
+{
+    hipStream_t s = nullptr;
+    stream_holder() { hip_check(hipStreamCreate(&s), "hipStreamCreate"); }
+    stream_holder(const stream_holder&) = delete;
+    stream_holder& operator=(const stream_holder&) = delete;
+    ~stream_holder()
+    {
+        if(s != nullptr)
+            (void)hipStreamDestroy(s);
+    }
+};
+
+context::context() : m_stream(std::make_shared<stream_holder>()) {}
+void* context::get_stream() const { return m_stream->s; }
+void context::finish() const { hip_check(hipStreamSynchronize(m_stream->s), "hipStreamSynchronize"); }
+
+argument allocate_device(const shape& s)
+{
+    void* p             = nullptr;
+    const std::size_t n = std::max<std::size_t>(s.bytes(), 16);
+    hip_check(hipMalloc(&p, n), "hipMalloc");
+    return {s, std::shared_ptr<char>(static_cast<char*>(p), [](char* q) { (void)hipFree(q); })};
+}
+
+argument to_device(const argument& host)
+{
+    // the device copy is dense in the host tensor's own memory order: same shape, same strides
+    argument d = allocate_device(host.get_shape());
+    if(host.get_shape().bytes() > 0)
+        hip_check(hipMemcpy(d.data(), host.data(), host.get_shape().bytes(), hipMemcpyHostToDevice),
+                  "hipMemcpy to device");
+    return d;
+}
+
+argument from_device(const argument& device)
+{
+    argument h{device.get_shape()};
+    if(device.get_shape().bytes() > 0)
+        hip_check(
+            hipMemcpy(h.data(), device.data(), device.get_shape().bytes(), hipMemcpyDeviceToHost),
+            "hipMemcpy from device");
+    return h;
+}
+
+// ----------------------------------------------------------------- helpers
+
+int to_mi355_type(shape::type_t t)
+{
+    switch(t)
+    {
+    case shape::int8_type: return MI355_I8;
+    case shape::uint8_type: return MI355_U8;
+    case shape::int32_type: return MI355_I32;
+    case shape::float_type: return MI355_F32;
+    case shape::half_type: return MI355_F16;
+    case shape::bf16_type: return MI355_BF16;
+    case shape::fp8e4m3fn_type: return MI355_FP8;
+    default: MIGRAPHX_THROW("mi355: no kernel takes " + shape::type_name(t));
+    }
+}
+
+matrix_view view_as_matrix(const shape& s)
+{
+    matrix_view v;
+    const std::size_t nd = s.ndim();
+    if(nd < 2)
+        return v;
+    v.rows     = static_cast<int64_t>(s.lens()[nd - 2]);
+    v.cols     = static_cast<int64_t>(s.lens()[nd - 1]);
+    v.stride_r = v.rows == 1 ? 0 : static_cast<int64_t>(s.strides()[nd - 2]);
+    v.stride_c = v.cols == 1 ? 0 : static_cast<int64_t>(s.strides()[nd - 1]);
+    if(v.cols == 1 or v.stride_c == 1)
+    {
+        v.trans = false;
+        v.ld    = v.rows == 1 ? v.cols : v.stride_r;
+        v.ok    = v.ld >= v.cols;
+    }
+    else if(v.rows == 1 or v.stride_r == 1)
+    {
+        v.trans = true;
+        v.ld    = v.stride_c;
+        v.ok    = v.ld >= v.rows;
+    }
+    if(not v.ok)
+        return v;
+    // leading dimensions must collapse into one batch stride
+    std::vector<std::pair<std::size_t, std::size_t>> dims; // (len, stride), length-1 dims dropped
+    for(std::size_t i = 0; i + 2 < nd; i++)
+    {
+        v.batch *= static_cast<int64_t>(s.lens()[i]);
+        if(s.lens()[i] > 1)
+            dims.emplace_back(s.lens()[i], s.strides()[i]);
+    }
+    for(std::size_t i = 0; i + 1 < dims.size(); i++)
+    {
+        if(dims[i].second != dims[i + 1].second * dims[i + 1].first)
+            v.ok = false;
+    }
+    v.batch_stride = dims.empty() ? 0 : static_cast<int64_t>(dims.back().second);
+    return v;
+}
+
+bool collapse_2d(const shape& s, int64_t& stride_r, int64_t& stride_c)
+{
+    const std::size_t nd = s.ndim();
+    if(nd == 0)
+        return false;
+    stride_c = s.lens()[nd - 1] == 1 ? 0 : static_cast<int64_t>(s.strides()[nd - 1]);
+    std::vector<std::pair<std::size_t, std::size_t>> dims;
+    for(std::size_t i = 0; i + 1 < nd; i++)
+    {
+        if(s.lens()[i] > 1)
+            dims.emplace_back(s.lens()[i], s.strides()[i]);
+    }
+    for(std::size_t i = 0; i + 1 < dims.size(); i++)
+    {
+        if(dims[i].second != dims[i + 1].second * dims[i + 1].first)
+            return false;
+    }
+    stride_r = dims.empty() ? 0 : static_cast<int64_t>(dims.back().second);
+    return true;
+}
+
+namespace {
+void rows_cols(const shape& s, int64_t& rows, int64_t& cols)
+{
+    cols = static_cast<int64_t>(s.lens().back());
+    rows = cols == 0 ? 0 : static_cast<int64_t>(s.elements()) / cols;
+}
+} // namespace
+
+// ----------------------------------------------------------------- memory operators
+
+argument allocate::compute(migraphx::context&, const shape&, const std::vector<argument>&) const
+{
+    if(buffer.empty())
+        MIGRAPHX_THROW("mi355::allocate: evaluated before finalize");
+    return buffer;
+}
+
+shape copy_to_device::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    if(inputs[0] != inputs[1])
+        MIGRAPHX_THROW("mi355::copy_to_device: host and device shapes differ");
+    return inputs[1];
+}
+
+argument copy_to_device::compute(migraphx::context& ctx,
+                                 const shape&,
+                                 const std::vector<argument>& args) const
+{
+    const auto n = args[0].get_shape().bytes();
+    if(n > 0)
+        hip_check(hipMemcpyAsync(args[1].data(),
+                                 args[0].data(),
+                                 n,
+                                 hipMemcpyHostToDevice,
+                                 static_cast<hipStream_t>(stream_of(ctx))),
+                  "hipMemcpyAsync to device");
+    return args[1];
+}
+
+shape copy_from_device::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 1, name());
+    return inputs[0];
+}
+
+argument copy_from_device::compute(migraphx::context& ctx,
+                                   const shape& out,
+                                   const std::vector<argument>& args) const
+{
+    argument h{out};
+    auto s = static_cast<hipStream_t>(stream_of(ctx));
+    if(out.bytes() > 0)
+        hip_check(hipMemcpyAsync(h.data(), args[0].data(), out.bytes(), hipMemcpyDeviceToHost, s),
+                  "hipMemcpyAsync from device");
+    hip_check(hipStreamSynchronize(s), "hipStreamSynchronize");
+    return h;
+}
+
+// ----------------------------------------------------------------- GEMM operators
+
+shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, expected_inputs(), name());
+    auto s = op::quant_dot{}.compute_shape({inputs[0], inputs[1]});
+    if(inputs[0].type() != shape::int8_type and inputs[0].type() != shape::fp8e4m3fn_type)
+        MIGRAPHX_THROW("mi355::quant_dot: kernels take int8 or fp8e4m3fn operands, not " +
+                       inputs[0].type_string());
+    if(not view_as_matrix(inputs[0]).ok or not view_as_matrix(inputs[1]).ok)
+        MIGRAPHX_THROW("mi355::quant_dot: operand strides are neither row-major nor transposed");
+    if(not dequant and out_type != s.type())
+        MIGRAPHX_THROW("mi355::quant_dot: output type must be " + s.type_string());
+    if(dequant)
+    {
+        if(out_type != shape::float_type and out_type != shape::half_type and
+           out_type != shape::bf16_type)
+            MIGRAPHX_THROW("mi355::quant_dot: dequantized output must be float, half or bf16");
+        if(inputs[2].type() != shape::float_type or inputs[3].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::quant_dot: scales must be float");
+        if((zp_a != 0 or zp_b != 0) and inputs[0].type() != shape::int8_type)
+            MIGRAPHX_THROW("mi355::quant_dot: zero points need int8 operands");
+    }
+    shape out{out_type, s.lens()};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::quant_dot: output buffer has the wrong shape");
+    return out;
+}
+
+argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto va = view_as_matrix(args[0].get_shape());
+    const auto vb = view_as_matrix(args[1].get_shape());
+    mi355_quant_dot_desc d{};
+    d.m        = va.rows;
+    d.k        = va.cols;
+    d.n        = vb.cols;
+    d.trans_a  = va.trans;
+    d.trans_b  = vb.trans;
+    d.lda      = va.ld;
+    d.ldb      = vb.ld;
+    d.ldc      = d.n;
+    d.batch    = va.batch;
+    d.stride_a = va.batch_stride;
+    d.stride_b = vb.batch_stride;
+    d.stride_c = d.m * d.n;
+    d.in_type  = to_mi355_type(args[0].get_shape().type());
+    d.out_type = to_mi355_type(out_type);
+    d.dequant  = dequant ? 1 : 0;
+    d.scale_a_mode = static_cast<int32_t>(scale_a_mode);
+    d.scale_b_mode = static_cast<int32_t>(scale_b_mode);
+    d.zp_a         = static_cast<int32_t>(zp_a);
+    d.zp_b         = static_cast<int32_t>(zp_b);
+    std::size_t next = 2;
+    const float* sa  = nullptr;
+    const float* sb  = nullptr;
+    if(dequant)
+    {
+        sa = reinterpret_cast<const float*>(args[next++].data());
+        sb = reinterpret_cast<const float*>(args[next++].data());
+    }
+    const int32_t* colsum_b = zp_a != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
+    const int32_t* rowsum_a = zp_b != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
+    if((zp_a != 0 or zp_b != 0) and d.batch != 1)
+        MIGRAPHX_THROW("mi355::quant_dot: zero points with batched operands are not supported");
+    status_check(mi355_quant_dot(&d,
+                                 args[0].data(),
+                                 args[1].data(),
+                                 args.back().data(),
+                                 sa,
+                                 sb,
+                                 colsum_b,
+                                 rowsum_a,
+                                 stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+shape colsum::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    const auto v = view_as_matrix(inputs[0]);
+    if(not v.ok or v.batch != 1 or inputs[0].type() != shape::int8_type)
+        MIGRAPHX_THROW("mi355::colsum: needs one int8 matrix");
+    shape out{shape::int32_type, {static_cast<std::size_t>(v.cols)}};
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::colsum: output buffer has the wrong shape");
+    return out;
+}
+
+argument colsum::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto v = view_as_matrix(args[0].get_shape());
+    status_check(mi355_colsum_i8(args[0].data(),
+                                 v.rows,
+                                 v.cols,
+                                 v.ld,
+                                 v.trans,
+                                 reinterpret_cast<int32_t*>(args[1].data()),
+                                 stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape rowsum::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    const auto v = view_as_matrix(inputs[0]);
+    if(not v.ok or v.batch != 1 or inputs[0].type() != shape::int8_type)
+        MIGRAPHX_THROW("mi355::rowsum: needs one int8 matrix");
+    shape out{shape::int32_type, {static_cast<std::size_t>(v.rows)}};
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::rowsum: output buffer has the wrong shape");
+    return out;
+}
+
+argument rowsum::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto v = view_as_matrix(args[0].get_shape());
+    status_check(mi355_rowsum_i8(args[0].data(),
+                                 v.rows,
+                                 v.cols,
+                                 v.ld,
+                                 v.trans,
+                                 reinterpret_cast<int32_t*>(args[1].data()),
+                                 stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape dot::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    auto s = op::dot{}.compute_shape({inputs[0], inputs[1]});
+    to_mi355_type(s.type());
+    if(s.type() != shape::float_type and s.type() != shape::half_type and s.type() != shape::bf16_type)
+        MIGRAPHX_THROW("mi355::dot: float, half or bf16 only");
+    // any strides are fine inside a matrix; the batch dimensions must collapse
+    for(int i = 0; i < 2; i++)
+    {
+        auto v = view_as_matrix(inputs[i].ndim() == 2 ? inputs[i] : inputs[i]);
+        int64_t sr = 0;
+        int64_t sc = 0;
+        std::vector<std::size_t> bl(inputs[i].lens().begin(), inputs[i].lens().end() - 1);
+        std::vector<std::size_t> bs(inputs[i].strides().begin(), inputs[i].strides().end() - 1);
+        if(bl.size() > 1 and not collapse_2d(shape{s.type(), bl, bs}, sr, sc))
+            MIGRAPHX_THROW("mi355::dot: batch dimensions do not collapse into one stride");
+        (void)v;
+    }
+    if(inputs.back() != s)
+        MIGRAPHX_THROW("mi355::dot: output buffer has the wrong shape");
+    return s;
+}
+
+argument dot::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const auto& sa       = args[0].get_shape();
+    const auto& sb       = args[1].get_shape();
+    const std::size_t nd = sa.ndim();
+    const auto m         = static_cast<int64_t>(sa.lens()[nd - 2]);
+    const auto k         = static_cast<int64_t>(sa.lens()[nd - 1]);
+    const auto n         = static_cast<int64_t>(sb.lens()[nd - 1]);
+    int64_t batch        = 1;
+    for(std::size_t i = 0; i + 2 < nd; i++)
+        batch *= static_cast<int64_t>(sa.lens()[i]);
+    auto batch_stride = [&](const shape& s) {
+        int64_t r = 0;
+        for(std::size_t i = 0; i + 2 < nd; i++)
+        {
+            if(s.lens()[i] > 1)
+                r = static_cast<int64_t>(s.strides()[i]);
+        }
+        return r;
+    };
+    status_check(mi355_dot(args[0].data(),
+                           args[1].data(),
+                           args[2].data(),
+                           to_mi355_type(out.type()),
+                           m,
+                           n,
+                           k,
+                           static_cast<int64_t>(sa.strides()[nd - 2]),
+                           static_cast<int64_t>(sa.strides()[nd - 1]),
+                           static_cast<int64_t>(sb.strides()[nd - 2]),
+                           static_cast<int64_t>(sb.strides()[nd - 1]),
+                           n,
+                           batch,
+                           batch_stride(sa),
+                           batch_stride(sb),
+                           m * n,
+                           stream_of(ctx)),
+                 name());
+    return args[2];
+}
+
+shape w4a16_gemm::compute_shape(const std::vector<shape>& inputs) const
+{
+    const std::size_t expect = zp_mode == MI355_W4_ZP_SCALAR ? 4 : 5;
+    check_inputs(inputs, expect, name());
+    const auto& a = inputs[0];
+    const auto& w = inputs[1];
+    const auto& s = inputs[2];
+    if(a.type() != shape::half_type or s.type() != shape::half_type or w.type() != shape::uint8_type)
+        MIGRAPHX_THROW("mi355::w4a16_gemm: needs half activations and scales, uint8 packed weights");
+    if(a.ndim() != 2 or w.ndim() != 2 or a.strides()[1] != 1 or not w.standard() or not s.standard())
+        MIGRAPHX_THROW("mi355::w4a16_gemm: needs 2-D row-major operands");
+    const auto k = a.lens()[1];
+    const auto n = w.lens()[0];
+    if(w.lens()[1] * 2 != k or group <= 0 or k % group != 0 or s.elements() != n * (k / group))
+        MIGRAPHX_THROW("mi355::w4a16_gemm: operand dimensions do not fit");
+    shape out{shape::half_type, {a.lens()[0], n}};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::w4a16_gemm: output buffer has the wrong shape");
+    return out;
+}
+
+argument w4a16_gemm::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const auto& a    = args[0].get_shape();
+    const void* zp   = zp_mode == MI355_W4_ZP_SCALAR ? nullptr : args[3].data();
+    const int64_t m  = static_cast<int64_t>(a.lens()[0]);
+    const int64_t k  = static_cast<int64_t>(a.lens()[1]);
+    const int64_t n  = static_cast<int64_t>(out.lens()[1]);
+    const int64_t lda = m == 1 ? k : static_cast<int64_t>(a.strides()[0]);
+    status_check(mi355_w4a16_gemm(args[0].data(),
+                                  lda,
+                                  args[1].data(),
+                                  args[2].data(),
+                                  zp,
+                                  static_cast<int32_t>(zp_mode),
+                                  static_cast<int32_t>(zp_scalar),
+                                  args.back().data(),
+                                  n,
+                                  m,
+                                  n,
+                                  k,
+                                  group,
+                                  stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+// ----------------------------------------------------------------- pointwise operators
+
+shape quantizelinear::compute_shape(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() != 3 and inputs.size() != 4)
+        MIGRAPHX_THROW("mi355::quantizelinear: expected 3 or 4 arguments");
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != inputs[1].type())
+        MIGRAPHX_THROW("mi355::quantizelinear: Scales and input must be the same type");
+    int64_t sr = 0;
+    int64_t sc = 0;
+    for(std::size_t i = 1; i + 1 < inputs.size(); i++)
+    {
+        if(inputs[i].lens() != inputs[0].lens() or not collapse_2d(inputs[i], sr, sc))
+            MIGRAPHX_THROW("mi355::quantizelinear: parameter strides do not collapse to two");
+    }
+    if(inputs.size() == 4 and inputs[2].type() != out_type)
+        MIGRAPHX_THROW("mi355::quantizelinear: zero point type differs from the output type");
+    shape out{out_type, inputs[0].lens()};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::quantizelinear: output buffer has the wrong shape");
+    return out;
+}
+
+argument
+quantizelinear::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(out, rows, cols);
+    int64_t s_sr = 0, s_sc = 0, z_sr = 0, z_sc = 0;
+    collapse_2d(args[1].get_shape(), s_sr, s_sc);
+    const void* zp = nullptr;
+    if(args.size() == 4)
+    {
+        zp = args[2].data();
+        collapse_2d(args[2].get_shape(), z_sr, z_sc);
+    }
+    status_check(mi355_quantizelinear(args[0].data(),
+                                      to_mi355_type(args[0].get_shape().type()),
+                                      args[1].data(),
+                                      s_sr,
+                                      s_sc,
+                                      zp,
+                                      z_sr,
+                                      z_sc,
+                                      args.back().data(),
+                                      to_mi355_type(out.type()),
+                                      rows,
+                                      cols,
+                                      stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+shape dequantizelinear::compute_shape(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() != 3 and inputs.size() != 4)
+        MIGRAPHX_THROW("mi355::dequantizelinear: expected 3 or 4 arguments");
+    check_standard(inputs[0], name());
+    int64_t sr = 0;
+    int64_t sc = 0;
+    for(std::size_t i = 1; i + 1 < inputs.size(); i++)
+    {
+        if(inputs[i].lens() != inputs[0].lens() or not collapse_2d(inputs[i], sr, sc))
+            MIGRAPHX_THROW("mi355::dequantizelinear: parameter strides do not collapse to two");
+    }
+    if(inputs.size() == 4 and inputs[2].type() != inputs[0].type())
+        MIGRAPHX_THROW("mi355::dequantizelinear: Zero point and input should be the same type.");
+    shape out{inputs[1].type(), inputs[0].lens()};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::dequantizelinear: output buffer has the wrong shape");
+    return out;
+}
+
+argument
+dequantizelinear::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(out, rows, cols);
+    int64_t s_sr = 0, s_sc = 0, z_sr = 0, z_sc = 0;
+    collapse_2d(args[1].get_shape(), s_sr, s_sc);
+    const void* zp = nullptr;
+    if(args.size() == 4)
+    {
+        zp = args[2].data();
+        collapse_2d(args[2].get_shape(), z_sr, z_sc);
+    }
+    status_check(mi355_dequantizelinear(args[0].data(),
+                                        to_mi355_type(args[0].get_shape().type()),
+                                        args[1].data(),
+                                        to_mi355_type(args[1].get_shape().type()),
+                                        s_sr,
+                                        s_sc,
+                                        zp,
+                                        z_sr,
+                                        z_sc,
+                                        args.back().data(),
+                                        rows,
+                                        cols,
+                                        stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+shape unpack_int4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    auto out = op::unpack_int4{}.compute_shape({inputs[0]});
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::unpack_int4: output buffer has the wrong shape");
+    return out;
+}
+
+argument unpack_int4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_unpack_int4(args[0].data(),
+                                   args[1].data(),
+                                   args[0].get_shape().type() == shape::int8_type,
+                                   rows,
+                                   cols,
+                                   stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape pack_int4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    auto out = op::pack_int4{}.compute_shape({inputs[0]});
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::pack_int4: output buffer has the wrong shape");
+    return out;
+}
+
+argument pack_int4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_pack_int4(args[0].data(),
+                                 args[1].data(),
+                                 args[0].get_shape().type() == shape::int8_type,
+                                 rows,
+                                 cols,
+                                 stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape convert::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    shape out{target_type, inputs[0].lens()};
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::convert: output buffer has the wrong shape");
+    return out;
+}
+
+argument convert::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    status_check(mi355_convert(args[0].data(),
+                               to_mi355_type(args[0].get_shape().type()),
+                               args[1].data(),
+                               to_mi355_type(out.type()),
+                               static_cast<int64_t>(out.elements()),
+                               stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape contiguous::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    if(inputs[0].ndim() > MI355_MAX_DIMS)
+        MIGRAPHX_THROW("mi355::contiguous: too many dimensions");
+    shape out{inputs[0].type(), inputs[0].lens()};
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::contiguous: output buffer has the wrong shape");
+    return out;
+}
+
+argument contiguous::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto& s = args[0].get_shape();
+    std::vector<int64_t> lens(s.lens().begin(), s.lens().end());
+    std::vector<int64_t> strides(s.strides().begin(), s.strides().end());
+    status_check(mi355_contiguous(args[0].data(),
+                                  args[1].data(),
+                                  static_cast<int32_t>(s.type_size()),
+                                  static_cast<int32_t>(s.ndim()),
+                                  lens.data(),
+                                  strides.data(),
+                                  stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+// ----------------------------------------------------------------- target
+
+std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_options& options) const
+{
+    auto& ctx = any_cast<context>(gctx);
+    return {simplify_qdq{},
+            dead_code_elimination{},
+            lowering{&ctx, options.offload_copy},
+            dead_code_elimination{}};
+}
+
+} // namespace mi355
+
+MIGRAPHX_REGISTER_OP(mi355::allocate);
+MIGRAPHX_REGISTER_OP(mi355::device_literal);
+MIGRAPHX_REGISTER_OP(mi355::copy_to_device);
+MIGRAPHX_REGISTER_OP(mi355::copy_from_device);
+MIGRAPHX_REGISTER_OP(mi355::quant_dot);
+MIGRAPHX_REGISTER_OP(mi355::colsum);
+MIGRAPHX_REGISTER_OP(mi355::rowsum);
+MIGRAPHX_REGISTER_OP(mi355::dot);
+MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
+MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
+MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);
+MIGRAPHX_REGISTER_OP(mi355::unpack_int4);
+MIGRAPHX_REGISTER_OP(mi355::pack_int4);
+MIGRAPHX_REGISTER_OP(mi355::convert);
+MIGRAPHX_REGISTER_OP(mi355::contiguous);
+MIGRAPHX_REGISTER_TARGET(mi355::target);
+
+} // namespace migraphx
