@@ -74,15 +74,9 @@ inline float widen(uint16_t h)
     {
         if(man == 0)
             return bits_float(sign);
-        // normalise the subnormal
-        int k = 0;
-        while((man & (1u << MB)) == 0)
-        {
-            man <<= 1;
-            k++;
-        }
-        man &= (1u << MB) - 1;
-        return bits_float(sign | uint32_t(1 - k - bias + 127) << 23 | (man << (23 - MB)));
+        // subnormal: man * 2^(1 - bias - MB); for bf16 this is a float subnormal
+        const float v = std::ldexp(static_cast<float>(man), 1 - bias - MB);
+        return sign != 0 ? -v : v;
     }
     return bits_float(sign | uint32_t(e - bias + 127) << 23 | (man << (23 - MB)));
 }

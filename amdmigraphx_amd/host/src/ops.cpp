@@ -273,7 +273,7 @@ argument reshape::compute(const shape& out, const std::vector<argument>& args) c
     const auto& in = args.at(0);
     if(in.get_shape().standard())
         return in.reshape(out);
-    return contiguous{}.compute(out.with_lens(in.get_shape().lens()), args).reshape(out);
+    return contiguous{}.compute(shape{out.type(), in.get_shape().lens()}, args).reshape(out);
 }
 
 shape unsqueeze::compute_shape(const std::vector<shape>& inputs) const

@@ -629,6 +629,22 @@ instruction_ref matmulnbits(module& m,
     }
     auto dq = m.add_instruction(make_op("dequantizelinear"), bq, sc, z);
     auto bt = m.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), dq);
+    // numpy matmul rules for A (the reference's matmul helper, src/onnx/parse_matmul.cpp): a vector
+    // is a one-row matrix, leading dimensions of A broadcast over B
+    const auto a_lens = a->get_shape().lens();
+    if(a_lens.size() == 1)
+    {
+        auto a2 = m.add_instruction(make_op("unsqueeze", {{"axes", {0}}}), a);
+        auto d  = m.add_instruction(make_op("dot"), a2, bt);
+        return m.add_instruction(make_op("squeeze", {{"axes", {0}}}), d);
+    }
+    if(a_lens.size() > 2)
+    {
+        std::vector<std::size_t> bl(a_lens.begin(), a_lens.end() - 2);
+        bl.push_back(k);
+        bl.push_back(n);
+        bt = m.add_instruction(make_op("multibroadcast", {{"out_lens", bl}}), bt);
+    }
     return m.add_instruction(make_op("dot"), a, bt);
 }
 

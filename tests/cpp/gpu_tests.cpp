@@ -1,0 +1,373 @@
+// GPU tests of the mi355 target: every program is compiled for the CPU oracle target and for
+// "mi355" from the same host inputs, as the reference's test/verify/run_verify.cpp:139-226 does
+// with `ref` and `gpu`.  Integer results and float results whose arithmetic the kernels reproduce
+// exactly (int8 quant_dot with the dequantize epilogue, the int4 chain, float dot) must be
+// bit-identical; fp8 results use the tolerances stated at the test.
+#include "common.hpp"
+#include "oracle_target.hpp"
+#include "test.hpp"
+#include <fstream>
+
+using namespace testutil;
+using migraphx::shape;
+
+static void expect_same(const program& p, const migraphx::parameter_map& params)
+{
+    auto want = run_on("oracle", p, params);
+    auto got  = run_on("mi355", p, params);
+    EXPECT(want.size() == got.size());
+    for(std::size_t i = 0; i < want.size(); i++)
+        EXPECT(same_bytes(got[i], want[i]));
+    // parameters and results copied inside eval give the same answer
+    auto got2 = run_on("mi355", p, params, true);
+    for(std::size_t i = 0; i < want.size(); i++)
+        EXPECT(same_bytes(got2[i], want[i]));
+}
+
+static bool has_op(const program& p, const std::string& name)
+{
+    return count_ops(*p.get_main_module(), name) > 0;
+}
+
+// BASELINE config 1: X fp32 [M, K] -> quantizelinear (scale 1/32, zp 0) -> int8; W int8 literal
+// with per-output-channel scales; dot of the two dequantized tensors
+static program qdq_matmul(std::size_t m,
+                          std::size_t k,
+                          std::size_t n,
+                          bool weight_nk,
+                          int zp_x,
+                          int zp_w,
+                          shape::type_t model_type,
+                          unsigned seed)
+{
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{model_type, {m, k}});
+    auto xin = x;
+    if(model_type != shape::float_type)
+        xin = mm->add_instruction(make_op("convert", {{"target_type", shape::float_type}}), x);
+    auto sx  = mm->add_literal(1.0f / 32);
+    auto zx  = mm->add_literal(static_cast<std::int8_t>(zp_x));
+    auto q   = add_quantize_op(*mm, "quantizelinear", xin, sx, zx);
+    auto dx  = add_quantize_op(*mm, "dequantizelinear", q, sx, zx);
+    std::vector<std::size_t> wl = weight_nk ? std::vector<std::size_t>{n, k} : std::vector<std::size_t>{k, n};
+    auto w  = mm->add_literal(literal{shape{shape::int8_type, wl}, uniform_ints<int>(k * n, -127, 127, seed)});
+    auto sw = mm->add_literal(literal{shape{shape::float_type, {n}}, uniform_floats(n, 0.001f, 0.01f, seed + 1)});
+    auto zw = mm->add_literal(literal{shape{shape::int8_type, {n}}, std::vector<int>(n, zp_w)});
+    const std::size_t axis = weight_nk ? 0 : 1;
+    auto swb = mm->add_instruction(make_op("broadcast", {{"axis", axis}, {"out_lens", wl}}), sw);
+    auto zwb = mm->add_instruction(make_op("broadcast", {{"axis", axis}, {"out_lens", wl}}), zw);
+    instruction_ref dw = mm->add_instruction(make_op("dequantizelinear"), w, swb, zwb);
+    if(weight_nk)
+        dw = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), dw);
+    if(model_type != shape::float_type)
+    {
+        dx = mm->add_instruction(make_op("convert", {{"target_type", model_type}}), dx);
+        dw = mm->add_instruction(make_op("convert", {{"target_type", model_type}}), dw);
+    }
+    mm->add_return({mm->add_instruction(make_op("dot"), dx, dw)});
+    return p;
+}
+
+TEST_CASE(config1_qdq_matmul)
+{
+    const std::size_t m = 256, k = 1024, n = 1024;
+    auto p = qdq_matmul(m, k, n, false, 0, 0, shape::float_type, 0);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(has_op(p, "quant_dot") and not has_op(p, "dot"));
+    argument x{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 0)};
+    expect_same(p, {{"x", x}});
+    // the target runs simplify_qdq itself: the fake-quantized graph compiles to the same program
+    auto raw  = qdq_matmul(m, k, n, false, 0, 0, shape::float_type, 0);
+    auto got  = run_on("mi355", raw, {{"x", x}});
+    auto want = run_on("oracle", p, {{"x", x}});
+    EXPECT(same_bytes(got[0], want[0]));
+    // one fused kernel instruction, nothing left of the zero-point or scale arithmetic
+    program c = raw;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::quant_dot") == 1);
+    EXPECT(count_ops(*c.get_main_module(), "mi355::quantizelinear") == 1);
+    EXPECT(not has_op(c, "mul") and not has_op(c, "dequantizelinear") and not has_op(c, "quant_dot"));
+}
+
+TEST_CASE(qdq_matmul_transposed_weight)
+{
+    const std::size_t m = 96, k = 320, n = 208;
+    auto p = qdq_matmul(m, k, n, true, 0, 0, shape::float_type, 3);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    argument x{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 4)};
+    expect_same(p, {{"x", x}});
+}
+
+TEST_CASE(qdq_matmul_zero_points)
+{
+    const std::size_t m = 64, k = 256, n = 128;
+    for(auto zp : {std::pair<int, int>{3, 0}, {0, -5}, {3, -5}, {-128, 127}})
+    {
+        auto p = qdq_matmul(m, k, n, false, zp.first, zp.second, shape::float_type, 5);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        argument x{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.5f, 6)};
+        expect_same(p, {{"x", x}});
+        program c = p;
+        c.compile(migraphx::make_target("mi355"));
+        // the three extra GEMMs of the zero-point terms became column / row sums
+        EXPECT(count_ops(*c.get_main_module(), "mi355::quant_dot") == 1);
+        EXPECT(not has_op(c, "add") and not has_op(c, "sub"));
+    }
+}
+
+TEST_CASE(qdq_matmul_fp16_model)
+{
+    const std::size_t m = 48, k = 192, n = 80;
+    auto p = qdq_matmul(m, k, n, false, 0, 0, shape::half_type, 7);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(p.get_output_shapes().front().type() == shape::half_type);
+    argument x{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 8)};
+    expect_same(p, {{"x", x}});
+}
+
+TEST_CASE(bare_quant_dot_views)
+{
+    // the shapes of test/verify/test_batch_quant_dot_{1..5}.cpp and test_quant_dot_3args_*:
+    // batches, transposed A, transposed B, both
+    for(int variant = 0; variant < 4; variant++)
+    {
+        const bool ta = (variant & 1) != 0;
+        const bool tb = (variant & 2) != 0;
+        const std::size_t b0 = 3, b1 = 2, m = 24, k = 40, n = 56;
+        program p;
+        auto* mm = p.get_main_module();
+        shape sa{shape::int8_type, ta ? std::vector<std::size_t>{b0, b1, k, m} : std::vector<std::size_t>{b0, b1, m, k}};
+        shape sb{shape::int8_type, tb ? std::vector<std::size_t>{b0, b1, n, k} : std::vector<std::size_t>{b0, b1, k, n}};
+        instruction_ref a = mm->add_parameter("a", sa);
+        instruction_ref b = mm->add_parameter("b", sb);
+        if(ta)
+            a = mm->add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), a);
+        if(tb)
+            b = mm->add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), b);
+        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b)});
+        argument aa{sa, uniform_ints<int>(sa.elements(), -128, 127, 10 + variant)};
+        argument ba{sb, uniform_ints<int>(sb.elements(), -128, 127, 20 + variant)};
+        expect_same(p, {{"a", aa}, {"b", ba}});
+    }
+}
+
+TEST_CASE(fp8_quantized_matmul)
+{
+    // BASELINE config 3 in small: activations and weights quantized to fp8 e4m3fn with amax-based
+    // per-tensor scales, fp32 accumulation, bf16 output.  The fp8 MFMA instructions add each
+    // group of 128 products with about 20 bits below the group's largest term, so the result is
+    // not bit-identical to the oracle's exact sum: the error must stay within 1e-3 of the
+    // output's RMS, and no element may be off by more than 2^-8 of the largest output (two bf16
+    // steps at that magnitude).
+    const std::size_t m = 128, k = 512, n = 256;
+    auto xv = normal_floats(m * k, 1.0f, 30);
+    auto wv = normal_floats(k * n, 0.02f, 31);
+    float ax = 0, aw = 0;
+    for(float v : xv)
+        ax = std::max(ax, std::fabs(v));
+    for(float v : wv)
+        aw = std::max(aw, std::fabs(v));
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, wv});
+    auto sx  = mm->add_literal(ax / 448.0f);
+    auto sw  = mm->add_literal(aw / 448.0f);
+    auto z   = mm->add_literal(literal{shape{shape::fp8e4m3fn_type}, std::vector<float>{0.0f}});
+    auto qx  = add_quantize_op(*mm, "quantizelinear", x, sx, z);
+    auto dx  = add_quantize_op(*mm, "dequantizelinear", qx, sx, z);
+    auto qw  = add_quantize_op(*mm, "quantizelinear", w, sw, z);
+    auto dw  = add_quantize_op(*mm, "dequantizelinear", qw, sw, z);
+    auto d   = mm->add_instruction(make_op("dot"), dx, dw);
+    mm->add_return({mm->add_instruction(make_op("convert", {{"target_type", shape::bf16_type}}), d)});
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(has_op(p, "quant_dot") and not has_op(p, "dot"));
+    argument xa{shape{shape::float_type, {m, k}}, xv};
+    auto want = run_on("oracle", p, {{"x", xa}});
+    auto got  = run_on("mi355", p, {{"x", xa}});
+    EXPECT(got[0].get_shape().type() == shape::bf16_type);
+    auto a = got[0].to_vector<double>();
+    auto b = want[0].to_vector<double>();
+    double num = 0, den = 0, peak = 0, worst = 0;
+    for(std::size_t i = 0; i < a.size(); i++)
+    {
+        num += (a[i] - b[i]) * (a[i] - b[i]);
+        den += b[i] * b[i];
+        peak  = std::max(peak, std::fabs(b[i]));
+        worst = std::max(worst, std::fabs(a[i] - b[i]));
+    }
+    EXPECT(std::sqrt(num / den) < 1e-3);
+    EXPECT(worst <= peak / 256);
+    // the weight was quantized once, at compile time
+    program c = p;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::quantizelinear") == 1);
+    EXPECT(count_ops(*c.get_main_module(), "mi355::quant_dot") == 1);
+    EXPECT(not has_op(c, "mi355::convert"));
+}
+
+// the MatMulNBits graph with random data (BASELINE config 4 layout: block 128, zero point 8)
+static program
+matmulnbits_program(std::size_t m, std::size_t k, std::size_t n, std::size_t blk, bool with_zp, shape::type_t ft, unsigned seed)
+{
+    const std::size_t nblk = (k + blk - 1) / blk;
+    program p;
+    auto* mm = p.get_main_module();
+    auto a   = mm->add_parameter("a", shape{ft, {m, k}});
+    auto b   = mm->add_literal(literal{shape{shape::uint8_type, {n, nblk, blk / 2}}, uniform_ints<int>(n * nblk * blk / 2, 0, 255, seed)});
+    auto s   = mm->add_literal(literal{shape{ft, {n * nblk}}, uniform_floats(n * nblk, 0.005f, 0.02f, seed + 1)});
+    auto zp  = mm->end();
+    if(with_zp)
+        zp = mm->add_literal(literal{shape{shape::uint8_type, {n * ((nblk + 1) / 2)}}, uniform_ints<int>(n * ((nblk + 1) / 2), 0, 255, seed + 2)});
+    mm->add_return({migraphx::op::builder::matmulnbits(*mm, a, b, s, zp, n, k, blk)});
+    return p;
+}
+
+TEST_CASE(int4_weight_only_gemv)
+{
+    // M = 1: the streaming kernel; the graph collapses into one instruction
+    for(auto kn : {std::pair<std::size_t, std::size_t>{4096, 512}, {2048, 1000}})
+    {
+        auto p = matmulnbits_program(1, kn.first, kn.second, 128, false, shape::half_type, 40);
+        argument a{shape{shape::half_type, {1, kn.first}}, normal_floats(kn.first, 1.0f, 41)};
+        expect_same(p, {{"a", a}});
+        program c = p;
+        c.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+        EXPECT(not has_op(c, "mi355::dequantizelinear") and not has_op(c, "mi355::unpack_int4") and
+               not has_op(c, "mi355::dot"));
+    }
+}
+
+TEST_CASE(int4_weight_only_gemm_small_batch)
+{
+    for(std::size_t m : {2, 16})
+    {
+        auto p = matmulnbits_program(m, 1024, 384, 128, false, shape::half_type, 50);
+        argument a{shape{shape::half_type, {m, 1024}}, normal_floats(m * 1024, 1.0f, 51)};
+        expect_same(p, {{"a", a}});
+    }
+    // per-block zero points packed two to a byte, block size 32
+    auto p = matmulnbits_program(4, 512, 96, 32, true, shape::half_type, 52);
+    argument a{shape{shape::half_type, {4, 512}}, normal_floats(4 * 512, 1.0f, 53)};
+    expect_same(p, {{"a", a}});
+    program c = p;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+}
+
+TEST_CASE(int4_general_path)
+{
+    // float activations, or K that is not a multiple of the block: no fused kernel, the chain
+    // runs operator by operator (the weight side once, at compile time) and still matches
+    auto p = matmulnbits_program(5, 200, 48, 64, true, shape::float_type, 60);
+    argument a{shape{shape::float_type, {5, 200}}, normal_floats(5 * 200, 1.0f, 61)};
+    expect_same(p, {{"a", a}});
+    program c = p;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::dot") == 1);
+    EXPECT(not has_op(c, "mi355::dequantizelinear")); // folded into a literal
+}
+
+TEST_CASE(quantize_int4_program)
+{
+    const std::size_t m = 8, k = 64, n = 96;
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, uniform_floats(k * n, -0.5f, 1.0f, 70)});
+    mm->add_return({mm->add_instruction(make_op("dot"), x, w)});
+    migraphx::quantize_int4_weights(p);
+    argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 71)};
+    expect_same(p, {{"x", xa}});
+}
+
+TEST_CASE(int8_calibration_on_device)
+{
+    const std::size_t m = 32, k = 128, n = 64;
+    program fp;
+    auto* mm = fp.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, normal_floats(k * n, 0.05f, 80)});
+    mm->add_return({mm->add_instruction(make_op("dot"), x, w)});
+    argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 81)};
+    program on_oracle = fp;
+    program on_device = fp;
+    migraphx::quantize_int8(on_oracle, migraphx::make_target("oracle"), {{{"x", xa}}});
+    migraphx::quantize_int8(on_device, migraphx::make_target("mi355"), {{{"x", xa}}});
+    // same captured ranges, hence the same quantized program
+    EXPECT(on_oracle == on_device);
+    expect_same(on_device, {{"x", xa}});
+    // and the float program itself runs on the device, bit-exact with the oracle's dot
+    expect_same(fp, {{"x", xa}});
+}
+
+TEST_CASE(standalone_operators)
+{
+    // operators of the path outside any fused pattern
+    const std::size_t r = 37, c = 50;
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {r, c}});
+    auto s   = mm->add_literal(literal{shape{shape::float_type, {c}}, uniform_floats(c, 0.01f, 0.1f, 90)});
+    auto z   = mm->add_literal(literal{shape{shape::int8_type, {c}}, uniform_ints<int>(c, -10, 10, 91)});
+    std::vector<std::size_t> lens = {r, c};
+    auto sb  = mm->add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", lens}}), s);
+    auto zb  = mm->add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", lens}}), z);
+    auto q   = mm->add_instruction(make_op("quantizelinear"), x, sb, zb);
+    auto dq  = mm->add_instruction(make_op("dequantizelinear"), q, sb, zb);
+    auto h   = mm->add_instruction(make_op("convert", {{"target_type", shape::half_type}}), dq);
+    auto t   = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), q);
+    auto ct  = mm->add_instruction(make_op("contiguous"), t);
+    auto pk  = mm->add_instruction(make_op("pack_int4"), q);
+    auto un  = mm->add_instruction(make_op("unpack_int4"), pk);
+    mm->add_return({q, h, ct, pk, un});
+    argument xa{shape{shape::float_type, {r, c}}, normal_floats(r * c, 1.0f, 92)};
+    expect_same(p, {{"x", xa}});
+}
+
+TEST_CASE(no_host_fallback)
+{
+    // an operator without a kernel stops compilation instead of running on the host
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {4, 4}});
+    mm->add_return({mm->add_instruction(make_op("add"), x, x)});
+    bool thrown = false;
+    try
+    {
+        p.compile(migraphx::make_target("mi355"));
+    }
+    catch(const migraphx::exception& e)
+    {
+        thrown = std::string(e.what()).find("no kernel for operator 'add'") != std::string::npos;
+    }
+    EXPECT(thrown);
+    // wrong parameter shape at eval
+    program q;
+    auto* qm = q.get_main_module();
+    auto a   = qm->add_parameter("a", shape{shape::int8_type, {16, 64}});
+    auto b   = qm->add_parameter("b", shape{shape::int8_type, {64, 16}});
+    qm->add_return({qm->add_instruction(make_op("quant_dot"), a, b)});
+    auto t = migraphx::make_target("mi355");
+    q.compile(t);
+    EXPECT(test::throws([&] { q.eval({{"a", t.allocate(shape{shape::int8_type, {16, 64}})}}); }));
+    EXPECT(test::throws([&] {
+        q.eval({{"a", t.allocate(shape{shape::int8_type, {16, 32}})},
+                {"b", t.allocate(shape{shape::int8_type, {64, 16}})}});
+    }));
+}
+
+int main(int argc, char** argv)
+{
+    try
+    {
+        return test::run(argc, argv);
+    }
+    catch(const std::exception& e)
+    {
+        std::cout << "error: " << e.what() << std::endl;
+        return 4;
+    }
+}

@@ -1,0 +1,748 @@
+// CPU tests of the host layer: element types, shapes, values, operator shape rules, module
+// editing, registries, and the passes of the quantized-GEMM path (simplify_qdq, quantize_int8 /
+// fp8 calibration, quantize_int4, the MatMulNBits graph).  Pass tests follow the reference's
+// test/simplify_qdq_test.cpp, test/int4_test.cpp and test/quantization.cpp: the rewritten module
+// is compared with one written out by hand, and both are evaluated on the CPU oracle target.
+#include "common.hpp"
+#include "oracle_target.hpp"
+#include "test.hpp"
+#include <algorithm>
+#include <fstream>
+
+extern "C" {
+float orc_fp8e4m3fn_to_f32(uint8_t x);
+uint8_t orc_fp8e4m3fn_from_f32(float x);
+uint16_t orc_half_from_f32(float x);
+float orc_half_to_f32(uint16_t h);
+uint16_t orc_bf16_from_f32(float x);
+float orc_bf16_to_f32(uint16_t h);
+}
+
+using namespace testutil;
+using migraphx::shape;
+
+// ---------------------------------------------------------------- element types
+
+TEST_CASE(fp8_matches_oracle)
+{
+    for(int c = 0; c < 256; c++)
+    {
+        const float a = migraphx::fp8e4m3fn::from_bits(c);
+        const float b = orc_fp8e4m3fn_to_f32(c);
+        EXPECT((std::isnan(a) and std::isnan(b)) or a == b);
+    }
+    std::mt19937 g(1);
+    for(int i = 0; i < 400000; i++)
+    {
+        uint32_t bits = g();
+        float f;
+        std::memcpy(&f, &bits, 4);
+        const float af = std::fabs(f);
+        if(af > 464.0f and af < 512.0f)
+            continue; // the reference's encoder returns NaN there; unreachable behind the clamp
+        EXPECT(migraphx::fp8e4m3fn(f).bits == orc_fp8e4m3fn_from_f32(f));
+    }
+    for(float f : {0.0f, -0.0f, 1.0f, 1.0625f, 1.1875f, 448.0f, 1000.0f, -1000.0f, 0.001953125f, 0.0009765625f})
+        EXPECT(migraphx::fp8e4m3fn(f).bits == orc_fp8e4m3fn_from_f32(f));
+}
+
+TEST_CASE(half_bf16_match_oracle)
+{
+    for(int c = 0; c < 65536; c++)
+    {
+        const float a = migraphx::half::from_bits(c);
+        const float b = orc_half_to_f32(c);
+        EXPECT((std::isnan(a) and std::isnan(b)) or a == b);
+        const float x = migraphx::bf16::from_bits(c);
+        const float y = orc_bf16_to_f32(c);
+        EXPECT((std::isnan(x) and std::isnan(y)) or x == y);
+    }
+    std::mt19937 g(2);
+    for(int i = 0; i < 400000; i++)
+    {
+        uint32_t bits = g();
+        float f;
+        std::memcpy(&f, &bits, 4);
+        if(std::isnan(f) or (std::fabs(f) < 1.2e-38f and f != 0.0f))
+            continue; // NaN payloads and float subnormals are off the path
+        EXPECT(migraphx::half(f).bits == orc_half_from_f32(f));
+        EXPECT(migraphx::bf16(f).bits == orc_bf16_from_f32(f));
+    }
+    // truncation, not rounding
+    EXPECT(float(migraphx::half(1.0f + 1.5f / 2048)) == 1.0f);
+    EXPECT(float(migraphx::bf16(1.0f + 1.5f / 256)) == 1.0f);
+    EXPECT(std::isinf(float(migraphx::half(65536.0f))));
+    EXPECT(float(migraphx::half(65519.0f)) == 65504.0f);
+}
+
+// ---------------------------------------------------------------- shape, value
+
+TEST_CASE(shape_predicates)
+{
+    shape s{shape::float_type, {2, 3, 4}};
+    EXPECT(s.standard() and s.packed() and not s.transposed() and not s.broadcasted());
+    EXPECT(s.strides() == std::vector<std::size_t>{12, 4, 1});
+    EXPECT(s.elements() == 24 and s.bytes() == 96 and s.element_space() == 24);
+    EXPECT(s.index({1, 2, 3}) == 23 and s.index(std::size_t{17}) == 17);
+    EXPECT(s.multi(17) == std::vector<std::size_t>{1, 1, 1});
+
+    shape t{shape::int8_type, {3, 2}, {1, 3}};
+    EXPECT(t.transposed() and t.packed() and not t.standard());
+    EXPECT(t.index(std::size_t{1}) == 3);
+
+    shape b{shape::half_type, {4, 5}, {0, 1}};
+    EXPECT(b.broadcasted() and not b.packed() and not b.scalar());
+    EXPECT(b.element_space() == 5 and b.bytes() == 10);
+
+    shape sc{shape::uint8_type};
+    EXPECT(sc.scalar() and sc.elements() == 1 and sc.lens() == std::vector<std::size_t>{1});
+
+    EXPECT(shape::from_permutation(shape::float_type, {2, 3}, {1, 0}).strides() ==
+           std::vector<std::size_t>{1, 2});
+    EXPECT(t.with_lens({5, 7}).strides() == std::vector<std::size_t>{1, 5});
+    EXPECT(shape::parse_type("int8_type") == shape::int8_type);
+    EXPECT(shape::type_size(shape::fp8e4m3fn_type) == 1 and shape::type_size(shape::bf16_type) == 2);
+    EXPECT(test::throws([] { shape(shape::float_type, {2, 3}, {1}); }));
+}
+
+TEST_CASE(value_and_make_op)
+{
+    auto op = make_op("slice", {{"axes", {1}}, {"starts", {0}}, {"ends", {5}}});
+    auto v  = op.to_value();
+    EXPECT(v.at("axes").to_vector<int64_t>() == std::vector<int64_t>{1});
+    EXPECT(v.at("ends").to_vector<int64_t>() == std::vector<int64_t>{5});
+    EXPECT(op == make_op("slice", {{"ends", {5}}, {"axes", {1}}, {"starts", {0}}}));
+    EXPECT(op != make_op("slice", {{"ends", {6}}, {"axes", {1}}, {"starts", {0}}}));
+    EXPECT(test::throws([] { make_op("slice", {{"axis", {1}}}); }));
+    EXPECT(test::throws([] { make_op("no_such_operator"); }));
+    std::vector<std::size_t> lens = {2, 3};
+    auto mb = make_op("multibroadcast", {{"out_lens", lens}});
+    EXPECT(migraphx::any_cast<migraphx::op::multibroadcast>(mb).out_lens == lens);
+    auto cv = make_op("convert", {{"target_type", shape::half_type}});
+    EXPECT(migraphx::any_cast<migraphx::op::convert>(cv).target_type == shape::half_type);
+    std::stringstream ss;
+    ss << make_op("transpose", {{"permutation", {1, 0}}});
+    EXPECT(ss.str() == "transpose[permutation=[1, 0]]");
+}
+
+// ---------------------------------------------------------------- operator shape rules
+
+TEST_CASE(quant_dot_shapes)
+{
+    // src/include/migraphx/op/quant_dot.hpp:51-121
+    auto qd = make_op("quant_dot");
+    shape a{shape::int8_type, {4, 8}};
+    shape b{shape::int8_type, {8, 6}};
+    EXPECT(qd.compute_shape({a, b}) == shape{shape::int32_type, {4, 6}});
+    shape af{shape::fp8e4m3fn_type, {2, 4, 8}};
+    shape bf{shape::fp8e4m3fn_type, {2, 8, 6}};
+    EXPECT(qd.compute_shape({af, bf}) == shape{shape::float_type, {2, 4, 6}});
+    shape sa{shape::float_type, {4, 8}};
+    shape sb{shape::float_type, {8, 6}};
+    EXPECT(qd.compute_shape({a, b, sa, sb}).type() == shape::float_type);
+    // transposed views are fine
+    EXPECT(qd.compute_shape({a, shape{shape::int8_type, {8, 6}, {1, 8}}}).lens() ==
+           std::vector<std::size_t>{4, 6});
+    EXPECT(test::throws([&] { qd.compute_shape({a}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({a, shape{shape::uint8_type, {8, 6}}}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({a, shape{shape::int8_type, {7, 6}}}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({shape{shape::half_type, {4, 8}}, shape{shape::half_type, {8, 6}}}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({shape{shape::int8_type, {8}}, shape{shape::int8_type, {8}}}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({af, shape{shape::fp8e4m3fn_type, {3, 8, 6}}}); }));
+    EXPECT(test::throws([&] { qd.compute_shape({a, b, sa, shape{shape::half_type, {8, 6}}}); }));
+}
+
+TEST_CASE(qdq_and_int4_shapes)
+{
+    shape x{shape::float_type, {3, 4}};
+    shape zi{shape::int8_type, {3, 4}};
+    EXPECT(make_op("quantizelinear").compute_shape({x, x}) == shape{shape::uint8_type, {3, 4}});
+    EXPECT(make_op("quantizelinear").compute_shape({x, x, zi}) == zi);
+    EXPECT(make_op("quantizelinear", {{"out_type", shape::fp8e4m3fn_type}}).compute_shape({x, x}).type() ==
+           shape::fp8e4m3fn_type);
+    EXPECT(test::throws([&] { make_op("quantizelinear").compute_shape({x, shape{shape::half_type, {3, 4}}}); }));
+    EXPECT(test::throws([&] { make_op("quantizelinear").compute_shape({x, shape{shape::float_type, {3, 5}}}); }));
+    EXPECT(make_op("dequantizelinear").compute_shape({zi, shape{shape::half_type, {3, 4}}, zi}) ==
+           shape{shape::half_type, {3, 4}});
+    EXPECT(test::throws([&] { make_op("dequantizelinear").compute_shape({zi, x, shape{shape::uint8_type, {3, 4}}}); }));
+    shape p{shape::uint8_type, {2, 5}};
+    EXPECT(make_op("unpack_int4").compute_shape({p}).lens() == std::vector<std::size_t>{2, 10});
+    EXPECT(make_op("unpack_int4", {{"axis", 0}}).compute_shape({p}).lens() == std::vector<std::size_t>{4, 5});
+    EXPECT(make_op("pack_int4").compute_shape({shape{shape::int8_type, {2, 6}}}).lens() ==
+           std::vector<std::size_t>{2, 3});
+    EXPECT(test::throws([&] { make_op("pack_int4").compute_shape({p}); })); // odd axis
+    EXPECT(test::throws([&] { make_op("unpack_int4").compute_shape({x}); }));
+    EXPECT(make_op("convert", {{"target_type", shape::bf16_type}}).compute_shape({x}) ==
+           shape{shape::bf16_type, {3, 4}});
+}
+
+TEST_CASE(view_shapes)
+{
+    shape x{shape::float_type, {3, 4}};
+    EXPECT(make_op("transpose", {{"permutation", {1, 0}}}).compute_shape({x}) ==
+           shape{shape::float_type, {4, 3}, {1, 4}});
+    EXPECT(test::throws([&] { make_op("transpose", {{"permutation", {1, 1}}}).compute_shape({x}); }));
+    shape v{shape::float_type, {4}};
+    std::vector<std::size_t> lens = {3, 4};
+    EXPECT(make_op("broadcast", {{"axis", 1}, {"out_lens", lens}}).compute_shape({v}) ==
+           shape{shape::float_type, {3, 4}, {0, 1}});
+    EXPECT(test::throws([&] { make_op("broadcast", {{"axis", 0}, {"out_lens", lens}}).compute_shape({v}); }));
+    EXPECT(make_op("multibroadcast", {{"out_lens", lens}}).compute_shape({shape{shape::float_type}}) ==
+           shape{shape::float_type, {3, 4}, {0, 0}});
+    EXPECT(make_op("multibroadcast", {{"out_lens", lens}}).compute_shape({shape{shape::float_type, {3, 1}}}) ==
+           shape{shape::float_type, {3, 4}, {1, 0}});
+    EXPECT(make_op("reshape", {{"dims", {2, -1}}}).compute_shape({x}).lens() == std::vector<std::size_t>{2, 6});
+    EXPECT(test::throws([&] { make_op("reshape", {{"dims", {5, -1}}}).compute_shape({x}); }));
+    EXPECT(make_op("unsqueeze", {{"axes", {2}}}).compute_shape({x}) ==
+           shape{shape::float_type, {3, 4, 1}, {4, 1, 1}});
+    EXPECT(make_op("squeeze", {{"axes", {0}}}).compute_shape({shape{shape::float_type, {1, 4}}}).lens() ==
+           std::vector<std::size_t>{4});
+    auto sl = make_op("slice", {{"axes", {1}}, {"starts", {1}}, {"ends", {3}}});
+    EXPECT(sl.compute_shape({x}) == shape{shape::float_type, {3, 2}, {4, 1}});
+    argument a{x, std::vector<float>{0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11}};
+    EXPECT(sl.compute(sl.compute_shape({x}), {a}).to_vector<float>() ==
+           std::vector<float>{1, 2, 5, 6, 9, 10});
+    auto tr = make_op("transpose", {{"permutation", {1, 0}}});
+    auto at = tr.compute(tr.compute_shape({x}), {a});
+    EXPECT(make_op("contiguous").compute(shape{shape::float_type, {4, 3}}, {at}).to_vector<float>() ==
+           std::vector<float>{0, 4, 8, 1, 5, 9, 2, 6, 10, 3, 7, 11});
+}
+
+// ---------------------------------------------------------------- module, registries
+
+TEST_CASE(module_editing)
+{
+    module m;
+    auto x   = m.add_parameter("x", shape{shape::float_type, {2, 3}});
+    auto y   = m.add_parameter("y", shape{shape::float_type, {2, 3}});
+    auto l   = m.add_literal(literal{shape{shape::float_type, {2, 3}}, std::vector<float>{1, 2, 3, 4, 5, 6}});
+    auto s   = m.add_instruction(make_op("add"), x, y);
+    auto d   = m.add_instruction(make_op("mul"), x, l); // dead
+    auto r   = m.add_instruction(make_op("sub"), s, y);
+    (void)d;
+    EXPECT(m.validate() == m.end());
+    EXPECT(m.get_parameter_names() == std::vector<std::string>{"x", "y"});
+    EXPECT(m.get_output_shapes().front() == shape{shape::float_type, {2, 3}});
+    EXPECT(s->outputs().size() == 1 and x->outputs().size() == 2);
+    migraphx::dead_code_elimination{}.apply(m);
+    EXPECT(count_ops(m, "mul") == 0 and count_ops(m, "@literal") == 0 and count_ops(m, "@param") == 2);
+    // replacing the last instruction keeps the replacement as the result
+    auto t = m.insert_instruction(r, make_op("add"), s, s);
+    m.replace_instruction(r, t);
+    EXPECT(std::prev(m.end()) == t and m.validate() == m.end());
+    // a shape change propagates to users
+    module m2;
+    auto p  = m2.add_parameter("p", shape{shape::float_type, {2, 3}});
+    auto tp = m2.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), p);
+    auto id = m2.add_instruction(make_op("identity"), tp);
+    m2.replace_instruction(tp, make_op("identity"), p);
+    EXPECT(id->get_shape().lens() == std::vector<std::size_t>{2, 3});
+    // copies are deep
+    module m3 = m;
+    EXPECT(m3 == m);
+    m3.add_instruction(make_op("identity"), std::prev(m3.end()));
+    EXPECT(m3 != m);
+    auto tq = m2.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), p);
+    EXPECT(test::throws([&] { m2.add_instruction(make_op("add"), p, tq); }));
+    EXPECT(test::throws([&] { m.remove_instruction(x); }));
+}
+
+TEST_CASE(registries)
+{
+    EXPECT(migraphx::has_op("quant_dot") and migraphx::has_op("unpack_int4") and
+           migraphx::has_op("dequantizelinear") and migraphx::has_op("quantizelinear"));
+    auto t = migraphx::make_target("oracle");
+    EXPECT(t.name() == "oracle");
+    bool thrown = false;
+    try
+    {
+        migraphx::make_target("no_such_target");
+    }
+    catch(const migraphx::exception& e)
+    {
+        thrown = std::string(e.what()).find("Requested target 'no_such_target' is not loaded") !=
+                 std::string::npos;
+    }
+    EXPECT(thrown);
+    // an uncompiled arithmetic operator cannot be evaluated: there is no host fallback
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::int8_type, {2, 2}});
+    mm->add_instruction(make_op("quant_dot"), x, x);
+    argument a{shape{shape::int8_type, {2, 2}}, std::vector<int>{1, 2, 3, 4}};
+    EXPECT(test::throws([&] { p.eval({{"x", a}}); }));
+}
+
+TEST_CASE(mi355_target_library_loads)
+{
+    // libmigraphx_mi355.so is found next to libmigraphx.so and registers the target and its
+    // operators from its static initialisers; no GPU is touched by that
+    auto t = migraphx::make_target("mi355");
+    EXPECT(t.name() == "mi355");
+    EXPECT(migraphx::has_op("mi355::quant_dot") and migraphx::has_op("mi355::w4a16_gemm"));
+}
+
+// ---------------------------------------------------------------- simplify_qdq
+
+static void run_pass(module& m)
+{
+    migraphx::run_passes(m, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+}
+
+// mul(broadcast s1, broadcast s2) as the pass emits it (test/simplify_qdq_test.cpp add_scale_mul)
+static instruction_ref add_scale_mul(module& m,
+                                     instruction_ref s1,
+                                     instruction_ref s2,
+                                     std::size_t axis1,
+                                     std::size_t axis2,
+                                     const std::vector<std::size_t>& out_lens)
+{
+    auto bc = [&](instruction_ref s, std::size_t axis) {
+        if(s->get_shape().scalar())
+            return m.add_instruction(make_op("multibroadcast", {{"out_lens", out_lens}}), s);
+        return m.add_instruction(make_op("broadcast", {{"axis", axis}, {"out_lens", out_lens}}), s);
+    };
+    return m.add_instruction(make_op("mul"), bc(s1, axis1), bc(s2, axis2));
+}
+
+TEST_CASE(remove_qdq)
+{
+    shape sh{shape::float_type, {100, 100}};
+    module m1;
+    {
+        auto t1    = m1.add_parameter("t1", sh);
+        auto t2    = m1.add_parameter("t2", sh);
+        auto scale = m1.add_literal(0.5f);
+        auto zero  = m1.add_literal(std::int8_t{0});
+        auto q1    = add_quantize_op(m1, "quantizelinear", t1, scale, zero);
+        auto d1    = add_quantize_op(m1, "dequantizelinear", q1, scale, zero);
+        auto q2    = add_quantize_op(m1, "quantizelinear", t2, scale, zero);
+        auto d2    = add_quantize_op(m1, "dequantizelinear", q2, scale, zero);
+        m1.add_return({m1.add_instruction(make_op("add"), d1, d2)});
+    }
+    module m2;
+    {
+        auto t1 = m2.add_parameter("t1", sh);
+        auto t2 = m2.add_parameter("t2", sh);
+        m2.add_return({m2.add_instruction(make_op("add"), t1, t2)});
+    }
+    run_pass(m1);
+    EXPECT(canonical(m1) == canonical(m2));
+}
+
+TEST_CASE(qdq_different_scales)
+{
+    shape sh{shape::float_type, {100, 100}};
+    module m1;
+    {
+        auto t1     = m1.add_parameter("t1", sh);
+        auto scale1 = m1.add_literal(0.5f);
+        auto scale2 = m1.add_literal(0.4f);
+        auto zero   = m1.add_literal(std::int8_t{1});
+        auto q1     = add_quantize_op(m1, "quantizelinear", t1, scale1, zero);
+        auto d1     = add_quantize_op(m1, "dequantizelinear", q1, scale2, zero);
+        m1.add_return({d1});
+    }
+    module m2 = m1;
+    run_pass(m1);
+    EXPECT(canonical(m1) == canonical(m2));
+}
+
+TEST_CASE(qdq_dot)
+{
+    // test/simplify_qdq_test.cpp:125-163
+    shape sh1{shape::float_type, {1280, 1000}};
+    shape sh2{shape::float_type, {1000, 1024}};
+    module m1;
+    {
+        auto t1    = m1.add_parameter("t1", sh1);
+        auto t2    = m1.add_parameter("t2", sh2);
+        auto scale = m1.add_literal(0.5f);
+        auto zero  = m1.add_literal(std::int8_t{0});
+        auto q1    = add_quantize_op(m1, "quantizelinear", t1, scale, zero);
+        auto d1    = add_quantize_op(m1, "dequantizelinear", q1, scale, zero);
+        auto q2    = add_quantize_op(m1, "quantizelinear", t2, scale, zero);
+        auto d2    = add_quantize_op(m1, "dequantizelinear", q2, scale, zero);
+        m1.add_return({m1.add_instruction(make_op("dot"), d1, d2)});
+    }
+    module m3;
+    {
+        auto t1    = m3.add_parameter("t1", sh1);
+        auto t2    = m3.add_parameter("t2", sh2);
+        auto scale = m3.add_literal(0.5f);
+        auto zero  = m3.add_literal(std::int8_t{0});
+        auto q1    = add_quantize_op(m3, "quantizelinear", t1, scale, zero);
+        auto q2    = add_quantize_op(m3, "quantizelinear", t2, scale, zero);
+        auto dot   = m3.add_instruction(make_op("quant_dot"), q1, q2);
+        auto os    = add_scale_mul(m3, scale, scale, 1, 1, dot->get_shape().lens());
+        m3.add_return({m3.add_instruction(make_op("dequantizelinear"), dot, os)});
+    }
+    run_pass(m1);
+    EXPECT(canonical(m1) == canonical(m3));
+    EXPECT(count_ops(m1, "dot") == 0 and count_ops(m1, "quant_dot") == 1);
+}
+
+TEST_CASE(qdq_dot_fp16)
+{
+    // test/simplify_qdq_test.cpp:165-216: float Q/DQ parameters around a half dot
+    shape sh1{shape::half_type, {64, 40}};
+    shape sh2{shape::half_type, {40, 48}};
+    module m1;
+    {
+        auto t1    = m1.add_parameter("t1", sh1);
+        auto t2    = m1.add_parameter("t2", sh2);
+        auto scale = m1.add_literal(0.5f);
+        auto zero  = m1.add_literal(std::int8_t{0});
+        auto c1 = m1.add_instruction(make_op("convert", {{"target_type", shape::float_type}}), t1);
+        auto c2 = m1.add_instruction(make_op("convert", {{"target_type", shape::float_type}}), t2);
+        auto q1 = add_quantize_op(m1, "quantizelinear", c1, scale, zero);
+        auto d1 = add_quantize_op(m1, "dequantizelinear", q1, scale, zero);
+        auto q2 = add_quantize_op(m1, "quantizelinear", c2, scale, zero);
+        auto d2 = add_quantize_op(m1, "dequantizelinear", q2, scale, zero);
+        auto h1 = m1.add_instruction(make_op("convert", {{"target_type", shape::half_type}}), d1);
+        auto h2 = m1.add_instruction(make_op("convert", {{"target_type", shape::half_type}}), d2);
+        m1.add_return({m1.add_instruction(make_op("dot"), h1, h2)});
+    }
+    run_pass(m1);
+    EXPECT(count_ops(m1, "dot") == 0 and count_ops(m1, "quant_dot") == 1);
+    auto last = m1.get_returns().front();
+    EXPECT(last->name() == "convert" and last->get_shape().type() == shape::half_type);
+    EXPECT(last->inputs().front()->name() == "dequantizelinear");
+    EXPECT(last->inputs().front()->inputs().front()->get_shape().type() == shape::int32_type);
+}
+
+TEST_CASE(qdq_dot_multi_scale_and_transposed)
+{
+    // per-output-channel weight scale, weight stored [N, K] with the transpose between DQ and dot
+    // (test/simplify_qdq_test.cpp:218-347)
+    const std::size_t m = 16, k = 32, n = 24;
+    module m1;
+    {
+        auto x   = m1.add_parameter("x", shape{shape::float_type, {m, k}});
+        auto w   = m1.add_literal(literal{shape{shape::int8_type, {n, k}}, uniform_ints<int>(n * k, -127, 127, 3)});
+        auto s1  = m1.add_literal(0.25f);
+        auto z1  = m1.add_literal(std::int8_t{0});
+        auto s2  = m1.add_literal(literal{shape{shape::float_type, {n}}, uniform_floats(n, 0.001f, 0.01f, 4)});
+        auto z2  = m1.add_literal(literal{shape{shape::int8_type, {n}}, std::vector<int>(n, 0)});
+        auto q1  = add_quantize_op(m1, "quantizelinear", x, s1, z1);
+        auto d1  = add_quantize_op(m1, "dequantizelinear", q1, s1, z1);
+        std::vector<std::size_t> wl = {n, k};
+        auto s2b = m1.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", wl}}), s2);
+        auto z2b = m1.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", wl}}), z2);
+        auto d2  = m1.add_instruction(make_op("dequantizelinear"), w, s2b, z2b);
+        auto wt  = m1.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), d2);
+        m1.add_return({m1.add_instruction(make_op("dot"), d1, wt)});
+    }
+    program before;
+    *before.get_main_module() = m1;
+    run_pass(m1);
+    EXPECT(count_ops(m1, "dot") == 0 and count_ops(m1, "quant_dot") == 1);
+    // the quantized weight reaches quant_dot through the re-applied transpose
+    auto dq = m1.get_returns().front();
+    EXPECT(dq->name() == "dequantizelinear" and dq->inputs().size() == 2);
+    auto qd = dq->inputs()[0];
+    EXPECT(qd->inputs()[1]->name() == "transpose" and qd->inputs()[1]->get_shape().type() == shape::int8_type);
+    auto mul = dq->inputs()[1];
+    EXPECT(mul->name() == "mul" and mul->inputs()[0]->name() == "multibroadcast" and
+           mul->inputs()[1]->name() == "broadcast");
+    EXPECT(migraphx::any_cast<migraphx::op::broadcast>(mul->inputs()[1]->get_operator()).axis == 1);
+    // same numbers before and after, up to the float rounding of the fake-quantized dot
+    program after;
+    *after.get_main_module() = m1;
+    argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 5)};
+    auto r0 = run_on("oracle", before, {{"x", xa}});
+    auto r1 = run_on("oracle", after, {{"x", xa}});
+    EXPECT(max_rel_diff(r1[0], r0[0], 1.0) < 1e-5);
+}
+
+TEST_CASE(qdq_dot_unsupported_axis_and_uint8)
+{
+    // a per-row scale on the weight (length K on axis 0 of [K, N]) cannot move behind the dot
+    // (test/simplify_qdq_test.cpp:445-477); uint8 tensors are left alone (:628-658)
+    const std::size_t m = 8, k = 16, n = 12;
+    module m1;
+    {
+        auto x  = m1.add_parameter("x", shape{shape::float_type, {m, k}});
+        auto w  = m1.add_parameter("w", shape{shape::float_type, {k, n}});
+        auto s1 = m1.add_literal(0.5f);
+        auto z1 = m1.add_literal(std::int8_t{0});
+        auto s2 = m1.add_literal(literal{shape{shape::float_type, {k}}, uniform_floats(k, 0.1f, 0.2f, 1)});
+        auto z2 = m1.add_literal(literal{shape{shape::int8_type, {k}}, std::vector<int>(k, 0)});
+        auto q1 = add_quantize_op(m1, "quantizelinear", x, s1, z1);
+        auto d1 = add_quantize_op(m1, "dequantizelinear", q1, s1, z1);
+        std::vector<std::size_t> wl = {k, n};
+        auto s2b = m1.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", wl}}), s2);
+        auto z2b = m1.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", wl}}), z2);
+        auto q2  = m1.add_instruction(make_op("quantizelinear"), w, s2b, z2b);
+        auto d2  = m1.add_instruction(make_op("dequantizelinear"), q2, s2b, z2b);
+        m1.add_return({m1.add_instruction(make_op("dot"), d1, d2)});
+    }
+    run_pass(m1);
+    EXPECT(count_ops(m1, "dot") == 1 and count_ops(m1, "quant_dot") == 0);
+
+    module m2;
+    {
+        auto x  = m2.add_parameter("x", shape{shape::float_type, {m, k}});
+        auto w  = m2.add_parameter("w", shape{shape::float_type, {k, n}});
+        auto s  = m2.add_literal(0.5f);
+        auto z  = m2.add_literal(std::uint8_t{0});
+        auto q1 = add_quantize_op(m2, "quantizelinear", x, s, z);
+        auto d1 = add_quantize_op(m2, "dequantizelinear", q1, s, z);
+        auto q2 = add_quantize_op(m2, "quantizelinear", w, s, z);
+        auto d2 = add_quantize_op(m2, "dequantizelinear", q2, s, z);
+        m2.add_return({m2.add_instruction(make_op("dot"), d1, d2)});
+    }
+    run_pass(m2);
+    // the fake-quantization pairs fold away, the dot stays a float dot
+    EXPECT(count_ops(m2, "dot") == 1 and count_ops(m2, "quant_dot") == 0);
+}
+
+static module asymmetric_dot(int zp1, int zp2, std::size_t m, std::size_t k, std::size_t n)
+{
+    module m1;
+    auto x  = m1.add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w  = m1.add_parameter("w", shape{shape::float_type, {k, n}});
+    auto s1 = m1.add_literal(0.05f);
+    auto s2 = m1.add_literal(0.02f);
+    auto z1 = m1.add_literal(static_cast<std::int8_t>(zp1));
+    auto z2 = m1.add_literal(static_cast<std::int8_t>(zp2));
+    auto q1 = add_quantize_op(m1, "quantizelinear", x, s1, z1);
+    auto d1 = add_quantize_op(m1, "dequantizelinear", q1, s1, z1);
+    auto q2 = add_quantize_op(m1, "quantizelinear", w, s2, z2);
+    auto d2 = add_quantize_op(m1, "dequantizelinear", q2, s2, z2);
+    m1.add_return({m1.add_instruction(make_op("dot"), d1, d2)});
+    return m1;
+}
+
+TEST_CASE(qdq_dot_asymmetric)
+{
+    // test/simplify_qdq_test.cpp:479-626 and :1471-1520: one extra quant_dot per non-zero zero
+    // point, a third for the cross term, and the same numbers as the fake-quantized graph
+    const std::size_t m = 12, k = 40, n = 20;
+    struct cfg
+    {
+        int zp1, zp2;
+        std::size_t quant_dots, adds, subs;
+    };
+    for(auto c : {cfg{3, 0, 2, 1, 0}, cfg{0, -5, 2, 1, 0}, cfg{3, -5, 4, 2, 1}, cfg{0, 0, 1, 0, 0}})
+    {
+        module m1 = asymmetric_dot(c.zp1, c.zp2, m, k, n);
+        program before;
+        *before.get_main_module() = m1;
+        run_pass(m1);
+        EXPECT(count_ops(m1, "dot") == 0);
+        EXPECT(count_ops(m1, "quant_dot") == c.quant_dots);
+        EXPECT(count_ops(m1, "add") == c.adds and count_ops(m1, "sub") == c.subs);
+        auto dq = m1.get_returns().front();
+        EXPECT(dq->inputs().size() == ((c.zp1 != 0 or c.zp2 != 0) ? 3u : 2u));
+        program after;
+        *after.get_main_module() = m1;
+        argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 6)};
+        argument wa{shape{shape::float_type, {k, n}}, normal_floats(k * n, 0.5f, 7)};
+        auto r0 = run_on("oracle", before, {{"x", xa}, {"w", wa}});
+        auto r1 = run_on("oracle", after, {{"x", xa}, {"w", wa}});
+        EXPECT(max_rel_diff(r1[0], r0[0], 1e-2) < 1e-4);
+    }
+}
+
+// ---------------------------------------------------------------- quantize_int4, quantize_int8
+
+TEST_CASE(int4_pass)
+{
+    // test/int4_test.cpp:38-90
+    const std::size_t m = 4, k = 6, n = 8;
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto wv  = uniform_floats(k * n, -1.0f, 2.0f, 9);
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, wv});
+    mm->add_return({mm->add_instruction(make_op("dot"), x, w)});
+    program fp = p;
+    migraphx::quantize_int4_weights(p);
+    EXPECT(count_ops(*mm, "quantizelinear") == 1 and count_ops(*mm, "pack_int4") == 1 and
+           count_ops(*mm, "unpack_int4") == 1 and count_ops(*mm, "dequantizelinear") == 1);
+    auto dot = mm->get_returns().front();
+    EXPECT(dot->name() == "dot" and dot->inputs()[0] == x);
+    auto dq = dot->inputs()[1];
+    EXPECT(dq->name() == "dequantizelinear" and dq->inputs()[0]->name() == "unpack_int4");
+    auto q = dq->inputs()[0]->inputs()[0]->inputs()[0];
+    EXPECT(q->name() == "quantizelinear" and q->get_shape().type() == shape::uint8_type);
+    // per-tensor parameters: scale = (max - min) / 15, zero point = round(-min / scale)
+    const float lo = std::min(0.0f, *std::min_element(wv.begin(), wv.end()));
+    const float hi = std::max(0.0f, *std::max_element(wv.begin(), wv.end()));
+    auto scale_lit = q->inputs()[1]->inputs()[0];
+    auto zp_lit    = q->inputs()[2]->inputs()[0];
+    EXPECT(scale_lit->get_literal().at<float>() == (hi - lo) / 15);
+    EXPECT(zp_lit->get_literal().at<int>() == static_cast<int>(std::round(-lo / ((hi - lo) / 15))));
+    // quantized weights stay within half a step of the originals
+    argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 10)};
+    auto r0 = run_on("oracle", fp, {{"x", xa}});
+    auto r1 = run_on("oracle", p, {{"x", xa}});
+    auto a  = r0[0].to_vector<double>();
+    auto b  = r1[0].to_vector<double>();
+    for(std::size_t i = 0; i < a.size(); i++)
+        EXPECT(std::fabs(a[i] - b[i]) < 0.5 * (hi - lo) / 15 * k * 3);
+    // an odd last dimension is left alone
+    program p2;
+    auto* m2 = p2.get_main_module();
+    auto x2  = m2->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w2  = m2->add_literal(literal{shape{shape::float_type, {k, 7}}, uniform_floats(k * 7, -1, 1, 1)});
+    m2->add_return({m2->add_instruction(make_op("dot"), x2, w2)});
+    migraphx::quantize_int4_weights(p2);
+    EXPECT(count_ops(*m2, "quantizelinear") == 0);
+}
+
+TEST_CASE(int8_calibration)
+{
+    // test/quantization.cpp:1066-1110: calibrated int8 dot stays close to the float dot
+    const std::size_t m = 16, k = 64, n = 32;
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto wv  = normal_floats(k * n, 0.05f, 11);
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, wv});
+    mm->add_return({mm->add_instruction(make_op("dot"), x, w)});
+    program fp = p;
+    auto xv    = normal_floats(m * k, 1.0f, 12);
+    argument xa{shape{shape::float_type, {m, k}}, xv};
+    migraphx::quantize_int8(p, migraphx::make_target("oracle"), {{{"x", xa}}});
+    EXPECT(count_ops(*mm, "capture") == 0);
+    EXPECT(count_ops(*mm, "quantizelinear") == 2 and count_ops(*mm, "dequantizelinear") == 2);
+    // Q scale literal = max|x| / 127 (the inverse of the calibrated multiplier)
+    float amax = 0;
+    for(float v : xv)
+        amax = std::max(amax, std::fabs(v));
+    auto dot = mm->get_returns().front();
+    auto dq  = dot->inputs()[0];
+    auto sc  = dq->inputs()[1]->inputs()[0]->get_literal().at<float>();
+    EXPECT(sc == 1.0f / (127.0f / amax));
+    EXPECT(dq->inputs()[2]->get_shape().type() == shape::int8_type);
+    EXPECT(test::throws([&] {
+        program q = fp;
+        migraphx::quantize_int8(q, migraphx::make_target("oracle"), {}, {"dot"});
+    }));
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(count_ops(*mm, "quant_dot") == 1 and count_ops(*mm, "dot") == 0);
+    auto r0 = run_on("oracle", fp, {{"x", xa}});
+    auto r1 = run_on("oracle", p, {{"x", xa}});
+    // root-mean-square error relative to the result's own RMS, as verify::rms_range compares
+    auto a = r0[0].to_vector<double>();
+    auto b = r1[0].to_vector<double>();
+    double num = 0, den = 0;
+    for(std::size_t i = 0; i < a.size(); i++)
+    {
+        num += (a[i] - b[i]) * (a[i] - b[i]);
+        den += a[i] * a[i];
+    }
+    EXPECT(std::sqrt(num / den) < 0.02);
+}
+
+TEST_CASE(fp8_calibration)
+{
+    const std::size_t m = 8, k = 32, n = 16;
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {k, n}}, normal_floats(k * n, 0.02f, 13)});
+    mm->add_return({mm->add_instruction(make_op("dot"), x, w)});
+    program fp = p;
+    argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 14)};
+    migraphx::quantize_fp8(p, migraphx::make_target("oracle"), {{{"x", xa}}});
+    auto dot = mm->get_returns().front();
+    EXPECT(dot->inputs()[0]->inputs()[0]->get_shape().type() == shape::fp8e4m3fn_type);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(count_ops(*mm, "quant_dot") == 1);
+    EXPECT(mm->get_returns().front()->inputs()[0]->get_shape().type() == shape::float_type);
+    auto r0 = run_on("oracle", fp, {{"x", xa}});
+    auto r1 = run_on("oracle", p, {{"x", xa}});
+    auto a  = r0[0].to_vector<double>();
+    auto b  = r1[0].to_vector<double>();
+    double num = 0, den = 0;
+    for(std::size_t i = 0; i < a.size(); i++)
+    {
+        num += (a[i] - b[i]) * (a[i] - b[i]);
+        den += a[i] * a[i];
+    }
+    EXPECT(std::sqrt(num / den) < 0.06);
+}
+
+// ---------------------------------------------------------------- MatMulNBits
+
+TEST_CASE(matmulnbits_graph_checks)
+{
+    module m;
+    auto a  = m.add_parameter("a", shape{shape::float_type, {2, 32}});
+    auto b  = m.add_parameter("b", shape{shape::uint8_type, {4, 2, 8}});
+    auto s  = m.add_parameter("s", shape{shape::float_type, {8}});
+    auto r  = migraphx::op::builder::matmulnbits(m, a, b, s, m.end(), 4, 32, 16);
+    EXPECT(r->get_shape() == shape{shape::float_type, {2, 4}});
+    EXPECT(count_ops(m, "unpack_int4") == 1 and count_ops(m, "dequantizelinear") == 1);
+    EXPECT(test::throws([&] { migraphx::op::builder::matmulnbits(m, a, b, s, m.end(), 4, 32, 24); }));
+    EXPECT(test::throws([&] { migraphx::op::builder::matmulnbits(m, a, b, s, m.end(), 5, 32, 16); }));
+    EXPECT(test::throws([&] { migraphx::op::builder::matmulnbits(m, a, b, a, m.end(), 4, 32, 16); }));
+}
+
+// `host_tests matmulnbits <target> <case file> <result file>`: build the MatMulNBits graph from a
+// text description and evaluate it.  The Python tests feed it the reference's known answers.
+static int matmulnbits_tool(int argc, char** argv)
+{
+    if(argc != 5)
+        return 2;
+    std::ifstream in(argv[3]);
+    std::size_t nda = 0, n = 0, nblk = 0, blob = 0;
+    int has_zp = 0, use_half = 0;
+    in >> nda;
+    std::vector<std::size_t> a_lens(nda);
+    for(auto& l : a_lens)
+        in >> l;
+    in >> n >> nblk >> blob >> has_zp >> use_half;
+    const std::size_t k   = a_lens.back();
+    const std::size_t blk = blob * 2;
+    std::size_t na        = 1;
+    for(auto l : a_lens)
+        na *= l;
+    std::vector<float> a(na), scales(n * nblk);
+    std::vector<int> b(n * nblk * blob), zp(has_zp != 0 ? n * ((nblk + 1) / 2) : 0);
+    for(auto& v : a)
+        in >> v;
+    for(auto& v : b)
+        in >> v;
+    for(auto& v : scales)
+        in >> v;
+    for(auto& v : zp)
+        in >> v;
+    if(not in)
+        return 3;
+    const auto ft = use_half != 0 ? shape::half_type : shape::float_type;
+    program p;
+    auto* mm = p.get_main_module();
+    auto ai  = mm->add_parameter("a", shape{ft, a_lens});
+    auto bi  = mm->add_literal(literal{shape{shape::uint8_type, {n, nblk, blob}}, b});
+    auto si  = mm->add_literal(literal{shape{ft, {n * nblk}}, scales});
+    auto zi  = mm->end();
+    if(has_zp != 0)
+        zi = mm->add_literal(literal{shape{shape::uint8_type, {zp.size()}}, zp});
+    mm->add_return({migraphx::op::builder::matmulnbits(*mm, ai, bi, si, zi, n, k, blk)});
+    argument aa{shape{ft, a_lens}, a};
+    auto r = run_on(argv[2], p, {{"a", aa}});
+    std::ofstream out(argv[4]);
+    out.precision(9);
+    for(auto v : r[0].to_vector<float>())
+        out << v << "\n";
+    return 0;
+}
+
+int main(int argc, char** argv)
+{
+    try
+    {
+        if(argc > 1 and std::string(argv[1]) == "matmulnbits")
+            return matmulnbits_tool(argc, argv);
+        return test::run(argc, argv);
+    }
+    catch(const std::exception& e)
+    {
+        std::cout << "error: " << e.what() << std::endl;
+        return 4;
+    }
+}

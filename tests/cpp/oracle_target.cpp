@@ -1,0 +1,211 @@
+#include "oracle_target.hpp"
+#include <migraphx/ops.hpp>
+#include <migraphx/passes.hpp>
+#include <migraphx/register_target.hpp>
+#include <cstdint>
+#include <cstring>
+
+extern "C" {
+// oracle/ref_oracle.c
+void orc_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, int64_t m, int64_t n,
+              int64_t k, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn, int64_t batch,
+              int64_t a_sb, int64_t b_sb);
+void orc_quantizelinear(void* out, int out_type, const void* x, int x_type, const void* scale,
+                        int64_t s_sr, int64_t s_sc, const void* zp, int64_t z_sr, int64_t z_sc,
+                        int64_t rows, int64_t cols);
+void orc_dequantizelinear(void* out, const void* x, int x_type, const void* scale, int s_type,
+                          int64_t s_sr, int64_t s_sc, const void* zp, int64_t z_sr, int64_t z_sc,
+                          int64_t rows, int64_t cols);
+void orc_unpack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len,
+                     int64_t inner);
+void orc_pack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len,
+                   int64_t inner);
+void orc_convert(void* out, int out_type, const void* x, int x_type, size_t n);
+}
+
+namespace oracle {
+
+using migraphx::argument;
+using migraphx::shape;
+
+namespace {
+
+enum
+{
+    ORC_I8,
+    ORC_U8,
+    ORC_I32,
+    ORC_F32,
+    ORC_F16,
+    ORC_BF16,
+    ORC_FP8,
+    ORC_F64
+};
+
+int orc_type(shape::type_t t)
+{
+    switch(t)
+    {
+    case shape::int8_type: return ORC_I8;
+    case shape::uint8_type: return ORC_U8;
+    case shape::int32_type: return ORC_I32;
+    case shape::float_type: return ORC_F32;
+    case shape::half_type: return ORC_F16;
+    case shape::bf16_type: return ORC_BF16;
+    case shape::fp8e4m3fn_type: return ORC_FP8;
+    case shape::double_type: return ORC_F64;
+    default: MIGRAPHX_THROW("oracle: unsupported type " + shape::type_name(t));
+    }
+}
+
+argument dense(const argument& a)
+{
+    if(a.get_shape().standard())
+        return a;
+    return migraphx::op::contiguous{}.compute(
+        shape{a.get_shape().type(), a.get_shape().lens()}, {a});
+}
+
+void rows_cols(const shape& s, int64_t& rows, int64_t& cols)
+{
+    cols = static_cast<int64_t>(s.lens().back());
+    rows = cols == 0 ? 0 : static_cast<int64_t>(s.elements()) / cols;
+}
+
+// Evaluates the wrapped reference operator on host memory.
+struct cpu_op
+{
+    migraphx::operation op;
+    std::string name() const { return "oracle::" + op.name(); }
+    shape compute_shape(const std::vector<shape>& inputs) const
+    {
+        auto s = op.compute_shape(inputs);
+        return shape{s.type(), s.lens()};
+    }
+    argument compute(migraphx::context&, const shape& out, const std::vector<argument>& args) const
+    {
+        const auto n = op.name();
+        argument r{out};
+        if(n == "quant_dot" or n == "dot")
+        {
+            // batches are gathered to dense tensors; inside a matrix the strides are used as
+            // they are, so that transposed views reach the GEMM untouched
+            argument a = args[0];
+            argument b = args[1];
+            if(a.get_shape().ndim() > 2)
+            {
+                a = dense(a);
+                b = dense(b);
+            }
+            const auto& sa       = a.get_shape();
+            const auto& sb       = b.get_shape();
+            const std::size_t nd = sa.ndim();
+            const int64_t m      = sa.lens()[nd - 2];
+            const int64_t k      = sa.lens()[nd - 1];
+            const int64_t nn     = sb.lens()[nd - 1];
+            const int64_t batch  = m * k == 0 ? 0 : sa.elements() / (m * k);
+            orc_gemm(r.data(), orc_type(out.type()), a.data(), b.data(), orc_type(sa.type()), m, nn, k,
+                     sa.strides()[nd - 2], sa.strides()[nd - 1], sb.strides()[nd - 2],
+                     sb.strides()[nd - 1], batch, nd > 2 ? m * k : 0, nd > 2 ? k * nn : 0);
+        }
+        else if(n == "quantizelinear" or n == "dequantizelinear")
+        {
+            int64_t rows = 0;
+            int64_t cols = 0;
+            rows_cols(out, rows, cols);
+            argument x  = dense(args[0]);
+            argument s  = dense(args[1]);
+            argument zp = args.size() > 2 ? dense(args[2]) : argument{};
+            if(n == "quantizelinear")
+                orc_quantizelinear(r.data(), orc_type(out.type()), x.data(),
+                                   orc_type(x.get_shape().type()), s.data(), cols, 1,
+                                   zp.empty() ? nullptr : zp.data(), cols, 1, rows, cols);
+            else
+                orc_dequantizelinear(r.data(), x.data(), orc_type(x.get_shape().type()), s.data(),
+                                     orc_type(s.get_shape().type()), cols, 1,
+                                     zp.empty() ? nullptr : zp.data(), cols, 1, rows, cols);
+        }
+        else if(n == "unpack_int4" or n == "pack_int4")
+        {
+            argument x      = dense(args[0]);
+            const auto& si  = x.get_shape();
+            const bool unpk = n == "unpack_int4";
+            int64_t axis    = unpk ? migraphx::any_cast<migraphx::op::unpack_int4>(op).axis
+                                   : migraphx::any_cast<migraphx::op::pack_int4>(op).axis;
+            if(axis < 0)
+                axis += static_cast<int64_t>(si.ndim());
+            int64_t outer = 1;
+            int64_t inner = 1;
+            for(int64_t i = 0; i < axis; i++)
+                outer *= si.lens()[i];
+            for(std::size_t i = axis + 1; i < si.ndim(); i++)
+                inner *= si.lens()[i];
+            const int is_signed = si.type() == shape::int8_type;
+            if(unpk)
+                orc_unpack_int4(reinterpret_cast<uint8_t*>(r.data()),
+                                reinterpret_cast<const uint8_t*>(x.data()), is_signed, outer,
+                                si.lens()[axis], inner);
+            else
+                orc_pack_int4(reinterpret_cast<uint8_t*>(r.data()),
+                              reinterpret_cast<const uint8_t*>(x.data()), is_signed, outer,
+                              out.lens()[axis], inner);
+        }
+        else if(n == "convert")
+        {
+            argument x = dense(args[0]);
+            orc_convert(r.data(), orc_type(out.type()), x.data(), orc_type(x.get_shape().type()),
+                        out.elements());
+        }
+        else if(n == "mul" or n == "add" or n == "sub")
+        {
+            // op/binary.hpp: the plain C++ operator on the tensor's type
+            migraphx::visit_type(out.type(), [&](auto t) {
+                using T = decltype(t);
+                auto x  = args[0].get<T>();
+                auto y  = args[1].get<T>();
+                auto o  = r.get<T>();
+                for(std::size_t i = 0; i < o.size(); i++)
+                {
+                    if constexpr(std::is_same<T, float>{} or std::is_same<T, int32_t>{} or
+                                 std::is_same<T, double>{})
+                        o[i] = n == "mul" ? x[i] * y[i] : (n == "add" ? x[i] + y[i] : x[i] - y[i]);
+                    else
+                        MIGRAPHX_THROW("oracle: " + n + " on " + out.type_string());
+                }
+            });
+        }
+        else
+        {
+            MIGRAPHX_THROW("oracle: no implementation of " + n);
+        }
+        return r;
+    }
+};
+
+} // namespace
+
+void lowering::apply(migraphx::module& m) const
+{
+    std::vector<migraphx::instruction_ref> all;
+    for(auto it = m.begin(); it != m.end(); ++it)
+        all.push_back(it);
+    for(auto ins : all)
+    {
+        const auto n = ins->name();
+        if(n[0] == '@' or n == "capture" or n == "reshape" or n == "contiguous")
+            continue;
+        if(ins->get_operator().is_context_free())
+            continue; // views
+        m.replace_instruction(ins, migraphx::operation{cpu_op{ins->get_operator()}}, ins->inputs());
+    }
+}
+
+std::vector<migraphx::pass> target::get_passes(migraphx::context&,
+                                               const migraphx::compile_options&) const
+{
+    return {lowering{}, migraphx::dead_code_elimination{}};
+}
+
+} // namespace oracle
+
+MIGRAPHX_REGISTER_TARGET(oracle::target);
