@@ -54,13 +54,16 @@ instruction_ref make_param(module& m, instruction_ref ins, instruction_ref p)
     return m.insert_instruction(ins, operation{contiguous{}}, p, out);
 }
 
-// value of a constant that is one element behind its broadcasts
+// value of a constant whose elements all are the same behind its broadcasts
 bool scalar_constant(instruction_ref i, int64_t& v)
 {
     auto base = skip_broadcasts(i);
-    if(not base->can_eval() or base->get_shape().elements() != 1)
+    if(not base->can_eval() or base->get_shape().elements() == 0)
         return false;
-    v = base->eval().to_vector<int64_t>().front();
+    auto vals = base->eval().to_vector<int64_t>();
+    if(not std::all_of(vals.begin(), vals.end(), [&](int64_t x) { return x == vals.front(); }))
+        return false;
+    v = vals.front();
     return true;
 }
 
@@ -406,8 +409,6 @@ void lower_instruction(module& m, instruction_ref ins)
     }
     else if(name == "dot")
     {
-        if(lower_w4a16(m, ins))
-            return;
         m.replace_instruction(ins, operation{dot{}}, ins->inputs()[0], ins->inputs()[1], standard_out());
     }
     else if(name == "quantizelinear" or name == "dequantizelinear")
@@ -527,7 +528,12 @@ void lowering::apply(module& m) const
         MIGRAPHX_THROW("mi355::lowering: no context");
     // 1. fused patterns; what they absorb dies
     for(auto ins : all_instructions(m))
-        fuse_quant_dot_dq(m, ins);
+    {
+        if(ins->name() == "dot")
+            lower_w4a16(m, ins);
+        else
+            fuse_quant_dot_dq(m, ins);
+    }
     dead_code_elimination{}.apply(m);
     // 2. everything else, one operator at a time
     for(auto ins : all_instructions(m))
