@@ -389,6 +389,8 @@ int launch_gemv_m1(const w4_params& p, hipStream_t s)
     return mi355_launch_status();
 }
 
+#include "w4a16_mfma.h"
+
 } // namespace
 
 extern "C" int mi355_w4a16_gemm(const void* a,
@@ -446,6 +448,8 @@ extern "C" int mi355_w4a16_gemm(const void* a,
     if(m == 1 && zp_mode == MI355_W4_ZP_SCALAR && k % 2048 == 0 && k <= GV_MAX_K &&
        (group & (group - 1)) == 0 && group <= 2048)
         return launch_gemv_m1(p, s);
+    if(m >= 2 && mfma_gemm_supported(p))
+        return launch_mfma_gemm(p, s);
     dim3 grid((unsigned)((n + 3) / 4));
     if(m == 1)
         hipLaunchKernelGGL(w4a16_gemv_kernel<1>, grid, dim3(W4_THREADS), 0, s, p);
