@@ -6,12 +6,16 @@
 // dequantized there; activations come from L2.
 //
 // Work split: a workgroup owns 16 output columns (weight rows n0 .. n0+15) for all M rows.  Its
-// NW waves split K between them in steps of 128: wave w takes steps w, w + NW, ...  In a step,
-// lane l = 16*kg + n holds the 32 weights W[n0+n, 128*t + 32*kg .. +32] (one 16-byte load) -- four
-// B operands of v_mfma_f32_16x16x32_f16 (8 consecutive k each) once dequantized.  The matching A
-// operand of M-tile i is A[16*i + (l & 15), same 8 k], a 16-byte load.  Each wave accumulates
-// its K share in fp32; the NW partial tiles are added through LDS in wave order, so the result
-// does not depend on timing.
+// NW waves split K between them in steps of 128 (runs of WM_DEPTH consecutive steps per wave).  In
+// a step, lane l = 16*kg + n loads the 32 weights W[n0+n, 128*t + 32*kg .. +32] with one 16-byte
+// load, so a wave instruction reads 64 contiguous bytes of each of its 16 rows.  The four dwords
+// are then transposed across the four 16-lane rows of the wave (v_permlane32_swap,
+// v_permlane16_swap: four instructions), after which dword j of lane-row kg holds the 8 weights
+// k = 128*t + 32*j + 8*kg .. +8: the B operand of the j-th v_mfma_f32_16x16x32_f16.  The matching
+// A operand of M-tile i is A[16*i + (l & 15), same 8 k]: for a given j the four lane-rows read 64
+// contiguous bytes of an activation row, so these loads use whole cache-line halves as well.
+// Each wave accumulates its K share in fp32; the NW partial tiles are added through LDS in wave
+// order, so the result does not depend on timing.
 //
 // Dequantization, two weights per instruction, in natural k order (the A operand needs no
 // shuffle): byte r of a dword (nibbles 2r, 2r+1) is copied to bytes 0 and 2 of a register with
@@ -24,7 +28,10 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int WM_DEPTH = 4; // weight loads in flight per lane
 
-template <int MT, int NW>
+// SIMPLE: one zero point for the tensor and a group size that is a multiple of 128, so a step
+// needs one scale and no zero-point loads (the MatMulNBits default); the general form looks
+// both up for each 32-k quarter of a step.
+template <int MT, int NW, bool SIMPLE>
 __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
 {
     __shared__ float red[NW][MT * 4][64];
@@ -43,20 +50,23 @@ __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
     // the fp32 accumulation of the matrix cores keeps round-to-nearest
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 2, 2), 3" ::: "memory");
 
-    const uint8_t* wrow   = p.w + (int64_t)n * kbytes + kg * 16;
+    // uniform base pointers plus 32-bit lane offsets keep the address arithmetic short
+    const uint8_t* wbase  = p.w;
+    const uint32_t woff   = (uint32_t)n * (uint32_t)kbytes + kg * 16;
     const uint16_t* srow  = p.scales + (int64_t)n * groups;
     const int zrow_groups = p.zp_mode == MI355_W4_ZP_PACKED ? (groups + 1) / 2 : groups;
     const uint8_t* zrow   = p.zp_mode == MI355_W4_ZP_SCALAR ? nullptr : p.zp + (int64_t)n * zrow_groups;
 
     // activation rows of this lane, clamped so that every load is in bounds; rows past M are
     // computed and dropped
-    const uint16_t* arow[MT];
+    const uint8_t* abase = reinterpret_cast<const uint8_t*>(p.a);
+    uint32_t aoff[MT];
 #pragma unroll
     for(int i = 0; i < MT; i++)
     {
         int r   = 16 * i + nl;
         r       = r < p.m ? r : p.m - 1;
-        arow[i] = p.a + (int64_t)r * p.lda + kg * 32;
+        aoff[i] = ((uint32_t)r * (uint32_t)p.lda + kg * 8) * 2;
     }
 
     v4f acc[MT];
@@ -65,56 +75,107 @@ __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
         acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
 
     v4u wbuf[WM_DEPTH];
-    uint16_t sbuf[WM_DEPTH];
-    uint8_t zbuf[WM_DEPTH];
-    int t_ld = wave;
-    auto issue = [&](int slot) {
-        if(t_ld < nsteps)
+    uint16_t sbuf[WM_DEPTH][4];
+    uint8_t zbuf[WM_DEPTH][4];
+    // the four 32-k quarters of a step share one scale when the group size is a multiple of 128
+    const bool one_group = SIMPLE || (p.group & 127) == 0;
+    auto step_of = [&](int round, int u) { return (round * NW + wave) * WM_DEPTH + u; };
+    auto issue = [&](int slot, int t) {
+        if(t < nsteps)
         {
-            wbuf[slot]  = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(wrow + t_ld * 64));
-            const int g = (t_ld * 128 + kg * 32) / p.group;
-            sbuf[slot]  = srow[g];
-            uint8_t z   = (uint8_t)p.zp_scalar;
-            if(p.zp_mode == MI355_W4_ZP_GROUP)
-                z = zrow[g];
-            else if(p.zp_mode == MI355_W4_ZP_PACKED)
+            wbuf[slot] = __builtin_nontemporal_load(
+                reinterpret_cast<const v4u*>(wbase + (woff + (uint32_t)t * 64)));
+#pragma unroll
+            for(int j = 0; j < 4; j++)
             {
-                const uint8_t zb = zrow[g >> 1];
-                z                = (g & 1) ? (zb >> 4) : (zb & 0xf);
+                if(j > 0 && one_group)
+                {
+                    sbuf[slot][j] = sbuf[slot][0];
+                    zbuf[slot][j] = zbuf[slot][0];
+                    continue;
+                }
+                const int g   = (t * 128 + j * 32) / p.group;
+                sbuf[slot][j] = srow[g];
+                uint8_t z     = (uint8_t)p.zp_scalar;
+                if(SIMPLE)
+                {
+                }
+                else if(p.zp_mode == MI355_W4_ZP_GROUP)
+                    z = zrow[g];
+                else if(p.zp_mode == MI355_W4_ZP_PACKED)
+                {
+                    const uint8_t zb = zrow[g >> 1];
+                    z                = (g & 1) ? (zb >> 4) : (zb & 0xf);
+                }
+                zbuf[slot][j] = z;
             }
-            zbuf[slot] = z;
         }
-        t_ld += NW;
     };
 #pragma unroll
     for(int u = 0; u < WM_DEPTH; u++)
-        issue(u);
+        issue(u, step_of(0, u));
 
     uint32_t pair_mask = 0x00F0000Fu, lo_mask = 0x000F000Fu, magic = 0x64006400u;
     asm volatile("" : "+v"(pair_mask), "+v"(lo_mask), "+v"(magic));
 
-    auto consume = [&](int slot, int t) {
-        const uint32_t sb    = sbuf[slot];
-        const uint32_t z     = zbuf[slot];
-        const uint32_t wa[4] = {wbuf[slot].x, wbuf[slot].y, wbuf[slot].z, wbuf[slot].w};
-        const uint32_t sexp  = (sb >> 10) & 0x1fu;
-        // wave-uniform choice; the separate-nibble form is right for any scale
-        const bool fast = __builtin_amdgcn_ballot_w64(sexp >= 5 && sexp <= 30) == ~0ull;
-        h2 zoff, scv;
-        if(fast)
+    // Activation operands.  Up to two M-tiles: the operands of the wave's next step are loaded
+    // while the current step is computed (two register sets).  More tiles: all operands of a
+    // step are requested before its first MFMA, so the loads overlap one another.
+    constexpr bool A_AHEAD = MT <= 2;
+    v8h abuf[A_AHEAD ? 2 : 1][4][MT];
+    auto load_a = [&](int set, int t) {
+        if(t < nsteps)
         {
-            zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | (z << 4)) << 16));
-            scv  = __builtin_bit_cast(h2, sb | ((sb - (4u << 10)) << 16));
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+#pragma unroll
+                for(int i = 0; i < MT; i++)
+                    abuf[set][j][i] = *reinterpret_cast<const v8h*>(
+                        abase + (aoff[i] + (uint32_t)t * 256 + j * 64));
         }
+    };
+    if(A_AHEAD)
+        load_a(0, step_of(0, 0));
+
+    auto consume = [&](int slot, int t, int t_next) {
+        const int set = A_AHEAD ? (slot & 1) : 0;
+        if(A_AHEAD)
+            load_a(set ^ 1, t_next);
         else
+            load_a(0, t);
+        // 4 x 4 transpose of the dwords over the wave's 16-lane rows: afterwards wa[j] of
+        // lane-row kg is what lane-row j loaded as dword kg
+        uint32_t wa[4] = {wbuf[slot].x, wbuf[slot].y, wbuf[slot].z, wbuf[slot].w};
         {
-            zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | z) << 16));
-            scv  = __builtin_bit_cast(h2, sb | (sb << 16));
+            auto s02 = __builtin_amdgcn_permlane32_swap(wa[0], wa[2], false, false);
+            auto s13 = __builtin_amdgcn_permlane32_swap(wa[1], wa[3], false, false);
+            auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+            auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+            wa[0]    = t01[0];
+            wa[1]    = t01[1];
+            wa[2]    = t23[0];
+            wa[3]    = t23[1];
         }
 #pragma unroll
         for(int j = 0; j < 4; j++)
         {
-            // B operand: the 8 weights k = 128*t + 32*kg + 8*j .. +8 of column n
+            const uint32_t sb   = sbuf[slot][j];
+            const uint32_t z    = zbuf[slot][j];
+            const uint32_t sexp = (sb >> 10) & 0x1fu;
+            // wave-uniform choice; the separate-nibble form is right for any scale
+            const bool fast = __builtin_amdgcn_ballot_w64(sexp >= 5 && sexp <= 30) == ~0ull;
+            h2 zoff, scv;
+            if(fast)
+            {
+                zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | (z << 4)) << 16));
+                scv  = __builtin_bit_cast(h2, sb | ((sb - (4u << 10)) << 16));
+            }
+            else
+            {
+                zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | z) << 16));
+                scv  = __builtin_bit_cast(h2, sb | (sb << 16));
+            }
+            // B operand: the 8 weights k = 128*t + 32*j + 8*kg .. +8 of column n
             h2 x[4];
 #pragma unroll
             for(int r = 0; r < 4; r++)
@@ -143,22 +204,22 @@ __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
 #pragma unroll
             for(int i = 0; i < MT; i++)
             {
-                const v8h afrag = *reinterpret_cast<const v8h*>(arow[i] + t * 128 + j * 8);
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(abuf[set][j][i], bfrag, acc[i], 0, 0, 0);
             }
         }
     };
 
-    for(int t = wave; t < nsteps; t += NW * WM_DEPTH)
+    const int rounds = (nsteps + NW * WM_DEPTH - 1) / (NW * WM_DEPTH);
+    for(int round = 0; round < rounds; round++)
     {
 #pragma unroll
         for(int u = 0; u < WM_DEPTH; u++)
         {
-            const int tt = t + u * NW;
+            const int tt = step_of(round, u);
             if(tt < nsteps)
             {
-                consume(u, tt);
-                issue(u);
+                consume(u, tt, u + 1 < WM_DEPTH ? step_of(round, u + 1) : step_of(round + 1, 0));
+                issue(u, step_of(round + 1, u));
             }
         }
     }
@@ -187,7 +248,9 @@ __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
 
 bool mfma_gemm_supported(const w4_params& p)
 {
-    return p.n % 16 == 0 && p.k % 128 == 0 && p.m >= 1;
+    // lane offsets are 32-bit
+    return p.n % 16 == 0 && p.k % 128 == 0 && p.m >= 1 && (int64_t)p.n * p.k / 2 < (1ll << 31) &&
+           (int64_t)p.m * p.lda * 2 < (1ll << 31);
 }
 
 template <int MT>
@@ -195,10 +258,19 @@ int launch_mfma_tiles(const w4_params& p, hipStream_t s)
 {
     const int grid = p.n / 16;
     // few column tiles: more waves per workgroup keep enough weight loads in flight
-    if(grid < 512 && (p.k >> 7) >= 32 && MT <= 4)
-        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 16>), dim3(grid), dim3(1024), 0, s, p);
+    const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
+    if constexpr(MT == 1)
+    {
+        if(grid < 512 && (p.k >> 7) >= 32 && simple)
+        {
+            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 16, true>), dim3(grid), dim3(1024), 0, s, p);
+            return mi355_launch_status();
+        }
+    }
+    if(simple)
+        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 8, true>), dim3(grid), dim3(512), 0, s, p);
     else
-        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 8>), dim3(grid), dim3(512), 0, s, p);
+        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 8, false>), dim3(grid), dim3(512), 0, s, p);
     return mi355_launch_status();
 }
 
