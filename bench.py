@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 PEAK_TOPS_INT8 = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_TFLOPS_FP8 = 5000.0  # dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes one 8192^3 int8 quant_dot launch moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# counter runs of this file scaled by the same counters' reading for a plain copy of known size
+# (profiles/quant_dot_int8_8192_hbm_traffic.md holds both runs and the arithmetic).
+HEADLINE_TRAFFIC_BYTES = 1.1128e9
 
 
 def _time_launches(fn, steps, warmup):
@@ -67,6 +71,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=768)
+    ap.add_argument("--only-headline", action="store_true",
+                    help="time the headline kernel only (for counter runs under rocprofv3)")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, run a plain device copy of MIB mebibytes a few "
+                         "times: the HBM counters of that kernel calibrate roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -77,6 +86,16 @@ def main():
     dev = "cuda:0"
     g = torch.Generator(device=dev)
     g.manual_seed(0)
+
+    if args.copy_calibration > 0:
+        n = args.copy_calibration << 20
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=dev, generator=g)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes": n, "launches": 5}))
+        return
 
     # ---- headline: int8 quant_dot 8192^3 -> int32 --------------------------------
     M = N = K = 8192
@@ -95,6 +114,8 @@ def main():
     also = {}
     # ---- fp8 quant_dot with dequant epilogue, Llama-3-8B shape (config 3) ----------
     try:
+        if args.only_headline:
+            raise RuntimeError("skipped (--only-headline)")
         m3, k3, n3 = 4096, 4096, 14336 * 2
         a8 = torch.randint(0, 0x7e, (m3, k3), dtype=torch.uint8, device=dev, generator=g)
         b8 = torch.randint(0, 0x7e, (k3, n3), dtype=torch.uint8, device=dev, generator=g)
@@ -117,6 +138,8 @@ def main():
     # kernel plus the device-side gap between dependent kernels (about 2.6 us for
     # an empty kernel on this machine), not the host's submission rate.
     try:
+        if args.only_headline:
+            raise RuntimeError("skipped (--only-headline)")
         for (k4, n4) in ((4096, 4096), (4096, 14336), (14336, 4096)):
             grp = 128
             bytes_per = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * k4 + 2 * n4
@@ -157,7 +180,7 @@ def main():
                    "m": M, "n": N, "k": K},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_TOPS_INT8,
                      "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
-                     "traffic": None},
+                     "traffic": HEADLINE_TRAFFIC_BYTES},
         "also": also,
     }
     if not args.no_cpu:
