@@ -56,6 +56,7 @@ struct dma_params
     const int32_t* rowsum_a;
     int scale_a_mode, scale_b_mode;
     int zp_a, zp_b;
+    int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
 };
 
 // s_waitcnt with only the vector-memory counter constrained
@@ -521,9 +522,15 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 // steps and double buffered across slabs, so the loop body exists for both
 // slab parities.
 // ---------------------------------------------------------------------------
-template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE>
+// SPLITK (bare int32 result only): blockIdx.z selects a share of the K slabs and the tile is
+// added into a zero-filled C with integer atomics.  Integer addition commutes, so the result is
+// the same bits whatever order the workgroups finish in.  This is what fills the machine when a
+// skinny problem (few rows of A against a large B) has too few output tiles; 16-row tiles past the
+// last row of A are skipped in the MFMA steps.
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE, bool SPLITK = false>
 __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 {
+    static_assert(!SPLITK || !DEQ, "split-K adds raw accumulators");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid    = threadIdx.x;
@@ -539,6 +546,21 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 
     const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
     const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+    int nk = p.k / BK;
+    if constexpr(SPLITK)
+    {
+        // slabs [s0, s1) of this workgroup
+        const int per = (nk + p.ksplit - 1) / p.ksplit;
+        const int s0  = min((int)blockIdx.z * per, nk);
+        const int s1  = min(s0 + per, nk);
+        ga += (int64_t)s0 * BK;
+        gb += TRANS_B ? (int64_t)s0 * BK : (int64_t)s0 * BK * p.ldb;
+        nk = s1 - s0;
+        if(nk <= 0)
+            return;
+    }
+    // 16-row tiles of this wave's 128-row block that hold rows of A
+    const int live_tiles = SPLITK ? max(0, min(8, (p.m - (m0 + wave_m * 128) + 15) / 16)) : 8;
 
     // ---- global -> LDS (identical to the kernel above) ------------------------
     uint32_t a_off[2], b_off[2];
@@ -665,9 +687,12 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     {                                                                                       \
         _Pragma("unroll") for(int i_ = 0; i_ < 4; i_++)                                     \
         {                                                                                   \
-            _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++) acc[4 * (S) + i_][j_] =         \
-                __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[P][j_], fa[S][i_],                \
-                                                      acc[4 * (S) + i_][j_], 0, 0, 0);      \
+            if(!SPLITK || 4 * (S) + i_ < live_tiles)                                        \
+            {                                                                               \
+                _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++) acc[4 * (S) + i_][j_] =     \
+                    __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[P][j_], fa[S][i_],            \
+                                                          acc[4 * (S) + i_][j_], 0, 0, 0);  \
+            }                                                                               \
         }                                                                                   \
     } while(0)
     // one slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P]
@@ -698,7 +723,6 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     } while(0)
 
     // ---- main loop (see the kernel above for the ordering argument) ----------
-    const int nk = p.k / BK;
 #pragma unroll
     for(int s = 0; s < STAGES - 1; s++)
         if(s < nk)
@@ -762,7 +786,14 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             if constexpr(!DEQ)
             {
                 int32_t* o = static_cast<int32_t*>(p.c) + idx;
-                if constexpr(VEC_STORE)
+                if constexpr(SPLITK)
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        __hip_atomic_fetch_add(o + e, acc[i][j][e], __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                }
+                else if constexpr(VEC_STORE)
                     *reinterpret_cast<v4i*>(o) = acc[i][j];
                 else
                 {
@@ -829,6 +860,52 @@ int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
     dim3 grid(p.tiles_m * p.tiles_n, batch);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
     return mi355_launch_status();
+}
+
+// zero C ahead of the split-K kernel (a kernel rather than a memset so that a captured graph
+// replays it faithfully)
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* c, int m, int n, int64_t ldc, int64_t stride_c)
+{
+    int32_t* base   = c + (int64_t)blockIdx.y * stride_c;
+    const int64_t t = (int64_t)m * n;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < t; i += (int64_t)gridDim.x * 256)
+        base[(i / n) * ldc + (i % n)] = 0;
+}
+
+template <bool TRANS_B>
+int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream)
+{
+    auto kern = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true>;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if(attr != hipSuccess)
+        return MI355_ERR_LAUNCH;
+    const int64_t total = (int64_t)p.m * p.n;
+    const int zb        = (int)min((int64_t)2048, (total + 255) / 256);
+    hipLaunchKernelGGL(zero_i32_kernel, dim3(zb, batch), dim3(256), 0, stream,
+                       static_cast<int32_t*>(p.c), p.m, p.n, p.ldc, p.stride_c);
+    dim3 grid(p.tiles_m * p.tiles_n, batch, p.ksplit);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+    return mi355_launch_status();
+}
+
+// K shares per tile for a bare int8 quant_dot whose tiles alone leave most of the 256 CUs idle;
+// 1 = no split.  Measured on this kernel: one workgroup streams its operands at about 25 GB/s, and
+// the atomic adds of a share cost about 11.5 us per 2^20 outputs, so the time is roughly
+// T1 / S + c * S with T1 = operand bytes / (workgroups * 25 GB/s) and c = 11.5 us * outputs / 2^20;
+// the minimum is at sqrt(T1 / c).
+int choose_ksplit(int tiles, int batch, int nk, int64_t m, int64_t n, int64_t k)
+{
+    const int64_t wgs = (int64_t)tiles * batch;
+    if(wgs >= 128 || nk < 8)
+        return 1;
+    const double bytes = (double)batch * ((double)m * k + (double)k * n);
+    const double t1_us = bytes / ((double)wgs * 25e3);
+    const double c_us  = 11.5 * (double)batch * (double)m * (double)n / 1048576.0;
+    int s              = (int)(0.75 * __builtin_sqrt(t1_us / c_us));
+    s                  = min(s, nk / 4); // at least four slabs per share keep the LDS ring busy
+    s                  = min((int64_t)s, (512 + wgs - 1) / wgs);
+    return max(s, 1);
 }
 
 template <bool TRANS_B, bool VEC>
@@ -947,6 +1024,14 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
         // the 16 x 16 kernel drops or keeps 4 columns together
         return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+    p.ksplit = 1;
+    if(vec && !deq)
+    {
+        p.ksplit = choose_ksplit(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);
+        if(p.ksplit > 1)
+            return d->trans_b ? launch_i8_splitk<true>(p, (int)d->batch, stream)
+                              : launch_i8_splitk<false>(p, (int)d->batch, stream);
+    }
     if(vec)
         return d->trans_b ? launch_i8_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_i8_out<false, true>(p, (int)d->batch, deq, d->out_type, stream);

@@ -85,8 +85,17 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
         odt = torch.float32 if fp8 else torch.int32
     if out is None:
         out = torch.empty(batch_shape + (m, n), dtype=odt, device=a.device)
-    d = QuantDotDesc(m=m, n=n, k=k, lda=lda, ldb=ldb, ldc=n, batch=nb, stride_a=sa, stride_b=sb,
-                     stride_c=m * n, trans_a=ta, trans_b=tb, in_type=in_type,
+    # C may be a row-strided view (columns contiguous, batches evenly spaced)
+    if out.stride(-1) != 1 and n > 1:
+        raise Mi355Error("quant_dot: the output's last dimension must be contiguous")
+    ldc = out.stride(-2) if m > 1 else max(n, out.stride(-2))
+    stride_c = m * ldc
+    if out.dim() > 2 and nb > 1:
+        if out.dim() > 3 and not out.flatten(0, -3).is_contiguous():
+            raise Mi355Error("quant_dot: batch dimensions of the output must be dense")
+        stride_c = out.stride(-3)
+    d = QuantDotDesc(m=m, n=n, k=k, lda=lda, ldb=ldb, ldc=ldc, batch=nb, stride_a=sa, stride_b=sb,
+                     stride_c=stride_c, trans_a=ta, trans_b=tb, in_type=in_type,
                      out_type=_TORCH2DT[odt], dequant=int(dequant),
                      scale_a_mode=QP.NONE if scale_a is None else
                      (QP.PER_TENSOR if scale_a.numel() == 1 else QP.PER_ROW),

@@ -62,6 +62,39 @@ def test_int8_accumulators_bit_exact(ops, m, n, k, trans_b):
     assert np.array_equal(got, want)
 
 
+# few output tiles and a long K: the split-K form of the kernel (shares of K added into C with
+# integer atomics) must still be bit-exact, for any split remainder and for rows past M
+SKINNY = [(16, 8192, 8192), (128, 2048, 4096), (1, 256, 2048), (37, 512, 1088), (300, 260, 1024),
+          (1024, 1024, 1024), (16, 768, 576)]
+
+
+@pytest.mark.parametrize("m,n,k", SKINNY)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_int8_skinny_split_k_bit_exact(ops, m, n, k, trans_b):
+    rng = np.random.default_rng(m + n * 5 + k * 11)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    want = orc.quant_dot(a, b, orc.I8)
+    tb = dev(np.ascontiguousarray(b.T)).t() if trans_b else dev(b)
+    print("skinny", m, n, k, trans_b, flush=True)
+    out = torch.full((m, n + 4), 7, dtype=torch.int32, device="cuda")
+    # a second call into the same buffer must not accumulate on top of the first
+    for _ in range(2):
+        ops.quant_dot(dev(a), tb, out=out[:, :n])
+    assert np.array_equal(out[:, :n].cpu().numpy(), want)
+    assert (out[:, n:] == 7).all()
+
+
+def test_int8_skinny_batched(ops):
+    rng = np.random.default_rng(5)
+    bt, m, n, k = 3, 24, 256, 1536
+    a = rng.integers(-128, 128, (bt, m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (bt, k, n), dtype=np.int8)
+    want = orc.quant_dot(a, b, orc.I8)
+    got = ops.quant_dot(dev(a), dev(b)).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 def test_int8_extremes_and_batch(ops):
     a = np.full((2, 256, 512), -128, np.int8)
     b = np.full((2, 512, 256), -128, np.int8)
