@@ -1,62 +1,116 @@
-// int4 weight-only GEMM for 2 <= M <= 128 on the matrix cores (included by w4a16.hip inside its
-// anonymous namespace).
+// int4 weight-only GEMM for M >= 2 on the matrix cores (included by w4a16.hip inside its anonymous
+// namespace).
 //
-// The shapes are still bound by the weight stream (K*N/2 bytes against 2*M*N*K flops), so the
-// weights are read once, in 16-byte loads, straight into the register layout the MFMA wants and
-// dequantized there; activations come from L2.
+// The shapes are bound by the weight stream (K*N/2 bytes against 2*M*N*K flops), so the weights are
+// read exactly once, in the largest contiguous pieces the layout allows, and dequantized in
+// registers; activations come from L2.
 //
-// Work split: a workgroup owns 16 output columns (weight rows n0 .. n0+15) for all M rows.  Its
-// NW waves split K between them in steps of 128 (runs of WM_DEPTH consecutive steps per wave).  In
-// a step, lane l = 16*kg + n loads the 32 weights W[n0+n, 128*t + 32*kg .. +32] with one 16-byte
-// load, so a wave instruction reads 64 contiguous bytes of each of its 16 rows.  The four dwords
-// are then transposed across the four 16-lane rows of the wave (v_permlane32_swap,
-// v_permlane16_swap: four instructions), after which dword j of lane-row kg holds the 8 weights
-// k = 128*t + 32*j + 8*kg .. +8: the B operand of the j-th v_mfma_f32_16x16x32_f16.  The matching
-// A operand of M-tile i is A[16*i + (l & 15), same 8 k]: for a given j the four lane-rows read 64
-// contiguous bytes of an activation row, so these loads use whole cache-line halves as well.
-// Each wave accumulates its K share in fp32; the NW partial tiles are added through LDS in wave
-// order, so the result does not depend on timing.
+// Work split.  A workgroup owns 16*NT output columns (weight rows n0 ..) for up to 128 rows of A.  It
+// has 8 compute waves and one fetch wave.  K is walked in chunks of 2048: every weight row
+// contributes 1 KiB to a chunk, fetched by ONE global_load_lds instruction (64 lanes x 16 bytes,
+// contiguous in memory) straight into an LDS ring of RING chunks; RING-1 chunks stay in flight.  The
+// fetch wave issues all of these and is the only wave whose vector-memory counter they occupy:
+// memory operations of a wave complete in order, so a compute wave that issued ring loads would
+// have every activation load queue behind a weight fetch still on its way from HBM.  Inside a
+// chunk the 16 steps of 128 k are dealt to the compute waves (wave w: steps w and w + 8).  For a step and a 16-column tile, lane
+// l = 16*kg + n reads its 16 bytes W[n, 128*t + 32*kg .. +32] from LDS (row pitch 1040 bytes: the 16
+// rows of a quarter wave fall into distinct banks), the four dwords are transposed across the wave's
+// 16-lane rows (v_permlane32_swap, v_permlane16_swap), and dword j of lane-row kg then holds the 8
+// weights k = 128*t + 32*j + 8*kg .. +8: the B operand of the j-th v_mfma_f32_16x16x32_f16.  The
+// matching A operand of M-tile i is A[16*i + (l & 15), same 8 k], a 16-byte load; for a given j
+// the four lane-rows read 64 contiguous bytes of an activation row.  With NT = 2 one A operand
+// feeds two column tiles.  Each wave accumulates its K share in fp32; the 8 partial tiles are added
+// through LDS in wave order, so the result does not depend on timing.
 //
-// Dequantization, two weights per instruction, in natural k order (the A operand needs no
-// shuffle): byte r of a dword (nibbles 2r, 2r+1) is copied to bytes 0 and 2 of a register with
-// v_perm_b32; (t & 0x00f0000f) | 0x64006400 then reads as the halves (1024 + q0, 1024 + 16*q1).
-// Subtracting (1024 + zp, 1024 + 16*zp) is exact, and the packed multiply by (s, s/16) under
-// round-toward-zero forms (q - zp) * s with the single truncation of the reference's
-// float -> half store.  s/16 must be a normal half (exponent field of s at least 5); a wave that
-// meets a smaller scale unpacks the high nibble separately instead.
+// Dequantization, two weights per instruction, in natural k order: byte r of a dword (nibbles 2r,
+// 2r+1) is copied to bytes 0 and 2 of a register with v_perm_b32; (t & 0x00f0000f) | 0x64006400
+// then reads as the halves (1024 + q0, 1024 + 16*q1).  Subtracting (1024 + zp, 1024 + 16*zp) is
+// exact, and the packed multiply by (s, s/16) under round-toward-zero forms (q - zp) * s with the
+// single truncation of the reference's float -> half store.  s/16 must be a normal half (exponent
+// field of s at least 5); a wave that meets a smaller scale unpacks the high nibble separately.
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
-constexpr int WM_DEPTH = 4; // weight loads in flight per lane
+constexpr int WL_CHUNK_K = 2048;                  // k per chunk
+constexpr int WL_ROW     = WL_CHUNK_K / 2;        // bytes of one weight row in a chunk
+constexpr int WL_PITCH   = WL_ROW + 16;           // LDS row pitch
+constexpr int WL_WAVES   = 8;                     // compute waves; one more wave fetches
+constexpr int WL_THREADS = (WL_WAVES + 1) * 64;
+
+MI355_DEVINL void wl_load_to_lds(const uint8_t* g, uint8_t* l)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g),
+                                     (__attribute__((address_space(3))) void*)(l), 16, 0, 0);
+}
+
+template <int N>
+MI355_DEVINL void wl_wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64);
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+MI355_DEVINL void wl_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 // SIMPLE: one zero point for the tensor and a group size that is a multiple of 128, so a step
-// needs one scale and no zero-point loads (the MatMulNBits default); the general form looks
-// both up for each 32-k quarter of a step.
-template <int MT, int NW, bool SIMPLE>
-__global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
+// needs one scale and no zero-point loads (the MatMulNBits default); the general form looks both
+// up for each 32-k quarter of a step.
+template <int MT, int NT, bool SIMPLE>
+__global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
 {
-    __shared__ float red[NW][MT * 4][64];
+    constexpr int RING        = NT == 1 ? 4 : 3;
+    constexpr int CHUNK_BYTES = 16 * NT * WL_PITCH;
+    constexpr int RED_BYTES   = WL_WAVES * NT * MT * 4 * 64 * 4;
+    constexpr int LDS_BYTES   = RING * CHUNK_BYTES > RED_BYTES ? RING * CHUNK_BYTES : RED_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
+
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl   = lane & 15;
     const int kg   = lane >> 4;
-    const int n0   = blockIdx.x * 16;
-    const int n    = n0 + nl;
-    const int kbytes = p.k >> 1;
-    const int groups = p.k / p.group;
-    const int nsteps = p.k >> 7;
+    const int n0   = blockIdx.x * (16 * NT);
+    const int kbytes  = p.k >> 1;
+    const int groups  = p.k / p.group;
+    const int nsteps  = p.k >> 7;
+    const int nchunks = (p.k + WL_CHUNK_K - 1) / WL_CHUNK_K;
 
-    // half-precision arithmetic of this wave truncates from here on (MODE.fp_round bits 3:2);
-    // the fp32 accumulation of the matrix cores keeps round-to-nearest
+    // half-precision arithmetic of this wave truncates from here on (MODE.fp_round bits 3:2); the
+    // fp32 accumulation of the matrix cores keeps round-to-nearest
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 2, 2), 3" ::: "memory");
 
-    // uniform base pointers plus 32-bit lane offsets keep the address arithmetic short
-    const uint8_t* wbase  = p.w;
-    const uint32_t woff   = (uint32_t)n * (uint32_t)kbytes + kg * 16;
-    const uint16_t* srow  = p.scales + (int64_t)n * groups;
-    const int zrow_groups = p.zp_mode == MI355_W4_ZP_PACKED ? (groups + 1) / 2 : groups;
-    const uint8_t* zrow   = p.zp_mode == MI355_W4_ZP_SCALAR ? nullptr : p.zp + (int64_t)n * zrow_groups;
+    // ---- weight stream: global -> LDS ring ----------------------------------------------------
+    // one instruction per weight row; lanes past the end of K in the last chunk stay off
+    const uint8_t* wbase = p.w + (int64_t)n0 * kbytes;
+    auto issue_chunk     = [&](int c) {
+        uint8_t* slot   = lds + (c % RING) * CHUNK_BYTES;
+        const int valid = min(WL_ROW, kbytes - c * WL_ROW);
+        if(lane * 16 < valid)
+        {
+#pragma unroll
+            for(int r = 0; r < 16 * NT; r++)
+                wl_load_to_lds(wbase + (int64_t)r * kbytes + c * WL_ROW + lane * 16,
+                               slot + r * WL_PITCH);
+        }
+    };
 
+    // ---- per-lane constants ---------------------------------------------------------------------
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    const uint32_t w_lane = nl * WL_PITCH + kg * 16;
+    const uint16_t* srow[NT];
+    const uint8_t* zrow[NT];
+#pragma unroll
+    for(int t = 0; t < NT; t++)
+    {
+        const int n           = n0 + 16 * t + nl;
+        srow[t]               = p.scales + (int64_t)n * groups;
+        const int zrow_groups = p.zp_mode == MI355_W4_ZP_PACKED ? (groups + 1) / 2 : groups;
+        zrow[t] = p.zp_mode == MI355_W4_ZP_SCALAR ? nullptr : p.zp + (int64_t)n * zrow_groups;
+    }
     // activation rows of this lane, clamped so that every load is in bounds; rows past M are
     // computed and dropped
     const uint8_t* abase = reinterpret_cast<const uint8_t*>(p.a);
@@ -69,186 +123,235 @@ __global__ __launch_bounds__(NW * 64) void w4a16_mfma_kernel(w4_params p)
         aoff[i] = ((uint32_t)r * (uint32_t)p.lda + kg * 8) * 2;
     }
 
-    v4f acc[MT];
+    v4f acc[NT][MT];
 #pragma unroll
-    for(int i = 0; i < MT; i++)
-        acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    v4u wbuf[WM_DEPTH];
-    uint16_t sbuf[WM_DEPTH][4];
-    uint8_t zbuf[WM_DEPTH][4];
-    // the four 32-k quarters of a step share one scale when the group size is a multiple of 128
-    const bool one_group = SIMPLE || (p.group & 127) == 0;
-    auto step_of = [&](int round, int u) { return (round * NW + wave) * WM_DEPTH + u; };
-    auto issue = [&](int slot, int t) {
-        if(t < nsteps)
-        {
-            wbuf[slot] = __builtin_nontemporal_load(
-                reinterpret_cast<const v4u*>(wbase + (woff + (uint32_t)t * 64)));
+    for(int t = 0; t < NT; t++)
 #pragma unroll
-            for(int j = 0; j < 4; j++)
-            {
-                if(j > 0 && one_group)
-                {
-                    sbuf[slot][j] = sbuf[slot][0];
-                    zbuf[slot][j] = zbuf[slot][0];
-                    continue;
-                }
-                const int g   = (t * 128 + j * 32) / p.group;
-                sbuf[slot][j] = srow[g];
-                uint8_t z     = (uint8_t)p.zp_scalar;
-                if(SIMPLE)
-                {
-                }
-                else if(p.zp_mode == MI355_W4_ZP_GROUP)
-                    z = zrow[g];
-                else if(p.zp_mode == MI355_W4_ZP_PACKED)
-                {
-                    const uint8_t zb = zrow[g >> 1];
-                    z                = (g & 1) ? (zb >> 4) : (zb & 0xf);
-                }
-                zbuf[slot][j] = z;
-            }
-        }
-    };
-#pragma unroll
-    for(int u = 0; u < WM_DEPTH; u++)
-        issue(u, step_of(0, u));
+        for(int i = 0; i < MT; i++)
+            acc[t][i] = v4f{0.f, 0.f, 0.f, 0.f};
 
     uint32_t pair_mask = 0x00F0000Fu, lo_mask = 0x000F000Fu, magic = 0x64006400u;
     asm volatile("" : "+v"(pair_mask), "+v"(lo_mask), "+v"(magic));
 
-    // Activation operands.  Up to two M-tiles: the operands of the wave's next step are loaded
-    // while the current step is computed (two register sets).  More tiles: all operands of a
-    // step are requested before its first MFMA, so the loads overlap one another.
+    // What a step needs from global memory, requested one step ahead so that the latency runs
+    // under the previous step (and, for a wave's first step, under the first weight fetch): the
+    // scales and zero points of its 32-k quarters and -- with at most two M-tiles, where the registers
+    // allow a second set -- its activation operands.
+    constexpr int NQ       = SIMPLE ? 1 : 4;
     constexpr bool A_AHEAD = MT <= 2;
-    v8h abuf[A_AHEAD ? 2 : 1][4][MT];
-    auto load_a = [&](int set, int t) {
-        if(t < nsteps)
+    struct step_inputs
+    {
+        uint16_t sb[NT][NQ];
+        uint8_t z[NT][NQ];
+        v8h af[A_AHEAD ? 4 : 1][MT];
+    };
+    auto request = [&](step_inputs& in, int step) {
+        if(step >= nsteps)
+            return;
+#pragma unroll
+        for(int t = 0; t < NT; t++)
+#pragma unroll
+            for(int q = 0; q < NQ; q++)
+            {
+                const int g = (step * 128 + q * 32) / p.group;
+                in.sb[t][q] = srow[t][g];
+                uint8_t z   = (uint8_t)p.zp_scalar;
+                if(!SIMPLE)
+                {
+                    if(p.zp_mode == MI355_W4_ZP_GROUP)
+                        z = zrow[t][g];
+                    else if(p.zp_mode == MI355_W4_ZP_PACKED)
+                    {
+                        const uint8_t zb = zrow[t][g >> 1];
+                        z                = (g & 1) ? (zb >> 4) : (zb & 0xf);
+                    }
+                }
+                in.z[t][q] = z;
+            }
+        if(A_AHEAD)
         {
 #pragma unroll
             for(int j = 0; j < 4; j++)
 #pragma unroll
                 for(int i = 0; i < MT; i++)
-                    abuf[set][j][i] = *reinterpret_cast<const v8h*>(
-                        abase + (aoff[i] + (uint32_t)t * 256 + j * 64));
-        }
-    };
-    if(A_AHEAD)
-        load_a(0, step_of(0, 0));
-
-    auto consume = [&](int slot, int t, int t_next) {
-        const int set = A_AHEAD ? (slot & 1) : 0;
-        if(A_AHEAD)
-            load_a(set ^ 1, t_next);
-        else
-            load_a(0, t);
-        // 4 x 4 transpose of the dwords over the wave's 16-lane rows: afterwards wa[j] of
-        // lane-row kg is what lane-row j loaded as dword kg
-        uint32_t wa[4] = {wbuf[slot].x, wbuf[slot].y, wbuf[slot].z, wbuf[slot].w};
-        {
-            auto s02 = __builtin_amdgcn_permlane32_swap(wa[0], wa[2], false, false);
-            auto s13 = __builtin_amdgcn_permlane32_swap(wa[1], wa[3], false, false);
-            auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
-            auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
-            wa[0]    = t01[0];
-            wa[1]    = t01[1];
-            wa[2]    = t23[0];
-            wa[3]    = t23[1];
-        }
-#pragma unroll
-        for(int j = 0; j < 4; j++)
-        {
-            const uint32_t sb   = sbuf[slot][j];
-            const uint32_t z    = zbuf[slot][j];
-            const uint32_t sexp = (sb >> 10) & 0x1fu;
-            // wave-uniform choice; the separate-nibble form is right for any scale
-            const bool fast = __builtin_amdgcn_ballot_w64(sexp >= 5 && sexp <= 30) == ~0ull;
-            h2 zoff, scv;
-            if(fast)
-            {
-                zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | (z << 4)) << 16));
-                scv  = __builtin_bit_cast(h2, sb | ((sb - (4u << 10)) << 16));
-            }
-            else
-            {
-                zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | z) << 16));
-                scv  = __builtin_bit_cast(h2, sb | (sb << 16));
-            }
-            // B operand: the 8 weights k = 128*t + 32*j + 8*kg .. +8 of column n
-            h2 x[4];
-#pragma unroll
-            for(int r = 0; r < 4; r++)
-            {
-                const uint32_t sel = 0x0c000c00u | (uint32_t)r | ((uint32_t)r << 16);
-                const uint32_t tb  = __builtin_amdgcn_perm(wa[j], wa[j], sel);
-                if(fast)
-                    x[r] = __builtin_bit_cast(h2, and_or(tb, pair_mask, magic));
-                else
-                    x[r] = __builtin_bit_cast(
-                        h2, and_or((tb & 0xfu) | ((tb >> 4) & 0x000f0000u), lo_mask, magic));
-            }
-#pragma unroll
-            for(int r = 0; r < 4; r++)
-                x[r] = x[r] - zoff;
-#pragma unroll
-            for(int r = 0; r < 4; r++)
-                x[r] = x[r] * scv;
-            v8h bfrag;
-#pragma unroll
-            for(int r = 0; r < 4; r++)
-            {
-                bfrag[2 * r]     = x[r][0];
-                bfrag[2 * r + 1] = x[r][1];
-            }
-#pragma unroll
-            for(int i = 0; i < MT; i++)
-            {
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(abuf[set][j][i], bfrag, acc[i], 0, 0, 0);
-            }
+                    in.af[A_AHEAD ? j : 0][i] = *reinterpret_cast<const v8h*>(
+                        abase + (aoff[i] + (uint32_t)step * 256 + j * 64));
         }
     };
 
-    const int rounds = (nsteps + NW * WM_DEPTH - 1) / (NW * WM_DEPTH);
-    for(int round = 0; round < rounds; round++)
+    // one step (128 k) of the workgroup's column tiles
+    auto do_step = [&](step_inputs& in, int step, uint32_t slot_addr, int s_in_chunk) {
+        // without the second register set: all operands of the step up front for up to four
+        // M-tiles, per quarter for eight
+        constexpr bool A_UPFRONT = !A_AHEAD && MT <= 4;
+        v8h af_now[A_UPFRONT ? 4 : 1][MT];
+        if(A_UPFRONT)
+        {
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+#pragma unroll
+                for(int i = 0; i < MT; i++)
+                    af_now[A_UPFRONT ? j : 0][i] = *reinterpret_cast<const v8h*>(
+                        abase + (aoff[i] + (uint32_t)step * 256 + j * 64));
+        }
+#pragma unroll
+        for(int t = 0; t < NT; t++)
+        {
+            v4u wv;
+            asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                         : "=v"(wv)
+                         : "v"(slot_addr + w_lane + (uint32_t)(t * 16 * WL_PITCH + s_in_chunk * 64))
+                         : "memory");
+            // 4 x 4 transpose of the dwords over the wave's 16-lane rows: afterwards wa[j] of
+            // lane-row kg is what lane-row j read as dword kg
+            uint32_t wa[4];
+            {
+                auto s02 = __builtin_amdgcn_permlane32_swap(wv.x, wv.z, false, false);
+                auto s13 = __builtin_amdgcn_permlane32_swap(wv.y, wv.w, false, false);
+                auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+                auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+                wa[0]    = t01[0];
+                wa[1]    = t01[1];
+                wa[2]    = t23[0];
+                wa[3]    = t23[1];
+            }
+            // scale and zero point as packed constants: (s, s/16) and (1024 + zp, 1024 + 16*zp) for
+            // the two-nibbles-at-once form, (s, s) and (1024 + zp, 1024 + zp) otherwise.  The choice
+            // is wave-uniform; the separate-nibble form is right for any scale.
+            bool fast = false;
+            h2 zoff = {}, scv = {};
+            auto constants = [&](uint32_t sb, uint32_t z) {
+                const uint32_t sexp = (sb >> 10) & 0x1fu;
+                fast = __builtin_amdgcn_ballot_w64(sexp >= 5 && sexp <= 30) == ~0ull;
+                const uint32_t zhi = fast ? (z << 4) : z;
+                const uint32_t shi = fast ? sb - (4u << 10) : sb;
+                zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | zhi) << 16));
+                scv  = __builtin_bit_cast(h2, sb | (shi << 16));
+            };
+            if(SIMPLE)
+                constants(in.sb[t][0], in.z[t][0]);
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+                if(!SIMPLE)
+                    constants(in.sb[t][SIMPLE ? 0 : j], in.z[t][SIMPLE ? 0 : j]);
+                // B operand: the 8 weights k = 128*step + 32*j + 8*kg .. +8 of column n
+                h2 x[4];
+#pragma unroll
+                for(int r = 0; r < 4; r++)
+                {
+                    const uint32_t sel = 0x0c000c00u | (uint32_t)r | ((uint32_t)r << 16);
+                    const uint32_t tb  = __builtin_amdgcn_perm(wa[j], wa[j], sel);
+                    if(fast)
+                        x[r] = __builtin_bit_cast(h2, and_or(tb, pair_mask, magic));
+                    else
+                        x[r] = __builtin_bit_cast(
+                            h2, and_or((tb & 0xfu) | ((tb >> 4) & 0x000f0000u), lo_mask, magic));
+                }
+#pragma unroll
+                for(int r = 0; r < 4; r++)
+                    x[r] = x[r] - zoff;
+#pragma unroll
+                for(int r = 0; r < 4; r++)
+                    x[r] = x[r] * scv;
+                // the four packed registers are the operand as they stand
+                const v8h bfrag = __builtin_bit_cast(v8h, v4u{__builtin_bit_cast(uint32_t, x[0]),
+                                                               __builtin_bit_cast(uint32_t, x[1]),
+                                                               __builtin_bit_cast(uint32_t, x[2]),
+                                                               __builtin_bit_cast(uint32_t, x[3])});
+                if(!A_AHEAD && !A_UPFRONT)
+                {
+#pragma unroll
+                    for(int i = 0; i < MT; i++)
+                        af_now[0][i] = *reinterpret_cast<const v8h*>(
+                            abase + (aoff[i] + (uint32_t)step * 256 + j * 64));
+                }
+#pragma unroll
+                for(int i = 0; i < MT; i++)
+                {
+                    const v8h a = A_AHEAD ? in.af[A_AHEAD ? j : 0][i]
+                                          : af_now[A_UPFRONT ? j : 0][i];
+                    acc[t][i]   = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag, acc[t][i], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    // ---- main loop ------------------------------------------------------------------------------
+    // Barrier c (one per chunk) says: chunk c has landed, and every compute wave is done with chunk
+    // c - 1, whose ring slot the next fetch overwrites.  The fetch wave issues 16*NT loads per chunk;
+    // they complete in order, so "at most (RING-2) chunks' worth outstanding" means chunk c is in.
+    const bool fetcher = wave == WL_WAVES;
+    if(fetcher)
     {
 #pragma unroll
-        for(int u = 0; u < WM_DEPTH; u++)
+        for(int c = 0; c < RING - 1; c++)
+            if(c < nchunks)
+                issue_chunk(c);
+        for(int c = 0; c < nchunks; c++)
         {
-            const int tt = step_of(round, u);
-            if(tt < nsteps)
-            {
-                consume(u, tt, u + 1 < WM_DEPTH ? step_of(round, u + 1) : step_of(round + 1, 0));
-                issue(u, step_of(round + 1, u));
-            }
+            if(c + RING - 2 < nchunks)
+                wl_wait_vmcnt<(RING - 2) * 16 * NT>();
+            else
+                wl_wait_vmcnt<0>();
+            wl_barrier();
+            if(c + RING - 1 < nchunks)
+                issue_chunk(c + RING - 1);
+        }
+    }
+    else
+    {
+        // this wave's steps: chunk c, step-in-chunk wave and wave + 8; two input sets alternate
+        step_inputs in[2];
+        request(in[0], wave);
+        for(int c = 0; c < nchunks; c++)
+        {
+            wl_barrier();
+            const uint32_t slot_addr = lds0 + (c % RING) * CHUNK_BYTES;
+            const int step0          = c * (WL_CHUNK_K / 128) + wave;
+            request(in[1], step0 + WL_WAVES);
+            if(step0 < nsteps)
+                do_step(in[0], step0, slot_addr, wave);
+            request(in[0], step0 + WL_CHUNK_K / 128);
+            if(step0 + WL_WAVES < nsteps)
+                do_step(in[1], step0 + WL_WAVES, slot_addr, wave + WL_WAVES);
         }
     }
 
-    // add the waves' partial tiles in wave order
-#pragma unroll
-    for(int i = 0; i < MT; i++)
-#pragma unroll
-        for(int r = 0; r < 4; r++)
-            red[wave][i * 4 + r][lane] = acc[i][r];
-    __syncthreads();
-    for(int idx = tid; idx < MT * 4 * 64; idx += NW * 64)
+    // ---- add the waves' partial tiles in wave order ------------------------------------------
+    wl_barrier(); // every chunk has been read: the ring's memory becomes the reduction buffer
+    float* red = reinterpret_cast<float*>(lds);
+    if(!fetcher)
     {
-        const int l  = idx & 63;
-        const int ir = idx >> 6;
-        float s      = 0.f;
 #pragma unroll
-        for(int w = 0; w < NW; w++)
-            s += red[w][ir][l];
+        for(int t = 0; t < NT; t++)
+#pragma unroll
+            for(int i = 0; i < MT; i++)
+#pragma unroll
+                for(int r = 0; r < 4; r++)
+                    red[((wave * NT + t) * MT * 4 + i * 4 + r) * 64 + lane] = acc[t][i][r];
+    }
+    __syncthreads();
+    for(int idx = tid; idx < NT * MT * 4 * 64; idx += WL_THREADS)
+    {
+        const int l   = idx & 63;
+        const int tir = idx >> 6; // (t * MT + i) * 4 + r
+        float s       = 0.f;
+#pragma unroll
+        for(int w = 0; w < WL_WAVES; w++)
+            s += red[(w * NT * MT * 4 + tir) * 64 + l];
         // accumulator register r of lane l is D[4*(l >> 4) + r][l & 15]
-        const int m = 16 * (ir >> 2) + 4 * (l >> 4) + (ir & 3);
+        const int t = tir / (MT * 4);
+        const int i = (tir >> 2) % MT;
+        const int m = 16 * i + 4 * (l >> 4) + (tir & 3);
         if(m < p.m)
-            p.out[(int64_t)m * p.ldc + n0 + (l & 15)] = f32_to_half_rtz(s);
+            p.out[(int64_t)m * p.ldc + n0 + 16 * t + (l & 15)] = f32_to_half_rtz(s);
     }
 }
 
 bool mfma_gemm_supported(const w4_params& p)
 {
-    // lane offsets are 32-bit
+    // lane offsets are 32-bit; the ring loads move whole 16-byte pieces of a packed row
     return p.n % 16 == 0 && p.k % 128 == 0 && p.m >= 1 && (int64_t)p.n * p.k / 2 < (1ll << 31) &&
            (int64_t)p.m * p.lda * 2 < (1ll << 31);
 }
@@ -256,21 +359,28 @@ bool mfma_gemm_supported(const w4_params& p)
 template <int MT>
 int launch_mfma_tiles(const w4_params& p, hipStream_t s)
 {
-    const int grid = p.n / 16;
-    // few column tiles: more waves per workgroup keep enough weight loads in flight
     const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
-    if constexpr(MT == 1)
+    // two column tiles per workgroup halve the activation traffic; taken when that still leaves
+    // every CU a workgroup
+    // (not with 8 M-tiles: the accumulators of two column tiles would not fit the registers)
+    const bool two = MT <= 4 && p.n % 32 == 0 && p.n / 32 >= 256;
+    if constexpr(MT <= 4)
     {
-        if(grid < 512 && (p.k >> 7) >= 32 && simple)
+        if(two)
         {
-            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 16, true>), dim3(grid), dim3(1024), 0, s, p);
+            if(simple)
+                hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 2, true>), dim3(p.n / 32), dim3(WL_THREADS), 0, s, p);
+            else
+                hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 2, false>), dim3(p.n / 32), dim3(WL_THREADS), 0, s, p);
             return mi355_launch_status();
         }
     }
-    if(simple)
-        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 8, true>), dim3(grid), dim3(512), 0, s, p);
-    else
-        hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 8, false>), dim3(grid), dim3(512), 0, s, p);
+    {
+        if(simple)
+            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 1, true>), dim3(p.n / 16), dim3(WL_THREADS), 0, s, p);
+        else
+            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 1, false>), dim3(p.n / 16), dim3(WL_THREADS), 0, s, p);
+    }
     return mi355_launch_status();
 }
 
