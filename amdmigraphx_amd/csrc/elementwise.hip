@@ -1,0 +1,265 @@
+// Float operators around the quantized GEMMs of an encoder graph: broadcasting binary operators,
+// unary functions, reduce_mean and softmax over the last axis, gather along axis 0.  They follow
+// the ref target's arithmetic (plain IEEE float operations; reductions accumulate in double as
+// accumulator_type<float> does, src/include/migraphx/type_traits.hpp:78-81) and are written for
+// correctness and coalesced access, not tuned: the GEMMs dominate the graph.
+#include "common.h"
+
+namespace {
+
+struct bcast_params
+{
+    const float* a;
+    const float* b;
+    float* out;
+    int64_t lens[MI355_MAX_DIMS];
+    int64_t a_strides[MI355_MAX_DIMS];
+    int64_t b_strides[MI355_MAX_DIMS];
+    int64_t total;
+    int ndim;
+    int op;
+};
+
+__global__ __launch_bounds__(256) void binary_kernel(bcast_params p)
+{
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < p.total; i += step)
+    {
+        int64_t rem = i, ao = 0, bo = 0;
+        for(int d = p.ndim - 1; d >= 0; d--)
+        {
+            const int64_t c = rem % p.lens[d];
+            rem /= p.lens[d];
+            ao += c * p.a_strides[d];
+            bo += c * p.b_strides[d];
+        }
+        const float x = p.a[ao], y = p.b[bo];
+        float r;
+        switch(p.op)
+        {
+        case MI355_BIN_ADD: r = x + y; break;
+        case MI355_BIN_SUB: r = x - y; break;
+        case MI355_BIN_MUL: r = x * y; break;
+        default: r = x / y; break; // correctly rounded IEEE division
+        }
+        p.out[i] = r;
+    }
+}
+
+__global__ __launch_bounds__(256) void unary_kernel(const float* in, float* out, int64_t n, int op)
+{
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step)
+    {
+        const float x = in[i];
+        float r;
+        switch(op)
+        {
+        case MI355_UN_ERF: r = erff(x); break;
+        case MI355_UN_SQRT: r = sqrtf(x); break; // correctly rounded (hipcc default)
+        case MI355_UN_RSQRT: r = 1.0f / sqrtf(x); break; // 1 / std::sqrt(x), two IEEE operations
+        case MI355_UN_EXP: r = expf(x); break;
+        case MI355_UN_TANH: r = tanhf(x); break;
+        default: r = -x; break;
+        }
+        out[i] = r;
+    }
+}
+
+// sum of 64 doubles across a wave, every lane receives it; fixed pairing, so deterministic
+MI355_DEVINL double wave_sum_f64(double v)
+{
+#pragma unroll
+    for(int off = 32; off > 0; off >>= 1)
+        v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+MI355_DEVINL double wave_max_f64(double v)
+{
+#pragma unroll
+    for(int off = 32; off > 0; off >>= 1)
+        v = fmax(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// one wave per row; double accumulation (the order differs from the reference's sequential sum,
+// which moves the float result by at most its last bit)
+__global__ __launch_bounds__(256) void reduce_mean_kernel(const float* in, float* out, int64_t rows, int64_t cols)
+{
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= rows)
+        return;
+    const float* x = in + row * cols;
+    double s       = 0.0;
+    for(int64_t c = lane; c < cols; c += 64)
+        s += (double)x[c];
+    s = wave_sum_f64(s);
+    if(lane == 0)
+        out[row] = (float)(s / (double)cols);
+}
+
+// ref_softmax (src/targets/ref/lowering.cpp:281-312): e = float(exp(double(x) - max)),
+// sum of e in double, out = float(double(e) / sum)
+__global__ __launch_bounds__(256) void softmax_kernel(const float* in, float* out, int64_t rows, int64_t cols)
+{
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= rows)
+        return;
+    const float* x = in + row * cols;
+    float* y       = out + row * cols;
+    double m       = -1.7976931348623157e308;
+    for(int64_t c = lane; c < cols; c += 64)
+        m = fmax(m, (double)x[c]);
+    m        = wave_max_f64(m);
+    double s = 0.0;
+    for(int64_t c = lane; c < cols; c += 64)
+    {
+        const float e = (float)exp((double)x[c] - m);
+        y[c]          = e;
+        s += (double)e;
+    }
+    s = wave_sum_f64(s);
+    for(int64_t c = lane; c < cols; c += 64)
+        y[c] = (float)((double)y[c] / s);
+}
+
+// out[i, :] = table[ids[i], :]; negative indices count from the end (op/gather.hpp:100-118)
+template <class I>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    const uint32_t* table, const I* ids, uint32_t* out, int64_t n_ids, int64_t table_rows, int64_t row_words)
+{
+    const int64_t total = n_ids * row_words;
+    const int64_t step  = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step)
+    {
+        const int64_t r = i / row_words;
+        int64_t id      = (int64_t)ids[r];
+        if(id < 0)
+            id += table_rows;
+        // an index outside the table reads row 0 rather than memory out of bounds
+        if(id < 0 || id >= table_rows)
+            id = 0;
+        out[i] = table[id * row_words + (i - r * row_words)];
+    }
+}
+
+unsigned blocks_for_n(int64_t n)
+{
+    int64_t b = (n + 255) / 256;
+    return (unsigned)(b > 256 * 16 ? 256 * 16 : (b < 1 ? 1 : b));
+}
+
+} // namespace
+
+extern "C" int mi355_binary_f32(int32_t op,
+                                const float* a,
+                                const int64_t* a_strides,
+                                const float* b,
+                                const int64_t* b_strides,
+                                float* out,
+                                int32_t ndim,
+                                const int64_t* lens,
+                                void* stream)
+{
+    if(op < MI355_BIN_ADD || op > MI355_BIN_DIV || ndim < 1 || ndim > MI355_MAX_DIMS ||
+       lens == nullptr || a_strides == nullptr || b_strides == nullptr)
+        return MI355_ERR_BAD_ARG;
+    bcast_params p{};
+    p.total = 1;
+    for(int d = 0; d < ndim; d++)
+    {
+        if(lens[d] < 0 || a_strides[d] < 0 || b_strides[d] < 0)
+            return MI355_ERR_BAD_ARG;
+        p.lens[d]      = lens[d];
+        p.a_strides[d] = a_strides[d];
+        p.b_strides[d] = b_strides[d];
+        p.total *= lens[d];
+    }
+    if(p.total == 0)
+        return MI355_OK;
+    if(a == nullptr || b == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    p.a    = a;
+    p.b    = b;
+    p.out  = out;
+    p.ndim = ndim;
+    p.op   = op;
+    hipLaunchKernelGGL(binary_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t n, void* stream)
+{
+    if(op < MI355_UN_ERF || op > MI355_UN_NEG || n < 0)
+        return MI355_ERR_BAD_ARG;
+    if(n == 0)
+        return MI355_OK;
+    if(in == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    hipLaunchKernelGGL(unary_kernel, dim3(blocks_for_n(n)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), in, out, n, op);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_reduce_mean_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream)
+{
+    if(rows < 0 || cols <= 0)
+        return MI355_ERR_BAD_ARG;
+    if(rows == 0)
+        return MI355_OK;
+    if(in == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if((rows + 3) / 4 > 0x7fffffff)
+        return MI355_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(reduce_mean_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), in, out, rows, cols);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_softmax_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream)
+{
+    if(rows < 0 || cols <= 0)
+        return MI355_ERR_BAD_ARG;
+    if(rows == 0)
+        return MI355_OK;
+    if(in == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if((rows + 3) / 4 > 0x7fffffff)
+        return MI355_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), in, out, rows, cols);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_gather_rows(const void* table,
+                                 const void* ids,
+                                 int32_t ids_are_int64,
+                                 void* out,
+                                 int64_t n_ids,
+                                 int64_t table_rows,
+                                 int64_t row_bytes,
+                                 void* stream)
+{
+    if(n_ids < 0 || table_rows <= 0 || row_bytes <= 0 || row_bytes % 4 != 0)
+        return MI355_ERR_BAD_ARG;
+    if(n_ids == 0)
+        return MI355_OK;
+    if(table == nullptr || ids == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    const int64_t words = row_bytes / 4;
+    const dim3 grid(blocks_for_n(n_ids * words));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if(ids_are_int64)
+        hipLaunchKernelGGL(gather_rows_kernel<int64_t>, grid, dim3(256), 0, s,
+                           static_cast<const uint32_t*>(table), static_cast<const int64_t*>(ids),
+                           static_cast<uint32_t*>(out), n_ids, table_rows, words);
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<int32_t>, grid, dim3(256), 0, s,
+                           static_cast<const uint32_t*>(table), static_cast<const int32_t*>(ids),
+                           static_cast<uint32_t*>(out), n_ids, table_rows, words);
+    return mi355_launch_status();
+}

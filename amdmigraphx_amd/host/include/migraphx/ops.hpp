@@ -103,6 +103,62 @@ struct binary
 struct mul : binary { mul() : binary{"mul"} {} };
 struct add : binary { add() : binary{"add"} {} };
 struct sub : binary { sub() : binary{"sub"} {} };
+struct div : binary { div() : binary{"div"} {} };
+
+// src/include/migraphx/op/unary.hpp (erf.hpp, sqrt.hpp, rsqrt.hpp, exp.hpp, tanh.hpp, neg.hpp): the
+// result has the input's shape
+struct unary
+{
+    std::string op_name;
+    std::string name() const { return op_name; }
+    value attributes() const { return {{"pointwise", true}}; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+struct erf : unary { erf() : unary{"erf"} {} };
+struct sqrt : unary { sqrt() : unary{"sqrt"} {} };
+struct rsqrt : unary { rsqrt() : unary{"rsqrt"} {} };
+struct exp : unary { exp() : unary{"exp"} {} };
+struct tanh : unary { tanh() : unary{"tanh"} {} };
+struct neg : unary { neg() : unary{"neg"} {} };
+
+// src/include/migraphx/op/reduce_mean.hpp:34-50, reduce_op.hpp:80-180: reduced axes keep length 1
+struct reduce_mean
+{
+    std::vector<int64_t> axes;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axes, "axes");
+    }
+    std::string name() const { return "reduce_mean"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
+// src/include/migraphx/op/softmax.hpp:36-60
+struct softmax
+{
+    int64_t axis = 1;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
+    std::string name() const { return "softmax"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
+// src/include/migraphx/op/gather.hpp:42-98
+struct gather
+{
+    int64_t axis = 0;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
+    std::string name() const { return "gather"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
 
 // src/include/migraphx/op/broadcast.hpp:52-128
 struct broadcast

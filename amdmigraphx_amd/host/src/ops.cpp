@@ -165,6 +165,53 @@ shape binary::compute_shape(const std::vector<shape>& inputs) const
     return {s0.type(), s0.lens()};
 }
 
+shape unary::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, op_name, 1, 1);
+    const auto& s = inputs[0];
+    if(s.scalar() or s.broadcasted() or s.packed())
+        return s;
+    return {s.type(), s.lens()};
+}
+
+shape reduce_mean::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "REDUCE_MEAN", 1, 1);
+    const auto& s = inputs[0];
+    auto lens     = s.lens();
+    if(axes.empty())
+        std::fill(lens.begin(), lens.end(), 1);
+    for(auto a : axes)
+        lens[normalize_axis(a, s.ndim(), "REDUCE_MEAN")] = 1;
+    return {s.type(), lens};
+}
+
+shape softmax::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "SOFTMAX", 1, 1);
+    const auto& s = inputs[0];
+    normalize_axis(axis, s.ndim(), "SOFTMAX");
+    if(s.broadcasted())
+        return {s.type(), s.lens()};
+    return s.packed() ? s.with_lens(s.lens()) : shape{s.type(), s.lens()};
+}
+
+shape gather::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "GATHER", 2, 2);
+    const auto& data = inputs[0];
+    const auto& idx  = inputs[1];
+    const auto ax    = normalize_axis(axis, data.ndim(), "GATHER");
+    auto lens        = data.lens();
+    lens.erase(lens.begin() + ax);
+    const bool scalar_indices = idx.ndim() == 1 and idx.scalar() and idx.elements() == 1;
+    if(not scalar_indices)
+        lens.insert(lens.begin() + ax, idx.lens().begin(), idx.lens().end());
+    if(lens.empty())
+        return shape{data.type()};
+    return {data.type(), lens};
+}
+
 shape broadcast::compute_shape(const std::vector<shape>& inputs) const
 {
     check_count(inputs, "BROADCAST", 1, 1);
@@ -401,6 +448,16 @@ MIGRAPHX_REGISTER_OP(op::convert);
 MIGRAPHX_REGISTER_OP(op::mul);
 MIGRAPHX_REGISTER_OP(op::add);
 MIGRAPHX_REGISTER_OP(op::sub);
+MIGRAPHX_REGISTER_OP(op::div);
+MIGRAPHX_REGISTER_OP(op::erf);
+MIGRAPHX_REGISTER_OP(op::sqrt);
+MIGRAPHX_REGISTER_OP(op::rsqrt);
+MIGRAPHX_REGISTER_OP(op::exp);
+MIGRAPHX_REGISTER_OP(op::tanh);
+MIGRAPHX_REGISTER_OP(op::neg);
+MIGRAPHX_REGISTER_OP(op::reduce_mean);
+MIGRAPHX_REGISTER_OP(op::softmax);
+MIGRAPHX_REGISTER_OP(op::gather);
 MIGRAPHX_REGISTER_OP(op::broadcast);
 MIGRAPHX_REGISTER_OP(op::multibroadcast);
 MIGRAPHX_REGISTER_OP(op::transpose);

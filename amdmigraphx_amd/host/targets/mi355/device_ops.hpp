@@ -33,6 +33,8 @@ matrix_view view_as_matrix(const shape& s);
 // strides (row, column) of a tensor seen as [prod(leading dims), last dim]; false when the
 // leading dimensions do not collapse into one stride
 bool collapse_2d(const shape& s, int64_t& stride_r, int64_t& stride_c);
+// true when the dimensions in front of the last two can be walked with one stride
+bool batch_collapses(const shape& s);
 
 struct allocate
 {
@@ -195,6 +197,61 @@ struct convert
         f(self.target_type, "target_type");
     }
     std::string name() const { return "mi355::convert"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: a, b (views with any strides, broadcast included), out
+struct binary
+{
+    int64_t op = MI355_BIN_ADD;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.op, "op");
+    }
+    std::string name() const { return "mi355::binary"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: x, out
+struct unary
+{
+    int64_t op = MI355_UN_ERF;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.op, "op");
+    }
+    std::string name() const { return "mi355::unary"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: x (standard), out; over the last axis
+struct reduce_mean
+{
+    std::string name() const { return "mi355::reduce_mean"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+struct softmax
+{
+    std::string name() const { return "mi355::softmax"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: table (standard), indices (standard int32 / int64), out; along axis 0
+struct gather
+{
+    std::string name() const { return "mi355::gather"; }
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }

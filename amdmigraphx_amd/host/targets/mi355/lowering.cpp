@@ -409,7 +409,13 @@ void lower_instruction(module& m, instruction_ref ins)
     }
     else if(name == "dot")
     {
-        m.replace_instruction(ins, operation{dot{}}, ins->inputs()[0], ins->inputs()[1], standard_out());
+        auto a = ins->inputs()[0];
+        auto b = ins->inputs()[1];
+        if(not batch_collapses(a->get_shape()))
+            a = make_standard(m, ins, a);
+        if(not batch_collapses(b->get_shape()))
+            b = make_standard(m, ins, b);
+        m.replace_instruction(ins, operation{dot{}}, a, b, standard_out());
     }
     else if(name == "quantizelinear" or name == "dequantizelinear")
     {
@@ -448,6 +454,52 @@ void lower_instruction(module& m, instruction_ref ins)
         op.target_type = any_cast<op::convert>(ins->get_operator()).target_type;
         auto x         = make_standard(m, ins, ins->inputs()[0]);
         m.replace_instruction(ins, operation{op}, x, standard_out());
+    }
+    else if(name == "add" or name == "sub" or name == "mul" or name == "div")
+    {
+        binary op;
+        op.op = name == "add" ? MI355_BIN_ADD
+                              : (name == "sub" ? MI355_BIN_SUB : (name == "mul" ? MI355_BIN_MUL : MI355_BIN_DIV));
+        m.replace_instruction(ins, operation{op}, ins->inputs()[0], ins->inputs()[1], standard_out());
+    }
+    else if(name == "erf" or name == "sqrt" or name == "rsqrt" or name == "exp" or name == "tanh" or
+            name == "neg")
+    {
+        unary op;
+        op.op  = name == "erf" ? MI355_UN_ERF
+                               : (name == "sqrt" ? MI355_UN_SQRT
+                                                 : (name == "rsqrt" ? MI355_UN_RSQRT
+                                                                    : (name == "exp" ? MI355_UN_EXP
+                                                                                     : (name == "tanh" ? MI355_UN_TANH
+                                                                                                       : MI355_UN_NEG))));
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        m.replace_instruction(ins, operation{op}, x, standard_out());
+    }
+    else if(name == "reduce_mean")
+    {
+        const auto& axes = any_cast<op::reduce_mean>(ins->get_operator()).axes;
+        const auto nd    = static_cast<int64_t>(ins->inputs()[0]->get_shape().ndim());
+        if(axes.size() != 1 or (axes[0] != -1 and axes[0] != nd - 1))
+            MIGRAPHX_THROW("mi355: reduce_mean over anything but the last axis has no kernel");
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        m.replace_instruction(ins, operation{reduce_mean{}}, x, standard_out());
+    }
+    else if(name == "softmax")
+    {
+        const auto axis = any_cast<op::softmax>(ins->get_operator()).axis;
+        const auto nd   = static_cast<int64_t>(ins->inputs()[0]->get_shape().ndim());
+        if(axis != -1 and axis != nd - 1)
+            MIGRAPHX_THROW("mi355: softmax over anything but the last axis has no kernel");
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        m.replace_instruction(ins, operation{softmax{}}, x, standard_out());
+    }
+    else if(name == "gather")
+    {
+        if(any_cast<op::gather>(ins->get_operator()).axis != 0)
+            MIGRAPHX_THROW("mi355: gather along an axis other than 0 has no kernel");
+        auto t = make_standard(m, ins, ins->inputs()[0]);
+        auto i = make_standard(m, ins, ins->inputs()[1]);
+        m.replace_instruction(ins, operation{gather{}}, t, i, standard_out());
     }
     else if(name == "contiguous")
     {

@@ -166,6 +166,19 @@ bool collapse_2d(const shape& s, int64_t& stride_r, int64_t& stride_c)
     return true;
 }
 
+bool batch_collapses(const shape& s)
+{
+    if(s.ndim() <= 3)
+        return true;
+    std::vector<std::size_t> bl(s.lens().begin(), s.lens().end() - 2);
+    std::vector<std::size_t> bs(s.strides().begin(), s.strides().end() - 2);
+    bl.push_back(1);
+    bs.push_back(1);
+    int64_t sr = 0;
+    int64_t sc = 0;
+    return collapse_2d(shape{s.type(), bl, bs}, sr, sc);
+}
+
 namespace {
 void rows_cols(const shape& s, int64_t& rows, int64_t& cols)
 {
@@ -362,17 +375,11 @@ shape dot::compute_shape(const std::vector<shape>& inputs) const
     to_mi355_type(s.type());
     if(s.type() != shape::float_type and s.type() != shape::half_type and s.type() != shape::bf16_type)
         MIGRAPHX_THROW("mi355::dot: float, half or bf16 only");
-    // any strides are fine inside a matrix; the batch dimensions must collapse
+    // any strides are fine inside a matrix; the batch dimensions must collapse into one stride
     for(int i = 0; i < 2; i++)
     {
-        auto v = view_as_matrix(inputs[i].ndim() == 2 ? inputs[i] : inputs[i]);
-        int64_t sr = 0;
-        int64_t sc = 0;
-        std::vector<std::size_t> bl(inputs[i].lens().begin(), inputs[i].lens().end() - 1);
-        std::vector<std::size_t> bs(inputs[i].strides().begin(), inputs[i].strides().end() - 1);
-        if(bl.size() > 1 and not collapse_2d(shape{s.type(), bl, bs}, sr, sc))
+        if(not batch_collapses(inputs[i]))
             MIGRAPHX_THROW("mi355::dot: batch dimensions do not collapse into one stride");
-        (void)v;
     }
     if(inputs.back() != s)
         MIGRAPHX_THROW("mi355::dot: output buffer has the wrong shape");
@@ -672,6 +679,155 @@ argument contiguous::compute(migraphx::context& ctx, const shape&, const std::ve
     return args[1];
 }
 
+// ----------------------------------------------------------------- float operators
+
+shape binary::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    if(inputs[0].type() != shape::float_type or inputs[1].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::binary: float tensors only, got " + inputs[0].type_string());
+    if(inputs[0].lens() != inputs[1].lens())
+        MIGRAPHX_THROW("mi355::binary: Dimensions do not match");
+    if(inputs[0].ndim() > MI355_MAX_DIMS)
+        MIGRAPHX_THROW("mi355::binary: too many dimensions");
+    shape out{shape::float_type, inputs[0].lens()};
+    if(inputs[2] != out)
+        MIGRAPHX_THROW("mi355::binary: output buffer has the wrong shape");
+    return out;
+}
+
+argument binary::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    std::vector<int64_t> lens(out.lens().begin(), out.lens().end());
+    auto strides_of = [&](const shape& s) {
+        std::vector<int64_t> r(s.strides().begin(), s.strides().end());
+        for(std::size_t i = 0; i < r.size(); i++)
+        {
+            if(s.lens()[i] == 1)
+                r[i] = 0;
+        }
+        return r;
+    };
+    const auto sa = strides_of(args[0].get_shape());
+    const auto sb = strides_of(args[1].get_shape());
+    status_check(mi355_binary_f32(static_cast<int32_t>(op),
+                                  reinterpret_cast<const float*>(args[0].data()),
+                                  sa.data(),
+                                  reinterpret_cast<const float*>(args[1].data()),
+                                  sb.data(),
+                                  reinterpret_cast<float*>(args[2].data()),
+                                  static_cast<int32_t>(lens.size()),
+                                  lens.data(),
+                                  stream_of(ctx)),
+                 name());
+    return args[2];
+}
+
+shape unary::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::unary: float tensors only");
+    if(inputs[1] != inputs[0])
+        MIGRAPHX_THROW("mi355::unary: output buffer has the wrong shape");
+    return inputs[0];
+}
+
+argument unary::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    status_check(mi355_unary_f32(static_cast<int32_t>(op),
+                                 reinterpret_cast<const float*>(args[0].data()),
+                                 reinterpret_cast<float*>(args[1].data()),
+                                 static_cast<int64_t>(out.elements()),
+                                 stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape reduce_mean::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::reduce_mean: float tensors only");
+    auto lens   = inputs[0].lens();
+    lens.back() = 1;
+    shape out{shape::float_type, lens};
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::reduce_mean: output buffer has the wrong shape");
+    return out;
+}
+
+argument reduce_mean::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_reduce_mean_f32(reinterpret_cast<const float*>(args[0].data()),
+                                       reinterpret_cast<float*>(args[1].data()),
+                                       rows,
+                                       cols,
+                                       stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape softmax::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::softmax: float tensors only");
+    if(inputs[1] != inputs[0])
+        MIGRAPHX_THROW("mi355::softmax: output buffer has the wrong shape");
+    return inputs[0];
+}
+
+argument softmax::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_softmax_f32(reinterpret_cast<const float*>(args[0].data()),
+                                   reinterpret_cast<float*>(args[1].data()),
+                                   rows,
+                                   cols,
+                                   stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
+shape gather::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    check_standard(inputs[0], name());
+    check_standard(inputs[1], name());
+    if(inputs[1].type() != shape::int32_type and inputs[1].type() != shape::int64_type)
+        MIGRAPHX_THROW("mi355::gather: indices must be int32 or int64");
+    auto out = op::gather{}.compute_shape({inputs[0], inputs[1]});
+    if((inputs[0].bytes() / inputs[0].lens()[0]) % 4 != 0)
+        MIGRAPHX_THROW("mi355::gather: rows must be a multiple of 4 bytes");
+    if(inputs[2] != out)
+        MIGRAPHX_THROW("mi355::gather: output buffer has the wrong shape");
+    return out;
+}
+
+argument gather::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto& t = args[0].get_shape();
+    status_check(mi355_gather_rows(args[0].data(),
+                                   args[1].data(),
+                                   args[1].get_shape().type() == shape::int64_type,
+                                   args[2].data(),
+                                   static_cast<int64_t>(args[1].get_shape().elements()),
+                                   static_cast<int64_t>(t.lens()[0]),
+                                   static_cast<int64_t>(t.bytes() / t.lens()[0]),
+                                   stream_of(ctx)),
+                 name());
+    return args[2];
+}
+
 // ----------------------------------------------------------------- target
 
 std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_options& options) const
@@ -700,6 +856,11 @@ MIGRAPHX_REGISTER_OP(mi355::unpack_int4);
 MIGRAPHX_REGISTER_OP(mi355::pack_int4);
 MIGRAPHX_REGISTER_OP(mi355::convert);
 MIGRAPHX_REGISTER_OP(mi355::contiguous);
+MIGRAPHX_REGISTER_OP(mi355::binary);
+MIGRAPHX_REGISTER_OP(mi355::unary);
+MIGRAPHX_REGISTER_OP(mi355::reduce_mean);
+MIGRAPHX_REGISTER_OP(mi355::softmax);
+MIGRAPHX_REGISTER_OP(mi355::gather);
 MIGRAPHX_REGISTER_TARGET(mi355::target);
 
 } // namespace migraphx

@@ -234,6 +234,37 @@ int mi355_dot(const void* a, const void* b, void* c, int32_t type,
 int mi355_contiguous(const void* in, void* out, int32_t elem_size, int32_t ndim,
                      const int64_t* lens, const int64_t* strides, void* stream);
 
+/*
+ * Float operators of the graph around the quantized GEMMs (an encoder layer's bias and residual
+ * adds, layer normalisation built from reduce_mean / sub / mul / rsqrt, GELU through erf, attention
+ * softmax, embedding lookup).  float32 only; not tuned.
+ *
+ * mi355_binary_f32   op::add / sub / mul / div (src/include/migraphx/op/binary.hpp:60-90): out is a
+ *                    dense row-major tensor of `lens`; a and b are addressed through element strides
+ *                    (zero = broadcast), HOST arrays of ndim entries.
+ * mi355_unary_f32    op::erf / sqrt / rsqrt (1 / sqrt(x)) / exp / tanh / neg on n dense elements
+ *                    (op/unary.hpp; erf.hpp, rsqrt.hpp, ...).  erf, exp and tanh use the device math
+ *                    library and may differ from the host's by a few units in the last place.
+ * mi355_reduce_mean_f32  op::reduce_mean over the last axis of [rows, cols] (op/reduce_mean.hpp:34-50,
+ *                    reduce_op.hpp:186-202): sum in double, divided by cols, rounded to float.
+ * mi355_softmax_f32  softmax over the last axis (ref_softmax, src/targets/ref/lowering.cpp:281-312):
+ *                    e = float(exp(double(x) - max)), out = float(double(e) / sum_double(e)).
+ * mi355_gather_rows  op::gather along axis 0 of a [table_rows, row_bytes] table with int32 or int64
+ *                    indices (op/gather.hpp:100-118); row_bytes must be a multiple of 4.
+ */
+typedef enum mi355_binary_op { MI355_BIN_ADD = 0, MI355_BIN_SUB = 1, MI355_BIN_MUL = 2, MI355_BIN_DIV = 3 } mi355_binary_op;
+typedef enum mi355_unary_op {
+    MI355_UN_ERF = 0, MI355_UN_SQRT = 1, MI355_UN_RSQRT = 2, MI355_UN_EXP = 3, MI355_UN_TANH = 4, MI355_UN_NEG = 5
+} mi355_unary_op;
+int mi355_binary_f32(int32_t op, const float* a, const int64_t* a_strides, const float* b,
+                     const int64_t* b_strides, float* out, int32_t ndim, const int64_t* lens,
+                     void* stream);
+int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t n, void* stream);
+int mi355_reduce_mean_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
+int mi355_softmax_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
+int mi355_gather_rows(const void* table, const void* ids, int32_t ids_are_int64, void* out,
+                      int64_t n_ids, int64_t table_rows, int64_t row_bytes, void* stream);
+
 /* Human-readable text for a status code (static storage). */
 const char* mi355_status_string(int status);
 

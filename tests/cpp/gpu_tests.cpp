@@ -4,8 +4,10 @@
 // exactly (int8 quant_dot with the dequantize epilogue, the int4 chain, float dot) must be
 // bit-identical; fp8 results use the tolerances stated at the test.
 #include "common.hpp"
+#include "encoder.hpp"
 #include "oracle_target.hpp"
 #include "test.hpp"
+#include <chrono>
 #include <fstream>
 
 using namespace testutil;
@@ -383,7 +385,7 @@ TEST_CASE(no_host_fallback)
     program p;
     auto* mm = p.get_main_module();
     auto x   = mm->add_parameter("x", shape{shape::float_type, {4, 4}});
-    mm->add_return({mm->add_instruction(make_op("add"), x, x)});
+    mm->add_return({mm->add_instruction(make_op("softmax", {{"axis", 0}}), x)});
     bool thrown = false;
     try
     {
@@ -391,7 +393,7 @@ TEST_CASE(no_host_fallback)
     }
     catch(const migraphx::exception& e)
     {
-        thrown = std::string(e.what()).find("no kernel for operator 'add'") != std::string::npos;
+        thrown = std::string(e.what()).find("has no kernel") != std::string::npos;
     }
     EXPECT(thrown);
     // wrong parameter shape at eval
@@ -409,10 +411,157 @@ TEST_CASE(no_host_fallback)
     }));
 }
 
+TEST_CASE(float_operators)
+{
+    // the float operators around the GEMMs, one by one against the CPU target: exact where the
+    // arithmetic is IEEE (add / sub / mul / div / sqrt / rsqrt, gather), within a few units in the
+    // last place where a math-library function or the summation order is involved
+    const std::size_t r = 33, c = 200;
+    auto run = [&](const std::function<instruction_ref(module&, instruction_ref, instruction_ref)>& f, bool exact) {
+        static int case_no = 0;
+        case_no++;
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, {r, c}});
+        auto y   = mm->add_parameter("y", shape{shape::float_type, {r, c}});
+        mm->add_return({f(*mm, x, y)});
+        argument xa{shape{shape::float_type, {r, c}}, normal_floats(r * c, 2.0f, 100)};
+        argument ya{shape{shape::float_type, {r, c}}, uniform_floats(r * c, 0.5f, 3.0f, 101)};
+        auto want = run_on("oracle", p, {{"x", xa}, {"y", ya}});
+        auto got  = run_on("mi355", p, {{"x", xa}, {"y", ya}});
+        if(not(exact ? same_bytes(got[0], want[0]) : max_rel_diff(got[0], want[0], 1e-30) < 4e-6))
+            std::cout << "float operator case " << case_no << ": max rel diff "
+                      << max_rel_diff(got[0], want[0], 1e-30) << std::endl;
+        if(exact)
+            EXPECT(same_bytes(got[0], want[0]));
+        else
+            EXPECT(max_rel_diff(got[0], want[0], 1e-30) < 4e-6);
+    };
+    for(auto name : {"add", "sub", "mul", "div"})
+        run([&](module& m, instruction_ref x, instruction_ref y) { return m.add_instruction(make_op(name), x, y); }, true);
+    // broadcast operands: a row vector and a column of means
+    run([&](module& m, instruction_ref x, instruction_ref) {
+        auto mean = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), x);
+        auto mb   = m.add_instruction(make_op("multibroadcast", {{"out_lens", x->get_shape().lens()}}), mean);
+        return m.add_instruction(make_op("sub"), x, mb);
+    }, false);
+    run([&](module& m, instruction_ref, instruction_ref y) { return m.add_instruction(make_op("sqrt"), y); }, true);
+    run([&](module& m, instruction_ref, instruction_ref y) { return m.add_instruction(make_op("rsqrt"), y); }, true);
+    for(auto name : {"erf", "exp", "tanh"})
+        run([&](module& m, instruction_ref x, instruction_ref) { return m.add_instruction(make_op(name), x); }, false);
+    run([&](module& m, instruction_ref x, instruction_ref) { return m.add_instruction(make_op("softmax", {{"axis", 1}}), x); }, false);
+    // gather rows, negative index included
+    program p;
+    auto* mm = p.get_main_module();
+    auto t   = mm->add_literal(literal{shape{shape::float_type, {50, 24}}, normal_floats(50 * 24, 1.0f, 102)});
+    auto i   = mm->add_parameter("i", shape{shape::int32_type, {7}});
+    mm->add_return({mm->add_instruction(make_op("gather", {{"axis", 0}}), t, i)});
+    argument ia{shape{shape::int32_type, {7}}, std::vector<int>{0, 49, 3, 3, -1, 17, -50}};
+    expect_same(p, {{"i", ia}});
+}
+
+// agreement of two float tensors as the reference's verify does it (verify.hpp:175-195): root mean
+// square of the difference against the root mean square of the expected values
+static double rms_error(const argument& got, const argument& want)
+{
+    auto a = got.to_vector<double>();
+    auto b = want.to_vector<double>();
+    double num = 0, den = 0;
+    for(std::size_t i = 0; i < a.size(); i++)
+    {
+        num += (a[i] - b[i]) * (a[i] - b[i]);
+        den += b[i] * b[i];
+    }
+    return std::sqrt(num / den);
+}
+
+TEST_CASE(encoder_int8_qdq)
+{
+    // BASELINE config 5 at a size the CPU oracle evaluates in seconds: 2 layers, hidden 128, 4 heads,
+    // FFN 512, batch 2 x seq 16, vocabulary 100.  Activation scales come from max-abs calibration of
+    // the float graph on the seeded input.  The device's erf / exp differ from the host's in the
+    // last place and a quantizelinear input that lands within that distance of a rounding boundary
+    // moves one int8 step, so the end-to-end outputs are compared by RMS error (1e-3) rather than
+    // bit by bit.
+    encoder::config c;
+    auto w = encoder::make_weights(c, 7);
+    argument ids{shape{shape::int32_type, {c.tokens()}}, uniform_ints<int>(c.tokens(), 0, static_cast<int>(c.vocab) - 1, 8)};
+    auto scales_cpu = encoder::calibrate(c, w, "oracle", ids);
+    auto scales_gpu = encoder::calibrate(c, w, "mi355", ids);
+    EXPECT(scales_cpu.size() == 4 * c.layers);
+    for(std::size_t i = 0; i < scales_cpu.size(); i++)
+        EXPECT(std::fabs(scales_cpu[i] - scales_gpu[i]) <= 1e-5 * scales_cpu[i]);
+    auto p = encoder::quantized(c, w, scales_cpu);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(count_ops(*p.get_main_module(), "quant_dot") == 6 * c.layers);
+    EXPECT(count_ops(*p.get_main_module(), "dot") == 2 * c.layers); // the attention products
+    auto want = run_on("oracle", p, {{"ids", ids}});
+    auto got  = run_on("mi355", p, {{"ids", ids}});
+    EXPECT(got[0].get_shape() == shape{shape::float_type, {c.tokens(), c.hidden}});
+    const double err = rms_error(got[0], want[0]);
+    std::cout << "encoder rms error " << err << std::endl;
+    EXPECT(err < 1e-3);
+    // every QDQ MatMul became one fused kernel launch
+    program compiled = p;
+    compiled.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 6 * c.layers);
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quantizelinear") == 4 * c.layers);
+    EXPECT(not has_op(compiled, "mi355::dequantizelinear"));
+    // and the quantized model stays close to the float one
+    encoder::builder fb{c, w, {}, {}};
+    fb.tap = [](std::size_t, std::vector<argument>) {};
+    auto fp = fb.build();
+    auto ref = run_on("oracle", fp, {{"ids", ids}});
+    EXPECT(rms_error(want[0], ref[0]) < 0.05);
+}
+
+// `gpu_tests encoder_bench [layers]`: the full BERT-base shape (hidden 768, 12 heads, FFN 3072, batch
+// 32 x seq 384 = 12288 tokens, vocabulary 30522) on the device: calibration, compile, timed forwards
+static int encoder_bench(int argc, char** argv)
+{
+    encoder::config c;
+    c.layers = argc > 2 ? std::atoi(argv[2]) : 12;
+    c.hidden = 768;
+    c.heads  = 12;
+    c.ffn    = 3072;
+    c.batch  = 32;
+    c.seq    = 384;
+    c.vocab  = 30522;
+    auto w   = encoder::make_weights(c, 1);
+    argument ids{shape{shape::int32_type, {c.tokens()}}, uniform_ints<int>(c.tokens(), 0, 30521, 2)};
+    auto t      = migraphx::make_target("mi355");
+    auto scales = encoder::calibrate(c, w, "mi355", ids);
+    auto p      = encoder::quantized(c, w, scales);
+    p.compile(t);
+    std::cout << "quantized MatMul launches per forward: "
+              << count_ops(*p.get_main_module(), "mi355::quant_dot") << std::endl;
+    auto dids = t.copy_to(ids);
+    for(int i = 0; i < 2; i++)
+        p.eval({{"ids", dids}});
+    p.finish();
+    const int iters = 5;
+    auto t0 = std::chrono::steady_clock::now();
+    for(int i = 0; i < iters; i++)
+        p.eval({{"ids", dids}});
+    p.finish();
+    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / iters;
+    const double gemm_ops = 2.0 * c.tokens() * c.layers * (4.0 * c.hidden * c.hidden + 2.0 * c.hidden * c.ffn);
+    std::cout << "layers " << c.layers << ": " << ms << " ms per forward, quantized MatMuls "
+              << gemm_ops / 1e12 << " TOP -> " << gemm_ops / (ms * 1e9) << " TOPS if they were all of it" << std::endl;
+    auto out = t.copy_from(p.eval({{"ids", dids}})[0]).to_vector<float>();
+    double s = 0;
+    for(float v : out)
+        s += std::fabs(v);
+    std::cout << "mean |output| " << s / out.size() << std::endl;
+    return std::isfinite(s) ? 0 : 1;
+}
+
 int main(int argc, char** argv)
 {
     try
     {
+        if(argc > 1 and std::string(argv[1]) == "encoder_bench")
+            return encoder_bench(argc, argv);
         return test::run(argc, argv);
     }
     catch(const std::exception& e)

@@ -4,6 +4,7 @@
 // test/simplify_qdq_test.cpp, test/int4_test.cpp and test/quantization.cpp: the rewritten module
 // is compared with one written out by hand, and both are evaluated on the CPU oracle target.
 #include "common.hpp"
+#include "encoder.hpp"
 #include "oracle_target.hpp"
 #include "test.hpp"
 #include <algorithm>
@@ -664,6 +665,46 @@ TEST_CASE(fp8_calibration)
         den += a[i] * a[i];
     }
     EXPECT(std::sqrt(num / den) < 0.06);
+}
+
+// ---------------------------------------------------------------- encoder graph
+
+TEST_CASE(encoder_graph_on_cpu)
+{
+    // the BERT-shaped graph of BASELINE config 5, small: calibration, QDQ rewrite and evaluation on
+    // the CPU oracle target; the int8 model must stay close to the float one
+    encoder::config c;
+    c.layers = 1;
+    auto w   = encoder::make_weights(c, 3);
+    argument ids{shape{shape::int32_type, {c.tokens()}}, uniform_ints<int>(c.tokens(), 0, static_cast<int>(c.vocab) - 1, 4)};
+    auto scales = encoder::calibrate(c, w, "oracle", ids);
+    EXPECT(scales.size() == 4);
+    for(float s : scales)
+        EXPECT(s > 0 and std::isfinite(s));
+    auto p = encoder::quantized(c, w, scales);
+    EXPECT(count_ops(*p.get_main_module(), "dot") == 8);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    EXPECT(count_ops(*p.get_main_module(), "quant_dot") == 6);
+    EXPECT(count_ops(*p.get_main_module(), "dot") == 2);
+    EXPECT(count_ops(*p.get_main_module(), "quantizelinear") == 4);
+    EXPECT(count_ops(*p.get_main_module(), "dequantizelinear") == 6);
+    auto q = run_on("oracle", p, {{"ids", ids}});
+    encoder::builder fb{c, w, {}, {}};
+    fb.tap  = [](std::size_t, std::vector<argument>) {};
+    auto fp = fb.build();
+    auto f  = run_on("oracle", fp, {{"ids", ids}});
+    auto a = q[0].to_vector<double>();
+    auto b = f[0].to_vector<double>();
+    double num = 0, den = 0;
+    for(std::size_t i = 0; i < a.size(); i++)
+    {
+        EXPECT(std::isfinite(a[i]));
+        num += (a[i] - b[i]) * (a[i] - b[i]);
+        den += b[i] * b[i];
+    }
+    EXPECT(std::sqrt(num / den) < 0.05);
+    // LayerNorm output: rows have mean ~beta and unit-scale spread
+    EXPECT(q[0].get_shape() == shape{shape::float_type, {c.tokens(), c.hidden}});
 }
 
 // ---------------------------------------------------------------- MatMulNBits

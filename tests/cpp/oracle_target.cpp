@@ -3,7 +3,9 @@
 #include <migraphx/passes.hpp>
 #include <migraphx/register_target.hpp>
 #include <cstdint>
+#include <cmath>
 #include <cstring>
+#include <limits>
 
 extern "C" {
 // oracle/ref_oracle.c
@@ -156,19 +158,92 @@ struct cpu_op
             orc_convert(r.data(), orc_type(out.type()), x.data(), orc_type(x.get_shape().type()),
                         out.elements());
         }
-        else if(n == "mul" or n == "add" or n == "sub")
+        else if(n == "erf" or n == "sqrt" or n == "rsqrt" or n == "exp" or n == "tanh" or n == "neg")
+        {
+            // op/unary.hpp with the lambdas of erf.hpp, sqrt.hpp, rsqrt.hpp (1 / std::sqrt(x)),
+            // exp.hpp, tanh.hpp, neg.hpp, applied in the tensor's type
+            argument x = dense(args[0]);
+            auto in    = x.get<float>();
+            auto o     = r.get<float>();
+            for(std::size_t i = 0; i < o.size(); i++)
+            {
+                const float v = in[i];
+                o[i] = n == "erf" ? std::erf(v)
+                                  : (n == "sqrt" ? std::sqrt(v)
+                                                 : (n == "rsqrt" ? 1 / std::sqrt(v)
+                                                                 : (n == "exp" ? std::exp(v)
+                                                                               : (n == "tanh" ? std::tanh(v) : -v))));
+            }
+        }
+        else if(n == "reduce_mean")
+        {
+            // op/reduce_op.hpp:186-202 with reduce_mean.hpp:40-49: double accumulator over the
+            // reduced elements in index order, val / double(count), stored as float.  Last axis.
+            argument x = dense(args[0]);
+            int64_t rows = 0;
+            int64_t cols = 0;
+            rows_cols(x.get_shape(), rows, cols);
+            auto in = x.get<float>();
+            auto o  = r.get<float>();
+            for(int64_t i = 0; i < rows; i++)
+            {
+                double val = 0;
+                for(int64_t c = 0; c < cols; c++)
+                    val = static_cast<double>(in[i * cols + c]) + val;
+                o[i] = static_cast<float>(val / static_cast<double>(cols));
+            }
+        }
+        else if(n == "softmax")
+        {
+            // ref_softmax, src/targets/ref/lowering.cpp:281-312, along the last axis
+            argument x = dense(args[0]);
+            int64_t rows = 0;
+            int64_t cols = 0;
+            rows_cols(x.get_shape(), rows, cols);
+            auto in = x.get<float>();
+            auto o  = r.get<float>();
+            for(int64_t i = 0; i < rows; i++)
+            {
+                double mx = std::numeric_limits<double>::lowest();
+                for(int64_t c = 0; c < cols; c++)
+                    mx = std::max<double>(mx, in[i * cols + c]);
+                for(int64_t c = 0; c < cols; c++)
+                    o[i * cols + c] = std::exp(in[i * cols + c] - mx);
+                double sum = 0;
+                for(int64_t c = 0; c < cols; c++)
+                    sum += o[i * cols + c];
+                for(int64_t c = 0; c < cols; c++)
+                    o[i * cols + c] = o[i * cols + c] / sum;
+            }
+        }
+        else if(n == "gather")
+        {
+            // op/gather.hpp:100-118, axis 0: negative indices wrap
+            argument t = dense(args[0]);
+            argument ix = dense(args[1]);
+            const auto rows      = static_cast<int64_t>(t.get_shape().lens()[0]);
+            const std::size_t rb = t.get_shape().bytes() / rows;
+            auto ids             = ix.to_vector<int64_t>();
+            for(std::size_t i = 0; i < ids.size(); i++)
+            {
+                int64_t id = ids[i] < 0 ? ids[i] + rows : ids[i];
+                std::memcpy(r.data() + i * rb, t.data() + id * rb, rb);
+            }
+        }
+        else if(n == "mul" or n == "add" or n == "sub" or n == "div")
         {
             // op/binary.hpp: the plain C++ operator on the tensor's type
             migraphx::visit_type(out.type(), [&](auto t) {
                 using T = decltype(t);
-                auto x  = args[0].get<T>();
-                auto y  = args[1].get<T>();
+                auto x  = args[0].template get<T>();
+                auto y  = args[1].template get<T>();
                 auto o  = r.get<T>();
                 for(std::size_t i = 0; i < o.size(); i++)
                 {
                     if constexpr(std::is_same<T, float>{} or std::is_same<T, int32_t>{} or
                                  std::is_same<T, double>{})
-                        o[i] = n == "mul" ? x[i] * y[i] : (n == "add" ? x[i] + y[i] : x[i] - y[i]);
+                        o[i] = n == "mul" ? x[i] * y[i]
+                                          : (n == "add" ? x[i] + y[i] : (n == "sub" ? x[i] - y[i] : x[i] / y[i]));
                     else
                         MIGRAPHX_THROW("oracle: " + n + " on " + out.type_string());
                 }
