@@ -170,6 +170,50 @@ def main():
     except Exception as e:
         also["w4a16_gemv_error"] = str(e)
 
+    # ---- skinny int8 quant_dot (config 2) and int4 GEMM at M = 16 / 128 (config 4) ----------
+    try:
+        if args.only_headline:
+            raise RuntimeError("skipped (--only-headline)")
+        for m2 in (16, 128):
+            a2 = torch.randint(-128, 128, (m2, 8192), dtype=torch.int8, device=dev, generator=g)
+            bs = [torch.randint(-128, 128, (8192, 8192), dtype=torch.int8, device=dev, generator=g)
+                  for _ in range(6)]  # 6 x 67 MB: more than the last-level cache
+            c2 = torch.empty((m2, 8192), dtype=torch.int32, device=dev)
+            it = [0]
+
+            def skinny():
+                ops.quant_dot(a2, bs[it[0] % 6], out=c2)
+                it[0] += 1
+
+            t2, _ = _time_launches(skinny, 18, 6)
+            byts = m2 * 8192 + 8192 * 8192 + 4 * m2 * 8192
+            also[f"int8_quant_dot_M{m2}_N8192_K8192"] = {
+                "GB/s": round(byts / t2 / 1e9, 1), "frac_hbm_peak": round(byts / t2 / 1e9 / PEAK_HBM_GBS, 4),
+                "us_per_launch": round(t2 * 1e6, 1)}
+            del bs
+        for m4 in (16, 128):
+            k4, n4, grp = 4096, 14336, 128
+            byts = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * m4 * k4 + 2 * m4 * n4
+            copies = int(640e6 // byts) + 1
+            ws = [torch.randint(0, 256, (n4, k4 // 2), dtype=torch.uint8, device=dev, generator=g)
+                  for _ in range(copies)]
+            sc = (torch.rand((n4, k4 // grp), device=dev, generator=g) * 0.015 + 0.005).half()
+            x = torch.randn((m4, k4), device=dev, generator=g).half()
+            y = torch.empty((m4, n4), dtype=torch.float16, device=dev)
+            it = [0]
+
+            def w4():
+                ops.w4a16_gemm(x, ws[it[0] % copies], sc, grp, zp=8, out=y)
+                it[0] += 1
+
+            t4, _ = _time_launches(w4, 2 * copies, copies)
+            also[f"w4a16_gemm_M{m4}_K{k4}_N{n4}"] = {
+                "GB/s": round(byts / t4 / 1e9, 1), "TFLOPS": round(2.0 * m4 * n4 * k4 / t4 / 1e12, 1),
+                "us_per_launch": round(t4 * 1e6, 1)}
+            del ws
+    except Exception as e:
+        also["skinny_error"] = str(e)
+
     line = {
         "metric": "quant_dot TOPS & % MFMA peak (int8/fp8); int4 W-only GEMV GB/s & % HBM",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
