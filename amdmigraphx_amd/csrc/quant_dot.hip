@@ -23,16 +23,6 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc*,
                           const int32_t*,
                           const int32_t*,
                           hipStream_t);
-bool mi355_skinny_gemm_supported(const mi355_quant_dot_desc*, const void*, const void*, const void*);
-int mi355_skinny_gemm_launch(const mi355_quant_dot_desc*,
-                             const void*,
-                             const void*,
-                             void*,
-                             const float*,
-                             const float*,
-                             const int32_t*,
-                             const int32_t*,
-                             hipStream_t);
 
 namespace {
 
@@ -254,8 +244,6 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
         return MI355_ERR_UNSUPPORTED;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if(d->k > 0 && mi355_skinny_gemm_supported(d, a, b, c))
-        return mi355_skinny_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
     if(d->k > 0 && mi355_dma_gemm_supported(d, a, b))
         return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
     if(d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
