@@ -295,3 +295,66 @@ def w4a16_matmul(a_h, w_packed, scales_h, zp, group):
         z_full = np.repeat(np.asarray(zp, np.uint8), group, axis=1)[:, :k]
     w = dequantizelinear(q, s_full, z_full, U8, F16)        # [N, K] half bits
     return dot(a_h, w.T, F16)
+
+
+# ---- float operators around the GEMMs of an encoder graph -------------------------------------
+
+BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+UN = {"erf": 0, "sqrt": 1, "rsqrt": 2, "exp": 3, "tanh": 4, "neg": 5}
+
+
+def binary_f32(op, a, b):
+    a, b = np.broadcast_arrays(np.float32(a), np.float32(b))
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    out = np.empty(a.shape, np.float32)
+    _lib.orc_binary_f32(BIN[op], _p(out), _p(a), _p(b), ctypes.c_size_t(a.size))
+    return out
+
+
+def unary_f32(op, x):
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(x.shape, np.float32)
+    _lib.orc_unary_f32(UN[op], _p(out), _p(x), ctypes.c_size_t(x.size))
+    return out
+
+
+def _reduced_last(x, axes):
+    """x with the reduced axes moved to the end and flattened: [outer, reduced]."""
+    axes = sorted(a % x.ndim for a in axes)
+    keep = [d for d in range(x.ndim) if d not in axes]
+    xt = np.ascontiguousarray(np.transpose(x, keep + axes))
+    outer = int(np.prod([x.shape[d] for d in keep], dtype=np.int64))
+    return xt.reshape(outer, -1), keep, axes
+
+
+def reduce_mean_f32(x, axes):
+    """Mean over `axes` (kept as length-1 dimensions), accumulated in double in index order."""
+    x = np.float32(x)
+    flat, keep, axes = _reduced_last(x, axes)
+    out = np.empty(flat.shape[0], np.float32)
+    _lib.orc_reduce_mean_f32(_p(out), _p(flat), ctypes.c_int64(flat.shape[0]),
+                             ctypes.c_int64(flat.shape[1]), ctypes.c_int64(1))
+    shp = [1 if d in axes else x.shape[d] for d in range(x.ndim)]
+    return out.reshape(shp)
+
+
+def softmax_f32(x, axis):
+    x = np.ascontiguousarray(x, np.float32)
+    axis, outer, alen, inner = _axis_split(x.shape, axis)
+    out = np.empty(x.shape, np.float32)
+    _lib.orc_softmax_f32(_p(out), _p(x), ctypes.c_int64(outer), ctypes.c_int64(alen),
+                         ctypes.c_int64(inner))
+    return out
+
+
+def gather(data, indices, axis=0):
+    data = np.ascontiguousarray(data)
+    idx = np.asarray(indices, np.int64)
+    axis, outer, alen, inner = _axis_split(data.shape, axis)
+    scalar = idx.ndim == 0
+    flat = np.ascontiguousarray(idx.reshape(-1))
+    out = np.empty((outer, flat.size, inner), data.dtype)
+    _lib.orc_gather(_p(out), _p(data), _p(flat), ctypes.c_int64(flat.size), ctypes.c_int64(outer),
+                    ctypes.c_int64(alen), ctypes.c_int64(inner), ctypes.c_int64(data.itemsize))
+    shp = list(data.shape[:axis]) + ([] if scalar else list(idx.shape)) + list(data.shape[axis + 1:])
+    return out.reshape(shp)

@@ -32,8 +32,20 @@
  *   orc_dot                       test/onnx/verify/matmulnbits_tests.cpp golds
  *                                 (whole unpack -> dequantize -> dot chain)
  *   orc_convert                   test/ref/convert.cpp + closed form
+ *   orc_softmax_f32               test/ref/softmax.cpp:33-107 (two cases, 122
+ *                                 expected values, axis inside the shape)
+ *   orc_reduce_mean_f32           test/ref/reduce_mean.cpp:33-195 (axes {0,2},
+ *                                 {1}, {1,2}, {2} of a 3x2x2 tensor)
+ *   orc_gather                    test/ref/gather.cpp:59-214 (seven cases:
+ *                                 axes 0 / 1 / -1, negative and scalar indices)
+ *   orc_binary_f32, orc_unary_f32 one C operator / libm call each, which is
+ *                                 also how the reference's tests form their
+ *                                 expected values (test/ref/div.cpp:33-50,
+ *                                 erf.cpp:33-49, rsqrt.cpp:33-46); checked
+ *                                 against numpy / math.erf
  */
 #include <fenv.h>
+#include <float.h>
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -643,4 +655,106 @@ void orc_mul_f32(float* out,
     for(int64_t r = 0; r < rows; r++)
         for(int64_t c = 0; c < cols; c++)
             out[r * cols + c] = a[r * a_sr + c * a_sc] * b[r * b_sr + c * b_sc];
+}
+
+/* ------------------------------------------------------------------------
+ * Float operators around the quantized GEMMs of an encoder graph.  Tensors
+ * are dense; a reduced / indexed axis is described as [outer, axis_len, inner].
+ * ---------------------------------------------------------------------- */
+
+/* op::add / sub / mul / div on float tensors: op/binary.hpp:60-90 applies the
+ * plain C++ operator element by element (add.hpp, sub.hpp, mul.hpp, div.hpp). */
+void orc_binary_f32(int op, float* out, const float* a, const float* b, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+    {
+        switch(op)
+        {
+        case 0: out[i] = a[i] + b[i]; break;
+        case 1: out[i] = a[i] - b[i]; break;
+        case 2: out[i] = a[i] * b[i]; break;
+        default: out[i] = a[i] / b[i]; break;
+        }
+    }
+}
+
+/* op::erf / sqrt / rsqrt / exp / tanh / neg on float tensors: op/unary.hpp with
+ * the lambdas std::erf(x) (erf.hpp), std::sqrt(x) (sqrt.hpp), 1 / std::sqrt(x)
+ * (rsqrt.hpp:36-39), std::exp(x), std::tanh(x), -x, each on a float argument. */
+void orc_unary_f32(int op, float* out, const float* x, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+    {
+        const float v = x[i];
+        switch(op)
+        {
+        case 0: out[i] = erff(v); break;
+        case 1: out[i] = sqrtf(v); break;
+        case 2: out[i] = 1 / sqrtf(v); break;
+        case 3: out[i] = expf(v); break;
+        case 4: out[i] = tanhf(v); break;
+        default: out[i] = -v; break;
+        }
+    }
+}
+
+/* op::reduce_mean: op/reduce_op.hpp:186-202 accumulates the reduced elements
+ * in accumulator_type<float> = double (type_traits.hpp:78-81) in index order,
+ * reduce_mean.hpp:45-48 divides by double(count); the store rounds to float. */
+void orc_reduce_mean_f32(float* out, const float* x, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t i = 0; i < inner; i++)
+        {
+            double val = 0.0;
+            for(int64_t a = 0; a < axis_len; a++)
+                val = (double)x[(o * axis_len + a) * inner + i] + val;
+            out[o * inner + i] = (float)(val / (double)axis_len);
+        }
+}
+
+/* softmax: ref_softmax::compute, src/targets/ref/lowering.cpp:281-312.  Per
+ * batch: max over the axis as double; out = float(exp(double(x) - max)); the
+ * sum of those floats in a double; out = float(double(out) / sum). */
+void orc_softmax_f32(float* out, const float* x, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t i = 0; i < inner; i++)
+        {
+            double mx = -DBL_MAX;
+            for(int64_t a = 0; a < axis_len; a++)
+            {
+                double v = (double)x[(o * axis_len + a) * inner + i];
+                mx       = mx < v ? v : mx;
+            }
+            for(int64_t a = 0; a < axis_len; a++)
+            {
+                size_t idx = (size_t)((o * axis_len + a) * inner + i);
+                out[idx]   = (float)exp((double)x[idx] - mx);
+            }
+            double sum = 0.0;
+            for(int64_t a = 0; a < axis_len; a++)
+                sum += (double)out[(o * axis_len + a) * inner + i];
+            for(int64_t a = 0; a < axis_len; a++)
+            {
+                size_t idx = (size_t)((o * axis_len + a) * inner + i);
+                out[idx]   = (float)((double)out[idx] / sum);
+            }
+        }
+}
+
+/* gather: op/gather.hpp:100-118.  data is [outer, axis_len, inner] elements of
+ * elem_size bytes, the n_idx indices replace the axis; a negative index counts
+ * from the end of the axis. */
+void orc_gather(void* out, const void* data, const int64_t* idx, int64_t n_idx, int64_t outer,
+                int64_t axis_len, int64_t inner, int64_t elem_size)
+{
+    const size_t run = (size_t)(inner * elem_size);
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t j = 0; j < n_idx; j++)
+        {
+            int64_t id = idx[j] < 0 ? idx[j] + axis_len : idx[j];
+            memcpy((char*)out + (size_t)(o * n_idx + j) * run,
+                   (const char*)data + (size_t)(o * axis_len + id) * run, run);
+        }
 }

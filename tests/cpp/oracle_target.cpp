@@ -23,6 +23,12 @@ void orc_unpack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t out
 void orc_pack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len,
                    int64_t inner);
 void orc_convert(void* out, int out_type, const void* x, int x_type, size_t n);
+void orc_binary_f32(int op, float* out, const float* a, const float* b, size_t n);
+void orc_unary_f32(int op, float* out, const float* x, size_t n);
+void orc_reduce_mean_f32(float* out, const float* x, int64_t outer, int64_t axis_len, int64_t inner);
+void orc_softmax_f32(float* out, const float* x, int64_t outer, int64_t axis_len, int64_t inner);
+void orc_gather(void* out, const void* data, const int64_t* idx, int64_t n_idx, int64_t outer,
+                int64_t axis_len, int64_t inner, int64_t elem_size);
 }
 
 namespace oracle {
@@ -160,75 +166,43 @@ struct cpu_op
         }
         else if(n == "erf" or n == "sqrt" or n == "rsqrt" or n == "exp" or n == "tanh" or n == "neg")
         {
-            // op/unary.hpp with the lambdas of erf.hpp, sqrt.hpp, rsqrt.hpp (1 / std::sqrt(x)),
-            // exp.hpp, tanh.hpp, neg.hpp, applied in the tensor's type
-            argument x = dense(args[0]);
-            auto in    = x.get<float>();
-            auto o     = r.get<float>();
-            for(std::size_t i = 0; i < o.size(); i++)
-            {
-                const float v = in[i];
-                o[i] = n == "erf" ? std::erf(v)
-                                  : (n == "sqrt" ? std::sqrt(v)
-                                                 : (n == "rsqrt" ? 1 / std::sqrt(v)
-                                                                 : (n == "exp" ? std::exp(v)
-                                                                               : (n == "tanh" ? std::tanh(v) : -v))));
-            }
+            argument x   = dense(args[0]);
+            const int op = n == "erf" ? 0 : (n == "sqrt" ? 1 : (n == "rsqrt" ? 2 : (n == "exp" ? 3 : (n == "tanh" ? 4 : 5))));
+            orc_unary_f32(op, reinterpret_cast<float*>(r.data()),
+                          reinterpret_cast<const float*>(x.data()), out.elements());
         }
-        else if(n == "reduce_mean")
+        else if(n == "reduce_mean" or n == "softmax")
         {
-            // op/reduce_op.hpp:186-202 with reduce_mean.hpp:40-49: double accumulator over the
-            // reduced elements in index order, val / double(count), stored as float.  Last axis.
-            argument x = dense(args[0]);
+            // the last axis: [rows, cols, 1]
+            argument x   = dense(args[0]);
             int64_t rows = 0;
             int64_t cols = 0;
             rows_cols(x.get_shape(), rows, cols);
-            auto in = x.get<float>();
-            auto o  = r.get<float>();
-            for(int64_t i = 0; i < rows; i++)
-            {
-                double val = 0;
-                for(int64_t c = 0; c < cols; c++)
-                    val = static_cast<double>(in[i * cols + c]) + val;
-                o[i] = static_cast<float>(val / static_cast<double>(cols));
-            }
-        }
-        else if(n == "softmax")
-        {
-            // ref_softmax, src/targets/ref/lowering.cpp:281-312, along the last axis
-            argument x = dense(args[0]);
-            int64_t rows = 0;
-            int64_t cols = 0;
-            rows_cols(x.get_shape(), rows, cols);
-            auto in = x.get<float>();
-            auto o  = r.get<float>();
-            for(int64_t i = 0; i < rows; i++)
-            {
-                double mx = std::numeric_limits<double>::lowest();
-                for(int64_t c = 0; c < cols; c++)
-                    mx = std::max<double>(mx, in[i * cols + c]);
-                for(int64_t c = 0; c < cols; c++)
-                    o[i * cols + c] = std::exp(in[i * cols + c] - mx);
-                double sum = 0;
-                for(int64_t c = 0; c < cols; c++)
-                    sum += o[i * cols + c];
-                for(int64_t c = 0; c < cols; c++)
-                    o[i * cols + c] = o[i * cols + c] / sum;
-            }
+            if(n == "reduce_mean")
+                orc_reduce_mean_f32(reinterpret_cast<float*>(r.data()),
+                                    reinterpret_cast<const float*>(x.data()), rows, cols, 1);
+            else
+                orc_softmax_f32(reinterpret_cast<float*>(r.data()),
+                                reinterpret_cast<const float*>(x.data()), rows, cols, 1);
         }
         else if(n == "gather")
         {
-            // op/gather.hpp:100-118, axis 0: negative indices wrap
-            argument t = dense(args[0]);
+            // axis 0
+            argument t  = dense(args[0]);
             argument ix = dense(args[1]);
-            const auto rows      = static_cast<int64_t>(t.get_shape().lens()[0]);
-            const std::size_t rb = t.get_shape().bytes() / rows;
-            auto ids             = ix.to_vector<int64_t>();
-            for(std::size_t i = 0; i < ids.size(); i++)
-            {
-                int64_t id = ids[i] < 0 ? ids[i] + rows : ids[i];
-                std::memcpy(r.data() + i * rb, t.data() + id * rb, rb);
-            }
+            auto ids    = ix.to_vector<int64_t>();
+            const auto rows = static_cast<int64_t>(t.get_shape().lens()[0]);
+            orc_gather(r.data(), t.data(), ids.data(), static_cast<int64_t>(ids.size()), 1, rows,
+                       static_cast<int64_t>(t.get_shape().elements()) / rows,
+                       static_cast<int64_t>(t.get_shape().type_size()));
+        }
+        else if((n == "mul" or n == "add" or n == "sub" or n == "div") and out.type() == shape::float_type)
+        {
+            argument x = dense(args[0]);
+            argument y = dense(args[1]);
+            orc_binary_f32(n == "add" ? 0 : (n == "sub" ? 1 : (n == "mul" ? 2 : 3)),
+                           reinterpret_cast<float*>(r.data()), reinterpret_cast<const float*>(x.data()),
+                           reinterpret_cast<const float*>(y.data()), out.elements());
         }
         else if(n == "mul" or n == "add" or n == "sub" or n == "div")
         {

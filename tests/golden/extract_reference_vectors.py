@@ -213,6 +213,46 @@ for name, body in test_cases(t).items():
     mn.append(c)
 out["matmulnbits"] = mn
 
+# ---- float operators of the encoder graph: softmax, reduce_mean, gather ----------------------
+t = read("test/ref/softmax.cpp")
+cases = test_cases(t)
+sm = []
+for name in ("softmax_simple_test", "softmax_test"):
+    body = cases[name]
+    ax = int(re.search(r'"softmax",\s*\{\{"axis",\s*(-?\d+)\}\}', body).group(1))
+    sm.append({"name": name, "source": "test/ref/softmax.cpp", "shape": shape(body, "a_shape"),
+               "axis": ax, "a": vec(body, "a"), "gold": vec(body, "gold")})
+out["softmax"] = sm
+
+t = read("test/ref/reduce_mean.cpp")
+cases = test_cases(t)
+rm = []
+for name in ("reduce_mean_axis02", "reduce_mean_axis1", "reduce_mean_axis12", "reduce_mean_axis2"):
+    body = cases[name]
+    axes = num_list(re.search(r'"reduce_mean",\s*\{\{"axes",\s*\{([^}]*)\}\}\}', body).group(1))
+    inp = num_list(re.search(r"migraphx::literal\{s,\s*\{([^}]*)\}\}", body).group(1))
+    rm.append({"name": name, "source": "test/ref/reduce_mean.cpp", "shape": shape(body, "s"),
+               "axes": axes, "input": inp, "gold": vec(body, "gold")})
+out["reduce_mean"] = rm
+
+t = read("test/ref/gather.cpp")
+cases = test_cases(t)
+ga = []
+for i in range(1, 8):
+    body = cases["gather_test_%d" % i]
+    n = num_list(re.search(r"std::vector<float> data\(([^)]*)\)", body).group(1).replace("*", ","))
+    count = 1
+    for v in n:
+        count *= v
+    sidx = re.search(r"migraphx::shape s_indices\{migraphx::shape::int32_type(?:,\s*\{([^}]*)\})?\}", body)
+    ga.append({"name": "gather_test_%d" % i, "source": "test/ref/gather.cpp",
+               "data_iota_start": 0.5, "data_count": count, "shape": shape(body, "s"),
+               "indices_lens": num_list(sidx.group(1)) if sidx.group(1) else None,
+               "indices": vec(body, "indices"),
+               "axis": int(re.search(r"int axis\s*=\s*(-?\d+);", body).group(1)),
+               "gold": vec(body, "golden")})
+out["gather"] = ga
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")
