@@ -57,6 +57,7 @@ struct dma_params
     int scale_a_mode, scale_b_mode;
     int zp_a, zp_b;
     int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
+    int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
 };
 
 // s_waitcnt with only the vector-memory counter constrained
@@ -383,7 +384,9 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
             for(int j = 0; j < 2; j++)
             {
                 const int tile = FP8 ? 2 * S + i : i;
-                acc[tile][j]   = mfma(fa[S][i], fb[S][j], acc[tile][j]);
+                // B tile first: the accumulator holds the tile transposed, so that a lane owns
+                // runs of 4 consecutive columns of C (see the epilogue)
+                acc[tile][j]   = mfma(fb[S][j], fa[S][i], acc[tile][j]);
             }
     };
 
@@ -438,67 +441,108 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #undef WAIT_STEP
 
     // ---- epilogue ------------------------------------------------------------------
-    // 32 x 32 accumulator: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4,
-    // column l % 32.
+    // The operands went in swapped, so element e of lane l belongs to row l % 32 of the A tile
+    // and column 8*(e/4) + 4*(l/32) + e%4 of the B tile: four groups of 4 consecutive columns,
+    // each written with one store when C allows it (p.vec_store).
 #pragma unroll
-    for(int j = 0; j < 2; j++)
+    for(int i = 0; i < 4; i++)
     {
-        const int col = n0 + wave_n * 64 + j * 32 + lrow;
-        if(col >= p.n)
+        const int row = m0 + wave_m * 128 + i * 32 + lrow;
+        if(row >= p.m)
             continue;
-        float sb    = 1.f;
-        int32_t csb = 0;
+        float sa     = 1.f;
+        int64_t zrow = 0;
         if constexpr(DEQ)
         {
-            if(p.scale_b_mode == MI355_QP_PER_TENSOR)
-                sb = p.scale_b[0];
-            else if(p.scale_b_mode == MI355_QP_PER_COL)
-                sb = p.scale_b[col];
-            if(p.zp_a != 0)
-                csb = p.colsum_b[col];
+            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                sa = p.scale_a[0];
+            else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                sa = p.scale_a[row];
+            if(!FP8 && p.zp_b != 0)
+                zrow = (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b;
         }
 #pragma unroll
-        for(int i = 0; i < 4; i++)
+        for(int j = 0; j < 2; j++)
         {
 #pragma unroll
-            for(int e = 0; e < 16; e++)
+            for(int g = 0; g < 4; g++)
             {
-                const int row = m0 + wave_m * 128 + i * 32 + 8 * (e >> 2) + 4 * lgrp + (e & 3);
-                if(row >= p.m)
+                const int col = n0 + wave_n * 64 + j * 32 + 8 * g + 4 * lgrp;
+                if(col >= p.n)
                     continue;
                 const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                const bool whole  = p.vec_store && col + 4 <= p.n;
+                float v[4];
+                if constexpr(DEQ)
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                    {
+                        const int c = min(col + e, p.n - 1);
+                        float sb    = 1.f;
+                        if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                            sb = p.scale_b[0];
+                        else if(p.scale_b_mode == MI355_QP_PER_COL)
+                            sb = p.scale_b[c];
+                        // scale = fp32 product of the two scales (the graph's `mul`), then
+                        // (double(acc) - double(zp)) * scale in double, one rounding to float
+                        // (dequantizelinear)
+                        const float s = sa * sb;
+                        if constexpr(FP8)
+                        {
+                            // the accumulator is a float: double(acc) * double(s) rounded once
+                            // to float is exactly the correctly rounded fp32 product
+                            v[e] = acc[i][j][4 * g + e] * s;
+                        }
+                        else
+                        {
+                            int64_t zp = zrow;
+                            if(p.zp_a != 0)
+                                zp += (int64_t)p.zp_a * p.colsum_b[c];
+                            const double d = (double)acc[i][j][4 * g + e] - (double)(int32_t)zp;
+                            v[e]           = (float)(d * (double)s);
+                        }
+                    }
+                }
                 if constexpr(!DEQ)
                 {
-                    if constexpr(FP8)
-                        static_cast<float*>(p.c)[idx] = acc[i][j][e];
+                    using out_t = std::conditional_t<FP8, float, int32_t>;
+                    out_t* o    = static_cast<out_t*>(p.c) + idx;
+                    if(whole)
+                    {
+                        using vec_t = out_t __attribute__((ext_vector_type(4)));
+                        *reinterpret_cast<vec_t*>(o) =
+                            vec_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                  acc[i][j][4 * g + 3]};
+                    }
                     else
-                        static_cast<int32_t*>(p.c)[idx] = acc[i][j][e];
+                    {
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            if(col + e < p.n)
+                                o[e] = acc[i][j][4 * g + e];
+                    }
+                }
+                else if(whole)
+                {
+                    if constexpr(OUT == MI355_F32)
+                        *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) =
+                            v4f{v[0], v[1], v[2], v[3]};
+                    else if constexpr(OUT == MI355_F16)
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                            convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+                    else
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
+                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
                 }
                 else
                 {
-                    float sa = 1.f;
-                    if(p.scale_a_mode == MI355_QP_PER_TENSOR)
-                        sa = p.scale_a[0];
-                    else if(p.scale_a_mode == MI355_QP_PER_ROW)
-                        sa = p.scale_a[row];
-                    // scale = fp32 product of the two scales (the graph's `mul`),
-                    // then (double(acc) - double(zp)) * scale in double, one
-                    // rounding to float (dequantizelinear)
-                    const float s = sa * sb;
-                    double d;
-                    if constexpr(FP8)
-                    {
-                        d = (double)acc[i][j][e];
-                    }
-                    else
-                    {
-                        int64_t zp = (int64_t)p.zp_a * csb;
-                        if(p.zp_b != 0)
-                            zp += (int64_t)p.zp_b * p.rowsum_a[row] -
-                                  (int64_t)p.k * p.zp_a * p.zp_b;
-                        d = (double)acc[i][j][e] - (double)(int32_t)zp;
-                    }
-                    store1<OUT>(p.c, idx, (float)(d * (double)s));
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        if(col + e < p.n)
+                            store1<OUT>(p.c, idx + e, v[e]);
                 }
             }
         }
@@ -1011,6 +1055,12 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     p.zp_b         = d->zp_b;
     const bool fp8 = d->in_type == MI355_FP8;
     const bool deq = d->dequant != 0;
+    {
+        const size_t esz = deq ? mi355_dtype_size(d->out_type) : 4;
+        p.vec_store = d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
+                      reinterpret_cast<uintptr_t>(c) % (4 * esz) == 0;
+    }
+    p.ksplit = 1;
     if(fp8)
         return d->trans_b ? launch_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_out<true, false>(p, (int)d->batch, deq, d->out_type, stream);
