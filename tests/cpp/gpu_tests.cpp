@@ -9,6 +9,7 @@
 #include "test.hpp"
 #include <chrono>
 #include <fstream>
+#include <thread>
 
 using namespace testutil;
 using migraphx::shape;
@@ -377,6 +378,41 @@ TEST_CASE(standalone_operators)
     mm->add_return({q, h, ct, pk, un});
     argument xa{shape{shape::float_type, {r, c}}, normal_floats(r * c, 1.0f, 92)};
     expect_same(p, {{"x", xa}});
+}
+
+TEST_CASE(concurrent_programs)
+{
+    // the reference's verify harness compiles and evaluates programs for several targets from
+    // separate threads (test/verify/run_verify.cpp:46-58): registries are read-only after load, each
+    // compiled program owns its context and stream
+    const std::size_t m = 64, k = 256, n = 128;
+    auto p = qdq_matmul(m, k, n, false, 2, -3, shape::float_type, 9);
+    argument x{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 10)};
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    auto want = run_on("oracle", p, {{"x", x}});
+    std::vector<int> ok(4, 0);
+    std::vector<std::thread> threads;
+    for(int t = 0; t < 4; t++)
+        threads.emplace_back([&, t] {
+            try
+            {
+                for(int rep = 0; rep < 3; rep++)
+                {
+                    auto got = run_on(t % 2 == 0 ? "mi355" : "oracle", p, {{"x", x}}, rep % 2 == 1 and t % 2 == 0);
+                    if(not same_bytes(got[0], want[0]))
+                        return;
+                }
+                ok[t] = 1;
+            }
+            catch(const std::exception& e)
+            {
+                std::cout << "thread " << t << ": " << e.what() << std::endl;
+            }
+        });
+    for(auto& th : threads)
+        th.join();
+    for(int t = 0; t < 4; t++)
+        EXPECT(ok[t] == 1);
 }
 
 TEST_CASE(no_host_fallback)

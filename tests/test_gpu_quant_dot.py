@@ -280,3 +280,31 @@ def test_full_size_int8_properties(ops):
     lhs = c.double().sum(0)
     rhs = a.double().sum(0) @ b.double()
     assert torch.equal(lhs, rhs)
+
+
+def test_graph_replay_of_split_k_and_int4_kernels(ops):
+    """A captured HIP graph holding the split-K quant_dot (zero-fill kernel + integer
+    atomics) and the int4 GEMM must give the eager result on every replay, with eager
+    work and synchronisation between the replays."""
+    rng = np.random.default_rng(21)
+    m, n, k = 16, 1024, 4096
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    want = orc.quant_dot(a, b, orc.I8)
+    ta, tb = dev(a), dev(b)
+    out = torch.empty((m, n), dtype=torch.int32, device="cuda")
+    ops.quant_dot(ta, tb, out=out)  # warm up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.quant_dot(ta, tb, out=out)
+    for rep in range(3):
+        out.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want), rep
+        # eager work between the replays
+        assert np.array_equal(ops.quant_dot(ta, tb).cpu().numpy(), want)
