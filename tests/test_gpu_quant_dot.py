@@ -308,3 +308,35 @@ def test_graph_replay_of_split_k_and_int4_kernels(ops):
         assert np.array_equal(out.cpu().numpy(), want), rep
         # eager work between the replays
         assert np.array_equal(ops.quant_dot(ta, tb).cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("k,n", [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)])
+def test_full_size_fp8_config3_shapes(ops, k, n):
+    """BASELINE config 3 at its real sizes (M = 4096).  fp8 codes that hold small integers
+    make every partial sum an integer below 2^24, which the fp32 accumulator and the MFMA's
+    internal alignment hold exactly: the fp8 quant_dot must then equal the int8 quant_dot of
+    the same integers, element for element, over the whole result.  The bf16 epilogue is
+    checked against the float result with the scale applied (one truncation)."""
+    m = 4096
+    g = torch.Generator(device="cuda")
+    g.manual_seed(k + n)
+    ai = torch.randint(-4, 5, (m, k), dtype=torch.int8, device="cuda", generator=g)
+    bi = torch.randint(-4, 5, (k, n), dtype=torch.int8, device="cuda", generator=g)
+    # e4m3 codes of the integers -4..4
+    lut = torch.tensor([int(orc.fp8_from_f32(np.float32([v]))[0]) for v in range(-4, 5)],
+                       dtype=torch.uint8, device="cuda")
+    a8 = lut[(ai.long() + 4)]
+    b8 = lut[(bi.long() + 4)]
+    print("fp8 full size", k, n, flush=True)
+    want = ops.quant_dot(ai, bi)                    # int32, exact
+    got = ops.quant_dot(a8, b8, fp8=True)           # float
+    assert torch.equal(got, want.float())
+    s1 = torch.tensor([0.0078125], device="cuda")    # powers of two: the scaled value is exact
+    s2 = torch.tensor([0.25], device="cuda")
+    out = ops.quant_dot(a8, b8, fp8=True, scale_a=s1, scale_b=s2, out_dtype=torch.bfloat16)
+    exact = want.float() * (0.0078125 * 0.25)
+    # bf16 by truncation: never above the exact value in magnitude, within one bf16 step
+    diff = (exact.abs() - out.float().abs())
+    assert (diff >= 0).all()
+    assert (diff <= exact.abs() * 2.0**-7).all()
+    assert (out.float().sign() * exact.sign() >= 0).all()

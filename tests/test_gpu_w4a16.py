@@ -146,3 +146,46 @@ def test_w4a16_matrix_core_kernel_strided_activations_and_output(ops):
                                orc.U8, orc.F16)
     _check(half_bits(out[:, :n].contiguous()), want, a, wdq)
     assert (out[:, n:] == 0).all()
+
+
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 14336), (14336, 4096)])
+def test_w4a16_full_size_config4_shapes(ops, k, n):
+    """BASELINE config 4 at its real sizes, M in {1, 16, 128}: one-hot activation rows pick
+    single dequantized weights out of the full matrix (exact, for every kernel), and the
+    batched kernels agree with the M = 1 kernel row by row within the summation tolerance."""
+    g = 128
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(k * 3 + n)
+    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda", generator=gen)
+    sc = (torch.rand((n, k // g), device="cuda", generator=gen) * 0.015 + 0.005).half()
+    print("w4a16 full size", k, n, flush=True)
+    # expected dequantized weights for a few k positions, computed with torch on the device:
+    # half((q - 8) * scale) with truncation = the float product's bits shifted
+    ks = [0, 1, 127, 128, k // 2 + 5, k - 1]
+    onehot = torch.zeros((len(ks), k), dtype=torch.float16, device="cuda")
+    for i, kk in enumerate(ks):
+        onehot[i, kk] = 1.0
+    want_rows = []
+    for kk in ks:
+        byte = w[:, kk // 2].int()
+        q = (byte >> 4) if kk % 2 else (byte & 0xF)
+        prod = (q - 8).float() * sc[:, kk // g].float()
+        want_rows.append(orc.half_from_f32(prod.cpu().numpy()))
+    want = np.stack(want_rows)
+    for m in (1, 16, 128):
+        a = torch.zeros((m, k), dtype=torch.float16, device="cuda")
+        rows = min(m, len(ks))
+        a[:rows] = onehot[:rows]
+        got = ops.w4a16_gemm(a, w, sc, g, zp=8)
+        assert np.array_equal(half_bits(got[:rows]), want[:rows]), m
+        assert (got[rows:] == 0).all()
+    # random activations: every row of the M = 16 / 128 result against the M = 1 kernel
+    x = torch.randn((128, k), device="cuda", generator=gen).half()
+    big = ops.w4a16_gemm(x, w, sc, g, zp=8)
+    mid = ops.w4a16_gemm(x[:16], w, sc, g, zp=8)
+    for r in (0, 7, 15):
+        one = ops.w4a16_gemm(x[r:r + 1], w, sc, g, zp=8)
+        for other in (big[r:r + 1], mid[r:r + 1]):
+            d = (other.float() - one.float()).abs()
+            tol = torch.maximum(one.float().abs() * 2e-3, torch.tensor(2e-3, device="cuda"))
+            assert (d <= tol).all(), (r, d.max().item())
