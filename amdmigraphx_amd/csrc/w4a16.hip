@@ -12,6 +12,7 @@
 // The products a*w are exact in fp32 (11 x 11 significant bits); only the
 // running sum differs from the reference's double accumulator in the last
 // bits, which the parity tolerance covers.
+#include <type_traits>
 #include "common.h"
 
 namespace {

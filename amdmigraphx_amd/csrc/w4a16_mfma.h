@@ -30,9 +30,6 @@
 // field of s at least 5); a wave that meets a smaller scale unpacks the high nibble separately.
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
-constexpr int WL_CHUNK_K = 2048;                  // k per chunk
-constexpr int WL_ROW     = WL_CHUNK_K / 2;        // bytes of one weight row in a chunk
-constexpr int WL_PITCH   = WL_ROW + 16;           // LDS row pitch
 constexpr int WL_WAVES   = 8;                     // compute waves; one more wave fetches
 constexpr int WL_THREADS = (WL_WAVES + 1) * 64;
 
@@ -62,8 +59,14 @@ MI355_DEVINL void wl_barrier()
 template <int MT, int NT, bool SIMPLE>
 __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
 {
+    constexpr int WL_CHUNK_K  = NT >= 4 ? 1024 : 2048; // k per chunk
+    constexpr int WL_ROW      = WL_CHUNK_K / 2;        // bytes of one weight row in a chunk
+    constexpr int WL_PITCH    = WL_ROW + 16;           // LDS row pitch
+    constexpr int SPC         = WL_CHUNK_K / 128;      // steps per chunk
+    constexpr int SPW         = SPC / WL_WAVES;        // steps of a chunk per wave: 1 or 2
     constexpr int RING        = NT == 1 ? 4 : 3;
     constexpr int CHUNK_BYTES = 16 * NT * WL_PITCH;
+    static_assert(RING * CHUNK_BYTES <= 160 * 1024 && WL_WAVES * NT * MT * 4 * 64 * 4 <= 160 * 1024);
     constexpr int RED_BYTES   = WL_WAVES * NT * MT * 4 * 64 * 4;
     constexpr int LDS_BYTES   = RING * CHUNK_BYTES > RED_BYTES ? RING * CHUNK_BYTES : RED_BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
@@ -145,9 +148,11 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
         uint8_t z[NT][NQ];
         v8h af[A_AHEAD ? 4 : 1][MT];
     };
-    auto request = [&](step_inputs& in, int step) {
-        if(step >= nsteps)
-            return;
+    // A request is unconditional -- past the end of K it repeats the last step and its result goes
+    // unused -- so that the number of loads in flight at any point is known at compile time and a
+    // step waits for its own inputs only, not for the request issued after them.
+    auto request = [&](step_inputs& in, int step) __attribute__((always_inline)) {
+        step = step < nsteps ? step : nsteps - 1;
 #pragma unroll
         for(int t = 0; t < NT; t++)
 #pragma unroll
@@ -180,7 +185,9 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
     };
 
     // one step (128 k) of the workgroup's column tiles
-    auto do_step = [&](step_inputs& in, int step, uint32_t slot_addr, int s_in_chunk) {
+    auto step_body = [&](auto fast_tag, step_inputs& in, int step, uint32_t slot_addr, int s_in_chunk)
+                         __attribute__((always_inline)) {
+        constexpr bool fast = decltype(fast_tag)::value;
         // without the second register set: all operands of the step up front for up to four
         // M-tiles, per quarter for eight
         constexpr bool A_UPFRONT = !A_AHEAD && MT <= 4;
@@ -216,13 +223,9 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
                 wa[3]    = t23[1];
             }
             // scale and zero point as packed constants: (s, s/16) and (1024 + zp, 1024 + 16*zp) for
-            // the two-nibbles-at-once form, (s, s) and (1024 + zp, 1024 + zp) otherwise.  The choice
-            // is wave-uniform; the separate-nibble form is right for any scale.
-            bool fast = false;
+            // the two-nibbles-at-once form, (s, s) and (1024 + zp, 1024 + zp) otherwise
             h2 zoff = {}, scv = {};
             auto constants = [&](uint32_t sb, uint32_t z) {
-                const uint32_t sexp = (sb >> 10) & 0x1fu;
-                fast = __builtin_amdgcn_ballot_w64(sexp >= 5 && sexp <= 30) == ~0ull;
                 const uint32_t zhi = fast ? (z << 4) : z;
                 const uint32_t shi = fast ? sb - (4u << 10) : sb;
                 zoff = __builtin_bit_cast(h2, (0x6400u | z) | ((0x6400u | zhi) << 16));
@@ -277,6 +280,25 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
         }
     };
 
+    // The two-nibbles-at-once form needs s/16 to be a normal half for every scale of the step; the
+    // choice is made once per step and is wave-uniform, so the inner loops carry no branch.  The
+    // separate-nibble form is right for any scale.
+    auto do_step = [&](step_inputs& in, int step, uint32_t slot_addr, int s_in_chunk) __attribute__((always_inline)) {
+        bool ok = true;
+#pragma unroll
+        for(int t = 0; t < NT; t++)
+#pragma unroll
+            for(int q = 0; q < NQ; q++)
+            {
+                const uint32_t sexp = ((uint32_t)in.sb[t][q] >> 10) & 0x1fu;
+                ok                  = ok && sexp >= 5 && sexp <= 30;
+            }
+        if(__builtin_amdgcn_ballot_w64(ok) == __builtin_amdgcn_ballot_w64(true))
+            step_body(std::true_type{}, in, step, slot_addr, s_in_chunk);
+        else
+            step_body(std::false_type{}, in, step, slot_addr, s_in_chunk);
+    };
+
     // ---- main loop ------------------------------------------------------------------------------
     // Barrier c (one per chunk) says: chunk c has landed, and every compute wave is done with chunk
     // c - 1, whose ring slot the next fetch overwrites.  The fetch wave issues 16*NT loads per chunk;
@@ -290,8 +312,10 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
                 issue_chunk(c);
         for(int c = 0; c < nchunks; c++)
         {
+            // (the counter holds at most 63: waiting for one load more than needed is harmless)
+            constexpr int AHEAD = (RING - 2) * 16 * NT;
             if(c + RING - 2 < nchunks)
-                wl_wait_vmcnt<(RING - 2) * 16 * NT>();
+                wl_wait_vmcnt<(AHEAD < 63 ? AHEAD : 63)>();
             else
                 wl_wait_vmcnt<0>();
             wl_barrier();
@@ -301,20 +325,42 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
     }
     else
     {
-        // this wave's steps: chunk c, step-in-chunk wave and wave + 8; two input sets alternate
+        // this wave's steps: step-in-chunk wave (and wave + 8 where a chunk has 16 steps) of every
+        // chunk; two input sets alternate from step to step
         step_inputs in[2];
         request(in[0], wave);
-        for(int c = 0; c < nchunks; c++)
+        if constexpr(SPW == 2)
         {
-            wl_barrier();
-            const uint32_t slot_addr = lds0 + (c % RING) * CHUNK_BYTES;
-            const int step0          = c * (WL_CHUNK_K / 128) + wave;
-            request(in[1], step0 + WL_WAVES);
-            if(step0 < nsteps)
-                do_step(in[0], step0, slot_addr, wave);
-            request(in[0], step0 + WL_CHUNK_K / 128);
-            if(step0 + WL_WAVES < nsteps)
-                do_step(in[1], step0 + WL_WAVES, slot_addr, wave + WL_WAVES);
+            for(int c = 0; c < nchunks; c++)
+            {
+                wl_barrier();
+                const uint32_t slot_addr = lds0 + (c % RING) * CHUNK_BYTES;
+                const int step0          = c * SPC + wave;
+                request(in[1], step0 + WL_WAVES);
+                if(step0 < nsteps)
+                    do_step(in[0], step0, slot_addr, wave);
+                request(in[0], step0 + SPC);
+                if(step0 + WL_WAVES < nsteps)
+                    do_step(in[1], step0 + WL_WAVES, slot_addr, wave + WL_WAVES);
+            }
+        }
+        else
+        {
+            for(int c = 0; c < nchunks; c += 2)
+            {
+                wl_barrier();
+                const int step0 = c * SPC + wave;
+                request(in[1], step0 + SPC);
+                if(step0 < nsteps)
+                    do_step(in[0], step0, lds0 + (c % RING) * CHUNK_BYTES, wave);
+                if(c + 1 < nchunks)
+                {
+                    wl_barrier();
+                    request(in[0], step0 + 2 * SPC);
+                    if(step0 + SPC < nsteps)
+                        do_step(in[1], step0 + SPC, lds0 + ((c + 1) % RING) * CHUNK_BYTES, wave);
+                }
+            }
         }
     }
 
@@ -356,32 +402,32 @@ bool mfma_gemm_supported(const w4_params& p)
            (int64_t)p.m * p.lda * 2 < (1ll << 31);
 }
 
-template <int MT>
+template <int MT, int NT, bool SIMPLE>
+int launch_mfma_variant(const w4_params& p, hipStream_t s)
+{
+    hipLaunchKernelGGL((w4a16_mfma_kernel<MT, NT, SIMPLE>), dim3(p.n / (16 * NT)), dim3(WL_THREADS), 0, s, p);
+    return mi355_launch_status();
+}
+
+// Every workgroup reads all of A's rows once, from L2: M*K*2 bytes per workgroup against the
+// 8*NT*K bytes of weights it owns, so the activations are most of what a CU pulls in unless a
+// workgroup's column tile is wide.  The widest tile (NT_MAX column tiles, as the registers allow)
+// that still leaves about one workgroup per CU is taken.
+template <int MT, int NT_MAX, bool SIMPLE>
 int launch_mfma_tiles(const w4_params& p, hipStream_t s)
 {
-    const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
-    // two column tiles per workgroup halve the activation traffic; taken when that still leaves
-    // every CU a workgroup
-    // (not with 8 M-tiles: the accumulators of two column tiles would not fit the registers)
-    const bool two = MT <= 4 && p.n % 32 == 0 && p.n / 32 >= 256;
-    if constexpr(MT <= 4)
+    constexpr int64_t enough = 200;
+    if constexpr(NT_MAX >= 4)
     {
-        if(two)
-        {
-            if(simple)
-                hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 2, true>), dim3(p.n / 32), dim3(WL_THREADS), 0, s, p);
-            else
-                hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 2, false>), dim3(p.n / 32), dim3(WL_THREADS), 0, s, p);
-            return mi355_launch_status();
-        }
+        if(p.n % 64 == 0 && p.n / 64 >= enough)
+            return launch_mfma_variant<MT, 4, SIMPLE>(p, s);
     }
+    if constexpr(NT_MAX >= 2)
     {
-        if(simple)
-            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 1, true>), dim3(p.n / 16), dim3(WL_THREADS), 0, s, p);
-        else
-            hipLaunchKernelGGL((w4a16_mfma_kernel<MT, 1, false>), dim3(p.n / 16), dim3(WL_THREADS), 0, s, p);
+        if(p.n % 32 == 0 && p.n / 32 >= enough)
+            return launch_mfma_variant<MT, 2, SIMPLE>(p, s);
     }
-    return mi355_launch_status();
+    return launch_mfma_variant<MT, 1, SIMPLE>(p, s);
 }
 
 // M rows in chunks of at most 128
@@ -394,14 +440,16 @@ int launch_mfma_gemm(const w4_params& p0, hipStream_t s)
         p.out       = p0.out + (int64_t)m0 * p0.ldc;
         p.m         = p0.m - m0 < 128 ? p0.m - m0 : 128;
         int st;
+        // (the general zero-point form keeps more per-step state and has room for narrower tiles)
+        const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
         if(p.m <= 16)
-            st = launch_mfma_tiles<1>(p, s);
+            st = simple ? launch_mfma_tiles<1, 4, true>(p, s) : launch_mfma_tiles<1, 2, false>(p, s);
         else if(p.m <= 32)
-            st = launch_mfma_tiles<2>(p, s);
+            st = simple ? launch_mfma_tiles<2, 4, true>(p, s) : launch_mfma_tiles<2, 2, false>(p, s);
         else if(p.m <= 64)
-            st = launch_mfma_tiles<4>(p, s);
+            st = simple ? launch_mfma_tiles<4, 2, true>(p, s) : launch_mfma_tiles<4, 1, false>(p, s);
         else
-            st = launch_mfma_tiles<8>(p, s);
+            st = simple ? launch_mfma_tiles<8, 1, true>(p, s) : launch_mfma_tiles<8, 1, false>(p, s);
         if(st != MI355_OK)
             return st;
     }
