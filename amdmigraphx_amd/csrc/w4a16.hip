@@ -13,6 +13,7 @@
 // running sum differs from the reference's double accumulator in the last
 // bits, which the parity tolerance covers.
 #include <type_traits>
+#include <utility>
 #include "common.h"
 
 namespace {
@@ -391,6 +392,7 @@ int launch_gemv_m1(const w4_params& p, hipStream_t s)
 }
 
 #include "w4a16_mfma.h"
+#include "w4a16_tile.h"
 
 } // namespace
 

@@ -430,6 +430,9 @@ int launch_mfma_tiles(const w4_params& p, hipStream_t s)
     return launch_mfma_variant<MT, 1, SIMPLE>(p, s);
 }
 
+bool tile_gemm_supported(const w4_params& p);
+int launch_tile_gemm(const w4_params& p, hipStream_t s);
+
 // M rows in chunks of at most 128
 int launch_mfma_gemm(const w4_params& p0, hipStream_t s)
 {
@@ -440,6 +443,13 @@ int launch_mfma_gemm(const w4_params& p0, hipStream_t s)
         p.out       = p0.out + (int64_t)m0 * p0.ldc;
         p.m         = p0.m - m0 < 128 ? p0.m - m0 : 128;
         int st;
+        if(tile_gemm_supported(p))
+        {
+            st = launch_tile_gemm(p, s);
+            if(st != MI355_OK)
+                return st;
+            continue;
+        }
         // (the general zero-point form keeps more per-step state and has room for narrower tiles)
         const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
         if(p.m <= 16)

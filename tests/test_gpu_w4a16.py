@@ -132,6 +132,70 @@ def test_w4a16_matrix_core_kernel_exact_weights_all_zero_point_forms(ops):
             assert np.array_equal(half_bits(got), want), (lo, zmode)
 
 
+# ---- more than 32 rows and N % 128 == 0: the 64 x 128 tile kernel ------------------------
+
+@pytest.mark.parametrize("m,n,k,g", [(33, 128, 128, 128), (64, 256, 384, 128), (65, 128, 1152, 64),
+                                     (100, 384, 2048 + 128, 32), (128, 128, 512, 128)])
+def test_w4a16_tile_kernel_matches_oracle(ops, m, n, k, g):
+    """K an even and an odd multiple of 128 (the last chunk of 256 is then half used), row
+    counts that leave the second 64-row block nearly empty, several groups per step."""
+    rng = np.random.default_rng(m * 11 + n + k + g)
+    a, packed, scales, wq = _case(rng, m, n, k, g)
+    want = orc.w4a16_matmul(a, packed, scales, 8, g)
+    print("w4a16 tile", m, n, k, g, flush=True)
+    got = ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8)
+    wdq = orc.dequantizelinear(wq, np.repeat(scales, g, axis=1), np.full(wq.shape, 8, np.uint8),
+                               orc.U8, orc.F16)
+    _check(half_bits(got), want, a, wdq)
+
+
+def test_w4a16_tile_kernel_exact_weights_all_zero_point_forms(ops):
+    """One-hot activations in 70 rows (both 64-row blocks): each output is one dequantized
+    weight and must match bit for bit, for scalar, per-group and packed zero points and
+    for scales on both sides of the range of the (s, s/16) form."""
+    rng = np.random.default_rng(21)
+    n, k, g = 256, 640, 32
+    m = 70
+    wq = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = orc.pack_int4(wq)
+    a = np.zeros((m, k), np.float32)
+    for i in range(m):
+        a[i, (i * 53 + 7) % k] = 1.0 if i % 2 == 0 else -2.0
+    ab = orc.half_from_f32(a)
+    for lo, hi in ((0.005, 0.02), (2.0**-16, 2.0**-12), (0.5, 3.0)):
+        scales = orc.half_from_f32(rng.uniform(lo, hi, (n, k // g)).astype(np.float32))
+        zp = rng.integers(0, 16, (n, k // g), dtype=np.uint8)
+        for zmode in ("scalar", "group", "packed"):
+            print("w4a16 tile exact", lo, zmode, flush=True)
+            if zmode == "scalar":
+                want = orc.w4a16_matmul(ab, packed, scales, 3, g)
+                got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=3)
+            elif zmode == "group":
+                want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+                got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=dev(zp))
+            else:
+                want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+                got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g,
+                                     zp=dev(orc.pack_int4(zp)), zp_mode=ops.W4ZP.PACKED)
+            assert np.array_equal(half_bits(got), want), (lo, zmode)
+
+
+def test_w4a16_tile_kernel_strided_activations_and_output(ops):
+    rng = np.random.default_rng(22)
+    m, n, k, g = 90, 128, 384, 128
+    a, packed, scales, wq = _case(rng, m, n, k, g)
+    want = orc.w4a16_matmul(a, packed, scales, 8, g)
+    big = np.zeros((m, k + 64), np.uint16)
+    big[:, :k] = a
+    a_dev = half_dev(big)[:, :k]
+    out = torch.zeros((m, n + 16), dtype=torch.float16, device="cuda")
+    ops.w4a16_gemm(a_dev, dev(packed), half_dev(scales), g, zp=8, out=out[:, :n])
+    wdq = orc.dequantizelinear(wq, np.repeat(scales, g, axis=1), np.full(wq.shape, 8, np.uint8),
+                               orc.U8, orc.F16)
+    _check(half_bits(out[:, :n].contiguous()), want, a, wdq)
+    assert (out[:, n:] == 0).all()
+
+
 def test_w4a16_matrix_core_kernel_strided_activations_and_output(ops):
     rng = np.random.default_rng(13)
     m, n, k, g = 20, 80, 384, 128
