@@ -633,16 +633,19 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
         }
     }
-    auto issue_slab = [&](int kt) {
+    // A wave's four loads of a slab go out one at a time, each between two runs of MFMAs: a load
+    // instruction occupies the CU's memory pipeline for about 47 cycles, so 32 of them issued
+    // together at the top of a slab would hold every wave at its issue for most of a slab's MFMA
+    // time with the matrix cores idle.
+    auto issue_a = [&](int kt, int h) {
         uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
         const uint8_t* a_base = ga + (int64_t)kt * BK;
+        load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
+    };
+    auto issue_b = [&](int kt, int h) {
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
         const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
-#pragma unroll
-        for(int h = 0; h < 2; h++)
-            load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
-#pragma unroll
-        for(int h = 0; h < 2; h++)
-            load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+        load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
     };
 
     // ---- LDS -> operand fragments ----------------------------------------------
@@ -688,89 +691,116 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 #define RDTR8(dst, addr, imm) \
     asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
 
-    // A tiles 4*S .. 4*S+3 of the slab in `stage` -> fa[S]
-#define READ_A(stage, S)                                              \
-    do                                                                \
-    {                                                                 \
-        const uint32_t q_ = lds0 + (stage) * STAGE_BYTES + a_lane;    \
-        RD128(fa[S][0], q_, (4 * (S) + 0) * 16 * BK);                 \
-        RD128(fa[S][1], q_, (4 * (S) + 1) * 16 * BK);                 \
-        RD128(fa[S][2], q_, (4 * (S) + 2) * 16 * BK);                 \
-        RD128(fa[S][3], q_, (4 * (S) + 3) * 16 * BK);                 \
+    // A tile 4*S + E of the slab in `stage` -> fa[S][E]
+#define READ_A1(stage, S, E) \
+    RD128(fa[S][E], lds0 + (stage) * STAGE_BYTES + a_lane, (4 * (S) + (E)) * 16 * BK)
+#define READ_A(stage, S)      \
+    do                        \
+    {                         \
+        READ_A1(stage, S, 0); \
+        READ_A1(stage, S, 1); \
+        READ_A1(stage, S, 2); \
+        READ_A1(stage, S, 3); \
     } while(0)
-    // the four B tiles of the slab in `stage` -> fb[P]
-#define READ_B(stage, P)                                                                   \
+    // B tile J of the slab in `stage` -> fb[P][J]
+#define READ_B1(stage, P, J)                                                               \
     do                                                                                     \
     {                                                                                      \
         const uint32_t s_ = lds0 + (stage) * STAGE_BYTES;                                  \
         if constexpr(TRANS_B)                                                              \
         {                                                                                  \
-            const uint32_t q_ = s_ + b_lane[0];                                            \
-            RD128(fb[P][0], q_, 0 * 16 * BK);                                              \
-            RD128(fb[P][1], q_, 1 * 16 * BK);                                              \
-            RD128(fb[P][2], q_, 2 * 16 * BK);                                              \
-            RD128(fb[P][3], q_, 3 * 16 * BK);                                              \
+            RD128(fb[P][J], s_ + b_lane[0], (J) * 16 * BK);                                \
         }                                                                                  \
         else                                                                               \
         {                                                                                  \
-            _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++)                                \
-            {                                                                              \
-                const uint32_t c_ = (uint32_t)(((wave_n * 4 + j_) ^ bsw) << 4);            \
-                v2i lo_, hi_;                                                              \
-                RDTR8(lo_, s_ + b_lane[0] + c_, 0);                                        \
-                RDTR8(hi_, s_ + b_lane[1] + c_, 0);                                        \
-                fb[P][j_] = v4i{lo_.x, lo_.y, hi_.x, hi_.y};                               \
-            }                                                                              \
+            const uint32_t c_ = (uint32_t)(((wave_n * 4 + (J)) ^ bsw) << 4);               \
+            v2i lo_, hi_;                                                                  \
+            RDTR8(lo_, s_ + b_lane[0] + c_, 0);                                            \
+            RDTR8(hi_, s_ + b_lane[1] + c_, 0);                                            \
+            fb[P][J] = v4i{lo_.x, lo_.y, hi_.x, hi_.y};                                    \
         }                                                                                  \
+    } while(0)
+#define READ_B(stage, P)      \
+    do                        \
+    {                         \
+        READ_B1(stage, P, 0); \
+        READ_B1(stage, P, 1); \
+        READ_B1(stage, P, 2); \
+        READ_B1(stage, P, 3); \
     } while(0)
 #define WAIT4(x) \
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3])::"memory")
-    // 16 MFMAs: A tiles 4*S.. against the four B tiles in fb[P]
-#define MFMA_STEP(S, P)                                                                     \
-    do                                                                                      \
-    {                                                                                       \
-        _Pragma("unroll") for(int i_ = 0; i_ < 4; i_++)                                     \
-        {                                                                                   \
-            if(!SPLITK || 4 * (S) + i_ < live_tiles)                                        \
-            {                                                                               \
-                _Pragma("unroll") for(int j_ = 0; j_ < 4; j_++) acc[4 * (S) + i_][j_] =     \
-                    __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[P][j_], fa[S][i_],            \
-                                                          acc[4 * (S) + i_][j_], 0, 0, 0);  \
-            }                                                                               \
-        }                                                                                   \
+    // one MFMA: A tile 4*S + I against B tile J in fb[P]
+#define MF(S, P, I, J)                                                                            \
+    do                                                                                            \
+    {                                                                                             \
+        if(!SPLITK || 4 * (S) + (I) < live_tiles)                                                 \
+            acc[4 * (S) + (I)][J] = __builtin_amdgcn_mfma_i32_16x16x64_i8(                        \
+                fb[P][J], fa[S][I], acc[4 * (S) + (I)][J], 0, 0, 0);                              \
     } while(0)
-    // one slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P]
-#define SLAB(kt, P)                                                     \
-    do                                                                  \
-    {                                                                   \
-        const int stage_ = (kt) & (STAGES - 1);                         \
-        if((kt) + STAGES - 1 < nk)                                      \
-            issue_slab((kt) + STAGES - 1);                              \
-        WAIT4(fa[0]);                                                   \
-        WAIT4(fb[P]);                                                   \
-        READ_A(stage_, 1);                                              \
-        MFMA_STEP(0, P);                                                \
-        if((kt) + 3 < nk)                                               \
-            wait_vmcnt<8>();                                            \
-        else if((kt) + 2 < nk)                                          \
-            wait_vmcnt<4>();                                            \
-        else                                                            \
-            wait_vmcnt<0>();                                            \
-        WAIT4(fa[1]);                                                   \
-        block_barrier();                                                \
-        if((kt) + 1 < nk)                                               \
-        {                                                               \
-            READ_A(((kt) + 1) & (STAGES - 1), 0);                       \
-            READ_B(((kt) + 1) & (STAGES - 1), 1 - (P));                 \
-        }                                                               \
-        MFMA_STEP(1, P);                                                \
+    // the instruction order below is the schedule: nothing moves across these
+#define SB() __builtin_amdgcn_sched_barrier(0)
+    // One slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P].  LDS reads and
+    // direct-to-LDS loads are dealt out between the MFMAs, one at a time: issued in a bunch (12 reads
+    // by each of 8 waves right behind the barrier, as an earlier version did) they fill the LDS and
+    // memory queues and every wave sits at its issue with MFMAs waiting behind it in program order --
+    // clock stamps showed more than half of a slab's time going that way.
+    // Loads in flight, in issue order, at the wait in front of the barrier: slab kt+1, kt+2, kt+3
+    // (its B blocks were issued in this first step, its A blocks in the previous slab's second step).
+#define SLAB(kt, P)                                                                   \
+    do                                                                                \
+    {                                                                                 \
+        const int stage_  = (kt) & (STAGES - 1);                                      \
+        const int nstage_ = ((kt) + 1) & (STAGES - 1);                                \
+        const bool more_  = (kt) + 1 < nk;                                            \
+        const bool ldb_   = (kt) + STAGES - 1 < nk;                                   \
+        const bool lda_   = (kt) + STAGES < nk;                                       \
+        WAIT4(fa[0]);                                                                 \
+        WAIT4(fb[P]);                                                                 \
+        SB();                                                                         \
+        READ_A1(stage_, 1, 0); SB(); MF(0, P, 0, 0); MF(0, P, 0, 1); SB();            \
+        READ_A1(stage_, 1, 1); SB(); MF(0, P, 0, 2); MF(0, P, 0, 3); SB();            \
+        READ_A1(stage_, 1, 2); SB(); MF(0, P, 1, 0); MF(0, P, 1, 1); SB();            \
+        READ_A1(stage_, 1, 3); SB(); MF(0, P, 1, 2); MF(0, P, 1, 3); SB();            \
+        if(ldb_) issue_b((kt) + STAGES - 1, 0);                                       \
+        SB(); MF(0, P, 2, 0); MF(0, P, 2, 1); MF(0, P, 2, 2); MF(0, P, 2, 3); SB();   \
+        if(ldb_) issue_b((kt) + STAGES - 1, 1);                                       \
+        SB(); MF(0, P, 3, 0); MF(0, P, 3, 1); MF(0, P, 3, 2); MF(0, P, 3, 3); SB();   \
+        if((kt) + 3 < nk)                                                             \
+            wait_vmcnt<8>();                                                          \
+        else if((kt) + 2 < nk)                                                        \
+            wait_vmcnt<4>();                                                          \
+        else                                                                          \
+            wait_vmcnt<0>();                                                          \
+        WAIT4(fa[1]);                                                                 \
+        block_barrier();                                                              \
+        SB();                                                                         \
+        if(more_) READ_A1(nstage_, 0, 0); SB(); MF(1, P, 0, 0); SB();                 \
+        if(more_) READ_A1(nstage_, 0, 1); SB(); MF(1, P, 0, 1); SB();                 \
+        if(more_) READ_A1(nstage_, 0, 2); SB(); MF(1, P, 0, 2); SB();                 \
+        if(more_) READ_A1(nstage_, 0, 3); SB(); MF(1, P, 0, 3); SB();                 \
+        if(more_) READ_B1(nstage_, 1 - (P), 0); SB(); MF(1, P, 1, 0); MF(1, P, 1, 1); SB(); \
+        if(more_) READ_B1(nstage_, 1 - (P), 1); SB(); MF(1, P, 1, 2); MF(1, P, 1, 3); SB(); \
+        if(more_) READ_B1(nstage_, 1 - (P), 2); SB(); MF(1, P, 2, 0); MF(1, P, 2, 1); SB(); \
+        if(more_) READ_B1(nstage_, 1 - (P), 3); SB(); MF(1, P, 2, 2); MF(1, P, 2, 3); SB(); \
+        if(lda_) issue_a((kt) + STAGES, 0);                                           \
+        SB(); MF(1, P, 3, 0); MF(1, P, 3, 1); SB();                                   \
+        if(lda_) issue_a((kt) + STAGES, 1);                                           \
+        SB(); MF(1, P, 3, 2); MF(1, P, 3, 3); SB();                                   \
     } while(0)
 
     // ---- main loop (see the kernel above for the ordering argument) ----------
+    // The stage of slab kt + 4 is the one slab kt sits in: its A blocks may be requested once every
+    // wave holds its last fragments of slab kt, i.e. after slab kt's barrier.
 #pragma unroll
     for(int s = 0; s < STAGES - 1; s++)
         if(s < nk)
-            issue_slab(s);
+        {
+            issue_a(s, 0);
+            issue_a(s, 1);
+            issue_b(s, 0);
+            issue_b(s, 1);
+        }
     if(nk >= 3)
         wait_vmcnt<8>();
     else if(nk == 2)
@@ -778,6 +808,11 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     else
         wait_vmcnt<0>();
     block_barrier();
+    if(STAGES - 1 < nk)
+    {
+        issue_a(STAGES - 1, 0);
+        issue_a(STAGES - 1, 1);
+    }
     READ_A(0, 0);
     READ_B(0, 0);
     int kt = 0;
@@ -789,10 +824,13 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     if(kt < nk)
         SLAB(kt, 0);
 #undef SLAB
-#undef MFMA_STEP
+#undef SB
+#undef MF
 #undef WAIT4
 #undef READ_B
+#undef READ_B1
 #undef READ_A
+#undef READ_A1
 #undef RDTR8
 #undef RD128
 
