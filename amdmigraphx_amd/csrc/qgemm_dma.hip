@@ -188,16 +188,23 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
             b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
         }
     }
-    auto issue_slab = [&](int kt) {
+    // one load at a time, so that the main loop can deal them out between runs of MFMAs (a load
+    // occupies the CU's memory pipeline for about 47 cycles; 32 issued together stall every wave)
+    auto issue_a = [&](int kt, int h) {
         uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
         const uint8_t* a_base = ga + (int64_t)kt * BK;
+        load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
+    };
+    auto issue_b = [&](int kt, int h) {
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
         const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
-#pragma unroll
-        for(int h = 0; h < 2; h++)
-            load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
-#pragma unroll
-        for(int h = 0; h < 2; h++)
-            load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+        load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+    };
+    auto issue_slab = [&](int kt) {
+        issue_a(kt, 0);
+        issue_a(kt, 1);
+        issue_b(kt, 0);
+        issue_b(kt, 1);
     };
 
     // ---- LDS -> operand fragments --------------------------------------------
@@ -376,10 +383,12 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
             for(int e = 0; e < 16; e++)
                 acc[i][j][e] = 0;
 
-    auto mfma_step = [&](auto step) {
+    // half H (0, 1) of the MFMAs of step S
+    auto mfma_half = [&](auto step, auto half) {
         constexpr int S = decltype(step)::value;
+        constexpr int H = decltype(half)::value;
 #pragma unroll
-        for(int i = 0; i < A_TILES; i++)
+        for(int i = H * (A_TILES / 2); i < (H + 1) * (A_TILES / 2); i++)
 #pragma unroll
             for(int j = 0; j < 2; j++)
             {
@@ -391,15 +400,16 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     };
 
     // ---- main loop ---------------------------------------------------------------
-    // Per slab: issue the loads of slab kt+3, multiply step 0 while the step-1
-    // fragments are read, barrier, multiply step 1 while the first fragments of
-    // slab kt+1 are read.  The barrier sits between the two steps so that the
-    // LDS latency of the next slab's first reads is covered by MFMAs.
+    // Per slab: multiply step 0 while the step-1 fragments are read, barrier, multiply step 1 while
+    // the first fragments of slab kt+1 are read.  The barrier sits between the two steps so that the
+    // LDS latency of the next slab's first reads is covered by MFMAs.  The wave's four loads go out
+    // singly behind the four halves of the MFMA work: the B blocks of slab kt+3 in step 0, the A
+    // blocks of slab kt+4 in step 1.
     //
-    // Slab kt+1 must be complete and visible to every wave, and every wave must
-    // have its last fragments of slab kt in registers, before that barrier: the
-    // loads issued at the top of the next iteration (slab kt+4) overwrite the
-    // stage slab kt sits in.
+    // Slab kt+1 must be complete and visible to every wave, and every wave must have its last
+    // fragments of slab kt in registers, before that barrier: the loads issued behind it (A blocks
+    // of slab kt+4) overwrite the stage slab kt sits in.  At the wait in front of the barrier the
+    // loads in flight are, in issue order, those of slabs kt+1, kt+2, kt+3.
     const int nk = p.k / BK;
 #pragma unroll
     for(int s = 0; s < STAGES - 1; s++)
@@ -413,18 +423,28 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     else
         wait_vmcnt<0>();
     block_barrier();
+    if(STAGES - 1 < nk)
+    {
+        issue_a(STAGES - 1, 0);
+        issue_a(STAGES - 1, 1);
+    }
     read_step(0, IMM(0));
 
     for(int kt = 0; kt < nk; kt++)
     {
         const int stage = kt & (STAGES - 1);
-        if(kt + STAGES - 1 < nk)
-            issue_slab(kt + STAGES - 1);
+        const bool ldb  = kt + STAGES - 1 < nk;
+        const bool lda  = kt + STAGES < nk;
         // lgkmcnt counts every outstanding LDS read, so the wait for step 0
         // comes before the step-1 reads are issued, not after
         WAIT_STEP(0);
         read_step(stage, IMM(1));
-        mfma_step(IMM(0));
+        mfma_half(IMM(0), IMM(0));
+        if(ldb)
+            issue_b(kt + STAGES - 1, 0);
+        mfma_half(IMM(0), IMM(1));
+        if(ldb)
+            issue_b(kt + STAGES - 1, 1);
         if(kt + 3 < nk)
             wait_vmcnt<8>();
         else if(kt + 2 < nk)
@@ -435,7 +455,12 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
         block_barrier();
         if(kt + 1 < nk)
             read_step((kt + 1) & (STAGES - 1), IMM(0));
-        mfma_step(IMM(1));
+        mfma_half(IMM(1), IMM(0));
+        if(lda)
+            issue_a(kt + STAGES, 0);
+        mfma_half(IMM(1), IMM(1));
+        if(lda)
+            issue_a(kt + STAGES, 1);
     }
 #undef IMM
 #undef WAIT_STEP
