@@ -469,23 +469,52 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     // The operands went in swapped, so element e of lane l belongs to row l % 32 of the A tile
     // and column 8*(e/4) + 4*(l/32) + e%4 of the B tile: four groups of 4 consecutive columns,
     // each written with one store when C allows it (p.vec_store).
+    // Every scale, column sum and row sum this lane needs is loaded before the first store: a
+    // load placed behind a store to C cannot be moved in front of it (C may alias), and 32 groups
+    // of "load, wait out the latency, compute, store" in a row cost more than the main loop of a
+    // short K.
+    float sa_r[4]     = {1.f, 1.f, 1.f, 1.f};
+    int64_t zrow_r[4] = {0, 0, 0, 0};
+    float sb_c[2][4][4];
+    int32_t cs_c[2][4][4];
+    if constexpr(DEQ)
+    {
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            const int row = min(m0 + wave_m * 128 + i * 32 + lrow, p.m - 1);
+            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                sa_r[i] = p.scale_a[0];
+            else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                sa_r[i] = p.scale_a[row];
+            if(!FP8 && p.zp_b != 0)
+                zrow_r[i] = (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b;
+        }
+#pragma unroll
+        for(int j = 0; j < 2; j++)
+#pragma unroll
+            for(int g = 0; g < 4; g++)
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    const int c = min(n0 + wave_n * 64 + j * 32 + 8 * g + 4 * lgrp + e, p.n - 1);
+                    float sb    = 1.f;
+                    if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                        sb = p.scale_b[0];
+                    else if(p.scale_b_mode == MI355_QP_PER_COL)
+                        sb = p.scale_b[c];
+                    sb_c[j][g][e] = sb;
+                    cs_c[j][g][e] = (!FP8 && p.zp_a != 0) ? p.colsum_b[c] : 0;
+                }
+    }
 #pragma unroll
     for(int i = 0; i < 4; i++)
     {
         const int row = m0 + wave_m * 128 + i * 32 + lrow;
         if(row >= p.m)
             continue;
-        float sa     = 1.f;
-        int64_t zrow = 0;
-        if constexpr(DEQ)
-        {
-            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
-                sa = p.scale_a[0];
-            else if(p.scale_a_mode == MI355_QP_PER_ROW)
-                sa = p.scale_a[row];
-            if(!FP8 && p.zp_b != 0)
-                zrow = (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b;
-        }
+        const float sa     = sa_r[i];
+        const int64_t zrow = zrow_r[i];
 #pragma unroll
         for(int j = 0; j < 2; j++)
         {
@@ -503,16 +532,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #pragma unroll
                     for(int e = 0; e < 4; e++)
                     {
-                        const int c = min(col + e, p.n - 1);
-                        float sb    = 1.f;
-                        if(p.scale_b_mode == MI355_QP_PER_TENSOR)
-                            sb = p.scale_b[0];
-                        else if(p.scale_b_mode == MI355_QP_PER_COL)
-                            sb = p.scale_b[c];
                         // scale = fp32 product of the two scales (the graph's `mul`), then
                         // (double(acc) - double(zp)) * scale in double, one rounding to float
                         // (dequantizelinear)
-                        const float s = sa * sb;
+                        const float s = sa * sb_c[j][g][e];
                         if constexpr(FP8)
                         {
                             // the accumulator is a float: double(acc) * double(s) rounded once
@@ -521,11 +544,9 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                         }
                         else
                         {
-                            int64_t zp = zrow;
-                            if(p.zp_a != 0)
-                                zp += (int64_t)p.zp_a * p.colsum_b[c];
-                            const double d = (double)acc[i][j][4 * g + e] - (double)(int32_t)zp;
-                            v[e]           = (float)(d * (double)s);
+                            const int64_t zp = zrow + (int64_t)p.zp_a * cs_c[j][g][e];
+                            const double d   = (double)acc[i][j][4 * g + e] - (double)(int32_t)zp;
+                            v[e]             = (float)(d * (double)s);
                         }
                     }
                 }
@@ -862,27 +883,47 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     // ---- epilogue ----------------------------------------------------------------
     // acc[i][j][e]: row 16*i + (l % 16) of the wave's A block, column
     // 16*j + 4*(l / 16) + e of its B block.
+    // Scales, column sums and row sums are all loaded before the first store (a load behind a
+    // store to C cannot move in front of it, and its latency would be paid once per group).
+    float sb_c[4][4];
+    int32_t cs_c[4][4];
+    float sa_r[8];
+    int64_t zrow_r[8];
+    if constexpr(DEQ)
+    {
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                const int c = min(n0 + wave_n * 64 + j * 16 + 4 * lgrp + e, p.n - 1);
+                float sb    = 1.f;
+                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                    sb = p.scale_b[0];
+                else if(p.scale_b_mode == MI355_QP_PER_COL)
+                    sb = p.scale_b[c];
+                sb_c[j][e] = sb;
+                cs_c[j][e] = p.zp_a != 0 ? p.colsum_b[c] : 0;
+            }
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+        {
+            const int row = min(m0 + wave_m * 128 + i * 16 + lrow, p.m - 1);
+            float sa      = 1.f;
+            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                sa = p.scale_a[0];
+            else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                sa = p.scale_a[row];
+            sa_r[i]   = sa;
+            zrow_r[i] = p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
+        }
+    }
 #pragma unroll
     for(int j = 0; j < 4; j++)
     {
         const int col = n0 + wave_n * 64 + j * 16 + 4 * lgrp;
         if(col >= p.n)
             continue; // N is a multiple of 4 on this path, so the 4 columns are in or out together
-        float sb[4]   = {1.f, 1.f, 1.f, 1.f};
-        int32_t cs[4] = {0, 0, 0, 0};
-        if constexpr(DEQ)
-        {
-#pragma unroll
-            for(int e = 0; e < 4; e++)
-            {
-                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
-                    sb[e] = p.scale_b[0];
-                else if(p.scale_b_mode == MI355_QP_PER_COL)
-                    sb[e] = p.scale_b[col + e];
-                if(p.zp_a != 0)
-                    cs[e] = p.colsum_b[col + e];
-            }
-        }
 #pragma unroll
         for(int i = 0; i < 8; i++)
         {
@@ -911,14 +952,6 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             }
             else
             {
-                float sa = 1.f;
-                if(p.scale_a_mode == MI355_QP_PER_TENSOR)
-                    sa = p.scale_a[0];
-                else if(p.scale_a_mode == MI355_QP_PER_ROW)
-                    sa = p.scale_a[row];
-                int64_t zrow = 0;
-                if(p.zp_b != 0)
-                    zrow = (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b;
                 float v[4];
 #pragma unroll
                 for(int e = 0; e < 4; e++)
@@ -926,9 +959,9 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                     // scale = fp32 product of the two scales (the graph's `mul`),
                     // then (double(acc) - double(zp)) * scale in double, one
                     // rounding to float (dequantizelinear)
-                    const float s  = sa * sb[e];
+                    const float s  = sa_r[i] * sb_c[j][e];
                     const double d = (double)acc[i][j][e] -
-                                     (double)(int32_t)(zrow + (int64_t)p.zp_a * cs[e]);
+                                     (double)(int32_t)(zrow_r[i] + (int64_t)p.zp_a * cs_c[j][e]);
                     v[e] = (float)(d * (double)s);
                 }
                 if constexpr(VEC_STORE)
