@@ -58,6 +58,7 @@ struct dma_params
     int zp_a, zp_b;
     int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
+    int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
 };
 
 // s_waitcnt with only the vector-memory counter constrained
@@ -518,6 +519,55 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #pragma unroll
         for(int j = 0; j < 2; j++)
         {
+            // 16-bit outputs: lanes l and l + 32 hold the two halves of the same 8 columns, for two
+            // column groups; one v_permlane32_swap per register gives each of them one whole group,
+            // which goes out as a single 16-byte store (half as many store instructions).  N % 8 == 0
+            // there, so the two lanes are in or out of the matrix together.
+            if constexpr(DEQ && (OUT == MI355_F16 || OUT == MI355_BF16))
+            {
+                if(p.vec8_store)
+                {
+#pragma unroll
+                    for(int gp = 0; gp < 4; gp += 2)
+                    {
+                        uint32_t pk[2][2];
+#pragma unroll
+                        for(int h = 0; h < 2; h++)
+                        {
+                            uint16_t q[4];
+#pragma unroll
+                            for(int e = 0; e < 4; e++)
+                            {
+                                const float s = sa * sb_c[j][gp + h][e];
+                                float v;
+                                if constexpr(FP8)
+                                    v = acc[i][j][4 * (gp + h) + e] * s;
+                                else
+                                {
+                                    const int64_t zp = zrow + (int64_t)p.zp_a * cs_c[j][gp + h][e];
+                                    const double d =
+                                        (double)acc[i][j][4 * (gp + h) + e] - (double)(int32_t)zp;
+                                    v = (float)(d * (double)s);
+                                }
+                                q[e] = OUT == MI355_F16 ? convert_f32_to_half(v) : convert_f32_to_bf16(v);
+                            }
+                            pk[h][0] = q[0] | ((uint32_t)q[1] << 16);
+                            pk[h][1] = q[2] | ((uint32_t)q[3] << 16);
+                        }
+                        const auto r0 = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
+                        const auto r1 = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
+                        const int col = n0 + wave_n * 64 + j * 32 + 8 * (gp + lgrp);
+                        if(col < p.n)
+                        {
+                            const int64_t idx =
+                                (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                            *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.c) + idx) =
+                                make_uint4(r0[0], r1[0], r0[1], r1[1]);
+                        }
+                    }
+                    continue;
+                }
+            }
 #pragma unroll
             for(int g = 0; g < 4; g++)
             {
@@ -1155,6 +1205,8 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
         const size_t esz = deq ? mi355_dtype_size(d->out_type) : 4;
         p.vec_store = d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
                       reinterpret_cast<uintptr_t>(c) % (4 * esz) == 0;
+        p.vec8_store = esz == 2 && d->n % 8 == 0 && d->ldc % 8 == 0 && d->stride_c % 8 == 0 &&
+                       reinterpret_cast<uintptr_t>(c) % 16 == 0;
     }
     p.ksplit = 1;
     if(fp8)

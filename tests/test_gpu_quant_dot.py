@@ -248,6 +248,37 @@ def test_fp8_dequant_epilogue(ops, out):
     assert ok.all(), (~ok).sum()
 
 
+@pytest.mark.parametrize("m,n", [(200, 264), (77, 512), (256, 260), (130, 1000)])
+@pytest.mark.parametrize("out", ["f16", "bf16"])
+def test_fp8_16bit_outputs_ragged_shapes(ops, m, n, out):
+    """16-bit outputs leave the kernel as 16-byte stores built from two lanes' halves when
+    N % 8 == 0 (first, second and fourth shape) and as 8-byte or single stores otherwise; rows
+    past M and column groups past N are dropped in pairs.  Per-column scales, so a swapped
+    half would show."""
+    rng = np.random.default_rng(m + n)
+    k = 320
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    xq = orc.quantizelinear(x, np.float32(np.abs(x).max() / 448), None, orc.F32, orc.FP8)
+    wq = orc.quantizelinear(w, np.float32(np.abs(w).max() / 448), None, orc.F32, orc.FP8)
+    sx = np.float32(0.03)
+    sw = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    ot = orc.F16 if out == "f16" else orc.BF16
+    want = orc.qdq_matmul_fp8(xq, wq, sx, sw, ot)
+    td = torch.float16 if out == "f16" else torch.bfloat16
+    print("fp8 16-bit out", m, n, out, flush=True)
+    got = ops.quant_dot(dev(xq), dev(wq), fp8=True, scale_a=dev(np.float32([sx])), scale_b=dev(sw),
+                        out_dtype=td)
+    gb = got.view(torch.int16).cpu().numpy().view(np.uint16)
+    to_f32 = orc.half_to_f32 if out == "f16" else orc.bf16_to_f32
+    bound = _fp8_bound(xq, wq) * float(sx) * sw[None, :]
+    ok = (ulp_distance_16(gb, want) <= 1) | _fp8_close(to_f32(gb), to_f32(want), bound)
+    assert ok.all(), (~ok).sum()
+    # most outputs are bit-identical (half keeps three more bits of the fp32 sum than bf16, so fewer
+    # of them); a misplaced half would be off by the ratio of two column scales
+    assert (gb == want).mean() > (0.97 if out == "bf16" else 0.8)
+
+
 def test_argument_errors(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((4, 8), dtype=torch.int8, device="cuda")
