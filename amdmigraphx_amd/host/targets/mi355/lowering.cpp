@@ -395,8 +395,31 @@ void lower_instruction(module& m, instruction_ref ins)
     auto standard_out = [&] { return out(shape{ins->get_shape().type(), ins->get_shape().lens()}); };
     if(name == "quant_dot")
     {
-        if(ins->inputs().size() != 2)
-            MIGRAPHX_THROW("mi355: quant_dot with block scales has no kernel");
+        if(ins->inputs().size() == 4)
+        {
+            // The four-input form (operands with element-wise scales, as the MX block formats
+            // arrive after their scales are broadcast): float(a) * float(scale_a), the same for b,
+            // then the float GEMM -- the three steps of ref_quant_gemm::compute
+            // (src/targets/ref/lowering.cpp:221-242), each on its device kernel.
+            auto as_float = [&](instruction_ref x) {
+                if(x->get_shape().type() == shape::float_type)
+                    return x;
+                convert cv;
+                cv.target_type = shape::float_type;
+                auto xs        = make_standard(m, ins, x);
+                return m.insert_instruction(ins, operation{cv}, xs, out(shape{shape::float_type, x->get_shape().lens()}));
+            };
+            auto scaled = [&](instruction_ref x, instruction_ref sc) {
+                binary mul;
+                mul.op = MI355_BIN_MUL;
+                return m.insert_instruction(ins, operation{mul}, as_float(x), as_float(sc),
+                                            out(shape{shape::float_type, x->get_shape().lens()}));
+            };
+            auto a = scaled(ins->inputs()[0], ins->inputs()[2]);
+            auto b = scaled(ins->inputs()[1], ins->inputs()[3]);
+            m.replace_instruction(ins, operation{dot{}}, a, b, standard_out());
+            return;
+        }
         auto a = ins->inputs()[0];
         auto b = ins->inputs()[1];
         if(not view_as_matrix(a->get_shape()).ok)

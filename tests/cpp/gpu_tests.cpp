@@ -200,6 +200,74 @@ TEST_CASE(bare_quant_dot_views)
     }
 }
 
+TEST_CASE(quant_dot_four_inputs)
+{
+    // the reference's known answer (test/ref/dot_op.cpp:1836-1865) on the device
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        shape sa{shape::float_type, {2, 3}};
+        shape sb{shape::float_type, {3, 2}};
+        auto a  = mm->add_parameter("a", sa);
+        auto b  = mm->add_parameter("b", sb);
+        auto s1 = mm->add_literal(literal{sa, std::vector<float>{0.5f, 1, 0.5f, 1, 0.5f, 1}});
+        auto s2 = mm->add_literal(literal{sb, std::vector<float>{1, 0.5f, 1, 0.5f, 1, 0.5f}});
+        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b, s1, s2)});
+        argument aa{sa, std::vector<float>{1, 2, 3, 4, 5, 6}};
+        argument ba{sb, std::vector<float>{1, 2, 3, 4, 5, 6}};
+        auto got = run_on("mi355", p, {{"a", aa}, {"b", ba}});
+        EXPECT(got[0].to_vector<float>() == std::vector<float>{14.0f, 9.0f, 41.5f, 27.0f});
+        expect_same(p, {{"a", aa}, {"b", ba}});
+    }
+    // fp8 operands with one power-of-two scale per block of 32 along K (the MX arrangement, scales
+    // already spread over the elements), batched; A's scales arrive as a dense tensor, B's as a
+    // broadcast view of one row
+    {
+        const std::size_t bt = 2, m = 48, k = 64, n = 40;
+        program p;
+        auto* mm = p.get_main_module();
+        shape sa{shape::fp8e4m3fn_type, {bt, m, k}};
+        shape sb{shape::fp8e4m3fn_type, {bt, k, n}};
+        shape ssa{shape::float_type, {bt, m, k}};
+        shape ssb{shape::float_type, {n}};
+        auto a   = mm->add_parameter("a", sa);
+        auto b   = mm->add_parameter("b", sb);
+        auto s1  = mm->add_parameter("sa", ssa);
+        auto s2  = mm->add_parameter("sb", ssb);
+        auto s2b = mm->add_instruction(make_op("broadcast", {{"axis", 2}, {"out_lens", {bt, k, n}}}), s2);
+        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b, s1, s2b)});
+        auto codes = [](std::size_t cnt, unsigned seed) {
+            auto v = uniform_ints<int>(cnt, 0, 0x7d, seed);
+            auto sg = uniform_ints<int>(cnt, 0, 1, seed + 1);
+            std::vector<uint8_t> out(cnt);
+            for(std::size_t i = 0; i < cnt; i++)
+                out[i] = static_cast<uint8_t>(v[i] | (sg[i] << 7));
+            return out;
+        };
+        std::vector<float> sav(ssa.elements());
+        auto e1 = uniform_ints<int>(bt * m * (k / 32), -6, 3, 77);
+        for(std::size_t i = 0; i < sav.size(); i++)
+            sav[i] = std::ldexp(1.0f, e1[i / 32]);
+        std::vector<float> sbv(n);
+        auto e2 = uniform_ints<int>(n, -5, 2, 78);
+        for(std::size_t i = 0; i < n; i++)
+            sbv[i] = std::ldexp(1.0f, e2[i]);
+        argument aa{sa};
+        argument ba{sb};
+        const auto ca = codes(sa.elements(), 70);
+        const auto cb = codes(sb.elements(), 72);
+        std::memcpy(aa.data(), ca.data(), ca.size());
+        std::memcpy(ba.data(), cb.data(), cb.size());
+        expect_same(p, {{"a", aa}, {"b", ba}, {"sa", argument{ssa, sav}}, {"sb", argument{ssb, sbv}}});
+        program c = p;
+        c.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*c.get_main_module(), "mi355::dot") == 1);
+        EXPECT(count_ops(*c.get_main_module(), "mi355::convert") == 2);
+        EXPECT(count_ops(*c.get_main_module(), "mi355::binary") == 2);
+        EXPECT(not has_op(c, "quant_dot"));
+    }
+}
+
 TEST_CASE(fp8_quantized_matmul)
 {
     // BASELINE config 3 in small: activations and weights quantized to fp8 e4m3fn with amax-based

@@ -153,6 +153,24 @@ TEST_CASE(quant_dot_shapes)
     EXPECT(test::throws([&] { qd.compute_shape({a, b, sa, shape{shape::half_type, {8, 6}}}); }));
 }
 
+TEST_CASE(quant_dot_four_inputs_known_answer)
+{
+    // test/ref/dot_op.cpp:1836-1865 (quant_dot_4args_scales): element-wise scales, float GEMM
+    program p;
+    auto* mm = p.get_main_module();
+    shape sa{shape::float_type, {2, 3}};
+    shape sb{shape::float_type, {3, 2}};
+    auto a  = mm->add_literal(literal{sa, std::vector<float>{1, 2, 3, 4, 5, 6}});
+    auto b  = mm->add_literal(literal{sb, std::vector<float>{1, 2, 3, 4, 5, 6}});
+    auto s1 = mm->add_literal(literal{sa, std::vector<float>{0.5f, 1, 0.5f, 1, 0.5f, 1}});
+    auto s2 = mm->add_literal(literal{sb, std::vector<float>{1, 0.5f, 1, 0.5f, 1, 0.5f}});
+    mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b, s1, s2)});
+    auto r = testutil::run_on("oracle", p, {});
+    EXPECT(r.size() == 1);
+    EXPECT(r[0].get_shape() == shape{shape::float_type, {2, 2}});
+    EXPECT(r[0].to_vector<float>() == std::vector<float>{14.0f, 9.0f, 41.5f, 27.0f});
+}
+
 TEST_CASE(qdq_and_int4_shapes)
 {
     shape x{shape::float_type, {3, 4}};

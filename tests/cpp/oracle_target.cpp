@@ -100,6 +100,29 @@ struct cpu_op
             // they are, so that transposed views reach the GEMM untouched
             argument a = args[0];
             argument b = args[1];
+            if(args.size() == 4)
+            {
+                // four-input quant_dot (ref/lowering.cpp:221-242): float(x) * float(scale), element
+                // by element, then the float GEMM
+                auto scaled = [&](const argument& x, const argument& sc) {
+                    const argument xd = dense(x);
+                    const argument sd = dense(sc);
+                    const shape fs{shape::float_type, xd.get_shape().lens()};
+                    argument xf{fs};
+                    argument sf{fs};
+                    argument prod{fs};
+                    orc_convert(xf.data(), orc_type(shape::float_type), xd.data(),
+                                orc_type(xd.get_shape().type()), fs.elements());
+                    orc_convert(sf.data(), orc_type(shape::float_type), sd.data(),
+                                orc_type(sd.get_shape().type()), fs.elements());
+                    orc_binary_f32(2, reinterpret_cast<float*>(prod.data()),
+                                   reinterpret_cast<const float*>(xf.data()),
+                                   reinterpret_cast<const float*>(sf.data()), fs.elements());
+                    return prod;
+                };
+                a = scaled(args[0], args[2]);
+                b = scaled(args[1], args[3]);
+            }
             if(a.get_shape().ndim() > 2)
             {
                 a = dense(a);
