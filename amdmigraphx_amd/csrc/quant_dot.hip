@@ -40,6 +40,7 @@ struct generic_params
     const int32_t* rowsum_a;
     int scale_a_mode, scale_b_mode, zp_a, zp_b;
     int fp8, dequant, out_type;
+    int is_unsigned; // uint8 operands (bare quant_dot only)
 };
 
 // 16 x 16 outputs per workgroup, K walked in steps of 16 through LDS.  int8
@@ -65,12 +66,12 @@ __global__ __launch_bounds__(256) void quant_dot_generic_kernel(generic_params p
         if(row < p.m && k0 + tx < p.k)
         {
             uint8_t raw = a[row * p.a_sm + (k0 + tx) * p.a_sk];
-            av          = p.fp8 ? fp8_to_f32(raw) : (float)(int8_t)raw;
+            av          = p.fp8 ? fp8_to_f32(raw) : (p.is_unsigned ? (float)raw : (float)(int8_t)raw);
         }
         if(col < p.n && k0 + ty < p.k)
         {
             uint8_t raw = b[(k0 + ty) * p.b_sk + col * p.b_sn];
-            bv          = p.fp8 ? fp8_to_f32(raw) : (float)(int8_t)raw;
+            bv          = p.fp8 ? fp8_to_f32(raw) : (p.is_unsigned ? (float)raw : (float)(int8_t)raw);
         }
         as[ty][tx] = av;
         bs[ty][tx] = bv;
@@ -201,9 +202,13 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
     const bool empty = d->m == 0 || d->n == 0 || d->batch == 0;
     if(!empty && (a == nullptr || b == nullptr || c == nullptr))
         return MI355_ERR_BAD_ARG;
-    if(d->in_type != MI355_I8 && d->in_type != MI355_FP8)
+    if(d->in_type != MI355_I8 && d->in_type != MI355_FP8 && d->in_type != MI355_U8)
         return MI355_ERR_UNSUPPORTED;
     const bool fp8 = d->in_type == MI355_FP8;
+    // uint8 x uint8 -> int32 (op/quant_dot.hpp:62-64 lists it): bare result only, correctness path
+    const bool u8 = d->in_type == MI355_U8;
+    if(u8 && d->dequant)
+        return MI355_ERR_UNSUPPORTED;
     if(d->dequant)
     {
         if(d->out_type != MI355_F32 && d->out_type != MI355_F16 && d->out_type != MI355_BF16)
@@ -244,9 +249,9 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
         return MI355_ERR_UNSUPPORTED;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if(d->k > 0 && mi355_dma_gemm_supported(d, a, b))
+    if(!u8 && d->k > 0 && mi355_dma_gemm_supported(d, a, b))
         return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
-    if(d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
+    if(!u8 && d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
         return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
 
     generic_params p;
@@ -273,6 +278,7 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
     p.zp_a         = d->zp_a;
     p.zp_b         = d->zp_b;
     p.fp8          = fp8;
+    p.is_unsigned  = u8;
     p.dequant      = d->dequant;
     p.out_type     = d->out_type;
     const int64_t gx = (d->n + 15) / 16, gy = (d->m + 15) / 16;

@@ -50,7 +50,8 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     """quant_dot, optionally with the fused dequantizelinear epilogue.
 
     a [..., M, K], b [..., K, N] int8 (or uint8 carrying fp8 e4m3fn bits with
-    fp8=True); transposed views are passed as they are.  Without scales the
+    fp8=True; plain uint8 operands give the bare int32 result only); transposed
+    views are passed as they are.  Without scales the
     bare accumulators come back (int32 / float32).  With ``scale_a`` (scalar
     or [M]) / ``scale_b`` (scalar or [N]) float32 tensors the epilogue
     (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied."""
@@ -78,7 +79,7 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     ta, lda = _mat_layout(a3)
     tb, ldb = _mat_layout(b3)
     dequant = scale_a is not None or scale_b is not None or out_dtype is not None
-    in_type = DT.FP8 if fp8 else DT.I8
+    in_type = DT.FP8 if fp8 else (DT.U8 if a.dtype == torch.uint8 else DT.I8)
     if dequant:
         odt = out_dtype or torch.float32
     else:

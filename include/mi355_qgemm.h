@@ -70,7 +70,7 @@ typedef struct mi355_quant_dot_desc {
     int64_t batch;
     int64_t stride_a, stride_b, stride_c;
     int32_t trans_a, trans_b;
-    int32_t in_type;  /* MI355_I8 or MI355_FP8 */
+    int32_t in_type;  /* MI355_I8 or MI355_FP8; MI355_U8 for the bare result only */
     int32_t out_type; /* MI355_I32 / MI355_F32: bare quant_dot result (int8 / fp8).
                          With an epilogue: MI355_F32, MI355_F16 or MI355_BF16. */
     /* ---- fused dequantizelinear epilogue (all zero = bare quant_dot) ---- */

@@ -198,6 +198,20 @@ TEST_CASE(bare_quant_dot_views)
         argument ba{sb, uniform_ints<int>(sb.elements(), -128, 127, 20 + variant)};
         expect_same(p, {{"a", aa}, {"b", ba}});
     }
+    // uint8 operands (op/quant_dot.hpp:62-64)
+    {
+        const std::size_t m = 33, k = 70, n = 21;
+        program p;
+        auto* mm = p.get_main_module();
+        shape sa{shape::uint8_type, {m, k}};
+        shape sb{shape::uint8_type, {k, n}};
+        auto a = mm->add_parameter("a", sa);
+        auto b = mm->add_parameter("b", sb);
+        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b)});
+        argument aa{sa, uniform_ints<int>(sa.elements(), 0, 255, 30)};
+        argument ba{sb, uniform_ints<int>(sb.elements(), 0, 255, 31)};
+        expect_same(p, {{"a", aa}, {"b", ba}});
+    }
 }
 
 TEST_CASE(quant_dot_four_inputs)

@@ -279,6 +279,24 @@ def test_fp8_16bit_outputs_ragged_shapes(ops, m, n, out):
     assert (gb == want).mean() > (0.97 if out == "bf16" else 0.8)
 
 
+@pytest.mark.parametrize("m,n,k", [(5, 7, 3), (64, 48, 300), (130, 257, 96)])
+def test_uint8_quant_dot_bare(ops, m, n, k):
+    """uint8 x uint8 -> int32 (op/quant_dot.hpp:62-64): exact, also for a transposed B view and
+    in batches; with an epilogue the library refuses instead of guessing."""
+    from amdmigraphx_amd import Mi355Error
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(0, 256, (2, k, n), dtype=np.uint8)
+    want = np.matmul(a.astype(np.int64), b.astype(np.int64))
+    assert np.array_equal(orc.quant_dot(a[0], b[0], orc.U8), want[0])
+    got = ops.quant_dot(dev(a), dev(b))
+    assert got.dtype == torch.int32 and np.array_equal(got.cpu().numpy(), want)
+    bt = dev(np.ascontiguousarray(b[0].T)).t()
+    assert np.array_equal(ops.quant_dot(dev(a[0]), bt).cpu().numpy(), want[0])
+    with pytest.raises(Mi355Error):
+        ops.quant_dot(dev(a[0]), dev(b[0]), scale_a=dev(np.float32([0.1])), scale_b=dev(np.float32([0.2])))
+
+
 def test_argument_errors(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((4, 8), dtype=torch.int8, device="cuda")
