@@ -156,6 +156,61 @@ __global__ __launch_bounds__(PW_THREADS) void unpack_int4_kernel(
     }
 }
 
+// fp4 (e2m1): sign, two exponent bits, one mantissa bit; magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6.
+// Their fp8 e4m3fn codes (exponent bias 7, three mantissa bits), indexed by the low three bits:
+__constant__ const uint8_t fp4_as_fp8[8] = {0x00, 0x30, 0x38, 0x3c, 0x40, 0x44, 0x48, 0x4c};
+
+// one packed byte -> two fp8 bytes, low nibble first; 8 packed bytes per thread
+__global__ __launch_bounds__(PW_THREADS) void unpack_fp4_kernel(const uint8_t* in, uint8_t* out, int64_t total)
+{
+    const int64_t i0 = ((int64_t)blockIdx.x * PW_THREADS + threadIdx.x) * 8;
+    if(i0 >= total)
+        return;
+    const int cnt = (int)min((int64_t)8, total - i0);
+    for(int e = 0; e < cnt; e++)
+    {
+        const uint8_t v       = in[i0 + e];
+        out[2 * (i0 + e)]     = fp4_as_fp8[v & 7] | ((v & 0x08) << 4);
+        out[2 * (i0 + e) + 1] = fp4_as_fp8[(v >> 4) & 7] | (v & 0x80);
+    }
+}
+
+// float -> fp4 code: nearest magnitude, a tie to the neighbour with the even code, beyond 5 -> 6
+// (infinity included), NaN -> 0, sign kept (also for zero)
+MI355_DEVINL uint8_t f32_to_fp4(float x)
+{
+    if(x != x)
+        return 0;
+    const uint8_t sign = (__builtin_bit_cast(uint32_t, x) >> 31) ? 8 : 0;
+    const float a      = __builtin_fabsf(x);
+    uint8_t i;
+    if(a <= 0.25f)
+        i = 0;
+    else if(a < 0.75f)
+        i = 1;
+    else if(a <= 1.25f)
+        i = 2;
+    else if(a < 1.75f)
+        i = 3;
+    else if(a <= 2.5f)
+        i = 4;
+    else if(a < 3.5f)
+        i = 5;
+    else if(a <= 5.0f)
+        i = 6;
+    else
+        i = 7;
+    return i | sign;
+}
+
+__global__ __launch_bounds__(PW_THREADS) void pack_fp4_kernel(const float* in, uint8_t* out, int64_t total_out)
+{
+    const int64_t i = (int64_t)blockIdx.x * PW_THREADS + threadIdx.x;
+    if(i >= total_out)
+        return;
+    out[i] = (uint8_t)((f32_to_fp4(in[2 * i + 1]) << 4) | f32_to_fp4(in[2 * i]));
+}
+
 __global__ __launch_bounds__(PW_THREADS) void pack_int4_kernel(
     const uint8_t* in, uint8_t* out, int is_signed, int64_t total_out)
 {
@@ -325,6 +380,33 @@ extern "C" int mi355_pack_int4(
     hipLaunchKernelGGL(pack_int4_kernel, dim3(blocks_for(total_out)), dim3(PW_THREADS), 0,
                        static_cast<hipStream_t>(stream), static_cast<const uint8_t*>(in),
                        static_cast<uint8_t*>(out), is_signed, total_out);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_unpack_fp4(const void* in, void* out, int64_t rows, int64_t cols, void* stream)
+{
+    if(in == nullptr || out == nullptr || rows < 0 || cols < 0)
+        return MI355_ERR_BAD_ARG;
+    const int64_t total = rows * cols;
+    if(total == 0)
+        return MI355_OK;
+    hipLaunchKernelGGL(unpack_fp4_kernel, dim3(blocks_for((total + 7) / 8)), dim3(PW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint8_t*>(in),
+                       static_cast<uint8_t*>(out), total);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_pack_fp4(const float* in, void* out, int64_t rows, int64_t cols, void* stream)
+{
+    if(in == nullptr || out == nullptr || rows < 0 || cols < 0)
+        return MI355_ERR_BAD_ARG;
+    if(cols % 2 != 0)
+        return MI355_ERR_BAD_ARG; // PACK_FP4: can not pack along an axis of odd length
+    const int64_t total_out = rows * (cols / 2);
+    if(total_out == 0)
+        return MI355_OK;
+    hipLaunchKernelGGL(pack_fp4_kernel, dim3(blocks_for(total_out)), dim3(PW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), in, static_cast<uint8_t*>(out), total_out);
     return mi355_launch_status();
 }
 

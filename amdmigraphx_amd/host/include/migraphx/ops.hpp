@@ -78,6 +78,32 @@ struct pack_int4
     shape compute_shape(const std::vector<shape>& inputs) const;
 };
 
+// src/include/migraphx/op/unpack_fp4.hpp:42-76: fp4x2 -> fp8e4m3fn, the axis doubled
+struct unpack_fp4
+{
+    int64_t axis = -1;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
+    std::string name() const { return "unpack_fp4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
+// src/include/migraphx/op/pack_fp4.hpp:43-80: any arithmetic type -> fp4x2, the axis halved
+struct pack_fp4
+{
+    int64_t axis = -1;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
+    std::string name() const { return "pack_fp4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
 // src/include/migraphx/op/convert.hpp:40-62
 struct convert
 {

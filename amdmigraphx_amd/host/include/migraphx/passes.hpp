@@ -26,6 +26,9 @@ struct dead_code_elimination
 struct simplify_qdq
 {
     bool remove_qdq_only = false;
+    // also rewrite dot(DQ(a, block scales), DQ(b, block scales)) to the four-input quant_dot
+    // (simplify_qdq.hpp:42, set by a target whose hardware has block-scaled matrix instructions)
+    bool use_mx_quant = false;
     std::string name() const { return "simplify_qdq"; }
     void apply(module& m) const;
 };

@@ -56,7 +56,8 @@ struct shape
         fp8e5m2_type     = 14,
         bf16_type        = 15,
         fp8e5m2fnuz_type = 16,
-        tuple_type       = 17
+        tuple_type       = 17,
+        fp4x2_type       = 18 // two e2m1 values packed in a byte, low nibble first; not visitable
     };
 
     template <class T>

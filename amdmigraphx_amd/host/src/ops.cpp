@@ -138,6 +138,29 @@ shape pack_int4::compute_shape(const std::vector<shape>& inputs) const
     return {in.type(), lens};
 }
 
+shape unpack_fp4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "UNPACK_FP4", 1, 1);
+    const auto& in = inputs[0];
+    if(in.type() != shape::fp4x2_type)
+        MIGRAPHX_THROW("UNPACK_FP4: Only fp4x2_type is supported for unpacking");
+    auto lens = in.lens();
+    lens[normalize_axis(axis, in.ndim(), "UNPACK_FP4")] *= 2;
+    return {shape::fp8e4m3fn_type, lens};
+}
+
+shape pack_fp4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "PACK_FP4", 1, 1);
+    const auto& in = inputs[0];
+    auto lens      = in.lens();
+    const auto ax  = normalize_axis(axis, in.ndim(), "PACK_FP4");
+    if(lens[ax] % 2 != 0)
+        MIGRAPHX_THROW("PACK_FP4: Can not pack along axis of odd length (" + std::to_string(lens[ax]) + ")");
+    lens[ax] /= 2;
+    return {shape::fp4x2_type, lens};
+}
+
 shape convert::compute_shape(const std::vector<shape>& inputs) const
 {
     check_count(inputs, "CONVERT", 1, 1);
@@ -443,6 +466,8 @@ MIGRAPHX_REGISTER_OP(op::dot);
 MIGRAPHX_REGISTER_OP(op::quantizelinear);
 MIGRAPHX_REGISTER_OP(op::dequantizelinear);
 MIGRAPHX_REGISTER_OP(op::unpack_int4);
+MIGRAPHX_REGISTER_OP(op::unpack_fp4);
+MIGRAPHX_REGISTER_OP(op::pack_fp4);
 MIGRAPHX_REGISTER_OP(op::pack_int4);
 MIGRAPHX_REGISTER_OP(op::convert);
 MIGRAPHX_REGISTER_OP(op::mul);

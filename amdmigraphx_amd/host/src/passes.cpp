@@ -223,6 +223,39 @@ void find_quantizable_dot(module& m, instruction_ref qop)
     m.replace_instruction(qop, dq);
 }
 
+// simplify_qdq.cpp:290-357: block quantization of the MX types.  Both operands of the dot come
+// (through view operators) from a two-input dequantizelinear whose scale, behind its broadcasts,
+// is neither a scalar nor one-dimensional, i.e. has the operand's own rank: one scale per block,
+// spread over the elements.  The dot becomes quant_dot(a, b, scale_a, scale_b), the operators that
+// stood between each DQ and the dot re-applied to its tensor and to its scales alike.
+bool is_block_dq(instruction_ref dq)
+{
+    if(dq->name() != "dequantizelinear" or dq->inputs().size() != 2)
+        return false;
+    auto scale = skip_broadcasts(dq->inputs()[1]);
+    return not scale->get_shape().scalar() and scale->get_shape().ndim() != 1;
+}
+
+void find_mx_quantizable_dot(module& m, instruction_ref qop)
+{
+    auto dq1 = find_dq(qop->inputs()[0]);
+    auto dq2 = find_dq(qop->inputs()[1]);
+    if(not is_block_dq(dq1) or not is_block_dq(dq2))
+        return;
+    bool is_fp16_model = false;
+    if(dq1->get_shape().type() != qop->get_shape().type() and
+       qop->get_shape().type() == shape::half_type)
+        is_fp16_model = true;
+    auto qop_args = qop->inputs();
+    auto between0 = get_between_ins(dq1, qop_args[0]);
+    auto between1 = get_between_ins(dq2, qop_args[1]);
+    qop_args[0]   = propagate_quantized_ins(m, dq1, dq1->inputs().front(), between0, is_fp16_model);
+    qop_args[1]   = propagate_quantized_ins(m, dq2, dq2->inputs().front(), between1, is_fp16_model);
+    qop_args.push_back(propagate_quantized_ins(m, dq1, dq1->inputs()[1], between0, is_fp16_model));
+    qop_args.push_back(propagate_quantized_ins(m, dq2, dq2->inputs()[1], between1, is_fp16_model));
+    m.replace_instruction(qop, make_op("quant_dot"), qop_args);
+}
+
 // simplify_qdq.cpp:360-394
 bool compare_literals(instruction_ref a, instruction_ref b)
 {
@@ -355,6 +388,15 @@ void simplify_qdq::apply(module& m) const
             find_quantizable_dot(m, ins);
     }
     dead_code_elimination{}.apply(m);
+    if(use_mx_quant)
+    {
+        for(auto ins : all_instructions(m))
+        {
+            if(ins->name() == "dot")
+                find_mx_quantizable_dot(m, ins);
+        }
+        dead_code_elimination{}.apply(m);
+    }
     remove_qdq_pairs(m);
     dead_code_elimination{}.apply(m);
     remove_zero_point(m);

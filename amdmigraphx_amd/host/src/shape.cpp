@@ -59,7 +59,8 @@ std::size_t shape::type_size(type_t t)
     case fp8e4m3fnuz_type:
     case fp8e4m3fn_type:
     case fp8e5m2_type:
-    case fp8e5m2fnuz_type: return 1;
+    case fp8e5m2fnuz_type:
+    case fp4x2_type: return 1;
     case half_type:
     case bf16_type:
     case uint16_type:
@@ -211,13 +212,14 @@ std::string shape::type_name(type_t t)
     case bf16_type: return "bf16_type";
     case fp8e5m2fnuz_type: return "fp8e5m2fnuz_type";
     case tuple_type: return "tuple_type";
+    case fp4x2_type: return "fp4x2_type";
     }
     return "unknown_type";
 }
 
 shape::type_t shape::parse_type(const std::string& s)
 {
-    for(int i = 0; i <= tuple_type; i++)
+    for(int i = 0; i <= fp4x2_type; i++)
     {
         auto n = type_name(static_cast<type_t>(i));
         if(s == n or s + "_type" == n)

@@ -188,6 +188,22 @@ struct pack_int4
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// inputs: x (fp4x2), out (fp8e4m3fn) / x (float), out (fp4x2).  The packed axis is the last one.
+struct unpack_fp4
+{
+    std::string name() const { return "mi355::unpack_fp4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+struct pack_fp4
+{
+    std::string name() const { return "mi355::pack_fp4"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 struct convert
 {
     shape::type_t target_type = shape::half_type;

@@ -471,6 +471,29 @@ void lower_instruction(module& m, instruction_ref ins)
         else
             m.replace_instruction(ins, operation{pack_int4{}}, x, standard_out());
     }
+    else if(name == "unpack_fp4" or name == "pack_fp4")
+    {
+        const auto nd   = static_cast<int64_t>(ins->inputs()[0]->get_shape().ndim());
+        const auto axis = name == "unpack_fp4" ? any_cast<op::unpack_fp4>(ins->get_operator()).axis
+                                               : any_cast<op::pack_fp4>(ins->get_operator()).axis;
+        if(axis != -1 and axis != nd - 1)
+            MIGRAPHX_THROW("mi355: " + name + " along an axis other than the last has no kernel");
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        if(name == "unpack_fp4")
+        {
+            m.replace_instruction(ins, operation{unpack_fp4{}}, x, standard_out());
+        }
+        else
+        {
+            if(x->get_shape().type() != shape::float_type)
+            {
+                convert cv;
+                cv.target_type = shape::float_type;
+                x = m.insert_instruction(ins, operation{cv}, x, out(shape{shape::float_type, x->get_shape().lens()}));
+            }
+            m.replace_instruction(ins, operation{pack_fp4{}}, x, standard_out());
+        }
+    }
     else if(name == "convert")
     {
         convert op;

@@ -606,6 +606,48 @@ argument unpack_int4::compute(migraphx::context& ctx, const shape&, const std::v
     return args[1];
 }
 
+shape unpack_fp4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    auto out = op::unpack_fp4{}.compute_shape({inputs[0]});
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::unpack_fp4: output buffer has the wrong shape");
+    return out;
+}
+
+argument unpack_fp4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_unpack_fp4(args[0].data(), args[1].data(), rows, cols, stream_of(ctx)), name());
+    return args[1];
+}
+
+shape pack_fp4::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::pack_fp4: the kernel takes float input");
+    auto out = op::pack_fp4{}.compute_shape({inputs[0]});
+    if(inputs[1] != out)
+        MIGRAPHX_THROW("mi355::pack_fp4: output buffer has the wrong shape");
+    return out;
+}
+
+argument pack_fp4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(args[0].get_shape(), rows, cols);
+    status_check(mi355_pack_fp4(reinterpret_cast<const float*>(args[0].data()), args[1].data(), rows, cols,
+                                stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
 shape pack_int4::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -834,7 +876,11 @@ argument gather::compute(migraphx::context& ctx, const shape&, const std::vector
 std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_options& options) const
 {
     auto& ctx = any_cast<context>(gctx);
-    return {simplify_qdq{},
+    // gfx950 has the block-scaled matrix instructions, so the MX rewrite is on, as the reference's
+    // gpu target switches it (src/targets/gpu/target.cpp:129)
+    simplify_qdq sq;
+    sq.use_mx_quant = true;
+    return {sq,
             dead_code_elimination{},
             lowering{&ctx, options.offload_copy},
             dead_code_elimination{}};
@@ -854,6 +900,8 @@ MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
 MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::unpack_int4);
+MIGRAPHX_REGISTER_OP(mi355::unpack_fp4);
+MIGRAPHX_REGISTER_OP(mi355::pack_fp4);
 MIGRAPHX_REGISTER_OP(mi355::pack_int4);
 MIGRAPHX_REGISTER_OP(mi355::convert);
 MIGRAPHX_REGISTER_OP(mi355::contiguous);

@@ -178,6 +178,32 @@ def dequantizelinear(x, scale, zp=None, x_type=None):
     return out
 
 
+def unpack_fp4(x):
+    """fp4x2 bytes (uint8) -> fp8 e4m3fn bits (uint8), last axis doubled."""
+    _require_cuda(x)
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    out = torch.empty(x.shape[:-1] + (cols * 2,), dtype=torch.uint8, device=x.device)
+    check(lib().mi355_unpack_fp4(_ptr(x), _ptr(out), rows, cols, _stream()), "mi355_unpack_fp4")
+    return out
+
+
+def pack_fp4(x):
+    """float32 -> fp4x2 bytes (uint8), last axis halved."""
+    _require_cuda(x)
+    if x.dtype != torch.float32:
+        raise Mi355Error("pack_fp4: float32 input")
+    x = x.contiguous()
+    cols = x.shape[-1]
+    if cols % 2:
+        raise Mi355Error("PACK_FP4: Can not pack along axis of odd length")
+    rows = x.numel() // max(cols, 1)
+    out = torch.empty(x.shape[:-1] + (cols // 2,), dtype=torch.uint8, device=x.device)
+    check(lib().mi355_pack_fp4(_ptr(x), _ptr(out), rows, cols, _stream()), "mi355_pack_fp4")
+    return out
+
+
 def unpack_int4(x):
     x = x.contiguous()
     cols = x.shape[-1]

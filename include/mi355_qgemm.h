@@ -169,6 +169,19 @@ int mi355_pack_int4(const void* in, void* out, int32_t is_signed,
                     int64_t rows, int64_t cols, void* stream);
 
 /*
+ * unpack_fp4 / pack_fp4 along the last axis of a dense [rows, cols] tensor (cols = packed length
+ * for unpack, unpacked length for pack).  fp4 is e2m1 (magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6), two
+ * codes per byte, low nibble = even element.
+ *
+ * Replaces: op::unpack_fp4::compute (src/include/migraphx/op/unpack_fp4.hpp:78-101), which writes
+ * fp8 e4m3fn, and op::pack_fp4::compute (src/include/migraphx/op/pack_fp4.hpp:82-106) with
+ * cast_to_fp4 of src/include/migraphx/fp4_casts.hpp:80-100 (nearest, ties to the even code,
+ * saturating at 6, NaN -> 0) for float input.
+ */
+int mi355_unpack_fp4(const void* in, void* out, int64_t rows, int64_t cols, void* stream);
+int mi355_pack_fp4(const float* in, void* out, int64_t rows, int64_t cols, void* stream);
+
+/*
  * convert float -> half / bf16 / fp8 and back on n dense elements.
  *
  * Replaces: op::convert::compute (src/include/migraphx/op/convert.hpp:64-87)

@@ -45,6 +45,14 @@ def _load():
     lib.orc_unpack_int4.restype = None
     lib.orc_pack_int4.argtypes = [vp, vp, ci, i64, i64, i64]
     lib.orc_pack_int4.restype = None
+    lib.orc_unpack_fp4.argtypes = [vp, vp, i64, i64, i64]
+    lib.orc_unpack_fp4.restype = None
+    lib.orc_pack_fp4.argtypes = [vp, vp, i64, i64, i64]
+    lib.orc_pack_fp4.restype = None
+    lib.orc_fp4_to_f32.argtypes = [ctypes.c_uint8]
+    lib.orc_fp4_to_f32.restype = ctypes.c_float
+    lib.orc_fp4_from_f32.argtypes = [ctypes.c_float]
+    lib.orc_fp4_from_f32.restype = ctypes.c_uint8
     lib.orc_convert.argtypes = [vp, ci, vp, ci, ctypes.c_size_t]
     lib.orc_convert.restype = None
     lib.orc_mul_f32.argtypes = [vp, vp, i64, i64, vp, i64, i64, i64, i64]
@@ -223,6 +231,38 @@ def pack_int4(x, axis=-1):
     out = np.empty(shp, xc.dtype)
     _lib.orc_pack_int4(_p(out), _p(xc), int(signed), outer, alen // 2, inner)
     return out
+
+
+def unpack_fp4(x, axis=-1):
+    """fp4x2 bytes -> fp8 e4m3fn bytes, the axis doubled (op/unpack_fp4.hpp:78-101)."""
+    xc = np.ascontiguousarray(x, dtype=np.uint8)
+    axis, outer, alen, inner = _axis_split(xc.shape, axis)
+    shp = list(xc.shape)
+    shp[axis] *= 2
+    out = np.empty(shp, np.uint8)
+    _lib.orc_unpack_fp4(_p(out), _p(xc), outer, alen, inner)
+    return out
+
+
+def pack_fp4(x, axis=-1):
+    """float32 -> fp4x2 bytes, the axis halved (op/pack_fp4.hpp:82-106)."""
+    xc = np.ascontiguousarray(x, dtype=np.float32)
+    axis, outer, alen, inner = _axis_split(xc.shape, axis)
+    if alen % 2:
+        raise ValueError("PACK_FP4: Can not pack along axis of odd length")
+    shp = list(xc.shape)
+    shp[axis] //= 2
+    out = np.empty(shp, np.uint8)
+    _lib.orc_pack_fp4(_p(out), _p(xc), outer, alen // 2, inner)
+    return out
+
+
+def fp4_to_f32(code):
+    return float(_lib.orc_fp4_to_f32(int(code) & 0xff))
+
+
+def fp4_from_f32(x):
+    return int(_lib.orc_fp4_from_f32(float(x)))
 
 
 def convert(x, x_type, out_type):

@@ -29,6 +29,10 @@
  *   orc_dequantizelinear          test/ref/dequantizelinear.cpp:32-83
  *   orc_unpack_int4/orc_pack_int4 test/ref/unpack_int4.cpp, pack_int4.cpp,
  *                                 pack_unpack_int4.cpp
+ *   orc_unpack_fp4/orc_pack_fp4   test/ref/pack_unpack_fp4.cpp:34-89 (three cases) +
+ *                                 all 16 codes against the e2m1 definition
+ *                                 (+-{0, .5, 1, 1.5, 2, 3, 4, 6}), nearest-even on
+ *                                 every midpoint, saturation, NaN -> 0
  *   orc_dot                       test/onnx/verify/matmulnbits_tests.cpp golds
  *                                 (whole unpack -> dequantize -> dot chain)
  *   orc_convert                   test/ref/convert.cpp + closed form
@@ -599,6 +603,70 @@ void orc_pack_int4(
                     u2 = in[i2] > 15 ? 15 : in[i2];
                 }
                 out[(o * axis_len + a) * inner + i] = (uint8_t)((u2 << 4) | (u1 & 0xf));
+            }
+}
+
+/* ------------------------------------------------------------------------
+ * fp4 (e2m1) casts  src/include/migraphx/fp4_casts.hpp:41-100
+ * unpack_fp4::compute  src/include/migraphx/op/unpack_fp4.hpp:78-101
+ * pack_fp4::compute    src/include/migraphx/op/pack_fp4.hpp:82-106
+ * A code is sign (bit 3), exponent (bits 2:1), mantissa (bit 0); the eight magnitudes are
+ * 0, 0.5, 1, 1.5, 2, 3, 4, 6.  float -> fp4 rounds to the nearest magnitude, a tie going to the
+ * neighbour with an even code (0.25 -> 0, 0.75 -> 1, 1.25 -> 1, 1.75 -> 2, 2.5 -> 2, 3.5 -> 4,
+ * 5 -> 4); anything above 5 (infinity included) gives 6; NaN gives code 0; the sign bit is kept,
+ * also for zero.  unpack writes fp8 e4m3fn (every fp4 value is one), low nibble first; pack reads
+ * floats.  Dense tensor seen as [outer, axis_len, inner] as for int4.
+ * ---------------------------------------------------------------------- */
+static const float orc_fp4_values[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+
+float orc_fp4_to_f32(uint8_t code)
+{
+    float v = orc_fp4_values[code & 7];
+    return (code & 8) ? -v : v;
+}
+
+uint8_t orc_fp4_from_f32(float x)
+{
+    if(isnan(x))
+        return 0;
+    uint8_t sign = signbit(x) ? 8 : 0;
+    float a      = fabsf(x);
+    uint8_t i    = 0;
+    /* first magnitude whose upper tie point is not passed; the tie belongs to the even code */
+    for(i = 0; i < 7; i++)
+    {
+        float tie = 0.5f * (orc_fp4_values[i] + orc_fp4_values[i + 1]);
+        if(a < tie || (a == tie && (i & 1) == 0))
+            break;
+    }
+    return (uint8_t)(i | sign);
+}
+
+void orc_unpack_fp4(uint8_t* out, const uint8_t* in, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t a = 0; a < axis_len; a++)
+            for(int64_t i = 0; i < inner; i++)
+            {
+                uint8_t v   = in[(o * axis_len + a) * inner + i];
+                size_t lo_i = (size_t)((o * 2 * axis_len + 2 * a) * inner + i);
+                size_t hi_i = lo_i + (size_t)inner;
+                out[lo_i]   = orc_fp8e4m3fn_from_f32(orc_fp4_to_f32(v & 0xf));
+                out[hi_i]   = orc_fp8e4m3fn_from_f32(orc_fp4_to_f32(v >> 4));
+            }
+}
+
+void orc_pack_fp4(uint8_t* out, const float* in, int64_t outer, int64_t axis_len, int64_t inner)
+{
+    /* axis_len is the OUTPUT axis length; the input axis is 2*axis_len */
+    for(int64_t o = 0; o < outer; o++)
+        for(int64_t a = 0; a < axis_len; a++)
+            for(int64_t i = 0; i < inner; i++)
+            {
+                size_t i1 = (size_t)((o * 2 * axis_len + 2 * a) * inner + i);
+                size_t i2 = i1 + (size_t)inner;
+                out[(o * axis_len + a) * inner + i] =
+                    (uint8_t)((orc_fp4_from_f32(in[i2]) << 4) | (orc_fp4_from_f32(in[i1]) & 0xf));
             }
 }
 

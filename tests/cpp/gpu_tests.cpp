@@ -282,6 +282,63 @@ TEST_CASE(quant_dot_four_inputs)
     }
 }
 
+TEST_CASE(mx_fp4_matmul)
+{
+    // MX fp4: packed e2m1 operands, one power-of-two scale per 32 elements along K, as a graph of
+    // unpack_fp4 -> dequantizelinear -> dot (test/simplify_qdq_test.cpp:1776-1860).  The target's
+    // simplify_qdq turns it into the four-input quant_dot; the result equals the CPU target's bit
+    // for bit (every product float(a) * scale is exact).
+    const std::size_t bt = 2, m = 40, k = 96, n = 24;
+    shape pa{shape::fp4x2_type, {bt, m, k / 2}};
+    shape pb{shape::fp4x2_type, {bt, n, k / 2}};
+    shape sa{shape::float_type, {bt, m, k}};
+    shape sb{shape::float_type, {bt, n, k}};
+    program p;
+    {
+        auto* mm = p.get_main_module();
+        auto a   = mm->add_parameter("a", pa);
+        auto b   = mm->add_parameter("b", pb);
+        auto s1  = mm->add_parameter("sa", sa);
+        auto s2  = mm->add_parameter("sb", sb);
+        auto ua  = mm->add_instruction(make_op("unpack_fp4"), a);
+        auto ub  = mm->add_instruction(make_op("unpack_fp4"), b);
+        auto da  = mm->add_instruction(make_op("dequantizelinear"), ua, s1);
+        auto db  = mm->add_instruction(make_op("dequantizelinear"), ub, s2);
+        auto tb  = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1}}}), db);
+        mm->add_return({mm->add_instruction(make_op("dot"), da, tb)});
+    }
+    argument aa{pa};
+    argument ba{pb};
+    const auto ca = uniform_ints<uint8_t>(pa.elements(), 0, 255, 41);
+    const auto cb = uniform_ints<uint8_t>(pb.elements(), 0, 255, 42);
+    std::memcpy(aa.data(), ca.data(), ca.size());
+    std::memcpy(ba.data(), cb.data(), cb.size());
+    auto block_scales = [](std::size_t rows, std::size_t kk, unsigned seed) {
+        auto e = uniform_ints<int>(rows * (kk / 32), -5, 5, seed);
+        std::vector<float> v(rows * kk);
+        for(std::size_t i = 0; i < v.size(); i++)
+            v[i] = std::ldexp(1.0f, e[i / 32]);
+        return v;
+    };
+    migraphx::parameter_map params = {{"a", aa}, {"b", ba}, {"sa", argument{sa, block_scales(bt * m, k, 43)}},
+                                      {"sb", argument{sb, block_scales(bt * n, k, 44)}}};
+    expect_same(p, params);
+    program c = p;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::unpack_fp4") == 2);
+    EXPECT(count_ops(*c.get_main_module(), "mi355::dot") == 1);
+    EXPECT(not has_op(c, "dequantizelinear") and not has_op(c, "mi355::dequantizelinear"));
+    // pack_fp4 on the device: float -> fp4x2 -> fp8, against the CPU target
+    program r;
+    {
+        auto* mm = r.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, {16, 64}});
+        auto pk  = mm->add_instruction(make_op("pack_fp4"), x);
+        mm->add_return({pk, mm->add_instruction(make_op("unpack_fp4"), pk)});
+    }
+    expect_same(r, {{"x", argument{shape{shape::float_type, {16, 64}}, uniform_floats(16 * 64, -7.0f, 7.0f, 45)}}});
+}
+
 TEST_CASE(fp8_quantized_matmul)
 {
     // BASELINE config 3 in small: activations and weights quantized to fp8 e4m3fn with amax-based

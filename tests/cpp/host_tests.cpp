@@ -566,6 +566,201 @@ TEST_CASE(qdq_dot_asymmetric)
 
 // ---------------------------------------------------------------- quantize_int4, quantize_int8
 
+// ---------------------------------------------------------------- MX block quantization (fp4)
+
+static void run_mx_pass(module& m)
+{
+    migraphx::simplify_qdq sq;
+    sq.use_mx_quant = true;
+    migraphx::run_passes(m, {sq, migraphx::dead_code_elimination{}});
+}
+
+TEST_CASE(fp4_shapes)
+{
+    // op/unpack_fp4.hpp:61-76, op/pack_fp4.hpp:64-80
+    auto un = make_op("unpack_fp4");
+    EXPECT(un.compute_shape({shape{shape::fp4x2_type, {1, 3, 6, 12}}}) ==
+           shape{shape::fp8e4m3fn_type, {1, 3, 6, 24}});
+    EXPECT(make_op("unpack_fp4", {{"axis", 1}}).compute_shape({shape{shape::fp4x2_type, {2, 1}}}) ==
+           shape{shape::fp8e4m3fn_type, {2, 2}});
+    EXPECT(test::throws([&] { un.compute_shape({shape{shape::uint8_type, {2, 2}}}); }));
+    auto pk = make_op("pack_fp4", {{"axis", 1}});
+    EXPECT(pk.compute_shape({shape{shape::float_type, {2, 2}}}) == shape{shape::fp4x2_type, {2, 1}});
+    EXPECT(test::throws([&] { pk.compute_shape({shape{shape::float_type, {2, 3}}}); }));
+    EXPECT(shape{shape::fp4x2_type, {4, 4}}.bytes() == 16);
+    EXPECT(shape::parse_type("fp4x2_type") == shape::fp4x2_type);
+}
+
+TEST_CASE(fp4_pack_unpack_known_answers)
+{
+    // test/ref/pack_unpack_fp4.cpp:34-89
+    program p;
+    auto* mm = p.get_main_module();
+    auto l0  = mm->add_literal(literal{shape{shape::float_type, {2, 2}}, std::vector<float>{-2.f, 3.4f, 3.5f, 0.f}});
+    auto pk  = mm->add_instruction(make_op("pack_fp4", {{"axis", 1}}), l0);
+    auto un  = mm->add_instruction(make_op("unpack_fp4", {{"axis", 1}}), pk);
+    mm->add_return({pk, un});
+    auto r = testutil::run_on("oracle", p, {});
+    EXPECT(r.size() == 2);
+    EXPECT(r[0].get_shape() == shape{shape::fp4x2_type, {2, 1}});
+    EXPECT(static_cast<uint8_t>(r[0].data()[0]) == 0x5C and static_cast<uint8_t>(r[0].data()[1]) == 0x06);
+    EXPECT(r[1].to_vector<float>() == std::vector<float>{-2.f, 3.f, 4.f, 0.f});
+}
+
+TEST_CASE(fp4x2_quant_dot_even)
+{
+    // test/simplify_qdq_test.cpp:1776-1814
+    shape pa{shape::fp4x2_type, {1, 3, 6, 12}};
+    shape pb{shape::fp4x2_type, {1, 3, 24, 4}};
+    shape sa{shape::float_type, {1, 3, 6, 24}};
+    shape sb{shape::float_type, {1, 3, 24, 8}};
+    module m1;
+    {
+        auto a   = m1.add_parameter("input", pa);
+        auto b   = m1.add_parameter("weights", pb);
+        auto s1  = m1.add_parameter("scale_a", sa);
+        auto s2  = m1.add_parameter("scale_b", sb);
+        auto ua  = m1.add_instruction(make_op("unpack_fp4"), a);
+        auto ub  = m1.add_instruction(make_op("unpack_fp4"), b);
+        auto da  = m1.add_instruction(make_op("dequantizelinear"), ua, s1);
+        auto db  = m1.add_instruction(make_op("dequantizelinear"), ub, s2);
+        m1.add_return({m1.add_instruction(make_op("dot"), da, db)});
+    }
+    module m2;
+    {
+        auto a  = m2.add_parameter("input", pa);
+        auto b  = m2.add_parameter("weights", pb);
+        auto s1 = m2.add_parameter("scale_a", sa);
+        auto s2 = m2.add_parameter("scale_b", sb);
+        auto ua = m2.add_instruction(make_op("unpack_fp4"), a);
+        auto ub = m2.add_instruction(make_op("unpack_fp4"), b);
+        m2.add_return({m2.add_instruction(make_op("quant_dot"), ua, ub, s1, s2)});
+    }
+    run_mx_pass(m1);
+    EXPECT(testutil::canonical(m1) == testutil::canonical(m2));
+    // without the option the graph stays as it is
+    module m3 = m2;
+    run_pass(m3);
+    EXPECT(testutil::canonical(m3) == testutil::canonical(m2));
+}
+
+TEST_CASE(fp4x2_quant_dot_trans_b)
+{
+    // test/simplify_qdq_test.cpp:1816-1860: the transpose between DQ and dot moves to the packed
+    // tensor's unpacked form and to its scales
+    shape pa{shape::fp4x2_type, {1, 3, 6, 12}};
+    shape pb{shape::fp4x2_type, {1, 3, 8, 12}};
+    shape sa{shape::float_type, {1, 3, 6, 24}};
+    shape sb{shape::float_type, {1, 3, 8, 24}};
+    module m1;
+    {
+        auto a  = m1.add_parameter("input", pa);
+        auto b  = m1.add_parameter("weights", pb);
+        auto s1 = m1.add_parameter("scale_a", sa);
+        auto s2 = m1.add_parameter("scale_b", sb);
+        auto ua = m1.add_instruction(make_op("unpack_fp4"), a);
+        auto ub = m1.add_instruction(make_op("unpack_fp4"), b);
+        auto da = m1.add_instruction(make_op("dequantizelinear"), ua, s1);
+        auto db = m1.add_instruction(make_op("dequantizelinear"), ub, s2);
+        auto tb = m1.add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), db);
+        m1.add_return({m1.add_instruction(make_op("dot"), da, tb)});
+    }
+    module m2;
+    {
+        auto a   = m2.add_parameter("input", pa);
+        auto b   = m2.add_parameter("weights", pb);
+        auto s1  = m2.add_parameter("scale_a", sa);
+        auto s2  = m2.add_parameter("scale_b", sb);
+        auto ua  = m2.add_instruction(make_op("unpack_fp4"), a);
+        auto ub  = m2.add_instruction(make_op("unpack_fp4"), b);
+        auto tb  = m2.add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), ub);
+        auto ts2 = m2.add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), s2);
+        m2.add_return({m2.add_instruction(make_op("quant_dot"), ua, tb, s1, ts2)});
+    }
+    run_mx_pass(m1);
+    EXPECT(testutil::canonical(m1) == testutil::canonical(m2));
+}
+
+TEST_CASE(fp4x2_quant_dot_const_b)
+{
+    // test/simplify_qdq_test.cpp:1862-1905: constant packed weights and scales
+    shape pa{shape::fp4x2_type, {1, 3, 6, 12}};
+    shape pb{shape::fp4x2_type, {1, 3, 24, 4}};
+    shape sa{shape::float_type, {1, 3, 6, 24}};
+    shape sb{shape::float_type, {1, 3, 24, 8}};
+    const auto bytes = testutil::uniform_ints<uint8_t>(pb.elements(), 0, 255, 826);
+    const auto sbv   = testutil::uniform_floats(sb.elements(), 0.25f, 4.0f, 826);
+    auto build = [&](module& m, bool rewritten) {
+        auto a  = m.add_parameter("input", pa);
+        auto b  = m.add_literal(literal{pb, reinterpret_cast<const char*>(bytes.data())});
+        auto s1 = m.add_parameter("scale_a", sa);
+        auto s2 = m.add_literal(literal{sb, sbv});
+        auto ua = m.add_instruction(make_op("unpack_fp4"), a);
+        auto ub = m.add_instruction(make_op("unpack_fp4"), b);
+        if(rewritten)
+        {
+            m.add_return({m.add_instruction(make_op("quant_dot"), ua, ub, s1, s2)});
+            return;
+        }
+        auto da = m.add_instruction(make_op("dequantizelinear"), ua, s1);
+        auto db = m.add_instruction(make_op("dequantizelinear"), ub, s2);
+        m.add_return({m.add_instruction(make_op("dot"), da, db)});
+    };
+    module m1;
+    module m2;
+    build(m1, false);
+    build(m2, true);
+    run_mx_pass(m1);
+    EXPECT(testutil::canonical(m1) == testutil::canonical(m2));
+}
+
+TEST_CASE(mx_quant_dot_equals_dequantized_dot)
+{
+    // the rewritten graph computes what the fake-quantized one does: bit for bit on the CPU target,
+    // because DQ of an fp8 value by a float scale is the same single float product
+    const std::size_t m = 6, k = 64, n = 8;
+    shape pa{shape::fp4x2_type, {m, k / 2}};
+    shape pb{shape::fp4x2_type, {n, k / 2}};
+    shape sa{shape::float_type, {m, k}};
+    shape sb{shape::float_type, {n, k}};
+    program p;
+    {
+        auto* mm = p.get_main_module();
+        auto a   = mm->add_parameter("a", pa);
+        auto b   = mm->add_parameter("b", pb);
+        auto s1  = mm->add_parameter("sa", sa);
+        auto s2  = mm->add_parameter("sb", sb);
+        auto ua  = mm->add_instruction(make_op("unpack_fp4"), a);
+        auto ub  = mm->add_instruction(make_op("unpack_fp4"), b);
+        auto da  = mm->add_instruction(make_op("dequantizelinear"), ua, s1);
+        auto db  = mm->add_instruction(make_op("dequantizelinear"), ub, s2);
+        auto tb  = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), db);
+        mm->add_return({mm->add_instruction(make_op("dot"), da, tb)});
+    }
+    program q = p;
+    run_mx_pass(*q.get_main_module());
+    EXPECT(testutil::count_ops(*q.get_main_module(), "quant_dot") == 1);
+    EXPECT(testutil::count_ops(*q.get_main_module(), "dequantizelinear") == 0);
+    argument aa{pa};
+    argument ba{pb};
+    const auto ca = testutil::uniform_ints<uint8_t>(pa.elements(), 0, 255, 1);
+    const auto cb = testutil::uniform_ints<uint8_t>(pb.elements(), 0, 255, 2);
+    std::memcpy(aa.data(), ca.data(), ca.size());
+    std::memcpy(ba.data(), cb.data(), cb.size());
+    auto block_scales = [](std::size_t rows, std::size_t kk, unsigned seed) {
+        auto e = testutil::uniform_ints<int>(rows * (kk / 32), -4, 4, seed);
+        std::vector<float> v(rows * kk);
+        for(std::size_t i = 0; i < v.size(); i++)
+            v[i] = std::ldexp(1.0f, e[i / 32]);
+        return v;
+    };
+    migraphx::parameter_map params = {{"a", aa}, {"b", ba}, {"sa", argument{sa, block_scales(m, k, 3)}},
+                                      {"sb", argument{sb, block_scales(n, k, 4)}}};
+    auto want = testutil::run_on("oracle", p, params);
+    auto got  = testutil::run_on("oracle", q, params);
+    EXPECT(testutil::same_bytes(got[0], want[0]));
+}
+
 TEST_CASE(int4_pass)
 {
     // test/int4_test.cpp:38-90

@@ -23,6 +23,8 @@ void orc_unpack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t out
 void orc_pack_int4(uint8_t* out, const uint8_t* in, int is_signed, int64_t outer, int64_t axis_len,
                    int64_t inner);
 void orc_convert(void* out, int out_type, const void* x, int x_type, size_t n);
+void orc_unpack_fp4(uint8_t* out, const uint8_t* in, int64_t outer, int64_t axis_len, int64_t inner);
+void orc_pack_fp4(uint8_t* out, const float* in, int64_t outer, int64_t axis_len, int64_t inner);
 void orc_binary_f32(int op, float* out, const float* a, const float* b, size_t n);
 void orc_unary_f32(int op, float* out, const float* x, size_t n);
 void orc_reduce_mean_f32(float* out, const float* x, int64_t outer, int64_t axis_len, int64_t inner);
@@ -180,6 +182,36 @@ struct cpu_op
                 orc_pack_int4(reinterpret_cast<uint8_t*>(r.data()),
                               reinterpret_cast<const uint8_t*>(x.data()), is_signed, outer,
                               out.lens()[axis], inner);
+        }
+        else if(n == "unpack_fp4" or n == "pack_fp4")
+        {
+            argument x      = dense(args[0]);
+            const bool unpk = n == "unpack_fp4";
+            int64_t axis    = unpk ? migraphx::any_cast<migraphx::op::unpack_fp4>(op).axis
+                                   : migraphx::any_cast<migraphx::op::pack_fp4>(op).axis;
+            const auto& si  = x.get_shape();
+            if(axis < 0)
+                axis += static_cast<int64_t>(si.ndim());
+            int64_t outer = 1;
+            int64_t inner = 1;
+            for(int64_t i = 0; i < axis; i++)
+                outer *= si.lens()[i];
+            for(std::size_t i = axis + 1; i < si.ndim(); i++)
+                inner *= si.lens()[i];
+            if(unpk)
+            {
+                orc_unpack_fp4(reinterpret_cast<uint8_t*>(r.data()),
+                               reinterpret_cast<const uint8_t*>(x.data()), outer, si.lens()[axis], inner);
+            }
+            else
+            {
+                // cast_to_fp4 converts its argument to float first (fp4_casts.hpp:83-85)
+                argument xf{shape{shape::float_type, si.lens()}};
+                orc_convert(xf.data(), orc_type(shape::float_type), x.data(), orc_type(si.type()),
+                            si.elements());
+                orc_pack_fp4(reinterpret_cast<uint8_t*>(r.data()),
+                             reinterpret_cast<const float*>(xf.data()), outer, out.lens()[axis], inner);
+            }
         }
         else if(n == "convert")
         {

@@ -253,6 +253,30 @@ for i in range(1, 8):
                "gold": vec(body, "golden")})
 out["gather"] = ga
 
+# ---- pack_fp4 / unpack_fp4 (test/ref/pack_unpack_fp4.cpp) ---------------------------
+t = read("test/ref/pack_unpack_fp4.cpp")
+cases = test_cases(t)
+fp4 = []
+body = cases["pack_fp4"]
+fp4.append({"name": "pack_fp4", "source": "test/ref/pack_unpack_fp4.cpp",
+            "lens": num_list(re.search(r"float_type,\s*\{([^}]*)\}", body).group(1)),
+            "input": num_list(re.search(r"migraphx::literal\{s,\s*\{([^}]*)\}\}", body).group(1)),
+            "axis": int(re.search(r'"axis",\s*(-?\d+)', body).group(1)),
+            "gold_bytes": num_list(re.search(r"std::vector<uint8_t> gold\{([^}]*)\}", body).group(1))})
+body = cases["unpack_fp4"]
+fp4.append({"name": "unpack_fp4", "source": "test/ref/pack_unpack_fp4.cpp",
+            "lens": num_list(re.search(r"fp4x2_type,\s*\{([^}]*)\}", body).group(1)),
+            "input_bytes": num_list(re.search(r"packed_data\s*=\s*\{([^}]*)\}", body).group(1)),
+            "axis": int(re.search(r'"axis",\s*(-?\d+)', body).group(1)),
+            "gold": num_list(re.search(r"std::vector<float> gold\{([^}]*)\}", body).group(1))})
+body = cases["pack_unpack_fp4"]
+fp4.append({"name": "pack_unpack_fp4", "source": "test/ref/pack_unpack_fp4.cpp",
+            "lens": num_list(re.search(r"float_type,\s*\{([^}]*)\}", body).group(1)),
+            "input": num_list(re.search(r"migraphx::literal\{s,\s*\{([^}]*)\}\}", body).group(1)),
+            "axis": int(re.search(r'"axis",\s*(-?\d+)', body).group(1)),
+            "gold": num_list(re.search(r"std::vector<float> gold\{([^}]*)\}", body).group(1))})
+out["fp4"] = fp4
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -163,3 +163,25 @@ def test_convert(ops):
     got = ops.convert(half_dev(hb), ops.DT.F32)
     want = orc.convert(hb, orc.F16, orc.F32)
     assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_fp4_unpack_and_pack_match_oracle(ops):
+    """All 256 packed bytes through unpack (fp8 e4m3fn out), and pack on every rounding boundary,
+    its float neighbours, saturation, infinities, NaN and signed zeros -- bit for bit."""
+    packed = np.arange(256, dtype=np.uint8).reshape(8, 32)
+    got = ops.unpack_fp4(dev(packed)).cpu().numpy()
+    assert np.array_equal(got, orc.unpack_fp4(packed))
+    ties = np.float32([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
+    pts = np.concatenate([ties, np.nextafter(ties, np.float32(0)), np.nextafter(ties, np.float32(10)),
+                          np.float32([0, 0.5, 1, 1.5, 2, 3, 4, 6, 6.5, 448, 1e30, np.inf, np.nan, 1e-30])])
+    x = np.concatenate([pts, -pts]).astype(np.float32)
+    rng = np.random.default_rng(5)
+    x = np.concatenate([x, rng.uniform(-7, 7, 4096 - x.size).astype(np.float32)]).reshape(64, 64)
+    got = ops.pack_fp4(dev(x)).cpu().numpy()
+    assert np.array_equal(got, orc.pack_fp4(x))
+    # round trip on the device equals the oracle's
+    back = ops.unpack_fp4(ops.pack_fp4(dev(x))).cpu().numpy()
+    assert np.array_equal(back, orc.unpack_fp4(orc.pack_fp4(x)))
+    from amdmigraphx_amd import Mi355Error
+    with pytest.raises(Mi355Error):
+        ops.pack_fp4(dev(np.zeros((2, 3), np.float32)))
