@@ -32,24 +32,38 @@ MI355_DEVINL float load_f32(const void* p, int type, int64_t i)
     }
 }
 
-// 64 x 64 outputs per workgroup of 256 threads, 4 x 4 per thread, K in steps of 16 through LDS.
-__global__ __launch_bounds__(256) void dot_float_kernel(dot_params p)
+typedef double v4d __attribute__((ext_vector_type(4)));
+
+// The sums run on the fp64 matrix cores.  v_mfma_f64_16x16x4_f64 adds its four products to the
+// accumulator one after the other, k ascending, each as a fused multiply-add in double -- the
+// order and the rounding of the reference's loop -- so the results are the same bits (the tests
+// compare them with the CPU restatement).  Operand layout (probed): lane l supplies A[l % 16][l / 16] and
+// B[l / 16][l % 16]; register r of lane l holds D[4*r + l / 16][l % 16].
+// 64 x 64 outputs per workgroup of four waves (2 x 2, each 32 x 32 = 2 x 2 instruction tiles), K in
+// steps of 16 through LDS, where the tiles are kept as doubles (converted once, when staged).  The
+// row pitch of 80 doubles puts the two k rows a half wave reads into disjoint halves of the banks.
+__global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
 {
-    __shared__ float as[16][65];
-    __shared__ float bs[16][65];
-    const int tid = threadIdx.x;
-    const int tx  = tid & 15;
-    const int ty  = tid >> 4;
+    constexpr int PITCH = 80;
+    __shared__ double as[16][PITCH];
+    __shared__ double bs[16][PITCH];
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm   = wave >> 1;
+    const int wn   = wave & 1;
+    const int l16  = lane & 15;
+    const int lk   = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.y * 64;
     const int64_t col0 = (int64_t)blockIdx.x * 64;
     const int64_t ao   = (int64_t)blockIdx.z * p.stride_a;
     const int64_t bo   = (int64_t)blockIdx.z * p.stride_b;
-    double acc[4][4];
+    v4d acc[2][2];
 #pragma unroll
-    for(int i = 0; i < 4; i++)
+    for(int i = 0; i < 2; i++)
 #pragma unroll
-        for(int j = 0; j < 4; j++)
-            acc[i][j] = 0.0;
+        for(int j = 0; j < 2; j++)
+            acc[i][j] = v4d{0.0, 0.0, 0.0, 0.0};
 
     for(int64_t k0 = 0; k0 < p.k; k0 += 16)
     {
@@ -57,68 +71,198 @@ __global__ __launch_bounds__(256) void dot_float_kernel(dot_params p)
         for(int e = 0; e < 4; e++)
         {
             const int idx = tid + e * 256; // 0..1023
-            // A tile: element (r, kk) with kk fastest so that K-contiguous rows coalesce
             {
                 const int r  = idx >> 4;
                 const int kk = idx & 15;
                 float v      = 0.f;
                 if(row0 + r < p.m && k0 + kk < p.k)
                     v = load_f32(p.a, p.type, ao + (row0 + r) * p.a_sm + (k0 + kk) * p.a_sk);
-                as[kk][r] = v;
+                as[kk][r] = (double)v;
             }
-            // B tile: element (kk, c) with c fastest (row-major B coalesces)
             {
                 const int kk = idx >> 6;
                 const int c  = idx & 63;
                 float v      = 0.f;
                 if(col0 + c < p.n && k0 + kk < p.k)
                     v = load_f32(p.b, p.type, bo + (k0 + kk) * p.b_sk + (col0 + c) * p.b_sn);
-                bs[kk][c] = v;
+                bs[kk][c] = (double)v;
             }
         }
         __syncthreads();
 #pragma unroll
-        for(int kk = 0; kk < 16; kk++)
+        for(int kk0 = 0; kk0 < 16; kk0 += 4)
         {
-            double av[4], bv[4];
+            double av[2], bv[2];
 #pragma unroll
-            for(int i = 0; i < 4; i++)
-                av[i] = (double)as[kk][ty * 4 + i];
+            for(int i = 0; i < 2; i++)
+                av[i] = as[kk0 + lk][wm * 32 + i * 16 + l16];
 #pragma unroll
-            for(int j = 0; j < 4; j++)
-                bv[j] = (double)bs[kk][tx + 16 * j];
+            for(int j = 0; j < 2; j++)
+                bv[j] = bs[kk0 + lk][wn * 32 + j * 16 + l16];
 #pragma unroll
-            for(int i = 0; i < 4; i++)
+            for(int i = 0; i < 2; i++)
 #pragma unroll
-                for(int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_fma(av[i], bv[j], acc[i][j]);
+                for(int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
 #pragma unroll
-    for(int i = 0; i < 4; i++)
-    {
-        const int64_t row = row0 + ty * 4 + i;
-        if(row >= p.m)
-            continue;
+    for(int i = 0; i < 2; i++)
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int r = 0; r < 4; r++)
         {
-            const int64_t col = col0 + tx + 16 * j;
-            if(col >= p.n)
+            const int64_t row = row0 + wm * 32 + i * 16 + 4 * r + lk;
+            if(row >= p.m)
                 continue;
-            const int64_t idx = (int64_t)blockIdx.z * p.stride_c + row * p.ldc + col;
-            // static_cast<T>(double): double -> float (nearest even), then float -> 16-bit
-            // float by truncation for half and bf16
-            const float f = (float)acc[i][j];
-            if(p.type == MI355_F32)
-                ((float*)p.c)[idx] = f;
-            else if(p.type == MI355_F16)
-                ((uint16_t*)p.c)[idx] = f32_to_half_rtz(f);
-            else
-                ((uint16_t*)p.c)[idx] = f32_to_bf16_rtz(f);
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+            {
+                const int64_t col = col0 + wn * 32 + j * 16 + l16;
+                if(col >= p.n)
+                    continue;
+                const int64_t idx = (int64_t)blockIdx.z * p.stride_c + row * p.ldc + col;
+                const float f     = (float)acc[i][j][r];
+                if(p.type == MI355_F32)
+                    ((float*)p.c)[idx] = f;
+                else if(p.type == MI355_F16)
+                    ((uint16_t*)p.c)[idx] = f32_to_half_rtz(f);
+                else
+                    ((uint16_t*)p.c)[idx] = f32_to_bf16_rtz(f);
+            }
         }
+}
+
+// fp32 operands whose rows or columns are contiguous: the same kernel with 16-byte loads (one per
+// thread and operand per K step) that are issued one step ahead, so that their latency runs under
+// the matrix instructions.  A_KCONT: A's K stride is 1 (else its row stride is 1); B_NCONT: B's
+// column stride is 1 (else its K stride is 1).  The host checks the alignment the vector loads need;
+// a vector that would cross the matrix edge is read element by element with zero fill.
+template <bool A_KCONT, bool B_NCONT>
+__global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
+{
+    constexpr int PITCH = 80;
+    __shared__ double as[16][PITCH];
+    __shared__ double bs[16][PITCH];
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm   = wave >> 1;
+    const int wn   = wave & 1;
+    const int l16  = lane & 15;
+    const int lk   = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * 64;
+    const int64_t col0 = (int64_t)blockIdx.x * 64;
+    const float* a = static_cast<const float*>(p.a) + (int64_t)blockIdx.z * p.stride_a;
+    const float* b = static_cast<const float*>(p.b) + (int64_t)blockIdx.z * p.stride_b;
+    // this thread's piece of each tile: `major` indexes the strided dimension, `minor` the
+    // contiguous one (4 elements)
+    const int a_major = A_KCONT ? tid >> 2 : tid >> 4;        // row       | k
+    const int a_minor = A_KCONT ? (tid & 3) * 4 : (tid & 15) * 4; // k     | row
+    const int b_major = B_NCONT ? tid >> 4 : tid >> 2;        // k         | column
+    const int b_minor = B_NCONT ? (tid & 15) * 4 : (tid & 3) * 4; // column | k
+
+    auto load_a = [&](int64_t k0) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        const int64_t row = row0 + (A_KCONT ? a_major : a_minor);
+        const int64_t kk  = k0 + (A_KCONT ? a_minor : a_major);
+        const float* src  = a + row * p.a_sm + kk * p.a_sk;
+        const int64_t lim = A_KCONT ? p.k - kk : p.m - row; // elements left along the contiguous axis
+        const bool inside = A_KCONT ? row < p.m : kk < p.k;
+        if(inside && lim >= 4)
+            v = *reinterpret_cast<const v4f*>(src);
+        else if(inside)
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+                if(e < lim)
+                    v[e] = src[e];
+        }
+        return v;
+    };
+    auto load_b = [&](int64_t k0) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        const int64_t col = col0 + (B_NCONT ? b_minor : b_major);
+        const int64_t kk  = k0 + (B_NCONT ? b_major : b_minor);
+        const float* src  = b + kk * p.b_sk + col * p.b_sn;
+        const int64_t lim = B_NCONT ? p.n - col : p.k - kk;
+        const bool inside = B_NCONT ? kk < p.k : col < p.n;
+        if(inside && lim >= 4)
+            v = *reinterpret_cast<const v4f*>(src);
+        else if(inside)
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+                if(e < lim)
+                    v[e] = src[e];
+        }
+        return v;
+    };
+
+    v4d acc[2][2];
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++)
+            acc[i][j] = v4d{0.0, 0.0, 0.0, 0.0};
+
+    v4f va = load_a(0);
+    v4f vb = load_b(0);
+    for(int64_t k0 = 0; k0 < p.k; k0 += 16)
+    {
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+        {
+            if(A_KCONT)
+                as[a_minor + e][a_major] = (double)va[e];
+            else
+                as[a_major][a_minor + e] = (double)va[e];
+            if(B_NCONT)
+                bs[b_major][b_minor + e] = (double)vb[e];
+            else
+                bs[b_minor + e][b_major] = (double)vb[e];
+        }
+        __syncthreads();
+        if(k0 + 16 < p.k)
+        {
+            va = load_a(k0 + 16);
+            vb = load_b(k0 + 16);
+        }
+#pragma unroll
+        for(int kk0 = 0; kk0 < 16; kk0 += 4)
+        {
+            double av[2], bv[2];
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+                av[i] = as[kk0 + lk][wm * 32 + i * 16 + l16];
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+                bv[j] = bs[kk0 + lk][wn * 32 + j * 16 + l16];
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
     }
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int r = 0; r < 4; r++)
+        {
+            const int64_t row = row0 + wm * 32 + i * 16 + 4 * r + lk;
+            if(row >= p.m)
+                continue;
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+            {
+                const int64_t col = col0 + wn * 32 + j * 16 + l16;
+                if(col < p.n)
+                    static_cast<float*>(p.c)[(int64_t)blockIdx.z * p.stride_c + row * p.ldc + col] =
+                        (float)acc[i][j][r];
+            }
+        }
 }
 
 struct gather_params
@@ -183,8 +327,28 @@ extern "C" int mi355_dot(const void* a,
         return MI355_ERR_UNSUPPORTED;
     dot_params p{a, b, c, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc,
                  stride_a, stride_b, stride_c, type};
-    hipLaunchKernelGGL(dot_float_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)batch), dim3(256),
-                       0, static_cast<hipStream_t>(stream), p);
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // fp32 with contiguous rows or columns, everything the 16-byte loads touch aligned
+    auto aligned4 = [](int64_t x) { return x % 4 == 0; };
+    const bool a_k = a_stride_k == 1 && aligned4(a_stride_m);
+    const bool a_m = a_stride_m == 1 && aligned4(a_stride_k);
+    const bool b_n = b_stride_n == 1 && aligned4(b_stride_k);
+    const bool b_k = b_stride_k == 1 && aligned4(b_stride_n);
+    if(type == MI355_F32 && k > 0 && (a_k || a_m) && (b_n || b_k) && aligned4(stride_a) && aligned4(stride_b) &&
+       reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0)
+    {
+        if(a_k && b_n)
+            hipLaunchKernelGGL((dot_f32_mfma_kernel<true, true>), grid, dim3(256), 0, s, p);
+        else if(a_k)
+            hipLaunchKernelGGL((dot_f32_mfma_kernel<true, false>), grid, dim3(256), 0, s, p);
+        else if(b_n)
+            hipLaunchKernelGGL((dot_f32_mfma_kernel<false, true>), grid, dim3(256), 0, s, p);
+        else
+            hipLaunchKernelGGL((dot_f32_mfma_kernel<false, false>), grid, dim3(256), 0, s, p);
+        return mi355_launch_status();
+    }
+    hipLaunchKernelGGL(dot_float_mfma_kernel, grid, dim3(256), 0, s, p);
     return mi355_launch_status();
 }
 

@@ -586,6 +586,43 @@ TEST_CASE(no_host_fallback)
     }));
 }
 
+TEST_CASE(float_dot_layouts)
+{
+    // op::dot on fp32 (bit-identical to gemm_naive's double accumulation): row-major and transposed
+    // operands, sizes with ragged edges in every dimension, K not a multiple of 4, batches -- the
+    // vector-load kernel, its element-wise edges and the generic kernel (odd leading dimension)
+    struct dims { std::size_t b, m, n, k; };
+    for(auto d : {dims{1, 64, 64, 16}, dims{3, 70, 66, 50}, dims{2, 130, 36, 19}, dims{1, 5, 7, 3}, dims{2, 96, 128, 64}})
+    {
+        for(int variant = 0; variant < 4; variant++)
+        {
+            const bool ta = (variant & 1) != 0;
+            const bool tb = (variant & 2) != 0;
+            program p;
+            auto* mm = p.get_main_module();
+            shape sa{shape::float_type, ta ? std::vector<std::size_t>{d.b, d.k, d.m} : std::vector<std::size_t>{d.b, d.m, d.k}};
+            shape sb{shape::float_type, tb ? std::vector<std::size_t>{d.b, d.n, d.k} : std::vector<std::size_t>{d.b, d.k, d.n}};
+            instruction_ref a = mm->add_parameter("a", sa);
+            instruction_ref b = mm->add_parameter("b", sb);
+            if(ta)
+                a = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1}}}), a);
+            if(tb)
+                b = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1}}}), b);
+            mm->add_return({mm->add_instruction(make_op("dot"), a, b)});
+            // wide dynamic range so that a different summation order would show
+            auto wide = [](std::size_t cnt, unsigned seed) {
+                auto v = normal_floats(cnt, 1.0f, seed);
+                auto e = uniform_ints<int>(cnt, -12, 12, seed + 1);
+                for(std::size_t i = 0; i < cnt; i++)
+                    v[i] = std::ldexp(v[i], e[i]);
+                return v;
+            };
+            expect_same(p, {{"a", argument{sa, wide(sa.elements(), 90 + variant)}},
+                            {"b", argument{sb, wide(sb.elements(), 95 + variant)}}});
+        }
+    }
+}
+
 TEST_CASE(float_operators)
 {
     // the float operators around the GEMMs, one by one against the CPU target: exact where the
