@@ -20,6 +20,8 @@ struct bcast_params
     int op;
 };
 
+MI355_DEVINL float binary_apply(int op, float x, float y);
+
 __global__ __launch_bounds__(256) void binary_kernel(bcast_params p)
 {
     const int64_t step = (int64_t)gridDim.x * 256;
@@ -33,16 +35,63 @@ __global__ __launch_bounds__(256) void binary_kernel(bcast_params p)
             ao += c * p.a_strides[d];
             bo += c * p.b_strides[d];
         }
-        const float x = p.a[ao], y = p.b[bo];
-        float r;
-        switch(p.op)
+        p.out[i] = binary_apply(p.op, p.a[ao], p.b[bo]);
+    }
+}
+
+MI355_DEVINL float binary_apply(int op, float x, float y)
+{
+    switch(op)
+    {
+    case MI355_BIN_ADD: return x + y;
+    case MI355_BIN_SUB: return x - y;
+    case MI355_BIN_MUL: return x * y;
+    default: return x / y; // correctly rounded IEEE division
+    }
+}
+
+// The shapes that matter collapse to [rows, cols] with each operand either running along the
+// columns (column stride 1) or constant along them (column stride 0: a per-row value or a scalar):
+// activations against a bias row, a per-row statistic, another activation.  Four columns per
+// thread as one 16-byte access, rows by grid stride; no index division at all.
+struct binary2d_params
+{
+    const float* a;
+    const float* b;
+    float* out;
+    int64_t rows, cols;
+    int64_t a_sr, b_sr;
+    int a_sc, b_sc; // 0 or 1
+    int op;
+};
+
+__global__ __launch_bounds__(256) void binary2d_kernel(binary2d_params p)
+{
+    const int64_t c4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if(c4 >= p.cols)
+        return;
+    for(int64_t r = blockIdx.y; r < p.rows; r += gridDim.y)
+    {
+        v4f x, y;
+        if(p.a_sc)
+            x = *reinterpret_cast<const v4f*>(p.a + r * p.a_sr + c4);
+        else
         {
-        case MI355_BIN_ADD: r = x + y; break;
-        case MI355_BIN_SUB: r = x - y; break;
-        case MI355_BIN_MUL: r = x * y; break;
-        default: r = x / y; break; // correctly rounded IEEE division
+            const float s = p.a[r * p.a_sr];
+            x             = v4f{s, s, s, s};
         }
-        p.out[i] = r;
+        if(p.b_sc)
+            y = *reinterpret_cast<const v4f*>(p.b + r * p.b_sr + c4);
+        else
+        {
+            const float s = p.b[r * p.b_sr];
+            y             = v4f{s, s, s, s};
+        }
+        v4f o;
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+            o[e] = binary_apply(p.op, x[e], y[e]);
+        *reinterpret_cast<v4f*>(p.out + r * p.cols + c4) = o;
     }
 }
 
@@ -187,6 +236,51 @@ extern "C" int mi355_binary_f32(int32_t op,
     p.out  = out;
     p.ndim = ndim;
     p.op   = op;
+    // collapse to [rows, cols]: leading dimensions merge into one row index when, for both
+    // operands, each stride continues the next one (or both are broadcast there)
+    {
+        int last = ndim - 1;
+        while(last > 0 && lens[last] == 1)
+            last--;
+        const int64_t cols = lens[last];
+        int64_t rows       = 1;
+        int64_t a_sr = 0, b_sr = 0;
+        bool ok      = true;
+        bool first   = true;
+        for(int d = last - 1; d >= 0 && ok; d--)
+        {
+            if(lens[d] == 1)
+                continue;
+            if(first)
+            {
+                a_sr  = a_strides[d];
+                b_sr  = b_strides[d];
+                first = false;
+            }
+            else
+            {
+                ok = a_strides[d] == a_sr * rows && b_strides[d] == b_sr * rows;
+            }
+            rows *= lens[d];
+        }
+        const int64_t a_sc = cols == 1 ? 0 : a_strides[last];
+        const int64_t b_sc = cols == 1 ? 0 : b_strides[last];
+        auto vec_ok        = [&](const float* q, int64_t sr, int64_t sc) {
+            if(sc == 0)
+                return true;
+            return sc == 1 && sr % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0;
+        };
+        if(ok && cols % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && vec_ok(a, a_sr, a_sc) &&
+           vec_ok(b, b_sr, b_sc))
+        {
+            binary2d_params q{a, b, out, rows, cols, a_sr, b_sr, (int)a_sc, (int)b_sc, op};
+            const int64_t gx = (cols / 4 + 255) / 256;
+            const int64_t gy = rows < 65535 ? rows : 65535;
+            hipLaunchKernelGGL(binary2d_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0,
+                               static_cast<hipStream_t>(stream), q);
+            return mi355_launch_status();
+        }
+    }
     hipLaunchKernelGGL(binary_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
     return mi355_launch_status();
