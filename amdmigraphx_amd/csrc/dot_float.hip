@@ -293,6 +293,38 @@ __global__ __launch_bounds__(256) void gather_kernel(gather_params p)
     }
 }
 
+// The innermost dimension is contiguous in the input too (a permutation of the outer dimensions, a
+// slice): rows of `run` 16-byte pieces are copied whole; only the row index is decomposed, in 32-bit
+// arithmetic, once per piece.
+struct row_copy_params
+{
+    const uint8_t* in;
+    uint8_t* out;
+    uint32_t lens[MI355_MAX_DIMS]; // outer dimensions
+    int64_t strides[MI355_MAX_DIMS]; // their input strides in bytes
+    uint32_t rows, run;              // run = 16-byte pieces per row
+    int ndim;                        // number of outer dimensions
+};
+
+__global__ __launch_bounds__(256) void row_copy_kernel(row_copy_params p)
+{
+    const uint64_t total = (uint64_t)p.rows * p.run;
+    const uint64_t step  = (uint64_t)gridDim.x * 256;
+    for(uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step)
+    {
+        uint32_t row       = (uint32_t)(i / p.run);
+        const uint32_t pc  = (uint32_t)(i - (uint64_t)row * p.run);
+        int64_t off        = 0;
+        for(int d = p.ndim - 1; d >= 0; d--)
+        {
+            const uint32_t q = row / p.lens[d];
+            off += (int64_t)(row - q * p.lens[d]) * p.strides[d];
+            row = q;
+        }
+        reinterpret_cast<v4u*>(p.out)[i] = *reinterpret_cast<const v4u*>(p.in + off + (int64_t)pc * 16);
+    }
+}
+
 } // namespace
 
 extern "C" int mi355_dot(const void* a,
@@ -382,11 +414,44 @@ extern "C" int mi355_contiguous(const void* in,
     p.out       = static_cast<uint8_t*>(out);
     p.ndim      = ndim;
     p.elem_size = elem_size;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // last dimension contiguous in the input, rows a whole number of aligned 16-byte pieces
+    {
+        int last = ndim - 1;
+        while(last > 0 && lens[last] == 1)
+            last--;
+        const int64_t row_bytes = lens[last] * elem_size;
+        bool ok = strides[last] == 1 && row_bytes % 16 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(out) % 16 == 0 && p.total / lens[last] < (1ll << 31) &&
+                  row_bytes / 16 < (1ll << 31);
+        row_copy_params q{};
+        q.ndim = 0;
+        for(int d = 0; d < last && ok; d++)
+        {
+            if(lens[d] == 1)
+                continue;
+            ok = (strides[d] * elem_size) % 16 == 0 && lens[d] < (1ll << 31);
+            q.lens[q.ndim]    = (uint32_t)lens[d];
+            q.strides[q.ndim] = strides[d] * elem_size;
+            q.ndim++;
+        }
+        if(ok)
+        {
+            q.in   = p.in;
+            q.out  = p.out;
+            q.rows = (uint32_t)(p.total / lens[last]);
+            q.run  = (uint32_t)(row_bytes / 16);
+            int64_t nb = ((int64_t)q.rows * q.run + 255) / 256;
+            if(nb > 256 * 16)
+                nb = 256 * 16;
+            hipLaunchKernelGGL(row_copy_kernel, dim3((unsigned)nb), dim3(256), 0, s, q);
+            return mi355_launch_status();
+        }
+    }
     int64_t blocks = (p.total + 255) / 256;
     if(blocks > 256 * 16)
         blocks = 256 * 16;
     const dim3 grid((unsigned)blocks);
-    hipStream_t s = static_cast<hipStream_t>(stream);
     switch(elem_size)
     {
     case 1: hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, dim3(256), 0, s, p); break;

@@ -95,22 +95,37 @@ __global__ __launch_bounds__(256) void binary2d_kernel(binary2d_params p)
     }
 }
 
+MI355_DEVINL float unary_apply(int op, float x)
+{
+    switch(op)
+    {
+    case MI355_UN_ERF: return erff(x);
+    case MI355_UN_SQRT: return sqrtf(x); // correctly rounded (hipcc default)
+    case MI355_UN_RSQRT: return 1.0f / sqrtf(x); // 1 / std::sqrt(x), two IEEE operations
+    case MI355_UN_EXP: return expf(x);
+    case MI355_UN_TANH: return tanhf(x);
+    default: return -x;
+    }
+}
+
 __global__ __launch_bounds__(256) void unary_kernel(const float* in, float* out, int64_t n, int op)
 {
     const int64_t step = (int64_t)gridDim.x * 256;
     for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step)
+        out[i] = unary_apply(op, in[i]);
+}
+
+// n a multiple of 4, both pointers 16-byte aligned
+__global__ __launch_bounds__(256) void unary4_kernel(const v4f* in, v4f* out, int64_t n4, int op)
+{
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += step)
     {
-        const float x = in[i];
-        float r;
-        switch(op)
-        {
-        case MI355_UN_ERF: r = erff(x); break;
-        case MI355_UN_SQRT: r = sqrtf(x); break; // correctly rounded (hipcc default)
-        case MI355_UN_RSQRT: r = 1.0f / sqrtf(x); break; // 1 / std::sqrt(x), two IEEE operations
-        case MI355_UN_EXP: r = expf(x); break;
-        case MI355_UN_TANH: r = tanhf(x); break;
-        default: r = -x; break;
-        }
+        const v4f x = in[i];
+        v4f r;
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+            r[e] = unary_apply(op, x[e]);
         out[i] = r;
     }
 }
@@ -173,6 +188,51 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* in, float* ou
     s = wave_sum_f64(s);
     for(int64_t c = lane; c < cols; c += 64)
         y[c] = (float)((double)y[c] / s);
+}
+
+// The same arithmetic with the row held in registers (up to 64*NV columns): one read and one write
+// of the tensor instead of three and two.  A lane's elements are summed in the same order as above,
+// so the results are the same bits.
+template <int NV>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* in, float* out, int64_t rows, int64_t cols)
+{
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= rows)
+        return;
+    const float* x = in + row * cols;
+    float* y       = out + row * cols;
+    float v[NV];
+    double m = -1.7976931348623157e308;
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        const int64_t c = lane + 64 * i;
+        if(c < cols)
+        {
+            v[i] = x[c];
+            m    = fmax(m, (double)v[i]);
+        }
+    }
+    m        = wave_max_f64(m);
+    double s = 0.0;
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        if(lane + 64 * i < cols)
+        {
+            v[i] = (float)exp((double)v[i] - m);
+            s += (double)v[i];
+        }
+    }
+    s = wave_sum_f64(s);
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        const int64_t c = lane + 64 * i;
+        if(c < cols)
+            y[c] = (float)((double)v[i] / s);
+    }
 }
 
 // out[i, :] = table[ids[i], :]; negative indices count from the end (op/gather.hpp:100-118)
@@ -294,8 +354,12 @@ extern "C" int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t 
         return MI355_OK;
     if(in == nullptr || out == nullptr)
         return MI355_ERR_BAD_ARG;
-    hipLaunchKernelGGL(unary_kernel, dim3(blocks_for_n(n)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), in, out, n, op);
+    if(n % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0)
+        hipLaunchKernelGGL(unary4_kernel, dim3(blocks_for_n(n / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           reinterpret_cast<const v4f*>(in), reinterpret_cast<v4f*>(out), n / 4, op);
+    else
+        hipLaunchKernelGGL(unary_kernel, dim3(blocks_for_n(n)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), in, out, n, op);
     return mi355_launch_status();
 }
 
@@ -324,8 +388,16 @@ extern "C" int mi355_softmax_f32(const float* in, float* out, int64_t rows, int6
         return MI355_ERR_BAD_ARG;
     if((rows + 3) / 4 > 0x7fffffff)
         return MI355_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), in, out, rows, cols);
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if(cols <= 64 * 2)
+        hipLaunchKernelGGL(softmax_rows_kernel<2>, grid, dim3(256), 0, s, in, out, rows, cols);
+    else if(cols <= 64 * 8)
+        hipLaunchKernelGGL(softmax_rows_kernel<8>, grid, dim3(256), 0, s, in, out, rows, cols);
+    else if(cols <= 64 * 16)
+        hipLaunchKernelGGL(softmax_rows_kernel<16>, grid, dim3(256), 0, s, in, out, rows, cols);
+    else
+        hipLaunchKernelGGL(softmax_kernel, grid, dim3(256), 0, s, in, out, rows, cols);
     return mi355_launch_status();
 }
 
