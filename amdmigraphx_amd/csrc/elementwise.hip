@@ -130,6 +130,95 @@ __global__ __launch_bounds__(256) void unary4_kernel(const v4f* in, v4f* out, in
     }
 }
 
+// A chain of binary and unary operators over [rows, cols] in one pass.  W columns per thread
+// (4 as one 16-byte access, or 1), rows by grid stride.  The step list is uniform over the grid,
+// so the switch costs scalar branches only; every operation is the one the single-operator
+// kernels perform, and separate steps are never contracted into a fused multiply-add.
+struct chain_params
+{
+    const float* in[MI355_CHAIN_MAX_INPUTS];
+    int64_t sr[MI355_CHAIN_MAX_INPUTS];
+    int sc[MI355_CHAIN_MAX_INPUTS];
+    mi355_chain_step steps[MI355_CHAIN_MAX_STEPS];
+    float* out;
+    int64_t rows, cols;
+    int n_steps;
+};
+
+template <int W>
+__global__ __launch_bounds__(256) void chain_kernel(chain_params p)
+{
+#pragma clang fp contract(off)
+    const int64_t c0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * W;
+    if(c0 >= p.cols)
+        return;
+    for(int64_t r = blockIdx.y; r < p.rows; r += gridDim.y)
+    {
+        float acc[W], saved[W], operand[W];
+#pragma unroll
+        for(int e = 0; e < W; e++)
+            acc[e] = saved[e] = 0.0f;
+        auto fetch = [&](int i, float(&dst)[W]) __attribute__((always_inline)) {
+            const float* q = p.in[i] + r * p.sr[i];
+            if(p.sc[i] == 0)
+            {
+                const float s = q[0];
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                    dst[e] = s;
+            }
+            else if constexpr(W == 4)
+            {
+                const v4f v = *reinterpret_cast<const v4f*>(q + c0);
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                    dst[e] = v[e];
+            }
+            else
+            {
+                dst[0] = q[c0];
+            }
+        };
+        for(int s = 0; s < p.n_steps; s++)
+        {
+            const mi355_chain_step st = p.steps[s];
+            switch(st.kind)
+            {
+            case MI355_CH_LOAD: fetch(st.src, acc); break;
+            case MI355_CH_BINARY: {
+                if(st.src >= 0)
+                    fetch(st.src, operand);
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < W; e++)
+                        operand[e] = st.src == MI355_CH_SAVED ? saved[e] : acc[e];
+                }
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                    acc[e] = st.reversed ? binary_apply(st.op, operand[e], acc[e])
+                                         : binary_apply(st.op, acc[e], operand[e]);
+                break;
+            }
+            case MI355_CH_UNARY:
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                    acc[e] = unary_apply(st.op, acc[e]);
+                break;
+            default:
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                    saved[e] = acc[e];
+                break;
+            }
+        }
+        if constexpr(W == 4)
+            *reinterpret_cast<v4f*>(p.out + r * p.cols + c0) = v4f{acc[0], acc[1], acc[2], acc[3]};
+        else
+            p.out[r * p.cols + c0] = acc[0];
+    }
+}
+
 // sum of 64 doubles across a wave, every lane receives it; fixed pairing, so deterministic
 MI355_DEVINL double wave_sum_f64(double v)
 {
@@ -343,6 +432,75 @@ extern "C" int mi355_binary_f32(int32_t op,
     }
     hipLaunchKernelGGL(binary_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
+                               int32_t n_steps,
+                               const float* const* inputs,
+                               const int64_t* row_strides,
+                               const int32_t* col_strides,
+                               int32_t n_inputs,
+                               float* out,
+                               int64_t rows,
+                               int64_t cols,
+                               void* stream)
+{
+    if(steps == nullptr || n_steps < 1 || n_steps > MI355_CHAIN_MAX_STEPS || n_inputs < 1 ||
+       n_inputs > MI355_CHAIN_MAX_INPUTS || inputs == nullptr || row_strides == nullptr ||
+       col_strides == nullptr || rows < 0 || cols < 0)
+        return MI355_ERR_BAD_ARG;
+    if(steps[0].kind != MI355_CH_LOAD)
+        return MI355_ERR_BAD_ARG;
+    chain_params p{};
+    for(int s = 0; s < n_steps; s++)
+    {
+        const mi355_chain_step& st = steps[s];
+        switch(st.kind)
+        {
+        case MI355_CH_LOAD:
+            if(st.src < 0 || st.src >= n_inputs)
+                return MI355_ERR_BAD_ARG;
+            break;
+        case MI355_CH_BINARY:
+            if(st.op < MI355_BIN_ADD || st.op > MI355_BIN_DIV || st.src >= n_inputs || st.src < MI355_CH_SELF)
+                return MI355_ERR_BAD_ARG;
+            break;
+        case MI355_CH_UNARY:
+            if(st.op < MI355_UN_ERF || st.op > MI355_UN_NEG)
+                return MI355_ERR_BAD_ARG;
+            break;
+        case MI355_CH_SAVE: break;
+        default: return MI355_ERR_BAD_ARG;
+        }
+        p.steps[s] = st;
+    }
+    if(rows == 0 || cols == 0)
+        return MI355_OK;
+    if(out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    bool vec = cols % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    for(int i = 0; i < n_inputs; i++)
+    {
+        if(inputs[i] == nullptr || row_strides[i] < 0 || (col_strides[i] != 0 && col_strides[i] != 1))
+            return MI355_ERR_BAD_ARG;
+        p.in[i] = inputs[i];
+        p.sr[i] = row_strides[i];
+        p.sc[i] = cols == 1 ? 0 : col_strides[i];
+        if(p.sc[i] == 1 && (row_strides[i] % 4 != 0 || reinterpret_cast<uintptr_t>(inputs[i]) % 16 != 0))
+            vec = false;
+    }
+    p.out     = out;
+    p.rows    = rows;
+    p.cols    = cols;
+    p.n_steps = n_steps;
+    const int64_t gy = rows < 65535 ? rows : 65535;
+    if(vec)
+        hipLaunchKernelGGL(chain_kernel<4>, dim3((unsigned)((cols / 4 + 255) / 256), (unsigned)gy), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), p);
+    else
+        hipLaunchKernelGGL(chain_kernel<1>, dim3((unsigned)((cols + 255) / 256), (unsigned)gy), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), p);
     return mi355_launch_status();
 }
 

@@ -36,6 +36,7 @@ argument from_device(const argument& device);
 // Replace the operators of the quantized-GEMM path by operators that call the kernel library:
 //   quant_dot -> dequantizelinear [-> convert]           one fused mi355::quant_dot
 //   dot(x, transpose(dequantizelinear(unpack_int4 ...)))   mi355::w4a16_gemm (MatMulNBits layout)
+//   chains of add / sub / mul / div / erf / sqrt / ...     one mi355::chain (fuse_pointwise)
 //   quant_dot, dot, quantizelinear, dequantizelinear, unpack_int4, pack_int4, convert, contiguous
 //                                                          the mi355:: operator of the same name
 // Literals move to device memory, constant subgraphs are evaluated once at compile time, and with
@@ -45,6 +46,7 @@ struct lowering
 {
     context* ctx      = nullptr;
     bool offload_copy = false;
+    bool fuse_pointwise = true;
     std::string name() const { return "mi355::lowering"; }
     void apply(module& m) const;
 };

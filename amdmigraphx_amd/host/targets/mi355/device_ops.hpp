@@ -248,6 +248,24 @@ struct unary
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// A chain of binary and unary float operators evaluated element by element in one kernel.
+// inputs: x0 .. x(n-1) (views of the output's dimensions whose strides collapse to a row stride
+// and a column stride of 0 or 1), out.  `steps` holds kind, op, src, reversed for every step of
+// the register machine mi355_chain_f32 describes.
+struct chain
+{
+    std::vector<int64_t> steps;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.steps, "steps");
+    }
+    std::string name() const { return "mi355::chain"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: x (standard), out; over the last axis
 struct reduce_mean
 {

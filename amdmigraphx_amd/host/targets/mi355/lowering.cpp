@@ -386,6 +386,198 @@ bool lower_w4a16(module& m, instruction_ref ins)
     return true;
 }
 
+// ---- chains of float pointwise operators ------------------------------------------------------
+//
+// add / sub / mul / div and the unary functions that feed one another through single-use values
+// become one mi355::chain, which keeps the intermediate values in registers.  The reference
+// groups such operators into pointwise modules (src/fuse_pointwise.cpp:364-385) and compiles
+// each module; here the group is restricted to what a machine with the running value and one
+// saved value can evaluate, which covers the encoder's GELU, bias + residual and the
+// scale-and-shift tail of layer normalisation.  The steps repeat the operators in their own
+// order, so the fused result equals the unfused one bit for bit.
+
+int binary_code(const std::string& name)
+{
+    if(name == "add")
+        return MI355_BIN_ADD;
+    if(name == "sub")
+        return MI355_BIN_SUB;
+    if(name == "mul")
+        return MI355_BIN_MUL;
+    if(name == "div")
+        return MI355_BIN_DIV;
+    return -1;
+}
+
+int unary_code(const std::string& name)
+{
+    if(name == "erf")
+        return MI355_UN_ERF;
+    if(name == "sqrt")
+        return MI355_UN_SQRT;
+    if(name == "rsqrt")
+        return MI355_UN_RSQRT;
+    if(name == "exp")
+        return MI355_UN_EXP;
+    if(name == "tanh")
+        return MI355_UN_TANH;
+    if(name == "neg")
+        return MI355_UN_NEG;
+    return -1;
+}
+
+struct chain_builder
+{
+    instruction_ref sink;
+    int max_depth = 0;
+    std::vector<instruction_ref> externals;
+    std::vector<instruction_ref> absorbed;
+    std::vector<int64_t> steps;
+    bool save_live = false;
+    bool failed    = false;
+
+    bool fusable(instruction_ref x) const
+    {
+        if(binary_code(x->name()) < 0 and unary_code(x->name()) < 0)
+            return false;
+        if(x->get_shape().type() != shape::float_type or x->get_shape().lens() != sink->get_shape().lens())
+            return false;
+        return std::all_of(x->inputs().begin(), x->inputs().end(), [&](instruction_ref i) {
+            return i->get_shape().type() == shape::float_type and
+                   i->get_shape().lens() == sink->get_shape().lens();
+        });
+    }
+
+    bool inlined(instruction_ref x, int depth) const
+    {
+        return depth <= max_depth and x->outputs().size() == 1 and fusable(x);
+    }
+
+    void push(int kind, int op, int src, int reversed)
+    {
+        if(steps.size() / 4 >= MI355_CHAIN_MAX_STEPS)
+        {
+            failed = true;
+            return;
+        }
+        steps.insert(steps.end(), {kind, op, src, reversed});
+    }
+
+    int external(instruction_ref x)
+    {
+        auto it = std::find(externals.begin(), externals.end(), x);
+        if(it != externals.end())
+            return static_cast<int>(it - externals.begin());
+        int64_t sr = 0;
+        int64_t sc = 0;
+        if(externals.size() >= MI355_CHAIN_MAX_INPUTS or not collapse_2d(x->get_shape(), sr, sc) or
+           (sc != 0 and sc != 1))
+        {
+            failed = true;
+            return 0;
+        }
+        externals.push_back(x);
+        return static_cast<int>(externals.size() - 1);
+    }
+
+    // leaves the value of x in the running register
+    void value(instruction_ref x, int depth)
+    {
+        if(inlined(x, depth))
+            emit(x, depth);
+        else
+            push(MI355_CH_LOAD, 0, external(x), 0);
+    }
+
+    void emit(instruction_ref x, int depth)
+    {
+        if(failed)
+            return;
+        if(x != sink)
+            absorbed.push_back(x);
+        const int un = unary_code(x->name());
+        if(un >= 0)
+        {
+            value(x->inputs()[0], depth + 1);
+            push(MI355_CH_UNARY, un, 0, 0);
+            return;
+        }
+        const int bin = binary_code(x->name());
+        auto a        = x->inputs()[0];
+        auto b        = x->inputs()[1];
+        if(a == b)
+        {
+            value(a, depth + 1);
+            push(MI355_CH_BINARY, bin, MI355_CH_SELF, 0);
+            return;
+        }
+        const bool ia = inlined(a, depth + 1);
+        const bool ib = inlined(b, depth + 1);
+        if(ia and ib and not save_live)
+        {
+            emit(a, depth + 1);
+            push(MI355_CH_SAVE, 0, 0, 0);
+            save_live = true;
+            emit(b, depth + 1);
+            save_live = false;
+            push(MI355_CH_BINARY, bin, MI355_CH_SAVED, 1);
+        }
+        else if(ia)
+        {
+            emit(a, depth + 1);
+            push(MI355_CH_BINARY, bin, external(b), 0);
+        }
+        else if(ib)
+        {
+            emit(b, depth + 1);
+            push(MI355_CH_BINARY, bin, external(a), 1);
+        }
+        else
+        {
+            push(MI355_CH_LOAD, 0, external(a), 0);
+            push(MI355_CH_BINARY, bin, external(b), 0);
+        }
+    }
+};
+
+void fuse_chains(module& m)
+{
+    std::unordered_set<const instruction*> taken;
+    auto order = all_instructions(m);
+    for(auto it = order.rbegin(); it != order.rend(); ++it)
+    {
+        auto ins = *it;
+        if(taken.count(&*ins) > 0)
+            continue;
+        if(binary_code(ins->name()) < 0 and unary_code(ins->name()) < 0)
+            continue;
+        // rows of fewer than four columns gain nothing from the row-wise kernel
+        if(ins->get_shape().ndim() == 0 or ins->get_shape().lens().back() < 4)
+            continue;
+        for(int depth : {MI355_CHAIN_MAX_STEPS, 6, 3, 1})
+        {
+            chain_builder cb;
+            cb.sink      = ins;
+            cb.max_depth = depth;
+            if(not cb.fusable(ins))
+                break;
+            cb.emit(ins, 0);
+            if(cb.failed)
+                continue;
+            if(cb.absorbed.empty())
+                break;
+            for(auto a : cb.absorbed)
+                taken.insert(&*a);
+            auto args = cb.externals;
+            args.push_back(insert_allocation(m, ins, shape{shape::float_type, ins->get_shape().lens()}));
+            chain op;
+            op.steps = cb.steps;
+            m.replace_instruction(ins, operation{op}, args);
+            break;
+        }
+    }
+}
+
 // ---- one operator at a time ------------------------------------------------------------------
 
 void lower_instruction(module& m, instruction_ref ins)
@@ -633,6 +825,11 @@ void lowering::apply(module& m) const
             fuse_quant_dot_dq(m, ins);
     }
     dead_code_elimination{}.apply(m);
+    if(fuse_pointwise)
+    {
+        fuse_chains(m);
+        dead_code_elimination{}.apply(m);
+    }
     // 2. everything else, one operator at a time
     for(auto ins : all_instructions(m))
         lower_instruction(m, ins);

@@ -2,6 +2,7 @@
 #include <migraphx/ops.hpp>
 #include <migraphx/passes.hpp>
 #include <migraphx/register_op.hpp>
+#include <cstdlib>
 #include <migraphx/register_target.hpp>
 #include <hip/hip_runtime_api.h>
 #include <algorithm>
@@ -788,6 +789,70 @@ argument unary::compute(migraphx::context& ctx, const shape& out, const std::vec
     return args[1];
 }
 
+shape chain::compute_shape(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() < 2 or inputs.size() > MI355_CHAIN_MAX_INPUTS + 1)
+        MIGRAPHX_THROW("mi355::chain: between 1 and " + std::to_string(MI355_CHAIN_MAX_INPUTS) +
+                       " inputs and the output buffer expected");
+    if(steps.empty() or steps.size() % 4 != 0 or steps.size() / 4 > MI355_CHAIN_MAX_STEPS)
+        MIGRAPHX_THROW("mi355::chain: malformed step list");
+    const shape& out = inputs.back();
+    if(out.type() != shape::float_type or not out.standard())
+        MIGRAPHX_THROW("mi355::chain: the output buffer must be a dense float tensor");
+    for(std::size_t i = 0; i + 1 < inputs.size(); i++)
+    {
+        int64_t sr = 0;
+        int64_t sc = 0;
+        if(inputs[i].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::chain: float tensors only, got " + inputs[i].type_string());
+        if(inputs[i].lens() != out.lens())
+            MIGRAPHX_THROW("mi355::chain: Dimensions do not match");
+        if(not collapse_2d(inputs[i], sr, sc) or (sc != 0 and sc != 1))
+            MIGRAPHX_THROW("mi355::chain: input strides do not collapse to rows and columns");
+    }
+    return out;
+}
+
+argument chain::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const std::size_t n = args.size() - 1;
+    std::vector<mi355_chain_step> st(steps.size() / 4);
+    for(std::size_t i = 0; i < st.size(); i++)
+    {
+        st[i].kind     = static_cast<int32_t>(steps[4 * i]);
+        st[i].op       = static_cast<int32_t>(steps[4 * i + 1]);
+        st[i].src      = static_cast<int32_t>(steps[4 * i + 2]);
+        st[i].reversed = static_cast<int32_t>(steps[4 * i + 3]);
+    }
+    std::vector<const float*> ptrs(n);
+    std::vector<int64_t> sr(n);
+    std::vector<int32_t> sc(n);
+    for(std::size_t i = 0; i < n; i++)
+    {
+        int64_t r = 0;
+        int64_t c = 0;
+        collapse_2d(args[i].get_shape(), r, c);
+        ptrs[i] = reinterpret_cast<const float*>(args[i].data());
+        sr[i]   = r;
+        sc[i]   = static_cast<int32_t>(c);
+    }
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(out, rows, cols);
+    status_check(mi355_chain_f32(st.data(),
+                                 static_cast<int32_t>(st.size()),
+                                 ptrs.data(),
+                                 sr.data(),
+                                 sc.data(),
+                                 static_cast<int32_t>(n),
+                                 reinterpret_cast<float*>(args[n].data()),
+                                 rows,
+                                 cols,
+                                 stream_of(ctx)),
+                 name());
+    return args[n];
+}
+
 shape reduce_mean::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -880,10 +945,11 @@ std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_opti
     // gpu target switches it (src/targets/gpu/target.cpp:129)
     simplify_qdq sq;
     sq.use_mx_quant = true;
-    return {sq,
-            dead_code_elimination{},
-            lowering{&ctx, options.offload_copy},
-            dead_code_elimination{}};
+    lowering low{&ctx, options.offload_copy};
+    // the reference's switch for its pointwise fusion (src/fuse_pointwise.cpp:39,369)
+    if(const char* off = std::getenv("MIGRAPHX_DISABLE_POINTWISE_FUSION"))
+        low.fuse_pointwise = std::string(off).empty() or std::string(off) == "0";
+    return {sq, dead_code_elimination{}, low, dead_code_elimination{}};
 }
 
 } // namespace mi355
@@ -899,6 +965,7 @@ MIGRAPHX_REGISTER_OP(mi355::dot);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
 MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);
+MIGRAPHX_REGISTER_OP(mi355::chain);
 MIGRAPHX_REGISTER_OP(mi355::unpack_int4);
 MIGRAPHX_REGISTER_OP(mi355::unpack_fp4);
 MIGRAPHX_REGISTER_OP(mi355::pack_fp4);

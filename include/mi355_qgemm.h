@@ -278,6 +278,38 @@ int mi355_softmax_f32(const float* in, float* out, int64_t rows, int64_t cols, v
 int mi355_gather_rows(const void* table, const void* ids, int32_t ids_are_int64, void* out,
                       int64_t n_ids, int64_t table_rows, int64_t row_bytes, void* stream);
 
+/* A chain of the float operators above applied element by element in one pass over a dense
+ * [rows, cols] result, so that the intermediate tensors of e.g. GELU (mul, erf, add, mul, mul) or
+ * bias + residual never reach memory.  It is the device counterpart of one fused pointwise module
+ * (src/fuse_pointwise.cpp:364-385 builds them for the reference's targets, which then compile each module;
+ * here nothing is compiled at run time).  Each element runs a small register machine with the running
+ * value and one saved value; every step is the same IEEE float operation the single operators
+ * perform, in the order the steps list them, so the result equals the unfused sequence bit for bit.
+ *   MI355_CH_LOAD    value = input[src]
+ *   MI355_CH_BINARY  value = value (op) operand, or operand (op) value when `reversed`;
+ *                    operand = input[src] for src >= 0, the saved value for MI355_CH_SAVED,
+ *                    the running value itself for MI355_CH_SELF
+ *   MI355_CH_UNARY   value = op(value)
+ *   MI355_CH_SAVE    saved = value
+ * Input i is addressed as inputs[i][row * row_strides[i] + col * col_strides[i]] with a column
+ * stride of 0 (constant along the row) or 1.  The first step must be a LOAD.  All arrays are HOST
+ * arrays; at most MI355_CHAIN_MAX_STEPS steps and MI355_CHAIN_MAX_INPUTS inputs. */
+typedef enum mi355_chain_kind { MI355_CH_LOAD = 0, MI355_CH_BINARY = 1, MI355_CH_UNARY = 2, MI355_CH_SAVE = 3 } mi355_chain_kind;
+#define MI355_CH_SAVED (-1)
+#define MI355_CH_SELF (-2)
+#define MI355_CHAIN_MAX_STEPS 24
+#define MI355_CHAIN_MAX_INPUTS 8
+typedef struct mi355_chain_step
+{
+    int32_t kind;     /* mi355_chain_kind */
+    int32_t op;       /* mi355_binary_op or mi355_unary_op; unused for LOAD and SAVE */
+    int32_t src;      /* LOAD: input index; BINARY: input index, MI355_CH_SAVED or MI355_CH_SELF */
+    int32_t reversed; /* BINARY only */
+} mi355_chain_step;
+int mi355_chain_f32(const mi355_chain_step* steps, int32_t n_steps, const float* const* inputs,
+                    const int64_t* row_strides, const int32_t* col_strides, int32_t n_inputs,
+                    float* out, int64_t rows, int64_t cols, void* stream);
+
 /* Human-readable text for a status code (static storage). */
 const char* mi355_status_string(int status);
 

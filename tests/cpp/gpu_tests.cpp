@@ -8,6 +8,7 @@
 #include "oracle_target.hpp"
 #include "test.hpp"
 #include <chrono>
+#include <cstdlib>
 #include <fstream>
 #include <thread>
 
@@ -670,6 +671,129 @@ TEST_CASE(float_operators)
     mm->add_return({mm->add_instruction(make_op("gather", {{"axis", 0}}), t, i)});
     argument ia{shape{shape::int32_type, {7}}, std::vector<int>{0, 49, 3, 3, -1, 17, -50}};
     expect_same(p, {{"i", ia}});
+}
+
+TEST_CASE(pointwise_chains)
+{
+    // Chains of float operators become one mi355::chain each.  With IEEE-exact operators the fused
+    // program must equal the CPU target bit for bit; with erf in the chain it must equal the
+    // unfused mi355 program bit for bit (same device functions, same order) and the CPU target
+    // within the math library's few units in the last place.
+    using builder = std::function<instruction_ref(module&, instruction_ref, instruction_ref, instruction_ref)>;
+    struct counts
+    {
+        std::size_t chains, singles;
+    };
+    auto run = [&](std::size_t r, std::size_t c, const builder& f, bool exact, counts expected) {
+        static int case_no = 0;
+        case_no++;
+        program p;
+        auto* mm = p.get_main_module();
+        shape s{shape::float_type, {r, c}};
+        auto x = mm->add_parameter("x", s);
+        auto y = mm->add_parameter("y", s);
+        auto v = mm->add_parameter("v", shape{shape::float_type, {c}});
+        mm->add_return({f(*mm, x, y, v)});
+        migraphx::parameter_map params{{"x", argument{s, normal_floats(r * c, 2.0f, 300 + case_no)}},
+                                       {"y", argument{s, uniform_floats(r * c, 0.5f, 3.0f, 400 + case_no)}},
+                                       {"v", argument{shape{shape::float_type, {c}}, uniform_floats(c, 0.5f, 2.0f, 500 + case_no)}}};
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        const auto chains  = count_ops(*compiled.get_main_module(), "mi355::chain");
+        const auto singles = count_ops(*compiled.get_main_module(), "mi355::binary") +
+                             count_ops(*compiled.get_main_module(), "mi355::unary");
+        if(chains != expected.chains or singles != expected.singles)
+            std::cout << "chain case " << case_no << ": " << chains << " chains, " << singles << " single operators"
+                      << std::endl;
+        EXPECT(chains == expected.chains);
+        EXPECT(singles == expected.singles);
+        auto got = run_on("mi355", p, params);
+        setenv("MIGRAPHX_DISABLE_POINTWISE_FUSION", "1", 1);
+        program plain = p;
+        plain.compile(migraphx::make_target("mi355"));
+        auto unfused = run_on("mi355", p, params);
+        unsetenv("MIGRAPHX_DISABLE_POINTWISE_FUSION");
+        EXPECT(not has_op(plain, "mi355::chain"));
+        EXPECT(same_bytes(got[0], unfused[0]));
+        auto want = run_on("oracle", p, params);
+        if(exact)
+        {
+            if(not same_bytes(got[0], want[0]))
+                std::cout << "chain case " << case_no << " differs from the CPU target, max rel diff "
+                          << max_rel_diff(got[0], want[0], 1e-30) << std::endl;
+            EXPECT(same_bytes(got[0], want[0]));
+        }
+        else
+        {
+            // 1 + erf(x) cancels for negative x, so small results carry the math library's
+            // absolute error: relative to max(|expected|, 0.25)
+            if(not(max_rel_diff(got[0], want[0], 0.25) < 4e-6))
+                std::cout << "chain case " << case_no << ": max rel diff " << max_rel_diff(got[0], want[0], 0.25)
+                          << std::endl;
+            EXPECT(max_rel_diff(got[0], want[0], 0.25) < 4e-6);
+        }
+    };
+    auto op = [](module& m, const std::string& name, auto... args) { return m.add_instruction(make_op(name), args...); };
+    auto bcast = [](module& m, instruction_ref v, instruction_ref like) {
+        return m.add_instruction(make_op("multibroadcast", {{"out_lens", like->get_shape().lens()}}), v);
+    };
+    // bias + residual
+    run(33, 200, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref v) {
+        return op(m, "add", op(m, "add", x, bcast(m, v, x)), y);
+    }, true, {1, 0});
+    // the tail of layer normalisation: (x / sigma) * gamma + beta with a per-row sigma
+    run(33, 200, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref v) {
+        auto var   = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), op(m, "mul", y, y));
+        auto sigma = bcast(m, op(m, "sqrt", var), x);
+        return op(m, "add", op(m, "mul", op(m, "div", x, sigma), bcast(m, v, x)), bcast(m, v, x));
+    }, false, {1, 2});
+    // an operand used on both sides, and the reversed forms of sub and div
+    run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        auto sq = op(m, "mul", x, x);
+        return op(m, "div", y, op(m, "sub", y, op(m, "neg", sq)));
+    }, true, {1, 0});
+    // two computed operands: the first is saved while the second is evaluated
+    run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        return op(m, "div", op(m, "add", x, y), op(m, "sqrt", op(m, "add", y, y)));
+    }, true, {1, 0});
+    run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        return op(m, "sub", op(m, "mul", x, y), op(m, "div", x, y));
+    }, true, {1, 0});
+    // a third computed operand while one is saved stays a kernel of its own
+    run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref v) {
+        auto inner = op(m, "div", op(m, "sub", x, y), op(m, "add", y, bcast(m, v, y)));
+        return op(m, "mul", op(m, "add", x, y), inner);
+    }, true, {1, 1});
+    // longer than one chain may be: split into several
+    run(8, 128, [&](module& m, instruction_ref, instruction_ref y, instruction_ref) {
+        auto t = y;
+        for(int i = 0; i < 20; i++)
+            t = op(m, "sqrt", op(m, "add", t, y));
+        return t;
+    }, true, {4, 0}); // 7 + 7 + 7 + 19 operators
+    // an operand whose strides do not reduce to rows and columns keeps the general kernel
+    run(64, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        auto xt = m.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), x);
+        return op(m, "mul", op(m, "add", xt, y), y);
+    }, true, {0, 2});
+    // a row length that is no multiple of four, and a view that starts off a 16-byte boundary
+    run(9, 203, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        return op(m, "mul", op(m, "sub", x, y), y);
+    }, true, {1, 0});
+    run(9, 204, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        auto xs = m.add_instruction(make_op("slice", {{"axes", {1}}, {"starts", {1}}, {"ends", {201}}}), x);
+        auto ys = m.add_instruction(make_op("slice", {{"axes", {1}}, {"starts", {4}}, {"ends", {204}}}), y);
+        return op(m, "mul", op(m, "sub", xs, ys), ys);
+    }, true, {1, 0});
+    // GELU as the exporters write it: x * 0.5 * (1 + erf(x / sqrt 2)) after a bias
+    run(33, 200, [&](module& m, instruction_ref x, instruction_ref, instruction_ref v) {
+        auto constant = [&](float c) {
+            return bcast(m, m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{c}}), x);
+        };
+        auto h = op(m, "add", x, bcast(m, v, x));
+        auto e = op(m, "add", op(m, "erf", op(m, "mul", h, constant(0.70710678f))), constant(1.0f));
+        return op(m, "mul", op(m, "mul", h, constant(0.5f)), e);
+    }, false, {1, 1});
 }
 
 // agreement of two float tensors as the reference's verify does it (verify.hpp:175-195): root mean
