@@ -36,6 +36,7 @@ class QuantDotDesc(ctypes.Structure):
 
 EXPORTS = {
     "mi355_quant_dot": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 8,
+    "mi355_quant_dot_bias": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9,
     "mi355_colsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                         ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p],
     "mi355_rowsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,

@@ -120,6 +120,15 @@ MI355_DEVINL uint16_t convert_f32_to_bf16(float x)
     return f32_to_bf16_rtz(x);
 }
 
+// The `add` of a bias behind dequantizelinear: its own fp32 rounding, never contracted with the
+// multiplication in front of it.  b = -0.0f leaves every value (signed zeros and NaN included) as
+// it is, which is how "no bias" is passed.
+MI355_DEVINL float add_bias(float v, float b)
+{
+#pragma clang fp contract(off)
+    return v + b;
+}
+
 // Typed loads as double / stores from double, mirroring
 // static_cast<double>(view[i]) and view[i] = d on the ref target.
 MI355_DEVINL double load_as_f64(const void* p, int type, int64_t i)

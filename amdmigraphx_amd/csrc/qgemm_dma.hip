@@ -54,6 +54,7 @@ struct dma_params
     const float* scale_b;
     const int32_t* colsum_b;
     const int32_t* rowsum_a;
+    const float* bias; // [N], added after the dequantization; null = none
     int scale_a_mode, scale_b_mode;
     int zp_a, zp_b;
     int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
@@ -478,6 +479,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     int64_t zrow_r[4] = {0, 0, 0, 0};
     float sb_c[2][4][4];
     int32_t cs_c[2][4][4];
+    float bias_c[2][4][4];
     if constexpr(DEQ)
     {
 #pragma unroll
@@ -506,8 +508,18 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                         sb = p.scale_b[c];
                     sb_c[j][g][e] = sb;
                     cs_c[j][g][e] = (!FP8 && p.zp_a != 0) ? p.colsum_b[c] : 0;
+                    if constexpr(FP8)
+                        bias_c[j][g][e] = p.bias != nullptr ? p.bias[c] : -0.0f;
                 }
     }
+    // the int8 form of this kernel has no registers left for a bias: the launcher never sends
+    // one here (only matrices whose N is no multiple of 4 come here with int8)
+    auto bias_of = [&](int j, int g, int e) __attribute__((always_inline)) {
+        if constexpr(FP8)
+            return bias_c[j][g][e];
+        else
+            return -0.0f;
+    };
 #pragma unroll
     for(int i = 0; i < 4; i++)
     {
@@ -549,6 +561,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                                         (double)acc[i][j][4 * (gp + h) + e] - (double)(int32_t)zp;
                                     v = (float)(d * (double)s);
                                 }
+                                v    = add_bias(v, bias_of(j, gp + h, e));
                                 q[e] = OUT == MI355_F16 ? convert_f32_to_half(v) : convert_f32_to_bf16(v);
                             }
                             pk[h][0] = q[0] | ((uint32_t)q[1] << 16);
@@ -598,6 +611,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                             const double d   = (double)acc[i][j][4 * g + e] - (double)(int32_t)zp;
                             v[e]             = (float)(d * (double)s);
                         }
+                        v[e] = add_bias(v[e], bias_of(j, g, e));
                     }
                 }
                 if constexpr(!DEQ)
@@ -937,6 +951,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     // store to C cannot move in front of it, and its latency would be paid once per group).
     float sb_c[4][4];
     int32_t cs_c[4][4];
+    float bias_c[4][4];
     float sa_r[8];
     int64_t zrow_r[8];
     if constexpr(DEQ)
@@ -954,6 +969,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                     sb = p.scale_b[c];
                 sb_c[j][e] = sb;
                 cs_c[j][e] = p.zp_a != 0 ? p.colsum_b[c] : 0;
+                bias_c[j][e] = p.bias != nullptr ? p.bias[c] : -0.0f;
             }
 #pragma unroll
         for(int i = 0; i < 8; i++)
@@ -1012,7 +1028,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                     const float s  = sa_r[i] * sb_c[j][e];
                     const double d = (double)acc[i][j][e] -
                                      (double)(int32_t)(zrow_r[i] + (int64_t)p.zp_a * cs_c[j][e]);
-                    v[e] = (float)(d * (double)s);
+                    v[e] = add_bias((float)(d * (double)s), bias_c[j][e]);
                 }
                 if constexpr(VEC_STORE)
                 {
@@ -1174,9 +1190,11 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                           const float* scale_b,
                           const int32_t* colsum_b,
                           const int32_t* rowsum_a,
+                          const float* bias,
                           hipStream_t stream)
 {
     dma_params p;
+    p.bias         = bias;
     p.a            = static_cast<const uint8_t*>(a);
     p.b            = static_cast<const uint8_t*>(b);
     p.c            = c;

@@ -46,6 +46,7 @@ struct gemm_params
     int tiles_m, tiles_n;
     const float* scale_a;
     const float* scale_b;
+    const float* bias; // [N], added after the dequantization; null = none
     const int32_t* colsum_b;
     const int32_t* rowsum_a;
     int scale_a_mode, scale_b_mode;
@@ -383,6 +384,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
         return;
     float sb[4]  = {1.f, 1.f, 1.f, 1.f};
     int32_t cs[4] = {0, 0, 0, 0};
+    float bias[4] = {-0.0f, -0.0f, -0.0f, -0.0f};
     if constexpr(DEQ)
     {
 #pragma unroll
@@ -394,6 +396,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
                 sb[j] = p.scale_b[col + j];
             if(p.zp_a != 0)
                 cs[j] = p.colsum_b[col + j];
+            if(p.bias != nullptr)
+                bias[j] = p.bias[col + j];
         }
     }
     uint8_t* cbase = static_cast<uint8_t*>(p.c);
@@ -448,7 +452,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
                     else
                         d = (double)acc[i][j][r] -
                             (double)(int32_t)(zrow + (int64_t)p.zp_a * cs[j]);
-                    v[j] = (float)(d * (double)s);
+                    v[j] = add_bias((float)(d * (double)s), bias[j]);
                 }
                 store4<OUT>(p.c, idx, v);
             }
@@ -542,9 +546,11 @@ int mi355_mfma_gemm_launch(const mi355_quant_dot_desc* d,
                            const float* scale_b,
                            const int32_t* colsum_b,
                            const int32_t* rowsum_a,
+                           const float* bias,
                            hipStream_t stream)
 {
     gemm_params p;
+    p.bias         = bias;
     p.a            = static_cast<const uint8_t*>(a);
     p.b            = static_cast<const uint8_t*>(b);
     p.c            = c;

@@ -12,6 +12,7 @@ int mi355_mfma_gemm_launch(const mi355_quant_dot_desc*,
                            const float*,
                            const int32_t*,
                            const int32_t*,
+                           const float*,
                            hipStream_t);
 bool mi355_dma_gemm_supported(const mi355_quant_dot_desc*, const void*, const void*);
 int mi355_dma_gemm_launch(const mi355_quant_dot_desc*,
@@ -22,6 +23,7 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc*,
                           const float*,
                           const int32_t*,
                           const int32_t*,
+                          const float*,
                           hipStream_t);
 
 namespace {
@@ -38,6 +40,7 @@ struct generic_params
     const float* scale_b;
     const int32_t* colsum_b;
     const int32_t* rowsum_a;
+    const float* bias;
     int scale_a_mode, scale_b_mode, zp_a, zp_b;
     int fp8, dequant, out_type;
     int is_unsigned; // uint8 operands (bare quant_dot only)
@@ -129,7 +132,9 @@ __global__ __launch_bounds__(256) void quant_dot_generic_kernel(generic_params p
             zp -= p.k * (int64_t)p.zp_a * p.zp_b;
         d = (double)iacc - (double)(int32_t)zp;
     }
-    const float v = (float)(d * (double)s);
+    float v = (float)(d * (double)s);
+    if(p.bias != nullptr)
+        v = add_bias(v, p.bias[col]);
     switch(p.out_type)
     {
     case MI355_F32: static_cast<float*>(p.c)[idx] = v; break;
@@ -195,6 +200,20 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
                                const int32_t* rowsum_a,
                                void* stream)
 {
+    return mi355_quant_dot_bias(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, nullptr, stream);
+}
+
+extern "C" int mi355_quant_dot_bias(const mi355_quant_dot_desc* d,
+                                    const void* a,
+                                    const void* b,
+                                    void* c,
+                                    const float* scale_a,
+                                    const float* scale_b,
+                                    const int32_t* colsum_b,
+                                    const int32_t* rowsum_a,
+                                    const float* bias,
+                                    void* stream)
+{
     if(d == nullptr)
         return MI355_ERR_BAD_ARG;
     if(d->m < 0 || d->n < 0 || d->k < 0 || d->batch < 0)
@@ -209,6 +228,8 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
     const bool u8 = d->in_type == MI355_U8;
     if(u8 && d->dequant)
         return MI355_ERR_UNSUPPORTED;
+    if(bias != nullptr && !d->dequant)
+        return MI355_ERR_BAD_ARG; // the bias is a float added to the dequantized value
     if(d->dequant)
     {
         if(d->out_type != MI355_F32 && d->out_type != MI355_F16 && d->out_type != MI355_BF16)
@@ -249,10 +270,12 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
         return MI355_ERR_UNSUPPORTED;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if(!u8 && d->k > 0 && mi355_dma_gemm_supported(d, a, b))
-        return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
+    // int8 with N % 4 != 0 would take the DMA path's 32 x 32 kernel, which applies no bias
+    const bool dma_has_bias = bias == nullptr || fp8 || d->n % 4 == 0;
+    if(!u8 && d->k > 0 && dma_has_bias && mi355_dma_gemm_supported(d, a, b))
+        return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
     if(!u8 && d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
-        return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, s);
+        return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
 
     generic_params p;
     p.a            = static_cast<const uint8_t*>(a);
@@ -273,6 +296,7 @@ extern "C" int mi355_quant_dot(const mi355_quant_dot_desc* d,
     p.scale_b      = scale_b;
     p.colsum_b     = colsum_b;
     p.rowsum_a     = rowsum_a;
+    p.bias         = bias;
     p.scale_a_mode = d->scale_a_mode;
     p.scale_b_mode = d->scale_b_mode;
     p.zp_a         = d->zp_a;

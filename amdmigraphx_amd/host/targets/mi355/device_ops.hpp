@@ -76,10 +76,12 @@ struct copy_from_device
     argument compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const;
 };
 
-// inputs: a, b, [scale_a, scale_b] (dequant), [colsum_b] (zp_a != 0), [rowsum_a] (zp_b != 0), out
+// inputs: a, b, [scale_a, scale_b] (dequant), [colsum_b] (zp_a != 0), [rowsum_a] (zp_b != 0),
+// [bias: float [N]] (has_bias), out
 struct quant_dot
 {
     bool dequant           = false;
+    bool has_bias          = false;
     int64_t zp_a           = 0;
     int64_t zp_b           = 0;
     int64_t scale_a_mode   = MI355_QP_NONE;
@@ -89,6 +91,7 @@ struct quant_dot
     static void reflect(Self& self, F f)
     {
         f(self.dequant, "dequant");
+        f(self.has_bias, "has_bias");
         f(self.zp_a, "zp_a");
         f(self.zp_b, "zp_b");
         f(self.scale_a_mode, "scale_a_mode");
@@ -98,7 +101,7 @@ struct quant_dot
     std::string name() const { return "mi355::quant_dot"; }
     std::size_t expected_inputs() const
     {
-        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0);
+        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0) + (has_bias ? 1 : 0);
     }
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;

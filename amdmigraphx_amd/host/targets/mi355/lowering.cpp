@@ -167,6 +167,25 @@ int scale_mode(const shape& s)
     return row ? MI355_QP_PER_ROW : (col ? MI355_QP_PER_COL : MI355_QP_PER_TENSOR);
 }
 
+// a float [N] vector broadcast over every row of `lens`
+bool is_column_bias(instruction_ref x, const std::vector<std::size_t>& lens)
+{
+    const shape& s = x->get_shape();
+    if(s.type() != shape::float_type or s.lens() != lens)
+        return false;
+    const std::size_t nd = s.ndim();
+    for(std::size_t i = 0; i + 1 < nd; i++)
+    {
+        if(s.lens()[i] != 1 and s.strides()[i] != 0)
+            return false;
+    }
+    if(s.lens()[nd - 1] != 1 and s.strides()[nd - 1] != 1)
+        return false;
+    auto base = skip_broadcasts(x);
+    return base != x and base->get_shape().type() == shape::float_type and base->get_shape().standard() and
+           base->get_shape().elements() == lens.back();
+}
+
 bool fuse_quant_dot_dq(module& m, instruction_ref dq)
 {
     if(dq->name() != "dequantizelinear")
@@ -249,8 +268,25 @@ bool fuse_quant_dot_dq(module& m, instruction_ref dq)
         }
     }
 
+    // so does the bias of a linear layer: an only user that adds a vector broadcast along the rows
+    // (the epilogue adds it in fp32 exactly as the `add` would)
+    bool has_bias = false;
+    instruction_ref bias;
+    if(last == dq and dq->outputs().size() == 1 and dq->outputs().front()->name() == "add")
+    {
+        auto add   = dq->outputs().front();
+        auto other = add->inputs()[0] == dq ? add->inputs()[1] : add->inputs()[0];
+        if(other != dq and is_column_bias(other, qd->get_shape().lens()))
+        {
+            has_bias = true;
+            bias     = skip_broadcasts(other);
+            last     = add;
+        }
+    }
+
     quant_dot op;
     op.dequant      = true;
+    op.has_bias     = has_bias;
     op.zp_a         = t.zp_a;
     op.zp_b         = t.zp_b;
     op.scale_a_mode = mode_a;
@@ -270,6 +306,8 @@ bool fuse_quant_dot_dq(module& m, instruction_ref dq)
         auto buf        = insert_allocation(m, last, shape{shape::int32_type, {rows}});
         args.push_back(m.insert_instruction(last, operation{rowsum{}}, a, buf));
     }
+    if(has_bias)
+        args.push_back(bias);
     args.push_back(insert_allocation(m, last, shape{out_type, qd->get_shape().lens()}));
     m.replace_instruction(last, operation{op}, args);
     return true;

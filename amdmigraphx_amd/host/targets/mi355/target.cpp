@@ -263,6 +263,14 @@ shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
         if((zp_a != 0 or zp_b != 0) and inputs[0].type() != shape::int8_type)
             MIGRAPHX_THROW("mi355::quant_dot: zero points need int8 operands");
     }
+    if(has_bias)
+    {
+        const shape& bias = inputs[inputs.size() - 2];
+        if(not dequant)
+            MIGRAPHX_THROW("mi355::quant_dot: a bias needs the dequantizing epilogue");
+        if(bias.type() != shape::float_type or not bias.standard() or bias.elements() != s.lens().back())
+            MIGRAPHX_THROW("mi355::quant_dot: the bias must be a dense float vector of N elements");
+    }
     shape out{out_type, s.lens()};
     if(inputs.back() != out)
         MIGRAPHX_THROW("mi355::quant_dot: output buffer has the wrong shape");
@@ -303,17 +311,19 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     }
     const int32_t* colsum_b = zp_a != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
     const int32_t* rowsum_a = zp_b != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
+    const float* bias = has_bias ? reinterpret_cast<const float*>(args[next++].data()) : nullptr;
     if((zp_a != 0 or zp_b != 0) and d.batch != 1)
         MIGRAPHX_THROW("mi355::quant_dot: zero points with batched operands are not supported");
-    status_check(mi355_quant_dot(&d,
-                                 args[0].data(),
-                                 args[1].data(),
-                                 args.back().data(),
-                                 sa,
-                                 sb,
-                                 colsum_b,
-                                 rowsum_a,
-                                 stream_of(ctx)),
+    status_check(mi355_quant_dot_bias(&d,
+                                      args[0].data(),
+                                      args[1].data(),
+                                      args.back().data(),
+                                      sa,
+                                      sb,
+                                      colsum_b,
+                                      rowsum_a,
+                                      bias,
+                                      stream_of(ctx)),
                  name());
     return args.back();
 }

@@ -46,7 +46,7 @@ def _mat_layout(t):
 
 
 def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
-              colsum_b=None, rowsum_a=None, out_dtype=None, out=None):
+              colsum_b=None, rowsum_a=None, out_dtype=None, out=None, bias=None):
     """quant_dot, optionally with the fused dequantizelinear epilogue.
 
     a [..., M, K], b [..., K, N] int8 (or uint8 carrying fp8 e4m3fn bits with
@@ -54,8 +54,9 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     views are passed as they are.  Without scales the
     bare accumulators come back (int32 / float32).  With ``scale_a`` (scalar
     or [M]) / ``scale_b`` (scalar or [N]) float32 tensors the epilogue
-    (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied."""
-    _require_cuda(a, b, scale_a, scale_b)
+    (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied; ``bias`` (float32 [N])
+    is then added in float32, before the conversion to a 16-bit ``out_dtype``."""
+    _require_cuda(a, b, scale_a, scale_b, bias)
     if a.dim() != b.dim() or a.dim() < 2:
         raise Mi355Error("QUANT_DOT: dot only accepts >= 2D operands of equal rank")
     if a.shape[:-2] != b.shape[:-2]:
@@ -107,6 +108,15 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
         raise Mi355Error("scale_a must be a scalar or have M elements")
     if scale_b is not None and scale_b.numel() not in (1, n):
         raise Mi355Error("scale_b must be a scalar or have N elements")
+    if bias is not None:
+        if not dequant:
+            raise Mi355Error("quant_dot: a bias needs the dequantizing epilogue")
+        if bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous():
+            raise Mi355Error("bias must be a dense float32 vector of N elements")
+        st = lib().mi355_quant_dot_bias(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
+                                        _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _ptr(bias), _stream())
+        check(st, "mi355_quant_dot_bias")
+        return out
     st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
                                _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
     check(st, "mi355_quant_dot")

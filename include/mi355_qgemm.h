@@ -111,6 +111,22 @@ int mi355_quant_dot(const mi355_quant_dot_desc* desc,
                     const int32_t* rowsum_a,
                     void* stream);
 
+/* The same with the bias `add` that follows the dequantizelinear of a linear layer
+ * (op::add, src/include/migraphx/op/binary.hpp:60-90, of a [N] vector broadcast over the rows):
+ *   out = float(dequantized) + bias[n]      one more fp32 rounding, never a fused multiply-add,
+ * applied before the `convert` to a 16-bit type.  bias is [N] fp32 (batches share it); NULL gives
+ * mi355_quant_dot.  Requires desc->dequant. */
+int mi355_quant_dot_bias(const mi355_quant_dot_desc* desc,
+                         const void* a,
+                         const void* b,
+                         void* c,
+                         const float* scale_a,
+                         const float* scale_b,
+                         const int32_t* colsum_b,
+                         const int32_t* rowsum_a,
+                         const float* bias,
+                         void* stream);
+
 /* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
  * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the
  * zero-point term of simplify_qdq.cpp:260-266 divided by the zero point. */

@@ -165,6 +165,58 @@ TEST_CASE(qdq_matmul_zero_points)
     }
 }
 
+TEST_CASE(qdq_linear_layer_bias)
+{
+    // MatMul + Add of a [N] bias, as a linear layer is exported: the add joins the GEMM's epilogue
+    // (one launch, no separate add) and the result stays bit-identical to the CPU target.  The
+    // second shape has a zero point on the activations, the third an N that is no multiple of 4
+    // (the any-stride kernel), the fourth a bias of shape [1, N] added from the left.
+    struct layer
+    {
+        std::size_t m, k, n;
+        int zp_x;
+        bool weight_nk, left;
+    };
+    for(auto c : {layer{256, 768, 768, 0, true, false}, layer{64, 256, 128, 3, false, false},
+                  layer{33, 96, 50, 0, false, false}, layer{128, 512, 3072, 0, true, true}})
+    {
+        auto p   = qdq_matmul(c.m, c.k, c.n, c.weight_nk, c.zp_x, 0, shape::float_type, 11);
+        auto* mm = p.get_main_module();
+        auto ret = std::prev(mm->end());
+        auto y   = ret->inputs().front();
+        std::vector<std::size_t> bl = c.left ? std::vector<std::size_t>{1, c.n} : std::vector<std::size_t>{c.n};
+        auto b   = mm->add_literal(literal{shape{shape::float_type, bl}, normal_floats(c.n, 2.0f, 12)});
+        auto bb  = mm->insert_instruction(ret, make_op("multibroadcast", {{"out_lens", {c.m, c.n}}}), b);
+        auto sum = c.left ? mm->insert_instruction(ret, make_op("add"), bb, y)
+                          : mm->insert_instruction(ret, make_op("add"), y, bb);
+        migraphx::instruction::replace_argument(ret, y, sum);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        argument x{shape{shape::float_type, {c.m, c.k}}, normal_floats(c.m * c.k, 1.0f, 13)};
+        expect_same(p, {{"x", x}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 1);
+        EXPECT(not has_op(compiled, "mi355::binary") and not has_op(compiled, "mi355::chain"));
+    }
+    // a bias along the rows is no epilogue bias: it stays an add
+    {
+        const std::size_t m = 64, k = 128, n = 64;
+        auto p   = qdq_matmul(m, k, n, false, 0, 0, shape::float_type, 14);
+        auto* mm = p.get_main_module();
+        auto ret = std::prev(mm->end());
+        auto y   = ret->inputs().front();
+        auto b   = mm->add_literal(literal{shape{shape::float_type, {m}}, normal_floats(m, 2.0f, 15)});
+        auto bb  = mm->insert_instruction(ret, make_op("broadcast", {{"axis", 0}, {"out_lens", {m, n}}}), b);
+        migraphx::instruction::replace_argument(ret, y, mm->insert_instruction(ret, make_op("add"), y, bb));
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        argument x{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 16)};
+        expect_same(p, {{"x", x}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(has_op(compiled, "mi355::binary"));
+    }
+}
+
 TEST_CASE(qdq_matmul_fp16_model)
 {
     const std::size_t m = 48, k = 192, n = 80;

@@ -279,6 +279,71 @@ def test_fp8_16bit_outputs_ragged_shapes(ops, m, n, out):
     assert (gb == want).mean() > (0.97 if out == "bf16" else 0.8)
 
 
+@pytest.mark.parametrize("m,n,k,trans_b", [(192, 320, 2048, False), (512, 768, 768, True), (100, 260, 128, False),
+                                           (33, 50, 40, False), (64, 130, 256, True), (300, 1002, 512, False)])
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_int8_bias_epilogue_bit_exact(ops, m, n, k, trans_b, out):
+    """quant_dot -> dequantizelinear -> add(bias) [-> convert] in one launch: the bias is one more
+    fp32 addition (op/binary.hpp:60-90 through add), rounded on its own.  The shapes cover the
+    three int8 kernels (N % 4 == 0 large, small, and the any-stride one)."""
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (n, k) if trans_b else (k, n), dtype=np.int8)
+    bm = b.T if trans_b else b
+    sa = np.float32(0.0371)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 3).astype(np.float32)
+    bias[:4] = [0.0, -0.0, 1e-30, -1e4]
+    zp_a = 3 if m % 2 else 0
+    want = orc.qdq_matmul_int8(a, np.ascontiguousarray(bm), sa, sb, zp_a, 0, orc.F32) + bias[None, :]
+    assert want.dtype == np.float32
+    tb = dev(b).T if trans_b else dev(b)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    print("int8 bias", m, n, k, trans_b, out, flush=True)
+    got = ops.quant_dot(dev(a), tb, scale_a=dev(np.float32([sa])), scale_b=dev(sb), zp_a=zp_a,
+                        colsum_b=ops.colsum_i8(tb) if zp_a else None, out_dtype=td, bias=dev(bias))
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        ot = orc.F16 if out == "f16" else orc.BF16
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 384, 2048), (200, 264, 320), (77, 130, 192)])
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_fp8_bias_epilogue(ops, m, n, k, out):
+    """The fp8 kernels add the bias to exactly the value they would have stored without one (no
+    fused multiply-add): biased output == convert(unbiased fp32 output + bias) bit for bit."""
+    rng = np.random.default_rng(m * 3 + n)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    sx = np.float32(np.abs(x).max() / 448)
+    sw = np.float32(np.abs(w).max() / 448)
+    xq = orc.quantizelinear(x, sx, None, orc.F32, orc.FP8)
+    wq = orc.quantizelinear(w, sw, None, orc.F32, orc.FP8)
+    bias = (rng.standard_normal(n) * 0.5).astype(np.float32)
+    bias[:2] = [0.0, -0.0]
+    dsx, dsw = dev(np.float32([sx])), dev(np.float32([sw]))
+    print("fp8 bias", m, n, k, out, flush=True)
+    plain = ops.quant_dot(dev(xq), dev(wq), fp8=True, scale_a=dsx, scale_b=dsw, out_dtype=torch.float32)
+    want = plain.cpu().numpy() + bias[None, :]
+    td = torch.float32 if out == "f32" else torch.bfloat16
+    got = ops.quant_dot(dev(xq), dev(wq), fp8=True, scale_a=dsx, scale_b=dsw, out_dtype=td, bias=dev(bias))
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(bf16_bits(got), orc.convert(want, orc.F32, orc.BF16))
+    # and the unbiased value is the oracle's within the fp8 accumulation bound
+    ref = orc.qdq_matmul_fp8(xq, wq, sx, sw, orc.F32)
+    assert _fp8_close(plain.cpu().numpy(), ref, _fp8_bound(xq, wq) * float(sx) * float(sw)).all()
+
+
+def test_bias_needs_the_epilogue(ops):
+    a = dev(np.ones((16, 16), np.int8))
+    with pytest.raises(Exception):
+        ops.quant_dot(a, a, bias=dev(np.zeros(16, np.float32)))
+
+
 @pytest.mark.parametrize("m,n,k", [(5, 7, 3), (64, 48, 300), (130, 257, 96)])
 def test_uint8_quant_dot_bare(ops, m, n, k):
     """uint8 x uint8 -> int32 (op/quant_dot.hpp:62-64): exact, also for a transposed B view and
