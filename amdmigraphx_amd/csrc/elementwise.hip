@@ -145,38 +145,56 @@ struct chain_params
     int n_steps;
 };
 
-template <int W>
+template <int W, int R>
 __global__ __launch_bounds__(256) void chain_kernel(chain_params p)
 {
 #pragma clang fp contract(off)
     const int64_t c0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * W;
     if(c0 >= p.cols)
         return;
-    for(int64_t r = blockIdx.y; r < p.rows; r += gridDim.y)
+    // R rows at a time: their loads are in flight together and the step list is walked once for
+    // all of them.  Rows past the end repeat the last one and are not stored.
+    for(int64_t r0 = (int64_t)blockIdx.y * R; r0 < p.rows; r0 += (int64_t)gridDim.y * R)
     {
-        float acc[W], saved[W], operand[W];
+        float acc[R][W], saved[R][W], operand[R][W];
 #pragma unroll
-        for(int e = 0; e < W; e++)
-            acc[e] = saved[e] = 0.0f;
-        auto fetch = [&](int i, float(&dst)[W]) __attribute__((always_inline)) {
-            const float* q = p.in[i] + r * p.sr[i];
-            if(p.sc[i] == 0)
+        for(int i = 0; i < R; i++)
+#pragma unroll
+            for(int e = 0; e < W; e++)
+                acc[i][e] = saved[i][e] = 0.0f;
+        auto fetch = [&](int in, float(&dst)[R][W]) __attribute__((always_inline)) {
+            const float* base = p.in[in];
+            const int64_t sr  = p.sr[in];
+            if(p.sc[in] == 0)
             {
-                const float s = q[0];
 #pragma unroll
-                for(int e = 0; e < W; e++)
-                    dst[e] = s;
-            }
-            else if constexpr(W == 4)
-            {
-                const v4f v = *reinterpret_cast<const v4f*>(q + c0);
+                for(int i = 0; i < R; i++)
+                {
+                    const int64_t r = min(r0 + i, p.rows - 1);
+                    const float s   = base[r * sr];
 #pragma unroll
-                for(int e = 0; e < W; e++)
-                    dst[e] = v[e];
+                    for(int e = 0; e < W; e++)
+                        dst[i][e] = s;
+                }
             }
             else
             {
-                dst[0] = q[c0];
+#pragma unroll
+                for(int i = 0; i < R; i++)
+                {
+                    const int64_t r = min(r0 + i, p.rows - 1);
+                    if constexpr(W == 4)
+                    {
+                        const v4f v = *reinterpret_cast<const v4f*>(base + r * sr + c0);
+#pragma unroll
+                        for(int e = 0; e < W; e++)
+                            dst[i][e] = v[e];
+                    }
+                    else
+                    {
+                        dst[i][0] = base[r * sr + c0];
+                    }
+                }
             }
         };
         for(int s = 0; s < p.n_steps; s++)
@@ -191,31 +209,46 @@ __global__ __launch_bounds__(256) void chain_kernel(chain_params p)
                 else
                 {
 #pragma unroll
-                    for(int e = 0; e < W; e++)
-                        operand[e] = st.src == MI355_CH_SAVED ? saved[e] : acc[e];
+                    for(int i = 0; i < R; i++)
+#pragma unroll
+                        for(int e = 0; e < W; e++)
+                            operand[i][e] = st.src == MI355_CH_SAVED ? saved[i][e] : acc[i][e];
                 }
 #pragma unroll
-                for(int e = 0; e < W; e++)
-                    acc[e] = st.reversed ? binary_apply(st.op, operand[e], acc[e])
-                                         : binary_apply(st.op, acc[e], operand[e]);
+                for(int i = 0; i < R; i++)
+#pragma unroll
+                    for(int e = 0; e < W; e++)
+                        acc[i][e] = st.reversed ? binary_apply(st.op, operand[i][e], acc[i][e])
+                                                : binary_apply(st.op, acc[i][e], operand[i][e]);
                 break;
             }
             case MI355_CH_UNARY:
 #pragma unroll
-                for(int e = 0; e < W; e++)
-                    acc[e] = unary_apply(st.op, acc[e]);
+                for(int i = 0; i < R; i++)
+#pragma unroll
+                    for(int e = 0; e < W; e++)
+                        acc[i][e] = unary_apply(st.op, acc[i][e]);
                 break;
             default:
 #pragma unroll
-                for(int e = 0; e < W; e++)
-                    saved[e] = acc[e];
+                for(int i = 0; i < R; i++)
+#pragma unroll
+                    for(int e = 0; e < W; e++)
+                        saved[i][e] = acc[i][e];
                 break;
             }
         }
-        if constexpr(W == 4)
-            *reinterpret_cast<v4f*>(p.out + r * p.cols + c0) = v4f{acc[0], acc[1], acc[2], acc[3]};
-        else
-            p.out[r * p.cols + c0] = acc[0];
+#pragma unroll
+        for(int i = 0; i < R; i++)
+        {
+            const int64_t r = r0 + i;
+            if(r >= p.rows)
+                break;
+            if constexpr(W == 4)
+                *reinterpret_cast<v4f*>(p.out + r * p.cols + c0) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+            else
+                p.out[r * p.cols + c0] = acc[i][0];
+        }
     }
 }
 
@@ -494,13 +527,20 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
     p.rows    = rows;
     p.cols    = cols;
     p.n_steps = n_steps;
-    const int64_t gy = rows < 65535 ? rows : 65535;
-    if(vec)
-        hipLaunchKernelGGL(chain_kernel<4>, dim3((unsigned)((cols / 4 + 255) / 256), (unsigned)gy), dim3(256), 0,
-                           static_cast<hipStream_t>(stream), p);
+    // four rows per pass when there are enough rows to keep every CU busy that way
+    const int64_t col_blocks = ((vec ? cols / 4 : cols) + 255) / 256;
+    const bool rows4         = rows * col_blocks >= 4 * 2048;
+    const int64_t row_groups = rows4 ? (rows + 3) / 4 : rows;
+    const dim3 grid((unsigned)col_blocks, (unsigned)(row_groups < 65535 ? row_groups : 65535));
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    if(vec && rows4)
+        hipLaunchKernelGGL((chain_kernel<4, 4>), grid, dim3(256), 0, hs, p);
+    else if(vec)
+        hipLaunchKernelGGL((chain_kernel<4, 1>), grid, dim3(256), 0, hs, p);
+    else if(rows4)
+        hipLaunchKernelGGL((chain_kernel<1, 4>), grid, dim3(256), 0, hs, p);
     else
-        hipLaunchKernelGGL(chain_kernel<1>, dim3((unsigned)((cols + 255) / 256), (unsigned)gy), dim3(256), 0,
-                           static_cast<hipStream_t>(stream), p);
+        hipLaunchKernelGGL((chain_kernel<1, 1>), grid, dim3(256), 0, hs, p);
     return mi355_launch_status();
 }
 

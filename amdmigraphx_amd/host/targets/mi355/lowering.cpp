@@ -486,9 +486,33 @@ struct chain_builder
         });
     }
 
+    static bool pointwise(instruction_ref x)
+    {
+        return binary_code(x->name()) >= 0 or unary_code(x->name()) >= 0;
+    }
+
+    // A value with several users is computed again inside each of them when that costs one
+    // operator on values that exist anyway and every user is a pointwise operator (x - mean in
+    // layer normalisation, used by the variance and by the normalised value): once all of them
+    // have taken it in, the tensor itself is never written.
+    bool recomputed(instruction_ref x) const
+    {
+        if(x->outputs().size() < 2 or not fusable(x))
+            return false;
+        const bool cheap = std::all_of(x->inputs().begin(), x->inputs().end(), [&](instruction_ref i) {
+            return not pointwise(i) or i->outputs().size() > 1;
+        });
+        return cheap and std::all_of(x->outputs().begin(), x->outputs().end(), [&](instruction_ref u) {
+            return pointwise(u) and u->get_shape().type() == shape::float_type and
+                   u->get_shape().lens() == x->get_shape().lens();
+        });
+    }
+
     bool inlined(instruction_ref x, int depth) const
     {
-        return depth <= max_depth and x->outputs().size() == 1 and fusable(x);
+        if(depth > max_depth or not fusable(x))
+            return false;
+        return x->outputs().size() == 1 or recomputed(x);
     }
 
     void push(int kind, int op, int src, int reversed)
@@ -533,6 +557,9 @@ struct chain_builder
             return;
         if(x != sink)
             absorbed.push_back(x);
+        // the operands of a recomputed value are read, not computed again in their turn
+        if(x != sink and x->outputs().size() > 1)
+            depth = max_depth;
         const int un = unary_code(x->name());
         if(un >= 0)
         {

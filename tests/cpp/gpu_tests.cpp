@@ -845,6 +845,22 @@ TEST_CASE(pointwise_chains)
         auto h = op(m, "add", x, bcast(m, v, x));
         auto e = op(m, "add", op(m, "erf", op(m, "mul", h, constant(0.70710678f))), constant(1.0f));
         return op(m, "mul", op(m, "mul", h, constant(0.5f)), e);
+    }, false, {1, 0}); // x + bias has two users: both compute it again, the sum is never stored
+    // layer normalisation: x - mean feeds the variance and the normalised value and is recomputed
+    // in both chains; the two operators on the [rows, 1] statistics stay single
+    run(33, 200, [&](module& m, instruction_ref x, instruction_ref, instruction_ref v) {
+        auto mean  = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), x);
+        auto xm    = op(m, "sub", x, bcast(m, mean, x));
+        auto var   = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), op(m, "mul", xm, xm));
+        auto eps   = m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{1e-5f}});
+        auto sigma = op(m, "sqrt", op(m, "add", var, bcast(m, eps, var)));
+        return op(m, "add", op(m, "mul", op(m, "div", xm, bcast(m, sigma, x)), bcast(m, v, x)), bcast(m, v, x));
+    }, false, {2, 2});
+    // a value with a user that is no pointwise operator is stored once and read by the others
+    run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        auto d  = op(m, "sub", x, y);
+        auto mu = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), d);
+        return op(m, "mul", op(m, "add", d, y), bcast(m, mu, x));
     }, false, {1, 1});
 }
 

@@ -41,7 +41,8 @@ def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
 
 
-@pytest.mark.parametrize("rows,cols", [(33, 200), (7, 203), (1, 4), (300, 1024), (5, 1)])
+# the last two shapes have enough rows for the four-rows-per-pass form, with a ragged last group
+@pytest.mark.parametrize("rows,cols", [(33, 200), (7, 203), (1, 4), (300, 1024), (5, 1), (9001, 256), (8195, 203)])
 def test_exact_operators_match_numpy(rows, cols):
     rng = np.random.default_rng(rows * 1000 + cols)
     x = rng.standard_normal((rows, cols)).astype(np.float32) * 3
