@@ -30,6 +30,45 @@ struct dot
     shape compute_shape(const std::vector<shape>& inputs) const;
 };
 
+// Attributes and shape rule shared by convolution and quant_convolution
+// (src/include/migraphx/op/quant_convolution.hpp:52-134, op/convolution.hpp:47-206): input
+// [N, C, spatial...], weights [O, C / group, window...]; `padding` holds one entry per spatial
+// dimension (both sides) or two (all the left ones, then all the right ones).
+struct convolution_attributes
+{
+    std::vector<int64_t> padding  = {0, 0};
+    std::vector<int64_t> stride   = {1, 1};
+    std::vector<int64_t> dilation = {1, 1};
+    int64_t padding_mode          = 0; // default_: the padding that is given
+    int64_t group                 = 1;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.padding, "padding");
+        f(self.stride, "stride");
+        f(self.dilation, "dilation");
+        f(self.padding_mode, "padding_mode");
+        f(self.group, "group");
+    }
+    std::size_t kdims() const;
+    std::vector<std::size_t> output_lens(const std::string& opname, const shape& input, const shape& weights) const;
+};
+
+// src/include/migraphx/op/convolution.hpp:47-206 (static shapes)
+struct convolution : convolution_attributes
+{
+    std::string name() const { return "convolution"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
+// src/include/migraphx/op/quant_convolution.hpp:52-134: int8 -> int32, fp8 / float / fp4x2 -> float
+struct quant_convolution : convolution_attributes
+{
+    value attributes() const { return {{"general_data_type", "convolution"}}; }
+    std::string name() const { return "quant_convolution"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
 // src/include/migraphx/op/quantizelinear.hpp:50-69
 struct quantizelinear
 {

@@ -19,10 +19,10 @@ struct dead_code_elimination
     void apply(module& m) const;
 };
 
-// Turn dequantizelinear -> dot into quant_dot -> dequantizelinear and drop the fake-quantization
-// pairs that remain (src/simplify_qdq.cpp:225-289, :498-594, :642-670).  The convolution branch,
-// the MX block-scale branch and the concat / reused-quantizelinear rewrites are not part of this
-// build.
+// Turn dequantizelinear -> dot into quant_dot -> dequantizelinear, dequantizelinear -> convolution
+// into quant_convolution -> dequantizelinear, and drop the fake-quantization pairs that remain
+// (src/simplify_qdq.cpp:126-289, :498-594, :642-670); with use_mx_quant also the block-scale
+// branch (:290-357).  The concat / reused-quantizelinear rewrites are not part of this build.
 struct simplify_qdq
 {
     bool remove_qdq_only = false;

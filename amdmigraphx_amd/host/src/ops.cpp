@@ -91,6 +91,69 @@ shape dot::compute_shape(const std::vector<shape>& inputs) const
     return dot_shape(inputs, "DOT", inputs[0].type());
 }
 
+std::size_t convolution_attributes::kdims() const
+{
+    if((padding.size() != stride.size() and padding.size() / 2 != stride.size()) or
+       stride.size() != dilation.size())
+        MIGRAPHX_THROW("CONVOLUTION: inconsistent attribute sizes");
+    return stride.size();
+}
+
+std::vector<std::size_t> convolution_attributes::output_lens(const std::string& opname,
+                                                             const shape& input,
+                                                             const shape& weights) const
+{
+    if(input.ndim() != weights.ndim() or input.ndim() < 3)
+        MIGRAPHX_THROW(opname + ": input and weights need the same rank of at least 3");
+    const std::size_t kd = input.ndim() - 2;
+    if(kd != kdims())
+        MIGRAPHX_THROW(opname + ": input k-dims does not match attribute size");
+    if(group < 1 or input.lens()[1] != weights.lens()[1] * static_cast<std::size_t>(group) or
+       weights.lens()[0] % static_cast<std::size_t>(group) != 0)
+        MIGRAPHX_THROW(opname + ": mismatched channel numbers");
+    std::vector<std::size_t> lens{input.lens()[0], weights.lens()[0]};
+    for(std::size_t i = 0; i < kd; i++)
+    {
+        auto padding_factor = 2 * padding[i];
+        if(padding.size() == 2 * kd)
+            padding_factor = padding[i] + padding[i + kd];
+        const auto span = static_cast<std::ptrdiff_t>(input.lens()[i + 2]) -
+                          (1 + dilation[i] * (static_cast<std::ptrdiff_t>(weights.lens()[i + 2]) - 1)) +
+                          padding_factor;
+        // the quotient truncates toward zero, as the reference's signed division does
+        lens.push_back(static_cast<std::size_t>(std::max<std::ptrdiff_t>(1, span / stride[i] + 1)));
+    }
+    return lens;
+}
+
+shape convolution::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "CONVOLUTION", 2, 2);
+    if(inputs[0].type() != inputs[1].type())
+        MIGRAPHX_THROW("CONVOLUTION: Types do not match");
+    return {inputs[0].type(), output_lens("CONVOLUTION", inputs[0], inputs[1])};
+}
+
+shape quant_convolution::compute_shape(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() != 2 and inputs.size() != 4)
+        MIGRAPHX_THROW("QUANT_CONVOLUTION: Wrong number of arguments: expected 2 or 4 but given " +
+                       std::to_string(inputs.size()));
+    if(inputs[0].type() != inputs[1].type())
+        MIGRAPHX_THROW("QUANT_CONVOLUTION: Types do not match");
+    if(inputs.size() == 4 and inputs[2].type() != inputs[3].type())
+        MIGRAPHX_THROW("QUANT_CONVOLUTION: Types do not match");
+    const auto t = inputs[0].type();
+    static const std::set<shape::type_t> fp8 = {shape::fp8e4m3fn_type,
+                                                shape::fp8e4m3fnuz_type,
+                                                shape::fp8e5m2_type,
+                                                shape::fp8e5m2fnuz_type};
+    if(fp8.count(t) == 0 and t != shape::int8_type and t != shape::float_type and t != shape::fp4x2_type)
+        MIGRAPHX_THROW("QUANT_CONVOLUTION: only supports int8_t, uint8_t, fp4x2, and fp8");
+    return {t == shape::int8_type ? shape::int32_type : shape::float_type,
+            output_lens("QUANT_CONVOLUTION", inputs[0], inputs[1])};
+}
+
 shape quantizelinear::compute_shape(const std::vector<shape>& inputs) const
 {
     check_count(inputs, "QUANTIZELINEAR", 2, 3);
@@ -463,6 +526,8 @@ argument contiguous::compute(const shape& out, const std::vector<argument>& args
 
 MIGRAPHX_REGISTER_OP(op::quant_dot);
 MIGRAPHX_REGISTER_OP(op::dot);
+MIGRAPHX_REGISTER_OP(op::convolution);
+MIGRAPHX_REGISTER_OP(op::quant_convolution);
 MIGRAPHX_REGISTER_OP(op::quantizelinear);
 MIGRAPHX_REGISTER_OP(op::dequantizelinear);
 MIGRAPHX_REGISTER_OP(op::unpack_int4);

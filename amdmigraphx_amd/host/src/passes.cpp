@@ -149,7 +149,7 @@ bool is_quantized_type(shape::type_t t)
            t == shape::fp8e5m2_type or t == shape::fp8e5m2fnuz_type;
 }
 
-// simplify_qdq.cpp:126-289, dot branch
+// simplify_qdq.cpp:126-289: the dot branch and the convolution branch (:171-222)
 void find_quantizable_dot(module& m, instruction_ref qop)
 {
     auto dq1 = find_dq(qop->inputs()[0]);
@@ -178,6 +178,48 @@ void find_quantizable_dot(module& m, instruction_ref qop)
     if(not is_quantized_type(dq1->inputs().front()->get_shape().type()) or
        not is_quantized_type(dq2->inputs().front()->get_shape().type()))
         return;
+
+    if(qop->name() == "convolution")
+    {
+        // simplify_qdq.cpp:171-222: the input may only carry one scale and zero point, the
+        // weights one per output channel (axis 0 of the weights, axis 1 of the result)
+        const auto conv_val = qop->get_operator().to_value();
+        auto qconv          = m.insert_instruction(qop, make_op("quant_convolution", conv_val), qop_args);
+        auto conv_lens      = qconv->get_shape().lens();
+        if(not(scale1->get_shape().elements() == 1 and zp1->get_shape().elements() == 1 and
+               is_valid_qparam(scale2, arg2_lens, 0) and is_valid_qparam(zp2, arg2_lens, 0)))
+            return;
+        auto s1 = m.insert_instruction(qop, qparam_broadcast_op(scale1, conv_lens, 1), scale1);
+        auto s2 = m.insert_instruction(qop, qparam_broadcast_op(scale2, conv_lens, 1), scale2);
+        auto conv_scale = m.insert_instruction(qop, make_op("mul"), s1, s2);
+        auto zero = m.add_literal(literal{shape{qconv->get_shape().type()}, std::vector<int>{0}});
+        auto conv_zp =
+            m.insert_instruction(qop, make_op("multibroadcast", {{"out_lens", conv_lens}}), zero);
+        auto in_zp_bc = m.insert_instruction(qop, qparam_broadcast_op(zp1, arg1_lens, 1), zp1);
+        auto w_zp_bc  = m.insert_instruction(qop, qparam_broadcast_op(zp2, arg2_lens, 0), zp2);
+        const bool s1z = is_symmetric_zero_point(zp1);
+        const bool s2z = is_symmetric_zero_point(zp2);
+        if(not s1z)
+        {
+            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), in_zp_bc, qop_args[1]);
+            conv_zp = m.insert_instruction(qop, make_op("add"), conv_zp, t);
+        }
+        if(not s2z)
+        {
+            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), qop_args[0], w_zp_bc);
+            conv_zp = m.insert_instruction(qop, make_op("add"), conv_zp, t);
+        }
+        if(not s1z and not s2z)
+        {
+            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), in_zp_bc, w_zp_bc);
+            conv_zp = m.insert_instruction(qop, make_op("sub"), conv_zp, t);
+        }
+        auto r = m.insert_instruction(qop, make_op("dequantizelinear"), qconv, conv_scale, conv_zp);
+        if(is_fp16_model)
+            r = m.insert_instruction(qop, make_op("convert", {{"target_type", shape::half_type}}), r);
+        m.replace_instruction(qop, r);
+        return;
+    }
 
     auto dq       = m.insert_instruction(qop, make_op("quant_dot"), qop_args);
     auto out_lens = dq->get_shape().lens();
@@ -384,7 +426,7 @@ void simplify_qdq::apply(module& m) const
     add_int4_pack_unpack_pair(m);
     for(auto ins : all_instructions(m))
     {
-        if(ins->name() == "dot")
+        if(ins->name() == "dot" or ins->name() == "convolution")
             find_quantizable_dot(m, ins);
     }
     dead_code_elimination{}.apply(m);

@@ -53,6 +53,8 @@ def _load():
     lib.orc_fp4_to_f32.restype = ctypes.c_float
     lib.orc_fp4_from_f32.argtypes = [ctypes.c_float]
     lib.orc_fp4_from_f32.restype = ctypes.c_uint8
+    lib.orc_convolution.argtypes = [vp, ci, vp, vp, ci] + [i64] * 16
+    lib.orc_convolution.restype = None
     lib.orc_convert.argtypes = [vp, ci, vp, ci, ctypes.c_size_t]
     lib.orc_convert.restype = None
     lib.orc_mul_f32.argtypes = [vp, vp, i64, i64, vp, i64, i64, i64, i64]
@@ -137,6 +139,29 @@ def gemm(a, b, ab_type, c_type):
     sa, sb = _elem_strides(a3), _elem_strides(b3)
     _lib.orc_gemm(_p(out), c_type, ctypes.c_void_p(a3.ctypes.data), ctypes.c_void_p(b3.ctypes.data),
                   ab_type, m, n, k, sa[1], sa[2], sb[1], sb[2], nb, sa[0], sb[0])
+    return out
+
+
+def conv_out_len(in_len, k, pad, stride, dilation):
+    """op/quant_convolution.hpp:113-126 with symmetric padding."""
+    return max(1, (in_len - (1 + dilation * (k - 1)) + 2 * pad) // stride + 1)
+
+
+def convolution(x, w, x_type, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1):
+    """convolution / quant_convolution of an [N, C, H, W] input with [O, C/group, KH, KW] weights:
+    int8 -> int32, fp8 -> float (double products), float -> float (float products, double sum)."""
+    x = _c(x, _NP[x_type])
+    w = _c(w, _NP[x_type])
+    n, c, h, wd = x.shape
+    o, cg, kh, kw = w.shape
+    assert cg * group == c and o % group == 0
+    oh = conv_out_len(h, kh, padding[0], stride[0], dilation[0])
+    ow = conv_out_len(wd, kw, padding[1], stride[1], dilation[1])
+    out_type = I32 if x_type == I8 else F32
+    out = np.empty((n, o, oh, ow), _NP[out_type])
+    _lib.orc_convolution(_p(out), out_type, _p(x), _p(w), x_type, n, c, h, wd, o, kh, kw,
+                         padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1],
+                         group, oh, ow)
     return out
 
 

@@ -35,6 +35,12 @@
  *                                 every midpoint, saturation, NaN -> 0
  *   orc_dot                       test/onnx/verify/matmulnbits_tests.cpp golds
  *                                 (whole unpack -> dequantize -> dot chain)
+ *   orc_convolution               test/ref/quant_convolution.cpp:33-133 (three int8
+ *                                 cases: plain, padding, padding + stride);
+ *                                 test/ref/convolution.cpp:674-701 (dilation) and
+ *                                 :761-857 (groups) for the window indexing;
+ *                                 brute force over every attribute against a
+ *                                 padded-array numpy restatement
  *   orc_convert                   test/ref/convert.cpp + closed form
  *   orc_softmax_f32               test/ref/softmax.cpp:33-107 (two cases, 122
  *                                 expected values, axis inside the shape)
@@ -450,6 +456,76 @@ void orc_gemm(void* c,
                      load_f64(b, ab_type, b0 + (size_t)(kk * b_sk));
         }
         store_f64(c, c_type, (size_t)idx, s);
+    }
+}
+
+/* ------------------------------------------------------------------------
+ * convolution  src/include/migraphx/convolution.hpp:37-100, called by
+ *   op::quant_convolution::compute  src/include/migraphx/op/quant_convolution.hpp:142-157
+ *   op::convolution::compute        src/include/migraphx/op/convolution.hpp:208-239
+ * Cross-correlation of an [N, C, H, W] input with [O, C/group, KH, KW] weights: the window of
+ * output (n, o, y, x) starts at (y*stride - pad, x*stride - pad), steps by the dilation, and
+ * positions outside the input contribute nothing.  Output channel o reads the input channels of
+ * group o / (O / group).  The sum runs over (channel, kh, kw) in that order in a double.
+ * quant_convolution converts both tensors to double first (get_all<double>), so each product is
+ * a double product; the float operator multiplies in float and adds the rounded product.
+ * One conversion to the output type at the end.
+ * ---------------------------------------------------------------------- */
+void orc_convolution(void* out,
+                     int out_type,
+                     const void* x,
+                     const void* w,
+                     int x_type,
+                     int64_t n,
+                     int64_t c,
+                     int64_t h,
+                     int64_t wd,
+                     int64_t o,
+                     int64_t kh,
+                     int64_t kw,
+                     int64_t pad_h,
+                     int64_t pad_w,
+                     int64_t stride_h,
+                     int64_t stride_w,
+                     int64_t dil_h,
+                     int64_t dil_w,
+                     int64_t group,
+                     int64_t oh,
+                     int64_t ow)
+{
+    const int64_t cg    = c / group; /* input channels per group = weights' second dimension */
+    const int64_t og    = o / group;
+    const int64_t total = n * o * oh * ow;
+#pragma omp parallel for schedule(static)
+    for(int64_t idx = 0; idx < total; idx++)
+    {
+        const int64_t ox = idx % ow;
+        const int64_t oy = (idx / ow) % oh;
+        const int64_t oc = (idx / (ow * oh)) % o;
+        const int64_t b  = idx / (ow * oh * o);
+        const int64_t g  = oc / og;
+        double acc       = 0.0;
+        for(int64_t k = 0; k < cg; k++)
+        {
+            const int64_t ic = g * cg + k;
+            for(int64_t r = 0; r < kh; r++)
+            {
+                const int64_t iy = oy * stride_h - pad_h + r * dil_h;
+                for(int64_t q = 0; q < kw; q++)
+                {
+                    const int64_t ix = ox * stride_w - pad_w + q * dil_w;
+                    if(iy < 0 || iy >= h || ix < 0 || ix >= wd)
+                        continue;
+                    const size_t xi = (size_t)(((b * c + ic) * h + iy) * wd + ix);
+                    const size_t wi = (size_t)(((oc * cg + k) * kh + r) * kw + q);
+                    if(x_type == ORC_F32)
+                        acc += ((const float*)x)[xi] * ((const float*)w)[wi];
+                    else
+                        acc += load_f64(x, x_type, xi) * load_f64(w, x_type, wi);
+                }
+            }
+        }
+        store_f64(out, out_type, (size_t)idx, acc);
     }
 }
 

@@ -564,6 +564,190 @@ TEST_CASE(qdq_dot_asymmetric)
     }
 }
 
+// ---------------------------------------------------------------- convolution
+
+static migraphx::operation conv_op(const std::string& name,
+                                   std::vector<int64_t> padding = {0, 0, 0, 0},
+                                   std::vector<int64_t> stride  = {1, 1},
+                                   std::vector<int64_t> dilation = {1, 1},
+                                   int64_t group                = 1)
+{
+    return make_op(name, {{"padding", padding}, {"stride", stride}, {"dilation", dilation}, {"group", group},
+                          {"padding_mode", 0}});
+}
+
+TEST_CASE(quant_convolution_shapes)
+{
+    // op/quant_convolution.hpp:85-134
+    auto out = [](shape x, shape w, const migraphx::operation& op) { return op.compute_shape({x, w}); };
+    EXPECT(out({shape::int8_type, {2, 3, 4, 4}}, {shape::int8_type, {2, 3, 3, 3}}, make_op("quant_convolution")) ==
+           shape{shape::int32_type, {2, 2, 2, 2}});
+    EXPECT(out({shape::int8_type, {2, 3, 4, 4}}, {shape::int8_type, {2, 3, 3, 3}},
+               make_op("quant_convolution", {{"padding", {1, 1}}, {"stride", {2, 2}}})) ==
+           shape{shape::int32_type, {2, 2, 2, 2}});
+    EXPECT(out({shape::fp8e4m3fn_type, {1, 8, 9, 9}}, {shape::fp8e4m3fn_type, {4, 4, 3, 3}},
+               conv_op("quant_convolution", {1, 1, 1, 1}, {1, 1}, {2, 2}, 2)) ==
+           shape{shape::float_type, {1, 4, 7, 7}});
+    // two padding entries per dimension: left ones first
+    EXPECT(out({shape::int8_type, {1, 1, 5, 5}}, {shape::int8_type, {1, 1, 3, 3}},
+               conv_op("quant_convolution", {0, 1, 2, 1})) == shape{shape::int32_type, {1, 1, 5, 5}});
+    EXPECT(out({shape::float_type, {1, 4, 10}}, {shape::float_type, {6, 2, 3}},
+               make_op("convolution", {{"padding", {1}}, {"stride", {2}}, {"dilation", {1}}, {"group", 2}})) ==
+           shape{shape::float_type, {1, 6, 5}});
+    EXPECT(test::throws([&] {
+        out({shape::int8_type, {2, 3, 4, 4}}, {shape::int8_type, {2, 2, 3, 3}}, make_op("quant_convolution"));
+    }));
+    EXPECT(test::throws([&] {
+        out({shape::uint8_type, {2, 3, 4, 4}}, {shape::uint8_type, {2, 3, 3, 3}}, make_op("quant_convolution"));
+    }));
+    EXPECT(test::throws([&] {
+        out({shape::int8_type, {2, 3, 4, 4}}, {shape::int8_type, {2, 3, 3, 3}},
+            make_op("quant_convolution", {{"stride", {1, 1, 1}}}));
+    }));
+}
+
+TEST_CASE(quant_convolution_known_answers)
+{
+    // test/ref/quant_convolution.cpp:33-133 on the CPU target
+    struct kat
+    {
+        std::vector<int64_t> padding, stride;
+        std::vector<int> gold;
+    };
+    const std::vector<kat> cases = {
+        {{0, 0}, {1, 1}, {10197, 10548, 11601, 11952, 25506, 26586, 29826, 30906, 27045, 27396, 28449, 28800,
+                          77346, 78426, 81666, 82746}},
+        {{1, 1}, {2, 2}, {4521, 7014, 7830, 11952, 10515, 16734, 19737, 30906, 13161, 19542, 19494, 28800,
+                          34707, 52590, 54729, 82746}}};
+    for(const auto& c : cases)
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        std::vector<int> a(2 * 3 * 4 * 4), w(2 * 3 * 3 * 3);
+        std::iota(a.begin(), a.end(), 0);
+        std::iota(w.begin(), w.end(), 0);
+        auto al = mm->add_literal(literal{shape{shape::int8_type, {2, 3, 4, 4}}, a});
+        auto wl = mm->add_literal(literal{shape{shape::int8_type, {2, 3, 3, 3}}, w});
+        mm->add_return({mm->add_instruction(
+            make_op("quant_convolution", {{"padding", c.padding}, {"stride", c.stride}}), al, wl)});
+        auto r = run_on("oracle", p, {});
+        EXPECT(r[0].get_shape() == shape{shape::int32_type, {2, 2, 2, 2}});
+        EXPECT(r[0].to_vector<int>() == c.gold);
+    }
+}
+
+TEST_CASE(qdq_conv)
+{
+    // test/simplify_qdq_test.cpp:762-811 (`conv`) and :876-926 (`conv_multi_scale`)
+    shape s4{shape::int8_type, {1280, 320, 1, 1}};
+    shape s7{shape::float_type, {1, 320, 7, 7}};
+    for(bool per_channel : {false, true})
+    {
+        auto weight_scale = [&](module& m) {
+            if(per_channel)
+                return m.add_literal(literal{shape{shape::float_type, {1280}}, uniform_floats(1280, 0.01f, 0.1f, 3)});
+            return m.add_literal(0.5f);
+        };
+        module m1;
+        {
+            auto input   = m1.add_parameter("input", s7);
+            auto weights = m1.add_parameter("weights", s4);
+            auto wscale  = weight_scale(m1);
+            auto scale   = m1.add_literal(0.5f);
+            auto zero    = m1.add_literal(std::int8_t{0});
+            instruction_ref d1;
+            if(per_channel)
+            {
+                auto sb = m1.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", s4.lens()}}), wscale);
+                auto zb = m1.add_instruction(make_op("multibroadcast", {{"out_lens", s4.lens()}}), zero);
+                d1      = m1.add_instruction(make_op("dequantizelinear"), weights, sb, zb);
+            }
+            else
+                d1 = add_quantize_op(m1, "dequantizelinear", weights, wscale, zero);
+            auto q1 = add_quantize_op(m1, "quantizelinear", input, scale, zero);
+            auto d5 = add_quantize_op(m1, "dequantizelinear", q1, scale, zero);
+            m1.add_return({m1.add_instruction(conv_op("convolution"), d5, d1)});
+        }
+        module m2;
+        {
+            auto input   = m2.add_parameter("input", s7);
+            auto weights = m2.add_parameter("weights", s4);
+            auto wscale  = weight_scale(m2);
+            auto scale   = m2.add_literal(0.5f);
+            auto zero    = m2.add_literal(std::int8_t{0});
+            auto q1      = add_quantize_op(m2, "quantizelinear", input, scale, zero);
+            auto c1      = m2.add_instruction(conv_op("quant_convolution"), q1, weights);
+            auto os      = add_scale_mul(m2, scale, wscale, 1, 1, c1->get_shape().lens());
+            m2.add_return({m2.add_instruction(make_op("dequantizelinear"), c1, os)});
+        }
+        run_pass(m1);
+        EXPECT(canonical(m1) == canonical(m2));
+        EXPECT(count_ops(m1, "convolution") == 0 and count_ops(m1, "quant_convolution") == 1);
+    }
+    // a scale per input channel of the weights is no valid quantization axis (:928-975): untouched
+    {
+        module m1;
+        auto input   = m1.add_parameter("input", s7);
+        auto weights = m1.add_parameter("weights", s4);
+        auto wscale  = m1.add_literal(literal{shape{shape::float_type, {320}}, uniform_floats(320, 0.01f, 0.1f, 4)});
+        auto scale   = m1.add_literal(0.5f);
+        auto zero    = m1.add_literal(std::int8_t{0});
+        auto sb = m1.add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", s4.lens()}}), wscale);
+        auto zb = m1.add_instruction(make_op("multibroadcast", {{"out_lens", s4.lens()}}), zero);
+        auto d1 = m1.add_instruction(make_op("dequantizelinear"), weights, sb, zb);
+        auto q1 = add_quantize_op(m1, "quantizelinear", input, scale, zero);
+        auto d5 = add_quantize_op(m1, "dequantizelinear", q1, scale, zero);
+        m1.add_return({m1.add_instruction(conv_op("convolution"), d5, d1)});
+        run_pass(m1);
+        EXPECT(count_ops(m1, "convolution") == 1 and count_ops(m1, "quant_convolution") == 0);
+    }
+}
+
+TEST_CASE(qdq_conv_asymmetric)
+{
+    // test/simplify_qdq_test.cpp:813-874 (`conv_asymmetric_input`): one more quant_convolution per
+    // non-zero zero point, a third for the cross term; the rewritten graph computes what the
+    // fake-quantized one does (padding included: the zero-point term sees the same zero border)
+    struct cfg
+    {
+        int zp_in, zp_w;
+        std::size_t convs, adds, subs;
+    };
+    shape sx{shape::float_type, {2, 4, 6, 6}};
+    shape sw{shape::float_type, {6, 4, 3, 3}};
+    for(auto c : {cfg{0, 0, 1, 0, 0}, cfg{1, 0, 2, 1, 0}, cfg{0, -2, 2, 1, 0}, cfg{3, -2, 4, 2, 1}})
+    {
+        module m1;
+        {
+            auto input   = m1.add_parameter("x", sx);
+            auto weights = m1.add_parameter("w", sw);
+            auto scale   = m1.add_literal(0.25f);
+            auto wscale  = m1.add_literal(0.125f);
+            auto zp_in   = m1.add_literal(static_cast<std::int8_t>(c.zp_in));
+            auto zp_w    = m1.add_literal(static_cast<std::int8_t>(c.zp_w));
+            auto qw = add_quantize_op(m1, "quantizelinear", weights, wscale, zp_w);
+            auto dw = add_quantize_op(m1, "dequantizelinear", qw, wscale, zp_w);
+            auto q1 = add_quantize_op(m1, "quantizelinear", input, scale, zp_in);
+            auto d5 = add_quantize_op(m1, "dequantizelinear", q1, scale, zp_in);
+            m1.add_return({m1.add_instruction(conv_op("convolution", {1, 1, 1, 1}, {2, 1}), d5, dw)});
+        }
+        program before;
+        *before.get_main_module() = m1;
+        run_pass(m1);
+        EXPECT(count_ops(m1, "convolution") == 0);
+        EXPECT(count_ops(m1, "quant_convolution") == c.convs);
+        EXPECT(count_ops(m1, "add") == c.adds and count_ops(m1, "sub") == c.subs);
+        program after;
+        *after.get_main_module() = m1;
+        argument xa{sx, normal_floats(sx.elements(), 2.0f, 21)};
+        argument wa{sw, normal_floats(sw.elements(), 1.0f, 22)};
+        auto r0 = run_on("oracle", before, {{"x", xa}, {"w", wa}});
+        auto r1 = run_on("oracle", after, {{"x", xa}, {"w", wa}});
+        EXPECT(r1[0].get_shape() == shape{shape::float_type, {2, 6, 3, 6}});
+        EXPECT(max_rel_diff(r1[0], r0[0], 1e-2) < 1e-4);
+    }
+}
+
 // ---------------------------------------------------------------- quantize_int4, quantize_int8
 
 // ---------------------------------------------------------------- MX block quantization (fp4)

@@ -277,6 +277,45 @@ fp4.append({"name": "pack_unpack_fp4", "source": "test/ref/pack_unpack_fp4.cpp",
             "gold": num_list(re.search(r"std::vector<float> gold\{([^}]*)\}", body).group(1))})
 out["fp4"] = fp4
 
+# ---- convolution known answers (test/ref/quant_convolution.cpp, convolution.cpp) ---------------
+def conv_attrs(body, opname):
+    m = re.search(r'make_op\(\s*"' + opname + r'"\s*(?:,\s*\{(.*?)\}\s*)?\)\s*,\s*al', body, re.S)
+    attrs = {"padding": [0, 0], "stride": [1, 1], "dilation": [1, 1], "group": 1}
+    if m and m.group(1):
+        for key in ("padding", "stride", "dilation"):
+            k = re.search(r'"' + key + r'",\s*\{([^}]*)\}', m.group(1))
+            if k:
+                attrs[key] = num_list(k.group(1))
+        g = re.search(r'"group",\s*(\d+)', m.group(1))
+        if g:
+            attrs["group"] = int(g.group(1))
+    return attrs
+
+
+conv = []
+cases = test_cases(read("test/ref/quant_convolution.cpp"))
+for name in ("quant_conv2d_test", "quant_conv2d_padding_test", "quant_conv2d_padding_stride_test"):
+    body = cases[name]
+    c = {"name": name, "source": "test/ref/quant_convolution.cpp", "type": "int8",
+         "x_lens": shape(body, "a_shape")["lens"], "w_lens": shape(body, "c_shape")["lens"],
+         "x": "iota", "w": "iota", "gold": vec(body, "gold")}
+    c.update(conv_attrs(body, "quant_convolution"))
+    conv.append(c)
+cases = test_cases(read("test/ref/convolution.cpp"))
+body = cases["conv2d_dilation_test"]
+c = {"name": "conv2d_dilation_test", "source": "test/ref/convolution.cpp:674-701", "type": "float",
+     "x_lens": shape(body, "a_shape")["lens"], "w_lens": shape(body, "c_shape")["lens"],
+     "x": "iota", "w": "iota", "gold": vec(body, "gold")}
+c.update(conv_attrs(body, "convolution"))
+conv.append(c)
+body = cases["conv2d_grouped_test"]
+c = {"name": "conv2d_grouped_test", "source": "test/ref/convolution.cpp:761-857", "type": "float",
+     "x_lens": shape(body, "a_shape")["lens"], "w_lens": shape(body, "c_shape")["lens"],
+     "x": vec(body, "a"), "w": vec(body, "c"), "gold": vec(body, "gold")}
+c.update(conv_attrs(body, "convolution"))
+conv.append(c)
+out["convolution"] = conv
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")
