@@ -34,7 +34,19 @@ class QuantDotDesc(ctypes.Structure):
                  "scale_b_mode", "zp_a", "zp_b")]
 
 
+class QuantConvDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in
+                ("n", "c", "h", "w", "o", "kh", "kw", "pad_h", "pad_w", "stride_h", "stride_w",
+                 "dil_h", "dil_w", "group")] + \
+               [(n, ctypes.c_int32) for n in
+                ("in_type", "out_type", "dequant", "scale_x_mode", "scale_w_mode")]
+
+
 EXPORTS = {
+    "mi355_quant_convolution_dims": [ctypes.POINTER(QuantConvDesc), ctypes.POINTER(ctypes.c_int64),
+                                     ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_size_t)],
+    "mi355_quant_convolution": [ctypes.POINTER(QuantConvDesc)] + [ctypes.c_void_p] * 6 +
+                               [ctypes.c_size_t, ctypes.c_void_p],
     "mi355_quant_dot": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 8,
     "mi355_quant_dot_bias": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9,
     "mi355_colsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,

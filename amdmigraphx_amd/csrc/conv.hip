@@ -1,0 +1,262 @@
+// quant_convolution as im2col + the quantized GEMM.  The windows of the input are gathered into a
+// [N, group, OH*OW, Kp] matrix (Kp = C/group * KH * KW rounded up to the GEMM's K step, zero
+// filled), the weights are copied to rows of the same pitch, and for every image the result
+// plane [O, OH*OW] = W [O, Kp] . col^T is one batched mi355_quant_dot with the col matrix as the
+// transposed operand: the GEMM writes NCHW directly and its dequantize epilogue applies the
+// per-output-channel scale as a per-row scale.  Zero padding adds exact zeros to every sum
+// (int8: 0 * w; fp8: the code 0 is +0.0 and the padded weights are +0.0 too), so the result is the
+// direct convolution's.
+#include "common.h"
+
+namespace {
+
+constexpr int64_t K_STEP = 64;
+
+struct im2col_params
+{
+    const uint8_t* x;
+    uint8_t* col;
+    int64_t rows;      // N * OH * OW
+    int64_t c, h, w;   // input channels (all groups), height, width
+    int64_t cg;        // channels per group
+    int64_t kh, kw, oh, ow;
+    int64_t pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+    int64_t group;
+    int64_t kg, kp;    // window elements per group, padded row length
+};
+
+// One thread writes 16 consecutive bytes of one row of one group's matrix.
+__global__ __launch_bounds__(256) void im2col_kernel(im2col_params p)
+{
+    const int64_t chunks = p.kp / 16;
+    const int64_t total  = p.rows * p.group * chunks;
+    const int64_t step   = (int64_t)gridDim.x * 256;
+    for(int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += step)
+    {
+        const int64_t chunk = t % chunks;
+        const int64_t rg    = t / chunks; // (row within the image batch, group) with the group inside
+        const int64_t g     = rg % p.group;
+        const int64_t row   = rg / p.group;
+        const int64_t ox    = row % p.ow;
+        const int64_t oy    = (row / p.ow) % p.oh;
+        const int64_t n     = row / (p.ow * p.oh);
+        const int64_t y0    = oy * p.stride_h - p.pad_h;
+        const int64_t x0    = ox * p.stride_w - p.pad_w;
+        int64_t k           = chunk * 16;
+        int64_t q           = k % p.kw;
+        int64_t r           = (k / p.kw) % p.kh;
+        int64_t ch          = k / (p.kw * p.kh);
+        const uint8_t* img  = p.x + (n * p.c + g * p.cg) * p.h * p.w;
+        uint32_t packed[4]  = {0, 0, 0, 0};
+#pragma unroll
+        for(int e = 0; e < 16; e++, k++)
+        {
+            uint32_t v = 0;
+            if(k < p.kg)
+            {
+                const int64_t iy = y0 + r * p.dil_h;
+                const int64_t ix = x0 + q * p.dil_w;
+                if(iy >= 0 && iy < p.h && ix >= 0 && ix < p.w)
+                    v = img[(ch * p.h + iy) * p.w + ix];
+            }
+            packed[e / 4] |= v << (8 * (e % 4));
+            if(++q == p.kw)
+            {
+                q = 0;
+                if(++r == p.kh)
+                {
+                    r = 0;
+                    ch++;
+                }
+            }
+        }
+        // layout [N, group, OH*OW, Kp]
+        const int64_t plane = p.oh * p.ow;
+        const int64_t pos   = row % plane;
+        uint8_t* dst        = p.col + (((n * p.group + g) * plane + pos) * p.kp + chunk * 16);
+        *reinterpret_cast<uint4*>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    }
+}
+
+int64_t out_len(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil)
+{
+    const int64_t span = in - (1 + dil * (k - 1)) + 2 * pad;
+    const int64_t v    = span / stride + 1; // truncating division, as the reference's shape rule
+    return v < 1 ? 1 : v;
+}
+
+bool valid(const mi355_quant_conv_desc* d)
+{
+    if(d == nullptr)
+        return false;
+    if(d->n < 0 || d->c < 1 || d->h < 1 || d->w < 1 || d->o < 1 || d->kh < 1 || d->kw < 1)
+        return false;
+    if(d->pad_h < 0 || d->pad_w < 0 || d->stride_h < 1 || d->stride_w < 1 || d->dil_h < 1 || d->dil_w < 1)
+        return false;
+    if(d->group < 1 || d->c % d->group != 0 || d->o % d->group != 0)
+        return false;
+    return d->in_type == MI355_I8 || d->in_type == MI355_FP8;
+}
+
+void launch_im2col(const im2col_params& p, hipStream_t stream)
+{
+    const int64_t total = p.rows * p.group * (p.kp / 16);
+    int64_t blocks      = (total + 255) / 256;
+    if(blocks > 256 * 64)
+        blocks = 256 * 64;
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+}
+
+} // namespace
+
+extern "C" int mi355_quant_convolution_dims(const mi355_quant_conv_desc* d,
+                                            int64_t* oh,
+                                            int64_t* ow,
+                                            size_t* workspace_bytes)
+{
+    if(!valid(d))
+        return MI355_ERR_BAD_ARG;
+    const int64_t h_out = out_len(d->h, d->kh, d->pad_h, d->stride_h, d->dil_h);
+    const int64_t w_out = out_len(d->w, d->kw, d->pad_w, d->stride_w, d->dil_w);
+    const int64_t kg    = d->c / d->group * d->kh * d->kw;
+    const int64_t kp    = (kg + K_STEP - 1) / K_STEP * K_STEP;
+    if(oh != nullptr)
+        *oh = h_out;
+    if(ow != nullptr)
+        *ow = w_out;
+    if(workspace_bytes != nullptr)
+        *workspace_bytes = (size_t)((d->n * d->group * h_out * w_out + d->o) * kp);
+    return MI355_OK;
+}
+
+extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
+                                       const void* x,
+                                       const void* w,
+                                       void* out,
+                                       const float* scale_x,
+                                       const float* scale_w,
+                                       void* workspace,
+                                       size_t workspace_bytes,
+                                       void* stream)
+{
+    int64_t oh = 0, ow = 0;
+    size_t need = 0;
+    const int st = mi355_quant_convolution_dims(d, &oh, &ow, &need);
+    if(st != MI355_OK)
+        return st;
+    const bool fp8 = d->in_type == MI355_FP8;
+    if(d->dequant)
+    {
+        if(d->out_type != MI355_F32 && d->out_type != MI355_F16 && d->out_type != MI355_BF16)
+            return MI355_ERR_BAD_ARG;
+        if(d->scale_x_mode != MI355_QP_NONE && d->scale_x_mode != MI355_QP_PER_TENSOR)
+            return MI355_ERR_BAD_ARG;
+        if(d->scale_w_mode != MI355_QP_NONE && d->scale_w_mode != MI355_QP_PER_TENSOR &&
+           d->scale_w_mode != MI355_QP_PER_ROW)
+            return MI355_ERR_BAD_ARG;
+        if((d->scale_x_mode != MI355_QP_NONE && scale_x == nullptr) ||
+           (d->scale_w_mode != MI355_QP_NONE && scale_w == nullptr))
+            return MI355_ERR_BAD_ARG;
+    }
+    else if(d->out_type != (fp8 ? MI355_F32 : MI355_I32))
+        return MI355_ERR_BAD_ARG;
+    if(d->n == 0)
+        return MI355_OK;
+    if(x == nullptr || w == nullptr || out == nullptr || workspace == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if(workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return MI355_ERR_BAD_ARG;
+    if(d->n > 65535)
+        return MI355_ERR_UNSUPPORTED;
+
+    hipStream_t hs      = static_cast<hipStream_t>(stream);
+    const int64_t cg    = d->c / d->group;
+    const int64_t og    = d->o / d->group;
+    const int64_t kg    = cg * d->kh * d->kw;
+    const int64_t kp    = (kg + K_STEP - 1) / K_STEP * K_STEP;
+    const int64_t plane = oh * ow;
+    uint8_t* col        = static_cast<uint8_t*>(workspace);
+    uint8_t* wp         = col + d->n * d->group * plane * kp;
+
+    im2col_params p{};
+    p.x        = static_cast<const uint8_t*>(x);
+    p.col      = col;
+    p.rows     = d->n * plane;
+    p.c        = d->c;
+    p.h        = d->h;
+    p.w        = d->w;
+    p.cg       = cg;
+    p.kh       = d->kh;
+    p.kw       = d->kw;
+    p.oh       = oh;
+    p.ow       = ow;
+    p.pad_h    = d->pad_h;
+    p.pad_w    = d->pad_w;
+    p.stride_h = d->stride_h;
+    p.stride_w = d->stride_w;
+    p.dil_h    = d->dil_h;
+    p.dil_w    = d->dil_w;
+    p.group    = d->group;
+    p.kg       = kg;
+    p.kp       = kp;
+    launch_im2col(p, hs);
+    if(mi355_launch_status() != MI355_OK)
+        return MI355_ERR_LAUNCH;
+
+    // the weights as O rows of Kp bytes: a 1 x 1 "convolution window" over [O, Kg, 1, 1]
+    im2col_params q{};
+    q.x        = static_cast<const uint8_t*>(w);
+    q.col      = wp;
+    q.rows     = d->o;
+    q.c        = kg;
+    q.h        = 1;
+    q.w        = 1;
+    q.cg       = kg;
+    q.kh       = 1;
+    q.kw       = 1;
+    q.oh       = 1;
+    q.ow       = 1;
+    q.stride_h = 1;
+    q.stride_w = 1;
+    q.dil_h    = 1;
+    q.dil_w    = 1;
+    q.group    = 1;
+    q.kg       = kg;
+    q.kp       = kp;
+    launch_im2col(q, hs);
+    if(mi355_launch_status() != MI355_OK)
+        return MI355_ERR_LAUNCH;
+
+    mi355_quant_dot_desc g{};
+    g.m            = og;
+    g.n            = plane;
+    g.k            = kp;
+    g.lda          = kp;
+    g.ldb          = kp;
+    g.ldc          = plane;
+    g.batch        = d->n;
+    g.stride_a     = 0;
+    g.stride_b     = d->group * plane * kp;
+    g.stride_c     = d->o * plane;
+    g.trans_a      = 0;
+    g.trans_b      = 1;
+    g.in_type      = d->in_type;
+    g.out_type     = d->out_type;
+    g.dequant      = d->dequant;
+    // the weights are the GEMM's first operand: one scale per output channel is one per row
+    g.scale_a_mode = d->dequant ? d->scale_w_mode : MI355_QP_NONE;
+    g.scale_b_mode = d->dequant ? d->scale_x_mode : MI355_QP_NONE;
+    const size_t esz = mi355_dtype_size(d->out_type);
+    for(int64_t grp = 0; grp < d->group; grp++)
+    {
+        const float* sw = scale_w;
+        if(d->dequant && d->scale_w_mode == MI355_QP_PER_ROW)
+            sw = scale_w + grp * og;
+        const int r = mi355_quant_dot(&g, wp + grp * og * kp, col + grp * plane * kp,
+                                      static_cast<uint8_t*>(out) + (size_t)(grp * og * plane) * esz, sw, scale_x,
+                                      nullptr, nullptr, stream);
+        if(r != MI355_OK)
+            return r;
+    }
+    return MI355_OK;
+}

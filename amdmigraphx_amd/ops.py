@@ -11,7 +11,7 @@ import ctypes
 
 import torch
 
-from .capi import DT, QP, W4ZP, QuantDotDesc, Mi355Error, check, lib
+from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConvDesc, Mi355Error, check, lib
 
 _TORCH2DT = {torch.int8: DT.I8, torch.uint8: DT.U8, torch.int32: DT.I32, torch.float32: DT.F32,
              torch.float16: DT.F16, torch.bfloat16: DT.BF16}
@@ -120,6 +120,46 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
                                _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
     check(st, "mi355_quant_dot")
+    return out
+
+
+def quant_convolution(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1, fp8=False,
+                      scale_x=None, scale_w=None, out_dtype=None):
+    """quant_convolution of a dense [N, C, H, W] tensor with dense [O, C/group, KH, KW] weights
+    (int8, or uint8 carrying fp8 e4m3fn codes with fp8=True), optionally with the dequantizing
+    epilogue: ``scale_x`` one float, ``scale_w`` one float or one per output channel."""
+    _require_cuda(x, w, scale_x, scale_w)
+    if x.dim() != 4 or w.dim() != 4:
+        raise Mi355Error("QUANT_CONVOLUTION: input and weights must have four dimensions")
+    if x.dtype != w.dtype:
+        raise Mi355Error("QUANT_CONVOLUTION: Types do not match")
+    if not x.is_contiguous() or not w.is_contiguous():
+        raise Mi355Error("quant_convolution: input and weights must be dense")
+    n, c, h, wd = x.shape
+    o, cg, kh, kw = w.shape
+    if group < 1 or cg * group != c or o % group != 0:
+        raise Mi355Error("QUANT_CONVOLUTION: mismatched channel numbers")
+    dequant = scale_x is not None or scale_w is not None or out_dtype is not None
+    odt = (out_dtype or torch.float32) if dequant else (torch.float32 if fp8 else torch.int32)
+    d = QuantConvDesc(n=n, c=c, h=h, w=wd, o=o, kh=kh, kw=kw, pad_h=padding[0], pad_w=padding[1],
+                      stride_h=stride[0], stride_w=stride[1], dil_h=dilation[0], dil_w=dilation[1],
+                      group=group, in_type=DT.FP8 if fp8 else DT.I8, out_type=_TORCH2DT[odt],
+                      dequant=int(dequant),
+                      scale_x_mode=QP.NONE if scale_x is None else QP.PER_TENSOR,
+                      scale_w_mode=QP.NONE if scale_w is None else
+                      (QP.PER_TENSOR if scale_w.numel() == 1 else QP.PER_ROW))
+    if scale_x is not None and scale_x.numel() != 1:
+        raise Mi355Error("scale_x must be a single value")
+    if scale_w is not None and scale_w.numel() not in (1, o):
+        raise Mi355Error("scale_w must be a scalar or have one value per output channel")
+    oh, ow, need = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_size_t()
+    check(lib().mi355_quant_convolution_dims(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow),
+                                             ctypes.byref(need)), "mi355_quant_convolution_dims")
+    out = torch.empty((n, o, oh.value, ow.value), dtype=odt, device=x.device)
+    workspace = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
+    check(lib().mi355_quant_convolution(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(out), _ptr(scale_x),
+                                        _ptr(scale_w), _ptr(workspace), need.value, _stream()),
+          "mi355_quant_convolution")
     return out
 
 

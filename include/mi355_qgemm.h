@@ -127,6 +127,39 @@ int mi355_quant_dot_bias(const mi355_quant_dot_desc* desc,
                          const float* bias,
                          void* stream);
 
+/*
+ * quant_convolution (+ fused dequantizelinear) of an [N, C, H, W] tensor with [O, C/group, KH, KW]
+ * weights, both dense; the result is dense [N, O, OH, OW].
+ *
+ * Replaces: op::quant_convolution::compute (src/include/migraphx/op/quant_convolution.hpp:142-157)
+ * -> convolution (src/include/migraphx/convolution.hpp:37-100) with the shape rule of
+ * quant_convolution.hpp:85-134: cross-correlation, `pad` zeros on the low side of each spatial
+ * dimension (and as many as the output size needs on the high side), window positions stepping
+ * by the dilation; int8 x int8 -> int32 (exact), fp8 e4m3fn -> float.  A one-dimensional
+ * convolution is passed with h = kh = 1.
+ * With desc->dequant it also replaces what simplify_qdq.cpp:171-222 puts behind it for symmetric
+ * zero points:  out = float(double(acc) * double(scale_x[0] * scale_w[o or 0]))  [-> half / bf16].
+ * scale_w_mode = MI355_QP_PER_ROW means one scale per output channel ([O]).
+ * workspace: device memory of at least the size mi355_quant_convolution_dims reports, 16-byte
+ * aligned; it holds the window matrix and is free again when the call's work has finished.
+ */
+typedef struct mi355_quant_conv_desc {
+    int64_t n, c, h, w;     /* input  [N, C, H, W] */
+    int64_t o, kh, kw;      /* weights [O, C / group, KH, KW] */
+    int64_t pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+    int64_t group;
+    int32_t in_type;        /* MI355_I8 or MI355_FP8 */
+    int32_t out_type;       /* bare: MI355_I32 / MI355_F32; dequant: MI355_F32 / F16 / BF16 */
+    int32_t dequant;
+    int32_t scale_x_mode;   /* MI355_QP_NONE / PER_TENSOR */
+    int32_t scale_w_mode;   /* MI355_QP_NONE / PER_TENSOR / PER_ROW (= per output channel) */
+} mi355_quant_conv_desc;
+int mi355_quant_convolution_dims(const mi355_quant_conv_desc* desc, int64_t* oh, int64_t* ow,
+                                 size_t* workspace_bytes);
+int mi355_quant_convolution(const mi355_quant_conv_desc* desc, const void* x, const void* w, void* out,
+                            const float* scale_x, const float* scale_w, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
 /* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
  * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the
  * zero-point term of simplify_qdq.cpp:260-266 divided by the zero point. */

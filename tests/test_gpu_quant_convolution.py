@@ -1,0 +1,113 @@
+"""GPU parity of quant_convolution (im2col + the quantized GEMM) through the C ABI against the
+CPU oracle: int32 results bit-exact, dequantized results bit-exact for int8, fp8 within the
+accumulation tolerance of the fp8 matrix instructions."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.gpu_util import dev, half_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from amdmigraphx_amd import ops
+    return ops
+
+
+def test_reference_known_answers_on_gpu(ops, golden):
+    for c in golden["convolution"]:
+        if c["type"] != "int8":
+            continue
+        x = np.arange(int(np.prod(c["x_lens"]))).astype(np.int8).reshape(c["x_lens"])
+        w = np.arange(int(np.prod(c["w_lens"]))).astype(np.int8).reshape(c["w_lens"])
+        got = ops.quant_convolution(dev(x), dev(w), c["padding"], c["stride"], c["dilation"], c["group"])
+        assert got.dtype == torch.int32
+        assert got.cpu().numpy().flatten().tolist() == c["gold"], c["name"]
+
+
+CASES = [
+    # x shape, w shape, padding, stride, dilation, group
+    ((2, 64, 14, 14), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # K = 576: no padding of K
+    ((1, 3, 33, 31), (16, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # K = 147 -> 192
+    ((3, 32, 9, 12), (48, 32, 1, 1), (0, 0), (1, 1), (1, 1), 1),       # pointwise
+    ((2, 16, 10, 10), (24, 4, 3, 3), (2, 1), (1, 2), (2, 1), 4),       # groups, dilation, mixed pads
+    ((1, 8, 12, 12), (8, 1, 3, 3), (1, 1), (1, 1), (1, 1), 8),         # depthwise
+    ((2, 5, 1, 40), (7, 5, 1, 5), (0, 2), (1, 3), (1, 1), 1),          # one-dimensional
+    ((1, 20, 6, 6), (300, 20, 3, 3), (0, 0), (1, 1), (1, 1), 1),       # more than one row tile of weights
+]
+
+
+@pytest.mark.parametrize("xs,ws,padding,stride,dilation,group", CASES)
+def test_int8_bit_exact(ops, xs, ws, padding, stride, dilation, group):
+    rng = np.random.default_rng(sum(xs) * 7 + sum(ws))
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    want = orc.convolution(x, w, orc.I8, padding, stride, dilation, group)
+    print("conv int8", xs, ws, padding, stride, dilation, group, flush=True)
+    got = ops.quant_convolution(dev(x), dev(w), padding, stride, dilation, group)
+    assert tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_int8_dequant_epilogue_bit_exact(ops, out, per_channel):
+    """quant_convolution -> dequantizelinear(scale_x * scale_w[o]) [-> convert], the graph
+    simplify_qdq.cpp:171-222 leaves for symmetric zero points."""
+    rng = np.random.default_rng(5)
+    xs, ws = (2, 32, 12, 12), (40, 16, 3, 3)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.0213)
+    sw = rng.uniform(0.001, 0.01, 40 if per_channel else 1).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (1, 1), (1, 1), (1, 1), 2)
+    scale = (sx * sw).astype(np.float32)                      # the graph's fp32 `mul`
+    scale_full = np.broadcast_to(scale.reshape(1, -1, 1, 1) if per_channel else scale.reshape(1, 1, 1, 1),
+                                 acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale_full), None, orc.I32, orc.F32)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 2, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        ot = orc.F16 if out == "f16" else orc.BF16
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+def test_fp8_convolution(ops):
+    rng = np.random.default_rng(8)
+    xs, ws = (2, 32, 10, 10), (24, 32, 3, 3)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.05).astype(np.float32)
+    xq = orc.quantizelinear(x.reshape(-1, xs[-1]), np.float32(np.abs(x).max() / 448), None, orc.F32,
+                            orc.FP8).reshape(xs)
+    wq = orc.quantizelinear(w.reshape(-1, ws[-1]), np.float32(np.abs(w).max() / 448), None, orc.F32,
+                            orc.FP8).reshape(ws)
+    want = orc.convolution(xq, wq, orc.FP8, (1, 1))
+    got = ops.quant_convolution(dev(xq), dev(wq), (1, 1), fp8=True).cpu().numpy()
+    # the fp8 matrix instructions keep about 20 bits below the largest product of a K-group
+    mag = orc.convolution(np.abs(orc.fp8_to_f32(xq)).astype(np.float32),
+                          np.abs(orc.fp8_to_f32(wq)).astype(np.float32), orc.F32, (1, 1))
+    assert np.all(np.abs(got - want) <= np.maximum(1e-3 * np.abs(want), 2.0 ** -14 * mag))
+    # small integers are exact
+    xi = rng.integers(-3, 4, xs).astype(np.float32)
+    wi = rng.integers(-2, 3, ws).astype(np.float32)
+    got = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(orc.fp8_from_f32(wi)), (1, 1), fp8=True)
+    assert np.array_equal(got.cpu().numpy(), orc.convolution(xi, wi, orc.F32, (1, 1)))
+
+
+def test_argument_errors(ops):
+    x = dev(np.zeros((1, 4, 5, 5), np.int8))
+    with pytest.raises(Exception):
+        ops.quant_convolution(x, dev(np.zeros((2, 3, 3, 3), np.int8)))          # channels do not match
+    with pytest.raises(Exception):
+        ops.quant_convolution(x, dev(np.zeros((3, 2, 3, 3), np.int8)), group=2)  # O % group
+    with pytest.raises(Exception):
+        ops.quant_convolution(x, dev(np.zeros((2, 4, 3, 3), np.int8)), stride=(0, 1))
+    # a window larger than the padded input gives the minimum output size of one
+    got = ops.quant_convolution(x, dev(np.ones((2, 4, 7, 7), np.int8)))
+    assert tuple(got.shape) == (1, 2, 1, 1)
