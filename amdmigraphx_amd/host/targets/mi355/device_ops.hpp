@@ -108,6 +108,36 @@ struct quant_dot
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// inputs: x [N, C, H, W] or [N, C, W], weights [O, C / group, window...] (both dense),
+// [scale_x (one float), scale_w (one float or one per output channel)] (dequant),
+// workspace (uint8, the size mi355_quant_convolution_dims reports), out
+struct quant_convolution
+{
+    std::vector<int64_t> padding  = {0, 0};
+    std::vector<int64_t> stride   = {1, 1};
+    std::vector<int64_t> dilation = {1, 1};
+    int64_t group                 = 1;
+    bool dequant                  = false;
+    int64_t scale_w_mode          = MI355_QP_NONE;
+    shape::type_t out_type        = shape::int32_type;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.padding, "padding");
+        f(self.stride, "stride");
+        f(self.dilation, "dilation");
+        f(self.group, "group");
+        f(self.dequant, "dequant");
+        f(self.scale_w_mode, "scale_w_mode");
+        f(self.out_type, "out_type");
+    }
+    std::string name() const { return "mi355::quant_convolution"; }
+    mi355_quant_conv_desc describe(const shape& x, const shape& w) const;
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: int8 matrix, out (int32 [cols] or [rows])
 struct colsum
 {

@@ -313,6 +313,110 @@ bool fuse_quant_dot_dq(module& m, instruction_ref dq)
     return true;
 }
 
+// ---- quant_convolution [-> dequantizelinear [-> convert]] --------------------------------------
+
+quant_convolution conv_operator(instruction_ref qc)
+{
+    const auto& ref = any_cast<op::quant_convolution>(qc->get_operator());
+    quant_convolution op;
+    op.padding  = ref.padding;
+    op.stride   = ref.stride;
+    op.dilation = ref.dilation;
+    op.group    = ref.group;
+    op.out_type = qc->get_shape().type();
+    return op;
+}
+
+instruction_ref insert_conv_workspace(module& m, instruction_ref pos, const quant_convolution& op,
+                                      instruction_ref x, instruction_ref w)
+{
+    const auto d = op.describe(x->get_shape(), w->get_shape());
+    size_t need  = 0;
+    if(mi355_quant_convolution_dims(&d, nullptr, nullptr, &need) != MI355_OK)
+        MIGRAPHX_THROW("mi355: quant_convolution attributes are not valid");
+    return insert_allocation(m, pos, shape{shape::uint8_type, {std::max<std::size_t>(need, 16)}});
+}
+
+// 0: one value, 1: one value per channel (axis 1) of `lens`, -1: anything else
+int channel_scale_mode(instruction_ref x, const std::vector<std::size_t>& lens)
+{
+    const shape& s = x->get_shape();
+    if(s.type() != shape::float_type or s.lens() != lens)
+        return -1;
+    auto base = skip_broadcasts(x);
+    if(not base->get_shape().standard())
+        return -1;
+    bool channel = false;
+    for(std::size_t i = 0; i < s.ndim(); i++)
+    {
+        if(s.lens()[i] == 1 or s.strides()[i] == 0)
+            continue;
+        if(i == 1 and s.strides()[i] == 1)
+            channel = true;
+        else
+            return -1;
+    }
+    if(channel)
+        return base->get_shape().elements() == lens[1] ? 1 : -1;
+    return base->get_shape().elements() == 1 ? 0 : -1;
+}
+
+// What simplify_qdq leaves of a convolution with symmetric zero points (simplify_qdq.cpp:171-222
+// after remove_zero_point): quant_convolution -> dequantizelinear(., mul(bcast(scale_x),
+// bcast(scale_w))) [-> convert to a 16-bit float].  One operator: the GEMM's epilogue scales.
+bool fuse_quant_conv_dq(module& m, instruction_ref dq)
+{
+    if(dq->name() != "dequantizelinear" or dq->inputs().size() != 2)
+        return false;
+    auto qc = dq->inputs()[0];
+    if(qc->name() != "quant_convolution" or qc->inputs().size() != 2 or qc->outputs().size() != 1)
+        return false;
+    auto scale = dq->inputs()[1];
+    if(scale->name() != "mul" or scale->get_shape().type() != shape::float_type)
+        return false;
+    const auto& lens = qc->get_shape().lens();
+    auto s1          = scale->inputs()[0];
+    auto s2          = scale->inputs()[1];
+    int m1           = channel_scale_mode(s1, lens);
+    int m2           = channel_scale_mode(s2, lens);
+    if(m1 == 1 and m2 == 0)
+    {
+        std::swap(s1, s2);
+        std::swap(m1, m2);
+    }
+    if(m1 != 0 or m2 < 0)
+        return false;
+    const auto t = qc->inputs()[0]->get_shape().type();
+    if(t != shape::int8_type and t != shape::fp8e4m3fn_type)
+        return false;
+    const std::size_t kd = qc->get_shape().ndim() - 2;
+    if(kd < 1 or kd > 2)
+        return false;
+
+    instruction_ref last   = dq;
+    shape::type_t out_type = shape::float_type;
+    if(dq->outputs().size() == 1 and dq->outputs().front()->name() == "convert")
+    {
+        auto cv = dq->outputs().front();
+        auto tt = any_cast<op::convert>(cv->get_operator()).target_type;
+        if(tt == shape::half_type or tt == shape::bf16_type)
+        {
+            last     = cv;
+            out_type = tt;
+        }
+    }
+    auto op         = conv_operator(qc);
+    op.dequant      = true;
+    op.scale_w_mode = m2 == 1 ? MI355_QP_PER_ROW : MI355_QP_PER_TENSOR;
+    op.out_type     = out_type;
+    auto x          = make_standard(m, last, qc->inputs()[0]);
+    auto w          = make_standard(m, last, qc->inputs()[1]);
+    auto ws         = insert_conv_workspace(m, last, op, x, w);
+    auto out        = insert_allocation(m, last, shape{out_type, lens});
+    m.replace_instruction(last, operation{op}, {x, w, skip_broadcasts(s1), skip_broadcasts(s2), ws, out});
+    return true;
+}
+
 // ---- dot(x, transpose(dequantizelinear(unpack_int4(w), blockwise scales, zero points))) -------
 
 instruction_ref skip_full_slice(instruction_ref x, bool& sliced)
@@ -687,6 +791,16 @@ void lower_instruction(module& m, instruction_ref ins)
         op.out_type = ins->get_shape().type();
         m.replace_instruction(ins, operation{op}, a, b, standard_out());
     }
+    else if(name == "quant_convolution")
+    {
+        if(ins->inputs().size() != 2)
+            MIGRAPHX_THROW("mi355: quant_convolution with scale inputs has no kernel");
+        auto op = conv_operator(ins);
+        auto x  = make_standard(m, ins, ins->inputs()[0]);
+        auto w  = make_standard(m, ins, ins->inputs()[1]);
+        auto ws = insert_conv_workspace(m, ins, op, x, w);
+        m.replace_instruction(ins, operation{op}, {x, w, ws, standard_out()});
+    }
     else if(name == "dot")
     {
         auto a = ins->inputs()[0];
@@ -886,8 +1000,8 @@ void lowering::apply(module& m) const
     {
         if(ins->name() == "dot")
             lower_w4a16(m, ins);
-        else
-            fuse_quant_dot_dq(m, ins);
+        else if(not fuse_quant_dot_dq(m, ins))
+            fuse_quant_conv_dq(m, ins);
     }
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)

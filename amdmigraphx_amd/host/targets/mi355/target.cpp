@@ -328,6 +328,99 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     return args.back();
 }
 
+mi355_quant_conv_desc quant_convolution::describe(const shape& x, const shape& w) const
+{
+    const std::size_t kd = stride.size();
+    if(kd < 1 or kd > 2 or dilation.size() != kd or (padding.size() != kd and padding.size() != 2 * kd))
+        MIGRAPHX_THROW("mi355::quant_convolution: one or two spatial dimensions with matching attributes");
+    if(x.ndim() != kd + 2 or w.ndim() != kd + 2)
+        MIGRAPHX_THROW("mi355::quant_convolution: input rank does not match the attributes");
+    for(std::size_t i = 0; i < kd and padding.size() == 2 * kd; i++)
+    {
+        if(padding[i] != padding[i + kd])
+            MIGRAPHX_THROW("mi355::quant_convolution: different padding on the two sides has no kernel");
+    }
+    const bool two = kd == 2;
+    mi355_quant_conv_desc d{};
+    d.n        = static_cast<int64_t>(x.lens()[0]);
+    d.c        = static_cast<int64_t>(x.lens()[1]);
+    d.h        = two ? static_cast<int64_t>(x.lens()[2]) : 1;
+    d.w        = static_cast<int64_t>(x.lens()[kd + 1]);
+    d.o        = static_cast<int64_t>(w.lens()[0]);
+    d.kh       = two ? static_cast<int64_t>(w.lens()[2]) : 1;
+    d.kw       = static_cast<int64_t>(w.lens()[kd + 1]);
+    d.pad_h    = two ? padding[0] : 0;
+    d.pad_w    = padding[kd - 1];
+    d.stride_h = two ? stride[0] : 1;
+    d.stride_w = stride[kd - 1];
+    d.dil_h    = two ? dilation[0] : 1;
+    d.dil_w    = dilation[kd - 1];
+    d.group    = group;
+    d.in_type  = to_mi355_type(x.type());
+    d.out_type = to_mi355_type(out_type);
+    d.dequant  = dequant ? 1 : 0;
+    d.scale_x_mode = dequant ? MI355_QP_PER_TENSOR : MI355_QP_NONE;
+    d.scale_w_mode = dequant ? static_cast<int32_t>(scale_w_mode) : MI355_QP_NONE;
+    return d;
+}
+
+shape quant_convolution::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, dequant ? 6 : 4, name());
+    op::quant_convolution ref;
+    ref.padding  = padding;
+    ref.stride   = stride;
+    ref.dilation = dilation;
+    ref.group    = group;
+    auto s = ref.compute_shape({inputs[0], inputs[1]});
+    if(inputs[0].type() != shape::int8_type and inputs[0].type() != shape::fp8e4m3fn_type)
+        MIGRAPHX_THROW("mi355::quant_convolution: kernels take int8 or fp8e4m3fn operands, not " +
+                       inputs[0].type_string());
+    check_standard(inputs[0], name());
+    check_standard(inputs[1], name());
+    if(not dequant and out_type != s.type())
+        MIGRAPHX_THROW("mi355::quant_convolution: output type must be " + s.type_string());
+    if(dequant)
+    {
+        if(out_type != shape::float_type and out_type != shape::half_type and out_type != shape::bf16_type)
+            MIGRAPHX_THROW("mi355::quant_convolution: dequantized output must be float, half or bf16");
+        if(inputs[2].type() != shape::float_type or inputs[3].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::quant_convolution: scales must be float");
+        if(scale_w_mode != MI355_QP_PER_TENSOR and scale_w_mode != MI355_QP_PER_ROW)
+            MIGRAPHX_THROW("mi355::quant_convolution: weight scales are per tensor or per output channel");
+    }
+    const auto d = describe(inputs[0], inputs[1]);
+    size_t need  = 0;
+    status_check(mi355_quant_convolution_dims(&d, nullptr, nullptr, &need), name());
+    const shape& ws = inputs[inputs.size() - 2];
+    if(ws.type() != shape::uint8_type or not ws.standard() or ws.bytes() < need)
+        MIGRAPHX_THROW("mi355::quant_convolution: workspace too small");
+    shape out{out_type, s.lens()};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::quant_convolution: output buffer has the wrong shape");
+    return out;
+}
+
+argument
+quant_convolution::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto d = describe(args[0].get_shape(), args[1].get_shape());
+    const float* sx = dequant ? reinterpret_cast<const float*>(args[2].data()) : nullptr;
+    const float* sw = dequant ? reinterpret_cast<const float*>(args[3].data()) : nullptr;
+    const argument& ws = args[args.size() - 2];
+    status_check(mi355_quant_convolution(&d,
+                                         args[0].data(),
+                                         args[1].data(),
+                                         args.back().data(),
+                                         sx,
+                                         sw,
+                                         ws.data(),
+                                         ws.get_shape().bytes(),
+                                         stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
 shape colsum::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -969,6 +1062,7 @@ MIGRAPHX_REGISTER_OP(mi355::device_literal);
 MIGRAPHX_REGISTER_OP(mi355::copy_to_device);
 MIGRAPHX_REGISTER_OP(mi355::copy_from_device);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot);
+MIGRAPHX_REGISTER_OP(mi355::quant_convolution);
 MIGRAPHX_REGISTER_OP(mi355::colsum);
 MIGRAPHX_REGISTER_OP(mi355::rowsum);
 MIGRAPHX_REGISTER_OP(mi355::dot);

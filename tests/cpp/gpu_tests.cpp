@@ -217,6 +217,113 @@ TEST_CASE(qdq_linear_layer_bias)
     }
 }
 
+// QDQ-wrapped convolution as a quantized ONNX model holds it: X float -> Q/DQ (one scale), W int8
+// literal -> DQ with one scale per output channel, convolution of the two dequantized tensors
+static program qdq_conv(std::vector<std::size_t> xl,
+                        std::vector<std::size_t> wl,
+                        const migraphx::operation& conv,
+                        bool per_channel,
+                        int zp_x,
+                        shape::type_t model_type,
+                        unsigned seed)
+{
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{model_type, xl});
+    auto xin = x;
+    if(model_type != shape::float_type)
+        xin = mm->add_instruction(make_op("convert", {{"target_type", shape::float_type}}), x);
+    auto sx = mm->add_literal(1.0f / 16);
+    auto zx = mm->add_literal(static_cast<std::int8_t>(zp_x));
+    auto q  = add_quantize_op(*mm, "quantizelinear", xin, sx, zx);
+    auto dx = add_quantize_op(*mm, "dequantizelinear", q, sx, zx);
+    const std::size_t o = wl[0];
+    std::size_t wn      = 1;
+    for(auto l : wl)
+        wn *= l;
+    auto w  = mm->add_literal(literal{shape{shape::int8_type, wl}, uniform_ints<int>(wn, -127, 127, seed)});
+    auto zw = mm->add_literal(std::int8_t{0});
+    instruction_ref dw;
+    if(per_channel)
+    {
+        auto sw  = mm->add_literal(literal{shape{shape::float_type, {o}}, uniform_floats(o, 0.001f, 0.01f, seed + 1)});
+        auto swb = mm->add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", wl}}), sw);
+        auto zwb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", wl}}), zw);
+        dw       = mm->add_instruction(make_op("dequantizelinear"), w, swb, zwb);
+    }
+    else
+    {
+        auto sw = mm->add_literal(0.004f);
+        dw      = add_quantize_op(*mm, "dequantizelinear", w, sw, zw);
+    }
+    if(model_type != shape::float_type)
+    {
+        dx = mm->add_instruction(make_op("convert", {{"target_type", model_type}}), dx);
+        dw = mm->add_instruction(make_op("convert", {{"target_type", model_type}}), dw);
+    }
+    mm->add_return({mm->add_instruction(conv, dx, dw)});
+    return p;
+}
+
+TEST_CASE(quant_convolution_programs)
+{
+    auto conv = [](std::vector<int64_t> padding, std::vector<int64_t> stride, std::vector<int64_t> dilation,
+                   int64_t group, const std::string& name = "convolution") {
+        return make_op(name, {{"padding", padding}, {"stride", stride}, {"dilation", dilation}, {"group", group}});
+    };
+    // bare quant_convolution, the shapes of test/ref/quant_convolution.cpp and of
+    // test/verify/test_quant_conv*.cpp, int8 parameters: bit-exact int32
+    struct bare
+    {
+        std::vector<std::size_t> xl, wl;
+        std::vector<int64_t> padding, stride;
+    };
+    for(const auto& c : {bare{{2, 3, 4, 4}, {2, 3, 3, 3}, {0, 0}, {1, 1}}, bare{{2, 3, 4, 4}, {2, 3, 3, 3}, {1, 1}, {2, 2}},
+                         bare{{4, 3, 32, 32}, {16, 3, 5, 5}, {2, 2}, {1, 1}}})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        shape sx{shape::int8_type, c.xl};
+        shape sw{shape::int8_type, c.wl};
+        auto x = mm->add_parameter("x", sx);
+        auto w = mm->add_parameter("w", sw);
+        mm->add_return({mm->add_instruction(conv(c.padding, c.stride, {1, 1}, 1, "quant_convolution"), x, w)});
+        expect_same(p, {{"x", argument{sx, uniform_ints<int>(sx.elements(), -128, 127, 31)}},
+                        {"w", argument{sw, uniform_ints<int>(sw.elements(), -128, 127, 32)}}});
+    }
+    // fake-quantized convolutions through simplify_qdq: one fused launch, bit-identical floats
+    struct layer
+    {
+        std::vector<std::size_t> xl, wl;
+        std::vector<int64_t> padding, stride, dilation;
+        int64_t group;
+        bool per_channel;
+        shape::type_t model;
+    };
+    for(const auto& c : {layer{{2, 16, 14, 14}, {32, 16, 3, 3}, {1, 1}, {1, 1}, {1, 1}, 1, true, shape::float_type},
+                         layer{{1, 3, 33, 31}, {8, 3, 7, 7}, {3, 3}, {2, 2}, {1, 1}, 1, true, shape::float_type},
+                         layer{{2, 8, 10, 10}, {12, 2, 3, 3}, {2, 1}, {1, 2}, {2, 1}, 4, false, shape::float_type},
+                         layer{{2, 16, 9, 9}, {16, 16, 1, 1}, {0, 0}, {1, 1}, {1, 1}, 1, true, shape::half_type},
+                         layer{{2, 6, 40}, {10, 6, 5}, {2}, {3}, {1}, 1, true, shape::float_type}})
+    {
+        auto p = qdq_conv(c.xl, c.wl, conv(c.padding, c.stride, c.dilation, c.group), c.per_channel, 0, c.model, 41);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        EXPECT(has_op(p, "quant_convolution") and not has_op(p, "convolution"));
+        shape sx{c.model, c.xl};
+        expect_same(p, {{"x", argument{sx, normal_floats(sx.elements(), 2.0f, 42)}}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_convolution") == 1);
+        EXPECT(not has_op(compiled, "mi355::dequantizelinear") and not has_op(compiled, "mi355::binary"));
+    }
+    // a zero point on the activations adds a second quant_convolution and an int32 add, for which
+    // the target has no kernel: compile says so instead of computing something else
+    {
+        auto p = qdq_conv({1, 4, 8, 8}, {4, 4, 3, 3}, conv({1, 1}, {1, 1}, {1, 1}, 1), true, 3, shape::float_type, 43);
+        EXPECT(test::throws([&] { p.compile(migraphx::make_target("mi355")); }));
+    }
+}
+
 TEST_CASE(qdq_matmul_fp16_model)
 {
     const std::size_t m = 48, k = 192, n = 80;
