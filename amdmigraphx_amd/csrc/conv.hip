@@ -25,56 +25,68 @@ struct im2col_params
     int64_t kg, kp;    // window elements per group, padded row length
 };
 
-// One thread writes 16 consecutive bytes of one row of one group's matrix.
+// A wave covers 64 consecutive output positions (lane = position) and one 16-byte piece of their
+// rows at a time: every byte load then reads neighbouring input bytes across the lanes (one or two
+// cache lines per instruction), and the (channel, window row, window column) of a piece is the
+// same for the whole wave.  The four waves of a workgroup write four neighbouring pieces of the
+// same rows, which the L2 merges into whole lines.  blockIdx.y is the group, blockIdx.z the set of
+// four pieces.
 __global__ __launch_bounds__(256) void im2col_kernel(im2col_params p)
 {
-    const int64_t chunks = p.kp / 16;
-    const int64_t total  = p.rows * p.group * chunks;
-    const int64_t step   = (int64_t)gridDim.x * 256;
-    for(int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += step)
+    const int lane      = threadIdx.x & 63;
+    const int wave      = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int chunks    = (int)(p.kp / 16);
+    const int g         = blockIdx.y;
+    const int64_t plane = p.oh * p.ow;
+    const int kw = (int)p.kw, kh = (int)p.kh, kg = (int)p.kg;
+    const int h = (int)p.h, w = (int)p.w;
+    const int dil_h = (int)p.dil_h, dil_w = (int)p.dil_w;
+    for(int64_t base = (int64_t)blockIdx.x * 64; base < p.rows; base += (int64_t)gridDim.x * 64)
     {
-        const int64_t chunk = t % chunks;
-        const int64_t rg    = t / chunks; // (row within the image batch, group) with the group inside
-        const int64_t g     = rg % p.group;
-        const int64_t row   = rg / p.group;
-        const int64_t ox    = row % p.ow;
-        const int64_t oy    = (row / p.ow) % p.oh;
-        const int64_t n     = row / (p.ow * p.oh);
-        const int64_t y0    = oy * p.stride_h - p.pad_h;
-        const int64_t x0    = ox * p.stride_w - p.pad_w;
-        int64_t k           = chunk * 16;
-        int64_t q           = k % p.kw;
-        int64_t r           = (k / p.kw) % p.kh;
-        int64_t ch          = k / (p.kw * p.kh);
-        const uint8_t* img  = p.x + (n * p.c + g * p.cg) * p.h * p.w;
-        uint32_t packed[4]  = {0, 0, 0, 0};
-#pragma unroll
-        for(int e = 0; e < 16; e++, k++)
+        const int64_t row = base + lane;
+        const bool live   = row < p.rows;
+        const int64_t rr  = live ? row : p.rows - 1;
+        const int64_t n   = rr / plane;
+        const int64_t pos = rr % plane;
+        const int oy      = (int)(pos / p.ow);
+        const int ox      = (int)(pos % p.ow);
+        const int y0      = oy * (int)p.stride_h - (int)p.pad_h;
+        const int x0      = ox * (int)p.stride_w - (int)p.pad_w;
+        const uint8_t* img = p.x + (n * p.c + g * p.cg) * h * w;
+        uint8_t* dst_row   = p.col + ((n * p.group + g) * plane + pos) * p.kp;
+        const int chunk = blockIdx.z * 4 + wave;
+        if(chunk < chunks)
         {
-            uint32_t v = 0;
-            if(k < p.kg)
+            int k  = chunk * 16;
+            int q  = k % kw;
+            int r  = (k / kw) % kh;
+            int ch = k / (kw * kh);
+            uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+            for(int e = 0; e < 16; e++, k++)
             {
-                const int64_t iy = y0 + r * p.dil_h;
-                const int64_t ix = x0 + q * p.dil_w;
-                if(iy >= 0 && iy < p.h && ix >= 0 && ix < p.w)
-                    v = img[(ch * p.h + iy) * p.w + ix];
-            }
-            packed[e / 4] |= v << (8 * (e % 4));
-            if(++q == p.kw)
-            {
-                q = 0;
-                if(++r == p.kh)
+                // always load (from a clamped address) and select afterwards: the 16 loads are then
+                // independent and in flight together
+                const int iy     = y0 + r * dil_h;
+                const int ix     = x0 + q * dil_w;
+                const bool valid = k < kg && iy >= 0 && iy < h && ix >= 0 && ix < w;
+                const int64_t at = valid ? ((int64_t)ch * h + iy) * w + ix : 0;
+                const uint32_t v = valid ? img[at] : (uint32_t)(img[at] & 0);
+                packed[e / 4] |= v << (8 * (e % 4));
+                if(++q == kw)
                 {
-                    r = 0;
-                    ch++;
+                    q = 0;
+                    if(++r == kh)
+                    {
+                        r = 0;
+                        ch++;
+                    }
                 }
             }
+            if(live)
+                *reinterpret_cast<uint4*>(dst_row + chunk * 16) =
+                    make_uint4(packed[0], packed[1], packed[2], packed[3]);
         }
-        // layout [N, group, OH*OW, Kp]
-        const int64_t plane = p.oh * p.ow;
-        const int64_t pos   = row % plane;
-        uint8_t* dst        = p.col + (((n * p.group + g) * plane + pos) * p.kp + chunk * 16);
-        *reinterpret_cast<uint4*>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     }
 }
 
@@ -100,11 +112,12 @@ bool valid(const mi355_quant_conv_desc* d)
 
 void launch_im2col(const im2col_params& p, hipStream_t stream)
 {
-    const int64_t total = p.rows * p.group * (p.kp / 16);
-    int64_t blocks      = (total + 255) / 256;
-    if(blocks > 256 * 64)
-        blocks = 256 * 64;
-    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    int64_t blocks = (p.rows + 63) / 64;
+    if(blocks > 65535 * 16)
+        blocks = 65535 * 16;
+    const int64_t chunk_blocks = (p.kp / 16 + 3) / 4;
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)blocks, (unsigned)p.group, (unsigned)chunk_blocks), dim3(256),
+                       0, stream, p);
 }
 
 } // namespace
@@ -166,7 +179,10 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
         return MI355_ERR_BAD_ARG;
     if(workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
         return MI355_ERR_BAD_ARG;
-    if(d->n > 65535)
+    // batch and group become grid dimensions, the spatial sizes 32-bit indices
+    const int64_t lim = (int64_t)1 << 30;
+    if(d->n > 65535 || d->group > 65535 || d->h >= lim || d->w >= lim || d->kh >= lim || d->kw >= lim ||
+       d->c / d->group * d->kh * d->kw >= 65535 * 64)
         return MI355_ERR_UNSUPPORTED;
 
     hipStream_t hs      = static_cast<hipStream_t>(stream);
@@ -203,7 +219,10 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
     if(mi355_launch_status() != MI355_OK)
         return MI355_ERR_LAUNCH;
 
-    // the weights as O rows of Kp bytes: a 1 x 1 "convolution window" over [O, Kg, 1, 1]
+    // the weights as O rows of Kp bytes: a 1 x 1 "convolution window" over [O, Kg, 1, 1]; rows that
+    // already have that length (and a 16-byte aligned start) are used where they are
+    const bool pad_weights = kg != kp || reinterpret_cast<uintptr_t>(w) % 16 != 0;
+    const uint8_t* wmat    = pad_weights ? wp : static_cast<const uint8_t*>(w);
     im2col_params q{};
     q.x        = static_cast<const uint8_t*>(w);
     q.col      = wp;
@@ -223,9 +242,12 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
     q.group    = 1;
     q.kg       = kg;
     q.kp       = kp;
-    launch_im2col(q, hs);
-    if(mi355_launch_status() != MI355_OK)
-        return MI355_ERR_LAUNCH;
+    if(pad_weights)
+    {
+        launch_im2col(q, hs);
+        if(mi355_launch_status() != MI355_OK)
+            return MI355_ERR_LAUNCH;
+    }
 
     mi355_quant_dot_desc g{};
     g.m            = og;
@@ -252,7 +274,7 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
         const float* sw = scale_w;
         if(d->dequant && d->scale_w_mode == MI355_QP_PER_ROW)
             sw = scale_w + grp * og;
-        const int r = mi355_quant_dot(&g, wp + grp * og * kp, col + grp * plane * kp,
+        const int r = mi355_quant_dot(&g, wmat + grp * og * kp, col + grp * plane * kp,
                                       static_cast<uint8_t*>(out) + (size_t)(grp * og * plane) * esz, sw, scale_x,
                                       nullptr, nullptr, stream);
         if(r != MI355_OK)

@@ -214,6 +214,22 @@ def main():
     except Exception as e:
         also["skinny_error"] = str(e)
 
+    # ---- quant_convolution with the dequantize epilogue (ResNet-50-shaped 3 x 3 layers, batch 32) --
+    try:
+        if args.only_headline:
+            raise RuntimeError("skipped (--only-headline)")
+        for (cc, hw, oo) in ((64, 56, 64), (256, 14, 256)):
+            xq = torch.randint(-128, 128, (32, cc, hw, hw), dtype=torch.int8, device=dev, generator=g)
+            wq = torch.randint(-128, 128, (oo, cc, 3, 3), dtype=torch.int8, device=dev, generator=g)
+            sx = torch.full((1,), 0.02, dtype=torch.float32, device=dev)
+            sw = torch.rand((oo,), device=dev, generator=g) * 0.01 + 0.001
+            tc, _ = _time_launches(lambda: ops.quant_convolution(xq, wq, (1, 1), scale_x=sx, scale_w=sw), 10, 3)
+            opsn = 2.0 * 32 * oo * hw * hw * cc * 9
+            also[f"quant_conv3x3_dq_N32_C{cc}_{hw}x{hw}_O{oo}"] = {
+                "TOPS": round(opsn / tc / 1e12, 1), "us_per_call": round(tc * 1e6, 1)}
+    except Exception as e:
+        also["quant_conv_error"] = str(e)
+
     line = {
         "metric": "quant_dot TOPS & % MFMA peak (int8/fp8); int4 W-only GEMV GB/s & % HBM",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
