@@ -80,6 +80,9 @@ EXPORTS = {
     "mi355_chain_f32": [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_void_p),
                         ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32), ctypes.c_int32,
                         ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
+    "mi355_binary_i32": [ctypes.c_int32, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p,
+                         ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p, ctypes.c_int32,
+                         ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p],
     "mi355_unary_f32": [ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p],
     "mi355_reduce_mean_f32": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
     "mi355_softmax_f32": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],

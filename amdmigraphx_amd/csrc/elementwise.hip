@@ -50,6 +50,41 @@ MI355_DEVINL float binary_apply(int op, float x, float y)
     }
 }
 
+// int32 add / sub / mul with the same addressing: the zero-point terms simplify_qdq adds up in
+// front of a dequantizelinear (src/simplify_qdq.cpp:196-222).  Wrapping arithmetic, as int32 in
+// the reference wraps on every target it is built for.
+struct bcast_params_i32
+{
+    const int32_t* a;
+    const int32_t* b;
+    int32_t* out;
+    int64_t lens[MI355_MAX_DIMS];
+    int64_t a_strides[MI355_MAX_DIMS];
+    int64_t b_strides[MI355_MAX_DIMS];
+    int64_t total;
+    int ndim;
+    int op;
+};
+
+__global__ __launch_bounds__(256) void binary_i32_kernel(bcast_params_i32 p)
+{
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < p.total; i += step)
+    {
+        int64_t rem = i, ao = 0, bo = 0;
+        for(int d = p.ndim - 1; d >= 0; d--)
+        {
+            const int64_t c = rem % p.lens[d];
+            rem /= p.lens[d];
+            ao += c * p.a_strides[d];
+            bo += c * p.b_strides[d];
+        }
+        const uint32_t x = (uint32_t)p.a[ao], y = (uint32_t)p.b[bo];
+        const uint32_t r = p.op == MI355_BIN_ADD ? x + y : (p.op == MI355_BIN_SUB ? x - y : x * y);
+        p.out[i]         = (int32_t)r;
+    }
+}
+
 // The shapes that matter collapse to [rows, cols] with each operand either running along the
 // columns (column stride 1) or constant along them (column stride 0: a per-row value or a scalar):
 // activations against a bias row, a per-row statistic, another activation.  Four columns per
@@ -541,6 +576,44 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
         hipLaunchKernelGGL((chain_kernel<1, 4>), grid, dim3(256), 0, hs, p);
     else
         hipLaunchKernelGGL((chain_kernel<1, 1>), grid, dim3(256), 0, hs, p);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_binary_i32(int32_t op,
+                                const int32_t* a,
+                                const int64_t* a_strides,
+                                const int32_t* b,
+                                const int64_t* b_strides,
+                                int32_t* out,
+                                int32_t ndim,
+                                const int64_t* lens,
+                                void* stream)
+{
+    if(op < MI355_BIN_ADD || op > MI355_BIN_MUL || ndim < 1 || ndim > MI355_MAX_DIMS || lens == nullptr ||
+       a_strides == nullptr || b_strides == nullptr)
+        return MI355_ERR_BAD_ARG;
+    bcast_params_i32 p{};
+    p.total = 1;
+    for(int d = 0; d < ndim; d++)
+    {
+        if(lens[d] < 0 || a_strides[d] < 0 || b_strides[d] < 0)
+            return MI355_ERR_BAD_ARG;
+        p.lens[d]      = lens[d];
+        p.a_strides[d] = a_strides[d];
+        p.b_strides[d] = b_strides[d];
+        p.total *= lens[d];
+    }
+    if(p.total == 0)
+        return MI355_OK;
+    if(a == nullptr || b == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    p.a    = a;
+    p.b    = b;
+    p.out  = out;
+    p.ndim = ndim;
+    p.op   = op;
+    hipLaunchKernelGGL(binary_i32_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
     return mi355_launch_status();
 }
 

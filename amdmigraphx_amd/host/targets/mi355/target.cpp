@@ -831,13 +831,17 @@ argument contiguous::compute(migraphx::context& ctx, const shape&, const std::ve
 shape binary::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 3, name());
-    if(inputs[0].type() != shape::float_type or inputs[1].type() != shape::float_type)
-        MIGRAPHX_THROW("mi355::binary: float tensors only, got " + inputs[0].type_string());
+    const auto t = inputs[0].type();
+    if(t != inputs[1].type() or (t != shape::float_type and t != shape::int32_type))
+        MIGRAPHX_THROW("mi355::binary: float or int32 tensors of one type only, got " + inputs[0].type_string() +
+                       " and " + inputs[1].type_string());
+    if(t == shape::int32_type and op == MI355_BIN_DIV)
+        MIGRAPHX_THROW("mi355::binary: int32 division has no kernel");
     if(inputs[0].lens() != inputs[1].lens())
         MIGRAPHX_THROW("mi355::binary: Dimensions do not match");
     if(inputs[0].ndim() > MI355_MAX_DIMS)
         MIGRAPHX_THROW("mi355::binary: too many dimensions");
-    shape out{shape::float_type, inputs[0].lens()};
+    shape out{t, inputs[0].lens()};
     if(inputs[2] != out)
         MIGRAPHX_THROW("mi355::binary: output buffer has the wrong shape");
     return out;
@@ -857,6 +861,20 @@ argument binary::compute(migraphx::context& ctx, const shape& out, const std::ve
     };
     const auto sa = strides_of(args[0].get_shape());
     const auto sb = strides_of(args[1].get_shape());
+    if(out.type() == shape::int32_type)
+    {
+        status_check(mi355_binary_i32(static_cast<int32_t>(op),
+                                      reinterpret_cast<const int32_t*>(args[0].data()),
+                                      sa.data(),
+                                      reinterpret_cast<const int32_t*>(args[1].data()),
+                                      sb.data(),
+                                      reinterpret_cast<int32_t*>(args[2].data()),
+                                      static_cast<int32_t>(lens.size()),
+                                      lens.data(),
+                                      stream_of(ctx)),
+                     name());
+        return args[2];
+    }
     status_check(mi355_binary_f32(static_cast<int32_t>(op),
                                   reinterpret_cast<const float*>(args[0].data()),
                                   sa.data(),

@@ -321,6 +321,11 @@ typedef enum mi355_unary_op {
 int mi355_binary_f32(int32_t op, const float* a, const int64_t* a_strides, const float* b,
                      const int64_t* b_strides, float* out, int32_t ndim, const int64_t* lens,
                      void* stream);
+/* add / sub / mul of int32 tensors (wrapping), same addressing as mi355_binary_f32: the
+ * zero-point terms of src/simplify_qdq.cpp:196-222 and :250-279 when they stay in the graph. */
+int mi355_binary_i32(int32_t op, const int32_t* a, const int64_t* a_strides, const int32_t* b,
+                     const int64_t* b_strides, int32_t* out, int32_t ndim, const int64_t* lens,
+                     void* stream);
 int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t n, void* stream);
 int mi355_reduce_mean_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
 int mi355_softmax_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);

@@ -316,11 +316,16 @@ TEST_CASE(quant_convolution_programs)
         EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_convolution") == 1);
         EXPECT(not has_op(compiled, "mi355::dequantizelinear") and not has_op(compiled, "mi355::binary"));
     }
-    // a zero point on the activations adds a second quant_convolution and an int32 add, for which
-    // the target has no kernel: compile says so instead of computing something else
+    // a zero point on the activations adds a second quant_convolution (of the broadcast zero point:
+    // the border it sees is zero-padded like the data's) and an int32 add; they stay separate
+    // operators in front of a dequantizelinear with a tensor zero point
+    for(int zp : {3, -7})
     {
-        auto p = qdq_conv({1, 4, 8, 8}, {4, 4, 3, 3}, conv({1, 1}, {1, 1}, {1, 1}, 1), true, 3, shape::float_type, 43);
-        EXPECT(test::throws([&] { p.compile(migraphx::make_target("mi355")); }));
+        auto p = qdq_conv({2, 4, 8, 8}, {6, 4, 3, 3}, conv({1, 1}, {2, 1}, {1, 1}, 1), true, zp, shape::float_type, 43);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        EXPECT(count_ops(*p.get_main_module(), "quant_convolution") == 2);
+        shape sx{shape::float_type, {2, 4, 8, 8}};
+        expect_same(p, {{"x", argument{sx, normal_floats(sx.elements(), 2.0f, 44)}}});
     }
 }
 
