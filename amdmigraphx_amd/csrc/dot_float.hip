@@ -20,6 +20,7 @@ struct dot_params
     int64_t a_sm, a_sk, b_sk, b_sn, ldc;
     int64_t stride_a, stride_b, stride_c;
     int type;
+    const float* scale; // fp32 only: the result is multiplied by scale[0] (a `mul` behind the dot); null = none
 };
 
 MI355_DEVINL float load_f32(const void* p, int type, int64_t i)
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
                 const int64_t idx = (int64_t)blockIdx.z * p.stride_c + row * p.ldc + col;
                 const float f     = (float)acc[i][j][r];
                 if(p.type == MI355_F32)
-                    ((float*)p.c)[idx] = f;
+                    ((float*)p.c)[idx] = p.scale != nullptr ? f * p.scale[0] : f;
                 else if(p.type == MI355_F16)
                     ((uint16_t*)p.c)[idx] = f32_to_half_rtz(f);
                 else
@@ -206,6 +207,8 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
         for(int j = 0; j < 2; j++)
             acc[i][j] = v4d{0.0, 0.0, 0.0, 0.0};
 
+    // x * 1.0f is x for every float, so "no scale" needs no second code path
+    const float alpha = p.scale != nullptr ? p.scale[0] : 1.0f;
     v4f va = load_a(0);
     v4f vb = load_b(0);
     for(int64_t k0 = 0; k0 < p.k; k0 += 16)
@@ -260,7 +263,7 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
                 const int64_t col = col0 + wn * 32 + j * 16 + l16;
                 if(col < p.n)
                     static_cast<float*>(p.c)[(int64_t)blockIdx.z * p.stride_c + row * p.ldc + col] =
-                        (float)acc[i][j][r];
+                        (float)acc[i][j][r] * alpha;
             }
         }
 }
@@ -345,8 +348,33 @@ extern "C" int mi355_dot(const void* a,
                          int64_t stride_c,
                          void* stream)
 {
+    return mi355_dot_scaled(a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc, batch,
+                            stride_a, stride_b, stride_c, nullptr, stream);
+}
+
+extern "C" int mi355_dot_scaled(const void* a,
+                                const void* b,
+                                void* c,
+                                int32_t type,
+                                int64_t m,
+                                int64_t n,
+                                int64_t k,
+                                int64_t a_stride_m,
+                                int64_t a_stride_k,
+                                int64_t b_stride_k,
+                                int64_t b_stride_n,
+                                int64_t ldc,
+                                int64_t batch,
+                                int64_t stride_a,
+                                int64_t stride_b,
+                                int64_t stride_c,
+                                const float* scale,
+                                void* stream)
+{
     if(type != MI355_F32 && type != MI355_F16 && type != MI355_BF16)
         return MI355_ERR_BAD_ARG;
+    if(scale != nullptr && type != MI355_F32)
+        return MI355_ERR_UNSUPPORTED;
     if(m < 0 || n < 0 || k < 0 || batch < 0 || a_stride_m < 0 || a_stride_k < 0 || b_stride_k < 0 ||
        b_stride_n < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0 || ldc < n)
         return MI355_ERR_BAD_ARG;
@@ -358,7 +386,7 @@ extern "C" int mi355_dot(const void* a,
     if(gy > 65535 || batch > 65535)
         return MI355_ERR_UNSUPPORTED;
     dot_params p{a, b, c, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc,
-                 stride_a, stride_b, stride_c, type};
+                 stride_a, stride_b, stride_c, type, scale};
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // fp32 with contiguous rows or columns, everything the 16-byte loads touch aligned

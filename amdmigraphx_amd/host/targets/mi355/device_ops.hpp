@@ -155,8 +155,15 @@ struct rowsum
 };
 
 // inputs: a, b, out
+// (with `scaled`: a, b, scale (one float), out -- the result times that value, fp32 only)
 struct dot
 {
+    bool scaled = false;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.scaled, "scaled");
+    }
     std::string name() const { return "mi355::dot"; }
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;

@@ -528,6 +528,38 @@ bool lower_w4a16(module& m, instruction_ref ins)
     return true;
 }
 
+// ---- dot -> mul by one value (attention scores) -------------------------------------------------
+// The multiplication joins the dot's store: float(sum) * value, the two roundings the two
+// operators perform.
+bool fuse_dot_scale(module& m, instruction_ref mul)
+{
+    if(mul->name() != "mul" or mul->get_shape().type() != shape::float_type)
+        return false;
+    for(int side = 0; side < 2; side++)
+    {
+        auto d = mul->inputs()[side];
+        auto s = mul->inputs()[1 - side];
+        if(d->name() != "dot" or d->outputs().size() != 1 or d->get_shape().type() != shape::float_type)
+            continue;
+        auto base = skip_broadcasts(s);
+        if(base == s or base->get_shape().elements() != 1 or base->get_shape().type() != shape::float_type or
+           s->get_shape().lens() != d->get_shape().lens())
+            continue;
+        auto a = d->inputs()[0];
+        auto b = d->inputs()[1];
+        if(not batch_collapses(a->get_shape()))
+            a = make_standard(m, mul, a);
+        if(not batch_collapses(b->get_shape()))
+            b = make_standard(m, mul, b);
+        dot op;
+        op.scaled = true;
+        auto out  = insert_allocation(m, mul, shape{shape::float_type, d->get_shape().lens()});
+        m.replace_instruction(mul, operation{op}, {a, b, base, out});
+        return true;
+    }
+    return false;
+}
+
 // ---- chains of float pointwise operators ------------------------------------------------------
 //
 // add / sub / mul / div and the unary functions that feed one another through single-use values
@@ -1000,8 +1032,8 @@ void lowering::apply(module& m) const
     {
         if(ins->name() == "dot")
             lower_w4a16(m, ins);
-        else if(not fuse_quant_dot_dq(m, ins))
-            fuse_quant_conv_dq(m, ins);
+        else if(not fuse_quant_dot_dq(m, ins) and not fuse_quant_conv_dq(m, ins))
+            fuse_dot_scale(m, ins);
     }
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)

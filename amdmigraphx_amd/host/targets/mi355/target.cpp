@@ -475,9 +475,12 @@ argument rowsum::compute(migraphx::context& ctx, const shape&, const std::vector
 
 shape dot::compute_shape(const std::vector<shape>& inputs) const
 {
-    check_inputs(inputs, 3, name());
+    check_inputs(inputs, scaled ? 4 : 3, name());
     auto s = op::dot{}.compute_shape({inputs[0], inputs[1]});
     to_mi355_type(s.type());
+    if(scaled and (s.type() != shape::float_type or inputs[2].type() != shape::float_type or
+                   inputs[2].elements() != 1))
+        MIGRAPHX_THROW("mi355::dot: the scale is one float and needs a float dot");
     if(s.type() != shape::float_type and s.type() != shape::half_type and s.type() != shape::bf16_type)
         MIGRAPHX_THROW("mi355::dot: float, half or bf16 only");
     // any strides are fine inside a matrix; the batch dimensions must collapse into one stride
@@ -511,9 +514,9 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
         }
         return r;
     };
-    status_check(mi355_dot(args[0].data(),
+    status_check(mi355_dot_scaled(args[0].data(),
                            args[1].data(),
-                           args[2].data(),
+                           args.back().data(),
                            to_mi355_type(out.type()),
                            m,
                            n,
@@ -527,9 +530,10 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
                            batch_stride(sa),
                            batch_stride(sb),
                            m * n,
+                           scaled ? reinterpret_cast<const float*>(args[2].data()) : nullptr,
                            stream_of(ctx)),
                  name());
-    return args[2];
+    return args.back();
 }
 
 shape w4a16_gemm::compute_shape(const std::vector<shape>& inputs) const

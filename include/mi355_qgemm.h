@@ -286,6 +286,17 @@ int mi355_dot(const void* a, const void* b, void* c, int32_t type,
               int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
               void* stream);
 
+/* The same followed by the `mul` with one float that scales attention scores
+ * (op::mul, src/include/migraphx/op/binary.hpp:60-90, of a broadcast scalar): fp32 only,
+ *   C = float(sum) * scale[0]       the sum is rounded to float first, then multiplied in fp32,
+ * which is what the two operators give one after the other.  scale is a DEVICE pointer; NULL gives
+ * mi355_dot. */
+int mi355_dot_scaled(const void* a, const void* b, void* c, int32_t type,
+                     int64_t m, int64_t n, int64_t k,
+                     int64_t a_stride_m, int64_t a_stride_k, int64_t b_stride_k, int64_t b_stride_n,
+                     int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                     const float* scale, void* stream);
+
 /*
  * contiguous: gather a strided view (ndim <= MI355_MAX_DIMS, element strides, zero = broadcast)
  * into a dense row-major tensor.  lens / strides are HOST arrays.

@@ -788,6 +788,64 @@ TEST_CASE(float_dot_layouts)
     }
 }
 
+TEST_CASE(dot_scale_epilogue)
+{
+    // attention scores: dot(q, k^T) * 1/sqrt(d) -- the multiplication joins the dot's store and the
+    // result stays the two operators' (float(sum) rounded, then one fp32 multiplication)
+    const std::size_t b = 3, h = 2, s = 48, d = 32;
+    for(bool left : {false, true})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        shape sq{shape::float_type, {b, h, s, d}};
+        auto q   = mm->add_parameter("q", sq);
+        auto k   = mm->add_parameter("k", sq);
+        auto kt  = mm->add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), k);
+        auto qk  = mm->add_instruction(make_op("dot"), q, kt);
+        auto c   = mm->add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{0.17677669f}});
+        auto cb  = mm->add_instruction(make_op("multibroadcast", {{"out_lens", qk->get_shape().lens()}}), c);
+        auto sc  = left ? mm->add_instruction(make_op("mul"), cb, qk) : mm->add_instruction(make_op("mul"), qk, cb);
+        mm->add_return({mm->add_instruction(make_op("softmax", {{"axis", 3}}), sc)});
+        migraphx::parameter_map params{{"q", argument{sq, normal_floats(sq.elements(), 1.0f, 61)}},
+                                       {"k", argument{sq, normal_floats(sq.elements(), 1.0f, 62)}}};
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::dot") == 1);
+        EXPECT(not has_op(compiled, "mi355::binary") and not has_op(compiled, "mi355::chain"));
+        auto want = run_on("oracle", p, params);
+        auto got  = run_on("mi355", p, params);
+        EXPECT(max_rel_diff(got[0], want[0], 1e-30) < 4e-6);
+        // the scaled scores themselves are bit-identical
+        program scores;
+        auto* sm = scores.get_main_module();
+        auto q2  = sm->add_parameter("q", sq);
+        auto k2  = sm->add_parameter("k", sq);
+        auto kt2 = sm->add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), k2);
+        auto qk2 = sm->add_instruction(make_op("dot"), q2, kt2);
+        auto c2  = sm->add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{0.17677669f}});
+        auto cb2 = sm->add_instruction(make_op("multibroadcast", {{"out_lens", qk2->get_shape().lens()}}), c2);
+        sm->add_return({left ? sm->add_instruction(make_op("mul"), cb2, qk2)
+                             : sm->add_instruction(make_op("mul"), qk2, cb2)});
+        expect_same(scores, params);
+    }
+    // a dot with a second user keeps its own result: nothing is fused
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        shape sa{shape::float_type, {16, 24}};
+        shape sb{shape::float_type, {24, 8}};
+        auto a  = mm->add_parameter("a", sa);
+        auto bb = mm->add_parameter("b", sb);
+        auto ab = mm->add_instruction(make_op("dot"), a, bb);
+        auto c  = mm->add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{3.0f}});
+        auto cb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", ab->get_shape().lens()}}), c);
+        auto sc = mm->add_instruction(make_op("mul"), ab, cb);
+        mm->add_return({mm->add_instruction(make_op("add"), sc, ab)});
+        expect_same(p, {{"a", argument{sa, normal_floats(sa.elements(), 1.0f, 63)}},
+                        {"b", argument{sb, normal_floats(sb.elements(), 1.0f, 64)}}});
+    }
+}
+
 TEST_CASE(float_operators)
 {
     // the float operators around the GEMMs, one by one against the CPU target: exact where the
