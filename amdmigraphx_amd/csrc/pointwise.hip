@@ -100,6 +100,38 @@ __global__ __launch_bounds__(PW_THREADS) void quantizelinear_kernel(
             o[e] = res[e];
 }
 
+// fp32 -> int8 with one scale and one zero point for the whole tensor (activations): 16 elements
+// per thread as four 16-byte loads and one 16-byte store, the same arithmetic as above.  n16 is
+// the element count / 16; x and out are 16-byte aligned.
+__global__ __launch_bounds__(PW_THREADS) void quantize_f32_i8_tensor_kernel(
+    const v4f* x, const float* scale, const int8_t* zp, uint4* out, int64_t n16)
+{
+    const float sv = scale[0];
+    const double z = zp != nullptr ? (double)zp[0] : 0.0;
+    const int64_t step = (int64_t)gridDim.x * PW_THREADS;
+    for(int64_t i = (int64_t)blockIdx.x * PW_THREADS + threadIdx.x; i < n16; i += step)
+    {
+        v4f v[4];
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            v[j] = x[4 * i + j];
+        uint32_t w[4];
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+        {
+            w[j] = 0;
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                const double qv = (double)rintf(v[j][e] / sv) + z;
+                const uint32_t b = (uint8_t)(int8_t)(int)clamp_like_ref(qv, -128.0, 127.0);
+                w[j] |= b << (8 * e);
+            }
+        }
+        out[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 __global__ __launch_bounds__(PW_THREADS) void dequantizelinear_kernel(const void* x,
                                                                       int x_type,
                                                                       qparams q,
@@ -315,6 +347,20 @@ extern "C" int mi355_quantizelinear(const void* x,
         return MI355_ERR_UNSUPPORTED;
     qparams q{scale, scale_stride_r, scale_stride_c, zp, zp_stride_r, zp_stride_c};
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t total = rows * cols;
+    if(x_type == MI355_F32 && out_type == MI355_I8 && scale_stride_r == 0 && scale_stride_c == 0 &&
+       (zp == nullptr || (zp_stride_r == 0 && zp_stride_c == 0)) && total % 16 == 0 &&
+       reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0)
+    {
+        const int64_t n16 = total / 16;
+        int64_t blocks    = (n16 + PW_THREADS - 1) / PW_THREADS;
+        if(blocks > 256 * 32)
+            blocks = 256 * 32;
+        hipLaunchKernelGGL(quantize_f32_i8_tensor_kernel, dim3((unsigned)blocks), dim3(PW_THREADS), 0, s,
+                           static_cast<const v4f*>(x), static_cast<const float*>(scale),
+                           static_cast<const int8_t*>(zp), static_cast<uint4*>(out), n16);
+        return mi355_launch_status();
+    }
     switch(x_type)
     {
     case MI355_F32: return launch_quantize<MI355_F32>(out_type, x, q, out, rows, cols, s);

@@ -56,6 +56,20 @@ def test_quantize_f32_to_int8(ops, scale, zp):
     assert np.array_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("scale,zp", [(1.0 / 32, 0), (0.0123, 5), (3.7, -7)])
+def test_quantize_f32_to_int8_whole_tensor_form(ops, scale, zp):
+    """A dense tensor of a multiple of 16 elements with one scale and zero point takes the
+    16-elements-per-thread kernel: same answers, ties, NaN and infinities included."""
+    rng = np.random.default_rng(2)
+    x = _adversarial_f32(rng, 5000)
+    x = x[:x.size // 64 * 64].reshape(-1, 64)
+    want = orc.quantizelinear(x, np.float32(scale), np.int8(zp), orc.F32, orc.I8)
+    got = ops.quantizelinear(dev(x), dev(np.float32([scale])), dev(np.int8([zp])), ops.DT.I8)
+    assert np.array_equal(got.cpu().numpy(), want)
+    got = ops.quantizelinear(dev(x), dev(np.float32([scale])), None, ops.DT.I8)
+    assert np.array_equal(got.cpu().numpy(), orc.quantizelinear(x, np.float32(scale), np.int8(0), orc.F32, orc.I8))
+
+
 def test_quantize_per_column_and_per_row(ops):
     rng = np.random.default_rng(1)
     x = (rng.standard_normal((37, 101)) * 3).astype(np.float32)
