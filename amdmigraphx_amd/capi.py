@@ -37,7 +37,7 @@ class QuantDotDesc(ctypes.Structure):
 class QuantConvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in
                 ("n", "c", "h", "w", "o", "kh", "kw", "pad_h", "pad_w", "stride_h", "stride_w",
-                 "dil_h", "dil_w", "group")] + \
+                 "dil_h", "dil_w", "group", "pad_h_hi", "pad_w_hi")] + \
                [(n, ctypes.c_int32) for n in
                 ("in_type", "out_type", "dequant", "scale_x_mode", "scale_w_mode")]
 

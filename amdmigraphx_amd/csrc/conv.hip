@@ -90,9 +90,9 @@ __global__ __launch_bounds__(256) void im2col_kernel(im2col_params p)
     }
 }
 
-int64_t out_len(int64_t in, int64_t k, int64_t pad, int64_t stride, int64_t dil)
+int64_t out_len(int64_t in, int64_t k, int64_t pad_lo, int64_t pad_hi, int64_t stride, int64_t dil)
 {
-    const int64_t span = in - (1 + dil * (k - 1)) + 2 * pad;
+    const int64_t span = in - (1 + dil * (k - 1)) + pad_lo + pad_hi;
     const int64_t v    = span / stride + 1; // truncating division, as the reference's shape rule
     return v < 1 ? 1 : v;
 }
@@ -103,7 +103,7 @@ bool valid(const mi355_quant_conv_desc* d)
         return false;
     if(d->n < 0 || d->c < 1 || d->h < 1 || d->w < 1 || d->o < 1 || d->kh < 1 || d->kw < 1)
         return false;
-    if(d->pad_h < 0 || d->pad_w < 0 || d->stride_h < 1 || d->stride_w < 1 || d->dil_h < 1 || d->dil_w < 1)
+    if(d->pad_h < 0 || d->pad_w < 0 || d->pad_h_hi < 0 || d->pad_w_hi < 0 || d->stride_h < 1 || d->stride_w < 1 || d->dil_h < 1 || d->dil_w < 1)
         return false;
     if(d->group < 1 || d->c % d->group != 0 || d->o % d->group != 0)
         return false;
@@ -129,8 +129,8 @@ extern "C" int mi355_quant_convolution_dims(const mi355_quant_conv_desc* d,
 {
     if(!valid(d))
         return MI355_ERR_BAD_ARG;
-    const int64_t h_out = out_len(d->h, d->kh, d->pad_h, d->stride_h, d->dil_h);
-    const int64_t w_out = out_len(d->w, d->kw, d->pad_w, d->stride_w, d->dil_w);
+    const int64_t h_out = out_len(d->h, d->kh, d->pad_h, d->pad_h_hi, d->stride_h, d->dil_h);
+    const int64_t w_out = out_len(d->w, d->kw, d->pad_w, d->pad_w_hi, d->stride_w, d->dil_w);
     const int64_t kg    = d->c / d->group * d->kh * d->kw;
     const int64_t kp    = (kg + K_STEP - 1) / K_STEP * K_STEP;
     if(oh != nullptr)

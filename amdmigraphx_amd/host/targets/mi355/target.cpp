@@ -335,12 +335,8 @@ mi355_quant_conv_desc quant_convolution::describe(const shape& x, const shape& w
         MIGRAPHX_THROW("mi355::quant_convolution: one or two spatial dimensions with matching attributes");
     if(x.ndim() != kd + 2 or w.ndim() != kd + 2)
         MIGRAPHX_THROW("mi355::quant_convolution: input rank does not match the attributes");
-    for(std::size_t i = 0; i < kd and padding.size() == 2 * kd; i++)
-    {
-        if(padding[i] != padding[i + kd])
-            MIGRAPHX_THROW("mi355::quant_convolution: different padding on the two sides has no kernel");
-    }
     const bool two = kd == 2;
+    const bool both_sides = padding.size() == 2 * kd; // low values first, then high values
     mi355_quant_conv_desc d{};
     d.n        = static_cast<int64_t>(x.lens()[0]);
     d.c        = static_cast<int64_t>(x.lens()[1]);
@@ -356,6 +352,8 @@ mi355_quant_conv_desc quant_convolution::describe(const shape& x, const shape& w
     d.dil_h    = two ? dilation[0] : 1;
     d.dil_w    = dilation[kd - 1];
     d.group    = group;
+    d.pad_h_hi = two ? padding[both_sides ? kd : 0] : 0;
+    d.pad_w_hi = padding[both_sides ? 2 * kd - 1 : kd - 1];
     d.in_type  = to_mi355_type(x.type());
     d.out_type = to_mi355_type(out_type);
     d.dequant  = dequant ? 1 : 0;

@@ -127,7 +127,8 @@ def quant_convolution(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), grou
                       scale_x=None, scale_w=None, out_dtype=None):
     """quant_convolution of a dense [N, C, H, W] tensor with dense [O, C/group, KH, KW] weights
     (int8, or uint8 carrying fp8 e4m3fn codes with fp8=True), optionally with the dequantizing
-    epilogue: ``scale_x`` one float, ``scale_w`` one float or one per output channel."""
+    epilogue: ``scale_x`` one float, ``scale_w`` one float or one per output channel.  ``padding``
+    is (h, w) for both sides or (h_low, w_low, h_high, w_high)."""
     _require_cuda(x, w, scale_x, scale_w)
     if x.dim() != 4 or w.dim() != 4:
         raise Mi355Error("QUANT_CONVOLUTION: input and weights must have four dimensions")
@@ -141,7 +142,9 @@ def quant_convolution(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), grou
         raise Mi355Error("QUANT_CONVOLUTION: mismatched channel numbers")
     dequant = scale_x is not None or scale_w is not None or out_dtype is not None
     odt = (out_dtype or torch.float32) if dequant else (torch.float32 if fp8 else torch.int32)
+    pad_hi = padding[2:] if len(padding) == 4 else padding
     d = QuantConvDesc(n=n, c=c, h=h, w=wd, o=o, kh=kh, kw=kw, pad_h=padding[0], pad_w=padding[1],
+                      pad_h_hi=pad_hi[0], pad_w_hi=pad_hi[1],
                       stride_h=stride[0], stride_w=stride[1], dil_h=dilation[0], dil_w=dilation[1],
                       group=group, in_type=DT.FP8 if fp8 else DT.I8, out_type=_TORCH2DT[odt],
                       dequant=int(dequant),

@@ -133,9 +133,9 @@ int mi355_quant_dot_bias(const mi355_quant_dot_desc* desc,
  *
  * Replaces: op::quant_convolution::compute (src/include/migraphx/op/quant_convolution.hpp:142-157)
  * -> convolution (src/include/migraphx/convolution.hpp:37-100) with the shape rule of
- * quant_convolution.hpp:85-134: cross-correlation, `pad` zeros on the low side of each spatial
- * dimension (and as many as the output size needs on the high side), window positions stepping
- * by the dilation; int8 x int8 -> int32 (exact), fp8 e4m3fn -> float.  A one-dimensional
+ * quant_convolution.hpp:85-134: cross-correlation, `pad` zeros on the low side and `pad_hi` on
+ * the high side of each spatial dimension (the reference's 2 * kdims padding form; equal values
+ * give its kdims form), window positions stepping by the dilation; int8 x int8 -> int32 (exact), fp8 e4m3fn -> float.  A one-dimensional
  * convolution is passed with h = kh = 1.
  * With desc->dequant it also replaces what simplify_qdq.cpp:171-222 puts behind it for symmetric
  * zero points:  out = float(double(acc) * double(scale_x[0] * scale_w[o or 0]))  [-> half / bf16].
@@ -146,8 +146,9 @@ int mi355_quant_dot_bias(const mi355_quant_dot_desc* desc,
 typedef struct mi355_quant_conv_desc {
     int64_t n, c, h, w;     /* input  [N, C, H, W] */
     int64_t o, kh, kw;      /* weights [O, C / group, KH, KW] */
-    int64_t pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+    int64_t pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;   /* pad: zeros on the low side */
     int64_t group;
+    int64_t pad_h_hi, pad_w_hi; /* zeros on the high side (enter the output size only) */
     int32_t in_type;        /* MI355_I8 or MI355_FP8 */
     int32_t out_type;       /* bare: MI355_I32 / MI355_F32; dequant: MI355_F32 / F16 / BF16 */
     int32_t dequant;

@@ -142,9 +142,10 @@ def gemm(a, b, ab_type, c_type):
     return out
 
 
-def conv_out_len(in_len, k, pad, stride, dilation):
-    """op/quant_convolution.hpp:113-126 with symmetric padding."""
-    return max(1, (in_len - (1 + dilation * (k - 1)) + 2 * pad) // stride + 1)
+def conv_out_len(in_len, k, pad, stride, dilation, pad_hi=None):
+    """op/quant_convolution.hpp:113-126 (the quotient truncates toward zero)."""
+    span = in_len - (1 + dilation * (k - 1)) + pad + (pad if pad_hi is None else pad_hi)
+    return max(1, int(span / stride) + 1)
 
 
 def convolution(x, w, x_type, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1):
@@ -155,8 +156,9 @@ def convolution(x, w, x_type, padding=(0, 0), stride=(1, 1), dilation=(1, 1), gr
     n, c, h, wd = x.shape
     o, cg, kh, kw = w.shape
     assert cg * group == c and o % group == 0
-    oh = conv_out_len(h, kh, padding[0], stride[0], dilation[0])
-    ow = conv_out_len(wd, kw, padding[1], stride[1], dilation[1])
+    hi = padding[2:] if len(padding) == 4 else padding   # (h_low, w_low, h_high, w_high) form
+    oh = conv_out_len(h, kh, padding[0], stride[0], dilation[0], hi[0])
+    ow = conv_out_len(wd, kw, padding[1], stride[1], dilation[1], hi[1])
     out_type = I32 if x_type == I8 else F32
     out = np.empty((n, o, oh, ow), _NP[out_type])
     _lib.orc_convolution(_p(out), out_type, _p(x), _p(w), x_type, n, c, h, wd, o, kh, kw,

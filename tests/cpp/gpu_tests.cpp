@@ -304,7 +304,9 @@ TEST_CASE(quant_convolution_programs)
                          layer{{1, 3, 33, 31}, {8, 3, 7, 7}, {3, 3}, {2, 2}, {1, 1}, 1, true, shape::float_type},
                          layer{{2, 8, 10, 10}, {12, 2, 3, 3}, {2, 1}, {1, 2}, {2, 1}, 4, false, shape::float_type},
                          layer{{2, 16, 9, 9}, {16, 16, 1, 1}, {0, 0}, {1, 1}, {1, 1}, 1, true, shape::half_type},
-                         layer{{2, 6, 40}, {10, 6, 5}, {2}, {3}, {1}, 1, true, shape::float_type}})
+                         layer{{2, 6, 40}, {10, 6, 5}, {2}, {3}, {1}, 1, true, shape::float_type},
+                         // SAME_UPPER-style padding: none in front, one behind
+                         layer{{1, 8, 8, 8}, {8, 8, 3, 3}, {0, 0, 1, 1}, {2, 2}, {1, 1}, 1, true, shape::float_type}})
     {
         auto p = qdq_conv(c.xl, c.wl, conv(c.padding, c.stride, c.dilation, c.group), c.per_channel, 0, c.model, 41);
         migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});

@@ -155,11 +155,6 @@ struct cpu_op
             const std::size_t kd = stride.size();
             if(args.size() != 2 or kd < 1 or kd > 2)
                 MIGRAPHX_THROW("oracle: convolution with " + std::to_string(kd) + " spatial dimensions");
-            for(std::size_t i = 0; i < kd and padding.size() == 2 * kd; i++)
-            {
-                if(padding[i] != padding[i + kd])
-                    MIGRAPHX_THROW("oracle: asymmetric padding");
-            }
             argument x = dense(args[0]);
             argument w = dense(args[1]);
             const auto& xl = x.get_shape().lens();

@@ -37,6 +37,7 @@ CASES = [
     ((1, 8, 12, 12), (8, 1, 3, 3), (1, 1), (1, 1), (1, 1), 8),         # depthwise
     ((2, 5, 1, 40), (7, 5, 1, 5), (0, 2), (1, 3), (1, 1), 1),          # one-dimensional
     ((1, 20, 6, 6), (300, 20, 3, 3), (0, 0), (1, 1), (1, 1), 1),       # more than one row tile of weights
+    ((2, 8, 9, 10), (8, 8, 3, 3), (0, 1, 2, 0), (2, 2), (1, 1), 1),    # low and high padding differ
 ]
 
 

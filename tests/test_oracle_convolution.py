@@ -28,11 +28,12 @@ def brute(x, w, padding, stride, dilation, group):
     """Independent form: pad with zeros, slice the dilated window, sum products in int64."""
     n, c, h, wd = x.shape
     o, cg, kh, kw = w.shape
-    ph, pw = padding
-    xp = np.zeros((n, c, h + 2 * ph, wd + 2 * pw), np.int64)
+    ph, pw = padding[0], padding[1]
+    ph2, pw2 = (padding[2], padding[3]) if len(padding) == 4 else (ph, pw)
+    xp = np.zeros((n, c, h + ph + ph2, wd + pw + pw2), np.int64)
     xp[:, :, ph:ph + h, pw:pw + wd] = x
-    oh = orc.conv_out_len(h, kh, ph, stride[0], dilation[0])
-    ow = orc.conv_out_len(wd, kw, pw, stride[1], dilation[1])
+    oh = orc.conv_out_len(h, kh, ph, stride[0], dilation[0], ph2)
+    ow = orc.conv_out_len(wd, kw, pw, stride[1], dilation[1], pw2)
     og = o // group
     out = np.zeros((n, o, oh, ow), np.int64)
     for oc in range(o):
@@ -53,6 +54,8 @@ def brute(x, w, padding, stride, dilation, group):
     ((3, 8, 5, 11), (8, 1, 3, 3), (2, 2), (1, 3), (2, 1), 8),
     ((2, 3, 6, 6), (5, 3, 1, 1), (0, 0), (2, 2), (1, 1), 1),
     ((1, 2, 7, 7), (2, 2, 5, 5), (2, 2), (1, 1), (1, 1), 1),
+    ((2, 3, 8, 9), (4, 3, 3, 3), (0, 1, 2, 0), (2, 2), (1, 1), 1),   # low and high padding differ
+    ((1, 2, 6, 6), (2, 2, 3, 3), (2, 0, 0, 1), (1, 1), (1, 1), 1),
 ])
 def test_int8_against_brute_force(shape, wshape, padding, stride, dilation, group):
     rng = np.random.default_rng(sum(shape) + sum(wshape))
