@@ -344,6 +344,87 @@ def test_bias_needs_the_epilogue(ops):
         ops.quant_dot(a, a, bias=dev(np.zeros(16, np.float32)))
 
 
+def _sweep_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    m = int(pick([1, 3, 16, 17, 64, 100, 255, 256, 257, 300]))
+    n = int(pick([1, 4, 7, 16, 60, 64, 128, 200, 256, 260]))
+    k = int(pick([1, 5, 16, 48, 64, 80, 128, 192, 256, 320, 400]))
+    return dict(m=m, n=n, k=k, trans_a=bool(rng.integers(0, 2)), trans_b=bool(rng.integers(0, 2)),
+                batch=int(pick([1, 1, 2, 3])), dequant=bool(rng.integers(0, 4) > 0),
+                sa_row=bool(rng.integers(0, 2)), sb_col=bool(rng.integers(0, 2)),
+                zp_a=int(pick([0, 0, 4, -9])), zp_b=int(pick([0, 0, -3, 11])),
+                bias=bool(rng.integers(0, 2)), out=pick(["f32", "f32", "f16", "bf16"]), rng=rng)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_int8_seeded_sweep_over_every_dispatch_path(ops, seed):
+    """Shapes on and around the tile sizes, transposed views of either operand, batches, every
+    epilogue mode: whichever of the three int8 kernels the dispatcher picks, the result is the
+    oracle's bit for bit."""
+    c = _sweep_case(seed)
+    rng, m, n, k, nb = c["rng"], c["m"], c["n"], c["k"], c["batch"]
+    a = rng.integers(-128, 128, (nb, m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (nb, k, n), dtype=np.int8)
+    da = dev(np.ascontiguousarray(a.transpose(0, 2, 1))).transpose(1, 2) if c["trans_a"] else dev(a)
+    db = dev(np.ascontiguousarray(b.transpose(0, 2, 1))).transpose(1, 2) if c["trans_b"] else dev(b)
+    if nb == 1:
+        da, db = da[0], db[0]
+    print("sweep", seed, {x: c[x] for x in c if x != "rng"}, flush=True)
+    if not c["dequant"]:
+        got = ops.quant_dot(da, db).cpu().numpy().reshape(nb, m, n)
+        for i in range(nb):
+            assert np.array_equal(got[i], orc.quant_dot(a[i], b[i], orc.I8))
+        return
+    zp_a, zp_b = (c["zp_a"], c["zp_b"]) if nb == 1 else (0, 0)
+    sa = rng.uniform(0.01, 0.05, m if c["sa_row"] else 1).astype(np.float32)
+    sb = rng.uniform(0.001, 0.01, n if c["sb_col"] else 1).astype(np.float32)
+    bias = (rng.standard_normal(n) * 2).astype(np.float32) if c["bias"] else None
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[c["out"]]
+    got = ops.quant_dot(da, db, scale_a=dev(sa), scale_b=dev(sb), zp_a=zp_a, zp_b=zp_b,
+                        colsum_b=ops.colsum_i8(db) if zp_a else None,
+                        rowsum_a=ops.rowsum_i8(da) if zp_b else None, out_dtype=td,
+                        bias=None if bias is None else dev(bias))
+    got = got.reshape(nb, m, n)
+    for i in range(nb):
+        want = orc.qdq_matmul_int8(a[i], b[i], sa.reshape(-1, 1) if c["sa_row"] else sa[0],
+                                   sb if c["sb_col"] else sb[0], zp_a, zp_b, orc.F32)
+        if bias is not None:
+            want = want + bias[None, :]
+        if c["out"] == "f32":
+            assert np.array_equal(got[i].cpu().numpy().view(np.uint32), want.view(np.uint32))
+        else:
+            ot = orc.F16 if c["out"] == "f16" else orc.BF16
+            assert np.array_equal(half_bits(got[i]), orc.convert(want, orc.F32, ot))
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_fp8_seeded_sweep_over_every_dispatch_path(ops, seed):
+    """The same sweep for fp8 e4m3fn operands (amax-quantized normal data): the float result stays
+    within the tolerance of the fp8 matrix instructions whichever kernel runs, with and without the
+    scaling epilogue."""
+    c = _sweep_case(100 + seed)
+    rng, m, n, k = c["rng"], c["m"], c["n"], c["k"]
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    xq = orc.quantizelinear(x, np.float32(max(np.abs(x).max(), 1e-3) / 448), None, orc.F32, orc.FP8)
+    wq = orc.quantizelinear(w, np.float32(max(np.abs(w).max(), 1e-3) / 448), None, orc.F32, orc.FP8)
+    da = dev(np.ascontiguousarray(xq.T)).t() if c["trans_a"] else dev(xq)
+    db = dev(np.ascontiguousarray(wq.T)).t() if c["trans_b"] else dev(wq)
+    print("fp8 sweep", seed, {x_: c[x_] for x_ in c if x_ != "rng"}, flush=True)
+    bound = _fp8_bound(xq, wq)
+    if not c["dequant"]:
+        got = ops.quant_dot(da, db, fp8=True).cpu().numpy()
+        assert _fp8_close(got, orc.quant_dot(xq, wq, orc.FP8), bound).all()
+        return
+    sa = np.float32(0.013)
+    sb = rng.uniform(0.001, 0.01, n if c["sb_col"] else 1).astype(np.float32)
+    want = orc.qdq_matmul_fp8(xq, wq, sa, sb if c["sb_col"] else sb[0], orc.F32)
+    got = ops.quant_dot(da, db, fp8=True, scale_a=dev(np.float32([sa])), scale_b=dev(sb),
+                        out_dtype=torch.float32).cpu().numpy()
+    assert _fp8_close(got, want, bound * float(sa) * (sb[None, :] if c["sb_col"] else float(sb[0]))).all()
+
+
 @pytest.mark.parametrize("m,n,k", [(5, 7, 3), (64, 48, 300), (130, 257, 96)])
 def test_uint8_quant_dot_bare(ops, m, n, k):
     """uint8 x uint8 -> int32 (op/quant_dot.hpp:62-64): exact, also for a transposed B view and
