@@ -90,6 +90,61 @@ __global__ __launch_bounds__(256) void im2col_kernel(im2col_params p)
     }
 }
 
+// The same matrix from a channels-last copy of the input (xt[n][y][x][c]) when every group has a
+// multiple of 16 channels: the window elements are ordered (window row, window column, channel),
+// so a 16-byte piece of a row is 16 consecutive channels of one input position -- one aligned
+// 16-byte load and one 16-byte store per thread, neighbouring threads on neighbouring pieces.
+// I: the type of the index arithmetic (32-bit when every count fits, which the launcher checks;
+// the byte offsets themselves are always 64-bit)
+template <class I>
+__global__ __launch_bounds__(256) void im2col_cl_kernel(im2col_params p)
+{
+    const I pieces = (I)(p.kp / 16);
+    const I plane  = (I)(p.oh * p.ow);
+    const I ow = (I)p.ow, group = (I)p.group, cg = (I)p.cg, kw = (I)p.kw;
+    const I total = (I)p.rows * group * pieces;
+    const I step  = (I)gridDim.x * 256;
+    for(I t = (I)blockIdx.x * 256 + threadIdx.x; t < total; t += step)
+    {
+        const I piece = t % pieces;
+        const I rg    = t / pieces;
+        const I g     = rg % group;
+        const I row   = rg / group;
+        const I pos   = row % plane;
+        const I n     = row / plane;
+        const I k     = piece * 16;
+        uint4 v       = make_uint4(0, 0, 0, 0);
+        if(k < (I)p.kg)
+        {
+            const I rq = k / cg;
+            const I c0 = k % cg;
+            const int64_t iy = (int64_t)(pos / ow) * p.stride_h - p.pad_h + (int64_t)(rq / kw) * p.dil_h;
+            const int64_t ix = (int64_t)(pos % ow) * p.stride_w - p.pad_w + (int64_t)(rq % kw) * p.dil_w;
+            if(iy >= 0 && iy < p.h && ix >= 0 && ix < p.w)
+                v = *reinterpret_cast<const uint4*>(p.x + (((int64_t)n * p.h + iy) * p.w + ix) * p.c +
+                                                    (int64_t)g * p.cg + c0);
+        }
+        *reinterpret_cast<uint4*>(p.col + (((int64_t)n * p.group + g) * plane + pos) * p.kp + k) = v;
+    }
+}
+
+// weights [O][Cg][KH*KW] -> rows of kp bytes in (window position, channel) order, zero filled
+__global__ __launch_bounds__(256) void weights_cl_kernel(
+    const uint8_t* w, uint8_t* out, int64_t o, int64_t cg, int64_t win, int64_t kp)
+{
+    const int64_t total = o * kp;
+    const int64_t step  = (int64_t)gridDim.x * 256;
+    for(int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += step)
+    {
+        const int64_t k  = t % kp;
+        const int64_t oc = t / kp;
+        uint8_t v        = 0;
+        if(k < cg * win)
+            v = w[(oc * cg + k % cg) * win + k / cg];
+        out[t] = v;
+    }
+}
+
 int64_t out_len(int64_t in, int64_t k, int64_t pad_lo, int64_t pad_hi, int64_t stride, int64_t dil)
 {
     const int64_t span = in - (1 + dil * (k - 1)) + pad_lo + pad_hi;
@@ -138,7 +193,7 @@ extern "C" int mi355_quant_convolution_dims(const mi355_quant_conv_desc* d,
     if(ow != nullptr)
         *ow = w_out;
     if(workspace_bytes != nullptr)
-        *workspace_bytes = (size_t)((d->n * d->group * h_out * w_out + d->o) * kp);
+        *workspace_bytes = (size_t)((d->n * d->group * h_out * w_out + d->o) * kp + d->n * d->c * d->h * d->w);
     return MI355_OK;
 }
 
@@ -194,8 +249,38 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
     uint8_t* col        = static_cast<uint8_t*>(workspace);
     uint8_t* wp         = col + d->n * d->group * plane * kp;
 
+    uint8_t* xt         = wp + d->o * kp; // channels-last copy of the input, when that form is used
+    // every group a multiple of 16 channels and a real window: gather through a channels-last copy
+    const bool channels_last = cg % 16 == 0 && d->kh * d->kw > 1 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    if(channels_last)
+    {
+        // [N][C][H*W] -> [N][H*W][C]: the window kernel with a 1 x 1 window and K = C does exactly this
+        im2col_params t{};
+        t.x        = static_cast<const uint8_t*>(x);
+        t.col      = xt;
+        t.rows     = d->n * d->h * d->w;
+        t.c        = d->c;
+        t.h        = d->h;
+        t.w        = d->w;
+        t.cg       = d->c;
+        t.kh       = 1;
+        t.kw       = 1;
+        t.oh       = d->h;
+        t.ow       = d->w;
+        t.stride_h = 1;
+        t.stride_w = 1;
+        t.dil_h    = 1;
+        t.dil_w    = 1;
+        t.group    = 1;
+        t.kg       = d->c;
+        t.kp       = d->c;
+        launch_im2col(t, hs);
+        if(mi355_launch_status() != MI355_OK)
+            return MI355_ERR_LAUNCH;
+    }
+
     im2col_params p{};
-    p.x        = static_cast<const uint8_t*>(x);
+    p.x        = channels_last ? xt : static_cast<const uint8_t*>(x);
     p.col      = col;
     p.rows     = d->n * plane;
     p.c        = d->c;
@@ -215,14 +300,38 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
     p.group    = d->group;
     p.kg       = kg;
     p.kp       = kp;
-    launch_im2col(p, hs);
+    if(channels_last)
+    {
+        const int64_t total = p.rows * p.group * (kp / 16);
+        int64_t blocks      = (total + 255) / 256;
+        if(blocks > 256 * 64)
+            blocks = 256 * 64;
+        if(total + blocks * 256 < ((int64_t)1 << 31))
+            hipLaunchKernelGGL(im2col_cl_kernel<uint32_t>, dim3((unsigned)blocks), dim3(256), 0, hs, p);
+        else
+            hipLaunchKernelGGL(im2col_cl_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, hs, p);
+    }
+    else
+        launch_im2col(p, hs);
     if(mi355_launch_status() != MI355_OK)
         return MI355_ERR_LAUNCH;
 
     // the weights as O rows of Kp bytes: a 1 x 1 "convolution window" over [O, Kg, 1, 1]; rows that
     // already have that length (and a 16-byte aligned start) are used where they are
-    const bool pad_weights = kg != kp || reinterpret_cast<uintptr_t>(w) % 16 != 0;
-    const uint8_t* wmat    = pad_weights ? wp : static_cast<const uint8_t*>(w);
+    const bool pad_weights = !channels_last && (kg != kp || reinterpret_cast<uintptr_t>(w) % 16 != 0);
+    const uint8_t* wmat    = (pad_weights || channels_last) ? wp : static_cast<const uint8_t*>(w);
+    if(channels_last)
+    {
+        // the same element order as the window matrix
+        const int64_t total = d->o * kp;
+        int64_t blocks      = (total + 255) / 256;
+        if(blocks > 256 * 16)
+            blocks = 256 * 16;
+        hipLaunchKernelGGL(weights_cl_kernel, dim3((unsigned)blocks), dim3(256), 0, hs,
+                           static_cast<const uint8_t*>(w), wp, d->o, cg, d->kh * d->kw, kp);
+        if(mi355_launch_status() != MI355_OK)
+            return MI355_ERR_LAUNCH;
+    }
     im2col_params q{};
     q.x        = static_cast<const uint8_t*>(w);
     q.col      = wp;

@@ -38,6 +38,10 @@ CASES = [
     ((2, 5, 1, 40), (7, 5, 1, 5), (0, 2), (1, 3), (1, 1), 1),          # one-dimensional
     ((1, 20, 6, 6), (300, 20, 3, 3), (0, 0), (1, 1), (1, 1), 1),       # more than one row tile of weights
     ((2, 8, 9, 10), (8, 8, 3, 3), (0, 1, 2, 0), (2, 2), (1, 1), 1),    # low and high padding differ
+    # 16 | channels per group: the window matrix is gathered from a channels-last copy
+    ((2, 64, 9, 11), (32, 32, 3, 2), (1, 0, 2, 1), (2, 1), (1, 2), 2),
+    ((1, 16, 7, 7), (5, 16, 5, 5), (2, 2), (1, 1), (1, 1), 1),         # K = 400 -> 448
+    ((3, 48, 6, 5), (7, 48, 2, 2), (0, 0), (1, 1), (1, 1), 1),
 ]
 
 
