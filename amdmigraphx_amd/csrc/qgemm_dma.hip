@@ -225,7 +225,6 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     // waits below.  Each fragment is tied ("+v") into the s_waitcnt statement
     // that must precede its first use, which is what orders the MFMAs.
     constexpr int A_TILES = FP8 ? 2 : 4;
-    constexpr int A_PARTS = FP8 ? 2 : 1; // 16-byte reads per K-contiguous fragment
     const int lrow        = lane & 31;
     const int lgrp        = lane >> 5;
     const int tr_i        = lane & 15;
