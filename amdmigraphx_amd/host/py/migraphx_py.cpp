@@ -7,6 +7,7 @@
 #include <pybind11/stl.h>
 #include <migraphx/make_op.hpp>
 #include <migraphx/mi355/target.hpp>
+#include <migraphx/onnx.hpp>
 #include <migraphx/ops.hpp>
 #include <migraphx/passes.hpp>
 #include <migraphx/program.hpp>
@@ -347,6 +348,13 @@ PYBIND11_MODULE(migraphx, m)
         .def("__ne__", [](const migraphx::program& a, const migraphx::program& b) { return a != b; })
         .def("__repr__", [](const migraphx::program& p) { return to_string(p); });
 
+    // src/py/migraphx_py.cpp:699-760 (static shapes; the keyword arguments for dynamic shapes and
+    // default dimensions are not part of this build)
+    m.def("parse_onnx", [](const std::string& filename) { return migraphx::parse_onnx(filename); },
+          "Parse onnx file", py::arg("filename"));
+    m.def("parse_onnx_buffer",
+          [](const py::bytes& buffer) { return migraphx::parse_onnx_buffer(std::string(buffer)); },
+          "Parse onnx file from a buffer", py::arg("onnx_buffer"));
     m.def("get_target", &get_target);
     m.def("create_argument", [](const shape& s, const std::vector<double>& values) {
         if(values.size() != s.elements())

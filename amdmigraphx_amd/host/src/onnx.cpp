@@ -1,0 +1,774 @@
+#include <migraphx/onnx.hpp>
+#include <migraphx/make_op.hpp>
+#include <migraphx/ops.hpp>
+#include <migraphx/passes.hpp>
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <map>
+#include <numeric>
+#include <sstream>
+#include <unordered_map>
+
+namespace migraphx {
+
+namespace {
+
+// ---- protobuf wire format ----------------------------------------------------------------------
+// A message is a sequence of (field number << 3 | wire type) keys, each followed by a varint (0),
+// eight bytes (1), a length and that many bytes (2) or four bytes (5).
+struct wire
+{
+    const unsigned char* p;
+    const unsigned char* end;
+
+    bool done() const { return p >= end; }
+
+    uint64_t varint()
+    {
+        uint64_t r = 0;
+        for(int shift = 0; shift < 64; shift += 7)
+        {
+            if(p >= end)
+                MIGRAPHX_THROW("parse_onnx: truncated varint");
+            const unsigned char b = *p++;
+            r |= static_cast<uint64_t>(b & 0x7f) << shift;
+            if((b & 0x80) == 0)
+                return r;
+        }
+        MIGRAPHX_THROW("parse_onnx: varint too long");
+    }
+
+    wire bytes()
+    {
+        const uint64_t n = varint();
+        if(n > static_cast<uint64_t>(end - p))
+            MIGRAPHX_THROW("parse_onnx: length-delimited field runs past the end");
+        wire r{p, p + n};
+        p += n;
+        return r;
+    }
+
+    std::string str()
+    {
+        wire w = bytes();
+        return {reinterpret_cast<const char*>(w.p), static_cast<std::size_t>(w.end - w.p)};
+    }
+
+    template <class T>
+    T fixed()
+    {
+        if(sizeof(T) > static_cast<std::size_t>(end - p))
+            MIGRAPHX_THROW("parse_onnx: truncated fixed-width field");
+        T v;
+        std::memcpy(&v, p, sizeof(T));
+        p += sizeof(T);
+        return v;
+    }
+
+    // next key; false at the end of the message
+    bool next(uint32_t& field, uint32_t& type)
+    {
+        if(done())
+            return false;
+        const uint64_t key = varint();
+        field              = static_cast<uint32_t>(key >> 3);
+        type               = static_cast<uint32_t>(key & 7);
+        return true;
+    }
+
+    void skip(uint32_t type)
+    {
+        switch(type)
+        {
+        case 0: varint(); break;
+        case 1: fixed<uint64_t>(); break;
+        case 2: bytes(); break;
+        case 5: fixed<uint32_t>(); break;
+        default: MIGRAPHX_THROW("parse_onnx: unsupported wire type " + std::to_string(type));
+        }
+    }
+
+    // repeated scalar field: packed (one length-delimited run) or one element per key
+    template <class F>
+    void repeated(uint32_t type, uint32_t element_type, F f)
+    {
+        if(type == 2 and element_type != 2)
+        {
+            wire run = bytes();
+            while(not run.done())
+                f(run);
+        }
+        else
+        {
+            f(*this);
+        }
+    }
+};
+
+// ---- the ONNX messages, reduced to the fields read here (onnx.proto field numbers) -------------
+struct tensor_proto
+{
+    std::vector<int64_t> dims;
+    int data_type = 0;
+    std::string name;
+    std::string raw;
+    std::vector<float> floats;
+    std::vector<int64_t> ints; // int32_data and int64_data
+    std::vector<double> doubles;
+};
+
+struct attribute_proto
+{
+    std::string name;
+    float f   = 0;
+    int64_t i = 0;
+    std::string s;
+    tensor_proto t;
+    std::vector<float> floats;
+    std::vector<int64_t> ints;
+};
+
+struct node_proto
+{
+    std::vector<std::string> inputs;
+    std::vector<std::string> outputs;
+    std::string name;
+    std::string op_type;
+    std::string domain;
+    std::map<std::string, attribute_proto> attributes;
+};
+
+struct value_info
+{
+    std::string name;
+    int elem_type = 0;
+    std::vector<int64_t> dims;
+    bool has_shape = false;
+};
+
+tensor_proto read_tensor(wire w)
+{
+    tensor_proto t;
+    uint32_t field = 0;
+    uint32_t type  = 0;
+    while(w.next(field, type))
+    {
+        switch(field)
+        {
+        case 1: w.repeated(type, 0, [&](wire& r) { t.dims.push_back(static_cast<int64_t>(r.varint())); }); break;
+        case 2: t.data_type = static_cast<int>(w.varint()); break;
+        case 4: w.repeated(type, 5, [&](wire& r) { t.floats.push_back(r.fixed<float>()); }); break;
+        case 5:
+            // int32 values are sign-extended to 64 bits on the wire
+            w.repeated(type, 0, [&](wire& r) { t.ints.push_back(static_cast<int32_t>(r.varint())); });
+            break;
+        case 7: w.repeated(type, 0, [&](wire& r) { t.ints.push_back(static_cast<int64_t>(r.varint())); }); break;
+        case 8: t.name = w.str(); break;
+        case 9: t.raw = w.str(); break;
+        case 10: w.repeated(type, 1, [&](wire& r) { t.doubles.push_back(r.fixed<double>()); }); break;
+        case 13: MIGRAPHX_THROW("parse_onnx: tensors with external data are not supported");
+        default: w.skip(type);
+        }
+    }
+    return t;
+}
+
+attribute_proto read_attribute(wire w)
+{
+    attribute_proto a;
+    uint32_t field = 0;
+    uint32_t type  = 0;
+    while(w.next(field, type))
+    {
+        switch(field)
+        {
+        case 1: a.name = w.str(); break;
+        case 2: a.f = w.fixed<float>(); break;
+        case 3: a.i = static_cast<int64_t>(w.varint()); break;
+        case 4: a.s = w.str(); break;
+        case 5: a.t = read_tensor(w.bytes()); break;
+        case 7: w.repeated(type, 5, [&](wire& r) { a.floats.push_back(r.fixed<float>()); }); break;
+        case 8: w.repeated(type, 0, [&](wire& r) { a.ints.push_back(static_cast<int64_t>(r.varint())); }); break;
+        default: w.skip(type);
+        }
+    }
+    return a;
+}
+
+node_proto read_node(wire w)
+{
+    node_proto n;
+    uint32_t field = 0;
+    uint32_t type  = 0;
+    while(w.next(field, type))
+    {
+        switch(field)
+        {
+        case 1: n.inputs.push_back(w.str()); break;
+        case 2: n.outputs.push_back(w.str()); break;
+        case 3: n.name = w.str(); break;
+        case 4: n.op_type = w.str(); break;
+        case 5: {
+            auto a               = read_attribute(w.bytes());
+            n.attributes[a.name] = a;
+            break;
+        }
+        case 7: n.domain = w.str(); break;
+        default: w.skip(type);
+        }
+    }
+    return n;
+}
+
+value_info read_value_info(wire w)
+{
+    value_info v;
+    uint32_t field = 0;
+    uint32_t type  = 0;
+    while(w.next(field, type))
+    {
+        if(field == 1)
+            v.name = w.str();
+        else if(field == 2)
+        {
+            // TypeProto { tensor_type = 1 { elem_type = 1; shape = 2 { dim = 1 { dim_value = 1 } } } }
+            wire tp = w.bytes();
+            uint32_t f2 = 0, t2 = 0;
+            while(tp.next(f2, t2))
+            {
+                if(f2 != 1)
+                {
+                    tp.skip(t2);
+                    continue;
+                }
+                wire tt = tp.bytes();
+                uint32_t f3 = 0, t3 = 0;
+                while(tt.next(f3, t3))
+                {
+                    if(f3 == 1)
+                        v.elem_type = static_cast<int>(tt.varint());
+                    else if(f3 == 2)
+                    {
+                        v.has_shape = true;
+                        wire sh = tt.bytes();
+                        uint32_t f4 = 0, t4 = 0;
+                        while(sh.next(f4, t4))
+                        {
+                            if(f4 != 1)
+                            {
+                                sh.skip(t4);
+                                continue;
+                            }
+                            wire dim    = sh.bytes();
+                            int64_t val = -1; // a symbolic or missing dimension
+                            uint32_t f5 = 0, t5 = 0;
+                            while(dim.next(f5, t5))
+                            {
+                                if(f5 == 1)
+                                    val = static_cast<int64_t>(dim.varint());
+                                else
+                                    dim.skip(t5);
+                            }
+                            v.dims.push_back(val);
+                        }
+                    }
+                    else
+                        tt.skip(t3);
+                }
+            }
+        }
+        else
+            w.skip(type);
+    }
+    return v;
+}
+
+// onnx.proto TensorProto.DataType -> shape::type_t (src/onnx/onnx_parser.cpp get_type)
+shape::type_t get_type(int dtype)
+{
+    switch(dtype)
+    {
+    case 1: return shape::float_type;
+    case 2: return shape::uint8_type;
+    case 3: return shape::int8_type;
+    case 4: return shape::uint16_type;
+    case 5: return shape::int16_type;
+    case 6: return shape::int32_type;
+    case 7: return shape::int64_type;
+    case 9: return shape::bool_type;
+    case 10: return shape::half_type;
+    case 11: return shape::double_type;
+    case 12: return shape::uint32_type;
+    case 13: return shape::uint64_type;
+    case 16: return shape::bf16_type;
+    case 17: return shape::fp8e4m3fn_type;
+    default: MIGRAPHX_THROW("parse_onnx: unsupported tensor data type " + std::to_string(dtype));
+    }
+}
+
+literal make_literal(const tensor_proto& t)
+{
+    const auto type = get_type(t.data_type);
+    std::vector<std::size_t> lens(t.dims.begin(), t.dims.end());
+    const shape s = lens.empty() ? shape{type} : shape{type, lens};
+    if(not t.raw.empty())
+    {
+        if(t.raw.size() != s.bytes())
+            MIGRAPHX_THROW("parse_onnx: raw_data of '" + t.name + "' has " + std::to_string(t.raw.size()) +
+                           " bytes, the shape needs " + std::to_string(s.bytes()));
+        return literal{s, t.raw.data()};
+    }
+    if(s.elements() == 0)
+        return literal{s, std::vector<float>{}};
+    switch(type)
+    {
+    case shape::float_type: return literal{s, t.floats};
+    case shape::double_type: return literal{s, t.doubles};
+    case shape::half_type:
+    case shape::bf16_type:
+    case shape::fp8e4m3fn_type: {
+        // the typed fields hold the bit patterns of these types
+        argument a{s};
+        for(std::size_t i = 0; i < t.ints.size() and i < s.elements(); i++)
+        {
+            const auto bits = static_cast<uint16_t>(t.ints[i]);
+            std::memcpy(a.data() + i * s.type_size(), &bits, s.type_size());
+        }
+        return literal{s, a.data()};
+    }
+    default: return literal{s, t.ints};
+    }
+}
+
+// ---- node parsers -------------------------------------------------------------------------------
+struct node_info
+{
+    const node_proto* node;
+    module* mod;
+    bool has(const std::string& a) const { return node->attributes.count(a) > 0; }
+    const attribute_proto& attr(const std::string& a) const { return node->attributes.at(a); }
+};
+
+using node_parser = std::function<instruction_ref(const node_info&, const std::vector<instruction_ref>&)>;
+
+std::string lens_string(const std::vector<std::size_t>& l)
+{
+    std::stringstream ss;
+    for(std::size_t i = 0; i < l.size(); i++)
+        ss << (i == 0 ? "" : ", ") << l[i];
+    return ss.str();
+}
+
+int64_t tune_axis(std::size_t rank, int64_t axis, const std::string& op_name)
+{
+    if(axis < -static_cast<int64_t>(rank) or axis >= static_cast<int64_t>(rank))
+        MIGRAPHX_THROW(op_name + ": axis is out of range.");
+    return axis < 0 ? axis + static_cast<int64_t>(rank) : axis;
+}
+
+// scale and zero point brought to x's dimensions:
+// src/op/builder/include/migraphx/op/builder/quantize_dequantize_linear.hpp:38-150
+std::vector<instruction_ref> transform_qdq_inputs(
+    module& m, const std::string& op_name, int64_t block_size, int64_t axis, std::vector<instruction_ref> args)
+{
+    const auto x_lens       = args.at(0)->get_shape().lens();
+    const auto x_rank       = x_lens.size();
+    const auto y_scale_lens = args.at(1)->get_shape().lens();
+    auto for_params = [&](auto f) {
+        for(std::size_t i = 1; i < args.size(); i++)
+            args[i] = f(args[i]);
+    };
+    if(args.at(1)->get_shape().elements() == 1)
+    {
+        // one value for the tensor
+        for_params([&](instruction_ref ins) {
+            return m.add_instruction(make_op("multibroadcast", {{"out_lens", x_lens}}), ins);
+        });
+    }
+    else if(y_scale_lens.size() == 1)
+    {
+        // one value per index of `axis`
+        axis = tune_axis(x_rank, axis, op_name);
+        if(x_lens[axis] != y_scale_lens[0])
+            MIGRAPHX_THROW(op_name + ": For per axis granularity the length of y_scale (actual: " +
+                           std::to_string(y_scale_lens[0]) + ") must be equal to size of x on axis " +
+                           std::to_string(axis) + "(actual: " + std::to_string(x_lens[axis]) + ")");
+        std::vector<int64_t> unsqueeze_axes(x_rank);
+        std::iota(unsqueeze_axes.begin(), unsqueeze_axes.end(), 0);
+        unsqueeze_axes.erase(unsqueeze_axes.begin() + axis);
+        for_params([&](instruction_ref ins) {
+            auto u = m.add_instruction(make_op("unsqueeze", {{"axes", unsqueeze_axes}}), ins);
+            return m.add_instruction(make_op("multibroadcast", {{"out_lens", x_lens}}), u);
+        });
+    }
+    else
+    {
+        // one value per block of `block_size` elements along `axis`
+        axis = tune_axis(x_rank, axis, op_name);
+        if(x_rank != y_scale_lens.size())
+            MIGRAPHX_THROW(op_name + ": x(rank: " + std::to_string(x_rank) + ") and y_scale(rank: " +
+                           std::to_string(y_scale_lens.size()) + ") must be of same rank for block granularity");
+        for(std::size_t i = 0; i < x_rank; i++)
+        {
+            if(x_lens[i] != y_scale_lens[i] and static_cast<int64_t>(i) != axis)
+                MIGRAPHX_THROW(op_name + ": x(shape: " + lens_string(x_lens) + ") and y_scale(shape: " +
+                               lens_string(y_scale_lens) + ") shapes may only differ along provided axis(" +
+                               std::to_string(axis) + ")");
+        }
+        const float di = static_cast<float>(x_lens[axis]);
+        const float si = static_cast<float>(y_scale_lens[axis]);
+        if(si <= 1.0f)
+            MIGRAPHX_THROW(op_name + ": y_scale(shape: " + lens_string(y_scale_lens) +
+                           ") must have size > 1 along provided axis(" + std::to_string(axis) +
+                           ") for block granularity");
+        const auto block_size_min = static_cast<int64_t>(std::ceil(di / si));
+        const auto block_size_max = static_cast<int64_t>(std::ceil(di / (si - 1))) - 1;
+        if(block_size == 0)
+            block_size = block_size_min;
+        if(block_size < block_size_min or block_size > block_size_max)
+            MIGRAPHX_THROW(op_name + ": Block size(actual: " + std::to_string(block_size) +
+                           ") must be within range [" + std::to_string(block_size_min) + ", " +
+                           std::to_string(block_size_max) + "]");
+        for_params([&](instruction_ref ins) {
+            if(block_size == 1)
+                return ins;
+            ins          = m.add_instruction(make_op("unsqueeze", {{"axes", {axis + 1}}}), ins);
+            auto bc_lens = ins->get_shape().lens();
+            bc_lens[axis + 1] = static_cast<std::size_t>(block_size);
+            ins = m.add_instruction(make_op("multibroadcast", {{"out_lens", bc_lens}}), ins);
+            std::vector<int64_t> reshape_lens(x_lens.begin(), x_lens.end());
+            reshape_lens[axis] = static_cast<int64_t>(ins->get_shape().lens()[axis]) * block_size;
+            ins = m.add_instruction(make_op("reshape", {{"dims", reshape_lens}}), ins);
+            if(static_cast<int64_t>(x_lens[axis]) < reshape_lens[axis]) // runt block
+                ins = m.add_instruction(
+                    make_op("slice", {{"axes", {axis}}, {"starts", {0}}, {"ends", {x_lens[axis]}}}), ins);
+            return ins;
+        });
+    }
+    return args;
+}
+
+// src/onnx/parse_dequantizelinear.cpp:41-81
+instruction_ref parse_dequantizelinear(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 2 or args.size() > 3)
+        MIGRAPHX_THROW("DequantizeLinear: must have either 2 or 3 inputs, " + std::to_string(args.size()) +
+                       " inputs provided");
+    if(args.size() == 3)
+    {
+        if(args[0]->get_shape().type() != args[2]->get_shape().type())
+            MIGRAPHX_THROW("DequantizeLinear: x and y_zero_point must be of same type");
+        if(args[1]->get_shape().lens() != args[2]->get_shape().lens())
+            MIGRAPHX_THROW("DequantizeLinear: y_scale and y_zero_point shape mismatch. Provided y_scale shape: " +
+                           lens_string(args[1]->get_shape().lens()) + ", provided y_zero_point shape: " +
+                           lens_string(args[2]->get_shape().lens()));
+    }
+    const int64_t axis  = info.has("axis") ? info.attr("axis").i : 1;
+    const int64_t block = info.has("block_size") ? info.attr("block_size").i : 0;
+    auto a = transform_qdq_inputs(*info.mod, "dequantizelinear", block, axis, args);
+    return info.mod->add_instruction(make_op("dequantizelinear"), a);
+}
+
+// src/onnx/parse_quantizelinear.cpp:40-100, src/op/builder/quantizelinear.cpp:86-116
+instruction_ref parse_quantizelinear(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 2 or args.size() > 3)
+        MIGRAPHX_THROW("QuantizeLinear: must have either 2 or 3 inputs, " + std::to_string(args.size()) +
+                       " input(s) provided");
+    if(args.size() == 3 and args[1]->get_shape().lens() != args[2]->get_shape().lens())
+        MIGRAPHX_THROW("QuantizeLinear: y_scale and y_zero_point shapes must be equal. Provided y_scale shape: " +
+                       lens_string(args[1]->get_shape().lens()) + ", provided y_zero_point shape: " +
+                       lens_string(args[2]->get_shape().lens()));
+    const int64_t axis  = info.has("axis") ? info.attr("axis").i : 1;
+    const int64_t block = info.has("block_size") ? info.attr("block_size").i : 0;
+    int64_t out_type    = -1;
+    if(info.has("output_dtype"))
+    {
+        out_type = get_type(static_cast<int>(info.attr("output_dtype").i));
+        if(args.size() == 3 and static_cast<shape::type_t>(out_type) != args[2]->get_shape().type())
+            MIGRAPHX_THROW("QuantizeLinear: output_type and y_zero_point type must match.");
+    }
+    auto a = transform_qdq_inputs(*info.mod, "quantizelinear", block, axis, args);
+    // x and the scale in one type (float wins over half)
+    const auto tx = a[0]->get_shape().type();
+    const auto ts = a[1]->get_shape().type();
+    if(tx != ts)
+    {
+        const auto common = (tx == shape::float_type or ts == shape::float_type) ? shape::float_type : tx;
+        for(int i = 0; i < 2; i++)
+        {
+            if(a[i]->get_shape().type() != common)
+                a[i] = info.mod->add_instruction(make_op("convert", {{"target_type", common}}), a[i]);
+        }
+    }
+    if(out_type >= 0)
+        return info.mod->add_instruction(make_op("quantizelinear", {{"out_type", out_type}}), a);
+    return info.mod->add_instruction(make_op("quantizelinear"), a);
+}
+
+// numpy matmul: a vector operand is a one-row / one-column matrix, leading dimensions broadcast
+// (src/onnx/parse_matmul.cpp:205-330, src/op/builder/include/migraphx/op/builder/broadcast_dimensions.hpp)
+instruction_ref parse_matmul(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() != 2)
+        MIGRAPHX_THROW("MatMul: two inputs expected");
+    module& m   = *info.mod;
+    auto a0     = args[0];
+    auto a1     = args[1];
+    const bool v0 = a0->get_shape().ndim() == 1;
+    const bool v1 = a1->get_shape().ndim() == 1;
+    if(v0)
+        a0 = m.add_instruction(make_op("unsqueeze", {{"axes", {0}}}), a0);
+    if(v1)
+        a1 = m.add_instruction(make_op("unsqueeze", {{"axes", {1}}}), a1);
+    auto l0 = a0->get_shape().lens();
+    auto l1 = a1->get_shape().lens();
+    if(not std::equal(l0.rbegin() + 2, l0.rend(), l1.rbegin() + 2, l1.rend()))
+    {
+        std::vector<std::size_t> b0(l0.begin(), l0.end() - 2);
+        std::vector<std::size_t> b1(l1.begin(), l1.end() - 2);
+        // broadcast the batch dimensions right-aligned
+        const std::size_t nb = std::max(b0.size(), b1.size());
+        std::vector<std::size_t> out(nb, 1);
+        for(std::size_t i = 0; i < nb; i++)
+        {
+            const std::size_t d0 = i < nb - b0.size() ? 1 : b0[i - (nb - b0.size())];
+            const std::size_t d1 = i < nb - b1.size() ? 1 : b1[i - (nb - b1.size())];
+            if(d0 != d1 and d0 != 1 and d1 != 1)
+                MIGRAPHX_THROW("MatMul: batch dimensions {" + lens_string(b0) + "} and {" + lens_string(b1) +
+                               "} do not broadcast");
+            out[i] = std::max(d0, d1);
+        }
+        auto n0 = out;
+        n0.insert(n0.end(), l0.end() - 2, l0.end());
+        auto n1 = out;
+        n1.insert(n1.end(), l1.end() - 2, l1.end());
+        if(l0 != n0)
+            a0 = m.add_instruction(make_op("multibroadcast", {{"out_lens", n0}}), a0);
+        if(l1 != n1)
+            a1 = m.add_instruction(make_op("multibroadcast", {{"out_lens", n1}}), a1);
+    }
+    auto r = m.add_instruction(make_op("dot"), a0, a1);
+    const auto nd = static_cast<int64_t>(r->get_shape().ndim());
+    if(v0)
+        r = m.add_instruction(make_op("squeeze", {{"axes", {nd - 2}}}), r);
+    if(v1)
+        r = m.add_instruction(make_op("squeeze", {{"axes", {v0 ? nd - 2 : nd - 1}}}), r);
+    return r;
+}
+
+// src/onnx/parse_matmulnbits.cpp:42-126
+instruction_ref parse_matmulnbits(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 3 or args.size() > 4)
+        MIGRAPHX_THROW("MatMulNBits: 3 or 4 inputs expected (a, b, scales, zero_points)");
+    for(const char* a : {"N", "K", "bits", "block_size"})
+    {
+        if(not info.has(a))
+            MIGRAPHX_THROW(std::string("MatMulNBits: Attribute ") + a + " is required");
+    }
+    const auto n     = static_cast<std::size_t>(info.attr("N").i);
+    const auto k     = static_cast<std::size_t>(info.attr("K").i);
+    const auto bits  = info.attr("bits").i;
+    const auto block = static_cast<std::size_t>(info.attr("block_size").i);
+    if(bits != 4)
+        MIGRAPHX_THROW("MatMulNBits: bits only supported for value of 4, actual value " + std::to_string(bits));
+    if(args[0]->get_shape().lens().back() != k)
+        MIGRAPHX_THROW("MatMulNBits: Input A last dimension does not match K");
+    return op::builder::matmulnbits(*info.mod, args[0], args[1], args[2],
+                                    args.size() == 4 ? args[3] : info.mod->end(), n, k, block);
+}
+
+instruction_ref parse_binary(const std::string& op, const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() != 2)
+        MIGRAPHX_THROW(info.node->op_type + ": two inputs expected");
+    module& m = *info.mod;
+    auto a    = args[0];
+    auto b    = args[1];
+    // numpy broadcasting of the two operands (src/onnx/onnx_parser.cpp add_broadcastable_binary_op)
+    if(a->get_shape().lens() != b->get_shape().lens())
+    {
+        const auto la = a->get_shape().lens();
+        const auto lb = b->get_shape().lens();
+        const std::size_t nd = std::max(la.size(), lb.size());
+        std::vector<std::size_t> out(nd, 1);
+        for(std::size_t i = 0; i < nd; i++)
+        {
+            const std::size_t da = i < nd - la.size() ? 1 : la[i - (nd - la.size())];
+            const std::size_t db = i < nd - lb.size() ? 1 : lb[i - (nd - lb.size())];
+            if(da != db and da != 1 and db != 1)
+                MIGRAPHX_THROW(info.node->op_type + ": shapes {" + lens_string(la) + "} and {" + lens_string(lb) +
+                               "} do not broadcast");
+            out[i] = std::max(da, db);
+        }
+        if(la != out)
+            a = m.add_instruction(make_op("multibroadcast", {{"out_lens", out}}), a);
+        if(lb != out)
+            b = m.add_instruction(make_op("multibroadcast", {{"out_lens", out}}), b);
+    }
+    return m.add_instruction(make_op(op), a, b);
+}
+
+const std::unordered_map<std::string, node_parser>& parsers()
+{
+    static const std::unordered_map<std::string, node_parser> table = {
+        {"MatMul", parse_matmul},
+        {"MatMulNBits", parse_matmulnbits},
+        {"DequantizeLinear", parse_dequantizelinear},
+        {"QuantizeLinear", parse_quantizelinear},
+        {"Add", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("add", i, a); }},
+        {"Sub", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("sub", i, a); }},
+        {"Mul", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("mul", i, a); }},
+        {"Div", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("div", i, a); }},
+        {"Identity",
+         [](const node_info& i, const std::vector<instruction_ref>& a) {
+             return i.mod->add_instruction(make_op("identity"), a.at(0));
+         }},
+        {"Transpose",
+         [](const node_info& i, const std::vector<instruction_ref>& a) {
+             std::vector<int64_t> perm;
+             if(i.has("perm"))
+                 perm = i.attr("perm").ints;
+             else
+             {
+                 // the default reverses the dimensions
+                 perm.resize(a.at(0)->get_shape().ndim());
+                 std::iota(perm.rbegin(), perm.rend(), 0);
+             }
+             return i.mod->add_instruction(make_op("transpose", {{"permutation", perm}}), a.at(0));
+         }},
+        {"Reshape",
+         [](const node_info& i, const std::vector<instruction_ref>& a) {
+             if(a.size() != 2 or not a[1]->can_eval())
+                 MIGRAPHX_THROW("Reshape: the target shape must be a constant input");
+             auto dims = a[1]->eval().to_vector<int64_t>();
+             // 0 keeps the input's dimension (allowzero = 0)
+             for(std::size_t d = 0; d < dims.size(); d++)
+             {
+                 if(dims[d] == 0 and d < a[0]->get_shape().ndim())
+                     dims[d] = static_cast<int64_t>(a[0]->get_shape().lens()[d]);
+             }
+             auto x = a[0];
+             if(not x->get_shape().standard())
+                 x = i.mod->add_instruction(make_op("contiguous"), x);
+             return i.mod->add_instruction(make_op("reshape", {{"dims", dims}}), x);
+         }},
+    };
+    return table;
+}
+
+program parse_model(wire model)
+{
+    // ModelProto.graph = 7
+    wire graph{nullptr, nullptr};
+    bool found     = false;
+    uint32_t field = 0;
+    uint32_t type  = 0;
+    while(model.next(field, type))
+    {
+        if(field == 7 and type == 2)
+        {
+            graph = model.bytes();
+            found = true;
+        }
+        else
+            model.skip(type);
+    }
+    if(not found)
+        MIGRAPHX_THROW("parse_onnx: Failed reading onnx file.");
+
+    std::vector<node_proto> nodes;
+    std::vector<tensor_proto> initializers;
+    std::vector<value_info> inputs;
+    std::vector<value_info> outputs;
+    while(graph.next(field, type))
+    {
+        switch(field)
+        {
+        case 1: nodes.push_back(read_node(graph.bytes())); break;
+        case 5: initializers.push_back(read_tensor(graph.bytes())); break;
+        case 11: inputs.push_back(read_value_info(graph.bytes())); break;
+        case 12: outputs.push_back(read_value_info(graph.bytes())); break;
+        default: graph.skip(type);
+        }
+    }
+
+    program p;
+    module* mm = p.get_main_module();
+    std::unordered_map<std::string, instruction_ref> values;
+    for(const auto& t : initializers)
+        values[t.name] = mm->add_literal(make_literal(t));
+    for(const auto& in : inputs)
+    {
+        if(values.count(in.name) > 0)
+            continue; // an initializer listed among the inputs
+        if(not in.has_shape)
+            MIGRAPHX_THROW("parse_onnx: input '" + in.name + "' has no shape");
+        std::vector<std::size_t> lens;
+        for(auto d : in.dims)
+        {
+            if(d <= 0)
+                MIGRAPHX_THROW("parse_onnx: input '" + in.name + "' has a dynamic dimension");
+            lens.push_back(static_cast<std::size_t>(d));
+        }
+        const auto t    = get_type(in.elem_type);
+        values[in.name] = mm->add_parameter(in.name, lens.empty() ? shape{t} : shape{t, lens});
+    }
+    for(const auto& n : nodes)
+    {
+        if(n.op_type == "Constant")
+        {
+            if(n.attributes.count("value") == 0)
+                MIGRAPHX_THROW("Constant: only the tensor form (attribute `value`) is supported");
+            values[n.outputs.at(0)] = mm->add_literal(make_literal(n.attributes.at("value").t));
+            continue;
+        }
+        auto it = parsers().find(n.op_type);
+        if(it == parsers().end())
+            MIGRAPHX_THROW("parse_onnx: operator '" + n.op_type + "' is outside the quantized-GEMM path of this build");
+        std::vector<instruction_ref> args;
+        for(const auto& name : n.inputs)
+        {
+            if(name.empty())
+                continue; // an omitted optional input
+            if(values.count(name) == 0)
+                MIGRAPHX_THROW("PARSE_GRAPH: invalid onnx file. Input \"" + name + "\" is unavailable due to unordered nodes!");
+            args.push_back(values.at(name));
+        }
+        values[n.outputs.at(0)] = it->second(node_info{&n, mm}, args);
+    }
+    std::vector<instruction_ref> rets;
+    for(const auto& o : outputs)
+    {
+        if(values.count(o.name) == 0)
+            MIGRAPHX_THROW("parse_onnx: graph output '" + o.name + "' is not produced by any node");
+        rets.push_back(values.at(o.name));
+    }
+    mm->add_return(rets);
+    return p;
+}
+
+} // namespace
+
+program parse_onnx_buffer(const void* data, std::size_t size)
+{
+    const auto* b = static_cast<const unsigned char*>(data);
+    return parse_model(wire{b, b + size});
+}
+
+program parse_onnx_buffer(const std::string& buffer) { return parse_onnx_buffer(buffer.data(), buffer.size()); }
+
+program parse_onnx(const std::string& filename)
+{
+    std::ifstream is(filename, std::ios::binary);
+    if(not is)
+        MIGRAPHX_THROW("parse_onnx: cannot open '" + filename + "'");
+    std::stringstream ss;
+    ss << is.rdbuf();
+    return parse_onnx_buffer(ss.str());
+}
+
+} // namespace migraphx

@@ -7,6 +7,8 @@
 #include "encoder.hpp"
 #include "oracle_target.hpp"
 #include "test.hpp"
+#include <sstream>
+#include <migraphx/onnx.hpp>
 #include <algorithm>
 #include <fstream>
 
@@ -1170,12 +1172,55 @@ static int matmulnbits_tool(int argc, char** argv)
     return 0;
 }
 
+// `host_tests onnx print <model>`: parse and print the program.
+// `host_tests onnx <target> <model> <inputs file> <result file>`: parse, evaluate with the parameter
+// values of the inputs file (one line per parameter: name, then its values) and write every output
+// value on a line of its own.  The Python tests drive it with the reference's ONNX test models.
+static int onnx_tool(int argc, char** argv)
+{
+    if(argc != 4 and argc != 6)
+        return 2;
+    auto p = migraphx::parse_onnx(argv[3]);
+    if(std::string(argv[2]) == "print")
+    {
+        std::cout << p << std::endl;
+        return 0;
+    }
+    if(argc != 6)
+        return 2;
+    std::ifstream in(argv[4]);
+    migraphx::parameter_map params;
+    std::string line;
+    while(std::getline(in, line))
+    {
+        std::stringstream ls(line);
+        std::string name;
+        if(not(ls >> name))
+            continue;
+        std::vector<double> values;
+        double v = 0;
+        while(ls >> v)
+            values.push_back(v);
+        const auto s = p.get_parameter_shape(name);
+        params[name] = argument{shape{s.type(), s.lens()}, values};
+    }
+    auto r = run_on(argv[2], p, params);
+    std::ofstream out(argv[5]);
+    out.precision(17);
+    for(const auto& a : r)
+        for(auto v : a.to_vector<double>())
+            out << v << "\n";
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     try
     {
         if(argc > 1 and std::string(argv[1]) == "matmulnbits")
             return matmulnbits_tool(argc, argv);
+        if(argc > 1 and std::string(argv[1]) == "onnx")
+            return onnx_tool(argc, argv);
         return test::run(argc, argv);
     }
     catch(const std::exception& e)

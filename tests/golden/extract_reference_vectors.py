@@ -316,6 +316,19 @@ c.update(conv_attrs(body, "convolution"))
 conv.append(c)
 out["convolution"] = conv
 
+# ---- ONNX Q/DQ models with their expected outputs (test/onnx/verify/*_blocked_test.cpp) ---------
+onnx_cases = []
+for rel in ("test/onnx/verify/dequantizelinear_blocked_test.cpp", "test/onnx/verify/quantizelinear_blocked_test.cpp"):
+    for name, body in test_cases(read(rel)).items():
+        model = re.search(r'read_onnx\("([^"]+)"\)', body).group(1)
+        c = {"name": name, "source": rel, "model": model, "inputs": {}}
+        # pm["<parameter>"] = migraphx::argument{<var>_shape, <var>.data()};
+        for param, var in re.findall(r'pm\["(\w+)"\]\s*=\s*migraphx::argument\{\w+,\s*(\w+)\.data\(\)\}', body):
+            c["inputs"][param] = vec(body, var)
+        c["gold"] = vec(body, "gold")
+        onnx_cases.append(c)
+out["onnx_qdq"] = onnx_cases
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -51,3 +51,27 @@ def run_matmulnbits(target, case, tmp_path, use_half=False):
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout + r.stderr
     return np.loadtxt(out, dtype=np.float32, ndmin=1)
+
+
+ONNX_DIR = os.path.join(ROOT, "tests", "golden", "onnx")
+
+
+def run_onnx(target, model, inputs, tmp_path):
+    """Parse tests/golden/onnx/<model> with the host layer and evaluate it on `target` with the
+    given parameter values (name -> flat list); returns the outputs as one flat float64 array."""
+    spec = tmp_path / (model + ".in")
+    with open(spec, "w") as f:
+        for name, values in inputs.items():
+            f.write(name + " " + " ".join(repr(float(v)) for v in values) + "\n")
+    out = tmp_path / (model + ".out")
+    r = subprocess.run([HOST_TESTS, "onnx", target, os.path.join(ONNX_DIR, model), str(spec), str(out)],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout + r.stderr
+    return np.loadtxt(out, dtype=np.float64, ndmin=1)
+
+
+def print_onnx(model):
+    """The parsed program as text, or the error message (return code 4) when parsing throws."""
+    r = subprocess.run([HOST_TESTS, "onnx", "print", os.path.join(ONNX_DIR, model)],
+                       capture_output=True, text=True, timeout=600)
+    return r.returncode, r.stdout

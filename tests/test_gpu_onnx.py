@@ -1,0 +1,33 @@
+"""The reference's ONNX test models of the quantized-GEMM path parsed by the host layer, compiled
+for the MI355X target and checked against the reference's expected outputs."""
+import numpy as np
+import pytest
+
+from host_util import ensure_built, run_onnx
+from test_onnx import matmulnbits_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def built():
+    ensure_built()
+
+
+def test_matmulnbits_models_on_device(golden, tmp_path):
+    # test/onnx/verify/matmulnbits_tests.cpp; float models take the bit-exact float dot behind the
+    # device's dequantization, so the tolerance is the reference's own
+    for c in golden["matmulnbits"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["name"] + ".onnx", matmulnbits_inputs(c), tmp_path)
+        np.testing.assert_allclose(got, np.float64(c["gold"]), rtol=1e-5, atol=1e-4, err_msg=c["name"])
+
+
+def test_blocked_quantize_dequantize_models_on_device(golden, tmp_path):
+    for c in golden["onnx_qdq"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], c["inputs"], tmp_path)
+        want = run_onnx("oracle", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == want.tolist(), c["name"]
+        if c["name"].startswith("quantize"):
+            assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
