@@ -581,6 +581,66 @@ instruction_ref parse_matmulnbits(const node_info& info, const std::vector<instr
                                     args.size() == 4 ? args[3] : info.mod->end(), n, k, block);
 }
 
+// scale and zero point spread over x: a vector along `axis`, anything else by multibroadcast
+// (src/onnx/broadcast_qdq.cpp:34-63)
+instruction_ref bcast_qdq(module& m,
+                          const std::string& op_name,
+                          instruction_ref x,
+                          instruction_ref scale,
+                          instruction_ref zp,
+                          std::size_t axis = 0)
+{
+    const auto lens = x->get_shape().lens();
+    auto spread     = [&](instruction_ref q) {
+        if(q->get_shape().ndim() == 1 and q->get_shape().elements() > 1)
+            return m.add_instruction(make_op("broadcast", {{"axis", axis}, {"out_lens", lens}}), q);
+        return m.add_instruction(make_op("multibroadcast", {{"out_lens", lens}}), q);
+    };
+    return m.add_instruction(make_op(op_name), x, spread(scale), spread(zp));
+}
+
+// src/onnx/parse_qlinearmatmul.cpp:93-196: dequantize both operands, dot, quantize the result
+instruction_ref parse_qlinearmatmul(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 8)
+        MIGRAPHX_THROW("QLINEARMATMUL: missing inputs");
+    module& m = *info.mod;
+    auto in_a = args[0];
+    auto in_b = args[3];
+    for(auto x : {in_a, in_b})
+    {
+        const auto t = x->get_shape().type();
+        if(t != shape::int8_type and t != shape::uint8_type)
+            MIGRAPHX_THROW("QLINEARMATMUL: unsupported input type");
+    }
+    auto lens_a = in_a->get_shape().lens();
+    auto lens_b = in_b->get_shape().lens();
+    if(lens_a.empty() or lens_b.empty())
+        MIGRAPHX_THROW("QLINEARMATMUL: empty input");
+    const bool a_vector = lens_a.size() == 1;
+    const bool b_vector = lens_b.size() == 1;
+    if(a_vector)
+        lens_a.insert(lens_a.begin(), 1);
+    if(b_vector)
+        lens_b.push_back(1);
+    if(lens_a.size() != lens_b.size() or lens_a.back() != *(lens_b.rbegin() + 1) or
+       not std::equal(lens_a.rbegin() + 2, lens_a.rend(), lens_b.rbegin() + 2, lens_b.rend()))
+        MIGRAPHX_THROW("QLINEARMATMUL: mismatched input dimensions");
+    const auto nd_a = in_a->get_shape().ndim();
+    auto dq_a = bcast_qdq(m, "dequantizelinear", in_a, args[1], args[2], nd_a >= 2 ? nd_a - 2 : 0);
+    auto dq_b = bcast_qdq(m, "dequantizelinear", in_b, args[4], args[5], in_b->get_shape().ndim() - 1);
+    if(a_vector)
+        dq_a = m.add_instruction(make_op("unsqueeze", {{"axes", {0}}}), dq_a);
+    if(b_vector)
+        dq_b = m.add_instruction(make_op("unsqueeze", {{"axes", {1}}}), dq_b);
+    auto y = m.add_instruction(make_op("dot"), dq_a, dq_b);
+    if(a_vector)
+        y = m.add_instruction(make_op("squeeze", {{"axes", {0}}}), y);
+    else if(b_vector)
+        y = m.add_instruction(make_op("squeeze", {{"axes", {1}}}), y);
+    return bcast_qdq(m, "quantizelinear", y, args[6], args[7]);
+}
+
 instruction_ref parse_binary(const std::string& op, const node_info& info, const std::vector<instruction_ref>& args)
 {
     if(args.size() != 2)
@@ -619,6 +679,7 @@ const std::unordered_map<std::string, node_parser>& parsers()
         {"MatMulNBits", parse_matmulnbits},
         {"DequantizeLinear", parse_dequantizelinear},
         {"QuantizeLinear", parse_quantizelinear},
+        {"QLinearMatMul", parse_qlinearmatmul},
         {"Add", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("add", i, a); }},
         {"Sub", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("sub", i, a); }},
         {"Mul", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("mul", i, a); }},

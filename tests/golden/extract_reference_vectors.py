@@ -329,6 +329,23 @@ for rel in ("test/onnx/verify/dequantizelinear_blocked_test.cpp", "test/onnx/ver
         onnx_cases.append(c)
 out["onnx_qdq"] = onnx_cases
 
+# ---- QLinearMatMul models (test/onnx/verify/qlinearmatmul_*_test.cpp, QLinearMatMul_2d_per_channel_test.cpp)
+qlm = []
+for rel in ("test/onnx/verify/qlinearmatmul_1D_test.cpp", "test/onnx/verify/qlinearmatmul_2D_test.cpp",
+            "test/onnx/verify/qlinearmatmul_3D_test.cpp", "test/onnx/verify/qlinearmatmul_N_D_perchannel_test.cpp",
+            "test/onnx/verify/QLinearMatMul_2d_per_channel_test.cpp"):
+    for name, body in test_cases(read(rel)).items():
+        model = re.search(r'read_onnx\("([^"]+)"\)', body).group(1)
+        c = {"name": name, "source": rel, "model": model, "inputs": {}}
+        for param, var in re.findall(r'pp\["(\w+)"\]\s*=\s*migraphx::argument\(\w+,\s*(\w+)\.data\(\)\)', body):
+            c["inputs"][param] = vec(body, var)
+        c["gold"] = vec(body, "gold")
+        # the 2-D per-channel case builds its input in code and its model holds a 2 MB weight: left out
+        if any(v is None for v in c["inputs"].values()):
+            continue
+        qlm.append(c)
+out["onnx_qlinearmatmul"] = qlm
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -31,3 +31,12 @@ def test_blocked_quantize_dequantize_models_on_device(golden, tmp_path):
         assert got.tolist() == want.tolist(), c["name"]
         if c["name"].startswith("quantize"):
             assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
+
+
+def test_qlinearmatmul_models_on_device(golden, tmp_path):
+    # uint8 operands are no quant_dot inputs of simplify_qdq (int8 and fp8 only), so these run as
+    # dequantize -> float dot -> quantize on the device; the answers are the reference's
+    for c in golden["onnx_qlinearmatmul"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == [float(v) for v in c["gold"]], c["name"]

@@ -39,6 +39,14 @@ def test_blocked_quantize_dequantize_models_reference_known_answers(golden, tmp_
             np.testing.assert_allclose(got, np.float64(c["gold"]), rtol=1e-6, atol=1e-6, err_msg=c["name"])
 
 
+def test_qlinearmatmul_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/qlinearmatmul_{1D,2D,3D,N_D_perchannel}_test.cpp: uint8 results, exact
+    assert len(golden["onnx_qlinearmatmul"]) == 4
+    for c in golden["onnx_qlinearmatmul"]:
+        got = run_onnx("oracle", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
+
+
 def test_per_tensor_and_per_axis_models(tmp_path):
     # test/onnx/parse/dequantizelinear_test.cpp, _zero_point_test, _axis_test, _neg_axis_test: shapes of
     # the models, values against the operator's definition
