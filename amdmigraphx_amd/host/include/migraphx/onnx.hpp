@@ -1,6 +1,6 @@
 // ONNX front end for the quantized-GEMM path: reads a ModelProto from its protobuf wire format and
 // builds a program from the nodes that path consists of -- MatMul, MatMulNBits (com.microsoft),
-// QLinearMatMul, QuantizeLinear, DequantizeLinear (per tensor, per axis, blocked), the float binary operators,
+// QLinearMatMul, Conv, QuantizeLinear, DequantizeLinear (per tensor, per axis, blocked), the float binary operators,
 // Transpose, Reshape, Identity.  Follows src/onnx/onnx_parser.cpp (graph inputs that are not
 // initializers become parameters in input order, initializers become literals, graph outputs the
 // return) and the node parsers named at each operator in onnx.cpp.  Any other operator type

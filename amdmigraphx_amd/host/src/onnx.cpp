@@ -641,6 +641,73 @@ instruction_ref parse_qlinearmatmul(const node_info& info, const std::vector<ins
     return bcast_qdq(m, "quantizelinear", y, args[6], args[7]);
 }
 
+// src/onnx/parse_convolution.cpp:49-106 with the attribute rules of src/op/builder/convolution.cpp:62-113
+// and the SAME_UPPER / SAME_LOWER padding of src/pad_calc.cpp:31-53, :96-120 (static shapes)
+instruction_ref parse_conv(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 2 or args.size() > 3)
+        MIGRAPHX_THROW("Conv: two or three inputs expected");
+    module& m = *info.mod;
+    auto x    = args[0];
+    auto w    = args[1];
+    if(x->get_shape().ndim() < 3 or w->get_shape().ndim() != x->get_shape().ndim())
+        MIGRAPHX_THROW("Conv: input and weights need the same rank of at least 3");
+    const std::size_t kdims = x->get_shape().ndim() - 2;
+    std::string auto_pad    = "NOTSET";
+    if(info.has("auto_pad"))
+    {
+        auto_pad = info.attr("auto_pad").s;
+        for(auto& ch : auto_pad)
+            ch = static_cast<char>(std::toupper(static_cast<unsigned char>(ch)));
+    }
+    if(info.has("pads") and auto_pad != "NOTSET")
+        MIGRAPHX_THROW("PARSE_CONV: auto_pad and padding cannot be specified simultaneously");
+    auto attr_or = [&](const char* name, int64_t fill) {
+        std::vector<int64_t> v = info.has(name) ? info.attr(name).ints : std::vector<int64_t>(kdims, fill);
+        return v;
+    };
+    auto strides   = attr_or("strides", 1);
+    auto dilations = attr_or("dilations", 1);
+    auto paddings  = attr_or("pads", 0);
+    if(strides.size() != kdims)
+        MIGRAPHX_THROW("Inconsistent strides size, is: " + std::to_string(strides.size()) +
+                       ", should be: " + std::to_string(kdims));
+    if(dilations.size() != kdims)
+        MIGRAPHX_THROW("Inconsistent dilations size, is: " + std::to_string(dilations.size()) +
+                       ", should be: " + std::to_string(kdims));
+    if(paddings.size() != kdims and paddings.size() != 2 * kdims)
+        MIGRAPHX_THROW("Inconsistent paddings size, is: " + std::to_string(paddings.size()) +
+                       ", should be: " + std::to_string(kdims) + " or: " + std::to_string(2 * kdims));
+    if(auto_pad.find("SAME") != std::string::npos)
+    {
+        const bool upper = auto_pad.find("SAME_UPPER") != std::string::npos;
+        paddings.assign(2 * kdims, 0);
+        for(std::size_t i = 0; i < kdims; i++)
+        {
+            const auto in_dim  = static_cast<int64_t>(x->get_shape().lens()[i + 2]);
+            const auto k_dim   = static_cast<int64_t>(w->get_shape().lens()[i + 2]);
+            const auto out_dim = (in_dim + strides[i] - 1) / strides[i];
+            const auto k_eff   = k_dim + (k_dim - 1) * (dilations[i] - 1);
+            const auto pad     = std::max<int64_t>(0, (out_dim - 1) * strides[i] + k_eff - in_dim);
+            paddings[upper ? i : i + kdims] = pad / 2;
+            paddings[upper ? i + kdims : i] = pad - pad / 2;
+        }
+    }
+    const int64_t group = info.has("group") ? info.attr("group").i : 1;
+    auto conv = m.add_instruction(
+        make_op("convolution",
+                {{"padding", paddings}, {"stride", strides}, {"dilation", dilations}, {"group", group}}),
+        x, w);
+    if(args.size() == 3)
+    {
+        if(args[2]->get_shape().ndim() != 1 or args[2]->get_shape().lens()[0] != conv->get_shape().lens()[1])
+            MIGRAPHX_THROW("Conv: the bias must be a vector with one value per output channel");
+        auto b = m.add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", conv->get_shape().lens()}}), args[2]);
+        return m.add_instruction(make_op("add"), conv, b);
+    }
+    return conv;
+}
+
 instruction_ref parse_binary(const std::string& op, const node_info& info, const std::vector<instruction_ref>& args)
 {
     if(args.size() != 2)
@@ -680,6 +747,7 @@ const std::unordered_map<std::string, node_parser>& parsers()
         {"DequantizeLinear", parse_dequantizelinear},
         {"QuantizeLinear", parse_quantizelinear},
         {"QLinearMatMul", parse_qlinearmatmul},
+        {"Conv", parse_conv},
         {"Add", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("add", i, a); }},
         {"Sub", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("sub", i, a); }},
         {"Mul", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("mul", i, a); }},

@@ -131,9 +131,25 @@ bool is_valid_qparam(instruction_ref q, const std::vector<std::size_t>& lens, st
 
 operation qparam_broadcast_op(instruction_ref q, const std::vector<std::size_t>& lens, std::size_t axis)
 {
-    if(q->get_shape().scalar())
+    // one value: spread it whatever shape it came in (a scalar, or the [1] tensor of an ONNX
+    // initializer)
+    if(q->get_shape().scalar() or q->get_shape().elements() == 1)
         return make_op("multibroadcast", {{"out_lens", lens}});
     return make_op("broadcast", {{"out_lens", lens}, {"axis", axis}});
+}
+
+// A per-axis parameter that arrives with unit dimensions around its axis (the ONNX parsers
+// unsqueeze a vector to the tensor's rank before they broadcast it) as the vector `broadcast`
+// takes.  The reference leaves this to the passes that run in front of simplify_qdq on its
+// targets; here the pass does it itself.
+instruction_ref as_vector(module& m, instruction_ref pos, instruction_ref q)
+{
+    const auto& s = q->get_shape();
+    if(s.scalar() or s.ndim() <= 1)
+        return q;
+    if(not s.standard())
+        q = m.insert_instruction(pos, make_op("contiguous"), q);
+    return m.insert_instruction(pos, make_op("reshape", {{"dims", {static_cast<int64_t>(s.elements())}}}), q);
 }
 
 bool is_symmetric_zero_point(instruction_ref zp)
@@ -189,6 +205,8 @@ void find_quantizable_dot(module& m, instruction_ref qop)
         if(not(scale1->get_shape().elements() == 1 and zp1->get_shape().elements() == 1 and
                is_valid_qparam(scale2, arg2_lens, 0) and is_valid_qparam(zp2, arg2_lens, 0)))
             return;
+        scale2 = as_vector(m, qop, scale2);
+        zp2    = as_vector(m, qop, zp2);
         auto s1 = m.insert_instruction(qop, qparam_broadcast_op(scale1, conv_lens, 1), scale1);
         auto s2 = m.insert_instruction(qop, qparam_broadcast_op(scale2, conv_lens, 1), scale2);
         auto conv_scale = m.insert_instruction(qop, make_op("mul"), s1, s2);
@@ -228,6 +246,10 @@ void find_quantizable_dot(module& m, instruction_ref qop)
     if(not(is_valid_qparam(scale1, out_lens, nd - 2) and is_valid_qparam(zp1, out_lens, nd - 2) and
            is_valid_qparam(scale2, out_lens, nd - 1) and is_valid_qparam(zp2, out_lens, nd - 1)))
         return;
+    scale1 = as_vector(m, qop, scale1);
+    zp1    = as_vector(m, qop, zp1);
+    scale2 = as_vector(m, qop, scale2);
+    zp2    = as_vector(m, qop, zp2);
 
     auto s1_bcast = m.insert_instruction(qop, qparam_broadcast_op(scale1, out_lens, nd - 2), scale1);
     auto s2_bcast = m.insert_instruction(qop, qparam_broadcast_op(scale2, out_lens, nd - 1), scale2);

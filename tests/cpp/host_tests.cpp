@@ -1173,20 +1173,23 @@ static int matmulnbits_tool(int argc, char** argv)
 }
 
 // `host_tests onnx print <model>`: parse and print the program.
-// `host_tests onnx <target> <model> <inputs file> <result file>`: parse, evaluate with the parameter
-// values of the inputs file (one line per parameter: name, then its values) and write every output
-// value on a line of its own.  The Python tests drive it with the reference's ONNX test models.
+// `host_tests onnx <target> <model> <inputs file> <result file> [simplify_qdq]`: parse (and, when asked,
+// run simplify_qdq as the mi355 target does on its own), evaluate with the parameter values of the
+// inputs file (one line per parameter: name, then its values) and write every output value on a
+// line of its own.  The Python tests drive it with the reference's ONNX test models.
 static int onnx_tool(int argc, char** argv)
 {
-    if(argc != 4 and argc != 6)
+    if(argc != 4 and argc != 6 and argc != 7)
         return 2;
     auto p = migraphx::parse_onnx(argv[3]);
+    if(argc == 7 and std::string(argv[6]) == "simplify_qdq")
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
     if(std::string(argv[2]) == "print")
     {
         std::cout << p << std::endl;
         return 0;
     }
-    if(argc != 6)
+    if(argc < 6)
         return 2;
     std::ifstream in(argv[4]);
     migraphx::parameter_map params;

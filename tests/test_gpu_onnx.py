@@ -40,3 +40,28 @@ def test_qlinearmatmul_models_on_device(golden, tmp_path):
         print("onnx", c["name"], flush=True)
         got = run_onnx("mi355", c["model"], c["inputs"], tmp_path)
         assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
+
+
+def test_written_qdq_conv_model_on_device(tmp_path):
+    """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
+    turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU
+    target on the same input."""
+    import subprocess
+    import host_util
+    from test_onnx import qdq_conv_model
+    rng = np.random.default_rng(3)
+    data, _, _, _ = qdq_conv_model(rng)
+    path = tmp_path / "qdq_conv.onnx"
+    path.write_bytes(data)
+    x = rng.standard_normal((2, 4, 9, 9)).astype(np.float32)
+    spec = tmp_path / "in.txt"
+    spec.write_text("x " + " ".join(repr(float(v)) for v in x.flatten()) + "\n")
+    results = {}
+    for target in ("oracle", "mi355"):
+        out = tmp_path / (target + ".txt")
+        # the CPU target evaluates what it is given, so it gets the graph simplify_qdq leaves
+        r = subprocess.run([host_util.HOST_TESTS, "onnx", target, str(path), str(spec), str(out), "simplify_qdq"],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stdout + r.stderr
+        results[target] = np.loadtxt(out)
+    assert results["mi355"].tolist() == results["oracle"].tolist()

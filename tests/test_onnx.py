@@ -121,3 +121,66 @@ def test_python_module_parses_files_and_buffers():
         mgx.parse_onnx_buffer(b"\x3a\x7f\x01")      # a graph field that claims more bytes than there are
     with pytest.raises(RuntimeError):
         mgx.parse_onnx(os.path.join(ONNX_DIR, "no_such_file.onnx"))
+
+
+def qdq_conv_model(rng):
+    """x float -> Q/DQ (one scale) ; int8 weights with one scale per output channel -> DQ (axis 0) ;
+    Conv with SAME_UPPER padding, stride 2 and a bias: what a QDQ-format quantized CNN layer holds."""
+    import onnx_writer as ow
+    w = rng.integers(-127, 128, (6, 4, 3, 3), dtype=np.int8)
+    sw = rng.uniform(0.002, 0.01, 6).astype(np.float32)
+    bias = rng.standard_normal(6).astype(np.float32)
+    inits = [("w", w), ("sw", sw), ("zw", np.zeros(6, np.int8)), ("sx", np.float32([0.05])),
+             ("zx", np.zeros(1, np.int8)), ("bias", bias)]
+    nodes = [ow.node("QuantizeLinear", ["x", "sx", "zx"], ["xq"]),
+             ow.node("DequantizeLinear", ["xq", "sx", "zx"], ["xd"]),
+             ow.node("DequantizeLinear", ["w", "sw", "zw"], ["wd"], axis=0),
+             ow.node("Conv", ["xd", "wd", "bias"], ["y"], auto_pad="SAME_UPPER", strides=[2, 2])]
+    data = ow.model(nodes, [("x", ow.FLOAT, [2, 4, 9, 9])], [("y", ow.FLOAT, [2, 6, 5, 5])], inits)
+    return data, w, sw, bias
+
+
+def test_written_qdq_conv_model_parses_and_matches_the_definition(tmp_path):
+    import os
+    from oracle import oracle as orc
+    rng = np.random.default_rng(3)
+    data, w, sw, bias = qdq_conv_model(rng)
+    path = tmp_path / "qdq_conv.onnx"
+    path.write_bytes(data)
+    import host_util
+    x = rng.standard_normal((2, 4, 9, 9)).astype(np.float32)
+    spec = tmp_path / "in.txt"
+    spec.write_text("x " + " ".join(repr(float(v)) for v in x.flatten()) + "\n")
+    out = tmp_path / "out.txt"
+    import subprocess
+    r = subprocess.run([host_util.HOST_TESTS, "onnx", "oracle", str(path), str(spec), str(out)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.loadtxt(out).reshape(2, 6, 5, 5)
+    xq = orc.quantizelinear(x.reshape(-1, 9), np.float32(0.05), np.int8(0), orc.F32, orc.I8).reshape(x.shape)
+    xd = xq.astype(np.float32) * np.float32(0.05)
+    wd = w.astype(np.float32) * sw[:, None, None, None]
+    # SAME_UPPER for 9 -> 5 with stride 2 and a 3-wide window: one zero in front, one behind
+    want = orc.convolution(xd, wd, orc.F32, (1, 1, 1, 1), (2, 2)) + bias[None, :, None, None]
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("model,fragment", [
+    # test/onnx/parse/conv_1d_test.cpp, conv_bias_test.cpp, conv_autopad_same_test.cpp
+    ("conv_1d_test.onnx", "convolution[padding=[0],stride=[1],dilation=[1]"),
+    ("conv_bias_test.onnx", "broadcast[axis=1,out_lens=[1, 1, 28, 28]]"),
+    ("conv_autopad_same_test.onnx", "convolution[padding=[1, 1, 1, 1],stride=[1, 1],dilation=[1, 1]"),
+])
+def test_conv_models_structure(model, fragment):
+    rc, text = print_onnx(model)
+    assert rc == 0 and fragment in text, text
+
+
+@pytest.mark.parametrize("model,message", [
+    ("conv_autopad_fail_test.onnx", "auto_pad and padding cannot be specified simultaneously"),
+    ("conv_attr_fail_test.onnx", "Inconsistent strides size, is: 2, should be: 1"),
+    ("conv_bad_bias_test.onnx", "Types do not match"),
+])
+def test_malformed_conv_models_are_rejected(model, message):
+    rc, text = print_onnx(model)
+    assert rc == 4 and message in text, text
