@@ -65,3 +65,22 @@ def test_written_qdq_conv_model_on_device(tmp_path):
         assert r.returncode == 0, r.stdout + r.stderr
         results[target] = np.loadtxt(out)
     assert results["mi355"].tolist() == results["oracle"].tolist()
+
+
+def test_written_qdq_matmul_model_on_device(tmp_path):
+    """BASELINE config 1 from ONNX bytes through the Python surface: one fused quant_dot launch
+    (dequantize and bias in its epilogue), bit-identical to the oracle."""
+    from oracle import oracle as orc
+    from amdmigraphx_amd import migraphx as mgx
+    from test_onnx import qdq_matmul_model
+    rng = np.random.default_rng(4)
+    data, w, sw, bias = qdq_matmul_model(rng, m=256, k=1024, n=1024)
+    p = mgx.parse_onnx_buffer(data)
+    p.compile(mgx.get_target("gpu"))
+    text = repr(p)
+    assert text.count("mi355::quant_dot") == 1 and "mi355::binary" not in text and "mi355::chain" not in text
+    x = rng.standard_normal((256, 1024)).astype(np.float32)
+    got = np.array(p.run({"x": x})[0])
+    xq = orc.quantizelinear(x, np.float32(1.0 / 32), np.int8(0), orc.F32, orc.I8)
+    want = orc.qdq_matmul_int8(xq, w, np.float32(1.0 / 32), sw) + bias[None, :]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -184,3 +184,51 @@ def test_conv_models_structure(model, fragment):
 def test_malformed_conv_models_are_rejected(model, message):
     rc, text = print_onnx(model)
     assert rc == 4 and message in text, text
+
+
+def qdq_matmul_model(rng, m=64, k=256, n=128, with_bias=True):
+    """BASELINE config 1 as a QDQ-format ONNX model: x float -> Q/DQ (scale 1/32) ; int8 weights with
+    one scale per output column -> DQ (axis 1) ; MatMul ; Add of a bias."""
+    import onnx_writer as ow
+    w = rng.integers(-127, 128, (k, n), dtype=np.int8)
+    sw = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    inits = [("w", w), ("sw", sw), ("zw", np.zeros(n, np.int8)), ("sx", np.float32([1.0 / 32])),
+             ("zx", np.zeros(1, np.int8)), ("bias", bias)]
+    nodes = [ow.node("QuantizeLinear", ["x", "sx", "zx"], ["xq"]),
+             ow.node("DequantizeLinear", ["xq", "sx", "zx"], ["xd"]),
+             ow.node("DequantizeLinear", ["w", "sw", "zw"], ["wd"], axis=1),
+             ow.node("MatMul", ["xd", "wd"], ["mm"])]
+    out = "mm"
+    if with_bias:
+        nodes.append(ow.node("Add", ["mm", "bias"], ["y"]))
+        out = "y"
+    data = ow.model(nodes, [("x", ow.FLOAT, [m, k])], [(out, ow.FLOAT, [m, n])], inits)
+    return data, w, sw, bias
+
+
+def test_written_qdq_matmul_model_becomes_quant_dot(tmp_path):
+    from oracle import oracle as orc
+    mgx = pytest.importorskip("amdmigraphx_amd.migraphx")
+    rng = np.random.default_rng(4)
+    data, w, sw, bias = qdq_matmul_model(rng)
+    p = mgx.parse_onnx_buffer(data)
+    assert p.get_parameter_shapes()["x"] == mgx.shape(type="float", lens=[64, 256])
+    text = repr(p)
+    assert text.count("dequantizelinear") == 2 and "dot(" in text and "quant_dot" not in text
+    # on the CPU target the parsed graph gives the fake-quantized product
+    import subprocess
+    import host_util
+    path = tmp_path / "qdq_matmul.onnx"
+    path.write_bytes(data)
+    x = rng.standard_normal((64, 256)).astype(np.float32)
+    spec = tmp_path / "in.txt"
+    spec.write_text("x " + " ".join(repr(float(v)) for v in x.flatten()) + "\n")
+    out = tmp_path / "out.txt"
+    r = subprocess.run([host_util.HOST_TESTS, "onnx", "oracle", str(path), str(spec), str(out), "simplify_qdq"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.loadtxt(out).reshape(64, 128).astype(np.float32)
+    xq = orc.quantizelinear(x, np.float32(1.0 / 32), np.int8(0), orc.F32, orc.I8)
+    want = orc.qdq_matmul_int8(xq, w, np.float32(1.0 / 32), sw) + bias[None, :]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
