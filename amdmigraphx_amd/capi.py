@@ -49,6 +49,9 @@ EXPORTS = {
                                [ctypes.c_size_t, ctypes.c_void_p],
     "mi355_quant_dot": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 8,
     "mi355_quant_dot_bias": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9,
+    "mi355_quant_dot_workspace_size": [ctypes.POINTER(QuantDotDesc)],
+    "mi355_quant_dot_ws": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9 +
+                          [ctypes.c_size_t, ctypes.c_void_p],
     "mi355_colsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                         ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p],
     "mi355_rowsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
@@ -128,7 +131,8 @@ def lib():
         for name, argtypes in EXPORTS.items():
             fn = getattr(h, name)
             fn.argtypes = argtypes
-            fn.restype = ctypes.c_char_p if name == "mi355_status_string" else ctypes.c_int
+            fn.restype = (ctypes.c_char_p if name == "mi355_status_string" else
+                          ctypes.c_size_t if name == "mi355_quant_dot_workspace_size" else ctypes.c_int)
         _handle = h
     return _handle
 

@@ -58,6 +58,8 @@ struct dma_params
     int scale_a_mode, scale_b_mode;
     int zp_a, zp_b;
     int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
+    int32_t* partial; // split-K with a workspace: share z of batch b writes its tile sums to
+                      // partial[(b * ksplit + z)][m][n] with plain stores; null = atomic adds into C
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
     int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
 };
@@ -1001,10 +1003,19 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                 int32_t* o = static_cast<int32_t*>(p.c) + idx;
                 if constexpr(SPLITK)
                 {
+                    if(p.partial != nullptr)
+                    {
+                        int32_t* w = p.partial +
+                                     (((int64_t)blockIdx.y * p.ksplit + blockIdx.z) * p.m + row) * p.n + col;
+                        *reinterpret_cast<v4i*>(w) = acc[i][j];
+                    }
+                    else
+                    {
 #pragma unroll
-                    for(int e = 0; e < 4; e++)
-                        __hip_atomic_fetch_add(o + e, acc[i][j][e], __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
+                        for(int e = 0; e < 4; e++)
+                            __hip_atomic_fetch_add(o + e, acc[i][j][e], __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
                 else if constexpr(VEC_STORE)
                     *reinterpret_cast<v4i*>(o) = acc[i][j];
@@ -1077,14 +1088,111 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* c, int m, int n,
         base[(i / n) * ldc + (i % n)] = 0;
 }
 
+// Second kernel of the split-K with a workspace: C = epilogue(sum of the shares' partial tiles).
+// A thread column (threadIdx.x) owns 4 adjacent outputs; the 4 waves of a workgroup (threadIdx.y)
+// each add every fourth share and the first one collects the four sums through the LDS.  Integer
+// sums: any order gives the same bits; the dequantizing epilogue is the arithmetic of the one-pass
+// kernel's.  N, ldc and the batch stride of C are multiples of 4 on this path.
+template <bool DEQ, int OUT>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int shares)
+{
+    __shared__ v4i part[3][64];
+    const int64_t mn    = (int64_t)p.m * p.n;
+    const int64_t q     = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    const bool inside   = 4 * q < mn;
+    const int32_t* src  = p.partial + (int64_t)blockIdx.y * p.ksplit * mn + 4 * q;
+    v4i sum             = {0, 0, 0, 0};
+    if(inside)
+    {
+#pragma unroll 4
+        for(int z = threadIdx.y; z < shares; z += 4)
+            sum += *reinterpret_cast<const v4i*>(src + (int64_t)z * mn);
+    }
+    if(threadIdx.y > 0)
+        part[threadIdx.y - 1][threadIdx.x] = sum;
+    __syncthreads();
+    if(threadIdx.y != 0 || !inside)
+        return;
+    sum += part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x];
+    const int row     = (int)(4 * q / p.n);
+    const int col     = (int)(4 * q % p.n);
+    const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+    if constexpr(!DEQ)
+        *reinterpret_cast<v4i*>(static_cast<int32_t*>(p.c) + idx) = sum;
+    else
+    {
+        float sa = 1.f;
+        if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+            sa = p.scale_a[0];
+        else if(p.scale_a_mode == MI355_QP_PER_ROW)
+            sa = p.scale_a[row];
+        const int64_t zrow =
+            p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
+        float v[4];
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+        {
+            float sb = 1.f;
+            if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                sb = p.scale_b[0];
+            else if(p.scale_b_mode == MI355_QP_PER_COL)
+                sb = p.scale_b[col + e];
+            const int32_t cs = p.zp_a != 0 ? p.colsum_b[col + e] : 0;
+            const float bias = p.bias != nullptr ? p.bias[col + e] : -0.0f;
+            const float s    = sa * sb;
+            const double d   = (double)sum[e] - (double)(int32_t)(zrow + (int64_t)p.zp_a * cs);
+            v[e]             = add_bias((float)(d * (double)s), bias);
+        }
+        if constexpr(OUT == MI355_F32)
+            *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) = v4f{v[0], v[1], v[2], v[3]};
+        else if constexpr(OUT == MI355_F16)
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) =
+                make_uint2(convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                           convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+        else
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) =
+                make_uint2(convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
+                           convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+    }
+}
+
+template <bool DEQ, int OUT>
+void launch_reduce(const dma_params& p, int batch, int shares, hipStream_t stream)
+{
+    const int64_t quads = (int64_t)p.m * p.n / 4;
+    hipLaunchKernelGGL((reduce_partials_kernel<DEQ, OUT>), dim3((unsigned)((quads + 63) / 64), batch),
+                       dim3(64, 4), 0, stream, p, shares);
+}
+
+// deq / out_type: the epilogue of the second kernel on the workspace path (the atomic path gives
+// the bare int32 product only)
 template <bool TRANS_B>
-int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream)
+int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream, bool deq = false, int out_type = MI355_F32)
 {
     auto kern = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true>;
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if(attr != hipSuccess)
         return MI355_ERR_LAUNCH;
+    if(p.partial != nullptr)
+    {
+        dim3 grid(p.tiles_m * p.tiles_n, batch, p.ksplit);
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+        // shares that hold slabs: the kernel gives ceil(nk / ksplit) slabs to each, the last ones
+        // may be left with none (they write nothing)
+        const int nk     = p.k / BK;
+        const int per    = (nk + p.ksplit - 1) / p.ksplit;
+        const int shares = (nk + per - 1) / per;
+        if(!deq)
+            launch_reduce<false, MI355_F32>(p, batch, shares, stream);
+        else if(out_type == MI355_F32)
+            launch_reduce<true, MI355_F32>(p, batch, shares, stream);
+        else if(out_type == MI355_F16)
+            launch_reduce<true, MI355_F16>(p, batch, shares, stream);
+        else
+            launch_reduce<true, MI355_BF16>(p, batch, shares, stream);
+        return mi355_launch_status();
+    }
     const int64_t total = (int64_t)p.m * p.n;
     const int zb        = (int)min((int64_t)2048, (total + 255) / 256);
     hipLaunchKernelGGL(zero_i32_kernel, dim3(zb, batch), dim3(256), 0, stream,
@@ -1111,6 +1219,21 @@ int choose_ksplit(int tiles, int batch, int nk, int64_t m, int64_t n, int64_t k)
     s                  = min(s, nk / 4); // at least four slabs per share keep the LDS ring busy
     s                  = min((int64_t)s, (512 + wgs - 1) / wgs);
     return max(s, 1);
+}
+
+// The same choice when the shares write partial tiles to a workspace and a second kernel adds them
+// up: no atomics, so the cost of a share is writing and reading its M x N partial sums once; as
+// many shares as keep every CU busy twice over, at least four slabs each, and not so many that the
+// partial sums outweigh the operands.
+int choose_ksplit_ws(int tiles, int batch, int nk, int64_t m, int64_t n, int64_t k)
+{
+    const int64_t wgs = (int64_t)tiles * batch;
+    if(wgs >= 128 || nk < 8)
+        return 1;
+    int64_t s = (512 + wgs - 1) / wgs;
+    s         = min(s, (int64_t)nk / 4);
+    s         = min(s, (m * k + k * n) / (8 * m * n));
+    return (int)max(s, (int64_t)1);
 }
 
 template <bool TRANS_B, bool VEC>
@@ -1181,6 +1304,18 @@ bool mi355_dma_gemm_supported(const mi355_quant_dot_desc* d, const void* a, cons
     return true;
 }
 
+// bytes of workspace that would let an int8 quant_dot of this description (bare or dequantizing)
+// split K without atomics (0: no use for one)
+size_t mi355_dma_gemm_workspace(const mi355_quant_dot_desc* d)
+{
+    if(d->in_type != MI355_I8 || d->trans_a || d->k % BK != 0 || d->k < BK || d->n % 4 != 0 ||
+       d->ldc % 4 != 0 || d->stride_c % 4 != 0 || d->m <= 0 || d->n <= 0 || d->batch <= 0)
+        return 0;
+    const int tiles = (int)(((d->m + BM - 1) / BM) * ((d->n + BN - 1) / BN));
+    const int s     = choose_ksplit_ws(tiles, (int)d->batch, (int)(d->k / BK), d->m, d->n, d->k);
+    return s > 1 ? (size_t)s * d->batch * d->m * d->n * 4 : 0;
+}
+
 int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                           const void* a,
                           const void* b,
@@ -1190,10 +1325,13 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                           const int32_t* colsum_b,
                           const int32_t* rowsum_a,
                           const float* bias,
+                          void* workspace,
+                          size_t workspace_bytes,
                           hipStream_t stream)
 {
     dma_params p;
     p.bias         = bias;
+    p.partial      = nullptr;
     p.a            = static_cast<const uint8_t*>(a);
     p.b            = static_cast<const uint8_t*>(b);
     p.c            = c;
@@ -1240,6 +1378,18 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
         return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
     p.ksplit = 1;
+    if(vec && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+       (!deq || d->out_type == MI355_F32 || d->out_type == MI355_F16 || d->out_type == MI355_BF16))
+    {
+        const int s = choose_ksplit_ws(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);
+        if(s > 1 && (size_t)s * d->batch * d->m * d->n * 4 <= workspace_bytes)
+        {
+            p.ksplit  = s;
+            p.partial = static_cast<int32_t*>(workspace);
+            return d->trans_b ? launch_i8_splitk<true>(p, (int)d->batch, stream, deq, d->out_type)
+                              : launch_i8_splitk<false>(p, (int)d->batch, stream, deq, d->out_type);
+        }
+    }
     if(vec && !deq)
     {
         p.ksplit = choose_ksplit(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);

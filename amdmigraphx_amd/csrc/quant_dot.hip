@@ -24,7 +24,10 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc*,
                           const int32_t*,
                           const int32_t*,
                           const float*,
+                          void*,
+                          size_t,
                           hipStream_t);
+size_t mi355_dma_gemm_workspace(const mi355_quant_dot_desc*);
 
 namespace {
 
@@ -214,6 +217,27 @@ extern "C" int mi355_quant_dot_bias(const mi355_quant_dot_desc* d,
                                     const float* bias,
                                     void* stream)
 {
+    return mi355_quant_dot_ws(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, nullptr, 0, stream);
+}
+
+extern "C" size_t mi355_quant_dot_workspace_size(const mi355_quant_dot_desc* d)
+{
+    return d == nullptr ? 0 : mi355_dma_gemm_workspace(d);
+}
+
+extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
+                                  const void* a,
+                                  const void* b,
+                                  void* c,
+                                  const float* scale_a,
+                                  const float* scale_b,
+                                  const int32_t* colsum_b,
+                                  const int32_t* rowsum_a,
+                                  const float* bias,
+                                  void* workspace,
+                                  size_t workspace_bytes,
+                                  void* stream)
+{
     if(d == nullptr)
         return MI355_ERR_BAD_ARG;
     if(d->m < 0 || d->n < 0 || d->k < 0 || d->batch < 0)
@@ -273,7 +297,7 @@ extern "C" int mi355_quant_dot_bias(const mi355_quant_dot_desc* d,
     // int8 with N % 4 != 0 would take the DMA path's 32 x 32 kernel, which applies no bias
     const bool dma_has_bias = bias == nullptr || fp8 || d->n % 4 == 0;
     if(!u8 && d->k > 0 && dma_has_bias && mi355_dma_gemm_supported(d, a, b))
-        return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
+        return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, workspace, workspace_bytes, s);
     if(!u8 && d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
         return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
 

@@ -82,6 +82,7 @@ struct quant_dot
 {
     bool dequant           = false;
     bool has_bias          = false;
+    bool workspace         = false; // a uint8 buffer before `out` (mi355_quant_dot_workspace_size)
     int64_t zp_a           = 0;
     int64_t zp_b           = 0;
     int64_t scale_a_mode   = MI355_QP_NONE;
@@ -92,6 +93,7 @@ struct quant_dot
     {
         f(self.dequant, "dequant");
         f(self.has_bias, "has_bias");
+        f(self.workspace, "workspace");
         f(self.zp_a, "zp_a");
         f(self.zp_b, "zp_b");
         f(self.scale_a_mode, "scale_a_mode");
@@ -101,8 +103,10 @@ struct quant_dot
     std::string name() const { return "mi355::quant_dot"; }
     std::size_t expected_inputs() const
     {
-        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0) + (has_bias ? 1 : 0);
+        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0) + (has_bias ? 1 : 0) +
+               (workspace ? 1 : 0);
     }
+    mi355_quant_dot_desc describe(const shape& a, const shape& b) const;
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }

@@ -186,6 +186,18 @@ bool is_column_bias(instruction_ref x, const std::vector<std::size_t>& lens)
            base->get_shape().elements() == lens.back();
 }
 
+// A skinny int8 product splits K over the chip when it is given room for the partial sums: ask
+// the library how much this shape can use and pass it as one more buffer.
+void add_dot_workspace(module& m, instruction_ref pos, quant_dot& op, std::vector<instruction_ref>& args)
+{
+    const auto d      = op.describe(args[0]->get_shape(), args[1]->get_shape());
+    const size_t need = mi355_quant_dot_workspace_size(&d);
+    if(need == 0)
+        return;
+    op.workspace = true;
+    args.push_back(insert_allocation(m, pos, shape{shape::uint8_type, {need}}));
+}
+
 bool fuse_quant_dot_dq(module& m, instruction_ref dq)
 {
     if(dq->name() != "dequantizelinear")
@@ -308,6 +320,7 @@ bool fuse_quant_dot_dq(module& m, instruction_ref dq)
     }
     if(has_bias)
         args.push_back(bias);
+    add_dot_workspace(m, last, op, args);
     args.push_back(insert_allocation(m, last, shape{out_type, qd->get_shape().lens()}));
     m.replace_instruction(last, operation{op}, args);
     return true;
@@ -821,7 +834,10 @@ void lower_instruction(module& m, instruction_ref ins)
             b = make_standard(m, ins, b);
         quant_dot op;
         op.out_type = ins->get_shape().type();
-        m.replace_instruction(ins, operation{op}, a, b, standard_out());
+        std::vector<instruction_ref> args = {a, b};
+        add_dot_workspace(m, ins, op, args);
+        args.push_back(standard_out());
+        m.replace_instruction(ins, operation{op}, args);
     }
     else if(name == "quant_convolution")
     {

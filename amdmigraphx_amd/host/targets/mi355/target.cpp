@@ -263,9 +263,11 @@ shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
         if((zp_a != 0 or zp_b != 0) and inputs[0].type() != shape::int8_type)
             MIGRAPHX_THROW("mi355::quant_dot: zero points need int8 operands");
     }
+    if(workspace and inputs[inputs.size() - 2].type() != shape::uint8_type)
+        MIGRAPHX_THROW("mi355::quant_dot: the workspace must be a uint8 buffer");
     if(has_bias)
     {
-        const shape& bias = inputs[inputs.size() - 2];
+        const shape& bias = inputs[inputs.size() - (workspace ? 3 : 2)];
         if(not dequant)
             MIGRAPHX_THROW("mi355::quant_dot: a bias needs the dequantizing epilogue");
         if(bias.type() != shape::float_type or not bias.standard() or bias.elements() != s.lens().back())
@@ -277,10 +279,10 @@ shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
     return out;
 }
 
-argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+mi355_quant_dot_desc quant_dot::describe(const shape& a, const shape& b) const
 {
-    const auto va = view_as_matrix(args[0].get_shape());
-    const auto vb = view_as_matrix(args[1].get_shape());
+    const auto va = view_as_matrix(a);
+    const auto vb = view_as_matrix(b);
     mi355_quant_dot_desc d{};
     d.m        = va.rows;
     d.k        = va.cols;
@@ -294,13 +296,19 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     d.stride_a = va.batch_stride;
     d.stride_b = vb.batch_stride;
     d.stride_c = d.m * d.n;
-    d.in_type  = to_mi355_type(args[0].get_shape().type());
+    d.in_type  = to_mi355_type(a.type());
     d.out_type = to_mi355_type(out_type);
     d.dequant  = dequant ? 1 : 0;
     d.scale_a_mode = static_cast<int32_t>(scale_a_mode);
     d.scale_b_mode = static_cast<int32_t>(scale_b_mode);
     d.zp_a         = static_cast<int32_t>(zp_a);
     d.zp_b         = static_cast<int32_t>(zp_b);
+    return d;
+}
+
+argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto d     = describe(args[0].get_shape(), args[1].get_shape());
     std::size_t next = 2;
     const float* sa  = nullptr;
     const float* sb  = nullptr;
@@ -314,16 +322,20 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     const float* bias = has_bias ? reinterpret_cast<const float*>(args[next++].data()) : nullptr;
     if((zp_a != 0 or zp_b != 0) and d.batch != 1)
         MIGRAPHX_THROW("mi355::quant_dot: zero points with batched operands are not supported");
-    status_check(mi355_quant_dot_bias(&d,
-                                      args[0].data(),
-                                      args[1].data(),
-                                      args.back().data(),
-                                      sa,
-                                      sb,
-                                      colsum_b,
-                                      rowsum_a,
-                                      bias,
-                                      stream_of(ctx)),
+    void* ws             = workspace ? args[next].data() : nullptr;
+    const size_t ws_size = workspace ? args[next].get_shape().bytes() : 0;
+    status_check(mi355_quant_dot_ws(&d,
+                                    args[0].data(),
+                                    args[1].data(),
+                                    args.back().data(),
+                                    sa,
+                                    sb,
+                                    colsum_b,
+                                    rowsum_a,
+                                    bias,
+                                    ws,
+                                    ws_size,
+                                    stream_of(ctx)),
                  name());
     return args.back();
 }

@@ -46,7 +46,7 @@ def _mat_layout(t):
 
 
 def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
-              colsum_b=None, rowsum_a=None, out_dtype=None, out=None, bias=None):
+              colsum_b=None, rowsum_a=None, out_dtype=None, out=None, bias=None, workspace=None):
     """quant_dot, optionally with the fused dequantizelinear epilogue.
 
     a [..., M, K], b [..., K, N] int8 (or uint8 carrying fp8 e4m3fn bits with
@@ -55,8 +55,10 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     bare accumulators come back (int32 / float32).  With ``scale_a`` (scalar
     or [M]) / ``scale_b`` (scalar or [N]) float32 tensors the epilogue
     (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied; ``bias`` (float32 [N])
-    is then added in float32, before the conversion to a 16-bit ``out_dtype``."""
-    _require_cuda(a, b, scale_a, scale_b, bias)
+    is then added in float32, before the conversion to a 16-bit ``out_dtype``.
+    ``workspace`` (any dense device tensor, see quant_dot_workspace_size) lets a skinny int8
+    product, bare or with the epilogue, split K over the chip without atomics."""
+    _require_cuda(a, b, scale_a, scale_b, bias, workspace)
     if a.dim() != b.dim() or a.dim() < 2:
         raise Mi355Error("QUANT_DOT: dot only accepts >= 2D operands of equal rank")
     if a.shape[:-2] != b.shape[:-2]:
@@ -113,14 +115,30 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
             raise Mi355Error("quant_dot: a bias needs the dequantizing epilogue")
         if bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous():
             raise Mi355Error("bias must be a dense float32 vector of N elements")
+    if workspace is not None:
+        if not workspace.is_contiguous():
+            raise Mi355Error("the workspace must be dense")
+        st = lib().mi355_quant_dot_ws(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
+                                      _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _ptr(bias), _ptr(workspace),
+                                      workspace.numel() * workspace.element_size(), _stream())
+        check(st, "mi355_quant_dot_ws")
+    elif bias is not None:
         st = lib().mi355_quant_dot_bias(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
                                         _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _ptr(bias), _stream())
         check(st, "mi355_quant_dot_bias")
-        return out
-    st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
-                               _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
-    check(st, "mi355_quant_dot")
+    else:
+        st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
+                                   _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
+        check(st, "mi355_quant_dot")
     return out
+
+
+def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False):
+    """Bytes of workspace an int8 quant_dot of that shape can use (0: none)."""
+    d = QuantDotDesc(m=m, n=n, k=k, batch=batch, lda=k, ldb=k if trans_b else n, ldc=n,
+                     stride_a=m * k, stride_b=k * n, stride_c=m * n, trans_a=0, trans_b=int(trans_b),
+                     in_type=DT.I8, out_type=DT.I32, dequant=0)
+    return int(lib().mi355_quant_dot_workspace_size(ctypes.byref(d)))
 
 
 def quant_convolution(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1, fp8=False,

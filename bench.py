@@ -204,11 +204,33 @@ def main():
                 ops.quant_dot(a2, bs[it[0] % 6], out=c2)
                 it[0] += 1
 
-            t2, _ = _time_launches(skinny, 18, 6)
+            # the same with room for partial sums: K split over the chip without atomics
+            room = torch.empty(max(ops.quant_dot_workspace_size(m2, 8192, 8192), 16), dtype=torch.uint8,
+                               device=dev)
+
+            def skinny_ws():
+                ops.quant_dot(a2, bs[it[0] % 6], out=c2, workspace=room)
+                it[0] += 1
+
+            # and as the fused linear layer (per-column scales, bias, bf16 out)
+            sa2 = torch.full((1,), 0.02, device=dev)
+            sb2 = torch.rand(8192, device=dev, generator=g) * 0.01
+            bias2 = torch.randn(8192, device=dev, generator=g)
+            y2 = torch.empty((m2, 8192), dtype=torch.bfloat16, device=dev)
+
+            def skinny_dq():
+                ops.quant_dot(a2, bs[it[0] % 6], scale_a=sa2, scale_b=sb2, bias=bias2, out_dtype=torch.bfloat16,
+                              out=y2, workspace=room)
+                it[0] += 1
+
+            t2a, _ = _time_launches(skinny, 18, 6)
+            t2, _ = _time_launches(skinny_ws, 18, 6)
+            t2d, _ = _time_launches(skinny_dq, 18, 6)
             byts = m2 * 8192 + 8192 * 8192 + 4 * m2 * 8192
             also[f"int8_quant_dot_M{m2}_N8192_K8192"] = {
                 "GB/s": round(byts / t2 / 1e9, 1), "frac_hbm_peak": round(byts / t2 / 1e9 / PEAK_HBM_GBS, 4),
-                "us_per_launch": round(t2 * 1e6, 1)}
+                "us_per_launch": round(t2 * 1e6, 1), "us_per_launch_no_workspace": round(t2a * 1e6, 1),
+                "us_per_launch_dq_bias_bf16": round(t2d * 1e6, 1), "workspace_MiB": room.numel() >> 20}
             del bs
         for m4 in (16, 128):
             k4, n4, grp = 4096, 14336, 128

@@ -161,6 +161,19 @@ int mi355_quant_convolution(const mi355_quant_conv_desc* desc, const void* x, co
                             const float* scale_x, const float* scale_w, void* workspace,
                             size_t workspace_bytes, void* stream);
 
+/* The same with a workspace.  A bare int8 quant_dot with few output tiles and a long K (a skinny
+ * A against a large B) is split along K over the workgroups of the chip; without a workspace the
+ * shares are added into C with integer atomics, with one they write partial tiles and a second
+ * kernel adds them up (no atomics, no clearing of C; the result is the same bits).
+ * mi355_quant_dot_workspace_size gives the bytes that description can use (0: none); a NULL or
+ * smaller workspace is not an error, the call then behaves like mi355_quant_dot_bias.  The
+ * workspace must be 16-byte aligned device memory and is free again when the call's work is done. */
+size_t mi355_quant_dot_workspace_size(const mi355_quant_dot_desc* desc);
+int mi355_quant_dot_ws(const mi355_quant_dot_desc* desc, const void* a, const void* b, void* c,
+                       const float* scale_a, const float* scale_b, const int32_t* colsum_b,
+                       const int32_t* rowsum_a, const float* bias, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
  * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the
  * zero-point term of simplify_qdq.cpp:260-266 divided by the zero point. */

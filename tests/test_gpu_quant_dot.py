@@ -535,3 +535,80 @@ def test_full_size_fp8_config3_shapes(ops, k, n):
     assert (diff >= 0).all()
     assert (diff <= exact.abs() * 2.0**-7).all()
     assert (out.float().sign() * exact.sign() >= 0).all()
+
+
+# skinny bare int8 products with a workspace: K is split over workgroups that write partial tiles,
+# a second kernel adds them; the result must be the bits of the one-pass product (int32 sums are
+# exact in any order) and of the oracle
+@pytest.mark.parametrize("m,n,k,batch,trans_b", [
+    (16, 1024, 4096, 1, False), (16, 1024, 4096, 1, True), (128, 512, 2048, 1, False), (1, 256, 8192, 1, True),
+    (33, 260, 1024, 2, False), (40, 300, 1600, 1, True), (8, 256, 2112, 1, False), (16, 8192, 8192, 1, False), (128, 8192, 8192, 1, True),
+])
+def test_int8_split_k_with_workspace_bit_exact(ops, m, n, k, batch, trans_b):
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    a = torch.randint(-128, 128, (batch, m, k), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (batch, n, k) if trans_b else (batch, k, n), dtype=torch.int8, generator=g)
+    da, db = a.cuda(), b.cuda()
+    dbv = db.transpose(1, 2) if trans_b else db
+    bytes_ = ops.quant_dot_workspace_size(m, n, k, batch, trans_b)
+    assert bytes_ > 0, "these shapes are meant to take the split"
+    assert bytes_ % (batch * m * n * 4) == 0
+    ws = torch.full((bytes_ // 4,), 0x55555555, dtype=torch.int32, device="cuda")
+    got = ops.quant_dot(da, dbv, workspace=ws)
+    ref = ops.quant_dot(da, dbv)
+    assert torch.equal(got, ref)
+    want = torch.matmul(a.double(), (b.transpose(1, 2) if trans_b else b).double()).to(torch.int32)
+    assert torch.equal(got.cpu(), want)
+    # a workspace that is too small is not an error: the call takes the path without one
+    small = torch.empty(64, dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.quant_dot(da, dbv, workspace=small), ref)
+    # second call with the same workspace (stale partial sums from the first), into a view of a
+    # wider buffer: the columns beside it stay as they were
+    wide = torch.full((batch, m, n + 8), 7, dtype=torch.int32, device="cuda")
+    ops.quant_dot(da, dbv, workspace=ws, out=wide[:, :, :n])
+    assert torch.equal(wide[:, :, :n], ref)
+    assert (wide[:, :, n:] == 7).all()
+
+
+def test_workspace_size_is_zero_where_no_split_pays(ops):
+    assert ops.quant_dot_workspace_size(8192, 8192, 8192) == 0
+    assert ops.quant_dot_workspace_size(16, 64, 128) == 0
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 300, 1600, False),
+                                           (1, 512, 8192, True), (8, 256, 2112, False)])
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b, out):
+    """The skinny fused linear layer: the second kernel of the workspace split applies the
+    dequantizelinear epilogue (scales per row and per column, both zero points, bias, convert) to
+    the summed partial tiles.  Required: the bits of the oracle, which are also those of the
+    one-pass kernel."""
+    rng = np.random.default_rng(m * 13 + n + k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (n, k) if trans_b else (k, n), dtype=np.int8)
+    bm = np.ascontiguousarray(b.T) if trans_b else b
+    sa = rng.uniform(0.01, 0.05, m).astype(np.float32)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 3).astype(np.float32)
+    bias[:2] = [0.0, -0.0]
+    zp_a, zp_b = (3, -2) if m % 16 else (0, 0)
+    want = orc.qdq_matmul_int8(a, bm, sa[:, None], sb[None, :], zp_a, zp_b, orc.F32) + bias[None, :]
+    assert want.dtype == np.float32
+    tb = dev(b).T if trans_b else dev(b)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    nbytes = ops.quant_dot_workspace_size(m, n, k, 1, trans_b)
+    assert nbytes > 0
+    ws = torch.full((nbytes,), 0xA5, dtype=torch.uint8, device="cuda")
+    print("int8 workspace dq", m, n, k, trans_b, out, flush=True)
+    kw = dict(scale_a=dev(sa), scale_b=dev(sb), zp_a=zp_a, zp_b=zp_b,
+              colsum_b=ops.colsum_i8(tb) if zp_a else None, rowsum_a=ops.rowsum_i8(dev(a)) if zp_b else None,
+              out_dtype=td, bias=dev(bias))
+    got = ops.quant_dot(dev(a), tb, workspace=ws, **kw)
+    one_pass = ops.quant_dot(dev(a), tb, **kw)
+    assert torch.equal(got.view(torch.int32 if out == "f32" else torch.int16),
+                       one_pass.view(torch.int32 if out == "f32" else torch.int16))
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        ot = orc.F16 if out == "f16" else orc.BF16
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
