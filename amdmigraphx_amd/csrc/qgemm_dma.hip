@@ -1090,35 +1090,39 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* c, int m, int n,
 
 // Second kernel of the split-K with a workspace: C = epilogue(sum of the shares' partial tiles).
 // A thread column (threadIdx.x) owns 4 adjacent outputs; the 4 waves of a workgroup (threadIdx.y)
-// each add every fourth share and the first one collects the four sums through the LDS.  Integer
-// sums: any order gives the same bits; the dequantizing epilogue is the arithmetic of the one-pass
-// kernel's.  N, ldc and the batch stride of C are multiples of 4 on this path.
-template <bool DEQ, int OUT>
+// each add every fourth share and the first one collects the four sums through the LDS.  int8:
+// integer sums, any order gives the same bits, and the dequantizing epilogue is the arithmetic of
+// the one-pass kernel's.  fp8: float partial sums added in this fixed order (the same bits on every
+// run; not those of the one-pass kernel, whose one accumulator walks K in another order).  N, ldc
+// and the batch stride of C are multiples of 4 on this path.
+template <bool FP8, bool DEQ, int OUT>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int shares)
 {
-    __shared__ v4i part[3][64];
-    const int64_t mn    = (int64_t)p.m * p.n;
-    const int64_t q     = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    const bool inside   = 4 * q < mn;
-    const int32_t* src  = p.partial + (int64_t)blockIdx.y * p.ksplit * mn + 4 * q;
-    v4i sum             = {0, 0, 0, 0};
+    using acc_t = std::conditional_t<FP8, float, int32_t>;
+    using vec_t = acc_t __attribute__((ext_vector_type(4)));
+    __shared__ vec_t part[3][64];
+    const int64_t mn  = (int64_t)p.m * p.n;
+    const int64_t q   = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    const bool inside = 4 * q < mn;
+    const acc_t* src  = reinterpret_cast<const acc_t*>(p.partial) + (int64_t)blockIdx.y * p.ksplit * mn + 4 * q;
+    vec_t sum         = {0, 0, 0, 0};
     if(inside)
     {
 #pragma unroll 4
         for(int z = threadIdx.y; z < shares; z += 4)
-            sum += *reinterpret_cast<const v4i*>(src + (int64_t)z * mn);
+            sum += *reinterpret_cast<const vec_t*>(src + (int64_t)z * mn);
     }
     if(threadIdx.y > 0)
         part[threadIdx.y - 1][threadIdx.x] = sum;
     __syncthreads();
     if(threadIdx.y != 0 || !inside)
         return;
-    sum += part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x];
+    sum               = ((sum + part[0][threadIdx.x]) + part[1][threadIdx.x]) + part[2][threadIdx.x];
     const int row     = (int)(4 * q / p.n);
     const int col     = (int)(4 * q % p.n);
     const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
     if constexpr(!DEQ)
-        *reinterpret_cast<v4i*>(static_cast<int32_t*>(p.c) + idx) = sum;
+        *reinterpret_cast<vec_t*>(static_cast<acc_t*>(p.c) + idx) = sum;
     else
     {
         float sa = 1.f;
@@ -1126,8 +1130,9 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
             sa = p.scale_a[0];
         else if(p.scale_a_mode == MI355_QP_PER_ROW)
             sa = p.scale_a[row];
-        const int64_t zrow =
-            p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
+        int64_t zrow = 0;
+        if constexpr(!FP8)
+            zrow = p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
         float v[4];
 #pragma unroll
         for(int e = 0; e < 4; e++)
@@ -1137,11 +1142,16 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
                 sb = p.scale_b[0];
             else if(p.scale_b_mode == MI355_QP_PER_COL)
                 sb = p.scale_b[col + e];
-            const int32_t cs = p.zp_a != 0 ? p.colsum_b[col + e] : 0;
             const float bias = p.bias != nullptr ? p.bias[col + e] : -0.0f;
             const float s    = sa * sb;
-            const double d   = (double)sum[e] - (double)(int32_t)(zrow + (int64_t)p.zp_a * cs);
-            v[e]             = add_bias((float)(d * (double)s), bias);
+            if constexpr(FP8)
+                v[e] = add_bias((float)sum[e] * s, bias);
+            else
+            {
+                const int32_t cs = p.zp_a != 0 ? p.colsum_b[col + e] : 0;
+                const double d   = (double)sum[e] - (double)(int32_t)(zrow + (int64_t)p.zp_a * cs);
+                v[e]             = add_bias((float)(d * (double)s), bias);
+            }
         }
         if constexpr(OUT == MI355_F32)
             *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) = v4f{v[0], v[1], v[2], v[3]};
@@ -1156,12 +1166,20 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
     }
 }
 
-template <bool DEQ, int OUT>
-void launch_reduce(const dma_params& p, int batch, int shares, hipStream_t stream)
+template <bool FP8>
+int launch_reduce(const dma_params& p, int batch, int shares, bool deq, int out_type, hipStream_t stream)
 {
     const int64_t quads = (int64_t)p.m * p.n / 4;
-    hipLaunchKernelGGL((reduce_partials_kernel<DEQ, OUT>), dim3((unsigned)((quads + 63) / 64), batch),
-                       dim3(64, 4), 0, stream, p, shares);
+    const dim3 grid((unsigned)((quads + 63) / 64), batch), block(64, 4);
+    if(!deq)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, false, MI355_F32>), grid, block, 0, stream, p, shares);
+    else if(out_type == MI355_F32)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F32>), grid, block, 0, stream, p, shares);
+    else if(out_type == MI355_F16)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F16>), grid, block, 0, stream, p, shares);
+    else
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_BF16>), grid, block, 0, stream, p, shares);
+    return mi355_launch_status();
 }
 
 // deq / out_type: the epilogue of the second kernel on the workspace path (the atomic path gives
@@ -1183,15 +1201,7 @@ int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream, bool de
         const int nk     = p.k / BK;
         const int per    = (nk + p.ksplit - 1) / p.ksplit;
         const int shares = (nk + per - 1) / per;
-        if(!deq)
-            launch_reduce<false, MI355_F32>(p, batch, shares, stream);
-        else if(out_type == MI355_F32)
-            launch_reduce<true, MI355_F32>(p, batch, shares, stream);
-        else if(out_type == MI355_F16)
-            launch_reduce<true, MI355_F16>(p, batch, shares, stream);
-        else
-            launch_reduce<true, MI355_BF16>(p, batch, shares, stream);
-        return mi355_launch_status();
+        return launch_reduce<false>(p, batch, shares, deq, out_type, stream);
     }
     const int64_t total = (int64_t)p.m * p.n;
     const int zb        = (int)min((int64_t)2048, (total + 255) / 256);
@@ -1304,10 +1314,31 @@ bool mi355_dma_gemm_supported(const mi355_quant_dot_desc* d, const void* a, cons
     return true;
 }
 
-// bytes of workspace that would let an int8 quant_dot of this description (bare or dequantizing)
-// split K without atomics (0: no use for one)
+// fp8: the shares are equal slices of K (the split goes through the kernel's batch index), so the
+// count from the model is lowered to the next divisor of the number of slabs; one batch only
+static int fp8_shares(const mi355_quant_dot_desc* d)
+{
+    if(d->batch != 1 || d->k % BK != 0 || d->m <= 0 || d->n <= 0)
+        return 1;
+    const int nk    = (int)(d->k / BK);
+    const int tiles = (int)(((d->m + BM - 1) / BM) * ((d->n + BN - 1) / BN));
+    int s           = choose_ksplit_ws(tiles, 1, nk, d->m, d->n, d->k);
+    while(s > 1 && nk % s != 0)
+        s--;
+    return s;
+}
+
+// bytes of workspace that would let a quant_dot of this description (bare or dequantizing) split K
+// without atomics (0: no use for one)
 size_t mi355_dma_gemm_workspace(const mi355_quant_dot_desc* d)
 {
+    if(d->in_type == MI355_FP8)
+    {
+        if(d->trans_a || d->n % 4 != 0 || d->ldc % 4 != 0)
+            return 0;
+        const int s = fp8_shares(d);
+        return s > 1 ? (size_t)s * d->m * d->n * 4 : 0;
+    }
     if(d->in_type != MI355_I8 || d->trans_a || d->k % BK != 0 || d->k < BK || d->n % 4 != 0 ||
        d->ldc % 4 != 0 || d->stride_c % 4 != 0 || d->m <= 0 || d->n <= 0 || d->batch <= 0)
         return 0;
@@ -1364,6 +1395,34 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                        reinterpret_cast<uintptr_t>(c) % 16 == 0;
     }
     p.ksplit = 1;
+    if(fp8 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && p.vec_store &&
+       d->n % 4 == 0)
+    {
+        // Split K through the batch index: share z is the bare product of A[:, z*kz : (z+1)*kz]
+        // and the matching rows of B, written to partial[z] (the kernel itself is unchanged);
+        // the second kernel adds the shares and applies the epilogue.
+        const int s = fp8_shares(d);
+        if(s > 1 && (size_t)s * d->m * d->n * 4 <= workspace_bytes)
+        {
+            dma_params q = p;
+            q.k          = p.k / s;
+            q.c          = workspace;
+            q.ldc        = d->n;
+            q.stride_c   = d->m * d->n;
+            q.stride_a   = q.k;
+            q.stride_b   = d->trans_b ? (int64_t)q.k : (int64_t)q.k * d->ldb;
+            q.vec_store  = 1;
+            q.vec8_store = 0;
+            q.bias       = nullptr;
+            const int st = d->trans_b ? launch_out<true, true>(q, s, false, MI355_F32, stream)
+                                      : launch_out<true, false>(q, s, false, MI355_F32, stream);
+            if(st != MI355_OK)
+                return st;
+            p.ksplit  = s;
+            p.partial = static_cast<int32_t*>(workspace);
+            return launch_reduce<true>(p, 1, s, deq, d->out_type, stream);
+        }
+    }
     if(fp8)
         return d->trans_b ? launch_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
                           : launch_out<true, false>(p, (int)d->batch, deq, d->out_type, stream);

@@ -133,11 +133,11 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     return out
 
 
-def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False):
-    """Bytes of workspace an int8 quant_dot of that shape can use (0: none)."""
+def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False, fp8=False):
+    """Bytes of workspace an int8 (or fp8) quant_dot of that shape can use (0: none)."""
     d = QuantDotDesc(m=m, n=n, k=k, batch=batch, lda=k, ldb=k if trans_b else n, ldc=n,
                      stride_a=m * k, stride_b=k * n, stride_c=m * n, trans_a=0, trans_b=int(trans_b),
-                     in_type=DT.I8, out_type=DT.I32, dequant=0)
+                     in_type=DT.FP8 if fp8 else DT.I8, out_type=DT.F32 if fp8 else DT.I32, dequant=0)
     return int(lib().mi355_quant_dot_workspace_size(ctypes.byref(d)))
 
 

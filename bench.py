@@ -223,9 +223,28 @@ def main():
                               out=y2, workspace=room)
                 it[0] += 1
 
+            # fp8 operands (the same bytes with the exponent's top bit cleared: finite codes)
+            a8 = a2.view(torch.uint8) & 0x77
+            b8 = [b.view(torch.uint8) & 0x77 for b in bs]
+            room8 = torch.empty(max(ops.quant_dot_workspace_size(m2, 8192, 8192, fp8=True), 16),
+                                dtype=torch.uint8, device=dev)
+
+            def skinny_fp8(workspace):
+                def run():
+                    ops.quant_dot(a8, b8[it[0] % 6], fp8=True, scale_a=sa2, scale_b=sb2, bias=bias2,
+                                  out_dtype=torch.bfloat16, out=y2, workspace=workspace)
+                    it[0] += 1
+                return run
+
             t2a, _ = _time_launches(skinny, 18, 6)
             t2, _ = _time_launches(skinny_ws, 18, 6)
             t2d, _ = _time_launches(skinny_dq, 18, 6)
+            t8, _ = _time_launches(skinny_fp8(room8), 18, 6)
+            t8a, _ = _time_launches(skinny_fp8(None), 18, 6)
+            also[f"fp8_quant_dot_dq_bias_bf16_M{m2}_N8192_K8192"] = {
+                "us_per_launch": round(t8 * 1e6, 1), "us_per_launch_no_workspace": round(t8a * 1e6, 1),
+                "workspace_MiB": room8.numel() >> 20}
+            del b8
             byts = m2 * 8192 + 8192 * 8192 + 4 * m2 * 8192
             also[f"int8_quant_dot_M{m2}_N8192_K8192"] = {
                 "GB/s": round(byts / t2 / 1e9, 1), "frac_hbm_peak": round(byts / t2 / 1e9 / PEAK_HBM_GBS, 4),

@@ -161,13 +161,16 @@ int mi355_quant_convolution(const mi355_quant_conv_desc* desc, const void* x, co
                             const float* scale_x, const float* scale_w, void* workspace,
                             size_t workspace_bytes, void* stream);
 
-/* The same with a workspace.  A bare int8 quant_dot with few output tiles and a long K (a skinny
- * A against a large B) is split along K over the workgroups of the chip; without a workspace the
- * shares are added into C with integer atomics, with one they write partial tiles and a second
- * kernel adds them up (no atomics, no clearing of C; the result is the same bits).
- * mi355_quant_dot_workspace_size gives the bytes that description can use (0: none); a NULL or
- * smaller workspace is not an error, the call then behaves like mi355_quant_dot_bias.  The
- * workspace must be 16-byte aligned device memory and is free again when the call's work is done. */
+/* The same with a workspace.  A quant_dot with few output tiles and a long K (a skinny A against a
+ * large B) is split along K over the workgroups of the chip.  Without a workspace only the bare
+ * int8 product is split (the shares are added into C with integer atomics); with one, the shares
+ * write partial tiles and a second kernel adds them up and applies the dequantizing epilogue (no
+ * atomics, no clearing of C).  int8: the same bits as the unsplit kernel.  fp8 (one batch only):
+ * float partial sums added in a fixed order, the same bits on every call, within the fp8
+ * tolerance of the unsplit kernel's.  mi355_quant_dot_workspace_size gives the bytes that
+ * description can use (0: none); a NULL or smaller workspace is not an error, the call then
+ * behaves like mi355_quant_dot_bias.  The workspace must be 16-byte aligned device memory and is
+ * free again when the call's work is done. */
 size_t mi355_quant_dot_workspace_size(const mi355_quant_dot_desc* desc);
 int mi355_quant_dot_ws(const mi355_quant_dot_desc* desc, const void* a, const void* b, void* c,
                        const float* scale_a, const float* scale_b, const int32_t* colsum_b,

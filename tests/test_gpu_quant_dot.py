@@ -612,3 +612,55 @@ def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b
     else:
         ot = orc.F16 if out == "f16" else orc.BF16
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 300, 1600, False),
+                                           (1, 512, 8192, True), (64, 256, 2112, False)])
+@pytest.mark.parametrize("out", ["bare", "f32", "bf16"])
+def test_fp8_split_k_with_workspace(ops, m, n, k, trans_b, out):
+    """fp8 skinny shapes with a workspace: K is cut into equal slices (float partial sums, added in
+    a fixed order by the second kernel, which also applies scale, bias and convert).  The sums are
+    floats in another order than the one-pass kernel's, so the requirement is the fp8 tolerance
+    against the oracle (as for the one-pass kernel) and the same bits on every call."""
+    rng = np.random.default_rng(m + 3 * n + k)
+    a = _fp8_codes(rng, (m, k), 100.0)
+    b = _fp8_codes(rng, (k, n), 100.0)
+    tb = dev(np.ascontiguousarray(b.T)).t() if trans_b else dev(b)
+    nbytes = ops.quant_dot_workspace_size(m, n, k, 1, trans_b, fp8=True)
+    assert nbytes > 0 and nbytes % (m * n * 4) == 0 and (k // 64) % (nbytes // (m * n * 4)) == 0
+    ws = torch.full((nbytes,), 0x7F, dtype=torch.uint8, device="cuda")  # NaN patterns if read unwritten
+    print("fp8 workspace", m, n, k, trans_b, out, flush=True)
+    if out == "bare":
+        want = orc.quant_dot(a, b, orc.FP8)
+        got = ops.quant_dot(dev(a), tb, fp8=True, workspace=ws)
+        again = ops.quant_dot(dev(a), tb, fp8=True, workspace=ws)
+        assert torch.equal(got.view(torch.int32), again.view(torch.int32))
+        assert _fp8_close(got.cpu().numpy(), want, _fp8_bound(a, b)).all()
+        rel = np.abs(got.cpu().numpy() - want) / np.maximum(np.abs(want), 1e-30)
+        assert np.median(rel) < 1e-4
+        return
+    sx, sw = np.float32(0.0123), np.float32(0.00371)
+    sb = (rng.uniform(0.5, 1.5, n) * sw).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.5).astype(np.float32)
+    td = torch.float32 if out == "f32" else torch.bfloat16
+    kw = dict(fp8=True, scale_a=dev(np.float32([sx])), scale_b=dev(sb), out_dtype=td, bias=dev(bias))
+    got = ops.quant_dot(dev(a), tb, workspace=ws, **kw)
+    again = ops.quant_dot(dev(a), tb, workspace=ws, **kw)
+    assert torch.equal(got.view(torch.int32 if out == "f32" else torch.int16),
+                       again.view(torch.int32 if out == "f32" else torch.int16))
+    # the epilogue on top of this path's own bare sums, bit for bit: fp32 scale product, one
+    # multiply, one add, convert
+    bare = ops.quant_dot(dev(a), tb, fp8=True, workspace=ws).cpu().numpy()
+    step = (bare * (sx * sb)[None, :]).astype(np.float32) + bias[None, :]
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), step.view(np.uint32))
+    else:
+        assert np.array_equal(bf16_bits(got), orc.convert(step, orc.F32, orc.BF16))
+    # and the oracle's value within the fp8 tolerance
+    ref = orc.quant_dot(a, b, orc.FP8).astype(np.float64) * (np.float64(sx) * sb.astype(np.float64))[None, :] + bias
+    bound = _fp8_bound(a, b) * float(sx) * sb.astype(np.float64)[None, :]
+    gf = got.float().cpu().numpy()
+    if out == "f32":
+        assert _fp8_close(gf, ref, bound).all()
+    else:
+        assert ((np.abs(gf - ref) <= np.abs(ref) * 2.0**-7) | _fp8_close(gf, ref, bound)).all()
