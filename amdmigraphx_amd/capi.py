@@ -97,6 +97,11 @@ EXPORTS = {
                          ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
                          ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                          ctypes.c_int64, ctypes.c_void_p],
+    "mi355_w4a16_gemm_workspace_size": [ctypes.c_int64] * 4,
+    "mi355_w4a16_gemm_ws": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+                            ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
+                            ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                            ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     "mi355_status_string": [ctypes.c_int],
     "mi355_version": [],
 }
@@ -132,7 +137,7 @@ def lib():
             fn = getattr(h, name)
             fn.argtypes = argtypes
             fn.restype = (ctypes.c_char_p if name == "mi355_status_string" else
-                          ctypes.c_size_t if name == "mi355_quant_dot_workspace_size" else ctypes.c_int)
+                          ctypes.c_size_t if name.endswith("_workspace_size") else ctypes.c_int)
         _handle = h
     return _handle
 

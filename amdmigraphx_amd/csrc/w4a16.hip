@@ -31,6 +31,9 @@ struct w4_params
     uint16_t* out;
     int64_t ldc;
     int m, n, k, group;
+    float* partial;        // room for split-K partial sums (null: none)
+    size_t partial_bytes;  // host side only
+    int chunks_per_share;  // set by the launcher when it splits
 };
 
 MI355_DEVINL float wave_sum(float v)
@@ -411,6 +414,36 @@ extern "C" int mi355_w4a16_gemm(const void* a,
                                 int64_t group,
                                 void* stream)
 {
+    return mi355_w4a16_gemm_ws(a, lda, w_packed, scales, zp, zp_mode, zp_scalar, out, ldc, m, n, k, group, nullptr,
+                               0, stream);
+}
+
+extern "C" size_t mi355_w4a16_gemm_workspace_size(int64_t m, int64_t n, int64_t k, int64_t group)
+{
+    if(m <= 32 || n <= 0 || k <= 0 || group <= 0 || n % TL_BN != 0 || k % 128 != 0 || k > (1 << 30) ||
+       n > (1 << 30) || m > (1 << 30))
+        return 0;
+    const int shares = tile_gemm_shares((int)m, (int)n, (int)k);
+    return shares > 1 ? (size_t)shares * m * n * 4 : 0;
+}
+
+extern "C" int mi355_w4a16_gemm_ws(const void* a,
+                                   int64_t lda,
+                                   const void* w_packed,
+                                   const void* scales,
+                                   const void* zp,
+                                   int32_t zp_mode,
+                                   int32_t zp_scalar,
+                                   void* out,
+                                   int64_t ldc,
+                                   int64_t m,
+                                   int64_t n,
+                                   int64_t k,
+                                   int64_t group,
+                                   void* workspace,
+                                   size_t workspace_bytes,
+                                   void* stream)
+{
     if(a == nullptr || w_packed == nullptr || scales == nullptr || out == nullptr)
         return MI355_ERR_BAD_ARG;
     if(m < 0 || n < 0 || k <= 0 || group <= 0)
@@ -447,6 +480,9 @@ extern "C" int mi355_w4a16_gemm(const void* a,
     p.n         = (int)n;
     p.k         = (int)k;
     p.group     = (int)group;
+    p.partial   = reinterpret_cast<uintptr_t>(workspace) % 16 == 0 ? static_cast<float*>(workspace) : nullptr;
+    p.partial_bytes    = p.partial != nullptr ? workspace_bytes : 0;
+    p.chunks_per_share = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if(m == 1 && zp_mode == MI355_W4_ZP_SCALAR && k % 2048 == 0 && k <= GV_MAX_K &&
        (group & (group - 1)) == 0 && group <= 2048)

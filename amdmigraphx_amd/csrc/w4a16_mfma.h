@@ -436,6 +436,9 @@ int launch_tile_gemm(const w4_params& p, hipStream_t s);
 // M rows in chunks of at most 128
 int launch_mfma_gemm(const w4_params& p0, hipStream_t s)
 {
+    // the tile kernel takes any number of rows in one launch (64 per workgroup)
+    if(tile_gemm_supported(p0))
+        return launch_tile_gemm(p0, s);
     for(int m0 = 0; m0 < p0.m; m0 += 128)
     {
         w4_params p = p0;

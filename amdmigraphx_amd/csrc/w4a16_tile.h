@@ -64,6 +64,10 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
     const int groups  = p.k / p.group;
     const int nsteps  = p.k >> 7;
     const int nchunks = (p.k + TL_CK - 1) / TL_CK;
+    // K split over blockIdx.z (p.partial set): this workgroup walks chunks cbase .. cbase + nloc - 1
+    // and leaves float sums in partial[blockIdx.z]; every share holds at least one chunk
+    const int cbase = p.partial != nullptr ? (int)blockIdx.z * p.chunks_per_share : 0;
+    const int nloc  = p.partial != nullptr ? min(p.chunks_per_share, nchunks - cbase) : nchunks;
 
     // half-precision arithmetic of this wave truncates from here on (MODE.fp_round bits 3:2); the
     // fp32 accumulation of the matrix cores keeps round-to-nearest
@@ -101,8 +105,9 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
             asrc[t]      = ((uint32_t)row * (uint32_t)p.lda + (uint32_t)(pc * 8)) * 2;
             a_second[t]  = pc >= 16;
         }
-        auto issue_chunk = [&](int c) {
-            uint8_t* slot = lds + (c % TL_RING) * SLOT;
+        auto issue_chunk = [&](int cl) {
+            uint8_t* slot = lds + (cl % TL_RING) * SLOT;
+            const int c   = cbase + cl;
             // only the first half of the last chunk exists when K is an odd multiple of 128
             const bool half = c * TL_CK + 128 >= p.k;
 #pragma unroll
@@ -127,16 +132,16 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
         // one chunk's worth outstanding" means chunk c is in.
 #pragma unroll
         for(int c = 0; c < TL_RING - 1; c++)
-            if(c < nchunks)
+            if(c < nloc)
                 issue_chunk(c);
-        for(int c = 0; c < nchunks; c++)
+        for(int c = 0; c < nloc; c++)
         {
-            if(c + TL_RING - 2 < nchunks)
+            if(c + TL_RING - 2 < nloc)
                 wl_wait_vmcnt<(TL_RING - 2) * PER_CHUNK>();
             else
                 wl_wait_vmcnt<0>();
             wl_barrier();
-            if(c + TL_RING - 1 < nchunks)
+            if(c + TL_RING - 1 < nloc)
                 issue_chunk(c + TL_RING - 1);
         }
         return;
@@ -299,15 +304,16 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
     };
 
     step_inputs in[2];
-    request(in[0], 0);
-    for(int c = 0; c < nchunks; c++)
+    request(in[0], 2 * cbase);
+    for(int c = 0; c < nloc; c++)
     {
         wl_barrier();
         const uint32_t slot_addr = lds0 + (c % TL_RING) * SLOT;
-        request(in[1], 2 * c + 1);
+        const int step           = 2 * (cbase + c);
+        request(in[1], step + 1);
         do_step(in[0], slot_addr, 0);
-        request(in[0], 2 * c + 2);
-        if(2 * c + 1 < nsteps)
+        request(in[0], step + 2);
+        if(step + 1 < nsteps)
             do_step(in[1], slot_addr, 1);
     }
 
@@ -318,9 +324,43 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
         for(int r = 0; r < 4; r++)
         {
             const int m = m0 + 16 * i + 4 * kg + r;
-            if(m < p.m)
+            if(m >= p.m)
+                continue;
+            if(p.partial != nullptr)
+                p.partial[((int64_t)blockIdx.z * p.m + m) * p.n + n] = acc[i][r];
+            else
                 p.out[(int64_t)m * p.ldc + n] = f32_to_half_rtz(acc[i][r]);
         }
+}
+
+// out = half(sum of the shares' float partial sums), 4 columns per thread, shares added in order
+__global__ __launch_bounds__(256) void w4a16_reduce_kernel(const float* partial, uint16_t* out, int m, int n,
+                                                            int64_t ldc, int shares)
+{
+    const int64_t mn = (int64_t)m * n;
+    const int64_t e  = 4 * ((int64_t)blockIdx.x * 256 + threadIdx.x);
+    if(e >= mn)
+        return;
+    v4f sum = *reinterpret_cast<const v4f*>(partial + e);
+    for(int z = 1; z < shares; z++)
+        sum += *reinterpret_cast<const v4f*>(partial + (int64_t)z * mn + e);
+    uint16_t* o = out + (e / n) * ldc + (e % n);
+#pragma unroll
+    for(int r = 0; r < 4; r++)
+        o[r] = f32_to_half_rtz(sum[r]);
+}
+
+// shares of K for `m` rows: enough workgroups for every CU (a workgroup
+// fills one), at least two chunks per share; 1 = no split
+int tile_gemm_shares(int m, int n, int k)
+{
+    const int tiles   = (n / TL_BN) * ((m + 63) / 64);
+    const int nchunks = (k + TL_CK - 1) / TL_CK;
+    if(tiles > 128 || nchunks < 4)
+        return 1;
+    int s = (256 + tiles - 1) / tiles;
+    s     = min(s, nchunks / 2);
+    return max(s, 1);
 }
 
 bool tile_gemm_supported(const w4_params& p)
@@ -328,14 +368,31 @@ bool tile_gemm_supported(const w4_params& p)
     return p.m > 32 && p.n % TL_BN == 0 && mfma_gemm_supported(p);
 }
 
-// at most 128 rows per call (the caller walks M in such pieces): 64 rows per workgroup
-int launch_tile_gemm(const w4_params& p, hipStream_t s)
+// 64 rows per workgroup
+int launch_tile_gemm(const w4_params& p0, hipStream_t s)
 {
+    w4_params p       = p0;
     const bool simple = p.zp_mode == MI355_W4_ZP_SCALAR && (p.group & 127) == 0;
-    const dim3 grid((unsigned)(p.n / TL_BN), (unsigned)((p.m + 63) / 64));
+    dim3 grid((unsigned)(p.n / TL_BN), (unsigned)((p.m + 63) / 64));
+    const int shares = tile_gemm_shares(p.m, p.n, p.k);
+    float* room      = p0.partial;
+    p.partial        = nullptr;
+    if(room != nullptr && shares > 1 && (size_t)shares * p.m * p.n * 4 <= p0.partial_bytes)
+    {
+        const int nchunks  = (p.k + TL_CK - 1) / TL_CK;
+        p.chunks_per_share = (nchunks + shares - 1) / shares;
+        p.partial          = room;
+        grid.z             = (unsigned)((nchunks + p.chunks_per_share - 1) / p.chunks_per_share);
+    }
     if(simple)
         hipLaunchKernelGGL((w4a16_tile_kernel<4, true>), grid, dim3(WL_THREADS), 0, s, p);
     else
         hipLaunchKernelGGL((w4a16_tile_kernel<4, false>), grid, dim3(WL_THREADS), 0, s, p);
+    if(p.partial != nullptr)
+    {
+        const int64_t quads = (int64_t)p.m * p.n / 4;
+        hipLaunchKernelGGL(w4a16_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p.partial,
+                           p.out, p.m, p.n, p.ldc, (int)grid.z);
+    }
     return mi355_launch_status();
 }

@@ -180,12 +180,14 @@ struct w4a16_gemm
     int64_t group     = 128;
     int64_t zp_mode   = MI355_W4_ZP_SCALAR;
     int64_t zp_scalar = 8;
+    bool workspace    = false; // a uint8 buffer before `out` (mi355_w4a16_gemm_workspace_size)
     template <class Self, class F>
     static void reflect(Self& self, F f)
     {
         f(self.group, "group");
         f(self.zp_mode, "zp_mode");
         f(self.zp_scalar, "zp_scalar");
+        f(self.workspace, "workspace");
     }
     std::string name() const { return "mi355::w4a16_gemm"; }
     shape compute_shape(const std::vector<shape>& inputs) const;

@@ -536,7 +536,16 @@ bool lower_w4a16(module& m, instruction_ref ins)
     }
     if(a->get_shape().strides()[1] != 1 and a->get_shape().lens()[1] != 1)
         args[0] = make_standard(m, ins, a);
-    args.push_back(insert_allocation(m, ins, shape{shape::half_type, {a->get_shape().lens()[0], n}}));
+    // room for split-K partial sums where the column tiles alone do not fill the chip
+    const auto rows   = a->get_shape().lens()[0];
+    const size_t need = mi355_w4a16_gemm_workspace_size(static_cast<int64_t>(rows), static_cast<int64_t>(n),
+                                                        static_cast<int64_t>(k), op.group);
+    if(need > 0)
+    {
+        op.workspace = true;
+        args.push_back(insert_allocation(m, ins, shape{shape::uint8_type, {need}}));
+    }
+    args.push_back(insert_allocation(m, ins, shape{shape::half_type, {rows, n}}));
     m.replace_instruction(ins, operation{op}, args);
     return true;
 }

@@ -548,8 +548,10 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
 
 shape w4a16_gemm::compute_shape(const std::vector<shape>& inputs) const
 {
-    const std::size_t expect = zp_mode == MI355_W4_ZP_SCALAR ? 4 : 5;
+    const std::size_t expect = (zp_mode == MI355_W4_ZP_SCALAR ? 4 : 5) + (workspace ? 1 : 0);
     check_inputs(inputs, expect, name());
+    if(workspace and inputs[inputs.size() - 2].type() != shape::uint8_type)
+        MIGRAPHX_THROW("mi355::w4a16_gemm: the workspace must be a uint8 buffer");
     const auto& a = inputs[0];
     const auto& w = inputs[1];
     const auto& s = inputs[2];
@@ -575,20 +577,23 @@ argument w4a16_gemm::compute(migraphx::context& ctx, const shape& out, const std
     const int64_t k  = static_cast<int64_t>(a.lens()[1]);
     const int64_t n  = static_cast<int64_t>(out.lens()[1]);
     const int64_t lda = m == 1 ? k : static_cast<int64_t>(a.strides()[0]);
-    status_check(mi355_w4a16_gemm(args[0].data(),
-                                  lda,
-                                  args[1].data(),
-                                  args[2].data(),
-                                  zp,
-                                  static_cast<int32_t>(zp_mode),
-                                  static_cast<int32_t>(zp_scalar),
-                                  args.back().data(),
-                                  n,
-                                  m,
-                                  n,
-                                  k,
-                                  group,
-                                  stream_of(ctx)),
+    const auto& room = args[args.size() - 2];
+    status_check(mi355_w4a16_gemm_ws(args[0].data(),
+                                     lda,
+                                     args[1].data(),
+                                     args[2].data(),
+                                     zp,
+                                     static_cast<int32_t>(zp_mode),
+                                     static_cast<int32_t>(zp_scalar),
+                                     args.back().data(),
+                                     n,
+                                     m,
+                                     n,
+                                     k,
+                                     group,
+                                     workspace ? room.data() : nullptr,
+                                     workspace ? room.get_shape().bytes() : 0,
+                                     stream_of(ctx)),
                  name());
     return args.back();
 }

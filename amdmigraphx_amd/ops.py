@@ -306,10 +306,12 @@ def convert(x, out_type, in_type=None):
     return out
 
 
-def w4a16_gemm(a, w_packed, scales, group, zp=8, zp_mode=None, out=None):
+def w4a16_gemm(a, w_packed, scales, group, zp=8, zp_mode=None, out=None, workspace=None):
     """fp16 activations [M, K] times int4 weights packed [N, K/2] with fp16
-    group scales [N, K/group]; zp is an int (per tensor) or a uint8 tensor."""
-    _require_cuda(a, w_packed, scales)
+    group scales [N, K/group]; zp is an int (per tensor) or a uint8 tensor.
+    ``workspace`` (a dense device tensor, see w4a16_gemm_workspace_size) lets shapes whose
+    column tiles do not fill the chip split K."""
+    _require_cuda(a, w_packed, scales, workspace)
     m, k = a.shape
     n = w_packed.shape[0]
     if w_packed.shape[1] * 2 != k:
@@ -321,7 +323,20 @@ def w4a16_gemm(a, w_packed, scales, group, zp=8, zp_mode=None, out=None):
     else:
         zptr, zs = _ptr(zp), 0
         mode = zp_mode if zp_mode is not None else W4ZP.GROUP
+    if workspace is not None:
+        if not workspace.is_contiguous():
+            raise Mi355Error("the workspace must be dense")
+        st = lib().mi355_w4a16_gemm_ws(_ptr(a), a.stride(0), _ptr(w_packed), _ptr(scales), zptr, mode, zs,
+                                       _ptr(out), out.stride(0), m, n, k, group, _ptr(workspace),
+                                       workspace.numel() * workspace.element_size(), _stream())
+        check(st, "mi355_w4a16_gemm_ws")
+        return out
     st = lib().mi355_w4a16_gemm(_ptr(a), a.stride(0), _ptr(w_packed), _ptr(scales), zptr, mode, zs,
                                 _ptr(out), out.stride(0), m, n, k, group, _stream())
     check(st, "mi355_w4a16_gemm")
     return out
+
+
+def w4a16_gemm_workspace_size(m, n, k, group):
+    """Bytes of workspace w4a16_gemm can use for that shape (0: none)."""
+    return int(lib().mi355_w4a16_gemm_workspace_size(m, n, k, group))

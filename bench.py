@@ -271,6 +271,33 @@ def main():
                 "GB/s": round(byts / t4 / 1e9, 1), "TFLOPS": round(2.0 * m4 * n4 * k4 / t4 / 1e12, 1),
                 "us_per_launch": round(t4 * 1e6, 1)}
             del ws
+        # shapes whose 128-column tiles do not fill the chip: K split with a workspace
+        for m4, k4, n4 in ((128, 4096, 4096), (128, 14336, 4096), (512, 4096, 4096)):
+            grp = 128
+            byts = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * m4 * k4 + 2 * m4 * n4
+            copies = int(640e6 // byts) + 1
+            ws = [torch.randint(0, 256, (n4, k4 // 2), dtype=torch.uint8, device=dev, generator=g)
+                  for _ in range(copies)]
+            sc = (torch.rand((n4, k4 // grp), device=dev, generator=g) * 0.015 + 0.005).half()
+            x = torch.randn((m4, k4), device=dev, generator=g).half()
+            y = torch.empty((m4, n4), dtype=torch.float16, device=dev)
+            room = torch.empty(max(ops.w4a16_gemm_workspace_size(m4, n4, k4, grp), 16), dtype=torch.uint8,
+                               device=dev)
+            it = [0]
+
+            def w4s(workspace):
+                def run():
+                    ops.w4a16_gemm(x, ws[it[0] % copies], sc, grp, zp=8, out=y, workspace=workspace)
+                    it[0] += 1
+                return run
+
+            t4, _ = _time_launches(w4s(room), 2 * copies, copies)
+            t4a, _ = _time_launches(w4s(None), 2 * copies, copies)
+            also[f"w4a16_gemm_M{m4}_K{k4}_N{n4}"] = {
+                "GB/s": round(byts / t4 / 1e9, 1), "TFLOPS": round(2.0 * m4 * n4 * k4 / t4 / 1e12, 1),
+                "us_per_launch": round(t4 * 1e6, 1), "us_per_launch_no_workspace": round(t4a * 1e6, 1),
+                "workspace_MiB": room.numel() >> 20}
+            del ws
     except Exception as e:
         also["skinny_error"] = str(e)
 

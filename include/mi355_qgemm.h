@@ -286,6 +286,23 @@ int mi355_w4a16_gemm(const void* a, int64_t lda,
                      int64_t m, int64_t n, int64_t k, int64_t group,
                      void* stream);
 
+/* The same with a workspace.  Between 33 and a few hundred rows against a weight matrix of few
+ * columns (N / 128 tiles do not fill the chip) the tile kernel splits K over more workgroups when
+ * it has room for their float partial sums; a second kernel adds them in a fixed order and
+ * converts to half.  Deterministic, within the path's fp tolerance of the unsplit result (another
+ * order of fp32 additions).  mi355_w4a16_gemm_workspace_size gives the bytes the shape can use
+ * (0: none); a NULL or smaller workspace is not an error.  16-byte aligned device memory, free
+ * again when the call's work is done. */
+size_t mi355_w4a16_gemm_workspace_size(int64_t m, int64_t n, int64_t k, int64_t group);
+int mi355_w4a16_gemm_ws(const void* a, int64_t lda,
+                        const void* w_packed,
+                        const void* scales,
+                        const void* zp, int32_t zp_mode, int32_t zp_scalar,
+                        void* out, int64_t ldc,
+                        int64_t m, int64_t n, int64_t k, int64_t group,
+                        void* workspace, size_t workspace_bytes,
+                        void* stream);
+
 /*
  * Float dot: C[b, m, n] = T( sum_k double(A[b, m, k]) * double(B[b, k, n]) ), k ascending,
  * T in {F32, F16, BF16} for all three tensors (16-bit results truncate, as the software

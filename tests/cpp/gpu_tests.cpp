@@ -662,6 +662,25 @@ TEST_CASE(int4_weight_only_gemm_small_batch)
     EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
 }
 
+TEST_CASE(int4_weight_only_gemm_larger_batch)
+{
+    // more than 32 rows and N a multiple of 128: the tile kernel; where its column tiles do not
+    // fill the chip the lowering adds a workspace and K is split (with packed zero points too)
+    for(bool with_zp : {false, true})
+    {
+        auto p = matmulnbits_program(96, 2048, 256, 128, with_zp, shape::half_type, 54);
+        argument a{shape{shape::half_type, {96, 2048}}, normal_floats(96 * 2048, 1.0f, 55)};
+        expect_close_half(p, {{"a", a}});
+        program c = p;
+        c.compile(migraphx::make_target("mi355"));
+        const auto& mod = *c.get_main_module();
+        EXPECT(count_ops(mod, "mi355::w4a16_gemm") == 1);
+        for(auto ins = mod.begin(); ins != mod.end(); ++ins)
+            if(ins->name() == "mi355::w4a16_gemm")
+                EXPECT(ins->get_operator().to_value().at("workspace").to<bool>());
+    }
+}
+
 TEST_CASE(int4_general_path)
 {
     // float activations, or K that is not a multiple of the block: no fused kernel, the chain

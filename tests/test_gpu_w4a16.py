@@ -135,7 +135,8 @@ def test_w4a16_matrix_core_kernel_exact_weights_all_zero_point_forms(ops):
 # ---- more than 32 rows and N % 128 == 0: the 64 x 128 tile kernel ------------------------
 
 @pytest.mark.parametrize("m,n,k,g", [(33, 128, 128, 128), (64, 256, 384, 128), (65, 128, 1152, 64),
-                                     (100, 384, 2048 + 128, 32), (128, 128, 512, 128)])
+                                     (100, 384, 2048 + 128, 32), (128, 128, 512, 128), (300, 256, 640, 128),
+                                     (129, 128, 384, 64)])
 def test_w4a16_tile_kernel_matches_oracle(ops, m, n, k, g):
     """K an even and an odd multiple of 128 (the last chunk of 256 is then half used), row
     counts that leave the second 64-row block nearly empty, several groups per step."""
@@ -253,3 +254,65 @@ def test_w4a16_full_size_config4_shapes(ops, k, n):
             d = (other.float() - one.float()).abs()
             tol = torch.maximum(one.float().abs() * 2e-3, torch.tensor(2e-3, device="cuda"))
             assert (d <= tol).all(), (r, d.max().item())
+
+
+# ---- the tile kernel with a workspace: K split over more workgroups --------------------------
+
+@pytest.mark.parametrize("m,n,k,g", [(64, 256, 1152, 64), (100, 384, 2048 + 128, 32), (130, 128, 1024, 128),
+                                     (128, 512, 4096, 128), (40, 128, 1536, 128), (300, 256, 1152, 64)])
+def test_w4a16_tile_kernel_split_k_with_workspace(ops, m, n, k, g):
+    """Shares of K leave float partial sums in the workspace, a second kernel adds them in a fixed
+    order: the oracle's value within the path's tolerance, the same bits on every call; K an odd
+    multiple of 128, shares of unequal length, more than 128 rows."""
+    rng = np.random.default_rng(m * 7 + n + k + g)
+    a, packed, scales, wq = _case(rng, m, n, k, g)
+    want = orc.w4a16_matmul(a, packed, scales, 8, g)
+    nbytes = ops.w4a16_gemm_workspace_size(m, n, k, g)
+    assert nbytes > 0
+    ws = torch.full((nbytes,), 0x7F, dtype=torch.uint8, device="cuda")
+    print("w4a16 tile workspace", m, n, k, g, nbytes, flush=True)
+    out = torch.zeros((m, n + 8), dtype=torch.float16, device="cuda")
+    ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8, out=out[:, :n], workspace=ws)
+    got = out[:, :n].contiguous()
+    again = ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8, workspace=ws)
+    assert torch.equal(got.view(torch.int16), again.view(torch.int16))
+    assert (out[:, n:] == 0).all()
+    wdq = orc.dequantizelinear(wq, np.repeat(scales, g, axis=1), np.full(wq.shape, 8, np.uint8),
+                               orc.U8, orc.F16)
+    _check(half_bits(got), want, a, wdq)
+    # a workspace that is too small is not an error
+    small = torch.empty(256, dtype=torch.uint8, device="cuda")
+    one_pass = ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8)
+    assert torch.equal(ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8,
+                                      workspace=small).view(torch.int16), one_pass.view(torch.int16))
+
+
+def test_w4a16_tile_kernel_split_k_exact_weights(ops):
+    """One-hot activations: every partial sum is one dequantized weight or zero, so the split
+    result must match the oracle bit for bit, for the three zero-point forms."""
+    rng = np.random.default_rng(23)
+    n, k, g, m = 256, 1280, 32, 70
+    wq = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = orc.pack_int4(wq)
+    a = np.zeros((m, k), np.float32)
+    for i in range(m):
+        a[i, (i * 53 + 7) % k] = 1.0 if i % 2 == 0 else -2.0
+    ab = orc.half_from_f32(a)
+    scales = orc.half_from_f32(rng.uniform(0.005, 0.02, (n, k // g)).astype(np.float32))
+    zp = rng.integers(0, 16, (n, k // g), dtype=np.uint8)
+    nbytes = ops.w4a16_gemm_workspace_size(m, n, k, g)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    for zmode in ("scalar", "group", "packed"):
+        print("w4a16 tile workspace exact", zmode, flush=True)
+        if zmode == "scalar":
+            want = orc.w4a16_matmul(ab, packed, scales, 3, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=3, workspace=ws)
+        elif zmode == "group":
+            want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=dev(zp), workspace=ws)
+        else:
+            want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g,
+                                 zp=dev(orc.pack_int4(zp)), zp_mode=ops.W4ZP.PACKED, workspace=ws)
+        assert np.array_equal(half_bits(got), want), zmode
