@@ -420,10 +420,21 @@ extern "C" int mi355_w4a16_gemm(const void* a,
 
 extern "C" size_t mi355_w4a16_gemm_workspace_size(int64_t m, int64_t n, int64_t k, int64_t group)
 {
-    if(m <= 32 || n <= 0 || k <= 0 || group <= 0 || n % TL_BN != 0 || k % 128 != 0 || k > (1 << 30) ||
-       n > (1 << 30) || m > (1 << 30))
+    if(m < 2 || n <= 0 || k <= 0 || group <= 0 || k % 128 != 0 || n % 16 != 0 || k > (1 << 30) || n > (1 << 30) ||
+       m > (1 << 30))
         return 0;
-    const int shares = tile_gemm_shares((int)m, (int)n, (int)k);
+    if(m > 32 && n % TL_BN == 0)
+    {
+        const int shares = tile_gemm_shares((int)m, (int)n, (int)k);
+        return shares > 1 ? (size_t)shares * m * n * 4 : 0;
+    }
+    // the matrix-core kernel for few rows: the widest column tile any zero-point form may take
+    // (an upper bound for the others)
+    int shares = 1;
+    if(m <= 32)
+        shares = mfma_gemm_shares<4>((int)n, (int)k);
+    else if(m <= 64)
+        shares = mfma_gemm_shares<2>((int)n, (int)k);
     return shares > 1 ? (size_t)shares * m * n * 4 : 0;
 }
 

@@ -81,6 +81,10 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
     const int groups  = p.k / p.group;
     const int nsteps  = p.k >> 7;
     const int nchunks = (p.k + WL_CHUNK_K - 1) / WL_CHUNK_K;
+    // K split over blockIdx.z (p.partial set): this workgroup walks chunks cbase .. cbase + nloc - 1
+    // and leaves float sums in partial[blockIdx.z]; every share holds at least one chunk
+    const int cbase = p.partial != nullptr ? (int)blockIdx.z * p.chunks_per_share : 0;
+    const int nloc  = p.partial != nullptr ? min(p.chunks_per_share, nchunks - cbase) : nchunks;
 
     // half-precision arithmetic of this wave truncates from here on (MODE.fp_round bits 3:2); the
     // fp32 accumulation of the matrix cores keeps round-to-nearest
@@ -89,8 +93,9 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
     // ---- weight stream: global -> LDS ring ----------------------------------------------------
     // one instruction per weight row; lanes past the end of K in the last chunk stay off
     const uint8_t* wbase = p.w + (int64_t)n0 * kbytes;
-    auto issue_chunk     = [&](int c) {
-        uint8_t* slot   = lds + (c % RING) * CHUNK_BYTES;
+    auto issue_chunk     = [&](int cl) {
+        uint8_t* slot   = lds + (cl % RING) * CHUNK_BYTES;
+        const int c     = cbase + cl;
         const int valid = min(WL_ROW, kbytes - c * WL_ROW);
         if(lane * 16 < valid)
         {
@@ -308,18 +313,18 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
     {
 #pragma unroll
         for(int c = 0; c < RING - 1; c++)
-            if(c < nchunks)
+            if(c < nloc)
                 issue_chunk(c);
-        for(int c = 0; c < nchunks; c++)
+        for(int c = 0; c < nloc; c++)
         {
             // (the counter holds at most 63: waiting for one load more than needed is harmless)
             constexpr int AHEAD = (RING - 2) * 16 * NT;
-            if(c + RING - 2 < nchunks)
+            if(c + RING - 2 < nloc)
                 wl_wait_vmcnt<(AHEAD < 63 ? AHEAD : 63)>();
             else
                 wl_wait_vmcnt<0>();
             wl_barrier();
-            if(c + RING - 1 < nchunks)
+            if(c + RING - 1 < nloc)
                 issue_chunk(c + RING - 1);
         }
     }
@@ -328,14 +333,14 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
         // this wave's steps: step-in-chunk wave (and wave + 8 where a chunk has 16 steps) of every
         // chunk; two input sets alternate from step to step
         step_inputs in[2];
-        request(in[0], wave);
+        request(in[0], cbase * SPC + wave);
         if constexpr(SPW == 2)
         {
-            for(int c = 0; c < nchunks; c++)
+            for(int c = 0; c < nloc; c++)
             {
                 wl_barrier();
                 const uint32_t slot_addr = lds0 + (c % RING) * CHUNK_BYTES;
-                const int step0          = c * SPC + wave;
+                const int step0          = (cbase + c) * SPC + wave;
                 request(in[1], step0 + WL_WAVES);
                 if(step0 < nsteps)
                     do_step(in[0], step0, slot_addr, wave);
@@ -346,14 +351,14 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
         }
         else
         {
-            for(int c = 0; c < nchunks; c += 2)
+            for(int c = 0; c < nloc; c += 2)
             {
                 wl_barrier();
-                const int step0 = c * SPC + wave;
+                const int step0 = (cbase + c) * SPC + wave;
                 request(in[1], step0 + SPC);
                 if(step0 < nsteps)
                     do_step(in[0], step0, lds0 + (c % RING) * CHUNK_BYTES, wave);
-                if(c + 1 < nchunks)
+                if(c + 1 < nloc)
                 {
                     wl_barrier();
                     request(in[0], step0 + 2 * SPC);
@@ -390,9 +395,53 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_mfma_kernel(w4_params p)
         const int t = tir / (MT * 4);
         const int i = (tir >> 2) % MT;
         const int m = 16 * i + 4 * (l >> 4) + (tir & 3);
-        if(m < p.m)
+        if(m >= p.m)
+            continue;
+        if(p.partial != nullptr)
+            p.partial[((int64_t)blockIdx.z * p.m + m) * p.n + n0 + 16 * t + (l & 15)] = s;
+        else
             p.out[(int64_t)m * p.ldc + n0 + 16 * t + (l & 15)] = f32_to_half_rtz(s);
     }
+}
+
+// out = half(sum of the shares' float partial sums), 4 columns per thread, shares added in order
+__global__ __launch_bounds__(256) void w4a16_reduce_kernel(const float* partial, uint16_t* out, int m, int n,
+                                                            int64_t ldc, int shares)
+{
+    const int64_t mn = (int64_t)m * n;
+    const int64_t e  = 4 * ((int64_t)blockIdx.x * 256 + threadIdx.x);
+    if(e >= mn)
+        return;
+    v4f sum = *reinterpret_cast<const v4f*>(partial + e);
+    for(int z = 1; z < shares; z++)
+        sum += *reinterpret_cast<const v4f*>(partial + (int64_t)z * mn + e);
+    uint16_t* o = out + (e / n) * ldc + (e % n);
+#pragma unroll
+    for(int r = 0; r < 4; r++)
+        o[r] = f32_to_half_rtz(sum[r]);
+}
+
+int launch_w4a16_reduce(const w4_params& p, int shares, hipStream_t s)
+{
+    const int64_t quads = (int64_t)p.m * p.n / 4;
+    hipLaunchKernelGGL(w4a16_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p.partial, p.out,
+                       p.m, p.n, p.ldc, shares);
+    return mi355_launch_status();
+}
+
+// shares of K for the widest column tile: one workgroup per CU, at least one chunk per share.
+// The second kernel costs 3-4 us, which the split only wins back with few column tiles and a
+// long K (measured at 16 and 32 rows: K = 14336, N = 4096 gains, 4096 x 4096 and 8192 x 8192 do
+// not).
+template <int NT>
+int mfma_gemm_shares(int n, int k)
+{
+    constexpr int chunk_k = NT >= 4 ? 1024 : 2048;
+    const int tiles       = n / (16 * NT);
+    const int nchunks     = (k + chunk_k - 1) / chunk_k;
+    if(n % (16 * NT) != 0 || n % 4 != 0 || tiles > 64 || nchunks < 8)
+        return 1;
+    return max(1, min((256 + tiles - 1) / tiles, nchunks));
 }
 
 bool mfma_gemm_supported(const w4_params& p)
@@ -403,10 +452,25 @@ bool mfma_gemm_supported(const w4_params& p)
 }
 
 template <int MT, int NT, bool SIMPLE>
-int launch_mfma_variant(const w4_params& p, hipStream_t s)
+int launch_mfma_variant(const w4_params& p0, hipStream_t s)
 {
+    w4_params p = p0;
+    p.partial   = nullptr;
     hipLaunchKernelGGL((w4a16_mfma_kernel<MT, NT, SIMPLE>), dim3(p.n / (16 * NT)), dim3(WL_THREADS), 0, s, p);
     return mi355_launch_status();
+}
+
+// the widest tile with K split over `shares` workgroups, then the sum of their partial tiles
+template <int MT, int NT, bool SIMPLE>
+int launch_mfma_split(const w4_params& p0, int shares, hipStream_t s)
+{
+    constexpr int chunk_k = NT >= 4 ? 1024 : 2048;
+    w4_params p           = p0;
+    const int nchunks     = (p.k + chunk_k - 1) / chunk_k;
+    p.chunks_per_share    = (nchunks + shares - 1) / shares;
+    const int z           = (nchunks + p.chunks_per_share - 1) / p.chunks_per_share;
+    hipLaunchKernelGGL((w4a16_mfma_kernel<MT, NT, SIMPLE>), dim3(p.n / (16 * NT), 1, z), dim3(WL_THREADS), 0, s, p);
+    return launch_w4a16_reduce(p, z, s);
 }
 
 // Every workgroup reads all of A's rows once, from L2: M*K*2 bytes per workgroup against the
@@ -417,6 +481,13 @@ template <int MT, int NT_MAX, bool SIMPLE>
 int launch_mfma_tiles(const w4_params& p, hipStream_t s)
 {
     constexpr int64_t enough = 200;
+    if constexpr(NT_MAX >= 2)
+    {
+        // with room for partial sums: the widest tile (fewest re-reads of A) and K split
+        const int shares = mfma_gemm_shares<NT_MAX>(p.n, p.k);
+        if(p.partial != nullptr && shares > 1 && (size_t)shares * p.m * p.n * 4 <= p.partial_bytes)
+            return launch_mfma_split<MT, NT_MAX, SIMPLE>(p, shares, s);
+    }
     if constexpr(NT_MAX >= 4)
     {
         if(p.n % 64 == 0 && p.n / 64 >= enough)

@@ -333,23 +333,6 @@ __global__ __launch_bounds__(WL_THREADS) void w4a16_tile_kernel(w4_params p)
         }
 }
 
-// out = half(sum of the shares' float partial sums), 4 columns per thread, shares added in order
-__global__ __launch_bounds__(256) void w4a16_reduce_kernel(const float* partial, uint16_t* out, int m, int n,
-                                                            int64_t ldc, int shares)
-{
-    const int64_t mn = (int64_t)m * n;
-    const int64_t e  = 4 * ((int64_t)blockIdx.x * 256 + threadIdx.x);
-    if(e >= mn)
-        return;
-    v4f sum = *reinterpret_cast<const v4f*>(partial + e);
-    for(int z = 1; z < shares; z++)
-        sum += *reinterpret_cast<const v4f*>(partial + (int64_t)z * mn + e);
-    uint16_t* o = out + (e / n) * ldc + (e % n);
-#pragma unroll
-    for(int r = 0; r < 4; r++)
-        o[r] = f32_to_half_rtz(sum[r]);
-}
-
 // shares of K for `m` rows: enough workgroups for every CU (a workgroup
 // fills one), at least two chunks per share; 1 = no split
 int tile_gemm_shares(int m, int n, int k)
@@ -389,10 +372,6 @@ int launch_tile_gemm(const w4_params& p0, hipStream_t s)
     else
         hipLaunchKernelGGL((w4a16_tile_kernel<4, false>), grid, dim3(WL_THREADS), 0, s, p);
     if(p.partial != nullptr)
-    {
-        const int64_t quads = (int64_t)p.m * p.n / 4;
-        hipLaunchKernelGGL(w4a16_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p.partial,
-                           p.out, p.m, p.n, p.ldc, (int)grid.z);
-    }
+        return launch_w4a16_reduce(p, (int)grid.z, s);
     return mi355_launch_status();
 }

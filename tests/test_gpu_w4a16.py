@@ -316,3 +316,57 @@ def test_w4a16_tile_kernel_split_k_exact_weights(ops):
             got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g,
                                  zp=dev(orc.pack_int4(zp)), zp_mode=ops.W4ZP.PACKED, workspace=ws)
         assert np.array_equal(half_bits(got), want), zmode
+
+
+# ---- the matrix-core kernel for few rows with a workspace: widest column tile, K split ----------
+
+@pytest.mark.parametrize("m,n,k,g", [(16, 256, 8192, 128), (2, 64, 8192 + 128, 64), (17, 320, 8192, 128),
+                                     (40, 96, 16384 + 128, 32), (48, 160, 16384 + 128, 128),
+                                     (32, 1024, 14336, 128)])
+def test_w4a16_matrix_core_kernel_split_k_with_workspace(ops, m, n, k, g):
+    rng = np.random.default_rng(m * 5 + n + k + g)
+    a, packed, scales, wq = _case(rng, m, n, k, g)
+    want = orc.w4a16_matmul(a, packed, scales, 8, g)
+    nbytes = ops.w4a16_gemm_workspace_size(m, n, k, g)
+    assert nbytes > 0
+    ws = torch.full((nbytes,), 0x7F, dtype=torch.uint8, device="cuda")
+    print("w4a16 mfma workspace", m, n, k, g, nbytes, flush=True)
+    out = torch.zeros((m, n + 8), dtype=torch.float16, device="cuda")
+    ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8, out=out[:, :n], workspace=ws)
+    got = out[:, :n].contiguous()
+    again = ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), g, zp=8, workspace=ws)
+    assert torch.equal(got.view(torch.int16), again.view(torch.int16))
+    assert (out[:, n:] == 0).all()
+    wdq = orc.dequantizelinear(wq, np.repeat(scales, g, axis=1), np.full(wq.shape, 8, np.uint8),
+                               orc.U8, orc.F16)
+    _check(half_bits(got), want, a, wdq)
+
+
+def test_w4a16_matrix_core_kernel_split_k_exact_weights(ops):
+    """One-hot activations, the three zero-point forms: bit for bit the oracle's weights."""
+    rng = np.random.default_rng(24)
+    n, k, g, m = 128, 8192, 32, 12
+    wq = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = orc.pack_int4(wq)
+    a = np.zeros((m, k), np.float32)
+    for i in range(m):
+        a[i, (i * 531 + 7) % k] = 1.0 if i % 2 == 0 else -2.0
+    ab = orc.half_from_f32(a)
+    scales = orc.half_from_f32(rng.uniform(0.005, 0.02, (n, k // g)).astype(np.float32))
+    zp = rng.integers(0, 16, (n, k // g), dtype=np.uint8)
+    nbytes = ops.w4a16_gemm_workspace_size(m, n, k, g)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    for zmode in ("scalar", "group", "packed"):
+        print("w4a16 mfma workspace exact", zmode, flush=True)
+        if zmode == "scalar":
+            want = orc.w4a16_matmul(ab, packed, scales, 3, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=3, workspace=ws)
+        elif zmode == "group":
+            want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g, zp=dev(zp), workspace=ws)
+        else:
+            want = orc.w4a16_matmul(ab, packed, scales, zp, g)
+            got = ops.w4a16_gemm(half_dev(ab), dev(packed), half_dev(scales), g,
+                                 zp=dev(orc.pack_int4(zp)), zp_mode=ops.W4ZP.PACKED, workspace=ws)
+        assert np.array_equal(half_bits(got), want), zmode
