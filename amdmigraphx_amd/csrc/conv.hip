@@ -175,6 +175,39 @@ void launch_im2col(const im2col_params& p, hipStream_t stream)
                        0, stream, p);
 }
 
+// the batched GEMM of one group: weights [O/G, Kp] times the group's window matrix [P, Kp]^T per image
+mi355_quant_dot_desc gemm_of(const mi355_quant_conv_desc* d, int64_t plane, int64_t kp)
+{
+    mi355_quant_dot_desc g{};
+    g.m            = d->o / d->group;
+    g.n            = plane;
+    g.k            = kp;
+    g.lda          = kp;
+    g.ldb          = kp;
+    g.ldc          = plane;
+    g.batch        = d->n;
+    g.stride_a     = 0;
+    g.stride_b     = d->group * plane * kp;
+    g.stride_c     = d->o * plane;
+    g.trans_a      = 0;
+    g.trans_b      = 1;
+    g.in_type      = d->in_type;
+    g.out_type     = d->out_type;
+    g.dequant      = d->dequant;
+    // the weights are the GEMM's first operand: one scale per output channel is one per row
+    g.scale_a_mode = d->dequant ? d->scale_w_mode : MI355_QP_NONE;
+    g.scale_b_mode = d->dequant ? d->scale_x_mode : MI355_QP_NONE;
+    return g;
+}
+
+// window matrix + reordered weights + channels-last copy, rounded up so that what follows (room for
+// the GEMM's split-K partial sums) is 16-byte aligned
+size_t staging_bytes(const mi355_quant_conv_desc* d, int64_t plane, int64_t kp)
+{
+    const size_t b = (size_t)((d->n * d->group * plane + d->o) * kp + d->n * d->c * d->h * d->w);
+    return (b + 15) / 16 * 16;
+}
+
 } // namespace
 
 extern "C" int mi355_quant_convolution_dims(const mi355_quant_conv_desc* d,
@@ -193,7 +226,11 @@ extern "C" int mi355_quant_convolution_dims(const mi355_quant_conv_desc* d,
     if(ow != nullptr)
         *ow = w_out;
     if(workspace_bytes != nullptr)
-        *workspace_bytes = (size_t)((d->n * d->group * h_out * w_out + d->o) * kp + d->n * d->c * d->h * d->w);
+    {
+        // few output tiles (small images, one image at a time): the GEMM splits K when it has room
+        const mi355_quant_dot_desc g = gemm_of(d, h_out * w_out, kp);
+        *workspace_bytes             = staging_bytes(d, h_out * w_out, kp) + mi355_quant_dot_workspace_size(&g);
+    }
     return MI355_OK;
 }
 
@@ -358,34 +395,19 @@ extern "C" int mi355_quant_convolution(const mi355_quant_conv_desc* d,
             return MI355_ERR_LAUNCH;
     }
 
-    mi355_quant_dot_desc g{};
-    g.m            = og;
-    g.n            = plane;
-    g.k            = kp;
-    g.lda          = kp;
-    g.ldb          = kp;
-    g.ldc          = plane;
-    g.batch        = d->n;
-    g.stride_a     = 0;
-    g.stride_b     = d->group * plane * kp;
-    g.stride_c     = d->o * plane;
-    g.trans_a      = 0;
-    g.trans_b      = 1;
-    g.in_type      = d->in_type;
-    g.out_type     = d->out_type;
-    g.dequant      = d->dequant;
-    // the weights are the GEMM's first operand: one scale per output channel is one per row
-    g.scale_a_mode = d->dequant ? d->scale_w_mode : MI355_QP_NONE;
-    g.scale_b_mode = d->dequant ? d->scale_x_mode : MI355_QP_NONE;
+    const mi355_quant_dot_desc g = gemm_of(d, plane, kp);
+    void* room                   = static_cast<uint8_t*>(workspace) + staging_bytes(d, plane, kp);
+    const size_t room_bytes      = need - staging_bytes(d, plane, kp);
     const size_t esz = mi355_dtype_size(d->out_type);
     for(int64_t grp = 0; grp < d->group; grp++)
     {
         const float* sw = scale_w;
         if(d->dequant && d->scale_w_mode == MI355_QP_PER_ROW)
             sw = scale_w + grp * og;
-        const int r = mi355_quant_dot(&g, wmat + grp * og * kp, col + grp * plane * kp,
-                                      static_cast<uint8_t*>(out) + (size_t)(grp * og * plane) * esz, sw, scale_x,
-                                      nullptr, nullptr, stream);
+        const int r = mi355_quant_dot_ws(&g, wmat + grp * og * kp, col + grp * plane * kp,
+                                         static_cast<uint8_t*>(out) + (size_t)(grp * og * plane) * esz, sw, scale_x,
+                                         nullptr, nullptr, nullptr, room_bytes > 0 ? room : nullptr, room_bytes,
+                                         stream);
         if(r != MI355_OK)
             return r;
     }

@@ -59,7 +59,9 @@ struct dma_params
     int zp_a, zp_b;
     int ksplit; // workgroups along K per output tile (blockIdx.z), int8 split-K kernel only
     int32_t* partial; // split-K with a workspace: share z of batch b writes its tile sums to
-                      // partial[(b * ksplit + z)][m][n] with plain stores; null = atomic adds into C
+                      // partial[(b * ksplit + z)][m][partial_ld] with plain stores; null = atomic adds
+                      // into C
+    int partial_ld;   // n rounded up to 4: a group of 4 columns that starts inside n is stored whole
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
     int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
 };
@@ -1006,7 +1008,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                     if(p.partial != nullptr)
                     {
                         int32_t* w = p.partial +
-                                     (((int64_t)blockIdx.y * p.ksplit + blockIdx.z) * p.m + row) * p.n + col;
+                                     (((int64_t)blockIdx.y * p.ksplit + blockIdx.z) * p.m + row) * p.partial_ld +
+                                     col;
                         *reinterpret_cast<v4i*>(w) = acc[i][j];
                     }
                     else
@@ -1093,15 +1096,16 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* c, int m, int n,
 // each add every fourth share and the first one collects the four sums through the LDS.  int8:
 // integer sums, any order gives the same bits, and the dequantizing epilogue is the arithmetic of
 // the one-pass kernel's.  fp8: float partial sums added in this fixed order (the same bits on every
-// run; not those of the one-pass kernel, whose one accumulator walks K in another order).  N, ldc
-// and the batch stride of C are multiples of 4 on this path.
-template <bool FP8, bool DEQ, int OUT>
+// run; not those of the one-pass kernel, whose one accumulator walks K in another order).  VEC: N,
+// ldc and the batch stride of C are multiples of 4 and C is aligned for a store of 4 outputs;
+// otherwise the outputs leave one by one (the partial rows are padded to a multiple of 4).
+template <bool FP8, bool DEQ, int OUT, bool VEC>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int shares)
 {
     using acc_t = std::conditional_t<FP8, float, int32_t>;
     using vec_t = acc_t __attribute__((ext_vector_type(4)));
     __shared__ vec_t part[3][64];
-    const int64_t mn  = (int64_t)p.m * p.n;
+    const int64_t mn  = (int64_t)p.m * p.partial_ld;
     const int64_t q   = (int64_t)blockIdx.x * 64 + threadIdx.x;
     const bool inside = 4 * q < mn;
     const acc_t* src  = reinterpret_cast<const acc_t*>(p.partial) + (int64_t)blockIdx.y * p.ksplit * mn + 4 * q;
@@ -1118,11 +1122,21 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
     if(threadIdx.y != 0 || !inside)
         return;
     sum               = ((sum + part[0][threadIdx.x]) + part[1][threadIdx.x]) + part[2][threadIdx.x];
-    const int row     = (int)(4 * q / p.n);
-    const int col     = (int)(4 * q % p.n);
+    const int row     = (int)(4 * q / p.partial_ld);
+    const int col     = (int)(4 * q % p.partial_ld);
     const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
     if constexpr(!DEQ)
-        *reinterpret_cast<vec_t*>(static_cast<acc_t*>(p.c) + idx) = sum;
+    {
+        if constexpr(VEC)
+            *reinterpret_cast<vec_t*>(static_cast<acc_t*>(p.c) + idx) = sum;
+        else
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+                if(col + e < p.n)
+                    static_cast<acc_t*>(p.c)[idx + e] = sum[e];
+        }
+    }
     else
     {
         float sa = 1.f;
@@ -1137,23 +1151,31 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
 #pragma unroll
         for(int e = 0; e < 4; e++)
         {
-            float sb = 1.f;
+            const int c = min(col + e, p.n - 1);
+            float sb    = 1.f;
             if(p.scale_b_mode == MI355_QP_PER_TENSOR)
                 sb = p.scale_b[0];
             else if(p.scale_b_mode == MI355_QP_PER_COL)
-                sb = p.scale_b[col + e];
-            const float bias = p.bias != nullptr ? p.bias[col + e] : -0.0f;
+                sb = p.scale_b[c];
+            const float bias = p.bias != nullptr ? p.bias[c] : -0.0f;
             const float s    = sa * sb;
             if constexpr(FP8)
                 v[e] = add_bias((float)sum[e] * s, bias);
             else
             {
-                const int32_t cs = p.zp_a != 0 ? p.colsum_b[col + e] : 0;
+                const int32_t cs = p.zp_a != 0 ? p.colsum_b[c] : 0;
                 const double d   = (double)sum[e] - (double)(int32_t)(zrow + (int64_t)p.zp_a * cs);
                 v[e]             = add_bias((float)(d * (double)s), bias);
             }
         }
-        if constexpr(OUT == MI355_F32)
+        if constexpr(!VEC)
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+                if(col + e < p.n)
+                    store1<OUT>(p.c, idx + e, v[e]);
+        }
+        else if constexpr(OUT == MI355_F32)
             *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) = v4f{v[0], v[1], v[2], v[3]};
         else if constexpr(OUT == MI355_F16)
             *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) =
@@ -1166,20 +1188,28 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
     }
 }
 
+template <bool FP8, bool VEC>
+int launch_reduce_vec(const dma_params& p, int batch, int shares, bool deq, int out_type, hipStream_t stream)
+{
+    const int64_t quads = (int64_t)p.m * p.partial_ld / 4;
+    const dim3 grid((unsigned)((quads + 63) / 64), batch), block(64, 4);
+    if(!deq)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, false, MI355_F32, VEC>), grid, block, 0, stream, p, shares);
+    else if(out_type == MI355_F32)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F32, VEC>), grid, block, 0, stream, p, shares);
+    else if(out_type == MI355_F16)
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F16, VEC>), grid, block, 0, stream, p, shares);
+    else
+        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_BF16, VEC>), grid, block, 0, stream, p, shares);
+    return mi355_launch_status();
+}
+
 template <bool FP8>
 int launch_reduce(const dma_params& p, int batch, int shares, bool deq, int out_type, hipStream_t stream)
 {
-    const int64_t quads = (int64_t)p.m * p.n / 4;
-    const dim3 grid((unsigned)((quads + 63) / 64), batch), block(64, 4);
-    if(!deq)
-        hipLaunchKernelGGL((reduce_partials_kernel<FP8, false, MI355_F32>), grid, block, 0, stream, p, shares);
-    else if(out_type == MI355_F32)
-        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F32>), grid, block, 0, stream, p, shares);
-    else if(out_type == MI355_F16)
-        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_F16>), grid, block, 0, stream, p, shares);
-    else
-        hipLaunchKernelGGL((reduce_partials_kernel<FP8, true, MI355_BF16>), grid, block, 0, stream, p, shares);
-    return mi355_launch_status();
+    const bool vec = p.vec_store && p.n % 4 == 0;
+    return vec ? launch_reduce_vec<FP8, true>(p, batch, shares, deq, out_type, stream)
+               : launch_reduce_vec<FP8, false>(p, batch, shares, deq, out_type, stream);
 }
 
 // deq / out_type: the epilogue of the second kernel on the workspace path (the atomic path gives
@@ -1352,17 +1382,17 @@ size_t mi355_dma_gemm_workspace(const mi355_quant_dot_desc* d)
 {
     if(d->in_type == MI355_FP8)
     {
-        if(d->trans_a || d->n % 4 != 0 || d->ldc % 4 != 0)
+        if(d->trans_a || d->n % 4 != 0 || d->ldc % 4 != 0 || (!d->trans_b && d->n % 16 != 0))
             return 0;
         const int s = fp8_shares(d);
         return s > 1 ? (size_t)s * d->m * d->n * 4 : 0;
     }
-    if(d->in_type != MI355_I8 || d->trans_a || d->k % BK != 0 || d->k < BK || d->n % 4 != 0 ||
-       d->ldc % 4 != 0 || d->stride_c % 4 != 0 || d->m <= 0 || d->n <= 0 || d->batch <= 0)
+    if(d->in_type != MI355_I8 || d->trans_a || d->k % BK != 0 || d->k < BK || d->m <= 0 || d->n <= 0 ||
+       d->batch <= 0 || (!d->trans_b && d->n % 16 != 0))
         return 0;
     const int tiles = (int)(((d->m + BM - 1) / BM) * ((d->n + BN - 1) / BN));
     const int s     = choose_ksplit_ws(tiles, (int)d->batch, (int)(d->k / BK), d->m, d->n, d->k);
-    return s > 1 ? (size_t)s * d->batch * d->m * d->n * 4 : 0;
+    return s > 1 ? (size_t)s * d->batch * d->m * ((d->n + 3) / 4 * 4) * 4 : 0;
 }
 
 int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
@@ -1381,6 +1411,7 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     dma_params p;
     p.bias         = bias;
     p.partial      = nullptr;
+    p.partial_ld   = (int)((d->n + 3) / 4 * 4);
     p.a            = static_cast<const uint8_t*>(a);
     p.b            = static_cast<const uint8_t*>(b);
     p.c            = c;
@@ -1450,16 +1481,11 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     const size_t osz = deq ? mi355_dtype_size(d->out_type) : 4;
     const bool vec   = d->n % 4 == 0 && d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
                      reinterpret_cast<uintptr_t>(c) % (4 * osz) == 0;
-    if(d->n % 4 != 0)
-        // the 16 x 16 kernel drops or keeps 4 columns together
-        return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
-                          : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
-    p.ksplit = 1;
-    if(vec && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+    if(workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
        (!deq || d->out_type == MI355_F32 || d->out_type == MI355_F16 || d->out_type == MI355_BF16))
     {
         const int s = choose_ksplit_ws(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);
-        if(s > 1 && (size_t)s * d->batch * d->m * d->n * 4 <= workspace_bytes)
+        if(s > 1 && (size_t)s * d->batch * d->m * p.partial_ld * 4 <= workspace_bytes)
         {
             p.ksplit  = s;
             p.partial = static_cast<int32_t*>(workspace);
@@ -1467,6 +1493,11 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                               : launch_i8_splitk<false>(p, (int)d->batch, stream, deq, d->out_type);
         }
     }
+    if(d->n % 4 != 0)
+        // the 16 x 16 kernel drops or keeps 4 columns together
+        return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+    p.ksplit = 1;
     if(vec && !deq)
     {
         p.ksplit = choose_ksplit(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);

@@ -221,8 +221,8 @@ TEST_CASE(qdq_linear_layer_skinny)
 {
     // A few rows against a large weight matrix (decoding, small batches): the lowering hands the
     // quant_dot a workspace so that K is split over the chip, the second kernel applies the
-    // epilogue.  Still one mi355::quant_dot, bit-identical to the CPU target; a large-M layer
-    // gets no workspace.
+    // epilogue.  Still one mi355::quant_dot, bit-identical to the CPU target; a layer
+    // with a short K gets no workspace.
     struct layer
     {
         std::size_t m, k, n;
@@ -232,9 +232,9 @@ TEST_CASE(qdq_linear_layer_skinny)
     };
     for(auto c : {layer{16, 4096, 1024, 0, 0, true, true, shape::float_type},
                   layer{1, 2048, 512, 0, 0, false, true, shape::float_type},
-                  layer{40, 1600, 300, 3, -2, false, true, shape::float_type},
+                  layer{40, 1600, 304, 3, -2, false, true, shape::float_type},
                   layer{128, 3072, 768, 0, 0, true, true, shape::half_type},
-                  layer{2048, 1024, 1024, 0, 0, true, false, shape::float_type}})
+                  layer{2048, 256, 1024, 0, 0, true, false, shape::float_type}})
     {
         auto p = qdq_matmul(c.m, c.k, c.n, c.weight_nk, c.zp_x, c.zp_w, c.type, 31);
         migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});

@@ -42,6 +42,10 @@ CASES = [
     ((2, 64, 9, 11), (32, 32, 3, 2), (1, 0, 2, 1), (2, 1), (1, 2), 2),
     ((1, 16, 7, 7), (5, 16, 5, 5), (2, 2), (1, 1), (1, 1), 1),         # K = 400 -> 448
     ((3, 48, 6, 5), (7, 48, 2, 2), (0, 0), (1, 1), (1, 1), 1),
+    # one image, deep K, one output tile: the GEMM splits K inside the convolution's workspace
+    ((1, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 128, 12, 12), (96, 64, 5, 5), (2, 2), (1, 1), (1, 1), 2),
+    ((1, 512, 7, 7), (64, 512, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # 49 positions: N % 4 != 0 in the split
 ]
 
 
@@ -81,6 +85,28 @@ def test_int8_dequant_epilogue_bit_exact(ops, out, per_channel):
     else:
         ot = orc.F16 if out == "f16" else orc.BF16
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_int8_dequant_epilogue_with_split_k(ops, out):
+    """One image of a deep layer: K is split over the chip and the second kernel applies the
+    per-output-channel scale (a row scale of the GEMM); same bits as the oracle."""
+    rng = np.random.default_rng(6)
+    xs, ws = (1, 256, 14, 14), (256, 256, 3, 3)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.0213)
+    sw = rng.uniform(0.001, 0.01, 256).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (1, 1), (1, 1), (1, 1), 1)
+    scale = np.broadcast_to((sx * sw).astype(np.float32).reshape(1, -1, 1, 1), acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    td = torch.float32 if out == "f32" else torch.bfloat16
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 1, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.BF16))
 
 
 def test_fp8_convolution(ops):

@@ -542,7 +542,8 @@ def test_full_size_fp8_config3_shapes(ops, k, n):
 # exact in any order) and of the oracle
 @pytest.mark.parametrize("m,n,k,batch,trans_b", [
     (16, 1024, 4096, 1, False), (16, 1024, 4096, 1, True), (128, 512, 2048, 1, False), (1, 256, 8192, 1, True),
-    (33, 260, 1024, 2, False), (40, 300, 1600, 1, True), (8, 256, 2112, 1, False), (16, 8192, 8192, 1, False), (128, 8192, 8192, 1, True),
+    (33, 260, 1024, 2, True), (40, 300, 1600, 1, True), (8, 256, 2112, 1, False),
+    (16, 1023, 4096, 1, True), (40, 301, 1600, 2, True),  # N % 4 != 0: padded partial rows, scalar stores (16, 8192, 8192, 1, False), (128, 8192, 8192, 1, True),
 ])
 def test_int8_split_k_with_workspace_bit_exact(ops, m, n, k, batch, trans_b):
     g = torch.Generator().manual_seed(m * 7 + n + k)
@@ -552,7 +553,7 @@ def test_int8_split_k_with_workspace_bit_exact(ops, m, n, k, batch, trans_b):
     dbv = db.transpose(1, 2) if trans_b else db
     bytes_ = ops.quant_dot_workspace_size(m, n, k, batch, trans_b)
     assert bytes_ > 0, "these shapes are meant to take the split"
-    assert bytes_ % (batch * m * n * 4) == 0
+    assert bytes_ % (batch * m * ((n + 3) // 4 * 4) * 4) == 0  # partial rows are padded to 4 columns
     ws = torch.full((bytes_ // 4,), 0x55555555, dtype=torch.int32, device="cuda")
     got = ops.quant_dot(da, dbv, workspace=ws)
     ref = ops.quant_dot(da, dbv)
@@ -575,8 +576,9 @@ def test_workspace_size_is_zero_where_no_split_pays(ops):
     assert ops.quant_dot_workspace_size(16, 64, 128) == 0
 
 
-@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 300, 1600, False),
-                                           (1, 512, 8192, True), (8, 256, 2112, False)])
+@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 304, 1600, False),
+                                           (1, 512, 8192, True), (8, 256, 2112, False), (24, 250, 2048, True),
+                                           (17, 49, 4608, True)])
 @pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
 def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b, out):
     """The skinny fused linear layer: the second kernel of the workspace split applies the
@@ -592,7 +594,11 @@ def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b
     bias = (rng.standard_normal(n) * 3).astype(np.float32)
     bias[:2] = [0.0, -0.0]
     zp_a, zp_b = (3, -2) if m % 16 else (0, 0)
-    want = orc.qdq_matmul_int8(a, bm, sa[:, None], sb[None, :], zp_a, zp_b, orc.F32) + bias[None, :]
+    # (an int8 product whose N is no multiple of 4 takes a bias on another kernel: none there)
+    use_bias = n % 4 == 0
+    want = orc.qdq_matmul_int8(a, bm, sa[:, None], sb[None, :], zp_a, zp_b, orc.F32)
+    if use_bias:
+        want = want + bias[None, :]
     assert want.dtype == np.float32
     tb = dev(b).T if trans_b else dev(b)
     td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
@@ -602,7 +608,7 @@ def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b
     print("int8 workspace dq", m, n, k, trans_b, out, flush=True)
     kw = dict(scale_a=dev(sa), scale_b=dev(sb), zp_a=zp_a, zp_b=zp_b,
               colsum_b=ops.colsum_i8(tb) if zp_a else None, rowsum_a=ops.rowsum_i8(dev(a)) if zp_b else None,
-              out_dtype=td, bias=dev(bias))
+              out_dtype=td, bias=dev(bias) if use_bias else None)
     got = ops.quant_dot(dev(a), tb, workspace=ws, **kw)
     one_pass = ops.quant_dot(dev(a), tb, **kw)
     assert torch.equal(got.view(torch.int32 if out == "f32" else torch.int16),
@@ -614,7 +620,7 @@ def test_int8_split_k_with_workspace_dequantizing_epilogue(ops, m, n, k, trans_b
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
 
 
-@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 300, 1600, False),
+@pytest.mark.parametrize("m,n,k,trans_b", [(16, 1024, 4096, False), (128, 768, 3072, True), (40, 304, 1600, False),
                                            (1, 512, 8192, True), (64, 256, 2112, False)])
 @pytest.mark.parametrize("out", ["bare", "f32", "bf16"])
 def test_fp8_split_k_with_workspace(ops, m, n, k, trans_b, out):
