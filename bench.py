@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one int8 quant_dot (A[8192,8192] . B[8192,8192] -> int32, row-major,
-uniform int8 operands: BASELINE config 2 at its largest size) launched through
+uniform int8 operands: benchmark config 2 at its largest size) launched through
 the C ABI with both operands resident in HBM.  One JSON line is printed with
 the whole-job throughput in TOPS (2*M*N*K operations per step), the MFMA
 roofline fraction of the kernel (HIP events around the launches, on the stream
@@ -323,7 +323,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(wall_s * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "int8 quant_dot A[8192,8192] x B[8192,8192] -> int32, row-major, "
-                               "uniform int8 (BASELINE config 2, M=N=K=8192)",
+                               "uniform int8 (benchmark config 2, M=N=K=8192)",
                    "m": M, "n": N, "k": K},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_TOPS_INT8,
                      "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),

@@ -1,4 +1,4 @@
-// A BERT-shaped encoder built in memory (BASELINE config 5): token + position embedding,
+// A BERT-shaped encoder built in memory (benchmark config 5): token + position embedding,
 // LayerNorm, then per layer multi-head self-attention and a GELU feed-forward block with residual
 // connections and LayerNorm.  Weights ~N(0, 0.02).  In the quantized form the six projections of a
 // layer (Q, K, V, O and the two feed-forward matrices) are QDQ MatMuls: int8 weights with one scale

@@ -1070,7 +1070,7 @@ TEST_CASE(fp8_calibration)
 
 TEST_CASE(encoder_graph_on_cpu)
 {
-    // the BERT-shaped graph of BASELINE config 5, small: calibration, QDQ rewrite and evaluation on
+    // the BERT-shaped graph of benchmark config 5, small: calibration, QDQ rewrite and evaluation on
     // the CPU oracle target; the int8 model must stay close to the float one
     encoder::config c;
     c.layers = 1;

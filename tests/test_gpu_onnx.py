@@ -68,7 +68,7 @@ def test_written_qdq_conv_model_on_device(tmp_path):
 
 
 def test_written_qdq_matmul_model_on_device(tmp_path):
-    """BASELINE config 1 from ONNX bytes through the Python surface: one fused quant_dot launch
+    """benchmark config 1 from ONNX bytes through the Python surface: one fused quant_dot launch
     (dequantize and bias in its epilogue), bit-identical to the oracle."""
     from oracle import oracle as orc
     from amdmigraphx_amd import migraphx as mgx

@@ -15,7 +15,7 @@ def mgx():
 
 
 def qdq_matmul(mgx, m, k, n, w, sw):
-    """X float -> Q/DQ (scale 1/32) ; W int8 -> DQ per output channel ; dot (BASELINE config 1)."""
+    """X float -> Q/DQ (scale 1/32) ; W int8 -> DQ per output channel ; dot (benchmark config 1)."""
     p = mgx.program()
     mm = p.get_main_module()
     x = mm.add_parameter("x", mgx.shape(type="float", lens=[m, k]))

@@ -108,7 +108,7 @@ def test_int8_extremes_and_batch(ops):
 
 
 def test_config1_qdq_matmul_bit_exact(ops):
-    """BASELINE config 1: X fp32 [256,1024] ~N(0,1) -> quantizelinear(1/32, 0) ->
+    """benchmark config 1: X fp32 [256,1024] ~N(0,1) -> quantizelinear(1/32, 0) ->
     quant_dot with W int8 U[-127,127] -> per-channel dequantizelinear, seed 0."""
     rng = np.random.default_rng(0)
     x = rng.standard_normal((256, 1024)).astype(np.float32)
@@ -220,7 +220,7 @@ def test_fp8_small_integers_are_exact(ops):
 
 @pytest.mark.parametrize("out", ["f32", "bf16"])
 def test_fp8_dequant_epilogue(ops, out):
-    """BASELINE config 3 at reduced size: amax-scaled fp8 operands, per-tensor
+    """benchmark config 3 at reduced size: amax-scaled fp8 operands, per-tensor
     scales, fp32 accumulate, truncating bf16 output."""
     rng = np.random.default_rng(3)
     m, n, k = 256, 384, 2048
@@ -457,7 +457,7 @@ def test_argument_errors(ops):
 
 
 def test_full_size_int8_properties(ops):
-    """BASELINE config 2 at 8192^3: sampled rows against the oracle and a
+    """benchmark config 2 at 8192^3: sampled rows against the oracle and a
     row-checksum identity over the whole result."""
     torch.manual_seed(0)
     n = 8192
@@ -507,7 +507,7 @@ def test_graph_replay_of_split_k_and_int4_kernels(ops):
 
 @pytest.mark.parametrize("k,n", [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)])
 def test_full_size_fp8_config3_shapes(ops, k, n):
-    """BASELINE config 3 at its real sizes (M = 4096).  fp8 codes that hold small integers
+    """benchmark config 3 at its real sizes (M = 4096).  fp8 codes that hold small integers
     make every partial sum an integer below 2^24, which the fp32 accumulator and the MFMA's
     internal alignment hold exactly: the fp8 quant_dot must then equal the int8 quant_dot of
     the same integers, element for element, over the whole result.  The bf16 epilogue is

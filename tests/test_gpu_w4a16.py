@@ -215,7 +215,7 @@ def test_w4a16_matrix_core_kernel_strided_activations_and_output(ops):
 
 @pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 14336), (14336, 4096)])
 def test_w4a16_full_size_config4_shapes(ops, k, n):
-    """BASELINE config 4 at its real sizes, M in {1, 16, 128}: one-hot activation rows pick
+    """benchmark config 4 at its real sizes, M in {1, 16, 128}: one-hot activation rows pick
     single dequantized weights out of the full matrix (exact, for every kernel), and the
     batched kernels agree with the M = 1 kernel row by row within the summation tolerance."""
     g = 128

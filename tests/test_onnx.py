@@ -187,7 +187,7 @@ def test_malformed_conv_models_are_rejected(model, message):
 
 
 def qdq_matmul_model(rng, m=64, k=256, n=128, with_bias=True):
-    """BASELINE config 1 as a QDQ-format ONNX model: x float -> Q/DQ (scale 1/32) ; int8 weights with
+    """benchmark config 1 as a QDQ-format ONNX model: x float -> Q/DQ (scale 1/32) ; int8 weights with
     one scale per output column -> DQ (axis 1) ; MatMul ; Add of a bias."""
     import onnx_writer as ow
     w = rng.integers(-127, 128, (k, n), dtype=np.int8)
