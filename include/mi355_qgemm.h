@@ -161,16 +161,17 @@ int mi355_quant_convolution(const mi355_quant_conv_desc* desc, const void* x, co
                             const float* scale_x, const float* scale_w, void* workspace,
                             size_t workspace_bytes, void* stream);
 
-/* The same with a workspace.  A quant_dot with few output tiles and a long K (a skinny A against a
- * large B) is split along K over the workgroups of the chip.  Without a workspace only the bare
- * int8 product is split (the shares are added into C with integer atomics); with one, the shares
- * write partial tiles and a second kernel adds them up and applies the dequantizing epilogue (no
- * atomics, no clearing of C).  int8: the same bits as the unsplit kernel.  fp8 (one batch only):
- * float partial sums added in a fixed order, the same bits on every call, within the fp8
- * tolerance of the unsplit kernel's.  mi355_quant_dot_workspace_size gives the bytes that
- * description can use (0: none); a NULL or smaller workspace is not an error, the call then
- * behaves like mi355_quant_dot_bias.  The workspace must be 16-byte aligned device memory and is
- * free again when the call's work is done. */
+/* The same with a workspace.  A quant_dot that launches fewer workgroups than the chip has CUs
+ * (a skinny or mid-size A against a large B, one image of a convolution) is split along K.
+ * Without a workspace only the bare int8 product is split (the shares are added into C with
+ * integer atomics); with one, the shares write partial tiles and a second kernel adds them up and
+ * applies the dequantizing epilogue (no atomics, no clearing of C).  int8: the same bits as the
+ * unsplit kernel, any N when B is [N, K].  fp8 (one batch, N % 4 == 0): float partial sums added
+ * in a fixed order, the same bits on every call, within the fp8 tolerance of the unsplit
+ * kernel's.  mi355_quant_dot_workspace_size gives the bytes that description can use (0: none);
+ * a NULL or smaller workspace is not an error, the call then behaves like mi355_quant_dot_bias.
+ * The workspace must be 16-byte aligned device memory and is free again when the call's work is
+ * done. */
 size_t mi355_quant_dot_workspace_size(const mi355_quant_dot_desc* desc);
 int mi355_quant_dot_ws(const mi355_quant_dot_desc* desc, const void* a, const void* b, void* c,
                        const float* scale_a, const float* scale_b, const int32_t* colsum_b,
@@ -286,13 +287,13 @@ int mi355_w4a16_gemm(const void* a, int64_t lda,
                      int64_t m, int64_t n, int64_t k, int64_t group,
                      void* stream);
 
-/* The same with a workspace.  Between 33 and a few hundred rows against a weight matrix of few
- * columns (N / 128 tiles do not fill the chip) the tile kernel splits K over more workgroups when
- * it has room for their float partial sums; a second kernel adds them in a fixed order and
- * converts to half.  Deterministic, within the path's fp tolerance of the unsplit result (another
- * order of fp32 additions).  mi355_w4a16_gemm_workspace_size gives the bytes the shape can use
- * (0: none); a NULL or smaller workspace is not an error.  16-byte aligned device memory, free
- * again when the call's work is done. */
+/* The same with a workspace.  Where the column tiles alone do not fill the chip (more than 32
+ * rows against N / 128 tiles; 2..64 rows against few 64-column tiles and K >= 8192) the kernels
+ * split K over more workgroups when they have room for the float partial sums; a second kernel
+ * adds them in a fixed order and converts to half.  Deterministic, within the path's fp tolerance
+ * of the unsplit result (another order of fp32 additions).  mi355_w4a16_gemm_workspace_size gives
+ * the bytes the shape can use (0: none); a NULL or smaller workspace is not an error.  16-byte
+ * aligned device memory, free again when the call's work is done. */
 size_t mi355_w4a16_gemm_workspace_size(int64_t m, int64_t n, int64_t k, int64_t group);
 int mi355_w4a16_gemm_ws(const void* a, int64_t lda,
                         const void* w_packed,
