@@ -68,6 +68,12 @@ EXPORTS = {
                           ctypes.c_int64, ctypes.c_void_p],
     "mi355_pack_int4": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64,
                         ctypes.c_int64, ctypes.c_void_p],
+    "mi355_unpack_int4_nd": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
+                             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_int32,
+                             ctypes.c_void_p],
+    "mi355_pack_int4_nd": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
+                           ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_int32,
+                           ctypes.c_void_p],
     "mi355_unpack_fp4": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
     "mi355_pack_fp4": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
     "mi355_convert": [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32,

@@ -429,6 +429,135 @@ extern "C" int mi355_pack_int4(
     return mi355_launch_status();
 }
 
+// ---- int4 pack / unpack along any axis of a strided view ------------------------------------
+// One thread per packed byte.  `lens` are the lengths of the packed tensor (unpack: the input,
+// pack: the output); the byte with multi-index idx pairs with the elements idx[axis] * 2 and
+// idx[axis] * 2 + 1 of the unpacked tensor.  The strided side (the input) is addressed through
+// element strides, zero for a broadcast dimension; the output is dense row-major.
+struct int4_nd_params
+{
+    const uint8_t* in;
+    uint8_t* out;
+    int64_t lens[MI355_MAX_DIMS];
+    int64_t in_strides[MI355_MAX_DIMS];
+    int64_t out_strides[MI355_MAX_DIMS];
+    int64_t total;
+    int ndim, axis, is_signed;
+};
+
+template <bool PACK>
+__global__ __launch_bounds__(PW_THREADS) void int4_nd_kernel(int4_nd_params p)
+{
+    for(int64_t i = (int64_t)blockIdx.x * PW_THREADS + threadIdx.x; i < p.total;
+        i += (int64_t)gridDim.x * PW_THREADS)
+    {
+        int64_t rest = i, in_off = 0, out_off = 0;
+        for(int d = p.ndim - 1; d >= 0; d--)
+        {
+            const int64_t idx = rest % p.lens[d];
+            rest /= p.lens[d];
+            // along the axis the unpacked side holds two elements per packed byte
+            in_off += idx * p.in_strides[d] * ((PACK && d == p.axis) ? 2 : 1);
+            out_off += idx * p.out_strides[d] * ((!PACK && d == p.axis) ? 2 : 1);
+        }
+        if constexpr(PACK)
+        {
+            const uint8_t r1 = p.in[in_off], r2 = p.in[in_off + p.in_strides[p.axis]];
+            uint8_t u1, u2;
+            if(p.is_signed)
+            {
+                u1 = (uint8_t)max(-8, min(7, (int)(int8_t)r1));
+                u2 = (uint8_t)max(-8, min(7, (int)(int8_t)r2));
+            }
+            else
+            {
+                u1 = (uint8_t)min((int)r1, 15);
+                u2 = (uint8_t)min((int)r2, 15);
+            }
+            p.out[out_off] = (uint8_t)((u2 << 4) | (u1 & 0xf));
+        }
+        else
+        {
+            const uint8_t v = p.in[in_off];
+            uint8_t lo, hi;
+            if(p.is_signed)
+            {
+                lo = (uint8_t)((int8_t)(uint8_t)(v << 4) >> 4);
+                hi = (uint8_t)((int8_t)v >> 4);
+            }
+            else
+            {
+                lo = v & 0xf;
+                hi = v >> 4;
+            }
+            p.out[out_off]                         = lo;
+            p.out[out_off + p.out_strides[p.axis]] = hi;
+        }
+    }
+}
+
+template <bool PACK>
+static int launch_int4_nd(const void* in, void* out, int32_t is_signed, int32_t ndim, const int64_t* lens,
+                          const int64_t* in_strides, int32_t axis, void* stream)
+{
+    if(ndim < 1 || ndim > MI355_MAX_DIMS || lens == nullptr || in_strides == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if(axis < 0)
+        axis += ndim;
+    if(axis < 0 || axis >= ndim)
+        return MI355_ERR_BAD_ARG;
+    int4_nd_params p{};
+    p.total = 1;
+    for(int d = 0; d < ndim; d++)
+    {
+        if(lens[d] < 0 || in_strides[d] < 0)
+            return MI355_ERR_BAD_ARG;
+        p.lens[d]       = lens[d]; // lengths of the INPUT
+        p.in_strides[d] = in_strides[d];
+    }
+    if(PACK)
+    {
+        if(lens[axis] % 2 != 0)
+            return MI355_ERR_BAD_ARG; // PACK_INT4: can not pack an axis of odd length
+        p.lens[axis] = lens[axis] / 2; // the kernel walks the packed tensor
+    }
+    // dense strides of the output
+    int64_t run = 1;
+    for(int d = ndim - 1; d >= 0; d--)
+    {
+        p.out_strides[d] = run;
+        run *= (!PACK && d == axis) ? p.lens[d] * 2 : p.lens[d];
+        p.total *= p.lens[d];
+    }
+    if(p.total == 0)
+        return MI355_OK;
+    if(in == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    p.in        = static_cast<const uint8_t*>(in);
+    p.out       = static_cast<uint8_t*>(out);
+    p.ndim      = ndim;
+    p.axis      = axis;
+    p.is_signed = is_signed;
+    int64_t blocks = (p.total + PW_THREADS - 1) / PW_THREADS;
+    if(blocks > 256 * 16)
+        blocks = 256 * 16;
+    hipLaunchKernelGGL(int4_nd_kernel<PACK>, dim3((unsigned)blocks), dim3(PW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_unpack_int4_nd(const void* in, void* out, int32_t is_signed, int32_t ndim,
+                                    const int64_t* lens, const int64_t* in_strides, int32_t axis, void* stream)
+{
+    return launch_int4_nd<false>(in, out, is_signed, ndim, lens, in_strides, axis, stream);
+}
+
+extern "C" int mi355_pack_int4_nd(const void* in, void* out, int32_t is_signed, int32_t ndim,
+                                  const int64_t* lens, const int64_t* in_strides, int32_t axis, void* stream)
+{
+    return launch_int4_nd<true>(in, out, is_signed, ndim, lens, in_strides, axis, stream);
+}
+
 extern "C" int mi355_unpack_fp4(const void* in, void* out, int64_t rows, int64_t cols, void* stream)
 {
     if(in == nullptr || out == nullptr || rows < 0 || cols < 0)

@@ -40,6 +40,15 @@ constexpr int NTHREADS    = 512;
 constexpr int A_BYTES     = BM * BK;
 constexpr int STAGE_BYTES = (BM + BN) * BK;
 constexpr int LDS_BYTES   = STAGES * STAGE_BYTES;
+// The 16 x 16 int8 kernel keeps the K-contiguous A operand in stages of 128 K bytes (two slabs), so
+// that every direct-to-LDS load instruction fetches whole 128-byte lines (8 rows x 128 bytes): a
+// load of 16 rows x 64 bytes moves the same 16 lines from L2 for half the payload, and with all
+// 256 CUs pulling such half lines the L2s deliver 28 instead of 40 bytes per clock and CU.
+constexpr int A2_STAGES   = 2;
+constexpr int A2_BYTES    = BM * 2 * BK; // one stage of A: 256 rows x 128 bytes
+constexpr int B_BYTES     = BN * BK;     // one stage of B: one slab
+constexpr int I8_B_BASE   = A2_STAGES * A2_BYTES;
+constexpr int I8_LDS_BYTES = I8_B_BASE + STAGES * B_BYTES;
 
 struct dma_params
 {
@@ -719,18 +728,27 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     // 16-row tiles of this wave's 128-row block that hold rows of A
     const int live_tiles = SPLITK ? max(0, min(8, (p.m - (m0 + wave_m * 128) + 15) / 16)) : 8;
 
-    // ---- global -> LDS (identical to the kernel above) ------------------------
-    uint32_t a_off[2], b_off[2];
+    // ---- global -> LDS ---------------------------------------------------------
+    // A: stages of two slabs (128 K bytes).  One load instruction fetches 8 rows x 128 bytes, whole
+    // lines; a wave issues blocks {wave, wave+8, wave+16, wave+24} of a stage.  Row r keeps its 8
+    // 16-byte chunks at positions c ^ ((r >> 1) & 7), which makes the 16 rows x one chunk of an
+    // operand read fall into 16 different bank groups.  B: one slab per stage as in the kernel above.
+    uint32_t a_off[4], b_off[2];
+    const int a_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7); // (r >> 1) & 7 of this lane's rows
+#pragma unroll
+    for(int h = 0; h < 4; h++)
+    {
+        const int r   = 8 * (wave + 8 * h) + (lane >> 3);
+        const int row = min(m0 + r, p.m - 1);
+        a_off[h]      = (uint32_t)row * (uint32_t)p.lda + a_chunk * 16;
+    }
+    // an odd number of slabs leaves the last stage half filled: the lanes of its second half
+    // fetch the first half again instead of bytes past the end of the rows
+    const uint32_t a_tail_back = a_chunk >= 4 ? 64u : 0u;
 #pragma unroll
     for(int h = 0; h < 2; h++)
     {
         const int blk = wave + 8 * h;
-        {
-            const int r     = 16 * blk + (lane >> 2);
-            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
-            const int row   = min(m0 + r, p.m - 1);
-            a_off[h]        = (uint32_t)row * (uint32_t)p.lda + chunk * 16;
-        }
         if constexpr(TRANS_B)
         {
             const int r     = 16 * blk + (lane >> 2);
@@ -746,19 +764,19 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
         }
     }
-    // A wave's four loads of a slab go out one at a time, each between two runs of MFMAs: a load
-    // instruction occupies the CU's memory pipeline for about 47 cycles, so 32 of them issued
-    // together at the top of a slab would hold every wave at its issue for most of a slab's MFMA
-    // time with the matrix cores idle.
-    auto issue_a = [&](int kt, int h) {
-        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
-        const uint8_t* a_base = ga + (int64_t)kt * BK;
-        load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
+    // Loads go out one at a time, each between two runs of MFMAs: 32 of them issued together at
+    // the top of a slab would hold every wave at its issue with the matrix cores idle.
+    // ss: index of the 128-byte K step (slabs 2*ss and 2*ss + 1)
+    auto issue_a = [&](int ss, int h) {
+        uint8_t* st           = lds + (ss % A2_STAGES) * A2_BYTES;
+        const uint8_t* a_base = ga + (int64_t)ss * (2 * BK);
+        const uint32_t back   = 2 * ss + 1 < nk ? 0u : a_tail_back;
+        load_to_lds(a_base + (a_off[h] - back), st + (wave + 8 * h) * 1024);
     };
     auto issue_b = [&](int kt, int h) {
-        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
+        uint8_t* st           = lds + I8_B_BASE + (kt & (STAGES - 1)) * B_BYTES;
         const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
-        load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+        load_to_lds(b_base + b_off[h], st + (wave + 8 * h) * 1024);
     };
 
     // ---- LDS -> operand fragments ----------------------------------------------
@@ -767,11 +785,15 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     const int lgrp      = lane >> 4;
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
     const int sw        = (lrow >> 2) & 3;
-    const uint32_t a_lane = (wave_m * 128 + lrow) * BK + ((lgrp ^ sw) << 4);
+    // A: row stride 128 bytes; slab parity h reads logical chunks 4h .. 4h+3
+    uint32_t a_lane[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+        a_lane[h] = (wave_m * 128 + lrow) * (2 * BK) + (((4 * h + lgrp) ^ ((lrow >> 1) & 7)) << 4);
     uint32_t b_lane[2]; // K-contiguous B: one offset; row-major B: one per 8-row k block
     if constexpr(TRANS_B)
     {
-        b_lane[0] = A_BYTES + (wave_n * 64 + lrow) * BK + ((lgrp ^ sw) << 4);
+        b_lane[0] = I8_B_BASE + (wave_n * 64 + lrow) * BK + ((lgrp ^ sw) << 4);
         b_lane[1] = 0;
     }
     else
@@ -785,7 +807,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             const int k = lgrp * 16 + 8 * r + (lrow >> 1);
             // chunk index of tile j is wave_n*4 + j; its low bits are XORed with
             // k & 7, which for j in 0..3 only needs (j ^ x) on the low two bits
-            b_lane[r] = A_BYTES + k * BN + 8 * (lrow & 1);
+            b_lane[r] = I8_B_BASE + k * BN + 8 * (lrow & 1);
         }
     }
     const int bsw = (lrow >> 1) & 7; // k & 7 of this lane's row in the transposing read
@@ -804,22 +826,23 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 #define RDTR8(dst, addr, imm) \
     asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
 
-    // A tile 4*S + E of the slab in `stage` -> fa[S][E]
-#define READ_A1(stage, S, E) \
-    RD128(fa[S][E], lds0 + (stage) * STAGE_BYTES + a_lane, (4 * (S) + (E)) * 16 * BK)
-#define READ_A(stage, S)      \
+    // A tile 4*S + E of slab kt (slab parity H = kt & 1, a constant where this is used) -> fa[S][E]
+#define READ_A1(kt, H, S, E)                                                                 \
+    RD128(fa[S][E], lds0 + (((kt) >> 1) % A2_STAGES) * A2_BYTES + a_lane[H],             \
+          (4 * (S) + (E)) * 16 * 2 * BK)
+#define READ_A(kt, H, S)      \
     do                        \
     {                         \
-        READ_A1(stage, S, 0); \
-        READ_A1(stage, S, 1); \
-        READ_A1(stage, S, 2); \
-        READ_A1(stage, S, 3); \
+        READ_A1(kt, H, S, 0); \
+        READ_A1(kt, H, S, 1); \
+        READ_A1(kt, H, S, 2); \
+        READ_A1(kt, H, S, 3); \
     } while(0)
-    // B tile J of the slab in `stage` -> fb[P][J]
+    // B tile J of the slab in B stage `stage` -> fb[P][J]
 #define READ_B1(stage, P, J)                                                               \
     do                                                                                     \
     {                                                                                      \
-        const uint32_t s_ = lds0 + (stage) * STAGE_BYTES;                                  \
+        const uint32_t s_ = lds0 + (stage) * B_BYTES;                                      \
         if constexpr(TRANS_B)                                                              \
         {                                                                                  \
             RD128(fb[P][J], s_ + b_lane[0], (J) * 16 * BK);                                \
@@ -853,80 +876,118 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     } while(0)
     // the instruction order below is the schedule: nothing moves across these
 #define SB() __builtin_amdgcn_sched_barrier(0)
-    // One slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P].  LDS reads and
-    // direct-to-LDS loads are dealt out between the MFMAs, one at a time: issued in a bunch (12 reads
-    // by each of 8 waves right behind the barrier, as an earlier version did) they fill the LDS and
-    // memory queues and every wave sits at its issue with MFMAs waiting behind it in program order --
-    // clock stamps showed more than half of a slab's time going that way.
-    // Loads in flight, in issue order, at the wait in front of the barrier: slab kt+1, kt+2, kt+3
-    // (its B blocks were issued in this first step, its A blocks in the previous slab's second step).
+    // One slab whose B fragments sit in fb[P]; the next slab's go to fb[1 - P].  P is also the slab's
+    // parity, i.e. which half of the A stage it multiplies.  LDS reads and direct-to-LDS loads are
+    // dealt out between the MFMAs, one at a time: issued in a bunch (12 reads by each of 8 waves right
+    // behind the barrier, as an earlier version did) they fill the LDS and memory queues and every
+    // wave sits at its issue with MFMAs waiting behind it in program order.
+    //
+    // Order of a wave's loads: B blocks of slab kt+3 in the first step of slab kt; the four A blocks
+    // of K step s + A2_STAGES behind the barrier of slab 2s+1 (every wave then holds its last
+    // fragments of K step s, whose stage they overwrite).  At the wait in front of the barrier of
+    // slab kt, slab kt+1 must have landed; behind its last load the wave has issued, with three A
+    // stages,
+    //   kt even: B(kt+2), A(kt/2+2), B(kt+3)        kt odd: A((kt+3)/2), B(kt+2), B(kt+3)
+    // and with two A stages
+    //   kt even: B(kt+2), A(kt/2+1), B(kt+3)        kt odd: B(kt+2), B(kt+3)
+    // (each where it exists): that many may stay in flight.
+#define WAIT_LOADS(P)                                                                 \
+    do                                                                                \
+    {                                                                                 \
+        int cnt_ = (kt_ + 2 < nk ? 2 : 0) + (kt_ + 3 < nk ? 2 : 0);                    \
+        if((P) == 0)                                                                  \
+            cnt_ += kt_ + 2 * A2_STAGES - 2 < nk ? 4 : 0;                             \
+        else if(A2_STAGES == 3)                                                       \
+            cnt_ += kt_ + 3 < nk ? 4 : 0;                                             \
+        if(cnt_ == 8)      wait_vmcnt<8>();                                           \
+        else if(cnt_ == 6) wait_vmcnt<6>();                                           \
+        else if(cnt_ == 4) wait_vmcnt<4>();                                           \
+        else if(cnt_ == 2) wait_vmcnt<2>();                                           \
+        else               wait_vmcnt<0>();                                           \
+    } while(0)
+#define LOAD_A(h) \
+    do { if((P_) == 1 && lda_) issue_a(((kt_) >> 1) + A2_STAGES, h); } while(0)
 #define SLAB(kt, P)                                                                   \
     do                                                                                \
     {                                                                                 \
-        const int stage_  = (kt) & (STAGES - 1);                                      \
-        const int nstage_ = ((kt) + 1) & (STAGES - 1);                                \
-        const bool more_  = (kt) + 1 < nk;                                            \
-        const bool ldb_   = (kt) + STAGES - 1 < nk;                                   \
-        const bool lda_   = (kt) + STAGES < nk;                                       \
+        constexpr int P_  = (P);                                                      \
+        const int kt_     = (kt);                                                     \
+        const int stage_  = kt_ & (STAGES - 1);                                       \
+        const int nstage_ = (kt_ + 1) & (STAGES - 1);                                 \
+        const bool more_  = kt_ + 1 < nk;                                             \
+        const bool ldb_   = kt_ + STAGES - 1 < nk;                                    \
+        const bool lda_   = 2 * ((kt_ >> 1) + A2_STAGES) < nk;                        \
+        (void)stage_;                                                                 \
         WAIT4(fa[0]);                                                                 \
         WAIT4(fb[P]);                                                                 \
         SB();                                                                         \
-        READ_A1(stage_, 1, 0); SB(); MF(0, P, 0, 0); MF(0, P, 0, 1); SB();            \
-        READ_A1(stage_, 1, 1); SB(); MF(0, P, 0, 2); MF(0, P, 0, 3); SB();            \
-        READ_A1(stage_, 1, 2); SB(); MF(0, P, 1, 0); MF(0, P, 1, 1); SB();            \
-        READ_A1(stage_, 1, 3); SB(); MF(0, P, 1, 2); MF(0, P, 1, 3); SB();            \
-        if(ldb_) issue_b((kt) + STAGES - 1, 0);                                       \
+        READ_A1(kt_, P_, 1, 0); SB(); MF(0, P, 0, 0); MF(0, P, 0, 1); SB();           \
+        READ_A1(kt_, P_, 1, 1); SB(); MF(0, P, 0, 2); MF(0, P, 0, 3); SB();           \
+        READ_A1(kt_, P_, 1, 2); SB(); MF(0, P, 1, 0); MF(0, P, 1, 1); SB();           \
+        READ_A1(kt_, P_, 1, 3); SB(); MF(0, P, 1, 2); MF(0, P, 1, 3); SB();           \
+        if(ldb_) issue_b(kt_ + STAGES - 1, 0);                                        \
         SB(); MF(0, P, 2, 0); MF(0, P, 2, 1); MF(0, P, 2, 2); MF(0, P, 2, 3); SB();   \
-        if(ldb_) issue_b((kt) + STAGES - 1, 1);                                       \
+        if(ldb_) issue_b(kt_ + STAGES - 1, 1);                                        \
         SB(); MF(0, P, 3, 0); MF(0, P, 3, 1); MF(0, P, 3, 2); MF(0, P, 3, 3); SB();   \
-        if((kt) + 3 < nk)                                                             \
-            wait_vmcnt<8>();                                                          \
-        else if((kt) + 2 < nk)                                                        \
-            wait_vmcnt<4>();                                                          \
-        else                                                                          \
-            wait_vmcnt<0>();                                                          \
+        WAIT_LOADS(P);                                                                \
         WAIT4(fa[1]);                                                                 \
         block_barrier();                                                              \
         SB();                                                                         \
-        if(more_) READ_A1(nstage_, 0, 0); SB(); MF(1, P, 0, 0); SB();                 \
-        if(more_) READ_A1(nstage_, 0, 1); SB(); MF(1, P, 0, 1); SB();                 \
-        if(more_) READ_A1(nstage_, 0, 2); SB(); MF(1, P, 0, 2); SB();                 \
-        if(more_) READ_A1(nstage_, 0, 3); SB(); MF(1, P, 0, 3); SB();                 \
+        if(more_) READ_A1(kt_ + 1, 1 - P_, 0, 0); SB(); MF(1, P, 0, 0); SB();         \
+        if(more_) READ_A1(kt_ + 1, 1 - P_, 0, 1); SB(); MF(1, P, 0, 1); SB();         \
+        if(more_) READ_A1(kt_ + 1, 1 - P_, 0, 2); SB(); MF(1, P, 0, 2); SB();         \
+        if(more_) READ_A1(kt_ + 1, 1 - P_, 0, 3); SB(); MF(1, P, 0, 3); SB();         \
         if(more_) READ_B1(nstage_, 1 - (P), 0); SB(); MF(1, P, 1, 0); MF(1, P, 1, 1); SB(); \
+        LOAD_A(0); SB();                                                              \
         if(more_) READ_B1(nstage_, 1 - (P), 1); SB(); MF(1, P, 1, 2); MF(1, P, 1, 3); SB(); \
+        LOAD_A(1); SB();                                                              \
         if(more_) READ_B1(nstage_, 1 - (P), 2); SB(); MF(1, P, 2, 0); MF(1, P, 2, 1); SB(); \
+        LOAD_A(2); SB();                                                              \
         if(more_) READ_B1(nstage_, 1 - (P), 3); SB(); MF(1, P, 2, 2); MF(1, P, 2, 3); SB(); \
-        if(lda_) issue_a((kt) + STAGES, 0);                                           \
-        SB(); MF(1, P, 3, 0); MF(1, P, 3, 1); SB();                                   \
-        if(lda_) issue_a((kt) + STAGES, 1);                                           \
-        SB(); MF(1, P, 3, 2); MF(1, P, 3, 3); SB();                                   \
+        LOAD_A(3);                                                                    \
+        SB(); MF(1, P, 3, 0); MF(1, P, 3, 1); MF(1, P, 3, 2); MF(1, P, 3, 3); SB();   \
     } while(0)
 
-    // ---- main loop (see the kernel above for the ordering argument) ----------
-    // The stage of slab kt + 4 is the one slab kt sits in: its A blocks may be requested once every
-    // wave holds its last fragments of slab kt, i.e. after slab kt's barrier.
-#pragma unroll
-    for(int s = 0; s < STAGES - 1; s++)
-        if(s < nk)
-        {
-            issue_a(s, 0);
-            issue_a(s, 1);
-            issue_b(s, 0);
-            issue_b(s, 1);
-        }
-    if(nk >= 3)
-        wait_vmcnt<8>();
-    else if(nk == 2)
-        wait_vmcnt<4>();
-    else
-        wait_vmcnt<0>();
-    block_barrier();
-    if(STAGES - 1 < nk)
+    // ---- main loop -----------------------------------------------------------------
+    // Prologue in the order the waits above assume: A(0), B(0), [A(1)], B(1), B(2), A(last stage).
     {
-        issue_a(STAGES - 1, 0);
-        issue_a(STAGES - 1, 1);
+#pragma unroll
+        for(int h = 0; h < 4; h++)
+            issue_a(0, h);
+        issue_b(0, 0);
+        issue_b(0, 1);
+        if(A2_STAGES == 3 && 2 < nk)
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_a(1, h);
+        }
+#pragma unroll
+        for(int s = 1; s < STAGES - 1; s++)
+            if(s < nk)
+            {
+                issue_b(s, 0);
+                issue_b(s, 1);
+            }
+        if(2 * (A2_STAGES - 1) < nk)
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_a(A2_STAGES - 1, h);
+        }
     }
-    READ_A(0, 0);
+    // slab 0 has landed when only what was issued behind B(0) is outstanding
+    {
+        const int cnt = (1 < nk ? 2 : 0) + (2 < nk ? 2 : 0) + (A2_STAGES == 3 && 2 < nk ? 4 : 0) +
+                        (2 * (A2_STAGES - 1) < nk ? 4 : 0);
+        if(cnt == 12)      wait_vmcnt<12>();
+        else if(cnt == 8)  wait_vmcnt<8>();
+        else if(cnt == 6)  wait_vmcnt<6>();
+        else if(cnt == 2)  wait_vmcnt<2>();
+        else               wait_vmcnt<0>();
+    }
+    block_barrier();
+    READ_A(0, 0, 0);
     READ_B(0, 0);
     int kt = 0;
     for(; kt + 1 < nk; kt += 2)
@@ -936,6 +997,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     }
     if(kt < nk)
         SLAB(kt, 0);
+#undef LOAD_A
+#undef WAIT_LOADS
 #undef SLAB
 #undef SB
 #undef MF
@@ -1073,11 +1136,11 @@ int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
 {
     auto kern = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
     if(attr != hipSuccess)
         return MI355_ERR_LAUNCH;
     dim3 grid(p.tiles_m * p.tiles_n, batch);
-    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
     return mi355_launch_status();
 }
 
@@ -1219,13 +1282,13 @@ int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream, bool de
 {
     auto kern = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true>;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
     if(attr != hipSuccess)
         return MI355_ERR_LAUNCH;
     if(p.partial != nullptr)
     {
         dim3 grid(p.tiles_m * p.tiles_n, batch, p.ksplit);
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
         // shares that hold slabs: the kernel gives ceil(nk / ksplit) slabs to each, the last ones
         // may be left with none (they write nothing)
         const int nk     = p.k / BK;
@@ -1238,7 +1301,7 @@ int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream, bool de
     hipLaunchKernelGGL(zero_i32_kernel, dim3(zb, batch), dim3(256), 0, stream,
                        static_cast<int32_t*>(p.c), p.m, p.n, p.ldc, p.stride_c);
     dim3 grid(p.tiles_m * p.tiles_n, batch, p.ksplit);
-    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
     return mi355_launch_status();
 }
 

@@ -221,6 +221,12 @@ struct dequantizelinear
 // inputs: x, out.  The packed axis is the last one.
 struct unpack_int4
 {
+    int64_t axis = -1; // the packed axis; any strided (also broadcast) input view is taken as it is
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
     std::string name() const { return "mi355::unpack_int4"; }
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
@@ -228,6 +234,12 @@ struct unpack_int4
 };
 struct pack_int4
 {
+    int64_t axis = -1; // the packed axis; any strided (also broadcast) input view is taken as it is
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axis, "axis");
+    }
     std::string name() const { return "mi355::pack_int4"; }
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;

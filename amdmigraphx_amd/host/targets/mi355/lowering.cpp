@@ -466,6 +466,12 @@ bool match_blockwise(instruction_ref x, std::size_t n, instruction_ref& base, st
     return true;
 }
 
+bool unpacks_last_axis(instruction_ref unpk)
+{
+    const auto axis = any_cast<op::unpack_int4>(unpk->get_operator()).axis;
+    return axis == -1 or axis == static_cast<int64_t>(unpk->get_shape().ndim()) - 1;
+}
+
 bool lower_w4a16(module& m, instruction_ref ins)
 {
     auto a  = ins->inputs()[0];
@@ -486,6 +492,10 @@ bool lower_w4a16(module& m, instruction_ref ins)
         return false;
     auto packed = unpk->inputs().front();
     if(not packed->get_shape().standard() or packed->get_shape().ndim() != 2)
+        return false;
+    // the kernel reads nibble pairs along K: the unpack must run along the last axis of [N, K/2]
+    // (a weight packed along axis 0 has the same byte count and would be read the wrong way)
+    if(not unpacks_last_axis(unpk) or packed->get_shape().lens() != std::vector<std::size_t>{n, k / 2} or k % 2 != 0)
         return false;
 
     instruction_ref scales;
@@ -511,6 +521,8 @@ bool lower_w4a16(module& m, instruction_ref ins)
         std::size_t zblk = 0;
         if(scalar_constant(z, v))
         {
+            if(v < 0 or v > 15)
+                return false; // not a 4-bit zero point: the generic operators take the graph
             op.zp_mode   = MI355_W4_ZP_SCALAR;
             op.zp_scalar = v;
         }
@@ -518,7 +530,9 @@ bool lower_w4a16(module& m, instruction_ref ins)
         {
             bool zsliced = false;
             auto zu      = skip_full_slice(zbase, zsliced);
-            if(zu->name() == "unpack_int4" and zu->inputs().front()->get_shape().standard())
+            if(zu->name() == "unpack_int4" and zu->inputs().front()->get_shape().standard() and
+               unpacks_last_axis(zu) and zu->inputs().front()->get_shape().ndim() == 2 and
+               zu->inputs().front()->get_shape().lens()[0] == n)
             {
                 op.zp_mode = MI355_W4_ZP_PACKED;
                 args.push_back(zu->inputs().front());
@@ -534,7 +548,9 @@ bool lower_w4a16(module& m, instruction_ref ins)
         else
             return false;
     }
-    if(a->get_shape().strides()[1] != 1 and a->get_shape().lens()[1] != 1)
+    // the kernels load 16 bytes of a row at a time: rows must start 16-byte aligned
+    if((a->get_shape().strides()[1] != 1 and a->get_shape().lens()[1] != 1) or
+       a->get_shape().strides()[0] % 8 != 0 or a->name() == "slice")
         args[0] = make_standard(m, ins, a);
     // room for split-K partial sums where the column tiles alone do not fill the chip
     const auto rows   = a->get_shape().lens()[0];
@@ -888,16 +904,23 @@ void lower_instruction(module& m, instruction_ref ins)
     }
     else if(name == "unpack_int4" or name == "pack_int4")
     {
-        const auto nd   = static_cast<int64_t>(ins->inputs()[0]->get_shape().ndim());
-        const auto axis = name == "unpack_int4" ? any_cast<op::unpack_int4>(ins->get_operator()).axis
-                                                : any_cast<op::pack_int4>(ins->get_operator()).axis;
-        if(axis != -1 and axis != nd - 1)
-            MIGRAPHX_THROW("mi355: " + name + " along an axis other than the last has no kernel");
-        auto x = make_standard(m, ins, ins->inputs()[0]);
+        // any axis, any view (transposed, broadcast): the kernel walks the input's strides
+        const auto nd = ins->inputs()[0]->get_shape().ndim();
+        auto x        = ins->inputs()[0];
+        if(nd > MI355_MAX_DIMS)
+            MIGRAPHX_THROW("mi355: " + name + " of more than 8 dimensions has no kernel");
         if(name == "unpack_int4")
-            m.replace_instruction(ins, operation{unpack_int4{}}, x, standard_out());
+        {
+            unpack_int4 op;
+            op.axis = any_cast<op::unpack_int4>(ins->get_operator()).axis;
+            m.replace_instruction(ins, operation{op}, x, standard_out());
+        }
         else
-            m.replace_instruction(ins, operation{pack_int4{}}, x, standard_out());
+        {
+            pack_int4 op;
+            op.axis = any_cast<op::pack_int4>(ins->get_operator()).axis;
+            m.replace_instruction(ins, operation{op}, x, standard_out());
+        }
     }
     else if(name == "unpack_fp4" or name == "pack_fp4")
     {

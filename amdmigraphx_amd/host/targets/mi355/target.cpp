@@ -707,24 +707,42 @@ dequantizelinear::compute(migraphx::context& ctx, const shape& out, const std::v
 shape unpack_int4::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
-    check_standard(inputs[0], name());
-    auto out = op::unpack_int4{}.compute_shape({inputs[0]});
+    op::unpack_int4 ref;
+    ref.axis = axis;
+    auto out = ref.compute_shape({inputs[0]});
     if(inputs[1] != out)
         MIGRAPHX_THROW("mi355::unpack_int4: output buffer has the wrong shape");
     return out;
 }
 
+// lengths and element strides of a view as the C ABI takes them
+static void lens_strides(const shape& s, std::vector<int64_t>& lens, std::vector<int64_t>& strides)
+{
+    lens.assign(s.lens().begin(), s.lens().end());
+    strides.assign(s.strides().begin(), s.strides().end());
+}
+
 argument unpack_int4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
 {
-    int64_t rows = 0;
-    int64_t cols = 0;
-    rows_cols(args[0].get_shape(), rows, cols);
-    status_check(mi355_unpack_int4(args[0].data(),
-                                   args[1].data(),
-                                   args[0].get_shape().type() == shape::int8_type,
-                                   rows,
-                                   cols,
-                                   stream_of(ctx)),
+    const auto& in = args[0].get_shape();
+    const auto nd  = static_cast<int64_t>(in.ndim());
+    if(in.standard() and (axis == -1 or axis == nd - 1))
+    {
+        int64_t rows = 0;
+        int64_t cols = 0;
+        rows_cols(in, rows, cols);
+        status_check(mi355_unpack_int4(args[0].data(), args[1].data(), in.type() == shape::int8_type, rows, cols,
+                                       stream_of(ctx)),
+                     name());
+        return args[1];
+    }
+    if(nd > MI355_MAX_DIMS)
+        MIGRAPHX_THROW("mi355::unpack_int4: more than 8 dimensions");
+    std::vector<int64_t> lens, strides;
+    lens_strides(in, lens, strides);
+    status_check(mi355_unpack_int4_nd(args[0].data(), args[1].data(), in.type() == shape::int8_type,
+                                      static_cast<int32_t>(nd), lens.data(), strides.data(),
+                                      static_cast<int32_t>(axis), stream_of(ctx)),
                  name());
     return args[1];
 }
@@ -774,8 +792,9 @@ argument pack_fp4::compute(migraphx::context& ctx, const shape&, const std::vect
 shape pack_int4::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
-    check_standard(inputs[0], name());
-    auto out = op::pack_int4{}.compute_shape({inputs[0]});
+    op::pack_int4 ref;
+    ref.axis = axis;
+    auto out = ref.compute_shape({inputs[0]});
     if(inputs[1] != out)
         MIGRAPHX_THROW("mi355::pack_int4: output buffer has the wrong shape");
     return out;
@@ -783,15 +802,25 @@ shape pack_int4::compute_shape(const std::vector<shape>& inputs) const
 
 argument pack_int4::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
 {
-    int64_t rows = 0;
-    int64_t cols = 0;
-    rows_cols(args[0].get_shape(), rows, cols);
-    status_check(mi355_pack_int4(args[0].data(),
-                                 args[1].data(),
-                                 args[0].get_shape().type() == shape::int8_type,
-                                 rows,
-                                 cols,
-                                 stream_of(ctx)),
+    const auto& in = args[0].get_shape();
+    const auto nd  = static_cast<int64_t>(in.ndim());
+    if(in.standard() and (axis == -1 or axis == nd - 1))
+    {
+        int64_t rows = 0;
+        int64_t cols = 0;
+        rows_cols(in, rows, cols);
+        status_check(mi355_pack_int4(args[0].data(), args[1].data(), in.type() == shape::int8_type, rows, cols,
+                                     stream_of(ctx)),
+                     name());
+        return args[1];
+    }
+    if(nd > MI355_MAX_DIMS)
+        MIGRAPHX_THROW("mi355::pack_int4: more than 8 dimensions");
+    std::vector<int64_t> lens, strides;
+    lens_strides(in, lens, strides);
+    status_check(mi355_pack_int4_nd(args[0].data(), args[1].data(), in.type() == shape::int8_type,
+                                    static_cast<int32_t>(nd), lens.data(), strides.data(),
+                                    static_cast<int32_t>(axis), stream_of(ctx)),
                  name());
     return args[1];
 }

@@ -275,26 +275,49 @@ def pack_fp4(x):
     return out
 
 
-def unpack_int4(x):
-    x = x.contiguous()
-    cols = x.shape[-1]
-    rows = x.numel() // max(cols, 1)
-    out = torch.empty(x.shape[:-1] + (cols * 2,), dtype=x.dtype, device=x.device)
-    check(lib().mi355_unpack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
-                                  _stream()), "mi355_unpack_int4")
+def _int4_nd(fn_name, x, axis, out_shape):
+    nd = x.dim()
+    if nd > 8:
+        raise Mi355Error("at most 8 dimensions")
+    lens = (ctypes.c_int64 * nd)(*x.shape)
+    strides = (ctypes.c_int64 * nd)(*x.stride())
+    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    check(getattr(lib(), fn_name)(_ptr(x), _ptr(out), int(x.dtype == torch.int8), nd, lens, strides,
+                                  axis, _stream()), fn_name)
     return out
 
 
-def pack_int4(x):
-    x = x.contiguous()
-    cols = x.shape[-1]
-    if cols % 2:
+def unpack_int4(x, axis=-1):
+    """unpack_int4 along ``axis`` of any strided view (transposed, expanded): the result is dense."""
+    _require_cuda(x)
+    ax = axis % x.dim()
+    shp = list(x.shape)
+    shp[ax] *= 2
+    if ax == x.dim() - 1 and x.is_contiguous():
+        cols = x.shape[-1]
+        rows = x.numel() // max(cols, 1)
+        out = torch.empty(shp, dtype=x.dtype, device=x.device)
+        check(lib().mi355_unpack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
+                                      _stream()), "mi355_unpack_int4")
+        return out
+    return _int4_nd("mi355_unpack_int4_nd", x, ax, shp)
+
+
+def pack_int4(x, axis=-1):
+    _require_cuda(x)
+    ax = axis % x.dim()
+    shp = list(x.shape)
+    if shp[ax] % 2:
         raise Mi355Error("PACK_INT4: Can not pack axis that has odd lengths")
-    rows = x.numel() // max(cols, 1)
-    out = torch.empty(x.shape[:-1] + (cols // 2,), dtype=x.dtype, device=x.device)
-    check(lib().mi355_pack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
-                                _stream()), "mi355_pack_int4")
-    return out
+    shp[ax] //= 2
+    if ax == x.dim() - 1 and x.is_contiguous():
+        cols = x.shape[-1]
+        rows = x.numel() // max(cols, 1)
+        out = torch.empty(shp, dtype=x.dtype, device=x.device)
+        check(lib().mi355_pack_int4(_ptr(x), _ptr(out), int(x.dtype == torch.int8), rows, cols,
+                                    _stream()), "mi355_pack_int4")
+        return out
+    return _int4_nd("mi355_pack_int4_nd", x, ax, shp)
 
 
 def convert(x, out_type, in_type=None):

@@ -70,6 +70,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the comparisons with the CPU oracle")
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--only-headline", action="store_true",
                     help="time the headline kernel only (for counter runs under rocprofv3)")
@@ -111,23 +112,54 @@ def main():
     tops = ops_per_step / wall_s / 1e12
     kern_tops = ops_per_step / kern_s / 1e12
 
+    # every timed result is compared with the CPU oracle on sampled rows / columns, outside the
+    # timed regions; "ok" in the output line is the conjunction
+    checks = {}
+    import numpy as np
+    from oracle import oracle as orc
+
+    def sampled_rows_equal(c_dev, a_dev, b_host, rows):
+        want = orc.quant_dot(a_dev[rows].cpu().numpy(), b_host, orc.I8)
+        return bool(np.array_equal(c_dev[rows].cpu().numpy(), want))
+
+    if not args.no_check:
+        checks["int8_quant_dot_8192"] = sampled_rows_equal(c, a, b.cpu().numpy(), [0, 255, 256, 4097, 8191])
+
     also = {}
     # ---- fp8 quant_dot with dequant epilogue, Llama-3-8B shape (config 3) ----------
     try:
         if args.only_headline:
             raise RuntimeError("skipped (--only-headline)")
         m3, k3, n3 = 4096, 4096, 14336 * 2
-        a8 = torch.randint(0, 0x7e, (m3, k3), dtype=torch.uint8, device=dev, generator=g)
-        b8 = torch.randint(0, 0x7e, (k3, n3), dtype=torch.uint8, device=dev, generator=g)
-        s1 = torch.full((1,), 0.01, dtype=torch.float32, device=dev)
-        s2 = torch.full((1,), 0.02, dtype=torch.float32, device=dev)
+        # config 3's own distribution: bf16 activations ~N(0,1), weights ~N(0,0.02), each quantized to
+        # fp8 e4m3fn with its per-tensor scale amax / 448
+        x3 = torch.randn((m3, k3), device=dev, generator=g).bfloat16().float()
+        w3 = (torch.randn((k3, n3), device=dev, generator=g) * 0.02).bfloat16().float()
+        s1 = (x3.abs().max() / 448).reshape(1)
+        s2 = (w3.abs().max() / 448).reshape(1)
+        a8 = ops.quantizelinear(x3, s1, None, out_type=ops.DT.FP8)
+        b8 = ops.quantizelinear(w3, s2, None, out_type=ops.DT.FP8)
+        del x3, w3
         o8 = torch.empty((m3, n3), dtype=torch.bfloat16, device=dev)
         t8, _ = _time_launches(lambda: ops.quant_dot(a8, b8, fp8=True, scale_a=s1, scale_b=s2,
                                                      out_dtype=torch.bfloat16, out=o8),
                                max(3, args.steps // 2), 2)
         f8 = 2.0 * m3 * k3 * n3 / t8 / 1e12
         also["fp8_quant_dot_bf16_out_M4096_K4096_N28672"] = {
-            "TFLOPS": round(f8, 1), "frac_mfma_peak": round(f8 / PEAK_TFLOPS_FP8, 4)}
+            "TFLOPS": round(f8, 1), "frac_mfma_peak": round(f8 / PEAK_TFLOPS_FP8, 4),
+            "data": "amax-quantized normal operands (config 3)"}
+        if not args.no_check:
+            rows = [0, 2047, 4095]
+            ah, bh = a8[rows].cpu().numpy(), b8.cpu().numpy()
+            want = orc.qdq_matmul_fp8(ah, bh, np.float32(s1.item()), np.float32(s2.item()), orc.BF16)
+            got = o8[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+            gf, wf = orc.bf16_to_f32(got).astype(np.float64), orc.bf16_to_f32(want).astype(np.float64)
+            mag = np.abs(orc.fp8_to_f32(ah)).astype(np.float64) @ np.abs(orc.fp8_to_f32(bh)).astype(np.float64)
+            d = np.abs(gf - wf)
+            # 1e-3 relative, or one bf16 step, or (cancelling sums) 2^-15 of sum|a||b| scaled
+            okm = (d <= 1e-3 * np.abs(wf)) | (d <= np.abs(wf) * 2.0**-7) | \
+                  (d <= mag * 2.0**-15 * s1.item() * s2.item())
+            checks["fp8_quant_dot_config3"] = bool(okm.all())
         del a8, b8, o8
     except Exception as e:  # report, never hide the headline
         also["fp8_quant_dot_error"] = str(e)
@@ -154,6 +186,15 @@ def main():
             for i in range(copies):
                 ops.w4a16_gemm(x, ws[i], sc[i], grp, zp=8, out=y)
             torch.cuda.synchronize()
+            if not args.no_check:
+                cols = list(range(0, 8)) + [n4 // 2, n4 - 1]
+                last = copies - 1
+                xh = x.view(torch.int16).cpu().numpy().view(np.uint16)
+                want = orc.half_to_f32(orc.w4a16_matmul(
+                    xh, ws[last][cols].cpu().numpy(),
+                    sc[last][cols].view(torch.int16).cpu().numpy().view(np.uint16), 8, grp))
+                got = y[:, cols].float().cpu().numpy()
+                checks[f"w4a16_gemv_K{k4}_N{n4}"] = bool(np.allclose(got, want, rtol=2e-3, atol=2e-3))
             graph = torch.cuda.CUDAGraph()
             side = torch.cuda.Stream()
             with torch.cuda.stream(side):
@@ -237,7 +278,13 @@ def main():
                 return run
 
             t2a, _ = _time_launches(skinny, 18, 6)
+            if not args.no_check:
+                checks[f"int8_quant_dot_M{m2}_atomics"] = sampled_rows_equal(
+                    c2, a2, bs[(it[0] - 1) % 6].cpu().numpy(), [0, m2 - 1])
             t2, _ = _time_launches(skinny_ws, 18, 6)
+            if not args.no_check:
+                checks[f"int8_quant_dot_M{m2}_workspace"] = sampled_rows_equal(
+                    c2, a2, bs[(it[0] - 1) % 6].cpu().numpy(), [0, m2 - 1])
             t2d, _ = _time_launches(skinny_dq, 18, 6)
             t8, _ = _time_launches(skinny_fp8(room8), 18, 6)
             t8a, _ = _time_launches(skinny_fp8(None), 18, 6)
@@ -329,6 +376,7 @@ def main():
                      "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
                      "traffic": HEADLINE_TRAFFIC_BYTES},
         "also": also,
+        "checks": checks, "ok": all(checks.values()),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(rows=args.cpu_rows)

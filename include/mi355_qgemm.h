@@ -236,6 +236,21 @@ int mi355_pack_int4(const void* in, void* out, int32_t is_signed,
                     int64_t rows, int64_t cols, void* stream);
 
 /*
+ * The same along any axis of a strided view: `lens` (HOST array, ndim <= MI355_MAX_DIMS entries)
+ * are the lengths of the INPUT, `in_strides` its element strides (zero = a broadcast dimension,
+ * as multibroadcast views carry), `axis` the packed axis (negative counts from the end).  The
+ * output is dense row-major with lens[axis] doubled (unpack) or halved (pack).
+ *
+ * Replaces the same two operators for every axis and for the non-standard input shapes they
+ * accept (op/unpack_int4.hpp:54-73 normalises the axis, :75-121 walks the multi-index with
+ * idx[axis] * 2 and idx[axis] * 2 + 1; op/pack_int4.hpp:79-124 likewise).
+ */
+int mi355_unpack_int4_nd(const void* in, void* out, int32_t is_signed, int32_t ndim,
+                         const int64_t* lens, const int64_t* in_strides, int32_t axis, void* stream);
+int mi355_pack_int4_nd(const void* in, void* out, int32_t is_signed, int32_t ndim,
+                       const int64_t* lens, const int64_t* in_strides, int32_t axis, void* stream);
+
+/*
  * unpack_fp4 / pack_fp4 along the last axis of a dense [rows, cols] tensor (cols = packed length
  * for unpack, unpacked length for pack).  fp4 is e2m1 (magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6), two
  * codes per byte, low nibble = even element.

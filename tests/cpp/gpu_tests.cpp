@@ -681,6 +681,50 @@ TEST_CASE(int4_weight_only_gemm_larger_batch)
     }
 }
 
+TEST_CASE(int4_weight_packed_along_axis_0_is_not_fused)
+{
+    // dot(a, transpose(dequantizelinear(unpack_int4{axis = 0}(w [N/2, K]), blockwise scales, 8))): the
+    // same byte count as a weight packed along K, but the nibble pairs run along N.  The fused
+    // kernel reads pairs along K, so this graph must go operator by operator, and match.
+    const std::size_t m = 4, k = 256, n = 64, blk = 128;
+    program p;
+    auto* mm = p.get_main_module();
+    auto a   = mm->add_parameter("a", shape{shape::half_type, {m, k}});
+    auto w   = mm->add_literal(literal{shape{shape::uint8_type, {n / 2, k}}, uniform_ints<int>(n / 2 * k, 0, 255, 70)});
+    auto s   = mm->add_literal(literal{shape{shape::half_type, {n, k / blk}}, uniform_floats(n * k / blk, 0.005f, 0.02f, 71)});
+    auto u   = mm->add_instruction(migraphx::make_op("unpack_int4", {{"axis", 0}}), w);
+    auto su  = mm->add_instruction(migraphx::make_op("unsqueeze", {{"axes", {2}}}), s);
+    auto sb  = mm->add_instruction(migraphx::make_op("multibroadcast", {{"out_lens", {n, k / blk, blk}}}), su);
+    auto sr  = mm->add_instruction(migraphx::make_op("reshape", {{"dims", {static_cast<int64_t>(n), -1}}}), sb);
+    auto z   = mm->add_literal(literal{shape{shape::uint8_type, {1}}, std::vector<int>{8}});
+    auto zb  = mm->add_instruction(migraphx::make_op("multibroadcast", {{"out_lens", {n, k}}}), z);
+    auto dq  = mm->add_instruction(migraphx::make_op("dequantizelinear"), u, sr, zb);
+    auto bt  = mm->add_instruction(migraphx::make_op("transpose", {{"permutation", {1, 0}}}), dq);
+    mm->add_return({mm->add_instruction(migraphx::make_op("dot"), a, bt)});
+    argument av{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 72)};
+    expect_same(p, {{"a", av}});
+    program c = p;
+    c.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 0);
+}
+
+TEST_CASE(int4_unpack_pack_any_axis_programs)
+{
+    // unpack_int4 / pack_int4 along axis 0 and of a transposed view, as operators of a program
+    for(int64_t axis : {0, 1})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::uint8_type, {6, 10}});
+        auto xt  = mm->add_instruction(migraphx::make_op("transpose", {{"permutation", {1, 0}}}), x);
+        auto u   = mm->add_instruction(migraphx::make_op("unpack_int4", {{"axis", axis}}), xt);
+        auto pk  = mm->add_instruction(migraphx::make_op("pack_int4", {{"axis", 1 - axis}}), u);
+        mm->add_return({u, pk});
+        argument xv{shape{shape::uint8_type, {6, 10}}, uniform_ints<int>(60, 0, 255, 73)};
+        expect_same(p, {{"x", xv}});
+    }
+}
+
 TEST_CASE(int4_general_path)
 {
     // float activations, or K that is not a multiple of the block: no fused kernel, the chain

@@ -139,15 +139,42 @@ def test_dequantize_int32_and_u8_half(ops):
 
 
 def test_reference_int4_known_answers_on_gpu(ops, golden):
+    """All 12 cases of test/ref/unpack_int4.cpp and pack_int4.cpp, including the transposed
+    literal, the multibroadcast view and axis 0, on the device with the views' own strides."""
+    assert len(golden["unpack_int4"]) + len(golden["pack_int4"]) == 12
     for c in golden["unpack_int4"] + golden["pack_int4"]:
-        if c["axis"] not in (-1, len(c["shape"]["lens"]) - 1) or c["multibroadcast"]:
-            continue     # the C ABI packs along the last axis of a dense tensor
         dt = np.int8 if c["shape"]["type"] == "int8" else np.uint8
         raw = np.array(c["data"], np.uint8)
-        x = (raw if dt == np.uint8 else raw.view(np.int8)).reshape(c["shape"]["lens"])
+        lens = c["shape"]["lens"]
+        x = dev((raw if dt == np.uint8 else raw.view(np.int8)).reshape(lens))
+        strides = c["shape"].get("strides")
+        if strides and len(lens) == 2 and strides[0] < strides[1]:
+            x = x.t().contiguous().t()           # same values, column-major storage
+            assert list(x.stride()) == strides
+        if c["multibroadcast"]:
+            x = x.expand(c["multibroadcast"])    # stride 0 along the new dimension
         fn = ops.unpack_int4 if "unpack" in c["name"] else ops.pack_int4
-        got = fn(dev(x)).cpu().numpy()
+        got = fn(x, c["axis"]).cpu().numpy()
         assert got.view(np.uint8).flatten().tolist() == (np.array(c["gold"]).astype(np.int64) & 0xff).tolist(), c["name"]
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, -1])
+def test_int4_any_axis_and_views_match_oracle(ops, axis):
+    rng = np.random.default_rng(50 + axis)
+    for dt, lo, hi in ((np.uint8, 0, 40), (np.int8, -30, 30)):
+        x = rng.integers(lo, hi, (6, 10, 14)).astype(dt)
+        p = ops.pack_int4(dev(x), axis)
+        assert np.array_equal(p.cpu().numpy(), orc.pack_int4(x, axis))
+        u = ops.unpack_int4(p, axis)
+        assert np.array_equal(u.cpu().numpy(), orc.unpack_int4(orc.pack_int4(x, axis), axis))
+        # a permuted view and a broadcast view, both along the same logical axis
+        xv = dev(x).permute(2, 0, 1)
+        xn = np.transpose(x, (2, 0, 1))
+        assert np.array_equal(ops.unpack_int4(xv, axis).cpu().numpy(), orc.unpack_int4(np.ascontiguousarray(xn), axis))
+        assert np.array_equal(ops.pack_int4(xv, axis).cpu().numpy(), orc.pack_int4(np.ascontiguousarray(xn), axis))
+        xb = dev(x[:, :1, :]).expand(6, 4, 14)
+        xbn = np.ascontiguousarray(np.broadcast_to(x[:, :1, :], (6, 4, 14)))
+        assert np.array_equal(ops.unpack_int4(xb, axis).cpu().numpy(), orc.unpack_int4(xbn, axis))
 
 
 def test_pack_unpack_random(ops):

@@ -256,6 +256,36 @@ def test_w4a16_full_size_config4_shapes(ops, k, n):
             assert (d <= tol).all(), (r, d.max().item())
 
 
+@pytest.mark.parametrize("m", [1, 16, 128])
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 14336), (14336, 4096)])
+def test_w4a16_full_size_config4_against_oracle(ops, m, k, n):
+    """benchmark config 4 at its real sizes: sampled output columns (weight rows) of the full
+    product against the oracle's unpack_int4 -> dequantizelinear -> dot chain, for the bare call
+    and the call with a workspace."""
+    g = 128
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(k * 5 + n + m)
+    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda", generator=gen)
+    sc = (torch.rand((n, k // g), device="cuda", generator=gen) * 0.015 + 0.005).half()
+    x = torch.randn((m, k), device="cuda", generator=gen).half()
+    print("w4a16 full size vs oracle", m, k, n, flush=True)
+    cols = sorted(set(list(range(0, 16)) + [127, 128, 129, n // 2 - 1, n // 2, n - 130, n - 17, n - 16, n - 2, n - 1]
+                      + list(range(1000, 1032))))
+    a = half_bits(x)
+    packed = w[cols].cpu().numpy()
+    scales = half_bits(sc[cols])
+    want = orc.w4a16_matmul(a, packed, scales, 8, g)
+    wq = orc.unpack_int4(packed)
+    wdq = orc.dequantizelinear(wq, np.repeat(scales, g, axis=1), np.full(wq.shape, 8, np.uint8), orc.U8, orc.F16)
+    got = ops.w4a16_gemm(x, w, sc, g, zp=8)
+    _check(half_bits(got[:, cols]), want, a, wdq)
+    nbytes = ops.w4a16_gemm_workspace_size(m, n, k, g)
+    if nbytes > 0:
+        ws = torch.full((nbytes,), 0x7F, dtype=torch.uint8, device="cuda")
+        got = ops.w4a16_gemm(x, w, sc, g, zp=8, workspace=ws)
+        _check(half_bits(got[:, cols]), want, a, wdq)
+
+
 # ---- the tile kernel with a workspace: K split over more workgroups --------------------------
 
 @pytest.mark.parametrize("m,n,k,g", [(64, 256, 1152, 64), (100, 384, 2048 + 128, 32), (130, 128, 1024, 128),
