@@ -52,6 +52,7 @@ EXPORTS = {
     "mi355_quant_dot_workspace_size": [ctypes.POINTER(QuantDotDesc)],
     "mi355_quant_dot_ws": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9 +
                           [ctypes.c_size_t, ctypes.c_void_p],
+    "mi355_quant_dot_static": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9,
     "mi355_colsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                         ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p],
     "mi355_rowsum_i8": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,

@@ -2,6 +2,8 @@
 // kernel that serves the shapes the MFMA kernel's load pattern does not fit
 // (transposed A, K not a multiple of 16, odd leading dimensions, tiny cases).
 #include "common.h"
+#include <atomic>
+#include <mutex>
 
 bool mi355_mfma_gemm_supported(const mi355_quant_dot_desc*, const void*, const void*, const void*);
 int mi355_mfma_gemm_launch(const mi355_quant_dot_desc*,
@@ -337,6 +339,73 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
     return mi355_launch_status();
 }
 
+// ---- quant_dot that allocates nothing and takes no workspace -------------------------------
+// The split-K partial sums of mi355_quant_dot_ws go to a device array that is part of the
+// library's code object: every GPU the library runs on holds its own copy from the moment the
+// module is loaded there until the process ends.  In host code the array's name only stands for
+// the symbol; the memory is reached through the address hipGetSymbolAddress reports on the
+// device that is current, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[MI355_QUANT_DOT_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int max_devices = 64;
+std::atomic<void*> scratch_of_device[max_devices];
+std::mutex scratch_lookup;
+
+// address of this device's copy of `scratch`; null with *status set when HIP reports an error
+void* device_scratch(int* status)
+{
+    int dev = -1;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= max_devices)
+    {
+        *status = MI355_ERR_LAUNCH;
+        return nullptr;
+    }
+    void* ptr = scratch_of_device[dev].load(std::memory_order_acquire);
+    if(ptr != nullptr)
+        return ptr;
+    std::lock_guard<std::mutex> guard(scratch_lookup);
+    ptr = scratch_of_device[dev].load(std::memory_order_acquire);
+    if(ptr != nullptr)
+        return ptr;
+    if(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr)
+    {
+        (void)hipGetLastError();
+        *status = MI355_ERR_LAUNCH;
+        return nullptr;
+    }
+    scratch_of_device[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+} // namespace
+
+extern "C" int mi355_quant_dot_static(const mi355_quant_dot_desc* d,
+                                      const void* a,
+                                      const void* b,
+                                      void* c,
+                                      const float* scale_a,
+                                      const float* scale_b,
+                                      const int32_t* colsum_b,
+                                      const int32_t* rowsum_a,
+                                      const float* bias,
+                                      void* stream)
+{
+    if(d == nullptr)
+        return MI355_ERR_BAD_ARG;
+    const size_t need = mi355_quant_dot_workspace_size(d);
+    if(need > MI355_QUANT_DOT_STATIC_SCRATCH_BYTES)
+        return MI355_ERR_SCRATCH_TOO_SMALL;
+    if(need == 0) // no split for this description: the one-pass kernels use no scratch memory
+        return mi355_quant_dot_ws(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, nullptr, 0, stream);
+    int status = MI355_OK;
+    void* ptr  = device_scratch(&status);
+    if(ptr == nullptr)
+        return status;
+    // every element of the partial sums that the second kernel reads is stored by the first one in
+    // the same call, so nothing has to be cleared between calls
+    return mi355_quant_dot_ws(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, ptr, need, stream);
+}
+
 extern "C" int mi355_colsum_i8(const void* b,
                                int64_t k,
                                int64_t n,
@@ -401,6 +470,7 @@ extern "C" const char* mi355_status_string(int status)
     case MI355_ERR_BAD_ARG: return "bad argument";
     case MI355_ERR_UNSUPPORTED: return "unsupported configuration";
     case MI355_ERR_LAUNCH: return "HIP launch error";
+    case MI355_ERR_SCRATCH_TOO_SMALL: return "the problem needs more scratch memory than the library's static buffer holds";
     default: return "unknown status";
     }
 }

@@ -57,8 +57,10 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     (double(acc) - zp) * (scale_a*scale_b) -> out_dtype is applied; ``bias`` (float32 [N])
     is then added in float32, before the conversion to a 16-bit ``out_dtype``.
     ``workspace`` (any dense device tensor, see quant_dot_workspace_size) lets a skinny int8
-    product, bare or with the epilogue, split K over the chip without atomics."""
-    _require_cuda(a, b, scale_a, scale_b, bias, workspace)
+    product, bare or with the epilogue, split K over the chip without atomics; the word
+    ``"static"`` takes the library's own static device buffer instead (nothing is allocated,
+    shapes that need more than it holds are refused)."""
+    _require_cuda(a, b, scale_a, scale_b, bias, None if isinstance(workspace, str) else workspace)
     if a.dim() != b.dim() or a.dim() < 2:
         raise Mi355Error("QUANT_DOT: dot only accepts >= 2D operands of equal rank")
     if a.shape[:-2] != b.shape[:-2]:
@@ -115,7 +117,13 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
             raise Mi355Error("quant_dot: a bias needs the dequantizing epilogue")
         if bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous():
             raise Mi355Error("bias must be a dense float32 vector of N elements")
-    if workspace is not None:
+    if isinstance(workspace, str):
+        if workspace != "static":
+            raise Mi355Error("workspace must be a device tensor or the word 'static'")
+        st = lib().mi355_quant_dot_static(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
+                                          _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _ptr(bias), _stream())
+        check(st, "mi355_quant_dot_static")
+    elif workspace is not None:
         if not workspace.is_contiguous():
             raise Mi355Error("the workspace must be dense")
         st = lib().mi355_quant_dot_ws(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),

@@ -28,7 +28,8 @@ typedef enum mi355_status {
     MI355_OK              = 0,
     MI355_ERR_BAD_ARG     = -1, /* null pointer, negative size, bad enum */
     MI355_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for */
-    MI355_ERR_LAUNCH      = -3  /* HIP reported an error at launch */
+    MI355_ERR_LAUNCH      = -3, /* HIP reported an error at launch */
+    MI355_ERR_SCRATCH_TOO_SMALL = -4 /* mi355_quant_dot_static: the split needs more than the static buffer */
 } mi355_status;
 
 /* Element types.  half / bf16 / fp8 are passed as their raw bits. */
@@ -177,6 +178,22 @@ int mi355_quant_dot_ws(const mi355_quant_dot_desc* desc, const void* a, const vo
                        const float* scale_a, const float* scale_b, const int32_t* colsum_b,
                        const int32_t* rowsum_a, const float* bias, void* workspace,
                        size_t workspace_bytes, void* stream);
+
+/* quant_dot for callers that cannot allocate.  No counterpart in the reference: it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, which can
+ * neither allocate the workspace of mi355_quant_dot_ws nor keep one around.  Same arguments and
+ * result as mi355_quant_dot_ws; the split-K partial sums go to a buffer of
+ * MI355_QUANT_DOT_STATIC_SCRATCH_BYTES that is part of the library's device code (one copy per
+ * GPU, held from module load until the process ends).  The call itself allocates and frees
+ * nothing; the first call on a device looks the buffer's address up once.  A description whose
+ * mi355_quant_dot_workspace_size exceeds the buffer is refused with MI355_ERR_SCRATCH_TOO_SMALL
+ * (nothing is launched).  All calls on one GPU share the buffer: calls that may run at the same
+ * time on one GPU (different streams, different threads) race on it and must be ordered by the
+ * caller.  The buffer keeps the last call's partial sums; no call depends on its contents. */
+#define MI355_QUANT_DOT_STATIC_SCRATCH_BYTES (32u << 20)
+int mi355_quant_dot_static(const mi355_quant_dot_desc* desc, const void* a, const void* b, void* c,
+                           const float* scale_a, const float* scale_b, const int32_t* colsum_b,
+                           const int32_t* rowsum_a, const float* bias, void* stream);
 
 /* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
  * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the
