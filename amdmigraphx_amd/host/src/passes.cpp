@@ -72,70 +72,95 @@ void dead_code_elimination::apply(module& m) const
 
 namespace {
 
-const std::set<std::string>& post_dq_ops()
+// ---- a product operand that comes out of a dequantizelinear ------------------------------------
+//
+// Between a dot / convolution argument and the dequantizelinear that made it there may stand
+// operators that only re-label or re-type the tensor (match/dq_helpers.hpp:40-57 lists them).
+// The rewrite moves the product in front of the dequantization, so those operators have to be
+// applied to the quantized tensor instead (simplify_qdq.cpp:49-82).
+struct dequantized_operand
 {
-    static const std::set<std::string> s = {
-        "broadcast", "multibroadcast", "contiguous", "transpose", "reshape", "convert"};
-    return s;
-}
+    instruction_ref dq;
+    std::vector<instruction_ref> views; // what stood between, the one next to dq first
 
-// dequantizelinear(x, const scale, const zp), looked for through the operators that may sit
-// between it and the dot (match/dq_helpers.hpp:40-57)
-instruction_ref find_dq(instruction_ref arg)
-{
-    while(contains(post_dq_ops(), arg->name()))
-        arg = arg->inputs().front();
-    return arg;
-}
-
-bool is_const_dq(instruction_ref dq)
-{
-    if(dq->name() != "dequantizelinear" or dq->inputs().size() != 3)
-        return false;
-    return skip_broadcasts(dq->inputs()[1])->can_eval() and
-           skip_broadcasts(dq->inputs()[2])->can_eval();
-}
-
-std::vector<instruction_ref> get_between_ins(instruction_ref dq, instruction_ref arg)
-{
-    std::vector<instruction_ref> r;
-    while(arg != dq)
+    static bool passes_through(const std::string& name)
     {
-        r.push_back(arg);
-        arg = arg->inputs().front();
+        static const std::set<std::string> names = {
+            "broadcast", "multibroadcast", "contiguous", "transpose", "reshape", "convert"};
+        return names.count(name) > 0;
     }
-    return r;
-}
 
-// re-apply the view operators that stood between DQ and dot to the quantized tensor
-// (simplify_qdq.cpp:64-82)
-instruction_ref propagate_quantized_ins(module& m,
-                                        instruction_ref dq,
-                                        instruction_ref input,
-                                        const std::vector<instruction_ref>& between,
-                                        bool is_fp16_model)
-{
-    for(auto it = between.rbegin(); it != between.rend(); ++it)
+    static dequantized_operand behind(instruction_ref arg)
     {
-        if((*it)->name() == "convert" and is_fp16_model)
-            continue;
-        input = m.insert_instruction(dq, (*it)->get_operator(), input);
+        dequantized_operand r;
+        while(passes_through(arg->name()))
+        {
+            r.views.insert(r.views.begin(), arg);
+            arg = arg->inputs().front();
+        }
+        r.dq = arg;
+        return r;
     }
-    return input;
+
+    bool is_dq() const { return dq->name() == "dequantizelinear"; }
+    instruction_ref tensor() const { return dq->inputs()[0]; }
+    instruction_ref scale() const { return skip_broadcasts(dq->inputs()[1]); }
+    instruction_ref zero_point() const { return skip_broadcasts(dq->inputs()[2]); }
+
+    // scale and zero point both present and known at compile time
+    bool constant_parameters() const
+    {
+        return is_dq() and dq->inputs().size() == 3 and scale()->can_eval() and zero_point()->can_eval();
+    }
+
+    // MX block quantization: no zero point, and a scale of the tensor's own rank (one value per
+    // block, spread over the block's elements by the broadcasts in front of it)
+    bool block_scaled() const
+    {
+        if(not is_dq() or dq->inputs().size() != 2)
+            return false;
+        const auto& s = scale()->get_shape();
+        return not s.scalar() and s.ndim() != 1;
+    }
+
+    // x with the operand's view operators on top, inserted in front of the dequantizelinear; a
+    // `convert` among them is dropped when the product's own type says the model runs in half
+    instruction_ref with_views(module& m, instruction_ref x, bool half_model) const
+    {
+        for(auto v : views)
+        {
+            if(half_model and v->name() == "convert")
+                continue;
+            x = m.insert_instruction(dq, v->get_operator(), x);
+        }
+        return x;
+    }
+};
+
+// the product's result is half while the dequantized operands are not: an fp16 model whose Q/DQ
+// pairs were inserted in float; the rewritten product converts its result back (:283-287)
+bool runs_in_half(instruction_ref product, const dequantized_operand& a)
+{
+    return product->get_shape().type() == shape::half_type and a.dq->get_shape().type() != shape::half_type;
 }
 
-bool is_valid_qparam(instruction_ref q, const std::vector<std::size_t>& lens, std::size_t axis)
+bool is_quantized_type(shape::type_t t)
 {
-    return q->get_shape().elements() == 1 or q->get_shape().elements() == lens.at(axis);
+    return t == shape::int8_type or t == shape::fp8e4m3fn_type or t == shape::fp8e4m3fnuz_type or
+           t == shape::fp8e5m2_type or t == shape::fp8e5m2fnuz_type;
 }
 
-operation qparam_broadcast_op(instruction_ref q, const std::vector<std::size_t>& lens, std::size_t axis)
+bool evaluates_to_zero(instruction_ref x) { return x->can_eval() and all_zero(x->eval()); }
+
+// one value, or one value per index of `axis`
+instruction_ref spread(module& m, instruction_ref pos, instruction_ref q, const std::vector<std::size_t>& lens,
+                       std::size_t axis)
 {
-    // one value: spread it whatever shape it came in (a scalar, or the [1] tensor of an ONNX
-    // initializer)
+    // a single value is spread whatever shape it came in (a scalar, or the [1] tensor of an
+    // ONNX initializer)
     if(q->get_shape().scalar() or q->get_shape().elements() == 1)
-        return make_op("multibroadcast", {{"out_lens", lens}});
-    return make_op("broadcast", {{"out_lens", lens}, {"axis", axis}});
+        return m.insert_instruction(pos, make_op("multibroadcast", {{"out_lens", lens}}), q);
+    return m.insert_instruction(pos, make_op("broadcast", {{"out_lens", lens}, {"axis", axis}}), q);
 }
 
 // A per-axis parameter that arrives with unit dimensions around its axis (the ONNX parsers
@@ -152,172 +177,111 @@ instruction_ref as_vector(module& m, instruction_ref pos, instruction_ref q)
     return m.insert_instruction(pos, make_op("reshape", {{"dims", {static_cast<int64_t>(s.elements())}}}), q);
 }
 
-bool is_symmetric_zero_point(instruction_ref zp)
+// ---- dot / convolution of two dequantized tensors -> quantized product + one dequantizelinear --
+//
+// simplify_qdq.cpp:128-289.  dot and convolution differ only in where a per-axis parameter of
+// each operand runs: along M / N of a dot's result and operands (:232-238), along the output
+// channels for a convolution's weights, while a convolution's input may carry one scale and one
+// zero point only (:171-195).  With x = sa (qa - za), w = sb (qb - zb):
+//   x * w = sa sb [ qa*qb - za*qb - qa*zb + za*zb ]
+// so the result is dequantizelinear(qa*qb, scale = sa sb, zero point = za*qb + qa*zb - za*zb),
+// each `*` the quantized product itself and the zero-point terms present only for non-zero
+// zero points (:196-222, :250-279).
+struct product_axes
 {
-    if(not zp->can_eval())
-        return false;
-    return all_zero(zp->eval());
-}
+    std::size_t in_result[2];  // axis of the result the parameters of operand 0 / 1 follow
+    std::size_t in_operand[2]; // the same axis in the operand itself
+    bool per_axis[2];          // may the operand carry one parameter per index at all
+};
 
-bool is_quantized_type(shape::type_t t)
+void quantize_product(module& m, instruction_ref product)
 {
-    return t == shape::int8_type or t == shape::fp8e4m3fn_type or t == shape::fp8e4m3fnuz_type or
-           t == shape::fp8e5m2_type or t == shape::fp8e5m2fnuz_type;
-}
-
-// simplify_qdq.cpp:126-289: the dot branch and the convolution branch (:171-222)
-void find_quantizable_dot(module& m, instruction_ref qop)
-{
-    auto dq1 = find_dq(qop->inputs()[0]);
-    auto dq2 = find_dq(qop->inputs()[1]);
-    if(not is_const_dq(dq1) or not is_const_dq(dq2))
+    const dequantized_operand side[2] = {dequantized_operand::behind(product->inputs()[0]),
+                                         dequantized_operand::behind(product->inputs()[1])};
+    if(not side[0].constant_parameters() or not side[1].constant_parameters())
         return;
-    auto scale1 = skip_broadcasts(dq1->inputs()[1]);
-    auto zp1    = skip_broadcasts(dq1->inputs()[2]);
-    auto scale2 = skip_broadcasts(dq2->inputs()[1]);
-    auto zp2    = skip_broadcasts(dq2->inputs()[2]);
+    const bool half_model = runs_in_half(product, side[0]);
+    const bool is_conv    = product->name() == "convolution";
 
-    bool is_fp16_model = false;
-    if(dq1->get_shape().type() != qop->get_shape().type() and
-       qop->get_shape().type() == shape::half_type)
-        is_fp16_model = true;
-
-    auto qop_args = qop->inputs();
-    auto between0 = get_between_ins(dq1, qop_args[0]);
-    auto between1 = get_between_ins(dq2, qop_args[1]);
-    qop_args[0]   = propagate_quantized_ins(m, dq1, dq1->inputs().front(), between0, is_fp16_model);
-    qop_args[1]   = propagate_quantized_ins(m, dq2, dq2->inputs().front(), between1, is_fp16_model);
-    auto arg1_lens = qop_args[0]->get_shape().lens();
-    auto arg2_lens = qop_args[1]->get_shape().lens();
-
+    instruction_ref q[2], scale[2], zp[2];
+    for(int i = 0; i < 2; i++)
+    {
+        q[i]     = side[i].with_views(m, side[i].tensor(), half_model);
+        scale[i] = side[i].scale();
+        zp[i]    = side[i].zero_point();
+    }
     // only int8 and fp8 tensors are rewritten; uint8 Q/DQ stays as it is (:157-165)
-    if(not is_quantized_type(dq1->inputs().front()->get_shape().type()) or
-       not is_quantized_type(dq2->inputs().front()->get_shape().type()))
+    if(not is_quantized_type(side[0].tensor()->get_shape().type()) or
+       not is_quantized_type(side[1].tensor()->get_shape().type()))
         return;
 
-    if(qop->name() == "convolution")
+    const operation qop = is_conv ? make_op("quant_convolution", product->get_operator().to_value())
+                                  : make_op("quant_dot");
+    auto multiply       = [&](instruction_ref x, instruction_ref w) { return m.insert_instruction(product, qop, x, w); };
+    auto acc            = multiply(q[0], q[1]);
+    const auto lens     = acc->get_shape().lens();
+    const std::vector<std::size_t> operand_lens[2] = {q[0]->get_shape().lens(), q[1]->get_shape().lens()};
+    const std::size_t nd = lens.size();
+    const product_axes ax =
+        is_conv ? product_axes{{1, 1}, {1, 0}, {false, true}}
+                : product_axes{{nd - 2, nd - 1}, {operand_lens[0].size() - 2, operand_lens[1].size() - 1}, {true, true}};
+    for(int i = 0; i < 2; i++)
     {
-        // simplify_qdq.cpp:171-222: the input may only carry one scale and zero point, the
-        // weights one per output channel (axis 0 of the weights, axis 1 of the result)
-        const auto conv_val = qop->get_operator().to_value();
-        auto qconv          = m.insert_instruction(qop, make_op("quant_convolution", conv_val), qop_args);
-        auto conv_lens      = qconv->get_shape().lens();
-        if(not(scale1->get_shape().elements() == 1 and zp1->get_shape().elements() == 1 and
-               is_valid_qparam(scale2, arg2_lens, 0) and is_valid_qparam(zp2, arg2_lens, 0)))
-            return;
-        scale2 = as_vector(m, qop, scale2);
-        zp2    = as_vector(m, qop, zp2);
-        auto s1 = m.insert_instruction(qop, qparam_broadcast_op(scale1, conv_lens, 1), scale1);
-        auto s2 = m.insert_instruction(qop, qparam_broadcast_op(scale2, conv_lens, 1), scale2);
-        auto conv_scale = m.insert_instruction(qop, make_op("mul"), s1, s2);
-        auto zero = m.add_literal(literal{shape{qconv->get_shape().type()}, std::vector<int>{0}});
-        auto conv_zp =
-            m.insert_instruction(qop, make_op("multibroadcast", {{"out_lens", conv_lens}}), zero);
-        auto in_zp_bc = m.insert_instruction(qop, qparam_broadcast_op(zp1, arg1_lens, 1), zp1);
-        auto w_zp_bc  = m.insert_instruction(qop, qparam_broadcast_op(zp2, arg2_lens, 0), zp2);
-        const bool s1z = is_symmetric_zero_point(zp1);
-        const bool s2z = is_symmetric_zero_point(zp2);
-        if(not s1z)
+        for(auto p : {scale[i], zp[i]})
         {
-            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), in_zp_bc, qop_args[1]);
-            conv_zp = m.insert_instruction(qop, make_op("add"), conv_zp, t);
+            const auto n = p->get_shape().elements();
+            if(n != 1 and not(ax.per_axis[i] and n == lens.at(ax.in_result[i])))
+                return; // parameters along another axis: the graph stays as it was
         }
-        if(not s2z)
-        {
-            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), qop_args[0], w_zp_bc);
-            conv_zp = m.insert_instruction(qop, make_op("add"), conv_zp, t);
-        }
-        if(not s1z and not s2z)
-        {
-            auto t  = m.insert_instruction(qop, make_op("quant_convolution", conv_val), in_zp_bc, w_zp_bc);
-            conv_zp = m.insert_instruction(qop, make_op("sub"), conv_zp, t);
-        }
-        auto r = m.insert_instruction(qop, make_op("dequantizelinear"), qconv, conv_scale, conv_zp);
-        if(is_fp16_model)
-            r = m.insert_instruction(qop, make_op("convert", {{"target_type", shape::half_type}}), r);
-        m.replace_instruction(qop, r);
-        return;
     }
-
-    auto dq       = m.insert_instruction(qop, make_op("quant_dot"), qop_args);
-    auto out_lens = dq->get_shape().lens();
-    const std::size_t nd = out_lens.size();
-    // valid quantization axes: M for the first input, N for the second (:232-238)
-    if(not(is_valid_qparam(scale1, out_lens, nd - 2) and is_valid_qparam(zp1, out_lens, nd - 2) and
-           is_valid_qparam(scale2, out_lens, nd - 1) and is_valid_qparam(zp2, out_lens, nd - 1)))
-        return;
-    scale1 = as_vector(m, qop, scale1);
-    zp1    = as_vector(m, qop, zp1);
-    scale2 = as_vector(m, qop, scale2);
-    zp2    = as_vector(m, qop, zp2);
-
-    auto s1_bcast = m.insert_instruction(qop, qparam_broadcast_op(scale1, out_lens, nd - 2), scale1);
-    auto s2_bcast = m.insert_instruction(qop, qparam_broadcast_op(scale2, out_lens, nd - 1), scale2);
-    auto out_scale = m.insert_instruction(qop, make_op("mul"), s1_bcast, s2_bcast);
-
-    // zero-point terms: 0 [+ zp1*B] [+ A*zp2] [- zp1*zp2] (:250-279)
-    auto zero_lit = m.add_literal(literal{shape{dq->get_shape().type()}, std::vector<int>{0}});
-    auto out_zp =
-        m.insert_instruction(qop, make_op("multibroadcast", {{"out_lens", out_lens}}), zero_lit);
-    auto zp1_bc =
-        m.insert_instruction(qop, qparam_broadcast_op(zp1, arg1_lens, arg1_lens.size() - 2), zp1);
-    auto zp2_bc =
-        m.insert_instruction(qop, qparam_broadcast_op(zp2, arg2_lens, arg2_lens.size() - 1), zp2);
-    const bool sym1 = is_symmetric_zero_point(zp1);
-    const bool sym2 = is_symmetric_zero_point(zp2);
-    if(not sym1)
+    for(int i = 0; i < 2; i++)
     {
-        auto t = m.insert_instruction(qop, make_op("quant_dot"), zp1_bc, qop_args[1]);
-        out_zp = m.insert_instruction(qop, make_op("add"), out_zp, t);
-    }
-    if(not sym2)
-    {
-        auto t = m.insert_instruction(qop, make_op("quant_dot"), qop_args[0], zp2_bc);
-        out_zp = m.insert_instruction(qop, make_op("add"), out_zp, t);
-    }
-    if(not sym1 and not sym2)
-    {
-        auto t = m.insert_instruction(qop, make_op("quant_dot"), zp1_bc, zp2_bc);
-        out_zp = m.insert_instruction(qop, make_op("sub"), out_zp, t);
+        if(not ax.per_axis[i])
+            continue;
+        scale[i] = as_vector(m, product, scale[i]);
+        zp[i]    = as_vector(m, product, zp[i]);
     }
 
-    dq = m.insert_instruction(qop, make_op("dequantizelinear"), dq, out_scale, out_zp);
-    if(is_fp16_model)
-        dq = m.insert_instruction(qop, make_op("convert", {{"target_type", shape::half_type}}), dq);
-    m.replace_instruction(qop, dq);
+    auto sa        = spread(m, product, scale[0], lens, ax.in_result[0]);
+    auto sb        = spread(m, product, scale[1], lens, ax.in_result[1]);
+    auto out_scale = m.insert_instruction(product, make_op("mul"), sa, sb);
+
+    auto zero      = m.add_literal(literal{shape{acc->get_shape().type()}, std::vector<int>{0}});
+    auto shift     = m.insert_instruction(product, make_op("multibroadcast", {{"out_lens", lens}}), zero);
+    auto za        = spread(m, product, zp[0], operand_lens[0], ax.in_operand[0]);
+    auto zb        = spread(m, product, zp[1], operand_lens[1], ax.in_operand[1]);
+    const bool has_za = not evaluates_to_zero(zp[0]);
+    const bool has_zb = not evaluates_to_zero(zp[1]);
+    if(has_za)
+        shift = m.insert_instruction(product, make_op("add"), shift, multiply(za, q[1]));
+    if(has_zb)
+        shift = m.insert_instruction(product, make_op("add"), shift, multiply(q[0], zb));
+    if(has_za and has_zb)
+        shift = m.insert_instruction(product, make_op("sub"), shift, multiply(za, zb));
+
+    auto result = m.insert_instruction(product, make_op("dequantizelinear"), acc, out_scale, shift);
+    if(half_model)
+        result = m.insert_instruction(product, make_op("convert", {{"target_type", shape::half_type}}), result);
+    m.replace_instruction(product, result);
 }
 
 // simplify_qdq.cpp:290-357: block quantization of the MX types.  Both operands of the dot come
-// (through view operators) from a two-input dequantizelinear whose scale, behind its broadcasts,
-// is neither a scalar nor one-dimensional, i.e. has the operand's own rank: one scale per block,
-// spread over the elements.  The dot becomes quant_dot(a, b, scale_a, scale_b), the operators that
-// stood between each DQ and the dot re-applied to its tensor and to its scales alike.
-bool is_block_dq(instruction_ref dq)
+// (through view operators) from a two-input dequantizelinear with one scale per block.  The dot
+// becomes quant_dot(a, b, scale_a, scale_b); what stood between each dequantizelinear and the dot
+// is applied to its tensor and to its scales alike.
+void quantize_block_scaled_dot(module& m, instruction_ref dot)
 {
-    if(dq->name() != "dequantizelinear" or dq->inputs().size() != 2)
-        return false;
-    auto scale = skip_broadcasts(dq->inputs()[1]);
-    return not scale->get_shape().scalar() and scale->get_shape().ndim() != 1;
-}
-
-void find_mx_quantizable_dot(module& m, instruction_ref qop)
-{
-    auto dq1 = find_dq(qop->inputs()[0]);
-    auto dq2 = find_dq(qop->inputs()[1]);
-    if(not is_block_dq(dq1) or not is_block_dq(dq2))
+    const auto a = dequantized_operand::behind(dot->inputs()[0]);
+    const auto b = dequantized_operand::behind(dot->inputs()[1]);
+    if(not a.block_scaled() or not b.block_scaled())
         return;
-    bool is_fp16_model = false;
-    if(dq1->get_shape().type() != qop->get_shape().type() and
-       qop->get_shape().type() == shape::half_type)
-        is_fp16_model = true;
-    auto qop_args = qop->inputs();
-    auto between0 = get_between_ins(dq1, qop_args[0]);
-    auto between1 = get_between_ins(dq2, qop_args[1]);
-    qop_args[0]   = propagate_quantized_ins(m, dq1, dq1->inputs().front(), between0, is_fp16_model);
-    qop_args[1]   = propagate_quantized_ins(m, dq2, dq2->inputs().front(), between1, is_fp16_model);
-    qop_args.push_back(propagate_quantized_ins(m, dq1, dq1->inputs()[1], between0, is_fp16_model));
-    qop_args.push_back(propagate_quantized_ins(m, dq2, dq2->inputs()[1], between1, is_fp16_model));
-    m.replace_instruction(qop, make_op("quant_dot"), qop_args);
+    const bool half_model = runs_in_half(dot, a);
+    std::vector<instruction_ref> args;
+    args.push_back(a.with_views(m, a.tensor(), half_model));
+    args.push_back(b.with_views(m, b.tensor(), half_model));
+    args.push_back(a.with_views(m, a.dq->inputs()[1], half_model));
+    args.push_back(b.with_views(m, b.dq->inputs()[1], half_model));
+    m.replace_instruction(dot, make_op("quant_dot"), args);
 }
 
 // simplify_qdq.cpp:360-394
@@ -449,7 +413,7 @@ void simplify_qdq::apply(module& m) const
     for(auto ins : all_instructions(m))
     {
         if(ins->name() == "dot" or ins->name() == "convolution")
-            find_quantizable_dot(m, ins);
+            quantize_product(m, ins);
     }
     dead_code_elimination{}.apply(m);
     if(use_mx_quant)
@@ -457,7 +421,7 @@ void simplify_qdq::apply(module& m) const
         for(auto ins : all_instructions(m))
         {
             if(ins->name() == "dot")
-                find_mx_quantizable_dot(m, ins);
+                quantize_block_scaled_dot(m, ins);
         }
         dead_code_elimination{}.apply(m);
     }
@@ -504,87 +468,121 @@ void capture_arguments_pass::apply(module& m) const
     }
 }
 
+namespace {
+
+// The scale a quantizelinear / dequantizelinear pair carries is the inverse of the calibrated
+// multiplier, held inside what the tensor's own type can represent: at least its epsilon, at
+// most its largest finite value (quantize_8bits.cpp:73-83).
+float qdq_scale_for(float multiplier, shape::type_t tensor_type)
+{
+    float smallest = 0.0f;
+    float largest  = std::numeric_limits<float>::max();
+    visit_type(tensor_type, [&](auto tag) {
+        using limits = std::numeric_limits<decltype(tag)>;
+        smallest     = static_cast<float>(limits::epsilon());
+        largest      = static_cast<float>(limits::max());
+    });
+    return std::clamp(1.0f / multiplier, smallest, largest);
+}
+
+} // namespace
+
+// Every `capture` that marks a float tensor is replaced by quantizelinear -> dequantizelinear with
+// that tensor's calibrated parameters (quantize_8bits.cpp:52-96); simplify_qdq later moves the
+// products in front of the dequantizations.
 void quantize_8bits_pass::apply(module& m) const
 {
-    for(auto ins : all_instructions(m))
+    for(auto marker : all_instructions(m))
     {
-        if(ins->name() != "capture")
+        if(marker->name() != "capture")
             continue;
-        const auto index = any_cast<op::capture>(ins->get_operator()).ins_index;
-        const auto param = quant_params.at(index);
-        auto input       = ins->inputs().front();
-        const auto s     = input->get_shape();
-        if(quantizable_types().count(s.type()) == 0 or s.type() == precision)
+        auto x           = marker->inputs().front();
+        const auto& xs   = x->get_shape();
+        if(quantizable_types().count(xs.type()) == 0 or xs.type() == precision)
             continue;
-        auto zero_point = m.add_literal(literal{shape{precision}, std::vector<float>{param.second}});
-        // the Q/DQ scale is the inverse of the calibrated multiplier, kept within the tensor
-        // type's [epsilon, max] (quantize_8bits.cpp:73-83)
-        float inverted_scale = 1.0f / param.first;
-        float epsilon        = 0.0f;
-        float max_val        = std::numeric_limits<float>::max();
-        visit_type(s.type(), [&](auto x) {
-            using T = decltype(x);
-            epsilon = static_cast<float>(std::numeric_limits<T>::epsilon());
-            max_val = static_cast<float>(std::numeric_limits<T>::max());
-        });
-        inverted_scale = std::max(epsilon, std::min(max_val, inverted_scale));
-        auto scale     = m.add_literal(literal{shape{s.type()}, std::vector<float>{inverted_scale}});
-        auto scale_bc =
-            m.insert_instruction(ins, make_op("multibroadcast", {{"out_lens", s.lens()}}), scale);
-        auto zp_bc = m.insert_instruction(
-            ins, make_op("multibroadcast", {{"out_lens", s.lens()}}), zero_point);
-        auto q  = m.insert_instruction(ins, make_op("quantizelinear"), input, scale_bc, zp_bc);
-        auto dq = m.insert_instruction(ins, make_op("dequantizelinear"), q, scale_bc, zp_bc);
-        m.replace_instruction(ins, dq);
+        const auto& calibrated = quant_params.at(any_cast<op::capture>(marker->get_operator()).ins_index);
+        auto shift  = m.add_literal(literal{shape{precision}, std::vector<float>{calibrated.second}});
+        auto scale  = m.add_literal(literal{shape{xs.type()}, std::vector<float>{qdq_scale_for(calibrated.first, xs.type())}});
+        const auto over_x = make_op("multibroadcast", {{"out_lens", xs.lens()}});
+        auto scales = m.insert_instruction(marker, over_x, scale);
+        auto shifts = m.insert_instruction(marker, over_x, shift);
+        auto stored = m.insert_instruction(marker, make_op("quantizelinear"), x, scales, shifts);
+        m.replace_instruction(marker, make_op("dequantizelinear"), stored, scales, shifts);
     }
 }
 
 namespace {
 
-void quantize_8bits(program& prog,
-                    const target& t,
-                    shape::type_t precision,
-                    const std::vector<parameter_map>& calibration,
-                    const std::unordered_set<std::string>& ins_names)
+// Calibration state of one quantization run: the largest magnitude every captured tensor has
+// shown so far and the (multiplier, shift) pair that follows from it.  The multiplier maps the
+// observed range onto the quantized type's, the shift stays 0 (quantization.cpp:88-130).
+class range_calibration
 {
-    auto params   = std::make_shared<std::vector<std::pair<float, float>>>();
-    auto max_abs  = std::make_shared<std::vector<float>>();
-    static const std::map<shape::type_t, float> ranges = {{shape::int8_type, 127.0f},
-                                                          {shape::fp8e4m3fnuz_type, 240.0f},
-                                                          {shape::fp8e4m3fn_type, 448.0f}};
-    const float quantized_range = ranges.at(precision);
-    // scale = range / max|x| over all calibration runs; the shift stays 0 (quantization.cpp:101-130)
-    auto calc = [=](std::size_t index, std::vector<argument> args) {
-        argument host = t.copy_from(args.front());
-        auto v        = host.to_vector<float>();
-        float m       = 0.0f;
-        for(float x : v)
-            m = std::max(m, std::fabs(x));
-        max_abs->at(index)   = std::max(max_abs->at(index), m);
-        std::pair<float, float> p{64.0f, 0.0f};
-        p.first           = float_equal(max_abs->at(index), 0.0f) ? 1.0f : quantized_range / max_abs->at(index);
-        params->at(index) = p;
-    };
-
-    std::size_t param_num = 0;
-    run_passes(prog, {capture_arguments_pass{ins_names, calc, &param_num}});
-    params->resize(param_num, std::pair<float, float>(64.0f, 0.0f));
-    max_abs->resize(param_num, 0.0f);
-
-    program capture_prog = prog;
-    capture_prog.compile(t);
-    for(const auto& arg : calibration)
+    public:
+    explicit range_calibration(shape::type_t precision)
     {
-        parameter_map pm;
-        for(const auto& x : capture_prog.get_parameter_shapes())
+        switch(precision)
         {
-            auto it = arg.find(x.first);
-            pm[x.first] = it != arg.end() ? t.copy_to(it->second) : t.allocate(x.second);
+        case shape::int8_type: target_range = 127.0f; break;
+        case shape::fp8e4m3fnuz_type: target_range = 240.0f; break;
+        case shape::fp8e4m3fn_type: target_range = 448.0f; break;
+        default: MIGRAPHX_THROW("quantize: no 8-bit range for this type");
         }
-        capture_prog.eval(pm);
-        capture_prog.finish();
     }
-    run_passes(prog, {quantize_8bits_pass{precision, *params}, dead_code_elimination{}});
+
+    void resize(std::size_t n)
+    {
+        largest.assign(n, 0.0f);
+        parameters.assign(n, {64.0f, 0.0f}); // what a tensor that is never observed keeps
+    }
+
+    void observe(std::size_t index, const std::vector<float>& values)
+    {
+        float seen = largest.at(index);
+        for(float v : values)
+            seen = std::max(seen, std::fabs(v));
+        largest.at(index)    = seen;
+        parameters.at(index) = {seen == 0.0f ? 1.0f : target_range / seen, 0.0f};
+    }
+
+    std::vector<std::pair<float, float>> parameters;
+
+    private:
+    float target_range = 0.0f;
+    std::vector<float> largest;
+};
+
+// quantization.cpp:132-174: mark the inputs of the named operators, run the marked program on
+// the calibration data (on whatever target the caller chose, this build's included), then turn
+// the marks into Q/DQ pairs
+void calibrate_and_insert_qdq(program& prog,
+                              const target& t,
+                              shape::type_t precision,
+                              const std::vector<parameter_map>& calibration,
+                              const std::unordered_set<std::string>& ins_names)
+{
+    auto state = std::make_shared<range_calibration>(precision);
+    auto on_capture = [state, t](std::size_t index, std::vector<argument> args) {
+        state->observe(index, t.copy_from(args.front()).to_vector<float>());
+    };
+    std::size_t marked = 0;
+    run_passes(prog, {capture_arguments_pass{ins_names, on_capture, &marked}});
+    state->resize(marked);
+
+    program marked_prog = prog;
+    marked_prog.compile(t);
+    for(const auto& sample : calibration)
+    {
+        parameter_map inputs;
+        for(const auto& [name, param_shape] : marked_prog.get_parameter_shapes())
+        {
+            const auto given = sample.find(name);
+            inputs[name]     = given != sample.end() ? t.copy_to(given->second) : t.allocate(param_shape);
+        }
+        marked_prog.eval(inputs);
+        marked_prog.finish();
+    }
+    run_passes(prog, {quantize_8bits_pass{precision, state->parameters}, dead_code_elimination{}});
 }
 
 } // namespace
@@ -597,7 +595,7 @@ void quantize_int8(program& prog,
     const std::unordered_set<std::string> op_names = {"convolution", "dot"};
     if(op_names != ins_names)
         MIGRAPHX_THROW("QUANTIZE_INT8: only support DOT and CONVOLUTION operation");
-    quantize_8bits(prog, t, shape::int8_type, calibration, ins_names);
+    calibrate_and_insert_qdq(prog, t, shape::int8_type, calibration, ins_names);
 }
 
 void quantize_fp8(program& prog, const target& t, const std::vector<parameter_map>& calibration)
@@ -609,55 +607,83 @@ void quantize_fp8(program& prog, const target& t, const std::vector<parameter_ma
             continue;
         names.insert(ins->name());
     }
-    quantize_8bits(prog, t, shape::fp8e4m3fn_type, calibration, names);
+    calibrate_and_insert_qdq(prog, t, shape::fp8e4m3fn_type, calibration, names);
 }
 
 // ---------------------------------------------------------------- quantize int4
 
+namespace {
+
+// Per-tensor affine 4-bit parameters: the value range, widened to contain 0, mapped onto 0..15
+// (quantize_int4.cpp:73-78)
+struct uint4_affine
+{
+    float scale;
+    int zero_point;
+
+    static uint4_affine covering(const std::vector<float>& values)
+    {
+        const auto [lo_it, hi_it] = std::minmax_element(values.begin(), values.end());
+        const float lo            = std::min(*lo_it, 0.0f);
+        const float hi            = std::max(*hi_it, 0.0f);
+        uint4_affine r{(hi - lo) / 15, 0};
+        if(r.scale != 0)
+            r.zero_point = static_cast<int>(std::round(-lo / r.scale));
+        return r;
+    }
+};
+
+// a constant float / half operand whose last axis can be packed two to a byte
+bool can_store_as_int4(instruction_ref x)
+{
+    const auto& s = x->get_shape();
+    if(s.broadcasted() or (s.type() != shape::float_type and s.type() != shape::half_type))
+        return false;
+    return s.lens().back() % 2 == 0 and x->can_eval();
+}
+
+// x -> dequantizelinear(unpack_int4(pack_int4(quantizelinear(x)))), all in front of `user`; the
+// scale literals take the user's result type (quantize_int4.cpp:80-100)
+instruction_ref through_int4(module& m, instruction_ref user, instruction_ref x)
+{
+    const auto values = x->eval().to_vector<float>();
+    if(values.empty())
+        return x;
+    const auto affine = uint4_affine::covering(values);
+    const auto over_x = make_op("multibroadcast", {{"out_lens", x->get_shape().lens()}});
+    // the quantizing and the dequantizing side get literals of their own, as the reference's do
+    auto parameters = [&] {
+        auto s = m.add_literal(literal{shape{user->get_shape().type()}, std::vector<float>{affine.scale}});
+        s      = m.insert_instruction(user, over_x, s);
+        auto z = m.add_literal(literal{shape{shape::uint8_type}, std::vector<int>{affine.zero_point}});
+        z      = m.insert_instruction(user, over_x, z);
+        return std::make_pair(s, z);
+    };
+    const auto [qs, qz] = parameters();
+    auto stored   = m.insert_instruction(user, make_op("quantizelinear"), x, qs, qz);
+    auto packed   = m.insert_instruction(user, make_op("pack_int4", {{"axis", -1}}), stored);
+    auto unpacked = m.insert_instruction(user, make_op("unpack_int4", {{"axis", -1}}), packed);
+    const auto [ds, dz] = parameters();
+    return m.insert_instruction(user, make_op("dequantizelinear"), unpacked, ds, dz);
+}
+
+} // namespace
+
+// quantize_int4.cpp:38-103: constant float / half operands of dot and convolution go through a
+// 4-bit store
 void quantize_int4_pass::apply(module& m) const
 {
-    for(auto ins : all_instructions(m))
+    for(auto user : all_instructions(m))
     {
-        if(ins->name() != "dot" or ins->inputs().empty())
+        if((user->name() != "dot" and user->name() != "convolution") or user->inputs().empty())
             continue;
-        const auto out_type = ins->get_shape().type();
-        auto inputs         = ins->inputs();
-        for(auto& inp : inputs)
+        auto operands = user->inputs();
+        for(auto& x : operands)
         {
-            const auto sh = inp->get_shape();
-            if(sh.broadcasted())
-                continue;
-            if(sh.type() != shape::float_type and sh.type() != shape::half_type)
-                continue;
-            const auto lens = sh.lens();
-            if(lens.back() % 2 != 0)
-                continue; // the packed axis must be even
-            if(not inp->can_eval())
-                continue;
-            auto val = inp->eval().to_vector<float>();
-            if(val.empty())
-                continue;
-            // per-tensor affine parameters over [min(0, min), max(0, max)] mapped to [0, 15]
-            float lo = std::min(0.0f, *std::min_element(val.begin(), val.end()));
-            float hi = std::max(0.0f, *std::max_element(val.begin(), val.end()));
-            const float fscale4 = (hi - lo) / 15;
-            const int zp4       = float_equal(fscale4, 0) ? 0 : static_cast<int>(std::round(-lo / fscale4));
-            auto bcast          = make_op("multibroadcast", {{"out_lens", lens}});
-            auto scale = m.add_literal(literal{shape{out_type}, std::vector<float>{fscale4}});
-            scale      = m.insert_instruction(ins, bcast, scale);
-            auto zp    = m.add_literal(literal{shape{shape::uint8_type}, std::vector<int>{zp4}});
-            zp         = m.insert_instruction(ins, bcast, zp);
-            auto q     = m.insert_instruction(ins, make_op("quantizelinear"), inp, scale, zp);
-            auto pk    = m.insert_instruction(ins, make_op("pack_int4", {{"axis", -1}}), q);
-            auto unpk  = m.insert_instruction(ins, make_op("unpack_int4", {{"axis", -1}}), pk);
-            auto dq_scale = m.add_literal(literal{shape{out_type}, std::vector<float>{fscale4}});
-            dq_scale      = m.insert_instruction(ins, bcast, dq_scale);
-            auto dq_zp = m.add_literal(literal{shape{shape::uint8_type}, std::vector<int>{zp4}});
-            dq_zp      = m.insert_instruction(ins, bcast, dq_zp);
-            inp = m.insert_instruction(ins, make_op("dequantizelinear"), unpk, dq_scale, dq_zp);
+            if(can_store_as_int4(x))
+                x = through_int4(m, user, x);
         }
-        auto converted = m.insert_instruction(ins, ins->get_operator(), inputs);
-        m.replace_instruction(ins, converted);
+        m.replace_instruction(user, m.insert_instruction(user, user->get_operator(), operands));
     }
 }
 

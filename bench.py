@@ -74,12 +74,22 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--only-headline", action="store_true",
                     help="time the headline kernel only (for counter runs under rocprofv3)")
+    ap.add_argument("--only", choices=["headline", "fp8", "gemv", "skinny", "conv"], default=None,
+                    help="run one section only, so that a rocprofv3 run holds that section's kernels alone")
+    ap.add_argument("--gemv-shape", default=None, metavar="K,N",
+                    help="with --only gemv: one (K, N) shape instead of the three of config 4")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB mebibytes a few "
                          "times: the HBM counters of that kernel calibrate roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+    if args.only_headline:
+        args.only = "headline"
+
+    def skip(section):
+        if args.only is not None and args.only != section:
+            raise RuntimeError(f"skipped (--only {args.only})")
 
     import torch
     from amdmigraphx_amd import ops
@@ -100,36 +110,39 @@ def main():
 
     # ---- headline: int8 quant_dot 8192^3 -> int32 --------------------------------
     M = N = K = 8192
-    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
-    b = torch.randint(-128, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
-    c = torch.empty((M, N), dtype=torch.int32, device=dev)
-
-    def step():
-        ops.quant_dot(a, b, out=c)
-
-    kern_s, wall_s = _time_launches(step, args.steps, args.warmup)
-    ops_per_step = 2.0 * M * N * K
-    tops = ops_per_step / wall_s / 1e12
-    kern_tops = ops_per_step / kern_s / 1e12
-
+    import numpy as np
+    from oracle import oracle as orc
     # every timed result is compared with the CPU oracle on sampled rows / columns, outside the
     # timed regions; "ok" in the output line is the conjunction
     checks = {}
-    import numpy as np
-    from oracle import oracle as orc
 
     def sampled_rows_equal(c_dev, a_dev, b_host, rows):
         want = orc.quant_dot(a_dev[rows].cpu().numpy(), b_host, orc.I8)
         return bool(np.array_equal(c_dev[rows].cpu().numpy(), want))
 
-    if not args.no_check:
-        checks["int8_quant_dot_8192"] = sampled_rows_equal(c, a, b.cpu().numpy(), [0, 255, 256, 4097, 8191])
+    kern_s = wall_s = float("nan")
+    if args.only in (None, "headline"):
+        a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+        b = torch.randint(-128, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+        c = torch.empty((M, N), dtype=torch.int32, device=dev)
+
+        def step():
+            ops.quant_dot(a, b, out=c)
+
+        kern_s, wall_s = _time_launches(step, args.steps, args.warmup)
+        if not args.no_check:
+            checks["int8_quant_dot_8192"] = sampled_rows_equal(c, a, b.cpu().numpy(), [0, 255, 256, 4097, 8191])
+        del a, b, c
+    ops_per_step = 2.0 * M * N * K
+    tops = ops_per_step / wall_s / 1e12
+    kern_tops = ops_per_step / kern_s / 1e12
+    if args.only not in (None, "headline"):     # a section run for the profiler: no headline figures
+        tops = kern_tops = wall_s = 0.0
 
     also = {}
     # ---- fp8 quant_dot with dequant epilogue, Llama-3-8B shape (config 3) ----------
     try:
-        if args.only_headline:
-            raise RuntimeError("skipped (--only-headline)")
+        skip("fp8")
         m3, k3, n3 = 4096, 4096, 14336 * 2
         # config 3's own distribution: bf16 activations ~N(0,1), weights ~N(0,0.02), each quantized to
         # fp8 e4m3fn with its per-tensor scale amax / 448
@@ -170,9 +183,11 @@ def main():
     # kernel plus the device-side gap between dependent kernels (about 2.6 us for
     # an empty kernel on this machine), not the host's submission rate.
     try:
-        if args.only_headline:
-            raise RuntimeError("skipped (--only-headline)")
-        for (k4, n4) in ((4096, 4096), (4096, 14336), (14336, 4096)):
+        skip("gemv")
+        shapes4 = ((4096, 4096), (4096, 14336), (14336, 4096))
+        if args.gemv_shape:
+            shapes4 = (tuple(int(v) for v in args.gemv_shape.split(",")),)
+        for (k4, n4) in shapes4:
             grp = 128
             bytes_per = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * k4 + 2 * n4
             # rotate through enough weight copies to exceed the 256 MB last-level cache
@@ -232,8 +247,7 @@ def main():
 
     # ---- skinny int8 quant_dot (config 2) and int4 GEMM at M = 16 / 128 (config 4) ----------
     try:
-        if args.only_headline:
-            raise RuntimeError("skipped (--only-headline)")
+        skip("skinny")
         for m2 in (16, 128):
             a2 = torch.randint(-128, 128, (m2, 8192), dtype=torch.int8, device=dev, generator=g)
             bs = [torch.randint(-128, 128, (8192, 8192), dtype=torch.int8, device=dev, generator=g)
@@ -350,8 +364,7 @@ def main():
 
     # ---- quant_convolution with the dequantize epilogue (ResNet-50-shaped 3 x 3 layers, batch 32) --
     try:
-        if args.only_headline:
-            raise RuntimeError("skipped (--only-headline)")
+        skip("conv")
         for (cc, hw, oo) in ((64, 56, 64), (256, 14, 256)):
             xq = torch.randint(-128, 128, (32, cc, hw, hw), dtype=torch.int8, device=dev, generator=g)
             wq = torch.randint(-128, 128, (oo, cc, 3, 3), dtype=torch.int8, device=dev, generator=g)
@@ -378,7 +391,7 @@ def main():
         "also": also,
         "checks": checks, "ok": all(checks.values()),
     }
-    if not args.no_cpu:
+    if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(rows=args.cpu_rows)
     print(json.dumps(line))
 

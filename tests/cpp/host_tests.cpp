@@ -992,6 +992,34 @@ TEST_CASE(int4_pass)
     EXPECT(count_ops(*m2, "quantizelinear") == 0);
 }
 
+TEST_CASE(int4_pass_takes_convolution_weights)
+{
+    // src/quantize_int4.cpp:40 lists convolution beside dot: constant weights with an even last
+    // dimension go through the 4-bit store, the data input (a parameter) does not
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {1, 3, 8, 8}});
+    auto wv  = uniform_floats(4 * 3 * 3 * 4, -0.5f, 1.0f, 19);
+    auto w   = mm->add_literal(literal{shape{shape::float_type, {4, 3, 3, 4}}, wv});
+    mm->add_return({mm->add_instruction(make_op("convolution"), x, w)});
+    program fp = p;
+    migraphx::quantize_int4_weights(p);
+    EXPECT(count_ops(*mm, "quantizelinear") == 1 and count_ops(*mm, "pack_int4") == 1 and
+           count_ops(*mm, "unpack_int4") == 1 and count_ops(*mm, "dequantizelinear") == 1);
+    auto conv = mm->get_returns().front();
+    EXPECT(conv->name() == "convolution" and conv->inputs()[0] == x);
+    EXPECT(conv->inputs()[1]->name() == "dequantizelinear");
+    EXPECT(conv->get_shape() == fp.get_main_module()->get_returns().front()->get_shape());
+    // 3 x 3 windows: the odd last dimension stays in float
+    program p2;
+    auto* m2 = p2.get_main_module();
+    auto x2  = m2->add_parameter("x", shape{shape::float_type, {1, 3, 8, 8}});
+    auto w2  = m2->add_literal(literal{shape{shape::float_type, {4, 3, 3, 3}}, uniform_floats(108, -1, 1, 2)});
+    m2->add_return({m2->add_instruction(make_op("convolution"), x2, w2)});
+    migraphx::quantize_int4_weights(p2);
+    EXPECT(count_ops(*m2, "quantizelinear") == 0);
+}
+
 TEST_CASE(int8_calibration)
 {
     // test/quantization.cpp:1066-1110: calibrated int8 dot stays close to the float dot
