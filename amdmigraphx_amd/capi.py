@@ -15,7 +15,7 @@ class Mi355Error(RuntimeError):
 
 
 class DT:
-    I8, U8, I32, F32, F16, BF16, FP8 = range(7)
+    I8, U8, I32, F32, F16, BF16, FP8, FP4X2 = range(8)
 
 
 class QP:
@@ -42,7 +42,16 @@ class QuantConvDesc(ctypes.Structure):
                 ("in_type", "out_type", "dequant", "scale_x_mode", "scale_w_mode")]
 
 
+class MxDotDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in
+                ("m", "n", "k", "batch", "lda", "ldb", "ldc", "stride_a", "stride_b", "stride_c",
+                 "sa_batch", "sa_row", "sa_block", "sa_elem", "sb_batch", "sb_row", "sb_block", "sb_elem")] + \
+               [(n, ctypes.c_int32) for n in ("a_type", "b_type")]
+
+
 EXPORTS = {
+    "mi355_quant_dot_mx_workspace_size": [ctypes.POINTER(MxDotDesc)],
+    "mi355_quant_dot_mx": [ctypes.POINTER(MxDotDesc)] + [ctypes.c_void_p] * 6 + [ctypes.c_size_t, ctypes.c_void_p],
     "mi355_quant_convolution_dims": [ctypes.POINTER(QuantConvDesc), ctypes.POINTER(ctypes.c_int64),
                                      ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_size_t)],
     "mi355_quant_convolution": [ctypes.POINTER(QuantConvDesc)] + [ctypes.c_void_p] * 6 +

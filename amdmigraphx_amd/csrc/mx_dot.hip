@@ -1,0 +1,328 @@
+// quant_dot with block scales (the MX formats): fp8 e4m3fn or packed fp4 e2m1 operands, one scale
+// per 32 elements along K for each row of A and each column of B, on the block-scaled matrix-core
+// instruction v_mfma_scale_f32_16x16x128_f8f6f4.
+//
+// The instruction takes, per lane, 32 consecutive K elements of one row (A) or column (B) and one
+// e8m0 scale (a power of two, the biased exponent byte of a float) for exactly those 32 elements:
+// a lane's fragment is one scale block.  The operator (ref_quant_gemm::compute, four inputs,
+// src/targets/ref/lowering.cpp:221-242) is more general: its scales are float tensors of the
+// operands' own shape, any value per element.  Three kernels keep every input right without a
+// host-side decision:
+//   mx_prepare_kernel   walks the scale tensors once: a block whose 32 scales are one normal power
+//                       of two becomes its exponent byte in a compact [rows, K/32] array; anything
+//                       else raises a flag in device memory;
+//   mx_gemm_kernel      the matrix-core product from the compact scales; returns at once when the
+//                       flag is up;
+//   mx_exact_kernel     the operator's arithmetic one output per thread -- float(a) * scale in
+//                       float, products and sum in double, one rounding to float -- and returns at
+//                       once when the flag is down.
+// With power-of-two block scales every float(a) * scale is exact, so the first path computes the
+// same sum as the second up to the fp32 accumulation of the instruction (the tolerance of the fp8
+// quant_dot); small sums are exact.
+#include "common.h"
+
+namespace {
+
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+struct mx_params
+{
+    const uint8_t* a;
+    const uint8_t* b;
+    float* c;
+    const float* scale_a;
+    const float* scale_b;
+    int m, n, k, nblk;
+    int64_t lda, ldb, ldc; // lda / ldb in bytes of the stored operand
+    int64_t stride_a, stride_b, stride_c;
+    int64_t sa_batch, sa_row, sa_block, sa_elem;
+    int64_t sb_batch, sb_row, sb_block, sb_elem;
+    int a4, b4; // operand stored as packed fp4 (two codes per byte, low nibble = even k)
+    uint32_t* flag;
+    uint8_t* ea; // [batch][m][nblk] exponent bytes
+    uint8_t* eb; // [batch][n][nblk]
+};
+
+__global__ void mx_clear_flag_kernel(uint32_t* flag) { *flag = 0; }
+
+// one thread per (operand, batch, row, block)
+__global__ __launch_bounds__(256) void mx_prepare_kernel(mx_params p, int batch)
+{
+    const bool is_b     = blockIdx.y != 0;
+    const int rows      = is_b ? p.n : p.m;
+    const int64_t total = (int64_t)batch * rows * p.nblk;
+    const int64_t i     = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if(i >= total)
+        return;
+    const int blk   = (int)(i % p.nblk);
+    const int row   = (int)((i / p.nblk) % rows);
+    const int bt    = (int)(i / ((int64_t)p.nblk * rows));
+    const float* s  = is_b ? p.scale_b + bt * p.sb_batch + row * p.sb_row + blk * p.sb_block
+                           : p.scale_a + bt * p.sa_batch + row * p.sa_row + blk * p.sa_block;
+    const int64_t e = is_b ? p.sb_elem : p.sa_elem;
+    const uint32_t first = __builtin_bit_cast(uint32_t, s[0]);
+    const uint32_t field = (first >> 23) & 0xffu;
+    // a positive normal power of two: no sign, no mantissa, exponent field 1..254
+    bool ok = (first & 0x807fffffu) == 0 && field >= 1 && field <= 254;
+    if(e != 0)
+    {
+        const int last = min(32, p.k - blk * 32);
+        for(int j = 1; j < last; j++)
+            ok = ok && __builtin_bit_cast(uint32_t, s[j * e]) == first;
+    }
+    (is_b ? p.eb : p.ea)[i] = (uint8_t)field;
+    if(!ok)
+        *p.flag = 1;
+}
+
+MI355_DEVINL float fp4_value(uint32_t code)
+{
+    // e2m1: sign, two exponent bits, one mantissa bit
+    const float mag[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+    const float v      = mag[code & 7];
+    return (code & 8) ? -v : v;
+}
+
+MI355_DEVINL float operand_value(const uint8_t* base, int k, int packed)
+{
+    if(packed)
+    {
+        const uint8_t byte = base[k >> 1];
+        return fp4_value((k & 1) ? (byte >> 4) : (byte & 0xf));
+    }
+    return fp8_to_f32(base[k]);
+}
+
+// the operator's own arithmetic, for scales the matrix-core path cannot take
+__global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p)
+{
+    if(*p.flag == 0)
+        return;
+    const int col = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int row = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int bt  = blockIdx.z;
+    if(row >= p.m || col >= p.n)
+        return;
+    const uint8_t* a = p.a + bt * p.stride_a + row * p.lda;
+    const uint8_t* b = p.b + bt * p.stride_b + col * p.ldb;
+    const float* sa  = p.scale_a + bt * p.sa_batch + row * p.sa_row;
+    const float* sb  = p.scale_b + bt * p.sb_batch + col * p.sb_row;
+    double sum       = 0;
+    for(int k = 0; k < p.k; k++)
+    {
+#pragma clang fp contract(off)
+        const float x = operand_value(a, k, p.a4) * sa[(k >> 5) * p.sa_block + (k & 31) * p.sa_elem];
+        const float w = operand_value(b, k, p.b4) * sb[(k >> 5) * p.sb_block + (k & 31) * p.sb_elem];
+        sum += (double)x * (double)w;
+    }
+    p.c[bt * p.stride_c + (int64_t)row * p.ldc + col] = (float)sum;
+}
+
+// 128 x 128 of C per workgroup of 4 waves (2 x 2), 64 x 64 per wave as 4 x 4 tiles of 16 x 16;
+// K in steps of 128.  A lane's fragment of a tile is the 32 K elements [32 g, 32 g + 32) of row
+// (or column) r, g = lane / 16, r = lane % 16: contiguous bytes of a K-contiguous operand, loaded
+// straight from memory (rows of one tile are read by the two waves beside each other; the
+// operands of block-scaled layers are a quarter to a half of an int8 layer's bytes).
+template <bool A4, bool B4>
+__global__ __launch_bounds__(256) void mx_gemm_kernel(mx_params p)
+{
+    if(*p.flag != 0)
+        return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wm   = wave >> 1, wn = wave & 1;
+    const int r    = lane & 15, g = lane >> 4;
+    const int bt   = blockIdx.z;
+    const int m0   = blockIdx.y * 128 + wm * 64;
+    const int n0   = blockIdx.x * 128 + wn * 64;
+    const uint8_t* a  = p.a + bt * p.stride_a;
+    const uint8_t* b  = p.b + bt * p.stride_b;
+    const uint8_t* ea = p.ea + (int64_t)bt * p.m * p.nblk;
+    const uint8_t* eb = p.eb + (int64_t)bt * p.n * p.nblk;
+
+    const uint8_t* arow[4];
+    const uint8_t* brow[4];
+    const uint8_t* earow[4];
+    const uint8_t* ebrow[4];
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+    {
+        const int row = min(m0 + i * 16 + r, p.m - 1);
+        const int col = min(n0 + i * 16 + r, p.n - 1);
+        arow[i]       = a + row * p.lda;
+        brow[i]       = b + col * p.ldb;
+        earow[i]      = ea + (int64_t)row * p.nblk;
+        ebrow[i]      = eb + (int64_t)col * p.nblk;
+    }
+    v4f32 acc[4][4];
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
+
+    // Operand registers of the instruction.  4-bit codes: lane group g holds K elements
+    // [32 g, 32 g + 32) of the step in four registers -- one scale block.  8-bit codes: the
+    // 128-deep instruction is laid out as two 64-deep halves, lane group g holding
+    // [16 g, 16 g + 16) in registers 0-3 and [64 + 16 g, 64 + 16 g + 16) in registers 4-7, while
+    // the scale a lane supplies is still that of block g, i.e. of K [32 g, 32 g + 32).
+    // Past the end of K: zeros, which add nothing whatever their scale.
+    auto fragment = [&](const uint8_t* row, int k0, auto packed) -> v8i {
+        v8i f = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr(decltype(packed)::value)
+        {
+            const int k = k0 + 32 * g;
+            if(k < p.k)
+            {
+                const v4i lo = *reinterpret_cast<const v4i*>(row + (k >> 1));
+                f            = v8i{lo.x, lo.y, lo.z, lo.w, 0, 0, 0, 0};
+            }
+        }
+        else
+        {
+            const int k = k0 + 16 * g;
+            v4i lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+            if(k < p.k)
+                lo = *reinterpret_cast<const v4i*>(row + k);
+            if(k + 64 < p.k)
+                hi = *reinterpret_cast<const v4i*>(row + k + 64);
+            f = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+        return f;
+    };
+
+    for(int k0 = 0; k0 < p.k; k0 += 128)
+    {
+        const int k   = k0 + 32 * g;
+        const int blk = min(k >> 5, p.nblk - 1);
+        v8i fa[4], fb[4];
+        int sa[4], sb[4];
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            fa[i] = fragment(arow[i], k0, std::integral_constant<bool, A4>{});
+            fb[i] = fragment(brow[i], k0, std::integral_constant<bool, B4>{});
+            sa[i] = earow[i][blk];
+            sb[i] = ebrow[i][blk];
+        }
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    fa[i], fb[j], acc[i][j], A4 ? 4 : 0, B4 ? 4 : 0, 0, sa[i], 0, sb[j]);
+    }
+    // element e of lane (r, g) of tile (i, j): row 16 i + 4 g + e, column 16 j + r
+    float* c = p.c + bt * p.stride_c;
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+        {
+            const int row = m0 + i * 16 + 4 * g + e;
+            if(row >= p.m)
+                continue;
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+                const int col = n0 + j * 16 + r;
+                if(col < p.n)
+                    c[(int64_t)row * p.ldc + col] = acc[i][j][e];
+            }
+        }
+}
+
+size_t align16(size_t x) { return (x + 15) / 16 * 16; }
+
+} // namespace
+
+extern "C" size_t mi355_quant_dot_mx_workspace_size(const mi355_mx_dot_desc* d)
+{
+    if(d == nullptr || d->m <= 0 || d->n <= 0 || d->k <= 0 || d->batch <= 0)
+        return 0;
+    const size_t nblk = (size_t)(d->k + 31) / 32;
+    return 16 + align16((size_t)d->batch * d->m * nblk) + align16((size_t)d->batch * d->n * nblk);
+}
+
+extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
+                                  const void* a,
+                                  const void* b,
+                                  float* c,
+                                  const float* scale_a,
+                                  const float* scale_b,
+                                  void* workspace,
+                                  size_t workspace_bytes,
+                                  void* stream)
+{
+    if(d == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if(d->m < 0 || d->n < 0 || d->k < 0 || d->batch < 0)
+        return MI355_ERR_BAD_ARG;
+    if((d->a_type != MI355_FP8 && d->a_type != MI355_FP4X2) || (d->b_type != MI355_FP8 && d->b_type != MI355_FP4X2))
+        return MI355_ERR_UNSUPPORTED;
+    if(d->m == 0 || d->n == 0 || d->batch == 0)
+        return MI355_OK;
+    if(a == nullptr || b == nullptr || c == nullptr || scale_a == nullptr || scale_b == nullptr || workspace == nullptr)
+        return MI355_ERR_BAD_ARG;
+    if(d->k == 0 || d->k % 32 != 0)
+        return MI355_ERR_UNSUPPORTED; // whole scale blocks only
+    const bool a4 = d->a_type == MI355_FP4X2, b4 = d->b_type == MI355_FP4X2;
+    const int64_t a_row = a4 ? d->k / 2 : d->k, b_row = b4 ? d->k / 2 : d->k;
+    if(d->lda < a_row || d->ldb < b_row || d->ldc < d->n)
+        return MI355_ERR_BAD_ARG;
+    // fragments are 16-byte loads
+    if(d->lda % 16 != 0 || d->ldb % 16 != 0 || d->stride_a % 16 != 0 || d->stride_b % 16 != 0 ||
+       reinterpret_cast<uintptr_t>(a) % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0 ||
+       reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return MI355_ERR_UNSUPPORTED;
+    if(d->m > (1 << 30) || d->n > (1 << 30) || d->k > (1 << 30) || d->batch > 65535 || (d->m + 15) / 16 > 65535)
+        return MI355_ERR_UNSUPPORTED;
+    if(workspace_bytes < mi355_quant_dot_mx_workspace_size(d))
+        return MI355_ERR_BAD_ARG;
+    mx_params p{};
+    p.a        = static_cast<const uint8_t*>(a);
+    p.b        = static_cast<const uint8_t*>(b);
+    p.c        = c;
+    p.scale_a  = scale_a;
+    p.scale_b  = scale_b;
+    p.m        = (int)d->m;
+    p.n        = (int)d->n;
+    p.k        = (int)d->k;
+    p.nblk     = (int)(d->k / 32);
+    p.lda      = d->lda;
+    p.ldb      = d->ldb;
+    p.ldc      = d->ldc;
+    p.stride_a = d->stride_a;
+    p.stride_b = d->stride_b;
+    p.stride_c = d->stride_c;
+    p.sa_batch = d->sa_batch;
+    p.sa_row   = d->sa_row;
+    p.sa_block = d->sa_block;
+    p.sa_elem  = d->sa_elem;
+    p.sb_batch = d->sb_batch;
+    p.sb_row   = d->sb_row;
+    p.sb_block = d->sb_block;
+    p.sb_elem  = d->sb_elem;
+    p.a4       = a4;
+    p.b4       = b4;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    p.flag      = reinterpret_cast<uint32_t*>(ws);
+    p.ea        = ws + 16;
+    p.eb        = p.ea + align16((size_t)d->batch * d->m * p.nblk);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(mx_clear_flag_kernel, dim3(1), dim3(1), 0, s, p.flag);
+    const int64_t most = (int64_t)d->batch * (d->m > d->n ? d->m : d->n) * p.nblk;
+    hipLaunchKernelGGL(mx_prepare_kernel, dim3((unsigned)((most + 255) / 256), 2), dim3(256), 0, s, p, (int)d->batch);
+    const dim3 grid((unsigned)((d->n + 127) / 128), (unsigned)((d->m + 127) / 128), (unsigned)d->batch);
+    if(a4 && b4)
+        hipLaunchKernelGGL((mx_gemm_kernel<true, true>), grid, dim3(256), 0, s, p);
+    else if(a4)
+        hipLaunchKernelGGL((mx_gemm_kernel<true, false>), grid, dim3(256), 0, s, p);
+    else if(b4)
+        hipLaunchKernelGGL((mx_gemm_kernel<false, true>), grid, dim3(256), 0, s, p);
+    else
+        hipLaunchKernelGGL((mx_gemm_kernel<false, false>), grid, dim3(256), 0, s, p);
+    const dim3 egrid((unsigned)((d->n + 15) / 16), (unsigned)((d->m + 15) / 16), (unsigned)d->batch);
+    hipLaunchKernelGGL(mx_exact_kernel, egrid, dim3(256), 0, s, p);
+    return mi355_launch_status();
+}

@@ -174,6 +174,33 @@ struct dot
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// The four-input quant_dot of block-scaled operands on the block-scaled matrix-core instruction.
+// inputs: a [.., M, K] fp8 codes or [.., M, K/2] fp4x2 (standard), b stored as [.., N, K] likewise,
+// scale_a, scale_b (float), workspace (uint8, mi355_quant_dot_mx_workspace_size), out float [.., M, N].
+// A scale is either a view with the operand's logical shape (scale_a [.., M, K], scale_b [.., K, N],
+// any strides: what the operator itself takes) or, with *_compact, a standard [.., rows, K/32] tensor
+// of one scale per block.
+struct quant_dot_mx
+{
+    bool a_fp4      = false;
+    bool b_fp4      = false;
+    bool sa_compact = false;
+    bool sb_compact = false;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.a_fp4, "a_fp4");
+        f(self.b_fp4, "b_fp4");
+        f(self.sa_compact, "sa_compact");
+        f(self.sb_compact, "sb_compact");
+    }
+    std::string name() const { return "mi355::quant_dot_mx"; }
+    mi355_mx_dot_desc describe(const std::vector<shape>& inputs) const;
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: a fp16 [M, K], packed weights uint8 [N, K/2], scales fp16 [N, K/group], [zero points], out
 struct w4a16_gemm
 {

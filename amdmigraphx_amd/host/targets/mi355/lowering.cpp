@@ -817,6 +817,137 @@ void fuse_chains(module& m)
     }
 }
 
+// ---- quant_dot(a, b, scale_a, scale_b): block-scaled operands ----------------------------------
+//
+// The four-input form simplify_qdq leaves for the MX formats (src/simplify_qdq.cpp:290-357) goes
+// to the block-scaled matrix-core kernel when both operands are fp8 e4m3fn tensors (what
+// unpack_fp4 yields) with whole blocks of 32 along K.  An operand that comes straight out of
+// unpack_fp4 along K is handed over still packed.  The kernel wants both operands K-contiguous:
+// a B that is the transpose view of [.., N, K] storage is used as it is, any other B is copied
+// into that layout.  The scales go in as the views they are (the kernel walks their strides and
+// finds out on the device whether they are per-block powers of two); a scale that is visibly one
+// value per block spread over 32 elements is passed in its compact form instead.
+
+// x = unpack_fp4 along the last axis of a standard tensor: the packed tensor, else x itself
+instruction_ref packed_fp4_source(instruction_ref x, bool& packed)
+{
+    packed = false;
+    if(x->name() != "unpack_fp4")
+        return x;
+    const auto axis = any_cast<op::unpack_fp4>(x->get_operator()).axis;
+    const auto nd   = static_cast<int64_t>(x->get_shape().ndim());
+    auto src        = x->inputs().front();
+    if((axis != -1 and axis != nd - 1) or not src->get_shape().standard())
+        return x;
+    packed = true;
+    return src;
+}
+
+bool swaps_last_two(instruction_ref t)
+{
+    if(t->name() != "transpose")
+        return false;
+    const auto perm = any_cast<op::transpose>(t->get_operator()).permutation;
+    const auto nd   = perm.size();
+    if(nd < 2 or perm[nd - 1] != static_cast<int64_t>(nd - 2) or perm[nd - 2] != static_cast<int64_t>(nd - 1))
+        return false;
+    for(std::size_t i = 0; i + 2 < nd; i++)
+        if(perm[i] != static_cast<int64_t>(i))
+            return false;
+    return true;
+}
+
+// s [.., rows, K] = reshape(multibroadcast{[.., rows, K/32, 32]}(unsqueeze(base [.., rows, K/32])))
+bool compact_block_scale(instruction_ref s, instruction_ref& base)
+{
+    if(s->name() != "reshape")
+        return false;
+    auto mb = s->inputs().front();
+    if(mb->name() != "multibroadcast")
+        return false;
+    auto us = mb->inputs().front();
+    if(us->name() != "unsqueeze")
+        return false;
+    base             = us->inputs().front();
+    const auto& bl   = base->get_shape().lens();
+    const auto& ml   = mb->get_shape().lens();
+    const auto& sl   = s->get_shape().lens();
+    if(not base->get_shape().standard() or base->get_shape().type() != shape::float_type)
+        return false;
+    if(ml.size() != bl.size() + 1 or sl.size() != bl.size() or ml.back() != 32)
+        return false;
+    for(std::size_t i = 0; i < bl.size(); i++)
+        if(ml[i] != bl[i])
+            return false;
+    for(std::size_t i = 0; i + 1 < bl.size(); i++)
+        if(sl[i] != bl[i])
+            return false;
+    return sl.back() == bl.back() * 32;
+}
+
+bool lower_mx_dot(module& m, instruction_ref ins)
+{
+    auto a  = ins->inputs()[0];
+    auto b  = ins->inputs()[1];
+    auto sa = ins->inputs()[2];
+    auto sb = ins->inputs()[3];
+    const auto& as = a->get_shape();
+    const auto& bs = b->get_shape();
+    const std::size_t nd = as.ndim();
+    if(as.type() != shape::fp8e4m3fn_type or bs.type() != shape::fp8e4m3fn_type or
+       ins->get_shape().type() != shape::float_type or sa->get_shape().type() != shape::float_type or
+       sb->get_shape().type() != shape::float_type)
+        return false;
+    const auto k = as.lens()[nd - 1];
+    if(nd < 2 or k == 0 or k % 32 != 0)
+        return false;
+    quant_dot_mx op;
+    // A
+    a = packed_fp4_source(a, op.a_fp4);
+    if(not a->get_shape().standard())
+        a = make_standard(m, ins, a);
+    // B as [.., N, K]
+    instruction_ref b_nk;
+    if(swaps_last_two(b))
+        b_nk = b->inputs().front();
+    else
+    {
+        std::vector<int64_t> perm(nd);
+        for(std::size_t i = 0; i < nd; i++)
+            perm[i] = static_cast<int64_t>(i);
+        std::swap(perm[nd - 1], perm[nd - 2]);
+        b_nk = m.insert_instruction(ins, make_op("transpose", {{"permutation", perm}}), b);
+    }
+    b_nk = packed_fp4_source(b_nk, op.b_fp4);
+    if(not b_nk->get_shape().standard())
+        b_nk = make_standard(m, ins, b_nk);
+    // scales: compact where the graph shows the block structure, else the view itself
+    instruction_ref base;
+    if(compact_block_scale(sa, base))
+    {
+        sa            = base;
+        op.sa_compact = true;
+    }
+    else if(not batch_collapses(sa->get_shape()))
+        sa = make_standard(m, ins, sa);
+    if(swaps_last_two(sb) and compact_block_scale(sb->inputs().front(), base))
+    {
+        sb            = base;
+        op.sb_compact = true;
+    }
+    else if(not batch_collapses(sb->get_shape()))
+        sb = make_standard(m, ins, sb);
+    auto out_lens   = ins->get_shape().lens();
+    auto out        = insert_allocation(m, ins, shape{shape::float_type, out_lens});
+    // the workspace size depends on the sizes only
+    std::vector<shape> probe = {a->get_shape(), b_nk->get_shape(), sa->get_shape(), sb->get_shape(),
+                                shape{shape::uint8_type, {16}}, out->get_shape()};
+    const auto d    = op.describe(probe);
+    auto ws         = insert_allocation(m, ins, shape{shape::uint8_type, {mi355_quant_dot_mx_workspace_size(&d)}});
+    m.replace_instruction(ins, operation{op}, {a, b_nk, sa, sb, ws, out});
+    return true;
+}
+
 // ---- one operator at a time ------------------------------------------------------------------
 
 void lower_instruction(module& m, instruction_ref ins)
@@ -828,7 +959,7 @@ void lower_instruction(module& m, instruction_ref ins)
     {
         if(ins->inputs().size() == 4)
         {
-            // The four-input form (operands with element-wise scales, as the MX block formats
+            // The four-input form the block-scaled kernel did not take (operands with element-wise scales, as the MX block formats
             // arrive after their scales are broadcast): float(a) * float(scale_a), the same for b,
             // then the float GEMM -- the three steps of ref_quant_gemm::compute
             // (src/targets/ref/lowering.cpp:221-242), each on its device kernel.
@@ -1080,6 +1211,8 @@ void lowering::apply(module& m) const
     {
         if(ins->name() == "dot")
             lower_w4a16(m, ins);
+        else if(ins->name() == "quant_dot" and ins->inputs().size() == 4)
+            lower_mx_dot(m, ins);
         else if(not fuse_quant_dot_dq(m, ins) and not fuse_quant_conv_dq(m, ins))
             fuse_dot_scale(m, ins);
     }

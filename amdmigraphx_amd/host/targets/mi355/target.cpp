@@ -483,6 +483,136 @@ argument rowsum::compute(migraphx::context& ctx, const shape&, const std::vector
     return args[1];
 }
 
+// ---- quant_dot_mx --------------------------------------------------------------------------
+
+mi355_mx_dot_desc quant_dot_mx::describe(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() != 6)
+        MIGRAPHX_THROW("mi355::quant_dot_mx: expects a, b, scale_a, scale_b, workspace, out");
+    const auto& a  = inputs[0];
+    const auto& b  = inputs[1];
+    const auto& sa = inputs[2];
+    const auto& sb = inputs[3];
+    const std::size_t nd = a.ndim();
+    if(nd < 2 or b.ndim() != nd or not a.standard() or not b.standard())
+        MIGRAPHX_THROW("mi355::quant_dot_mx: operands are standard tensors [.., M, K] and [.., N, K]");
+    auto storage_ok = [](const shape& s, bool fp4) {
+        return fp4 ? s.type() == shape::fp4x2_type : s.type() == shape::fp8e4m3fn_type;
+    };
+    if(not storage_ok(a, a_fp4) or not storage_ok(b, b_fp4))
+        MIGRAPHX_THROW("mi355::quant_dot_mx: operand types are fp8e4m3fn or fp4x2");
+    if(sa.type() != shape::float_type or sb.type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::quant_dot_mx: scales are float");
+    mi355_mx_dot_desc d{};
+    d.m     = static_cast<int64_t>(a.lens()[nd - 2]);
+    d.n     = static_cast<int64_t>(b.lens()[nd - 2]);
+    d.k     = static_cast<int64_t>(a.lens()[nd - 1]) * (a_fp4 ? 2 : 1);
+    d.batch = 1;
+    for(std::size_t i = 0; i + 2 < nd; i++)
+    {
+        if(a.lens()[i] != b.lens()[i])
+            MIGRAPHX_THROW("mi355::quant_dot_mx: outer dimensions of A and B mismatch");
+        d.batch *= static_cast<int64_t>(a.lens()[i]);
+    }
+    if(static_cast<int64_t>(b.lens()[nd - 1]) * (b_fp4 ? 2 : 1) != d.k)
+        MIGRAPHX_THROW("mi355::quant_dot_mx: inner dimensions are not compatible");
+    if(d.k % 32 != 0)
+        MIGRAPHX_THROW("mi355::quant_dot_mx: K must be whole blocks of 32");
+    d.lda      = static_cast<int64_t>(a.lens()[nd - 1]);
+    d.ldb      = static_cast<int64_t>(b.lens()[nd - 1]);
+    d.ldc      = d.n;
+    d.stride_a = d.m * d.lda;
+    d.stride_b = d.n * d.ldb;
+    d.stride_c = d.m * d.n;
+    d.a_type   = a_fp4 ? MI355_FP4X2 : MI355_FP8;
+    d.b_type   = b_fp4 ? MI355_FP4X2 : MI355_FP8;
+    // the one stride the batch dimensions of a view collapse into (0: no batch, or broadcast)
+    auto batch_stride = [&](const shape& s) {
+        int64_t r = 0;
+        for(std::size_t i = 0; i + 2 < s.ndim(); i++)
+        {
+            if(s.lens()[i] > 1)
+                r = static_cast<int64_t>(s.strides()[i]);
+        }
+        return r;
+    };
+    const auto nblk = d.k / 32;
+    auto check_scale = [&](const shape& s, bool compact, int64_t rows, bool transposed) {
+        if(s.ndim() != nd or not batch_collapses(s))
+            MIGRAPHX_THROW("mi355::quant_dot_mx: scale has the wrong rank or batch layout");
+        const auto r = static_cast<int64_t>(s.lens()[nd - 2]);
+        const auto c = static_cast<int64_t>(s.lens()[nd - 1]);
+        const bool ok = compact ? (s.standard() and r == rows and c == nblk)
+                                : (transposed ? (r == d.k and c == rows) : (r == rows and c == d.k));
+        if(not ok)
+            MIGRAPHX_THROW("mi355::quant_dot_mx: scale has the wrong shape");
+    };
+    check_scale(sa, sa_compact, d.m, false);
+    check_scale(sb, sb_compact, d.n, true);
+    if(sa_compact)
+    {
+        d.sa_batch = d.m * nblk;
+        d.sa_row   = nblk;
+        d.sa_block = 1;
+        d.sa_elem  = 0;
+    }
+    else
+    {
+        d.sa_batch = batch_stride(sa);
+        d.sa_row   = static_cast<int64_t>(sa.strides()[nd - 2]);
+        d.sa_elem  = static_cast<int64_t>(sa.strides()[nd - 1]);
+        d.sa_block = 32 * d.sa_elem;
+    }
+    if(sb_compact)
+    {
+        d.sb_batch = d.n * nblk;
+        d.sb_row   = nblk;
+        d.sb_block = 1;
+        d.sb_elem  = 0;
+    }
+    else
+    {
+        // scale_b has the operator's [.., K, N] shape
+        d.sb_batch = batch_stride(sb);
+        d.sb_elem  = static_cast<int64_t>(sb.strides()[nd - 2]);
+        d.sb_row   = static_cast<int64_t>(sb.strides()[nd - 1]);
+        d.sb_block = 32 * d.sb_elem;
+    }
+    return d;
+}
+
+shape quant_dot_mx::compute_shape(const std::vector<shape>& inputs) const
+{
+    const auto d = describe(inputs);
+    auto lens    = inputs[0].lens();
+    lens.back()  = static_cast<std::size_t>(d.n);
+    shape out{shape::float_type, lens};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::quant_dot_mx: output buffer has the wrong shape");
+    if(inputs[4].bytes() < mi355_quant_dot_mx_workspace_size(&d))
+        MIGRAPHX_THROW("mi355::quant_dot_mx: workspace is too small");
+    return out;
+}
+
+argument quant_dot_mx::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    std::vector<shape> shapes;
+    for(const auto& a : args)
+        shapes.push_back(a.get_shape());
+    const auto d = describe(shapes);
+    status_check(mi355_quant_dot_mx(&d,
+                                    args[0].data(),
+                                    args[1].data(),
+                                    reinterpret_cast<float*>(args[5].data()),
+                                    reinterpret_cast<const float*>(args[2].data()),
+                                    reinterpret_cast<const float*>(args[3].data()),
+                                    args[4].data(),
+                                    args[4].get_shape().bytes(),
+                                    stream_of(ctx)),
+                 name());
+    return args[5];
+}
+
 shape dot::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, scaled ? 4 : 3, name());
@@ -1132,6 +1262,7 @@ MIGRAPHX_REGISTER_OP(mi355::quant_convolution);
 MIGRAPHX_REGISTER_OP(mi355::colsum);
 MIGRAPHX_REGISTER_OP(mi355::rowsum);
 MIGRAPHX_REGISTER_OP(mi355::dot);
+MIGRAPHX_REGISTER_OP(mi355::quant_dot_mx);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
 MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);

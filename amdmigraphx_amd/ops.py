@@ -11,7 +11,7 @@ import ctypes
 
 import torch
 
-from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConvDesc, Mi355Error, check, lib
+from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConvDesc, MxDotDesc, Mi355Error, check, lib
 
 _TORCH2DT = {torch.int8: DT.I8, torch.uint8: DT.U8, torch.int32: DT.I32, torch.float32: DT.F32,
              torch.float16: DT.F16, torch.bfloat16: DT.BF16}
@@ -138,6 +138,55 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
         st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
                                    _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
         check(st, "mi355_quant_dot")
+    return out
+
+
+def quant_dot_mx(a, b_nk, scale_a, scale_b, a_fp4=False, b_fp4=False, out=None):
+    """Four-input quant_dot of block-scaled operands: C = (float(A) * SA) . (float(B) * SB)^T.
+
+    ``a`` [..., M, K] and ``b_nk`` [..., N, K] are uint8 tensors of e4m3fn codes, or with
+    ``a_fp4`` / ``b_fp4`` of packed e2m1 pairs ([..., M, K/2], low nibble = even k).  The scales are
+    float32, either of the operand's logical shape ([..., M, K], the operator's form) or compact
+    ([..., M, K/32], one per block).  Returns float32 [..., M, N]."""
+    _require_cuda(a, b_nk, scale_a, scale_b)
+    if a.dtype != torch.uint8 or b_nk.dtype != torch.uint8:
+        raise Mi355Error("quant_dot_mx: operands are uint8 tensors of fp8 codes or packed fp4 pairs")
+    a, b_nk = a.contiguous(), b_nk.contiguous()
+    scale_a, scale_b = scale_a.contiguous(), scale_b.contiguous()
+    batch_shape = a.shape[:-2]
+    if b_nk.shape[:-2] != batch_shape:
+        raise Mi355Error("QUANT_DOT: outer dimensions of A and B mismatch")
+    m, n = a.shape[-2], b_nk.shape[-2]
+    k = a.shape[-1] * (2 if a_fp4 else 1)
+    if b_nk.shape[-1] * (2 if b_fp4 else 1) != k:
+        raise Mi355Error("QUANT_DOT: inner dimensions are not compatible")
+    nb = 1
+    for v in batch_shape:
+        nb *= v
+
+    def scale_strides(sc, rows):
+        if sc.dtype != torch.float32 or sc.shape[:-1] != batch_shape + (rows,):
+            raise Mi355Error("quant_dot_mx: scales must be float32 of the operand's shape or [rows, K/32]")
+        cols = sc.shape[-1]
+        if cols == k:
+            return rows * k, k, 32, 1
+        if cols * 32 == k:
+            return rows * cols, cols, 1, 0
+        raise Mi355Error("quant_dot_mx: scales must have K or K/32 columns")
+
+    sab, sar, sak, sae = scale_strides(scale_a, m)
+    sbb, sbr, sbk, sbe = scale_strides(scale_b, n)
+    if out is None:
+        out = torch.empty(batch_shape + (m, n), dtype=torch.float32, device=a.device)
+    d = MxDotDesc(m=m, n=n, k=k, batch=nb, lda=a.shape[-1], ldb=b_nk.shape[-1], ldc=n,
+                  stride_a=m * a.shape[-1], stride_b=n * b_nk.shape[-1], stride_c=m * n,
+                  sa_batch=sab, sa_row=sar, sa_block=sak, sa_elem=sae,
+                  sb_batch=sbb, sb_row=sbr, sb_block=sbk, sb_elem=sbe,
+                  a_type=DT.FP4X2 if a_fp4 else DT.FP8, b_type=DT.FP4X2 if b_fp4 else DT.FP8)
+    need = int(lib().mi355_quant_dot_mx_workspace_size(ctypes.byref(d)))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=a.device)
+    check(lib().mi355_quant_dot_mx(ctypes.byref(d), _ptr(a), _ptr(b_nk), _ptr(out), _ptr(scale_a), _ptr(scale_b),
+                                   _ptr(ws), need, _stream()), "mi355_quant_dot_mx")
     return out
 
 

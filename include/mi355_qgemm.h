@@ -40,7 +40,8 @@ typedef enum mi355_dtype {
     MI355_F32  = 3,
     MI355_F16  = 4, /* IEEE binary16 */
     MI355_BF16 = 5,
-    MI355_FP8  = 6  /* OCP e4m3fn */
+    MI355_FP8  = 6, /* OCP e4m3fn */
+    MI355_FP4X2 = 7 /* two OCP e2m1 codes per byte, low nibble = even element (block-scaled operands) */
 } mi355_dtype;
 
 /* How a quantization parameter is broadcast over an [M, N] result. */
@@ -194,6 +195,42 @@ int mi355_quant_dot_ws(const mi355_quant_dot_desc* desc, const void* a, const vo
 int mi355_quant_dot_static(const mi355_quant_dot_desc* desc, const void* a, const void* b, void* c,
                            const float* scale_a, const float* scale_b, const int32_t* colsum_b,
                            const int32_t* rowsum_a, const float* bias, void* stream);
+
+/*
+ * quant_dot with element-wise scales, the MX block formats' form:
+ *   C[b, m, n] = float( sum_k double(float(A[b,m,k]) * SA[b,m,k]) * double(float(B[b,k,n]) * SB[b,k,n]) )
+ *
+ * Replaces: ref_quant_gemm::compute with four inputs (src/targets/ref/lowering.cpp:221-242:
+ * float(a) * scale_a and float(b) * scale_b element by element in float, then gemm_naive,
+ * src/gemm.cpp:42-63), which is what simplify_qdq.cpp:290-357 leaves of
+ * unpack_fp4 -> dequantizelinear -> dot for block-quantized operands.
+ *
+ * A is [batch, M, K] and B is given as [batch, N, K] (K contiguous for both: the transpose view
+ * the operator sees as [K, N]); each either one e4m3fn code per element (MI355_FP8) or two e2m1
+ * codes per byte along K (MI355_FP4X2, what unpack_fp4 reads); lda / ldb / stride_a / stride_b count
+ * BYTES of the stored operand.  C is float, row-major.  The scales are float tensors addressed as
+ *   SA(b, m, k) = scale_a[b * sa_batch + m * sa_row + (k / 32) * sa_block + (k % 32) * sa_elem]
+ * (element strides), so the operator's full-size scale tensor is (M*K, K, 32, 1) and a compact
+ * [M, K/32] tensor of block scales is (M*K/32, K/32, 1, 0); likewise SB(b, n, k).
+ * Where every block of 32 scales along K is one positive normal power of two (what the MX formats
+ * store as e8m0) the product runs on v_mfma_scale_f32_16x16x128_f8f6f4 with the scales as the
+ * instruction's block-scale operands; any other scale values are detected on the device and the
+ * call then evaluates the formula above as written (slowly).  K must be a multiple of 32, rows
+ * 16-byte aligned.  workspace: mi355_quant_dot_mx_workspace_size bytes of device memory, 16-byte
+ * aligned, free again when the call's work is done.
+ */
+typedef struct mi355_mx_dot_desc {
+    int64_t m, n, k, batch;
+    int64_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;
+    int64_t sa_batch, sa_row, sa_block, sa_elem;
+    int64_t sb_batch, sb_row, sb_block, sb_elem;
+    int32_t a_type, b_type; /* MI355_FP8 or MI355_FP4X2 */
+} mi355_mx_dot_desc;
+size_t mi355_quant_dot_mx_workspace_size(const mi355_mx_dot_desc* desc);
+int mi355_quant_dot_mx(const mi355_mx_dot_desc* desc, const void* a, const void* b, float* c,
+                       const float* scale_a, const float* scale_b, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* int32 column sums of an int8 [K, N] matrix (same addressing as B above,
  * batch 1): out[n] = sum_k B[k, n].  Equals quant_dot(ones[1,K], B), the

@@ -45,6 +45,32 @@ static void expect_same(const program& p, const migraphx::parameter_map& params)
         EXPECT(same_bytes(got2[i], want[i]));
 }
 
+// The fp8 / block-scaled matrix-core instructions accumulate in fp32 where the CPU target holds the
+// exact sum: the device result must stay within 1e-3 of the output's RMS, no element off by more
+// than 2^-8 of the largest output.
+static void expect_close_rms(const program& p, const migraphx::parameter_map& params)
+{
+    auto want_all = run_on("oracle", p, params);
+    auto got_all  = run_on("mi355", p, params);
+    EXPECT(want_all.size() == got_all.size());
+    for(std::size_t o = 0; o < want_all.size(); o++)
+    {
+        auto want = want_all[o].to_vector<double>();
+        auto got  = got_all[o].to_vector<double>();
+        EXPECT(want.size() == got.size());
+        double num = 0, den = 0, peak = 0, worst = 0;
+        for(std::size_t i = 0; i < want.size(); i++)
+        {
+            num += (got[i] - want[i]) * (got[i] - want[i]);
+            den += want[i] * want[i];
+            peak  = std::max(peak, std::fabs(want[i]));
+            worst = std::max(worst, std::fabs(got[i] - want[i]));
+        }
+        EXPECT(std::sqrt(num / den) < 1e-3);
+        EXPECT(worst <= peak / 256);
+    }
+}
+
 // The int4 kernel dequantizes every weight exactly as the reference does but accumulates the
 // dot product in fp32 (v_dot2_f32_f16 partial sums, then a wavefront reduction) where the reference
 // accumulates in double: outputs may differ by the last half-precision bit.  Allowed: one fp16
@@ -453,7 +479,9 @@ TEST_CASE(quant_dot_four_inputs)
     }
     // fp8 operands with one power-of-two scale per block of 32 along K (the MX arrangement, scales
     // already spread over the elements), batched; A's scales arrive as a dense tensor, B's as a
-    // broadcast view of one row
+    // broadcast view of one row.  B is row-major [K, N]: the lowering copies it into the
+    // K-contiguous layout the block-scaled kernel reads.  The codes span the whole e4m3 range, so
+    // the fp32 accumulation of the instruction shows: the fp8 tolerance, not bit equality.
     {
         const std::size_t bt = 2, m = 48, k = 64, n = 40;
         program p;
@@ -490,13 +518,14 @@ TEST_CASE(quant_dot_four_inputs)
         const auto cb = codes(sb.elements(), 72);
         std::memcpy(aa.data(), ca.data(), ca.size());
         std::memcpy(ba.data(), cb.data(), cb.size());
+        expect_close_rms(p, {{"a", aa}, {"b", ba}, {"sa", argument{ssa, sav}}, {"sb", argument{ssb, sbv}}});
+        // a scale that is no power of two: the same graph, now bit for bit (exact path on the device)
+        sbv[3] = 0.75f;
         expect_same(p, {{"a", aa}, {"b", ba}, {"sa", argument{ssa, sav}}, {"sb", argument{ssb, sbv}}});
         program c = p;
         c.compile(migraphx::make_target("mi355"));
-        EXPECT(count_ops(*c.get_main_module(), "mi355::dot") == 1);
-        EXPECT(count_ops(*c.get_main_module(), "mi355::convert") == 2);
-        EXPECT(count_ops(*c.get_main_module(), "mi355::binary") == 2);
-        EXPECT(not has_op(c, "quant_dot"));
+        EXPECT(count_ops(*c.get_main_module(), "mi355::quant_dot_mx") == 1);
+        EXPECT(not has_op(c, "quant_dot") and not has_op(c, "mi355::dot"));
     }
 }
 
@@ -504,8 +533,12 @@ TEST_CASE(mx_fp4_matmul)
 {
     // MX fp4: packed e2m1 operands, one power-of-two scale per 32 elements along K, as a graph of
     // unpack_fp4 -> dequantizelinear -> dot (test/simplify_qdq_test.cpp:1776-1860).  The target's
-    // simplify_qdq turns it into the four-input quant_dot; the result equals the CPU target's bit
-    // for bit (every product float(a) * scale is exact).
+    // simplify_qdq turns it into the four-input quant_dot, which runs on the block-scaled
+    // matrix-core kernel with the operands still packed.  Every product float(a) * scale is exact,
+    // so the CPU target's result is the exact sum rounded once; the instruction accumulates in
+    // fp32 (the tolerance of the fp8 quant_dot: 1e-3 of the output's RMS here, no element off by
+    // more than 2^-8 of the largest).  With scales close together every partial sum is exact and
+    // the results are the same bits.
     const std::size_t bt = 2, m = 40, k = 96, n = 24;
     shape pa{shape::fp4x2_type, {bt, m, k / 2}};
     shape pb{shape::fp4x2_type, {bt, n, k / 2}};
@@ -531,21 +564,78 @@ TEST_CASE(mx_fp4_matmul)
     const auto cb = uniform_ints<uint8_t>(pb.elements(), 0, 255, 42);
     std::memcpy(aa.data(), ca.data(), ca.size());
     std::memcpy(ba.data(), cb.data(), cb.size());
-    auto block_scales = [](std::size_t rows, std::size_t kk, unsigned seed) {
-        auto e = uniform_ints<int>(rows * (kk / 32), -5, 5, seed);
+    auto block_scales = [](std::size_t rows, std::size_t kk, int spread, unsigned seed) {
+        auto e = uniform_ints<int>(rows * (kk / 32), -spread, spread, seed);
         std::vector<float> v(rows * kk);
         for(std::size_t i = 0; i < v.size(); i++)
             v[i] = std::ldexp(1.0f, e[i / 32]);
         return v;
     };
-    migraphx::parameter_map params = {{"a", aa}, {"b", ba}, {"sa", argument{sa, block_scales(bt * m, k, 43)}},
-                                      {"sb", argument{sb, block_scales(bt * n, k, 44)}}};
-    expect_same(p, params);
+    for(int spread : {1, 5})
+    {
+        migraphx::parameter_map params = {{"a", aa}, {"b", ba}, {"sa", argument{sa, block_scales(bt * m, k, spread, 43)}},
+                                          {"sb", argument{sb, block_scales(bt * n, k, spread, 44)}}};
+        if(spread == 1)
+        {
+            expect_same(p, params);
+            continue;
+        }
+        expect_close_rms(p, params);
+    }
+    // scales that are no powers of two: found on the device, evaluated as the operator is written
+    {
+        auto v1 = uniform_floats(sa.elements(), 0.25f, 2.0f, 46);
+        auto v2 = uniform_floats(sb.elements(), 0.25f, 2.0f, 47);
+        expect_same(p, {{"a", aa}, {"b", ba}, {"sa", argument{sa, v1}}, {"sb", argument{sb, v2}}});
+    }
     program c = p;
     c.compile(migraphx::make_target("mi355"));
-    EXPECT(count_ops(*c.get_main_module(), "mi355::unpack_fp4") == 2);
-    EXPECT(count_ops(*c.get_main_module(), "mi355::dot") == 1);
+    EXPECT(count_ops(*c.get_main_module(), "mi355::quant_dot_mx") == 1);
+    EXPECT(not has_op(c, "mi355::unpack_fp4") and not has_op(c, "mi355::dot"));
     EXPECT(not has_op(c, "dequantizelinear") and not has_op(c, "mi355::dequantizelinear"));
+    // block scales that the graph spreads itself (one value per block, unsqueeze -> multibroadcast
+    // -> reshape): the kernel gets the compact tensors
+    program q;
+    {
+        auto* mm = q.get_main_module();
+        auto a   = mm->add_parameter("a", pa);
+        auto b   = mm->add_parameter("b", pb);
+        auto s1  = mm->add_parameter("sa", shape{shape::float_type, {bt, m, k / 32}});
+        auto s2  = mm->add_parameter("sb", shape{shape::float_type, {bt, n, k / 32}});
+        auto spread32 = [&](instruction_ref x, std::size_t rows) {
+            auto u  = mm->add_instruction(make_op("unsqueeze", {{"axes", {3}}}), x);
+            auto mb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {bt, rows, k / 32, std::size_t{32}}}}), u);
+            return mm->add_instruction(make_op("reshape", {{"dims", {static_cast<int64_t>(bt), static_cast<int64_t>(rows), static_cast<int64_t>(k)}}}), mb);
+        };
+        auto ua = mm->add_instruction(make_op("unpack_fp4"), a);
+        auto ub = mm->add_instruction(make_op("unpack_fp4"), b);
+        auto da = mm->add_instruction(make_op("dequantizelinear"), ua, spread32(s1, m));
+        auto db = mm->add_instruction(make_op("dequantizelinear"), ub, spread32(s2, n));
+        auto tb = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1}}}), db);
+        mm->add_return({mm->add_instruction(make_op("dot"), da, tb)});
+    }
+    {
+        auto compact = [](std::size_t count, unsigned seed) {
+            auto e = uniform_ints<int>(count, -1, 1, seed);
+            std::vector<float> v(count);
+            for(std::size_t i = 0; i < count; i++)
+                v[i] = std::ldexp(1.0f, e[i]);
+            return v;
+        };
+        shape c1{shape::float_type, {bt, m, k / 32}};
+        shape c2{shape::float_type, {bt, n, k / 32}};
+        expect_same(q, {{"a", aa}, {"b", ba}, {"sa", argument{c1, compact(c1.elements(), 48)}},
+                        {"sb", argument{c2, compact(c2.elements(), 49)}}});
+        program qc = q;
+        qc.compile(migraphx::make_target("mi355"));
+        for(auto ins = qc.get_main_module()->begin(); ins != qc.get_main_module()->end(); ++ins)
+            if(ins->name() == "mi355::quant_dot_mx")
+            {
+                EXPECT(ins->get_operator().to_value().at("sa_compact").to<bool>());
+                EXPECT(ins->get_operator().to_value().at("sb_compact").to<bool>());
+            }
+        EXPECT(count_ops(*qc.get_main_module(), "mi355::quant_dot_mx") == 1);
+    }
     // pack_fp4 on the device: float -> fp4x2 -> fp8, against the CPU target
     program r;
     {
