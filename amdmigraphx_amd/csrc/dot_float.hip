@@ -8,6 +8,7 @@
 // double, so the fused multiply-add used here rounds exactly as the reference's separate multiply
 // and add do.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -139,12 +140,17 @@ __global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
 // the matrix instructions.  A_KCONT: A's K stride is 1 (else its row stride is 1); B_NCONT: B's
 // column stride is 1 (else its K stride is 1).  The host checks the alignment the vector loads need;
 // a vector that would cross the matrix edge is read element by element with zero fill.
-template <bool A_KCONT, bool B_NCONT>
+// FP32ACC: the sums run on the fp32 matrix cores instead (v_mfma_f32_16x16x4_f32, twice the rate):
+// fp32 products and fp32 accumulation, no longer the bits of the reference's double sum but within
+// K * 2^-24 of sum|a||b| of them.  Register r of lane l then holds D[4 * (l / 16) + r][l % 16].
+template <bool A_KCONT, bool B_NCONT, bool FP32ACC = false>
 __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
 {
     constexpr int PITCH = 80;
-    __shared__ double as[16][PITCH];
-    __shared__ double bs[16][PITCH];
+    using stage_t = std::conditional_t<FP32ACC, float, double>;
+    using acc_t   = std::conditional_t<FP32ACC, v4f, v4d>;
+    __shared__ stage_t as[16][PITCH];
+    __shared__ stage_t bs[16][PITCH];
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -200,12 +206,12 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
         return v;
     };
 
-    v4d acc[2][2];
+    acc_t acc[2][2];
 #pragma unroll
     for(int i = 0; i < 2; i++)
 #pragma unroll
         for(int j = 0; j < 2; j++)
-            acc[i][j] = v4d{0.0, 0.0, 0.0, 0.0};
+            acc[i][j] = acc_t{0, 0, 0, 0};
 
     // x * 1.0f is x for every float, so "no scale" needs no second code path
     const float alpha = p.scale != nullptr ? p.scale[0] : 1.0f;
@@ -217,13 +223,13 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
         for(int e = 0; e < 4; e++)
         {
             if(A_KCONT)
-                as[a_minor + e][a_major] = (double)va[e];
+                as[a_minor + e][a_major] = (stage_t)va[e];
             else
-                as[a_major][a_minor + e] = (double)va[e];
+                as[a_major][a_minor + e] = (stage_t)va[e];
             if(B_NCONT)
-                bs[b_major][b_minor + e] = (double)vb[e];
+                bs[b_major][b_minor + e] = (stage_t)vb[e];
             else
-                bs[b_minor + e][b_major] = (double)vb[e];
+                bs[b_minor + e][b_major] = (stage_t)vb[e];
         }
         __syncthreads();
         if(k0 + 16 < p.k)
@@ -234,7 +240,7 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
 #pragma unroll
         for(int kk0 = 0; kk0 < 16; kk0 += 4)
         {
-            double av[2], bv[2];
+            stage_t av[2], bv[2];
 #pragma unroll
             for(int i = 0; i < 2; i++)
                 av[i] = as[kk0 + lk][wm * 32 + i * 16 + l16];
@@ -245,7 +251,12 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
             for(int i = 0; i < 2; i++)
 #pragma unroll
                 for(int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
+                {
+                    if constexpr(FP32ACC)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
+                }
         }
         __syncthreads();
     }
@@ -254,7 +265,7 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
 #pragma unroll
         for(int r = 0; r < 4; r++)
         {
-            const int64_t row = row0 + wm * 32 + i * 16 + 4 * r + lk;
+            const int64_t row = row0 + wm * 32 + i * 16 + (FP32ACC ? 4 * lk + r : 4 * r + lk);
             if(row >= p.m)
                 continue;
 #pragma unroll
@@ -352,7 +363,8 @@ extern "C" int mi355_dot(const void* a,
                             stride_a, stride_b, stride_c, nullptr, stream);
 }
 
-extern "C" int mi355_dot_scaled(const void* a,
+static int dot_launch(bool fp32acc,
+                      const void* a,
                                 const void* b,
                                 void* c,
                                 int32_t type,
@@ -373,7 +385,7 @@ extern "C" int mi355_dot_scaled(const void* a,
 {
     if(type != MI355_F32 && type != MI355_F16 && type != MI355_BF16)
         return MI355_ERR_BAD_ARG;
-    if(scale != nullptr && type != MI355_F32)
+    if((scale != nullptr || fp32acc) && type != MI355_F32)
         return MI355_ERR_UNSUPPORTED;
     if(m < 0 || n < 0 || k < 0 || batch < 0 || a_stride_m < 0 || a_stride_k < 0 || b_stride_k < 0 ||
        b_stride_n < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0 || ldc < n)
@@ -398,6 +410,18 @@ extern "C" int mi355_dot_scaled(const void* a,
     if(type == MI355_F32 && k > 0 && (a_k || a_m) && (b_n || b_k) && aligned4(stride_a) && aligned4(stride_b) &&
        reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0)
     {
+        if(fp32acc)
+        {
+            if(a_k && b_n)
+                hipLaunchKernelGGL((dot_f32_mfma_kernel<true, true, true>), grid, dim3(256), 0, s, p);
+            else if(a_k)
+                hipLaunchKernelGGL((dot_f32_mfma_kernel<true, false, true>), grid, dim3(256), 0, s, p);
+            else if(b_n)
+                hipLaunchKernelGGL((dot_f32_mfma_kernel<false, true, true>), grid, dim3(256), 0, s, p);
+            else
+                hipLaunchKernelGGL((dot_f32_mfma_kernel<false, false, true>), grid, dim3(256), 0, s, p);
+            return mi355_launch_status();
+        }
         if(a_k && b_n)
             hipLaunchKernelGGL((dot_f32_mfma_kernel<true, true>), grid, dim3(256), 0, s, p);
         else if(a_k)
@@ -410,6 +434,52 @@ extern "C" int mi355_dot_scaled(const void* a,
     }
     hipLaunchKernelGGL(dot_float_mfma_kernel, grid, dim3(256), 0, s, p);
     return mi355_launch_status();
+}
+
+extern "C" int mi355_dot_scaled(const void* a,
+                                const void* b,
+                                void* c,
+                                int32_t type,
+                                int64_t m,
+                                int64_t n,
+                                int64_t k,
+                                int64_t a_stride_m,
+                                int64_t a_stride_k,
+                                int64_t b_stride_k,
+                                int64_t b_stride_n,
+                                int64_t ldc,
+                                int64_t batch,
+                                int64_t stride_a,
+                                int64_t stride_b,
+                                int64_t stride_c,
+                                const float* scale,
+                                void* stream)
+{
+    return dot_launch(false, a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc, batch,
+                      stride_a, stride_b, stride_c, scale, stream);
+}
+
+extern "C" int mi355_dot_fp32acc(const void* a,
+                                 const void* b,
+                                 void* c,
+                                 int32_t type,
+                                 int64_t m,
+                                 int64_t n,
+                                 int64_t k,
+                                 int64_t a_stride_m,
+                                 int64_t a_stride_k,
+                                 int64_t b_stride_k,
+                                 int64_t b_stride_n,
+                                 int64_t ldc,
+                                 int64_t batch,
+                                 int64_t stride_a,
+                                 int64_t stride_b,
+                                 int64_t stride_c,
+                                 const float* scale,
+                                 void* stream)
+{
+    return dot_launch(true, a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc, batch,
+                      stride_a, stride_b, stride_c, scale, stream);
 }
 
 extern "C" int mi355_contiguous(const void* in,

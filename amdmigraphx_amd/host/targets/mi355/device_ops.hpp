@@ -162,11 +162,13 @@ struct rowsum
 // (with `scaled`: a, b, scale (one float), out -- the result times that value, fp32 only)
 struct dot
 {
-    bool scaled = false;
+    bool scaled  = false;
+    bool fp32acc = false; // fp32 matrix cores: faster, within fp32 accumulation error of the exact sum
     template <class Self, class F>
     static void reflect(Self& self, F f)
     {
         f(self.scaled, "scaled");
+        f(self.fp32acc, "fp32acc");
     }
     std::string name() const { return "mi355::dot"; }
     shape compute_shape(const std::vector<shape>& inputs) const;

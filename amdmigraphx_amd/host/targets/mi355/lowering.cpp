@@ -1,3 +1,4 @@
+#include <cstdlib>
 #include "device_ops.hpp"
 #include <migraphx/ops.hpp>
 #include <migraphx/passes.hpp>
@@ -566,6 +567,14 @@ bool lower_w4a16(module& m, instruction_ref ins)
     return true;
 }
 
+// MIGRAPHX_MI355_FP32_DOT set (to anything but 0) when a program is compiled: float `dot`s run on
+// the fp32 matrix cores instead of reproducing the reference's double sum bit for bit
+bool fp32_dot_requested()
+{
+    const char* v = std::getenv("MIGRAPHX_MI355_FP32_DOT");
+    return v != nullptr and std::string(v) != "0" and std::string(v) != "";
+}
+
 // ---- dot -> mul by one value (attention scores) -------------------------------------------------
 // The multiplication joins the dot's store: float(sum) * value, the two roundings the two
 // operators perform.
@@ -590,8 +599,9 @@ bool fuse_dot_scale(module& m, instruction_ref mul)
         if(not batch_collapses(b->get_shape()))
             b = make_standard(m, mul, b);
         dot op;
-        op.scaled = true;
-        auto out  = insert_allocation(m, mul, shape{shape::float_type, d->get_shape().lens()});
+        op.scaled  = true;
+        op.fp32acc = fp32_dot_requested();
+        auto out   = insert_allocation(m, mul, shape{shape::float_type, d->get_shape().lens()});
         m.replace_instruction(mul, operation{op}, {a, b, base, out});
         return true;
     }
@@ -1013,7 +1023,9 @@ void lower_instruction(module& m, instruction_ref ins)
             a = make_standard(m, ins, a);
         if(not batch_collapses(b->get_shape()))
             b = make_standard(m, ins, b);
-        m.replace_instruction(ins, operation{dot{}}, a, b, standard_out());
+        dot op;
+        op.fp32acc = fp32_dot_requested() and ins->get_shape().type() == shape::float_type;
+        m.replace_instruction(ins, operation{op}, a, b, standard_out());
     }
     else if(name == "quantizelinear" or name == "dequantizelinear")
     {

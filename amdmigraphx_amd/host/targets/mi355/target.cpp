@@ -654,7 +654,8 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
         }
         return r;
     };
-    status_check(mi355_dot_scaled(args[0].data(),
+    const bool fast = fp32acc and out.type() == shape::float_type;
+    status_check((fast ? mi355_dot_fp32acc : mi355_dot_scaled)(args[0].data(),
                            args[1].data(),
                            args.back().data(),
                            to_mi355_type(out.type()),

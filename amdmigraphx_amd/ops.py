@@ -190,6 +190,31 @@ def quant_dot_mx(a, b_nk, scale_a, scale_b, a_fp4=False, b_fp4=False, out=None):
     return out
 
 
+def dot(a, b, scale=None, fp32acc=False):
+    """Float `dot` of float32 / float16 / bfloat16 tensors [..., M, K] . [..., K, N] (any strides
+    inside a matrix, batches dense).  By default the reference's double sum bit for bit; with
+    ``fp32acc`` (float32 only) on the fp32 matrix cores.  ``scale``: one float32 the result is
+    multiplied by."""
+    _require_cuda(a, b, scale)
+    if a.dtype != b.dtype or a.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise Mi355Error("dot: float32, float16 or bfloat16 operands of one type")
+    if a.dim() != b.dim() or a.dim() < 2 or a.shape[:-2] != b.shape[:-2] or a.shape[-1] != b.shape[-2]:
+        raise Mi355Error("DOT: operands do not fit")
+    m, k = a.shape[-2:]
+    n = b.shape[-1]
+    nb = 1
+    for v in a.shape[:-2]:
+        nb *= v
+    a3 = a.reshape((nb, m, k)) if a.dim() != 3 else a
+    b3 = b.reshape((nb, k, n)) if b.dim() != 3 else b
+    out = torch.empty(a.shape[:-2] + (m, n), dtype=a.dtype, device=a.device)
+    fn = lib().mi355_dot_fp32acc if fp32acc else lib().mi355_dot_scaled
+    check(fn(_ptr(a3), _ptr(b3), _ptr(out), _TORCH2DT[a.dtype], m, n, k, a3.stride(1), a3.stride(2),
+             b3.stride(1), b3.stride(2), n, nb, a3.stride(0) if nb > 1 else 0, b3.stride(0) if nb > 1 else 0,
+             m * n, _ptr(scale), _stream()), "mi355_dot")
+    return out
+
+
 def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False, fp8=False):
     """Bytes of workspace an int8 (or fp8) quant_dot of that shape can use (0: none)."""
     d = QuantDotDesc(m=m, n=n, k=k, batch=batch, lda=k, ldb=k if trans_b else n, ldc=n,

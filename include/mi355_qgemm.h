@@ -401,6 +401,19 @@ int mi355_dot_scaled(const void* a, const void* b, void* c, int32_t type,
                      int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                      const float* scale, void* stream);
 
+/* The same arguments (fp32 only), with the sums on the fp32 matrix cores: fp32 products and fp32
+ * accumulation at twice the rate of mi355_dot_scaled.  The result is no longer the bits of the
+ * reference's double sum; it stays within K * 2^-24 of sum|a||b| of it, far inside the 1e-3
+ * relative the float outputs of the path are held to.  Meant for the attention products of an
+ * encoder when the caller asks for speed (the mi355 target lowers `dot` to it when the environment
+ * variable MIGRAPHX_MI355_FP32_DOT is set at compile time); op::dot::compute
+ * (src/include/migraphx/op/dot.hpp:102-107) is the operator it stands in for. */
+int mi355_dot_fp32acc(const void* a, const void* b, void* c, int32_t type,
+                      int64_t m, int64_t n, int64_t k,
+                      int64_t a_stride_m, int64_t a_stride_k, int64_t b_stride_k, int64_t b_stride_n,
+                      int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                      const float* scale, void* stream);
+
 /*
  * contiguous: gather a strided view (ndim <= MI355_MAX_DIMS, element strides, zero = broadcast)
  * into a dense row-major tensor.  lens / strides are HOST arrays.

@@ -1,0 +1,47 @@
+"""Float `dot` on the device against the CPU oracle (gemm_naive: double accumulation, one rounding):
+the default entry point bit for bit, the fp32 matrix-core entry point within fp32 accumulation
+error -- K * 2^-24 of sum|a||b| -- which is far inside the 1e-3 relative the path's float outputs
+are held to."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from amdmigraphx_amd import ops
+    return ops
+
+
+@pytest.mark.parametrize("bt,m,n,k,trans_b", [(1, 64, 64, 64, False), (12, 384, 384, 64, True), (12, 384, 64, 384, False),
+                                              (3, 100, 36, 52, False), (2, 33, 130, 260, True)])
+def test_float_dot_exact_and_fp32_accumulating(ops, bt, m, n, k, trans_b):
+    rng = np.random.default_rng(bt + m + n + k)
+    a = rng.standard_normal((bt, m, k)).astype(np.float32)
+    b = rng.standard_normal((bt, n, k) if trans_b else (bt, k, n)).astype(np.float32)
+    bv = np.swapaxes(b, 1, 2) if trans_b else b
+    want = orc.dot(a, bv, orc.F32)
+    tb = dev(b).transpose(1, 2) if trans_b else dev(b)
+    got = ops.dot(dev(a), tb).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    fast = ops.dot(dev(a), tb, fp32acc=True).cpu().numpy()
+    mag = np.abs(a).astype(np.float64) @ np.abs(bv).astype(np.float64)
+    err = np.abs(fast.astype(np.float64) - want.astype(np.float64))
+    assert (err <= mag * k * 2.0**-24).all(), (err / mag).max()
+    # with the scale of attention scores: float(sum) * scale, one more fp32 rounding
+    s = torch.tensor([0.125], device="cuda")
+    assert np.array_equal(ops.dot(dev(a), tb, scale=s).cpu().numpy(), want * np.float32(0.125))
+    scaled = ops.dot(dev(a), tb, scale=s, fp32acc=True).cpu().numpy()
+    assert (np.abs(scaled.astype(np.float64) - want * 0.125) <= mag * k * 2.0**-27 + 1e-30).all()
+
+
+def test_fp32_accumulation_is_float32_only(ops):
+    from amdmigraphx_amd import Mi355Error
+    a = torch.zeros((16, 16), dtype=torch.float16, device="cuda")
+    with pytest.raises(Mi355Error):
+        ops.dot(a, a, fp32acc=True)
