@@ -73,6 +73,7 @@ struct dma_params
     int partial_ld;   // n rounded up to 4: a group of 4 columns that starts inside n is stored whole
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
     int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
+    int stream_c;   // C is far larger than the caches: streaming stores
 };
 
 // s_waitcnt with only the vector-memory counter constrained
@@ -140,6 +141,19 @@ struct types<true>
     using acc  = v16f;
     using frag = v8i;
 };
+
+// One vector of C.  `stream`: the result is large against the last-level cache and is written
+// once: a streaming (nontemporal) store keeps it from pushing out the operand panels that every
+// L2 miss of the main loop is served from (8192^3 int8: 479 -> 468 us).  Small results stay
+// cached for whatever reads them next.
+template <class V>
+MI355_DEVINL void store_c(V* dst, V v, bool stream)
+{
+    if(stream)
+        __builtin_nontemporal_store(v, dst);
+    else
+        *dst = v;
+}
 
 template <int OUT>
 MI355_DEVINL void store1(void* c, int64_t idx, float v)
@@ -586,8 +600,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                         {
                             const int64_t idx =
                                 (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
-                            *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.c) + idx) =
-                                make_uint4(r0[0], r1[0], r0[1], r1[1]);
+                            store_c(reinterpret_cast<v4u*>(static_cast<uint16_t*>(p.c) + idx),
+                                    v4u{r0[0], r1[0], r0[1], r1[1]}, p.stream_c);
                         }
                     }
                     continue;
@@ -633,9 +647,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                     if(whole)
                     {
                         using vec_t = out_t __attribute__((ext_vector_type(4)));
-                        *reinterpret_cast<vec_t*>(o) =
-                            vec_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                                  acc[i][j][4 * g + 3]};
+                        store_c(reinterpret_cast<vec_t*>(o),
+                                vec_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                      acc[i][j][4 * g + 3]},
+                                p.stream_c);
                     }
                     else
                     {
@@ -648,8 +663,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                 else if(whole)
                 {
                     if constexpr(OUT == MI355_F32)
-                        *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) =
-                            v4f{v[0], v[1], v[2], v[3]};
+                        store_c(reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx), v4f{v[0], v[1], v[2], v[3]}, p.stream_c);
                     else if constexpr(OUT == MI355_F16)
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
                             convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
@@ -1084,7 +1098,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                     }
                 }
                 else if constexpr(VEC_STORE)
-                    *reinterpret_cast<v4i*>(o) = acc[i][j];
+                    store_c(reinterpret_cast<v4i*>(o), acc[i][j], p.stream_c);
                 else
                 {
 #pragma unroll
@@ -1109,8 +1123,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                 if constexpr(VEC_STORE)
                 {
                     if constexpr(OUT == MI355_F32)
-                        *reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx) =
-                            v4f{v[0], v[1], v[2], v[3]};
+                        store_c(reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx), v4f{v[0], v[1], v[2], v[3]}, p.stream_c);
                     else if constexpr(OUT == MI355_F16)
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
                             convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
@@ -1505,6 +1518,8 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                       reinterpret_cast<uintptr_t>(c) % (4 * esz) == 0;
         p.vec8_store = esz == 2 && d->n % 8 == 0 && d->ldc % 8 == 0 && d->stride_c % 8 == 0 &&
                        reinterpret_cast<uintptr_t>(c) % 16 == 0;
+        // half of the 256 MB last-level cache and more: the result streams past it
+        p.stream_c = (double)d->batch * (double)d->m * (double)d->n * (double)esz >= 128.0 * 1048576.0;
     }
     p.ksplit = 1;
     if(fp8 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && p.vec_store &&
