@@ -26,8 +26,8 @@ PEAK_TFLOPS_FP8 = 5000.0  # dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes one 8192^3 int8 quant_dot launch moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # counter runs of this file scaled by the same counters' reading for a plain copy of known size
-# (profiles/quant_dot_int8_8192_hbm_traffic.md holds both runs and the arithmetic).
-HEADLINE_TRAFFIC_BYTES = 1.0911e9
+# (profiles/quant_dot_int8_8192_counters.md holds both runs and the arithmetic).
+HEADLINE_TRAFFIC_BYTES = 1.1169e9
 
 
 def _time_launches(fn, steps, warmup, settle_ms=0.0):
