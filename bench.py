@@ -193,7 +193,10 @@ def main():
     # an empty kernel on this machine), not the host's submission rate.
     try:
         skip("gemv")
-        shapes4 = ((4096, 4096), (4096, 14336), (14336, 4096))
+        # config 4's three shapes, then the same-input projections of a Llama-3-8B layer as one launch
+        # each (weights concatenated along N, which a graph-level fusion of GEMVs that share their
+        # input gives): q | k | v = 4096 + 1024 + 1024 columns, gate | up = 2 x 14336
+        shapes4 = ((4096, 4096), (4096, 14336), (14336, 4096), (4096, 6144), (4096, 28672))
         if args.gemv_shape:
             shapes4 = (tuple(int(v) for v in args.gemv_shape.split(",")),)
         for (k4, n4) in shapes4:
