@@ -61,6 +61,9 @@ struct module
     }
     instruction_ref insert_literal(instruction_ref ins, literal l);
     instruction_ref add_parameter(std::string name, shape s);
+    // a parameter at a given position and rank among the parameters, as a saved program lists it
+    instruction_ref
+    insert_parameter(instruction_ref ins, std::string name, shape s, std::size_t order);
     instruction_ref add_return(std::vector<instruction_ref> args);
 
     std::vector<std::string> get_parameter_names() const;

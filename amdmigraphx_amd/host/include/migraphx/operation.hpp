@@ -7,6 +7,7 @@
 //   std::ptrdiff_t output_alias(const std::vector<shape>&) const;
 //   void finalize(context&, const shape&, const std::vector<shape>&);
 //   template <class Self, class F> static void reflect(Self&, F f);   // f(self.member, "member")
+//   value to_value() const; void from_value(const value&);            // instead of reflect
 //   value attributes() const;
 // reflect gives to_value / from_value, equality and printing.
 #ifndef MIGRAPHX_GUARD_OPERATION_HPP
@@ -20,6 +21,7 @@
 #include <vector>
 #include <migraphx/argument.hpp>
 #include <migraphx/context.hpp>
+#include <migraphx/serialize.hpp>
 #include <migraphx/value.hpp>
 
 namespace migraphx {
@@ -80,13 +82,22 @@ struct has_attributes : std::false_type {};
 template <class T>
 struct has_attributes<T, void_t<decltype(std::declval<const T&>().attributes())>> : std::true_type {};
 
+// a type may write and read its fields itself: value to_value() const; void from_value(const value&)
+template <class T, class = void>
+struct has_own_value : std::false_type {};
+template <class T>
+struct has_own_value<T,
+                     void_t<decltype(std::declval<const T&>().to_value()),
+                            decltype(std::declval<T&>().from_value(std::declval<const value&>()))>>
+    : std::true_type {};
+
 struct to_value_visitor
 {
     value* v;
     template <class U>
     void operator()(const U& x, const char* name) const
     {
-        (*v)[name] = value(std::string(name), value(x));
+        (*v)[name] = value(std::string(name), migraphx::to_value(x));
     }
 };
 
@@ -97,7 +108,7 @@ struct from_value_visitor
     void operator()(U& x, const char* name) const
     {
         if(v->contains(name))
-            v->at(name).get(x);
+            migraphx::from_value(v->at(name), x);
     }
 };
 
@@ -238,13 +249,17 @@ struct operation
         value to_value() const override
         {
             value v = value::object();
-            if constexpr(detail::has_reflect<T>{})
+            if constexpr(detail::has_own_value<T>{})
+                v = x.to_value();
+            else if constexpr(detail::has_reflect<T>{})
                 T::reflect(x, detail::to_value_visitor{&v});
             return v;
         }
         void from_value(const value& v) override
         {
-            if constexpr(detail::has_reflect<T>{})
+            if constexpr(detail::has_own_value<T>{})
+                x.from_value(v);
+            else if constexpr(detail::has_reflect<T>{})
                 T::reflect(x, detail::from_value_visitor{&v});
         }
         value attributes() const override

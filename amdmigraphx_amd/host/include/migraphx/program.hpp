@@ -42,6 +42,15 @@ struct program
     void finish() const { m_ctx.finish(); }
     context& get_context() { return m_ctx; }
 
+    // The saved form (src/program.cpp:720-777): version numbers, the target's name and context
+    // when compiled, and per module the instructions in order, each with the name of its
+    // result, operator fields, literal data and the names of its inputs.
+    value to_value() const;
+    // Rebuild from the saved form; a compiled program loads its target's library, takes a new
+    // context from it and finalizes again (src/program.cpp:851-902).
+    void from_value(const value& v);
+    static constexpr int program_file_version = 8;
+
     friend std::ostream& operator<<(std::ostream& os, const program& p);
     friend bool operator==(const program& x, const program& y) { return *x.m_main == *y.m_main; }
     friend bool operator!=(const program& x, const program& y) { return not(x == y); }
@@ -49,6 +58,7 @@ struct program
     private:
     std::unique_ptr<module> m_main;
     mutable context m_ctx;
+    std::string m_target; // name of the target it was compiled for
     bool m_compiled = false;
 };
 

@@ -26,7 +26,8 @@ struct value
         float_kind,
         string_kind,
         array_kind,
-        object_kind
+        object_kind,
+        binary_kind // raw bytes (literal data in a saved program)
     };
 
     value() = default;
@@ -52,6 +53,13 @@ struct value
     value(std::initializer_list<value> i);                                 // NOLINT
     value(const std::string& key, const value& v) : value(v) { m_key = key; }
 
+    static value binary(const void* bytes, std::size_t n)
+    {
+        value v;
+        v.m_kind = binary_kind;
+        v.m_str.assign(static_cast<const char*>(bytes), n);
+        return v;
+    }
     static value array() { value v; v.m_kind = array_kind; return v; }
     static value object() { value v; v.m_kind = object_kind; return v; }
 
@@ -60,6 +68,14 @@ struct value
     bool is_string() const { return m_kind == string_kind; }
     bool is_array() const { return m_kind == array_kind; }
     bool is_object() const { return m_kind == object_kind; }
+    bool is_binary() const { return m_kind == binary_kind; }
+    // the bytes of a binary value
+    const std::string& get_binary() const;
+    value without_key() const { value v = *this; v.m_key.clear(); return v; }
+    bool get_bool() const { return as_int() != 0; }
+    int64_t get_int64() const { return as_int(); }
+    double get_double() const { return as_float(); }
+    const std::string& get_string() const;
     const std::string& get_key() const { return m_key; }
 
     bool contains(const std::string& key) const;

@@ -7,6 +7,7 @@
 #include <pybind11/stl.h>
 #include <migraphx/make_op.hpp>
 #include <migraphx/mi355/target.hpp>
+#include <migraphx/load_save.hpp>
 #include <migraphx/onnx.hpp>
 #include <migraphx/ops.hpp>
 #include <migraphx/passes.hpp>
@@ -355,6 +356,37 @@ PYBIND11_MODULE(migraphx, m)
     m.def("parse_onnx_buffer",
           [](const py::bytes& buffer) { return migraphx::parse_onnx_buffer(std::string(buffer)); },
           "Parse onnx file from a buffer", py::arg("onnx_buffer"));
+    // programs on disk (src/py/migraphx_py.cpp:753-793)
+    m.def(
+        "load",
+        [](const std::string& filename, const std::string& format) {
+            migraphx::file_options o;
+            o.format = format;
+            return migraphx::load(filename, o);
+        },
+        "Load MIGraphX program", py::arg("filename"), py::arg("format") = "msgpack");
+    m.def(
+        "save",
+        [](const migraphx::program& p, const std::string& filename, const std::string& format) {
+            migraphx::file_options o;
+            o.format = format;
+            migraphx::save(p, filename, o);
+        },
+        "Save MIGraphX program", py::arg("p"), py::arg("filename"), py::arg("format") = "msgpack");
+    m.def(
+        "save_buffer",
+        [](const migraphx::program& p) {
+            auto buffer = migraphx::save_buffer(p);
+            return py::bytes(buffer.data(), buffer.size());
+        },
+        "Serialize MIGraphX program", py::arg("p"));
+    m.def(
+        "load_buffer",
+        [](const py::bytes& b) {
+            const std::string bytes = b;
+            return migraphx::load_buffer(bytes.data(), bytes.size());
+        },
+        "Deserialize MIGraphX program", py::arg("b"));
     m.def("get_target", &get_target);
     m.def("create_argument", [](const shape& s, const std::vector<double>& values) {
         if(values.size() != s.elements())

@@ -192,6 +192,13 @@ instruction_ref module::add_parameter(std::string name, shape s)
     return m_ins.begin();
 }
 
+instruction_ref
+module::insert_parameter(instruction_ref ins, std::string name, shape s, std::size_t order)
+{
+    return m_ins.insert(
+        ins, instruction{operation{builtin::param{std::move(name), order}}, std::move(s), {}});
+}
+
 instruction_ref module::add_return(std::vector<instruction_ref> args)
 {
     m_ins.push_back(instruction{operation{builtin::returns{}}, shape{}, std::move(args)});

@@ -683,7 +683,8 @@ void quantize_int4_pass::apply(module& m) const
             if(can_store_as_int4(x))
                 x = through_int4(m, user, x);
         }
-        m.replace_instruction(user, m.insert_instruction(user, user->get_operator(), operands));
+        if(operands != user->inputs())
+            m.replace_instruction(user, user->get_operator(), operands);
     }
 }
 

@@ -1,6 +1,7 @@
 #include <migraphx/program.hpp>
 #include <migraphx/register_op.hpp>
 #include <migraphx/register_target.hpp>
+#include <migraphx/serialize.hpp>
 #include <algorithm>
 #include <iostream>
 #include <map>
@@ -159,7 +160,10 @@ void run_passes(program& p, const std::vector<pass>& passes)
 // --------------------------------------------------------------------- program
 
 program::program(const program& p)
-    : m_main(std::make_unique<module>(*p.m_main)), m_ctx(p.m_ctx), m_compiled(p.m_compiled)
+    : m_main(std::make_unique<module>(*p.m_main)),
+      m_ctx(p.m_ctx),
+      m_target(p.m_target),
+      m_compiled(p.m_compiled)
 {
 }
 
@@ -167,6 +171,7 @@ program& program::operator=(program p)
 {
     std::swap(m_main, p.m_main);
     std::swap(m_ctx, p.m_ctx);
+    std::swap(m_target, p.m_target);
     std::swap(m_compiled, p.m_compiled);
     return *this;
 }
@@ -182,7 +187,134 @@ void program::compile(const target& t, compile_options options)
         MIGRAPHX_THROW("Invalid program from compilation at instruction " + bad->name());
     m_main->finalize(m_ctx);
     m_ctx.finish();
+    m_target   = t.name();
     m_compiled = true;
+}
+
+// --------------------------------------------------------------- saved programs
+
+static const char* const library_version = "2.16.0";
+
+value program::to_value() const
+{
+    value result                = value::object();
+    result["version"]           = value("version", program_file_version);
+    result["migraphx_version"]  = value("migraphx_version", library_version);
+    value targets               = value::array();
+    value contexts              = value::array();
+    if(m_compiled)
+    {
+        value t   = value::object();
+        t["name"] = value("name", m_target);
+        targets.push_back(t);
+        contexts.push_back(value::object()); // the stream is made anew on load
+    }
+    result["targets"]  = value("targets", targets);
+    result["contexts"] = value("contexts", contexts);
+
+    // results are named by position, parameters by their own name (src/module.cpp:1473-1500)
+    std::unordered_map<const instruction*, std::string> names;
+    value nodes       = value::array();
+    std::size_t count = 0;
+    for(auto ins = m_main->begin(); ins != m_main->end(); ++ins, ++count)
+    {
+        const bool is_param = ins->name() == "@param";
+        const auto out      = is_param ? any_cast<builtin::param>(ins->get_operator()).parameter
+                                       : "@" + std::to_string(count);
+        names[&*ins]        = out;
+        value node          = value::object();
+        node["output"]      = value("output", out);
+        node["name"]        = value("name", ins->name());
+        node["shape"]       = value("shape", migraphx::to_value(ins->get_shape()));
+        node["normalized"]  = value("normalized", true);
+        if(ins->name() == "@literal")
+            node["literal"] = value("literal", migraphx::to_value(ins->get_literal()));
+        node["operator"] = value("operator", ins->get_operator().to_value());
+        value inputs     = value::array();
+        for(auto a : ins->inputs())
+            inputs.push_back(value(names.at(&*a)));
+        node["inputs"] = value("inputs", inputs);
+        nodes.push_back(node);
+    }
+    value main_module     = value::object();
+    main_module["name"]   = value("name", m_main->name());
+    main_module["nodes"]  = value("nodes", nodes);
+    value modules         = value::object();
+    modules[m_main->name()] = value(m_main->name(), main_module);
+    result["modules"]     = value("modules", modules);
+    return result;
+}
+
+void program::from_value(const value& v)
+{
+    const auto version = v.at("version").to<int>();
+    if(version != program_file_version)
+        MIGRAPHX_THROW(
+            "Error: Program version mismatch. MXR file was created using program file version: " +
+            std::to_string(version) + ", while installed MIGraphX is using program file version: " +
+            std::to_string(program_file_version) +
+            ", Try regenerating MXR file using installed MIGraphX and running again.");
+    const auto& targets = v.at("targets");
+    if(targets.size() > 1)
+        MIGRAPHX_THROW("from_value: programs compiled for several targets are not supported");
+    const auto& modules = v.at("modules");
+    if(modules.size() != 1 or not modules.contains("main"))
+        MIGRAPHX_THROW("from_value: programs with submodules are not supported");
+
+    // make_target loads the target's library, which registers its operators
+    target tgt;
+    if(not targets.empty())
+        tgt = make_target(targets.at(0).at("name").to<std::string>());
+
+    auto fresh = std::make_unique<module>("main");
+    std::unordered_map<std::string, instruction_ref> by_name;
+    for(const auto& node : modules.at("main").at("nodes").items())
+    {
+        const auto name    = node.at("name").to<std::string>();
+        const auto& fields = node.at("operator");
+        instruction_ref out;
+        if(name == "@param")
+        {
+            out = fresh->insert_parameter(fresh->end(),
+                                          fields.at("parameter").to<std::string>(),
+                                          migraphx::from_value<shape>(node.at("shape")),
+                                          fields.contains("order")
+                                              ? fields.at("order").to<std::size_t>()
+                                              : fresh->get_parameter_names().size());
+        }
+        else if(name == "@literal")
+        {
+            out = fresh->insert_literal(fresh->end(), migraphx::from_value<literal>(node.at("literal")));
+        }
+        else
+        {
+            std::vector<instruction_ref> inputs;
+            for(const auto& i : node.at("inputs").items())
+            {
+                auto it = by_name.find(i.to<std::string>());
+                if(it == by_name.end())
+                    MIGRAPHX_THROW("from_value: " + name + " uses '" + i.to<std::string>() +
+                                   "' before it is defined");
+                inputs.push_back(it->second);
+            }
+            out = name == "@return" ? fresh->add_return(inputs)
+                                    : fresh->add_instruction(make_op(name, fields), inputs);
+        }
+        by_name[node.at("output").to<std::string>()] = out;
+    }
+
+    m_main     = std::move(fresh);
+    m_ctx      = context{};
+    m_target   = "";
+    m_compiled = false;
+    if(not tgt.empty())
+    {
+        m_ctx = tgt.get_context();
+        m_main->finalize(m_ctx);
+        m_ctx.finish();
+        m_target   = tgt.name();
+        m_compiled = true;
+    }
 }
 
 std::vector<argument> program::eval(const parameter_map& params) const

@@ -65,6 +65,20 @@ void value::push_back(const value& v)
 
 void value::get(bool& b) const { b = as_int() != 0; }
 
+const std::string& value::get_binary() const
+{
+    if(m_kind != binary_kind)
+        MIGRAPHX_THROW("value: expected binary data");
+    return m_str;
+}
+
+const std::string& value::get_string() const
+{
+    if(m_kind != string_kind)
+        MIGRAPHX_THROW("value: expected a string");
+    return m_str;
+}
+
 void value::get(std::string& s) const
 {
     if(m_kind != string_kind)
@@ -107,7 +121,7 @@ bool operator==(const value& x, const value& y)
         return x.as_float() == y.as_float();
     if(x.m_kind != y.m_kind)
         return false;
-    if(x.m_kind == value::string_kind)
+    if(x.m_kind == value::string_kind or x.m_kind == value::binary_kind)
         return x.m_str == y.m_str;
     return x.m_items == y.m_items;
 }
@@ -121,6 +135,7 @@ std::ostream& operator<<(std::ostream& os, const value& v)
     case value::int_kind: os << v.m_int; break;
     case value::float_kind: os << v.m_float; break;
     case value::string_kind: os << v.m_str; break;
+    case value::binary_kind: os << "binary[" << v.m_str.size() << "]"; break;
     case value::array_kind:
     case value::object_kind: {
         const bool obj = v.m_kind == value::object_kind;

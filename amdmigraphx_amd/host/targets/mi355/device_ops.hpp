@@ -40,6 +40,11 @@ struct allocate
 {
     shape s;
     argument buffer; // set by finalize
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.s, "shape");
+    }
     std::string name() const { return "mi355::allocate"; }
     shape compute_shape(const std::vector<shape>&) const { return s; }
     void finalize(migraphx::context&, const shape&, const std::vector<shape>&)
@@ -53,6 +58,9 @@ struct allocate
 struct device_literal
 {
     argument data;
+    // saved as host bytes: written from a copy of the device buffer, read straight into a new one
+    value to_value() const;
+    void from_value(const value& v);
     std::string name() const { return "mi355::literal"; }
     shape compute_shape(const std::vector<shape>&) const { return data.get_shape(); }
     argument compute(migraphx::context&, const shape&, const std::vector<argument>&) const

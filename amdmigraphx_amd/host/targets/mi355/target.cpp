@@ -197,6 +197,21 @@ argument allocate::compute(migraphx::context&, const shape&, const std::vector<a
     return buffer;
 }
 
+value device_literal::to_value() const
+{
+    // the key is always there: make_op checks attribute names against a default instance
+    value v   = value::object();
+    v["data"] = value("data", data.empty() ? value{} : migraphx::to_value(from_device(data)));
+    return v;
+}
+
+void device_literal::from_value(const value& v)
+{
+    if(not v.contains("data") or v.at("data").is_null())
+        return;
+    data = to_device(migraphx::from_value<argument>(v.at("data")));
+}
+
 shape copy_to_device::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());

@@ -7,6 +7,7 @@
 #include "encoder.hpp"
 #include "oracle_target.hpp"
 #include "test.hpp"
+#include <migraphx/load_save.hpp>
 #include <chrono>
 #include <cstdlib>
 #include <fstream>
@@ -1293,6 +1294,70 @@ TEST_CASE(encoder_int8_qdq)
     auto fp = fb.build();
     auto ref = run_on("oracle", fp, {{"ids", ids}});
     EXPECT(rms_error(want[0], ref[0]) < 0.05);
+}
+
+TEST_CASE(compiled_program_saved_and_loaded)
+{
+    // A program compiled for the device (fused quant_dot launches, device literals holding the
+    // folded int8 weights and column sums, scratch allocations, copies inside eval) is written to
+    // a file, read back in the same process and run: same instructions, bit-identical results
+    // (test/serialize_program.cpp:88-95, on this target).
+    encoder::config c;
+    auto w = encoder::make_weights(c, 7);
+    argument ids{shape{shape::int32_type, {c.tokens()}}, uniform_ints<int>(c.tokens(), 0, static_cast<int>(c.vocab) - 1, 8)};
+    auto scales = encoder::calibrate(c, w, "mi355", ids);
+    auto p      = encoder::quantized(c, w, scales);
+    migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    program compiled = p;
+    migraphx::compile_options opts;
+    opts.offload_copy = true;
+    compiled.compile(migraphx::make_target("mi355"), opts);
+    auto want = compiled.eval({{"ids", ids}});
+    compiled.finish();
+
+    const std::string filename = "/tmp/mi355_gpu_tests_encoder.mxr";
+    migraphx::save(compiled, filename);
+    auto loaded = migraphx::load(filename);
+    std::remove(filename.c_str());
+    EXPECT(loaded.is_compiled());
+    EXPECT(loaded == compiled);
+    EXPECT(count_ops(*loaded.get_main_module(), "mi355::quant_dot") == 6 * c.layers);
+    EXPECT(count_ops(*loaded.get_main_module(), "mi355::literal") ==
+           count_ops(*compiled.get_main_module(), "mi355::literal"));
+    for(int rep = 0; rep < 2; rep++)
+    {
+        auto got = loaded.eval({{"ids", ids}});
+        loaded.finish();
+        EXPECT(got.size() == 1 and same_bytes(got[0], want[0]));
+    }
+    // the JSON form carries the same program
+    migraphx::file_options json;
+    json.format  = "json";
+    auto loaded2 = migraphx::load_buffer(migraphx::save_buffer(compiled, json), json);
+    auto got2    = loaded2.eval({{"ids", ids}});
+    loaded2.finish();
+    EXPECT(same_bytes(got2[0], want[0]));
+
+    // weight-only int4: the packed weights and their scales travel as device literals
+    {
+        const std::size_t m = 4, k = 256, n = 192;
+        program q;
+        auto* mm = q.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::half_type, {m, k}});
+        auto wl  = mm->add_literal(literal{shape{shape::half_type, {k, n}}, normal_floats(k * n, 0.05f, 21)});
+        mm->add_return({mm->add_instruction(make_op("dot"), x, wl)});
+        migraphx::quantize_int4_weights(q);
+        program cq = q;
+        cq.compile(migraphx::make_target("mi355"), opts);
+        argument xa{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 22)};
+        auto r1 = cq.eval({{"x", xa}});
+        cq.finish();
+        auto lq = migraphx::load_buffer(migraphx::save_buffer(cq));
+        auto r2 = lq.eval({{"x", xa}});
+        lq.finish();
+        EXPECT(lq == cq);
+        EXPECT(same_bytes(r1[0], r2[0]));
+    }
 }
 
 TEST_CASE(encoder_int8_qdq_real_width)

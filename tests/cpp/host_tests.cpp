@@ -8,6 +8,9 @@
 #include "oracle_target.hpp"
 #include "test.hpp"
 #include <sstream>
+#include <migraphx/json.hpp>
+#include <migraphx/load_save.hpp>
+#include <migraphx/msgpack.hpp>
 #include <migraphx/onnx.hpp>
 #include <algorithm>
 #include <fstream>
@@ -1132,6 +1135,316 @@ TEST_CASE(encoder_graph_on_cpu)
     EXPECT(std::sqrt(num / den) < 0.05);
     // LayerNorm output: rows have mean ~beta and unit-scale spread
     EXPECT(q[0].get_shape() == shape{shape::float_type, {c.tokens(), c.hidden}});
+}
+
+// ---------------------------------------------------------------- saved programs
+// Follows test/msgpack.cpp (encodings compared with the MessagePack format's own byte layouts),
+// test/json.cpp and test/serialize_program.cpp (a program equals the one read back from its value,
+// MessagePack, JSON and file forms, compiled or not).
+
+static std::vector<char> bytes_of(std::initializer_list<int> b)
+{
+    std::vector<char> r;
+    for(int x : b)
+        r.push_back(static_cast<char>(x));
+    return r;
+}
+
+TEST_CASE(msgpack_known_encodings)
+{
+    using migraphx::to_msgpack;
+    using migraphx::value;
+    // the MessagePack specification's formats: fixint, uint8/16/32/64, negative fixint, int8/16/32
+    EXPECT(to_msgpack(value{}) == bytes_of({0xc0}));
+    EXPECT(to_msgpack(value(true)) == bytes_of({0xc3}));
+    EXPECT(to_msgpack(value(false)) == bytes_of({0xc2}));
+    EXPECT(to_msgpack(value(3)) == bytes_of({0x03}));
+    EXPECT(to_msgpack(value(127)) == bytes_of({0x7f}));
+    EXPECT(to_msgpack(value(128)) == bytes_of({0xcc, 0x80}));
+    EXPECT(to_msgpack(value(256)) == bytes_of({0xcd, 0x01, 0x00}));
+    EXPECT(to_msgpack(value(65536)) == bytes_of({0xce, 0x00, 0x01, 0x00, 0x00}));
+    EXPECT(to_msgpack(value(int64_t{1} << 32)) ==
+           bytes_of({0xcf, 0, 0, 0, 1, 0, 0, 0, 0}));
+    EXPECT(to_msgpack(value(-1)) == bytes_of({0xff}));
+    EXPECT(to_msgpack(value(-32)) == bytes_of({0xe0}));
+    EXPECT(to_msgpack(value(-33)) == bytes_of({0xd0, 0xdf}));
+    EXPECT(to_msgpack(value(-129)) == bytes_of({0xd1, 0xff, 0x7f}));
+    EXPECT(to_msgpack(value(-32769)) == bytes_of({0xd2, 0xff, 0xff, 0x7f, 0xff}));
+    EXPECT(to_msgpack(value(-(int64_t{1} << 40))) ==
+           bytes_of({0xd3, 0xff, 0xff, 0xff, 0, 0, 0, 0, 0}));
+    // doubles are float64, big endian: 1.5 = 0x3ff8000000000000
+    EXPECT(to_msgpack(value(1.5)) == bytes_of({0xcb, 0x3f, 0xf8, 0, 0, 0, 0, 0, 0}));
+    EXPECT(to_msgpack(value("abc")) == bytes_of({0xa3, 'a', 'b', 'c'}));
+    {
+        const std::string s40(40, 'x');
+        auto b = to_msgpack(value(s40));
+        EXPECT(b.size() == 42 and static_cast<unsigned char>(b[0]) == 0xd9 and b[1] == 40);
+    }
+    EXPECT(to_msgpack(value(std::vector<int>{1, 2, 3})) == bytes_of({0x93, 1, 2, 3}));
+    EXPECT(to_msgpack(value::array()) == bytes_of({0x90}));
+    // keyed items make a map, in order
+    EXPECT(to_msgpack(value{{"a", 1}, {"b", true}}) ==
+           bytes_of({0x82, 0xa1, 'a', 0x01, 0xa1, 'b', 0xc3}));
+    // binary data: an array of bin chunks (one here)
+    const unsigned char raw[3] = {0, 200, 7};
+    EXPECT(to_msgpack(value::binary(raw, 3)) == bytes_of({0x91, 0xc4, 3, 0, 200, 7}));
+    {
+        std::vector<int> many(20, 5);
+        auto b = to_msgpack(value(many));
+        EXPECT(static_cast<unsigned char>(b[0]) == 0xdc and b[1] == 0 and b[2] == 20 and b.size() == 23);
+    }
+}
+
+TEST_CASE(msgpack_reads_every_number_format)
+{
+    using migraphx::from_msgpack;
+    EXPECT(from_msgpack(bytes_of({0xca, 0x3f, 0xc0, 0, 0})).to<double>() == 1.5); // float32
+    EXPECT(from_msgpack(bytes_of({0xcc, 0xff})).to<int>() == 255);
+    EXPECT(from_msgpack(bytes_of({0xd0, 0x80})).to<int>() == -128);
+    EXPECT(from_msgpack(bytes_of({0xd1, 0x80, 0x00})).to<int>() == -32768);
+    EXPECT(from_msgpack(bytes_of({0xd2, 0x80, 0, 0, 0})).to<int64_t>() == -2147483648ll);
+    EXPECT(from_msgpack(bytes_of({0xd3, 0xff, 0xff, 0xff, 0xff, 0xff, 0xff, 0xff, 0xfe})).to<int>() == -2);
+    EXPECT(from_msgpack(bytes_of({0xda, 0, 2, 'h', 'i'})).to<std::string>() == "hi");
+    EXPECT(from_msgpack(bytes_of({0xdd, 0, 0, 0, 2, 1, 2})).to_vector<int>() == std::vector<int>{1, 2});
+    EXPECT(from_msgpack(bytes_of({0xde, 0, 1, 0xa1, 'k', 0x05})).at("k").to<int>() == 5);
+    // a lone bin object (the older layout) and chunked binary both read as binary
+    EXPECT(from_msgpack(bytes_of({0xc4, 2, 9, 8})).get_binary() == std::string("\x09\x08"));
+    EXPECT(from_msgpack(bytes_of({0x92, 0xc4, 1, 9, 0xc5, 0, 1, 8})).get_binary() == std::string("\x09\x08"));
+    EXPECT(test::throws([] { from_msgpack(bytes_of({0xc7, 1, 1, 0})); }));       // ext
+    EXPECT(test::throws([] { from_msgpack(bytes_of({0xa5, 'a', 'b'})); }));      // truncated
+    EXPECT(test::throws([] { from_msgpack(bytes_of({0x93, 1, 2})); }));          // truncated array
+    EXPECT(test::throws([] { from_msgpack(std::vector<char>{}); }));
+}
+
+static migraphx::value sample_value()
+{
+    using migraphx::value;
+    const unsigned char raw[5] = {1, 0, 255, 128, 3};
+    value v                    = value::object();
+    v["none"]                  = value("none", value{});
+    v["flag"]                  = value("flag", true);
+    v["count"]                 = value("count", -70000);
+    v["big"]                   = value("big", int64_t{1} << 50);
+    v["ratio"]                 = value("ratio", 0.1);
+    v["whole"]                 = value("whole", 2.0);
+    v["text"]                  = value("text", "line\n\"quoted\"\t\\ \x01 caf\xc3\xa9");
+    v["list"]                  = value("list", std::vector<int>{1, -2, 3});
+    v["empty"]                 = value("empty", value::array());
+    v["bytes"]                 = value("bytes", value::binary(raw, 5));
+    value inner                = value::object();
+    inner["lens"]              = value("lens", std::vector<std::size_t>{2, 3});
+    inner["nested"]            = value("nested", value{{"k", 1.25}});
+    v["inner"]                 = value("inner", inner);
+    return v;
+}
+
+TEST_CASE(msgpack_and_json_round_trips)
+{
+    auto v = sample_value();
+    auto m = migraphx::from_msgpack(migraphx::to_msgpack(v));
+    EXPECT(m == v);
+    EXPECT(m.at("bytes").is_binary() and m.at("bytes").get_binary().size() == 5);
+    EXPECT(m.at("whole").kind() == migraphx::value::float_kind);
+    auto text = migraphx::to_json_string(v);
+    auto j    = migraphx::from_json_string(text);
+    EXPECT(j == v);
+    EXPECT(j.at("whole").kind() == migraphx::value::float_kind);
+    EXPECT(j.at("text").to<std::string>() == v.at("text").to<std::string>());
+    // hand-written JSON: whitespace, escapes, exponents, nesting
+    auto h = migraphx::from_json_string(
+        " { \"a\" : [ 1 , 2.5e1 , -3 ] , \"s\" : \"\\u0041\\u00e9\\ud83d\\ude00\\/\" , \"o\" : { } , \"n\" : null }");
+    EXPECT(h.at("a").to_vector<double>() == std::vector<double>{1, 25, -3});
+    EXPECT(h.at("s").to<std::string>() == "A\xc3\xa9\xf0\x9f\x98\x80/");
+    EXPECT(h.at("o").is_object() and h.at("o").empty());
+    EXPECT(h.at("n").is_null());
+    EXPECT(migraphx::to_json_string(migraphx::value{{"a", 1}, {"b", "x"}}) == "{\"a\":1,\"b\":\"x\"}");
+    EXPECT(migraphx::to_json_string(migraphx::value(std::vector<int>{1, 2})) == "[1,2]");
+    EXPECT(test::throws([] { migraphx::from_json_string("{\"a\": }"); }));
+    EXPECT(test::throws([] { migraphx::from_json_string("[1, 2"); }));
+    EXPECT(test::throws([] { migraphx::from_json_string("[1] x"); }));
+}
+
+TEST_CASE(shape_and_literal_values)
+{
+    shape s{shape::half_type, {2, 3, 4}, {12, 1, 3}};
+    auto v = migraphx::to_value(s);
+    EXPECT(v.at("type").to<std::string>() == "half_type");
+    EXPECT(v.at("lens").to_vector<std::size_t>() == s.lens());
+    EXPECT(v.at("strides").to_vector<std::size_t>() == s.strides());
+    EXPECT(v.at("dynamic_dimensions").empty() and v.at("sub_shapes").empty());
+    EXPECT(migraphx::from_value<shape>(v) == s);
+    literal l{shape{shape::int8_type, {2, 2}}, std::vector<int>{-128, 127, 0, 5}};
+    auto lv = migraphx::to_value(l);
+    EXPECT(lv.at("data").get_binary() == std::string("\x80\x7f\x00\x05", 4));
+    EXPECT(migraphx::from_value<literal>(lv) == l);
+    // a literal whose byte count disagrees with its shape is refused
+    lv["data"] = migraphx::value("data", migraphx::value::binary("ab", 2));
+    EXPECT(test::throws([&] { migraphx::from_value<literal>(lv); }));
+    // a scalar
+    literal one{1.5f};
+    EXPECT(migraphx::from_value<literal>(migraphx::to_value(one)) == one);
+}
+
+static program qdq_program_for_saving()
+{
+    // three parameters added in order, literals of several types, operators with list, number,
+    // type and string attributes, views, and the quantize / dequantize pair
+    program p;
+    auto* mm = p.get_main_module();
+    auto x   = mm->add_parameter("x", shape{shape::float_type, {2, 4, 8}});
+    auto w   = mm->add_parameter("w", shape{shape::float_type, {8, 6}});
+    auto b   = mm->add_parameter("bias", shape{shape::half_type, {6}});
+    auto sc  = mm->add_literal(literal{0.05f});
+    auto zp  = mm->add_literal(literal{shape{shape::int8_type}, std::vector<int>{3}});
+    auto qx  = add_quantize_op(*mm, "quantizelinear", x, sc, zp);
+    auto dx  = add_quantize_op(*mm, "dequantizelinear", qx, sc, zp);
+    auto wt  = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), w);
+    auto wtt = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), wt);
+    auto wb  = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {2, 8, 6}}}), wtt);
+    auto d   = mm->add_instruction(make_op("dot"), dx, wb);
+    auto bf  = mm->add_instruction(make_op("convert", {{"target_type", shape::float_type}}), b);
+    auto bb  = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {2, 4, 6}}}), bf);
+    auto sum = mm->add_instruction(make_op("add"), d, bb);
+    auto sl  = mm->add_instruction(
+        make_op("slice", {{"axes", {2}}, {"starts", {1}}, {"ends", {5}}}), sum);
+    auto sm = mm->add_instruction(make_op("softmax", {{"axis", -1}}), sl);
+    mm->add_return({sm, sum});
+    return p;
+}
+
+static std::string printed(const program& p)
+{
+    std::stringstream ss;
+    ss << p;
+    return ss.str();
+}
+
+TEST_CASE(program_value_round_trip)
+{
+    auto p1 = qdq_program_for_saving();
+    auto v  = p1.to_value();
+    EXPECT(v.at("version").to<int>() == 8);
+    EXPECT(v.at("targets").empty() and v.at("contexts").empty());
+    const auto& nodes = v.at("modules").at("main").at("nodes");
+    EXPECT(nodes.size() == p1.get_main_module()->size());
+    // results are named by position, parameters by name; inputs refer to those names
+    std::size_t i = 0;
+    for(const auto& node : nodes.items())
+    {
+        const auto name = node.at("name").to<std::string>();
+        if(name == "@param")
+            EXPECT(node.at("output").to<std::string>() == node.at("operator").at("parameter").to<std::string>());
+        else
+            EXPECT(node.at("output").to<std::string>() == "@" + std::to_string(i));
+        EXPECT(node.contains("literal") == (name == "@literal"));
+        i++;
+    }
+    program p2;
+    p2.from_value(v);
+    EXPECT(p1 == p2);
+    EXPECT(printed(p1) == printed(p2));
+    EXPECT(p2.get_parameter_names() == p1.get_parameter_names());
+    EXPECT(p2.get_output_shapes() == p1.get_output_shapes());
+    EXPECT(not p2.is_compiled());
+    EXPECT(p2.to_value() == v);
+}
+
+TEST_CASE(program_saved_as_msgpack_json_and_file)
+{
+    auto p1 = qdq_program_for_saving();
+    for(const std::string format : {"msgpack", "json"})
+    {
+        migraphx::file_options o;
+        o.format    = format;
+        auto buffer = migraphx::save_buffer(p1, o);
+        auto p2     = migraphx::load_buffer(buffer, o);
+        EXPECT(p1 == p2);
+        EXPECT(printed(p1) == printed(p2));
+        auto p3 = migraphx::load_buffer(buffer.data(), buffer.size(), o);
+        EXPECT(p1 == p3);
+    }
+    const std::string filename = "/tmp/mi355_host_tests_program.mxr";
+    migraphx::save(p1, filename);
+    auto p4 = migraphx::load(filename);
+    std::remove(filename.c_str());
+    EXPECT(p1 == p4);
+    EXPECT(test::throws([&] { migraphx::load(filename); })); // gone
+    migraphx::file_options bad;
+    bad.format = "???";
+    EXPECT(test::throws([&] { migraphx::save_buffer(p1, bad); }));
+    EXPECT(test::throws([&] { migraphx::load_buffer(std::vector<char>{}, bad); }));
+}
+
+TEST_CASE(program_load_rejects_bad_files)
+{
+    auto v = qdq_program_for_saving().to_value();
+    {
+        auto w       = v;
+        w["version"] = migraphx::value("version", 7);
+        program p;
+        EXPECT(test::throws([&] { p.from_value(w); }));
+    }
+    {
+        // an input that is not defined yet
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, {2}});
+        mm->add_instruction(make_op("neg"), x);
+        auto text = migraphx::to_json_string(p.to_value());
+        auto at   = text.find("\"inputs\":[\"x\"]");
+        EXPECT(at != std::string::npos);
+        text.replace(at, 14, "\"inputs\":[\"y\"]");
+        migraphx::file_options o;
+        o.format = "json";
+        EXPECT(test::throws([&] { migraphx::load_buffer(text.data(), text.size(), o); }));
+    }
+    {
+        // an operator this library does not have
+        auto text = migraphx::to_json_string(v);
+        auto at   = text.find("\"name\":\"softmax\"");
+        EXPECT(at != std::string::npos);
+        text.replace(at, 16, "\"name\":\"softmin\"");
+        migraphx::file_options o;
+        o.format = "json";
+        EXPECT(test::throws([&] { migraphx::load_buffer(text.data(), text.size(), o); }));
+    }
+    // cut short
+    auto buffer = migraphx::save_buffer(qdq_program_for_saving());
+    buffer.resize(buffer.size() / 2);
+    EXPECT(test::throws([&] { migraphx::load_buffer(buffer); }));
+}
+
+TEST_CASE(saved_program_evaluates_the_same)
+{
+    // the quantized form of a program (after the QDQ rewrite) is saved, read back, and both are
+    // evaluated on the CPU oracle target; compiled there, it is saved and read back once more
+    auto p1 = qdq_program_for_saving();
+    migraphx::run_passes(p1, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+    auto p2 = migraphx::load_buffer(migraphx::save_buffer(p1));
+    EXPECT(p1 == p2);
+    migraphx::parameter_map params;
+    params["x"]    = argument{shape{shape::float_type, {2, 4, 8}}, normal_floats(64, 1.0f, 1)};
+    params["w"]    = argument{shape{shape::float_type, {8, 6}}, normal_floats(48, 0.5f, 2)};
+    params["bias"] = argument{shape{shape::half_type, {6}}, normal_floats(6, 0.5f, 3)};
+    auto r1 = run_on("oracle", p1, params);
+    auto r2 = run_on("oracle", p2, params);
+    EXPECT(r1.size() == 2 and r2.size() == 2);
+    EXPECT(same_bytes(r1[0], r2[0]) and same_bytes(r1[1], r2[1]));
+
+    program c1 = p1;
+    c1.compile(migraphx::make_target("oracle"));
+    auto v = c1.to_value();
+    EXPECT(v.at("targets").size() == 1);
+    EXPECT(v.at("targets").at(0).at("name").to<std::string>() == "oracle");
+    EXPECT(v.at("contexts").size() == 1);
+    auto c2 = migraphx::load_buffer(migraphx::save_buffer(c1));
+    EXPECT(c2.is_compiled());
+    EXPECT(c1 == c2);
+    auto r3 = c2.eval(params);
+    c2.finish();
+    EXPECT(same_bytes(r1[0], r3[0]) and same_bytes(r1[1], r3[1]));
+    // a compiled program cannot be compiled again, loaded or not
+    EXPECT(test::throws([&] { c2.compile(migraphx::make_target("oracle")); }));
 }
 
 // ---------------------------------------------------------------- MatMulNBits

@@ -91,6 +91,9 @@ struct cpu_op
 {
     migraphx::operation op;
     std::string name() const { return "oracle::" + op.name(); }
+    // saved with the wrapped operator's own fields
+    migraphx::value to_value() const { return op.to_value(); }
+    void from_value(const migraphx::value& v) { op.from_value(v); }
     shape compute_shape(const std::vector<shape>& inputs) const
     {
         auto s = op.compute_shape(inputs);
@@ -313,6 +316,8 @@ struct cpu_op
 
 } // namespace
 
+migraphx::operation wrap(const migraphx::operation& op) { return migraphx::operation{cpu_op{op}}; }
+
 void lowering::apply(migraphx::module& m) const
 {
     std::vector<migraphx::instruction_ref> all;
@@ -338,3 +343,13 @@ std::vector<migraphx::pass> target::get_passes(migraphx::context&,
 } // namespace oracle
 
 MIGRAPHX_REGISTER_TARGET(oracle::target);
+
+// every operator of the library can come back from a saved program in its wrapped form
+static const int register_wrapped_operators = [] {
+    for(const auto& name : migraphx::get_operators())
+    {
+        if(name[0] != '@' and name.rfind("oracle::", 0) != 0)
+            migraphx::register_op(migraphx::operation{oracle::wrap(migraphx::load_op(name))});
+    }
+    return 0;
+}();

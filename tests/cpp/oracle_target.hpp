@@ -8,6 +8,7 @@
 #include <string>
 #include <vector>
 #include <migraphx/context.hpp>
+#include <migraphx/operation.hpp>
 #include <migraphx/pass.hpp>
 #include <migraphx/target.hpp>
 
@@ -17,6 +18,9 @@ struct context
 {
     void finish() const {}
 };
+
+// the operator that evaluates `op` with the oracle
+migraphx::operation wrap(const migraphx::operation& op);
 
 struct lowering
 {

@@ -111,3 +111,89 @@ def test_targets():
     assert mgx.get_target("mi355").name() == "mi355"
     with pytest.raises(RuntimeError):
         mgx.get_target("no_such_target")
+
+
+def quantized_matmul_program():
+    p, _ = build_matmul(k=256, n=64)
+    mgx.quantize_int4_weights(p)
+    return p
+
+
+def test_save_and_load(tmp_path):
+    # src/py/migraphx_py.cpp:753-793: load / save with a format keyword, save_buffer / load_buffer
+    p = quantized_matmul_program()
+    for fmt in ("msgpack", "json"):
+        name = str(tmp_path / ("prog." + fmt))
+        mgx.save(p, name, format=fmt)
+        q = mgx.load(name, format=fmt)
+        assert q == p and repr(q) == repr(p)
+    name = str(tmp_path / "default.mxr")
+    mgx.save(p, name)
+    assert mgx.load(name) == p
+    buf = mgx.save_buffer(p)
+    assert isinstance(buf, bytes) and open(name, "rb").read() == buf
+    assert mgx.load_buffer(buf) == p
+    with pytest.raises(RuntimeError):
+        mgx.load(str(tmp_path / "missing.mxr"))
+    with pytest.raises(RuntimeError):
+        mgx.save(p, str(tmp_path / "x"), format="yaml")
+    with pytest.raises(RuntimeError):
+        mgx.load_buffer(buf[: len(buf) // 2])
+
+
+def test_saved_program_is_standard_messagepack():
+    """The saved bytes are checked against an independent MessagePack implementation (the `msgpack`
+    Python package): it decodes them to the fields src/program.cpp:720-777 writes, re-encoding what
+    it decoded gives the same bytes (every number and length is in its shortest form), and bytes it
+    encodes load as the same program."""
+    msgpack = pytest.importorskip("msgpack")
+    p = quantized_matmul_program()
+    buf = mgx.save_buffer(p)
+    doc = msgpack.unpackb(buf, raw=False, strict_map_key=True)
+    assert doc["version"] == 8 and isinstance(doc["migraphx_version"], str)
+    assert doc["targets"] == [] and doc["contexts"] == []
+    assert list(doc["modules"]) == ["main"] and doc["modules"]["main"]["name"] == "main"
+    nodes = doc["modules"]["main"]["nodes"]
+    assert [n["name"] for n in nodes].count("@literal") >= 2          # packed weights and scales
+    by_output = {n["output"]: n for n in nodes}
+    assert len(by_output) == len(nodes)
+    for i, n in enumerate(nodes):
+        assert set(n) >= {"output", "name", "shape", "normalized", "operator", "inputs"}
+        assert n["output"] == (n["operator"]["parameter"] if n["name"] == "@param" else "@%d" % i)
+        assert all(j in by_output for j in n["inputs"])
+        assert set(n["shape"]) == {"type", "sub_shapes", "lens", "strides", "dynamic_dimensions", "dyn_strides"}
+    x = by_output["x"]
+    assert x["shape"]["type"] == "float_type" and x["shape"]["lens"] == [4, 256]
+    lit = next(n for n in nodes if n["name"] == "@literal" and n["shape"]["type"] == "uint8_type")
+    data = lit["literal"]["data"]
+    # binary data is an array of bin chunks
+    assert isinstance(data, list) and len(data) == 1 and isinstance(data[0], bytes)
+    assert len(data[0]) == int(np.prod(lit["shape"]["lens"]))
+    unpack = next(n for n in nodes if n["name"] == "unpack_int4")
+    assert unpack["operator"] == {"axis": -1}
+    assert msgpack.packb(doc, use_bin_type=True) == buf
+    assert mgx.load_buffer(msgpack.packb(doc, use_bin_type=True)) == p
+    # an edit made outside survives the trip: rename the parameter
+    for n in nodes:
+        if n["name"] == "@param":
+            n["output"] = n["operator"]["parameter"] = "activations"
+        n["inputs"] = ["activations" if j == "x" else j for j in n["inputs"]]
+    q = mgx.load_buffer(msgpack.packb(doc, use_bin_type=True))
+    assert q.get_parameter_names() == ["activations"] and q.get_output_shapes() == p.get_output_shapes()
+    # JSON form: standard JSON with the same fields
+    import json
+    name_json = json.loads(open_json(p))
+    assert name_json["version"] == 8 and [n["name"] for n in name_json["modules"]["main"]["nodes"]] == \
+        [n["name"] for n in nodes]
+    jl = next(n for n in name_json["modules"]["main"]["nodes"]
+              if n["name"] == "@literal" and n["shape"]["type"] == "uint8_type")
+    assert bytes(jl["literal"]["data"]["bytes"]) == data[0]
+
+
+def open_json(p):
+    import os
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        name = os.path.join(d, "p.json")
+        mgx.save(p, name, format="json")
+        return open(name).read()
