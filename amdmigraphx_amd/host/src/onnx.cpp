@@ -789,7 +789,7 @@ const std::unordered_map<std::string, node_parser>& parsers()
     return table;
 }
 
-program parse_model(wire model)
+program parse_model(wire model, const onnx_options& options)
 {
     // ModelProto.graph = 7
     wire graph{nullptr, nullptr};
@@ -834,14 +834,20 @@ program parse_model(wire model)
     {
         if(values.count(in.name) > 0)
             continue; // an initializer listed among the inputs
-        if(not in.has_shape)
+        if(not in.has_shape and options.map_input_dims.count(in.name) == 0)
             MIGRAPHX_THROW("parse_onnx: input '" + in.name + "' has no shape");
         std::vector<std::size_t> lens;
-        for(auto d : in.dims)
+        auto given = options.map_input_dims.find(in.name);
+        if(given != options.map_input_dims.end())
         {
-            if(d <= 0)
-                MIGRAPHX_THROW("parse_onnx: input '" + in.name + "' has a dynamic dimension");
-            lens.push_back(static_cast<std::size_t>(d));
+            lens = given->second;
+        }
+        else
+        {
+            // an open dimension takes the default size (onnx.cpp:50-66 of the reference: 1 unless set)
+            for(auto d : in.dims)
+                lens.push_back(d > 0 ? static_cast<std::size_t>(d)
+                                     : std::max<std::size_t>(options.default_dim_value, 1));
         }
         const auto t    = get_type(in.elem_type);
         values[in.name] = mm->add_parameter(in.name, lens.empty() ? shape{t} : shape{t, lens});
@@ -882,22 +888,25 @@ program parse_model(wire model)
 
 } // namespace
 
-program parse_onnx_buffer(const void* data, std::size_t size)
+program parse_onnx_buffer(const void* data, std::size_t size, const onnx_options& options)
 {
     const auto* b = static_cast<const unsigned char*>(data);
-    return parse_model(wire{b, b + size});
+    return parse_model(wire{b, b + size}, options);
 }
 
-program parse_onnx_buffer(const std::string& buffer) { return parse_onnx_buffer(buffer.data(), buffer.size()); }
+program parse_onnx_buffer(const std::string& buffer, const onnx_options& options)
+{
+    return parse_onnx_buffer(buffer.data(), buffer.size(), options);
+}
 
-program parse_onnx(const std::string& filename)
+program parse_onnx(const std::string& filename, const onnx_options& options)
 {
     std::ifstream is(filename, std::ios::binary);
     if(not is)
         MIGRAPHX_THROW("parse_onnx: cannot open '" + filename + "'");
     std::stringstream ss;
     ss << is.rdbuf();
-    return parse_onnx_buffer(ss.str());
+    return parse_onnx_buffer(ss.str(), options);
 }
 
 } // namespace migraphx

@@ -14,8 +14,8 @@ def ensure_built():
     """Build the libraries and test programs when they are not there yet."""
     lib = os.path.join(ROOT, "amdmigraphx_amd", "lib")
     need = [os.path.join(lib, "libmi355_qgemm.so"), os.path.join(lib, "libmigraphx.so"),
-            os.path.join(lib, "libmigraphx_mi355.so"), os.path.join(ROOT, "oracle", "liboracle.so"),
-            HOST_TESTS, GPU_TESTS]
+            os.path.join(lib, "libmigraphx_mi355.so"), os.path.join(lib, "libmigraphx_c.so"),
+            os.path.join(ROOT, "oracle", "liboracle.so"), HOST_TESTS, GPU_TESTS, os.path.join(BIN, "capi_tests")]
     if all(os.path.exists(p) for p in need):
         return
     import sys
