@@ -42,6 +42,14 @@ class QuantConvDesc(ctypes.Structure):
                 ("in_type", "out_type", "dequant", "scale_x_mode", "scale_w_mode")]
 
 
+class QuantConv3dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("n", "c", "d", "h", "w", "o", "kd", "kh", "kw")] + \
+               [(n, ctypes.c_int64 * 3) for n in ("pad", "pad_hi", "stride", "dil")] + \
+               [("group", ctypes.c_int64)] + \
+               [(n, ctypes.c_int32) for n in
+                ("in_type", "out_type", "dequant", "scale_x_mode", "scale_w_mode")]
+
+
 class MxDotDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in
                 ("m", "n", "k", "batch", "lda", "ldb", "ldc", "stride_a", "stride_b", "stride_c",
@@ -56,6 +64,10 @@ EXPORTS = {
                                      ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_size_t)],
     "mi355_quant_convolution": [ctypes.POINTER(QuantConvDesc)] + [ctypes.c_void_p] * 6 +
                                [ctypes.c_size_t, ctypes.c_void_p],
+    "mi355_quant_convolution3d_dims": [ctypes.POINTER(QuantConv3dDesc), ctypes.POINTER(ctypes.c_int64),
+                                       ctypes.POINTER(ctypes.c_size_t)],
+    "mi355_quant_convolution3d": [ctypes.POINTER(QuantConv3dDesc)] + [ctypes.c_void_p] * 6 +
+                                 [ctypes.c_size_t, ctypes.c_void_p],
     "mi355_quant_dot": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 8,
     "mi355_quant_dot_bias": [ctypes.POINTER(QuantDotDesc)] + [ctypes.c_void_p] * 9,
     "mi355_quant_dot_workspace_size": [ctypes.POINTER(QuantDotDesc)],

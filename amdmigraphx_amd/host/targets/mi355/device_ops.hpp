@@ -120,9 +120,9 @@ struct quant_dot
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
-// inputs: x [N, C, H, W] or [N, C, W], weights [O, C / group, window...] (both dense),
+// inputs: x [N, C, D, H, W], [N, C, H, W] or [N, C, W], weights [O, C / group, window...] (both dense),
 // [scale_x (one float), scale_w (one float or one per output channel)] (dequant),
-// workspace (uint8, the size mi355_quant_convolution_dims reports), out
+// workspace (uint8, the size mi355_quant_convolution3d_dims reports), out
 struct quant_convolution
 {
     std::vector<int64_t> padding  = {0, 0};
@@ -144,7 +144,7 @@ struct quant_convolution
         f(self.out_type, "out_type");
     }
     std::string name() const { return "mi355::quant_convolution"; }
-    mi355_quant_conv_desc describe(const shape& x, const shape& w) const;
+    mi355_quant_conv3d_desc describe(const shape& x, const shape& w) const;
     shape compute_shape(const std::vector<shape>& inputs) const;
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }

@@ -346,7 +346,7 @@ instruction_ref insert_conv_workspace(module& m, instruction_ref pos, const quan
 {
     const auto d = op.describe(x->get_shape(), w->get_shape());
     size_t need  = 0;
-    if(mi355_quant_convolution_dims(&d, nullptr, nullptr, &need) != MI355_OK)
+    if(mi355_quant_convolution3d_dims(&d, nullptr, &need) != MI355_OK)
         MIGRAPHX_THROW("mi355: quant_convolution attributes are not valid");
     return insert_allocation(m, pos, shape{shape::uint8_type, {std::max<std::size_t>(need, 16)}});
 }
@@ -404,7 +404,7 @@ bool fuse_quant_conv_dq(module& m, instruction_ref dq)
     if(t != shape::int8_type and t != shape::fp8e4m3fn_type)
         return false;
     const std::size_t kd = qc->get_shape().ndim() - 2;
-    if(kd < 1 or kd > 2)
+    if(kd < 1 or kd > 3)
         return false;
 
     instruction_ref last   = dq;

@@ -355,32 +355,38 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     return args.back();
 }
 
-mi355_quant_conv_desc quant_convolution::describe(const shape& x, const shape& w) const
+mi355_quant_conv3d_desc quant_convolution::describe(const shape& x, const shape& w) const
 {
     const std::size_t kd = stride.size();
-    if(kd < 1 or kd > 2 or dilation.size() != kd or (padding.size() != kd and padding.size() != 2 * kd))
-        MIGRAPHX_THROW("mi355::quant_convolution: one or two spatial dimensions with matching attributes");
+    if(kd < 1 or kd > 3 or dilation.size() != kd or (padding.size() != kd and padding.size() != 2 * kd))
+        MIGRAPHX_THROW("mi355::quant_convolution: one to three spatial dimensions with matching attributes");
     if(x.ndim() != kd + 2 or w.ndim() != kd + 2)
         MIGRAPHX_THROW("mi355::quant_convolution: input rank does not match the attributes");
-    const bool two = kd == 2;
     const bool both_sides = padding.size() == 2 * kd; // low values first, then high values
-    mi355_quant_conv_desc d{};
-    d.n        = static_cast<int64_t>(x.lens()[0]);
-    d.c        = static_cast<int64_t>(x.lens()[1]);
-    d.h        = two ? static_cast<int64_t>(x.lens()[2]) : 1;
-    d.w        = static_cast<int64_t>(x.lens()[kd + 1]);
-    d.o        = static_cast<int64_t>(w.lens()[0]);
-    d.kh       = two ? static_cast<int64_t>(w.lens()[2]) : 1;
-    d.kw       = static_cast<int64_t>(w.lens()[kd + 1]);
-    d.pad_h    = two ? padding[0] : 0;
-    d.pad_w    = padding[kd - 1];
-    d.stride_h = two ? stride[0] : 1;
-    d.stride_w = stride[kd - 1];
-    d.dil_h    = two ? dilation[0] : 1;
-    d.dil_w    = dilation[kd - 1];
+    const std::size_t lead = 3 - kd;                  // missing leading axes have length one
+    mi355_quant_conv3d_desc d{};
+    int64_t in[3]  = {1, 1, 1};
+    int64_t win[3] = {1, 1, 1};
+    for(std::size_t i = 0; i < 3; i++)
+    {
+        d.stride[i] = 1;
+        d.dil[i]    = 1;
+    }
+    for(std::size_t i = 0; i < kd; i++)
+    {
+        in[lead + i]       = static_cast<int64_t>(x.lens()[2 + i]);
+        win[lead + i]      = static_cast<int64_t>(w.lens()[2 + i]);
+        d.pad[lead + i]    = padding[i];
+        d.pad_hi[lead + i] = padding[both_sides ? kd + i : i];
+        d.stride[lead + i] = stride[i];
+        d.dil[lead + i]    = dilation[i];
+    }
+    d.n = static_cast<int64_t>(x.lens()[0]);
+    d.c = static_cast<int64_t>(x.lens()[1]);
+    d.o = static_cast<int64_t>(w.lens()[0]);
+    d.d = in[0], d.h = in[1], d.w = in[2];
+    d.kd = win[0], d.kh = win[1], d.kw = win[2];
     d.group    = group;
-    d.pad_h_hi = two ? padding[both_sides ? kd : 0] : 0;
-    d.pad_w_hi = padding[both_sides ? 2 * kd - 1 : kd - 1];
     d.in_type  = to_mi355_type(x.type());
     d.out_type = to_mi355_type(out_type);
     d.dequant  = dequant ? 1 : 0;
@@ -416,7 +422,7 @@ shape quant_convolution::compute_shape(const std::vector<shape>& inputs) const
     }
     const auto d = describe(inputs[0], inputs[1]);
     size_t need  = 0;
-    status_check(mi355_quant_convolution_dims(&d, nullptr, nullptr, &need), name());
+    status_check(mi355_quant_convolution3d_dims(&d, nullptr, &need), name());
     const shape& ws = inputs[inputs.size() - 2];
     if(ws.type() != shape::uint8_type or not ws.standard() or ws.bytes() < need)
         MIGRAPHX_THROW("mi355::quant_convolution: workspace too small");
@@ -433,7 +439,7 @@ quant_convolution::compute(migraphx::context& ctx, const shape&, const std::vect
     const float* sx = dequant ? reinterpret_cast<const float*>(args[2].data()) : nullptr;
     const float* sw = dequant ? reinterpret_cast<const float*>(args[3].data()) : nullptr;
     const argument& ws = args[args.size() - 2];
-    status_check(mi355_quant_convolution(&d,
+    status_check(mi355_quant_convolution3d(&d,
                                          args[0].data(),
                                          args[1].data(),
                                          args.back().data(),

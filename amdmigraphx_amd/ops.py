@@ -11,7 +11,7 @@ import ctypes
 
 import torch
 
-from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConvDesc, MxDotDesc, Mi355Error, check, lib
+from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConv3dDesc, QuantConvDesc, MxDotDesc, Mi355Error, check, lib
 
 _TORCH2DT = {torch.int8: DT.I8, torch.uint8: DT.U8, torch.int32: DT.I32, torch.float32: DT.F32,
              torch.float16: DT.F16, torch.bfloat16: DT.BF16}
@@ -223,46 +223,69 @@ def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False, fp8=False):
     return int(lib().mi355_quant_dot_workspace_size(ctypes.byref(d)))
 
 
-def quant_convolution(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1, fp8=False,
+def quant_convolution(x, w, padding=None, stride=None, dilation=None, group=1, fp8=False,
                       scale_x=None, scale_w=None, out_dtype=None):
-    """quant_convolution of a dense [N, C, H, W] tensor with dense [O, C/group, KH, KW] weights
-    (int8, or uint8 carrying fp8 e4m3fn codes with fp8=True), optionally with the dequantizing
-    epilogue: ``scale_x`` one float, ``scale_w`` one float or one per output channel.  ``padding``
-    is (h, w) for both sides or (h_low, w_low, h_high, w_high)."""
+    """quant_convolution of a dense [N, C, spatial...] tensor with dense [O, C/group, window...]
+    weights over one, two or three spatial axes (int8, or uint8 carrying fp8 e4m3fn codes with
+    fp8=True), optionally with the dequantizing epilogue: ``scale_x`` one float, ``scale_w`` one
+    float or one per output channel.  ``padding`` holds one value per spatial axis for both sides,
+    or the low values followed by the high ones."""
     _require_cuda(x, w, scale_x, scale_w)
-    if x.dim() != 4 or w.dim() != 4:
-        raise Mi355Error("QUANT_CONVOLUTION: input and weights must have four dimensions")
+    nd = x.dim() - 2
+    if nd < 1 or nd > 3 or w.dim() != x.dim():
+        raise Mi355Error("QUANT_CONVOLUTION: input and weights must have 3 to 5 dimensions, and the same number")
     if x.dtype != w.dtype:
         raise Mi355Error("QUANT_CONVOLUTION: Types do not match")
     if not x.is_contiguous() or not w.is_contiguous():
         raise Mi355Error("quant_convolution: input and weights must be dense")
-    n, c, h, wd = x.shape
-    o, cg, kh, kw = w.shape
+    padding = list(padding) if padding is not None else [0] * nd
+    stride = list(stride) if stride is not None else [1] * nd
+    dilation = list(dilation) if dilation is not None else [1] * nd
+    if len(padding) not in (nd, 2 * nd) or len(stride) != nd or len(dilation) != nd:
+        raise Mi355Error("QUANT_CONVOLUTION: inconsistent attribute sizes")
+    n, c = x.shape[:2]
+    o, cg = w.shape[:2]
     if group < 1 or cg * group != c or o % group != 0:
         raise Mi355Error("QUANT_CONVOLUTION: mismatched channel numbers")
     dequant = scale_x is not None or scale_w is not None or out_dtype is not None
     odt = (out_dtype or torch.float32) if dequant else (torch.float32 if fp8 else torch.int32)
-    pad_hi = padding[2:] if len(padding) == 4 else padding
-    d = QuantConvDesc(n=n, c=c, h=h, w=wd, o=o, kh=kh, kw=kw, pad_h=padding[0], pad_w=padding[1],
-                      pad_h_hi=pad_hi[0], pad_w_hi=pad_hi[1],
-                      stride_h=stride[0], stride_w=stride[1], dil_h=dilation[0], dil_w=dilation[1],
-                      group=group, in_type=DT.FP8 if fp8 else DT.I8, out_type=_TORCH2DT[odt],
-                      dequant=int(dequant),
-                      scale_x_mode=QP.NONE if scale_x is None else QP.PER_TENSOR,
-                      scale_w_mode=QP.NONE if scale_w is None else
-                      (QP.PER_TENSOR if scale_w.numel() == 1 else QP.PER_ROW))
+    pad_hi = padding[nd:] if len(padding) == 2 * nd else padding
     if scale_x is not None and scale_x.numel() != 1:
         raise Mi355Error("scale_x must be a single value")
     if scale_w is not None and scale_w.numel() not in (1, o):
         raise Mi355Error("scale_w must be a scalar or have one value per output channel")
-    oh, ow, need = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_size_t()
-    check(lib().mi355_quant_convolution_dims(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow),
-                                             ctypes.byref(need)), "mi355_quant_convolution_dims")
-    out = torch.empty((n, o, oh.value, ow.value), dtype=odt, device=x.device)
+    common = dict(group=group, in_type=DT.FP8 if fp8 else DT.I8, out_type=_TORCH2DT[odt], dequant=int(dequant),
+                  scale_x_mode=QP.NONE if scale_x is None else QP.PER_TENSOR,
+                  scale_w_mode=QP.NONE if scale_w is None else
+                  (QP.PER_TENSOR if scale_w.numel() == 1 else QP.PER_ROW))
+    need = ctypes.c_size_t()
+    if nd == 2:
+        d = QuantConvDesc(n=n, c=c, h=x.shape[2], w=x.shape[3], o=o, kh=w.shape[2], kw=w.shape[3],
+                          pad_h=padding[0], pad_w=padding[1], pad_h_hi=pad_hi[0], pad_w_hi=pad_hi[1],
+                          stride_h=stride[0], stride_w=stride[1], dil_h=dilation[0], dil_w=dilation[1], **common)
+        oh, ow = ctypes.c_int64(), ctypes.c_int64()
+        check(lib().mi355_quant_convolution_dims(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow),
+                                                 ctypes.byref(need)), "mi355_quant_convolution_dims")
+        out_spatial = [oh.value, ow.value]
+        run, what = lib().mi355_quant_convolution, "mi355_quant_convolution"
+    else:
+        # one spatial axis: a depth and a height of one in front
+        lead = 3 - nd
+        three = ctypes.c_int64 * 3
+        sp = [1] * lead + list(x.shape[2:])
+        win = [1] * lead + list(w.shape[2:])
+        d = QuantConv3dDesc(n=n, c=c, d=sp[0], h=sp[1], w=sp[2], o=o, kd=win[0], kh=win[1], kw=win[2],
+                            pad=three(*([0] * lead + padding[:nd])), pad_hi=three(*([0] * lead + list(pad_hi))),
+                            stride=three(*([1] * lead + stride)), dil=three(*([1] * lead + dilation)), **common)
+        lens = three()
+        check(lib().mi355_quant_convolution3d_dims(ctypes.byref(d), lens, ctypes.byref(need)),
+              "mi355_quant_convolution3d_dims")
+        out_spatial = list(lens)[lead:]
+        run, what = lib().mi355_quant_convolution3d, "mi355_quant_convolution3d"
+    out = torch.empty((n, o, *out_spatial), dtype=odt, device=x.device)
     workspace = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
-    check(lib().mi355_quant_convolution(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(out), _ptr(scale_x),
-                                        _ptr(scale_w), _ptr(workspace), need.value, _stream()),
-          "mi355_quant_convolution")
+    check(run(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(out), _ptr(scale_x), _ptr(scale_w), _ptr(workspace),
+              need.value, _stream()), what)
     return out
 
 

@@ -163,6 +163,25 @@ int mi355_quant_convolution(const mi355_quant_conv_desc* desc, const void* x, co
                             const float* scale_x, const float* scale_w, void* workspace,
                             size_t workspace_bytes, void* stream);
 
+/* The same over three spatial axes: input [N, C, D, H, W], weights [O, C / group, KD, KH, KW],
+ * output [N, O, OD, OH, OW]  (ref: convolution.hpp:37-100 loops over any number of spatial axes;
+ * op/quant_convolution.hpp:52-157 accepts one to three).  pad / pad_hi / stride / dil hold one
+ * value per spatial axis in the order depth, height, width.  The two-dimensional entry points are
+ * this one with a depth of one. */
+typedef struct mi355_quant_conv3d_desc {
+    int64_t n, c, d, h, w;
+    int64_t o, kd, kh, kw;
+    int64_t pad[3], pad_hi[3], stride[3], dil[3];
+    int64_t group;
+    int32_t in_type, out_type, dequant, scale_x_mode, scale_w_mode;   /* as in mi355_quant_conv_desc */
+} mi355_quant_conv3d_desc;
+/* out_lens: OD, OH, OW */
+int mi355_quant_convolution3d_dims(const mi355_quant_conv3d_desc* desc, int64_t* out_lens,
+                                   size_t* workspace_bytes);
+int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* desc, const void* x, const void* w, void* out,
+                              const float* scale_x, const float* scale_w, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* The same with a workspace.  A quant_dot that launches fewer workgroups than the chip has CUs
  * (a skinny or mid-size A against a large B, one image of a convolution) is split along K.
  * Without a workspace only the bare int8 product is split (the shares are added into C with

@@ -55,6 +55,8 @@ def _load():
     lib.orc_fp4_from_f32.restype = ctypes.c_uint8
     lib.orc_convolution.argtypes = [vp, ci, vp, vp, ci] + [i64] * 16
     lib.orc_convolution.restype = None
+    lib.orc_convolution3d.argtypes = [vp, ci, vp, vp, ci, i64, i64, vp, i64, vp, vp, vp, vp, i64, vp]
+    lib.orc_convolution3d.restype = None
     lib.orc_convert.argtypes = [vp, ci, vp, ci, ctypes.c_size_t]
     lib.orc_convert.restype = None
     lib.orc_mul_f32.argtypes = [vp, vp, i64, i64, vp, i64, i64, i64, i64]
@@ -148,22 +150,34 @@ def conv_out_len(in_len, k, pad, stride, dilation, pad_hi=None):
     return max(1, int(span / stride) + 1)
 
 
-def convolution(x, w, x_type, padding=(0, 0), stride=(1, 1), dilation=(1, 1), group=1):
-    """convolution / quant_convolution of an [N, C, H, W] input with [O, C/group, KH, KW] weights:
-    int8 -> int32, fp8 -> float (double products), float -> float (float products, double sum)."""
+def convolution(x, w, x_type, padding=None, stride=None, dilation=None, group=1):
+    """convolution / quant_convolution of an [N, C, spatial...] input with [O, C/group, window...]
+    weights over one, two or three spatial axes: int8 -> int32, fp8 -> float (double products),
+    float -> float (float products, double sum).  `padding` holds one value per axis, or the low
+    values followed by the high ones."""
     x = _c(x, _NP[x_type])
     w = _c(w, _NP[x_type])
-    n, c, h, wd = x.shape
-    o, cg, kh, kw = w.shape
+    nd = x.ndim - 2
+    assert 1 <= nd <= 3 and w.ndim == x.ndim
+    padding = list(padding) if padding is not None else [0] * nd
+    stride = list(stride) if stride is not None else [1] * nd
+    dilation = list(dilation) if dilation is not None else [1] * nd
+    n, c = x.shape[:2]
+    o, cg = w.shape[:2]
     assert cg * group == c and o % group == 0
-    hi = padding[2:] if len(padding) == 4 else padding   # (h_low, w_low, h_high, w_high) form
-    oh = conv_out_len(h, kh, padding[0], stride[0], dilation[0], hi[0])
-    ow = conv_out_len(wd, kw, padding[1], stride[1], dilation[1], hi[1])
+    hi = padding[nd:] if len(padding) == 2 * nd else padding   # (low..., high...) form
+    out_sp = [conv_out_len(x.shape[2 + i], w.shape[2 + i], padding[i], stride[i], dilation[i], hi[i])
+              for i in range(nd)]
     out_type = I32 if x_type == I8 else F32
-    out = np.empty((n, o, oh, ow), _NP[out_type])
-    _lib.orc_convolution(_p(out), out_type, _p(x), _p(w), x_type, n, c, h, wd, o, kh, kw,
-                         padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1],
-                         group, oh, ow)
+    out = np.empty((n, o, *out_sp), _NP[out_type])
+    lead = 3 - nd                                              # missing leading axes have length one
+
+    def arr(v, fill):
+        return np.ascontiguousarray([fill] * lead + [int(e) for e in v[:nd]], np.int64)
+
+    a = [arr(x.shape[2:], 1), arr(w.shape[2:], 1), arr(padding, 0), arr(stride, 1), arr(dilation, 1), arr(out_sp, 1)]
+    _lib.orc_convolution3d(_p(out), out_type, _p(x), _p(w), x_type, n, c, _p(a[0]), o, _p(a[1]), _p(a[2]),
+                           _p(a[3]), _p(a[4]), group, _p(a[5]))
     return out
 
 

@@ -463,14 +463,77 @@ void orc_gemm(void* c,
  * convolution  src/include/migraphx/convolution.hpp:37-100, called by
  *   op::quant_convolution::compute  src/include/migraphx/op/quant_convolution.hpp:142-157
  *   op::convolution::compute        src/include/migraphx/op/convolution.hpp:208-239
- * Cross-correlation of an [N, C, H, W] input with [O, C/group, KH, KW] weights: the window of
- * output (n, o, y, x) starts at (y*stride - pad, x*stride - pad), steps by the dilation, and
- * positions outside the input contribute nothing.  Output channel o reads the input channels of
- * group o / (O / group).  The sum runs over (channel, kh, kw) in that order in a double.
+ * Cross-correlation of an [N, C, D, H, W] input with [O, C/group, KD, KH, KW] weights (the
+ * reference's loop runs over any number of spatial axes; one, two and three are what its operators
+ * accept): the window of output (n, o, z, y, x) starts at (z*stride - pad, y*stride - pad,
+ * x*stride - pad), steps by the dilation, and positions outside the input contribute nothing.
+ * Output channel o reads the input channels of group o / (O / group).  The sum runs over
+ * (channel, kd, kh, kw) in that order in a double.
  * quant_convolution converts both tensors to double first (get_all<double>), so each product is
  * a double product; the float operator multiplies in float and adds the rounded product.
  * One conversion to the output type at the end.
  * ---------------------------------------------------------------------- */
+void orc_convolution3d(void* out,
+                       int out_type,
+                       const void* x,
+                       const void* w,
+                       int x_type,
+                       int64_t n,
+                       int64_t c,
+                       const int64_t* in_lens,  /* D, H, W of the input */
+                       int64_t o,
+                       const int64_t* win_lens, /* KD, KH, KW */
+                       const int64_t* pad,      /* zeros in front of each spatial axis */
+                       const int64_t* stride,
+                       const int64_t* dil,
+                       int64_t group,
+                       const int64_t* out_lens) /* OD, OH, OW */
+{
+    const int64_t cg    = c / group; /* input channels per group = weights' second dimension */
+    const int64_t og    = o / group;
+    const int64_t d = in_lens[0], h = in_lens[1], wd = in_lens[2];
+    const int64_t kd = win_lens[0], kh = win_lens[1], kw = win_lens[2];
+    const int64_t od = out_lens[0], oh = out_lens[1], ow = out_lens[2];
+    const int64_t total = n * o * od * oh * ow;
+#pragma omp parallel for schedule(static)
+    for(int64_t idx = 0; idx < total; idx++)
+    {
+        const int64_t ox = idx % ow;
+        const int64_t oy = (idx / ow) % oh;
+        const int64_t oz = (idx / (ow * oh)) % od;
+        const int64_t oc = (idx / (ow * oh * od)) % o;
+        const int64_t b  = idx / (ow * oh * od * o);
+        const int64_t g  = oc / og;
+        double acc       = 0.0;
+        for(int64_t k = 0; k < cg; k++)
+        {
+            const int64_t ic = g * cg + k;
+            for(int64_t t = 0; t < kd; t++)
+            {
+                const int64_t iz = oz * stride[0] - pad[0] + t * dil[0];
+                for(int64_t r = 0; r < kh; r++)
+                {
+                    const int64_t iy = oy * stride[1] - pad[1] + r * dil[1];
+                    for(int64_t q = 0; q < kw; q++)
+                    {
+                        const int64_t ix = ox * stride[2] - pad[2] + q * dil[2];
+                        if(iz < 0 || iz >= d || iy < 0 || iy >= h || ix < 0 || ix >= wd)
+                            continue;
+                        const size_t xi = (size_t)((((b * c + ic) * d + iz) * h + iy) * wd + ix);
+                        const size_t wi = (size_t)((((oc * cg + k) * kd + t) * kh + r) * kw + q);
+                        if(x_type == ORC_F32)
+                            acc += ((const float*)x)[xi] * ((const float*)w)[wi];
+                        else
+                            acc += load_f64(x, x_type, xi) * load_f64(w, x_type, wi);
+                    }
+                }
+            }
+        }
+        store_f64(out, out_type, (size_t)idx, acc);
+    }
+}
+
+/* the two-dimensional case: a depth of one */
 void orc_convolution(void* out,
                      int out_type,
                      const void* x,
@@ -493,40 +556,13 @@ void orc_convolution(void* out,
                      int64_t oh,
                      int64_t ow)
 {
-    const int64_t cg    = c / group; /* input channels per group = weights' second dimension */
-    const int64_t og    = o / group;
-    const int64_t total = n * o * oh * ow;
-#pragma omp parallel for schedule(static)
-    for(int64_t idx = 0; idx < total; idx++)
-    {
-        const int64_t ox = idx % ow;
-        const int64_t oy = (idx / ow) % oh;
-        const int64_t oc = (idx / (ow * oh)) % o;
-        const int64_t b  = idx / (ow * oh * o);
-        const int64_t g  = oc / og;
-        double acc       = 0.0;
-        for(int64_t k = 0; k < cg; k++)
-        {
-            const int64_t ic = g * cg + k;
-            for(int64_t r = 0; r < kh; r++)
-            {
-                const int64_t iy = oy * stride_h - pad_h + r * dil_h;
-                for(int64_t q = 0; q < kw; q++)
-                {
-                    const int64_t ix = ox * stride_w - pad_w + q * dil_w;
-                    if(iy < 0 || iy >= h || ix < 0 || ix >= wd)
-                        continue;
-                    const size_t xi = (size_t)(((b * c + ic) * h + iy) * wd + ix);
-                    const size_t wi = (size_t)(((oc * cg + k) * kh + r) * kw + q);
-                    if(x_type == ORC_F32)
-                        acc += ((const float*)x)[xi] * ((const float*)w)[wi];
-                    else
-                        acc += load_f64(x, x_type, xi) * load_f64(w, x_type, wi);
-                }
-            }
-        }
-        store_f64(out, out_type, (size_t)idx, acc);
-    }
+    const int64_t in_lens[3]  = {1, h, wd};
+    const int64_t win_lens[3] = {1, kh, kw};
+    const int64_t pad[3]      = {0, pad_h, pad_w};
+    const int64_t stride[3]   = {1, stride_h, stride_w};
+    const int64_t dil[3]      = {1, dil_h, dil_w};
+    const int64_t out_lens[3] = {1, oh, ow};
+    orc_convolution3d(out, out_type, x, w, x_type, n, c, in_lens, o, win_lens, pad, stride, dil, group, out_lens);
 }
 
 /* ------------------------------------------------------------------------

@@ -356,8 +356,11 @@ TEST_CASE(quant_convolution_programs)
         std::vector<std::size_t> xl, wl;
         std::vector<int64_t> padding, stride;
     };
+    // and volumes: the shapes of test/ref/convolution.cpp:991-1060 and test/verify/test_conv3d.cpp
     for(const auto& c : {bare{{2, 3, 4, 4}, {2, 3, 3, 3}, {0, 0}, {1, 1}}, bare{{2, 3, 4, 4}, {2, 3, 3, 3}, {1, 1}, {2, 2}},
-                         bare{{4, 3, 32, 32}, {16, 3, 5, 5}, {2, 2}, {1, 1}}})
+                         bare{{4, 3, 32, 32}, {16, 3, 5, 5}, {2, 2}, {1, 1}},
+                         bare{{2, 3, 4, 4, 1}, {2, 3, 3, 3, 1}, {0, 0, 0}, {1, 1, 1}},
+                         bare{{4, 3, 5, 5, 5}, {4, 3, 3, 3, 3}, {1, 0, 2}, {1, 2, 1}}})
     {
         program p;
         auto* mm = p.get_main_module();
@@ -365,7 +368,8 @@ TEST_CASE(quant_convolution_programs)
         shape sw{shape::int8_type, c.wl};
         auto x = mm->add_parameter("x", sx);
         auto w = mm->add_parameter("w", sw);
-        mm->add_return({mm->add_instruction(conv(c.padding, c.stride, {1, 1}, 1, "quant_convolution"), x, w)});
+        mm->add_return({mm->add_instruction(
+            conv(c.padding, c.stride, std::vector<int64_t>(c.stride.size(), 1), 1, "quant_convolution"), x, w)});
         expect_same(p, {{"x", argument{sx, uniform_ints<int>(sx.elements(), -128, 127, 31)}},
                         {"w", argument{sw, uniform_ints<int>(sw.elements(), -128, 127, 32)}}});
     }
@@ -383,6 +387,10 @@ TEST_CASE(quant_convolution_programs)
                          layer{{2, 8, 10, 10}, {12, 2, 3, 3}, {2, 1}, {1, 2}, {2, 1}, 4, false, shape::float_type},
                          layer{{2, 16, 9, 9}, {16, 16, 1, 1}, {0, 0}, {1, 1}, {1, 1}, 1, true, shape::half_type},
                          layer{{2, 6, 40}, {10, 6, 5}, {2}, {3}, {1}, 1, true, shape::float_type},
+                         // three spatial axes: per-channel scales, groups, low / high padding
+                         layer{{2, 8, 6, 7, 5}, {12, 8, 3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {1, 1, 1}, 1, true, shape::float_type},
+                         layer{{1, 32, 5, 6, 6}, {8, 16, 2, 3, 2}, {0, 1, 0, 1, 0, 1}, {1, 2, 1}, {2, 1, 1}, 2, false,
+                               shape::float_type},
                          // SAME_UPPER-style padding: none in front, one behind
                          layer{{1, 8, 8, 8}, {8, 8, 3, 3}, {0, 0, 1, 1}, {2, 2}, {1, 1}, 1, true, shape::float_type}})
     {

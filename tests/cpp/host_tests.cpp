@@ -599,6 +599,14 @@ TEST_CASE(quant_convolution_shapes)
     EXPECT(out({shape::float_type, {1, 4, 10}}, {shape::float_type, {6, 2, 3}},
                make_op("convolution", {{"padding", {1}}, {"stride", {2}}, {"dilation", {1}}, {"group", 2}})) ==
            shape{shape::float_type, {1, 6, 5}});
+    // three spatial axes, the shapes of test/ref/convolution.cpp:859-1060 and one with every attribute
+    EXPECT(out({shape::int8_type, {2, 3, 4, 4, 1}}, {shape::int8_type, {2, 3, 3, 3, 1}},
+               make_op("quant_convolution", {{"padding", {0, 0, 0}}, {"stride", {1, 1, 1}}, {"dilation", {1, 1, 1}}})) ==
+           shape{shape::int32_type, {2, 2, 2, 2, 1}});
+    EXPECT(out({shape::int8_type, {1, 4, 9, 8, 7}}, {shape::int8_type, {6, 2, 3, 2, 3}},
+               make_op("quant_convolution",
+                       {{"padding", {1, 0, 2, 0, 1, 2}}, {"stride", {2, 1, 3}}, {"dilation", {1, 2, 1}}, {"group", 2}})) ==
+           shape{shape::int32_type, {1, 6, 4, 7, 3}});
     EXPECT(test::throws([&] {
         out({shape::int8_type, {2, 3, 4, 4}}, {shape::int8_type, {2, 2, 3, 3}}, make_op("quant_convolution"));
     }));
@@ -639,6 +647,30 @@ TEST_CASE(quant_convolution_known_answers)
         EXPECT(r[0].get_shape() == shape{shape::int32_type, {2, 2, 2, 2}});
         EXPECT(r[0].to_vector<int>() == c.gold);
     }
+}
+
+TEST_CASE(convolution_three_spatial_axes_on_cpu)
+{
+    // int8 operands over a volume on the CPU target against sums written out here: every output of
+    // a 2 x 2 x 2 window over a 3 x 3 x 3 volume of ones times weights 1..8 is 36, a border of
+    // zeros removes the weights that fall outside
+    program p;
+    auto* mm = p.get_main_module();
+    std::vector<int> w(8);
+    std::iota(w.begin(), w.end(), 1);
+    auto x  = mm->add_literal(literal{shape{shape::int8_type, {1, 1, 3, 3, 3}}, std::vector<int>(27, 1)});
+    auto wl = mm->add_literal(literal{shape{shape::int8_type, {1, 1, 2, 2, 2}}, w});
+    auto plain = mm->add_instruction(
+        make_op("quant_convolution", {{"padding", {0, 0, 0}}, {"stride", {1, 1, 1}}, {"dilation", {1, 1, 1}}}), x, wl);
+    auto padded = mm->add_instruction(
+        make_op("quant_convolution", {{"padding", {1, 0, 0}}, {"stride", {2, 1, 1}}, {"dilation", {1, 1, 1}}}), x, wl);
+    mm->add_return({plain, padded});
+    auto r = run_on("oracle", p, {});
+    EXPECT(r[0].get_shape() == shape{shape::int32_type, {1, 1, 2, 2, 2}});
+    EXPECT(r[0].to_vector<int>() == std::vector<int>(8, 36));
+    // depth positions -1..0 (only the window's second plane, weights 5..8, sees data) and 1..2
+    EXPECT(r[1].get_shape() == shape{shape::int32_type, {1, 1, 2, 2, 2}});
+    EXPECT(r[1].to_vector<int>() == std::vector<int>{26, 26, 26, 26, 36, 36, 36, 36});
 }
 
 TEST_CASE(qdq_conv)

@@ -12,10 +12,10 @@ extern "C" {
 void orc_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, int64_t m, int64_t n,
               int64_t k, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn, int64_t batch,
               int64_t a_sb, int64_t b_sb);
-void orc_convolution(void* out, int out_type, const void* x, const void* w, int x_type, int64_t n,
-                     int64_t c, int64_t h, int64_t wd, int64_t o, int64_t kh, int64_t kw, int64_t pad_h,
-                     int64_t pad_w, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w,
-                     int64_t group, int64_t oh, int64_t ow);
+void orc_convolution3d(void* out, int out_type, const void* x, const void* w, int x_type, int64_t n,
+                       int64_t c, const int64_t* in_lens, int64_t o, const int64_t* win_lens,
+                       const int64_t* pad, const int64_t* stride, const int64_t* dil, int64_t group,
+                       const int64_t* out_lens);
 void orc_quantizelinear(void* out, int out_type, const void* x, int x_type, const void* scale,
                         int64_t s_sr, int64_t s_sc, const void* zp, int64_t z_sr, int64_t z_sc,
                         int64_t rows, int64_t cols);
@@ -150,24 +150,32 @@ struct cpu_op
         }
         else if(n == "convolution" or n == "quant_convolution")
         {
-            // one or two spatial dimensions (a 1-D convolution is a 2-D one of height 1)
+            // one to three spatial dimensions; missing leading ones have length one
             const auto v        = op.to_value();
             const auto padding  = v.at("padding").to_vector<int64_t>();
             const auto stride   = v.at("stride").to_vector<int64_t>();
             const auto dilation = v.at("dilation").to_vector<int64_t>();
             const std::size_t kd = stride.size();
-            if(args.size() != 2 or kd < 1 or kd > 2)
+            if(args.size() != 2 or kd < 1 or kd > 3)
                 MIGRAPHX_THROW("oracle: convolution with " + std::to_string(kd) + " spatial dimensions");
             argument x = dense(args[0]);
             argument w = dense(args[1]);
             const auto& xl = x.get_shape().lens();
             const auto& wl = w.get_shape().lens();
-            const bool two = kd == 2;
-            orc_convolution(r.data(), orc_type(out.type()), x.data(), w.data(), orc_type(x.get_shape().type()),
-                            xl[0], xl[1], two ? xl[2] : 1, xl[kd + 1], wl[0], two ? wl[2] : 1, wl[kd + 1],
-                            two ? padding[0] : 0, padding[kd - 1], two ? stride[0] : 1, stride[kd - 1],
-                            two ? dilation[0] : 1, dilation[kd - 1], v.at("group").to<int64_t>(),
-                            two ? out.lens()[2] : 1, out.lens()[kd + 1]);
+            const std::size_t lead = 3 - kd;
+            int64_t in[3] = {1, 1, 1}, win[3] = {1, 1, 1}, pad[3] = {0, 0, 0}, st[3] = {1, 1, 1},
+                    dil[3] = {1, 1, 1}, ol[3] = {1, 1, 1};
+            for(std::size_t i = 0; i < kd; i++)
+            {
+                in[lead + i]  = xl[2 + i];
+                win[lead + i] = wl[2 + i];
+                pad[lead + i] = padding[i]; // the low side; the high side only enters the output size
+                st[lead + i]  = stride[i];
+                dil[lead + i] = dilation[i];
+                ol[lead + i]  = out.lens()[2 + i];
+            }
+            orc_convolution3d(r.data(), orc_type(out.type()), x.data(), w.data(), orc_type(x.get_shape().type()),
+                              xl[0], xl[1], in, wl[0], win, pad, st, dil, v.at("group").to<int64_t>(), ol);
         }
         else if(n == "quantizelinear" or n == "dequantizelinear")
         {

@@ -314,6 +314,16 @@ c = {"name": "conv2d_grouped_test", "source": "test/ref/convolution.cpp:761-857"
      "x": vec(body, "a"), "w": vec(body, "c"), "gold": vec(body, "gold")}
 c.update(conv_attrs(body, "convolution"))
 conv.append(c)
+# three spatial axes: the float operator's known answers pin the loop order and the indexing of
+# the shared convolution routine (quant_convolution calls the same one)
+for name, where in (("conv3d_test", "test/ref/convolution.cpp:991-1060"),
+                    ("conv3d_grouped_test", "test/ref/convolution.cpp:859-989")):
+    body = cases[name]
+    c = {"name": name, "source": where, "type": "float",
+         "x_lens": shape(body, "a_shape")["lens"], "w_lens": shape(body, "c_shape")["lens"],
+         "x": vec(body, "a"), "w": vec(body, "c"), "gold": vec(body, "gold")}
+    c.update(conv_attrs(body, "convolution"))
+    conv.append(c)
 out["convolution"] = conv
 
 # ---- ONNX Q/DQ models with their expected outputs (test/onnx/verify/*_blocked_test.cpp) ---------

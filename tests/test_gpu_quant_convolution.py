@@ -1,5 +1,5 @@
-"""GPU parity of quant_convolution (im2col + the quantized GEMM) through the C ABI against the
-CPU oracle: int32 results bit-exact, dequantized results bit-exact for int8, fp8 within the
+"""GPU parity of quant_convolution (im2col + the quantized GEMM, one to three spatial axes) through
+the C ABI against the CPU oracle: int32 results bit-exact, dequantized results bit-exact for int8, fp8 within the
 accumulation tolerance of the fp8 matrix instructions."""
 import numpy as np
 import pytest
@@ -109,6 +109,66 @@ def test_int8_dequant_epilogue_with_split_k(ops, out):
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.BF16))
 
 
+VOLUME_CASES = [
+    # x shape, w shape, padding, stride, dilation, group: three spatial axes, then one
+    ((2, 4, 5, 6, 7), (6, 4, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),           # K = 108 -> 128
+    ((1, 6, 6, 5, 4), (4, 3, 2, 3, 1), (1, 0, 2), (2, 1, 1), (1, 2, 1), 2),           # groups, strides, dilation
+    ((2, 4, 7, 4, 5), (4, 1, 3, 2, 2), (0, 1, 0, 2, 0, 1), (1, 2, 3), (2, 1, 1), 4),  # depthwise, low / high padding
+    ((1, 3, 4, 4, 4), (2, 3, 1, 1, 1), (0, 0, 0), (2, 2, 2), (1, 1, 1), 1),           # pointwise with strides
+    ((2, 32, 4, 6, 5), (24, 16, 3, 3, 3), (1, 1, 1), (1, 2, 1), (1, 1, 1), 2),        # channels-last gather
+    ((1, 16, 8, 7, 6), (40, 16, 2, 3, 2), (0, 1, 1, 1, 0, 0), (1, 1, 1), (2, 1, 2), 1),
+    ((1, 64, 6, 6, 6), (64, 64, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),        # K = 1728: split K
+    ((3, 2, 9), (4, 2, 3), (1,), (2,), (2,), 1),                                      # [N, C, W]
+    ((2, 32, 40), (6, 16, 5), (2, 0), (1,), (3,), 2),
+]
+
+
+@pytest.mark.parametrize("xs,ws,padding,stride,dilation,group", VOLUME_CASES)
+def test_int8_one_and_three_spatial_axes_bit_exact(ops, xs, ws, padding, stride, dilation, group):
+    rng = np.random.default_rng(sum(xs) * 5 + sum(ws))
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    want = orc.convolution(x, w, orc.I8, padding, stride, dilation, group)
+    print("conv int8", xs, ws, padding, stride, dilation, group, flush=True)
+    got = ops.quant_convolution(dev(x), dev(w), padding, stride, dilation, group)
+    assert got.dtype == torch.int32 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_volume_of_depth_one_equals_the_image(ops):
+    """The two-dimensional entry point and the three-dimensional one agree where they overlap."""
+    rng = np.random.default_rng(12)
+    x = rng.integers(-128, 128, (2, 16, 9, 8), dtype=np.int8)
+    w = rng.integers(-128, 128, (12, 16, 3, 3), dtype=np.int8)
+    flat = ops.quant_convolution(dev(x), dev(w), (1, 0), (1, 2), (1, 1))
+    vol = ops.quant_convolution(dev(x[:, :, None]), dev(w[:, :, None]), (0, 1, 0), (1, 1, 2), (1, 1, 1))
+    assert torch.equal(vol[:, :, 0], flat)
+
+
+def test_three_axis_dequant_epilogue_and_fp8(ops):
+    rng = np.random.default_rng(13)
+    xs, ws = (2, 16, 5, 6, 6), (20, 16, 3, 3, 3)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.017)
+    sw = rng.uniform(0.001, 0.01, 20).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (1, 1, 1))
+    scale = np.broadcast_to((sx * sw).astype(np.float32).reshape(1, -1, 1, 1, 1), acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1, 1), scale_x=dev(np.float32([sx])), scale_w=dev(sw))
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    got16 = ops.quant_convolution(dev(x), dev(w), (1, 1, 1), scale_x=dev(np.float32([sx])), scale_w=dev(sw),
+                                  out_dtype=torch.float16)
+    assert np.array_equal(half_bits(got16), orc.convert(want, orc.F32, orc.F16))
+    # fp8: small integers are exact, and the float reference's known 3-D answer is met on operands
+    # that fp8 represents exactly
+    xi = rng.integers(-3, 4, xs).astype(np.float32)
+    wi = rng.integers(-2, 3, ws).astype(np.float32)
+    gotf = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(orc.fp8_from_f32(wi)), (1, 1, 1), fp8=True)
+    assert gotf.dtype == torch.float32
+    assert np.array_equal(gotf.cpu().numpy(), orc.convolution(xi, wi, orc.F32, (1, 1, 1)))
+
+
 def test_fp8_convolution(ops):
     rng = np.random.default_rng(8)
     xs, ws = (2, 32, 10, 10), (24, 32, 3, 3)
@@ -139,6 +199,11 @@ def test_argument_errors(ops):
         ops.quant_convolution(x, dev(np.zeros((3, 2, 3, 3), np.int8)), group=2)  # O % group
     with pytest.raises(Exception):
         ops.quant_convolution(x, dev(np.zeros((2, 4, 3, 3), np.int8)), stride=(0, 1))
+    with pytest.raises(Exception):
+        ops.quant_convolution(x, dev(np.zeros((2, 4, 1, 3, 3), np.int8)))       # ranks differ
+    with pytest.raises(Exception):
+        ops.quant_convolution(dev(np.zeros((1, 4, 5, 5, 5), np.int8)), dev(np.zeros((2, 4, 3, 3, 3), np.int8)),
+                              stride=(1, 1))                                      # two strides for three axes
     # a window larger than the padded input gives the minimum output size of one
     got = ops.quant_convolution(x, dev(np.ones((2, 4, 7, 7), np.int8)))
     assert tuple(got.shape) == (1, 2, 1, 1)

@@ -88,3 +88,52 @@ def test_fp8_products_are_exact_in_double():
     want = orc.convolution(x, w, orc.F32, (1, 1))
     assert got.dtype == np.float32
     assert np.array_equal(got, want)
+
+
+def brute_nd(x, w, padding, stride, dilation, group):
+    """Independent form for any number of spatial axes: pad with zeros, slice the dilated window,
+    sum products in int64."""
+    nd = x.ndim - 2
+    lo, hi = list(padding[:nd]), list(padding[nd:] if len(padding) == 2 * nd else padding[:nd])
+    xp = np.zeros(x.shape[:2] + tuple(x.shape[2 + i] + lo[i] + hi[i] for i in range(nd)), np.int64)
+    xp[(slice(None), slice(None)) + tuple(slice(lo[i], lo[i] + x.shape[2 + i]) for i in range(nd))] = x
+    out_sp = [orc.conv_out_len(x.shape[2 + i], w.shape[2 + i], lo[i], stride[i], dilation[i], hi[i]) for i in range(nd)]
+    o, cg = w.shape[:2]
+    og = o // group
+    out = np.zeros((x.shape[0], o, *out_sp), np.int64)
+    for oc in range(o):
+        g = oc // og
+        xs = xp[:, g * cg:(g + 1) * cg]
+        for pos in np.ndindex(*out_sp):
+            win = xs[(slice(None), slice(None)) + tuple(
+                slice(pos[i] * stride[i], pos[i] * stride[i] + dilation[i] * (w.shape[2 + i] - 1) + 1, dilation[i])
+                for i in range(nd))]
+            out[(slice(None), oc) + pos] = (win * w[oc].astype(np.int64)[None]).sum(axis=tuple(range(1, nd + 2)))
+    return out
+
+
+@pytest.mark.parametrize("shape,wshape,padding,stride,dilation,group", [
+    ((2, 4, 5, 6, 7), (6, 4, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    ((1, 6, 6, 5, 4), (4, 3, 2, 3, 1), (1, 0, 2), (2, 1, 1), (1, 2, 1), 2),
+    ((2, 4, 7, 4, 5), (4, 1, 3, 2, 2), (0, 1, 0, 2, 0, 1), (1, 2, 3), (2, 1, 1), 4),   # low / high padding
+    ((1, 3, 4, 4, 4), (2, 3, 1, 1, 1), (0, 0, 0), (2, 2, 2), (1, 1, 1), 1),
+    ((3, 2, 9), (4, 2, 3), (1,), (2,), (2,), 1),                                      # one spatial axis
+    ((2, 4, 11), (6, 2, 4), (2, 0), (1,), (1,), 2),
+])
+def test_int8_one_and_three_spatial_axes_against_brute_force(shape, wshape, padding, stride, dilation, group):
+    rng = np.random.default_rng(sum(shape) * 7 + sum(wshape))
+    x = rng.integers(-128, 128, shape, dtype=np.int8)
+    w = rng.integers(-128, 128, wshape, dtype=np.int8)
+    got = orc.convolution(x, w, orc.I8, padding, stride, dilation, group)
+    want = brute_nd(x, w, padding, stride, dilation, group)
+    assert got.shape == want.shape
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_depth_one_volume_is_the_two_dimensional_convolution():
+    rng = np.random.default_rng(11)
+    x = rng.integers(-128, 128, (2, 4, 6, 7), dtype=np.int8)
+    w = rng.integers(-128, 128, (3, 4, 3, 2), dtype=np.int8)
+    flat = orc.convolution(x, w, orc.I8, (1, 0), (1, 2), (1, 1))
+    vol = orc.convolution(x[:, :, None], w[:, :, None], orc.I8, (0, 1, 0), (1, 1, 2), (1, 1, 1))
+    assert np.array_equal(vol[:, :, 0], flat)
