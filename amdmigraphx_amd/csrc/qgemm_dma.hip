@@ -1144,16 +1144,431 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// The same 256 x 256 tile with four waves, one per SIMD, each owning a 128 x 128 quadrant
+// (8 x 8 MFMA tiles of 16 x 16: 256 accumulator registers, which the compiler keeps in the
+// accumulation half of the register file).  Against the eight-wave kernel above every operand
+// byte in LDS is read by half as many waves: 64 KiB of fragment reads per slab instead of 96,
+// next to the 32 KiB the direct-to-LDS loads write.  The LDS serves about 146 bytes per clock to
+// both together, so the eight-wave kernel needs 88 % of it at the full MFMA rate, this one 66 %.
+//
+// A slab's fragments are all in registers when its MFMAs start: they are read (into the other
+// half of a double buffer) while the previous slab is multiplied, right behind the one barrier per
+// slab.  That barrier tells a wave that slab kt+1 is complete in LDS and that every wave has
+// finished reading slab kt, whose B stage then takes the loads of slab kt+4.  A has three stages
+// of two slabs each; K step s is loaded in two halves during slabs 2s-5 and 2s-4, so every slab
+// issues 4 B and 4 A load instructions per wave.
+constexpr int W4_THREADS  = 256;
+constexpr int W4_A_STAGES = 3;
+constexpr int W4_B_BASE   = W4_A_STAGES * A2_BYTES;
+constexpr int W4_LDS_BYTES = W4_B_BASE + STAGES * B_BYTES; // 96 + 64 KiB
+
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE>
+__global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 1; // 0..1
+    const int wave_n = wave & 1;  // 0..1
+
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
+    const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+    const int nk = p.k / BK;
+
+    // ---- global -> LDS: the layouts of the eight-wave kernel, blocks dealt to four waves ----
+    uint32_t a_off[8], b_off[4];
+    const int a_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7); // (r >> 1) & 7 of this lane's rows
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+    {
+        const int r   = 8 * (wave + 4 * h) + (lane >> 3);
+        const int row = min(m0 + r, p.m - 1);
+        a_off[h]      = (uint32_t)row * (uint32_t)p.lda + a_chunk * 16;
+    }
+    const uint32_t a_tail_back = a_chunk >= 4 ? 64u : 0u;
+#pragma unroll
+    for(int h = 0; h < 4; h++)
+    {
+        const int blk = wave + 4 * h;
+        if constexpr(TRANS_B)
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int col   = min(n0 + r, p.n - 1);
+            b_off[h]        = (uint32_t)col * (uint32_t)p.ldb + chunk * 16;
+        }
+        else
+        {
+            const int k     = 4 * blk + (lane >> 4);
+            const int chunk = (lane & 15) ^ (k & 7);
+            const int col   = min(n0 + chunk * 16, p.n - 16);
+            b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
+        }
+    }
+    // ss: index of the 128-byte K step (slabs 2*ss and 2*ss + 1); h: block 0..7 of this wave
+    auto issue_a = [&](int ss, int h) {
+        uint8_t* st           = lds + (ss % W4_A_STAGES) * A2_BYTES;
+        const uint8_t* a_base = ga + (int64_t)ss * (2 * BK);
+        const uint32_t back   = 2 * ss + 1 < nk ? 0u : a_tail_back;
+        load_to_lds(a_base + (a_off[h] - back), st + (wave + 4 * h) * 1024);
+    };
+    auto issue_b = [&](int kt, int h) {
+        uint8_t* st           = lds + W4_B_BASE + (kt & (STAGES - 1)) * B_BYTES;
+        const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
+        load_to_lds(b_base + b_off[h], st + (wave + 4 * h) * 1024);
+    };
+    // what a wave issues during slab kt (kt from -4: the prologue runs the same sequence): the B
+    // blocks of slab kt+4 and one half of an A step, K step (kt+5)/2 first half when kt is odd,
+    // (kt+4)/2 second half when it is even
+    auto a_step_of   = [](int kt) { return (kt & 1) != 0 ? (kt + 5) / 2 : (kt + 4) / 2; };
+    auto issues_b    = [&](int kt) { return kt + 4 >= 0 && kt + 4 < nk; };
+    auto issues_a    = [&](int kt) { const int ss = a_step_of(kt); return ss >= 1 && 2 * ss < nk; };
+    auto issued_in   = [&](int kt) { return (issues_b(kt) ? 4 : 0) + (issues_a(kt) ? 4 : 0); };
+
+    // ---- LDS -> operand fragments -------------------------------------------------------------
+    const int lrow      = lane & 15;
+    const int lgrp      = lane >> 4;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    const int sw        = (lrow >> 2) & 3;
+    uint32_t a_lane[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+        a_lane[h] = (wave_m * 128 + lrow) * (2 * BK) + (((4 * h + lgrp) ^ ((lrow >> 1) & 7)) << 4);
+    uint32_t b_lane[2];
+    if constexpr(TRANS_B)
+    {
+        b_lane[0] = W4_B_BASE + (wave_n * 128 + lrow) * BK + ((lgrp ^ sw) << 4);
+        b_lane[1] = 0;
+    }
+    else
+    {
+#pragma unroll
+        for(int r = 0; r < 2; r++)
+        {
+            const int k = lgrp * 16 + 8 * r + (lrow >> 1);
+            b_lane[r]   = W4_B_BASE + k * BN + 8 * (lrow & 1);
+        }
+    }
+    const int bsw = (lrow >> 1) & 7; // k & 7 of this lane's row in the transposing read
+
+    v4i fa[2][8];
+    v4i fb[2][8];
+    v4i acc[8][8];
+#pragma unroll
+    for(int i = 0; i < 8; i++)
+#pragma unroll
+        for(int j = 0; j < 8; j++)
+            acc[i][j] = v4i{0, 0, 0, 0};
+
+#define RD128(dst, addr, imm) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define RDTR8(dst, addr, imm) \
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define SB() __builtin_amdgcn_sched_barrier(0)
+    // A tile I of slab kt -> fa[Q][I]
+#define RA(kt, Q, I) \
+    RD128(fa[Q][I], lds0 + (((kt) >> 1) % W4_A_STAGES) * A2_BYTES + a_lane[(kt) & 1], (I) * 16 * 2 * BK)
+    // B tile J of slab kt: row-major B takes two reads (R = 0, 1), K-contiguous B one
+#define RB(kt, Q, J, R)                                                                        \
+    do                                                                                         \
+    {                                                                                          \
+        const uint32_t s_ = lds0 + ((kt) & (STAGES - 1)) * B_BYTES;                            \
+        if constexpr(TRANS_B)                                                                  \
+        {                                                                                      \
+            if((R) == 0)                                                                       \
+                RD128(fb[Q][J], s_ + b_lane[0], (J) * 16 * BK);                                \
+        }                                                                                      \
+        else                                                                                   \
+        {                                                                                      \
+            const uint32_t c_ = (uint32_t)(((wave_n * 8 + (J)) ^ bsw) << 4);                   \
+            v2i t_;                                                                            \
+            if((R) == 0)                                                                       \
+            {                                                                                  \
+                RDTR8(t_, s_ + b_lane[0] + c_, 0);                                             \
+                fb[Q][J].x = t_.x;                                                             \
+                fb[Q][J].y = t_.y;                                                             \
+            }                                                                                  \
+            else                                                                               \
+            {                                                                                  \
+                RDTR8(t_, s_ + b_lane[1] + c_, 0);                                             \
+                fb[Q][J].z = t_.x;                                                             \
+                fb[Q][J].w = t_.y;                                                             \
+            }                                                                                  \
+        }                                                                                      \
+    } while(0)
+    // every fragment of buffer Q has arrived
+#define WAIT_FRAGS(Q)                                                                              \
+    do                                                                                             \
+    {                                                                                              \
+        asm volatile("s_waitcnt lgkmcnt(0)"                                                        \
+                     : "+v"(fa[Q][0]), "+v"(fa[Q][1]), "+v"(fa[Q][2]), "+v"(fa[Q][3]),             \
+                       "+v"(fa[Q][4]), "+v"(fa[Q][5]), "+v"(fa[Q][6]), "+v"(fa[Q][7]),             \
+                       "+v"(fb[Q][0]), "+v"(fb[Q][1]), "+v"(fb[Q][2]), "+v"(fb[Q][3]),             \
+                       "+v"(fb[Q][4]), "+v"(fb[Q][5]), "+v"(fb[Q][6]), "+v"(fb[Q][7])::"memory");   \
+    } while(0)
+    // The MFMA as an assembly statement with the accumulator tied to the accumulation registers:
+    // left to the register allocator, a part of the 256 accumulators ends up in ordinary
+    // registers and scratch memory and is copied in and out around every instruction.  The
+    // statements are volatile, so together with the LDS reads they stay in program order.
+#define MF(Q, I, J)                                                   \
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"              \
+                 : "+a"(acc[I][J])                                    \
+                 : "v"(fb[Q][J]), "v"(fa[Q][I]))
+    // two MFMAs, then one other instruction: slot N of 32 in a slab.  Slots 0..23 read the next
+    // slab's fragments (8 A tiles, then 8 B tiles in two halves), slots 24..31 issue this slab's
+    // share of the loads.
+#define OTHER(kt, Q, N)                                                                     \
+    do                                                                                      \
+    {                                                                                       \
+        if constexpr((N) < 8)                                                               \
+        {                                                                                   \
+            if(fast_ || more_) RA((kt) + 1, 1 - (Q), (N));                                  \
+        }                                                                                   \
+        else if constexpr((N) < 24)                                                         \
+        {                                                                                   \
+            if(fast_ || more_) RB((kt) + 1, 1 - (Q), ((N) - 8) >> 1, ((N) - 8) & 1);        \
+        }                                                                                   \
+        else if constexpr((N) < 28)                                                         \
+        {                                                                                   \
+            if(fast_ || ldb_) issue_b((kt) + 4, (N) - 24);                                  \
+        }                                                                                   \
+        else                                                                                \
+        {                                                                                   \
+            if(fast_ || lda_) issue_a(ass_, (1 - (Q)) * 4 + (N) - 28);                      \
+        }                                                                                   \
+    } while(0)
+#define ROW(kt, Q, I)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        SB(); MF(Q, I, 0); MF(Q, I, 1); SB(); OTHER(kt, Q, 4 * (I) + 0);                     \
+        SB(); MF(Q, I, 2); MF(Q, I, 3); SB(); OTHER(kt, Q, 4 * (I) + 1);                     \
+        SB(); MF(Q, I, 4); MF(Q, I, 5); SB(); OTHER(kt, Q, 4 * (I) + 2);                     \
+        SB(); MF(Q, I, 6); MF(Q, I, 7); SB(); OTHER(kt, Q, 4 * (I) + 3);                     \
+    } while(0)
+    // vector-memory operations that may stay in flight when slab kt+1 must be complete: what the
+    // wave issued during slabs kt-2 and kt-1
+#define WAIT_SLAB(kt)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        const int cnt_ = issued_in((kt) - 2) + issued_in((kt) - 1);                          \
+        if(cnt_ >= 16)      wait_vmcnt<16>();                                               \
+        else if(cnt_ >= 12) wait_vmcnt<12>();                                               \
+        else if(cnt_ >= 8)  wait_vmcnt<8>();                                                \
+        else if(cnt_ >= 4)  wait_vmcnt<4>();                                                \
+        else                wait_vmcnt<0>();                                                \
+    } while(0)
+    // Q: the slab's parity (which fragment buffer it multiplies; an even slab issues the second
+    // half of an A step, an odd one the first).  FAST: a slab of the steady state, where the next
+    // slab and every load of the slab's share exist and the wait is for 16 operations.
+#define SLAB(kt, Q, FAST)                                                                   \
+    do                                                                                      \
+    {                                                                                       \
+        constexpr bool fast_ = (FAST);                                                      \
+        const int kt_     = (kt);                                                           \
+        const bool more_  = kt_ + 1 < nk;                                                   \
+        const bool ldb_   = issues_b(kt_);                                                  \
+        const bool lda_   = issues_a(kt_);                                                  \
+        const int ass_    = a_step_of(kt_);                                                 \
+        (void)more_; (void)ldb_; (void)lda_;                                                \
+        WAIT_FRAGS(Q);                                                                      \
+        if constexpr(fast_)                                                                 \
+            wait_vmcnt<16>();                                                               \
+        else if(more_)                                                                      \
+            WAIT_SLAB(kt_);                                                                 \
+        block_barrier();                                                                    \
+        ROW(kt_, Q, 0); ROW(kt_, Q, 1); ROW(kt_, Q, 2); ROW(kt_, Q, 3);                     \
+        ROW(kt_, Q, 4); ROW(kt_, Q, 5); ROW(kt_, Q, 6); ROW(kt_, Q, 7);                     \
+        SB();                                                                               \
+    } while(0)
+
+    // ---- main loop -----------------------------------------------------------------------------
+    // Prologue: K step 0 of A, then what slabs -4 .. -1 would have issued.
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+        issue_a(0, h);
+#pragma unroll
+    for(int kt = -4; kt < 0; kt++)
+    {
+        if(issues_b(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_b(kt + 4, h);
+        }
+        if(issues_a(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_a(a_step_of(kt), ((kt & 1) != 0 ? 0 : 4) + h);
+        }
+    }
+    // slab 0 is complete when only what came behind B(0) is in flight
+    {
+        const int cnt = issued_in(-3) + issued_in(-2) + issued_in(-1);
+        if(cnt >= 24)      wait_vmcnt<24>();
+        else if(cnt == 20) wait_vmcnt<20>();
+        else if(cnt == 16) wait_vmcnt<16>();
+        else if(cnt == 12) wait_vmcnt<12>();
+        else if(cnt == 8)  wait_vmcnt<8>();
+        else if(cnt == 4)  wait_vmcnt<4>();
+        else               wait_vmcnt<0>();
+    }
+    block_barrier();
+#pragma unroll
+    for(int i = 0; i < 8; i++)
+        RA(0, 0, i);
+#pragma unroll
+    for(int j = 0; j < 8; j++)
+    {
+        RB(0, 0, j, 0);
+        RB(0, 0, j, 1);
+    }
+    int kt = 0;
+    for(; kt + 6 < nk; kt += 2)
+    {
+        SLAB(kt, 0, true);
+        SLAB(kt + 1, 1, true);
+    }
+    for(; kt + 1 < nk; kt += 2)
+    {
+        SLAB(kt, 0, false);
+        SLAB(kt + 1, 1, false);
+    }
+    if(kt < nk)
+        SLAB(kt, 0, false);
+    // the last MFMAs' results are read by ordinary instructions next: the wait states the compiler
+    // would put behind an MFMA it knows
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
+#undef SLAB
+#undef WAIT_SLAB
+#undef ROW
+#undef OTHER
+#undef MF
+#undef WAIT_FRAGS
+#undef RB
+#undef RA
+#undef SB
+#undef RDTR8
+#undef RD128
+
+    // ---- epilogue: as in the eight-wave kernel, 8 x 8 tiles per wave ---------------------------
+    // acc[i][j][e]: row 16*i + (l % 16) of the wave's A block, column 16*j + 4*(l / 16) + e of its
+    // B block.
+    float sa_r[8];
+    int64_t zrow_r[8];
+    if constexpr(DEQ)
+    {
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+        {
+            const int row = min(m0 + wave_m * 128 + i * 16 + lrow, p.m - 1);
+            float sa      = 1.f;
+            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                sa = p.scale_a[0];
+            else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                sa = p.scale_a[row];
+            sa_r[i]   = sa;
+            zrow_r[i] = p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
+        }
+    }
+#pragma unroll
+    for(int j = 0; j < 8; j++)
+    {
+        const int col = n0 + wave_n * 128 + j * 16 + 4 * lgrp;
+        if(col >= p.n)
+            continue; // N is a multiple of 4 on this path, so the 4 columns are in or out together
+        float sb_c[4];
+        int32_t cs_c[4];
+        float bias_c[4];
+        if constexpr(DEQ)
+        {
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                const int c = min(col + e, p.n - 1);
+                float sb    = 1.f;
+                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                    sb = p.scale_b[0];
+                else if(p.scale_b_mode == MI355_QP_PER_COL)
+                    sb = p.scale_b[c];
+                sb_c[e]   = sb;
+                cs_c[e]   = p.zp_a != 0 ? p.colsum_b[c] : 0;
+                bias_c[e] = p.bias != nullptr ? p.bias[c] : -0.0f;
+            }
+        }
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+        {
+            const int row = m0 + wave_m * 128 + i * 16 + lrow;
+            if(row >= p.m)
+                continue;
+            const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+            if constexpr(!DEQ)
+            {
+                int32_t* o = static_cast<int32_t*>(p.c) + idx;
+                if constexpr(VEC_STORE)
+                    store_c(reinterpret_cast<v4i*>(o), acc[i][j], p.stream_c);
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        o[e] = acc[i][j][e];
+                }
+            }
+            else
+            {
+                float v[4];
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    const float s  = sa_r[i] * sb_c[e];
+                    const double d = (double)acc[i][j][e] -
+                                     (double)(int32_t)(zrow_r[i] + (int64_t)p.zp_a * cs_c[e]);
+                    v[e] = add_bias((float)(d * (double)s), bias_c[e]);
+                }
+                if constexpr(VEC_STORE)
+                {
+                    if constexpr(OUT == MI355_F32)
+                        store_c(reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx), v4f{v[0], v[1], v[2], v[3]}, p.stream_c);
+                    else if constexpr(OUT == MI355_F16)
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                            convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+                    else
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
+                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                }
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        store1<OUT>(p.c, idx + e, v[e]);
+                }
+            }
+        }
+    }
+}
+
 template <bool TRANS_B, bool DEQ, int OUT, bool VEC>
 int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
 {
-    auto kern = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
+    auto kern = qgemm_w4_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
+        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
     if(attr != hipSuccess)
         return MI355_ERR_LAUNCH;
     dim3 grid(p.tiles_m * p.tiles_n, batch);
-    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(W4_THREADS), W4_LDS_BYTES, stream, p);
     return mi355_launch_status();
 }
 
