@@ -1562,13 +1562,28 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 template <bool TRANS_B, bool DEQ, int OUT, bool VEC>
 int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
 {
-    auto kern = qgemm_w4_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
-    static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
-    if(attr != hipSuccess)
-        return MI355_ERR_LAUNCH;
     dim3 grid(p.tiles_m * p.tiles_n, batch);
-    hipLaunchKernelGGL(kern, grid, dim3(W4_THREADS), W4_LDS_BYTES, stream, p);
+    // The four-wave kernel pays more per tile (a deeper pipeline to fill, 64 stores per wave at
+    // the end) and less per slab: measured against the eight-wave kernel at 8192 x 8192 x K it is
+    // 12 % slower at K = 1024, even at 2048, 2-15 % faster from 4096 on.
+    if(p.k >= 3072)
+    {
+        auto kern = qgemm_w4_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
+        static const hipError_t attr = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
+        if(attr != hipSuccess)
+            return MI355_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, dim3(W4_THREADS), W4_LDS_BYTES, stream, p);
+    }
+    else
+    {
+        auto kern = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
+        static const hipError_t attr = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
+        if(attr != hipSuccess)
+            return MI355_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
+    }
     return mi355_launch_status();
 }
 

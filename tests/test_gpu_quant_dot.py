@@ -149,6 +149,74 @@ def test_int8_dequant_epilogue_bit_exact(ops, zp_a, zp_b, out):
         assert np.array_equal(half_bits(got), want)
 
 
+# ---- the four-wave kernel: one-pass int8 products with K >= 3072 --------------------------------
+# Bare products reach it when the tiles alone fill half the chip (here through the batch), products
+# with the dequantizing epilogue whenever no workspace is given.
+
+@pytest.mark.parametrize("m,n,k,batch,trans_b", [
+    (300, 520, 3136, 32, False),      # ragged M and N tiles, an odd number of slabs (49)
+    (300, 520, 3136, 32, True),
+    (256, 512, 3072, 64, False),      # whole tiles, 48 slabs
+    (513, 260, 3200, 24, True),       # three tile rows with one live row in the last
+])
+def test_four_wave_kernel_bare_bit_exact(ops, m, n, k, batch, trans_b):
+    rng = np.random.default_rng(m + 3 * n + 7 * k + batch)
+    a = rng.integers(-128, 128, (batch, m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (batch, k, n), dtype=np.int8)
+    a[0, :4] = 127
+    b[0, :, :4] = -128
+    want = np.stack([orc.quant_dot(a[i], b[i], orc.I8) for i in range(batch)])
+    tb = dev(np.ascontiguousarray(b.transpose(0, 2, 1))).transpose(1, 2) if trans_b else dev(b)
+    print("w4 bare", m, n, k, batch, trans_b, flush=True)
+    got = ops.quant_dot(dev(a), tb).cpu().numpy()
+    assert got.dtype == np.int32 and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(260, 264, 3072, False), (512, 520, 3136, True), (100, 1028, 4160, False)])
+@pytest.mark.parametrize("zp_a,zp_b", [(0, 0), (7, -9)])
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_four_wave_kernel_dequantizing_epilogue_bit_exact(ops, m, n, k, trans_b, zp_a, zp_b, out):
+    """Per-row and per-column scales, both zero points, a bias and the truncating converts in the
+    epilogue of the four-wave kernel; accumulators beyond 2^24."""
+    rng = np.random.default_rng(m + n + k + zp_a)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (n, k) if trans_b else (k, n), dtype=np.int8)
+    bm = np.ascontiguousarray(b.T) if trans_b else b
+    a[:8] = 127
+    bm[:, :8] = 127
+    b = np.ascontiguousarray(bm.T) if trans_b else bm
+    sa = np.float32(0.0371)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 3).astype(np.float32)
+    want = orc.qdq_matmul_int8(a, bm, sa, sb, zp_a, zp_b, orc.F32) + bias[None, :]
+    ta = dev(a)
+    tb = dev(b).T if trans_b else dev(b)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    print("w4 dq", m, n, k, trans_b, zp_a, zp_b, out, flush=True)
+    got = ops.quant_dot(ta, tb, scale_a=dev(np.float32([sa])), scale_b=dev(sb), zp_a=zp_a, zp_b=zp_b,
+                        colsum_b=ops.colsum_i8(tb) if zp_a else None,
+                        rowsum_a=ops.rowsum_i8(ta) if zp_b else None, out_dtype=td, bias=dev(bias))
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        ot = orc.F16 if out == "f16" else orc.BF16
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+def test_four_wave_kernel_per_row_scales(ops):
+    rng = np.random.default_rng(77)
+    m, n, k = 300, 260, 3072
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    sa = rng.uniform(0.01, 0.05, m).astype(np.float32)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    acc = orc.quant_dot(a, b, orc.I8)
+    scale = (sa[:, None] * sb[None, :]).astype(np.float32)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    got = ops.quant_dot(dev(a), dev(b), scale_a=dev(sa), scale_b=dev(sb))
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_rowsum_colsum(ops):
     rng = np.random.default_rng(5)
     a = rng.integers(-128, 128, (130, 1000), dtype=np.int8)
