@@ -93,31 +93,30 @@ MI355_DEVINL uint8_t f32_to_fp8_rne(float x)
 // `convert` op (op/convert.hpp:64-87) from float to a 16-bit float type.
 MI355_DEVINL uint16_t convert_f32_to_half(float x)
 {
-    if(x != x)
-        return 0x7e00;
-    uint32_t ax = __builtin_bit_cast(uint32_t, x) & 0x7fffffffu;
-    if(ax == 0x7f800000u)
-        return x > 0 ? 0x7c00 : 0xfc00;
-    if(x >= 65504.0f)
-        return 0x7bff;
-    if(x <= -65504.0f)
-        return 0xfbff;
-    return f32_to_half_rtz(x);
+    // selects, not branches: the epilogues convert thousands of values per wave
+    const uint32_t ux   = __builtin_bit_cast(uint32_t, x);
+    const uint32_t ax   = ux & 0x7fffffffu;
+    const uint32_t sign = (ux >> 16) & 0x8000u;
+    const auto p        = __builtin_amdgcn_cvt_pkrtz(x, 0.0f);
+    uint32_t h          = __builtin_bit_cast(uint32_t, p) & 0xffffu;
+    // float subnormals: the software conversion shifts the mantissa, the hardware gives +-0
+    h = (ax != 0 && ax < 0x00800000u) ? (sign | ((ux & 0x7fffffu) >> 13)) : h;
+    h = ax >= 0x477fe000u ? (sign | 0x7bffu) : h; // |x| >= 65504: the largest finite half
+    h = ax == 0x7f800000u ? (sign | 0x7c00u) : h; // infinities stay
+    h = ax > 0x7f800000u ? 0x7e00u : h;           // NaN
+    return (uint16_t)h;
 }
 
 MI355_DEVINL uint16_t convert_f32_to_bf16(float x)
 {
-    if(x != x)
-        return 0x7fc0;
-    uint32_t ax = __builtin_bit_cast(uint32_t, x) & 0x7fffffffu;
-    if(ax == 0x7f800000u)
-        return x > 0 ? 0x7f80 : 0xff80;
-    const float bmax = __builtin_bit_cast(float, 0x7f7f0000u);
-    if(x >= bmax)
-        return 0x7f7f;
-    if(x <= -bmax)
-        return 0xff7f;
-    return f32_to_bf16_rtz(x);
+    const uint32_t ux   = __builtin_bit_cast(uint32_t, x);
+    const uint32_t ax   = ux & 0x7fffffffu;
+    const uint32_t sign = (ux >> 16) & 0x8000u;
+    uint32_t h          = ux >> 16;                // toward zero
+    h = ax >= 0x7f7f0000u ? (sign | 0x7f7fu) : h; // |x| >= the largest finite bf16
+    h = ax == 0x7f800000u ? (sign | 0x7f80u) : h; // infinities stay
+    h = ax > 0x7f800000u ? 0x7fc0u : h;           // NaN
+    return (uint16_t)h;
 }
 
 // The `add` of a bias behind dequantizelinear: its own fp32 rounding, never contracted with the

@@ -1445,9 +1445,12 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     }
     if(kt < nk)
         SLAB(kt, 0, false);
-    // the last MFMAs' results are read by ordinary instructions next: the wait states the compiler
-    // would put behind an MFMA it knows
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
+    // The last MFMAs' results are read by ordinary instructions next: the wait states the compiler
+    // would put behind an MFMA it knows.  The last row of accumulators passes through the statement,
+    // so no read of it can move ahead; the rows before are at least eight MFMAs old.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3"
+                 : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
+                   "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]));
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
@@ -1480,31 +1483,48 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
             zrow_r[i] = p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
         }
     }
+    // The scales, column sums and biases of a block of 16 columns are loaded ahead of the stores of
+    // the block before it: a load issued behind a store waits for it.
+    float sb_c[4], bias_c[4], sb_next[4], bias_next[4];
+    int32_t cs_c[4], cs_next[4];
+    auto load_block = [&](int j, float (&sb_o)[4], int32_t (&cs_o)[4], float (&bias_o)[4]) {
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+        {
+            const int c = min(n0 + wave_n * 128 + j * 16 + 4 * lgrp + e, p.n - 1);
+            float sb    = 1.f;
+            if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                sb = p.scale_b[0];
+            else if(p.scale_b_mode == MI355_QP_PER_COL)
+                sb = p.scale_b[c];
+            sb_o[e]   = sb;
+            cs_o[e]   = p.zp_a != 0 ? p.colsum_b[c] : 0;
+            bias_o[e] = p.bias != nullptr ? p.bias[c] : -0.0f;
+        }
+    };
+    if constexpr(DEQ)
+        load_block(0, sb_c, cs_c, bias_c);
 #pragma unroll
     for(int j = 0; j < 8; j++)
     {
+        if constexpr(DEQ)
+        {
+            if(j > 0)
+            {
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    sb_c[e]   = sb_next[e];
+                    cs_c[e]   = cs_next[e];
+                    bias_c[e] = bias_next[e];
+                }
+            }
+            if(j + 1 < 8)
+                load_block(j + 1, sb_next, cs_next, bias_next);
+        }
         const int col = n0 + wave_n * 128 + j * 16 + 4 * lgrp;
         if(col >= p.n)
             continue; // N is a multiple of 4 on this path, so the 4 columns are in or out together
-        float sb_c[4];
-        int32_t cs_c[4];
-        float bias_c[4];
-        if constexpr(DEQ)
-        {
-#pragma unroll
-            for(int e = 0; e < 4; e++)
-            {
-                const int c = min(col + e, p.n - 1);
-                float sb    = 1.f;
-                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
-                    sb = p.scale_b[0];
-                else if(p.scale_b_mode == MI355_QP_PER_COL)
-                    sb = p.scale_b[c];
-                sb_c[e]   = sb;
-                cs_c[e]   = p.zp_a != 0 ? p.colsum_b[c] : 0;
-                bias_c[e] = p.bias != nullptr ? p.bias[c] : -0.0f;
-            }
-        }
 #pragma unroll
         for(int i = 0; i < 8; i++)
         {
@@ -1814,9 +1834,505 @@ int launch_i8_out(const dma_params& p, int batch, bool deq, int out, hipStream_t
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// fp8 (e4m3fn) on the four-wave plan: the same loads, LDS stages, barrier and one-slab-ahead
+// fragment reads as qgemm_w4_i8_kernel, with v_mfma_f32_32x32x64_f8f6f4.  A wave's 128 x 128
+// quadrant is 4 x 4 tiles of 32 x 32 (16 accumulator registers each, 256 in all); a 32-row operand
+// tile of one slab is 32 bytes per lane (lane l: row l % 32, K bytes 32 * (l / 32)..), read as two
+// 16-byte chunks (A, or B given as [N, K]) or four transposing 8-byte reads (row-major B).
+// 16 MFMAs of 64 cycles per slab, two other instructions behind each.
+// The kernel is for C whose rows keep groups of 4 outputs whole and aligned (N % 4 == 0 and
+// p.vec_store); VEC8: 16-bit outputs in groups of 8 (p.vec8_store).  The way C is stored is fixed at
+// compile time: with both ways behind a run-time branch the compiler keeps the accumulators in
+// scratch memory across the epilogue.
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC8>
+__global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 1; // 0..1
+    const int wave_n = wave & 1;  // 0..1
+
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
+    const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+    const int nk = p.k / BK;
+
+    // ---- global -> LDS: exactly as in qgemm_w4_i8_kernel -------------------------------------
+    uint32_t a_off[8], b_off[4];
+    const int a_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+    {
+        const int r   = 8 * (wave + 4 * h) + (lane >> 3);
+        const int row = min(m0 + r, p.m - 1);
+        a_off[h]      = (uint32_t)row * (uint32_t)p.lda + a_chunk * 16;
+    }
+    const uint32_t a_tail_back = a_chunk >= 4 ? 64u : 0u;
+#pragma unroll
+    for(int h = 0; h < 4; h++)
+    {
+        const int blk = wave + 4 * h;
+        if constexpr(TRANS_B)
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int col   = min(n0 + r, p.n - 1);
+            b_off[h]        = (uint32_t)col * (uint32_t)p.ldb + chunk * 16;
+        }
+        else
+        {
+            const int k     = 4 * blk + (lane >> 4);
+            const int chunk = (lane & 15) ^ (k & 7);
+            const int col   = min(n0 + chunk * 16, p.n - 16);
+            b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
+        }
+    }
+    auto issue_a = [&](int ss, int h) {
+        uint8_t* st           = lds + (ss % W4_A_STAGES) * A2_BYTES;
+        const uint8_t* a_base = ga + (int64_t)ss * (2 * BK);
+        const uint32_t back   = 2 * ss + 1 < nk ? 0u : a_tail_back;
+        load_to_lds(a_base + (a_off[h] - back), st + (wave + 4 * h) * 1024);
+    };
+    auto issue_b = [&](int kt, int h) {
+        uint8_t* st           = lds + W4_B_BASE + (kt & (STAGES - 1)) * B_BYTES;
+        const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
+        load_to_lds(b_base + b_off[h], st + (wave + 4 * h) * 1024);
+    };
+    auto a_step_of   = [](int kt) { return (kt & 1) != 0 ? (kt + 5) / 2 : (kt + 4) / 2; };
+    auto issues_b    = [&](int kt) { return kt + 4 >= 0 && kt + 4 < nk; };
+    auto issues_a    = [&](int kt) { const int ss = a_step_of(kt); return ss >= 1 && 2 * ss < nk; };
+    auto issued_in   = [&](int kt) { return (issues_b(kt) ? 4 : 0) + (issues_a(kt) ? 4 : 0); };
+
+    // ---- LDS -> operand fragments -------------------------------------------------------------
+    const int lrow      = lane & 31;
+    const int lgrp      = lane >> 5;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    // A: rows of 128 bytes (two slabs); slab parity h, chunk x of this lane's 32 bytes is logical
+    // chunk 4h + 2*lgrp + x at position c ^ ((row >> 1) & 7)
+    uint32_t a_lane[2][2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+            a_lane[h][x] = (wave_m * 128 + lrow) * (2 * BK) + (((4 * h + 2 * lgrp + x) ^ ((lrow >> 1) & 7)) << 4);
+    uint32_t b_lane[2];
+    int bsw = 0, bcol = 0;
+    if constexpr(TRANS_B)
+    {
+        const int sw = (lrow >> 2) & 3;
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+            b_lane[x] = W4_B_BASE + (wave_n * 128 + lrow) * BK + (((2 * lgrp + x) ^ sw) << 4);
+    }
+    else
+    {
+        // transposing read: lane 16g + i supplies row k = 32 * (g >> 1) + 8r + (i >> 1) (r = 0..3),
+        // byte half (i & 1) of the 16-byte chunk with columns 16 * (g & 1).. of the tile, and
+        // receives column 16 * (g & 1) + i with 8 consecutive k
+        const int tr_i = lane & 15;
+        const int tr_g = lane >> 4;
+        const int krow = (tr_g >> 1) * 32 + (tr_i >> 1);
+        b_lane[0]      = W4_B_BASE + krow * BN + 8 * (tr_i & 1);
+        b_lane[1]      = 0;
+        bsw            = krow & 7;
+        bcol           = tr_g & 1;
+    }
+
+    v8i fa[2][4];
+    v8i fb[2][4];
+    v16f acc[4][4];
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int e = 0; e < 16; e++)
+                acc[i][j][e] = 0.f;
+
+#define RD128(dst, addr, imm) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define RDTR8(dst, addr, imm) \
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define PUT4(frag, X, t)                \
+    do                                  \
+    {                                   \
+        frag[4 * (X) + 0] = t.x;        \
+        frag[4 * (X) + 1] = t.y;        \
+        frag[4 * (X) + 2] = t.z;        \
+        frag[4 * (X) + 3] = t.w;        \
+    } while(0)
+    // half X of A tile I of slab kt -> fa[Q][I]
+#define RA(kt, Q, I, X)                                                                         \
+    do                                                                                          \
+    {                                                                                           \
+        v4i t_;                                                                                 \
+        RD128(t_, lds0 + (((kt) >> 1) % W4_A_STAGES) * A2_BYTES + a_lane[(kt) & 1][X],          \
+              (I) * 32 * 2 * BK);                                                               \
+        PUT4(fa[Q][I], X, t_);                                                                  \
+    } while(0)
+    // part R of B tile J of slab kt: row-major B four transposing reads, K-contiguous B two
+#define RB(kt, Q, J, R)                                                                         \
+    do                                                                                          \
+    {                                                                                           \
+        const uint32_t s_ = lds0 + ((kt) & (STAGES - 1)) * B_BYTES;                             \
+        if constexpr(TRANS_B)                                                                   \
+        {                                                                                       \
+            if((R) < 2)                                                                         \
+            {                                                                                   \
+                v4i t_;                                                                         \
+                RD128(t_, s_ + b_lane[(R) & 1], (J) * 32 * BK);                                 \
+                PUT4(fb[Q][J], (R) & 1, t_);                                                    \
+            }                                                                                   \
+        }                                                                                       \
+        else                                                                                    \
+        {                                                                                       \
+            const uint32_t c_ = (uint32_t)(((wave_n * 8 + (J) * 2 + bcol) ^ bsw) << 4);         \
+            v2i t_;                                                                             \
+            RDTR8(t_, s_ + b_lane[0] + c_, (R) * 8 * BN);                                       \
+            fb[Q][J][2 * (R) + 0] = t_.x;                                                       \
+            fb[Q][J][2 * (R) + 1] = t_.y;                                                       \
+        }                                                                                       \
+    } while(0)
+#define WAIT_FRAGS(Q)                                                                           \
+    asm volatile("s_waitcnt lgkmcnt(0)"                                                         \
+                 : "+v"(fa[Q][0]), "+v"(fa[Q][1]), "+v"(fa[Q][2]), "+v"(fa[Q][3]),              \
+                   "+v"(fb[Q][0]), "+v"(fb[Q][1]), "+v"(fb[Q][2]), "+v"(fb[Q][3])::"memory")
+    // The B tile goes in first: the accumulator then holds the tile transposed and a lane owns runs
+    // of four consecutive columns of C (see the epilogue).  Assembly for the reason given in
+    // qgemm_w4_i8_kernel.  The compiler does not know that the statement is an MFMA and adds none
+    // of the wait states a 16-pass MFMA needs before its result may be read.  In the steady-state
+    // loop nothing reads an accumulator.  In the last slabs, whose loads and reads are conditional,
+    // the compiler keeps copies of the accumulators in scratch memory and stores them right behind
+    // the MFMA, so there the statement carries the wait states itself.
+#define MF(Q, I, J)                                                                        \
+    do                                                                                     \
+    {                                                                                      \
+        if constexpr(fast_)                                                                \
+            asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0"                       \
+                         : "+a"(acc[I][J])                                                 \
+                         : "v"(fb[Q][J]), "v"(fa[Q][I]));                                  \
+        else                                                                               \
+            asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0\n\t"                   \
+                         "s_nop 7\n\ts_nop 7\n\ts_nop 3"                                   \
+                         : "+a"(acc[I][J])                                                 \
+                         : "v"(fb[Q][J]), "v"(fa[Q][I]));                                  \
+    } while(0)
+    // slot N of 32: 0..7 A reads, 8..23 B reads (8..15 when B is K-contiguous), 24..31 loads.
+#define OTHER(kt, Q, N)                                                                     \
+    do                                                                                      \
+    {                                                                                       \
+        if constexpr((N) < 8)                                                               \
+        {                                                                                   \
+            if(fast_ || more_) RA((kt) + 1, 1 - (Q), (N) >> 1, (N) & 1);                   \
+        }                                                                                   \
+        else if constexpr((N) < 24)                                                         \
+        {                                                                                   \
+            if(fast_ || more_) RB((kt) + 1, 1 - (Q), ((N) - 8) >> 2, ((N) - 8) & 3);       \
+        }                                                                                   \
+        else if constexpr((N) < 28)                                                         \
+        {                                                                                   \
+            if(fast_ || ldb_) issue_b((kt) + 4, (N) - 24);                                  \
+        }                                                                                   \
+        else                                                                                \
+        {                                                                                   \
+            if(fast_ || lda_) issue_a(ass_, (1 - (Q)) * 4 + (N) - 28);                      \
+        }                                                                                   \
+    } while(0)
+#define ROW(kt, Q, I)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        SB(); MF(Q, I, 0); SB(); OTHER(kt, Q, 8 * (I) + 0); SB(); OTHER(kt, Q, 8 * (I) + 1);  \
+        SB(); MF(Q, I, 1); SB(); OTHER(kt, Q, 8 * (I) + 2); SB(); OTHER(kt, Q, 8 * (I) + 3);  \
+        SB(); MF(Q, I, 2); SB(); OTHER(kt, Q, 8 * (I) + 4); SB(); OTHER(kt, Q, 8 * (I) + 5);  \
+        SB(); MF(Q, I, 3); SB(); OTHER(kt, Q, 8 * (I) + 6); SB(); OTHER(kt, Q, 8 * (I) + 7);  \
+    } while(0)
+#define WAIT_SLAB(kt)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        const int cnt_ = issued_in((kt) - 2) + issued_in((kt) - 1);                          \
+        if(cnt_ >= 16)      wait_vmcnt<16>();                                               \
+        else if(cnt_ >= 12) wait_vmcnt<12>();                                               \
+        else if(cnt_ >= 8)  wait_vmcnt<8>();                                                \
+        else if(cnt_ >= 4)  wait_vmcnt<4>();                                                \
+        else                wait_vmcnt<0>();                                                \
+    } while(0)
+#define SLAB(kt, Q, FAST)                                                                   \
+    do                                                                                      \
+    {                                                                                       \
+        constexpr bool fast_ = (FAST);                                                      \
+        const int kt_     = (kt);                                                           \
+        const bool more_  = kt_ + 1 < nk;                                                   \
+        const bool ldb_   = issues_b(kt_);                                                  \
+        const bool lda_   = issues_a(kt_);                                                  \
+        const int ass_    = a_step_of(kt_);                                                 \
+        (void)more_; (void)ldb_; (void)lda_;                                                \
+        WAIT_FRAGS(Q);                                                                      \
+        if constexpr(fast_)                                                                 \
+            wait_vmcnt<16>();                                                               \
+        else if(more_)                                                                      \
+            WAIT_SLAB(kt_);                                                                 \
+        block_barrier();                                                                    \
+        ROW(kt_, Q, 0); ROW(kt_, Q, 1); ROW(kt_, Q, 2); ROW(kt_, Q, 3);                     \
+        SB();                                                                               \
+    } while(0)
+
+    // ---- main loop: the schedule of qgemm_w4_i8_kernel ------------------------------------------
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+        issue_a(0, h);
+#pragma unroll
+    for(int kt = -4; kt < 0; kt++)
+    {
+        if(issues_b(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_b(kt + 4, h);
+        }
+        if(issues_a(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_a(a_step_of(kt), ((kt & 1) != 0 ? 0 : 4) + h);
+        }
+    }
+    {
+        const int cnt = issued_in(-3) + issued_in(-2) + issued_in(-1);
+        if(cnt >= 24)      wait_vmcnt<24>();
+        else if(cnt == 20) wait_vmcnt<20>();
+        else if(cnt == 16) wait_vmcnt<16>();
+        else if(cnt == 12) wait_vmcnt<12>();
+        else if(cnt == 8)  wait_vmcnt<8>();
+        else if(cnt == 4)  wait_vmcnt<4>();
+        else               wait_vmcnt<0>();
+    }
+    block_barrier();
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+    {
+        RA(0, 0, i, 0);
+        RA(0, 0, i, 1);
+    }
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+    {
+        RB(0, 0, j, 0);
+        RB(0, 0, j, 1);
+        RB(0, 0, j, 2);
+        RB(0, 0, j, 3);
+    }
+    int kt = 0;
+    for(; kt + 6 < nk; kt += 2)
+    {
+        SLAB(kt, 0, true);
+        SLAB(kt + 1, 1, true);
+    }
+    // The second half of the accumulators was written last: it passes through a statement that
+    // holds the wait states before anything the compiler places here can read it.  The first half
+    // is at least eight MFMAs old.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3"
+                 : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
+                   "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
+    for(; kt + 1 < nk; kt += 2)
+    {
+        SLAB(kt, 0, false);
+        SLAB(kt + 1, 1, false);
+    }
+    if(kt < nk)
+        SLAB(kt, 0, false);
+#undef SLAB
+#undef WAIT_SLAB
+#undef ROW
+#undef OTHER
+#undef MF
+#undef WAIT_FRAGS
+#undef RB
+#undef RA
+#undef PUT4
+#undef SB
+#undef RDTR8
+#undef RD128
+
+    // ---- epilogue: the fp8 part of qgemm_dma_kernel's, 4 x 4 tiles per wave ---------------------
+    // Element e of lane l belongs to row l % 32 of the A tile and column 8*(e/4) + 4*(l/32) + e%4
+    // of the B tile: four groups of 4 consecutive columns, each written with one store.  One block
+    // of 32 columns at a time; its scales and biases are loaded ahead of the stores of the block
+    // before it (a load issued behind a store waits for it), and no more than two blocks' worth is
+    // held in registers.
+    float sa_r[4] = {1.f, 1.f, 1.f, 1.f};
+    if constexpr(DEQ)
+    {
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            const int row = min(m0 + wave_m * 128 + i * 32 + lrow, p.m - 1);
+            if(p.scale_a_mode == MI355_QP_PER_TENSOR)
+                sa_r[i] = p.scale_a[0];
+            else if(p.scale_a_mode == MI355_QP_PER_ROW)
+                sa_r[i] = p.scale_a[row];
+        }
+    }
+    float sb_c[4][4], bias_c[4][4], sb_next[4][4], bias_next[4][4];
+    auto load_block = [&](int j, float (&sb_o)[4][4], float (&bias_o)[4][4]) {
+#pragma unroll
+        for(int g = 0; g < 4; g++)
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                const int c = min(n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp + e, p.n - 1);
+                float sb    = 1.f;
+                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                    sb = p.scale_b[0];
+                else if(p.scale_b_mode == MI355_QP_PER_COL)
+                    sb = p.scale_b[c];
+                sb_o[g][e]   = sb;
+                bias_o[g][e] = p.bias != nullptr ? p.bias[c] : -0.0f;
+            }
+    };
+    if constexpr(DEQ)
+        load_block(0, sb_c, bias_c);
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+    {
+        if constexpr(DEQ)
+        {
+            if(j + 1 < 4)
+                load_block(j + 1, sb_next, bias_next);
+        }
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            const int row = m0 + wave_m * 128 + i * 32 + lrow;
+            if(row >= p.m)
+                continue;
+            const float sa = sa_r[i];
+            // 16-bit outputs: lanes l and l + 32 hold the two halves of the same 8 columns, for two
+            // column groups; one v_permlane32_swap per register gives each of them one whole group,
+            // which goes out as a single 16-byte store.  N % 8 == 0 there, so the two lanes are in
+            // or out of the matrix together (and they share their row).
+            if constexpr(VEC8)
+            {
+                static_assert(!VEC8 || (DEQ && (OUT == MI355_F16 || OUT == MI355_BF16)), "16-bit outputs only");
+#pragma unroll
+                for(int gp = 0; gp < 4; gp += 2)
+                {
+                    uint32_t pk[2][2];
+#pragma unroll
+                    for(int h = 0; h < 2; h++)
+                    {
+                        uint16_t q[4];
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            float v = acc[i][j][4 * (gp + h) + e] * (sa * sb_c[gp + h][e]);
+                            v       = add_bias(v, bias_c[gp + h][e]);
+                            q[e]    = OUT == MI355_F16 ? convert_f32_to_half(v) : convert_f32_to_bf16(v);
+                        }
+                        pk[h][0] = q[0] | ((uint32_t)q[1] << 16);
+                        pk[h][1] = q[2] | ((uint32_t)q[3] << 16);
+                    }
+                    const auto r0 = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
+                    const auto r1 = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
+                    const int col = n0 + wave_n * 128 + j * 32 + 8 * (gp + lgrp);
+                    if(col < p.n)
+                    {
+                        const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                        store_c(reinterpret_cast<v4u*>(static_cast<uint16_t*>(p.c) + idx),
+                                v4u{r0[0], r1[0], r0[1], r1[1]}, p.stream_c);
+                    }
+                }
+            }
+            else
+            {
+#pragma unroll
+                for(int g = 0; g < 4; g++)
+                {
+                    const int col = n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp;
+                    if(col >= p.n)
+                        continue;
+                    const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                    float v[4];
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                    {
+                        v[e] = acc[i][j][4 * g + e];
+                        if constexpr(DEQ)
+                            // the accumulator is a float: double(acc) * double(s) rounded once to float
+                            // is exactly the correctly rounded fp32 product
+                            v[e] = add_bias(v[e] * (sa * sb_c[g][e]), bias_c[g][e]);
+                    }
+                    if constexpr(!DEQ || OUT == MI355_F32)
+                        store_c(reinterpret_cast<v4f*>(static_cast<float*>(p.c) + idx), v4f{v[0], v[1], v[2], v[3]},
+                                p.stream_c);
+                    else if constexpr(OUT == MI355_F16)
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                            convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+                    else
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
+                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
+                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                }
+            }
+        }
+        if constexpr(DEQ)
+        {
+            if(j + 1 < 4)
+            {
+#pragma unroll
+                for(int g = 0; g < 4; g++)
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                    {
+                        sb_c[g][e]   = sb_next[g][e];
+                        bias_c[g][e] = bias_next[g][e];
+                    }
+            }
+        }
+    }
+}
+
 template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
 int launch_one(const dma_params& p, int batch, hipStream_t stream)
 {
+    if constexpr(FP8)
+    {
+        // as for int8 (launch_i8_one): the four-wave kernel from K = 3072 on, where C takes whole
+        // groups of 4 outputs
+        if(p.k >= 3072 && p.vec_store && p.n % 4 == 0)
+        {
+            constexpr bool half_out = DEQ && (OUT == MI355_F16 || OUT == MI355_BF16);
+            auto kern4 = qgemm_w4_f8_kernel<TRANS_B, DEQ, OUT, false>;
+            if constexpr(half_out)
+            {
+                if(p.vec8_store)
+                    kern4 = qgemm_w4_f8_kernel<TRANS_B, DEQ, OUT, true>;
+            }
+            // once per kernel: above the 64 KiB default
+            static const hipError_t attr4 = hipFuncSetAttribute(
+                reinterpret_cast<const void*>(qgemm_w4_f8_kernel<TRANS_B, DEQ, OUT, false>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
+            static const hipError_t attr8 =
+                half_out ? hipFuncSetAttribute(reinterpret_cast<const void*>(qgemm_w4_f8_kernel<TRANS_B, DEQ, OUT, half_out>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES)
+                         : hipSuccess;
+            if(attr4 != hipSuccess || attr8 != hipSuccess)
+                return MI355_ERR_LAUNCH;
+            dim3 grid4(p.tiles_m * p.tiles_n, batch);
+            hipLaunchKernelGGL(kern4, grid4, dim3(W4_THREADS), W4_LDS_BYTES, stream, p);
+            return mi355_launch_status();
+        }
+    }
     auto kern = qgemm_dma_kernel<FP8, TRANS_B, DEQ, OUT>;
     // above the 64 KiB default: opt in once per kernel instantiation
     static const hipError_t attr = hipFuncSetAttribute(

@@ -413,6 +413,70 @@ def test_fp8_bias_epilogue(ops, m, n, k, out):
     assert _fp8_close(plain.cpu().numpy(), ref, _fp8_bound(xq, wq) * float(sx) * float(sw)).all()
 
 
+@pytest.mark.parametrize("m,n,k,batch,trans_b", [
+    (260, 264, 3072, 1, False), (512, 520, 3200, 1, True), (100, 1028, 4224, 1, False),
+    (256, 256, 3072, 2, True), (1024, 768, 3968, 1, False)])
+def test_fp8_four_wave_kernel_small_integers_exact(ops, m, n, k, batch, trans_b):
+    """From K = 3072 on fp8 runs on four waves of 128 x 128 (K a whole number of 128-wide slabs or
+    not, an odd and an even number of them, ragged M and N, batches).  Small-integer operands make
+    every partial sum exact in fp32, so each element must equal the reference bit for bit whatever
+    the order of accumulation: a misplaced fragment, slab or tile shows."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k + batch)
+    a = orc.fp8_from_f32(rng.integers(-8, 9, (batch, m, k)).astype(np.float32))
+    b = orc.fp8_from_f32(rng.integers(-8, 9, (batch, k, n)).astype(np.float32))
+    want = np.stack([orc.quant_dot(a[i], b[i], orc.FP8) for i in range(batch)])
+    tb = dev(np.ascontiguousarray(b.transpose(0, 2, 1))).transpose(1, 2) if trans_b else dev(b)
+    print("fp8 w4 exact", m, n, k, batch, trans_b, flush=True)
+    got = ops.quant_dot(dev(a), tb, fp8=True).cpu().numpy()
+    assert got.dtype == np.float32 and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(384, 512, 4096, False), (200, 264, 3072, True)])
+def test_fp8_four_wave_kernel_accumulators(ops, m, n, k, trans_b):
+    """Operands over the whole e4m3 range: the tolerance of the fp8 path, as for the shorter K."""
+    rng = np.random.default_rng(m + n + k)
+    a = _fp8_codes(rng, (m, k), 1.0 * 100)
+    b = _fp8_codes(rng, (k, n), 0.02 * 5000)
+    want = orc.quant_dot(a, b, orc.FP8)
+    tb = dev(np.ascontiguousarray(b.T)).t() if trans_b else dev(b)
+    print("fp8 w4 acc", m, n, k, trans_b, flush=True)
+    got = ops.quant_dot(dev(a), tb, fp8=True).cpu().numpy()
+    ok = _fp8_close(got, want, _fp8_bound(a, b))
+    assert ok.all(), (np.abs(got - want).max(), (~ok).sum())
+    rel = np.abs(got - want) / np.maximum(np.abs(want), 1e-30)
+    assert np.median(rel) < 1e-4
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(260, 264, 3072, False), (512, 520, 3200, True), (100, 1028, 4224, False),
+                                           (77, 130, 3072, False)])
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("row_scales", [False, True])
+def test_fp8_four_wave_kernel_dequantizing_epilogue(ops, m, n, k, trans_b, out, row_scales):
+    """Scales per column and per tensor or per row, a bias and the truncating converts in the
+    four-wave kernel's epilogue, with 16-byte, 8-byte and single stores (N % 8 == 0, N % 4 == 0,
+    neither).  Small-integer operands: the accumulators are exact, so the output must be the
+    reference's dequantizelinear -> add -> convert bit for bit."""
+    rng = np.random.default_rng(m + n + k)
+    a = orc.fp8_from_f32(rng.integers(-8, 9, (m, k)).astype(np.float32))
+    bm = orc.fp8_from_f32(rng.integers(-8, 9, (k, n)).astype(np.float32))
+    sa = rng.uniform(0.01, 0.05, m).astype(np.float32) if row_scales else np.float32([0.0371])
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 3).astype(np.float32)
+    acc = orc.quant_dot(a, bm, orc.FP8)
+    scale = (sa.reshape(-1, 1) * sb[None, :]).astype(np.float32) * np.ones((m, 1), np.float32)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.F32, orc.F32) + bias[None, :]
+    assert want.dtype == np.float32
+    tb = dev(np.ascontiguousarray(bm.T)).t() if trans_b else dev(bm)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    print("fp8 w4 dq", m, n, k, trans_b, out, row_scales, flush=True)
+    got = ops.quant_dot(dev(a), tb, fp8=True, scale_a=dev(sa), scale_b=dev(sb), out_dtype=td, bias=dev(bias))
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        ot = orc.F16 if out == "f16" else orc.BF16
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
 def test_bias_needs_the_epilogue(ops):
     a = dev(np.ones((16, 16), np.int8))
     with pytest.raises(Exception):
