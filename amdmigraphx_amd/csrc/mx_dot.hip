@@ -21,6 +21,14 @@
 // quant_dot); small sums are exact.
 #include "common.h"
 
+// the LDS-staged kernel for packed fp4 x packed fp4 and fp8 x fp8 (qgemm_dma.hip)
+bool mi355_dma_mx_supported(int64_t m, int64_t n, int64_t kbytes, int64_t lda, int64_t ldb, int64_t ldc,
+                            int64_t stride_a, int64_t stride_b, const void* a, const void* b);
+int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64_t n, int64_t kbytes,
+                        int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
+                        int64_t stride_c, int64_t batch, const uint8_t* ea, const uint8_t* eb,
+                        const uint32_t* flag, int bits, hipStream_t stream);
+
 namespace {
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
@@ -41,36 +49,65 @@ struct mx_params
     uint32_t* flag;
     uint8_t* ea; // [batch][m][nblk] exponent bytes
     uint8_t* eb; // [batch][n][nblk]
+    // staged: the layout the LDS-staged kernel loads, [batch][slab][rows rounded up to 256][4]: the
+    // blocks of a 64-byte slab of one row side by side (4 of packed fp4, 2 of fp8 and two bytes
+    // unused); rows past the end are not written and their products are dropped
+    int staged;
+    int group; // blocks per thread of mx_prepare_kernel: 4, or the slab's 2 when staged fp8
+    int rows_a, rows_b; // m and n rounded up to 256
 };
 
 __global__ void mx_clear_flag_kernel(uint32_t* flag) { *flag = 0; }
 
-// one thread per (operand, batch, row, block)
+// one thread per (operand, batch, row, group of p.group blocks): the exponent bytes of a group leave
+// as one word where the layout keeps them together
 __global__ __launch_bounds__(256) void mx_prepare_kernel(mx_params p, int batch)
 {
     const bool is_b     = blockIdx.y != 0;
     const int rows      = is_b ? p.n : p.m;
-    const int64_t total = (int64_t)batch * rows * p.nblk;
+    const int groups    = (p.nblk + p.group - 1) / p.group;
+    const int64_t total = (int64_t)batch * rows * groups;
     const int64_t i     = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if(i >= total)
         return;
-    const int blk   = (int)(i % p.nblk);
-    const int row   = (int)((i / p.nblk) % rows);
-    const int bt    = (int)(i / ((int64_t)p.nblk * rows));
-    const float* s  = is_b ? p.scale_b + bt * p.sb_batch + row * p.sb_row + blk * p.sb_block
-                           : p.scale_a + bt * p.sa_batch + row * p.sa_row + blk * p.sa_block;
-    const int64_t e = is_b ? p.sb_elem : p.sa_elem;
-    const uint32_t first = __builtin_bit_cast(uint32_t, s[0]);
-    const uint32_t field = (first >> 23) & 0xffu;
-    // a positive normal power of two: no sign, no mantissa, exponent field 1..254
-    bool ok = (first & 0x807fffffu) == 0 && field >= 1 && field <= 254;
-    if(e != 0)
+    const int grp  = (int)(i % groups);
+    const int row  = (int)((i / groups) % rows);
+    const int bt   = (int)(i / ((int64_t)groups * rows));
+    const float* s = is_b ? p.scale_b + bt * p.sb_batch + row * p.sb_row : p.scale_a + bt * p.sa_batch + row * p.sa_row;
+    const int64_t sblock = is_b ? p.sb_block : p.sa_block;
+    const int64_t e      = is_b ? p.sb_elem : p.sa_elem;
+    bool ok        = true;
+    uint32_t word  = 0;
+    const int nb   = min(p.group, p.nblk - p.group * grp);
+    for(int c = 0; c < nb; c++)
     {
-        const int last = min(32, p.k - blk * 32);
-        for(int j = 1; j < last; j++)
-            ok = ok && __builtin_bit_cast(uint32_t, s[j * e]) == first;
+        const int blk        = p.group * grp + c;
+        const float* sp      = s + blk * sblock;
+        const uint32_t first = __builtin_bit_cast(uint32_t, sp[0]);
+        const uint32_t field = (first >> 23) & 0xffu;
+        // a positive normal power of two: no sign, no mantissa, exponent field 1..254
+        ok = ok && (first & 0x807fffffu) == 0 && field >= 1 && field <= 254;
+        if(e != 0)
+        {
+            const int last = min(32, p.k - blk * 32);
+            for(int j = 1; j < last; j++)
+                ok = ok && __builtin_bit_cast(uint32_t, sp[j * e]) == first;
+        }
+        word |= field << (8 * c);
     }
-    (is_b ? p.eb : p.ea)[i] = (uint8_t)field;
+    uint8_t* out = is_b ? p.eb : p.ea;
+    if(p.staged)
+    {
+        // whole slabs only, one word each
+        const int padded = is_b ? p.rows_b : p.rows_a;
+        *reinterpret_cast<uint32_t*>(out + (((int64_t)bt * groups + grp) * padded + row) * 4) = word;
+    }
+    else
+    {
+        uint8_t* o = out + ((int64_t)bt * rows + row) * p.nblk + p.group * grp;
+        for(int c = 0; c < nb; c++)
+            o[c] = (uint8_t)(word >> (8 * c));
+    }
     if(!ok)
         *p.flag = 1;
 }
@@ -94,15 +131,22 @@ MI355_DEVINL float operand_value(const uint8_t* base, int k, int packed)
 }
 
 // the operator's own arithmetic, for scales the matrix-core path cannot take
-__global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p)
+// (a fixed, modest number of workgroups walks the 16 x 16 tiles: when the flag is down -- the usual
+// case -- the launch is over after that many reads of it, whatever the size of C)
+__global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p, int batch)
 {
     if(*p.flag == 0)
         return;
-    const int col = blockIdx.x * 16 + (threadIdx.x & 15);
-    const int row = blockIdx.y * 16 + (threadIdx.x >> 4);
-    const int bt  = blockIdx.z;
+    const int tiles_n   = (p.n + 15) / 16;
+    const int tiles_m   = (p.m + 15) / 16;
+    const int64_t tiles = (int64_t)batch * tiles_m * tiles_n;
+    for(int64_t t = blockIdx.x; t < tiles; t += gridDim.x)
+    {
+    const int col = (int)(t % tiles_n) * 16 + (threadIdx.x & 15);
+    const int row = (int)((t / tiles_n) % tiles_m) * 16 + (threadIdx.x >> 4);
+    const int bt  = (int)(t / ((int64_t)tiles_n * tiles_m));
     if(row >= p.m || col >= p.n)
-        return;
+        continue;
     const uint8_t* a = p.a + bt * p.stride_a + row * p.lda;
     const uint8_t* b = p.b + bt * p.stride_b + col * p.ldb;
     const float* sa  = p.scale_a + bt * p.sa_batch + row * p.sa_row;
@@ -116,6 +160,7 @@ __global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p)
         sum += (double)x * (double)w;
     }
     p.c[bt * p.stride_c + (int64_t)row * p.ldc + col] = (float)sum;
+    }
 }
 
 // 128 x 128 of C per workgroup of 4 waves (2 x 2), 64 x 64 per wave as 4 x 4 tiles of 16 x 16;
@@ -240,8 +285,11 @@ extern "C" size_t mi355_quant_dot_mx_workspace_size(const mi355_mx_dot_desc* d)
 {
     if(d == nullptr || d->m <= 0 || d->n <= 0 || d->k <= 0 || d->batch <= 0)
         return 0;
-    const size_t nblk = (size_t)(d->k + 31) / 32;
-    return 16 + align16((size_t)d->batch * d->m * nblk) + align16((size_t)d->batch * d->n * nblk);
+    // rows rounded up to the 256 of the staged layout (mx_params::staged), which spends four bytes
+    // on the two blocks of an fp8 slab
+    const size_t nblk = (size_t)(d->k + 31) / 32 * (d->a_type == MI355_FP8 && d->b_type == MI355_FP8 ? 2 : 1);
+    const size_t ra = (size_t)(d->m + 255) / 256 * 256, rb = (size_t)(d->n + 255) / 256 * 256;
+    return 16 + align16((size_t)d->batch * ra * nblk) + align16((size_t)d->batch * rb * nblk);
 }
 
 extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
@@ -308,13 +356,26 @@ extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     p.flag      = reinterpret_cast<uint32_t*>(ws);
     p.ea        = ws + 16;
-    p.eb        = p.ea + align16((size_t)d->batch * d->m * p.nblk);
+    p.rows_a    = (int)((d->m + 255) / 256 * 256);
+    p.rows_b    = (int)((d->n + 255) / 256 * 256);
+    p.eb        = p.ea + align16((size_t)d->batch * p.rows_a * p.nblk * (!a4 && !b4 ? 2 : 1));
+    // both operands packed fp4 or both fp8, whole 64-byte slabs: the LDS-staged kernel
+    p.staged = a4 == b4 && d->k % (a4 ? 128 : 64) == 0 &&
+               mi355_dma_mx_supported(d->m, d->n, a_row, d->lda, d->ldb, d->ldc, d->stride_a, d->stride_b, a, b);
+    p.group = p.staged && !a4 ? 2 : 4;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(mx_clear_flag_kernel, dim3(1), dim3(1), 0, s, p.flag);
-    const int64_t most = (int64_t)d->batch * (d->m > d->n ? d->m : d->n) * p.nblk;
+    const int64_t most = (int64_t)d->batch * (d->m > d->n ? d->m : d->n) * ((p.nblk + p.group - 1) / p.group);
     hipLaunchKernelGGL(mx_prepare_kernel, dim3((unsigned)((most + 255) / 256), 2), dim3(256), 0, s, p, (int)d->batch);
     const dim3 grid((unsigned)((d->n + 127) / 128), (unsigned)((d->m + 127) / 128), (unsigned)d->batch);
-    if(a4 && b4)
+    if(p.staged)
+    {
+        const int st = mi355_dma_mx_launch(a, b, c, d->m, d->n, a_row, d->lda, d->ldb, d->ldc, d->stride_a,
+                                           d->stride_b, d->stride_c, d->batch, p.ea, p.eb, p.flag, a4 ? 4 : 8, s);
+        if(st != MI355_OK)
+            return st;
+    }
+    else if(a4 && b4)
         hipLaunchKernelGGL((mx_gemm_kernel<true, true>), grid, dim3(256), 0, s, p);
     else if(a4)
         hipLaunchKernelGGL((mx_gemm_kernel<true, false>), grid, dim3(256), 0, s, p);
@@ -322,7 +383,8 @@ extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
         hipLaunchKernelGGL((mx_gemm_kernel<false, true>), grid, dim3(256), 0, s, p);
     else
         hipLaunchKernelGGL((mx_gemm_kernel<false, false>), grid, dim3(256), 0, s, p);
-    const dim3 egrid((unsigned)((d->n + 15) / 16), (unsigned)((d->m + 15) / 16), (unsigned)d->batch);
-    hipLaunchKernelGGL(mx_exact_kernel, egrid, dim3(256), 0, s, p);
+    const int64_t etiles = (int64_t)d->batch * ((d->n + 15) / 16) * ((d->m + 15) / 16);
+    hipLaunchKernelGGL(mx_exact_kernel, dim3((unsigned)(etiles < 2048 ? etiles : 2048)), dim3(256), 0, s, p,
+                       (int)d->batch);
     return mi355_launch_status();
 }

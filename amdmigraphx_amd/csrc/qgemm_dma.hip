@@ -74,6 +74,14 @@ struct dma_params
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
     int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
     int stream_c;   // C is far larger than the caches: streaming stores
+    // block-scaled operands (qgemm_dma_kernel<.., MX>): exponent bytes of the scales as
+    // [batch][slab][rows rounded up to 256][4] (a slab of 64 operand bytes is 128 fp4 elements = 4
+    // blocks of 32, or 64 fp8 elements = 2 blocks in bytes 0 and 1), and a word that, when not
+    // zero, says the scales are not such exponents
+    const uint8_t* mx_ea  = nullptr;
+    const uint8_t* mx_eb  = nullptr;
+    const uint32_t* mx_flag = nullptr;
+    int mx_rows_a = 0, mx_rows_b = 0;
 };
 
 // s_waitcnt with only the vector-memory counter constrained
@@ -166,12 +174,28 @@ MI355_DEVINL void store1(void* c, int64_t idx, float v)
         static_cast<uint16_t*>(c)[idx] = convert_f32_to_bf16(v);
 }
 
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+// MX = 4 or 8: the operands are packed fp4 (e2m1) or fp8 (e4m3fn) codes with one power-of-two scale
+// per 32 elements along K, both K-contiguous.  Bytes are bytes: the loads, the LDS layout and the
+// fragment reads are those of fp8 with B as [N, K].  fp4: a lane's two 16-byte chunks of a slab are
+// two scale blocks, multiplied by two v_mfma_scale_f32_32x32x64_f8f6f4 (32 elements per lane each);
+// fp8: its 32 bytes are one block and one instruction.  The exponent bytes of a row's slab (four,
+// or two and two unused) travel through the LDS with the operands (2 KiB more per stage: one more
+// load per wave and slab, sixteen lanes of it), and a lane shifts its own down to byte 0 (and 1).
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT, int MX = 0>
 __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 {
+    static_assert(MX == 0 || ((MX == 4 || MX == 8) && FP8 && TRANS_B && !DEQ),
+                  "block scales: K-contiguous operands, bare result");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     using acc_t  = typename types<FP8>::acc;
     using frag_t = typename types<FP8>::frag;
+    constexpr int ST        = MX ? STAGE_BYTES + 2048 : STAGE_BYTES; // bytes of one stage
+    constexpr int PER_SLAB  = MX ? 5 : 4;                            // loads per wave and slab
+    if constexpr(MX)
+    {
+        if(*p.mx_flag != 0)
+            return;
+    }
 
     const int tid    = threadIdx.x;
     const int lane   = tid & 63;
@@ -220,20 +244,41 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     // one load at a time, so that the main loop can deal them out between runs of MFMAs (a load
     // occupies the CU's memory pipeline for about 47 cycles; 32 issued together stall every wave)
     auto issue_a = [&](int kt, int h) {
-        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * ST;
         const uint8_t* a_base = ga + (int64_t)kt * BK;
         load_to_lds(a_base + a_off[h], st + (wave + 8 * h) * 1024);
     };
     auto issue_b = [&](int kt, int h) {
-        uint8_t* st           = lds + (kt & (STAGES - 1)) * STAGE_BYTES;
+        uint8_t* st           = lds + (kt & (STAGES - 1)) * ST;
         const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
         load_to_lds(b_base + b_off[h], st + A_BYTES + (wave + 8 * h) * 1024);
+    };
+    // MX: the slab's exponent bytes, 1 KiB for the 256 rows of A (waves 0..3, a quarter each) and
+    // 1 KiB for B (waves 4..7); issued with the B blocks
+    const uint8_t* gs = nullptr;
+    if constexpr(MX)
+    {
+        const bool for_b   = wave >= 4;
+        const int rows     = for_b ? p.mx_rows_b : p.mx_rows_a;
+        const int64_t per  = (int64_t)(p.k / BK) * rows * 4; // one batch
+        gs = (for_b ? p.mx_eb : p.mx_ea) + (int64_t)blockIdx.y * per +
+             ((int64_t)(for_b ? n0 : m0) + 64 * (wave & 3)) * 4 + (lane & 15) * 16;
+    }
+    auto issue_s = [&](int kt) {
+        if constexpr(MX)
+        {
+            uint8_t* st    = lds + (kt & (STAGES - 1)) * ST + STAGE_BYTES + (wave >= 4 ? 1024 : 0) + (wave & 3) * 256;
+            const int rows = wave >= 4 ? p.mx_rows_b : p.mx_rows_a;
+            if(lane < 16)
+                load_to_lds(gs + (int64_t)kt * rows * 4, st);
+        }
     };
     auto issue_slab = [&](int kt) {
         issue_a(kt, 0);
         issue_a(kt, 1);
         issue_b(kt, 0);
         issue_b(kt, 1);
+        issue_s(kt);
     };
 
     // ---- LDS -> operand fragments --------------------------------------------
@@ -265,8 +310,11 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #pragma unroll
         for(int x = 0; x < 2; x++)
         {
-            // int8: x = step (chunk 2x + lgrp); fp8: x = part (chunk 2*lgrp + x)
-            const int chunk = FP8 ? 2 * lgrp + x : 2 * x + lgrp;
+            // int8: x = step (chunk 2x + lgrp); fp8: x = part (chunk 2*lgrp + x).  Block-scaled fp8:
+            // the instruction takes K [16 g, 16 g + 16) and [32 + 16 g, ..) from lane group g and
+            // scales K [32 g, 32 g + 32) by that group's exponent, so the group holds chunks g and
+            // 2 + g, and the two groups' first halves are the block whose scale group 0 supplies.
+            const int chunk = FP8 && MX != 8 ? 2 * lgrp + x : 2 * x + lgrp;
             a_lane[x]       = (wave_m * 128 + lrow) * BK + ((chunk ^ sw) << 4);
             if constexpr(TRANS_B)
                 b_lane[x] = A_BYTES + (wave_n * 64 + lrow) * BK + ((chunk ^ sw) << 4);
@@ -288,6 +336,12 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 
     frag_t fa[2][A_TILES];
     frag_t fb[2][2];
+    // MX: the exponent bytes of the lane's rows, [step][tile of the step]
+    int sca[2][2] = {{0, 0}, {0, 0}}, scb[2][2] = {{0, 0}, {0, 0}};
+    const uint32_t sa_lane = STAGE_BYTES + (wave_m * 128 + lrow) * 4;
+    const uint32_t sb_lane = STAGE_BYTES + 1024 + (wave_n * 64 + lrow) * 4;
+    const int sc_shift     = (MX == 4 ? 16 : 8) * lgrp;
+    (void)sa_lane; (void)sb_lane; (void)sc_shift;
 
     auto rd128 = [](uint32_t addr, auto imm) -> v4i {
         v4i r;
@@ -305,12 +359,17 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                      : "memory");
         return r;
     };
+    auto rd32 = [](uint32_t addr, auto imm) -> int {
+        int r;
+        asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(decltype(imm)::value) : "memory");
+        return r;
+    };
 #define IMM(x) std::integral_constant<int, (x)>{}
 
     // Issues the LDS reads of step S of the slab in `stage` into fa[S], fb[S].
     auto read_step = [&](int stage, auto step) {
         constexpr int S     = decltype(step)::value;
-        const uint32_t base = lds0 + stage * STAGE_BYTES;
+        const uint32_t base = lds0 + stage * ST;
         if constexpr(FP8)
         {
             const uint32_t a0 = base + a_lane[0], a1 = base + a_lane[1];
@@ -337,6 +396,13 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                 v4i lo1 = rd128(b0, IMM(32 * BK)), hi1 = rd128(b1, IMM(32 * BK));
                 fb[S][0] = v8i{lo0.x, lo0.y, lo0.z, lo0.w, hi0.x, hi0.y, hi0.z, hi0.w};
                 fb[S][1] = v8i{lo1.x, lo1.y, lo1.z, lo1.w, hi1.x, hi1.y, hi1.z, hi1.w};
+                if constexpr(MX)
+                {
+                    sca[S][0] = rd32(base + sa_lane, IMM((2 * S) * 128));
+                    sca[S][1] = rd32(base + sa_lane, IMM((2 * S + 1) * 128));
+                    scb[S][0] = rd32(base + sb_lane, IMM(0));
+                    scb[S][1] = rd32(base + sb_lane, IMM(128));
+                }
             }
             else
             {
@@ -381,7 +447,17 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #define WAIT_STEP(S)                                                                            \
     do                                                                                          \
     {                                                                                           \
-        if constexpr(FP8)                                                                       \
+        if constexpr(MX)                                                                        \
+        {                                                                                       \
+            asm volatile("s_waitcnt lgkmcnt(0)"                                                 \
+                         : "+v"(fa[S][0]), "+v"(fa[S][1]), "+v"(fb[S][0]), "+v"(fb[S][1]),      \
+                           "+v"(sca[S][0]), "+v"(sca[S][1]), "+v"(scb[S][0]), "+v"(scb[S][1])   \
+                         :                                                                      \
+                         : "memory");                                                           \
+            sca[S][0] >>= sc_shift; sca[S][1] >>= sc_shift;                                     \
+            scb[S][0] >>= sc_shift; scb[S][1] >>= sc_shift;                                     \
+        }                                                                                       \
+        else if constexpr(FP8)                                                                  \
             asm volatile("s_waitcnt lgkmcnt(0)"                                                 \
                          : "+v"(fa[S][0]), "+v"(fa[S][1]), "+v"(fb[S][0]), "+v"(fb[S][1])       \
                          :                                                                      \
@@ -423,7 +499,22 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                 const int tile = FP8 ? 2 * S + i : i;
                 // B tile first: the accumulator holds the tile transposed, so that a lane owns
                 // runs of 4 consecutive columns of C (see the epilogue)
-                acc[tile][j]   = mfma(fb[S][j], fa[S][i], acc[tile][j]);
+                if constexpr(MX == 8)
+                    acc[tile][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        fb[S][j], fa[S][i], acc[tile][j], 0, 0, 0, scb[S][j], 0, sca[S][i]);
+                else if constexpr(MX == 4)
+                {
+                    // chunk 0 of both lanes' pairs, then chunk 1 (registers 4..7 moved down: for
+                    // 4-bit codes the instruction reads four registers per operand)
+                    acc[tile][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        fb[S][j], fa[S][i], acc[tile][j], 4, 4, 0, scb[S][j], 0, sca[S][i]);
+                    acc[tile][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        __builtin_shufflevector(fb[S][j], fb[S][j], 4, 5, 6, 7, 0, 1, 2, 3),
+                        __builtin_shufflevector(fa[S][i], fa[S][i], 4, 5, 6, 7, 0, 1, 2, 3), acc[tile][j], 4, 4, 1,
+                        scb[S][j], 1, sca[S][i]);
+                }
+                else
+                    acc[tile][j] = mfma(fb[S][j], fa[S][i], acc[tile][j]);
             }
     };
 
@@ -445,9 +536,9 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
             issue_slab(s);
     // slab 0 has landed when at most the loads of slabs 1 and 2 are outstanding
     if(nk >= 3)
-        wait_vmcnt<8>();
+        wait_vmcnt<2 * PER_SLAB>();
     else if(nk == 2)
-        wait_vmcnt<4>();
+        wait_vmcnt<PER_SLAB>();
     else
         wait_vmcnt<0>();
     block_barrier();
@@ -472,11 +563,14 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
             issue_b(kt + STAGES - 1, 0);
         mfma_half(IMM(0), IMM(1));
         if(ldb)
+        {
             issue_b(kt + STAGES - 1, 1);
+            issue_s(kt + STAGES - 1);
+        }
         if(kt + 3 < nk)
-            wait_vmcnt<8>();
+            wait_vmcnt<2 * PER_SLAB>();
         else if(kt + 2 < nk)
-            wait_vmcnt<4>();
+            wait_vmcnt<PER_SLAB>();
         else
             wait_vmcnt<0>();
         WAIT_STEP(1);
@@ -2359,6 +2453,65 @@ int launch_out(const dma_params& p, int batch, bool deq, int out, hipStream_t s)
 }
 
 } // namespace
+
+// Block-scaled fp4 x fp4 or fp8 x fp8 (see qgemm_dma_kernel<.., MX>): kbytes = bytes per row of A
+// [M, kbytes] and of B [N, kbytes] (K / 2 or K), a multiple of the 64-byte slab; bits = 4 or 8;
+// ea / eb as described at dma_params::mx_ea.
+bool mi355_dma_mx_supported(int64_t m, int64_t n, int64_t kbytes, int64_t lda, int64_t ldb, int64_t ldc,
+                            int64_t stride_a, int64_t stride_b, const void* a, const void* b)
+{
+    (void)ldc;
+    if(m <= 0 || n <= 0 || kbytes < BK || kbytes % BK != 0)
+        return false;
+    if(lda % 16 != 0 || ldb % 16 != 0 || stride_a % 16 != 0 || stride_b % 16 != 0 ||
+       reinterpret_cast<uintptr_t>(a) % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0)
+        return false;
+    const int64_t lim = (int64_t)1 << 31;
+    return m * lda < lim && n * ldb < lim && m < (1 << 30) && n < (1 << 30);
+}
+
+int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64_t n, int64_t kbytes,
+                        int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
+                        int64_t stride_c, int64_t batch, const uint8_t* ea, const uint8_t* eb,
+                        const uint32_t* flag, int bits, hipStream_t stream)
+{
+    dma_params p{};
+    p.a          = static_cast<const uint8_t*>(a);
+    p.b          = static_cast<const uint8_t*>(b);
+    p.c          = c;
+    p.m          = (int)m;
+    p.n          = (int)n;
+    p.k          = (int)kbytes;
+    p.lda        = lda;
+    p.ldb        = ldb;
+    p.ldc        = ldc;
+    p.stride_a   = stride_a;
+    p.stride_b   = stride_b;
+    p.stride_c   = stride_c;
+    p.tiles_m    = (p.m + BM - 1) / BM;
+    p.tiles_n    = (p.n + BN - 1) / BN;
+    p.ksplit     = 1;
+    p.partial_ld = (int)((n + 3) / 4 * 4);
+    p.vec_store  = ldc % 4 == 0 && stride_c % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+    p.stream_c   = (double)batch * (double)m * (double)n * 4.0 >= 128.0 * 1048576.0;
+    p.mx_ea      = ea;
+    p.mx_eb      = eb;
+    p.mx_flag    = flag;
+    p.mx_rows_a  = p.tiles_m * BM;
+    p.mx_rows_b  = p.tiles_n * BN;
+    constexpr int lds_bytes = STAGES * (STAGE_BYTES + 2048);
+    auto kern4 = qgemm_dma_kernel<true, true, false, MI355_F32, 4>;
+    auto kern8 = qgemm_dma_kernel<true, true, false, MI355_F32, 8>;
+    static const hipError_t attr4 = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern4), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    static const hipError_t attr8 = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern8), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if(attr4 != hipSuccess || attr8 != hipSuccess || (bits != 4 && bits != 8))
+        return MI355_ERR_LAUNCH;
+    dim3 grid(p.tiles_m * p.tiles_n, (unsigned)batch);
+    hipLaunchKernelGGL(bits == 4 ? kern4 : kern8, grid, dim3(NTHREADS), lds_bytes, stream, p);
+    return mi355_launch_status();
+}
 
 // The direct-to-LDS kernel moves whole 16-byte chunks and cannot zero-fill a
 // partial one: K must be a multiple of the 64-byte slab, row-major B needs N a

@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_TOPS_INT8 = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_TFLOPS_FP8 = 5000.0  # dense fp8 MFMA
+PEAK_TFLOPS_FP4 = 10100.0  # dense fp4 / fp6 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes one 8192^3 int8 quant_dot launch moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # counter runs of this file scaled by the same counters' reading for a plain copy of known size
@@ -83,7 +84,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--only-headline", action="store_true",
                     help="time the headline kernel only (for counter runs under rocprofv3)")
-    ap.add_argument("--only", choices=["headline", "fp8", "gemv", "skinny", "conv"], default=None,
+    ap.add_argument("--only", choices=["headline", "fp8", "gemv", "skinny", "conv", "mx"], default=None,
                     help="run one section only, so that a rocprofv3 run holds that section's kernels alone")
     ap.add_argument("--gemv-shape", default=None, metavar="K,N",
                     help="with --only gemv: one (K, N) shape instead of the three of config 4")
@@ -388,6 +389,33 @@ def main():
                 "TOPS": round(opsn / tc / 1e12, 1), "us_per_call": round(tc * 1e6, 1)}
     except Exception as e:
         also["quant_conv_error"] = str(e)
+
+    # ---- block-scaled quant_dot (MX): packed fp4 x packed fp4 and fp8 x fp8, one exponent per 32 ----
+    # The time is that of the whole entry point: flag clear, scale preparation, product, and the
+    # launch of the exact path that finds nothing to do.
+    try:
+        skip("mx")
+        for (mm, nn, kk, fp4) in ((4096, 4096, 4096, True), (8192, 8192, 8192, True), (4096, 4096, 4096, False)):
+            kb = kk // 2 if fp4 else kk
+            am = torch.randint(0, 256, (mm, kb), dtype=torch.uint8, device=dev, generator=g)
+            bm = torch.randint(0, 256, (nn, kb), dtype=torch.uint8, device=dev, generator=g)
+            if not fp4:     # no NaN codes
+                am &= 0x77
+                bm &= 0x77
+            ea = torch.randint(-3, 4, (mm, kk // 32), device=dev, generator=g)
+            eb = torch.randint(-3, 4, (nn, kk // 32), device=dev, generator=g)
+            sam, sbm = torch.ldexp(torch.ones_like(ea, dtype=torch.float32), ea), \
+                torch.ldexp(torch.ones_like(eb, dtype=torch.float32), eb)
+            om = torch.empty((mm, nn), dtype=torch.float32, device=dev)
+            tm, _ = _time_launches(lambda: ops.quant_dot_mx(am, bm, sam, sbm, a_fp4=fp4, b_fp4=fp4, out=om),
+                                   20, 3, settle_ms=60)
+            fm = 2.0 * mm * nn * kk / tm / 1e12
+            peak = PEAK_TFLOPS_FP4 if fp4 else PEAK_TFLOPS_FP8
+            also[f"mx_quant_dot_{'fp4' if fp4 else 'fp8'}_M{mm}_N{nn}_K{kk}"] = {
+                "TFLOPS": round(fm, 1), "us_per_call": round(tm * 1e6, 1), "frac_mfma_peak": round(fm / peak, 4)}
+            del am, bm, om
+    except Exception as e:
+        also["mx_quant_dot_error"] = str(e)
 
     line = {
         "metric": "quant_dot TOPS & % MFMA peak (int8/fp8); int4 W-only GEMV GB/s & % HBM",

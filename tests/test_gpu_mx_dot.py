@@ -124,6 +124,50 @@ def test_batched(ops):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("fp4,bt,m,n,k", [
+    (True, 1, 300, 520, 128), (True, 1, 257, 260, 384), (True, 2, 130, 300, 640), (True, 1, 512, 256, 2048),
+    (False, 1, 300, 520, 64), (False, 1, 257, 260, 192), (False, 2, 130, 300, 320), (False, 1, 512, 256, 1024)])
+def test_staged_kernel_exact_sums(ops, fp4, bt, m, n, k):
+    """Packed fp4 x fp4 with K % 128 == 0 and fp8 x fp8 with K % 64 == 0 run on the LDS-staged
+    kernel (256 x 256 tiles, 64-byte slabs: one, three, five and many of them; several tiles with
+    ragged edges; batches).  Operands and scales are chosen so that every partial sum is exact in
+    fp32 (small codes, scales within a factor of four), so each output must carry the reference's
+    bits: a misplaced chunk, slab, tile or exponent byte shows."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k + bt)
+    if fp4:
+        # codes of magnitude 0, 0.5, 1, 1.5 with either sign
+        pa = rng.integers(0, 4, (bt, m, k // 2), dtype=np.uint8) | (rng.integers(0, 4, (bt, m, k // 2), dtype=np.uint8) << 4)
+        pb = rng.integers(0, 4, (bt, n, k // 2), dtype=np.uint8) | (rng.integers(0, 4, (bt, n, k // 2), dtype=np.uint8) << 4)
+        pa |= rng.integers(0, 2, pa.shape, dtype=np.uint8) << 3
+        pb |= rng.integers(0, 2, pb.shape, dtype=np.uint8) << 7
+        av = _fp4_values(pa.reshape(-1, k // 2)).reshape(bt, m, k)
+        bv = _fp4_values(pb.reshape(-1, k // 2)).reshape(bt, n, k)
+    else:
+        pa = orc.fp8_from_f32(rng.integers(-4, 5, (bt, m, k)).astype(np.float32))
+        pb = orc.fp8_from_f32(rng.integers(-4, 5, (bt, n, k)).astype(np.float32))
+        av, bv = orc.fp8_to_f32(pa), orc.fp8_to_f32(pb)
+    sa = _block_scales(rng, (bt, m), k, -1, 1)
+    sb = _block_scales(rng, (bt, n), k, -1, 1)
+    want = _reference(av, bv, np.repeat(sa, 32, axis=2), np.repeat(sb, 32, axis=2))
+    print("mx staged", fp4, bt, m, n, k, flush=True)
+    got = ops.quant_dot_mx(dev(pa), dev(pb), dev(sa), dev(sb), a_fp4=fp4, b_fp4=fp4).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+def test_staged_kernel_full_range_operands(ops):
+    """The staged kernel on operands and exponents over their whole range: the path's tolerance."""
+    rng = np.random.default_rng(21)
+    m, n, k = 384, 512, 1024
+    pa = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    pb = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    av, bv = _fp4_values(pa), _fp4_values(pb)
+    sa_c, sb_c = _block_scales(rng, (m,), k), _block_scales(rng, (n,), k)
+    sa, sb = np.repeat(sa_c, 32, axis=1), np.repeat(sb_c, 32, axis=1)
+    want = _reference(av, bv, sa, sb)
+    got = ops.quant_dot_mx(dev(pa), dev(pb), dev(sa_c), dev(sb_c), a_fp4=True, b_fp4=True).cpu().numpy()
+    assert _close(got, want, av, bv, sa, sb).all()
+
+
 @pytest.mark.parametrize("kind", ["not_a_power_of_two", "varies_inside_a_block", "negative", "zero"])
 def test_general_scales_take_the_exact_path(ops, kind):
     """Scales the instruction cannot take are found on the device; the result is then the
