@@ -1,0 +1,84 @@
+"""Scan of gfx950 assembly for the one hazard the compiler cannot see in this library's kernels.
+
+The four-wave GEMM kernels issue their MFMAs from inline assembly (so that the accumulators stay in
+the accumulation registers).  To the compiler such a statement is opaque: it does not know that the
+result arrives some passes later, and inserts none of the wait states that an ordinary instruction
+reading (or overwriting) the result registers needs behind an MFMA -- the kernels carry them
+themselves.  This scan checks that they do: for every MFMA inside an inline-assembly region it
+follows the instruction stream and reports any non-MFMA instruction that names one of the MFMA's
+destination accumulation registers before enough wait states have gone by (every instruction
+counts one, ``s_nop N`` counts N + 1).  The stream is read in layout order, branches are not
+followed: a block laid out behind an MFMA but reached another way can give a false alarm, never a
+miss on the fall-through path.
+
+Wait states (XDL write of a VGPR followed by a VALU / VMEM / LDS access, gfx940 and later):
+passes + 3, with 4 passes for v_mfma_i32_16x16x64_i8, 8 for the 4-bit and 16 for the 8-bit forms
+of v_mfma[_scale]_f32_32x32x64_f8f6f4.
+"""
+import re
+
+_RANGE = re.compile(r"^a\[(\d+):(\d+)\]$")
+_ONE = re.compile(r"^a(\d+)$")
+
+
+def _acc_regs(token):
+    m = _RANGE.match(token)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = _ONE.match(token)
+    if m:
+        return {int(m.group(1))}
+    return set()
+
+
+def _wait_states_needed(line):
+    if "i32_16x16x64_i8" in line:
+        return 4 + 3
+    if "32x32x64_f8f6f4" in line:
+        return (8 if "cbsz:4" in line and "blgp:4" in line else 16) + 3
+    if "16x16x128_f8f6f4" in line:
+        return (4 if "cbsz:4" in line and "blgp:4" in line else 8) + 3
+    return 16 + 3   # unknown form: the longest
+
+
+def scan(path, only=None):
+    """Returns (number of inline-assembly MFMAs seen, list of hazard descriptions).  ``only``: a
+    substring that a kernel's mangled name must contain to be scanned."""
+    hazards, seen = [], 0
+    kernel, in_asm, pending = None, False, []
+    with open(path) as f:
+        for number, raw in enumerate(f, 1):
+            text = raw.strip()
+            if text.startswith(";;#ASMSTART"):
+                in_asm = True
+                continue
+            if text.startswith(";;#ASMEND"):
+                in_asm = False
+                continue
+            if text.endswith(":") and not text.startswith("."):
+                kernel, pending = text[:-1], []
+                continue
+            if not text or text[0] in ".;":
+                continue
+            if only is not None and (kernel is None or only not in kernel):
+                continue
+            text = text.split(";")[0].strip()
+            parts = text.replace(",", " ").split()
+            op, operands = parts[0], parts[1:]
+            states = int(operands[0]) + 1 if op == "s_nop" else 1
+            if op.startswith("v_mfma") or op.startswith("v_smfmac"):
+                # an MFMA that accumulates into the registers of the one before it is interlocked
+                pending = [(r, w - states, n) for (r, w, n) in pending if w - states > 0]
+                if in_asm:
+                    seen += 1
+                    pending.append((_acc_regs(operands[0]), _wait_states_needed(text), number))
+                continue
+            touched = set()
+            for token in operands:
+                touched |= _acc_regs(token)
+            for regs, left, at in pending:
+                if touched & regs:
+                    hazards.append(f"{kernel}: line {number} `{text}` touches a{min(touched & regs)}.. "
+                                   f"{left} wait states early (MFMA at line {at})")
+            pending = [(r, w - states, n) for (r, w, n) in pending if w - states > 0]
+    return seen, hazards

@@ -1,0 +1,52 @@
+"""The generated code of the kernels whose MFMAs are inline assembly keeps the wait states between
+an MFMA and the first ordinary access to its result (see tests/isa_lint.py).  Compiles
+csrc/qgemm_dma.hip to assembly (about a minute and a half), no GPU needed."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+from tests import isa_lint
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+def test_lint_finds_a_read_right_behind_an_assembly_mfma(tmp_path):
+    listing = tmp_path / "sample.s"
+    listing.write_text("""
+_Z6samplev:
+	;;#ASMSTART
+	v_mfma_i32_16x16x64_i8 a[0:3], v[0:3], v[4:7], a[0:3]
+	;;#ASMEND
+	s_nop 3
+	v_accvgpr_read_b32 v8, a1
+	;;#ASMSTART
+	v_mfma_f32_32x32x64_f8f6f4 a[16:31], v[0:7], v[8:15], a[16:31]
+	;;#ASMEND
+	s_nop 7
+	s_nop 7
+	s_nop 2
+	scratch_store_dwordx4 off, a[28:31], off
+	v_mfma_i32_16x16x64_i8 a[4:7], v[0:3], v[4:7], a[4:7]
+	v_accvgpr_read_b32 v9, a5
+""")
+    seen, hazards = isa_lint.scan(str(listing))
+    # the int8 read comes 4 + 1 wait states behind (7 needed); the fp8 store 19 behind (19 needed: fine);
+    # the last MFMA is the compiler's own (outside an assembly region) and not this scan's business
+    assert seen == 2
+    assert len(hazards) == 1 and "a1" in hazards[0]
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_four_wave_kernels_keep_their_wait_states(tmp_path):
+    out = tmp_path / "qgemm_dma.s"
+    cmd = [HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"),
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only",
+           "-o", str(out), os.path.join(ROOT, "amdmigraphx_amd", "csrc", "qgemm_dma.hip")]
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=900)
+    seen, hazards = isa_lint.scan(str(out))
+    # 64 (int8) or 16 (fp8) MFMAs per slab body, several bodies per kernel, 28 kernels
+    assert seen > 5000
+    assert hazards == [], hazards[:5]
