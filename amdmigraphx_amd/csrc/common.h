@@ -93,30 +93,33 @@ MI355_DEVINL uint8_t f32_to_fp8_rne(float x)
 // `convert` op (op/convert.hpp:64-87) from float to a 16-bit float type.
 MI355_DEVINL uint16_t convert_f32_to_half(float x)
 {
-    // selects, not branches: the epilogues convert thousands of values per wave
-    const uint32_t ux   = __builtin_bit_cast(uint32_t, x);
-    const uint32_t ax   = ux & 0x7fffffffu;
-    const uint32_t sign = (ux >> 16) & 0x8000u;
-    const auto p        = __builtin_amdgcn_cvt_pkrtz(x, 0.0f);
-    uint32_t h          = __builtin_bit_cast(uint32_t, p) & 0xffffu;
-    // float subnormals: the software conversion shifts the mantissa, the hardware gives +-0
-    h = (ax != 0 && ax < 0x00800000u) ? (sign | ((ux & 0x7fffffu) >> 13)) : h;
-    h = ax >= 0x477fe000u ? (sign | 0x7bffu) : h; // |x| >= 65504: the largest finite half
-    h = ax == 0x7f800000u ? (sign | 0x7c00u) : h; // infinities stay
-    h = ax > 0x7f800000u ? 0x7e00u : h;           // NaN
+    // selects, not branches: the epilogues convert thousands of values per wave.  The hardware
+    // conversion under round-toward-zero already gives the largest finite half for every finite
+    // |x| >= 65504 and keeps infinities; what is left are NaN (one canonical result) and float
+    // subnormals (the software conversion shifts the mantissa, the hardware gives +-0).
+    const uint32_t ux = __builtin_bit_cast(uint32_t, x);
+    const uint32_t ax = ux & 0x7fffffffu;
+    const auto p      = __builtin_amdgcn_cvt_pkrtz(x, 0.0f);
+    uint32_t h        = __builtin_bit_cast(uint32_t, p) & 0xffffu;
+    h = (ax - 1u < 0x007fffffu) ? (((ux >> 16) & 0x8000u) | ((ux & 0x7fffffu) >> 13)) : h;
+    h = x != x ? 0x7e00u : h;
     return (uint16_t)h;
 }
 
 MI355_DEVINL uint16_t convert_f32_to_bf16(float x)
 {
-    const uint32_t ux   = __builtin_bit_cast(uint32_t, x);
-    const uint32_t ax   = ux & 0x7fffffffu;
-    const uint32_t sign = (ux >> 16) & 0x8000u;
-    uint32_t h          = ux >> 16;                // toward zero
-    h = ax >= 0x7f7f0000u ? (sign | 0x7f7fu) : h; // |x| >= the largest finite bf16
-    h = ax == 0x7f800000u ? (sign | 0x7f80u) : h; // infinities stay
-    h = ax > 0x7f800000u ? 0x7fc0u : h;           // NaN
-    return (uint16_t)h;
+    // toward zero: every finite value at or beyond the largest finite bf16 has that number's upper
+    // half already, infinities keep theirs; NaN gets the one canonical result
+    const uint32_t ux = __builtin_bit_cast(uint32_t, x);
+    return (uint16_t)(x != x ? 0x7fc0u : ux >> 16);
+}
+
+// two of them side by side (lo in the low half): one v_perm_b32 takes both upper halves
+MI355_DEVINL uint32_t convert_f32_to_bf16x2(float lo, float hi)
+{
+    const uint32_t ulo = lo != lo ? 0x7fc00000u : __builtin_bit_cast(uint32_t, lo);
+    const uint32_t uhi = hi != hi ? 0x7fc00000u : __builtin_bit_cast(uint32_t, hi);
+    return __builtin_amdgcn_perm(uhi, ulo, 0x07060302u);
 }
 
 // The `add` of a bias behind dequantizelinear: its own fp32 rounding, never contracted with the

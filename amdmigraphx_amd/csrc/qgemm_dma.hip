@@ -74,6 +74,8 @@ struct dma_params
     int vec_store; // rows of C keep groups of 4 outputs aligned to 4 elements
     int vec8_store; // 16-bit outputs: N % 8 == 0 and rows of C keep groups of 8 aligned to 16 bytes
     int stream_c;   // C is far larger than the caches: streaming stores
+    int vec_cols;   // the per-column arrays in use (scale_b, colsum_b, bias) are 16-byte aligned and
+                    // N % 4 == 0: four columns' values come with one load
     // block-scaled operands (qgemm_dma_kernel<.., MX>): exponent bytes of the scales as
     // [batch][slab][rows rounded up to 256][4] (a slab of 64 operand bytes is 128 fp4 elements = 4
     // blocks of 32, or 64 fp8 elements = 2 blocks in bytes 0 and 1), and a word that, when not
@@ -161,6 +163,16 @@ MI355_DEVINL void store_c(V* dst, V v, bool stream)
         __builtin_nontemporal_store(v, dst);
     else
         *dst = v;
+}
+
+// two outputs of a 16-bit type in one word, the first in the low half
+template <int OUT>
+MI355_DEVINL uint32_t pack16(float lo, float hi)
+{
+    if constexpr(OUT == MI355_F16)
+        return convert_f32_to_half(lo) | ((uint32_t)convert_f32_to_half(hi) << 16);
+    else
+        return convert_f32_to_bf16x2(lo, hi);
 }
 
 template <int OUT>
@@ -666,7 +678,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 #pragma unroll
                         for(int h = 0; h < 2; h++)
                         {
-                            uint16_t q[4];
+                            float q[4];
 #pragma unroll
                             for(int e = 0; e < 4; e++)
                             {
@@ -682,10 +694,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                                     v = (float)(d * (double)s);
                                 }
                                 v    = add_bias(v, bias_of(j, gp + h, e));
-                                q[e] = OUT == MI355_F16 ? convert_f32_to_half(v) : convert_f32_to_bf16(v);
+                                q[e] = v;
                             }
-                            pk[h][0] = q[0] | ((uint32_t)q[1] << 16);
-                            pk[h][1] = q[2] | ((uint32_t)q[3] << 16);
+                            pk[h][0] = pack16<OUT>(q[0], q[1]);
+                            pk[h][1] = pack16<OUT>(q[2], q[3]);
                         }
                         const auto r0 = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
                         const auto r1 = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
@@ -764,8 +776,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                             convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
                     else
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
-                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
-                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                            convert_f32_to_bf16x2(v[0], v[1]),
+                            convert_f32_to_bf16x2(v[2], v[3]));
                 }
                 else
                 {
@@ -1224,8 +1236,8 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                             convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
                     else
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
-                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
-                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                            convert_f32_to_bf16x2(v[0], v[1]),
+                            convert_f32_to_bf16x2(v[2], v[3]));
                 }
                 else
                 {
@@ -1582,6 +1594,29 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     float sb_c[4], bias_c[4], sb_next[4], bias_next[4];
     int32_t cs_c[4], cs_next[4];
     auto load_block = [&](int j, float (&sb_o)[4], int32_t (&cs_o)[4], float (&bias_o)[4]) {
+        if(p.vec_cols)
+        {
+            const int cv = min(n0 + wave_n * 128 + j * 16 + 4 * lgrp, p.n - 4);
+            v4f sb4      = {1.f, 1.f, 1.f, 1.f};
+            v4f bi4      = {-0.0f, -0.0f, -0.0f, -0.0f};
+            v4i cs4      = {0, 0, 0, 0};
+            if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                sb4 = v4f{p.scale_b[0], p.scale_b[0], p.scale_b[0], p.scale_b[0]};
+            else if(p.scale_b_mode == MI355_QP_PER_COL)
+                sb4 = *reinterpret_cast<const v4f*>(p.scale_b + cv);
+            if(p.zp_a != 0)
+                cs4 = *reinterpret_cast<const v4i*>(p.colsum_b + cv);
+            if(p.bias != nullptr)
+                bi4 = *reinterpret_cast<const v4f*>(p.bias + cv);
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+            {
+                sb_o[e]   = sb4[e];
+                cs_o[e]   = cs4[e];
+                bias_o[e] = bi4[e];
+            }
+            return;
+        }
 #pragma unroll
         for(int e = 0; e < 4; e++)
         {
@@ -1659,8 +1694,8 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                             convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
                     else
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
-                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
-                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                            convert_f32_to_bf16x2(v[0], v[1]),
+                            convert_f32_to_bf16x2(v[2], v[3]));
                 }
                 else
                 {
@@ -1803,8 +1838,8 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(dma_params p, int 
                            convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
         else
             *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) =
-                make_uint2(convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
-                           convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                make_uint2(convert_f32_to_bf16x2(v[0], v[1]),
+                           convert_f32_to_bf16x2(v[2], v[3]));
     }
 }
 
@@ -2276,14 +2311,75 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                 sa_r[i] = p.scale_a[row];
         }
     }
+    if constexpr(!DEQ)
+    {
+        // the bare result: row block by row block
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            const int row = m0 + wave_m * 128 + i * 32 + lrow;
+            if(row >= p.m)
+                continue;
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+#pragma unroll
+                for(int g = 0; g < 4; g++)
+                {
+                    const int col = n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp;
+                    if(col >= p.n)
+                        continue;
+                    const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
+                    const bool whole  = p.vec_store && col + 4 <= p.n;
+                    float v[4];
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        v[e] = acc[i][j][4 * g + e];
+                    float* o = static_cast<float*>(p.c) + idx;
+                    if(whole)
+                        store_c(reinterpret_cast<v4f*>(o), v4f{v[0], v[1], v[2], v[3]}, p.stream_c);
+                    else
+                    {
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            if(col + e < p.n)
+                                o[e] = v[e];
+                    }
+                }
+            }
+        }
+        return;
+    }
     float sb_c[4][4], bias_c[4][4], sb_next[4][4], bias_next[4][4];
     auto load_block = [&](int j, float (&sb_o)[4][4], float (&bias_o)[4][4]) {
 #pragma unroll
         for(int g = 0; g < 4; g++)
+        {
+            const int c0 = n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp;
+            if(p.vec_cols)
+            {
+                // N % 4 == 0: a group that starts inside N lies inside it
+                const int cv = min(c0, p.n - 4);
+                v4f sb4      = {1.f, 1.f, 1.f, 1.f};
+                v4f bi4      = {-0.0f, -0.0f, -0.0f, -0.0f};
+                if(p.scale_b_mode == MI355_QP_PER_TENSOR)
+                    sb4 = v4f{p.scale_b[0], p.scale_b[0], p.scale_b[0], p.scale_b[0]};
+                else if(p.scale_b_mode == MI355_QP_PER_COL)
+                    sb4 = *reinterpret_cast<const v4f*>(p.scale_b + cv);
+                if(p.bias != nullptr)
+                    bi4 = *reinterpret_cast<const v4f*>(p.bias + cv);
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    sb_o[g][e]   = sb4[e];
+                    bias_o[g][e] = bi4[e];
+                }
+                continue;
+            }
 #pragma unroll
             for(int e = 0; e < 4; e++)
             {
-                const int c = min(n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp + e, p.n - 1);
+                const int c = min(c0 + e, p.n - 1);
                 float sb    = 1.f;
                 if(p.scale_b_mode == MI355_QP_PER_TENSOR)
                     sb = p.scale_b[0];
@@ -2292,6 +2388,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                 sb_o[g][e]   = sb;
                 bias_o[g][e] = p.bias != nullptr ? p.bias[c] : -0.0f;
             }
+        }
     };
     if constexpr(DEQ)
         load_block(0, sb_c, bias_c);
@@ -2324,16 +2421,16 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
 #pragma unroll
                     for(int h = 0; h < 2; h++)
                     {
-                        uint16_t q[4];
+                        float q[4];
 #pragma unroll
                         for(int e = 0; e < 4; e++)
                         {
                             float v = acc[i][j][4 * (gp + h) + e] * (sa * sb_c[gp + h][e]);
                             v       = add_bias(v, bias_c[gp + h][e]);
-                            q[e]    = OUT == MI355_F16 ? convert_f32_to_half(v) : convert_f32_to_bf16(v);
+                            q[e]    = v;
                         }
-                        pk[h][0] = q[0] | ((uint32_t)q[1] << 16);
-                        pk[h][1] = q[2] | ((uint32_t)q[3] << 16);
+                        pk[h][0] = pack16<OUT>(q[0], q[1]);
+                        pk[h][1] = pack16<OUT>(q[2], q[3]);
                     }
                     const auto r0 = __builtin_amdgcn_permlane32_swap(pk[0][0], pk[1][0], false, false);
                     const auto r1 = __builtin_amdgcn_permlane32_swap(pk[0][1], pk[1][1], false, false);
@@ -2374,8 +2471,8 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                             convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
                     else
                         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.c) + idx) = make_uint2(
-                            convert_f32_to_bf16(v[0]) | ((uint32_t)convert_f32_to_bf16(v[1]) << 16),
-                            convert_f32_to_bf16(v[2]) | ((uint32_t)convert_f32_to_bf16(v[3]) << 16));
+                            convert_f32_to_bf16x2(v[0], v[1]),
+                            convert_f32_to_bf16x2(v[2], v[3]));
                 }
             }
         }
@@ -2619,6 +2716,9 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
                        reinterpret_cast<uintptr_t>(c) % 16 == 0;
         // half of the 256 MB last-level cache and more: the result streams past it
         p.stream_c = (double)d->batch * (double)d->m * (double)d->n * (double)esz >= 128.0 * 1048576.0;
+        auto aligned16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+        p.vec_cols = d->n % 4 == 0 && (d->scale_b_mode != MI355_QP_PER_COL || aligned16(scale_b)) &&
+                     (d->zp_a == 0 || aligned16(colsum_b)) && (bias == nullptr || aligned16(bias));
     }
     p.ksplit = 1;
     if(fp8 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && p.vec_store &&

@@ -203,6 +203,40 @@ def test_four_wave_kernel_dequantizing_epilogue_bit_exact(ops, m, n, k, trans_b,
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_four_wave_kernel_unaligned_column_arrays(ops, fp8):
+    """Per-column scales, column sums and biases normally come four at a time; arrays that start
+    off a 16-byte boundary are read one value at a time.  Both must give the same bits."""
+    rng = np.random.default_rng(123 + fp8)
+    m, n, k = 260, 264, 3072
+    if fp8:
+        a = orc.fp8_from_f32(rng.integers(-8, 9, (m, k)).astype(np.float32))
+        b = orc.fp8_from_f32(rng.integers(-8, 9, (k, n)).astype(np.float32))
+    else:
+        a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+        b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    sa = dev(np.float32([0.0371]))
+    sb = rng.uniform(0.001, 0.01, n + 1).astype(np.float32)
+    bias = (rng.standard_normal(n + 1) * 3).astype(np.float32)
+    ta, tb = dev(a), dev(b)
+    kw = dict(fp8=True) if fp8 else dict(zp_a=5, colsum_b=None)
+    outs = []
+    for shift in (0, 1):
+        sbt = dev(sb)[shift:shift + n] if shift else dev(np.ascontiguousarray(sb[1:]))
+        bt = dev(bias)[shift:shift + n] if shift else dev(np.ascontiguousarray(bias[1:]))
+        assert (sbt.data_ptr() % 16 == 0) == (shift == 0)
+        if not fp8:
+            cs = ops.colsum_i8(tb)
+            pad = torch.zeros(n + 1, dtype=torch.int32, device="cuda")
+            pad[1:] = cs
+            kw["colsum_b"] = pad[1:] if shift else cs
+        outs.append(ops.quant_dot(ta, tb, scale_a=sa, scale_b=sbt, out_dtype=torch.float32, bias=bt, **kw))
+    assert torch.equal(outs[0], outs[1])
+    if not fp8:
+        want = orc.qdq_matmul_int8(a, b, np.float32(0.0371), sb[1:], 5, 0, orc.F32) + bias[None, 1:]
+        assert np.array_equal(outs[0].cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_four_wave_kernel_per_row_scales(ops):
     rng = np.random.default_rng(77)
     m, n, k = 300, 260, 3072
