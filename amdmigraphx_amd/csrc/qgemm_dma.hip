@@ -1572,6 +1572,41 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     // ---- epilogue: as in the eight-wave kernel, 8 x 8 tiles per wave ---------------------------
     // acc[i][j][e]: row 16*i + (l % 16) of the wave's A block, column 16*j + 4*(l / 16) + e of its
     // B block.
+    if constexpr(!DEQ && VEC_STORE)
+    {
+        // The bare result through the LDS: stored straight from the accumulators an instruction
+        // writes 64 bytes of each of 16 rows; re-read from a row-major copy in the LDS it writes the
+        // 512 bytes of two whole rows of the wave's quadrant.  32 rows at a time, in two buffers of
+        // the wave's own 40 KiB (the operand stages are dead: every wave is past its last fragment
+        // read behind this barrier, and no load is in flight).
+        block_barrier();
+        constexpr int PITCH = 512 + 16; // bytes per row of the copy: rows start 4 banks apart
+        uint8_t* mine       = lds + wave * 40960;
+        const int out_col   = n0 + wave_n * 128 + 4 * (lane & 31);
+        int32_t* out_base   = static_cast<int32_t*>(p.c) + (int64_t)blockIdx.y * p.stride_c + out_col;
+#pragma unroll
+        for(int pass = 0; pass < 4; pass++)
+        {
+            uint8_t* buf = mine + (pass & 1) * (32 * PITCH);
+#pragma unroll
+            for(int i2 = 0; i2 < 2; i2++)
+#pragma unroll
+                for(int j = 0; j < 8; j++)
+                    *reinterpret_cast<v4i*>(buf + (16 * i2 + lrow) * PITCH + (16 * j + 4 * lgrp) * 4) =
+                        acc[2 * pass + i2][j];
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the wave's own writes are in the LDS
+#pragma unroll
+            for(int t = 0; t < 16; t++)
+            {
+                const int r   = 2 * t + (lane >> 5);
+                const v4i v   = *reinterpret_cast<const v4i*>(buf + r * PITCH + (lane & 31) * 16);
+                const int row = m0 + wave_m * 128 + 32 * pass + r;
+                if(row < p.m && out_col < p.n)
+                    store_c(reinterpret_cast<v4i*>(out_base + (int64_t)row * p.ldc), v, p.stream_c);
+            }
+        }
+        return;
+    }
     float sa_r[8];
     int64_t zrow_r[8];
     if constexpr(DEQ)
@@ -1633,6 +1668,75 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     };
     if constexpr(DEQ)
         load_block(0, sb_c, cs_c, bias_c);
+    // fp32 outputs, and 16-bit ones in whole groups of 8: through the LDS like the bare result.  The
+    // wave's copy holds 256 bytes of each of its 128 rows: all 128 columns of a 16-bit type, or half
+    // of them in fp32 (two rounds); an instruction then stores 256 contiguous bytes of 4 rows.
+    if constexpr(DEQ && VEC_STORE)
+    {
+        if(OUT == MI355_F32 || p.vec8_store)
+        {
+            block_barrier();
+            constexpr int ROWB = 256 + 16;               // rows start 4 banks apart
+            constexpr int ESZ  = OUT == MI355_F32 ? 4 : 2;
+            constexpr int JP   = OUT == MI355_F32 ? 4 : 8; // 16-column blocks per round
+            uint8_t* mine      = lds + wave * 40960;
+#pragma unroll
+            for(int round = 0; round < 8 / JP; round++)
+            {
+#pragma unroll
+                for(int jj = 0; jj < JP; jj++)
+                {
+                    const int j = round * JP + jj;
+                    if(j > 0)
+                    {
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            sb_c[e]   = sb_next[e];
+                            cs_c[e]   = cs_next[e];
+                            bias_c[e] = bias_next[e];
+                        }
+                    }
+                    if(j + 1 < 8)
+                        load_block(j + 1, sb_next, cs_next, bias_next);
+#pragma unroll
+                    for(int i = 0; i < 8; i++)
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            const float s  = sa_r[i] * sb_c[e];
+                            const double d = (double)acc[i][j][e] -
+                                             (double)(int32_t)(zrow_r[i] + (int64_t)p.zp_a * cs_c[e]);
+                            v[e] = add_bias((float)(d * (double)s), bias_c[e]);
+                        }
+                        uint8_t* dst = mine + (16 * i + lrow) * ROWB + (16 * jj + 4 * lgrp) * ESZ;
+                        if constexpr(OUT == MI355_F32)
+                            *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+                        else
+                            *reinterpret_cast<uint2*>(dst) =
+                                make_uint2(pack16<OUT>(v[0], v[1]), pack16<OUT>(v[2], v[3]));
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+                const int col = n0 + wave_n * 128 + round * (JP * 16) + (lane & 15) * (16 / ESZ);
+#pragma unroll
+                for(int t = 0; t < 32; t++)
+                {
+                    const int r   = 4 * t + (lane >> 4);
+                    const v4u val = *reinterpret_cast<const v4u*>(mine + r * ROWB + (lane & 15) * 16);
+                    const int row = m0 + wave_m * 128 + r;
+                    if(row < p.m && col < p.n)
+                        store_c(reinterpret_cast<v4u*>(
+                                    static_cast<uint8_t*>(p.c) +
+                                    ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
+                                val, p.stream_c);
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for(int j = 0; j < 8; j++)
     {
@@ -2313,6 +2417,39 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
     }
     if constexpr(!DEQ)
     {
+        if(p.vec_store && p.n % 4 == 0)
+        {
+            // The bare result through the LDS, as in qgemm_w4_i8_kernel: straight from the
+            // accumulators a store instruction writes 32 bytes of each of 32 rows, from a row-major
+            // copy in the LDS the 512 bytes of two whole rows of the wave's quadrant.
+            block_barrier();
+            constexpr int PITCH = 512 + 16;
+            uint8_t* mine       = lds + wave * 40960;
+            const int out_col   = n0 + wave_n * 128 + 4 * (lane & 31);
+            float* out_base     = static_cast<float*>(p.c) + (int64_t)blockIdx.y * p.stride_c + out_col;
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                uint8_t* buf = mine + (i & 1) * (32 * PITCH);
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                        *reinterpret_cast<v4f*>(buf + lrow * PITCH + (32 * j + 8 * g + 4 * lgrp) * 4) =
+                            v4f{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                {
+                    const int r   = 2 * t + (lane >> 5);
+                    const v4f v   = *reinterpret_cast<const v4f*>(buf + r * PITCH + (lane & 31) * 16);
+                    const int row = m0 + wave_m * 128 + 32 * i + r;
+                    if(row < p.m && out_col < p.n)
+                        store_c(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), v, p.stream_c);
+                }
+            }
+            return;
+        }
         // the bare result: row block by row block
 #pragma unroll
         for(int i = 0; i < 4; i++)
@@ -2392,6 +2529,74 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
     };
     if constexpr(DEQ)
         load_block(0, sb_c, bias_c);
+    // fp32 outputs, and 16-bit ones in whole groups of 8: through the LDS like the bare result.  The
+    // wave's copy holds 256 bytes of each of its 128 rows: all 128 columns of a 16-bit type, or half
+    // of them in fp32 (two rounds); an instruction then stores 256 contiguous bytes of 4 rows.
+    if constexpr(DEQ && (OUT == MI355_F32 || VEC8))
+    {
+        block_barrier();
+        constexpr int ROWB = 256 + 16;               // rows start 4 banks apart
+        constexpr int ESZ  = OUT == MI355_F32 ? 4 : 2;
+        constexpr int JP   = OUT == MI355_F32 ? 2 : 4; // 32-column blocks per round
+        uint8_t* mine      = lds + wave * 40960;
+#pragma unroll
+        for(int round = 0; round < 4 / JP; round++)
+        {
+#pragma unroll
+            for(int jj = 0; jj < JP; jj++)
+            {
+                const int j = round * JP + jj;
+                if(j + 1 < 4)
+                    load_block(j + 1, sb_next, bias_next);
+#pragma unroll
+                for(int i = 0; i < 4; i++)
+                {
+                    const float sa = sa_r[i];
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            // the accumulator is a float: double(acc) * double(s) rounded once to
+                            // float is exactly the correctly rounded fp32 product
+                            v[e] = add_bias(acc[i][j][4 * g + e] * (sa * sb_c[g][e]), bias_c[g][e]);
+                        uint8_t* dst = mine + (32 * i + lrow) * ROWB + (32 * jj + 8 * g + 4 * lgrp) * ESZ;
+                        if constexpr(OUT == MI355_F32)
+                            *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+                        else
+                            *reinterpret_cast<uint2*>(dst) =
+                                make_uint2(pack16<OUT>(v[0], v[1]), pack16<OUT>(v[2], v[3]));
+                    }
+                }
+                if(j + 1 < 4)
+                {
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            sb_c[g][e]   = sb_next[g][e];
+                            bias_c[g][e] = bias_next[g][e];
+                        }
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+            const int col = n0 + wave_n * 128 + round * (JP * 32) + (lane & 15) * (16 / ESZ);
+#pragma unroll
+            for(int t = 0; t < 32; t++)
+            {
+                const int r   = 4 * t + (lane >> 4);
+                const v4u val = *reinterpret_cast<const v4u*>(mine + r * ROWB + (lane & 15) * 16);
+                const int row = m0 + wave_m * 128 + r;
+                if(row < p.m && col < p.n)
+                    store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                                                   ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
+                            val, p.stream_c);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for(int j = 0; j < 4; j++)
     {
