@@ -193,7 +193,11 @@ MI355_DEVINL void store1(void* c, int64_t idx, float v)
 // fp8: its 32 bytes are one block and one instruction.  The exponent bytes of a row's slab (four,
 // or two and two unused) travel through the LDS with the operands (2 KiB more per stage: one more
 // load per wave and slab, sixteen lanes of it), and a lane shifts its own down to byte 0 (and 1).
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT, int MX = 0>
+// VIA_LDS: the result leaves through a row-major copy in the LDS (see the epilogue).  A separate
+// instantiation: compiled into the same kernel behind a run-time choice, the copy's code made the
+// direct stores of a large result 25 % slower (8192^3 block-scaled fp4: 382 -> 479 us) although the
+// main loop and the direct epilogue came out instruction for instruction the same.
+template <bool FP8, bool TRANS_B, bool DEQ, int OUT, int MX = 0, bool VIA_LDS = false>
 __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 {
     static_assert(MX == 0 || ((MX == 4 || MX == 8) && FP8 && TRANS_B && !DEQ),
@@ -652,6 +656,75 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
         else
             return -0.0f;
     };
+    // fp8 (and the block-scaled products) where C takes whole groups: through a row-major copy in
+    // the LDS, 32 rows of the wave's 128 x 64 part at a time (the operand stages are dead behind the
+    // barrier).  Straight from the accumulators a store instruction writes 32 bytes of each of 32
+    // rows; from the copy, the whole 256 bytes (fp32) of 4 rows or 128 bytes (16-bit) of 8.
+    // Measured on this kernel (block-scaled products, whole call): 4096^3 fp4 68 -> 63 us and fp8
+    // 96 -> 86 us, but 8192^3 fp4 424 -> 466 us and 4096 x 28672 x 4096 391 -> 423 us: with many
+    // rounds of tiles and a result far larger than the caches the direct stores are faster here
+    // (unlike in the four-wave kernels), so the launcher takes this form for results that stay
+    // cached.  It requires p.vec_store, N % 4 == 0 and, for 16-bit outputs, p.vec8_store.
+    if constexpr(FP8 && VIA_LDS)
+    {
+        constexpr int ESZ = DEQ && (OUT == MI355_F16 || OUT == MI355_BF16) ? 2 : 4;
+        {
+            block_barrier();
+            constexpr int ROWB  = 64 * ESZ + 16;  // rows start 4 banks apart
+            constexpr int PER   = 16 / ESZ;       // outputs per 16-byte piece
+            constexpr int LANES = 64 / PER;       // lanes per row of the copy
+            uint8_t* mine       = lds + wave * 16384;
+            const int col       = n0 + wave_n * 64 + (lane % LANES) * PER;
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                const float sa = sa_r[i];
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            v[e] = acc[i][j][4 * g + e];
+                            if constexpr(DEQ)
+                                v[e] = add_bias(v[e] * (sa * sb_c[j][g][e]), bias_of(j, g, e));
+                        }
+                        uint8_t* dst = mine + lrow * ROWB + (32 * j + 8 * g + 4 * lgrp) * ESZ;
+                        if constexpr(ESZ == 4)
+                            *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+                        else
+                            *reinterpret_cast<uint2*>(dst) =
+                                make_uint2(pack16<OUT>(v[0], v[1]), pack16<OUT>(v[2], v[3]));
+                    }
+                __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+                // every read before the first store (left to itself the compiler moves each read
+                // into the branch of its store: read, wait, store, one at a time)
+                constexpr int T = 32 * LANES / 64;
+                v4u val[T];
+#pragma unroll
+                for(int t = 0; t < T; t++)
+                    val[t] = *reinterpret_cast<const v4u*>(mine + (t * (64 / LANES) + lane / LANES) * ROWB +
+                                                           (lane % LANES) * 16);
+#pragma unroll
+                for(int t = 0; t < T; t++)
+                    asm volatile("" : "+v"(val[t]));
+#pragma unroll
+                for(int t = 0; t < T; t++)
+                {
+                    const int row = m0 + wave_m * 128 + 32 * i + t * (64 / LANES) + lane / LANES;
+                    if(row < p.m && col < p.n)
+                        store_c(reinterpret_cast<v4u*>(
+                                    static_cast<uint8_t*>(p.c) +
+                                    ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
+                                val[t], p.stream_c);
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for(int i = 0; i < 4; i++)
     {
@@ -1595,14 +1668,21 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                     *reinterpret_cast<v4i*>(buf + (16 * i2 + lrow) * PITCH + (16 * j + 4 * lgrp) * 4) =
                         acc[2 * pass + i2][j];
             __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the wave's own writes are in the LDS
+            // every read before the first store (left to itself the compiler moves each read into
+            // the branch of its store: read, wait, store, one at a time)
+            v4i val[16];
+#pragma unroll
+            for(int t = 0; t < 16; t++)
+                val[t] = *reinterpret_cast<const v4i*>(buf + (2 * t + (lane >> 5)) * PITCH + (lane & 31) * 16);
+#pragma unroll
+            for(int t = 0; t < 16; t++)
+                asm volatile("" : "+v"(val[t]));
 #pragma unroll
             for(int t = 0; t < 16; t++)
             {
-                const int r   = 2 * t + (lane >> 5);
-                const v4i v   = *reinterpret_cast<const v4i*>(buf + r * PITCH + (lane & 31) * 16);
-                const int row = m0 + wave_m * 128 + 32 * pass + r;
+                const int row = m0 + wave_m * 128 + 32 * pass + 2 * t + (lane >> 5);
                 if(row < p.m && out_col < p.n)
-                    store_c(reinterpret_cast<v4i*>(out_base + (int64_t)row * p.ldc), v, p.stream_c);
+                    store_c(reinterpret_cast<v4i*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
             }
         }
         return;
@@ -1673,7 +1753,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     // of them in fp32 (two rounds); an instruction then stores 256 contiguous bytes of 4 rows.
     if constexpr(DEQ && VEC_STORE)
     {
-        if(OUT == MI355_F32 || p.vec8_store)
+        // (16-bit outputs come here in whole groups of 8 only: launch_i8_one)
         {
             block_barrier();
             constexpr int ROWB = 256 + 16;               // rows start 4 banks apart
@@ -1722,16 +1802,25 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                 __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
                 const int col = n0 + wave_n * 128 + round * (JP * 16) + (lane & 15) * (16 / ESZ);
 #pragma unroll
-                for(int t = 0; t < 32; t++)
+                for(int t8 = 0; t8 < 32; t8 += 8)
                 {
-                    const int r   = 4 * t + (lane >> 4);
-                    const v4u val = *reinterpret_cast<const v4u*>(mine + r * ROWB + (lane & 15) * 16);
-                    const int row = m0 + wave_m * 128 + r;
-                    if(row < p.m && col < p.n)
-                        store_c(reinterpret_cast<v4u*>(
-                                    static_cast<uint8_t*>(p.c) +
-                                    ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
-                                val, p.stream_c);
+                    // eight reads before their eight stores (see the bare result above)
+                    v4u val[8];
+#pragma unroll
+                    for(int t = 0; t < 8; t++)
+                        val[t] = *reinterpret_cast<const v4u*>(mine + (4 * (t8 + t) + (lane >> 4)) * ROWB + (lane & 15) * 16);
+#pragma unroll
+                    for(int t = 0; t < 8; t++)
+                        asm volatile("" : "+v"(val[t]));
+#pragma unroll
+                    for(int t = 0; t < 8; t++)
+                    {
+                        const int row = m0 + wave_m * 128 + 4 * (t8 + t) + (lane >> 4);
+                        if(row < p.m && col < p.n)
+                            store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                                                           ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
+                                    val[t], p.stream_c);
+                    }
                 }
             }
             return;
@@ -1819,7 +1908,8 @@ int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
     // The four-wave kernel pays more per tile (a deeper pipeline to fill, 64 stores per wave at
     // the end) and less per slab: measured against the eight-wave kernel at 8192 x 8192 x K it is
     // 12 % slower at K = 1024, even at 2048, 2-15 % faster from 4096 on.
-    if(p.k >= 3072)
+    constexpr bool half_out = DEQ && (OUT == MI355_F16 || OUT == MI355_BF16);
+    if(p.k >= 3072 && (!VEC || !half_out || p.vec8_store))
     {
         auto kern = qgemm_w4_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
         static const hipError_t attr = hipFuncSetAttribute(
@@ -2417,7 +2507,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
     }
     if constexpr(!DEQ)
     {
-        if(p.vec_store && p.n % 4 == 0)
         {
             // The bare result through the LDS, as in qgemm_w4_i8_kernel: straight from the
             // accumulators a store instruction writes 32 bytes of each of 32 rows, from a row-major
@@ -2438,54 +2527,24 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                         *reinterpret_cast<v4f*>(buf + lrow * PITCH + (32 * j + 8 * g + 4 * lgrp) * 4) =
                             v4f{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
                 __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+                // (every read before the first store, see qgemm_w4_i8_kernel)
+                v4f val[16];
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                    val[t] = *reinterpret_cast<const v4f*>(buf + (2 * t + (lane >> 5)) * PITCH + (lane & 31) * 16);
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                    asm volatile("" : "+v"(val[t]));
 #pragma unroll
                 for(int t = 0; t < 16; t++)
                 {
-                    const int r   = 2 * t + (lane >> 5);
-                    const v4f v   = *reinterpret_cast<const v4f*>(buf + r * PITCH + (lane & 31) * 16);
-                    const int row = m0 + wave_m * 128 + 32 * i + r;
+                    const int row = m0 + wave_m * 128 + 32 * i + 2 * t + (lane >> 5);
                     if(row < p.m && out_col < p.n)
-                        store_c(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), v, p.stream_c);
+                        store_c(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
                 }
             }
             return;
         }
-        // the bare result: row block by row block
-#pragma unroll
-        for(int i = 0; i < 4; i++)
-        {
-            const int row = m0 + wave_m * 128 + i * 32 + lrow;
-            if(row >= p.m)
-                continue;
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-            {
-#pragma unroll
-                for(int g = 0; g < 4; g++)
-                {
-                    const int col = n0 + wave_n * 128 + j * 32 + 8 * g + 4 * lgrp;
-                    if(col >= p.n)
-                        continue;
-                    const int64_t idx = (int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col;
-                    const bool whole  = p.vec_store && col + 4 <= p.n;
-                    float v[4];
-#pragma unroll
-                    for(int e = 0; e < 4; e++)
-                        v[e] = acc[i][j][4 * g + e];
-                    float* o = static_cast<float*>(p.c) + idx;
-                    if(whole)
-                        store_c(reinterpret_cast<v4f*>(o), v4f{v[0], v[1], v[2], v[3]}, p.stream_c);
-                    else
-                    {
-#pragma unroll
-                        for(int e = 0; e < 4; e++)
-                            if(col + e < p.n)
-                                o[e] = v[e];
-                    }
-                }
-            }
-        }
-        return;
     }
     float sb_c[4][4], bias_c[4][4], sb_next[4][4], bias_next[4][4];
     auto load_block = [&](int j, float (&sb_o)[4][4], float (&bias_o)[4][4]) {
@@ -2584,15 +2643,25 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
             __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
             const int col = n0 + wave_n * 128 + round * (JP * 32) + (lane & 15) * (16 / ESZ);
 #pragma unroll
-            for(int t = 0; t < 32; t++)
+            for(int t8 = 0; t8 < 32; t8 += 8)
             {
-                const int r   = 4 * t + (lane >> 4);
-                const v4u val = *reinterpret_cast<const v4u*>(mine + r * ROWB + (lane & 15) * 16);
-                const int row = m0 + wave_m * 128 + r;
-                if(row < p.m && col < p.n)
-                    store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
-                                                   ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
-                            val, p.stream_c);
+                // eight reads before their eight stores (see the bare result above)
+                v4u val[8];
+#pragma unroll
+                for(int t = 0; t < 8; t++)
+                    val[t] = *reinterpret_cast<const v4u*>(mine + (4 * (t8 + t) + (lane >> 4)) * ROWB + (lane & 15) * 16);
+#pragma unroll
+                for(int t = 0; t < 8; t++)
+                    asm volatile("" : "+v"(val[t]));
+#pragma unroll
+                for(int t = 0; t < 8; t++)
+                {
+                    const int row = m0 + wave_m * 128 + 4 * (t8 + t) + (lane >> 4);
+                    if(row < p.m && col < p.n)
+                        store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                                                       ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
+                                val[t], p.stream_c);
+                }
             }
         }
         return;
@@ -2802,16 +2871,24 @@ int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64
     p.mx_rows_a  = p.tiles_m * BM;
     p.mx_rows_b  = p.tiles_n * BN;
     constexpr int lds_bytes = STAGES * (STAGE_BYTES + 2048);
-    auto kern4 = qgemm_dma_kernel<true, true, false, MI355_F32, 4>;
-    auto kern8 = qgemm_dma_kernel<true, true, false, MI355_F32, 8>;
-    static const hipError_t attr4 = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern4), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    static const hipError_t attr8 = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kern8), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if(attr4 != hipSuccess || attr8 != hipSuccess || (bits != 4 && bits != 8))
+    using kernel_t = void (*)(dma_params);
+    static const kernel_t kerns[4] = {qgemm_dma_kernel<true, true, false, MI355_F32, 4, false>,
+                                      qgemm_dma_kernel<true, true, false, MI355_F32, 8, false>,
+                                      qgemm_dma_kernel<true, true, false, MI355_F32, 4, true>,
+                                      qgemm_dma_kernel<true, true, false, MI355_F32, 8, true>};
+    static const bool attrs_ok = [] {
+        bool ok = true;
+        for(kernel_t k : kerns)
+            ok = ok && hipFuncSetAttribute(reinterpret_cast<const void*>(k),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) == hipSuccess;
+        return ok;
+    }();
+    if(!attrs_ok || (bits != 4 && bits != 8))
         return MI355_ERR_LAUNCH;
+    // a result that stays in the caches leaves through the LDS copy (whole groups of 4 outputs)
+    const bool via_lds = !p.stream_c && p.vec_store && p.n % 4 == 0;
     dim3 grid(p.tiles_m * p.tiles_n, (unsigned)batch);
-    hipLaunchKernelGGL(bits == 4 ? kern4 : kern8, grid, dim3(NTHREADS), lds_bytes, stream, p);
+    hipLaunchKernelGGL(kerns[(bits == 8 ? 1 : 0) + (via_lds ? 2 : 0)], grid, dim3(NTHREADS), lds_bytes, stream, p);
     return mi355_launch_status();
 }
 
