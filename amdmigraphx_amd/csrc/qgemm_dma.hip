@@ -886,10 +886,13 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
 // the same bits whatever order the workgroups finish in.  This is what fills the machine when a
 // skinny problem (few rows of A against a large B) has too few output tiles; 16-row tiles past the
 // last row of A are skipped in the MFMA steps.
-template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE, bool SPLITK = false>
+// VIA_LDS: the result (int32, or dequantized to fp32) leaves through a row-major copy in the LDS, as
+// in qgemm_dma_kernel and for the reason given there a separate instantiation.
+template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE, bool SPLITK = false, bool VIA_LDS = false>
 __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 {
     static_assert(!SPLITK || !DEQ, "split-K adds raw accumulators");
+    static_assert(!VIA_LDS || (VEC_STORE && !SPLITK && (!DEQ || OUT == MI355_F32)), "32-bit results in groups of 4");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid    = threadIdx.x;
@@ -1242,6 +1245,61 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             sa_r[i]   = sa;
             zrow_r[i] = p.zp_b != 0 ? (int64_t)p.zp_b * p.rowsum_a[row] - (int64_t)p.k * p.zp_a * p.zp_b : 0;
         }
+    }
+    if constexpr(VIA_LDS)
+    {
+        // 32 rows of the wave's 128 x 64 part at a time: written in the accumulators' layout (an
+        // instruction's 64 bytes of each of 16 rows), read back along the rows, stored as the whole
+        // 256 bytes of 4 rows per instruction.  The operand stages are dead behind the barrier.
+        block_barrier();
+        constexpr int ROWB = 256 + 16; // rows start 4 banks apart
+        uint8_t* mine      = lds + wave * 16384;
+        const int col      = n0 + wave_n * 64 + 4 * (lane & 15);
+#pragma unroll
+        for(int round = 0; round < 4; round++)
+        {
+#pragma unroll
+            for(int i2 = 0; i2 < 2; i2++)
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                {
+                    const int i  = 2 * round + i2;
+                    uint8_t* dst = mine + (16 * i2 + lrow) * ROWB + (16 * j + 4 * lgrp) * 4;
+                    if constexpr(!DEQ)
+                        *reinterpret_cast<v4i*>(dst) = acc[i][j];
+                    else
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                        {
+                            const float s  = sa_r[i] * sb_c[j][e];
+                            const double d = (double)acc[i][j][e] -
+                                             (double)(int32_t)(zrow_r[i] + (int64_t)p.zp_a * cs_c[j][e]);
+                            v[e] = add_bias((float)(d * (double)s), bias_c[j][e]);
+                        }
+                        *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+                    }
+                }
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+            v4u val[8];
+#pragma unroll
+            for(int t = 0; t < 8; t++)
+                val[t] = *reinterpret_cast<const v4u*>(mine + (4 * t + (lane >> 4)) * ROWB + (lane & 15) * 16);
+#pragma unroll
+            for(int t = 0; t < 8; t++)
+                asm volatile("" : "+v"(val[t]));
+#pragma unroll
+            for(int t = 0; t < 8; t++)
+            {
+                const int row = m0 + wave_m * 128 + 32 * round + 4 * t + (lane >> 4);
+                if(row < p.m && col < p.n)
+                    store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                                                   ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * 4),
+                            val[t], p.stream_c);
+            }
+        }
+        return;
     }
 #pragma unroll
     for(int j = 0; j < 4; j++)
@@ -1920,7 +1978,9 @@ int launch_i8_one(const dma_params& p, int batch, hipStream_t stream)
     }
     else
     {
-        auto kern = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC>;
+        // 32-bit results in whole groups of 4 leave through the LDS copy
+        constexpr bool lds_out = VEC && (!DEQ || OUT == MI355_F32);
+        auto kern              = qgemm_dma_i8_kernel<TRANS_B, DEQ, OUT, VEC, false, lds_out>;
         static const hipError_t attr = hipFuncSetAttribute(
             reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
         if(attr != hipSuccess)
