@@ -154,13 +154,16 @@ struct types<true>
 
 // One vector of C.  `stream`: the result is large against the last-level cache and is written
 // once: a streaming (nontemporal) store keeps it from pushing out the operand panels that every
-// L2 miss of the main loop is served from (8192^3 int8: 479 -> 468 us).  Small results stay
-// cached for whatever reads them next.
+// L2 miss of the main loop is served from (fp8 4096 x 28672 x 4096 -> fp32: 475 -> 461 us; no
+// difference at 8192^3).  Small results stay cached for whatever reads them next.  Assembly: the
+// compiler folds a nontemporal and a plain store of the same value behind a branch into one plain
+// store.
 template <class V>
 MI355_DEVINL void store_c(V* dst, V v, bool stream)
 {
+    static_assert(sizeof(V) == 16);
     if(stream)
-        __builtin_nontemporal_store(v, dst);
+        asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
     else
         *dst = v;
 }
