@@ -224,12 +224,14 @@ def quant_dot_workspace_size(m, n, k, batch=1, trans_b=False, fp8=False):
 
 
 def quant_convolution(x, w, padding=None, stride=None, dilation=None, group=1, fp8=False,
-                      scale_x=None, scale_w=None, out_dtype=None):
+                      scale_x=None, scale_w=None, out_dtype=None, out=None, workspace=None):
     """quant_convolution of a dense [N, C, spatial...] tensor with dense [O, C/group, window...]
     weights over one, two or three spatial axes (int8, or uint8 carrying fp8 e4m3fn codes with
     fp8=True), optionally with the dequantizing epilogue: ``scale_x`` one float, ``scale_w`` one
     float or one per output channel.  ``padding`` holds one value per spatial axis for both sides,
-    or the low values followed by the high ones."""
+    or the low values followed by the high ones.  ``out`` (dense, of the result's shape and type)
+    and ``workspace`` (a uint8 tensor of at least the size the library asks for) are allocated
+    here unless the caller brings them, e.g. to reuse them from call to call."""
     _require_cuda(x, w, scale_x, scale_w)
     nd = x.dim() - 2
     if nd < 1 or nd > 3 or w.dim() != x.dim():
@@ -254,6 +256,36 @@ def quant_convolution(x, w, padding=None, stride=None, dilation=None, group=1, f
         raise Mi355Error("scale_x must be a single value")
     if scale_w is not None and scale_w.numel() not in (1, o):
         raise Mi355Error("scale_w must be a scalar or have one value per output channel")
+    # the descriptor and the result's size depend on the shapes and attributes only: kept per
+    # combination, so that a layer called again costs one library call
+    key = (tuple(x.shape), tuple(w.shape), tuple(padding), tuple(stride), tuple(dilation), group, fp8, odt, dequant,
+           scale_x is None, None if scale_w is None else scale_w.numel() == 1)
+    plan = _CONV_PLANS.get(key)
+    if plan is None:
+        plan = _conv_plan(x, w, nd, n, c, o, padding, pad_hi, stride, dilation, group, fp8, odt, dequant, scale_x,
+                          scale_w)
+        if len(_CONV_PLANS) < 256:
+            _CONV_PLANS[key] = plan
+    d, out_spatial, need_bytes, run, what = plan
+    shape = (n, o, *out_spatial)
+    if out is None:
+        out = torch.empty(shape, dtype=odt, device=x.device)
+    elif tuple(out.shape) != shape or out.dtype != odt or not out.is_contiguous() or out.device != x.device:
+        raise Mi355Error("quant_convolution: out must be a dense tensor of the result's shape and type")
+    if workspace is None:
+        workspace = torch.empty(max(need_bytes, 16), dtype=torch.uint8, device=x.device)
+    elif workspace.dtype != torch.uint8 or workspace.numel() < need_bytes or workspace.device != x.device:
+        raise Mi355Error(f"quant_convolution: workspace must be a uint8 tensor of at least {need_bytes} bytes")
+    check(run(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(out), _ptr(scale_x), _ptr(scale_w), _ptr(workspace),
+              need_bytes, _stream()), what)
+    return out
+
+
+_CONV_PLANS = {}
+
+
+def _conv_plan(x, w, nd, n, c, o, padding, pad_hi, stride, dilation, group, fp8, odt, dequant, scale_x, scale_w):
+    """(descriptor, spatial lengths of the result, workspace bytes, entry point, its name)"""
     common = dict(group=group, in_type=DT.FP8 if fp8 else DT.I8, out_type=_TORCH2DT[odt], dequant=int(dequant),
                   scale_x_mode=QP.NONE if scale_x is None else QP.PER_TENSOR,
                   scale_w_mode=QP.NONE if scale_w is None else
@@ -282,11 +314,7 @@ def quant_convolution(x, w, padding=None, stride=None, dilation=None, group=1, f
               "mi355_quant_convolution3d_dims")
         out_spatial = list(lens)[lead:]
         run, what = lib().mi355_quant_convolution3d, "mi355_quant_convolution3d"
-    out = torch.empty((n, o, *out_spatial), dtype=odt, device=x.device)
-    workspace = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
-    check(run(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(out), _ptr(scale_x), _ptr(scale_w), _ptr(workspace),
-              need.value, _stream()), what)
-    return out
+    return d, out_spatial, need.value, run, what
 
 
 def colsum_i8(b):

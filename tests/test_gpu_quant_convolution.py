@@ -207,3 +207,20 @@ def test_argument_errors(ops):
     # a window larger than the padded input gives the minimum output size of one
     got = ops.quant_convolution(x, dev(np.ones((2, 4, 7, 7), np.int8)))
     assert tuple(got.shape) == (1, 2, 1, 1)
+
+
+def test_caller_provided_result_and_workspace(ops):
+    """The result and the workspace may be the caller's (reused from call to call): the same bits,
+    written in place; a workspace that is too small or a result of the wrong shape is refused."""
+    rng = np.random.default_rng(31)
+    x = rng.integers(-128, 128, (2, 8, 9, 9), dtype=np.int8)
+    w = rng.integers(-128, 128, (16, 8, 3, 3), dtype=np.int8)
+    want = ops.quant_convolution(dev(x), dev(w), (1, 1))
+    out = torch.full_like(want, -1)
+    room = torch.empty(1 << 22, dtype=torch.uint8, device="cuda")
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1), out=out, workspace=room)
+    assert got.data_ptr() == out.data_ptr() and torch.equal(out, want)
+    with pytest.raises(Exception):
+        ops.quant_convolution(dev(x), dev(w), (1, 1), workspace=torch.empty(8, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(Exception):
+        ops.quant_convolution(dev(x), dev(w), (1, 1), out=torch.empty((2, 16, 9, 8), dtype=torch.int32, device="cuda"))
