@@ -895,7 +895,8 @@ template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE, bool SPLITK = false, 
 __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
 {
     static_assert(!SPLITK || !DEQ, "split-K adds raw accumulators");
-    static_assert(!VIA_LDS || (VEC_STORE && !SPLITK && (!DEQ || OUT == MI355_F32)), "32-bit results in groups of 4");
+    // (with SPLITK: the partial sums of the workspace form, p.partial set)
+    static_assert(!VIA_LDS || (VEC_STORE && (!DEQ || OUT == MI355_F32)), "32-bit results in groups of 4");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid    = threadIdx.x;
@@ -1297,9 +1298,17 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
             {
                 const int row = m0 + wave_m * 128 + 32 * round + 4 * t + (lane >> 4);
                 if(row < p.m && col < p.n)
-                    store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
-                                                   ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * 4),
-                            val[t], p.stream_c);
+                {
+                    if constexpr(SPLITK)
+                        *reinterpret_cast<v4u*>(
+                            p.partial + (((int64_t)blockIdx.y * p.ksplit + blockIdx.z) * p.m + row) * p.partial_ld +
+                            col) = val[t];
+                    else
+                        store_c(reinterpret_cast<v4u*>(
+                                    static_cast<uint8_t*>(p.c) +
+                                    ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * 4),
+                                val[t], p.stream_c);
+                }
             }
         }
         return;
@@ -2129,15 +2138,21 @@ int launch_reduce(const dma_params& p, int batch, int shares, bool deq, int out_
 template <bool TRANS_B>
 int launch_i8_splitk(const dma_params& p, int batch, hipStream_t stream, bool deq = false, int out_type = MI355_F32)
 {
-    auto kern = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true>;
+    auto kern    = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true>;
+    auto kern_ws = qgemm_dma_i8_kernel<TRANS_B, false, MI355_F32, true, true, true>;
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
-    if(attr != hipSuccess)
+    static const hipError_t attr_ws = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kern_ws), hipFuncAttributeMaxDynamicSharedMemorySize, I8_LDS_BYTES);
+    if(attr != hipSuccess || attr_ws != hipSuccess)
         return MI355_ERR_LAUNCH;
     if(p.partial != nullptr)
     {
+        // the partial tiles of many rows leave through the LDS copy (whole rows of the wave's part
+        // per store: M = 128, N = K = 8192 33.4 -> 32.0 us); a few rows are faster straight from the
+        // accumulators (M = 16: 22.3 against 23.7 us with the copy's barrier and round trip)
         dim3 grid(p.tiles_m * p.tiles_n, batch, p.ksplit);
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
+        hipLaunchKernelGGL(p.m > 64 ? kern_ws : kern, grid, dim3(NTHREADS), I8_LDS_BYTES, stream, p);
         // shares that hold slabs: the kernel gives ceil(nk / ksplit) slabs to each, the last ones
         // may be left with none (they write nothing)
         const int nk     = p.k / BK;
