@@ -152,14 +152,23 @@ struct types<true>
     using frag = v8i;
 };
 
-// One vector of C.  `stream`: the result is large against the last-level cache and is written
-// once: a streaming (nontemporal) store keeps it from pushing out the operand panels that every
-// L2 miss of the main loop is served from (fp8 4096 x 28672 x 4096 -> fp32: 475 -> 461 us; no
-// difference at 8192^3).  Small results stay cached for whatever reads them next.  Assembly: the
+// 16 bytes of C.  store_c: straight from the accumulators, where an instruction writes 32 or 64
+// bytes of each of 16 or 32 rows.  store_rows: from the row-major copy in the LDS, where it writes
+// whole 128-byte lines; `stream`: the result is large against the last-level cache and is written
+// once, so a streaming (nontemporal) store keeps it from pushing out the operand panels that every L2
+// miss of the main loop is served from (fp8 4096 x 28672 x 4096 -> fp32: 475 -> 461 us; no
+// difference at 8192^3).  Only there: nontemporal stores of pieces of lines are far slower than
+// plain ones (block-scaled 8192^3 through the eight-wave kernel: 376 -> 630 us).  Assembly: the
 // compiler folds a nontemporal and a plain store of the same value behind a branch into one plain
 // store.
 template <class V>
-MI355_DEVINL void store_c(V* dst, V v, bool stream)
+MI355_DEVINL void store_c(V* dst, V v, bool)
+{
+    *dst = v;
+}
+
+template <class V>
+MI355_DEVINL void store_rows(V* dst, V v, bool stream)
 {
     static_assert(sizeof(V) == 16);
     if(stream)
@@ -523,13 +532,14 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                         fb[S][j], fa[S][i], acc[tile][j], 0, 0, 0, scb[S][j], 0, sca[S][i]);
                 else if constexpr(MX == 4)
                 {
-                    // chunk 0 of both lanes' pairs, then chunk 1 (registers 4..7 moved down: for
-                    // 4-bit codes the instruction reads four registers per operand)
+                    // chunk 0 of both lanes' pairs, then chunk 1: for 4-bit codes the instruction reads
+                    // four registers per operand, so registers 4..7 serve as they are (the upper half
+                    // of the shuffled vector is left undefined, which costs no copies)
                     acc[tile][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                         fb[S][j], fa[S][i], acc[tile][j], 4, 4, 0, scb[S][j], 0, sca[S][i]);
                     acc[tile][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                        __builtin_shufflevector(fb[S][j], fb[S][j], 4, 5, 6, 7, 0, 1, 2, 3),
-                        __builtin_shufflevector(fa[S][i], fa[S][i], 4, 5, 6, 7, 0, 1, 2, 3), acc[tile][j], 4, 4, 1,
+                        __builtin_shufflevector(fb[S][j], fb[S][j], 4, 5, 6, 7, -1, -1, -1, -1),
+                        __builtin_shufflevector(fa[S][i], fa[S][i], 4, 5, 6, 7, -1, -1, -1, -1), acc[tile][j], 4, 4, 1,
                         scb[S][j], 1, sca[S][i]);
                 }
                 else
@@ -719,7 +729,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
                 {
                     const int row = m0 + wave_m * 128 + 32 * i + t * (64 / LANES) + lane / LANES;
                     if(row < p.m && col < p.n)
-                        store_c(reinterpret_cast<v4u*>(
+                        store_rows(reinterpret_cast<v4u*>(
                                     static_cast<uint8_t*>(p.c) +
                                     ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
                                 val[t], p.stream_c);
@@ -1304,7 +1314,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
                             p.partial + (((int64_t)blockIdx.y * p.ksplit + blockIdx.z) * p.m + row) * p.partial_ld +
                             col) = val[t];
                     else
-                        store_c(reinterpret_cast<v4u*>(
+                        store_rows(reinterpret_cast<v4u*>(
                                     static_cast<uint8_t*>(p.c) +
                                     ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * 4),
                                 val[t], p.stream_c);
@@ -1752,7 +1762,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
             {
                 const int row = m0 + wave_m * 128 + 32 * pass + 2 * t + (lane >> 5);
                 if(row < p.m && out_col < p.n)
-                    store_c(reinterpret_cast<v4i*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
+                    store_rows(reinterpret_cast<v4i*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
             }
         }
         return;
@@ -1887,7 +1897,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                     {
                         const int row = m0 + wave_m * 128 + 4 * (t8 + t) + (lane >> 4);
                         if(row < p.m && col < p.n)
-                            store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                            store_rows(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
                                                            ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
                                     val[t], p.stream_c);
                     }
@@ -2618,7 +2628,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                 {
                     const int row = m0 + wave_m * 128 + 32 * i + 2 * t + (lane >> 5);
                     if(row < p.m && out_col < p.n)
-                        store_c(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
+                        store_rows(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
                 }
             }
             return;
@@ -2736,7 +2746,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                 {
                     const int row = m0 + wave_m * 128 + 4 * (t8 + t) + (lane >> 4);
                     if(row < p.m && col < p.n)
-                        store_c(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
+                        store_rows(reinterpret_cast<v4u*>(static_cast<uint8_t*>(p.c) +
                                                        ((int64_t)blockIdx.y * p.stride_c + (int64_t)row * p.ldc + col) * ESZ),
                                 val[t], p.stream_c);
                 }
