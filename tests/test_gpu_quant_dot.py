@@ -237,6 +237,51 @@ def test_four_wave_kernel_unaligned_column_arrays(ops, fp8):
         assert np.array_equal(outs[0].cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("k", [1024, 3072])
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("out", ["bare", "f32", "bf16"])
+def test_results_through_the_lds_copy_into_strided_batched_views(ops, k, fp8, out):
+    """The kernels write C from a row-major copy in the LDS, whole rows of a wave's part per store.
+    C here is a view with a row pitch beyond N and a batch stride beyond M x pitch, ragged in M and
+    N: every element inside must carry the oracle's bits (operands are small integers, so fp8 sums
+    are exact too) and everything around the view must stay untouched.  K = 1024 runs on the
+    eight-wave kernels, K = 3072 on the four-wave ones."""
+    rng = np.random.default_rng(k + 7 * fp8 + len(out))
+    bt, m, n, pitch, rows = 2, 300, 264, 280, 310
+    if fp8:
+        a = orc.fp8_from_f32(rng.integers(-8, 9, (bt, m, k)).astype(np.float32))
+        b = orc.fp8_from_f32(rng.integers(-8, 9, (bt, k, n)).astype(np.float32))
+    else:
+        a = rng.integers(-128, 128, (bt, m, k), dtype=np.int8)
+        b = rng.integers(-128, 128, (bt, k, n), dtype=np.int8)
+    sa = np.float32(0.0371)
+    sb = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    td = {"bare": torch.float32 if fp8 else torch.int32, "f32": torch.float32, "bf16": torch.bfloat16}[out]
+    whole = torch.full((bt, rows, pitch), 7, dtype=td, device="cuda")
+    view = whole[:, :m, :n]
+    print("lds copy", k, fp8, out, flush=True)
+    if out == "bare":
+        ops.quant_dot(dev(a), dev(b), fp8=fp8, out=view)
+        want = np.stack([orc.quant_dot(a[i], b[i], orc.FP8 if fp8 else orc.I8) for i in range(bt)])
+        assert np.array_equal(view.cpu().numpy(), want)
+    else:
+        ops.quant_dot(dev(a), dev(b), fp8=fp8, scale_a=dev(np.float32([sa])), scale_b=dev(sb), out_dtype=td, out=view)
+        ot = orc.F32 if out == "f32" else orc.BF16
+        if fp8:
+            want = np.stack([orc.qdq_matmul_fp8(a[i], b[i], sa, sb, ot) for i in range(bt)])
+        else:
+            want = np.stack([orc.qdq_matmul_int8(a[i], b[i], sa, sb, 0, 0, ot) for i in range(bt)])
+        got = view.contiguous()
+        if out == "f32":
+            assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        else:
+            assert np.array_equal(half_bits(got), want)
+    # nothing outside the view was written
+    outside = whole.clone()
+    outside[:, :m, :n] = 7
+    assert bool((outside == 7).all())
+
+
 def test_four_wave_kernel_per_row_scales(ops):
     rng = np.random.default_rng(77)
     m, n, k = 300, 260, 3072
