@@ -10,7 +10,8 @@
 // host-side decision:
 //   mx_prepare_kernel   walks the scale tensors once: a block whose 32 scales are one normal power
 //                       of two becomes its exponent byte in a compact [rows, K/32] array; anything
-//                       else raises a flag in device memory;
+//                       else raises a flag in device memory (by writing the call's number there:
+//                       the word needs no clearing, see next_ticket);
 //   mx_gemm_kernel      the matrix-core product from the compact scales; returns at once when the
 //                       flag is up;
 //   mx_exact_kernel     the operator's arithmetic one output per thread -- float(a) * scale in
@@ -21,13 +22,15 @@
 // quant_dot); small sums are exact.
 #include "common.h"
 
+#include <atomic>
+
 // the LDS-staged kernel for packed fp4 x packed fp4 and fp8 x fp8 (qgemm_dma.hip)
 bool mi355_dma_mx_supported(int64_t m, int64_t n, int64_t kbytes, int64_t lda, int64_t ldb, int64_t ldc,
                             int64_t stride_a, int64_t stride_b, const void* a, const void* b);
 int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64_t n, int64_t kbytes,
                         int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
                         int64_t stride_c, int64_t batch, const uint8_t* ea, const uint8_t* eb,
-                        const uint32_t* flag, int bits, hipStream_t stream);
+                        const uint32_t* flag, uint32_t ticket, int bits, hipStream_t stream);
 
 namespace {
 
@@ -46,7 +49,8 @@ struct mx_params
     int64_t sa_batch, sa_row, sa_block, sa_elem;
     int64_t sb_batch, sb_row, sb_block, sb_elem;
     int a4, b4; // operand stored as packed fp4 (two codes per byte, low nibble = even k)
-    uint32_t* flag;
+    uint32_t* flag;   // holds `ticket` when this call's scales are not what the matrix-core path takes
+    uint32_t ticket; // this call's number, never 0
     uint8_t* ea; // [batch][m][nblk] exponent bytes
     uint8_t* eb; // [batch][n][nblk]
     // staged: the layout the LDS-staged kernel loads, [batch][slab][rows rounded up to 256][4]: the
@@ -57,7 +61,6 @@ struct mx_params
     int rows_a, rows_b; // m and n rounded up to 256
 };
 
-__global__ void mx_clear_flag_kernel(uint32_t* flag) { *flag = 0; }
 
 // one thread per (operand, batch, row, group of p.group blocks): the exponent bytes of a group leave
 // as one word where the layout keeps them together
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(256) void mx_prepare_kernel(mx_params p, int batch)
             o[c] = (uint8_t)(word >> (8 * c));
     }
     if(!ok)
-        *p.flag = 1;
+        *p.flag = p.ticket;
 }
 
 MI355_DEVINL float fp4_value(uint32_t code)
@@ -135,7 +138,7 @@ MI355_DEVINL float operand_value(const uint8_t* base, int k, int packed)
 // case -- the launch is over after that many reads of it, whatever the size of C)
 __global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p, int batch)
 {
-    if(*p.flag == 0)
+    if(*p.flag != p.ticket)
         return;
     const int tiles_n   = (p.n + 15) / 16;
     const int tiles_m   = (p.m + 15) / 16;
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(256) void mx_exact_kernel(mx_params p, int batch)
 template <bool A4, bool B4>
 __global__ __launch_bounds__(256) void mx_gemm_kernel(mx_params p)
 {
-    if(*p.flag != 0)
+    if(*p.flag == p.ticket)
         return;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -279,6 +282,18 @@ __global__ __launch_bounds__(256) void mx_gemm_kernel(mx_params p)
 
 size_t align16(size_t x) { return (x + 15) / 16 * 16; }
 
+// The flag word of the workspace is never cleared: a call raises it by writing its own number, and
+// only that number counts.  Whatever the word held before -- an earlier call's number, or anything
+// at all in a fresh workspace -- reads as "not raised", except the one value in 2^32 that happens
+// to be this call's number; then (as after a replay of a captured call whose earlier run raised it)
+// the exact path computes the result, which is right for every input, only slower.
+uint32_t next_ticket()
+{
+    static std::atomic<uint32_t> counter{0};
+    uint32_t t = counter.fetch_add(1, std::memory_order_relaxed) + 1;
+    return t != 0 ? t : counter.fetch_add(1, std::memory_order_relaxed) + 1;
+}
+
 } // namespace
 
 extern "C" size_t mi355_quant_dot_mx_workspace_size(const mi355_mx_dot_desc* d)
@@ -355,6 +370,7 @@ extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
     p.b4       = b4;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     p.flag      = reinterpret_cast<uint32_t*>(ws);
+    p.ticket    = next_ticket();
     p.ea        = ws + 16;
     p.rows_a    = (int)((d->m + 255) / 256 * 256);
     p.rows_b    = (int)((d->n + 255) / 256 * 256);
@@ -364,14 +380,13 @@ extern "C" int mi355_quant_dot_mx(const mi355_mx_dot_desc* d,
                mi355_dma_mx_supported(d->m, d->n, a_row, d->lda, d->ldb, d->ldc, d->stride_a, d->stride_b, a, b);
     p.group = p.staged && !a4 ? 2 : 4;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(mx_clear_flag_kernel, dim3(1), dim3(1), 0, s, p.flag);
     const int64_t most = (int64_t)d->batch * (d->m > d->n ? d->m : d->n) * ((p.nblk + p.group - 1) / p.group);
     hipLaunchKernelGGL(mx_prepare_kernel, dim3((unsigned)((most + 255) / 256), 2), dim3(256), 0, s, p, (int)d->batch);
     const dim3 grid((unsigned)((d->n + 127) / 128), (unsigned)((d->m + 127) / 128), (unsigned)d->batch);
     if(p.staged)
     {
         const int st = mi355_dma_mx_launch(a, b, c, d->m, d->n, a_row, d->lda, d->ldb, d->ldc, d->stride_a,
-                                           d->stride_b, d->stride_c, d->batch, p.ea, p.eb, p.flag, a4 ? 4 : 8, s);
+                                           d->stride_b, d->stride_c, d->batch, p.ea, p.eb, p.flag, p.ticket, a4 ? 4 : 8, s);
         if(st != MI355_OK)
             return st;
     }

@@ -78,11 +78,12 @@ struct dma_params
                     // N % 4 == 0: four columns' values come with one load
     // block-scaled operands (qgemm_dma_kernel<.., MX>): exponent bytes of the scales as
     // [batch][slab][rows rounded up to 256][4] (a slab of 64 operand bytes is 128 fp4 elements = 4
-    // blocks of 32, or 64 fp8 elements = 2 blocks in bytes 0 and 1), and a word that, when not
-    // zero, says the scales are not such exponents
+    // blocks of 32, or 64 fp8 elements = 2 blocks in bytes 0 and 1), and a word that, when it holds
+    // this call's number, says the scales are not such exponents
     const uint8_t* mx_ea  = nullptr;
     const uint8_t* mx_eb  = nullptr;
     const uint32_t* mx_flag = nullptr;
+    uint32_t mx_ticket      = 0; // the value of *mx_flag that says so
     int mx_rows_a = 0, mx_rows_b = 0;
 };
 
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_kernel(dma_params p)
     constexpr int PER_SLAB  = MX ? 5 : 4;                            // loads per wave and slab
     if constexpr(MX)
     {
-        if(*p.mx_flag != 0)
+        if(*p.mx_flag == p.mx_ticket)
             return;
     }
 
@@ -2932,7 +2933,7 @@ bool mi355_dma_mx_supported(int64_t m, int64_t n, int64_t kbytes, int64_t lda, i
 int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64_t n, int64_t kbytes,
                         int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b,
                         int64_t stride_c, int64_t batch, const uint8_t* ea, const uint8_t* eb,
-                        const uint32_t* flag, int bits, hipStream_t stream)
+                        const uint32_t* flag, uint32_t ticket, int bits, hipStream_t stream)
 {
     dma_params p{};
     p.a          = static_cast<const uint8_t*>(a);
@@ -2956,6 +2957,7 @@ int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64
     p.mx_ea      = ea;
     p.mx_eb      = eb;
     p.mx_flag    = flag;
+    p.mx_ticket  = ticket;
     p.mx_rows_a  = p.tiles_m * BM;
     p.mx_rows_b  = p.tiles_n * BN;
     constexpr int lds_bytes = STAGES * (STAGE_BYTES + 2048);

@@ -398,7 +398,7 @@ def main():
         also["quant_conv_error"] = str(e)
 
     # ---- block-scaled quant_dot (MX): packed fp4 x packed fp4 and fp8 x fp8, one exponent per 32 ----
-    # The time is that of the whole entry point: flag clear, scale preparation, product, and the
+    # The time is that of the whole entry point: scale preparation, product, and the
     # launch of the exact path that finds nothing to do.
     try:
         skip("mx")
