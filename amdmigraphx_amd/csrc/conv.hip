@@ -155,6 +155,524 @@ __global__ __launch_bounds__(256) void weights_cl_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Direct (implicit-GEMM) int8 convolution for groups with a multiple of 16 channels.
+//
+// The input is first copied channels-last WITH its zero padding (xt[n][z][y][x][c], the padded
+// volume), so a 16-byte piece of a window row -- 16 consecutive channels of one window element
+// -- is one aligned 16-byte load at (position of the output element) + (offset of the window
+// element), with no bounds to check.  The main kernel is a GEMM whose rows are output positions
+// (all images flattened), whose columns are a group's output channels and whose K is
+// (window element, channel); its row operand is never materialised: every direct-to-LDS load
+// forms its address from the row's base and the K piece's offset (a table in LDS).
+//
+// Workgroup: 4 waves, 128 rows x 64 output channels, K in steps of 128 bytes through a ring of
+// LDS stages (16 KiB of rows + 8 KiB of weights each).  A load instruction fetches 8 rows x 128
+// bytes: whole cache lines when a group has 128 channels or more (64-byte pieces of 16 rows, as a
+// 64-byte K step would fetch, cost the CU's cache two line slots for one line of payload); the
+// weights are stored [group][K step][channel][128 bytes] by the kernel in front, so their loads
+// are 1 KiB contiguous.  A wave multiplies 32 rows by the 64 channels (2 x 4
+// v_mfma_i32_16x16x64_i8 per half step, rows as the first operand, so a lane ends up with four
+// consecutive output positions of one channel: 16 contiguous bytes of an NC(D)HW float result).
+// LDS rows are 128 bytes as eight 16-byte chunks, logical chunk c at position c ^ ((r >> 1) & 7);
+// a direct-to-LDS load writes lane l at base + 16 l, so the swizzle goes into the address a lane
+// fetches.
+// ---------------------------------------------------------------------------------------------
+constexpr int DC_ROWS    = 128;
+constexpr int DC_COLS    = 64;
+constexpr int DC_KSTEP   = 128;
+constexpr int DC_A_BYTES = DC_ROWS * DC_KSTEP;
+constexpr int DC_STAGE   = (DC_ROWS + DC_COLS) * DC_KSTEP;
+constexpr int DC_MAX_PIECES = 1024; // K pieces of 16 bytes a layer may have (the table is LDS)
+constexpr int DC_PITCH   = DC_ROWS * 4 + 16; // bytes of one channel's 128 results in the LDS copy
+
+struct direct_params
+{
+    const uint8_t* xt;  // padded channels-last input
+    const uint8_t* wp;  // weights [group][nk][ogp][128], (window element, channel) order, zero filled
+    void* out;
+    const float* scale_x;
+    const float* scale_w;
+    int64_t rows;       // N * plane
+    int plane, oh, ow;  // output positions per image; od = plane / (oh * ow)
+    int o, og, ogp, c, cg;
+    int kh, kw;         // kd is not needed: window element index / (kh * kw)
+    int dp, hp, wp_;    // padded input volume
+    int stride_d, stride_h, stride_w, dil_d, dil_h, dil_w;
+    int kg, nk;         // K bytes of a group's window, K steps
+    int col_tiles;      // 64-channel tiles per group
+    int dequant, scale_x_mode, scale_w_mode;
+};
+
+MI355_DEVINL void dc_load_to_lds(const uint8_t* g, uint8_t* l)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g),
+                                     (__attribute__((address_space(3))) void*)(l), 16, 0, 0);
+}
+
+template <int N>
+MI355_DEVINL void dc_wait_vmcnt()
+{
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// at most `steps` K steps of six loads may stay in flight
+MI355_DEVINL void dc_wait_steps(int steps)
+{
+    switch(steps)
+    {
+    case 0: dc_wait_vmcnt<0>(); break;
+    case 1: dc_wait_vmcnt<6>(); break;
+    case 2: dc_wait_vmcnt<12>(); break;
+    case 3: dc_wait_vmcnt<18>(); break;
+    default: dc_wait_vmcnt<24>(); break;
+    }
+}
+
+template <int OUT>
+MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
+{
+    if constexpr(OUT == MI355_I32)
+        *reinterpret_cast<v4i*>(static_cast<int32_t*>(out) + idx) = a;
+    else
+    {
+        float v[4];
+#pragma unroll
+        for(int e = 0; e < 4; e++)
+            v[e] = (float)((double)a[e] * (double)s);
+        if constexpr(OUT == MI355_F32)
+            *reinterpret_cast<v4f*>(static_cast<float*>(out) + idx) = v4f{v[0], v[1], v[2], v[3]};
+        else if constexpr(OUT == MI355_F16)
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + idx) =
+                make_uint2(convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
+                           convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+        else
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + idx) =
+                make_uint2(convert_f32_to_bf16x2(v[0], v[1]), convert_f32_to_bf16x2(v[2], v[3]));
+    }
+}
+
+// OUT: MI355_I32 (bare sums), MI355_F32 / F16 / BF16 (dequantized); VEC: the plane is a multiple of
+// 4 positions, so a lane's four rows are one image's and their store is one aligned vector.
+// STAGES: LDS ring; the loads of K step s + STAGES go out when step s has been read.
+template <int OUT, bool VEC, int STAGES>
+__global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
+{
+    static_assert(STAGES * DC_STAGE >= DC_COLS * DC_PITCH, "the result copy reuses the ring");
+    static_assert(STAGES >= 2 && STAGES <= 6);
+    constexpr int AHEAD = STAGES - 1;
+    extern __shared__ __align__(1024) uint8_t lds[];
+    int32_t* table  = reinterpret_cast<int32_t*>(lds + STAGES * DC_STAGE);
+    const int lane  = threadIdx.x & 63;
+    const int wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g     = blockIdx.y / p.col_tiles;
+    const int o0    = (blockIdx.y % p.col_tiles) * DC_COLS; // first output channel, within the group
+    const int64_t row0 = (int64_t)blockIdx.x * DC_ROWS;
+    const int nk    = p.nk;
+    const int pieces = nk * 8;
+
+    // byte offset of every K piece from a row's base: (window element, first channel)
+    for(int q = threadIdx.x; q < pieces; q += 256)
+    {
+        int off = 0;
+        if(q * 16 < p.kg)
+        {
+            const int tap = q * 16 / p.cg;
+            const int c0  = q * 16 % p.cg;
+            const int kx  = tap % p.kw;
+            const int ky  = tap / p.kw % p.kh;
+            const int kz  = tap / (p.kw * p.kh);
+            off = ((kz * p.dil_d * p.hp + ky * p.dil_h) * p.wp_ + kx * p.dil_w) * p.c + c0;
+        }
+        table[q] = off;
+    }
+    __syncthreads();
+
+    // ---- global -> LDS: a wave issues row blocks {wave + 4 h} (8 rows each) and weight blocks
+    // {wave, wave + 4} of a K step; (r >> 1) & 7 of a lane's row only depends on the block's parity
+    const int chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7); // logical chunk of this lane's position
+    const uint8_t* row_base[4];
+#pragma unroll
+    for(int h = 0; h < 4; h++)
+    {
+        int64_t r = row0 + 8 * (wave + 4 * h) + (lane >> 3);
+        r         = r < p.rows ? r : p.rows - 1;
+        int n, pos;
+        if(p.rows < ((int64_t)1 << 31))
+        {
+            n   = (int)((uint32_t)r / (uint32_t)p.plane);
+            pos = (int)((uint32_t)r - (uint32_t)n * (uint32_t)p.plane);
+        }
+        else
+        {
+            n   = (int)(r / p.plane);
+            pos = (int)(r - (int64_t)n * p.plane);
+        }
+        const int ox = pos % p.ow;
+        const int oy = pos / p.ow % p.oh;
+        const int oz = pos / (p.ow * p.oh);
+        row_base[h] = p.xt + (((((int64_t)n * p.dp + oz * p.stride_d) * p.hp + oy * p.stride_h) * (int64_t)p.wp_ +
+                               ox * p.stride_w) * p.c + g * p.cg);
+    }
+    uint32_t w_off[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+        w_off[h] = (uint32_t)((o0 + 8 * (wave + 4 * h) + (lane >> 3)) * DC_KSTEP + chunk * 16);
+    const uint8_t* w_base  = p.wp + (int64_t)g * nk * p.ogp * DC_KSTEP;
+    const uint32_t w_step  = (uint32_t)p.ogp * DC_KSTEP;
+    const uint32_t lds0    = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    const uint32_t tab0    = lds0 + STAGES * DC_STAGE;
+
+    auto read_offset = [&](int s, int& dst) {
+        const int q = min(8 * s + chunk, pieces - 1);
+        asm volatile("ds_read_b32 %0, %1" : "=v"(dst) : "v"(tab0 + 4 * q) : "memory");
+    };
+    auto issue = [&](int s, int off) {
+        uint8_t* st        = lds + (s % STAGES) * DC_STAGE;
+        const uint8_t* wgt = w_base + (int64_t)s * w_step;
+#pragma unroll
+        for(int h = 0; h < 4; h++)
+            dc_load_to_lds(row_base[h] + off, st + (wave + 4 * h) * 1024);
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+            dc_load_to_lds(wgt + w_off[h], st + DC_A_BYTES + (wave + 4 * h) * 1024);
+    };
+
+    // ---- LDS -> operand fragments: lane l supplies row l % 16 and K bytes 16 (l / 16) .. of a half step
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    uint32_t a_lane[2], b_lane[2];
+#pragma unroll
+    for(int hf = 0; hf < 2; hf++)
+    {
+        const uint32_t f = (uint32_t)(lrow * DC_KSTEP + (((4 * hf + lgrp) ^ ((lrow >> 1) & 7)) << 4));
+        a_lane[hf]       = (uint32_t)(wave * 32 * DC_KSTEP) + f;
+        b_lane[hf]       = (uint32_t)DC_A_BYTES + f;
+    }
+
+    v4i acc[2][4];
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            acc[i][j] = v4i{0, 0, 0, 0};
+    v4i fa[2][2], fb[2][4]; // [register set][tile]: set 0 holds first halves, set 1 second halves
+    int off_next = 0;
+
+    // half HF of K step s_ -> register set HF
+#define DC_READ(s_, HF)                                                                                  \
+    do                                                                                                   \
+    {                                                                                                    \
+        const uint32_t st_ = lds0 + ((s_) % STAGES) * DC_STAGE;                                          \
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fa[HF][0]) : "v"(st_ + a_lane[HF]) : "memory");        \
+        asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(fa[HF][1]) : "v"(st_ + a_lane[HF]) : "memory"); \
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fb[HF][0]) : "v"(st_ + b_lane[HF]) : "memory");        \
+        asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(fb[HF][1]) : "v"(st_ + b_lane[HF]) : "memory"); \
+        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fb[HF][2]) : "v"(st_ + b_lane[HF]) : "memory"); \
+        asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(fb[HF][3]) : "v"(st_ + b_lane[HF]) : "memory"); \
+    } while(0)
+#define DC_WAIT(HF)                                                                                      \
+    asm volatile("s_waitcnt lgkmcnt(0)"                                                                  \
+                 : "+v"(fa[HF][0]), "+v"(fa[HF][1]), "+v"(fb[HF][0]), "+v"(fb[HF][1]), "+v"(fb[HF][2]),  \
+                   "+v"(fb[HF][3]), "+v"(off_next)                                                       \
+                 :                                                                                       \
+                 : "memory")
+    // Inline assembly pins each accumulator to its registers (the builtin lets the compiler rename
+    // them per instruction and shuffle them back at the loop head) and keeps the order reads ->
+    // MFMAs -> wait.  Inside the loop an accumulator is next touched eight MFMAs later; behind the
+    // loop the results are read after the wait states below.
+#define DC_MFMA(HF)                                                                                      \
+    _Pragma("unroll") for(int i = 0; i < 2; i++)                                                         \
+        _Pragma("unroll") for(int j = 0; j < 4; j++)                                                     \
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"                                         \
+                         : "+v"(acc[i][j])                                                               \
+                         : "v"(fa[HF][i]), "v"(fb[HF][j]))
+
+    for(int t = 0; t <= AHEAD && t < nk; t++)
+    {
+        int off;
+        read_offset(t, off);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(off)::"memory");
+        issue(t, off);
+    }
+    read_offset(AHEAD + 1, off_next);
+    dc_wait_steps(min(nk - 1, AHEAD));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    DC_READ(0, 0);
+    DC_WAIT(0);
+    // From a read to the wait that covers it the code is one straight line: across a branch the
+    // compiler may copy a fragment to other registers, and it would do so before the data has
+    // arrived (it cannot see that the read is asynchronous).  The last step therefore reads a
+    // "next" first half too (the stage after it, which nothing is written to any more) and drops it.
+    for(int s = 0; s < nk; s++)
+    {
+        DC_READ(s, 1);
+        DC_MFMA(0);
+        DC_WAIT(1);
+        // every wave has read step s: its stage is free for step s + STAGES, once step s + 1 has landed
+        dc_wait_steps(max(0, min(nk - 1, s + AHEAD) - (s + 1)));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if(s + 1 + AHEAD < nk)
+            issue(s + 1 + AHEAD, off_next);
+        DC_READ(s + 1, 0);
+        read_offset(s + 2 + AHEAD, off_next);
+        DC_MFMA(1);
+        DC_WAIT(0);
+    }
+#undef DC_MFMA
+#undef DC_WAIT
+#undef DC_READ
+    // a 4-pass MFMA's result may be read 7 wait states after it issued at the earliest
+    asm volatile("s_nop 7\n\ts_nop 7"
+                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]),
+                   "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]));
+
+    // ---- result: lane holds rows 4 (l / 16) .. + 3 of its 16-row block for channel l % 16
+    const float sx = (p.dequant && p.scale_x_mode != MI355_QP_NONE) ? p.scale_x[0] : 1.f;
+    auto scale_of = [&](int och) {
+        float sw = 1.f;
+        if(p.scale_w_mode == MI355_QP_PER_TENSOR)
+            sw = p.scale_w[0];
+        else if(p.scale_w_mode == MI355_QP_PER_ROW)
+            sw = p.scale_w[och];
+        return sw * sx;
+    };
+    if constexpr(VEC)
+    {
+        // Through LDS as [channel][128 rows]: a store instruction then writes 512 contiguous bytes
+        // (float) of each of two channels instead of 64-byte pieces of sixteen.
+        __syncthreads(); // every wave has read its last fragments
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+                *reinterpret_cast<v4i*>(lds + (16 * j + lrow) * DC_PITCH + (wave * 32 + 16 * i + 4 * lgrp) * 4) =
+                    acc[i][j];
+        __syncthreads();
+            const int quad  = threadIdx.x & 31;
+        const int64_t r = row0 + 4 * quad;
+        if(r < p.rows)
+        {
+            const int64_t n   = r / p.plane;
+            const int64_t at  = (n * p.o + (int64_t)g * p.og + o0) * p.plane + (r - n * p.plane);
+            const int osub    = threadIdx.x >> 5;
+            // all scales first: a load between two stores would wait for the store in front of it
+            float sc[8];
+#pragma unroll
+            for(int it = 0; it < 8; it++)
+            {
+                sc[it] = 1.f;
+                if constexpr(OUT != MI355_I32)
+                    sc[it] = scale_of(g * p.og + min(o0 + 8 * it + osub, p.og - 1));
+            }
+#pragma unroll
+            for(int it = 0; it < 8; it++)
+            {
+                const int oc = 8 * it + osub;
+                if(o0 + oc < p.og)
+                {
+                    const v4i a = *reinterpret_cast<const v4i*>(lds + oc * DC_PITCH + quad * 16);
+                    dc_store4<OUT>(p.out, at + (int64_t)oc * p.plane, a, sc[it]);
+                }
+            }
+        }
+    }
+    else
+    {
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+        {
+            const int oc = o0 + 16 * j + lrow; // within the group
+            if(oc >= p.og)
+                continue;
+            const int och = g * p.og + oc;
+            float s       = 1.f;
+            if constexpr(OUT != MI355_I32)
+                s = scale_of(och);
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+            {
+                const int64_t r = row0 + wave * 32 + 16 * i + 4 * lgrp;
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                {
+                    const int64_t re = r + e;
+                    if(re >= p.rows)
+                        break;
+                    const int64_t idx = (re / p.plane * p.o + och) * p.plane + re % p.plane;
+                    if constexpr(OUT == MI355_I32)
+                        static_cast<int32_t*>(p.out)[idx] = acc[i][j][e];
+                    else
+                    {
+                        const float v = (float)((double)acc[i][j][e] * (double)s);
+                        if constexpr(OUT == MI355_F32)
+                            static_cast<float*>(p.out)[idx] = v;
+                        else if constexpr(OUT == MI355_F16)
+                            static_cast<uint16_t*>(p.out)[idx] = convert_f32_to_half(v);
+                        else
+                            static_cast<uint16_t*>(p.out)[idx] = convert_f32_to_bf16(v);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// What runs in front of it, as one launch.  Blocks [0, tiles): the channels-last copy, 64 channels
+// x 64 or 256 input positions per block through LDS (loads along the positions, which are
+// contiguous per channel; 16-byte stores of 16 channels per position).  Blocks [tiles, tiles +
+// border_rows): the zero borders, one row (n, z, y) of the padded volume each.  The blocks behind
+// them share the reordered weights ([O][Cg][window] -> [group][K step][channel, padded to 64][128
+// bytes] in (window element, channel) order, zero filled).  All counts fit 32 bits (the launcher
+// checks).
+struct prep_params
+{
+    const uint8_t* x;
+    const uint8_t* w;
+    uint8_t* xt;
+    uint8_t* wp;
+    int n, c, d, h, w_;    // input
+    int dp, hp, wp_;       // padded volume
+    int pad_d, pad_h, pad_w;
+    int group, og, ogp, cg, window, nk;
+    int tiles_s, tiles_c;  // tiles along the positions and the channels of one image
+    int tiles;             // n * tiles_c * tiles_s
+    int border_rows;       // n * dp * hp, or 0 when nothing is padded
+};
+
+// PW: input positions per load, 1 (bytes) or 4 (dwords, when the volume is a multiple of 4
+// positions); a tile is 64 channels x 64 PW positions
+template <int PW>
+__global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
+{
+    constexpr int TILE_S = 64 * PW;
+    __shared__ __align__(16) uint8_t tile[64][TILE_S + 4];
+    const int space = p.d * p.h * p.w_;
+    if((int)blockIdx.x < p.tiles)
+    {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int t    = blockIdx.x;
+        const int ts   = t % p.tiles_s;
+        const int tc   = t / p.tiles_s % p.tiles_c;
+        const int n    = t / (p.tiles_s * p.tiles_c);
+        const int s    = ts * TILE_S + lane * PW;
+        const int c0   = tc * 64;
+        // all 16 loads first, so that they are in flight together
+        uint32_t v[16];
+#pragma unroll
+        for(int i = 0; i < 16; i++)
+        {
+            const int ch = c0 + 16 * wave + i;
+            v[i]         = 0;
+            if(ch < p.c && s < space)
+            {
+                const uint8_t* src = p.x + ((int64_t)n * p.c + ch) * space + s;
+                if constexpr(PW == 4)
+                    v[i] = *reinterpret_cast<const uint32_t*>(src);
+                else
+                    v[i] = *src;
+            }
+        }
+#pragma unroll
+        for(int i = 0; i < 16; i++)
+        {
+            if constexpr(PW == 4)
+                *reinterpret_cast<uint32_t*>(&tile[16 * wave + i][4 * lane]) = v[i];
+            else
+                tile[16 * wave + i][lane] = (uint8_t)v[i];
+        }
+        __syncthreads();
+        // a thread gathers the 16 channels of one piece at one position; the four pieces of 16
+        // neighbouring positions make a wave's store 1 KiB contiguous when C = 64
+        const int piece = threadIdx.x & 3;
+        if(c0 + 16 * piece >= p.c)
+            return;
+#pragma unroll
+        for(int q = 0; q < PW; q++)
+        {
+            const int sl = 64 * q + (threadIdx.x >> 2);
+            const int so = ts * TILE_S + sl;
+            if(so >= space)
+                continue;
+            uint32_t packed[4] = {0, 0, 0, 0};
+            if constexpr(PW == 4)
+            {
+                // byte (sl & 3) of 16 dwords; selector bytes 0x0c give zero
+                const uint32_t b   = sl & 3;
+                const uint32_t sel = 0x0c0c0000u | ((4 + b) << 8) | b;
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                {
+                    const uint32_t r0 = *reinterpret_cast<const uint32_t*>(&tile[16 * piece + 4 * j + 0][sl & ~3]);
+                    const uint32_t r1 = *reinterpret_cast<const uint32_t*>(&tile[16 * piece + 4 * j + 1][sl & ~3]);
+                    const uint32_t r2 = *reinterpret_cast<const uint32_t*>(&tile[16 * piece + 4 * j + 2][sl & ~3]);
+                    const uint32_t r3 = *reinterpret_cast<const uint32_t*>(&tile[16 * piece + 4 * j + 3][sl & ~3]);
+                    const uint32_t lo = __builtin_amdgcn_perm(r1, r0, sel);
+                    const uint32_t hi = __builtin_amdgcn_perm(r3, r2, sel);
+                    packed[j]         = lo | (hi << 16);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for(int e = 0; e < 16; e++)
+                    packed[e / 4] |= (uint32_t)tile[16 * piece + e][sl] << (8 * (e % 4));
+            }
+            const int ix = so % p.w_;
+            const int iy = so / p.w_ % p.h;
+            const int iz = so / (p.w_ * p.h);
+            const int64_t at =
+                ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * p.c + c0 +
+                16 * piece;
+            *reinterpret_cast<uint4*>(p.xt + at) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        }
+        return;
+    }
+    const int cp = p.c / 16;
+    if((int)blockIdx.x < p.tiles + p.border_rows)
+    {
+        const int row = blockIdx.x - p.tiles;
+        const int y   = row % p.hp - p.pad_h;
+        const int z   = row / p.hp % p.dp - p.pad_d;
+        uint8_t* dst  = p.xt + (int64_t)row * p.wp_ * p.c;
+        const bool whole = y < 0 || y >= p.h || z < 0 || z >= p.d;
+        for(int t = threadIdx.x; t < p.wp_ * cp; t += 256)
+        {
+            const int x = t / cp - p.pad_w;
+            if(whole || x < 0 || x >= p.w_)
+                *reinterpret_cast<uint4*>(dst + (int64_t)t * 16) = make_uint4(0, 0, 0, 0);
+        }
+        return;
+    }
+    // weights: a thread fills 16 bytes of K for one channel
+    const int first    = p.tiles + p.border_rows;
+    const int nthreads = ((int)gridDim.x - first) * 256;
+    const int total    = p.group * p.nk * p.ogp * (DC_KSTEP / 16);
+    const int kg       = p.cg * p.window;
+    for(int t = ((int)blockIdx.x - first) * 256 + threadIdx.x; t < total; t += nthreads)
+    {
+        const int k0 = t % (DC_KSTEP / 16) * 16;
+        const int oc = t / (DC_KSTEP / 16) % p.ogp;
+        const int s  = t / (DC_KSTEP / 16) / p.ogp % p.nk;
+        const int g  = t / (DC_KSTEP / 16) / p.ogp / p.nk;
+        uint32_t packed[4] = {0, 0, 0, 0};
+        const int k  = s * DC_KSTEP + k0;
+        if(oc < p.og && k < kg)
+        {
+            // 16 | cg: the 16 bytes are 16 consecutive channels of one window element
+            const int tap      = k / p.cg;
+            const uint8_t* src = p.w + (((int64_t)g * p.og + oc) * p.cg + k % p.cg) * p.window + tap;
+#pragma unroll
+            for(int e = 0; e < 16; e++)
+                packed[e / 4] |= (uint32_t)src[(int64_t)e * p.window] << (8 * (e % 4));
+        }
+        *reinterpret_cast<uint4*>(p.wp + (int64_t)t * 16) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    }
+}
+
 int64_t out_len(int64_t in, int64_t k, int64_t pad_lo, int64_t pad_hi, int64_t stride, int64_t dil)
 {
     const int64_t span = in - (1 + dil * (k - 1)) + pad_lo + pad_hi;
@@ -239,6 +757,88 @@ size_t staging_bytes(const mi355_quant_conv3d_desc* d, int64_t plane, int64_t kp
     return (b + 15) / 16 * 16;
 }
 
+// K steps and padded channel count of the direct kernel's weights
+int64_t direct_steps(const mi355_quant_conv3d_desc* d)
+{
+    return (d->c / d->group * d->kd * d->kh * d->kw + DC_KSTEP - 1) / DC_KSTEP;
+}
+int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
+{
+    return (d->o / d->group + DC_COLS - 1) / DC_COLS * DC_COLS;
+}
+
+// The direct kernel's form of a layer: int8, every group a multiple of 16 channels, a real
+// window, every window inside the padded volume, counts that fit the kernels' 32-bit indices.
+bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
+{
+    const int64_t lim    = (int64_t)1 << 31;
+    const int64_t cg     = d->c / d->group;
+    const int64_t window = d->kd * d->kh * d->kw;
+    if(d->in_type != MI355_I8 || cg % 16 != 0 || window <= 1)
+        return false;
+    const int64_t in[3]  = {d->d, d->h, d->w};
+    const int64_t win[3] = {d->kd, d->kh, d->kw};
+    int64_t volume       = d->c;
+    for(int i = 0; i < 3; i++)
+    {
+        const int64_t padded = in[i] + d->pad[i] + d->pad_hi[i];
+        if((ol[i] - 1) * d->stride[i] + d->dil[i] * (win[i] - 1) + 1 > padded)
+            return false;
+        volume *= padded;
+        if(volume >= lim)
+            return false;
+    }
+    if(d->n * (volume / d->c) >= lim || d->n * d->c >= lim) // padded positions; channel planes
+        return false;
+    const int64_t nk = direct_steps(d);
+    if(nk * 8 > DC_MAX_PIECES)
+        return false;
+    return direct_ogp(d) / DC_COLS * d->group <= 65535 && d->group * nk * direct_ogp(d) * (DC_KSTEP / 16) < lim;
+}
+
+// reordered weights + padded channels-last copy
+size_t direct_bytes(const mi355_quant_conv3d_desc* d)
+{
+    return (size_t)(d->group * direct_steps(d) * direct_ogp(d) * DC_KSTEP +
+                    d->n * d->c * (d->d + d->pad[0] + d->pad_hi[0]) * (d->h + d->pad[1] + d->pad_hi[1]) *
+                        (d->w + d->pad[2] + d->pad_hi[2]));
+}
+
+template <int OUT, bool VEC, int STAGES>
+void launch_direct_as(const direct_params& p, dim3 grid, hipStream_t hs)
+{
+    // ring + offset table; may be above the 64 KiB default: opt in once per instantiation
+    auto kern = conv_direct_i8_kernel<OUT, VEC, STAGES>;
+    static const hipError_t attr =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            STAGES * DC_STAGE + DC_MAX_PIECES * 4);
+    (void)attr;
+    hipLaunchKernelGGL(kern, grid, dim3(256), STAGES * DC_STAGE + p.nk * 8 * 4, hs, p);
+}
+
+// The ring is as deep as the workgroups a CU gets at a time allow (160 KiB of LDS per CU): one
+// workgroup has to hide its load latency itself, three hide each other's.
+template <int OUT, bool VEC>
+void launch_direct_vec(const direct_params& p, dim3 grid, hipStream_t hs)
+{
+    const int64_t per_cu = ((int64_t)grid.x * grid.y + 255) / 256;
+    if(per_cu <= 1)
+        launch_direct_as<OUT, VEC, 6>(p, grid, hs);
+    else if(per_cu == 2)
+        launch_direct_as<OUT, VEC, 3>(p, grid, hs);
+    else
+        launch_direct_as<OUT, VEC, 2>(p, grid, hs);
+}
+
+template <int OUT>
+void launch_direct(const direct_params& p, bool vec, dim3 grid, hipStream_t hs)
+{
+    if(vec)
+        launch_direct_vec<OUT, true>(p, grid, hs);
+    else
+        launch_direct_vec<OUT, false>(p, grid, hs);
+}
+
 // a depth of one in front of the two-dimensional description
 mi355_quant_conv3d_desc with_unit_depth(const mi355_quant_conv_desc* d)
 {
@@ -284,6 +884,8 @@ extern "C" int mi355_quant_convolution3d_dims(const mi355_quant_conv3d_desc* d,
         const int64_t plane          = o[0] * o[1] * o[2];
         const mi355_quant_dot_desc g = gemm_of(d, plane, kp);
         *workspace_bytes             = staging_bytes(d, plane, kp) + mi355_quant_dot_workspace_size(&g);
+        if(direct_form(d, o) && *workspace_bytes < direct_bytes(d))
+            *workspace_bytes = direct_bytes(d);
     }
     return MI355_OK;
 }
@@ -346,6 +948,75 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
     const int64_t plane = ol[0] * ol[1] * ol[2];
     uint8_t* col        = static_cast<uint8_t*>(workspace);
     uint8_t* wp         = col + d->n * d->group * plane * kp;
+
+    if(direct_form(d, ol) && reinterpret_cast<uintptr_t>(x) % 16 == 0)
+    {
+        uint8_t* ws = static_cast<uint8_t*>(workspace);
+        const int64_t nk  = direct_steps(d);
+        const int64_t ogp = direct_ogp(d);
+        prep_params q{};
+        q.x = static_cast<const uint8_t*>(x);
+        q.w = static_cast<const uint8_t*>(w);
+        q.wp = ws;
+        q.xt = ws + d->group * nk * ogp * DC_KSTEP;
+        q.n = (int)d->n;
+        q.c = (int)d->c, q.d = (int)d->d, q.h = (int)d->h, q.w_ = (int)d->w;
+        q.pad_d = (int)d->pad[0], q.pad_h = (int)d->pad[1], q.pad_w = (int)d->pad[2];
+        q.dp = (int)(d->d + d->pad[0] + d->pad_hi[0]);
+        q.hp = (int)(d->h + d->pad[1] + d->pad_hi[1]);
+        q.wp_ = (int)(d->w + d->pad[2] + d->pad_hi[2]);
+        q.group = (int)d->group, q.og = (int)og, q.ogp = (int)ogp;
+        q.cg = (int)cg, q.window = (int)window, q.nk = (int)nk;
+        const int64_t space = d->d * d->h * d->w;
+        const bool dwords   = space % 4 == 0;
+        q.tiles_s = (int)((space + (dwords ? 255 : 63)) / (dwords ? 256 : 64));
+        q.tiles_c = (int)((d->c + 63) / 64);
+        const int64_t tiles = d->n * q.tiles_c * q.tiles_s;
+        const bool padded   = q.dp != q.d || q.hp != q.h || q.wp_ != q.w_;
+        const int64_t border_rows = padded ? d->n * q.dp * q.hp : 0;
+        // blocks behind them: the weights, one piece of 16 bytes per thread up to 1024 blocks
+        int64_t extra = d->group * nk * ogp * (DC_KSTEP / 16) / 256 + 1;
+        extra         = extra > 1024 ? 1024 : extra;
+        if(tiles + border_rows + extra >= ((int64_t)1 << 31))
+            return MI355_ERR_UNSUPPORTED;
+        q.tiles       = (int)tiles;
+        q.border_rows = (int)border_rows;
+        const dim3 prep_grid((unsigned)(tiles + border_rows + extra));
+        if(dwords)
+            hipLaunchKernelGGL(conv_prep_kernel<4>, prep_grid, dim3(256), 0, hs, q);
+        else
+            hipLaunchKernelGGL(conv_prep_kernel<1>, prep_grid, dim3(256), 0, hs, q);
+        if(mi355_launch_status() != MI355_OK)
+            return MI355_ERR_LAUNCH;
+
+        direct_params p{};
+        p.xt = q.xt, p.wp = q.wp, p.out = out;
+        p.scale_x = scale_x, p.scale_w = scale_w;
+        p.rows = d->n * plane;
+        p.plane = (int)plane, p.oh = (int)ol[1], p.ow = (int)ol[2];
+        p.o = (int)d->o, p.og = (int)og, p.ogp = (int)ogp, p.c = (int)d->c, p.cg = (int)cg;
+        p.kh = (int)d->kh, p.kw = (int)d->kw;
+        p.dp = q.dp, p.hp = q.hp, p.wp_ = q.wp_;
+        p.stride_d = (int)d->stride[0], p.stride_h = (int)d->stride[1], p.stride_w = (int)d->stride[2];
+        p.dil_d = (int)d->dil[0], p.dil_h = (int)d->dil[1], p.dil_w = (int)d->dil[2];
+        p.kg = (int)kg, p.nk = (int)nk;
+        p.col_tiles = (int)(ogp / DC_COLS);
+        p.dequant = d->dequant, p.scale_x_mode = d->scale_x_mode, p.scale_w_mode = d->scale_w_mode;
+        const int64_t row_tiles = (p.rows + DC_ROWS - 1) / DC_ROWS;
+        if(row_tiles >= ((int64_t)1 << 31))
+            return MI355_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)row_tiles, (unsigned)(p.col_tiles * d->group));
+        const bool vec = plane % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+        if(!d->dequant)
+            launch_direct<MI355_I32>(p, vec, grid, hs);
+        else if(d->out_type == MI355_F32)
+            launch_direct<MI355_F32>(p, vec, grid, hs);
+        else if(d->out_type == MI355_F16)
+            launch_direct<MI355_F16>(p, vec, grid, hs);
+        else
+            launch_direct<MI355_BF16>(p, vec, grid, hs);
+        return mi355_launch_status();
+    }
 
     uint8_t* xt         = wp + d->o * kp; // channels-last copy of the input, when that form is used
     // every group a multiple of 16 channels and a real window: gather through a channels-last copy

@@ -1,12 +1,12 @@
 """Scan of gfx950 assembly for the one hazard the compiler cannot see in this library's kernels.
 
-The four-wave GEMM kernels issue their MFMAs from inline assembly (so that the accumulators stay in
-the accumulation registers).  To the compiler such a statement is opaque: it does not know that the
+The four-wave GEMM kernels and the direct convolution kernel issue their MFMAs from inline assembly
+(so that every accumulator stays in its registers).  To the compiler such a statement is opaque: it does not know that the
 result arrives some passes later, and inserts none of the wait states that an ordinary instruction
 reading (or overwriting) the result registers needs behind an MFMA -- the kernels carry them
 themselves.  This scan checks that they do: for every MFMA inside an inline-assembly region it
 follows the instruction stream and reports any non-MFMA instruction that names one of the MFMA's
-destination accumulation registers before enough wait states have gone by (every instruction
+destination registers before enough wait states have gone by (every instruction
 counts one, ``s_nop N`` counts N + 1).  The stream is read in layout order, branches are not
 followed: a block laid out behind an MFMA but reached another way can give a false alarm, never a
 miss on the fall-through path.
@@ -17,17 +17,20 @@ of v_mfma[_scale]_f32_32x32x64_f8f6f4.
 """
 import re
 
-_RANGE = re.compile(r"^a\[(\d+):(\d+)\]$")
-_ONE = re.compile(r"^a(\d+)$")
+_RANGE = re.compile(r"^([av])\[(\d+):(\d+)\]$")
+_ONE = re.compile(r"^([av])(\d+)$")
+_LABEL = re.compile(r"^([A-Za-z_][\w$]*):")
 
 
 def _acc_regs(token):
+    """The registers a token names, as (file, index) pairs: accumulation registers and ordinary vector
+    registers both (the direct convolution kernel accumulates in the latter)."""
     m = _RANGE.match(token)
     if m:
-        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
     m = _ONE.match(token)
     if m:
-        return {int(m.group(1))}
+        return {(m.group(1), int(m.group(2)))}
     return set()
 
 
@@ -55,8 +58,9 @@ def scan(path, only=None):
             if text.startswith(";;#ASMEND"):
                 in_asm = False
                 continue
-            if text.endswith(":") and not text.startswith("."):
-                kernel, pending = text[:-1], []
+            label = _LABEL.match(text)   # a function's label (block labels start with a dot)
+            if label:
+                kernel, pending = label.group(1), []
                 continue
             if not text or text[0] in ".;":
                 continue
@@ -78,7 +82,8 @@ def scan(path, only=None):
                 touched |= _acc_regs(token)
             for regs, left, at in pending:
                 if touched & regs:
-                    hazards.append(f"{kernel}: line {number} `{text}` touches a{min(touched & regs)}.. "
+                    first = min(touched & regs)
+                    hazards.append(f"{kernel}: line {number} `{text}` touches {first[0]}{first[1]}.. "
                                    f"{left} wait states early (MFMA at line {at})")
             pending = [(r, w - states, n) for (r, w, n) in pending if w - states > 0]
     return seen, hazards

@@ -1,4 +1,4 @@
-"""GPU parity of quant_convolution (im2col + the quantized GEMM, one to three spatial axes) through
+"""GPU parity of quant_convolution (the direct kernel, or im2col + the quantized GEMM; one to three spatial axes) through
 the C ABI against the CPU oracle: int32 results bit-exact, dequantized results bit-exact for int8, fp8 within the
 accumulation tolerance of the fp8 matrix instructions."""
 import numpy as np
@@ -46,6 +46,16 @@ CASES = [
     ((1, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((1, 128, 12, 12), (96, 64, 5, 5), (2, 2), (1, 1), (1, 1), 2),
     ((1, 512, 7, 7), (64, 512, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # 49 positions: N % 4 != 0 in the split
+    # the direct kernel (int8, 16 | channels per group): channel tiles with a ragged end, row tiles that
+    # straddle images, K steps with a zero-filled second half, windows over the zero border only
+    ((3, 32, 10, 13), (80, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # 80 channels: tiles of 64 + 16; 130 positions
+    ((2, 96, 8, 8), (144, 48, 3, 3), (2, 2), (1, 1), (2, 2), 2),       # 72 channels per group, dilation, K = 432 -> 512
+    ((5, 16, 6, 6), (16, 16, 2, 2), (3, 3), (2, 2), (1, 1), 1),        # padding wider than the window
+    ((4, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # the benchmark's first layer shape, 4 images
+    ((4, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1), (1, 1), 1),   # and its second
+    ((2, 128, 28, 28), (128, 128, 3, 3), (1, 1), (2, 2), (1, 1), 1),   # stride 2
+    # not the direct kernel's form (200 channels): one image of a deep layer through im2col and the GEMM's split K
+    ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
 
 
@@ -85,6 +95,30 @@ def test_int8_dequant_epilogue_bit_exact(ops, out, per_channel):
     else:
         ot = orc.F16 if out == "f16" else orc.BF16
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
+
+
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_direct_kernel_dequant_without_vector_stores(ops, out):
+    """49 positions per image: a lane's four results are not one aligned vector of the NCHW result, so the direct
+    kernel stores them one by one; two groups of 24 channels (a ragged channel tile), three images in one row tile."""
+    rng = np.random.default_rng(16)
+    xs, ws = (3, 64, 7, 7), (48, 32, 3, 3)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.0371)
+    sw = rng.uniform(0.001, 0.01, 48).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (1, 1), (1, 1), (1, 1), 2)
+    scale = np.broadcast_to((sx * sw).astype(np.float32).reshape(1, -1, 1, 1), acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 2, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
+    bare = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 2)
+    assert np.array_equal(bare.cpu().numpy(), acc)
 
 
 @pytest.mark.parametrize("out", ["f32", "bf16"])

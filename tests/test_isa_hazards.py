@@ -1,6 +1,6 @@
 """The generated code of the kernels whose MFMAs are inline assembly keeps the wait states between
 an MFMA and the first ordinary access to its result (see tests/isa_lint.py).  Compiles
-csrc/qgemm_dma.hip to assembly (about a minute and a half), no GPU needed."""
+csrc/qgemm_dma.hip (about a minute and a half) and csrc/conv.hip to assembly, no GPU needed."""
 import os
 import shutil
 import subprocess
@@ -39,14 +39,26 @@ _Z6samplev:
     assert len(hazards) == 1 and "a1" in hazards[0]
 
 
-@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
-def test_four_wave_kernels_keep_their_wait_states(tmp_path):
-    out = tmp_path / "qgemm_dma.s"
+def _listing(tmp_path, source):
+    out = tmp_path / (source + ".s")
     cmd = [HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"),
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only",
-           "-o", str(out), os.path.join(ROOT, "amdmigraphx_amd", "csrc", "qgemm_dma.hip")]
+           "-o", str(out), os.path.join(ROOT, "amdmigraphx_amd", "csrc", source)]
     subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=900)
-    seen, hazards = isa_lint.scan(str(out))
+    return str(out)
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_direct_convolution_kernel_keeps_its_wait_states(tmp_path):
+    seen, hazards = isa_lint.scan(_listing(tmp_path, "conv.hip"), only="conv_direct")
+    # 16 MFMAs per K step body, 24 instantiations (4 result types, vector stores or not, 3 ring depths)
+    assert seen >= 16 * 24
+    assert hazards == [], hazards[:5]
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_four_wave_kernels_keep_their_wait_states(tmp_path):
+    seen, hazards = isa_lint.scan(_listing(tmp_path, "qgemm_dma.hip"))
     # 64 (int8) or 16 (fp8) MFMAs per slab body, several bodies per kernel, 28 kernels
     assert seen > 5000
     assert hazards == [], hazards[:5]
