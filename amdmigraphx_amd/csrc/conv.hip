@@ -793,7 +793,13 @@ bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
     const int64_t nk = direct_steps(d);
     if(nk * 8 > DC_MAX_PIECES)
         return false;
-    return direct_ogp(d) / DC_COLS * d->group <= 65535 && d->group * nk * direct_ogp(d) * (DC_KSTEP / 16) < lim;
+    if(direct_ogp(d) / DC_COLS * d->group > 65535 || d->group * nk * direct_ogp(d) * (DC_KSTEP / 16) >= lim)
+        return false;
+    // a handful of workgroups with a long K each (one image of a deep 7x7 layer: 8 workgroups x 36
+    // steps) is what the GEMM's split of K over the chip is for
+    const int64_t plane      = ol[0] * ol[1] * ol[2];
+    const int64_t workgroups = (d->n * plane + DC_ROWS - 1) / DC_ROWS * (direct_ogp(d) / DC_COLS) * d->group;
+    return !(workgroups < 32 && nk >= 24);
 }
 
 // reordered weights + padded channels-last copy
