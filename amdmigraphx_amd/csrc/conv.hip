@@ -210,6 +210,13 @@ MI355_DEVINL void dc_load_to_lds(const uint8_t* g, uint8_t* l)
                                      (__attribute__((address_space(3))) void*)(l), 16, 0, 0);
 }
 
+// 8 of a fragment's 16 bytes
+MI355_DEVINL long dc_half(v4i f, int hi)
+{
+    const v2i h = hi ? v2i{f[2], f[3]} : v2i{f[0], f[1]};
+    return __builtin_bit_cast(long, h);
+}
+
 template <int N>
 MI355_DEVINL void dc_wait_vmcnt()
 {
@@ -229,7 +236,19 @@ MI355_DEVINL void dc_wait_steps(int steps)
     }
 }
 
-template <int OUT>
+// one dequantized value as the GEMM's epilogue forms it: int8 through a double product, fp8 (the
+// accumulator's bits are a float) as a float product
+template <bool FP8>
+MI355_DEVINL float dc_scaled(int32_t a, float s)
+{
+    if constexpr(FP8)
+        return __builtin_bit_cast(float, a) * s;
+    else
+        return (float)((double)a * (double)s);
+}
+
+// OUT == MI355_I32 stands for the bare accumulators (int32, or the float sums of fp8 operands)
+template <bool FP8, int OUT>
 MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
 {
     if constexpr(OUT == MI355_I32)
@@ -239,7 +258,7 @@ MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
         float v[4];
 #pragma unroll
         for(int e = 0; e < 4; e++)
-            v[e] = (float)((double)a[e] * (double)s);
+            v[e] = dc_scaled<FP8>(a[e], s);
         if constexpr(OUT == MI355_F32)
             *reinterpret_cast<v4f*>(static_cast<float*>(out) + idx) = v4f{v[0], v[1], v[2], v[3]};
         else if constexpr(OUT == MI355_F16)
@@ -252,11 +271,13 @@ MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
     }
 }
 
-// OUT: MI355_I32 (bare sums), MI355_F32 / F16 / BF16 (dequantized); VEC: the plane is a multiple of
-// 4 positions, so a lane's four rows are one image's and their store is one aligned vector.
-// STAGES: LDS ring; the loads of K step s + STAGES go out when step s has been read.
-template <int OUT, bool VEC, int STAGES>
-__global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
+// FP8: e4m3fn operands on v_mfma_f32_16x16x32_fp8_fp8 (two per 64 K bytes; the lanes' K bytes are
+// assigned as for int8, the same for both operands, so the sum runs over the same products in another
+// order).  OUT: MI355_I32 (bare sums), MI355_F32 / F16 / BF16 (dequantized); VEC: the plane is a
+// multiple of 4 positions, so a lane's four rows are one image's and their store is one aligned
+// vector.  STAGES: LDS ring; the loads of K step s + STAGES go out when step s has been read.
+template <bool FP8, int OUT, bool VEC, int STAGES>
+__global__ __launch_bounds__(256) void conv_direct_kernel(direct_params p)
 {
     static_assert(STAGES * DC_STAGE >= DC_COLS * DC_PITCH, "the result copy reuses the ring");
     static_assert(STAGES >= 2 && STAGES <= 6);
@@ -274,6 +295,9 @@ __global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
     // byte offset of every K piece from a row's base: (window element, first channel)
     for(int q = threadIdx.x; q < pieces; q += 256)
     {
+        // past the window (the zero-filled tail of the last K step): the row's first piece again,
+        // times zero weights.  (An fp8 NaN there is in the true sum as well: it is the row's first
+        // window element.)
         int off = 0;
         if(q * 16 < p.kg)
         {
@@ -380,12 +404,24 @@ __global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
     // them per instruction and shuffle them back at the loop head) and keeps the order reads ->
     // MFMAs -> wait.  Inside the loop an accumulator is next touched eight MFMAs later; behind the
     // loop the results are read after the wait states below.
+    // fp8 goes through the builtin (its operands are halves of a fragment; every fragment is tied
+    // into the wait in front, so the compiler takes them behind it).
 #define DC_MFMA(HF)                                                                                      \
     _Pragma("unroll") for(int i = 0; i < 2; i++)                                                         \
         _Pragma("unroll") for(int j = 0; j < 4; j++)                                                     \
-            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"                                         \
-                         : "+v"(acc[i][j])                                                               \
-                         : "v"(fa[HF][i]), "v"(fb[HF][j]))
+        {                                                                                                \
+            if constexpr(FP8)                                                                            \
+            {                                                                                            \
+                v4f c_ = __builtin_bit_cast(v4f, acc[i][j]);                                             \
+                c_ = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(dc_half(fa[HF][i], 0), dc_half(fb[HF][j], 0), c_, 0, 0, 0); \
+                c_ = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(dc_half(fa[HF][i], 1), dc_half(fb[HF][j], 1), c_, 0, 0, 0); \
+                acc[i][j] = __builtin_bit_cast(v4i, c_);                                                 \
+            }                                                                                            \
+            else                                                                                         \
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"                                     \
+                             : "+v"(acc[i][j])                                                           \
+                             : "v"(fa[HF][i]), "v"(fb[HF][j]));                                          \
+        }
 
     for(int t = 0; t <= AHEAD && t < nk; t++)
     {
@@ -475,7 +511,7 @@ __global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
                 if(o0 + oc < p.og)
                 {
                     const v4i a = *reinterpret_cast<const v4i*>(lds + oc * DC_PITCH + quad * 16);
-                    dc_store4<OUT>(p.out, at + (int64_t)oc * p.plane, a, sc[it]);
+                    dc_store4<FP8, OUT>(p.out, at + (int64_t)oc * p.plane, a, sc[it]);
                 }
             }
         }
@@ -507,7 +543,7 @@ __global__ __launch_bounds__(256) void conv_direct_i8_kernel(direct_params p)
                         static_cast<int32_t*>(p.out)[idx] = acc[i][j][e];
                     else
                     {
-                        const float v = (float)((double)acc[i][j][e] * (double)s);
+                        const float v = dc_scaled<FP8>(acc[i][j][e], s);
                         if constexpr(OUT == MI355_F32)
                             static_cast<float*>(p.out)[idx] = v;
                         else if constexpr(OUT == MI355_F16)
@@ -767,14 +803,14 @@ int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
     return (d->o / d->group + DC_COLS - 1) / DC_COLS * DC_COLS;
 }
 
-// The direct kernel's form of a layer: int8, every group a multiple of 16 channels, a real
+// The direct kernel's form of a layer: every group a multiple of 16 channels, a real
 // window, every window inside the padded volume, counts that fit the kernels' 32-bit indices.
 bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
 {
     const int64_t lim    = (int64_t)1 << 31;
     const int64_t cg     = d->c / d->group;
     const int64_t window = d->kd * d->kh * d->kw;
-    if(d->in_type != MI355_I8 || cg % 16 != 0 || window <= 1)
+    if(cg % 16 != 0 || window <= 1)
         return false;
     const int64_t in[3]  = {d->d, d->h, d->w};
     const int64_t win[3] = {d->kd, d->kh, d->kw};
@@ -810,11 +846,11 @@ size_t direct_bytes(const mi355_quant_conv3d_desc* d)
                         (d->w + d->pad[2] + d->pad_hi[2]));
 }
 
-template <int OUT, bool VEC, int STAGES>
+template <bool FP8, int OUT, bool VEC, int STAGES>
 void launch_direct_as(const direct_params& p, dim3 grid, hipStream_t hs)
 {
     // ring + offset table; may be above the 64 KiB default: opt in once per instantiation
-    auto kern = conv_direct_i8_kernel<OUT, VEC, STAGES>;
+    auto kern = conv_direct_kernel<FP8, OUT, VEC, STAGES>;
     static const hipError_t attr =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             STAGES * DC_STAGE + DC_MAX_PIECES * 4);
@@ -824,25 +860,29 @@ void launch_direct_as(const direct_params& p, dim3 grid, hipStream_t hs)
 
 // The ring is as deep as the workgroups a CU gets at a time allow (160 KiB of LDS per CU): one
 // workgroup has to hide its load latency itself, three hide each other's.
-template <int OUT, bool VEC>
+template <bool FP8, int OUT, bool VEC>
 void launch_direct_vec(const direct_params& p, dim3 grid, hipStream_t hs)
 {
     const int64_t per_cu = ((int64_t)grid.x * grid.y + 255) / 256;
     if(per_cu <= 1)
-        launch_direct_as<OUT, VEC, 6>(p, grid, hs);
+        launch_direct_as<FP8, OUT, VEC, 6>(p, grid, hs);
     else if(per_cu == 2)
-        launch_direct_as<OUT, VEC, 3>(p, grid, hs);
+        launch_direct_as<FP8, OUT, VEC, 3>(p, grid, hs);
     else
-        launch_direct_as<OUT, VEC, 2>(p, grid, hs);
+        launch_direct_as<FP8, OUT, VEC, 2>(p, grid, hs);
 }
 
-template <int OUT>
-void launch_direct(const direct_params& p, bool vec, dim3 grid, hipStream_t hs)
+template <bool FP8>
+void launch_direct(const direct_params& p, bool dequant, int out_type, bool vec, dim3 grid, hipStream_t hs)
 {
-    if(vec)
-        launch_direct_vec<OUT, true>(p, grid, hs);
+    if(!dequant)
+        vec ? launch_direct_vec<FP8, MI355_I32, true>(p, grid, hs) : launch_direct_vec<FP8, MI355_I32, false>(p, grid, hs);
+    else if(out_type == MI355_F32)
+        vec ? launch_direct_vec<FP8, MI355_F32, true>(p, grid, hs) : launch_direct_vec<FP8, MI355_F32, false>(p, grid, hs);
+    else if(out_type == MI355_F16)
+        vec ? launch_direct_vec<FP8, MI355_F16, true>(p, grid, hs) : launch_direct_vec<FP8, MI355_F16, false>(p, grid, hs);
     else
-        launch_direct_vec<OUT, false>(p, grid, hs);
+        vec ? launch_direct_vec<FP8, MI355_BF16, true>(p, grid, hs) : launch_direct_vec<FP8, MI355_BF16, false>(p, grid, hs);
 }
 
 // a depth of one in front of the two-dimensional description
@@ -1013,14 +1053,10 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
             return MI355_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)row_tiles, (unsigned)(p.col_tiles * d->group));
         const bool vec = plane % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
-        if(!d->dequant)
-            launch_direct<MI355_I32>(p, vec, grid, hs);
-        else if(d->out_type == MI355_F32)
-            launch_direct<MI355_F32>(p, vec, grid, hs);
-        else if(d->out_type == MI355_F16)
-            launch_direct<MI355_F16>(p, vec, grid, hs);
+        if(fp8)
+            launch_direct<true>(p, d->dequant != 0, d->out_type, vec, grid, hs);
         else
-            launch_direct<MI355_BF16>(p, vec, grid, hs);
+            launch_direct<false>(p, d->dequant != 0, d->out_type, vec, grid, hs);
         return mi355_launch_status();
     }
 

@@ -225,6 +225,37 @@ def test_fp8_convolution(ops):
     assert np.array_equal(got.cpu().numpy(), orc.convolution(xi, wi, orc.F32, (1, 1)))
 
 
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_fp8_direct_kernel_shapes_and_dequant_epilogue(ops, out):
+    """fp8 through the direct kernel (16 | channels per group): two groups, a ragged channel tile, a K step whose
+    second half is padding, row tiles over three images; scales applied as float(sum) * (scale_x * scale_w[o]),
+    the fp8 GEMM's epilogue (quant_dot -> dequantizelinear, simplify_qdq.cpp:171-222)."""
+    rng = np.random.default_rng(18)
+    xs, ws = (3, 96, 9, 12), (80, 48, 3, 3)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.05).astype(np.float32)
+    sx = np.float32(np.abs(x).max() / 448)
+    swt = np.float32(np.abs(w).max() / 448)
+    xq = orc.quantizelinear(x.reshape(-1, xs[-1]), sx, None, orc.F32, orc.FP8).reshape(xs)
+    wq = orc.quantizelinear(w.reshape(-1, ws[-1]), swt, None, orc.F32, orc.FP8).reshape(ws)
+    acc = orc.convolution(xq, wq, orc.FP8, (1, 1), (1, 1), (1, 1), 2)
+    mag = orc.convolution(np.abs(orc.fp8_to_f32(xq)).astype(np.float32),
+                          np.abs(orc.fp8_to_f32(wq)).astype(np.float32), orc.F32, (1, 1), (1, 1), (1, 1), 2)
+    bare = ops.quant_convolution(dev(xq), dev(wq), (1, 1), (1, 1), (1, 1), 2, fp8=True).cpu().numpy()
+    assert np.all(np.abs(bare - acc) <= np.maximum(1e-3 * np.abs(acc), 2.0 ** -14 * mag))
+    sw = (swt * rng.uniform(0.5, 2.0, 80)).astype(np.float32)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_convolution(dev(xq), dev(wq), (1, 1), (1, 1), (1, 1), 2, fp8=True, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    # the kernel's own sums, scaled and converted as the reference does, are the result bit for bit
+    scale = (sw * sx).astype(np.float32).reshape(1, -1, 1, 1)
+    want = (bare * scale).astype(np.float32)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
+
+
 def test_argument_errors(ops):
     x = dev(np.zeros((1, 4, 5, 5), np.int8))
     with pytest.raises(Exception):
