@@ -567,6 +567,93 @@ bool lower_w4a16(module& m, instruction_ref ins)
     return true;
 }
 
+// ---- weight-only GEMMs that share their activations -> one launch -------------------------------
+//
+// The q / k / v projections of an attention layer and the gate / up projections of its MLP multiply
+// the same activations by different constant weights.  At one row of activations such a product
+// is a few microseconds of weight streaming behind a launch and a fetch of the activations that
+// cost as much; with the weights (and their scales) stacked along N at compile time the products
+// become one launch, and each original result is a `slice` of its columns.  A column's sum does
+// not depend on which other columns are computed with it, so the results keep their bits.
+// Taken: scalar zero points, weights and scales known at compile time, the same activations,
+// K, group size and zero point.
+void fuse_shared_w4a16(module& m)
+{
+    std::vector<instruction_ref> gemms;
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() == "mi355::w4a16_gemm")
+            gemms.push_back(ins);
+    }
+    auto constant = [](instruction_ref x) { return x->can_eval() and x->get_shape().standard(); };
+    std::unordered_set<const instruction*> taken;
+    for(std::size_t i = 0; i < gemms.size(); i++)
+    {
+        auto first = gemms[i];
+        if(taken.count(&*first) > 0)
+            continue;
+        const auto op = any_cast<w4a16_gemm>(first->get_operator());
+        if(op.zp_mode != MI355_W4_ZP_SCALAR or not constant(first->inputs()[1]) or not constant(first->inputs()[2]))
+            continue;
+        const auto k2 = first->inputs()[1]->get_shape().lens()[1];
+        const auto kb = first->inputs()[2]->get_shape().lens()[1];
+        std::vector<instruction_ref> members = {first};
+        for(std::size_t j = i + 1; j < gemms.size(); j++)
+        {
+            auto other = gemms[j];
+            if(taken.count(&*other) > 0 or other->inputs()[0] != first->inputs()[0])
+                continue;
+            const auto oop = any_cast<w4a16_gemm>(other->get_operator());
+            if(oop.zp_mode != MI355_W4_ZP_SCALAR or oop.zp_scalar != op.zp_scalar or oop.group != op.group or
+               not constant(other->inputs()[1]) or not constant(other->inputs()[2]) or
+               other->inputs()[1]->get_shape().lens()[1] != k2 or other->inputs()[2]->get_shape().lens()[1] != kb or
+               other->inputs()[2]->get_shape().type() != first->inputs()[2]->get_shape().type())
+                continue;
+            members.push_back(other);
+        }
+        if(members.size() < 2)
+            continue;
+        std::size_t n = 0;
+        std::string weights, scales;
+        for(auto g : members)
+        {
+            taken.insert(&*g);
+            const argument w = g->inputs()[1]->eval();
+            const argument s = g->inputs()[2]->eval();
+            weights.append(w.data(), w.get_shape().bytes());
+            scales.append(s.data(), s.get_shape().bytes());
+            n += g->inputs()[1]->get_shape().lens()[0];
+        }
+        auto a          = first->inputs()[0];
+        const auto rows = a->get_shape().lens()[0];
+        auto wl = m.add_literal(literal{shape{shape::uint8_type, {n, k2}}, weights.data()});
+        auto sl = m.add_literal(literal{shape{first->inputs()[2]->get_shape().type(), {n, kb}}, scales.data()});
+        w4a16_gemm fused = op;
+        fused.workspace  = false;
+        std::vector<instruction_ref> args = {a, wl, sl};
+        const size_t need = mi355_w4a16_gemm_workspace_size(static_cast<int64_t>(rows), static_cast<int64_t>(n),
+                                                            static_cast<int64_t>(2 * k2), op.group);
+        if(need > 0)
+        {
+            fused.workspace = true;
+            args.push_back(insert_allocation(m, first, shape{shape::uint8_type, {need}}));
+        }
+        args.push_back(insert_allocation(m, first, shape{shape::half_type, {rows, n}}));
+        auto all = m.insert_instruction(first, operation{fused}, args);
+        std::size_t at = 0;
+        for(auto g : members)
+        {
+            const auto cols = g->inputs()[1]->get_shape().lens()[0];
+            m.replace_instruction(g,
+                                  make_op("slice", {{"axes", {1}},
+                                                    {"starts", {static_cast<int64_t>(at)}},
+                                                    {"ends", {static_cast<int64_t>(at + cols)}}}),
+                                  {all});
+            at += cols;
+        }
+    }
+}
+
 // MIGRAPHX_MI355_FP32_DOT set (to anything but 0) when a program is compiled: float `dot`s run on
 // the fp32 matrix cores instead of reproducing the reference's double sum bit for bit
 bool fp32_dot_requested()
@@ -1228,6 +1315,8 @@ void lowering::apply(module& m) const
         else if(not fuse_quant_dot_dq(m, ins) and not fuse_quant_conv_dq(m, ins))
             fuse_dot_scale(m, ins);
     }
+    dead_code_elimination{}.apply(m);
+    fuse_shared_w4a16(m);
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)
     {

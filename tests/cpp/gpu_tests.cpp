@@ -744,6 +744,52 @@ TEST_CASE(int4_weight_only_gemv)
     }
 }
 
+TEST_CASE(int4_projections_sharing_activations)
+{
+    // q / k / v: three MatMulNBits of the same activations with constant weights become one launch
+    // over the stacked weights; every result is a slice of it with the bits of its own launch
+    for(std::size_t m : {1, 5})
+    {
+        const std::size_t k = 1024, blk = 128, nblk = k / blk;
+        const std::vector<std::size_t> ns = {256, 64, 96};
+        auto weights = [&](module& mod, std::size_t n, unsigned seed) {
+            auto b = mod.add_literal(literal{shape{shape::uint8_type, {n, nblk, blk / 2}}, uniform_ints<int>(n * nblk * blk / 2, 0, 255, seed)});
+            auto s = mod.add_literal(literal{shape{shape::half_type, {n * nblk}}, uniform_floats(n * nblk, 0.005f, 0.02f, seed + 1)});
+            return std::make_pair(b, s);
+        };
+        program all;
+        {
+            auto* mm = all.get_main_module();
+            auto a   = mm->add_parameter("a", shape{shape::half_type, {m, k}});
+            std::vector<migraphx::instruction_ref> outs;
+            for(std::size_t i = 0; i < ns.size(); i++)
+            {
+                auto ws = weights(*mm, ns[i], 70 + 10 * static_cast<unsigned>(i));
+                outs.push_back(migraphx::op::builder::matmulnbits(*mm, a, ws.first, ws.second, mm->end(), ns[i], k, blk));
+            }
+            mm->add_return(outs);
+        }
+        argument a{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 69)};
+        program c = all;
+        c.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+        auto got = run_on("mi355", all, {{"a", a}});
+        EXPECT(got.size() == ns.size());
+        for(std::size_t i = 0; i < ns.size(); i++)
+        {
+            program one;
+            auto* mm = one.get_main_module();
+            auto ap  = mm->add_parameter("a", shape{shape::half_type, {m, k}});
+            auto ws  = weights(*mm, ns[i], 70 + 10 * static_cast<unsigned>(i));
+            mm->add_return({migraphx::op::builder::matmulnbits(*mm, ap, ws.first, ws.second, mm->end(), ns[i], k, blk)});
+            expect_close_half(one, {{"a", a}});
+            auto alone = run_on("mi355", one, {{"a", a}});
+            EXPECT(alone.size() == 1 and got[i].get_shape().lens() == alone[0].get_shape().lens());
+            EXPECT(got[i].to_vector<double>() == alone[0].to_vector<double>());
+        }
+    }
+}
+
 TEST_CASE(int4_weight_only_gemm_small_batch)
 {
     for(std::size_t m : {2, 16})
