@@ -247,12 +247,14 @@ MI355_DEVINL float dc_scaled(int32_t a, float s)
         return (float)((double)a * (double)s);
 }
 
-// OUT == MI355_I32 stands for the bare accumulators (int32, or the float sums of fp8 operands)
+// OUT == MI355_I32 stands for the bare accumulators (int32, or the float sums of fp8 operands).
+// Nontemporal stores: the workgroup's stores cover whole lines of the result, which nothing on
+// this CU reads again.
 template <bool FP8, int OUT>
 MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
 {
     if constexpr(OUT == MI355_I32)
-        *reinterpret_cast<v4i*>(static_cast<int32_t*>(out) + idx) = a;
+        __builtin_nontemporal_store(a, reinterpret_cast<v4i*>(static_cast<int32_t*>(out) + idx));
     else
     {
         float v[4];
@@ -260,14 +262,17 @@ MI355_DEVINL void dc_store4(void* out, int64_t idx, v4i a, float s)
         for(int e = 0; e < 4; e++)
             v[e] = dc_scaled<FP8>(a[e], s);
         if constexpr(OUT == MI355_F32)
-            *reinterpret_cast<v4f*>(static_cast<float*>(out) + idx) = v4f{v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]},
+                                        reinterpret_cast<v4f*>(static_cast<float*>(out) + idx));
         else if constexpr(OUT == MI355_F16)
-            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + idx) =
-                make_uint2(convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16),
-                           convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16));
+            __builtin_nontemporal_store(
+                v2i{(int)(convert_f32_to_half(v[0]) | ((uint32_t)convert_f32_to_half(v[1]) << 16)),
+                    (int)(convert_f32_to_half(v[2]) | ((uint32_t)convert_f32_to_half(v[3]) << 16))},
+                reinterpret_cast<v2i*>(static_cast<uint16_t*>(out) + idx));
         else
-            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + idx) =
-                make_uint2(convert_f32_to_bf16x2(v[0], v[1]), convert_f32_to_bf16x2(v[2], v[3]));
+            __builtin_nontemporal_store(
+                v2i{(int)convert_f32_to_bf16x2(v[0], v[1]), (int)convert_f32_to_bf16x2(v[2], v[3])},
+                reinterpret_cast<v2i*>(static_cast<uint16_t*>(out) + idx));
     }
 }
 
@@ -663,7 +668,7 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
             const int64_t at =
                 ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * p.c + c0 +
                 16 * piece;
-            *reinterpret_cast<uint4*>(p.xt + at) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+            __builtin_nontemporal_store(v4u{packed[0], packed[1], packed[2], packed[3]}, reinterpret_cast<v4u*>(p.xt + at));
         }
         return;
     }
@@ -679,7 +684,7 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         {
             const int x = t / cp - p.pad_w;
             if(whole || x < 0 || x >= p.w_)
-                *reinterpret_cast<uint4*>(dst + (int64_t)t * 16) = make_uint4(0, 0, 0, 0);
+                __builtin_nontemporal_store(v4u{0, 0, 0, 0}, reinterpret_cast<v4u*>(dst + (int64_t)t * 16));
         }
         return;
     }
