@@ -389,6 +389,15 @@ def main():
             room = torch.empty(1 << 28, dtype=torch.uint8, device=dev)
             tk, _ = _time_launches(lambda: ops.quant_convolution(xq, wq, (1, 1), scale_x=sx, scale_w=sw, out=first,
                                                                  workspace=room), 20, 5, settle_ms=60)
+            if not args.no_check:
+                # the last image of the batch against the oracle: int8 sums and their dequantization are exact
+                xi = xq[31:32].cpu().numpy()
+                acc = orc.convolution(xi, wq.cpu().numpy(), orc.I8, (1, 1), (1, 1), (1, 1), 1)
+                scale = np.ascontiguousarray(np.broadcast_to(
+                    (np.float32(0.02) * sw.cpu().numpy()).astype(np.float32).reshape(1, -1, 1, 1), acc.shape))
+                want = orc.dequantizelinear(acc, scale, None, orc.I32, orc.F32)
+                checks[f"quant_conv3x3_C{cc}_{hw}x{hw}"] = bool(np.array_equal(
+                    first[31:32].cpu().numpy().view(np.uint32), want.view(np.uint32)))
             opsn = 2.0 * 32 * oo * hw * hw * cc * 9
             also[f"quant_conv3x3_dq_N32_C{cc}_{hw}x{hw}_O{oo}"] = {
                 "TOPS": round(opsn / tk / 1e12, 1), "us_per_call": round(tk * 1e6, 1),
