@@ -154,6 +154,41 @@ def test_staged_kernel_exact_sums(ops, fp4, bt, m, n, k):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("bt,m,n,k", [(1, 300, 520, 4096), (2, 257, 260, 4352), (1, 512, 256, 4224), (1, 130, 300, 8192),
+                                      (1, 600, 256, 5120)])
+def test_four_wave_fp4_kernel_exact_sums(ops, bt, m, n, k):
+    """Packed fp4 x fp4 with K >= 4096: the four-wave kernel (exponent words loaded per lane, two scaled
+    MFMAs per tile pair and slab).  Even and odd slab counts, batches, ragged tiles; sums exact in fp32 as in
+    test_staged_kernel_exact_sums, so every output carries the reference's bits."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k + bt)
+    pa = rng.integers(0, 4, (bt, m, k // 2), dtype=np.uint8) | (rng.integers(0, 4, (bt, m, k // 2), dtype=np.uint8) << 4)
+    pb = rng.integers(0, 4, (bt, n, k // 2), dtype=np.uint8) | (rng.integers(0, 4, (bt, n, k // 2), dtype=np.uint8) << 4)
+    pa |= rng.integers(0, 2, pa.shape, dtype=np.uint8) << 3
+    pb |= rng.integers(0, 2, pb.shape, dtype=np.uint8) << 7
+    av = _fp4_values(pa.reshape(-1, k // 2)).reshape(bt, m, k)
+    bv = _fp4_values(pb.reshape(-1, k // 2)).reshape(bt, n, k)
+    sa = _block_scales(rng, (bt, m), k, -1, 1)
+    sb = _block_scales(rng, (bt, n), k, -1, 1)
+    want = _reference(av, bv, np.repeat(sa, 32, axis=2), np.repeat(sb, 32, axis=2))
+    print("mx four-wave fp4", bt, m, n, k, flush=True)
+    got = ops.quant_dot_mx(dev(pa), dev(pb), dev(sa), dev(sb), a_fp4=True, b_fp4=True).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+def test_four_wave_fp4_kernel_full_range_operands(ops):
+    """The same kernel on codes and exponents over their whole range: the path's tolerance."""
+    rng = np.random.default_rng(23)
+    m, n, k = 384, 512, 4096
+    pa = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    pb = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    av, bv = _fp4_values(pa), _fp4_values(pb)
+    sa_c, sb_c = _block_scales(rng, (m,), k), _block_scales(rng, (n,), k)
+    sa, sb = np.repeat(sa_c, 32, axis=1), np.repeat(sb_c, 32, axis=1)
+    want = _reference(av, bv, sa, sb)
+    got = ops.quant_dot_mx(dev(pa), dev(pb), dev(sa_c), dev(sb_c), a_fp4=True, b_fp4=True).cpu().numpy()
+    assert _close(got, want, av, bv, sa, sb).all()
+
+
 def test_staged_kernel_full_range_operands(ops):
     """The staged kernel on operands and exponents over their whole range: the path's tolerance."""
     rng = np.random.default_rng(21)
