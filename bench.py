@@ -29,6 +29,7 @@ PEAK_HBM_GBS = 8000.0
 # counter runs of this file scaled by the same counters' reading for a plain copy of known size
 # (profiles/quant_dot_int8_8192_counters.md holds both runs and the arithmetic).
 HEADLINE_TRAFFIC_BYTES = 1.0745e9
+RANDOM_OPERAND_CEILING_TOPS = 4080.0   # v_mfma_i32_16x16x64_i8 from registers, uniformly random operands, this chip
 
 
 def _time_launches(fn, steps, warmup, settle_ms=0.0):
@@ -443,7 +444,11 @@ def main():
                    "m": M, "n": N, "k": K},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_TOPS_INT8,
                      "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
-                     "traffic": HEADLINE_TRAFFIC_BYTES},
+                     "traffic": HEADLINE_TRAFFIC_BYTES,
+                     # what a register-only loop of the same MFMA sustains on uniformly random int8
+                     # operands (the chip is power limited on them: 1.95-2.0 instead of 2.4 GHz)
+                     "measured_mfma_ceiling_random_operands": RANDOM_OPERAND_CEILING_TOPS,
+                     "frac_of_measured_ceiling": round(kern_tops / RANDOM_OPERAND_CEILING_TOPS, 4)},
         "also": also,
         "checks": checks, "ok": all(checks.values()),
     }
