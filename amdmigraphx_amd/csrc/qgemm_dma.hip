@@ -3265,6 +3265,398 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
     }
 }
 
+// The same for fp8 x fp8 (a slab row is 64 codes in two blocks): the fragments, slots and MFMA count
+// of qgemm_w4_f8_kernel, one scaled MFMA per tile pair; lane group g holds chunks g and 2 + g of a
+// slab row (the instruction scales K [32 g, 32 g + 32) by group g's exponent), byte g of the row's
+// exponent word is its scale.
+__global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
+{
+    constexpr bool TRANS_B = true;
+    constexpr bool DEQ     = false;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    if(*p.mx_flag == p.mx_ticket)
+        return;
+
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 1; // 0..1
+    const int wave_n = wave & 1;  // 0..1
+
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const uint8_t* __restrict__ ga = p.a + (int64_t)blockIdx.y * p.stride_a;
+    const uint8_t* __restrict__ gb = p.b + (int64_t)blockIdx.y * p.stride_b;
+    const int nk = p.k / BK;
+
+    // ---- global -> LDS: exactly as in qgemm_w4_i8_kernel -------------------------------------
+    uint32_t a_off[8], b_off[4];
+    const int a_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+    {
+        const int r   = 8 * (wave + 4 * h) + (lane >> 3);
+        const int row = min(m0 + r, p.m - 1);
+        a_off[h]      = (uint32_t)row * (uint32_t)p.lda + a_chunk * 16;
+    }
+    const uint32_t a_tail_back = a_chunk >= 4 ? 64u : 0u;
+#pragma unroll
+    for(int h = 0; h < 4; h++)
+    {
+        const int blk = wave + 4 * h;
+        if constexpr(TRANS_B)
+        {
+            const int r     = 16 * blk + (lane >> 2);
+            const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+            const int col   = min(n0 + r, p.n - 1);
+            b_off[h]        = (uint32_t)col * (uint32_t)p.ldb + chunk * 16;
+        }
+        else
+        {
+            const int k     = 4 * blk + (lane >> 4);
+            const int chunk = (lane & 15) ^ (k & 7);
+            const int col   = min(n0 + chunk * 16, p.n - 16);
+            b_off[h]        = (uint32_t)k * (uint32_t)p.ldb + col;
+        }
+    }
+    auto issue_a = [&](int ss, int h) {
+        uint8_t* st           = lds + (ss % W4_A_STAGES) * A2_BYTES;
+        const uint8_t* a_base = ga + (int64_t)ss * (2 * BK);
+        const uint32_t back   = 2 * ss + 1 < nk ? 0u : a_tail_back;
+        load_to_lds(a_base + (a_off[h] - back), st + (wave + 4 * h) * 1024);
+    };
+    auto issue_b = [&](int kt, int h) {
+        uint8_t* st           = lds + W4_B_BASE + (kt & (STAGES - 1)) * B_BYTES;
+        const uint8_t* b_base = TRANS_B ? gb + (int64_t)kt * BK : gb + (int64_t)kt * BK * p.ldb;
+        load_to_lds(b_base + b_off[h], st + (wave + 4 * h) * 1024);
+    };
+    auto a_step_of   = [](int kt) { return (kt & 1) != 0 ? (kt + 5) / 2 : (kt + 4) / 2; };
+    auto issues_b    = [&](int kt) { return kt + 4 >= 0 && kt + 4 < nk; };
+    auto issues_a    = [&](int kt) { const int ss = a_step_of(kt); return ss >= 1 && 2 * ss < nk; };
+    auto issued_in   = [&](int kt) { return (issues_b(kt) ? 4 : 0) + (issues_a(kt) ? 4 : 0); };
+
+    // ---- LDS -> operand fragments -------------------------------------------------------------
+    const int lrow      = lane & 31;
+    const int lgrp      = lane >> 5;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    // A: rows of 128 bytes (two slabs); slab parity h, chunk x of this lane's 32 bytes is logical
+    // chunk 4h + 2*lgrp + x at position c ^ ((row >> 1) & 7)
+    uint32_t a_lane[2][2];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+            a_lane[h][x] = (wave_m * 128 + lrow) * (2 * BK) + (((4 * h + 2 * x + lgrp) ^ ((lrow >> 1) & 7)) << 4);
+    uint32_t b_lane[2];
+    {
+        const int sw = (lrow >> 2) & 3;
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+            b_lane[x] = W4_B_BASE + (wave_n * 128 + lrow) * BK + (((2 * x + lgrp) ^ sw) << 4);
+    }
+
+    v8i fa[2][4];
+    v8i fb[2][4];
+    // exponent bytes of the lane's rows (0..3: A tiles, 4..7: B tiles): in flight, one set per slab
+    // parity, and the current slab's, shifted so that byte 0 is the lane group's block
+    int sin[2][8] = {{0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0}};
+    int sc[8]     = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int sc_shift = 8 * lgrp;
+    const uint8_t* sa_ptr = p.mx_ea + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_a * 4 +
+                            (int64_t)(m0 + wave_m * 128 + lrow) * 4;
+    const uint8_t* sb_ptr = p.mx_eb + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_b * 4 +
+                            (int64_t)(n0 + wave_n * 128 + lrow) * 4;
+    const int64_t sa_step = (int64_t)p.mx_rows_a * 4, sb_step = (int64_t)p.mx_rows_b * 4;
+    v16f acc[4][4];
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int e = 0; e < 16; e++)
+                acc[i][j][e] = 0.f;
+
+#define RD128(dst, addr, imm) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define RDTR8(dst, addr, imm) \
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm) : "memory")
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define LDS1(dst, ptr, imm) \
+    asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(dst) : "v"(ptr), "n"(imm) : "memory")
+#define LOAD_SCALES(s, Q)                                                   \
+    do                                                                      \
+    {                                                                       \
+        const int s_          = min((s), nk - 1);                           \
+        const uint8_t* pa_    = sa_ptr + (int64_t)s_ * sa_step;             \
+        const uint8_t* pb_    = sb_ptr + (int64_t)s_ * sb_step;             \
+        LDS1(sin[Q][0], pa_, 0);   LDS1(sin[Q][1], pa_, 128);               \
+        LDS1(sin[Q][2], pa_, 256); LDS1(sin[Q][3], pa_, 384);               \
+        LDS1(sin[Q][4], pb_, 0);   LDS1(sin[Q][5], pb_, 128);               \
+        LDS1(sin[Q][6], pb_, 256); LDS1(sin[Q][7], pb_, 384);               \
+    } while(0)
+#define PUT4(frag, X, t)                \
+    do                                  \
+    {                                   \
+        frag[4 * (X) + 0] = t.x;        \
+        frag[4 * (X) + 1] = t.y;        \
+        frag[4 * (X) + 2] = t.z;        \
+        frag[4 * (X) + 3] = t.w;        \
+    } while(0)
+    // half X of A tile I of slab kt -> fa[Q][I]
+#define RA(kt, Q, I, X)                                                                         \
+    do                                                                                          \
+    {                                                                                           \
+        v4i t_;                                                                                 \
+        RD128(t_, lds0 + (((kt) >> 1) % W4_A_STAGES) * A2_BYTES + a_lane[(kt) & 1][X],          \
+              (I) * 32 * 2 * BK);                                                               \
+        PUT4(fa[Q][I], X, t_);                                                                  \
+    } while(0)
+    // part R of B tile J of slab kt: row-major B four transposing reads, K-contiguous B two
+#define RB(kt, Q, J, R)                                                                         \
+    do                                                                                          \
+    {                                                                                           \
+        const uint32_t s_ = lds0 + ((kt) & (STAGES - 1)) * B_BYTES;                             \
+        if constexpr(TRANS_B)                                                                   \
+        {                                                                                       \
+            if((R) < 2)                                                                         \
+            {                                                                                   \
+                v4i t_;                                                                         \
+                RD128(t_, s_ + b_lane[(R) & 1], (J) * 32 * BK);                                 \
+                PUT4(fb[Q][J], (R) & 1, t_);                                                    \
+            }                                                                                   \
+        }                                                                                       \
+        else                                                                                    \
+        {                                                                                       \
+            (void)s_;                                                                           \
+        }                                                                                       \
+    } while(0)
+#define WAIT_FRAGS(Q)                                                                           \
+    asm volatile("s_waitcnt lgkmcnt(0)"                                                         \
+                 : "+v"(fa[Q][0]), "+v"(fa[Q][1]), "+v"(fa[Q][2]), "+v"(fa[Q][3]),              \
+                   "+v"(fb[Q][0]), "+v"(fb[Q][1]), "+v"(fb[Q][2]), "+v"(fb[Q][3])::"memory")
+    // The B tile goes in first: the accumulator then holds the tile transposed and a lane owns runs
+    // of four consecutive columns of C (see the epilogue).  Assembly for the reason given in
+    // qgemm_w4_i8_kernel.  The compiler does not know that the statement is an MFMA and adds none
+    // of the wait states a 16-pass MFMA needs before its result may be read.  In the steady-state
+    // loop nothing reads an accumulator.  In the last slabs, whose loads and reads are conditional,
+    // the compiler keeps copies of the accumulators in scratch memory and stores them right behind
+    // the MFMA, so there the statement carries the wait states itself.
+#define MF(Q, I, J)                                                                        \
+    do                                                                                     \
+    {                                                                                      \
+        if constexpr(fast_)                                                                \
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" \
+                         : "+a"(acc[I][J])                                                 \
+                         : "v"(fb[Q][J]), "v"(fa[Q][I]), "v"(sc[4 + (J)]), "v"(sc[I]));    \
+        else                                                                               \
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]\n\t" \
+                         "s_nop 7\n\ts_nop 7\n\ts_nop 3"                                   \
+                         : "+a"(acc[I][J])                                                 \
+                         : "v"(fb[Q][J]), "v"(fa[Q][I]), "v"(sc[4 + (J)]), "v"(sc[I]));    \
+    } while(0)
+    // slot N of 32: 0..7 A reads, 8..23 B reads (8..15 when B is K-contiguous), 24..31 loads.
+#define OTHER(kt, Q, N)                                                                     \
+    do                                                                                      \
+    {                                                                                       \
+        if constexpr((N) < 8)                                                               \
+        {                                                                                   \
+            if(fast_ || more_) RA((kt) + 1, 1 - (Q), (N) >> 1, (N) & 1);                   \
+        }                                                                                   \
+        else if constexpr((N) < 24)                                                         \
+        {                                                                                   \
+            if(fast_ || more_) RB((kt) + 1, 1 - (Q), ((N) - 8) >> 2, ((N) - 8) & 3);       \
+        }                                                                                   \
+        else if constexpr((N) < 28)                                                         \
+        {                                                                                   \
+            if(fast_ || ldb_) issue_b((kt) + 4, (N) - 24);                                  \
+        }                                                                                   \
+        else                                                                                \
+        {                                                                                   \
+            if(fast_ || lda_) issue_a(ass_, (1 - (Q)) * 4 + (N) - 28);                      \
+        }                                                                                   \
+    } while(0)
+#define ROW(kt, Q, I)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        SB(); MF(Q, I, 0); SB(); OTHER(kt, Q, 8 * (I) + 0); SB(); OTHER(kt, Q, 8 * (I) + 1);  \
+        SB(); MF(Q, I, 1); SB(); OTHER(kt, Q, 8 * (I) + 2); SB(); OTHER(kt, Q, 8 * (I) + 3);  \
+        SB(); MF(Q, I, 2); SB(); OTHER(kt, Q, 8 * (I) + 4); SB(); OTHER(kt, Q, 8 * (I) + 5);  \
+        SB(); MF(Q, I, 3); SB(); OTHER(kt, Q, 8 * (I) + 6); SB(); OTHER(kt, Q, 8 * (I) + 7);  \
+    } while(0)
+#define WAIT_SLAB(kt)                                                                       \
+    do                                                                                      \
+    {                                                                                       \
+        const int cnt_ = issued_in((kt) - 2) + issued_in((kt) - 1) + 8;                      \
+        if(cnt_ >= 24)      wait_vmcnt<24>();                                               \
+        else if(cnt_ >= 20) wait_vmcnt<20>();                                               \
+        else if(cnt_ >= 16) wait_vmcnt<16>();                                               \
+        else if(cnt_ >= 12) wait_vmcnt<12>();                                               \
+        else                wait_vmcnt<8>();                                                \
+    } while(0)
+#define SLAB(kt, Q, FAST)                                                                   \
+    do                                                                                      \
+    {                                                                                       \
+        constexpr bool fast_ = (FAST);                                                      \
+        const int kt_     = (kt);                                                           \
+        const bool more_  = kt_ + 1 < nk;                                                   \
+        const bool ldb_   = issues_b(kt_);                                                  \
+        const bool lda_   = issues_a(kt_);                                                  \
+        const int ass_    = a_step_of(kt_);                                                 \
+        (void)more_; (void)ldb_; (void)lda_;                                                \
+        WAIT_FRAGS(Q);                                                                      \
+        if constexpr(fast_)                                                                 \
+            wait_vmcnt<24>();                                                               \
+        else                                                                                \
+            WAIT_SLAB(kt_);                                                                 \
+        block_barrier();                                                                    \
+        asm volatile("" : "+v"(sin[Q][0]), "+v"(sin[Q][1]), "+v"(sin[Q][2]), "+v"(sin[Q][3]), \
+                          "+v"(sin[Q][4]), "+v"(sin[Q][5]), "+v"(sin[Q][6]), "+v"(sin[Q][7])); \
+        _Pragma("unroll") for(int t_ = 0; t_ < 8; t_++) sc[t_] = sin[Q][t_] >> sc_shift;     \
+        asm volatile("" : "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]),               \
+                          "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));               \
+        LOAD_SCALES(kt_ + 2, Q);                                                            \
+        ROW(kt_, Q, 0); ROW(kt_, Q, 1); ROW(kt_, Q, 2); ROW(kt_, Q, 3);                     \
+        SB();                                                                               \
+    } while(0)
+
+    // ---- main loop: the schedule of qgemm_w4_i8_kernel ------------------------------------------
+#pragma unroll
+    for(int h = 0; h < 8; h++)
+        issue_a(0, h);
+#pragma unroll
+    for(int kt = -4; kt < 0; kt++)
+    {
+        if(kt == -2)
+            LOAD_SCALES(0, 0);
+        if(kt == -1)
+            LOAD_SCALES(1, 1);
+        if(issues_b(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_b(kt + 4, h);
+        }
+        if(issues_a(kt))
+        {
+#pragma unroll
+            for(int h = 0; h < 4; h++)
+                issue_a(a_step_of(kt), ((kt & 1) != 0 ? 0 : 4) + h);
+        }
+    }
+    {
+        const int cnt = issued_in(-2) + 8 + issued_in(-1);
+        if(cnt >= 24)      wait_vmcnt<24>();
+        else if(cnt == 20) wait_vmcnt<20>();
+        else if(cnt == 16) wait_vmcnt<16>();
+        else if(cnt == 12) wait_vmcnt<12>();
+        else               wait_vmcnt<8>();
+    }
+    block_barrier();
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+    {
+        RA(0, 0, i, 0);
+        RA(0, 0, i, 1);
+    }
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+    {
+        RB(0, 0, j, 0);
+        RB(0, 0, j, 1);
+        RB(0, 0, j, 2);
+        RB(0, 0, j, 3);
+    }
+    int kt = 0;
+    for(; kt + 6 < nk; kt += 2)
+    {
+        SLAB(kt, 0, true);
+        SLAB(kt + 1, 1, true);
+    }
+    // The second half of the accumulators was written last: it passes through a statement that
+    // holds the wait states before anything the compiler places here can read it.  The first half
+    // is at least eight MFMAs old.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3"
+                 : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]),
+                   "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));
+    for(; kt + 1 < nk; kt += 2)
+    {
+        SLAB(kt, 0, false);
+        SLAB(kt + 1, 1, false);
+    }
+    if(kt < nk)
+        SLAB(kt, 0, false);
+    wait_vmcnt<0>();
+    asm volatile("" : "+v"(sin[0][0]), "+v"(sin[0][1]), "+v"(sin[0][2]), "+v"(sin[0][3]), "+v"(sin[0][4]),
+                      "+v"(sin[0][5]), "+v"(sin[0][6]), "+v"(sin[0][7]), "+v"(sin[1][0]), "+v"(sin[1][1]),
+                      "+v"(sin[1][2]), "+v"(sin[1][3]), "+v"(sin[1][4]), "+v"(sin[1][5]), "+v"(sin[1][6]),
+                      "+v"(sin[1][7]));
+#undef SLAB
+#undef WAIT_SLAB
+#undef ROW
+#undef OTHER
+#undef MF
+#undef WAIT_FRAGS
+#undef RB
+#undef RA
+#undef PUT4
+#undef LOAD_SCALES
+#undef LDS1
+#undef SB
+#undef RDTR8
+#undef RD128
+
+    // ---- epilogue: the fp8 part of qgemm_dma_kernel's, 4 x 4 tiles per wave ---------------------
+    // Element e of lane l belongs to row l % 32 of the A tile and column 8*(e/4) + 4*(l/32) + e%4
+    // of the B tile: four groups of 4 consecutive columns, each written with one store.  One block
+    // of 32 columns at a time; its scales and biases are loaded ahead of the stores of the block
+    // before it (a load issued behind a store waits for it), and no more than two blocks' worth is
+    // held in registers.
+    if constexpr(!DEQ)
+    {
+        {
+            // The bare result through the LDS, as in qgemm_w4_i8_kernel: straight from the
+            // accumulators a store instruction writes 32 bytes of each of 32 rows, from a row-major
+            // copy in the LDS the 512 bytes of two whole rows of the wave's quadrant.
+            block_barrier();
+            constexpr int PITCH = 512 + 16;
+            uint8_t* mine       = lds + wave * 40960;
+            const int out_col   = n0 + wave_n * 128 + 4 * (lane & 31);
+            float* out_base     = static_cast<float*>(p.c) + (int64_t)blockIdx.y * p.stride_c + out_col;
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                uint8_t* buf = mine + (i & 1) * (32 * PITCH);
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                        *reinterpret_cast<v4f*>(buf + lrow * PITCH + (32 * j + 8 * g + 4 * lgrp) * 4) =
+                            v4f{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+                // (every read before the first store, see qgemm_w4_i8_kernel)
+                v4f val[16];
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                    val[t] = *reinterpret_cast<const v4f*>(buf + (2 * t + (lane >> 5)) * PITCH + (lane & 31) * 16);
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                    asm volatile("" : "+v"(val[t]));
+#pragma unroll
+                for(int t = 0; t < 16; t++)
+                {
+                    const int row = m0 + wave_m * 128 + 32 * i + 2 * t + (lane >> 5);
+                    if(row < p.m && out_col < p.n)
+                        store_rows(reinterpret_cast<v4f*>(out_base + (int64_t)row * p.ldc), val[t], p.stream_c);
+                }
+            }
+            return;
+        }
+    }
+}
+
 template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
 int launch_one(const dma_params& p, int batch, hipStream_t stream)
 {
@@ -3385,16 +3777,20 @@ int mi355_dma_mx_launch(const void* a, const void* b, float* c, int64_t m, int64
     if(!attrs_ok || (bits != 4 && bits != 8))
         return MI355_ERR_LAUNCH;
     dim3 grid(p.tiles_m * p.tiles_n, (unsigned)batch);
-    // fp4 with a K of 4096 codes or more: the four-wave kernel (as for int8 and fp8: it pays more per
-    // tile and less per slab)
-    if(bits == 4 && kbytes >= 2048 && p.vec_store && p.n % 4 == 0)
+    // rows of 2048 bytes and more (4096 fp4 codes, 2048 fp8 codes): the four-wave kernels (as for int8
+    // and fp8: they pay more per tile and less per slab)
+    if(kbytes >= 2048 && p.vec_store && p.n % 4 == 0)
     {
         static const hipError_t attr4 =
             hipFuncSetAttribute(reinterpret_cast<const void*>(qgemm_w4_mx4_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
-        if(attr4 != hipSuccess)
+        static const hipError_t attr8 =
+            hipFuncSetAttribute(reinterpret_cast<const void*>(qgemm_w4_mx8_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, W4_LDS_BYTES);
+        if(attr4 != hipSuccess || attr8 != hipSuccess)
             return MI355_ERR_LAUNCH;
-        hipLaunchKernelGGL(qgemm_w4_mx4_kernel, grid, dim3(W4_THREADS), W4_LDS_BYTES, stream, p);
+        hipLaunchKernelGGL(bits == 4 ? qgemm_w4_mx4_kernel : qgemm_w4_mx8_kernel, grid, dim3(W4_THREADS),
+                           W4_LDS_BYTES, stream, p);
         return mi355_launch_status();
     }
     // a result that stays in the caches leaves through the LDS copy (whole groups of 4 outputs)

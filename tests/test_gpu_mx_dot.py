@@ -175,6 +175,22 @@ def test_four_wave_fp4_kernel_exact_sums(ops, bt, m, n, k):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("bt,m,n,k", [(1, 300, 520, 2048), (2, 257, 260, 2176), (1, 512, 256, 2112), (1, 130, 300, 4096)])
+def test_four_wave_fp8_kernel_exact_sums(ops, bt, m, n, k):
+    """fp8 x fp8 with K >= 2048: the four-wave kernel (one scaled MFMA per tile pair and slab, byte g of the
+    row's exponent word for lane group g).  Even and odd slab counts, batches, ragged tiles; exact sums."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k + bt)
+    pa = orc.fp8_from_f32(rng.integers(-4, 5, (bt, m, k)).astype(np.float32))
+    pb = orc.fp8_from_f32(rng.integers(-4, 5, (bt, n, k)).astype(np.float32))
+    av, bv = orc.fp8_to_f32(pa), orc.fp8_to_f32(pb)
+    sa = _block_scales(rng, (bt, m), k, -1, 1)
+    sb = _block_scales(rng, (bt, n), k, -1, 1)
+    want = _reference(av, bv, np.repeat(sa, 32, axis=2), np.repeat(sb, 32, axis=2))
+    print("mx four-wave fp8", bt, m, n, k, flush=True)
+    got = ops.quant_dot_mx(dev(pa), dev(pb), dev(sa), dev(sb), a_fp4=False, b_fp4=False).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 def test_four_wave_fp4_kernel_full_range_operands(ops):
     """The same kernel on codes and exponents over their whole range: the path's tolerance."""
     rng = np.random.default_rng(23)
