@@ -1000,6 +1000,37 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
     uint8_t* col        = static_cast<uint8_t*>(workspace);
     uint8_t* wp         = col + d->n * d->group * plane * kp;
 
+    // A window of one element with unit strides and no padding is a product of matrices as the
+    // tensors lie: out[n] [O/G, P] = W [O/G, C/G] . x[n] [C/G, P], the input row-major as the second
+    // operand.  Nothing is gathered or copied.
+    // (channels in whole K steps and positions in fours: the GEMM's matrix-core kernels; other shapes would fall to
+    // its general kernel, which the gathered form below beats)
+    bool pointwise = window == 1 && plane % 4 == 0 && cg % K_STEP == 0 &&
+                     reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+    for(int i = 0; i < 3; i++)
+        pointwise = pointwise && d->stride[i] == 1 && d->pad[i] == 0 && d->pad_hi[i] == 0;
+    if(pointwise)
+    {
+        mi355_quant_dot_desc g = gemm_of(d, plane, cg);
+        g.ldb      = plane;
+        g.stride_b = d->c * plane;
+        g.trans_b  = 0;
+        const size_t esz1 = mi355_dtype_size(d->out_type);
+        for(int64_t grp = 0; grp < d->group; grp++)
+        {
+            const float* sw = scale_w;
+            if(d->dequant && d->scale_w_mode == MI355_QP_PER_ROW)
+                sw = scale_w + grp * og;
+            const int r = mi355_quant_dot_ws(&g, static_cast<const uint8_t*>(w) + grp * og * cg,
+                                             static_cast<const uint8_t*>(x) + grp * cg * plane,
+                                             static_cast<uint8_t*>(out) + (size_t)(grp * og * plane) * esz1, sw,
+                                             scale_x, nullptr, nullptr, nullptr, workspace, workspace_bytes, stream);
+            if(r != MI355_OK)
+                return r;
+        }
+        return MI355_OK;
+    }
+
     if(direct_form(d, ol) && reinterpret_cast<uintptr_t>(x) % 16 == 0)
     {
         uint8_t* ws = static_cast<uint8_t*>(workspace);

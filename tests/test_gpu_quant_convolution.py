@@ -54,6 +54,10 @@ CASES = [
     ((4, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # the benchmark's first layer shape, 4 images
     ((4, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1), (1, 1), 1),   # and its second
     ((2, 128, 28, 28), (128, 128, 3, 3), (1, 1), (2, 2), (1, 1), 1),   # stride 2
+    # windows of one element, unit strides, no padding: the GEMM on the tensors as they lie (row-major second operand)
+    ((2, 64, 28, 28), (128, 64, 1, 1), (0, 0), (1, 1), (1, 1), 1),     # 784 positions: the direct-to-LDS GEMM
+    ((3, 128, 16, 16), (96, 64, 1, 1), (0, 0), (1, 1), (1, 1), 2),     # two groups
+    ((2, 40, 7, 9), (24, 40, 1, 1), (0, 0), (1, 1), (3, 2), 1),        # 63 positions, 40 channels: the general GEMM
     # not the direct kernel's form (200 channels): one image of a deep layer through im2col and the GEMM's split K
     ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
@@ -119,6 +123,28 @@ def test_direct_kernel_dequant_without_vector_stores(ops, out):
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
     bare = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 2)
     assert np.array_equal(bare.cpu().numpy(), acc)
+
+
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_pointwise_convolution_dequant_epilogue(ops, out):
+    """A 1 x 1 convolution is the quantized GEMM on the tensors as they lie; the per-output-channel scale is the
+    GEMM's per-row scale.  Two groups, 256 positions."""
+    rng = np.random.default_rng(26)
+    xs, ws = (2, 128, 16, 16), (80, 64, 1, 1)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.0151)
+    sw = rng.uniform(0.001, 0.01, 80).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (0, 0), (1, 1), (1, 1), 2)
+    scale = np.broadcast_to((sx * sw).astype(np.float32).reshape(1, -1, 1, 1), acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_convolution(dev(x), dev(w), (0, 0), (1, 1), (1, 1), 2, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
 
 
 @pytest.mark.parametrize("out", ["f32", "bf16"])
