@@ -808,14 +808,17 @@ int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
     return (d->o / d->group + DC_COLS - 1) / DC_COLS * DC_COLS;
 }
 
-// The direct kernel's form of a layer: every group a multiple of 16 channels, a real
-// window, every window inside the padded volume, counts that fit the kernels' 32-bit indices.
+// The direct kernel's form of a layer: every group a multiple of 16 channels, every window
+// inside the padded volume, counts that fit the kernels' 32-bit indices.
 bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
 {
     const int64_t lim    = (int64_t)1 << 31;
     const int64_t cg     = d->c / d->group;
     const int64_t window = d->kd * d->kh * d->kw;
-    if(cg % 16 != 0 || window <= 1)
+    // a window of one element with unit strides is served better by the GEMM itself (the pointwise
+    // form of mi355_quant_convolution3d, or the gathered form for odd sizes); with strides the
+    // direct kernel's addressing does the subsampling
+    if(cg % 16 != 0 || (window <= 1 && d->stride[0] == 1 && d->stride[1] == 1 && d->stride[2] == 1))
         return false;
     const int64_t in[3]  = {d->d, d->h, d->w};
     const int64_t win[3] = {d->kd, d->kh, d->kw};

@@ -58,6 +58,7 @@ CASES = [
     ((2, 64, 28, 28), (128, 64, 1, 1), (0, 0), (1, 1), (1, 1), 1),     # 784 positions: the direct-to-LDS GEMM
     ((3, 128, 16, 16), (96, 64, 1, 1), (0, 0), (1, 1), (1, 1), 2),     # two groups
     ((2, 40, 7, 9), (24, 40, 1, 1), (0, 0), (1, 1), (3, 2), 1),        # 63 positions, 40 channels: the general GEMM
+    ((2, 64, 14, 14), (96, 64, 1, 1), (0, 0), (2, 2), (1, 1), 1),      # 1 x 1 with strides: the direct kernel subsamples
     # not the direct kernel's form (200 channels): one image of a deep layer through im2col and the GEMM's split K
     ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
