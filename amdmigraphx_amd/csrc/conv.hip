@@ -576,6 +576,7 @@ struct prep_params
     uint8_t* xt;
     uint8_t* wp;
     int n, c, d, h, w_;    // input
+    int cp;                // channels of the copy: c, or c rounded up to 16 (one group) with zeros behind
     int dp, hp, wp_;       // padded volume
     int pad_d, pad_h, pad_w;
     int group, og, ogp, cg, window, nk;
@@ -629,7 +630,7 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         // a thread gathers the 16 channels of one piece at one position; the four pieces of 16
         // neighbouring positions make a wave's store 1 KiB contiguous when C = 64
         const int piece = threadIdx.x & 3;
-        if(c0 + 16 * piece >= p.c)
+        if(c0 + 16 * piece >= p.cp)
             return;
 #pragma unroll
         for(int q = 0; q < PW; q++)
@@ -666,19 +667,19 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
             const int iy = so / p.w_ % p.h;
             const int iz = so / (p.w_ * p.h);
             const int64_t at =
-                ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * p.c + c0 +
+                ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * p.cp + c0 +
                 16 * piece;
             __builtin_nontemporal_store(v4u{packed[0], packed[1], packed[2], packed[3]}, reinterpret_cast<v4u*>(p.xt + at));
         }
         return;
     }
-    const int cp = p.c / 16;
+    const int cp = p.cp / 16;
     if((int)blockIdx.x < p.tiles + p.border_rows)
     {
         const int row = blockIdx.x - p.tiles;
         const int y   = row % p.hp - p.pad_h;
         const int z   = row / p.hp % p.dp - p.pad_d;
-        uint8_t* dst  = p.xt + (int64_t)row * p.wp_ * p.c;
+        uint8_t* dst  = p.xt + (int64_t)row * p.wp_ * p.cp;
         const bool whole = y < 0 || y >= p.h || z < 0 || z >= p.d;
         for(int t = threadIdx.x; t < p.wp_ * cp; t += 256)
         {
@@ -692,7 +693,8 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
     const int first    = p.tiles + p.border_rows;
     const int nthreads = ((int)gridDim.x - first) * 256;
     const int total    = p.group * p.nk * p.ogp * (DC_KSTEP / 16);
-    const int kg       = p.cg * p.window;
+    const int cgp      = p.group == 1 ? p.cp : p.cg; // a group's channels in the copy
+    const int kg       = cgp * p.window;
     for(int t = ((int)blockIdx.x - first) * 256 + threadIdx.x; t < total; t += nthreads)
     {
         const int k0 = t % (DC_KSTEP / 16) * 16;
@@ -703,12 +705,15 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         const int k  = s * DC_KSTEP + k0;
         if(oc < p.og && k < kg)
         {
-            // 16 | cg: the 16 bytes are 16 consecutive channels of one window element
-            const int tap      = k / p.cg;
-            const uint8_t* src = p.w + (((int64_t)g * p.og + oc) * p.cg + k % p.cg) * p.window + tap;
+            // the 16 bytes are 16 consecutive channels of one window element (zeros for the channels
+            // the copy adds)
+            const int tap      = k / cgp;
+            const int c0       = k % cgp;
+            const uint8_t* src = p.w + (((int64_t)g * p.og + oc) * p.cg + c0) * p.window + tap;
 #pragma unroll
             for(int e = 0; e < 16; e++)
-                packed[e / 4] |= (uint32_t)src[(int64_t)e * p.window] << (8 * (e % 4));
+                if(c0 + e < p.cg)
+                    packed[e / 4] |= (uint32_t)src[(int64_t)e * p.window] << (8 * (e % 4));
         }
         *reinterpret_cast<uint4*>(p.wp + (int64_t)t * 16) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     }
@@ -798,31 +803,39 @@ size_t staging_bytes(const mi355_quant_conv3d_desc* d, int64_t plane, int64_t kp
     return (b + 15) / 16 * 16;
 }
 
+// A group's channels in the direct kernel's copy of the input: with one group, any channel count
+// is rounded up to 16 (the copy and the reordered weights hold zeros there)
+int64_t direct_cgp(const mi355_quant_conv3d_desc* d)
+{
+    const int64_t cg = d->c / d->group;
+    return d->group == 1 ? (cg + 15) / 16 * 16 : cg;
+}
+
 // K steps and padded channel count of the direct kernel's weights
 int64_t direct_steps(const mi355_quant_conv3d_desc* d)
 {
-    return (d->c / d->group * d->kd * d->kh * d->kw + DC_KSTEP - 1) / DC_KSTEP;
+    return (direct_cgp(d) * d->kd * d->kh * d->kw + DC_KSTEP - 1) / DC_KSTEP;
 }
 int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
 {
     return (d->o / d->group + DC_COLS - 1) / DC_COLS * DC_COLS;
 }
 
-// The direct kernel's form of a layer: every group a multiple of 16 channels, every window
-// inside the padded volume, counts that fit the kernels' 32-bit indices.
+// The direct kernel's form of a layer: one group, or every group a multiple of 16 channels; every
+// window inside the padded volume, counts that fit the kernels' 32-bit indices.
 bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
 {
     const int64_t lim    = (int64_t)1 << 31;
-    const int64_t cg     = d->c / d->group;
     const int64_t window = d->kd * d->kh * d->kw;
     // a window of one element with unit strides is served better by the GEMM itself (the pointwise
     // form of mi355_quant_convolution3d, or the gathered form for odd sizes); with strides the
     // direct kernel's addressing does the subsampling
-    if(cg % 16 != 0 || (window <= 1 && d->stride[0] == 1 && d->stride[1] == 1 && d->stride[2] == 1))
+    if(direct_cgp(d) % 16 != 0 || (window <= 1 && d->stride[0] == 1 && d->stride[1] == 1 && d->stride[2] == 1))
         return false;
     const int64_t in[3]  = {d->d, d->h, d->w};
     const int64_t win[3] = {d->kd, d->kh, d->kw};
-    int64_t volume       = d->c;
+    const int64_t cp     = direct_cgp(d) * d->group;
+    int64_t volume       = cp;
     for(int i = 0; i < 3; i++)
     {
         const int64_t padded = in[i] + d->pad[i] + d->pad_hi[i];
@@ -832,7 +845,7 @@ bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
         if(volume >= lim)
             return false;
     }
-    if(d->n * (volume / d->c) >= lim || d->n * d->c >= lim) // padded positions; channel planes
+    if(d->n * (volume / cp) >= lim || d->n * d->c >= lim) // padded positions; channel planes
         return false;
     const int64_t nk = direct_steps(d);
     if(nk * 8 > DC_MAX_PIECES)
@@ -850,7 +863,7 @@ bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
 size_t direct_bytes(const mi355_quant_conv3d_desc* d)
 {
     return (size_t)(d->group * direct_steps(d) * direct_ogp(d) * DC_KSTEP +
-                    d->n * d->c * (d->d + d->pad[0] + d->pad_hi[0]) * (d->h + d->pad[1] + d->pad_hi[1]) *
+                    d->n * direct_cgp(d) * d->group * (d->d + d->pad[0] + d->pad_hi[0]) * (d->h + d->pad[1] + d->pad_hi[1]) *
                         (d->w + d->pad[2] + d->pad_hi[2]));
 }
 
@@ -1046,6 +1059,7 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         q.xt = ws + d->group * nk * ogp * DC_KSTEP;
         q.n = (int)d->n;
         q.c = (int)d->c, q.d = (int)d->d, q.h = (int)d->h, q.w_ = (int)d->w;
+        q.cp = (int)(direct_cgp(d) * d->group);
         q.pad_d = (int)d->pad[0], q.pad_h = (int)d->pad[1], q.pad_w = (int)d->pad[2];
         q.dp = (int)(d->d + d->pad[0] + d->pad_hi[0]);
         q.hp = (int)(d->h + d->pad[1] + d->pad_hi[1]);
@@ -1055,7 +1069,7 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         const int64_t space = d->d * d->h * d->w;
         const bool dwords   = space % 4 == 0;
         q.tiles_s = (int)((space + (dwords ? 255 : 63)) / (dwords ? 256 : 64));
-        q.tiles_c = (int)((d->c + 63) / 64);
+        q.tiles_c = (int)((q.cp + 63) / 64);
         const int64_t tiles = d->n * q.tiles_c * q.tiles_s;
         const bool padded   = q.dp != q.d || q.hp != q.h || q.wp_ != q.w_;
         const int64_t border_rows = padded ? d->n * q.dp * q.hp : 0;
@@ -1079,12 +1093,12 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         p.scale_x = scale_x, p.scale_w = scale_w;
         p.rows = d->n * plane;
         p.plane = (int)plane, p.oh = (int)ol[1], p.ow = (int)ol[2];
-        p.o = (int)d->o, p.og = (int)og, p.ogp = (int)ogp, p.c = (int)d->c, p.cg = (int)cg;
+        p.o = (int)d->o, p.og = (int)og, p.ogp = (int)ogp, p.c = q.cp, p.cg = (int)direct_cgp(d);
         p.kh = (int)d->kh, p.kw = (int)d->kw;
         p.dp = q.dp, p.hp = q.hp, p.wp_ = q.wp_;
         p.stride_d = (int)d->stride[0], p.stride_h = (int)d->stride[1], p.stride_w = (int)d->stride[2];
         p.dil_d = (int)d->dil[0], p.dil_h = (int)d->dil[1], p.dil_w = (int)d->dil[2];
-        p.kg = (int)kg, p.nk = (int)nk;
+        p.kg = (int)(direct_cgp(d) * window), p.nk = (int)nk;
         p.col_tiles = (int)(ogp / DC_COLS);
         p.dequant = d->dequant, p.scale_x_mode = d->scale_x_mode, p.scale_w_mode = d->scale_w_mode;
         const int64_t row_tiles = (p.rows + DC_ROWS - 1) / DC_ROWS;

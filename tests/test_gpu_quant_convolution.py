@@ -38,7 +38,7 @@ CASES = [
     ((2, 5, 1, 40), (7, 5, 1, 5), (0, 2), (1, 3), (1, 1), 1),          # one-dimensional
     ((1, 20, 6, 6), (300, 20, 3, 3), (0, 0), (1, 1), (1, 1), 1),       # more than one row tile of weights
     ((2, 8, 9, 10), (8, 8, 3, 3), (0, 1, 2, 0), (2, 2), (1, 1), 1),    # low and high padding differ
-    # 16 | channels per group: the window matrix is gathered from a channels-last copy
+    # 16 | channels per group, two groups
     ((2, 64, 9, 11), (32, 32, 3, 2), (1, 0, 2, 1), (2, 1), (1, 2), 2),
     ((1, 16, 7, 7), (5, 16, 5, 5), (2, 2), (1, 1), (1, 1), 1),         # K = 400 -> 448
     ((3, 48, 6, 5), (7, 48, 2, 2), (0, 0), (1, 1), (1, 1), 1),
@@ -59,8 +59,13 @@ CASES = [
     ((3, 128, 16, 16), (96, 64, 1, 1), (0, 0), (1, 1), (1, 1), 2),     # two groups
     ((2, 40, 7, 9), (24, 40, 1, 1), (0, 0), (1, 1), (3, 2), 1),        # 63 positions, 40 channels: the general GEMM
     ((2, 64, 14, 14), (96, 64, 1, 1), (0, 0), (2, 2), (1, 1), 1),      # 1 x 1 with strides: the direct kernel subsamples
-    # not the direct kernel's form (200 channels): one image of a deep layer through im2col and the GEMM's split K
-    ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # not the direct kernel's form (two groups of 100 channels): one image of a deep layer through im2col and the
+    # GEMM's split K
+    ((1, 200, 7, 7), (64, 100, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    # one group with any channel count: the direct kernel on a copy whose channels are rounded up to 16 (zeros)
+    ((2, 3, 40, 36), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # an image network's first layer
+    ((2, 24, 14, 14), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # 200 -> 208 channels
 ]
 
 
