@@ -719,6 +719,115 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Many groups of a few channels each (depthwise layers: one channel per group).  A GEMM per group
+// would be a launch per group with K of a few bytes; here a thread computes one output element
+// from its C/G x window products (the input read along x, coalesced; a group's weights are a few
+// bytes that stay in the cache), in int32 / float, and applies the dequantizing epilogue.
+// ---------------------------------------------------------------------------------------------
+struct small_params
+{
+    const uint8_t* x;
+    const uint8_t* w;
+    void* out;
+    const float* scale_x;
+    const float* scale_w;
+    int64_t total; // N * O * plane
+    int c, d, h, w_;
+    int o, og, cg;
+    int kd, kh, kw, od, oh, ow;
+    int pad_d, pad_h, pad_w, stride_d, stride_h, stride_w, dil_d, dil_h, dil_w;
+    int dequant, scale_x_mode, scale_w_mode;
+};
+
+template <bool FP8, int OUT>
+__global__ __launch_bounds__(256) void conv_small_groups_kernel(small_params p)
+{
+    const int64_t step  = (int64_t)gridDim.x * 256;
+    const int plane     = p.od * p.oh * p.ow;
+    const int64_t space = (int64_t)p.d * p.h * p.w_;
+    const int window    = p.kd * p.kh * p.kw;
+    const float sx      = (p.dequant && p.scale_x_mode != MI355_QP_NONE) ? p.scale_x[0] : 1.f;
+    for(int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < p.total; t += step)
+    {
+        const int pos   = (int)(t % plane);
+        const int64_t r = t / plane;
+        const int oc    = (int)(r % p.o);
+        const int64_t n = r / p.o;
+        const int ox = pos % p.ow, oy = pos / p.ow % p.oh, oz = pos / (p.ow * p.oh);
+        const int g  = oc / p.og;
+        const uint8_t* xg = p.x + (n * p.c + (int64_t)g * p.cg) * space;
+        const uint8_t* wo = p.w + (int64_t)oc * p.cg * window;
+        int32_t acc_i = 0;
+        float acc_f   = 0.f;
+        for(int c = 0; c < p.cg; c++)
+            for(int kz = 0; kz < p.kd; kz++)
+            {
+                const int iz = oz * p.stride_d - p.pad_d + kz * p.dil_d;
+                if(iz < 0 || iz >= p.d)
+                    continue;
+                for(int ky = 0; ky < p.kh; ky++)
+                {
+                    const int iy = oy * p.stride_h - p.pad_h + ky * p.dil_h;
+                    if(iy < 0 || iy >= p.h)
+                        continue;
+                    for(int kx = 0; kx < p.kw; kx++)
+                    {
+                        const int ix = ox * p.stride_w - p.pad_w + kx * p.dil_w;
+                        if(ix < 0 || ix >= p.w_)
+                            continue;
+                        const uint8_t xv = xg[c * space + ((int64_t)iz * p.h + iy) * p.w_ + ix];
+                        const uint8_t wv = wo[(c * p.kd + kz) * p.kh * p.kw + ky * p.kw + kx];
+                        if constexpr(FP8)
+                            acc_f += __builtin_amdgcn_cvt_f32_fp8(xv, 0) * __builtin_amdgcn_cvt_f32_fp8(wv, 0);
+                        else
+                            acc_i += (int32_t)(int8_t)xv * (int32_t)(int8_t)wv;
+                    }
+                }
+            }
+        if constexpr(OUT == MI355_I32)
+        {
+            // the bare sums: int32, or float for fp8 operands
+            if constexpr(FP8)
+                static_cast<float*>(p.out)[t] = acc_f;
+            else
+                static_cast<int32_t*>(p.out)[t] = acc_i;
+        }
+        else
+        {
+            float sw = 1.f;
+            if(p.scale_w_mode == MI355_QP_PER_TENSOR)
+                sw = p.scale_w[0];
+            else if(p.scale_w_mode == MI355_QP_PER_ROW)
+                sw = p.scale_w[oc];
+            const float s = sw * sx;
+            const float v = FP8 ? acc_f * s : (float)((double)acc_i * (double)s);
+            if constexpr(OUT == MI355_F32)
+                static_cast<float*>(p.out)[t] = v;
+            else if constexpr(OUT == MI355_F16)
+                static_cast<uint16_t*>(p.out)[t] = convert_f32_to_half(v);
+            else
+                static_cast<uint16_t*>(p.out)[t] = convert_f32_to_bf16(v);
+        }
+    }
+}
+
+template <bool FP8>
+void launch_small_groups(const small_params& p, bool dequant, int out_type, hipStream_t hs)
+{
+    int64_t blocks = (p.total + 255) / 256;
+    blocks         = blocks > 256 * 64 ? 256 * 64 : blocks;
+    const dim3 grid((unsigned)blocks), block(256);
+    if(!dequant)
+        hipLaunchKernelGGL((conv_small_groups_kernel<FP8, MI355_I32>), grid, block, 0, hs, p);
+    else if(out_type == MI355_F32)
+        hipLaunchKernelGGL((conv_small_groups_kernel<FP8, MI355_F32>), grid, block, 0, hs, p);
+    else if(out_type == MI355_F16)
+        hipLaunchKernelGGL((conv_small_groups_kernel<FP8, MI355_F16>), grid, block, 0, hs, p);
+    else
+        hipLaunchKernelGGL((conv_small_groups_kernel<FP8, MI355_BF16>), grid, block, 0, hs, p);
+}
+
 int64_t out_len(int64_t in, int64_t k, int64_t pad_lo, int64_t pad_hi, int64_t stride, int64_t dil)
 {
     const int64_t span = in - (1 + dil * (k - 1)) + pad_lo + pad_hi;
@@ -1045,6 +1154,28 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
                 return r;
         }
         return MI355_OK;
+    }
+
+    // several groups of few channels (and not the direct kernel's form): one thread per output
+    if(d->group > 1 && cg % 16 != 0 && cg * window <= 256)
+    {
+        small_params q{};
+        q.x = static_cast<const uint8_t*>(x), q.w = static_cast<const uint8_t*>(w), q.out = out;
+        q.scale_x = scale_x, q.scale_w = scale_w;
+        q.total = d->n * d->o * plane;
+        q.c = (int)d->c, q.d = (int)d->d, q.h = (int)d->h, q.w_ = (int)d->w;
+        q.o = (int)d->o, q.og = (int)og, q.cg = (int)cg;
+        q.kd = (int)d->kd, q.kh = (int)d->kh, q.kw = (int)d->kw;
+        q.od = (int)ol[0], q.oh = (int)ol[1], q.ow = (int)ol[2];
+        q.pad_d = (int)d->pad[0], q.pad_h = (int)d->pad[1], q.pad_w = (int)d->pad[2];
+        q.stride_d = (int)d->stride[0], q.stride_h = (int)d->stride[1], q.stride_w = (int)d->stride[2];
+        q.dil_d = (int)d->dil[0], q.dil_h = (int)d->dil[1], q.dil_w = (int)d->dil[2];
+        q.dequant = d->dequant, q.scale_x_mode = d->scale_x_mode, q.scale_w_mode = d->scale_w_mode;
+        if(fp8)
+            launch_small_groups<true>(q, d->dequant != 0, d->out_type, hs);
+        else
+            launch_small_groups<false>(q, d->dequant != 0, d->out_type, hs);
+        return mi355_launch_status();
     }
 
     if(direct_form(d, ol) && reinterpret_cast<uintptr_t>(x) % 16 == 0)

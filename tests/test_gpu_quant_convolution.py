@@ -62,6 +62,9 @@ CASES = [
     # not the direct kernel's form (two groups of 100 channels): one image of a deep layer through im2col and the
     # GEMM's split K
     ((1, 200, 7, 7), (64, 100, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    # many groups of few channels (one thread per output): depthwise with strides, groups of 3 with dilation
+    ((3, 48, 15, 17), (48, 1, 3, 3), (1, 1), (2, 2), (1, 1), 48),
+    ((2, 24, 9, 9), (40, 3, 3, 3), (2, 2), (1, 1), (2, 2), 8),
     # one group with any channel count: the direct kernel on a copy whose channels are rounded up to 16 (zeros)
     ((2, 3, 40, 36), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # an image network's first layer
     ((2, 24, 14, 14), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1), 1),
@@ -129,6 +132,41 @@ def test_direct_kernel_dequant_without_vector_stores(ops, out):
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
     bare = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 2)
     assert np.array_equal(bare.cpu().numpy(), acc)
+
+
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+def test_depthwise_convolution_dequant_epilogue_and_fp8(ops, out):
+    """One channel per group: the one-thread-per-output kernel with the per-channel scale; fp8 operands on it give
+    exact sums for small integers and the fp8 tolerance otherwise."""
+    rng = np.random.default_rng(27)
+    xs, ws = (2, 40, 11, 13), (40, 1, 3, 3)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    sx = np.float32(0.0191)
+    sw = rng.uniform(0.001, 0.01, 40).astype(np.float32)
+    acc = orc.convolution(x, w, orc.I8, (1, 1), (1, 1), (1, 1), 40)
+    scale = np.broadcast_to((sx * sw).astype(np.float32).reshape(1, -1, 1, 1), acc.shape)
+    want = orc.dequantizelinear(acc, np.ascontiguousarray(scale), None, orc.I32, orc.F32)
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[out]
+    got = ops.quant_convolution(dev(x), dev(w), (1, 1), (1, 1), (1, 1), 40, scale_x=dev(np.float32([sx])),
+                                scale_w=dev(sw), out_dtype=td)
+    if out == "f32":
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, orc.F16 if out == "f16" else orc.BF16))
+    xi = rng.integers(-3, 4, xs).astype(np.float32)
+    wi = rng.integers(-2, 3, ws).astype(np.float32)
+    gotf = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(orc.fp8_from_f32(wi)), (1, 1), (1, 1), (1, 1), 40, fp8=True)
+    assert np.array_equal(gotf.cpu().numpy(), orc.convolution(xi, wi, orc.F32, (1, 1), (1, 1), (1, 1), 40))
+    xf = rng.standard_normal(xs).astype(np.float32)
+    wf = (rng.standard_normal(ws) * 0.05).astype(np.float32)
+    xq = orc.quantizelinear(xf.reshape(-1, xs[-1]), np.float32(np.abs(xf).max() / 448), None, orc.F32, orc.FP8).reshape(xs)
+    wq = orc.quantizelinear(wf.reshape(-1, ws[-1]), np.float32(np.abs(wf).max() / 448), None, orc.F32, orc.FP8).reshape(ws)
+    wantq = orc.convolution(xq, wq, orc.FP8, (1, 1), (1, 1), (1, 1), 40)
+    mag = orc.convolution(np.abs(orc.fp8_to_f32(xq)).astype(np.float32), np.abs(orc.fp8_to_f32(wq)).astype(np.float32),
+                          orc.F32, (1, 1), (1, 1), (1, 1), 40)
+    gotq = ops.quant_convolution(dev(xq), dev(wq), (1, 1), (1, 1), (1, 1), 40, fp8=True).cpu().numpy()
+    assert np.all(np.abs(gotq - wantq) <= np.maximum(1e-3 * np.abs(wantq), 2.0 ** -14 * mag))
 
 
 @pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
