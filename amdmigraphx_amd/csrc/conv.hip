@@ -1,12 +1,18 @@
-// quant_convolution as im2col + the quantized GEMM, over one, two or three spatial axes (a missing
-// leading axis is a depth of one).  The windows of the input are gathered into a
-// [N, group, OD*OH*OW, Kp] matrix (Kp = C/group * KD * KH * KW rounded up to the GEMM's K step, zero
-// filled), the weights are copied to rows of the same pitch, and for every image the result
-// plane [O, OD*OH*OW] = W [O, Kp] . col^T is one batched mi355_quant_dot with the col matrix as the
-// transposed operand: the GEMM writes NC(D)HW directly and its dequantize epilogue applies the
-// per-output-channel scale as a per-row scale.  Zero padding adds exact zeros to every sum
-// (int8: 0 * w; fp8: the code 0 is +0.0 and the padded weights are +0.0 too), so the result is the
-// direct convolution's.
+// quant_convolution over one, two or three spatial axes (a missing leading axis is a depth of one),
+// in four forms that mi355_quant_convolution3d chooses between:
+//   - a window of one element with unit strides and no padding: the batched quantized GEMM on the
+//     tensors as they lie (the input is its row-major second operand);
+//   - many groups of a few channels (depthwise): one thread per output element;
+//   - one group, or groups of a multiple of 16 channels: the direct kernel (an implicit GEMM over a
+//     padded channels-last copy of the input, see conv_direct_kernel);
+//   - everything else, im2col + GEMM: the windows of the input are gathered into a
+//     [N, group, OD*OH*OW, Kp] matrix (Kp = C/group * KD * KH * KW rounded up to the GEMM's K step,
+//     zero filled), the weights are copied to rows of the same pitch, and for every image the result
+//     plane [O, OD*OH*OW] = W [O, Kp] . col^T is one batched mi355_quant_dot with the col matrix as
+//     the transposed operand: the GEMM writes NC(D)HW directly and its dequantize epilogue applies
+//     the per-output-channel scale as a per-row scale.
+// Zero padding adds exact zeros to every sum (int8: 0 * w; fp8: the code 0 is +0.0 and the padded
+// weights are +0.0 too), so every form gives the direct convolution's result.
 #include "common.h"
 
 namespace {
