@@ -134,6 +134,35 @@ def test_direct_kernel_dequant_without_vector_stores(ops, out):
     assert np.array_equal(bare.cpu().numpy(), acc)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_layers_bit_exact(ops, seed):
+    """Random layers over every form the entry point chooses between (one to three spatial axes, any channel counts,
+    groups, windows, strides, dilations, low / high padding, batches that make row tiles straddle images): int32 sums
+    equal to the oracle's."""
+    rng = np.random.default_rng(1000 + seed)
+    nd = int(rng.integers(1, 4))
+    group = int(rng.choice([1, 1, 1, 2, 3, 8]))
+    cg = int(rng.choice([1, 3, 5, 16, 24, 32, 48])) if group == 1 or rng.random() < 0.5 else int(rng.choice([1, 2, 16, 32]))
+    og = int(rng.choice([1, 7, 16, 40, 70]))
+    win = [int(rng.integers(1, 4)) for _ in range(nd)]
+    stride = [int(rng.integers(1, 3)) for _ in range(nd)]
+    dil = [int(rng.integers(1, 3)) for _ in range(nd)]
+    pad_lo = [int(rng.integers(0, 3)) for _ in range(nd)]
+    pad_hi = [int(rng.integers(0, 3)) for _ in range(nd)]
+    size = [int(rng.integers(d * (k - 1) + 1, d * (k - 1) + 9)) for k, d in zip(win, dil)]
+    n = int(rng.integers(1, 5))
+    xs = (n, group * cg, *size)
+    ws = (group * og, cg, *win)
+    x = rng.integers(-128, 128, xs, dtype=np.int8)
+    w = rng.integers(-128, 128, ws, dtype=np.int8)
+    padding = tuple(pad_lo) + tuple(pad_hi)
+    want = orc.convolution(x, w, orc.I8, padding, tuple(stride), tuple(dil), group)
+    print("conv seeded", seed, xs, ws, padding, stride, dil, group, flush=True)
+    got = ops.quant_convolution(dev(x), dev(w), padding, tuple(stride), tuple(dil), group)
+    assert tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
 def test_depthwise_convolution_dequant_epilogue_and_fp8(ops, out):
     """One channel per group: the one-thread-per-output kernel with the per-channel scale; fp8 operands on it give
