@@ -65,6 +65,11 @@ CASES = [
     # many groups of few channels (one thread per output): depthwise with strides, groups of 3 with dilation
     ((3, 48, 15, 17), (48, 1, 3, 3), (1, 1), (2, 2), (1, 1), 48),
     ((2, 24, 9, 9), (40, 3, 3, 3), (2, 2), (1, 1), (2, 2), 8),
+    # the same kernel's four-outputs-of-a-row form (unit stride and dilation along x, at most 4 columns): a window
+    # 4 wide with padding 2 and a ragged last group, one column, and 5 columns (one output per thread again)
+    ((2, 12, 9, 10), (12, 1, 3, 4), (1, 2), (1, 1), (1, 1), 12),
+    ((1, 6, 5, 3), (6, 1, 3, 1), (1, 0), (2, 1), (1, 1), 6),
+    ((2, 12, 9, 11), (24, 2, 2, 5), (0, 2), (1, 1), (1, 1), 6),
     # one group with any channel count: the direct kernel on a copy whose channels are rounded up to 16 (zeros)
     ((2, 3, 40, 36), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # an image network's first layer
     ((2, 24, 14, 14), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1), 1),
