@@ -908,6 +908,13 @@ void launch_small_groups(const small_params& p, bool dequant, int out_type, hipS
         launch_small_groups_as<FP8, MI355_BF16>(p, hs);
 }
 
+// several groups of few channels each (and not the direct kernel's form): the vector-ALU kernel above
+bool small_groups_form(const mi355_quant_conv3d_desc* d)
+{
+    const int64_t cg = d->c / d->group;
+    return d->group > 1 && cg % 16 != 0 && cg * d->kd * d->kh * d->kw <= 256;
+}
+
 int64_t out_len(int64_t in, int64_t k, int64_t pad_lo, int64_t pad_hi, int64_t stride, int64_t dil)
 {
     const int64_t span = in - (1 + dil * (k - 1)) + pad_lo + pad_hi;
@@ -1142,6 +1149,9 @@ extern "C" int mi355_quant_convolution3d_dims(const mi355_quant_conv3d_desc* d,
         *workspace_bytes             = staging_bytes(d, plane, kp) + mi355_quant_dot_workspace_size(&g);
         if(direct_form(d, o) && *workspace_bytes < direct_bytes(d))
             *workspace_bytes = direct_bytes(d);
+        // the kernel for many small groups stages nothing (the entry point still wants a pointer)
+        if(small_groups_form(d))
+            *workspace_bytes = 16;
     }
     return MI355_OK;
 }
@@ -1236,8 +1246,8 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         return MI355_OK;
     }
 
-    // several groups of few channels (and not the direct kernel's form): one thread per output
-    if(d->group > 1 && cg % 16 != 0 && cg * window <= 256)
+    // several groups of few channels: one or four outputs per thread, nothing staged
+    if(small_groups_form(d))
     {
         small_params q{};
         q.x = static_cast<const uint8_t*>(x), q.w = static_cast<const uint8_t*>(w), q.out = out;

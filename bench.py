@@ -404,6 +404,29 @@ def main():
                 "TOPS": round(opsn / tk / 1e12, 1), "us_per_call": round(tk * 1e6, 1),
                 "us_per_call_allocating": round(tc * 1e6, 1)}
             del first, room
+        # the other forms the entry point chooses between: 1 x 1 (the batched GEMM on the tensors as they lie),
+        # depthwise (the vector-ALU kernel), an image network's first layer (3 channels padded to 16 in the copy)
+        for (name, xs, ws, pad, stride, group) in (
+                ("quant_conv1x1_dq_N32_C256_56x56_O64", (32, 256, 56, 56), (64, 256, 1, 1), (0, 0), (1, 1), 1),
+                ("quant_conv3x3_depthwise_dq_N32_C256_28x28", (32, 256, 28, 28), (256, 1, 3, 3), (1, 1), (1, 1), 256),
+                ("quant_conv7x7s2_dq_N32_C3_224x224_O64", (32, 3, 224, 224), (64, 3, 7, 7), (3, 3), (2, 2), 1)):
+            xq = torch.randint(-128, 128, xs, dtype=torch.int8, device=dev, generator=g)
+            wq = torch.randint(-128, 128, ws, dtype=torch.int8, device=dev, generator=g)
+            sx = torch.full((1,), 0.02, dtype=torch.float32, device=dev)
+            sw = torch.rand((ws[0],), device=dev, generator=g) * 0.01 + 0.001
+            first = ops.quant_convolution(xq, wq, pad, stride, (1, 1), group, scale_x=sx, scale_w=sw)
+            room = torch.empty(1 << 28, dtype=torch.uint8, device=dev)
+            tk, _ = _time_launches(lambda: ops.quant_convolution(xq, wq, pad, stride, (1, 1), group, scale_x=sx, scale_w=sw,
+                                                                 out=first, workspace=room), 20, 5, settle_ms=60)
+            if not args.no_check:
+                acc = orc.convolution(xq[31:32].cpu().numpy(), wq.cpu().numpy(), orc.I8, pad, stride, (1, 1), group)
+                scale = np.ascontiguousarray(np.broadcast_to(
+                    (np.float32(0.02) * sw.cpu().numpy()).astype(np.float32).reshape(1, -1, 1, 1), acc.shape))
+                want = orc.dequantizelinear(acc, scale, None, orc.I32, orc.F32)
+                checks[name] = bool(np.array_equal(first[31:32].cpu().numpy().view(np.uint32), want.view(np.uint32)))
+            moved = xq.numel() + wq.numel() + first.numel() * 4
+            also[name] = {"us_per_call": round(tk * 1e6, 1), "GB_per_s_tensors": round(moved / tk / 1e9, 1)}
+            del first, room
     except Exception as e:
         also["quant_conv_error"] = str(e)
 
