@@ -40,6 +40,25 @@ def test_float_dot_exact_and_fp32_accumulating(ops, bt, m, n, k, trans_b):
     assert (np.abs(scaled.astype(np.float64) - want * 0.125) <= mag * k * 2.0**-27 + 1e-30).all()
 
 
+@pytest.mark.parametrize("trans_a", [False, True])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_float_dot_whole_tiles_every_layout(ops, trans_a, trans_b):
+    """Each of the four operand layouts of the 16-byte-load kernel on whole tiles (rows or columns contiguous, for
+    either operand), bit for bit."""
+    bt, m, n, k = 2, 128, 192, 192
+    rng = np.random.default_rng(77 + 2 * trans_a + trans_b)
+    a = rng.standard_normal((bt, k, m) if trans_a else (bt, m, k)).astype(np.float32)
+    b = rng.standard_normal((bt, n, k) if trans_b else (bt, k, n)).astype(np.float32)
+    av = np.swapaxes(a, 1, 2) if trans_a else a
+    bv = np.swapaxes(b, 1, 2) if trans_b else b
+    want = orc.dot(np.ascontiguousarray(av), np.ascontiguousarray(bv), orc.F32)
+    ta = dev(a).transpose(1, 2) if trans_a else dev(a)
+    tb = dev(b).transpose(1, 2) if trans_b else dev(b)
+    print("float dot whole tiles", trans_a, trans_b, flush=True)
+    got = ops.dot(ta, tb).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_fp32_accumulation_is_float32_only(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((16, 16), dtype=torch.float16, device="cuda")
