@@ -2,7 +2,8 @@
 // in four forms that mi355_quant_convolution3d chooses between:
 //   - a window of one element with unit strides and no padding: the batched quantized GEMM on the
 //     tensors as they lie (the input is its row-major second operand);
-//   - many groups of a few channels (depthwise): one thread per output element;
+//   - many groups of a few channels: one or four outputs per thread on the vector ALU; depthwise
+//     layers over images from input rows staged in LDS (conv_depthwise_rows_kernel);
 //   - one group, or groups of a multiple of 16 channels: the direct kernel (an implicit GEMM over a
 //     padded channels-last copy of the input, see conv_direct_kernel);
 //   - everything else, im2col + GEMM: the windows of the input are gathered into a
@@ -873,9 +874,195 @@ __global__ __launch_bounds__(256) void conv_small_groups_kernel(small_params p)
     }
 }
 
+// Depthwise layers over images (one input channel per group, unit stride and dilation along x, at
+// most 4 window columns, at most 4 columns of padding on the left): a workgroup stages the input
+// rows that `th` output rows of one (image, output channel) need in LDS, zero border included, and
+// the window in front of them; a thread then computes four neighbouring outputs of a row from three
+// aligned LDS dwords per window row.  The one-output-per-thread form is bound by the number of
+// global byte loads (16 cycles of the address unit each); here a plane is fetched once, in dwords
+// where the rows are dword aligned (DW).
+// LDS: 64 bytes of window, then rows of `pitch` bytes; input column ix lies at byte 4 + ix.
+template <bool FP8, int OUT, bool DW>
+__global__ __launch_bounds__(256) void conv_depthwise_rows_kernel(small_params p, int th, int chunks, int pitch)
+{
+    extern __shared__ uint32_t dw_lds[];
+    uint8_t* wl        = reinterpret_cast<uint8_t*>(dw_lds);
+    uint32_t* tile32   = dw_lds + 16;
+    uint8_t* tile      = reinterpret_cast<uint8_t*>(tile32);
+    const int tid      = threadIdx.x;
+    const int nt       = blockDim.x; // 64, 128 or 256: a small plane takes one wave, and all of a layer's are resident at once
+    const int chunk    = blockIdx.x % chunks;
+    const int64_t noc  = blockIdx.x / chunks;
+    const int oc       = (int)(noc % p.o);
+    const int64_t n    = noc / p.o;
+    const int c        = oc / p.og;
+    const int window   = p.kh * p.kw;
+    const int oy0      = chunk * th;
+    const int nrows    = p.oh - oy0 < th ? p.oh - oy0 : th;
+    const int iy_base  = oy0 * p.stride_h - p.pad_h;
+    const int rows_in  = (nrows - 1) * p.stride_h + (p.kh - 1) * p.dil_h + 1;
+    const int pitch4   = pitch / 4;
+    for(int i = tid; i < rows_in * pitch4; i += nt)
+        tile32[i] = 0;
+    if(tid < window)
+        wl[tid] = p.w[(int64_t)oc * window + tid];
+    __syncthreads();
+    const uint8_t* xp = p.x + (n * p.c + c) * (int64_t)(p.h * p.w_);
+    if constexpr(DW)
+    {
+        const int wq = p.w_ / 4;
+        for(int i = tid; i < rows_in * wq; i += nt)
+        {
+            const int r = i / wq, q = i - r * wq, iy = iy_base + r;
+            if(iy >= 0 && iy < p.h)
+                tile32[r * pitch4 + 1 + q] = reinterpret_cast<const uint32_t*>(xp)[iy * wq + q];
+        }
+    }
+    else
+    {
+        for(int i = tid; i < rows_in * p.w_; i += nt)
+        {
+            const int r = i / p.w_, ix = i - r * p.w_, iy = iy_base + r;
+            if(iy >= 0 && iy < p.h)
+                tile[r * pitch + 4 + ix] = xp[iy * p.w_ + ix];
+        }
+    }
+    __syncthreads();
+
+    const int owq     = (p.ow + 3) / 4;
+    const int first   = p.pad_w == 0 ? 1 : 0;  // dword of a row that holds column 4 q - pad_w, minus q
+    const int shift   = (4 - p.pad_w) & 3;     // and that column's byte in it
+    const float sx    = (p.dequant && p.scale_x_mode != MI355_QP_NONE) ? p.scale_x[0] : 1.f;
+    float s           = 1.f;
+    if constexpr(OUT != MI355_I32)
+    {
+        float sw = 1.f;
+        if(p.scale_w_mode == MI355_QP_PER_TENSOR)
+            sw = p.scale_w[0];
+        else if(p.scale_w_mode == MI355_QP_PER_ROW)
+            sw = p.scale_w[oc];
+        s = sw * sx;
+    }
+    const bool vec = p.ow % 4 == 0 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0;
+    for(int it = tid; it < nrows * owq; it += nt)
+    {
+        const int ry = it / owq, q = it - ry * owq;
+        int32_t acc_i[4] = {0, 0, 0, 0};
+        float acc_f[4]   = {0.f, 0.f, 0.f, 0.f};
+        // columns outside the image hold zeros; an fp8 product with them is left out all the same (a NaN weight)
+        bool okx[7];
+#pragma unroll
+        for(int j = 0; j < 7; j++)
+            okx[j] = 4 * q - p.pad_w + j >= 0 && 4 * q - p.pad_w + j < p.w_;
+        for(int ky = 0; ky < p.kh; ky++)
+        {
+            const int r         = ry * p.stride_h + ky * p.dil_h;
+            const uint32_t* row = tile32 + r * pitch4 + q + first;
+            const uint32_t d0 = row[0], d1 = row[1], d2 = row[2];
+            const uint32_t lo = __builtin_amdgcn_alignbyte(d1, d0, shift);
+            const uint32_t hi = __builtin_amdgcn_alignbyte(d2, d1, shift);
+            const bool oky    = iy_base + r >= 0 && iy_base + r < p.h;
+#pragma unroll
+            for(int kx = 0; kx < 4; kx++)
+            {
+                if(kx < p.kw)
+                {
+                    const uint8_t wv = wl[ky * p.kw + kx];
+#pragma unroll
+                    for(int o4 = 0; o4 < 4; o4++)
+                    {
+                        const int j       = o4 + kx;
+                        const uint32_t xb = ((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu;
+                        if constexpr(FP8)
+                            acc_f[o4] += (okx[j] && oky) ? __builtin_amdgcn_cvt_f32_fp8(xb, 0) * __builtin_amdgcn_cvt_f32_fp8(wv, 0) : 0.f;
+                        else
+                            acc_i[o4] += (int32_t)(int8_t)xb * (int32_t)(int8_t)wv;
+                    }
+                }
+            }
+        }
+        const int64_t at = (noc * p.oh + oy0 + ry) * (int64_t)p.ow + 4 * q;
+        float v[4];
+#pragma unroll
+        for(int o4 = 0; o4 < 4; o4++)
+            v[o4] = FP8 ? (OUT == MI355_I32 ? acc_f[o4] : acc_f[o4] * s) : (float)((double)acc_i[o4] * (double)s);
+        if constexpr(OUT == MI355_I32 || OUT == MI355_F32)
+        {
+            if(vec)
+            {
+                if constexpr(OUT == MI355_I32 && !FP8)
+                    *reinterpret_cast<v4i*>(static_cast<int32_t*>(p.out) + at) = v4i{acc_i[0], acc_i[1], acc_i[2], acc_i[3]};
+                else
+                    *reinterpret_cast<v4f*>(static_cast<float*>(p.out) + at) = v4f{v[0], v[1], v[2], v[3]};
+                continue;
+            }
+        }
+#pragma unroll
+        for(int o4 = 0; o4 < 4; o4++)
+        {
+            if(4 * q + o4 >= p.ow)
+                break;
+            if constexpr(OUT == MI355_I32 && !FP8)
+                static_cast<int32_t*>(p.out)[at + o4] = acc_i[o4];
+            else if constexpr(OUT == MI355_I32 || OUT == MI355_F32)
+                static_cast<float*>(p.out)[at + o4] = v[o4];
+            else if constexpr(OUT == MI355_F16)
+                static_cast<uint16_t*>(p.out)[at + o4] = convert_f32_to_half(v[o4]);
+            else
+                static_cast<uint16_t*>(p.out)[at + o4] = convert_f32_to_bf16(v[o4]);
+        }
+    }
+}
+
+// rows of output per workgroup of the kernel above (0: not its form), and its LDS
+int depthwise_rows(const small_params& p, int* chunks, int* pitch, size_t* lds)
+{
+    if(p.cg != 1 || p.kd != 1 || p.d != 1 || p.od != 1 || p.pad_d != 0 || p.stride_w != 1 || p.dil_w != 1 || p.kw > 4 ||
+       p.pad_w > 4 || p.kh * p.kw > 64)
+        return 0;
+    const int owq = (p.ow + 3) / 4;
+    *pitch        = 4 * (owq + 3);
+    if(4 + p.w_ > *pitch) // (cannot be with unit stride and dilation; the staging loop relies on it)
+        return 0;
+    const int64_t halo    = (int64_t)(p.kh - 1) * p.dil_h + 1;
+    const int64_t rows_in = (32768 - 64) / *pitch;
+    if(rows_in < halo)
+        return 0;
+    int64_t th = (rows_in - halo) / p.stride_h + 1;
+    // about four work items per thread at most, so that large planes give several workgroups
+    const int64_t few = (1024 + owq - 1) / owq;
+    th                = th > few ? few : th;
+    th                = th > p.oh ? p.oh : th;
+    *chunks           = (int)((p.oh + th - 1) / th);
+    th                = (p.oh + *chunks - 1) / *chunks; // chunks of equal size
+    if((int64_t)p.total / p.ow / p.oh * *chunks >= ((int64_t)1 << 31))
+        return 0;
+    *lds = 64 + (size_t)(((th - 1) * p.stride_h + halo) * *pitch);
+    return (int)th;
+}
+
+template <bool FP8, int OUT>
+bool launch_depthwise_rows(const small_params& p, hipStream_t hs)
+{
+    int chunks = 0, pitch = 0;
+    size_t lds = 0;
+    const int th = depthwise_rows(p, &chunks, &pitch, &lds);
+    if(th == 0)
+        return false;
+    const int64_t items = (int64_t)th * ((p.ow + 3) / 4);
+    const dim3 grid((unsigned)(p.total / p.ow / p.oh * chunks)), block(items <= 256 ? 64 : items <= 512 ? 128 : 256);
+    if(p.w_ % 4 == 0 && reinterpret_cast<uintptr_t>(p.x) % 4 == 0)
+        hipLaunchKernelGGL((conv_depthwise_rows_kernel<FP8, OUT, true>), grid, block, lds, hs, p, th, chunks, pitch);
+    else
+        hipLaunchKernelGGL((conv_depthwise_rows_kernel<FP8, OUT, false>), grid, block, lds, hs, p, th, chunks, pitch);
+    return true;
+}
+
 template <bool FP8, int OUT>
 void launch_small_groups_as(small_params p, hipStream_t hs)
 {
+    if(launch_depthwise_rows<FP8, OUT>(p, hs))
+        return;
     const bool row4 = p.stride_w == 1 && p.dil_w == 1 && p.kw <= 4;
     p.items         = p.total / p.ow * ((p.ow + (row4 ? 3 : 0)) / (row4 ? 4 : 1));
     int64_t blocks  = (p.items + 255) / 256;

@@ -70,6 +70,13 @@ CASES = [
     ((2, 12, 9, 10), (12, 1, 3, 4), (1, 2), (1, 1), (1, 1), 12),
     ((1, 6, 5, 3), (6, 1, 3, 1), (1, 0), (2, 1), (1, 1), 6),
     ((2, 12, 9, 11), (24, 2, 2, 5), (0, 2), (1, 1), (1, 1), 6),
+    # depthwise over images with unit stride along x: rows staged in LDS.  Dword-aligned rows; several row chunks per
+    # plane with a strided, dilated 5 x 4 window and 4 columns of padding; two output channels per input channel;
+    # no padding on the left
+    ((2, 16, 28, 28), (16, 1, 3, 3), (1, 1), (1, 1), (1, 1), 16),
+    ((1, 2, 300, 64), (2, 1, 5, 4), (3, 4), (2, 1), (2, 1), 2),
+    ((2, 8, 12, 12), (16, 1, 3, 3), (1, 1), (1, 1), (1, 1), 8),
+    ((1, 4, 20, 24), (4, 1, 3, 3), (0, 0, 2, 3), (1, 1), (1, 1), 4),
     # one group with any channel count: the direct kernel on a copy whose channels are rounded up to 16 (zeros)
     ((2, 3, 40, 36), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # an image network's first layer
     ((2, 24, 14, 14), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1), 1),
