@@ -175,12 +175,13 @@ def test_seeded_random_layers_bit_exact(ops, seed):
     assert np.array_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("size", [(11, 13), (12, 16)])
 @pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
-def test_depthwise_convolution_dequant_epilogue_and_fp8(ops, out):
-    """One channel per group: the one-thread-per-output kernel with the per-channel scale; fp8 operands on it give
-    exact sums for small integers and the fp8 tolerance otherwise."""
+def test_depthwise_convolution_dequant_epilogue_and_fp8(ops, out, size):
+    """One channel per group: the kernel that stages rows in LDS (bytewise, and in dwords for rows of 16) with the
+    per-channel scale; fp8 operands on it give exact sums for small integers."""
     rng = np.random.default_rng(27)
-    xs, ws = (2, 40, 11, 13), (40, 1, 3, 3)
+    xs, ws = (2, 40, *size), (40, 1, 3, 3)
     x = rng.integers(-128, 128, xs, dtype=np.int8)
     w = rng.integers(-128, 128, ws, dtype=np.int8)
     sx = np.float32(0.0191)
@@ -199,6 +200,16 @@ def test_depthwise_convolution_dequant_epilogue_and_fp8(ops, out):
     wi = rng.integers(-2, 3, ws).astype(np.float32)
     gotf = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(orc.fp8_from_f32(wi)), (1, 1), (1, 1), (1, 1), 40, fp8=True)
     assert np.array_equal(gotf.cpu().numpy(), orc.convolution(xi, wi, orc.F32, (1, 1), (1, 1), (1, 1), 40))
+    # a NaN weight spoils the outputs whose window has that element inside the image only: products with the zero
+    # border are left out, as in the reference's loop (op/convolution.hpp skips positions outside the input)
+    wc = orc.fp8_from_f32(wi)
+    wc[0, 0, 0, 0] = 0x7F
+    wn = wi.copy()
+    wn[0, 0, 0, 0] = np.nan
+    gotn = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(wc), (1, 1), (1, 1), (1, 1), 40, fp8=True).cpu().numpy()
+    wantn = orc.convolution(xi, wn, orc.F32, (1, 1), (1, 1), (1, 1), 40)
+    assert np.isnan(wantn[:, 0, 1:, 1:]).all() and not np.isnan(wantn[:, 0, 0, :]).any()
+    assert np.array_equal(gotn, wantn, equal_nan=True)
     xf = rng.standard_normal(xs).astype(np.float32)
     wf = (rng.standard_normal(ws) * 0.05).astype(np.float32)
     xq = orc.quantizelinear(xf.reshape(-1, xs[-1]), np.float32(np.abs(xf).max() / 448), None, orc.F32, orc.FP8).reshape(xs)
