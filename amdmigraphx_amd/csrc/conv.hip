@@ -209,6 +209,7 @@ struct direct_params
     int kg, nk;         // K bytes of a group's window, K steps
     int col_tiles;      // 64-channel tiles per group
     int dequant, scale_x_mode, scale_w_mode;
+    int narrow;         // pixels of 4 channels; a K piece is 4 neighbouring window columns of one window row
 };
 
 MI355_DEVINL void dc_load_to_lds(const uint8_t* g, uint8_t* l)
@@ -311,7 +312,18 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(direct_params p)
         // times zero weights.  (An fp8 NaN there is in the true sum as well: it is the row's first
         // window element.)
         int off = 0;
-        if(q * 16 < p.kg)
+        if(p.narrow)
+        {
+            const int kwq = (p.kw + 3) / 4;
+            if(q * 16 < p.kg)
+            {
+                const int kxq = q % kwq;
+                const int ky  = q / kwq % p.kh;
+                const int kz  = q / (kwq * p.kh);
+                off = ((kz * p.dil_d * p.hp + ky * p.dil_h) * p.wp_ + 4 * kxq) * 4;
+            }
+        }
+        else if(q * 16 < p.kg)
         {
             const int tap = q * 16 / p.cg;
             const int c0  = q * 16 % p.cg;
@@ -590,6 +602,7 @@ struct prep_params
     int tiles_s, tiles_c;  // tiles along the positions and the channels of one image
     int tiles;             // n * tiles_c * tiles_s
     int border_rows;       // n * dp * hp, or 0 when nothing is padded
+    int narrow, kh, kw;    // pixels of 4 channels (cp = 4): a K piece of the weights is 4 window columns x 4 channels
 };
 
 // PW: input positions per load, 1 (bytes) or 4 (dwords, when the volume is a multiple of 4
@@ -637,6 +650,27 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         // a thread gathers the 16 channels of one piece at one position; the four pieces of 16
         // neighbouring positions make a wave's store 1 KiB contiguous when C = 64
         const int piece = threadIdx.x & 3;
+        if(p.narrow)
+        {
+            // four channels per position, one dword each (rows 4.. of the tile hold zeros: c <= 4)
+            for(int sl = threadIdx.x; sl < TILE_S; sl += 256)
+            {
+                const int so = ts * TILE_S + sl;
+                if(so >= space)
+                    break;
+                uint32_t px = 0;
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                    px |= (uint32_t)tile[e][sl] << (8 * e);
+                const int ix = so % p.w_;
+                const int iy = so / p.w_ % p.h;
+                const int iz = so / (p.w_ * p.h);
+                const int64_t at =
+                    ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * 4;
+                __builtin_nontemporal_store(px, reinterpret_cast<uint32_t*>(p.xt + at));
+            }
+            return;
+        }
         if(c0 + 16 * piece >= p.cp)
             return;
 #pragma unroll
@@ -688,6 +722,13 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         const int z   = row / p.hp % p.dp - p.pad_d;
         uint8_t* dst  = p.xt + (int64_t)row * p.wp_ * p.cp;
         const bool whole = y < 0 || y >= p.h || z < 0 || z >= p.d;
+        if(p.narrow)
+        {
+            for(int t = threadIdx.x; t < p.wp_; t += 256)
+                if(whole || t < p.pad_w || t >= p.pad_w + p.w_)
+                    __builtin_nontemporal_store(0u, reinterpret_cast<uint32_t*>(dst + (int64_t)t * 4));
+            return;
+        }
         for(int t = threadIdx.x; t < p.wp_ * cp; t += 256)
         {
             const int x = t / cp - p.pad_w;
@@ -710,7 +751,25 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         const int g  = t / (DC_KSTEP / 16) / p.ogp / p.nk;
         uint32_t packed[4] = {0, 0, 0, 0};
         const int k  = s * DC_KSTEP + k0;
-        if(oc < p.og && k < kg)
+        if(p.narrow)
+        {
+            const int kwq = (p.kw + 3) / 4;
+            const int q   = k / 16;
+            if(oc < p.og && q < p.window / p.kw * kwq)
+            {
+                const int kxq      = q % kwq;
+                const int rowk     = q / kwq; // (kz, ky)
+                const uint8_t* src = p.w + (int64_t)oc * p.cg * p.window + rowk * p.kw;
+#pragma unroll
+                for(int e = 0; e < 16; e++)
+                {
+                    const int kx = 4 * kxq + e / 4, ch = e % 4;
+                    if(kx < p.kw && ch < p.cg)
+                        packed[e / 4] |= (uint32_t)src[(int64_t)ch * p.window + kx] << (8 * (e % 4));
+                }
+            }
+        }
+        else if(oc < p.og && k < kg)
         {
             // the 16 bytes are 16 consecutive channels of one window element (zeros for the channels
             // the copy adds)
@@ -1188,15 +1247,28 @@ size_t staging_bytes(const mi355_quant_conv3d_desc* d, int64_t plane, int64_t kp
 
 // A group's channels in the direct kernel's copy of the input: with one group, any channel count
 // is rounded up to 16 (the copy and the reordered weights hold zeros there)
+// One group of at most 4 channels with several window columns (an image network's first layer), int8:
+// pixels of 4 channels, and a K piece of 16 bytes is 4 neighbouring window columns of a window row (unit
+// dilation along x) -- 16 x kd x kh x ceil(kw / 4) bytes of K per output instead of 16 x kd x kh x kw.
+// (Not for fp8: a piece reaches up to 3 pixels past the window, whose zero weights would not silence a NaN.)
+bool direct_narrow(const mi355_quant_conv3d_desc* d)
+{
+    return d->group == 1 && d->c <= 4 && d->kw >= 2 && d->dil[2] == 1 && d->in_type == MI355_I8;
+}
+
 int64_t direct_cgp(const mi355_quant_conv3d_desc* d)
 {
     const int64_t cg = d->c / d->group;
+    if(direct_narrow(d))
+        return 4;
     return d->group == 1 ? (cg + 15) / 16 * 16 : cg;
 }
 
 // K steps and padded channel count of the direct kernel's weights
 int64_t direct_steps(const mi355_quant_conv3d_desc* d)
 {
+    if(direct_narrow(d))
+        return (16 * d->kd * d->kh * ((d->kw + 3) / 4) + DC_KSTEP - 1) / DC_KSTEP;
     return (direct_cgp(d) * d->kd * d->kh * d->kw + DC_KSTEP - 1) / DC_KSTEP;
 }
 int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
@@ -1213,7 +1285,7 @@ bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
     // a window of one element with unit strides is served better by the GEMM itself (the pointwise
     // form of mi355_quant_convolution3d, or the gathered form for odd sizes); with strides the
     // direct kernel's addressing does the subsampling
-    if(direct_cgp(d) % 16 != 0 || (window <= 1 && d->stride[0] == 1 && d->stride[1] == 1 && d->stride[2] == 1))
+    if((direct_cgp(d) % 16 != 0 && !direct_narrow(d)) || (window <= 1 && d->stride[0] == 1 && d->stride[1] == 1 && d->stride[2] == 1))
         return false;
     const int64_t in[3]  = {d->d, d->h, d->w};
     const int64_t win[3] = {d->kd, d->kh, d->kw};
@@ -1247,7 +1319,8 @@ size_t direct_bytes(const mi355_quant_conv3d_desc* d)
 {
     return (size_t)(d->group * direct_steps(d) * direct_ogp(d) * DC_KSTEP +
                     d->n * direct_cgp(d) * d->group * (d->d + d->pad[0] + d->pad_hi[0]) * (d->h + d->pad[1] + d->pad_hi[1]) *
-                        (d->w + d->pad[2] + d->pad_hi[2]));
+                        (d->w + d->pad[2] + d->pad_hi[2]) +
+                    16); // (a narrow layer's last piece reaches up to 3 pixels past the copy's end)
 }
 
 template <bool FP8, int OUT, bool VEC, int STAGES>
@@ -1474,6 +1547,7 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         q.wp_ = (int)(d->w + d->pad[2] + d->pad_hi[2]);
         q.group = (int)d->group, q.og = (int)og, q.ogp = (int)ogp;
         q.cg = (int)cg, q.window = (int)window, q.nk = (int)nk;
+        q.narrow = direct_narrow(d) ? 1 : 0, q.kh = (int)d->kh, q.kw = (int)d->kw;
         const int64_t space = d->d * d->h * d->w;
         const bool dwords   = space % 4 == 0;
         q.tiles_s = (int)((space + (dwords ? 255 : 63)) / (dwords ? 256 : 64));
@@ -1507,6 +1581,9 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         p.stride_d = (int)d->stride[0], p.stride_h = (int)d->stride[1], p.stride_w = (int)d->stride[2];
         p.dil_d = (int)d->dil[0], p.dil_h = (int)d->dil[1], p.dil_w = (int)d->dil[2];
         p.kg = (int)(direct_cgp(d) * window), p.nk = (int)nk;
+        p.narrow = q.narrow;
+        if(p.narrow)
+            p.kg = (int)(16 * d->kd * d->kh * ((d->kw + 3) / 4));
         p.col_tiles = (int)(ogp / DC_COLS);
         p.dequant = d->dequant, p.scale_x_mode = d->scale_x_mode, p.scale_w_mode = d->scale_w_mode;
         const int64_t row_tiles = (p.rows + DC_ROWS - 1) / DC_ROWS;

@@ -79,6 +79,12 @@ CASES = [
     ((1, 4, 20, 24), (4, 1, 3, 3), (0, 0, 2, 3), (1, 1), (1, 1), 4),
     # one group with any channel count: the direct kernel on a copy whose channels are rounded up to 16 (zeros)
     ((2, 3, 40, 36), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),        # an image network's first layer
+    # at most 4 channels in one group: pixels of 4 channels, K pieces of 4 window columns.  4 channels with a window
+    # of exactly 4 columns and a dilated, strided y; one channel with 5 columns (the second piece reaches past the
+    # window, and past the copy's end at the last row); 2 columns
+    ((2, 4, 17, 19), (10, 4, 3, 4), (2, 1), (2, 1), (2, 1), 1),
+    ((3, 1, 9, 12), (70, 1, 3, 5), (0, 0), (1, 1), (1, 1), 1),
+    ((2, 2, 11, 8), (16, 2, 2, 2), (1, 0, 0, 1), (1, 2), (1, 1), 1),
     ((2, 24, 14, 14), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((1, 200, 7, 7), (64, 200, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # 200 -> 208 channels
 ]
