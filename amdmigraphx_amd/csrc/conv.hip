@@ -5,7 +5,8 @@
 //   - many groups of a few channels: one or four outputs per thread on the vector ALU; depthwise
 //     layers over images from input rows staged in LDS (conv_depthwise_rows_kernel);
 //   - one group, or groups of a multiple of 16 channels: the direct kernel (an implicit GEMM over a
-//     padded channels-last copy of the input, see conv_direct_kernel);
+//     padded channels-last copy of the input, see conv_direct_kernel; pixels of 4 channels for a
+//     first layer's 1 to 4 channels, see direct_narrow);
 //   - everything else, im2col + GEMM: the windows of the input are gathered into a
 //     [N, group, OD*OH*OW, Kp] matrix (Kp = C/group * KD * KH * KW rounded up to the GEMM's K step,
 //     zero filled), the weights are copied to rows of the same pitch, and for every image the result
@@ -613,6 +614,36 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
     constexpr int TILE_S = 64 * PW;
     __shared__ __align__(16) uint8_t tile[64][TILE_S + 4];
     const int space = p.d * p.h * p.w_;
+    if(p.narrow && (int)blockIdx.x < p.tiles)
+    {
+        // pixels of 4 channels (at most 4 channel planes): a thread forms 4 pixels of the padded copy, zero border
+        // included, from one byte per channel; a tile is 1024 pixels
+        const int64_t total = (int64_t)p.n * p.dp * p.hp * p.wp_;
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+        {
+            const int64_t px = ((int64_t)blockIdx.x * 4 + j) * 256 + threadIdx.x;
+            if(px >= total)
+                break;
+            const int ix = (int)(px % p.wp_) - p.pad_w;
+            int64_t r    = px / p.wp_;
+            const int iy = (int)(r % p.hp) - p.pad_h;
+            r /= p.hp;
+            const int iz = (int)(r % p.dp) - p.pad_d;
+            const int n  = (int)(r / p.dp);
+            uint32_t v   = 0;
+            if(ix >= 0 && ix < p.w_ && iy >= 0 && iy < p.h && iz >= 0 && iz < p.d)
+            {
+                const uint8_t* src = p.x + (int64_t)n * p.c * space + (iz * p.h + iy) * p.w_ + ix;
+#pragma unroll
+                for(int e = 0; e < 4; e++)
+                    if(e < p.c)
+                        v |= (uint32_t)src[(int64_t)e * space] << (8 * e);
+            }
+            __builtin_nontemporal_store(v, reinterpret_cast<uint32_t*>(p.xt + px * 4));
+        }
+        return;
+    }
     if((int)blockIdx.x < p.tiles)
     {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -650,27 +681,6 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         // a thread gathers the 16 channels of one piece at one position; the four pieces of 16
         // neighbouring positions make a wave's store 1 KiB contiguous when C = 64
         const int piece = threadIdx.x & 3;
-        if(p.narrow)
-        {
-            // four channels per position, one dword each (rows 4.. of the tile hold zeros: c <= 4)
-            for(int sl = threadIdx.x; sl < TILE_S; sl += 256)
-            {
-                const int so = ts * TILE_S + sl;
-                if(so >= space)
-                    break;
-                uint32_t px = 0;
-#pragma unroll
-                for(int e = 0; e < 4; e++)
-                    px |= (uint32_t)tile[e][sl] << (8 * e);
-                const int ix = so % p.w_;
-                const int iy = so / p.w_ % p.h;
-                const int iz = so / (p.w_ * p.h);
-                const int64_t at =
-                    ((((int64_t)n * p.dp + iz + p.pad_d) * p.hp + iy + p.pad_h) * (int64_t)p.wp_ + ix + p.pad_w) * 4;
-                __builtin_nontemporal_store(px, reinterpret_cast<uint32_t*>(p.xt + at));
-            }
-            return;
-        }
         if(c0 + 16 * piece >= p.cp)
             return;
 #pragma unroll
@@ -722,13 +732,6 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(prep_params p)
         const int z   = row / p.hp % p.dp - p.pad_d;
         uint8_t* dst  = p.xt + (int64_t)row * p.wp_ * p.cp;
         const bool whole = y < 0 || y >= p.h || z < 0 || z >= p.d;
-        if(p.narrow)
-        {
-            for(int t = threadIdx.x; t < p.wp_; t += 256)
-                if(whole || t < p.pad_w || t >= p.pad_w + p.w_)
-                    __builtin_nontemporal_store(0u, reinterpret_cast<uint32_t*>(dst + (int64_t)t * 4));
-            return;
-        }
         for(int t = threadIdx.x; t < p.wp_ * cp; t += 256)
         {
             const int x = t / cp - p.pad_w;
@@ -1552,9 +1555,15 @@ extern "C" int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* d,
         const bool dwords   = space % 4 == 0;
         q.tiles_s = (int)((space + (dwords ? 255 : 63)) / (dwords ? 256 : 64));
         q.tiles_c = (int)((q.cp + 63) / 64);
-        const int64_t tiles = d->n * q.tiles_c * q.tiles_s;
+        int64_t tiles       = d->n * q.tiles_c * q.tiles_s;
         const bool padded   = q.dp != q.d || q.hp != q.h || q.wp_ != q.w_;
-        const int64_t border_rows = padded ? d->n * q.dp * q.hp : 0;
+        int64_t border_rows = padded ? d->n * q.dp * q.hp : 0;
+        if(q.narrow)
+        {
+            // the narrow copy writes every pixel of the padded volume, the border among them
+            tiles       = (d->n * q.dp * q.hp * q.wp_ + 1023) / 1024;
+            border_rows = 0;
+        }
         // blocks behind them: the weights, one piece of 16 bytes per thread up to 1024 blocks
         int64_t extra = d->group * nk * ogp * (DC_KSTEP / 16) / 256 + 1;
         extra         = extra > 1024 ? 1024 : extra;
