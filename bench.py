@@ -29,6 +29,7 @@ PEAK_HBM_GBS = 8000.0
 # counter runs of this file scaled by the same counters' reading for a plain copy of known size
 # (profiles/quant_dot_int8_8192_counters.md holds both runs and the arithmetic).
 HEADLINE_TRAFFIC_BYTES = 1.0745e9
+HEADLINE_SETTLE_MS = 250.0
 RANDOM_OPERAND_CEILING_TOPS = 4080.0   # v_mfma_i32_16x16x64_i8 from registers, uniformly random operands, this chip
 
 
@@ -54,6 +55,28 @@ def _time_launches(fn, steps, warmup, settle_ms=0.0):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     return e0.elapsed_time(e1) / steps * 1e-3, wall
+
+
+def _w4a16_within_tolerance(got_bits, want_bits, x_bits, packed, scale_bits, group):
+    """The tolerance the GPU tests hold the int4 weight-only kernels to: 1e-3 relative, or one
+    half ulp, or 2^-19 of sum|a||w| where the dot product cancels (the reference sums exact
+    products in double and rounds once; the kernel sums in fp32)."""
+    import numpy as np
+    from oracle import oracle as orc
+    wq = orc.unpack_int4(packed)
+    wdq = orc.dequantizelinear(wq, np.repeat(scale_bits, group, axis=1),
+                               np.full(wq.shape, 8, np.uint8), orc.U8, orc.F16)
+    g = orc.half_to_f32(got_bits).astype(np.float64)
+    w = orc.half_to_f32(want_bits).astype(np.float64)
+    bound = np.abs(orc.half_to_f32(x_bits)).astype(np.float64) @ \
+        np.abs(orc.half_to_f32(wdq)).astype(np.float64).T
+    diff = np.abs(g - w)
+
+    def key(b):    # sign-magnitude half bits on one integer line
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7fff), b & 0x7fff)
+    one_ulp = np.abs(key(got_bits) - key(want_bits)) <= 1
+    return bool(((diff <= 1e-3 * np.abs(w)) | one_ulp | (diff <= bound * 2.0**-19)).all())
 
 
 def cpu_baseline(rows=16, n=8192, k=8192):
@@ -140,7 +163,9 @@ def main():
         def step():
             ops.quant_dot(a, b, out=c)
 
-        kern_s, wall_s = _time_launches(step, args.steps, args.warmup)
+        # whatever --warmup says, keep launching until the device has worked for well over the
+        # ~50 ms its clocks need to settle under this kernel; the timed region is the K steps after it
+        kern_s, wall_s = _time_launches(step, args.steps, args.warmup, settle_ms=HEADLINE_SETTLE_MS)
         if not args.no_check:
             checks["int8_quant_dot_8192"] = sampled_rows_equal(c, a, b.cpu().numpy(), [0, 255, 256, 4097, 8191])
         del a, b, c
@@ -180,9 +205,10 @@ def main():
             gf, wf = orc.bf16_to_f32(got).astype(np.float64), orc.bf16_to_f32(want).astype(np.float64)
             mag = np.abs(orc.fp8_to_f32(ah)).astype(np.float64) @ np.abs(orc.fp8_to_f32(bh)).astype(np.float64)
             d = np.abs(gf - wf)
-            # 1e-3 relative, or one bf16 step, or (cancelling sums) 2^-15 of sum|a||b| scaled
+            # 1e-3 relative, or one bf16 step, or (cancelling sums) 2^-18 of sum|a||b| scaled:
+            # the tolerance the GPU tests hold this distribution to
             okm = (d <= 1e-3 * np.abs(wf)) | (d <= np.abs(wf) * 2.0**-7) | \
-                  (d <= mag * 2.0**-15 * s1.item() * s2.item())
+                  (d <= mag * 2.0**-18 * s1.item() * s2.item())
             checks["fp8_quant_dot_config3"] = bool(okm.all())
         del a8, b8, o8
     except Exception as e:  # report, never hide the headline
@@ -219,11 +245,12 @@ def main():
                 cols = list(range(0, 8)) + [n4 // 2, n4 - 1]
                 last = copies - 1
                 xh = x.view(torch.int16).cpu().numpy().view(np.uint16)
-                want = orc.half_to_f32(orc.w4a16_matmul(
-                    xh, ws[last][cols].cpu().numpy(),
-                    sc[last][cols].view(torch.int16).cpu().numpy().view(np.uint16), 8, grp))
-                got = y[:, cols].float().cpu().numpy()
-                checks[f"w4a16_gemv_K{k4}_N{n4}"] = bool(np.allclose(got, want, rtol=2e-3, atol=2e-3))
+                wcols = ws[last][cols].cpu().numpy()
+                scols = sc[last][cols].view(torch.int16).cpu().numpy().view(np.uint16)
+                want_bits = orc.w4a16_matmul(xh, wcols, scols, 8, grp)
+                got_bits = y[:, cols].view(torch.int16).cpu().numpy().view(np.uint16)
+                checks[f"w4a16_gemv_K{k4}_N{n4}"] = _w4a16_within_tolerance(
+                    got_bits, want_bits, xh, wcols, scols, grp)
             graph = torch.cuda.CUDAGraph()
             side = torch.cuda.Stream()
             with torch.cuda.stream(side):
@@ -466,7 +493,7 @@ def main():
                                "uniform int8 (benchmark config 2, M=N=K=8192)",
                    "m": M, "n": N, "k": K},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_TOPS_INT8,
-                     "unit": "TFLOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
+                     "unit": "TOP/s", "frac": round(kern_tops / PEAK_TOPS_INT8, 4),
                      "traffic": HEADLINE_TRAFFIC_BYTES,
                      # what a register-only loop of the same MFMA sustains on uniformly random int8
                      # operands (the chip is power limited on them: 1.95-2.0 instead of 2.4 GHz)

@@ -1460,6 +1460,57 @@ TEST_CASE(encoder_int8_qdq_real_width)
     EXPECT(fast_dots == 2 * c.layers);
 }
 
+TEST_CASE(encoder_int8_qdq_full_size_replicated)
+{
+    // benchmark config 5 at its full size -- 12 layers, hidden 768, 12 heads, FFN 3072, 32 sequences
+    // of 384 tokens -- which the CPU oracle cannot evaluate in test time.  Every operator of the graph
+    // treats the sequences of a batch independently (the MatMuls row by row, attention per sequence and
+    // head, LayerNorm / softmax per row), the int8 sums are exact and the float `dot`s add in the
+    // reference's order whatever the batch, so a batch of 32 copies of one sequence must give 32 copies,
+    // bit for bit, of what the same 12 layers give for that sequence alone -- although the batch takes
+    // other kernels (M = 12288 instead of 384: other tiles, no split of K).  The one-sequence program is
+    // the shape that `encoder_int8_qdq_real_width` pins against the CPU target layer by layer.
+    encoder::config c1;
+    c1.layers = 12;
+    c1.hidden = 768;
+    c1.heads  = 12;
+    c1.ffn    = 3072;
+    c1.batch  = 1;
+    c1.seq    = 384;
+    c1.vocab  = 30522;
+    encoder::config c32 = c1;
+    c32.batch           = 32;
+    auto w              = encoder::make_weights(c1, 31);
+    auto one            = uniform_ints<int>(c1.tokens(), 0, static_cast<int>(c1.vocab) - 1, 32);
+    std::vector<int> many;
+    for(std::size_t b = 0; b < c32.batch; b++)
+        many.insert(many.end(), one.begin(), one.end());
+    argument ids1{shape{shape::int32_type, {c1.tokens()}}, one};
+    argument ids32{shape{shape::int32_type, {c32.tokens()}}, many};
+    auto scales = encoder::calibrate(c1, w, "mi355", ids1);
+    // max-abs calibration sees the same values 32 times over: the same scales
+    EXPECT(encoder::calibrate(c32, w, "mi355", ids32) == scales);
+    auto p1  = encoder::quantized(c1, w, scales);
+    auto p32 = encoder::quantized(c32, w, scales);
+    program compiled = p32;
+    compiled.compile(migraphx::make_target("mi355"));
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 6 * c32.layers);
+    auto alone = run_on("mi355", p1, {{"ids", ids1}})[0];
+    auto batch = run_on("mi355", p32, {{"ids", ids32}})[0];
+    const std::size_t bytes = alone.get_shape().bytes();
+    EXPECT(batch.get_shape().bytes() == bytes * c32.batch);
+    std::size_t differing = 0;
+    for(std::size_t b = 0; b < c32.batch; b++)
+        if(std::memcmp(batch.data() + b * bytes, alone.data(), bytes) != 0)
+            differing++;
+    EXPECT(differing == 0);
+    auto v = alone.to_vector<float>();
+    double s = 0;
+    for(float f : v)
+        s += std::fabs(f);
+    EXPECT(std::isfinite(s) and s / v.size() > 0.1);   // LayerNorm output: mean |x| is about 0.8
+}
+
 // `gpu_tests encoder_bench [layers]`: the full BERT-base shape (hidden 768, 12 heads, FFN 3072, batch
 // 32 x seq 384 = 12288 tokens, vocabulary 30522) on the device: calibration, compile, timed forwards
 static int encoder_bench(int argc, char** argv)

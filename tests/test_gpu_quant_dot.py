@@ -327,18 +327,23 @@ def _fp8_bound(a, b):
 # reference, or (bf16/half outputs) within 1 ulp of the output type, or --
 # where the exact sum cancels far below its terms, so that no fp32
 # accumulation in another order than the reference's can hold 1e-3 of the
-# result -- within 2^-15 of sum|a||b| (times the scale).  The last clause is a
+# result -- within 2^-15.5 of sum|a||b| (times the scale).  The last clause is a
 # declared deviation from "1e-3 relative or 1 bf16 ulp"; on the benchmark's own
-# operand distribution the measured error stays below 2^-18 of sum|a||b| and
-# test_full_size_fp8_config3_against_oracle holds the kernel to 2^-17 there and
+# operand distribution the measured error stays below 2^-19 of sum|a||b| and
+# test_full_size_fp8_config3_against_oracle holds the kernel to 2^-18 there and
 # bounds the share of outputs that need the clause at all.
-FP8_ABS_FLOOR = 2.0**-15
-FP8_CONFIG3_FLOOR = 2.0**-17
+FP8_ABS_FLOOR = 2.0**-15.5
+FP8_CONFIG3_FLOOR = 2.0**-18
 
 
 def _fp8_close(got, want, bound):
     diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    return (diff <= 1e-3 * np.abs(want)) | (diff <= bound * FP8_ABS_FLOOR)
+    rel = diff <= 1e-3 * np.abs(want)
+    need = ~rel & (bound > 0)
+    if need.any():    # what the floor clause was asked to cover (shown with pytest -s)
+        print("  fp8: %.2e of outputs outside 1e-3 relative, worst error / sum|a||b| = 2^%.2f"
+              % (need.mean(), np.log2((diff[need] / bound[need]).max())), flush=True)
+    return rel | (diff <= bound * FP8_ABS_FLOOR)
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (256, 512, 1024), (512, 384, 4096), (96, 132, 272)])
@@ -705,6 +710,39 @@ def test_full_size_int8_properties(ops, m, n, k, workspace):
     lhs = c.double().sum(0)
     rhs = a.double().sum(0) @ b.double()
     assert torch.equal(lhs, rhs)
+
+
+@pytest.mark.parametrize("n,k", [(768, 768), (3072, 768), (768, 3072)])
+def test_full_size_config5_linear_layers(ops, n, k):
+    """The quantized MatMuls of benchmark config 5 at their real size -- 32 x 384 = 12288 tokens
+    against hidden 768 / FFN 3072, per-tensor activation scale, per-output-channel weight scales,
+    bias, fp32 result -- as the one fused launch the lowering makes of them: sampled rows against
+    the oracle bit for bit (simplify_qdq.cpp:225-289, dequantizelinear.hpp:60-83, then the add), the
+    bare int32 accumulators of the same rows, and a checksum identity over the whole bare result."""
+    m = 12288
+    torch.manual_seed(n * 3 + k)
+    a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+    b = torch.randint(-127, 128, (k, n), dtype=torch.int8, device="cuda")
+    rng = np.random.default_rng(n + k)
+    sa = np.float32(0.0317)
+    sb = rng.uniform(0.0005, 0.002, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    print("config 5 linear layer", m, n, k, flush=True)
+    got = ops.quant_dot(a, b, scale_a=dev(np.float32([sa])), scale_b=dev(sb), bias=dev(bias),
+                        out_dtype=torch.float32)
+    bare = ops.quant_dot(a, b)
+    rows = [0, 1, 63, 64, 255, 256, 383, 384, 6143, 6144, 12031, 12287]
+    ah, bh = a[rows].cpu().numpy(), b.cpu().numpy()
+    assert np.array_equal(bare[rows].cpu().numpy(), orc.quant_dot(ah, bh, orc.I8))
+    want = orc.qdq_matmul_int8(ah, bh, sa, sb, 0, 0, orc.F32) + bias[None, :]
+    assert want.dtype == np.float32
+    assert np.array_equal(got[rows].cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.equal(bare.double().sum(1), a.double() @ b.double().sum(1))
+    assert torch.equal(bare.double().sum(0), a.double().sum(0) @ b.double())
+    # every row of the fused result is the dequantized bare row plus the bias, over the whole result
+    scale = torch.from_numpy(np.float32(sa) * sb).cuda()
+    whole = (bare.double() * scale.double()[None, :]).float() + dev(bias)[None, :]
+    assert torch.equal(got, whole)
 
 
 def test_graph_replay_of_split_k_and_int4_kernels(ops):
