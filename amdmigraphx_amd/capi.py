@@ -132,6 +132,12 @@ EXPORTS = {
                             ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
                             ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                             ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    "mi355_w4a16_prepacked_size": [ctypes.c_int64] * 3,
+    "mi355_w4a16_prepack": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
+                            ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p],
+    "mi355_w4a16_gemm_prepacked": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+                                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                   ctypes.c_void_p],
     "mi355_status_string": [ctypes.c_int],
     "mi355_version": [],
 }
@@ -167,7 +173,8 @@ def lib():
             fn = getattr(h, name)
             fn.argtypes = argtypes
             fn.restype = (ctypes.c_char_p if name == "mi355_status_string" else
-                          ctypes.c_size_t if name.endswith("_workspace_size") else ctypes.c_int)
+                          ctypes.c_size_t if name.endswith("_workspace_size") or name.endswith("_prepacked_size")
+                          else ctypes.c_int)
         _handle = h
     return _handle
 

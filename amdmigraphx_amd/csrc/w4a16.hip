@@ -380,7 +380,7 @@ __global__ __launch_bounds__(GV_THREADS) void w4a16_gemv_m1_kernel(w4_params p)
     }
 }
 
-constexpr int GV_MAX_K = 32768; // activations staged in LDS: 64 KiB; 4 slots per thread
+constexpr int GV_MAX_K = 16384; // activations staged in LDS: 4 slots of 8 halves per thread, 512 threads
 
 int launch_gemv_m1(const w4_params& p, hipStream_t s)
 {

@@ -493,6 +493,34 @@ def w4a16_gemm(a, w_packed, scales, group, zp=8, zp_mode=None, out=None, workspa
     return out
 
 
+def w4a16_prepack(w_packed, scales, group, zp=8):
+    """Reorder constant int4 weights [N, K/2] and their fp16 group scales [N, K/group] once for
+    w4a16_gemm_prepacked; returns the device buffer, or None when the reordered form does not
+    take the shape."""
+    _require_cuda(w_packed, scales)
+    n, k = w_packed.shape[0], w_packed.shape[1] * 2
+    size = int(lib().mi355_w4a16_prepacked_size(n, k, group))
+    if size == 0:
+        return None
+    if not (w_packed.is_contiguous() and scales.is_contiguous()):
+        raise Mi355Error("weights and scales must be dense")
+    out = torch.empty(size, dtype=torch.uint8, device=w_packed.device)
+    check(lib().mi355_w4a16_prepack(_ptr(w_packed), _ptr(scales), zp, n, k, group, _ptr(out), _stream()),
+          "mi355_w4a16_prepack")
+    return out
+
+
+def w4a16_gemm_prepacked(a, prepacked, n, out=None):
+    """fp16 activations [M, K] times weights reordered by w4a16_prepack (N rows)."""
+    _require_cuda(a, prepacked)
+    m, k = a.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    check(lib().mi355_w4a16_gemm_prepacked(_ptr(a), a.stride(0), _ptr(prepacked), _ptr(out), out.stride(0),
+                                           m, n, k, _stream()), "mi355_w4a16_gemm_prepacked")
+    return out
+
+
 def w4a16_gemm_workspace_size(m, n, k, group):
     """Bytes of workspace w4a16_gemm can use for that shape (0: none)."""
     return int(lib().mi355_w4a16_gemm_workspace_size(m, n, k, group))

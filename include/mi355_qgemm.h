@@ -393,6 +393,32 @@ int mi355_w4a16_gemm_ws(const void* a, int64_t lda,
                         void* stream);
 
 /*
+ * The same product for constant weights, reordered once ahead of time (a target does this when it
+ * compiles the program: the packed weights and scales of a weight-only layer are literals).
+ * mi355_w4a16_prepack writes, from the operator's own tensors (w_packed uint8 [N, K/2], scales fp16
+ * [N, K/128], one zero point for the tensor), a device buffer of mi355_w4a16_prepacked_size bytes
+ * that holds the same nibbles and scales -- 256 bytes more than the two tensors -- in the order
+ * the kernel's lanes read them; mi355_w4a16_gemm_prepacked then computes out = half(sum_k a * w)
+ * with w = half((q - zp) * scale) exactly as mi355_w4a16_gemm does (same reference chain:
+ * src/onnx/parse_matmulnbits.cpp:85-159, op/unpack_int4.hpp:75-121, op/dequantizelinear.hpp:60-83,
+ * op/dot.hpp:102-107), within the same tolerance of the fp32 sum.
+ * Shapes: group 128, N % 16 == 0, K % 512 == 0, K <= 28672, M == 1 (other M: MI355_ERR_UNSUPPORTED;
+ * the caller keeps mi355_w4a16_gemm for them).  mi355_w4a16_prepacked_size returns 0 for a shape
+ * the reordered form does not take.  Any scale values are accepted; the fastest form needs
+ * 2^-10 <= scale < 2^-4 and a zero point of 0, 1, 2, 4 or 8, which the reordering checks on the
+ * device and records in the buffer.
+ */
+size_t mi355_w4a16_prepacked_size(int64_t n, int64_t k, int64_t group);
+int mi355_w4a16_prepack(const void* w_packed, const void* scales, int32_t zp_scalar,
+                        int64_t n, int64_t k, int64_t group,
+                        void* prepacked, void* stream);
+int mi355_w4a16_gemm_prepacked(const void* a, int64_t lda,
+                               const void* prepacked,
+                               void* out, int64_t ldc,
+                               int64_t m, int64_t n, int64_t k,
+                               void* stream);
+
+/*
  * Float dot: C[b, m, n] = T( sum_k double(A[b, m, k]) * double(B[b, k, n]) ), k ascending,
  * T in {F32, F16, BF16} for all three tensors (16-bit results truncate, as the software
  * floats do).
