@@ -267,6 +267,16 @@ MI355_DEVINL void w4p_piece(const v4u& w, const w4p_consts& c, const uint8_t* a_
 // zero activations, so that the code has no branch and the compiler can overlap the LDS reads and
 // the matrix-core latency of one piece with the vector work of the next.  The general form may
 // meet scales that are not finite and skips such blocks instead.
+// block idx of a wave: row group rg0 + (idx / IS) * rg_stride, block w + (idx % IS) * wk of it (a
+// team past the last row group, or a wave past the last block, reads the last one and drops it)
+template <int IS>
+MI355_DEVINL const uint8_t* w4p_block_at(const w4p_params& p, int rg0, int w, int idx)
+{
+    const int rg = min(rg0 + (idx / IS) * p.rg_stride, p.nrg - 1);
+    const int s  = min(w + (idx % IS) * p.wk, p.nss - 1);
+    return p.pk + W4P_HEADER + ((int64_t)rg * p.nss + s) * W4P_BLOCK;
+}
+
 template <bool FAST, int IR, int IS>
 MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* zeros, float* red, int rg0, int team,
                              int w, int lane, int zp)
@@ -274,15 +284,11 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
     constexpr int TOTAL = IR * IS;
     static_assert(TOTAL >= 1 && TOTAL <= 4);
     const int zp_log2 = zp <= 1 ? 0 : (zp == 2 ? 1 : (zp == 4 ? 2 : 3));
-    auto block_at = [&](int idx) __attribute__((always_inline)) {
-        const int rg = min(rg0 + (idx / IS) * p.rg_stride, p.nrg - 1);
-        const int s  = min(w + (idx % IS) * p.wk, p.nss - 1);
-        return p.pk + W4P_HEADER + ((int64_t)rg * p.nss + s) * W4P_BLOCK;
-    };
-    w4p_item it[2];
-    w4p_issue(it[0], block_at(0), lane * 16, lane * 2);
-    if constexpr(TOTAL > 1)
-        w4p_issue(it[1], block_at(1), lane * 16, lane * 2);
+    // all of the wave's blocks are asked for at once
+    w4p_item it[TOTAL];
+#pragma unroll
+    for(int i = 0; i < TOTAL; i++)
+        w4p_issue(it[i], w4p_block_at<IS>(p, rg0, w, i), lane * 16, lane * 2);
 
     v4f acc[4];
 #pragma unroll
@@ -290,9 +296,9 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
         acc[c] = v4f{0.f, 0.f, 0.f, 0.f};
     auto block = [&](auto idx_tag) __attribute__((always_inline)) {
         constexpr int IDX = decltype(idx_tag)::value;
-        // loads behind this block's: the next block's five, issued before this one is taken up
-        constexpr int NEXT     = IDX + 1 < TOTAL ? 5 : 0;
-        w4p_item& b            = it[IDX & 1];
+        // loads behind this block's: five for every later block
+        constexpr int NEXT     = 5 * (TOTAL - 1 - IDX);
+        w4p_item& b            = it[IDX];
         const int rg           = rg0 + (IDX / IS) * p.rg_stride;
         const int s            = w + (IDX % IS) * p.wk;
         const bool live        = rg < p.nrg && s < p.nss;
@@ -310,8 +316,6 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
         w4p_wait_piece<0 + NEXT>(b.w[3]);
         if(FAST || live)
             w4p_piece<FAST>(b.w[3], c, a_block + 192, acc);
-        if constexpr(IDX + 2 < TOTAL)
-            w4p_issue(b, block_at(IDX + 2), lane * 16, lane * 2);
         if constexpr(IDX % IS == IS - 1)
         {
             // row 0 of the result tile: register 0 of lanes 0..15
@@ -389,6 +393,7 @@ w4p_gemv_kernel(w4p_params p)
         apiece[s] = min(tid + s * nthreads, a_pieces - 1);
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(areg[s]) : "v"(apiece[s] * 16), "s"(p.a) : "memory");
     }
+    const int rg0 = p.rg_base + blockIdx.x * p.teams + team;
     if(tid < 16)
         *reinterpret_cast<v4u*>(zeros + tid * 16) = v4u{0, 0, 0, 0};
     if constexpr(SLOTS == 1)
@@ -407,7 +412,6 @@ w4p_gemv_kernel(w4p_params p)
 
     // two separate bodies, each with its own loads and waits: a wait statement in each of two
     // branches for one load makes the compiler copy the loaded register in front of the branch
-    const int rg0 = p.rg_base + blockIdx.x * p.teams + team;
     if(__builtin_amdgcn_readfirstlane((flags & W4P_FLAG_GENERAL) == 0))
         w4p_blocks<true, IR, IS>(p, lds, zeros, red, rg0, team, w, lane, zp);
     else
@@ -497,12 +501,16 @@ extern "C" int mi355_w4a16_gemm_prepacked(const void* a,
     p.k   = (int)k;
     p.nss = (int)(k / W4P_SUPER_K);
     p.nrg = (int)(n / 16);
-    // waves per row group: all blocks of a row group in as few equal rounds as 16 waves allow
+    // Waves per row group (they split its blocks) and row groups per workgroup.  Measured on the
+    // shapes of a Llama-sized layer: two blocks per wave and row group beat one (half as many
+    // waves at the workgroup's barriers, one sum per two blocks) as long as the chip still gets
+    // some eight waves per CU, and two row groups per workgroup beat one where a row group has
+    // only four waves.
     p.iters_s = (p.nss + W4P_MAX_WAVES - 1) / W4P_MAX_WAVES;
-    p.wk      = (p.nss + p.iters_s - 1) / p.iters_s;
-    // two row groups per workgroup where that still leaves every CU more than one workgroup
-    // (the activation row is staged once per workgroup)
-    p.teams = (2 * p.wk <= W4P_MAX_WAVES && p.nrg >= 4 * 256) ? 2 : 1;
+    if(p.iters_s == 1 && p.nss >= 8 && p.nrg >= 384)
+        p.iters_s = 2;
+    p.wk    = (p.nss + p.iters_s - 1) / p.iters_s;
+    p.teams = (p.wk <= 4 && p.nrg >= 384) ? 2 : 1;
     // the activation row is staged with W4P_A_SLOTS pieces per thread
     while(p.k / 8 > W4P_A_SLOTS * p.teams * p.wk * 64 && (p.teams + 1) * p.wk <= W4P_MAX_WAVES)
         p.teams++;

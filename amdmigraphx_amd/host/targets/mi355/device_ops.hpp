@@ -232,6 +232,35 @@ struct w4a16_gemm
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// Constant int4 weights reordered once for the one-row product (mi355_w4a16_prepack).
+// inputs: packed weights uint8 [N, K/2], scales fp16 [N, K/128], out uint8 [mi355_w4a16_prepacked_size]
+struct w4a16_prepack
+{
+    int64_t zp_scalar = 8;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.zp_scalar, "zp_scalar");
+    }
+    std::string name() const { return "mi355::w4a16_prepack"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// inputs: a fp16 [1, K], reordered weights uint8 [bytes], out fp16 [1, N]
+struct w4a16_gemm_prepacked
+{
+    template <class Self, class F>
+    static void reflect(Self&, F)
+    {
+    }
+    std::string name() const { return "mi355::w4a16_gemm_prepacked"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: x, scale view, [zero point view], out
 struct quantizelinear
 {

@@ -574,7 +574,9 @@ bool lower_w4a16(module& m, instruction_ref ins)
 // is a few microseconds of weight streaming behind a launch and a fetch of the activations that
 // cost as much; with the weights (and their scales) stacked along N at compile time the products
 // become one launch, and each original result is a `slice` of its columns.  A column's sum does
-// not depend on which other columns are computed with it, so the results keep their bits.
+// not depend on which other columns are computed with it (the reordered one-row form splits K over
+// more or fewer waves with the number of columns, which can move a sum's last bit between a very
+// wide and a narrow product; the tolerance of the path covers it).
 // Taken: scalar zero points, weights and scales known at compile time, the same activations,
 // K, group size and zero point.
 void fuse_shared_w4a16(module& m)
@@ -651,6 +653,40 @@ void fuse_shared_w4a16(module& m)
                                   {all});
             at += cols;
         }
+    }
+}
+
+// ---- one-row weight-only products over constant weights -> the reordered form -------------------
+//
+// With one row of activations the product is a stream of weights, and constant weights can lie in
+// memory in whatever order the kernel reads fastest.  mi355::w4a16_prepack writes that order; its
+// operands are literals, so it runs once when the program is compiled (constant folding, below)
+// and the program keeps only the reordered copy.  Taken: one zero point for the tensor, group size
+// 128 and the shapes mi355_w4a16_prepacked_size accepts; everything else stays on mi355::w4a16_gemm.
+void prepack_w4a16(module& m)
+{
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "mi355::w4a16_gemm")
+            continue;
+        const auto op = any_cast<w4a16_gemm>(ins->get_operator());
+        auto a        = ins->inputs()[0];
+        auto w        = ins->inputs()[1];
+        auto s        = ins->inputs()[2];
+        if(op.zp_mode != MI355_W4_ZP_SCALAR or op.group != 128 or a->get_shape().lens()[0] != 1)
+            continue;
+        if(not(w->can_eval() and w->get_shape().standard() and s->can_eval() and s->get_shape().standard()))
+            continue;
+        const auto n       = static_cast<int64_t>(w->get_shape().lens()[0]);
+        const auto k       = static_cast<int64_t>(w->get_shape().lens()[1] * 2);
+        const size_t bytes = mi355_w4a16_prepacked_size(n, k, op.group);
+        if(bytes == 0)
+            continue;
+        w4a16_prepack pre;
+        pre.zp_scalar = op.zp_scalar;
+        auto room     = insert_allocation(m, ins, shape{shape::uint8_type, {bytes}});
+        auto packed   = m.insert_instruction(ins, operation{pre}, w, s, room);
+        m.replace_instruction(ins, operation{w4a16_gemm_prepacked{}}, a, packed, ins->inputs().back());
     }
 }
 
@@ -1317,6 +1353,8 @@ void lowering::apply(module& m) const
     }
     dead_code_elimination{}.apply(m);
     fuse_shared_w4a16(m);
+    dead_code_elimination{}.apply(m);
+    prepack_w4a16(m);
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)
     {

@@ -750,6 +750,66 @@ argument w4a16_gemm::compute(migraphx::context& ctx, const shape& out, const std
     return args.back();
 }
 
+shape w4a16_prepack::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    const auto& w = inputs[0];
+    const auto& s = inputs[1];
+    if(w.type() != shape::uint8_type or s.type() != shape::half_type or w.ndim() != 2 or not w.standard() or
+       not s.standard())
+        MIGRAPHX_THROW("mi355::w4a16_prepack: needs dense uint8 [N, K/2] weights and half scales");
+    const auto n       = static_cast<int64_t>(w.lens()[0]);
+    const auto k       = static_cast<int64_t>(w.lens()[1] * 2);
+    const size_t bytes = mi355_w4a16_prepacked_size(n, k, 128);
+    if(bytes == 0 or s.elements() != static_cast<std::size_t>(n * (k / 128)))
+        MIGRAPHX_THROW("mi355::w4a16_prepack: the reordered form does not take this shape");
+    shape out{shape::uint8_type, {bytes}};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::w4a16_prepack: output buffer has the wrong size");
+    return out;
+}
+
+argument w4a16_prepack::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto& w = args[0].get_shape();
+    status_check(mi355_w4a16_prepack(args[0].data(),
+                                     args[1].data(),
+                                     static_cast<int32_t>(zp_scalar),
+                                     static_cast<int64_t>(w.lens()[0]),
+                                     static_cast<int64_t>(w.lens()[1] * 2),
+                                     128,
+                                     args.back().data(),
+                                     stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+shape w4a16_gemm_prepacked::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    const auto& a   = inputs[0];
+    const auto& out = inputs.back();
+    if(a.type() != shape::half_type or out.type() != shape::half_type or inputs[1].type() != shape::uint8_type)
+        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: needs half activations and a uint8 buffer of reordered weights");
+    if(a.ndim() != 2 or out.ndim() != 2 or a.lens()[0] != 1 or out.lens()[0] != 1 or not out.standard())
+        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: takes one row of activations");
+    if(mi355_w4a16_prepacked_size(static_cast<int64_t>(out.lens()[1]), static_cast<int64_t>(a.lens()[1]), 128) !=
+       inputs[1].bytes())
+        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: the reordered weights do not fit the operands");
+    return out;
+}
+
+argument
+w4a16_gemm_prepacked::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const auto k = static_cast<int64_t>(args[0].get_shape().lens()[1]);
+    const auto n = static_cast<int64_t>(out.lens()[1]);
+    status_check(
+        mi355_w4a16_gemm_prepacked(args[0].data(), k, args[1].data(), args.back().data(), n, 1, n, k, stream_of(ctx)),
+        name());
+    return args.back();
+}
+
 // ----------------------------------------------------------------- pointwise operators
 
 shape quantizelinear::compute_shape(const std::vector<shape>& inputs) const
@@ -1286,6 +1346,8 @@ MIGRAPHX_REGISTER_OP(mi355::rowsum);
 MIGRAPHX_REGISTER_OP(mi355::dot);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot_mx);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
+MIGRAPHX_REGISTER_OP(mi355::w4a16_prepack);
+MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm_prepacked);
 MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::chain);

@@ -738,9 +738,24 @@ TEST_CASE(int4_weight_only_gemv)
         expect_close_half(p, {{"a", a}});
         program c = p;
         c.compile(migraphx::make_target("mi355"));
-        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+        // constant weights of a shape the reordered form takes (N % 16 == 0, K % 512 == 0) are
+        // reordered when the program is compiled; the program keeps the reordered copy only
+        const bool reordered = kn.second % 16 == 0 and kn.first % 512 == 0;
+        EXPECT(count_ops(*c.get_main_module(), reordered ? "mi355::w4a16_gemm_prepacked" : "mi355::w4a16_gemm") == 1);
+        EXPECT(not has_op(c, "mi355::w4a16_prepack"));
         EXPECT(not has_op(c, "mi355::dequantizelinear") and not has_op(c, "mi355::unpack_int4") and
                not has_op(c, "mi355::dot"));
+        if(reordered)
+        {
+            EXPECT(count_ops(*c.get_main_module(), "mi355::literal") == 1);
+            auto t  = migraphx::make_target("mi355");
+            auto r1 = c.eval({{"a", t.copy_to(a)}});
+            c.finish();
+            auto loaded = migraphx::load_buffer(migraphx::save_buffer(c));
+            auto r2     = loaded.eval({{"a", t.copy_to(a)}});
+            loaded.finish();
+            EXPECT(same_bytes(t.copy_from(r1[0]), t.copy_from(r2[0])));
+        }
     }
 }
 
@@ -772,7 +787,9 @@ TEST_CASE(int4_projections_sharing_activations)
         argument a{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 69)};
         program c = all;
         c.compile(migraphx::make_target("mi355"));
-        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+        // (one row of activations: the stacked constant weights are reordered at compile time)
+        EXPECT(count_ops(*c.get_main_module(), m == 1 ? "mi355::w4a16_gemm_prepacked" : "mi355::w4a16_gemm") == 1);
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") + count_ops(*c.get_main_module(), "mi355::w4a16_gemm_prepacked") == 1);
         auto got = run_on("mi355", all, {{"a", a}});
         EXPECT(got.size() == ns.size());
         for(std::size_t i = 0; i < ns.size(); i++)

@@ -48,7 +48,7 @@ def _dequantized(wq, scales, zp):
 
 
 @pytest.mark.parametrize("n,k", [(16, 512), (64, 1024), (512, 4096), (272, 3584), (256, 14336), (48, 28672),
-                                 (17600, 1536)])
+                                 (17600, 1536), (6160, 4096)])
 @pytest.mark.parametrize("zp", [8, 0, 3])
 def test_prepacked_gemv_matches_oracle(ops, n, k, zp):
     """Row groups x blocks of every launch shape: one block per wave, several blocks per wave,
