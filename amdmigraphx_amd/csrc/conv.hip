@@ -1281,6 +1281,10 @@ int64_t direct_ogp(const mi355_quant_conv3d_desc* d)
 
 // The direct kernel's form of a layer: one group, or every group a multiple of 16 channels; every
 // window inside the padded volume, counts that fit the kernels' 32-bit indices.
+// fp8 layers with padding are taken like any other.  The kernel multiplies the zero border of the
+// padded copy by the weights, where the reference (op/convolution.hpp:84-92) leaves window elements
+// outside the image out of the sum: the same number unless a weight is NaN, which then reaches the
+// border outputs as well (0 * NaN); the gathered form does the same, the vector-ALU forms mask.
 bool direct_form(const mi355_quant_conv3d_desc* d, const int64_t* ol)
 {
     const int64_t lim    = (int64_t)1 << 31;

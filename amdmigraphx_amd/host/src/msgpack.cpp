@@ -246,7 +246,13 @@ struct reader
         case 0xcc: return value(static_cast<int64_t>(be(1)));
         case 0xcd: return value(static_cast<int64_t>(be(2)));
         case 0xce: return value(static_cast<int64_t>(be(4)));
-        case 0xcf: return value(static_cast<int64_t>(be(8)));
+        case 0xcf: {
+            // `value` holds signed 64-bit integers only: a larger unsigned number would read back negative
+            const uint64_t u = be(8);
+            if(u > static_cast<uint64_t>(INT64_MAX))
+                MIGRAPHX_THROW("msgpack: unsigned integer above the signed 64-bit range");
+            return value(static_cast<int64_t>(u));
+        }
         case 0xd0: return value(sign_extend<int8_t>(be(1)));
         case 0xd1: return value(sign_extend<int16_t>(be(2)));
         case 0xd2: return value(sign_extend<int32_t>(be(4)));

@@ -613,7 +613,14 @@ void fuse_shared_w4a16(module& m)
                 continue;
             members.push_back(other);
         }
-        if(members.size() < 2)
+        // Each member's result becomes a column slice of the stacked one, a view whose rows start
+        // at the member's first column: a kernel that takes such a view as its activations reads 16
+        // bytes at a time, so every member's column count must keep the slices 16-byte aligned.
+        members.erase(std::remove_if(members.begin() + 1,
+                                     members.end(),
+                                     [](instruction_ref g) { return g->inputs()[1]->get_shape().lens()[0] % 8 != 0; }),
+                      members.end());
+        if(members.size() < 2 or first->inputs()[1]->get_shape().lens()[0] % 8 != 0)
             continue;
         std::size_t n = 0;
         std::string weights, scales;

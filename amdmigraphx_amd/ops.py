@@ -141,13 +141,14 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     return out
 
 
-def quant_dot_mx(a, b_nk, scale_a, scale_b, a_fp4=False, b_fp4=False, out=None):
+def quant_dot_mx(a, b_nk, scale_a, scale_b, a_fp4=False, b_fp4=False, out=None, workspace=None):
     """Four-input quant_dot of block-scaled operands: C = (float(A) * SA) . (float(B) * SB)^T.
 
     ``a`` [..., M, K] and ``b_nk`` [..., N, K] are uint8 tensors of e4m3fn codes, or with
     ``a_fp4`` / ``b_fp4`` of packed e2m1 pairs ([..., M, K/2], low nibble = even k).  The scales are
     float32, either of the operand's logical shape ([..., M, K], the operator's form) or compact
-    ([..., M, K/32], one per block).  Returns float32 [..., M, N]."""
+    ([..., M, K/32], one per block).  Returns float32 [..., M, N].  ``workspace``: a dense uint8
+    device tensor to use (and keep between calls) instead of a fresh allocation."""
     _require_cuda(a, b_nk, scale_a, scale_b)
     if a.dtype != torch.uint8 or b_nk.dtype != torch.uint8:
         raise Mi355Error("quant_dot_mx: operands are uint8 tensors of fp8 codes or packed fp4 pairs")
@@ -184,7 +185,9 @@ def quant_dot_mx(a, b_nk, scale_a, scale_b, a_fp4=False, b_fp4=False, out=None):
                   sb_batch=sbb, sb_row=sbr, sb_block=sbk, sb_elem=sbe,
                   a_type=DT.FP4X2 if a_fp4 else DT.FP8, b_type=DT.FP4X2 if b_fp4 else DT.FP8)
     need = int(lib().mi355_quant_dot_mx_workspace_size(ctypes.byref(d)))
-    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=a.device)
+    ws = workspace if workspace is not None else torch.empty(max(need, 16), dtype=torch.uint8, device=a.device)
+    if ws.numel() * ws.element_size() < need or not ws.is_contiguous():
+        raise Mi355Error("quant_dot_mx: the workspace is too small or not dense")
     check(lib().mi355_quant_dot_mx(ctypes.byref(d), _ptr(a), _ptr(b_nk), _ptr(out), _ptr(scale_a), _ptr(scale_b),
                                    _ptr(ws), need, _stream()), "mi355_quant_dot_mx")
     return out

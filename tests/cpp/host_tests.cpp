@@ -1242,6 +1242,9 @@ TEST_CASE(msgpack_reads_every_number_format)
     // a lone bin object (the older layout) and chunked binary both read as binary
     EXPECT(from_msgpack(bytes_of({0xc4, 2, 9, 8})).get_binary() == std::string("\x09\x08"));
     EXPECT(from_msgpack(bytes_of({0x92, 0xc4, 1, 9, 0xc5, 0, 1, 8})).get_binary() == std::string("\x09\x08"));
+    // unsigned 64-bit: up to the signed range; above it the reader refuses instead of wrapping negative
+    EXPECT(from_msgpack(bytes_of({0xcf, 0x7f, 0xff, 0xff, 0xff, 0xff, 0xff, 0xff, 0xff})).to<int64_t>() == INT64_MAX);
+    EXPECT(test::throws([] { from_msgpack(bytes_of({0xcf, 0x80, 0, 0, 0, 0, 0, 0, 0})); }));
     EXPECT(test::throws([] { from_msgpack(bytes_of({0xc7, 1, 1, 0})); }));       // ext
     EXPECT(test::throws([] { from_msgpack(bytes_of({0xa5, 'a', 'b'})); }));      // truncated
     EXPECT(test::throws([] { from_msgpack(bytes_of({0x93, 1, 2})); }));          // truncated array

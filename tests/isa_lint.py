@@ -87,3 +87,66 @@ def scan(path, only=None):
                                    f"{left} wait states early (MFMA at line {at})")
             pending = [(r, w - states, n) for (r, w, n) in pending if w - states > 0]
     return seen, hazards
+
+
+def scan_assembly_loads(path, only=None):
+    """The second hazard of this kind: vector-memory loads issued from inline assembly.
+
+    The int4 GEMV over reordered weights issues its global loads as assembly statements and waits
+    for them with counted ``s_waitcnt vmcnt(N)`` statements of its own; the compiler believes a
+    load's destination registers hold their value from the load on and may copy them
+    (``v_mov``) before the wait, which reads whatever the registers held before.  For every
+    ``global_load`` inside an inline-assembly region this scan follows the stream in layout order and
+    reports any instruction that names one of its destination registers before a
+    ``s_waitcnt vmcnt(N)`` with N at most the number of assembly loads issued since (a wave's loads
+    return in order).  A load into the same registers ends the watch as well.  Branches are not
+    followed.  Returns (loads seen, hazards)."""
+    hazards, seen = [], 0
+    kernel, in_asm, pending = None, False, []   # pending: [registers, loads issued behind, line]
+    with open(path) as f:
+        for number, raw in enumerate(f, 1):
+            text = raw.strip()
+            if text.startswith(";;#ASMSTART"):
+                in_asm = True
+                continue
+            if text.startswith(";;#ASMEND"):
+                in_asm = False
+                continue
+            label = _LABEL.match(text)
+            if label:
+                kernel, pending = label.group(1), []
+                continue
+            if not text or text[0] in ".;":
+                continue
+            if only is not None and (kernel is None or only not in kernel):
+                continue
+            text = text.split(";")[0].strip()
+            parts = text.replace(",", " ").split()
+            op, operands = parts[0], parts[1:]
+            if op == "s_waitcnt":
+                m = re.search(r"vmcnt\((\d+)\)", text)
+                if m:
+                    pending = [p for p in pending if p[1] < int(m.group(1))]
+                continue
+            if op == "s_endpgm":
+                pending = []
+                continue
+            touched = set()
+            for token in operands:
+                touched |= _acc_regs(token)
+            is_load = op.startswith("global_load") or op.startswith("buffer_load") or op.startswith("scratch_load")
+            dest = _acc_regs(operands[0]) if is_load and operands else set()
+            for regs, behind, at in pending:
+                hit = (touched - dest) & regs if is_load else touched & regs
+                if hit:
+                    first = min(hit)
+                    hazards.append(f"{kernel}: line {number} `{text}` names {first[0]}{first[1]} before the load "
+                                   f"at line {at} has been waited for")
+            if is_load:
+                pending = [p for p in pending if not (p[0] & dest)]
+                for p in pending:
+                    p[1] += 1
+                if in_asm:
+                    seen += 1
+                    pending.append([dest, 0, number])
+    return seen, hazards

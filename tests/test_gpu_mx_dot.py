@@ -242,6 +242,30 @@ def test_general_scales_take_the_exact_path(ops, kind):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_good_scales_after_flagged_ones_in_one_workspace(ops):
+    """The workspace word that marks "this call's scales need the exact path" is never cleared; every
+    eager call writes and compares its own number.  A call with power-of-two scales that follows a
+    flagged call in the same workspace must therefore be back on the matrix cores: it gives the bits
+    of the same call in a fresh workspace (the exact path would give the oracle's bits instead, which
+    differ from the matrix cores' in the last places on these operands)."""
+    rng = np.random.default_rng(12)
+    m, n, k = 96, 80, 512
+    a = orc.fp8_from_f32(rng.normal(0, 1.0, (m, k)).astype(np.float32))
+    b = orc.fp8_from_f32(rng.normal(0, 1.0, (n, k)).astype(np.float32))
+    sa, sb = _block_scales(rng, (m,), k), _block_scales(rng, (n,), k)
+    bad = sb.copy()
+    bad[3, 1] = 0.3
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    fresh = ops.quant_dot_mx(dev(a), dev(b), dev(sa), dev(sb)).cpu().numpy()
+    exact = ops.quant_dot_mx(dev(a), dev(b), dev(sa), dev(bad), workspace=ws).cpu().numpy()
+    want_bad = _reference(orc.fp8_to_f32(a), orc.fp8_to_f32(b), np.repeat(sa, 32, axis=1), np.repeat(bad, 32, axis=1))
+    assert np.array_equal(exact.view(np.uint32), want_bad.view(np.uint32))
+    again = ops.quant_dot_mx(dev(a), dev(b), dev(sa), dev(sb), workspace=ws).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), fresh.view(np.uint32))
+    want = _reference(orc.fp8_to_f32(a), orc.fp8_to_f32(b), np.repeat(sa, 32, axis=1), np.repeat(sb, 32, axis=1))
+    assert not np.array_equal(fresh.view(np.uint32), want.view(np.uint32)), "operands too tame to tell the paths apart"
+
+
 def test_argument_errors(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((4, 48), dtype=torch.uint8, device="cuda")      # K = 48: not whole blocks

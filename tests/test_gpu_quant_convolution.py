@@ -417,3 +417,28 @@ def test_caller_provided_result_and_workspace(ops):
         ops.quant_convolution(dev(x), dev(w), (1, 1), workspace=torch.empty(8, dtype=torch.uint8, device="cuda"))
     with pytest.raises(Exception):
         ops.quant_convolution(dev(x), dev(w), (1, 1), out=torch.empty((2, 16, 9, 8), dtype=torch.int32, device="cuda"))
+
+
+@pytest.mark.parametrize("xs,ws,group", [((2, 32, 12, 12), (24, 32, 3, 3), 1),      # direct kernel
+                                         ((1, 20, 9, 9), (8, 10, 3, 3), 2)])       # gathered form (10 channels per group)
+def test_fp8_nan_weight_on_zero_padded_forms(ops, xs, ws, group):
+    """A NaN weight in an fp8 layer with padding.  The reference skips window elements outside the image, so
+    the NaN spoils only outputs whose window has that element inside; the forms that work on a zero-padded
+    copy (direct kernel, gathered form) also return NaN where the element falls on the border (0 * NaN).
+    Pinned here: interior outputs agree with the oracle exactly, NaN included; border outputs are either the
+    oracle's value or NaN, and every other output channel is untouched."""
+    rng = np.random.default_rng(sum(xs) + sum(ws))
+    xi = rng.integers(-3, 4, xs).astype(np.float32)
+    wi = rng.integers(-2, 3, ws).astype(np.float32)
+    wc = orc.fp8_from_f32(wi)
+    wc[1, 0, 0, 0] = 0x7F
+    wn = wi.copy()
+    wn[1, 0, 0, 0] = np.nan
+    got = ops.quant_convolution(dev(orc.fp8_from_f32(xi)), dev(wc), (1, 1), (1, 1), (1, 1), group, fp8=True).cpu().numpy()
+    want = orc.convolution(xi, wn, orc.F32, (1, 1), (1, 1), (1, 1), group)
+    assert np.isnan(want[:, 1, 1:, 1:]).all() and not np.isnan(want[:, 1, 0, :]).any()
+    assert np.array_equal(got[:, :, 1:, 1:], want[:, :, 1:, 1:], equal_nan=True)
+    others = [o for o in range(ws[0]) if o != 1]
+    assert np.array_equal(got[:, others], want[:, others])
+    border = got[:, 1, 0, :]
+    assert (np.isnan(border) | (border == want[:, 1, 0, :])).all()

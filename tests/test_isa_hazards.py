@@ -39,6 +39,36 @@ _Z6samplev:
     assert len(hazards) == 1 and "a1" in hazards[0]
 
 
+def test_lint_finds_a_copy_of_a_loaded_register_in_front_of_its_wait(tmp_path):
+    listing = tmp_path / "loads.s"
+    listing.write_text("""
+_Z5loadsv:
+	;;#ASMSTART
+	global_load_ushort v9, v1, s[2:3] nt
+	;;#ASMEND
+	;;#ASMSTART
+	global_load_dwordx4 v[4:7], v0, s[2:3] offset:128 nt
+	;;#ASMEND
+	v_add_u32_e32 v8, 1, v0
+	v_mov_b32_e32 v10, v9
+	;;#ASMSTART
+	s_waitcnt vmcnt(1)
+	;;#ASMEND
+	v_and_b32_e32 v11, 15, v9
+	v_mov_b32_e32 v12, v5
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	v_mov_b32_e32 v13, v5
+	s_endpgm
+""")
+    seen, hazards = isa_lint.scan_assembly_loads(str(listing))
+    # v9 is copied before its wait (vmcnt(1) covers it: one load behind it) and read properly after;
+    # v5 is read once before vmcnt(0) and once after
+    assert seen == 2
+    assert len(hazards) == 2 and "v9" in hazards[0] and "v5" in hazards[1]
+
+
 def _listing(tmp_path, source):
     out = tmp_path / (source + ".s")
     cmd = [HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"),
@@ -54,6 +84,14 @@ def test_direct_convolution_kernel_keeps_its_wait_states(tmp_path):
     # 16 MFMAs per K step body, 24 int8 instantiations (4 result types, vector stores or not, 3 ring
     # depths); the fp8 ones use the compiler's own MFMAs
     assert seen >= 16 * 24
+    assert hazards == [], hazards[:5]
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_reordered_int4_gemv_reads_no_load_before_its_wait(tmp_path):
+    seen, hazards = isa_lint.scan_assembly_loads(_listing(tmp_path, "w4a16_prepacked.hip"), only="w4p_gemv_kernel")
+    # per kernel: the activation loads and, in each of the two bodies, five loads per block
+    assert seen >= 24 * (1 + 2 * 5)
     assert hazards == [], hazards[:5]
 
 
