@@ -55,6 +55,56 @@ struct allocate
     argument compute(migraphx::context&, const shape&, const std::vector<argument>&) const;
 };
 
+// One block of device memory that holds the program's intermediate buffers (memory_coloring).
+struct arena
+{
+    std::size_t bytes = 0;
+    argument buffer; // set by finalize
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.bytes, "bytes");
+    }
+    std::string name() const { return "mi355::arena"; }
+    shape compute_shape(const std::vector<shape>&) const { return shape{shape::uint8_type, {bytes}}; }
+    void finalize(migraphx::context&, const shape&, const std::vector<shape>&)
+    {
+        if(buffer.empty())
+            buffer = allocate_device(shape{shape::uint8_type, {bytes}});
+    }
+    argument compute(migraphx::context&, const shape&, const std::vector<argument>&) const;
+};
+
+// A buffer at a fixed place of the arena.  inputs: the arena
+struct load
+{
+    shape s;
+    std::size_t offset = 0;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.s, "shape");
+        f(self.offset, "offset");
+    }
+    std::string name() const { return "mi355::load"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context&, const shape&, const std::vector<argument>& args) const
+    {
+        return args.front().offset(offset, s);
+    }
+};
+
+// Buffer reuse (the counterpart of src/memory_coloring.cpp with "mi355::allocate" as the allocation
+// operator): every mi355::allocate of the lowered program lives from the instruction that writes
+// it to the last instruction that reads it or a view of it; allocations whose lives do not overlap
+// share memory.  All of them become mi355::load at fixed offsets of one mi355::arena, allocated
+// once when the program is finalized.
+struct memory_coloring
+{
+    std::string name() const { return "mi355::memory_coloring"; }
+    void apply(module& m) const;
+};
+
 struct device_literal
 {
     argument data;

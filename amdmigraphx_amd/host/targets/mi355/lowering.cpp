@@ -1414,5 +1414,123 @@ void lowering::apply(module& m) const
     fold_constants(m, *ctx);
 }
 
+// ---- buffer reuse -------------------------------------------------------------------------------
+
+void memory_coloring::apply(module& m) const
+{
+    const auto order = all_instructions(m);
+    std::unordered_map<const instruction*, int> index;
+    for(std::size_t i = 0; i < order.size(); i++)
+        index[&*order[i]] = static_cast<int>(i);
+    // the allocation an instruction's result lives in: its own (mi355::allocate), or that of the
+    // argument it returns (device operators return their output buffer, views their input)
+    std::unordered_map<const instruction*, const instruction*> root;
+    struct life
+    {
+        instruction_ref ins;
+        int first = -1, last = -1;
+        std::size_t bytes = 0, offset = 0;
+    };
+    std::unordered_map<const instruction*, life> lives;
+    const int forever = static_cast<int>(order.size());
+    auto touch        = [&](const instruction* r, int at) {
+        auto& l = lives.at(r);
+        l.first = l.first < 0 ? at : std::min(l.first, at);
+        l.last  = std::max(l.last, at);
+    };
+    for(std::size_t i = 0; i < order.size(); i++)
+    {
+        auto ins        = order[i];
+        const auto name = ins->name();
+        if(name == "mi355::allocate")
+        {
+            root[&*ins]  = &*ins;
+            lives[&*ins] = life{ins, -1, -1, (std::max<std::size_t>(ins->get_shape().bytes(), 16) + 255) / 256 * 256, 0};
+            continue;
+        }
+        std::vector<shape> in_shapes;
+        for(auto x : ins->inputs())
+            in_shapes.push_back(x->get_shape());
+        const auto alias = ins->inputs().empty() ? -1 : ins->get_operator().output_alias(in_shapes);
+        const instruction* mine = nullptr;
+        if(alias >= 0 and alias < static_cast<std::ptrdiff_t>(ins->inputs().size()))
+        {
+            auto it = root.find(&*ins->inputs()[alias]);
+            mine    = it == root.end() ? nullptr : it->second;
+        }
+        root[&*ins] = mine;
+        // results of the program, and arguments of anything that is neither a device operator nor a
+        // view (it may hand its argument on without saying so), stay for good
+        const bool known = name.rfind("mi355::", 0) == 0 or (alias >= 0 and ins->get_operator().is_context_free());
+        const int until  = (name == "@return" or not known) ? forever : static_cast<int>(i);
+        for(auto x : ins->inputs())
+        {
+            auto it = root.find(&*x);
+            if(it != root.end() and it->second != nullptr)
+                touch(it->second, until);
+        }
+        // (a use marks the allocation from its own position on, whatever `until` says)
+        for(auto x : ins->inputs())
+        {
+            auto it = root.find(&*x);
+            if(it != root.end() and it->second != nullptr)
+                lives.at(it->second).first = std::min(lives.at(it->second).first, static_cast<int>(i));
+        }
+    }
+    if(not order.empty() and order.back()->name() != "@return")
+    {
+        auto it = root.find(&*order.back());
+        if(it != root.end() and it->second != nullptr)
+            touch(it->second, forever);
+    }
+    std::vector<life*> todo;
+    for(auto& kv : lives)
+    {
+        if(kv.second.first < 0) // never used: dead code elimination's business
+            kv.second.first = kv.second.last = index.at(kv.first);
+        todo.push_back(&kv.second);
+    }
+    if(todo.empty())
+        return;
+    // largest first, each at the lowest offset that is free for the whole of its life
+    std::sort(todo.begin(), todo.end(), [&](const life* a, const life* b) {
+        if(a->bytes != b->bytes)
+            return a->bytes > b->bytes;
+        return index.at(&*a->ins) < index.at(&*b->ins);
+    });
+    std::vector<life*> placed;
+    std::size_t total = 0;
+    for(auto* l : todo)
+    {
+        std::vector<std::pair<std::size_t, std::size_t>> busy;
+        for(auto* o : placed)
+        {
+            if(o->first <= l->last and l->first <= o->last)
+                busy.emplace_back(o->offset, o->offset + o->bytes);
+        }
+        std::sort(busy.begin(), busy.end());
+        std::size_t at = 0;
+        for(const auto& b : busy)
+        {
+            if(at + l->bytes <= b.first)
+                break;
+            at = std::max(at, b.second);
+        }
+        l->offset = at;
+        total     = std::max(total, at + l->bytes);
+        placed.push_back(l);
+    }
+    arena whole;
+    whole.bytes = total;
+    auto block  = m.insert_instruction(m.begin(), operation{whole});
+    for(auto* l : placed)
+    {
+        load at;
+        at.s      = l->ins->get_shape();
+        at.offset = l->offset;
+        m.replace_instruction(l->ins, operation{at}, std::vector<instruction_ref>{block});
+    }
+}
+
 } // namespace mi355
 } // namespace migraphx

@@ -197,6 +197,21 @@ argument allocate::compute(migraphx::context&, const shape&, const std::vector<a
     return buffer;
 }
 
+argument arena::compute(migraphx::context&, const shape&, const std::vector<argument>&) const
+{
+    if(buffer.empty())
+        MIGRAPHX_THROW("mi355::arena: evaluated before finalize");
+    return buffer;
+}
+
+shape load::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 1, name());
+    if(offset + s.bytes() > inputs.front().bytes())
+        MIGRAPHX_THROW("mi355::load: reaches past the end of the arena");
+    return s;
+}
+
 value device_literal::to_value() const
 {
     // the key is always there: make_op checks attribute names against a default instance
@@ -1330,12 +1345,20 @@ std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_opti
     // the reference's switch for its pointwise fusion (src/fuse_pointwise.cpp:39,369)
     if(const char* off = std::getenv("MIGRAPHX_DISABLE_POINTWISE_FUSION"))
         low.fuse_pointwise = std::string(off).empty() or std::string(off) == "0";
-    return {sq, dead_code_elimination{}, low, dead_code_elimination{}};
+    // MIGRAPHX_MI355_DISABLE_MEMORY_COLORING: every intermediate buffer keeps an allocation of its own
+    if(const char* off = std::getenv("MIGRAPHX_MI355_DISABLE_MEMORY_COLORING"))
+    {
+        if(not std::string(off).empty() and std::string(off) != "0")
+            return {sq, dead_code_elimination{}, low, dead_code_elimination{}};
+    }
+    return {sq, dead_code_elimination{}, low, dead_code_elimination{}, memory_coloring{}};
 }
 
 } // namespace mi355
 
 MIGRAPHX_REGISTER_OP(mi355::allocate);
+MIGRAPHX_REGISTER_OP(mi355::arena);
+MIGRAPHX_REGISTER_OP(mi355::load);
 MIGRAPHX_REGISTER_OP(mi355::device_literal);
 MIGRAPHX_REGISTER_OP(mi355::copy_to_device);
 MIGRAPHX_REGISTER_OP(mi355::copy_from_device);

@@ -1209,6 +1209,63 @@ TEST_CASE(float_operators)
     expect_same(p, {{"i", ia}});
 }
 
+TEST_CASE(intermediate_buffers_share_one_arena)
+{
+    // memory_coloring: the buffers of a compiled program are places in one block of device memory,
+    // shared by buffers whose lives do not overlap.  A long chain of matrix products (each needs
+    // the one before it only) must come out the size of a few buffers, not of all of them; an early
+    // result that is returned must survive everything computed after it; a view of a buffer keeps
+    // the buffer alive; and the results are those of the program with a buffer per instruction.
+    const std::size_t n = 96;
+    program p;
+    auto* mm = p.get_main_module();
+    shape s{shape::float_type, {n, n}};
+    auto x     = mm->add_parameter("x", s);
+    auto w     = mm->add_literal(literal{s, normal_floats(n * n, 0.1f, 901)});
+    auto early = mm->add_instruction(make_op("dot"), x, w);
+    auto early_t = mm->add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), early);
+    auto y     = early;
+    for(int i = 0; i < 12; i++)
+        y = mm->add_instruction(make_op("dot"), y, w);
+    auto late = mm->add_instruction(make_op("dot"), early_t, y); // the view of `early`, read at the end
+    mm->add_return({early, y, late});
+    argument xa{s, normal_floats(n * n, 1.0f, 902)};
+
+    program colored = p;
+    colored.compile(migraphx::make_target("mi355"));
+    const auto& mod = *colored.get_main_module();
+    EXPECT(count_ops(mod, "mi355::arena") == 1 and count_ops(mod, "mi355::allocate") == 0);
+    EXPECT(count_ops(mod, "mi355::load") >= 14);
+    std::size_t arena_bytes = 0;
+    for(auto ins = mod.begin(); ins != mod.end(); ++ins)
+        if(ins->name() == "mi355::arena")
+            arena_bytes = ins->get_shape().bytes();
+    // 14 products of 36 KiB: `early`, the two last results and one or two buffers in rotation
+    EXPECT(arena_bytes >= 3 * n * n * 4 and arena_bytes <= 6 * n * n * 4);
+
+    auto got = run_on("mi355", p, {{"x", xa}});
+    setenv("MIGRAPHX_MI355_DISABLE_MEMORY_COLORING", "1", 1);
+    program plain = p;
+    plain.compile(migraphx::make_target("mi355"));
+    auto want = run_on("mi355", p, {{"x", xa}});
+    unsetenv("MIGRAPHX_MI355_DISABLE_MEMORY_COLORING");
+    EXPECT(count_ops(*plain.get_main_module(), "mi355::arena") == 0 and
+           count_ops(*plain.get_main_module(), "mi355::allocate") >= 14);
+    EXPECT(got.size() == 3 and want.size() == 3);
+    for(std::size_t i = 0; i < 3; i++)
+        EXPECT(same_bytes(got[i], want[i]));
+    auto cpu = run_on("oracle", p, {{"x", xa}});
+    for(std::size_t i = 0; i < 3; i++)
+        EXPECT(same_bytes(got[i], cpu[i]));
+    // a saved and reloaded program keeps its places
+    auto loaded = migraphx::load_buffer(migraphx::save_buffer(colored));
+    auto t      = migraphx::make_target("mi355");
+    auto again  = loaded.eval({{"x", t.copy_to(xa)}});
+    loaded.finish();
+    for(std::size_t i = 0; i < 3; i++)
+        EXPECT(same_bytes(t.copy_from(again[i]), got[i]));
+}
+
 TEST_CASE(pointwise_chains)
 {
     // Chains of float operators become one mi355::chain each.  With IEEE-exact operators the fused
@@ -1584,6 +1641,21 @@ static int encoder_bench(int argc, char** argv)
     p.compile(t);
     std::cout << "quantized MatMul launches per forward: "
               << count_ops(*p.get_main_module(), "mi355::quant_dot") << std::endl;
+    {
+        std::size_t arena = 0, separate = 0, buffers = 0;
+        for(auto ins = p.get_main_module()->begin(); ins != p.get_main_module()->end(); ++ins)
+        {
+            if(ins->name() == "mi355::arena")
+                arena = ins->get_shape().bytes();
+            if(ins->name() == "mi355::load" or ins->name() == "mi355::allocate")
+            {
+                separate += ins->get_shape().bytes();
+                buffers++;
+            }
+        }
+        std::cout << "intermediate buffers: " << buffers << " of " << separate / 1048576.0 << " MiB in all, arena "
+                  << arena / 1048576.0 << " MiB" << std::endl;
+    }
     auto dids = t.copy_to(ids);
     for(int i = 0; i < 2; i++)
         p.eval({{"ids", dids}});
