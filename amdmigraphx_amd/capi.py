@@ -15,7 +15,7 @@ class Mi355Error(RuntimeError):
 
 
 class DT:
-    I8, U8, I32, F32, F16, BF16, FP8, FP4X2 = range(8)
+    I8, U8, I32, F32, F16, BF16, FP8, FP4X2, BF8 = range(9)   # FP8: OCP e4m3fn, BF8: OCP e5m2
 
 
 class QP:

@@ -24,7 +24,8 @@ static inline size_t mi355_dtype_size(int t)
     {
     case MI355_I8:
     case MI355_U8:
-    case MI355_FP8: return 1;
+    case MI355_FP8:
+    case MI355_BF8: return 1;
     case MI355_F16:
     case MI355_BF16: return 2;
     case MI355_I32:
@@ -90,6 +91,20 @@ MI355_DEVINL uint8_t f32_to_fp8_rne(float x)
     return (uint8_t)(r & 0xff);
 }
 
+// OCP e5m2 decode (float8_impl.hpp:249-325 with Wm = 2, We = 5): an e5m2 code is the upper byte
+// of the half with the same value, infinities and NaN included.
+MI355_DEVINL float bf8_to_f32(uint8_t v)
+{
+    return half_to_f32((uint16_t)((uint32_t)v << 8));
+}
+
+// float -> e5m2, nearest even.  The caller has clamped to [-57344, 57344], as for e4m3fn above.
+MI355_DEVINL uint8_t f32_to_bf8_rne(float x)
+{
+    int r = __builtin_amdgcn_cvt_pk_bf8_f32(x, 0.0f, 0, false);
+    return (uint8_t)(r & 0xff);
+}
+
 // `convert` op (op/convert.hpp:64-87) from float to a 16-bit float type.
 MI355_DEVINL uint16_t convert_f32_to_half(float x)
 {
@@ -144,6 +159,7 @@ MI355_DEVINL double load_as_f64(const void* p, int type, int64_t i)
     case MI355_F16: return (double)half_to_f32(((const uint16_t*)p)[i]);
     case MI355_BF16: return (double)bf16_to_f32(((const uint16_t*)p)[i]);
     case MI355_FP8: return (double)fp8_to_f32(((const uint8_t*)p)[i]);
+    case MI355_BF8: return (double)bf8_to_f32(((const uint8_t*)p)[i]);
     default: return 0.0;
     }
 }

@@ -74,6 +74,14 @@ __global__ __launch_bounds__(PW_THREADS) void quantizelinear_kernel(
             double v = clamp_like_ref((double)xv / (double)sv + z, -448.0, 448.0);
             res[e]   = f32_to_fp8_rne((float)v);
         }
+        else if constexpr(OT == MI355_BF8)
+        {
+            double z = 0.0;
+            if(q.zp != nullptr)
+                z = (double)bf8_to_f32(static_cast<const uint8_t*>(q.zp)[r * q.z_sr + c * q.z_sc]);
+            double v = clamp_like_ref((double)xv / (double)sv + z, -57344.0, 57344.0);
+            res[e]   = f32_to_bf8_rne((float)v);
+        }
         else
         {
             double z = 0.0;
@@ -288,6 +296,15 @@ __global__ __launch_bounds__(PW_THREADS) void convert_kernel(
             static_cast<uint8_t*>(out)[i] =
                 f32_to_fp8_rne((float)fmin(448.0, fmax(-448.0, dx)));
         break;
+    case MI355_BF8:
+        // numeric_limits<fp8e5m2>::quiet_NaN() is 0xff (float8.hpp:364); infinities go through
+        // the clipping constructor
+        if(dx != dx)
+            static_cast<uint8_t*>(out)[i] = 0xff;
+        else
+            static_cast<uint8_t*>(out)[i] =
+                f32_to_bf8_rne((float)fmin(57344.0, fmax(-57344.0, dx)));
+        break;
     default: break;
     }
 }
@@ -316,6 +333,10 @@ int launch_quantize(int out_type,
         break;
     case MI355_FP8:
         hipLaunchKernelGGL((quantizelinear_kernel<XT, MI355_FP8>), dim3(blocks_for(work)),
+                           dim3(PW_THREADS), 0, s, x, q, out, rows, cols);
+        break;
+    case MI355_BF8:
+        hipLaunchKernelGGL((quantizelinear_kernel<XT, MI355_BF8>), dim3(blocks_for(work)),
                            dim3(PW_THREADS), 0, s, x, q, out, rows, cols);
         break;
     default: return MI355_ERR_UNSUPPORTED;
@@ -387,7 +408,7 @@ extern "C" int mi355_dequantizelinear(const void* x,
     if(x == nullptr || scale == nullptr || out == nullptr || rows < 0 || cols < 0)
         return MI355_ERR_BAD_ARG;
     if(x_type != MI355_I8 && x_type != MI355_U8 && x_type != MI355_I32 && x_type != MI355_F32 &&
-       x_type != MI355_FP8)
+       x_type != MI355_FP8 && x_type != MI355_BF8)
         return MI355_ERR_UNSUPPORTED;
     if(scale_type != MI355_F32 && scale_type != MI355_F16 && scale_type != MI355_BF16)
         return MI355_ERR_UNSUPPORTED;
@@ -593,7 +614,7 @@ extern "C" int mi355_convert(
     if(mi355_dtype_size(in_type) == 0 || mi355_dtype_size(out_type) == 0)
         return MI355_ERR_BAD_ARG;
     if(out_type != MI355_F32 && out_type != MI355_F16 && out_type != MI355_BF16 &&
-       out_type != MI355_FP8)
+       out_type != MI355_FP8 && out_type != MI355_BF8)
         return MI355_ERR_UNSUPPORTED;
     if(n == 0)
         return MI355_OK;

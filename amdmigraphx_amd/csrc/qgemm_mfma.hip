@@ -138,13 +138,14 @@ MI355_DEVINL void store4(void* c, int64_t idx, const float v[4])
     }
 }
 
-// FP8: element type; TRANS_B: B stored [N, K]; DEQ: apply the epilogue;
-// OUT: output element type; KFULL: K is a multiple of the 128-byte slab, so no
+// FMT: element type (0 int8, 1 fp8 e4m3fn, 2 fp8 e5m2); TRANS_B: B stored [N, K]; DEQ: apply the
+// epilogue; OUT: output element type; KFULL: K is a multiple of the 128-byte slab, so no
 // load needs a bounds predicate (a predicate per load costs a branch each).
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
+template <int FMT, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
 __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr bool FP8 = FMT != 0;
     using acc_t  = typename acc_traits<FP8>::type;
     using frag_t = typename frag_traits<FP8>::type;
 
@@ -304,7 +305,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
             return read_frag(q + h * 64);
     };
     auto mfma = [&](const frag_t& a, const frag_t& b, acc_t c) -> acc_t {
-        if constexpr(FP8)
+        if constexpr(FMT == 2)
+            // cbsz = blgp = 1: e5m2 for both operands
+            return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 1, 1, 0, 0, 0, 0);
+        else if constexpr(FP8)
             // zero scale operands select the unscaled v_mfma_f32_16x16x128_f8f6f4;
             // cbsz = blgp = 0 means e4m3 for both operands
             return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
@@ -460,10 +464,10 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_mfma_kernel(gemm_params p)
     }
 }
 
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
+template <int FMT, bool TRANS_B, bool DEQ, int OUT, bool KFULL>
 int launch_k(const gemm_params& p, int batch, hipStream_t stream)
 {
-    auto kern = qgemm_mfma_kernel<FP8, TRANS_B, DEQ, OUT, KFULL>;
+    auto kern = qgemm_mfma_kernel<FMT, TRANS_B, DEQ, OUT, KFULL>;
     // above the 64 KiB default: opt in once per kernel instantiation
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -474,23 +478,23 @@ int launch_k(const gemm_params& p, int batch, hipStream_t stream)
     return mi355_launch_status();
 }
 
-template <bool FP8, bool TRANS_B, bool DEQ, int OUT>
+template <int FMT, bool TRANS_B, bool DEQ, int OUT>
 int launch_one(const gemm_params& p, int batch, hipStream_t stream)
 {
-    return p.k % BK == 0 ? launch_k<FP8, TRANS_B, DEQ, OUT, true>(p, batch, stream)
-                         : launch_k<FP8, TRANS_B, DEQ, OUT, false>(p, batch, stream);
+    return p.k % BK == 0 ? launch_k<FMT, TRANS_B, DEQ, OUT, true>(p, batch, stream)
+                         : launch_k<FMT, TRANS_B, DEQ, OUT, false>(p, batch, stream);
 }
 
-template <bool FP8, bool TRANS_B>
+template <int FMT, bool TRANS_B>
 int launch_out(const gemm_params& p, int batch, bool deq, int out, hipStream_t s)
 {
     if(!deq)
-        return launch_one<FP8, TRANS_B, false, MI355_F32>(p, batch, s);
+        return launch_one<FMT, TRANS_B, false, MI355_F32>(p, batch, s);
     switch(out)
     {
-    case MI355_F32: return launch_one<FP8, TRANS_B, true, MI355_F32>(p, batch, s);
-    case MI355_F16: return launch_one<FP8, TRANS_B, true, MI355_F16>(p, batch, s);
-    case MI355_BF16: return launch_one<FP8, TRANS_B, true, MI355_BF16>(p, batch, s);
+    case MI355_F32: return launch_one<FMT, TRANS_B, true, MI355_F32>(p, batch, s);
+    case MI355_F16: return launch_one<FMT, TRANS_B, true, MI355_F16>(p, batch, s);
+    case MI355_BF16: return launch_one<FMT, TRANS_B, true, MI355_BF16>(p, batch, s);
     default: return MI355_ERR_UNSUPPORTED;
     }
 }
@@ -573,11 +577,13 @@ int mi355_mfma_gemm_launch(const mi355_quant_dot_desc* d,
     p.scale_b_mode = d->scale_b_mode;
     p.zp_a         = d->zp_a;
     p.zp_b         = d->zp_b;
-    const bool fp8 = d->in_type == MI355_FP8;
     const bool deq = d->dequant != 0;
-    if(fp8)
-        return d->trans_b ? launch_out<true, true>(p, (int)d->batch, deq, d->out_type, stream)
-                          : launch_out<true, false>(p, (int)d->batch, deq, d->out_type, stream);
-    return d->trans_b ? launch_out<false, true>(p, (int)d->batch, deq, d->out_type, stream)
-                      : launch_out<false, false>(p, (int)d->batch, deq, d->out_type, stream);
+    if(d->in_type == MI355_BF8)
+        return d->trans_b ? launch_out<2, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_out<2, false>(p, (int)d->batch, deq, d->out_type, stream);
+    if(d->in_type == MI355_FP8)
+        return d->trans_b ? launch_out<1, true>(p, (int)d->batch, deq, d->out_type, stream)
+                          : launch_out<1, false>(p, (int)d->batch, deq, d->out_type, stream);
+    return d->trans_b ? launch_out<0, true>(p, (int)d->batch, deq, d->out_type, stream)
+                      : launch_out<0, false>(p, (int)d->batch, deq, d->out_type, stream);
 }

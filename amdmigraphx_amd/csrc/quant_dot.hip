@@ -47,9 +47,18 @@ struct generic_params
     const int32_t* rowsum_a;
     const float* bias;
     int scale_a_mode, scale_b_mode, zp_a, zp_b;
-    int fp8, dequant, out_type;
+    int fp8, dequant, out_type; // fp8: 0 integers, 1 e4m3fn, 2 e5m2
     int is_unsigned; // uint8 operands (bare quant_dot only)
 };
+
+MI355_DEVINL float decode_operand(uint8_t raw, const generic_params& p)
+{
+    if(p.fp8 == 1)
+        return fp8_to_f32(raw);
+    if(p.fp8 == 2)
+        return bf8_to_f32(raw);
+    return p.is_unsigned ? (float)raw : (float)(int8_t)raw;
+}
 
 // 16 x 16 outputs per workgroup, K walked in steps of 16 through LDS.  int8
 // accumulates in int32 (exact); fp8 accumulates in double, which holds the
@@ -74,12 +83,12 @@ __global__ __launch_bounds__(256) void quant_dot_generic_kernel(generic_params p
         if(row < p.m && k0 + tx < p.k)
         {
             uint8_t raw = a[row * p.a_sm + (k0 + tx) * p.a_sk];
-            av          = p.fp8 ? fp8_to_f32(raw) : (p.is_unsigned ? (float)raw : (float)(int8_t)raw);
+            av          = decode_operand(raw, p);
         }
         if(col < p.n && k0 + ty < p.k)
         {
             uint8_t raw = b[(k0 + ty) * p.b_sk + col * p.b_sn];
-            bv          = p.fp8 ? fp8_to_f32(raw) : (p.is_unsigned ? (float)raw : (float)(int8_t)raw);
+            bv          = decode_operand(raw, p);
         }
         as[ty][tx] = av;
         bs[ty][tx] = bv;
@@ -247,9 +256,13 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
     const bool empty = d->m == 0 || d->n == 0 || d->batch == 0;
     if(!empty && (a == nullptr || b == nullptr || c == nullptr))
         return MI355_ERR_BAD_ARG;
-    if(d->in_type != MI355_I8 && d->in_type != MI355_FP8 && d->in_type != MI355_U8)
+    if(d->in_type != MI355_I8 && d->in_type != MI355_FP8 && d->in_type != MI355_U8 &&
+       d->in_type != MI355_BF8)
         return MI355_ERR_UNSUPPORTED;
-    const bool fp8 = d->in_type == MI355_FP8;
+    // e5m2 x e5m2 -> float (op/quant_dot.hpp:62-66 takes every fp8 type): the 16x16x128 MFMA
+    // kernel or the generic one
+    const bool bf8 = d->in_type == MI355_BF8;
+    const bool fp8 = d->in_type == MI355_FP8 || bf8;
     // uint8 x uint8 -> int32 (op/quant_dot.hpp:62-64 lists it): bare result only, correctness path
     const bool u8 = d->in_type == MI355_U8;
     if(u8 && d->dequant)
@@ -298,7 +311,7 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
     hipStream_t s = static_cast<hipStream_t>(stream);
     // int8 with N % 4 != 0 would take the DMA path's 32 x 32 kernel, which applies no bias
     const bool dma_has_bias = bias == nullptr || fp8 || d->n % 4 == 0;
-    if(!u8 && d->k > 0 && dma_has_bias && mi355_dma_gemm_supported(d, a, b))
+    if(!u8 && !bf8 && d->k > 0 && dma_has_bias && mi355_dma_gemm_supported(d, a, b))
         return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, workspace, workspace_bytes, s);
     if(!u8 && d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
         return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
@@ -327,7 +340,7 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
     p.scale_b_mode = d->scale_b_mode;
     p.zp_a         = d->zp_a;
     p.zp_b         = d->zp_b;
-    p.fp8          = fp8;
+    p.fp8          = bf8 ? 2 : (fp8 ? 1 : 0);
     p.is_unsigned  = u8;
     p.dequant      = d->dequant;
     p.out_type     = d->out_type;

@@ -164,6 +164,69 @@ struct fp8e4m3fn
     }
 };
 
+// fp8 e5m2 (src/include/migraphx/float8.hpp:102-116 with cast_to_f8<2, 5, float, false, true> /
+// cast_from_f8<2, 5, float, false>): exponent 31 is +-infinity with a zero mantissa and NaN
+// otherwise; conversion from float rounds to the nearest value, ties to the even code, and clips
+// everything from 57344 up (infinities included) to +-57344.
+struct fp8e5m2
+{
+    uint8_t bits = 0;
+    fp8e5m2() = default;
+    template <class T, std::enable_if_t<std::is_arithmetic<T>{}, int> = 0>
+    fp8e5m2(T x) : bits(encode(static_cast<float>(x))) // NOLINT
+    {
+    }
+    operator float() const { return decode(bits); }               // NOLINT
+    static fp8e5m2 from_bits(uint8_t b)
+    {
+        fp8e5m2 r;
+        r.bits = b;
+        return r;
+    }
+
+    static float decode(uint8_t b)
+    {
+        const int e     = (b >> 2) & 0x1f;
+        const int m     = b & 3;
+        const float sgn = (b & 0x80) != 0 ? -1.0f : 1.0f;
+        if(e == 0x1f)
+            return m == 0 ? sgn * std::numeric_limits<float>::infinity()
+                          : std::numeric_limits<float>::quiet_NaN();
+        if(e == 0)
+            return sgn * std::ldexp(static_cast<float>(m), -16);
+        return sgn * std::ldexp(static_cast<float>(4 + m), e - 17);
+    }
+
+    static uint8_t encode(float f)
+    {
+        const uint8_t sign = std::signbit(f) ? 0x80 : 0;
+        if(std::isnan(f))
+            return sign | 0x7f;
+        const float a = std::fabs(f);
+        if(a >= 57344.0f)
+            return sign | 0x7b;
+        // spacing of the grid around a: 2^-16 below 2^-14, else 2^(floor(log2 a) - 2)
+        int ex = 0;
+        std::frexp(a, &ex);
+        int step_exp = (ex - 1) - 2;
+        if(step_exp < -16)
+            step_exp = -16;
+        const float q = std::ldexp(a, -step_exp);   // exact
+        const float r = std::nearbyint(q);          // FE_TONEAREST: ties to even
+        const float v = std::ldexp(r, step_exp);
+        if(v > 57344.0f)
+            return sign | 0x7b;
+        if(v == 0.0f)
+            return sign;
+        int e2 = 0;
+        const float m2 = std::frexp(v, &e2);
+        if(e2 - 1 < -14)
+            return sign | static_cast<uint8_t>(std::ldexp(v, 16));
+        const int mant = static_cast<int>(std::ldexp(m2, 3)) - 4;
+        return sign | static_cast<uint8_t>(((e2 - 1 + 15) << 2) | mant);
+    }
+};
+
 } // namespace migraphx
 
 namespace std {
@@ -186,6 +249,18 @@ struct numeric_limits<migraphx::fp8e4m3fn>
     static T lowest() { return T::from_bits(0xfe); }
     static T min() { return T::from_bits(0x08); }
     static T epsilon() { return T::from_bits(0x20); }
+};
+template <>
+struct numeric_limits<migraphx::fp8e5m2> // float8.hpp:357-375
+{
+    using T = migraphx::fp8e5m2;
+    static constexpr bool is_specialized = true;
+    static T max() { return T::from_bits(0x7b); }
+    static T lowest() { return T::from_bits(0xfb); }
+    static T min() { return T::from_bits(0x04); }
+    static T epsilon() { return T::from_bits(0x34); }
+    static T infinity() { return T::from_bits(0x7c); }
+    static T quiet_NaN() { return T::from_bits(0xff); } // NOLINT
 };
 } // namespace std
 

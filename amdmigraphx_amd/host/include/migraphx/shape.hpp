@@ -30,12 +30,13 @@ namespace migraphx {
     m(uint32_type, uint32_t) \
     m(uint64_type, uint64_t) \
     m(fp8e4m3fn_type, migraphx::fp8e4m3fn) \
+    m(fp8e5m2_type, migraphx::fp8e5m2) \
     m(bf16_type, migraphx::bf16)
 // clang-format on
 
 struct shape
 {
-    // numbering of the reference's enum (shape.hpp:57-73); the fnuz / e5m2 fp8 variants keep their
+    // numbering of the reference's enum (shape.hpp:57-73); the fnuz fp8 variants keep their
     // slots but no kernel of this build takes them
     enum type_t
     {

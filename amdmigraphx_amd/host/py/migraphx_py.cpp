@@ -210,6 +210,7 @@ PYBIND11_MODULE(migraphx, m)
         .value("uint32_type", shape::uint32_type)
         .value("uint64_type", shape::uint64_type)
         .value("fp8e4m3fn_type", shape::fp8e4m3fn_type)
+        .value("fp8e5m2_type", shape::fp8e5m2_type)
         .value("bf16_type", shape::bf16_type)
         .value("fp4x2_type", shape::fp4x2_type);
     shape_cls

@@ -101,6 +101,7 @@ int to_mi355_type(shape::type_t t)
     case shape::half_type: return MI355_F16;
     case shape::bf16_type: return MI355_BF16;
     case shape::fp8e4m3fn_type: return MI355_FP8;
+    case shape::fp8e5m2_type: return MI355_BF8;
     default: MIGRAPHX_THROW("mi355: no kernel takes " + shape::type_name(t));
     }
 }
@@ -276,9 +277,10 @@ shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
     check_inputs(inputs, expected_inputs(), name());
     auto s = op::quant_dot{}.compute_shape({inputs[0], inputs[1]});
     const bool bare_u8 = inputs[0].type() == shape::uint8_type and not dequant;
-    if(inputs[0].type() != shape::int8_type and inputs[0].type() != shape::fp8e4m3fn_type and not bare_u8)
-        MIGRAPHX_THROW("mi355::quant_dot: kernels take int8 or fp8e4m3fn operands (uint8 for the bare "
-                       "result), not " + inputs[0].type_string());
+    if(inputs[0].type() != shape::int8_type and inputs[0].type() != shape::fp8e4m3fn_type and
+       inputs[0].type() != shape::fp8e5m2_type and not bare_u8)
+        MIGRAPHX_THROW("mi355::quant_dot: kernels take int8, fp8e4m3fn or fp8e5m2 operands (uint8 for the "
+                       "bare result), not " + inputs[0].type_string());
     if(not view_as_matrix(inputs[0]).ok or not view_as_matrix(inputs[1]).ok)
         MIGRAPHX_THROW("mi355::quant_dot: operand strides are neither row-major nor transposed");
     if(not dequant and out_type != s.type())

@@ -16,7 +16,7 @@ from .capi import DT, QP, W4ZP, QuantDotDesc, QuantConv3dDesc, QuantConvDesc, Mx
 _TORCH2DT = {torch.int8: DT.I8, torch.uint8: DT.U8, torch.int32: DT.I32, torch.float32: DT.F32,
              torch.float16: DT.F16, torch.bfloat16: DT.BF16}
 _DT2TORCH = {DT.I8: torch.int8, DT.U8: torch.uint8, DT.I32: torch.int32, DT.F32: torch.float32,
-             DT.F16: torch.float16, DT.BF16: torch.bfloat16, DT.FP8: torch.uint8}
+             DT.F16: torch.float16, DT.BF16: torch.bfloat16, DT.FP8: torch.uint8, DT.BF8: torch.uint8}
 
 
 def _stream():
@@ -50,7 +50,8 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     """quant_dot, optionally with the fused dequantizelinear epilogue.
 
     a [..., M, K], b [..., K, N] int8 (or uint8 carrying fp8 e4m3fn bits with
-    fp8=True; plain uint8 operands give the bare int32 result only); transposed
+    fp8=True, fp8 e5m2 bits with fp8="e5m2"; plain uint8 operands give the bare int32 result
+    only); transposed
     views are passed as they are.  Without scales the
     bare accumulators come back (int32 / float32).  With ``scale_a`` (scalar
     or [M]) / ``scale_b`` (scalar or [N]) float32 tensors the epilogue
@@ -84,7 +85,7 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     ta, lda = _mat_layout(a3)
     tb, ldb = _mat_layout(b3)
     dequant = scale_a is not None or scale_b is not None or out_dtype is not None
-    in_type = DT.FP8 if fp8 else (DT.U8 if a.dtype == torch.uint8 else DT.I8)
+    in_type = DT.BF8 if fp8 == "e5m2" else DT.FP8 if fp8 else (DT.U8 if a.dtype == torch.uint8 else DT.I8)
     if dequant:
         odt = out_dtype or torch.float32
     else:

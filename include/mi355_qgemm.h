@@ -41,7 +41,8 @@ typedef enum mi355_dtype {
     MI355_F16  = 4, /* IEEE binary16 */
     MI355_BF16 = 5,
     MI355_FP8  = 6, /* OCP e4m3fn */
-    MI355_FP4X2 = 7 /* two OCP e2m1 codes per byte, low nibble = even element (block-scaled operands) */
+    MI355_FP4X2 = 7, /* two OCP e2m1 codes per byte, low nibble = even element (block-scaled operands) */
+    MI355_BF8  = 8  /* OCP e5m2 (shape::fp8e5m2_type, src/include/migraphx/float8.hpp:102-116) */
 } mi355_dtype;
 
 /* How a quantization parameter is broadcast over an [M, N] result. */
@@ -72,7 +73,7 @@ typedef struct mi355_quant_dot_desc {
     int64_t batch;
     int64_t stride_a, stride_b, stride_c;
     int32_t trans_a, trans_b;
-    int32_t in_type;  /* MI355_I8 or MI355_FP8; MI355_U8 for the bare result only */
+    int32_t in_type;  /* MI355_I8, MI355_FP8 or MI355_BF8; MI355_U8 for the bare result only */
     int32_t out_type; /* MI355_I32 / MI355_F32: bare quant_dot result (int8 / fp8).
                          With an epilogue: MI355_F32, MI355_F16 or MI355_BF16. */
     /* ---- fused dequantizelinear epilogue (all zero = bare quant_dot) ---- */
@@ -88,7 +89,8 @@ typedef struct mi355_quant_dot_desc {
  * Replaces: ref_quant_gemm::compute (src/targets/ref/lowering.cpp:218-248) ->
  * gemm_naive (src/gemm.cpp:42-63) with the shape rules of
  * op::quant_dot::compute_shape (src/include/migraphx/op/quant_dot.hpp:51-121):
- * int8 x int8 -> int32 (exact), fp8 e4m3fn x fp8 e4m3fn -> float.
+ * int8 x int8 -> int32 (exact), fp8 e4m3fn x fp8 e4m3fn -> float, fp8 e5m2 x fp8 e5m2 -> float
+ * (op/quant_dot.hpp:62-66 takes every fp8 type; both operands have the same one).
  *
  * With desc->dequant it also replaces the instructions simplify_qdq.cpp:225-289
  * emits behind the quant_dot and that the ref target evaluates one by one:
@@ -269,7 +271,8 @@ int mi355_rowsum_i8(const void* a, int64_t m, int64_t k, int64_t lda, int32_t tr
  * (src/include/migraphx/op/quantizelinear.hpp:71-108).
  *   integral out: clamp(double(nearbyint(x / s)) + double(zp)), x / s divided
  *                 in x's own type, ties to even;
- *   fp8 out:      clamp(double(x)/double(s) + double(zp), -448, 448) -> fp8.
+ *   fp8 out:      clamp(double(x)/double(s) + double(zp), -448, 448) -> fp8 e4m3fn;
+ *                 the same with +-57344 for MI355_BF8 (fp8 e5m2).
  * scale has x's element type, zp (may be NULL = 0) has the output's.  Both are
  * addressed as p[r*stride_r + c*stride_c] so a per-tensor parameter uses
  * strides (0,0), a per-column one (0,1), a per-row one (1,0), a full one
@@ -341,7 +344,8 @@ int mi355_pack_fp4(const float* in, void* out, int64_t rows, int64_t cols, void*
  *
  * Replaces: op::convert::compute (src/include/migraphx/op/convert.hpp:64-87)
  * with the software-float conversions of generic_float.hpp:172-222 (half and
- * bf16: round toward zero) and float8_impl.hpp:38-247 (fp8: nearest even).
+ * bf16: round toward zero) and float8_impl.hpp:38-247 (fp8 e4m3fn and e5m2: nearest even,
+ * clipping; NaN becomes numeric_limits::quiet_NaN of the type, 0x7f and 0xff).
  */
 int mi355_convert(const void* in, int32_t in_type, void* out, int32_t out_type,
                   int64_t n, void* stream);

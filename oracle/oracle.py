@@ -18,9 +18,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-I8, U8, I32, F32, F16, BF16, FP8, F64 = range(8)
+I8, U8, I32, F32, F16, BF16, FP8, F64, BF8 = range(9)
 _NP = {I8: np.int8, U8: np.uint8, I32: np.int32, F32: np.float32,
-       F16: np.uint16, BF16: np.uint16, FP8: np.uint8, F64: np.float64}
+       F16: np.uint16, BF16: np.uint16, FP8: np.uint8, F64: np.float64, BF8: np.uint8}
 
 
 def build():
@@ -61,7 +61,7 @@ def _load():
     lib.orc_convert.restype = None
     lib.orc_mul_f32.argtypes = [vp, vp, i64, i64, vp, i64, i64, i64, i64]
     lib.orc_mul_f32.restype = None
-    for name in ("half", "bf16", "fp8e4m3fn"):
+    for name in ("half", "bf16", "fp8e4m3fn", "fp8e5m2"):
         getattr(lib, f"orc_{name}_from_f32_n").argtypes = [vp, vp, ctypes.c_size_t]
         getattr(lib, f"orc_{name}_from_f32_n").restype = None
         getattr(lib, f"orc_{name}_to_f32_n").argtypes = [vp, vp, ctypes.c_size_t]
@@ -112,6 +112,15 @@ def fp8_from_f32(x):
 
 def fp8_to_f32(x):
     return _conv("orc_fp8e4m3fn_to_f32_n", x, np.uint8, np.float32)
+
+
+def bf8_from_f32(x):
+    """float -> fp8 e5m2 bits (float8.hpp:102-116)."""
+    return _conv("orc_fp8e5m2_from_f32_n", x, np.float32, np.uint8)
+
+
+def bf8_to_f32(x):
+    return _conv("orc_fp8e5m2_to_f32_n", x, np.uint8, np.float32)
 
 
 # --- ops ---------------------------------------------------------------------
@@ -349,10 +358,10 @@ def qdq_matmul_int8(x_q, w_q, s_x, s_w, zp_x=0, zp_w=0, out_type=F32):
     return out
 
 
-def qdq_matmul_fp8(x_q, w_q, s_x, s_w, out_type=F32):
+def qdq_matmul_fp8(x_q, w_q, s_x, s_w, out_type=F32, fp8_type=FP8):
     m = x_q.shape[0]
     n = w_q.shape[1]
-    acc = quant_dot(x_q, w_q, FP8)
+    acc = quant_dot(x_q, w_q, fp8_type)
     scale = mul_f32(np.asarray(s_x, np.float32), np.asarray(s_w, np.float32), m, n)
     out = dequantizelinear(acc, scale, None, F32, F32)
     if out_type != F32:

@@ -19,6 +19,10 @@
  *                                 force "nearest table entry, ties to even
  *                                 mantissa, saturate to 448" over random and
  *                                 adversarial floats
+ *   orc_fp8e5m2_to_f32            256-entry table of test/fp8e5m2.cpp:34-292
+ *   orc_fp8e5m2_from_f32          samples test/fp8e5m2.cpp:320-360 + the same
+ *                                 brute force against the table, saturating
+ *                                 to 57344
  *   orc_half_* / orc_bf16_*       tables test/half.cpp, test/bf16.cpp + closed
  *                                 form (mantissa shift == round toward zero,
  *                                 compared with numpy bit arithmetic)
@@ -70,7 +74,8 @@ enum {
     ORC_F16  = 4,
     ORC_BF16 = 5,
     ORC_FP8  = 6, /* OCP e4m3fn */
-    ORC_F64  = 7
+    ORC_F64  = 7,
+    ORC_BF8  = 8  /* OCP e5m2 */
 };
 
 static inline uint32_t f32_bits(float f)
@@ -194,18 +199,26 @@ float orc_bf16_to_f32(uint16_t h) { return gf_to_f32(h, 7, 8); }
  * Round to nearest even, saturate to +-448 (0x7e/0xfe), +-inf -> +-448,
  * NaN -> 0x7f / 0xff.
  * ---------------------------------------------------------------------- */
-float orc_fp8e4m3fn_to_f32(uint8_t x)
+static float f8_to_f32(uint8_t x, int wm, int we)
 {
-    const int wm = 3, we = 4;
     if(x == 0)
         return 0.0f;
     if(x == 0x80)
         return bits_f32(0x80000000u);
-    if(x == 0x7f || x == 0xff)
-        return bits_f32(0x7f800001u);
     uint32_t sign     = x >> 7;
     uint32_t mantissa = x & ((1u << wm) - 1u);
     int exponent      = (x & 0x7f) >> wm;
+    if(we == 4)
+    {
+        if(x == 0x7f || x == 0xff)
+            return bits_f32(0x7f800001u);
+    }
+    else if(exponent == 31) /* e5m2: +-inf, else NaN (float8_impl.hpp:286-291) */
+    {
+        if(mantissa == 0)
+            return bits_f32(sign ? 0xff800000u : 0x7f800000u);
+        return bits_f32(0x7f800001u);
+    }
     const int exp_low_cutoff = (1 << (8 - 1)) - (1 << (we - 1)) + 1; /* 121 */
     if(exponent == 0)
     {
@@ -219,9 +232,9 @@ float orc_fp8e4m3fn_to_f32(uint8_t x)
     return bits_f32((sign << 31) | ((uint32_t)exponent << 23) | mantissa);
 }
 
-uint8_t orc_fp8e4m3fn_from_f32(float fx)
+static uint8_t f8_from_f32(float fx, uint32_t wm, uint32_t we)
 {
-    const uint32_t wm = 3, we = 4, mfmt = 23;
+    const uint32_t mfmt = 23;
     uint32_t x        = f32_bits(fx);
     uint32_t head     = x & 0xFF800000u;
     uint32_t mantissa = x & 0x7FFFFFu;
@@ -231,21 +244,22 @@ uint8_t orc_fp8e4m3fn_from_f32(float fx)
 
     uint32_t signed_inf      = (sign << 7) + (((1u << we) - 1u) << wm);
     uint32_t signed_all_ones = (sign << 7) + ((((1u << we) - 1u) << wm) + ((1u << wm) - 1u));
-    uint32_t signed_max      = signed_all_ones - 1u; /* wm == 3 */
+    /* float8_impl.hpp:81-83: e4m3fn max is all ones - 1, e5m2 max is all ones - 4 */
+    uint32_t signed_max = wm == 2 ? signed_all_ones - 4u : signed_all_ones - 1u;
 
     if((x & 0x7F800000u) == 0x7F800000u)
     {
         if(mantissa == 0)
-            return sign == 0 ? 0x7E : 0xFE;
-        return (uint8_t)(signed_inf + 7u); /* all-ones mantissa NaN */
+            return (uint8_t)signed_max;                      /* float8_impl.hpp:103-109 */
+        return (uint8_t)(signed_inf + ((1u << wm) - 1u));    /* all-ones mantissa NaN */
     }
     if(x == 0)
         return 0;
     if(x == 0x80000000u)
         return 0x80;
 
-    const int f8_bias                  = (1 << (we - 1u)) - 1; /* 7 */
-    const int f8_denormal_act_exponent = 1 - f8_bias;          /* -6 */
+    const int f8_bias                  = (1 << (we - 1u)) - 1; /* 7 | 15 */
+    const int f8_denormal_act_exponent = 1 - f8_bias;          /* -6 | -14 */
     int act_exponent, f8_exponent, exponent_diff;
 
     if(exponent == 0 && mantissa != 0)
@@ -296,18 +310,31 @@ uint8_t orc_fp8e4m3fn_from_f32(float fx)
     }
     mantissa >>= (mfmt - wm);
 
-    const int max_exp = (1 << we) - 1; /* wm == 3 */
+    /* float8_impl.hpp:228: exponent 31 of e5m2 belongs to inf and NaN */
+    const int max_exp = (1 << we) - (wm == 3 ? 1 : 2);
     if(f8_exponent > max_exp)
         return (uint8_t)signed_max;
     if(f8_exponent == 0 && mantissa == 0)
         return (uint8_t)(sign << 7);
     mantissa &= (1u << wm) - 1u;
     uint8_t r = (uint8_t)((sign << 7) | ((uint32_t)f8_exponent << wm) | mantissa);
-    /* exponent 15 with mantissa 7 is the NaN code: the clip branch above is
+    /* e4m3fn: exponent 15 with mantissa 7 is the NaN code: the clip branch above is
        reached only for f8_exponent > 15, so 0x7f can come out of the rounding
        carry; the reference returns it unchanged (float8_impl.hpp:243-246). */
     return r;
 }
+
+float orc_fp8e4m3fn_to_f32(uint8_t x) { return f8_to_f32(x, 3, 4); }
+uint8_t orc_fp8e4m3fn_from_f32(float fx) { return f8_from_f32(fx, 3, 4); }
+
+/* ------------------------------------------------------------------------
+ * fp8 e5m2 (OCP: exponent 31 is +-inf with mantissa 0, NaN otherwise; max 57344 = 0x7b)
+ * cast_from_f8<2,5,float,false> / cast_to_f8<2,5,float,false,true(clip)>, selected by
+ * float8.hpp:102-116.  Round to nearest even, saturate to +-57344, +-inf -> +-57344,
+ * NaN -> 0x7f / 0xff.
+ * ---------------------------------------------------------------------- */
+float orc_fp8e5m2_to_f32(uint8_t x) { return f8_to_f32(x, 2, 5); }
+uint8_t orc_fp8e5m2_from_f32(float fx) { return f8_from_f32(fx, 2, 5); }
 
 /* vector forms for the Python side */
 void orc_half_from_f32_n(const float* x, uint16_t* y, size_t n)
@@ -329,6 +356,16 @@ void orc_bf16_to_f32_n(const uint16_t* x, float* y, size_t n)
 {
     for(size_t i = 0; i < n; i++)
         y[i] = orc_bf16_to_f32(x[i]);
+}
+void orc_fp8e5m2_from_f32_n(const float* x, uint8_t* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_fp8e5m2_from_f32(x[i]);
+}
+void orc_fp8e5m2_to_f32_n(const uint8_t* x, float* y, size_t n)
+{
+    for(size_t i = 0; i < n; i++)
+        y[i] = orc_fp8e5m2_to_f32(x[i]);
 }
 void orc_fp8e4m3fn_from_f32_n(const float* x, uint8_t* y, size_t n)
 {
@@ -356,6 +393,7 @@ static inline double load_f64(const void* p, int type, size_t i)
     case ORC_F16: return (double)orc_half_to_f32(((const uint16_t*)p)[i]);
     case ORC_BF16: return (double)orc_bf16_to_f32(((const uint16_t*)p)[i]);
     case ORC_FP8: return (double)orc_fp8e4m3fn_to_f32(((const uint8_t*)p)[i]);
+    case ORC_BF8: return (double)orc_fp8e5m2_to_f32(((const uint8_t*)p)[i]);
     case ORC_F64: return ((const double*)p)[i];
     default: return NAN;
     }
@@ -376,6 +414,7 @@ static inline void store_f64(void* p, int type, size_t i, double d)
     case ORC_F16: ((uint16_t*)p)[i] = orc_half_from_f32((float)d); break;
     case ORC_BF16: ((uint16_t*)p)[i] = orc_bf16_from_f32((float)d); break;
     case ORC_FP8: ((uint8_t*)p)[i] = orc_fp8e4m3fn_from_f32((float)d); break;
+    case ORC_BF8: ((uint8_t*)p)[i] = orc_fp8e5m2_from_f32((float)d); break;
     case ORC_F64: ((double*)p)[i] = d; break;
     default: break;
     }
@@ -392,6 +431,7 @@ static inline double type_max(int type)
     case ORC_F16: return 65504.0;
     case ORC_BF16: return 3.38953138925153547590470800371487867e+38;
     case ORC_FP8: return 448.0;
+    case ORC_BF8: return 57344.0; /* float8.hpp:361-373 */
     default: return INFINITY;
     }
 }
@@ -802,6 +842,7 @@ void orc_convert(void* out, int out_type, const void* x, int x_type, size_t n)
             case ORC_F16: ((uint16_t*)out)[i] = 0x7e00; break;
             case ORC_BF16: ((uint16_t*)out)[i] = 0x7fc0; break;
             case ORC_FP8: ((uint8_t*)out)[i] = 0x7f; break;
+            case ORC_BF8: ((uint8_t*)out)[i] = 0xff; break; /* float8.hpp:364 */
             default: store_f64(out, out_type, i, 0.0); break;
             }
             continue;

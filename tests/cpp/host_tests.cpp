@@ -18,6 +18,8 @@
 extern "C" {
 float orc_fp8e4m3fn_to_f32(uint8_t x);
 uint8_t orc_fp8e4m3fn_from_f32(float x);
+float orc_fp8e5m2_to_f32(uint8_t x);
+uint8_t orc_fp8e5m2_from_f32(float x);
 uint16_t orc_half_from_f32(float x);
 float orc_half_to_f32(uint16_t h);
 uint16_t orc_bf16_from_f32(float x);
@@ -50,6 +52,35 @@ TEST_CASE(fp8_matches_oracle)
     }
     for(float f : {0.0f, -0.0f, 1.0f, 1.0625f, 1.1875f, 448.0f, 1000.0f, -1000.0f, 0.001953125f, 0.0009765625f})
         EXPECT(migraphx::fp8e4m3fn(f).bits == orc_fp8e4m3fn_from_f32(f));
+}
+
+TEST_CASE(fp8e5m2_matches_oracle)
+{
+    for(int c = 0; c < 256; c++)
+    {
+        const float a = migraphx::fp8e5m2::from_bits(c);
+        const float b = orc_fp8e5m2_to_f32(c);
+        EXPECT((std::isnan(a) and std::isnan(b)) or (a == b and std::signbit(a) == std::signbit(b)));
+        if(not std::isnan(b) and not std::isinf(b))
+            EXPECT(migraphx::fp8e5m2(b).bits == c);
+    }
+    std::mt19937 g(2);
+    for(int i = 0; i < 400000; i++)
+    {
+        uint32_t bits = g();
+        if(i % 2 == 1) // half of the samples inside the format's range, where the rounding happens
+            bits = (bits & 0x807fffffu) | ((100u + (g() % 46u)) << 23);
+        float f;
+        std::memcpy(&f, &bits, 4);
+        EXPECT(migraphx::fp8e5m2(f).bits == orc_fp8e5m2_from_f32(f));
+    }
+    for(float f : {0.0f, -0.0f, 1.0f, 1.125f, 1.375f, 57344.0f, 61440.0f, 1e9f, -1e9f, 7.62939453125e-06f,
+                   2.288818359375e-05f, std::numeric_limits<float>::infinity()})
+        EXPECT(migraphx::fp8e5m2(f).bits == orc_fp8e5m2_from_f32(f));
+    EXPECT(std::numeric_limits<migraphx::fp8e5m2>::max().bits == 0x7b);
+    EXPECT(float(std::numeric_limits<migraphx::fp8e5m2>::lowest()) == -57344.0f);
+    EXPECT(shape::type_size(shape::fp8e5m2_type) == 1);
+    EXPECT(shape::get_type<migraphx::fp8e5m2>::value == shape::fp8e5m2_type);
 }
 
 TEST_CASE(half_bf16_match_oracle)

@@ -53,7 +53,8 @@ enum
     ORC_F16,
     ORC_BF16,
     ORC_FP8,
-    ORC_F64
+    ORC_F64,
+    ORC_BF8
 };
 
 int orc_type(shape::type_t t)
@@ -67,6 +68,7 @@ int orc_type(shape::type_t t)
     case shape::half_type: return ORC_F16;
     case shape::bf16_type: return ORC_BF16;
     case shape::fp8e4m3fn_type: return ORC_FP8;
+    case shape::fp8e5m2_type: return ORC_BF8;
     case shape::double_type: return ORC_F64;
     default: MIGRAPHX_THROW("oracle: unsupported type " + shape::type_name(t));
     }

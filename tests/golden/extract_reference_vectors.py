@@ -95,6 +95,15 @@ pairs = re.findall(r"\{\s*([-+0-9.eE]+)\s*,\s*(0x[0-9a-fA-F]+)\s*\}", m.group(1)
 out["fp8e4m3fn_from_float"] = {"source": "test/fp8e4m3fn.cpp:121-140",
                                "pairs": [[float(a), int(b, 16)] for a, b in pairs]}
 
+# ---- fp8 e5m2 table and cast samples (test/fp8e5m2.cpp) ----------------------
+t = read("test/fp8e5m2.cpp")
+m = re.search(r"e4m3fnuz_lut = \{(.*?)\};", t, re.S)     # (the table keeps that name in this file too)
+out["fp8e5m2_lut"] = {"source": "test/fp8e5m2.cpp:37-295", "values": num_list(m.group(1))}
+m = re.search(r"test_vals = \{\s*\{(.*?)\}\s*,?\s*\};", t, re.S)
+pairs = re.findall(r"\{\s*([-+0-9.eE]+)\s*,\s*(0x[0-9a-fA-F]+)\s*\}", "{" + m.group(1) + "}")
+out["fp8e5m2_from_float"] = {"source": "test/fp8e5m2.cpp:320-360",
+                             "pairs": [[float(a), int(b, 16)] for a, b in pairs]}
+
 # ---- half / bf16 tables ------------------------------------------------------
 for nm, rel in (("half", "test/half.cpp"), ("bf16", "test/bf16.cpp")):
     t = read(rel)
@@ -163,6 +172,12 @@ body = m.group(1)
 out["quantizelinear_fp8e4m3"] = {
     "source": "test/ref/quantizelinear.cpp:86-127 (gold is computed there as "
               "fp8(clamp(x/s + fp8(zp))) in double)",
+    "x": vec(body, "xv"), "scale": vec(body, "sv"), "zp_float": vec(body, "tmp"), "lens": [2, 2, 2]}
+m = re.search(r"static void quantizelinear_fp8e5m2\(\)(.*?)TEST_CASE_REGISTER", t, re.S)
+body = m.group(1)
+out["quantizelinear_fp8e5m2"] = {
+    "source": "test/ref/quantizelinear.cpp:129-168 (gold is computed there as "
+              "fp8(clamp(x/s) + fp8(zp)) in double)",
     "x": vec(body, "xv"), "scale": vec(body, "sv"), "zp_float": vec(body, "tmp"), "lens": [2, 2, 2]}
 
 t = read("test/ref/dequantizelinear.cpp")

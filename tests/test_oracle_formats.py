@@ -1,4 +1,4 @@
-"""Pins the oracle's number formats (fp8 e4m3fn, half, bf16) against the tables
+"""Pins the oracle's number formats (fp8 e4m3fn and e5m2, half, bf16) against the tables
 the reference's own tests hold and against closed forms that do not share code
 with the oracle."""
 import numpy as np
@@ -78,6 +78,80 @@ def test_fp8_round_trip_all_codes():
     finite = (codes & 0x7f) != 0x7f
     back = orc.fp8_from_f32(orc.fp8_to_f32(codes))
     assert np.array_equal(back[finite], codes[finite])
+
+
+def _lut_e5m2(golden):
+    return np.array([float(v) for v in golden["fp8e5m2_lut"]["values"]], np.float64)
+
+
+def test_bf8_decode_matches_reference_table(golden):
+    lut = _lut_e5m2(golden)
+    got = orc.bf8_to_f32(np.arange(256, dtype=np.uint8)).astype(np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(lut))
+    ok = ~np.isnan(lut)
+    assert np.array_equal(got[ok], lut[ok])                    # +-inf at 0x7c / 0xfc included
+    assert np.isinf(got[0x7c]) and np.isinf(got[0xfc]) and got[0xfc] < 0
+    assert np.signbit(got[0x80]) and not np.signbit(got[0])
+    # an e5m2 value is the upper byte of the half with the same value
+    half = orc.half_to_f32((np.arange(256, dtype=np.uint16) << 8)).astype(np.float64)
+    assert np.array_equal(got[ok], half[ok])
+
+
+def test_bf8_encode_reference_samples(golden):
+    pairs = golden["fp8e5m2_from_float"]["pairs"]
+    x = np.array([p[0] for p in pairs], np.float32)
+    want = np.array([p[1] for p in pairs], np.uint8)
+    got = orc.bf8_from_f32(x)
+    # test/fp8e5m2.cpp compares through float_equal; every sample but +-7.6e-06 has a non-zero
+    # result, and for those two the sign of the zero is kept (test_negative_zero of that file)
+    assert np.array_equal(got, want)
+
+
+def test_bf8_encode_is_rne_saturating(golden):
+    """Independent of the oracle's bit arithmetic: nearest finite table value, ties to the even
+    code, everything at or beyond 57344 (rounded) saturates to 0x7b."""
+    lut = _lut_e5m2(golden)
+    pos = lut[:0x7c]                                           # 0 .. 57344 ascending
+    rng = np.random.default_rng(1)
+    mids = (pos[:-1] + pos[1:]) / 2
+    adv = np.concatenate([mids, np.nextafter(mids.astype(np.float32), np.float32(0)),
+                          np.nextafter(mids.astype(np.float32), np.float32(1e9)), pos,
+                          [57344.0, 57345.0, 61439.0, 61440.0, 61441.0, 65536.0, 1e6, 3e38,
+                           2.0**-17, 2.0**-18, 1e-30, 1e-45]])
+    rnd = np.concatenate([rng.normal(0, 1, 200000), rng.normal(0, 1000, 200000),
+                          rng.uniform(-70000, 70000, 100000), rng.normal(0, 1e-4, 100000)])
+    x = np.concatenate([adv, -adv, rnd]).astype(np.float32)
+    ax = np.abs(x.astype(np.float64))
+    idx = np.clip(np.searchsorted(pos, ax, side="left"), 1, len(pos) - 1)
+    lo, hi = pos[idx - 1], pos[idx]
+    dlo, dhi = ax - lo, hi - ax
+    pick_hi = (dhi < dlo) | ((dhi == dlo) & ((idx % 2) == 0))
+    code = np.where(pick_hi, idx, idx - 1)
+    # 61440 is the tie between 57344 (odd code 0x7b) and 65536: it rounds up and out of range,
+    # and out of range clips to the largest finite value (float8_impl.hpp:228-233)
+    code = np.where(ax >= 57344.0, 0x7b, code)
+    want = (code | (np.signbit(x).astype(np.int64) << 7)).astype(np.uint8)
+    assert np.array_equal(orc.bf8_from_f32(x), want)
+    sp = np.array([np.inf, -np.inf, np.nan], np.float32)
+    g = orc.bf8_from_f32(sp)
+    assert g[0] == 0x7b and g[1] == 0xfb and (g[2] & 0x7f) == 0x7f
+
+
+def test_bf8_round_trip_all_codes():
+    codes = np.arange(256, dtype=np.uint8)
+    finite = (codes & 0x7c) != 0x7c
+    back = orc.bf8_from_f32(orc.bf8_to_f32(codes))
+    assert np.array_equal(back[finite], codes[finite])
+
+
+def test_bf8_convert_and_quantize_follow_the_type_limits():
+    """convert (op/convert.hpp:64-87): NaN -> numeric_limits::quiet_NaN (0xff), infinities go
+    through the constructor (which clips), everything else clamps to +-57344."""
+    x = np.array([np.nan, np.inf, -np.inf, 1e9, -1e9, 57344.0, 3.0, -0.0], np.float32)
+    got = orc.convert(x, orc.F32, orc.BF8)
+    assert list(got) == [0xff, 0x7b, 0xfb, 0x7b, 0xfb, 0x7b, 0x42, 0x80]
+    back = orc.convert(np.array([0x7c, 0xfc, 0x7d, 0x42], np.uint8), orc.BF8, orc.F32)
+    assert np.isinf(back[0]) and back[1] == -np.inf and np.isnan(back[2]) and back[3] == 3.0
 
 
 def _check_lut(pairs, from_f32, to_f32):

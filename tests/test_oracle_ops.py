@@ -108,6 +108,41 @@ def test_quantizelinear_fp8_reference_case(golden):
     assert got.flatten()[0] == 0x43 and got.flatten()[1] == 0x3e
 
 
+def test_quantizelinear_fp8e5m2_reference_case(golden):
+    c = golden["quantizelinear_fp8e5m2"]
+    x = np.float32(c["x"]).reshape(c["lens"])
+    s = np.float32(c["scale"]).reshape(c["lens"])
+    z = orc.bf8_from_f32(np.float32(c["zp_float"])).reshape(c["lens"])
+    got = orc.quantizelinear(x, s, z, orc.F32, orc.BF8)
+    # the reference test builds its gold as fp8(clamp(x/s, -57344, 57344) + zp) in double
+    zf = orc.bf8_to_f32(z).astype(np.float64)
+    q = np.clip(x.astype(np.float64) / s.astype(np.float64), -57344, 57344) + zf
+    want = orc.bf8_from_f32(q.astype(np.float32))
+    assert np.array_equal(got, want)
+    # hand-checked entries: the zero point 0.6875 is the tie between 0.625 (0x39) and 0.75 (0x3a)
+    # and goes to the even code, 0.75; 0.5/0.25 + 0.75 = 2.75 is the tie between 2.5 (0x41) and
+    # 3 (0x42) -> 3; 0.75/0.75 + 0.75 = 1.75 (0x3f)
+    assert got.flatten()[0] == 0x42 and got.flatten()[1] == 0x3f
+
+
+def test_quant_dot_fp8e5m2_is_the_exact_sum_rounded_once():
+    """quant_dot over e5m2 (op/quant_dot.hpp:62-77 -> gemm in double, float out): every product of
+    two e5m2 values is a multiple of 2^-32 below 2^32, so the sum is exact in Python integers."""
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (5, 48)).astype(np.uint8)
+    b = rng.integers(0, 256, (48, 7)).astype(np.uint8)
+    a[(a & 0x7c) == 0x7c] = 0x3c
+    b[(b & 0x7c) == 0x7c] = 0xbc
+    a = (a & 0xbf) | 0x20            # exponents 8..15 and 24..: keep magnitudes in a narrow range
+    got = orc.quant_dot(a, b, orc.BF8)
+    af, bf = orc.bf8_to_f32(a).astype(np.float64), orc.bf8_to_f32(b).astype(np.float64)
+    from fractions import Fraction
+    for i in range(5):
+        for j in range(7):
+            exact = sum(Fraction(float(af[i, k])) * Fraction(float(bf[k, j])) for k in range(48))
+            assert got[i, j] == np.float32(float(exact)), (i, j)
+
+
 def test_quantizelinear_int8_ties_to_even_and_true_division():
     x = np.float32([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 1e9, -1e9, 3.0])
     got = orc.quantizelinear(x, np.float32(1.0), np.int8(0), orc.F32, orc.I8)
