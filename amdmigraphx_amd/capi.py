@@ -132,6 +132,10 @@ EXPORTS = {
                             ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
                             ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                             ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    "mi355_quant_dot_prepacked_size": [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64],
+    "mi355_quant_dot_prepack": [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p],
+    "mi355_quant_dot_prepacked": [ctypes.c_void_p] * 10,
     "mi355_w4a16_prepacked_size": [ctypes.c_int64] * 3,
     "mi355_w4a16_prepack": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
                             ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p],

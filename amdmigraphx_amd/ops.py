@@ -85,7 +85,7 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
     ta, lda = _mat_layout(a3)
     tb, ldb = _mat_layout(b3)
     dequant = scale_a is not None or scale_b is not None or out_dtype is not None
-    in_type = DT.BF8 if fp8 == "e5m2" else DT.FP8 if fp8 else (DT.U8 if a.dtype == torch.uint8 else DT.I8)
+    in_type = _fp8_dt(fp8, a)
     if dequant:
         odt = out_dtype or torch.float32
     else:
@@ -139,6 +139,54 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
         st = lib().mi355_quant_dot(ctypes.byref(d), _ptr(a3), _ptr(b3), _ptr(out), _ptr(scale_a),
                                    _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _stream())
         check(st, "mi355_quant_dot")
+    return out
+
+
+def _fp8_dt(fp8, t):
+    return DT.BF8 if fp8 == "e5m2" else DT.FP8 if fp8 else (DT.U8 if t.dtype == torch.uint8 else DT.I8)
+
+
+def quant_dot_prepack(b, fp8=False):
+    """Reorder a constant B [K, N] (any strides: a transposed view is read as it lies) once, for
+    quant_dot_prepacked.  Returns None for a shape or type the reordered form does not take."""
+    _require_cuda(b)
+    if b.dim() != 2:
+        raise Mi355Error("quant_dot_prepack: B is a matrix")
+    k, n = b.shape
+    it = _fp8_dt(fp8, b)
+    size = lib().mi355_quant_dot_prepacked_size(it, n, k)
+    if size == 0:
+        return None
+    out = torch.empty(size, dtype=torch.uint8, device=b.device)
+    check(lib().mi355_quant_dot_prepack(_ptr(b), it, n, k, b.stride(0), b.stride(1), _ptr(out), _stream()),
+          "mi355_quant_dot_prepack")
+    return out
+
+
+def quant_dot_prepacked(a, b_prepacked, n, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
+                        colsum_b=None, rowsum_a=None, out_dtype=None, out=None, bias=None):
+    """quant_dot of a [M <= 16, K] against a B reordered by quant_dot_prepack, with the epilogue
+    arguments of quant_dot; one launch, no workspace."""
+    _require_cuda(a, b_prepacked, scale_a, scale_b, bias)
+    if a.dim() != 2 or a.stride(1) != 1:
+        raise Mi355Error("quant_dot_prepacked: A is a row-major matrix")
+    m, k = a.shape
+    dequant = scale_a is not None or scale_b is not None or out_dtype is not None
+    odt = (out_dtype or torch.float32) if dequant else (torch.float32 if fp8 else torch.int32)
+    if out is None:
+        out = torch.empty((m, n), dtype=odt, device=a.device)
+    d = QuantDotDesc(m=m, n=n, k=k, lda=a.stride(0) if m > 1 else max(k, a.stride(0)), ldb=n,
+                     ldc=out.stride(0) if m > 1 else max(n, out.stride(0)), batch=1, stride_a=0, stride_b=0,
+                     stride_c=0, trans_a=0, trans_b=0, in_type=_fp8_dt(fp8, a), out_type=_TORCH2DT[out.dtype],
+                     dequant=int(dequant),
+                     scale_a_mode=QP.NONE if scale_a is None else
+                     (QP.PER_TENSOR if scale_a.numel() == 1 else QP.PER_ROW),
+                     scale_b_mode=QP.NONE if scale_b is None else
+                     (QP.PER_TENSOR if scale_b.numel() == 1 else QP.PER_COL),
+                     zp_a=int(zp_a), zp_b=int(zp_b))
+    check(lib().mi355_quant_dot_prepacked(ctypes.byref(d), _ptr(a), _ptr(b_prepacked), _ptr(out), _ptr(scale_a),
+                                          _ptr(scale_b), _ptr(colsum_b), _ptr(rowsum_a), _ptr(bias), _stream()),
+          "mi355_quant_dot_prepacked")
     return out
 
 

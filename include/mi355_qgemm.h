@@ -423,6 +423,33 @@ int mi355_w4a16_gemm_prepacked(const void* a, int64_t lda,
                                void* stream);
 
 /*
+ * quant_dot (+ fused dequantizelinear) of a few rows against a constant B reordered once ahead of
+ * time (a target does this when it compiles the program: the weights of a linear layer are
+ * literals).  mi355_quant_dot_prepack writes B -- addressed as b[k * stride_k + n * stride_n], so
+ * [K, N] and [N, K] sources need no copy -- into a device buffer of mi355_quant_dot_prepacked_size
+ * bytes (the size of B) as the 16-column x 64-k operand tiles of the matrix-core instruction;
+ * mi355_quant_dot_prepacked then computes what mi355_quant_dot_bias computes for the same
+ * descriptor (same reference chain: src/targets/ref/lowering.cpp:218-248 -> src/gemm.cpp:42-63,
+ * the epilogue of simplify_qdq.cpp:225-289) in one launch without a workspace: bit-identical for
+ * int8, within the fp8 tolerance for fp8 (its own fixed summation order).  desc->trans_b, ldb and
+ * stride_b are not read.
+ * Shapes: M <= 16, N % 16 == 0, K % 64 == 0, one batch, A row-major with lda % 16 == 0 and a
+ * 16-byte aligned base (otherwise MI355_ERR_UNSUPPORTED: the caller keeps mi355_quant_dot_bias).
+ * mi355_quant_dot_prepacked_size returns 0 for an N, K or element type the reordered form does
+ * not take.
+ */
+size_t mi355_quant_dot_prepacked_size(int32_t in_type, int64_t n, int64_t k);
+int mi355_quant_dot_prepack(const void* b, int32_t in_type, int64_t n, int64_t k,
+                            int64_t stride_k, int64_t stride_n,
+                            void* prepacked, void* stream);
+int mi355_quant_dot_prepacked(const mi355_quant_dot_desc* desc,
+                              const void* a, const void* b_prepacked, void* c,
+                              const float* scale_a, const float* scale_b,
+                              const int32_t* colsum_b, const int32_t* rowsum_a,
+                              const float* bias,
+                              void* stream);
+
+/*
  * Float dot: C[b, m, n] = T( sum_k double(A[b, m, k]) * double(B[b, k, n]) ), k ascending,
  * T in {F32, F16, BF16} for all three tensors (16-bit results truncate, as the software
  * floats do).
