@@ -170,6 +170,54 @@ struct quant_dot
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// A constant B of a quant_dot reordered once into the matrix-core operand tiles
+// (mi355_quant_dot_prepack).  inputs: b [K, N] (any matrix view), out uint8 [N * K]
+struct quant_dot_prepack
+{
+    template <class Self, class F>
+    static void reflect(Self&, F)
+    {
+    }
+    std::string name() const { return "mi355::quant_dot_prepack"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
+// mi355::quant_dot of at most 16 rows against a reordered B (mi355_quant_dot_prepacked): the
+// attributes and inputs of mi355::quant_dot without the workspace, the second input being the
+// uint8 buffer mi355::quant_dot_prepack wrote.
+struct quant_dot_prepacked
+{
+    bool dequant           = false;
+    bool has_bias          = false;
+    int64_t zp_a           = 0;
+    int64_t zp_b           = 0;
+    int64_t scale_a_mode   = MI355_QP_NONE;
+    int64_t scale_b_mode   = MI355_QP_NONE;
+    shape::type_t out_type = shape::int32_type;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.dequant, "dequant");
+        f(self.has_bias, "has_bias");
+        f(self.zp_a, "zp_a");
+        f(self.zp_b, "zp_b");
+        f(self.scale_a_mode, "scale_a_mode");
+        f(self.scale_b_mode, "scale_b_mode");
+        f(self.out_type, "out_type");
+    }
+    std::string name() const { return "mi355::quant_dot_prepacked"; }
+    std::size_t expected_inputs() const
+    {
+        return 3 + (dequant ? 2 : 0) + (zp_a != 0 ? 1 : 0) + (zp_b != 0 ? 1 : 0) + (has_bias ? 1 : 0);
+    }
+    mi355_quant_dot_desc describe(const shape& a, const shape& out) const;
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: x [N, C, D, H, W], [N, C, H, W] or [N, C, W], weights [O, C / group, window...] (both dense),
 // [scale_x (one float), scale_w (one float or one per output channel)] (dequant),
 // workspace (uint8, the size mi355_quant_convolution3d_dims reports), out

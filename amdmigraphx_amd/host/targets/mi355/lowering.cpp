@@ -697,6 +697,87 @@ void prepack_w4a16(module& m)
     }
 }
 
+// ---- quant_dot of a few rows against a constant B -> the reordered form --------------------------
+//
+// A linear layer applied to at most 16 rows (decoding, small batches) is a stream of its weight
+// matrix.  When B is built from literals only, mi355::quant_dot_prepack -- folded when the program
+// is compiled, like the step above -- stores it as the matrix-core operand tiles, and
+// mi355::quant_dot_prepacked computes the layer in one launch, without the split-K workspace and
+// its second kernel.  Taken: one batch, A dense [M <= 16, K], the shapes
+// mi355_quant_dot_prepacked_size accepts; everything else stays on mi355::quant_dot.
+bool built_from_literals(instruction_ref ins, std::unordered_map<const instruction*, bool>& seen)
+{
+    auto it = seen.find(&*ins);
+    if(it != seen.end())
+        return it->second;
+    bool r = false;
+    if(ins->name() == "@literal" or ins->name() == "mi355::literal")
+        r = true;
+    else if(ins->name()[0] != '@' and ins->name() != "mi355::allocate" and not ins->inputs().empty())
+    {
+        r = true;
+        for(auto i : ins->inputs())
+        {
+            if(i->name() == "mi355::allocate")
+                continue;
+            r = r and built_from_literals(i, seen);
+        }
+    }
+    seen[&*ins] = r;
+    return r;
+}
+
+// Off unless MIGRAPHX_MI355_PREPACK_QUANT_DOT is set (to anything but 0) when a program is compiled.
+// The kernels behind the two operators pass their own tests on the device, called through the C
+// interface; the one device run of programs compiled with this step ended with the device
+// reporting a fault before the test had printed anything, and reading the code has not shown a
+// cause.  Until one is shown, a program keeps mi355::quant_dot (and its split-K workspace) for
+// these layers.
+bool prepack_quant_dot_enabled()
+{
+    const char* v = std::getenv("MIGRAPHX_MI355_PREPACK_QUANT_DOT");
+    return v != nullptr and std::string(v) != "0" and std::string(v) != "";
+}
+
+void prepack_quant_dot(module& m)
+{
+    std::unordered_map<const instruction*, bool> seen;
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "mi355::quant_dot")
+            continue;
+        const auto op = any_cast<quant_dot>(ins->get_operator());
+        auto inputs   = ins->inputs();
+        auto a        = inputs[0];
+        auto b        = inputs[1];
+        const auto& as = a->get_shape();
+        const auto& bs = b->get_shape();
+        if(as.ndim() != 2 or bs.ndim() != 2 or not as.standard() or as.lens()[0] > 16)
+            continue;
+        if(as.type() == shape::uint8_type or not view_as_matrix(bs).ok)
+            continue;
+        const size_t bytes =
+            mi355_quant_dot_prepacked_size(to_mi355_type(as.type()), bs.lens()[1], bs.lens()[0]);
+        if(bytes == 0 or not built_from_literals(b, seen))
+            continue;
+        quant_dot_prepacked pre;
+        pre.dequant      = op.dequant;
+        pre.has_bias     = op.has_bias;
+        pre.zp_a         = op.zp_a;
+        pre.zp_b         = op.zp_b;
+        pre.scale_a_mode = op.scale_a_mode;
+        pre.scale_b_mode = op.scale_b_mode;
+        pre.out_type     = op.out_type;
+        auto room   = insert_allocation(m, ins, shape{shape::uint8_type, {bytes}});
+        auto packed = m.insert_instruction(ins, operation{quant_dot_prepack{}}, b, room);
+        std::vector<instruction_ref> args = inputs;
+        args[1] = packed;
+        if(op.workspace) // the buffer in front of the output
+            args.erase(args.end() - 2);
+        m.replace_instruction(ins, operation{pre}, args);
+    }
+}
+
 // MIGRAPHX_MI355_FP32_DOT set (to anything but 0) when a program is compiled: float `dot`s run on
 // the fp32 matrix cores instead of reproducing the reference's double sum bit for bit
 bool fp32_dot_requested()
@@ -1372,6 +1453,11 @@ void lowering::apply(module& m) const
     for(auto ins : all_instructions(m))
         lower_instruction(m, ins);
     dead_code_elimination{}.apply(m);
+    if(prepack_quant_dot_enabled())
+    {
+        prepack_quant_dot(m);
+        dead_code_elimination{}.apply(m);
+    }
     // 3. literals live in device memory
     for(auto ins : all_instructions(m))
     {

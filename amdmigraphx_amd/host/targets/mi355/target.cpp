@@ -372,6 +372,115 @@ argument quant_dot::compute(migraphx::context& ctx, const shape&, const std::vec
     return args.back();
 }
 
+shape quant_dot_prepack::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    const shape& b = inputs[0];
+    const auto vb  = view_as_matrix(b);
+    if(b.ndim() != 2 or not vb.ok)
+        MIGRAPHX_THROW("mi355::quant_dot_prepack: B is a row-major or transposed matrix");
+    const size_t bytes = mi355_quant_dot_prepacked_size(to_mi355_type(b.type()), vb.cols, vb.rows);
+    if(bytes == 0)
+        MIGRAPHX_THROW("mi355::quant_dot_prepack: the reordered form does not take this shape");
+    shape out{shape::uint8_type, {bytes}};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::quant_dot_prepack: output buffer has the wrong size");
+    return out;
+}
+
+argument quant_dot_prepack::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const shape& b = args[0].get_shape();
+    const auto vb  = view_as_matrix(b);
+    status_check(mi355_quant_dot_prepack(args[0].data(),
+                                         to_mi355_type(b.type()),
+                                         vb.cols,
+                                         vb.rows,
+                                         vb.trans ? 1 : vb.ld,
+                                         vb.trans ? vb.ld : 1,
+                                         args.back().data(),
+                                         stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
+mi355_quant_dot_desc quant_dot_prepacked::describe(const shape& a, const shape& out) const
+{
+    mi355_quant_dot_desc d{};
+    d.m        = static_cast<int64_t>(a.lens()[0]);
+    d.k        = static_cast<int64_t>(a.lens()[1]);
+    d.n        = static_cast<int64_t>(out.lens()[1]);
+    d.lda      = d.k;
+    d.ldb      = d.n;
+    d.ldc      = d.n;
+    d.batch    = 1;
+    d.in_type  = to_mi355_type(a.type());
+    d.out_type = to_mi355_type(out_type);
+    d.dequant  = dequant ? 1 : 0;
+    d.scale_a_mode = static_cast<int32_t>(scale_a_mode);
+    d.scale_b_mode = static_cast<int32_t>(scale_b_mode);
+    d.zp_a         = static_cast<int32_t>(zp_a);
+    d.zp_b         = static_cast<int32_t>(zp_b);
+    return d;
+}
+
+shape quant_dot_prepacked::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, expected_inputs(), name());
+    const shape& a   = inputs[0];
+    const shape& out = inputs.back();
+    if(a.ndim() != 2 or not a.standard() or out.ndim() != 2 or not out.standard() or out.lens()[0] != a.lens()[0])
+        MIGRAPHX_THROW("mi355::quant_dot_prepacked: A and the output are dense matrices with the same rows");
+    if(a.lens()[0] > 16)
+        MIGRAPHX_THROW("mi355::quant_dot_prepacked: takes at most 16 rows");
+    if(inputs[1].type() != shape::uint8_type or
+       inputs[1].elements() != mi355_quant_dot_prepacked_size(to_mi355_type(a.type()), out.lens()[1], a.lens()[1]) or
+       inputs[1].elements() == 0)
+        MIGRAPHX_THROW("mi355::quant_dot_prepacked: the reordered B does not fit the operands");
+    const bool fp8 = a.type() != shape::int8_type;
+    if(out.type() != out_type or (not dequant and out_type != (fp8 ? shape::float_type : shape::int32_type)))
+        MIGRAPHX_THROW("mi355::quant_dot_prepacked: output buffer has the wrong type");
+    if(dequant)
+    {
+        if(out_type != shape::float_type and out_type != shape::half_type and out_type != shape::bf16_type)
+            MIGRAPHX_THROW("mi355::quant_dot_prepacked: dequantized output must be float, half or bf16");
+        if(inputs[2].type() != shape::float_type or inputs[3].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::quant_dot_prepacked: scales must be float");
+        if((zp_a != 0 or zp_b != 0) and fp8)
+            MIGRAPHX_THROW("mi355::quant_dot_prepacked: zero points need int8 operands");
+    }
+    if(has_bias)
+    {
+        const shape& bias = inputs[inputs.size() - 2];
+        if(not dequant or bias.type() != shape::float_type or not bias.standard() or
+           bias.elements() != out.lens()[1])
+            MIGRAPHX_THROW("mi355::quant_dot_prepacked: the bias is a dense float vector of N elements behind "
+                           "the dequantizing epilogue");
+    }
+    return out;
+}
+
+argument
+quant_dot_prepacked::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    const auto d     = describe(args[0].get_shape(), args.back().get_shape());
+    std::size_t next = 2;
+    const float* sa  = nullptr;
+    const float* sb  = nullptr;
+    if(dequant)
+    {
+        sa = reinterpret_cast<const float*>(args[next++].data());
+        sb = reinterpret_cast<const float*>(args[next++].data());
+    }
+    const int32_t* colsum_b = zp_a != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
+    const int32_t* rowsum_a = zp_b != 0 ? reinterpret_cast<const int32_t*>(args[next++].data()) : nullptr;
+    const float* bias = has_bias ? reinterpret_cast<const float*>(args[next++].data()) : nullptr;
+    status_check(mi355_quant_dot_prepacked(
+                     &d, args[0].data(), args[1].data(), args.back().data(), sa, sb, colsum_b, rowsum_a, bias, stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
 mi355_quant_conv3d_desc quant_convolution::describe(const shape& x, const shape& w) const
 {
     const std::size_t kd = stride.size();
@@ -1372,6 +1481,8 @@ MIGRAPHX_REGISTER_OP(mi355::dot);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot_mx);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_prepack);
+MIGRAPHX_REGISTER_OP(mi355::quant_dot_prepack);
+MIGRAPHX_REGISTER_OP(mi355::quant_dot_prepacked);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm_prepacked);
 MIGRAPHX_REGISTER_OP(mi355::quantizelinear);
 MIGRAPHX_REGISTER_OP(mi355::dequantizelinear);

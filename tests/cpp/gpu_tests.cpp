@@ -302,6 +302,84 @@ TEST_CASE(qdq_linear_layer_skinny)
     }
 }
 
+TEST_CASE(qdq_linear_layer_reordered_weights)
+{
+    // needs the lowering step that MIGRAPHX_MI355_PREPACK_QUANT_DOT switches on (off by default)
+    if(std::getenv("MIGRAPHX_MI355_PREPACK_QUANT_DOT") == nullptr)
+    {
+        std::cout << "skipped: MIGRAPHX_MI355_PREPACK_QUANT_DOT is not set" << std::endl;
+        return;
+    }
+    // A few rows against a large weight matrix (decoding, small batches).  Up to 16 rows against
+    // constant weights: the weights are reordered when the program is compiled and the layer is
+    // one launch of mi355::quant_dot_prepacked.  More rows (or shapes the reordered form does not
+    // take): the lowering hands mi355::quant_dot a workspace so that K is split over the chip, the
+    // second kernel applies the epilogue; a layer with a short K gets no workspace.  All
+    // bit-identical to the CPU target.
+    struct layer
+    {
+        std::size_t m, k, n;
+        int zp_x, zp_w;
+        bool weight_nk, skinny, reordered;
+        shape::type_t type;
+    };
+    for(auto c : {layer{16, 4096, 1024, 0, 0, true, true, true, shape::float_type},
+                  layer{1, 2048, 512, 0, 0, false, true, true, shape::float_type},
+                  layer{5, 1600, 304, 3, -2, false, true, true, shape::half_type},
+                  layer{16, 1608, 304, 0, 0, false, true, false, shape::float_type},
+                  layer{40, 1600, 304, 3, -2, false, true, false, shape::float_type},
+                  layer{128, 3072, 768, 0, 0, true, true, false, shape::half_type},
+                  layer{2048, 256, 1024, 0, 0, true, false, false, shape::float_type}})
+    {
+        auto p = qdq_matmul(c.m, c.k, c.n, c.weight_nk, c.zp_x, c.zp_w, c.type, 31);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        const auto& mod = *compiled.get_main_module();
+        EXPECT(count_ops(mod, "mi355::quant_dot_prepacked") == (c.reordered ? 1 : 0));
+        EXPECT(count_ops(mod, "mi355::quant_dot") == (c.reordered ? 0 : 1));
+        EXPECT(count_ops(mod, "mi355::quant_dot_prepack") == 0); // ran when the program was compiled
+        for(auto ins = mod.begin(); ins != mod.end(); ++ins)
+        {
+            if(ins->name() != "mi355::quant_dot")
+                continue;
+            EXPECT(ins->get_operator().to_value().at("workspace").to<bool>() == c.skinny);
+        }
+        argument x{shape{c.type, {c.m, c.k}}, normal_floats(c.m * c.k, 1.0f, 32)};
+        expect_same(p, {{"x", x}});
+        // and after a round trip through a file
+        if(c.reordered)
+        {
+            const std::string file = "/tmp/mi355_skinny_layer.mxr";
+            migraphx::save(compiled, file);
+            auto loaded = migraphx::load(file);
+            auto r1 = compiled.eval({{"x", x}});
+            auto r2 = loaded.eval({{"x", x}});
+            EXPECT(same_bytes(r1[0], r2[0]));
+            std::remove(file.c_str());
+        }
+    }
+    // the bare product: int32 from int8 for few rows against a constant B, a variable B, more rows
+    for(std::size_t rows : {12, 24})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        auto a   = mm->add_parameter("a", shape{shape::int8_type, {rows, 2048}});
+        auto b   = mm->add_literal(literal{shape{shape::int8_type, {2048, 640}}, uniform_ints<std::int8_t>(2048 * 640, -128, 127, 33)});
+        auto bv  = mm->add_parameter("b", shape{shape::int8_type, {2048, 640}});
+        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b), mm->add_instruction(make_op("quant_dot"), a, bv)});
+        argument av{shape{shape::int8_type, {rows, 2048}}, uniform_ints<std::int8_t>(rows * 2048, -128, 127, 34)};
+        argument bb{shape{shape::int8_type, {2048, 640}}, uniform_ints<std::int8_t>(2048 * 640, -128, 127, 35)};
+        expect_same(p, {{"a", av}, {"b", bb}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot_prepacked") == (rows <= 16 ? 1 : 0));
+        for(auto ins = compiled.get_main_module()->begin(); ins != compiled.get_main_module()->end(); ++ins)
+            if(ins->name() == "mi355::quant_dot")
+                EXPECT(ins->get_operator().to_value().at("workspace").to<bool>());
+    }
+}
+
 // QDQ-wrapped convolution as a quantized ONNX model holds it: X float -> Q/DQ (one scale), W int8
 // literal -> DQ with one scale per output channel, convolution of the two dequantized tensors
 static program qdq_conv(std::vector<std::size_t> xl,
