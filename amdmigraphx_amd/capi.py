@@ -137,6 +137,7 @@ EXPORTS = {
                                 ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p],
     "mi355_quant_dot_prepacked": [ctypes.c_void_p] * 10,
     "mi355_w4a16_prepacked_size": [ctypes.c_int64] * 3,
+    "mi355_w4a16_prepacked_max_rows": [ctypes.c_int64] * 3,
     "mi355_w4a16_prepack": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_int64,
                             ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p],
     "mi355_w4a16_gemm_prepacked": [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
@@ -178,6 +179,7 @@ def lib():
             fn.argtypes = argtypes
             fn.restype = (ctypes.c_char_p if name == "mi355_status_string" else
                           ctypes.c_size_t if name.endswith("_workspace_size") or name.endswith("_prepacked_size")
+                          else ctypes.c_int64 if name.endswith("_max_rows")
                           else ctypes.c_int)
         _handle = h
     return _handle

@@ -131,6 +131,12 @@ struct w4p_params
     int iters_r;         // row groups per team
     int rg_stride;       // distance between a team's row groups
     int rg_base;         // first row group of this launch
+    // several activation rows (the MR = 16 kernels)
+    int m;               // activation rows, 1 .. 16
+    int lda, ldc;        // halves between rows of a and of out
+    int a_pitch;         // bytes between activation rows in the LDS: 2 k + 16
+    uint32_t row_magic;  // i / (k / 8)        = umulhi(i, row_magic)   for the piece numbers staged
+    uint32_t all_magic;  // i / (m * (k / 8))  = umulhi(i, all_magic)
 };
 
 
@@ -277,10 +283,13 @@ MI355_DEVINL const uint8_t* w4p_block_at(const w4p_params& p, int rg0, int w, in
     return p.pk + W4P_HEADER + ((int64_t)rg * p.nss + s) * W4P_BLOCK;
 }
 
-template <bool FAST, int IR, int IS>
+template <bool FAST, int MR, int IR, int IS>
 MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* zeros, float* red, int rg0, int team,
                              int w, int lane, int zp)
 {
+    // MR = 16: lane l multiplies activation row l % 16 (rows past the last read the last one
+    // again: rows of the result tile that nobody stores)
+    const uint8_t* a_rows = MR == 1 ? lds : lds + min(lane & 15, p.m - 1) * p.a_pitch;
     constexpr int TOTAL = IR * IS;
     static_assert(TOTAL >= 1 && TOTAL <= 4);
     const int zp_log2 = zp <= 1 ? 0 : (zp == 2 ? 1 : (zp == 4 ? 2 : 3));
@@ -302,7 +311,7 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
         const int rg           = rg0 + (IDX / IS) * p.rg_stride;
         const int s            = w + (IDX % IS) * p.wk;
         const bool live        = rg < p.nrg && s < p.nss;
-        const uint8_t* a_block = live || !FAST ? lds + s * 1024 + (lane >> 4) * 256 : zeros;
+        const uint8_t* a_block = live || !FAST ? a_rows + s * 1024 + (lane >> 4) * 256 : zeros;
         w4p_wait_piece<3 + NEXT>(b.w[0], b.sb);
         const w4p_consts c = w4p_scale_consts<FAST>(b.sb, zp, zp_log2);
         if(FAST || live)
@@ -316,7 +325,34 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
         w4p_wait_piece<0 + NEXT>(b.w[3]);
         if(FAST || live)
             w4p_piece<FAST>(b.w[3], c, a_block + 192, acc);
-        if constexpr(IDX % IS == IS - 1)
+        if constexpr(IDX % IS == IS - 1 && MR != 1)
+        {
+            // the whole result tile: lane l holds column l % 16 (a weight row) of activation rows
+            // 4 * (l / 16) .. + 3.  One buffer for the partial sums, so a second barrier keeps the
+            // next row group's sums out of it until the first wave has read these.
+            const v4f mine = (acc[0] + acc[1]) + (acc[2] + acc[3]) * (FAST ? 16.0f : 1.0f);
+            v4f* slot      = reinterpret_cast<v4f*>(red) + team * p.wk * 64;
+            slot[w * 64 + lane] = mine;
+            __syncthreads();
+            if(w == 0 && rg < p.nrg)
+            {
+                v4f sum = slot[lane];
+                for(int j = 1; j < p.wk; j++)
+                    sum += slot[j * 64 + lane];
+#pragma unroll
+                for(int r = 0; r < 4; r++)
+                {
+                    const int row = 4 * (lane >> 4) + r;
+                    if(row < p.m)
+                        p.out[(int64_t)row * p.ldc + rg * 16 + (lane & 15)] = f32_to_half_rtz(sum[r]);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for(int c2 = 0; c2 < 4; c2++)
+                acc[c2] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        else if constexpr(IDX % IS == IS - 1)
         {
             // row 0 of the result tile: register 0 of lanes 0..15
             const float mine = (acc[0][0] + acc[1][0]) + (acc[2][0] + acc[3][0]) * (FAST ? 16.0f : 1.0f);
@@ -355,7 +391,7 @@ MI355_DEVINL void w4p_blocks(const w4p_params& p, uint8_t* lds, const uint8_t* z
 // barrier.  A CU takes load instructions only at the rate the memory returns data, so a wave with
 // many loads to issue sits at its issue for microseconds; with the weights' loads in front of the
 // barrier the workgroup could not start to multiply until its last wave had issued its last load.
-template <int SLOTS, int IR, int IS>
+template <int MR, int SLOTS, int IR, int IS>
 __global__ __launch_bounds__(W4P_MAX_WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 w4p_gemv_kernel(w4p_params p)
 {
@@ -370,7 +406,7 @@ w4p_gemv_kernel(w4p_params p)
         team++;
     }
     const int nthreads = p.teams * p.wk * 64;
-    uint8_t* zeros     = lds + p.k * 2;                           // 256 bytes
+    uint8_t* zeros     = lds + (MR == 1 ? p.k * 2 : p.m * p.a_pitch); // 256 bytes
     float* red         = reinterpret_cast<float*>(zeros + 256);
 
     // half-precision arithmetic of this wave truncates from here on (MODE.fp_round bits 3:2); the
@@ -382,16 +418,32 @@ w4p_gemv_kernel(w4p_params p)
     uint64_t zp_flags;
     asm volatile("s_load_dwordx2 %0, %1, 0x10" : "=s"(zp_flags) : "s"(p.pk) : "memory");
 
-    // The activation row: loads and LDS stores are unconditional with the piece index clamped
-    // (threads past the end store the last piece once more).
-    const int a_pieces = p.k >> 3;
+    // The activations, 16-byte pieces: loads and LDS stores are unconditional.  A thread past the
+    // end takes piece (number mod count) once more -- not one fixed piece: the same 16 bytes asked
+    // for by half the threads of every workgroup on the chip queue up at one cache channel.
+    const int row_pieces = p.k >> 3;
+    const int a_pieces   = MR == 1 ? row_pieces : p.m * row_pieces;
     v4u areg[SLOTS];
-    int apiece[SLOTS];
+    int aslot[SLOTS]; // byte offset of the piece in the LDS
 #pragma unroll
     for(int s = 0; s < SLOTS; s++)
     {
-        apiece[s] = min(tid + s * nthreads, a_pieces - 1);
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(areg[s]) : "v"(apiece[s] * 16), "s"(p.a) : "memory");
+        int i = tid + s * nthreads;
+        i -= (int)__umulhi((uint32_t)i, p.all_magic) * a_pieces;
+        int goff;
+        if constexpr(MR == 1)
+        {
+            goff     = i * 16;
+            aslot[s] = i * 16;
+        }
+        else
+        {
+            const int row = (int)__umulhi((uint32_t)i, p.row_magic);
+            const int col = i - row * row_pieces;
+            goff          = row * p.lda * 2 + col * 16;
+            aslot[s]      = row * p.a_pitch + col * 16;
+        }
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(areg[s]) : "v"(goff), "s"(p.a) : "memory");
     }
     const int rg0 = p.rg_base + blockIdx.x * p.teams + team;
     if(tid < 16)
@@ -400,11 +452,18 @@ w4p_gemv_kernel(w4p_params p)
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(areg[0])::"memory");
     else if constexpr(SLOTS == 2)
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(areg[0]), "+v"(areg[1])::"memory");
-    else
+    else if constexpr(SLOTS == 4)
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(areg[0]), "+v"(areg[1]), "+v"(areg[2]), "+v"(areg[3])::"memory");
+    else
+    {
+        static_assert(SLOTS == 8);
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(areg[0]), "+v"(areg[1]), "+v"(areg[2]), "+v"(areg[3]), "+v"(areg[4]), "+v"(areg[5]),
+                       "+v"(areg[6]), "+v"(areg[7])::"memory");
+    }
 #pragma unroll
     for(int s = 0; s < SLOTS; s++)
-        *reinterpret_cast<v4u*>(lds + apiece[s] * 16) = areg[s];
+        *reinterpret_cast<v4u*>(lds + aslot[s]) = areg[s];
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(zp_flags)::"memory");
     const uint32_t flags = (uint32_t)(zp_flags >> 32);
     const int zp         = (int)(uint32_t)zp_flags;
@@ -413,17 +472,28 @@ w4p_gemv_kernel(w4p_params p)
     // two separate bodies, each with its own loads and waits: a wait statement in each of two
     // branches for one load makes the compiler copy the loaded register in front of the branch
     if(__builtin_amdgcn_readfirstlane((flags & W4P_FLAG_GENERAL) == 0))
-        w4p_blocks<true, IR, IS>(p, lds, zeros, red, rg0, team, w, lane, zp);
+        w4p_blocks<true, MR, IR, IS>(p, lds, zeros, red, rg0, team, w, lane, zp);
     else
-        w4p_blocks<false, IR, IS>(p, lds, zeros, red, rg0, team, w, lane, zp);
+        w4p_blocks<false, MR, IR, IS>(p, lds, zeros, red, rg0, team, w, lane, zp);
 }
 
-template <int SLOTS>
-void w4p_launch(const w4p_params& p, int grid, int threads, int lds, hipStream_t s)
+template <int MR, int SLOTS>
+int w4p_launch(const w4p_params& p, int grid, int threads, int lds, hipStream_t s)
 {
 #define W4P_CASE(R, S)                                                                                    \
     if(p.iters_r == R && p.iters_s == S)                                                                  \
-        hipLaunchKernelGGL((w4p_gemv_kernel<SLOTS, R, S>), dim3(grid), dim3(threads), lds, s, p);
+    {                                                                                                     \
+        auto kern = w4p_gemv_kernel<MR, SLOTS, R, S>;                                                     \
+        if(lds > 64 * 1024)                                                                               \
+        {                                                                                                 \
+            /* above the default limit: opt in once per kernel instantiation */                          \
+            static const hipError_t attr = hipFuncSetAttribute(                                           \
+                reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if(attr != hipSuccess)                                                                        \
+                return MI355_ERR_LAUNCH;                                                                  \
+        }                                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, s, p);                                   \
+    }
     W4P_CASE(1, 1)
     W4P_CASE(2, 1)
     W4P_CASE(3, 1)
@@ -433,6 +503,7 @@ void w4p_launch(const w4p_params& p, int grid, int threads, int lds, hipStream_t
     W4P_CASE(1, 3)
     W4P_CASE(1, 4)
 #undef W4P_CASE
+    return MI355_OK;
 }
 
 bool w4p_shape_ok(int64_t n, int64_t k, int64_t group)
@@ -448,6 +519,16 @@ extern "C" size_t mi355_w4a16_prepacked_size(int64_t n, int64_t k, int64_t group
     if(!w4p_shape_ok(n, k, group))
         return 0;
     return (size_t)W4P_HEADER + (size_t)(n / 16) * (size_t)(k / W4P_SUPER_K) * W4P_BLOCK;
+}
+
+// rows of activations the reordered form takes for this shape: one always; up to 16 as long as the
+// rows (2 k + 16 bytes each), 256 zero bytes and one result tile per wave (16 KiB) fit the LDS
+extern "C" int64_t mi355_w4a16_prepacked_max_rows(int64_t n, int64_t k, int64_t group)
+{
+    if(!w4p_shape_ok(n, k, group))
+        return 0;
+    const int64_t fit = (160 * 1024 - 256 - W4P_MAX_WAVES * 1024) / (2 * k + 16);
+    return fit < 1 ? 1 : (fit > 16 ? 16 : fit);
 }
 
 extern "C" int mi355_w4a16_prepack(const void* w_packed,
@@ -491,7 +572,11 @@ extern "C" int mi355_w4a16_gemm_prepacked(const void* a,
         return MI355_ERR_UNSUPPORTED;
     if(m == 0)
         return MI355_OK;
-    if(m != 1)
+    if(m > 16)
+        return MI355_ERR_UNSUPPORTED;
+    const bool rows = m > 1;
+    // several rows: 16-byte loads of every row, 32-bit byte offsets inside a
+    if(rows && (lda % 8 != 0 || lda * 2 * 16 >= (1ll << 31) || ldc * 16 >= (1ll << 31)))
         return MI355_ERR_UNSUPPORTED;
     w4p_params p;
     p.pk  = static_cast<const uint8_t*>(prepacked);
@@ -501,6 +586,14 @@ extern "C" int mi355_w4a16_gemm_prepacked(const void* a,
     p.k   = (int)k;
     p.nss = (int)(k / W4P_SUPER_K);
     p.nrg = (int)(n / 16);
+    p.m   = (int)m;
+    p.lda = (int)lda;
+    p.ldc = (int)ldc;
+    p.a_pitch = (int)(2 * k + 16);
+    const int row_pieces = (int)(k / 8);
+    const int a_pieces   = (int)m * row_pieces;
+    p.row_magic = (uint32_t)((((uint64_t)1 << 32) / (uint64_t)row_pieces) + 1);
+    p.all_magic = (uint32_t)((((uint64_t)1 << 32) / (uint64_t)a_pieces) + 1);
     // Waves per row group (they split its blocks) and row groups per workgroup.  Measured on the
     // shapes of a Llama-sized layer: two blocks per wave and row group beat one (half as many
     // waves at the workgroup's barriers, one sum per two blocks) as long as the chip still gets
@@ -511,20 +604,26 @@ extern "C" int mi355_w4a16_gemm_prepacked(const void* a,
         p.iters_s = 2;
     p.wk    = (p.nss + p.iters_s - 1) / p.iters_s;
     p.teams = (p.wk <= 4 && p.nrg >= 384) ? 2 : 1;
-    // the activation row is staged with W4P_A_SLOTS pieces per thread
-    while(p.k / 8 > W4P_A_SLOTS * p.teams * p.wk * 64 && (p.teams + 1) * p.wk <= W4P_MAX_WAVES)
+    // the activations are staged with at most W4P_A_SLOTS (several rows: 8) pieces per thread
+    const int max_slots = rows ? 8 : W4P_A_SLOTS;
+    while(a_pieces > max_slots * p.teams * p.wk * 64 && (p.teams + 1) * p.wk <= W4P_MAX_WAVES)
         p.teams++;
-    if(p.k / 8 > W4P_A_SLOTS * p.teams * p.wk * 64)
+    if(a_pieces > max_slots * p.teams * p.wk * 64)
         return MI355_ERR_UNSUPPORTED;
     const int threads  = p.teams * p.wk * 64;
-    const int lds      = p.k * 2 + 256 + 2 * p.teams * W4P_MAX_WAVES * 16 * 4;
+    // one row: the row, 256 zero bytes, two buffers of 16 partial sums per wave; several rows: the
+    // rows 2 k + 16 bytes apart, the zero bytes, one buffer of a whole result tile per wave
+    const int lds = rows ? (int)m * p.a_pitch + 256 + p.teams * p.wk * 1024
+                         : p.k * 2 + 256 + 2 * p.teams * W4P_MAX_WAVES * 16 * 4;
+    if(lds > 160 * 1024)
+        return MI355_ERR_UNSUPPORTED;
     const int wgs      = (p.nrg + p.teams - 1) / p.teams;
     // One resident set of workgroups (the kernel is built for 16 waves per CU), each walking up to
     // 4 / iters_s row groups; more rows than that take further launches over the rows behind.
     const int per_cu   = max(1, min(W4P_MAX_WAVES * 64 / threads, (160 * 1024) / lds));
     const int resident = 256 * per_cu;
     const int max_r    = 4 / p.iters_s;
-    const int slots    = (p.k / 8 + threads - 1) / threads;
+    const int slots    = (a_pieces + threads - 1) / threads;
     hipStream_t s      = static_cast<hipStream_t>(stream);
     for(int done = 0; done < wgs;)
     {
@@ -533,12 +632,21 @@ extern "C" int mi355_w4a16_gemm_prepacked(const void* a,
         const int grid = left <= resident * p.iters_r ? (left + p.iters_r - 1) / p.iters_r : resident;
         p.rg_stride    = grid * p.teams;
         p.rg_base      = done * p.teams;
-        if(slots <= 1)
-            w4p_launch<1>(p, grid, threads, lds, s);
+        int st;
+        if(rows && slots <= 2)
+            st = w4p_launch<16, 2>(p, grid, threads, lds, s);
+        else if(rows && slots <= 4)
+            st = w4p_launch<16, 4>(p, grid, threads, lds, s);
+        else if(rows)
+            st = w4p_launch<16, 8>(p, grid, threads, lds, s);
+        else if(slots <= 1)
+            st = w4p_launch<1, 1>(p, grid, threads, lds, s);
         else if(slots <= 2)
-            w4p_launch<2>(p, grid, threads, lds, s);
+            st = w4p_launch<1, 2>(p, grid, threads, lds, s);
         else
-            w4p_launch<W4P_A_SLOTS>(p, grid, threads, lds, s);
+            st = w4p_launch<1, W4P_A_SLOTS>(p, grid, threads, lds, s);
+        if(st != MI355_OK)
+            return st;
         done += grid * p.iters_r;
     }
     return mi355_launch_status();

@@ -346,7 +346,7 @@ struct w4a16_prepack
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
-// inputs: a fp16 [1, K], reordered weights uint8 [bytes], out fp16 [1, N]
+// inputs: a fp16 [M, K] (M <= mi355_w4a16_prepacked_max_rows), reordered weights uint8 [bytes], out fp16 [M, N]
 struct w4a16_gemm_prepacked
 {
     template <class Self, class F>

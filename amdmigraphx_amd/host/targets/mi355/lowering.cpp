@@ -663,13 +663,14 @@ void fuse_shared_w4a16(module& m)
     }
 }
 
-// ---- one-row weight-only products over constant weights -> the reordered form -------------------
+// ---- weight-only products of a few rows over constant weights -> the reordered form -------------
 //
-// With one row of activations the product is a stream of weights, and constant weights can lie in
+// With one row of activations (or a few: a small batch) the product is a stream of weights, and constant weights can lie in
 // memory in whatever order the kernel reads fastest.  mi355::w4a16_prepack writes that order; its
 // operands are literals, so it runs once when the program is compiled (constant folding, below)
 // and the program keeps only the reordered copy.  Taken: one zero point for the tensor, group size
-// 128 and the shapes mi355_w4a16_prepacked_size accepts; everything else stays on mi355::w4a16_gemm.
+// 128, the shapes mi355_w4a16_prepacked_size accepts and at most mi355_w4a16_prepacked_max_rows rows
+// (dense when more than one); everything else stays on mi355::w4a16_gemm.
 void prepack_w4a16(module& m)
 {
     for(auto ins : all_instructions(m))
@@ -680,7 +681,7 @@ void prepack_w4a16(module& m)
         auto a        = ins->inputs()[0];
         auto w        = ins->inputs()[1];
         auto s        = ins->inputs()[2];
-        if(op.zp_mode != MI355_W4_ZP_SCALAR or op.group != 128 or a->get_shape().lens()[0] != 1)
+        if(op.zp_mode != MI355_W4_ZP_SCALAR or op.group != 128)
             continue;
         if(not(w->can_eval() and w->get_shape().standard() and s->can_eval() and s->get_shape().standard()))
             continue;
@@ -688,6 +689,12 @@ void prepack_w4a16(module& m)
         const auto k       = static_cast<int64_t>(w->get_shape().lens()[1] * 2);
         const size_t bytes = mi355_w4a16_prepacked_size(n, k, op.group);
         if(bytes == 0)
+            continue;
+        // one row always; a few rows (small batches) while they fit the LDS, rows 16-byte aligned
+        const auto rows = static_cast<int64_t>(a->get_shape().lens()[0]);
+        if(rows > mi355_w4a16_prepacked_max_rows(n, k, op.group))
+            continue;
+        if(rows > 1 and not a->get_shape().standard())
             continue;
         w4a16_prepack pre;
         pre.zp_scalar = op.zp_scalar;

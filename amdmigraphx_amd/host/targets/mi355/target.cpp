@@ -917,8 +917,14 @@ shape w4a16_gemm_prepacked::compute_shape(const std::vector<shape>& inputs) cons
     const auto& out = inputs.back();
     if(a.type() != shape::half_type or out.type() != shape::half_type or inputs[1].type() != shape::uint8_type)
         MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: needs half activations and a uint8 buffer of reordered weights");
-    if(a.ndim() != 2 or out.ndim() != 2 or a.lens()[0] != 1 or out.lens()[0] != 1 or not out.standard())
-        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: takes one row of activations");
+    if(a.ndim() != 2 or out.ndim() != 2 or a.lens()[0] != out.lens()[0] or not out.standard() or
+       (a.lens()[1] > 1 and a.strides()[1] != 1))
+        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: needs row-major activations and a dense result with the same rows");
+    const auto max_rows =
+        mi355_w4a16_prepacked_max_rows(static_cast<int64_t>(out.lens()[1]), static_cast<int64_t>(a.lens()[1]), 128);
+    if(static_cast<int64_t>(a.lens()[0]) > max_rows)
+        MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: takes at most " + std::to_string(max_rows) +
+                       " rows of activations at this K");
     if(mi355_w4a16_prepacked_size(static_cast<int64_t>(out.lens()[1]), static_cast<int64_t>(a.lens()[1]), 128) !=
        inputs[1].bytes())
         MIGRAPHX_THROW("mi355::w4a16_gemm_prepacked: the reordered weights do not fit the operands");
@@ -928,10 +934,13 @@ shape w4a16_gemm_prepacked::compute_shape(const std::vector<shape>& inputs) cons
 argument
 w4a16_gemm_prepacked::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
 {
-    const auto k = static_cast<int64_t>(args[0].get_shape().lens()[1]);
-    const auto n = static_cast<int64_t>(out.lens()[1]);
+    const auto& a  = args[0].get_shape();
+    const auto m   = static_cast<int64_t>(a.lens()[0]);
+    const auto k   = static_cast<int64_t>(a.lens()[1]);
+    const auto n   = static_cast<int64_t>(out.lens()[1]);
+    const auto lda = m == 1 ? k : static_cast<int64_t>(a.strides()[0]);
     status_check(
-        mi355_w4a16_gemm_prepacked(args[0].data(), k, args[1].data(), args.back().data(), n, 1, n, k, stream_of(ctx)),
+        mi355_w4a16_gemm_prepacked(args[0].data(), lda, args[1].data(), args.back().data(), n, m, n, k, stream_of(ctx)),
         name());
     return args.back();
 }

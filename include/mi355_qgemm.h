@@ -406,13 +406,16 @@ int mi355_w4a16_gemm_ws(const void* a, int64_t lda,
  * with w = half((q - zp) * scale) exactly as mi355_w4a16_gemm does (same reference chain:
  * src/onnx/parse_matmulnbits.cpp:85-159, op/unpack_int4.hpp:75-121, op/dequantizelinear.hpp:60-83,
  * op/dot.hpp:102-107), within the same tolerance of the fp32 sum.
- * Shapes: group 128, N % 16 == 0, K % 512 == 0, K <= 28672, M == 1 (other M: MI355_ERR_UNSUPPORTED;
- * the caller keeps mi355_w4a16_gemm for them).  mi355_w4a16_prepacked_size returns 0 for a shape
+ * Shapes: group 128, N % 16 == 0, K % 512 == 0, K <= 28672, M <= mi355_w4a16_prepacked_max_rows (1 for
+ * any K; up to 16 while the rows fit the LDS: 16 at K <= 4096, 8 at K <= 8192, 4 at K <= 16384; rows
+ * of a 16-byte aligned with lda % 8 == 0); other M: MI355_ERR_UNSUPPORTED, the caller keeps
+ * mi355_w4a16_gemm for them.  Row r of a several-row call carries the bits of the one-row call on row r.  mi355_w4a16_prepacked_size returns 0 for a shape
  * the reordered form does not take.  Any scale values are accepted; the fastest form needs
  * 2^-10 <= scale < 2^-4 and a zero point of 0, 1, 2, 4 or 8, which the reordering checks on the
  * device and records in the buffer.
  */
 size_t mi355_w4a16_prepacked_size(int64_t n, int64_t k, int64_t group);
+int64_t mi355_w4a16_prepacked_max_rows(int64_t n, int64_t k, int64_t group);
 int mi355_w4a16_prepack(const void* w_packed, const void* scales, int32_t zp_scalar,
                         int64_t n, int64_t k, int64_t group,
                         void* prepacked, void* stream);

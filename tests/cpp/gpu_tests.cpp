@@ -920,9 +920,10 @@ TEST_CASE(int4_projections_sharing_activations)
         argument a{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 69)};
         program c = all;
         c.compile(migraphx::make_target("mi355"));
-        // (one row of activations: the stacked constant weights are reordered at compile time)
-        EXPECT(count_ops(*c.get_main_module(), m == 1 ? "mi355::w4a16_gemm_prepacked" : "mi355::w4a16_gemm") == 1);
-        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") + count_ops(*c.get_main_module(), "mi355::w4a16_gemm_prepacked") == 1);
+        // (one row or a few rows of activations: the stacked constant weights are reordered at
+        // compile time)
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm_prepacked") == 1);
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 0);
         auto got = run_on("mi355", all, {{"a", a}});
         EXPECT(got.size() == ns.size());
         for(std::size_t i = 0; i < ns.size(); i++)
@@ -963,7 +964,9 @@ TEST_CASE(int4_projections_with_odd_column_counts_are_not_stacked)
         mm->add_return(outs);
         program c = p;
         c.compile(migraphx::make_target("mi355"));
-        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 2);
+        // (the stacked pair has 160 columns and takes the reordered form, the odd one cannot)
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm") == 1);
+        EXPECT(count_ops(*c.get_main_module(), "mi355::w4a16_gemm_prepacked") == 1);
         argument av{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 169)};
         expect_close_half(p, {{"a", av}});
     }
@@ -971,11 +974,19 @@ TEST_CASE(int4_projections_with_odd_column_counts_are_not_stacked)
 
 TEST_CASE(int4_weight_only_gemm_small_batch)
 {
-    for(std::size_t m : {2, 16})
+    // constant weights, block size 128, a few rows that fit the LDS: the reordered form (as for one
+    // row); K = 8192 takes 8 rows of it, 16 rows stay on mi355::w4a16_gemm
+    for(auto mk : {std::pair<std::size_t, std::size_t>{2, 1024}, {16, 1024}, {8, 8192}, {16, 8192}})
     {
-        auto p = matmulnbits_program(m, 1024, 384, 128, false, shape::half_type, 50);
-        argument a{shape{shape::half_type, {m, 1024}}, normal_floats(m * 1024, 1.0f, 51)};
+        const std::size_t m = mk.first, k = mk.second;
+        auto p = matmulnbits_program(m, k, 384, 128, false, shape::half_type, 50);
+        argument a{shape{shape::half_type, {m, k}}, normal_floats(m * k, 1.0f, 51)};
         expect_close_half(p, {{"a", a}});
+        program c = p;
+        c.compile(migraphx::make_target("mi355"));
+        const bool reordered = not(m == 16 and k == 8192);
+        EXPECT(count_ops(*c.get_main_module(), reordered ? "mi355::w4a16_gemm_prepacked" : "mi355::w4a16_gemm") == 1);
+        EXPECT(not has_op(c, "mi355::w4a16_prepack"));
     }
     // per-block zero points packed two to a byte, block size 32
     auto p = matmulnbits_program(4, 512, 96, 32, true, shape::half_type, 52);

@@ -127,6 +127,59 @@ def test_prepacked_full_size_config4_against_oracle(ops, k, n):
     assert np.abs(orc.half_to_f32(gb) - orc.half_to_f32(ob)).max() < 0.05
 
 
+@pytest.mark.parametrize("m", [2, 5, 16])
+@pytest.mark.parametrize("n,k", [(16, 512), (64, 1024), (512, 4096), (272, 3584), (6160, 4096), (14336, 4096)])
+@pytest.mark.parametrize("zp", [8, 3])
+def test_prepacked_rows_match_oracle(ops, m, n, k, zp):
+    """2 .. 16 activation rows (each lane of the matrix-core operand its own row from the LDS),
+    every launch shape of the one-row tests that fits the LDS, both dequantization forms; rows of
+    a strided view."""
+    if m * (2 * k + 16) + 256 + 16384 > 160 * 1024:
+        pytest.skip("the rows do not fit the LDS")
+    rng = np.random.default_rng(m * 7 + n + k + zp)
+    _, packed, scales, wq = _case(rng, n, k)
+    a = orc.half_from_f32(rng.standard_normal((m, k)).astype(np.float32))
+    print("w4a16 prepacked rows", m, n, k, zp, flush=True)
+    pk = ops.w4a16_prepack(dev(packed), half_dev(scales), G, zp=zp)
+    got = ops.w4a16_gemm_prepacked(half_dev(a), pk, n)
+    wdq = _dequantized(wq, scales, zp)
+    if n * k <= 1 << 22:
+        want = orc.w4a16_matmul(a, packed, scales, zp, G)
+        _check(half_bits(got), want, a, wdq)
+    else:       # the oracle on sampled columns
+        cols = sorted(set(range(0, n, max(1, n // 97))) | {n - 1})
+        want = orc.w4a16_matmul(a, packed[cols], scales[cols], zp, G)
+        _check(half_bits(got)[:, cols], want, a, wdq[cols])
+    other = ops.w4a16_gemm(half_dev(a), dev(packed), half_dev(scales), G, zp=zp)
+    _check(half_bits(got), half_bits(other), a, wdq, identical=0.8)
+    # every row equals the one-row product of that row (same kernel arithmetic, same order)
+    for r in (0, m - 1):
+        one = ops.w4a16_gemm_prepacked(half_dev(a[r:r + 1]), pk, n)
+        assert np.array_equal(half_bits(one)[0], half_bits(got)[r])
+    # rows 24 halves apart in memory, output rows wider than N
+    wide = torch.zeros((m, k + 24), dtype=torch.float16, device="cuda")
+    wide[:, :k] = half_dev(a)
+    out = torch.zeros((m, n + 8), dtype=torch.float16, device="cuda")
+    ops.w4a16_gemm_prepacked(wide[:, :k], pk, n, out=out[:, :n])
+    assert np.array_equal(half_bits(out[:, :n]), half_bits(got)) and (out[:, n:] == 0).all()
+
+
+def test_prepacked_rows_dequantized_weights_are_exact(ops):
+    """one-hot activation rows, a different position per row: every output is one dequantized
+    weight, bit for bit"""
+    rng = np.random.default_rng(99)
+    n, k, m = 64, 1024, 16
+    _, packed, scales, wq = _case(rng, n, k)
+    for zp in (8, 5):
+        wdq = orc.half_to_f32(_dequantized(wq, scales, zp))
+        pk = ops.w4a16_prepack(dev(packed), half_dev(scales), G, zp=zp)
+        ks = rng.integers(0, k, m)
+        a = np.zeros((m, k), np.float32)
+        a[np.arange(m), ks] = 1.0
+        got = orc.half_to_f32(half_bits(ops.w4a16_gemm_prepacked(half_dev(orc.half_from_f32(a)), pk, n)))
+        assert np.array_equal(got, wdq[:, ks].T)
+
+
 def test_prepacked_form_declines_other_shapes(ops):
     from amdmigraphx_amd import Mi355Error
     w = torch.zeros((24, 256), dtype=torch.uint8, device="cuda")          # N % 16 != 0
@@ -139,5 +192,9 @@ def test_prepacked_form_declines_other_shapes(ops):
     s = torch.ones((32, 8), dtype=torch.float16, device="cuda")
     assert ops.w4a16_prepack(w, s, 64) is None
     pk = ops.w4a16_prepack(w, torch.ones((32, 4), dtype=torch.float16, device="cuda"), G)
-    with pytest.raises(Mi355Error):                                       # two rows: the other entry point's
-        ops.w4a16_gemm_prepacked(torch.zeros((2, 512), dtype=torch.float16, device="cuda"), pk, 32)
+    with pytest.raises(Mi355Error):                                       # 17 rows: the other entry point's
+        ops.w4a16_gemm_prepacked(torch.zeros((17, 512), dtype=torch.float16, device="cuda"), pk, 32)
+    w = torch.zeros((32, 8192), dtype=torch.uint8, device="cuda")         # 16 rows of K = 16384: more than the LDS
+    pk = ops.w4a16_prepack(w, torch.ones((32, 128), dtype=torch.float16, device="cuda"), G)
+    with pytest.raises(Mi355Error):
+        ops.w4a16_gemm_prepacked(torch.zeros((16, 16384), dtype=torch.float16, device="cuda"), pk, 32)
