@@ -643,15 +643,10 @@ instruction_ref parse_qlinearmatmul(const node_info& info, const std::vector<ins
 
 // src/onnx/parse_convolution.cpp:49-106 with the attribute rules of src/op/builder/convolution.cpp:62-113
 // and the SAME_UPPER / SAME_LOWER padding of src/pad_calc.cpp:31-53, :96-120 (static shapes)
-instruction_ref parse_conv(const node_info& info, const std::vector<instruction_ref>& args)
+migraphx::operation conv_operator(const node_info& info, instruction_ref x, instruction_ref w, const std::string& what)
 {
-    if(args.size() < 2 or args.size() > 3)
-        MIGRAPHX_THROW("Conv: two or three inputs expected");
-    module& m = *info.mod;
-    auto x    = args[0];
-    auto w    = args[1];
     if(x->get_shape().ndim() < 3 or w->get_shape().ndim() != x->get_shape().ndim())
-        MIGRAPHX_THROW("Conv: input and weights need the same rank of at least 3");
+        MIGRAPHX_THROW(what + ": input and weights need the same rank of at least 3");
     const std::size_t kdims = x->get_shape().ndim() - 2;
     std::string auto_pad    = "NOTSET";
     if(info.has("auto_pad"))
@@ -694,10 +689,18 @@ instruction_ref parse_conv(const node_info& info, const std::vector<instruction_
         }
     }
     const int64_t group = info.has("group") ? info.attr("group").i : 1;
-    auto conv = m.add_instruction(
-        make_op("convolution",
-                {{"padding", paddings}, {"stride", strides}, {"dilation", dilations}, {"group", group}}),
-        x, w);
+    return make_op("convolution",
+                   {{"padding", paddings}, {"stride", strides}, {"dilation", dilations}, {"group", group}});
+}
+
+instruction_ref parse_conv(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 2 or args.size() > 3)
+        MIGRAPHX_THROW("Conv: two or three inputs expected");
+    module& m = *info.mod;
+    auto x    = args[0];
+    auto w    = args[1];
+    auto conv = m.add_instruction(conv_operator(info, x, w, "Conv"), x, w);
     if(args.size() == 3)
     {
         if(args[2]->get_shape().ndim() != 1 or args[2]->get_shape().lens()[0] != conv->get_shape().lens()[1])
@@ -708,14 +711,49 @@ instruction_ref parse_conv(const node_info& info, const std::vector<instruction_
     return conv;
 }
 
-instruction_ref parse_binary(const std::string& op, const node_info& info, const std::vector<instruction_ref>& args)
+// src/onnx/parse_qlinearconv.cpp:84-250: dequantize the input and the weights, convolution, the
+// int32 bias dequantized with scale_x * scale_w and added, the result quantized
+instruction_ref parse_qlinearconv(const node_info& info, const std::vector<instruction_ref>& args)
 {
-    if(args.size() != 2)
-        MIGRAPHX_THROW(info.node->op_type + ": two inputs expected");
+    if(args.size() < 8)
+        MIGRAPHX_THROW("QLINEARCONV: missing inputs");
     module& m = *info.mod;
-    auto a    = args[0];
-    auto b    = args[1];
-    // numpy broadcasting of the two operands (src/onnx/onnx_parser.cpp add_broadcastable_binary_op)
+    auto in_x = args[0];
+    auto in_w = args[3];
+    for(auto x : {in_x, in_w})
+    {
+        const auto t = x->get_shape().type();
+        if(t != shape::int8_type and t != shape::uint8_type)
+            MIGRAPHX_THROW(x == in_x ? "QLINEARCONV: unsupported input type" : "QLINEARCONV: unsupported weight type");
+    }
+    if(args[1]->get_shape().type() != shape::float_type)
+        MIGRAPHX_THROW("QLINEARCONV x scale type should be float");
+    if(args[4]->get_shape().type() != shape::float_type)
+        MIGRAPHX_THROW("QLINEARCONV: wt scale type should be float");
+    if(args[6]->get_shape().type() != shape::float_type)
+        MIGRAPHX_THROW("QLINEARCONV: y scale type should be float");
+    if(args.size() > 8 and args[8]->get_shape().type() != shape::int32_type)
+        MIGRAPHX_THROW("QLINEARCONV y bias should be int32");
+    auto dq_x = bcast_qdq(m, "dequantizelinear", in_x, args[1], args[2]);
+    auto dq_w = bcast_qdq(m, "dequantizelinear", in_w, args[4], args[5]);
+    auto y    = m.add_instruction(conv_operator(info, in_x, in_w, "QLINEARCONV"), dq_x, dq_w);
+    if(args.size() > 8)
+    {
+        auto sx = m.add_instruction(make_op("multibroadcast", {{"out_lens", args[4]->get_shape().lens()}}), args[1]);
+        auto bs = m.add_instruction(make_op("mul"), sx, args[4]);
+        auto db = m.add_instruction(make_op("dequantizelinear"), args[8], bs);
+        auto bb = m.add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", y->get_shape().lens()}}), db);
+        auto fb = m.add_instruction(make_op("convert", {{"target_type", y->get_shape().type()}}), bb);
+        y       = m.add_instruction(make_op("add"), y, fb);
+    }
+    return bcast_qdq(m, "quantizelinear", y, args[6], args[7]);
+}
+
+// numpy broadcasting of the two operands, then the operator (src/common.cpp insert_common_op /
+// src/onnx/onnx_parser.cpp add_broadcastable_binary_op)
+instruction_ref common_binary(module& m, const std::string& op, instruction_ref a, instruction_ref b,
+                              const std::string& what)
+{
     if(a->get_shape().lens() != b->get_shape().lens())
     {
         const auto la = a->get_shape().lens();
@@ -727,7 +765,7 @@ instruction_ref parse_binary(const std::string& op, const node_info& info, const
             const std::size_t da = i < nd - la.size() ? 1 : la[i - (nd - la.size())];
             const std::size_t db = i < nd - lb.size() ? 1 : lb[i - (nd - lb.size())];
             if(da != db and da != 1 and db != 1)
-                MIGRAPHX_THROW(info.node->op_type + ": shapes {" + lens_string(la) + "} and {" + lens_string(lb) +
+                MIGRAPHX_THROW(what + ": shapes {" + lens_string(la) + "} and {" + lens_string(lb) +
                                "} do not broadcast");
             out[i] = std::max(da, db);
         }
@@ -739,6 +777,190 @@ instruction_ref parse_binary(const std::string& op, const node_info& info, const
     return m.add_instruction(make_op(op), a, b);
 }
 
+instruction_ref parse_binary(const std::string& op, const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() != 2)
+        MIGRAPHX_THROW(info.node->op_type + ": two inputs expected");
+    return common_binary(*info.mod, op, args[0], args[1], info.node->op_type);
+}
+
+// ---- MatMulInteger / MatMulIntegerToFloat (src/onnx/parse_matmul.cpp:36-330) ---------------------
+
+// a zero point that changes nothing: all zeros, or all 128 for uint8 (which is shifted to int8)
+bool is_symmetric_zero_point(instruction_ref zp)
+{
+    if(not zp->can_eval())
+        return false;
+    const double neutral = zp->get_shape().type() == shape::uint8_type ? 128.0 : 0.0;
+    const auto v         = zp->eval().to_vector<double>();
+    return std::all_of(v.begin(), v.end(), [&](double x) { return x == neutral; });
+}
+
+// src/op/builder/bias_uint8.cpp:49-100: uint8 data (and its zero point) move to int8 through half,
+// the zero point is subtracted in the data's type; returns {data, data - zero point}
+std::pair<instruction_ref, instruction_ref>
+bias_uint8(module& m, instruction_ref arg, instruction_ref bias_arg, bool has_bias, const std::string& what)
+{
+    auto shift = [&](instruction_ref x) {
+        auto offset = m.add_literal(literal{shape{shape::half_type}, std::vector<float>{-128.0f}});
+        auto h      = m.add_instruction(make_op("convert", {{"target_type", shape::half_type}}), x);
+        auto moved  = common_binary(m, "add", h, offset, what);
+        return m.add_instruction(make_op("convert", {{"target_type", shape::int8_type}}), moved);
+    };
+    if(arg->get_shape().type() == shape::uint8_type)
+    {
+        arg      = shift(arg);
+        bias_arg = has_bias ? shift(bias_arg) : arg;
+    }
+    if(has_bias)
+        bias_arg = common_binary(m, "sub", arg, bias_arg, what);
+    return {arg, bias_arg};
+}
+
+instruction_ref parse_matmul_integer(const node_info& info, const std::vector<instruction_ref>& args, bool scaled)
+{
+    const std::string op_name = scaled ? "quant_dot_scaled" : "quant_dot";
+    module& m = *info.mod;
+    if(args.size() < 2)
+        MIGRAPHX_THROW(op_name + ": two operands expected");
+    auto a0 = args[0];
+    auto a1 = args[1];
+    const bool a_prepended = a0->get_shape().ndim() == 1;
+    const bool b_appended  = a1->get_shape().ndim() == 1;
+    if(a_prepended)
+        a0 = m.add_instruction(make_op("unsqueeze", {{"axes", {0}}}), a0);
+    if(b_appended)
+        a1 = m.add_instruction(make_op("unsqueeze", {{"axes", {1}}}), a1);
+
+    std::size_t a0_zp_index = 2, a1_zp_index = 3;
+    instruction_ref scale_a0, scale_a1;
+    auto scale_arg = [&](instruction_ref mat, std::size_t index) {
+        if(args.size() <= index)
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: missing scale");
+        auto sc        = args[index];
+        const auto& ss = sc->get_shape();
+        if(ss.type() != shape::float_type and ss.type() != shape::half_type)
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Scales must be float or half_type");
+        if(ss.lens().at(0) != mat->get_shape().lens().back() and not ss.scalar())
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Scale must have same dim as matrix column");
+        if(ss.lens().size() > 1 and not ss.scalar())
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Scales shape must be scalar or 1-D tensor");
+        return sc;
+    };
+    if(scaled)
+    {
+        a0_zp_index = 4;
+        a1_zp_index = 5;
+        scale_a0    = scale_arg(a0, 2);
+        scale_a1    = scale_arg(a1, 3);
+        if(scale_a0->get_shape().type() != scale_a1->get_shape().type())
+            MIGRAPHX_THROW(op_name + ": Scales must be the same type");
+    }
+    // the zero point of an operand, or the operand itself when it has none that matters
+    auto bias_arg = [&](std::size_t index, instruction_ref input, bool& has) {
+        has = false;
+        if(args.size() <= index)
+            return input;
+        auto b = args[index];
+        if(b->get_shape().type() != input->get_shape().type())
+            MIGRAPHX_THROW(op_name + ": zero point must be the same type as data");
+        if(is_symmetric_zero_point(b))
+            return input;
+        has = true;
+        return b;
+    };
+    bool has_ba0 = false, has_ba1 = false, has_scale_bias = false;
+    auto ba0 = bias_arg(a0_zp_index, a0, has_ba0);
+    auto ba1 = bias_arg(a1_zp_index, a1, has_ba1);
+    instruction_ref scaled_bias;
+    if(scaled and args.size() > 6)
+    {
+        scaled_bias    = args[6];
+        const auto& bs = scaled_bias->get_shape();
+        if(bs.type() != shape::float_type and bs.type() != shape::half_type)
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Bias must be float or half_type");
+        if(bs.type() != scale_a1->get_shape().type())
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Bias must be the same type as scales");
+        if(bs.lens().at(0) != a1->get_shape().lens().back())
+            MIGRAPHX_THROW("PARSE_QUANT_DOT_SCALED: Bias have same dim as matrix B column");
+        has_scale_bias = true;
+    }
+    for(auto x : {a0, a1})
+    {
+        const auto t = x->get_shape().type();
+        if(t != shape::uint8_type and t != shape::int8_type)
+            MIGRAPHX_THROW(op_name + ": Unsupported type");
+    }
+
+    instruction_ref res;
+    if(scaled)
+    {
+        // dequantize both operands (the axis is the dimension the scale's length matches, counted
+        // from the back; 1 when none does), a float dot, the bias subtracted behind it
+        auto dequantized = [&](instruction_ref x, instruction_ref sc, instruction_ref zp, bool no_zp) {
+            const auto& lens     = x->get_shape().lens();
+            const auto scale_len = sc->get_shape().lens().at(0);
+            const auto rit       = std::find(lens.rbegin(), lens.rend(), scale_len);
+            const int64_t axis   = rit != lens.rend() ? static_cast<int64_t>(lens.rend() - rit - 1) : 1;
+            std::vector<instruction_ref> dq_args{x, sc};
+            if(not no_zp)
+                dq_args.push_back(zp);
+            auto t = transform_qdq_inputs(m, "dequantizelinear", 0, axis, dq_args);
+            return m.add_instruction(make_op("dequantizelinear"), t);
+        };
+        auto dq0 = dequantized(a0, scale_a0, ba0, a0 == ba0);
+        auto dq1 = dequantized(a1, scale_a1, ba1, a1 == ba1);
+        res      = parse_matmul(info, {dq0, dq1});
+        if(has_scale_bias)
+            res = common_binary(m, "sub", res, scaled_bias, op_name);
+    }
+    else
+    {
+        if(a0->get_shape().type() == shape::uint8_type or a1->get_shape().type() == shape::uint8_type)
+        {
+            std::tie(a0, ba0) = bias_uint8(m, a0, ba0, has_ba0, op_name);
+            std::tie(a1, ba1) = bias_uint8(m, a1, ba1, has_ba1, op_name);
+        }
+        // src/op/builder/dot.cpp:36-44 with broadcast_dimensions.hpp:39-71: the operands with
+        // their zero points taken off are multiplied -- unless the batch dimensions differ, where
+        // the broadcast (of the operand as it came in) takes the place of the biased one
+        const auto l0 = a0->get_shape().lens();
+        const auto l1 = a1->get_shape().lens();
+        if(not std::equal(l0.rbegin() + 2, l0.rend(), l1.rbegin() + 2, l1.rend()))
+        {
+            std::vector<std::size_t> b0(l0.begin(), l0.end() - 2), b1(l1.begin(), l1.end() - 2);
+            const std::size_t nb = std::max(b0.size(), b1.size());
+            std::vector<std::size_t> out(nb, 1);
+            for(std::size_t i = 0; i < nb; i++)
+            {
+                const std::size_t d0 = i < nb - b0.size() ? 1 : b0[i - (nb - b0.size())];
+                const std::size_t d1 = i < nb - b1.size() ? 1 : b1[i - (nb - b1.size())];
+                if(d0 != d1 and d0 != 1 and d1 != 1)
+                    MIGRAPHX_THROW(op_name + ": batch dimensions do not broadcast");
+                out[i] = std::max(d0, d1);
+            }
+            auto n0 = out;
+            n0.insert(n0.end(), l0.end() - 2, l0.end());
+            auto n1 = out;
+            n1.insert(n1.end(), l1.end() - 2, l1.end());
+            if(l0 != n0)
+                ba0 = m.add_instruction(make_op("multibroadcast", {{"out_lens", n0}}), a0);
+            if(l1 != n1)
+                ba1 = m.add_instruction(make_op("multibroadcast", {{"out_lens", n1}}), a1);
+        }
+        res = m.add_instruction(make_op("quant_dot"), ba0, ba1);
+    }
+    int64_t num_axis = static_cast<int64_t>(res->get_shape().ndim());
+    if(a_prepended)
+    {
+        res = m.add_instruction(make_op("squeeze", {{"axes", {num_axis - 2}}}), res);
+        --num_axis;
+    }
+    if(b_appended)
+        res = m.add_instruction(make_op("squeeze", {{"axes", {num_axis - 1}}}), res);
+    return res;
+}
+
 const std::unordered_map<std::string, node_parser>& parsers()
 {
     static const std::unordered_map<std::string, node_parser> table = {
@@ -747,6 +969,11 @@ const std::unordered_map<std::string, node_parser>& parsers()
         {"DequantizeLinear", parse_dequantizelinear},
         {"QuantizeLinear", parse_quantizelinear},
         {"QLinearMatMul", parse_qlinearmatmul},
+        {"QLinearConv", parse_qlinearconv},
+        {"MatMulInteger",
+         [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_matmul_integer(i, a, false); }},
+        {"MatMulIntegerToFloat",
+         [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_matmul_integer(i, a, true); }},
         {"Conv", parse_conv},
         {"Add", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("add", i, a); }},
         {"Sub", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_binary("sub", i, a); }},

@@ -311,6 +311,22 @@ struct cpu_op
                                  std::is_same<T, double>{})
                         o[i] = n == "mul" ? x[i] * y[i]
                                           : (n == "add" ? x[i] + y[i] : (n == "sub" ? x[i] - y[i] : x[i] / y[i]));
+                    else if constexpr(std::is_same<T, int8_t>{} or std::is_same<T, uint8_t>{})
+                    {
+                        // the operands promote to int, the result converts back (wrapping)
+                        const int a = x[i], b = y[i];
+                        if(n == "div" and b == 0)
+                            MIGRAPHX_THROW("oracle: integer division by zero");
+                        const int v = n == "mul" ? a * b : (n == "add" ? a + b : (n == "sub" ? a - b : a / b));
+                        o[i]        = static_cast<T>(static_cast<unsigned>(v));
+                    }
+                    else if constexpr(std::is_same<T, migraphx::half>{} or std::is_same<T, migraphx::bf16>{})
+                    {
+                        // generic_float.hpp:303-326: the operator works on floats and the result
+                        // converts back to the narrow type
+                        const float a = x[i], b = y[i];
+                        o[i] = T(n == "mul" ? a * b : (n == "add" ? a + b : (n == "sub" ? a - b : a / b)));
+                    }
                     else
                         MIGRAPHX_THROW("oracle: " + n + " on " + out.type_string());
                 }

@@ -371,6 +371,46 @@ for rel in ("test/onnx/verify/qlinearmatmul_1D_test.cpp", "test/onnx/verify/qlin
         qlm.append(c)
 out["onnx_qlinearmatmul"] = qlm
 
+# ---- integer MatMul / QLinearConv models (test/onnx/verify/matmulinteger*_test.cpp, qlinearconv_*_test.cpp)
+ints = []
+for stem in ("matmulinteger_int8_uint8_test", "matmulinteger_int8_uint8_one_zp_test",
+             "matmulinteger_int8_uint8_dual_zp_test", "matmulinteger_uns_test", "matmulinteger_uns_zp_test",
+             "matmulintegertofloat_int8_uint8_scales_zp_bias", "matmulintegertofloat_int8_uint8_scales_zp_bias_3d",
+             "qlinearconv_test", "qlinearconv_pad_0_test", "qlinearconv_pad_1_test", "qlinearconv_scale_1D_test",
+             "qlinearconv_perchannel_weightbias_test"):
+    rel = "test/onnx/verify/" + stem + ".cpp"
+    for name, body in test_cases(read(rel)).items():
+        model = re.search(r'read_onnx\("([^"]+)"\)', body).group(1)
+        c = {"name": name, "source": rel, "model": model, "inputs": {}}
+        for param, var in re.findall(r'pp\["(\w+)"\]\s*=\s*migraphx::argument\(\w+,\s*(\w+)\.data\(\)\)', body):
+            v = vec(body, var)
+            if v is None and re.search(r"std::iota\(" + var + r"\.begin\(\)", body):
+                # std::vector<T> var(shape.elements(), 0); std::iota(...): 0, 1, 2, ...
+                shp = re.search(r"std::vector<\w+>\s+" + var + r"\((\w+)\.elements\(\)", body).group(1)
+                n = 1
+                for d in shape(body, shp)["lens"]:
+                    n *= d
+                v = list(range(n))
+            if v is None and re.search(var + r"\[i\]\s*=\s*static_cast<uint8_t>\(i % 256\)", body):
+                # for(i ...) var[i] = i % 256 over the whole tensor
+                shp = re.search(r"std::vector<\w+>\s+" + var + r"\((\w+)\.elements\(\)\)", body).group(1)
+                n = 1
+                for d in shape(body, shp)["lens"]:
+                    n *= d
+                v = {"rule": "index mod 256", "count": n}
+            c["inputs"][param] = v
+        c["gold"] = vec(body, "gold")
+        if c["gold"] is None:
+            # only the first outputs are listed
+            c["gold"] = vec(body, "gold_prefix")
+            c["gold_is_prefix"] = True
+        assert c["gold"] is not None and all(v is not None for v in c["inputs"].values()), name
+        ints.append(c)
+        # the model itself is a data file of the reference's tests: kept beside the vectors
+        import shutil
+        shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
+out["onnx_integer"] = ints
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -47,6 +47,33 @@ def test_qlinearmatmul_models_reference_known_answers(golden, tmp_path):
         assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
 
 
+def _integer_case_inputs(c):
+    inputs = {}
+    for name, v in c["inputs"].items():
+        inputs[name] = [i % 256 for i in range(v["count"])] if isinstance(v, dict) else v
+    return inputs
+
+
+def test_integer_matmul_and_qlinearconv_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/matmulinteger_*_test.cpp, matmulintegertofloat_*.cpp, qlinearconv_*_test.cpp.
+    # MatMulInteger: int32 results, exact.  MatMulIntegerToFloat: the reference test reads the float
+    # result as int32 (truncating) and compares by RMS; QLinearConv: uint8 results compared by RMS
+    # there -- here every value must be within one step and 95 % must be equal.
+    assert len(golden["onnx_integer"]) == 12
+    for c in golden["onnx_integer"]:
+        got = run_onnx("oracle", c["model"], _integer_case_inputs(c), tmp_path)
+        gold = np.float64(c["gold"])
+        if c.get("gold_is_prefix"):
+            got = got[:len(gold)]
+        assert got.shape == gold.shape, c["name"]
+        if c["name"].startswith("matmulinteger_"):
+            assert got.tolist() == gold.tolist(), c["name"]
+        elif c["name"].startswith("matmulintegertofloat"):
+            assert np.trunc(got).tolist() == gold.tolist(), c["name"]
+        else:
+            assert np.abs(got - gold).max() <= 1 and (got == gold).mean() >= 0.95, (c["name"], got, gold)
+
+
 def test_per_tensor_and_per_axis_models(tmp_path):
     # test/onnx/parse/dequantizelinear_test.cpp, _zero_point_test, _axis_test, _neg_axis_test: shapes of
     # the models, values against the operator's definition
@@ -184,6 +211,42 @@ def test_conv_models_structure(model, fragment):
 def test_malformed_conv_models_are_rejected(model, message):
     rc, text = print_onnx(model)
     assert rc == 4 and message in text, text
+
+
+@pytest.mark.parametrize("model,message", [
+    # test/onnx/parse/matmulinteger_zp_mismatch_error_test.cpp, matmulinteger_invalid_type_error.cpp,
+    # matmulintegerToFloat_bad_{bias,scale}*_test.cpp: each must throw (messages of parse_matmul.cpp)
+    ("matmulinteger_int8_uint8_one_zp_error_test.onnx", "zero point must be the same type as data"),
+    ("matmulinteger_invalid_type_error.onnx", "Unsupported type"),
+    ("matmulintegertofloat_bad_bias_test.onnx", "PARSE_QUANT_DOT_SCALED"),
+    ("matmulintegertofloat_bad_bias_test2.onnx", "PARSE_QUANT_DOT_SCALED"),
+    ("matmulintegertofloat_bad_bias_test3.onnx", "PARSE_QUANT_DOT_SCALED"),
+    ("matmulintegertofloat_bad_scale_test.onnx", "Scales must be float or half_type"),
+    ("matmulintegertofloat_bad_scale2_test.onnx", "PARSE_QUANT_DOT_SCALED"),
+    ("matmulintegertofloat_bad_scale3_test.onnx", "PARSE_QUANT_DOT_SCALED"),
+    ("matmulintegertofloat_bad_scale4_test.onnx", "Scales must be float or half_type"),
+    ("matmulintegertofloat_bad_scale5_test.onnx", "Scales must be float or half_type"),
+])
+def test_malformed_integer_matmul_models_are_rejected(model, message):
+    rc, text = print_onnx(model)
+    assert rc == 4 and message in text, text
+
+
+def test_integer_matmul_and_qlinearconv_program_structure():
+    # test/onnx/parse/matmulinteger_test.cpp, matmulinteger_dual_zp_test.cpp, qlinearconv_test.cpp: what the
+    # parsed programs consist of
+    rc, text = print_onnx("matmulinteger_int8_uint8_dual_zp_test.onnx")
+    assert rc == 0, text
+    # the uint8 operand and its zero point move to int8 through half, each zero point is subtracted
+    assert text.count("convert[target_type=1]") == 2 and text.count("convert[target_type=5]") == 2, text
+    assert text.count("sub(") == 2 and text.count("quant_dot(") == 1, text
+    rc, text = print_onnx("matmulinteger_int8_uint8_test.onnx")
+    assert rc == 0 and text.count("sub(") == 0 and text.count("quant_dot(") == 1, text
+    rc, text = print_onnx("qlinearconv_test.onnx")
+    assert rc == 0 and text.count("dequantizelinear(") == 2 and text.count("convolution[") == 1 and \
+        text.count("quantizelinear[") == 1, text
+    rc, text = print_onnx("matmulintegertofloat_zp_bias_test.onnx")
+    assert rc == 0 and text.count("dequantizelinear(") == 2 and text.count("dot(") == 1 and text.count("sub(") == 1, text
 
 
 def qdq_matmul_model(rng, m=64, k=256, n=128, with_bias=True):
