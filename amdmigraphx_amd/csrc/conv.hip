@@ -1390,6 +1390,107 @@ mi355_quant_conv3d_desc with_unit_depth(const mi355_quant_conv_desc* d)
 
 } // namespace
 
+// ---- float convolution: a correctness path ------------------------------------------------------
+// op::convolution::compute (src/include/migraphx/op/convolution.hpp:208-239 -> convolution.hpp:37-100)
+// as the reference evaluates it: the float product rounded, added into a double over (channel,
+// kd, kh, kw) in that order, one conversion to float at the end.  One thread per output; what the
+// integer front ends leave of a layer whose tensors are uint8 (QLinearConv) runs here.
+struct convf_params
+{
+    const float* x;
+    const float* w;
+    float* out;
+    int64_t n, c, d, h, w_, o, kd, kh, kw, od, oh, ow;
+    int64_t pad[3], stride[3], dil[3];
+    int64_t group;
+};
+
+__global__ __launch_bounds__(256) void conv_f32_kernel(convf_params p)
+{
+#pragma clang fp contract(off)
+    const int64_t total = p.n * p.o * p.od * p.oh * p.ow;
+    const int64_t step  = (int64_t)gridDim.x * 256;
+    const int64_t cg = p.c / p.group, og = p.o / p.group;
+    for(int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += step)
+    {
+        const int64_t ox = idx % p.ow;
+        const int64_t oy = (idx / p.ow) % p.oh;
+        const int64_t oz = (idx / (p.ow * p.oh)) % p.od;
+        const int64_t oc = (idx / (p.ow * p.oh * p.od)) % p.o;
+        const int64_t b  = idx / (p.ow * p.oh * p.od * p.o);
+        const int64_t g  = oc / og;
+        double acc       = 0.0;
+        for(int64_t k = 0; k < cg; k++)
+        {
+            const int64_t ic = g * cg + k;
+            for(int64_t t = 0; t < p.kd; t++)
+            {
+                const int64_t iz = oz * p.stride[0] - p.pad[0] + t * p.dil[0];
+                if(iz < 0 || iz >= p.d)
+                    continue;
+                for(int64_t r = 0; r < p.kh; r++)
+                {
+                    const int64_t iy = oy * p.stride[1] - p.pad[1] + r * p.dil[1];
+                    if(iy < 0 || iy >= p.h)
+                        continue;
+                    for(int64_t q = 0; q < p.kw; q++)
+                    {
+                        const int64_t ix = ox * p.stride[2] - p.pad[2] + q * p.dil[2];
+                        if(ix < 0 || ix >= p.w_)
+                            continue;
+                        const float prod = p.x[(((b * p.c + ic) * p.d + iz) * p.h + iy) * p.w_ + ix] *
+                                           p.w[(((oc * cg + k) * p.kd + t) * p.kh + r) * p.kw + q];
+                        acc += (double)prod;
+                    }
+                }
+            }
+        }
+        p.out[idx] = (float)acc;
+    }
+}
+
+extern "C" int mi355_convolution_f32(const mi355_quant_conv3d_desc* d,
+                                     const float* x,
+                                     const float* w,
+                                     float* out,
+                                     void* stream)
+{
+    if(d == nullptr || d->in_type != MI355_F32)
+        return MI355_ERR_BAD_ARG;
+    mi355_quant_conv3d_desc q = *d;
+    q.in_type                 = MI355_I8; // the shape rules are those of the quantized operator
+    if(!valid(&q))
+        return MI355_ERR_BAD_ARG;
+    convf_params p;
+    const int64_t in[3]  = {d->d, d->h, d->w};
+    const int64_t win[3] = {d->kd, d->kh, d->kw};
+    int64_t o[3];
+    for(int i = 0; i < 3; i++)
+    {
+        o[i]        = out_len(in[i], win[i], d->pad[i], d->pad_hi[i], d->stride[i], d->dil[i]);
+        p.pad[i]    = d->pad[i];
+        p.stride[i] = d->stride[i];
+        p.dil[i]    = d->dil[i];
+        if(o[i] < 1)
+            return MI355_ERR_BAD_ARG;
+    }
+    const int64_t total = d->n * d->o * o[0] * o[1] * o[2];
+    if(total == 0)
+        return MI355_OK;
+    if(x == nullptr || w == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    p.x = x; p.w = w; p.out = out;
+    p.n = d->n; p.c = d->c; p.d = d->d; p.h = d->h; p.w_ = d->w;
+    p.o = d->o; p.kd = d->kd; p.kh = d->kh; p.kw = d->kw;
+    p.od = o[0]; p.oh = o[1]; p.ow = o[2];
+    p.group = d->group;
+    int64_t blocks = (total + 255) / 256;
+    if(blocks > 256 * 64)
+        blocks = 256 * 64;
+    hipLaunchKernelGGL(conv_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return mi355_launch_status();
+}
+
 extern "C" int mi355_quant_convolution3d_dims(const mi355_quant_conv3d_desc* d,
                                               int64_t* out_lens,
                                               size_t* workspace_bytes)

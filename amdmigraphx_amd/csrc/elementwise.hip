@@ -85,6 +85,57 @@ __global__ __launch_bounds__(256) void binary_i32_kernel(bcast_params_i32 p)
     }
 }
 
+// The same for the narrow types that the integer-MatMul front end leaves in a graph: int8 / uint8
+// (the operands promote to int and the result converts back, wrapping; division is not offered)
+// and half / bf16 (op/binary.hpp with generic_float.hpp:303-326: the operator works on floats and
+// the result converts back, toward zero).
+struct bcast_params_typed
+{
+    const void* a;
+    const void* b;
+    void* out;
+    int64_t lens[MI355_MAX_DIMS];
+    int64_t a_strides[MI355_MAX_DIMS];
+    int64_t b_strides[MI355_MAX_DIMS];
+    int64_t total;
+    int ndim;
+    int op;
+    int type;
+};
+
+__global__ __launch_bounds__(256) void binary_typed_kernel(bcast_params_typed p)
+{
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < p.total; i += step)
+    {
+        int64_t rem = i, ao = 0, bo = 0;
+        for(int d = p.ndim - 1; d >= 0; d--)
+        {
+            const int64_t c = rem % p.lens[d];
+            rem /= p.lens[d];
+            ao += c * p.a_strides[d];
+            bo += c * p.b_strides[d];
+        }
+        if(p.type == MI355_I8 || p.type == MI355_U8)
+        {
+            const int x = p.type == MI355_I8 ? (int)static_cast<const int8_t*>(p.a)[ao]
+                                             : (int)static_cast<const uint8_t*>(p.a)[ao];
+            const int y = p.type == MI355_I8 ? (int)static_cast<const int8_t*>(p.b)[bo]
+                                             : (int)static_cast<const uint8_t*>(p.b)[bo];
+            const int r = p.op == MI355_BIN_ADD ? x + y : (p.op == MI355_BIN_SUB ? x - y : x * y);
+            static_cast<uint8_t*>(p.out)[i] = (uint8_t)(unsigned)r;
+        }
+        else
+        {
+            const uint16_t xb = static_cast<const uint16_t*>(p.a)[ao], yb = static_cast<const uint16_t*>(p.b)[bo];
+            const float x = p.type == MI355_F16 ? half_to_f32(xb) : bf16_to_f32(xb);
+            const float y = p.type == MI355_F16 ? half_to_f32(yb) : bf16_to_f32(yb);
+            const float r = binary_apply(p.op, x, y);
+            static_cast<uint16_t*>(p.out)[i] = p.type == MI355_F16 ? f32_to_half_rtz(r) : f32_to_bf16_rtz(r);
+        }
+    }
+}
+
 // The shapes that matter collapse to [rows, cols] with each operand either running along the
 // columns (column stride 1) or constant along them (column stride 0: a per-row value or a scalar):
 // activations against a bias row, a per-row statistic, another activation.  Four columns per
@@ -613,6 +664,51 @@ extern "C" int mi355_binary_i32(int32_t op,
     p.ndim = ndim;
     p.op   = op;
     hipLaunchKernelGGL(binary_i32_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return mi355_launch_status();
+}
+
+extern "C" int mi355_binary_typed(int32_t op,
+                                  int32_t type,
+                                  const void* a,
+                                  const int64_t* a_strides,
+                                  const void* b,
+                                  const int64_t* b_strides,
+                                  void* out,
+                                  int32_t ndim,
+                                  const int64_t* lens,
+                                  void* stream)
+{
+    if(op < MI355_BIN_ADD || op > MI355_BIN_DIV || ndim < 1 || ndim > MI355_MAX_DIMS || lens == nullptr ||
+       a_strides == nullptr || b_strides == nullptr)
+        return MI355_ERR_BAD_ARG;
+    const bool integer = type == MI355_I8 || type == MI355_U8;
+    if(!integer && type != MI355_F16 && type != MI355_BF16)
+        return MI355_ERR_UNSUPPORTED;
+    if(integer && op == MI355_BIN_DIV)
+        return MI355_ERR_UNSUPPORTED;
+    bcast_params_typed p{};
+    p.total = 1;
+    for(int d = 0; d < ndim; d++)
+    {
+        if(lens[d] < 0 || a_strides[d] < 0 || b_strides[d] < 0)
+            return MI355_ERR_BAD_ARG;
+        p.lens[d]      = lens[d];
+        p.a_strides[d] = a_strides[d];
+        p.b_strides[d] = b_strides[d];
+        p.total *= lens[d];
+    }
+    if(p.total == 0)
+        return MI355_OK;
+    if(a == nullptr || b == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    p.a    = a;
+    p.b    = b;
+    p.out  = out;
+    p.ndim = ndim;
+    p.op   = op;
+    p.type = type;
+    hipLaunchKernelGGL(binary_typed_kernel, dim3(blocks_for_n(p.total)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
     return mi355_launch_status();
 }

@@ -296,6 +296,17 @@ __global__ __launch_bounds__(PW_THREADS) void convert_kernel(
             static_cast<uint8_t*>(out)[i] =
                 f32_to_fp8_rne((float)fmin(448.0, fmax(-448.0, dx)));
         break;
+    case MI355_I8:
+        // integral targets: NaN -> numeric_limits::quiet_NaN() = 0, saturate, then truncate toward zero
+        static_cast<int8_t*>(out)[i] = dx != dx ? (int8_t)0 : (int8_t)(int)fmin(127.0, fmax(-128.0, dx));
+        break;
+    case MI355_U8:
+        static_cast<uint8_t*>(out)[i] = dx != dx ? (uint8_t)0 : (uint8_t)(int)fmin(255.0, fmax(0.0, dx));
+        break;
+    case MI355_I32:
+        static_cast<int32_t*>(out)[i] =
+            dx != dx ? 0 : (int32_t)fmin(2147483647.0, fmax(-2147483648.0, dx));
+        break;
     case MI355_BF8:
         // numeric_limits<fp8e5m2>::quiet_NaN() is 0xff (float8.hpp:364); infinities go through
         // the clipping constructor
@@ -614,7 +625,8 @@ extern "C" int mi355_convert(
     if(mi355_dtype_size(in_type) == 0 || mi355_dtype_size(out_type) == 0)
         return MI355_ERR_BAD_ARG;
     if(out_type != MI355_F32 && out_type != MI355_F16 && out_type != MI355_BF16 &&
-       out_type != MI355_FP8 && out_type != MI355_BF8)
+       out_type != MI355_FP8 && out_type != MI355_BF8 && out_type != MI355_I8 && out_type != MI355_U8 &&
+       out_type != MI355_I32)
         return MI355_ERR_UNSUPPORTED;
     if(n == 0)
         return MI355_OK;

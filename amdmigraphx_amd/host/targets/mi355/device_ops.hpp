@@ -248,6 +248,27 @@ struct quant_convolution
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// Float convolution (mi355_convolution_f32, a correctness path).  inputs: x, weights (dense float), out
+struct convolution
+{
+    std::vector<int64_t> padding  = {0, 0};
+    std::vector<int64_t> stride   = {1, 1};
+    std::vector<int64_t> dilation = {1, 1};
+    int64_t group                 = 1;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.padding, "padding");
+        f(self.stride, "stride");
+        f(self.dilation, "dilation");
+        f(self.group, "group");
+    }
+    std::string name() const { return "mi355::convolution"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: int8 matrix, out (int32 [cols] or [rows])
 struct colsum
 {

@@ -1306,6 +1306,19 @@ void lower_instruction(module& m, instruction_ref ins)
             m.replace_instruction(ins, operation{pack_fp4{}}, x, standard_out());
         }
     }
+    else if(name == "convolution" and ins->get_shape().type() == shape::float_type)
+    {
+        // what no quantization pass turned into quant_convolution: the float kernel (bit-exact, slow)
+        const auto& ref = any_cast<op::convolution>(ins->get_operator());
+        convolution op;
+        op.padding  = ref.padding;
+        op.stride   = ref.stride;
+        op.dilation = ref.dilation;
+        op.group    = ref.group;
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        auto w = make_standard(m, ins, ins->inputs()[1]);
+        m.replace_instruction(ins, operation{op}, x, w, standard_out());
+    }
     else if(name == "convert")
     {
         convert op;

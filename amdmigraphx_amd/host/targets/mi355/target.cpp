@@ -578,6 +578,43 @@ quant_convolution::compute(migraphx::context& ctx, const shape&, const std::vect
     return args.back();
 }
 
+shape convolution::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 3, name());
+    op::convolution ref;
+    ref.padding  = padding;
+    ref.stride   = stride;
+    ref.dilation = dilation;
+    ref.group    = group;
+    auto s = ref.compute_shape({inputs[0], inputs[1]});
+    if(inputs[0].type() != shape::float_type or inputs[1].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::convolution: float tensors only, not " + inputs[0].type_string());
+    check_standard(inputs[0], name());
+    check_standard(inputs[1], name());
+    shape out{shape::float_type, s.lens()};
+    if(inputs.back() != out)
+        MIGRAPHX_THROW("mi355::convolution: output buffer has the wrong shape");
+    return out;
+}
+
+argument convolution::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    quant_convolution q;
+    q.padding  = padding;
+    q.stride   = stride;
+    q.dilation = dilation;
+    q.group    = group;
+    q.out_type = shape::float_type;
+    const auto d = q.describe(args[0].get_shape(), args[1].get_shape());
+    status_check(mi355_convolution_f32(&d,
+                                       reinterpret_cast<const float*>(args[0].data()),
+                                       reinterpret_cast<const float*>(args[1].data()),
+                                       reinterpret_cast<float*>(args.back().data()),
+                                       stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
 shape colsum::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -1227,11 +1264,14 @@ shape binary::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 3, name());
     const auto t = inputs[0].type();
-    if(t != inputs[1].type() or (t != shape::float_type and t != shape::int32_type))
-        MIGRAPHX_THROW("mi355::binary: float or int32 tensors of one type only, got " + inputs[0].type_string() +
-                       " and " + inputs[1].type_string());
-    if(t == shape::int32_type and op == MI355_BIN_DIV)
-        MIGRAPHX_THROW("mi355::binary: int32 division has no kernel");
+    const bool narrow_int = t == shape::int8_type or t == shape::uint8_type;
+    const bool narrow_flt = t == shape::half_type or t == shape::bf16_type;
+    if(t != inputs[1].type() or
+       (t != shape::float_type and t != shape::int32_type and not narrow_int and not narrow_flt))
+        MIGRAPHX_THROW("mi355::binary: float, half, bf16, int32, int8 or uint8 tensors of one type only, got " +
+                       inputs[0].type_string() + " and " + inputs[1].type_string());
+    if((t == shape::int32_type or narrow_int) and op == MI355_BIN_DIV)
+        MIGRAPHX_THROW("mi355::binary: integer division has no kernel");
     if(inputs[0].lens() != inputs[1].lens())
         MIGRAPHX_THROW("mi355::binary: Dimensions do not match");
     if(inputs[0].ndim() > MI355_MAX_DIMS)
@@ -1256,6 +1296,21 @@ argument binary::compute(migraphx::context& ctx, const shape& out, const std::ve
     };
     const auto sa = strides_of(args[0].get_shape());
     const auto sb = strides_of(args[1].get_shape());
+    if(out.type() != shape::int32_type and out.type() != shape::float_type)
+    {
+        status_check(mi355_binary_typed(static_cast<int32_t>(op),
+                                        to_mi355_type(out.type()),
+                                        args[0].data(),
+                                        sa.data(),
+                                        args[1].data(),
+                                        sb.data(),
+                                        args[2].data(),
+                                        static_cast<int32_t>(lens.size()),
+                                        lens.data(),
+                                        stream_of(ctx)),
+                     name());
+        return args[2];
+    }
     if(out.type() == shape::int32_type)
     {
         status_check(mi355_binary_i32(static_cast<int32_t>(op),
@@ -1489,6 +1544,7 @@ MIGRAPHX_REGISTER_OP(mi355::rowsum);
 MIGRAPHX_REGISTER_OP(mi355::dot);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot_mx);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_gemm);
+MIGRAPHX_REGISTER_OP(mi355::convolution);
 MIGRAPHX_REGISTER_OP(mi355::w4a16_prepack);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot_prepack);
 MIGRAPHX_REGISTER_OP(mi355::quant_dot_prepacked);

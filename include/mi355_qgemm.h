@@ -184,6 +184,14 @@ int mi355_quant_convolution3d(const mi355_quant_conv3d_desc* desc, const void* x
                               const float* scale_x, const float* scale_w, void* workspace,
                               size_t workspace_bytes, void* stream);
 
+/* Float convolution of the same description (in_type = MI355_F32; out_type, dequant and the scale
+ * modes are not read): op::convolution::compute (src/include/migraphx/op/convolution.hpp:208-239)
+ * as the reference evaluates it -- float products added into a double over (channel, kd, kh, kw),
+ * one rounding at the end -- bit for bit.  A correctness path (one thread per output) for what the
+ * integer front ends leave of layers with uint8 tensors (QLinearConv) and for unquantized models. */
+int mi355_convolution_f32(const mi355_quant_conv3d_desc* desc, const float* x, const float* w, float* out,
+                          void* stream);
+
 /* The same with a workspace.  A quant_dot that launches fewer workgroups than the chip has CUs
  * (a skinny or mid-size A against a large B, one image of a convolution) is split along K.
  * Without a workspace only the bare int8 product is split (the shares are added into C with
@@ -340,7 +348,8 @@ int mi355_unpack_fp4(const void* in, void* out, int64_t rows, int64_t cols, void
 int mi355_pack_fp4(const float* in, void* out, int64_t rows, int64_t cols, void* stream);
 
 /*
- * convert float -> half / bf16 / fp8 and back on n dense elements.
+ * convert float -> half / bf16 / fp8 and back on n dense elements; also to int8 / uint8 / int32
+ * (NaN -> 0, saturating, truncating toward zero: the integral branch of op/convert.hpp:64-87).
  *
  * Replaces: op::convert::compute (src/include/migraphx/op/convert.hpp:64-87)
  * with the software-float conversions of generic_float.hpp:172-222 (half and
@@ -528,6 +537,14 @@ typedef enum mi355_unary_op {
 int mi355_binary_f32(int32_t op, const float* a, const int64_t* a_strides, const float* b,
                      const int64_t* b_strides, float* out, int32_t ndim, const int64_t* lens,
                      void* stream);
+/* The same operators on the narrow types the integer-MatMul front end leaves in a graph
+ * (src/op/builder/bias_uint8.cpp:49-100: uint8 data moved to int8 through half, zero points
+ * subtracted in int8): MI355_I8 / MI355_U8 (add / sub / mul; operands promote to int, the result
+ * converts back, wrapping) and MI355_F16 / MI355_BF16 (the operator on floats, the result converted
+ * back toward zero: generic_float.hpp:303-326).  Addressing as mi355_binary_f32. */
+int mi355_binary_typed(int32_t op, int32_t type, const void* a, const int64_t* a_strides, const void* b,
+                       const int64_t* b_strides, void* out, int32_t ndim, const int64_t* lens,
+                       void* stream);
 /* add / sub / mul of int32 tensors (wrapping), same addressing as mi355_binary_f32: the
  * zero-point terms of src/simplify_qdq.cpp:196-222 and :250-279 when they stay in the graph. */
 int mi355_binary_i32(int32_t op, const int32_t* a, const int64_t* a_strides, const int32_t* b,

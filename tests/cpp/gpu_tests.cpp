@@ -1346,6 +1346,100 @@ TEST_CASE(float_operators)
     expect_same(p, {{"i", ia}});
 }
 
+TEST_CASE(narrow_type_operators_and_float_convolution)
+{
+    // What the integer-MatMul / QLinearConv front ends leave in a graph besides the GEMMs: add / sub /
+    // mul on int8, uint8 (wrapping) and half, bf16 (the operator on floats, the result truncated),
+    // convert to the integer types (NaN -> 0, saturating, truncating), and a float convolution --
+    // each bit for bit against the CPU target.
+    const std::size_t r = 19, c = 77;
+    for(auto t : {shape::int8_type, shape::uint8_type, shape::half_type, shape::bf16_type})
+    {
+        const bool integer = t == shape::int8_type or t == shape::uint8_type;
+        for(auto name : {"add", "sub", "mul", "div"})
+        {
+            if(integer and std::string(name) == "div")
+                continue;
+            program p;
+            auto* mm = p.get_main_module();
+            auto x   = mm->add_parameter("x", shape{t, {r, c}});
+            auto y   = mm->add_parameter("y", shape{t, {c}});
+            auto yb  = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {r, c}}}), y);
+            auto z   = mm->add_literal(literal{shape{t}, std::vector<float>{3.0f}});
+            auto zb  = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {r, c}}}), z);
+            auto v   = mm->add_instruction(make_op(name), x, yb);
+            mm->add_return({mm->add_instruction(make_op(name), v, zb)});
+            std::vector<float> xv, yv;
+            if(integer)
+            {
+                const int lo = t == shape::int8_type ? -128 : 0, hi = t == shape::int8_type ? 127 : 255;
+                auto xi = uniform_ints<int>(r * c, lo, hi, 400);
+                auto yi = uniform_ints<int>(c, lo, hi, 401);
+                xv.assign(xi.begin(), xi.end());
+                yv.assign(yi.begin(), yi.end());
+            }
+            else
+            {
+                xv = normal_floats(r * c, 30.0f, 402);
+                yv = uniform_floats(c, 0.01f, 5.0f, 403);
+            }
+            expect_same(p, {{"x", argument{shape{t, {r, c}}, xv}}, {"y", argument{shape{t, {c}}, yv}}});
+        }
+    }
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, {r, c}});
+        std::vector<instruction_ref> outs;
+        for(auto t : {shape::int8_type, shape::uint8_type, shape::int32_type})
+            outs.push_back(mm->add_instruction(make_op("convert", {{"target_type", t}}), x));
+        auto h = mm->add_instruction(make_op("convert", {{"target_type", shape::half_type}}), x);
+        outs.push_back(mm->add_instruction(make_op("convert", {{"target_type", shape::int8_type}}), h));
+        mm->add_return(outs);
+        auto xv = normal_floats(r * c, 90.0f, 404);
+        xv[0]   = std::numeric_limits<float>::quiet_NaN();
+        xv[1]   = std::numeric_limits<float>::infinity();
+        xv[2]   = -std::numeric_limits<float>::infinity();
+        xv[3]   = 3e9f;
+        xv[4]   = -3e9f;
+        xv[5]   = 127.9f;
+        xv[6]   = -128.9f;
+        xv[7]   = -0.9f;
+        xv[8]   = 255.5f;
+        expect_same(p, {{"x", argument{shape{shape::float_type, {r, c}}, xv}}});
+    }
+    // float convolution: groups, strides, dilation, padding on one side more than on the other, one
+    // to three spatial axes
+    struct conv_case
+    {
+        std::vector<std::size_t> x, w;
+        std::vector<int64_t> pad, stride, dil;
+        int64_t group;
+    };
+    for(auto k : {conv_case{{2, 6, 11, 9}, {8, 3, 3, 2}, {1, 0, 2, 1}, {2, 1}, {1, 2}, 2},
+                  conv_case{{1, 3, 20}, {5, 3, 4}, {2}, {3}, {1}, 1},
+                  conv_case{{1, 4, 5, 6, 7}, {4, 1, 2, 3, 3}, {0, 1, 1}, {1, 2, 1}, {2, 1, 1}, 4}})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, k.x});
+        std::size_t wn = 1;
+        for(auto l : k.w)
+            wn *= l;
+        auto w = mm->add_literal(literal{shape{shape::float_type, k.w}, normal_floats(wn, 0.5f, 405)});
+        mm->add_return({mm->add_instruction(
+            make_op("convolution", {{"padding", k.pad}, {"stride", k.stride}, {"dilation", k.dil}, {"group", k.group}}),
+            x, w)});
+        std::size_t xn = 1;
+        for(auto l : k.x)
+            xn *= l;
+        expect_same(p, {{"x", argument{shape{shape::float_type, k.x}, normal_floats(xn, 1.0f, 406)}}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::convolution") == 1);
+    }
+}
+
 TEST_CASE(intermediate_buffers_share_one_arena)
 {
     // memory_coloring: the buffers of a compiled program are places in one block of device memory,

@@ -42,6 +42,39 @@ def test_qlinearmatmul_models_on_device(golden, tmp_path):
         assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
 
 
+def test_integer_matmul_models_on_device(golden, tmp_path):
+    # test/onnx/verify/matmulinteger_*_test.cpp: uint8 operands move to int8 through half on the
+    # device (convert, half add, convert), zero points are subtracted in int8, the product is the
+    # int8 quant_dot -- int32 results, exact; matmulintegertofloat_*: dequantize, float dot, bias
+    from test_onnx import _integer_case_inputs
+    cases = [c for c in golden["onnx_integer"] if c["name"].startswith("matmulinteger")]
+    assert len(cases) == 7
+    for c in cases:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], _integer_case_inputs(c), tmp_path)
+        want = run_onnx("oracle", c["model"], _integer_case_inputs(c), tmp_path)
+        assert got.tolist() == want.tolist(), c["name"]
+        gold = [float(v) for v in c["gold"]]
+        assert (np.trunc(got) if c["name"].startswith("matmulintegertofloat") else got).tolist() == gold, c["name"]
+
+
+def test_qlinearconv_models_on_device(golden, tmp_path):
+    # test/onnx/verify/qlinearconv_*_test.cpp: uint8 tensors are no quant_convolution inputs of
+    # simplify_qdq, so the layer runs as dequantize -> float convolution -> (bias) -> quantize on the
+    # device, each step bit-identical to the CPU target's; the answers are the reference's
+    from test_onnx import _integer_case_inputs
+    cases = [c for c in golden["onnx_integer"] if c["name"].startswith("qlinearconv")]
+    assert len(cases) == 5
+    for c in cases:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], _integer_case_inputs(c), tmp_path)
+        want = run_onnx("oracle", c["model"], _integer_case_inputs(c), tmp_path)
+        assert got.tolist() == want.tolist(), c["name"]
+        gold = np.float64(c["gold"])
+        part = got[:len(gold)] if c.get("gold_is_prefix") else got
+        assert np.abs(part - gold).max() <= 1 and (part == gold).mean() >= 0.95, c["name"]
+
+
 def test_written_qdq_conv_model_on_device(tmp_path):
     """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
     turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU
