@@ -734,16 +734,12 @@ bool built_from_literals(instruction_ref ins, std::unordered_map<const instructi
     return r;
 }
 
-// Off unless MIGRAPHX_MI355_PREPACK_QUANT_DOT is set (to anything but 0) when a program is compiled.
-// The kernels behind the two operators pass their own tests on the device, called through the C
-// interface; the one device run of programs compiled with this step ended with the device
-// reporting a fault before the test had printed anything, and reading the code has not shown a
-// cause.  Until one is shown, a program keeps mi355::quant_dot (and its split-K workspace) for
-// these layers.
+// MIGRAPHX_MI355_DISABLE_PREPACK_QUANT_DOT set (to anything but 0) when a program is compiled keeps
+// these layers on mi355::quant_dot with its split-K workspace.
 bool prepack_quant_dot_enabled()
 {
-    const char* v = std::getenv("MIGRAPHX_MI355_PREPACK_QUANT_DOT");
-    return v != nullptr and std::string(v) != "0" and std::string(v) != "";
+    const char* v = std::getenv("MIGRAPHX_MI355_DISABLE_PREPACK_QUANT_DOT");
+    return v == nullptr or std::string(v) == "0" or std::string(v) == "";
 }
 
 void prepack_quant_dot(module& m)

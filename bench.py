@@ -112,6 +112,9 @@ def main():
                     help="run one section only, so that a rocprofv3 run holds that section's kernels alone")
     ap.add_argument("--gemv-shape", default=None, metavar="K,N",
                     help="with --only gemv: one (K, N) shape instead of the three of config 4")
+    ap.add_argument("--skinny-m", type=int, default=0, metavar="M", choices=[0, 16, 128],
+                    help="with --only skinny: the int8 M x 8192 x 8192 product alone, through the split-K "
+                         "workspace and (M = 16) over reordered weights, so that a profile holds one shape")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB mebibytes a few "
                          "times: the HBM counters of that kernel calibrate roofline.traffic")
@@ -313,7 +316,8 @@ def main():
     # ---- skinny int8 quant_dot (config 2) and int4 GEMM at M = 16 / 128 (config 4) ----------
     try:
         skip("skinny")
-        for m2 in (16, 128):
+        prof = args.skinny_m != 0
+        for m2 in ((args.skinny_m,) if prof else (16, 128)):
             a2 = torch.randint(-128, 128, (m2, 8192), dtype=torch.int8, device=dev, generator=g)
             bs = [torch.randint(-128, 128, (8192, 8192), dtype=torch.int8, device=dev, generator=g)
                   for _ in range(6)]  # 6 x 67 MB: more than the last-level cache
@@ -356,6 +360,22 @@ def main():
                     it[0] += 1
                 return run
 
+            if prof:
+                # one shape, two paths, many launches: what a kernel profile of this shape should hold
+                t2, _ = _time_launches(skinny_ws, 120, 12, settle_ms=60)
+                row = {"us_per_launch": round(t2 * 1e6, 1), "workspace_MiB": room.numel() >> 20}
+                if m2 <= 16:
+                    pk = [ops.quant_dot_prepack(b) for b in bs]
+                    c3 = torch.empty_like(c2)
+
+                    def skinny_pk():
+                        ops.quant_dot_prepacked(a2, pk[it[0] % 6], 8192, out=c3)
+                        it[0] += 1
+
+                    tp, _ = _time_launches(skinny_pk, 120, 12, settle_ms=60)
+                    row["reordered_weights_us_per_launch_eager"] = round(tp * 1e6, 1)
+                also[f"int8_quant_dot_M{m2}_N8192_K8192"] = row
+                continue
             t2a, _ = _time_launches(skinny, 18, 6, settle_ms=60)
             if not args.no_check:
                 checks[f"int8_quant_dot_M{m2}_atomics"] = sampled_rows_equal(
@@ -419,7 +439,7 @@ def main():
             del b8
             also[f"int8_quant_dot_M{m2}_N8192_K8192"] = row
             del bs
-        for m4 in (16, 128):
+        for m4 in (() if prof else (16, 128)):
             k4, n4, grp = 4096, 14336, 128
             byts = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * m4 * k4 + 2 * m4 * n4
             copies = int(640e6 // byts) + 1
@@ -463,7 +483,7 @@ def main():
             also[f"w4a16_gemm_M{m4}_K{k4}_N{n4}"] = row4
             del ws
         # shapes whose 128-column tiles do not fill the chip: K split with a workspace
-        for m4, k4, n4 in ((128, 4096, 4096), (128, 14336, 4096), (512, 4096, 4096)):
+        for m4, k4, n4 in (() if prof else ((128, 4096, 4096), (128, 14336, 4096), (512, 4096, 4096))):
             grp = 128
             byts = k4 * n4 // 2 + 2 * (k4 // grp) * n4 + 2 * m4 * k4 + 2 * m4 * n4
             copies = int(640e6 // byts) + 1

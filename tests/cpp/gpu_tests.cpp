@@ -253,63 +253,6 @@ TEST_CASE(qdq_linear_layer_bias)
 
 TEST_CASE(qdq_linear_layer_skinny)
 {
-    // A few rows against a large weight matrix (decoding, small batches): the lowering hands the
-    // quant_dot a workspace so that K is split over the chip, the second kernel applies the
-    // epilogue.  Still one mi355::quant_dot, bit-identical to the CPU target; a layer
-    // with a short K gets no workspace.
-    struct layer
-    {
-        std::size_t m, k, n;
-        int zp_x, zp_w;
-        bool weight_nk, skinny;
-        shape::type_t type;
-    };
-    for(auto c : {layer{16, 4096, 1024, 0, 0, true, true, shape::float_type},
-                  layer{1, 2048, 512, 0, 0, false, true, shape::float_type},
-                  layer{40, 1600, 304, 3, -2, false, true, shape::float_type},
-                  layer{128, 3072, 768, 0, 0, true, true, shape::half_type},
-                  layer{2048, 256, 1024, 0, 0, true, false, shape::float_type}})
-    {
-        auto p = qdq_matmul(c.m, c.k, c.n, c.weight_nk, c.zp_x, c.zp_w, c.type, 31);
-        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
-        program compiled = p;
-        compiled.compile(migraphx::make_target("mi355"));
-        const auto& mod = *compiled.get_main_module();
-        EXPECT(count_ops(mod, "mi355::quant_dot") == 1);
-        for(auto ins = mod.begin(); ins != mod.end(); ++ins)
-        {
-            if(ins->name() != "mi355::quant_dot")
-                continue;
-            EXPECT(ins->get_operator().to_value().at("workspace").to<bool>() == c.skinny);
-        }
-        argument x{shape{c.type, {c.m, c.k}}, normal_floats(c.m * c.k, 1.0f, 32)};
-        expect_same(p, {{"x", x}});
-    }
-    // the bare int32 product of a skinny shape takes the same path
-    {
-        program p;
-        auto* mm = p.get_main_module();
-        auto a   = mm->add_parameter("a", shape{shape::int8_type, {24, 2048}});
-        auto b   = mm->add_literal(literal{shape{shape::int8_type, {2048, 640}}, uniform_ints<std::int8_t>(2048 * 640, -128, 127, 33)});
-        mm->add_return({mm->add_instruction(make_op("quant_dot"), a, b)});
-        argument av{shape{shape::int8_type, {24, 2048}}, uniform_ints<std::int8_t>(24 * 2048, -128, 127, 34)};
-        expect_same(p, {{"a", av}});
-        program compiled = p;
-        compiled.compile(migraphx::make_target("mi355"));
-        for(auto ins = compiled.get_main_module()->begin(); ins != compiled.get_main_module()->end(); ++ins)
-            if(ins->name() == "mi355::quant_dot")
-                EXPECT(ins->get_operator().to_value().at("workspace").to<bool>());
-    }
-}
-
-TEST_CASE(qdq_linear_layer_reordered_weights)
-{
-    // needs the lowering step that MIGRAPHX_MI355_PREPACK_QUANT_DOT switches on (off by default)
-    if(std::getenv("MIGRAPHX_MI355_PREPACK_QUANT_DOT") == nullptr)
-    {
-        std::cout << "skipped: MIGRAPHX_MI355_PREPACK_QUANT_DOT is not set" << std::endl;
-        return;
-    }
     // A few rows against a large weight matrix (decoding, small batches).  Up to 16 rows against
     // constant weights: the weights are reordered when the program is compiled and the layer is
     // one launch of mi355::quant_dot_prepacked.  More rows (or shapes the reordered form does not
@@ -326,7 +269,7 @@ TEST_CASE(qdq_linear_layer_reordered_weights)
     for(auto c : {layer{16, 4096, 1024, 0, 0, true, true, true, shape::float_type},
                   layer{1, 2048, 512, 0, 0, false, true, true, shape::float_type},
                   layer{5, 1600, 304, 3, -2, false, true, true, shape::half_type},
-                  layer{16, 1608, 304, 0, 0, false, true, false, shape::float_type},
+                  layer{16, 1608, 304, 0, 0, false, false, false, shape::float_type}, // K % 64 != 0: neither form
                   layer{40, 1600, 304, 3, -2, false, true, false, shape::float_type},
                   layer{128, 3072, 768, 0, 0, true, true, false, shape::half_type},
                   layer{2048, 256, 1024, 0, 0, true, false, false, shape::float_type}})
@@ -353,9 +296,13 @@ TEST_CASE(qdq_linear_layer_reordered_weights)
             const std::string file = "/tmp/mi355_skinny_layer.mxr";
             migraphx::save(compiled, file);
             auto loaded = migraphx::load(file);
-            auto r1 = compiled.eval({{"x", x}});
-            auto r2 = loaded.eval({{"x", x}});
-            EXPECT(same_bytes(r1[0], r2[0]));
+            // (compiled without offload_copy: parameters and results live in device memory)
+            auto t  = migraphx::make_target("mi355");
+            auto r1 = compiled.eval({{"x", t.copy_to(x)}});
+            compiled.finish();
+            auto r2 = loaded.eval({{"x", t.copy_to(x)}});
+            loaded.finish();
+            EXPECT(same_bytes(t.copy_from(r1[0]), t.copy_from(r2[0])));
             std::remove(file.c_str());
         }
     }

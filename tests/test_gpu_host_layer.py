@@ -1,6 +1,5 @@
 """The mi355 target end to end (C++): programs compiled for the CPU oracle target
 and for "mi355" from the same inputs must agree (tests/cpp/gpu_tests.cpp)."""
-import os
 import subprocess
 
 import numpy as np
@@ -13,19 +12,8 @@ ensure_built()
 pytestmark = pytest.mark.gpu
 
 
-# Cases kept off the device, with the reason.
-SKIPPED = {
-    "qdq_linear_layer_reordered_weights":
-        "the lowering step it tests (MIGRAPHX_MI355_PREPACK_QUANT_DOT) is off by default: the one device run of "
-        "programs compiled with it ended with the device reporting a fault before any output, and no cause has "
-        "been shown; the kernels themselves are covered by tests/test_gpu_quant_dot_prepacked.py",
-}
-
-
 @pytest.mark.parametrize("case", list_cases(GPU_TESTS))
 def test_target_case(case):
-    if case in SKIPPED and os.environ.get("MIGRAPHX_MI355_PREPACK_QUANT_DOT") is None:
-        pytest.skip(SKIPPED[case])
     print("gpu_tests", case, flush=True)
     r = subprocess.run([GPU_TESTS, case], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout + r.stderr
