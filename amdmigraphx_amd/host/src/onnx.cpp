@@ -961,6 +961,87 @@ instruction_ref parse_matmul_integer(const node_info& info, const std::vector<in
     return res;
 }
 
+// ---- ConvInteger (src/onnx/parse_convolution.cpp:44-46 -> src/op/builder/convolution.cpp:185-380) ---
+//
+// quant_convolution(x - x_zp, w - w_zp) written out as
+// conv(x, w) - conv(x_zp, w) - conv(x, w_zp) + conv(x_zp, w_zp), every term a quant_convolution of
+// int8 tensors; uint8 tensors (and their zero points) move to int8 through half first, and a zero
+// point that changes nothing (absent, all zeros, or all 128 for uint8) adds no term.
+instruction_ref parse_convinteger(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 2 or args.size() > 4)
+        MIGRAPHX_THROW("ConvInteger: two to four inputs expected");
+    module& m = *info.mod;
+    auto x    = args[0];
+    auto w    = args[1];
+    for(auto t : {x, w})
+    {
+        const auto ty = t->get_shape().type();
+        if(ty != shape::int8_type and ty != shape::uint8_type)
+            MIGRAPHX_THROW("ConvInteger: int8 or uint8 tensors expected");
+    }
+    auto conv = conv_operator(info, x, w, "ConvInteger");
+    auto attrs = conv.to_value();
+    auto op    = make_op("quant_convolution", {{"padding", attrs.at("padding").to_vector<int64_t>()},
+                                               {"stride", attrs.at("stride").to_vector<int64_t>()},
+                                               {"dilation", attrs.at("dilation").to_vector<int64_t>()},
+                                               {"group", attrs.at("group").to<int64_t>()}});
+    auto neutral_literal = [&](instruction_ref like) {
+        const float v = like->get_shape().type() == shape::uint8_type ? 128.0f : 0.0f;
+        return m.add_literal(literal{shape{like->get_shape().type(), {1}, {0}}, std::vector<float>{v}});
+    };
+    auto zero_point = [&](instruction_ref input, std::size_t index) {
+        if(args.size() <= index)
+            return neutral_literal(input);
+        if(input->get_shape().type() != args[index]->get_shape().type())
+            MIGRAPHX_THROW("PARSE:Conv Data and Data Zero Point must have same type");
+        return is_symmetric_zero_point(args[index]) ? neutral_literal(args[index]) : args[index];
+    };
+    auto x_zp = zero_point(x, 2);
+    auto w_zp = zero_point(w, 3);
+    auto shift = [&](instruction_ref v) {
+        auto offset = m.add_literal(literal{shape{shape::half_type}, std::vector<float>{-128.0f}});
+        auto h      = m.add_instruction(make_op("convert", {{"target_type", shape::half_type}}), v);
+        auto moved  = common_binary(m, "add", h, offset, "ConvInteger");
+        return m.add_instruction(make_op("convert", {{"target_type", shape::int8_type}}), moved);
+    };
+    if(x->get_shape().type() == shape::uint8_type)
+    {
+        const bool has = not is_symmetric_zero_point(x_zp);
+        x              = shift(x);
+        if(has)
+            x_zp = shift(x_zp);
+    }
+    if(w->get_shape().type() == shape::uint8_type)
+    {
+        const bool has = not is_symmetric_zero_point(w_zp);
+        w              = shift(w);
+        if(has)
+            w_zp = shift(w_zp);
+    }
+    auto ret = m.add_instruction(op, x, w);
+    // the zero points spread over their tensors: x's is one value, w's one value or one per output channel
+    auto spread_x = [&] { return m.add_instruction(make_op("multibroadcast", {{"out_lens", x->get_shape().lens()}}), x_zp); };
+    auto spread_w = [&] {
+        if(w_zp->get_shape().elements() == 1)
+            return m.add_instruction(make_op("multibroadcast", {{"out_lens", w->get_shape().lens()}}), w_zp);
+        return m.add_instruction(make_op("broadcast", {{"axis", 0}, {"out_lens", w->get_shape().lens()}}), w_zp);
+    };
+    const bool x_term = not is_symmetric_zero_point(x_zp);
+    const bool w_term = not is_symmetric_zero_point(w_zp);
+    if(x_term)
+        ret = common_binary(m, "sub", ret, m.add_instruction(op, spread_x(), w), "ConvInteger");
+    if(w_term)
+        ret = common_binary(m, "sub", ret, m.add_instruction(op, x, spread_w()), "ConvInteger");
+    if(x_term and w_term)
+    {
+        auto xs = spread_x();
+        auto ws = spread_w();
+        ret     = common_binary(m, "add", ret, m.add_instruction(op, xs, ws), "ConvInteger");
+    }
+    return ret;
+}
+
 const std::unordered_map<std::string, node_parser>& parsers()
 {
     static const std::unordered_map<std::string, node_parser> table = {
@@ -970,6 +1051,7 @@ const std::unordered_map<std::string, node_parser>& parsers()
         {"QuantizeLinear", parse_quantizelinear},
         {"QLinearMatMul", parse_qlinearmatmul},
         {"QLinearConv", parse_qlinearconv},
+        {"ConvInteger", parse_convinteger},
         {"MatMulInteger",
          [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_matmul_integer(i, a, false); }},
         {"MatMulIntegerToFloat",

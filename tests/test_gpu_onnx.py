@@ -75,6 +75,17 @@ def test_qlinearconv_models_on_device(golden, tmp_path):
         assert np.abs(part - gold).max() <= 1 and (part == gold).mean() >= 0.95, c["name"]
 
 
+def test_convinteger_models_on_device(tmp_path):
+    # test/onnx/parse/convinteger_*.cpp models against the operator's definition: every term is an
+    # int8 quant_convolution on the device, the zero-point tensors go in as dense copies
+    from test_onnx import CONVINTEGER_MODELS, convinteger_case
+    for case in CONVINTEGER_MODELS:
+        print("onnx", case[0], flush=True)
+        inputs, want = convinteger_case(*case)
+        got = run_onnx("mi355", case[0], inputs, tmp_path)
+        assert got.tolist() == want.flatten().astype(np.float64).tolist(), case[0]
+
+
 def test_written_qdq_conv_model_on_device(tmp_path):
     """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
     turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU

@@ -74,6 +74,63 @@ def test_integer_matmul_and_qlinearconv_models_reference_known_answers(golden, t
             assert np.abs(got - gold).max() <= 1 and (got == gold).mean() >= 0.95, (c["name"], got, gold)
 
 
+def _conv_int64(x, w):
+    n, c, h, wd = x.shape
+    o, _, kh, kw = w.shape
+    out = np.zeros((n, o, h - kh + 1, wd - kw + 1), np.int64)
+    for r in range(kh):
+        for q in range(kw):
+            out += np.einsum("nchw,oc->nohw", x[:, :, r:r + out.shape[2], q:q + out.shape[3]], w[:, :, r, q])
+    return out
+
+
+CONVINTEGER_MODELS = [
+    # test/onnx/parse/convinteger_*.cpp: (model, x type and shape, w type and shape, which zero points are inputs)
+    ("convinteger_no_bias_test.onnx", np.int8, (1, 3, 5, 5), np.int8, (1, 3, 2, 2), ()),
+    ("convinteger_bias_test.onnx", np.int8, (2, 3, 32, 32), np.int8, (4, 3, 5, 5), ("2",)),
+    ("convinteger_dual_bias_test.onnx", np.int8, (2, 3, 10, 10), np.int8, (4, 3, 3, 3), ("2", "3")),
+    ("convinteger_no_bias_uint8_test.onnx", np.uint8, (1, 3, 32, 32), np.uint8, (1, 3, 5, 5), ()),
+    ("convinteger_mismatched_input_types_test.onnx", np.int8, (1, 3, 32, 32), np.uint8, (1, 3, 5, 5), ()),
+]
+
+
+def convinteger_case(model, xt, xs, wt, ws, zps, seed=0):
+    rng = np.random.default_rng(seed + len(model))
+    lim = lambda t: (0, 256) if t == np.uint8 else (-128, 128)
+    x = rng.integers(*lim(xt), xs).astype(xt)
+    w = rng.integers(*lim(wt), ws).astype(wt)
+    inputs = {"0": x.flatten(), "1": w.flatten()}
+    xz = wz = 0
+    if "2" in zps:
+        xz = int(rng.integers(-20, 20))
+        inputs["2"] = [xz]
+    if "3" in zps:
+        wz = int(rng.integers(-20, 20))
+        inputs["3"] = [wz]
+    # uint8 tensors without a zero point are taken as they are shifted by 128 (the operator's own rule)
+    xv = x.astype(np.int64) - (xz if "2" in zps else (128 if xt == np.uint8 else 0))
+    wv = w.astype(np.int64) - (wz if "3" in zps else (128 if wt == np.uint8 else 0))
+    return inputs, _conv_int64(xv, wv)
+
+
+@pytest.mark.parametrize("case", CONVINTEGER_MODELS, ids=[c[0] for c in CONVINTEGER_MODELS])
+def test_convinteger_models_against_the_definition(case, tmp_path):
+    inputs, want = convinteger_case(*case)
+    got = run_onnx("oracle", case[0], inputs, tmp_path)
+    assert got.tolist() == want.flatten().astype(np.float64).tolist()
+
+
+def test_convinteger_program_structure_and_rejections():
+    # test/onnx/parse/convinteger_dual_bias_test.cpp: conv - conv(x_zp, w) - conv(x, w_zp) + conv(x_zp, w_zp)
+    rc, text = print_onnx("convinteger_dual_bias_test.onnx")
+    assert rc == 0 and text.count("quant_convolution[") == 4 and text.count("sub(") == 2 and text.count("add(") == 1, text
+    rc, text = print_onnx("convinteger_no_bias_uint8_test.onnx")
+    assert rc == 0 and text.count("quant_convolution[") == 1 and text.count("convert[target_type=5]") == 2, text
+    for model in ("convinteger_mismatched_data_bias_test.onnx", "convinteger_mismatched_weight_bias_test.onnx"):
+        rc, text = print_onnx(model)
+        assert rc == 4 and "Zero Point must have same type" in text, text
+
+
 def test_per_tensor_and_per_axis_models(tmp_path):
     # test/onnx/parse/dequantizelinear_test.cpp, _zero_point_test, _axis_test, _neg_axis_test: shapes of
     # the models, values against the operator's definition
