@@ -46,6 +46,8 @@ MI355_DEVINL float binary_apply(int op, float x, float y)
     case MI355_BIN_ADD: return x + y;
     case MI355_BIN_SUB: return x - y;
     case MI355_BIN_MUL: return x * y;
+    case MI355_BIN_MAX: return x < y ? y : x; // std::max(x, y) (op/max.hpp)
+    case MI355_BIN_MIN: return y < x ? y : x; // std::min(x, y) (op/min.hpp)
     default: return x / y; // correctly rounded IEEE division
     }
 }
@@ -190,6 +192,7 @@ MI355_DEVINL float unary_apply(int op, float x)
     case MI355_UN_RSQRT: return 1.0f / sqrtf(x); // 1 / std::sqrt(x), two IEEE operations
     case MI355_UN_EXP: return expf(x);
     case MI355_UN_TANH: return tanhf(x);
+    case MI355_UN_NEARBYINT: return rintf(x); // std::nearbyint under round-to-nearest-even
     default: return -x;
     }
 }
@@ -481,7 +484,7 @@ extern "C" int mi355_binary_f32(int32_t op,
                                 const int64_t* lens,
                                 void* stream)
 {
-    if(op < MI355_BIN_ADD || op > MI355_BIN_DIV || ndim < 1 || ndim > MI355_MAX_DIMS ||
+    if(op < MI355_BIN_ADD || op > MI355_BIN_MIN || ndim < 1 || ndim > MI355_MAX_DIMS ||
        lens == nullptr || a_strides == nullptr || b_strides == nullptr)
         return MI355_ERR_BAD_ARG;
     bcast_params p{};
@@ -668,6 +671,40 @@ extern "C" int mi355_binary_i32(int32_t op,
     return mi355_launch_status();
 }
 
+// reduce_max / reduce_min over every element (op/reduce_max.hpp, reduce_min.hpp with all axes: what
+// DynamicQuantizeLinear asks for): one workgroup, a correctness path.  op 0: max, 1: min.
+__global__ __launch_bounds__(1024) void reduce_all_kernel(const float* in, float* out, int64_t n, int op)
+{
+    __shared__ float part[1024];
+    float v = in[0];
+    for(int64_t i = threadIdx.x; i < n; i += 1024)
+    {
+        const float x = in[i];
+        v             = op == 0 ? (v < x ? x : v) : (x < v ? x : v);
+    }
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for(int s = 512; s > 0; s >>= 1)
+    {
+        if((int)threadIdx.x < s)
+        {
+            const float a = part[threadIdx.x], b = part[threadIdx.x + s];
+            part[threadIdx.x] = op == 0 ? (a < b ? b : a) : (b < a ? b : a);
+        }
+        __syncthreads();
+    }
+    if(threadIdx.x == 0)
+        out[0] = part[0];
+}
+
+extern "C" int mi355_reduce_all_f32(int32_t op, const float* in, float* out, int64_t n, void* stream)
+{
+    if((op != 0 && op != 1) || n <= 0 || in == nullptr || out == nullptr)
+        return MI355_ERR_BAD_ARG;
+    hipLaunchKernelGGL(reduce_all_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), in, out, n, op);
+    return mi355_launch_status();
+}
+
 extern "C" int mi355_binary_typed(int32_t op,
                                   int32_t type,
                                   const void* a,
@@ -715,7 +752,7 @@ extern "C" int mi355_binary_typed(int32_t op,
 
 extern "C" int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t n, void* stream)
 {
-    if(op < MI355_UN_ERF || op > MI355_UN_NEG || n < 0)
+    if(op < MI355_UN_ERF || op > MI355_UN_NEARBYINT || n < 0)
         return MI355_ERR_BAD_ARG;
     if(n == 0)
         return MI355_OK;

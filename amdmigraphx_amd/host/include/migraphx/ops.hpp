@@ -169,6 +169,8 @@ struct mul : binary { mul() : binary{"mul"} {} };
 struct add : binary { add() : binary{"add"} {} };
 struct sub : binary { sub() : binary{"sub"} {} };
 struct div : binary { div() : binary{"div"} {} };
+struct max : binary { max() : binary{"max"} {} }; // op/max.hpp: std::max(x, y)
+struct min : binary { min() : binary{"min"} {} }; // op/min.hpp: std::min(x, y)
 
 // src/include/migraphx/op/unary.hpp (erf.hpp, sqrt.hpp, rsqrt.hpp, exp.hpp, tanh.hpp, neg.hpp): the
 // result has the input's shape
@@ -185,6 +187,7 @@ struct rsqrt : unary { rsqrt() : unary{"rsqrt"} {} };
 struct exp : unary { exp() : unary{"exp"} {} };
 struct tanh : unary { tanh() : unary{"tanh"} {} };
 struct neg : unary { neg() : unary{"neg"} {} };
+struct nearbyint : unary { nearbyint() : unary{"nearbyint"} {} }; // op/nearbyint.hpp: ties to even
 
 // src/include/migraphx/op/reduce_mean.hpp:34-50, reduce_op.hpp:80-180: reduced axes keep length 1
 struct reduce_mean
@@ -196,6 +199,30 @@ struct reduce_mean
         f(self.axes, "axes");
     }
     std::string name() const { return "reduce_mean"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+
+// src/include/migraphx/op/reduce_max.hpp, reduce_min.hpp (reduce_op.hpp:80-180): as reduce_mean
+struct reduce_extreme
+{
+    std::string op_name;
+    std::vector<int64_t> axes;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.axes, "axes");
+    }
+    std::string name() const { return op_name; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+};
+struct reduce_max : reduce_extreme { reduce_max() : reduce_extreme{"reduce_max", {}} {} };
+struct reduce_min : reduce_extreme { reduce_min() : reduce_extreme{"reduce_min", {}} {} };
+
+// src/include/migraphx/op/clip.hpp:44-70: min(max(lowest, x), highest), the three inputs of one shape
+struct clip
+{
+    std::string name() const { return "clip"; }
+    value attributes() const { return {{"pointwise", true}}; }
     shape compute_shape(const std::vector<shape>& inputs) const;
 };
 

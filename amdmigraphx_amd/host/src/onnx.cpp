@@ -1042,6 +1042,51 @@ instruction_ref parse_convinteger(const node_info& info, const std::vector<instr
     return ret;
 }
 
+// ---- DynamicQuantizeLinear (src/onnx/parse_dynamicquantizelinear.cpp:83-147) ----------------------
+// y_scale = (max(0, max(x)) - min(0, min(x))) / 255, y_zero_point = uint8(round(clip(0 - min / y_scale,
+// 0, 255))), y = quantizelinear(x, y_scale, y_zero_point): three outputs
+std::vector<instruction_ref> parse_dynamicquantizelinear(const node_info& info,
+                                                         const std::vector<instruction_ref>& args)
+{
+    if(args.size() != 1)
+        MIGRAPHX_THROW("DYNAMICQUANTIZELINEAR: one input expected");
+    module& m     = *info.mod;
+    auto x        = args[0];
+    const auto xt = x->get_shape().type();
+    auto lit_0    = m.add_literal(literal{shape{xt}, std::vector<float>{0.0f}});
+    std::vector<int64_t> axes(x->get_shape().ndim());
+    std::iota(axes.begin(), axes.end(), 0);
+    auto reduce_max_x = m.add_instruction(make_op("reduce_max", {{"axes", axes}}), x);
+    auto max_x        = common_binary(m, "max", lit_0, reduce_max_x, "DynamicQuantizeLinear");
+    auto reduce_min_x = m.add_instruction(make_op("reduce_min", {{"axes", axes}}), x);
+    auto min_x        = common_binary(m, "min", lit_0, reduce_min_x, "DynamicQuantizeLinear");
+    const auto lens   = max_x->get_shape().lens();
+    const std::size_t n = max_x->get_shape().elements();
+    auto q_range = m.add_literal(literal{shape{xt, lens}, std::vector<float>(n, 255.0f)});
+    auto q_min   = m.add_literal(literal{shape{xt, lens}, std::vector<float>(n, 0.0f)});
+    auto q_max   = m.add_literal(literal{shape{xt, lens}, std::vector<float>(n, 255.0f)});
+    auto sub0    = common_binary(m, "sub", max_x, min_x, "DynamicQuantizeLinear");
+    auto y_scale = common_binary(m, "div", sub0, q_range, "DynamicQuantizeLinear");
+    auto div1    = common_binary(m, "div", min_x, y_scale, "DynamicQuantizeLinear");
+    auto interm  = common_binary(m, "sub", q_min, div1, "DynamicQuantizeLinear");
+    auto sat     = m.add_instruction(make_op("clip"), interm, q_min, q_max);
+    auto round   = m.add_instruction(make_op("nearbyint"), sat);
+    auto y_zp    = m.add_instruction(make_op("convert", {{"target_type", shape::uint8_type}}), round);
+    auto quant   = bcast_qdq(m, "quantizelinear", x, y_scale, y_zp);
+    return {quant, y_scale, y_zp};
+}
+
+using multi_parser = std::function<std::vector<instruction_ref>(const node_info&, const std::vector<instruction_ref>&)>;
+
+// operators with several outputs
+const std::unordered_map<std::string, multi_parser>& multi_parsers()
+{
+    static const std::unordered_map<std::string, multi_parser> table = {
+        {"DynamicQuantizeLinear", parse_dynamicquantizelinear},
+    };
+    return table;
+}
+
 const std::unordered_map<std::string, node_parser>& parsers()
 {
     static const std::unordered_map<std::string, node_parser> table = {
@@ -1170,8 +1215,9 @@ program parse_model(wire model, const onnx_options& options)
             values[n.outputs.at(0)] = mm->add_literal(make_literal(n.attributes.at("value").t));
             continue;
         }
-        auto it = parsers().find(n.op_type);
-        if(it == parsers().end())
+        auto it    = parsers().find(n.op_type);
+        auto multi = multi_parsers().find(n.op_type);
+        if(it == parsers().end() and multi == multi_parsers().end())
             MIGRAPHX_THROW("parse_onnx: operator '" + n.op_type + "' is outside the quantized-GEMM path of this build");
         std::vector<instruction_ref> args;
         for(const auto& name : n.inputs)
@@ -1181,6 +1227,16 @@ program parse_model(wire model, const onnx_options& options)
             if(values.count(name) == 0)
                 MIGRAPHX_THROW("PARSE_GRAPH: invalid onnx file. Input \"" + name + "\" is unavailable due to unordered nodes!");
             args.push_back(values.at(name));
+        }
+        if(multi != multi_parsers().end())
+        {
+            const auto outs = multi->second(node_info{&n, mm}, args);
+            for(std::size_t i = 0; i < outs.size() and i < n.outputs.size(); i++)
+            {
+                if(not n.outputs[i].empty())
+                    values[n.outputs[i]] = outs[i];
+            }
+            continue;
         }
         values[n.outputs.at(0)] = it->second(node_info{&n, mm}, args);
     }

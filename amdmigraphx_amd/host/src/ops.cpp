@@ -272,6 +272,27 @@ shape reduce_mean::compute_shape(const std::vector<shape>& inputs) const
     return {s.type(), lens};
 }
 
+shape reduce_extreme::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, op_name, 1, 1);
+    const auto& s = inputs[0];
+    auto lens     = s.lens();
+    if(axes.empty())
+        std::fill(lens.begin(), lens.end(), 1);
+    for(auto a : axes)
+        lens[normalize_axis(a, s.ndim(), op_name)] = 1;
+    return {s.type(), lens};
+}
+
+shape clip::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_count(inputs, "clip", 3, 3);
+    if(inputs[0].type() != inputs[1].type() or inputs[0].type() != inputs[2].type())
+        MIGRAPHX_THROW("clip: Types do not match");
+    check_same_dims(inputs, "clip");
+    return {inputs[0].type(), inputs[0].lens()};
+}
+
 shape softmax::compute_shape(const std::vector<shape>& inputs) const
 {
     check_count(inputs, "SOFTMAX", 1, 1);
@@ -539,6 +560,12 @@ MIGRAPHX_REGISTER_OP(op::mul);
 MIGRAPHX_REGISTER_OP(op::add);
 MIGRAPHX_REGISTER_OP(op::sub);
 MIGRAPHX_REGISTER_OP(op::div);
+MIGRAPHX_REGISTER_OP(op::max);
+MIGRAPHX_REGISTER_OP(op::min);
+MIGRAPHX_REGISTER_OP(op::nearbyint);
+MIGRAPHX_REGISTER_OP(op::reduce_max);
+MIGRAPHX_REGISTER_OP(op::reduce_min);
+MIGRAPHX_REGISTER_OP(op::clip);
 MIGRAPHX_REGISTER_OP(op::erf);
 MIGRAPHX_REGISTER_OP(op::sqrt);
 MIGRAPHX_REGISTER_OP(op::rsqrt);

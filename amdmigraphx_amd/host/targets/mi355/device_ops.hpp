@@ -517,6 +517,20 @@ struct reduce_mean
     argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
+// reduce_max (op 0) / reduce_min (op 1) over every element.  inputs: x (dense float), out (one element)
+struct reduce_all
+{
+    int64_t op = 0;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.op, "op");
+    }
+    std::string name() const { return "mi355::reduce_all"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
 struct softmax
 {
     std::string name() const { return "mi355::softmax"; }

@@ -1322,18 +1322,40 @@ void lower_instruction(module& m, instruction_ref ins)
         auto x         = make_standard(m, ins, ins->inputs()[0]);
         m.replace_instruction(ins, operation{op}, x, standard_out());
     }
-    else if(name == "add" or name == "sub" or name == "mul" or name == "div")
+    else if(name == "add" or name == "sub" or name == "mul" or name == "div" or name == "max" or name == "min")
     {
         binary op;
-        op.op = name == "add" ? MI355_BIN_ADD
-                              : (name == "sub" ? MI355_BIN_SUB : (name == "mul" ? MI355_BIN_MUL : MI355_BIN_DIV));
+        op.op = name == "add"   ? MI355_BIN_ADD
+                : name == "sub" ? MI355_BIN_SUB
+                : name == "mul" ? MI355_BIN_MUL
+                : name == "div" ? MI355_BIN_DIV
+                : name == "max" ? MI355_BIN_MAX
+                                : MI355_BIN_MIN;
         m.replace_instruction(ins, operation{op}, ins->inputs()[0], ins->inputs()[1], standard_out());
     }
+    else if(name == "clip")
+    {
+        // op/clip.hpp:62-66: std::min(std::max(lowest, x), highest), as two launches
+        binary mx, mn;
+        mx.op    = MI355_BIN_MAX;
+        mn.op    = MI355_BIN_MIN;
+        auto low = m.insert_instruction(ins, operation{mx}, ins->inputs()[1], ins->inputs()[0], standard_out());
+        m.replace_instruction(ins, operation{mn}, low, ins->inputs()[2], standard_out());
+    }
+    else if(name == "reduce_max" or name == "reduce_min")
+    {
+        if(ins->get_shape().elements() != 1)
+            MIGRAPHX_THROW("mi355: " + name + " over part of the axes has no kernel");
+        reduce_all op;
+        op.op  = name == "reduce_max" ? 0 : 1;
+        auto x = make_standard(m, ins, ins->inputs()[0]);
+        m.replace_instruction(ins, operation{op}, x, standard_out());
+    }
     else if(name == "erf" or name == "sqrt" or name == "rsqrt" or name == "exp" or name == "tanh" or
-            name == "neg")
+            name == "neg" or name == "nearbyint")
     {
         unary op;
-        op.op  = name == "erf" ? MI355_UN_ERF
+        op.op  = name == "nearbyint" ? MI355_UN_NEARBYINT : name == "erf" ? MI355_UN_ERF
                                : (name == "sqrt" ? MI355_UN_SQRT
                                                  : (name == "rsqrt" ? MI355_UN_RSQRT
                                                                     : (name == "exp" ? MI355_UN_EXP

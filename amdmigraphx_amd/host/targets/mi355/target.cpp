@@ -1272,6 +1272,8 @@ shape binary::compute_shape(const std::vector<shape>& inputs) const
                        inputs[0].type_string() + " and " + inputs[1].type_string());
     if((t == shape::int32_type or narrow_int) and op == MI355_BIN_DIV)
         MIGRAPHX_THROW("mi355::binary: integer division has no kernel");
+    if(t != shape::float_type and (op == MI355_BIN_MAX or op == MI355_BIN_MIN))
+        MIGRAPHX_THROW("mi355::binary: max and min have a float kernel only");
     if(inputs[0].lens() != inputs[1].lens())
         MIGRAPHX_THROW("mi355::binary: Dimensions do not match");
     if(inputs[0].ndim() > MI355_MAX_DIMS)
@@ -1452,6 +1454,28 @@ argument reduce_mean::compute(migraphx::context& ctx, const shape&, const std::v
     return args[1];
 }
 
+shape reduce_all::compute_shape(const std::vector<shape>& inputs) const
+{
+    check_inputs(inputs, 2, name());
+    check_standard(inputs[0], name());
+    if(inputs[0].type() != shape::float_type or inputs[1].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::reduce_all: float tensors only");
+    if(inputs[0].elements() == 0 or inputs[1].elements() != 1 or (op != 0 and op != 1))
+        MIGRAPHX_THROW("mi355::reduce_all: reduces a tensor that is not empty to one element (op 0: max, 1: min)");
+    return inputs[1];
+}
+
+argument reduce_all::compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const
+{
+    status_check(mi355_reduce_all_f32(static_cast<int32_t>(op),
+                                      reinterpret_cast<const float*>(args[0].data()),
+                                      reinterpret_cast<float*>(args[1].data()),
+                                      static_cast<int64_t>(args[0].get_shape().elements()),
+                                      stream_of(ctx)),
+                 name());
+    return args[1];
+}
+
 shape softmax::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -1561,6 +1585,7 @@ MIGRAPHX_REGISTER_OP(mi355::contiguous);
 MIGRAPHX_REGISTER_OP(mi355::binary);
 MIGRAPHX_REGISTER_OP(mi355::unary);
 MIGRAPHX_REGISTER_OP(mi355::reduce_mean);
+MIGRAPHX_REGISTER_OP(mi355::reduce_all);
 MIGRAPHX_REGISTER_OP(mi355::softmax);
 MIGRAPHX_REGISTER_OP(mi355::gather);
 MIGRAPHX_REGISTER_TARGET(mi355::target);

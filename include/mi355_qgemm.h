@@ -530,9 +530,13 @@ int mi355_contiguous(const void* in, void* out, int32_t elem_size, int32_t ndim,
  * mi355_gather_rows  op::gather along axis 0 of a [table_rows, row_bytes] table with int32 or int64
  *                    indices (op/gather.hpp:100-118); row_bytes must be a multiple of 4.
  */
-typedef enum mi355_binary_op { MI355_BIN_ADD = 0, MI355_BIN_SUB = 1, MI355_BIN_MUL = 2, MI355_BIN_DIV = 3 } mi355_binary_op;
+typedef enum mi355_binary_op {
+    MI355_BIN_ADD = 0, MI355_BIN_SUB = 1, MI355_BIN_MUL = 2, MI355_BIN_DIV = 3,
+    MI355_BIN_MAX = 4, MI355_BIN_MIN = 5 /* std::max / std::min (op/max.hpp, min.hpp): mi355_binary_f32 only */
+} mi355_binary_op;
 typedef enum mi355_unary_op {
-    MI355_UN_ERF = 0, MI355_UN_SQRT = 1, MI355_UN_RSQRT = 2, MI355_UN_EXP = 3, MI355_UN_TANH = 4, MI355_UN_NEG = 5
+    MI355_UN_ERF = 0, MI355_UN_SQRT = 1, MI355_UN_RSQRT = 2, MI355_UN_EXP = 3, MI355_UN_TANH = 4, MI355_UN_NEG = 5,
+    MI355_UN_NEARBYINT = 6 /* op/nearbyint.hpp: ties to even */
 } mi355_unary_op;
 int mi355_binary_f32(int32_t op, const float* a, const int64_t* a_strides, const float* b,
                      const int64_t* b_strides, float* out, int32_t ndim, const int64_t* lens,
@@ -551,6 +555,9 @@ int mi355_binary_i32(int32_t op, const int32_t* a, const int64_t* a_strides, con
                      const int64_t* b_strides, int32_t* out, int32_t ndim, const int64_t* lens,
                      void* stream);
 int mi355_unary_f32(int32_t op, const float* in, float* out, int64_t n, void* stream);
+/* reduce_max (op 0) / reduce_min (op 1) over all n elements into out[0] (op/reduce_max.hpp,
+ * reduce_min.hpp with every axis reduced: the range DynamicQuantizeLinear needs); one workgroup. */
+int mi355_reduce_all_f32(int32_t op, const float* in, float* out, int64_t n, void* stream);
 int mi355_reduce_mean_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
 int mi355_softmax_f32(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
 int mi355_gather_rows(const void* table, const void* ids, int32_t ids_are_int64, void* out,

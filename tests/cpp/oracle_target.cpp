@@ -264,6 +264,60 @@ struct cpu_op
             orc_unary_f32(op, reinterpret_cast<float*>(r.data()),
                           reinterpret_cast<const float*>(x.data()), out.elements());
         }
+        else if((n == "max" or n == "min" or n == "clip" or n == "nearbyint") and out.type() == shape::float_type)
+        {
+            // op/max.hpp, min.hpp (std::max / std::min of the two values), op/clip.hpp:62-66
+            // (std::min(std::max(lowest, x), highest)), op/nearbyint.hpp (ties to even)
+            std::vector<argument> d;
+            for(const auto& a : args)
+                d.push_back(dense(a));
+            auto* o       = reinterpret_cast<float*>(r.data());
+            const auto* x = reinterpret_cast<const float*>(d[0].data());
+            for(std::size_t i = 0; i < out.elements(); i++)
+            {
+                if(n == "nearbyint")
+                    o[i] = std::nearbyint(x[i]);
+                else if(n == "max")
+                    o[i] = std::max(x[i], reinterpret_cast<const float*>(d[1].data())[i]);
+                else if(n == "min")
+                    o[i] = std::min(x[i], reinterpret_cast<const float*>(d[1].data())[i]);
+                else
+                    o[i] = std::min(std::max(reinterpret_cast<const float*>(d[1].data())[i], x[i]),
+                                    reinterpret_cast<const float*>(d[2].data())[i]);
+            }
+        }
+        else if((n == "reduce_max" or n == "reduce_min") and out.type() == shape::float_type)
+        {
+            // op/reduce_max.hpp, reduce_min.hpp over the listed axes (reduce_op.hpp:186-202): every
+            // output element folds the elements that differ from it in the reduced axes only
+            argument x     = dense(args[0]);
+            const auto& xs = x.get_shape();
+            const auto* in = reinterpret_cast<const float*>(x.data());
+            auto* o        = reinterpret_cast<float*>(r.data());
+            std::vector<bool> seen(out.elements(), false);
+            for(std::size_t i = 0; i < xs.elements(); i++)
+            {
+                // the output element of input element i: reduced axes have length one
+                std::size_t rem = i, oi = 0, mul = 1;
+                for(std::size_t d = xs.ndim(); d-- > 0;)
+                {
+                    const std::size_t c = rem % xs.lens()[d];
+                    rem /= xs.lens()[d];
+                    if(out.lens()[d] != 1)
+                    {
+                        oi += c * mul;
+                        mul *= out.lens()[d];
+                    }
+                }
+                if(not seen[oi])
+                {
+                    o[oi]    = in[i];
+                    seen[oi] = true;
+                }
+                else
+                    o[oi] = n == "reduce_max" ? std::max(o[oi], in[i]) : std::min(o[oi], in[i]);
+            }
+        }
         else if(n == "reduce_mean" or n == "softmax")
         {
             // the last axis: [rows, cols, 1]

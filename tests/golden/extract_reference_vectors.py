@@ -411,6 +411,18 @@ for stem in ("matmulinteger_int8_uint8_test", "matmulinteger_int8_uint8_one_zp_t
         shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
 out["onnx_integer"] = ints
 
+# ---- DynamicQuantizeLinear models (test/onnx/verify/dynamicquantizelinear_{1d,2d}_test.cpp): three outputs
+dql = []
+for stem in ("dynamicquantizelinear_1d_test", "dynamicquantizelinear_2d_test"):
+    rel = "test/onnx/verify/" + stem + ".cpp"
+    for name, body in test_cases(read(rel)).items():
+        model = re.search(r'read_onnx\("([^"]+)"\)', body).group(1)
+        dql.append({"name": name, "source": rel, "model": model, "x": vec(body, "data"),
+                    "y": vec(body, "y_gold"), "y_scale": vec(body, "y_scale_gold"), "y_zero_point": vec(body, "y_zpt_gold")})
+        import shutil
+        shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
+out["onnx_dynamicquantizelinear"] = dql
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

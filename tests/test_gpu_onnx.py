@@ -86,6 +86,17 @@ def test_convinteger_models_on_device(tmp_path):
         assert got.tolist() == want.flatten().astype(np.float64).tolist(), case[0]
 
 
+def test_dynamicquantizelinear_models_on_device(golden, tmp_path):
+    # test/onnx/verify/dynamicquantizelinear_*_test.cpp: the range (reduce_max / reduce_min over all
+    # elements), the scale and zero point arithmetic and the quantization all run on the device
+    for c in golden["onnx_dynamicquantizelinear"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], {"x": c["x"]}, tmp_path)
+        want = run_onnx("oracle", c["model"], {"x": c["x"]}, tmp_path)
+        assert got.tolist() == want.tolist(), c["name"]
+        assert got[:len(c["y"])].tolist() == [float(v) for v in c["y"]], c["name"]
+
+
 def test_written_qdq_conv_model_on_device(tmp_path):
     """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
     turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU

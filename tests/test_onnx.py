@@ -131,6 +131,17 @@ def test_convinteger_program_structure_and_rejections():
         assert rc == 4 and "Zero Point must have same type" in text, text
 
 
+def test_dynamicquantizelinear_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/dynamicquantizelinear_1d_test.cpp, _2d_test.cpp: y, y_scale and y_zero_point
+    assert len(golden["onnx_dynamicquantizelinear"]) == 3
+    for c in golden["onnx_dynamicquantizelinear"]:
+        got = run_onnx("oracle", c["model"], {"x": c["x"]}, tmp_path)
+        n = len(c["y"])
+        assert got[:n].tolist() == [float(v) for v in c["y"]], c["name"]
+        np.testing.assert_allclose(got[n], c["y_scale"][0], rtol=1e-6)
+        assert got[n + 1] == c["y_zero_point"][0]
+
+
 def test_per_tensor_and_per_axis_models(tmp_path):
     # test/onnx/parse/dequantizelinear_test.cpp, _zero_point_test, _axis_test, _neg_axis_test: shapes of
     # the models, values against the operator's definition
