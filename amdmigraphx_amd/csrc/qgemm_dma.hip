@@ -1650,6 +1650,121 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
         SB();                                                                               \
     } while(0)
 
+    // ---- the steady state, twelve slabs per trip ---------------------------------------------
+    // A wave issues in order and nothing it issues runs in the shadow of its own MFMAs: every
+    // other instruction of the loop adds its issue time (about 4 cycles for a vector instruction,
+    // 2.6 for a scalar one) to the 1024 cycles of a slab's 64 MFMAs.  The A stage of a slab repeats
+    // every six slabs and its B stage every four, so in a trip of twelve every LDS address is a
+    // register that never changes plus an immediate, every LDS destination of a load the wave's
+    // base plus an immediate (written to M0 ahead of the MFMA pair the load follows, which also
+    // covers the wait state between the two), and every global address a scalar base that advances
+    // once per slab plus the lane's fixed 32-bit offset: a slab is its 64 MFMAs, 24 LDS reads,
+    // 8 loads with their 8 M0 writes, three scalar additions, the waits and the barrier.
+    uint32_t a_vaddr[2][2]; // [slab parity][0: stages 0 and 1, 1: stage 2 (beyond a 16-bit immediate)]
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+    {
+        a_vaddr[h][0] = lds0 + a_lane[h];
+        a_vaddr[h][1] = lds0 + a_lane[h] + 2 * A2_BYTES;
+    }
+    uint32_t b_vaddr[8][2];
+#pragma unroll
+    for(int j2 = 0; j2 < 8; j2++)
+    {
+        if constexpr(TRANS_B)
+        {
+            b_vaddr[j2][0] = lds0 + b_lane[0];
+            b_vaddr[j2][1] = 0;
+        }
+        else
+        {
+            const uint32_t c_ = (uint32_t)(((wave_n * 8 + j2) ^ bsw) << 4);
+            b_vaddr[j2][0]    = lds0 + b_lane[0] + c_;
+            b_vaddr[j2][1]    = lds0 + b_lane[1] + c_;
+        }
+    }
+    const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
+#define RA12(U1, Q, I)                                                                         \
+    RD128(fa[Q][I], a_vaddr[(U1) & 1][A_STAGE12(U1) == 2 ? 1 : 0],                             \
+          (A_STAGE12(U1) == 2 ? 0 : A_STAGE12(U1) * A2_BYTES) + (I) * 16 * 2 * BK)
+#define RB12(U1, Q, J, R)                                                                      \
+    do                                                                                         \
+    {                                                                                          \
+        if constexpr(TRANS_B)                                                                  \
+        {                                                                                      \
+            if((R) == 0)                                                                       \
+                RD128(fb[Q][J], b_vaddr[0][0], ((U1) & (STAGES - 1)) * B_BYTES + (J) * 16 * BK); \
+        }                                                                                      \
+        else                                                                                   \
+        {                                                                                      \
+            v2i t_;                                                                            \
+            RDTR8(t_, b_vaddr[J][R], ((U1) & (STAGES - 1)) * B_BYTES);                         \
+            if((R) == 0)                                                                       \
+            {                                                                                  \
+                fb[Q][J].x = t_.x;                                                             \
+                fb[Q][J].y = t_.y;                                                             \
+            }                                                                                  \
+            else                                                                               \
+            {                                                                                  \
+                fb[Q][J].z = t_.x;                                                             \
+                fb[Q][J].w = t_.y;                                                             \
+            }                                                                                  \
+        }                                                                                      \
+    } while(0)
+    // two MFMAs with one load behind them; M0 (the load's LDS destination) is written first
+#define MF2_LOAD(Q, I, J0, J1, LDS_CONST, OFF, BASE)                                           \
+    asm volatile("s_add_i32 m0, %[wl], %[lc]\n\t"                                              \
+                 "v_mfma_i32_16x16x64_i8 %[c0], %[b0], %[a], %[c0]\n\t"                        \
+                 "v_mfma_i32_16x16x64_i8 %[c1], %[b1], %[a], %[c1]\n\t"                        \
+                 "global_load_lds_dwordx4 %[off], %[base]"                                     \
+                 : [c0] "+a"(acc[I][J0]), [c1] "+a"(acc[I][J1])                                \
+                 : [b0] "v"(fb[Q][J0]), [b1] "v"(fb[Q][J1]), [a] "v"(fa[Q][I]),                \
+                   [wl] "s"(wave_lds), [lc] "n"(LDS_CONST), [off] "v"(OFF), [base] "s"(BASE)   \
+                 : "memory", "scc")
+    // the A step whose half slab U loads, as a stage, and the first block of that half
+#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
+#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
+#define ROW12_READS(U, Q, I, N0)                                                               \
+    do                                                                                         \
+    {                                                                                          \
+        SB(); MF(Q, I, 0); MF(Q, I, 1); SB(); OTHER12(U, Q, (N0) + 0);                          \
+        SB(); MF(Q, I, 2); MF(Q, I, 3); SB(); OTHER12(U, Q, (N0) + 1);                          \
+        SB(); MF(Q, I, 4); MF(Q, I, 5); SB(); OTHER12(U, Q, (N0) + 2);                          \
+        SB(); MF(Q, I, 6); MF(Q, I, 7); SB(); OTHER12(U, Q, (N0) + 3);                          \
+    } while(0)
+#define OTHER12(U, Q, N)                                                                       \
+    do                                                                                         \
+    {                                                                                          \
+        if constexpr((N) < 8)                                                                  \
+            RA12((U) + 1, 1 - (Q), (N));                                                       \
+        else                                                                                   \
+            RB12((U) + 1, 1 - (Q), ((N) - 8) >> 1, ((N) - 8) & 1);                             \
+    } while(0)
+#define SLAB12(U)                                                                              \
+    do                                                                                         \
+    {                                                                                          \
+        constexpr int q_ = (U) & 1;                                                            \
+        WAIT_FRAGS(q_);                                                                        \
+        wait_vmcnt<16>();                                                                      \
+        block_barrier();                                                                       \
+        ROW12_READS(U, q_, 0, 0);  ROW12_READS(U, q_, 1, 4);  ROW12_READS(U, q_, 2, 8);        \
+        ROW12_READS(U, q_, 3, 12); ROW12_READS(U, q_, 4, 16); ROW12_READS(U, q_, 5, 20);       \
+        SB();                                                                                  \
+        MF2_LOAD(q_, 6, 0, 1, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 0 * 4096, b_off[0], b_ptr); \
+        MF2_LOAD(q_, 6, 2, 3, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 1 * 4096, b_off[1], b_ptr); \
+        MF2_LOAD(q_, 6, 4, 5, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 2 * 4096, b_off[2], b_ptr); \
+        MF2_LOAD(q_, 6, 6, 7, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 3 * 4096, b_off[3], b_ptr); \
+        MF2_LOAD(q_, 7, 0, 1, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 0) * 4096, a_off[A_LOAD_BLOCK12(U) + 0], a_ptr); \
+        MF2_LOAD(q_, 7, 2, 3, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 1) * 4096, a_off[A_LOAD_BLOCK12(U) + 1], a_ptr); \
+        MF2_LOAD(q_, 7, 4, 5, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 2) * 4096, a_off[A_LOAD_BLOCK12(U) + 2], a_ptr); \
+        MF2_LOAD(q_, 7, 6, 7, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 3) * 4096, a_off[A_LOAD_BLOCK12(U) + 3], a_ptr); \
+        SB();                                                                                  \
+        b_ptr += b_step;                                                                       \
+        if constexpr(((U) & 1) == 0)                                                           \
+            a_ptr += 2 * BK;                                                                   \
+    } while(0)
+
     // ---- main loop -----------------------------------------------------------------------------
     // Prologue: K step 0 of A, then what slabs -4 .. -1 would have issued.
 #pragma unroll
@@ -1693,6 +1808,22 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
         RB(0, 0, j, 1);
     }
     int kt = 0;
+    if(nk > 17)
+    {
+        // b_ptr: slab kt + 4 of B; a_ptr: K step a_step_of(kt) of A; both for the slab about to run
+        const int64_t b_step = TRANS_B ? (int64_t)BK : (int64_t)BK * p.ldb;
+        const uint8_t* b_ptr = gb + 4 * b_step;
+        const uint8_t* a_ptr = ga + 2 * (2 * BK);
+        uint32_t m0_saved;
+        asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
+        for(; kt + 17 < nk; kt += 12)
+        {
+            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
+            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
+            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
+        }
+        asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
+    }
     for(; kt + 6 < nk; kt += 2)
     {
         SLAB(kt, 0, true);
@@ -1711,6 +1842,15 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3"
                  : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
                    "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]));
+#undef SLAB12
+#undef OTHER12
+#undef ROW12_READS
+#undef A_LOAD_BLOCK12
+#undef A_LOAD_STAGE12
+#undef MF2_LOAD
+#undef RB12
+#undef RA12
+#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
