@@ -1575,6 +1575,16 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                        "+v"(fb[Q][0]), "+v"(fb[Q][1]), "+v"(fb[Q][2]), "+v"(fb[Q][3]),             \
                        "+v"(fb[Q][4]), "+v"(fb[Q][5]), "+v"(fb[Q][6]), "+v"(fb[Q][7])::"memory");   \
     } while(0)
+    // the same and at most 16 vector-memory operations in flight, as one instruction
+#define WAIT_FRAGS_VM16(Q)                                                                         \
+    do                                                                                             \
+    {                                                                                              \
+        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)"                                              \
+                     : "+v"(fa[Q][0]), "+v"(fa[Q][1]), "+v"(fa[Q][2]), "+v"(fa[Q][3]),             \
+                       "+v"(fa[Q][4]), "+v"(fa[Q][5]), "+v"(fa[Q][6]), "+v"(fa[Q][7]),             \
+                       "+v"(fb[Q][0]), "+v"(fb[Q][1]), "+v"(fb[Q][2]), "+v"(fb[Q][3]),             \
+                       "+v"(fb[Q][4]), "+v"(fb[Q][5]), "+v"(fb[Q][6]), "+v"(fb[Q][7])::"memory");   \
+    } while(0)
     // The MFMA as an assembly statement with the accumulator tied to the accumulation registers:
     // left to the register allocator, a part of the 256 accumulators ends up in ordinary
     // registers and scratch memory and is copied in and out around every instruction.  The
@@ -1712,15 +1722,36 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
             }                                                                                  \
         }                                                                                      \
     } while(0)
-    // two MFMAs with one load behind them; M0 (the load's LDS destination) is written first
-#define MF2_LOAD(Q, I, J0, J1, LDS_CONST, OFF, BASE)                                           \
-    asm volatile("s_add_i32 m0, %[wl], %[lc]\n\t"                                              \
-                 "v_mfma_i32_16x16x64_i8 %[c0], %[b0], %[a], %[c0]\n\t"                        \
+    // a row of eight MFMAs with a load behind every pair; M0 (the load's LDS destination) is
+    // written between the two MFMAs of the pair, an MFMA away from the load that uses it and from
+    // the load before (one statement: between two statements the compiler puts a wait state)
+#define MF8_LOAD4(Q, I, LDS_CONST, OFF0, OFF1, OFF2, OFF3, BASE)                                 \
+    asm volatile("v_mfma_i32_16x16x64_i8 %[c0], %[b0], %[a], %[c0]\n\t"                        \
+                 "s_add_i32 m0, %[wl], %[lc0]\n\t"                                             \
                  "v_mfma_i32_16x16x64_i8 %[c1], %[b1], %[a], %[c1]\n\t"                        \
-                 "global_load_lds_dwordx4 %[off], %[base]"                                     \
-                 : [c0] "+a"(acc[I][J0]), [c1] "+a"(acc[I][J1])                                \
-                 : [b0] "v"(fb[Q][J0]), [b1] "v"(fb[Q][J1]), [a] "v"(fa[Q][I]),                \
-                   [wl] "s"(wave_lds), [lc] "n"(LDS_CONST), [off] "v"(OFF), [base] "s"(BASE)   \
+                 "global_load_lds_dwordx4 %[o0], %[base]\n\t"                                  \
+                 "v_mfma_i32_16x16x64_i8 %[c2], %[b2], %[a], %[c2]\n\t"                        \
+                 "s_add_i32 m0, %[wl], %[lc1]\n\t"                                             \
+                 "v_mfma_i32_16x16x64_i8 %[c3], %[b3], %[a], %[c3]\n\t"                        \
+                 "global_load_lds_dwordx4 %[o1], %[base]\n\t"                                  \
+                 "v_mfma_i32_16x16x64_i8 %[c4], %[b4], %[a], %[c4]\n\t"                        \
+                 "s_add_i32 m0, %[wl], %[lc2]\n\t"                                             \
+                 "v_mfma_i32_16x16x64_i8 %[c5], %[b5], %[a], %[c5]\n\t"                        \
+                 "global_load_lds_dwordx4 %[o2], %[base]\n\t"                                  \
+                 "v_mfma_i32_16x16x64_i8 %[c6], %[b6], %[a], %[c6]\n\t"                        \
+                 "s_add_i32 m0, %[wl], %[lc3]\n\t"                                             \
+                 "v_mfma_i32_16x16x64_i8 %[c7], %[b7], %[a], %[c7]\n\t"                        \
+                 "global_load_lds_dwordx4 %[o3], %[base]"                                      \
+                 : [c0] "+a"(acc[I][0]), [c1] "+a"(acc[I][1]), [c2] "+a"(acc[I][2]),           \
+                   [c3] "+a"(acc[I][3]), [c4] "+a"(acc[I][4]), [c5] "+a"(acc[I][5]),           \
+                   [c6] "+a"(acc[I][6]), [c7] "+a"(acc[I][7])                                  \
+                 : [b0] "v"(fb[Q][0]), [b1] "v"(fb[Q][1]), [b2] "v"(fb[Q][2]),                 \
+                   [b3] "v"(fb[Q][3]), [b4] "v"(fb[Q][4]), [b5] "v"(fb[Q][5]),                 \
+                   [b6] "v"(fb[Q][6]), [b7] "v"(fb[Q][7]), [a] "v"(fa[Q][I]),                  \
+                   [wl] "s"(wave_lds), [lc0] "n"((LDS_CONST) + 0 * 4096),                      \
+                   [lc1] "n"((LDS_CONST) + 1 * 4096), [lc2] "n"((LDS_CONST) + 2 * 4096),       \
+                   [lc3] "n"((LDS_CONST) + 3 * 4096), [o0] "v"(OFF0), [o1] "v"(OFF1),          \
+                   [o2] "v"(OFF2), [o3] "v"(OFF3), [base] "s"(BASE)                            \
                  : "memory", "scc")
     // the A step whose half slab U loads, as a stage, and the first block of that half
 #define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
@@ -1745,20 +1776,16 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
     do                                                                                         \
     {                                                                                          \
         constexpr int q_ = (U) & 1;                                                            \
-        WAIT_FRAGS(q_);                                                                        \
-        wait_vmcnt<16>();                                                                      \
+        WAIT_FRAGS_VM16(q_);                                                                   \
         block_barrier();                                                                       \
         ROW12_READS(U, q_, 0, 0);  ROW12_READS(U, q_, 1, 4);  ROW12_READS(U, q_, 2, 8);        \
         ROW12_READS(U, q_, 3, 12); ROW12_READS(U, q_, 4, 16); ROW12_READS(U, q_, 5, 20);       \
         SB();                                                                                  \
-        MF2_LOAD(q_, 6, 0, 1, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 0 * 4096, b_off[0], b_ptr); \
-        MF2_LOAD(q_, 6, 2, 3, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 1 * 4096, b_off[1], b_ptr); \
-        MF2_LOAD(q_, 6, 4, 5, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 2 * 4096, b_off[2], b_ptr); \
-        MF2_LOAD(q_, 6, 6, 7, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES + 3 * 4096, b_off[3], b_ptr); \
-        MF2_LOAD(q_, 7, 0, 1, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 0) * 4096, a_off[A_LOAD_BLOCK12(U) + 0], a_ptr); \
-        MF2_LOAD(q_, 7, 2, 3, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 1) * 4096, a_off[A_LOAD_BLOCK12(U) + 1], a_ptr); \
-        MF2_LOAD(q_, 7, 4, 5, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 2) * 4096, a_off[A_LOAD_BLOCK12(U) + 2], a_ptr); \
-        MF2_LOAD(q_, 7, 6, 7, A_LOAD_STAGE12(U) * A2_BYTES + (A_LOAD_BLOCK12(U) + 3) * 4096, a_off[A_LOAD_BLOCK12(U) + 3], a_ptr); \
+        MF8_LOAD4(q_, 6, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES,                     \
+                  b_off[0], b_off[1], b_off[2], b_off[3], b_ptr);                              \
+        MF8_LOAD4(q_, 7, A_LOAD_STAGE12(U) * A2_BYTES + A_LOAD_BLOCK12(U) * 4096,              \
+                  a_off[A_LOAD_BLOCK12(U) + 0], a_off[A_LOAD_BLOCK12(U) + 1],                  \
+                  a_off[A_LOAD_BLOCK12(U) + 2], a_off[A_LOAD_BLOCK12(U) + 3], a_ptr);          \
         SB();                                                                                  \
         b_ptr += b_step;                                                                       \
         if constexpr(((U) & 1) == 0)                                                           \
@@ -1847,7 +1874,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 #undef ROW12_READS
 #undef A_LOAD_BLOCK12
 #undef A_LOAD_STAGE12
-#undef MF2_LOAD
+#undef MF8_LOAD4
 #undef RB12
 #undef RA12
 #undef A_STAGE12
@@ -1856,6 +1883,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 #undef ROW
 #undef OTHER
 #undef MF
+#undef WAIT_FRAGS_VM16
 #undef WAIT_FRAGS
 #undef RB
 #undef RA
