@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes one 8192^3 int8 quant_dot launch moves, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # counter runs of this file scaled by the same counters' reading for a plain copy of known size
 # (profiles/quant_dot_int8_8192_counters.md holds both runs and the arithmetic).
-HEADLINE_TRAFFIC_BYTES = 1.0745e9
+HEADLINE_TRAFFIC_BYTES = 1.0750e9
 HEADLINE_SETTLE_MS = 250.0
 RANDOM_OPERAND_CEILING_TOPS = 4080.0   # v_mfma_i32_16x16x64_i8 from registers, uniformly random operands, this chip
 
