@@ -4014,6 +4014,129 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
         SB();                                                                               \
     } while(0)
 
+    // ---- the steady state in trips of twelve slabs, as in qgemm_w4_mx4_kernel: the 16 fragment
+    // reads follow the first eight of a slab's 16 MFMAs (two each), the eight loads the last eight.
+    uint32_t a_vaddr[2][2][2]; // [slab parity][chunk][0: stages 0 and 1, 1: stage 2]
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+#pragma unroll
+        for(int x = 0; x < 2; x++)
+        {
+            a_vaddr[h][x][0] = lds0 + a_lane[h][x];
+            a_vaddr[h][x][1] = lds0 + a_lane[h][x] + 2 * A2_BYTES;
+        }
+    const uint32_t b_vaddr[2] = {lds0 + b_lane[0], lds0 + b_lane[1]};
+    const uint32_t wave_lds   = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    const uint32_t sa_off     = (uint32_t)(m0 + wave_m * 128 + lrow) * 4u;
+    const uint32_t sb_off     = (uint32_t)(n0 + wave_n * 128 + lrow) * 4u;
+#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
+#define RA12(U1, Q, I, X)                                                                       \
+    do                                                                                          \
+    {                                                                                           \
+        v4i t_;                                                                                 \
+        RD128(t_, a_vaddr[(U1) & 1][X][A_STAGE12(U1) == 2 ? 1 : 0],                             \
+              (A_STAGE12(U1) == 2 ? 0 : A_STAGE12(U1) * A2_BYTES) + (I) * 32 * 2 * BK);         \
+        PUT4(fa[Q][I], X, t_);                                                                  \
+    } while(0)
+#define RB12(U1, Q, J, R)                                                                       \
+    do                                                                                          \
+    {                                                                                           \
+        v4i t_;                                                                                 \
+        RD128(t_, b_vaddr[R], ((U1) & (STAGES - 1)) * B_BYTES + (J) * 32 * BK);                 \
+        PUT4(fb[Q][J], R, t_);                                                                  \
+    } while(0)
+#define LDS1S(dst, off, base, imm)                                                              \
+    asm volatile("global_load_dword %0, %1, %2 offset:%3"                                       \
+                 : "=v"(dst)                                                                    \
+                 : "v"(off), "s"(base), "n"(imm)                                                \
+                 : "memory")
+#define LOAD_SCALES12(Q)                                                                        \
+    do                                                                                          \
+    {                                                                                           \
+        LDS1S(sin[Q][0], sa_off, sa_run, 0);   LDS1S(sin[Q][1], sa_off, sa_run, 128);           \
+        LDS1S(sin[Q][2], sa_off, sa_run, 256); LDS1S(sin[Q][3], sa_off, sa_run, 384);           \
+        LDS1S(sin[Q][4], sb_off, sb_run, 0);   LDS1S(sin[Q][5], sb_off, sb_run, 128);           \
+        LDS1S(sin[Q][6], sb_off, sb_run, 256); LDS1S(sin[Q][7], sb_off, sb_run, 384);           \
+    } while(0)
+#define MF12(Q, I, J)                                                                           \
+    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]"    \
+                 : "+a"(acc[I][J])                                                              \
+                 : "v"(fb[Q][J]), "v"(fa[Q][I]), "v"(sc[4 + (J)]), "v"(sc[I]))
+#define READ12(U, Q, N)                                                                         \
+    do                                                                                          \
+    {                                                                                           \
+        if constexpr((N) < 8)                                                                   \
+            RA12((U) + 1, 1 - (Q), (N) >> 1, (N) & 1);                                          \
+        else                                                                                    \
+            RB12((U) + 1, 1 - (Q), ((N) - 8) >> 1, ((N) - 8) & 1);                              \
+    } while(0)
+#define ROW12_READS(U, Q, I, N0)                                                                \
+    do                                                                                          \
+    {                                                                                           \
+        SB(); MF12(Q, I, 0); SB(); READ12(U, Q, (N0) + 0); READ12(U, Q, (N0) + 1);              \
+        SB(); MF12(Q, I, 1); SB(); READ12(U, Q, (N0) + 2); READ12(U, Q, (N0) + 3);              \
+        SB(); MF12(Q, I, 2); SB(); READ12(U, Q, (N0) + 4); READ12(U, Q, (N0) + 5);              \
+        SB(); MF12(Q, I, 3); SB(); READ12(U, Q, (N0) + 6); READ12(U, Q, (N0) + 7);              \
+    } while(0)
+#define MF4_LOAD4(Q, I, LDS_CONST, OFF0, OFF1, OFF2, OFF3, BASE)                                \
+    asm volatile("s_add_i32 m0, %[wl], %[lc0]\n\t"                                              \
+                 "v_mfma_scale_f32_32x32x64_f8f6f4 %[c0], %[b0], %[a], %[c0], %[s0], %[sa] op_sel_hi:[0,0,0]\n\t" \
+                 "global_load_lds_dwordx4 %[o0], %[base]\n\t"                                   \
+                 "s_nop 0\n\t"                                                                  \
+                 "s_add_i32 m0, %[wl], %[lc1]\n\t"                                              \
+                 "v_mfma_scale_f32_32x32x64_f8f6f4 %[c1], %[b1], %[a], %[c1], %[s1], %[sa] op_sel_hi:[0,0,0]\n\t" \
+                 "global_load_lds_dwordx4 %[o1], %[base]\n\t"                                   \
+                 "s_nop 0\n\t"                                                                  \
+                 "s_add_i32 m0, %[wl], %[lc2]\n\t"                                              \
+                 "v_mfma_scale_f32_32x32x64_f8f6f4 %[c2], %[b2], %[a], %[c2], %[s2], %[sa] op_sel_hi:[0,0,0]\n\t" \
+                 "global_load_lds_dwordx4 %[o2], %[base]\n\t"                                   \
+                 "s_nop 0\n\t"                                                                  \
+                 "s_add_i32 m0, %[wl], %[lc3]\n\t"                                              \
+                 "v_mfma_scale_f32_32x32x64_f8f6f4 %[c3], %[b3], %[a], %[c3], %[s3], %[sa] op_sel_hi:[0,0,0]\n\t" \
+                 "global_load_lds_dwordx4 %[o3], %[base]"                                       \
+                 : [c0] "+a"(acc[I][0]), [c1] "+a"(acc[I][1]), [c2] "+a"(acc[I][2]),            \
+                   [c3] "+a"(acc[I][3])                                                         \
+                 : [b0] "v"(fb[Q][0]), [b1] "v"(fb[Q][1]), [b2] "v"(fb[Q][2]),                  \
+                   [b3] "v"(fb[Q][3]), [a] "v"(fa[Q][I]), [s0] "v"(sc[4]), [s1] "v"(sc[5]),     \
+                   [s2] "v"(sc[6]), [s3] "v"(sc[7]), [sa] "v"(sc[I]), [wl] "s"(wave_lds),       \
+                   [lc0] "n"((LDS_CONST) + 0 * 4096), [lc1] "n"((LDS_CONST) + 1 * 4096),        \
+                   [lc2] "n"((LDS_CONST) + 2 * 4096), [lc3] "n"((LDS_CONST) + 3 * 4096),        \
+                   [o0] "v"(OFF0), [o1] "v"(OFF1), [o2] "v"(OFF2), [o3] "v"(OFF3),              \
+                   [base] "s"(BASE)                                                             \
+                 : "memory", "scc")
+#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
+#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
+#define SLAB12(U)                                                                               \
+    do                                                                                          \
+    {                                                                                           \
+        constexpr int q_ = (U) & 1;                                                             \
+        /* may stay in flight: the loads of the last two slabs and the next slab's scale words */ \
+        asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)"                                           \
+                     : "+v"(fa[q_][0]), "+v"(fa[q_][1]), "+v"(fa[q_][2]), "+v"(fa[q_][3]),      \
+                       "+v"(fb[q_][0]), "+v"(fb[q_][1]), "+v"(fb[q_][2]), "+v"(fb[q_][3])::"memory"); \
+        block_barrier();                                                                        \
+        asm volatile("" : "+v"(sin[q_][0]), "+v"(sin[q_][1]), "+v"(sin[q_][2]), "+v"(sin[q_][3]), \
+                          "+v"(sin[q_][4]), "+v"(sin[q_][5]), "+v"(sin[q_][6]), "+v"(sin[q_][7])); \
+        _Pragma("unroll") for(int t_ = 0; t_ < 8; t_++) sc[t_] = sin[q_][t_] >> sc_shift;        \
+        asm volatile("" : "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]),                   \
+                          "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));                   \
+        LOAD_SCALES12(q_);                                                                      \
+        ROW12_READS(U, q_, 0, 0);                                                               \
+        ROW12_READS(U, q_, 1, 8);                                                               \
+        SB();                                                                                   \
+        MF4_LOAD4(q_, 2, W4_B_BASE + (((U) + 4) & (STAGES - 1)) * B_BYTES,                      \
+                  b_off[0], b_off[1], b_off[2], b_off[3], b_ptr);                               \
+        MF4_LOAD4(q_, 3, A_LOAD_STAGE12(U) * A2_BYTES + A_LOAD_BLOCK12(U) * 4096,               \
+                  a_off[A_LOAD_BLOCK12(U) + 0], a_off[A_LOAD_BLOCK12(U) + 1],                   \
+                  a_off[A_LOAD_BLOCK12(U) + 2], a_off[A_LOAD_BLOCK12(U) + 3], a_ptr);           \
+        SB();                                                                                   \
+        b_ptr += b_step;                                                                        \
+        sa_run += sa_step;                                                                      \
+        sb_run += sb_step;                                                                      \
+        if constexpr(((U) & 1) == 0)                                                            \
+            a_ptr += 2 * BK;                                                                    \
+    } while(0)
+
     // ---- main loop: the schedule of qgemm_w4_i8_kernel ------------------------------------------
 #pragma unroll
     for(int h = 0; h < 8; h++)
@@ -4062,6 +4185,25 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
         RB(0, 0, j, 3);
     }
     int kt = 0;
+    if(nk > 17)
+    {
+        // b_ptr: slab kt + 4 of B; a_ptr: K step a_step_of(kt) of A; sa_run / sb_run: the exponent
+        // words of slab kt + 2; all for the slab about to run
+        const int64_t b_step = BK;
+        const uint8_t* b_ptr = gb + 4 * b_step;
+        const uint8_t* a_ptr = ga + 2 * (2 * BK);
+        const uint8_t* sa_run = p.mx_ea + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_a * 4 + 2 * sa_step;
+        const uint8_t* sb_run = p.mx_eb + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_b * 4 + 2 * sb_step;
+        uint32_t m0_saved;
+        asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
+        for(; kt + 17 < nk; kt += 12)
+        {
+            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
+            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
+            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
+        }
+        asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
+    }
     for(; kt + 6 < nk; kt += 2)
     {
         SLAB(kt, 0, true);
@@ -4085,6 +4227,18 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
                       "+v"(sin[0][5]), "+v"(sin[0][6]), "+v"(sin[0][7]), "+v"(sin[1][0]), "+v"(sin[1][1]),
                       "+v"(sin[1][2]), "+v"(sin[1][3]), "+v"(sin[1][4]), "+v"(sin[1][5]), "+v"(sin[1][6]),
                       "+v"(sin[1][7]));
+#undef SLAB12
+#undef A_LOAD_BLOCK12
+#undef A_LOAD_STAGE12
+#undef MF4_LOAD4
+#undef ROW12_READS
+#undef READ12
+#undef MF12
+#undef LOAD_SCALES12
+#undef LDS1S
+#undef RB12
+#undef RA12
+#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
