@@ -150,3 +150,42 @@ def scan_assembly_loads(path, only=None):
                     seen += 1
                     pending.append([dest, 0, number])
     return seen, hazards
+
+
+def scan_m0_writes(path, only=None):
+    """A third hazard the compiler cannot see: inside inline assembly, a write of M0 needs one wait
+    state (any instruction) before a direct-to-LDS load reads it as its LDS destination.  The
+    twelve-slab loops of the four-wave GEMM kernels write M0 themselves.  Returns (M0 writes seen
+    inside assembly regions, hazards): a hazard is an assembly M0 write whose next instruction is a
+    ``global_load_lds_*`` / ``buffer_load_* ... lds``."""
+    hazards, seen = [], 0
+    kernel, in_asm, m0_just_written = None, False, None
+    with open(path) as f:
+        for number, raw in enumerate(f, 1):
+            text = raw.strip()
+            if text.startswith(";;#ASMSTART"):
+                in_asm = True
+                continue
+            if text.startswith(";;#ASMEND"):
+                in_asm = False
+                continue
+            label = _LABEL.match(text)
+            if label:
+                kernel, m0_just_written = label.group(1), None
+                continue
+            if not text or text[0] in ".;":
+                continue
+            if only is not None and (kernel is None or only not in kernel):
+                continue
+            text = text.split(";")[0].strip()
+            parts = text.replace(",", " ").split()
+            op, operands = parts[0], parts[1:]
+            is_lds_load = op.startswith("global_load_lds") or (op.startswith("buffer_load") and "lds" in operands)
+            if is_lds_load and m0_just_written is not None:
+                hazards.append(f"{kernel}: line {number} `{text}` reads M0 written by the instruction before it "
+                               f"(line {m0_just_written})")
+            m0_just_written = None
+            if in_asm and op.startswith("s_") and operands and operands[0] == "m0":
+                seen += 1
+                m0_just_written = number
+    return seen, hazards
