@@ -172,6 +172,32 @@ def test_four_wave_kernel_bare_bit_exact(ops, m, n, k, batch, trans_b):
     assert got.dtype == np.int32 and np.array_equal(got, want)
 
 
+# The steady state of the four-wave kernels runs in trips of twelve slabs while kt + 17 < K / 64; what
+# is left goes through the two-slab loops.  K / 64 = 53 ends the trips at slab 36, 54 at 48; 59 and
+# 60 (odd / even with one more trip's worth missing), 65 (a trip boundary plus the longest tail) and
+# a K that is not a multiple of 128 (the last A step is half a step).
+@pytest.mark.parametrize("k", [3392, 3456, 3776, 3840, 4160, 7744])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_four_wave_kernels_trip_boundaries_bit_exact(ops, k, trans_b):
+    m, n, batch = 300, 520, 22   # 132 tiles: at least half the chip, so no K split (see above)
+    rng = np.random.default_rng(k + trans_b)
+    a = rng.integers(-128, 128, (batch, m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (batch, k, n), dtype=np.int8)
+    want = np.stack([orc.quant_dot(a[i], b[i], orc.I8) for i in range(batch)])
+    tb = dev(np.ascontiguousarray(b.transpose(0, 2, 1))).transpose(1, 2) if trans_b else dev(b)
+    print("w4 trips int8", k, trans_b, flush=True)
+    got = ops.quant_dot(dev(a), tb).cpu().numpy()
+    assert np.array_equal(got, want)
+    # fp8 on small integers: every partial sum is exact, so the result is the reference's bit for bit
+    a8 = orc.fp8_from_f32(rng.integers(-8, 9, (2, m, k)).astype(np.float32))
+    b8 = orc.fp8_from_f32(rng.integers(-8, 9, (2, k, n)).astype(np.float32))
+    want8 = np.stack([orc.quant_dot(a8[i], b8[i], orc.FP8) for i in range(2)])
+    tb8 = dev(np.ascontiguousarray(b8.transpose(0, 2, 1))).transpose(1, 2) if trans_b else dev(b8)
+    print("w4 trips fp8", k, trans_b, flush=True)
+    got8 = ops.quant_dot(dev(a8), tb8, fp8=True).cpu().numpy()
+    assert np.array_equal(got8, want8)
+
+
 @pytest.mark.parametrize("m,n,k,trans_b", [(260, 264, 3072, False), (512, 520, 3136, True), (100, 1028, 4160, False)])
 @pytest.mark.parametrize("zp_a,zp_b", [(0, 0), (7, -9)])
 @pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
