@@ -1079,6 +1079,93 @@ std::vector<instruction_ref> parse_dynamicquantizelinear(const node_info& info,
 using multi_parser = std::function<std::vector<instruction_ref>(const node_info&, const std::vector<instruction_ref>&)>;
 
 // operators with several outputs
+// MatMulBnb4 (src/onnx/parse_matmulbnb4.cpp:38-275): B holds N * K 4-bit codes, two per byte, low
+// nibble first, row n of the [N, K] weight after row n - 1; absmax one float per block of
+// block_size consecutive codes.  quant_type 0 (FP4 there): weight = code / 8 * absmax; 1 (NF4):
+// weight = table[code] * absmax.  The result is A x weight^T with the vector and batch rules of
+// :249-275.  The codes index the table as int32 here (the reference converts to int64).
+instruction_ref parse_matmulbnb4(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    auto& m = *info.mod;
+    auto need = [&](const char* a) {
+        if(not info.has(a))
+            MIGRAPHX_THROW(std::string("MatMulBnb4: Attribute ") + a + " is required but missing");
+        return info.attr(a).i;
+    };
+    const auto n     = static_cast<std::size_t>(need("N"));
+    const auto k     = static_cast<std::size_t>(need("K"));
+    const auto block = need("block_size");
+    if(block < 16 or (block & (block - 1)) != 0)
+        MIGRAPHX_THROW("MatMulBnb4: block_size must be a power of 2 and >= 16, actual value: " +
+                       std::to_string(block));
+    const auto quant = need("quant_type");
+    if(quant != 0 and quant != 1)
+        MIGRAPHX_THROW("MatMulBnb4: quant_type must be 0 (FP4) or 1 (NF4), actual value: " + std::to_string(quant));
+    if(args.size() < 3)
+        MIGRAPHX_THROW("MatMulBnb4: requires exactly 3 inputs (A, B, absmax)");
+    auto a             = args[0];
+    const auto a_shape = a->get_shape();
+    if(a_shape.scalar())
+        MIGRAPHX_THROW("MatMulBnb4: Input A must have at least 1 dimension");
+    if(a_shape.lens().back() != k)
+        MIGRAPHX_THROW("MatMulBnb4: Input A inner dimension (" + std::to_string(a_shape.lens().back()) +
+                       ") must match attribute K (" + std::to_string(k) + ")");
+    const std::size_t codes = n * k, bs = static_cast<std::size_t>(block);
+    const std::vector<std::size_t> b_lens{(codes + 1) / 2}, s_lens{(codes + bs - 1) / bs};
+    if(args[1]->get_shape().lens() != b_lens)
+        MIGRAPHX_THROW("MatMulBnb4: Input B does not match expected dims: {" + lens_string(b_lens) +
+                       "}. Actual dims: {" + lens_string(args[1]->get_shape().lens()) + "}");
+    if(args[2]->get_shape().lens() != s_lens)
+        MIGRAPHX_THROW("MatMulBnb4: Input absmax does not match expected dims: {" + lens_string(s_lens) +
+                       "}. Actual dims: {" + lens_string(args[2]->get_shape().lens()) + "}");
+
+    auto first = [&](instruction_ref x, std::size_t have) {
+        if(have > codes)
+            x = m.add_instruction(make_op("slice", {{"axes", {0}}, {"starts", {0}}, {"ends", {codes}}}), x);
+        return m.add_instruction(make_op("reshape", {{"dims", {n, k}}}), x);
+    };
+    auto w = first(m.add_instruction(make_op("unpack_int4"), args[1]), 2 * b_lens[0]);
+    // every absmax repeated over its block, then cut to the N * K codes
+    auto s = m.add_instruction(make_op("unsqueeze", {{"axes", {1}}}), args[2]);
+    s      = m.add_instruction(make_op("multibroadcast", {{"out_lens", {s_lens[0], bs}}}), s);
+    s      = first(m.add_instruction(make_op("reshape", {{"dims", {s_lens[0] * bs}}}), s), s_lens[0] * bs);
+    instruction_ref value;
+    if(quant == 0)
+    {
+        auto f     = m.add_instruction(make_op("convert", {{"target_type", shape::float_type}}), w);
+        auto eight = m.add_literal(literal{shape{shape::float_type}, std::vector<float>{8.0f}});
+        eight      = m.add_instruction(make_op("multibroadcast", {{"out_lens", {n, k}}}), eight);
+        value      = m.add_instruction(make_op("div"), f, eight);
+    }
+    else
+    {
+        const std::vector<float> nf4 = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+                                        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+                                        0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f,
+                                        0.33791524171829224f, 0.44070982933044434f, 0.5626170039176941f,
+                                        0.7229568362236023f, 1.0f};
+        auto table = m.add_literal(literal{shape{shape::float_type, {16}}, nf4});
+        auto index = m.add_instruction(make_op("convert", {{"target_type", shape::int32_type}}), w);
+        value      = m.add_instruction(make_op("gather", {{"axis", 0}}), table, index);
+    }
+    auto wt = m.add_instruction(make_op("mul"), value, s);
+    wt      = m.add_instruction(make_op("transpose", {{"permutation", {1, 0}}}), wt);
+    const auto rank = a_shape.ndim();
+    if(rank == 1)
+        a = m.add_instruction(make_op("unsqueeze", {{"axes", {0}}}), a);
+    if(rank > 2)
+    {
+        auto lens = a_shape.lens();
+        lens[rank - 2] = k;
+        lens[rank - 1] = n;
+        wt = m.add_instruction(make_op("multibroadcast", {{"out_lens", lens}}), wt);
+    }
+    auto out = m.add_instruction(make_op("dot"), a, wt);
+    if(rank == 1)
+        out = m.add_instruction(make_op("squeeze", {{"axes", {0}}}), out);
+    return out;
+}
+
 const std::unordered_map<std::string, multi_parser>& multi_parsers()
 {
     static const std::unordered_map<std::string, multi_parser> table = {
@@ -1092,6 +1179,7 @@ const std::unordered_map<std::string, node_parser>& parsers()
     static const std::unordered_map<std::string, node_parser> table = {
         {"MatMul", parse_matmul},
         {"MatMulNBits", parse_matmulnbits},
+        {"MatMulBnb4", parse_matmulbnb4},
         {"DequantizeLinear", parse_dequantizelinear},
         {"QuantizeLinear", parse_quantizelinear},
         {"QLinearMatMul", parse_qlinearmatmul},

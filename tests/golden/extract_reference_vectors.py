@@ -423,6 +423,32 @@ for stem in ("dynamicquantizelinear_1d_test", "dynamicquantizelinear_2d_test"):
         shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
 out["onnx_dynamicquantizelinear"] = dql
 
+# ---- MatMulBnb4 models (test/onnx/verify/matmulbnb4_tests.cpp): A, the packed 4-bit codes, absmax, result
+bnb = []
+rel = "test/onnx/verify/matmulbnb4_tests.cpp"
+for name, body in test_cases(read(rel)).items():
+    model = re.search(r'optimize_onnx\("([^"]+)"\)', body).group(1)
+    c = {"name": name, "source": rel, "model": model, "inputs": {}}
+    for param, var in re.findall(r'pm\["(\w+)"\]\s*=\s*migraphx::argument\(\w+,\s*(\w+)\.data\(\)\)', body):
+        v = vec(body, var)
+        if v is None:
+            # std::vector<float> a(a_shape.elements()); std::iota(a.begin(), a.end(), start)
+            start = num(re.search(r"std::iota\(" + var + r"\.begin\(\),\s*" + var + r"\.end\(\),\s*([^)]+)\)", body).group(1))
+            n = 1
+            for d in shape(body, var + "_shape")["lens"]:
+                n *= d
+            v = [start + i for i in range(n)]
+        c["inputs"][param] = v
+    c["gold"] = vec(body, "gold")
+    c["lens"] = num_list(re.search(r"get_shape\(\)\.lens\(\) == std::vector<size_t>\{([^}]*)\}", body).group(1))
+    assert c["gold"] is not None and all(v is not None for v in c["inputs"].values()), name
+    bnb.append(c)
+import glob
+import shutil
+for f in sorted(glob.glob(os.path.join(REF, "test/onnx", "matmulbnb4_*.onnx"))):
+    shutil.copyfile(f, os.path.join(os.path.dirname(OUT), "onnx", os.path.basename(f)))
+out["onnx_matmulbnb4"] = bnb
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -97,6 +97,25 @@ def test_dynamicquantizelinear_models_on_device(golden, tmp_path):
         assert got[:len(c["y"])].tolist() == [float(v) for v in c["y"]], c["name"]
 
 
+def test_matmulbnb4_models_on_device(golden, tmp_path):
+    # test/onnx/verify/matmulbnb4_tests.cpp: codes and absmax are inputs of these models, so the
+    # unpacking, the table lookup (or code / 8), the scaling and the product all run on the device;
+    # every step is exact or correctly rounded, the product is the double sum of the CPU target
+    for c in golden["onnx_matmulbnb4"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], c["inputs"], tmp_path)
+        want = run_onnx("oracle", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == want.tolist(), c["name"]
+        np.testing.assert_allclose(got, np.float64(c["gold"]), rtol=2e-5, atol=1e-3, err_msg=c["name"])
+    # a larger layer (N = 64, K = 128, block 64; four rows of A) with seeded inputs
+    rng = np.random.default_rng(5)
+    inputs = {"A": rng.standard_normal(4 * 128).astype(np.float32), "B": rng.integers(0, 256, 64 * 128 // 2),
+              "absmax": (rng.random(128) + 0.5).astype(np.float32)}
+    got = run_onnx("mi355", "matmulbnb4_large_test.onnx", inputs, tmp_path)
+    want = run_onnx("oracle", "matmulbnb4_large_test.onnx", inputs, tmp_path)
+    assert got.tolist() == want.tolist()
+
+
 def test_written_qdq_conv_model_on_device(tmp_path):
     """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
     turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU

@@ -195,6 +195,16 @@ def test_matmul_vector_times_vector_value(tmp_path):
     ("dequantizelinear_too_many_inputs_test.onnx", "must have either 2 or 3 inputs, 4 inputs provided"),
     ("dequantizelinear_x_and_zp_type_mismatch_test.onnx", "x and y_zero_point must be of same type"),
     ("dequantizelinear_scale_and_zp_shape_mismatch_test.onnx", "y_scale and y_zero_point shape mismatch"),
+    # test/onnx/parse/matmulbnb4_tests.cpp
+    ("matmulbnb4_invalid_quant_type_test.onnx", "quant_type must be 0 (FP4) or 1 (NF4), actual value: "),
+    ("matmulbnb4_invalid_block_size_test.onnx", "block_size must be a power of 2 and >= 16, actual value: "),
+    ("matmulbnb4_invalid_block_size_small_test.onnx", "block_size must be a power of 2 and >= 16, actual value: "),
+    ("matmulbnb4_wrong_input_count_test.onnx", "requires exactly 3 inputs (A, B, absmax)"),
+    ("matmulbnb4_wrong_a_dims_test.onnx", "Input A must have at least 1 dimension"),
+    ("matmulbnb4_wrong_a_inner_dim_test.onnx", "must match attribute K"),
+    ("matmulbnb4_wrong_b_dims_test.onnx", "Input B does not match expected dims"),
+    ("matmulbnb4_wrong_absmax_dims_test.onnx", "Input absmax does not match expected dims"),
+    ("matmulbnb4_missing_n_attr_test.onnx", "Attribute N is required but missing"),
 ])
 def test_malformed_models_are_rejected_with_the_reference_messages(model, message):
     rc, text = print_onnx(model)
@@ -363,3 +373,54 @@ def test_written_qdq_matmul_model_becomes_quant_dot(tmp_path):
     xq = orc.quantizelinear(x, np.float32(1.0 / 32), np.int8(0), orc.F32, orc.I8)
     want = orc.qdq_matmul_int8(xq, w, np.float32(1.0 / 32), sw) + bias[None, :]
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+NF4_TABLE = np.float32([-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+                        -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+                        0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+                        0.7229568362236023, 1.0])
+
+
+def matmulbnb4_definition(a, b, absmax, n, k, block, nf4):
+    """The operator's definition in numpy: low nibble first, row n of the [N, K] weight behind row n - 1,
+    one absmax per block of consecutive codes; code / 8 or table[code], times absmax; A x W^T."""
+    b = np.asarray(b, np.uint8)
+    codes = np.stack([b & 15, b >> 4], axis=1).reshape(-1)[:n * k]
+    scale = np.repeat(np.float32(absmax), block)[:n * k]
+    value = NF4_TABLE[codes] if nf4 else codes.astype(np.float32) / np.float32(8)
+    w = (value * scale).reshape(n, k)
+    return np.float32(a).reshape(-1, k).astype(np.float64) @ w.T.astype(np.float64)
+
+
+MATMULBNB4_MODELS = {
+    # model: (N, K, block_size, NF4 table?) -- the attributes of test/onnx/gen_onnx.py's models
+    "matmulbnb4_fp4_test.onnx": (4, 8, 16, False), "matmulbnb4_nf4_test.onnx": (8, 16, 16, True),
+    "matmulbnb4_block32_test.onnx": (4, 16, 32, False), "matmulbnb4_fp4_1d_input_test.onnx": (4, 8, 16, False),
+    "matmulbnb4_fp4_3d_input_test.onnx": (4, 8, 16, False),
+}
+
+
+def test_matmulbnb4_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/matmulbnb4_tests.cpp (compared by RMS there; its NF4 numbers have six digits)
+    assert len(golden["onnx_matmulbnb4"]) == 5
+    for c in golden["onnx_matmulbnb4"]:
+        got = run_onnx("oracle", c["model"], c["inputs"], tmp_path)
+        gold = np.float64(c["gold"])
+        assert got.shape == gold.shape, c["name"]
+        np.testing.assert_allclose(got, gold, rtol=2e-5, atol=1e-3, err_msg=c["name"])
+        n, k, block, nf4 = MATMULBNB4_MODELS[c["model"]]
+        want = matmulbnb4_definition(c["inputs"]["A"], c["inputs"]["B"], c["inputs"]["absmax"], n, k, block, nf4)
+        np.testing.assert_allclose(got, want.reshape(-1), rtol=1e-6, err_msg=c["name"])
+
+
+def test_matmulbnb4_structure():
+    rc, text = print_onnx("matmulbnb4_nf4_test.onnx")
+    assert rc == 0, text
+    for op in ("unpack_int4", "gather[", "multibroadcast[", "transpose[", "dot"):
+        assert op in text, (op, text)
+    rc, text = print_onnx("matmulbnb4_fp4_3d_input_test.onnx")
+    assert rc == 0 and "div" in text and "gather[" not in text, text
+    ret = [l for l in text.splitlines() if "@return(" in l][0]
+    src = ret.split("@return(")[1].split(")")[0]
+    line = [l for l in text.splitlines() if l.startswith(src + " =")][0]
+    assert "float_type, {2, 3, 4}" in line, text
