@@ -1424,6 +1424,24 @@ constexpr int W4_A_STAGES = 3;
 constexpr int W4_B_BASE   = W4_A_STAGES * A2_BYTES;
 constexpr int W4_LDS_BYTES = W4_B_BASE + STAGES * B_BYTES; // 96 + 64 KiB
 
+// The steady state of the four-wave kernels runs in trips of twelve slabs (see qgemm_w4_i8_kernel).
+// For slab U = 0 .. 11 of a trip (kt = 12 t + U), as compile-time constants:
+// the A stage slab U is read from,
+#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
+// the A stage that the half K step loaded during slab U goes to (K step (kt + 5) / 2 in an odd
+// slab, (kt + 4) / 2 in an even one), and the first of that half's four blocks
+#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
+#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
+// The trips themselves: SLAB(U) is the kernel's slab body; a trip runs only while every load of
+// its slabs' shares exists (slab kt + 15 of B and K step (kt + 16) / 2 of A: kt + 17 < nk).
+#define W4_TRIPS_OF_TWELVE(kt, nk, SLAB)                   \
+    for(; (kt) + 17 < (nk); (kt) += 12)                    \
+    {                                                      \
+        SLAB(0); SLAB(1); SLAB(2);  SLAB(3);               \
+        SLAB(4); SLAB(5); SLAB(6);  SLAB(7);               \
+        SLAB(8); SLAB(9); SLAB(10); SLAB(11);              \
+    }
+
 template <bool TRANS_B, bool DEQ, int OUT, bool VEC_STORE>
 __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 {
@@ -1694,7 +1712,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
         }
     }
     const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
 #define RA12(U1, Q, I)                                                                         \
     RD128(fa[Q][I], a_vaddr[(U1) & 1][A_STAGE12(U1) == 2 ? 1 : 0],                             \
           (A_STAGE12(U1) == 2 ? 0 : A_STAGE12(U1) * A2_BYTES) + (I) * 16 * 2 * BK)
@@ -1753,9 +1770,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
                    [lc3] "n"((LDS_CONST) + 3 * 4096), [o0] "v"(OFF0), [o1] "v"(OFF1),          \
                    [o2] "v"(OFF2), [o3] "v"(OFF3), [base] "s"(BASE)                            \
                  : "memory", "scc")
-    // the A step whose half slab U loads, as a stage, and the first block of that half
-#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
-#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
 #define ROW12_READS(U, Q, I, N0)                                                               \
     do                                                                                         \
     {                                                                                          \
@@ -1843,12 +1857,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
         const uint8_t* a_ptr = ga + 2 * (2 * BK);
         uint32_t m0_saved;
         asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
-        for(; kt + 17 < nk; kt += 12)
-        {
-            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
-            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
-            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
-        }
+        W4_TRIPS_OF_TWELVE(kt, nk, SLAB12);
         asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
     }
     for(; kt + 6 < nk; kt += 2)
@@ -1872,12 +1881,9 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 #undef SLAB12
 #undef OTHER12
 #undef ROW12_READS
-#undef A_LOAD_BLOCK12
-#undef A_LOAD_STAGE12
 #undef MF8_LOAD4
 #undef RB12
 #undef RA12
-#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
@@ -2689,7 +2695,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
             b_vaddr[j2] = lds0 + b_lane[0] + (uint32_t)(((wave_n * 8 + j2 * 2 + bcol) ^ bsw) << 4);
     }
     const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
 #define RA12(U1, Q, I, X)                                                                       \
     do                                                                                          \
     {                                                                                           \
@@ -2766,8 +2771,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
                    [o0] "v"(OFF0), [o1] "v"(OFF1), [o2] "v"(OFF2), [o3] "v"(OFF3),              \
                    [base] "s"(BASE)                                                             \
                  : "memory", "scc")
-#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
-#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
 #define SLAB12(U)                                                                               \
     do                                                                                          \
     {                                                                                           \
@@ -2844,12 +2847,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
         const uint8_t* a_ptr = ga + 2 * (2 * BK);
         uint32_t m0_saved;
         asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
-        for(; kt + 17 < nk; kt += 12)
-        {
-            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
-            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
-            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
-        }
+        W4_TRIPS_OF_TWELVE(kt, nk, SLAB12);
         asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
     }
     for(; kt + 6 < nk; kt += 2)
@@ -2871,15 +2869,12 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_f8_kernel(dma_params p)
     if(kt < nk)
         SLAB(kt, 0, false);
 #undef SLAB12
-#undef A_LOAD_BLOCK12
-#undef A_LOAD_STAGE12
 #undef MF4_LOAD4
 #undef ROW12_READS
 #undef MF12
 #undef READ12
 #undef RB12
 #undef RA12
-#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
@@ -3464,7 +3459,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
     const uint32_t wave_lds   = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const uint32_t sa_off     = (uint32_t)(m0 + wave_m * 128 + lrow) * 4u;
     const uint32_t sb_off     = (uint32_t)(n0 + wave_n * 128 + lrow) * 4u;
-#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
 #define RA12(U1, Q, I, X)                                                                       \
     RD128(fa[Q][I][X], a_vaddr[(U1) & 1][X][A_STAGE12(U1) == 2 ? 1 : 0],                        \
           (A_STAGE12(U1) == 2 ? 0 : A_STAGE12(U1) * A2_BYTES) + (I) * 32 * 2 * BK)
@@ -3552,8 +3546,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
                    [o0] "v"(OFF0), [o1] "v"(OFF1), [o2] "v"(OFF2), [o3] "v"(OFF3),              \
                    [base] "s"(BASE)                                                             \
                  : "memory", "scc")
-#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
-#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
 #define SLAB12(U)                                                                               \
     do                                                                                          \
     {                                                                                           \
@@ -3649,12 +3641,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
         const uint8_t* sb_run = p.mx_eb + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_b * 4 + 2 * sb_step;
         uint32_t m0_saved;
         asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
-        for(; kt + 17 < nk; kt += 12)
-        {
-            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
-            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
-            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
-        }
+        W4_TRIPS_OF_TWELVE(kt, nk, SLAB12);
         asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
     }
     for(; kt + 6 < nk; kt += 2)
@@ -3682,8 +3669,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
                       "+v"(sin[1][2]), "+v"(sin[1][3]), "+v"(sin[1][4]), "+v"(sin[1][5]), "+v"(sin[1][6]),
                       "+v"(sin[1][7]));
 #undef SLAB12
-#undef A_LOAD_BLOCK12
-#undef A_LOAD_STAGE12
 #undef MF4_LOAD4
 #undef ROW12_PLAIN
 #undef ROW12_READS
@@ -3693,7 +3678,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx4_kernel(dma_params p)
 #undef LDS1S
 #undef RB12
 #undef RA12
-#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
@@ -4029,7 +4013,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
     const uint32_t wave_lds   = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const uint32_t sa_off     = (uint32_t)(m0 + wave_m * 128 + lrow) * 4u;
     const uint32_t sb_off     = (uint32_t)(n0 + wave_n * 128 + lrow) * 4u;
-#define A_STAGE12(U) ((((U) >> 1)) % W4_A_STAGES)
 #define RA12(U1, Q, I, X)                                                                       \
     do                                                                                          \
     {                                                                                           \
@@ -4104,8 +4087,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
                    [o0] "v"(OFF0), [o1] "v"(OFF1), [o2] "v"(OFF2), [o3] "v"(OFF3),              \
                    [base] "s"(BASE)                                                             \
                  : "memory", "scc")
-#define A_LOAD_STAGE12(U) ((((U) & 1) != 0 ? ((U) + 5) / 2 : ((U) + 4) / 2) % W4_A_STAGES)
-#define A_LOAD_BLOCK12(U) (((U) & 1) != 0 ? 0 : 4)
 #define SLAB12(U)                                                                               \
     do                                                                                          \
     {                                                                                           \
@@ -4196,12 +4177,7 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
         const uint8_t* sb_run = p.mx_eb + (int64_t)blockIdx.y * (int64_t)nk * p.mx_rows_b * 4 + 2 * sb_step;
         uint32_t m0_saved;
         asm volatile("s_mov_b32 %0, m0" : "=s"(m0_saved));
-        for(; kt + 17 < nk; kt += 12)
-        {
-            SLAB12(0); SLAB12(1); SLAB12(2);  SLAB12(3);
-            SLAB12(4); SLAB12(5); SLAB12(6);  SLAB12(7);
-            SLAB12(8); SLAB12(9); SLAB12(10); SLAB12(11);
-        }
+        W4_TRIPS_OF_TWELVE(kt, nk, SLAB12);
         asm volatile("s_mov_b32 m0, %0" ::"s"(m0_saved));
     }
     for(; kt + 6 < nk; kt += 2)
@@ -4228,8 +4204,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
                       "+v"(sin[1][2]), "+v"(sin[1][3]), "+v"(sin[1][4]), "+v"(sin[1][5]), "+v"(sin[1][6]),
                       "+v"(sin[1][7]));
 #undef SLAB12
-#undef A_LOAD_BLOCK12
-#undef A_LOAD_STAGE12
 #undef MF4_LOAD4
 #undef ROW12_READS
 #undef READ12
@@ -4238,7 +4212,6 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_mx8_kernel(dma_params p)
 #undef LDS1S
 #undef RB12
 #undef RA12
-#undef A_STAGE12
 #undef SLAB
 #undef WAIT_SLAB
 #undef ROW
