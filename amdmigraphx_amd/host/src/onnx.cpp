@@ -1079,6 +1079,33 @@ std::vector<instruction_ref> parse_dynamicquantizelinear(const node_info& info,
 using multi_parser = std::function<std::vector<instruction_ref>(const node_info&, const std::vector<instruction_ref>&)>;
 
 // operators with several outputs
+// QLinearAdd / QLinearMul (src/onnx/parse_qlinearbinary.cpp:107-161): both operands dequantized with
+// their per-tensor scale and zero point, the float operation with numpy broadcasting, the result
+// quantized with the output's scale and (optional) zero point.
+instruction_ref parse_qlinearbinary(const std::string& op, const std::string& onnx_name, const node_info& info,
+                                    const std::vector<instruction_ref>& args)
+{
+    if(args.size() < 7)
+        MIGRAPHX_THROW(onnx_name + ": missing inputs");
+    const auto ta = args[0]->get_shape().type();
+    const auto tb = args[3]->get_shape().type();
+    for(auto t : {ta, tb})
+    {
+        if(t != shape::int8_type and t != shape::uint8_type)
+            MIGRAPHX_THROW(onnx_name + ": unsupported input type");
+    }
+    if(ta != tb)
+        MIGRAPHX_THROW(onnx_name + ": mismatched input types");
+    module& m = *info.mod;
+    auto a    = bcast_qdq(m, "dequantizelinear", args[0], args[1], args[2]);
+    auto b    = bcast_qdq(m, "dequantizelinear", args[3], args[4], args[5]);
+    auto c    = common_binary(m, op, a, b, onnx_name);
+    if(args.size() == 8)
+        return bcast_qdq(m, "quantizelinear", c, args[6], args[7]);
+    auto scale = m.add_instruction(make_op("multibroadcast", {{"out_lens", c->get_shape().lens()}}), args[6]);
+    return m.add_instruction(make_op("quantizelinear"), c, scale);
+}
+
 // MatMulBnb4 (src/onnx/parse_matmulbnb4.cpp:38-275): B holds N * K 4-bit codes, two per byte, low
 // nibble first, row n of the [N, K] weight after row n - 1; absmax one float per block of
 // block_size consecutive codes.  quant_type 0 (FP4 there): weight = code / 8 * absmax; 1 (NF4):
@@ -1180,6 +1207,8 @@ const std::unordered_map<std::string, node_parser>& parsers()
         {"MatMul", parse_matmul},
         {"MatMulNBits", parse_matmulnbits},
         {"MatMulBnb4", parse_matmulbnb4},
+        {"QLinearAdd", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_qlinearbinary("add", "QLinearAdd", i, a); }},
+        {"QLinearMul", [](const node_info& i, const std::vector<instruction_ref>& a) { return parse_qlinearbinary("mul", "QLinearMul", i, a); }},
         {"DequantizeLinear", parse_dequantizelinear},
         {"QuantizeLinear", parse_quantizelinear},
         {"QLinearMatMul", parse_qlinearmatmul},

@@ -449,6 +449,21 @@ for f in sorted(glob.glob(os.path.join(REF, "test/onnx", "matmulbnb4_*.onnx"))):
     shutil.copyfile(f, os.path.join(os.path.dirname(OUT), "onnx", os.path.basename(f)))
 out["onnx_matmulbnb4"] = bnb
 
+# ---- QLinearAdd / QLinearMul models (test/onnx/verify/qlinear{add,mul}[_bcast]_test.cpp): 8-bit results
+qlb = []
+for stem in ("qlinearadd_test", "qlinearadd_bcast_test", "qlinearmul_test", "qlinearmul_bcast_test"):
+    rel = "test/onnx/verify/" + stem + ".cpp"
+    for name, body in test_cases(read(rel)).items():
+        model = re.search(r'read_onnx\("([^"]+)"\)', body).group(1)
+        c = {"name": name, "source": rel, "model": model, "inputs": {}}
+        for param, var in re.findall(r'pp\["(\w+)"\]\s*=\s*migraphx::argument\(\w+,\s*(\w+)\.data\(\)\)', body):
+            c["inputs"][param] = vec(body, var)
+        c["gold"] = vec(body, "gold")
+        assert c["gold"] is not None and all(v is not None for v in c["inputs"].values()), name
+        qlb.append(c)
+        shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
+out["onnx_qlinearbinary"] = qlb
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

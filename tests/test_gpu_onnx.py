@@ -116,6 +116,14 @@ def test_matmulbnb4_models_on_device(golden, tmp_path):
     assert got.tolist() == want.tolist()
 
 
+def test_qlinearadd_and_qlinearmul_models_on_device(golden, tmp_path):
+    # test/onnx/verify/qlinear{add,mul}[_bcast]_test.cpp: dequantize, add / mul, quantize on the device
+    for c in golden["onnx_qlinearbinary"]:
+        print("onnx", c["name"], flush=True)
+        got = run_onnx("mi355", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
+
+
 def test_written_qdq_conv_model_on_device(tmp_path):
     """A QDQ-format convolution layer written as ONNX bytes: parse, compile for mi355 (simplify_qdq
     turns it into quant_convolution with the dequantize epilogue fused), bit-identical to the CPU

@@ -424,3 +424,25 @@ def test_matmulbnb4_structure():
     src = ret.split("@return(")[1].split(")")[0]
     line = [l for l in text.splitlines() if l.startswith(src + " =")][0]
     assert "float_type, {2, 3, 4}" in line, text
+
+
+def test_qlinearadd_and_qlinearmul_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/qlinearadd_test.cpp, qlinearadd_bcast_test.cpp, qlinearmul_test.cpp,
+    # qlinearmul_bcast_test.cpp: 8-bit results (compared by RMS there; here every value must be equal)
+    assert len(golden["onnx_qlinearbinary"]) == 4
+    for c in golden["onnx_qlinearbinary"]:
+        got = run_onnx("oracle", c["model"], c["inputs"], tmp_path)
+        assert got.tolist() == [float(v) for v in c["gold"]], c["name"]
+
+
+def test_qlinearbinary_rejects_mismatched_types(tmp_path):
+    import onnx_writer as ow
+    # A uint8, B int8: src/onnx/parse_qlinearbinary.cpp:124-125
+    inits = [("sa", np.float32([0.1])), ("za", np.uint8([0])), ("sb", np.float32([0.1])), ("zb", np.int8([0])),
+             ("sc", np.float32([0.1])), ("zc", np.uint8([0]))]
+    nodes = [ow.node("QLinearAdd", ["A", "sa", "za", "B", "sb", "zb", "sc", "zc"], ["C"], domain="com.microsoft")]
+    data = ow.model(nodes, [("A", ow.UINT8, [4]), ("B", ow.INT8, [4])], [("C", ow.UINT8, [4])], inits)
+    path = tmp_path / "bad.onnx"
+    path.write_bytes(data)
+    rc, text = print_onnx(str(path))
+    assert rc == 4 and "QLinearAdd: mismatched input types" in text, text
