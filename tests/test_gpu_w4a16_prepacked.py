@@ -101,11 +101,12 @@ def test_prepacked_dequantized_weights_are_exact(ops, zp, lo, hi):
         assert np.array_equal(orc.half_to_f32(got[0]), w1.astype(np.float32))
 
 
-@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 14336), (14336, 4096), (4096, 28672)])
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 14336), (14336, 4096), (4096, 28672), (8192, 28672), (28672, 8192)])
 def test_prepacked_full_size_config4_against_oracle(ops, k, n):
     """benchmark config 4 at its real sizes (M = 1) and the fused gate | up projection: sampled
     output columns against the oracle, every output against the kernel that reads the operator's
-    layout."""
+    layout.  (8192, 28672) has more row groups than one resident set of workgroups walks: one row
+    group per workgroup in a grid larger than the device holds at once; (28672, 8192) is the largest K."""
     g = torch.Generator(device="cuda")
     g.manual_seed(k + n)
     w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda", generator=g)
