@@ -163,3 +163,12 @@ MI355_DEVINL double load_as_f64(const void* p, int type, int64_t i)
     default: return 0.0;
     }
 }
+
+// quantizelinear's saturation: std::max(lo, std::min(hi, q)) with std::min / std::max's comparison
+// order, so a NaN ends up at hi exactly as on the reference's CPU target
+// (src/include/migraphx/op/quantizelinear.hpp:95-104)
+MI355_DEVINL double clamp_like_ref(double q, double lo, double hi)
+{
+    double v = (q < hi) ? q : hi;
+    return (lo < v) ? v : lo;
+}

@@ -232,9 +232,14 @@ struct chain_params
     float* out;
     int64_t rows, cols;
     int n_steps;
+    // Q: the chain's last value leaves as int8, quantized with one scale and one zero point for the
+    // whole tensor (quantizelinear's arithmetic: rintf(v / scale) + zp, clamped), instead of as float
+    int8_t* qout;
+    const float* qscale;
+    const int8_t* qzp;
 };
 
-template <int W, int R>
+template <int W, int R, bool Q = false>
 __global__ __launch_bounds__(256) void chain_kernel(chain_params p)
 {
 #pragma clang fp contract(off)
@@ -333,7 +338,23 @@ __global__ __launch_bounds__(256) void chain_kernel(chain_params p)
             const int64_t r = r0 + i;
             if(r >= p.rows)
                 break;
-            if constexpr(W == 4)
+            if constexpr(Q)
+            {
+                const float sv = p.qscale[0];
+                const double z = p.qzp != nullptr ? (double)p.qzp[0] : 0.0;
+                uint32_t w     = 0;
+#pragma unroll
+                for(int e = 0; e < W; e++)
+                {
+                    const double qv = clamp_like_ref((double)rintf(acc[i][e] / sv) + z, -128.0, 127.0);
+                    w |= (uint32_t)(uint8_t)(int8_t)(int)qv << (8 * e);
+                }
+                if constexpr(W == 4)
+                    *reinterpret_cast<uint32_t*>(p.qout + r * p.cols + c0) = w;
+                else
+                    p.qout[r * p.cols + c0] = (int8_t)w;
+            }
+            else if constexpr(W == 4)
                 *reinterpret_cast<v4f*>(p.out + r * p.cols + c0) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
             else
                 p.out[r * p.cols + c0] = acc[i][0];
@@ -557,16 +578,20 @@ extern "C" int mi355_binary_f32(int32_t op,
     return mi355_launch_status();
 }
 
-extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
-                               int32_t n_steps,
-                               const float* const* inputs,
-                               const int64_t* row_strides,
-                               const int32_t* col_strides,
-                               int32_t n_inputs,
-                               float* out,
-                               int64_t rows,
-                               int64_t cols,
-                               void* stream)
+namespace {
+int chain_launch(const mi355_chain_step* steps,
+                 int32_t n_steps,
+                 const float* const* inputs,
+                 const int64_t* row_strides,
+                 const int32_t* col_strides,
+                 int32_t n_inputs,
+                 float* out,
+                 int8_t* qout,
+                 const float* qscale,
+                 const int8_t* qzp,
+                 int64_t rows,
+                 int64_t cols,
+                 void* stream)
 {
     if(steps == nullptr || n_steps < 1 || n_steps > MI355_CHAIN_MAX_STEPS || n_inputs < 1 ||
        n_inputs > MI355_CHAIN_MAX_INPUTS || inputs == nullptr || row_strides == nullptr ||
@@ -599,9 +624,11 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
     }
     if(rows == 0 || cols == 0)
         return MI355_OK;
-    if(out == nullptr)
+    const bool quant = qout != nullptr;
+    if(out == nullptr && !quant)
         return MI355_ERR_BAD_ARG;
-    bool vec = cols % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    bool vec = cols % 4 == 0 && (quant ? reinterpret_cast<uintptr_t>(qout) % 4 == 0
+                                       : reinterpret_cast<uintptr_t>(out) % 16 == 0);
     for(int i = 0; i < n_inputs; i++)
     {
         if(inputs[i] == nullptr || row_strides[i] < 0 || (col_strides[i] != 0 && col_strides[i] != 1))
@@ -613,6 +640,9 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
             vec = false;
     }
     p.out     = out;
+    p.qout    = qout;
+    p.qscale  = qscale;
+    p.qzp     = qzp;
     p.rows    = rows;
     p.cols    = cols;
     p.n_steps = n_steps;
@@ -622,7 +652,18 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
     const int64_t row_groups = rows4 ? (rows + 3) / 4 : rows;
     const dim3 grid((unsigned)col_blocks, (unsigned)(row_groups < 65535 ? row_groups : 65535));
     hipStream_t hs = static_cast<hipStream_t>(stream);
-    if(vec && rows4)
+    if(quant)
+    {
+        if(vec && rows4)
+            hipLaunchKernelGGL((chain_kernel<4, 4, true>), grid, dim3(256), 0, hs, p);
+        else if(vec)
+            hipLaunchKernelGGL((chain_kernel<4, 1, true>), grid, dim3(256), 0, hs, p);
+        else if(rows4)
+            hipLaunchKernelGGL((chain_kernel<1, 4, true>), grid, dim3(256), 0, hs, p);
+        else
+            hipLaunchKernelGGL((chain_kernel<1, 1, true>), grid, dim3(256), 0, hs, p);
+    }
+    else if(vec && rows4)
         hipLaunchKernelGGL((chain_kernel<4, 4>), grid, dim3(256), 0, hs, p);
     else if(vec)
         hipLaunchKernelGGL((chain_kernel<4, 1>), grid, dim3(256), 0, hs, p);
@@ -631,6 +672,41 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
     else
         hipLaunchKernelGGL((chain_kernel<1, 1>), grid, dim3(256), 0, hs, p);
     return mi355_launch_status();
+}
+} // namespace
+
+extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
+                               int32_t n_steps,
+                               const float* const* inputs,
+                               const int64_t* row_strides,
+                               const int32_t* col_strides,
+                               int32_t n_inputs,
+                               float* out,
+                               int64_t rows,
+                               int64_t cols,
+                               void* stream)
+{
+    return chain_launch(steps, n_steps, inputs, row_strides, col_strides, n_inputs, out, nullptr, nullptr, nullptr,
+                        rows, cols, stream);
+}
+
+extern "C" int mi355_chain_f32_q8(const mi355_chain_step* steps,
+                                  int32_t n_steps,
+                                  const float* const* inputs,
+                                  const int64_t* row_strides,
+                                  const int32_t* col_strides,
+                                  int32_t n_inputs,
+                                  const float* scale,
+                                  const int8_t* zero_point,
+                                  int8_t* out,
+                                  int64_t rows,
+                                  int64_t cols,
+                                  void* stream)
+{
+    if(scale == nullptr || (out == nullptr && rows > 0 && cols > 0))
+        return MI355_ERR_BAD_ARG;
+    return chain_launch(steps, n_steps, inputs, row_strides, col_strides, n_inputs, nullptr, out, scale, zero_point,
+                        rows, cols, stream);
 }
 
 extern "C" int mi355_binary_i32(int32_t op,

@@ -8,14 +8,6 @@ namespace {
 
 constexpr int PW_THREADS = 256;
 
-MI355_DEVINL double clamp_like_ref(double q, double lo, double hi)
-{
-    // std::max(lo, std::min(hi, q)) with std::min/max's comparison order, so a
-    // NaN ends up at hi exactly as on the ref target.
-    double v = (q < hi) ? q : hi;
-    return (lo < v) ? v : lo;
-}
-
 template <int XT>
 MI355_DEVINL float load_x(const void* x, int64_t i)
 {

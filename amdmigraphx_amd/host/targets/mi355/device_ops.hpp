@@ -509,6 +509,25 @@ struct chain
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// The same chain with a per-tensor quantizelinear to int8 as its last operation (the float value is
+// not stored).  inputs: the chain's inputs, scale (float, every element the same: any broadcast of one
+// value), zero point (int8, likewise) when has_zero_point, out (dense int8)
+struct chain_q8
+{
+    std::vector<int64_t> steps;
+    bool has_zero_point = false;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.steps, "steps");
+        f(self.has_zero_point, "has_zero_point");
+    }
+    std::string name() const { return "mi355::chain_q8"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: x (standard), out; over the last axis
 struct reduce_mean
 {

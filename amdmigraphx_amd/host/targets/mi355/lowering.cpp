@@ -1041,6 +1041,37 @@ void fuse_chains(module& m)
     }
 }
 
+// A chain whose only reader is a quantizelinear to int8 with one scale (and one zero point) for the
+// whole tensor -- the activations in front of a quantized layer, e.g. the GELU of a feed-forward
+// block -- becomes one mi355::chain_q8: the float tensor is neither written nor read back.  Runs
+// behind the lowering of the single operators (it matches mi355:: operators).
+void fuse_chain_quantize(module& m)
+{
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "mi355::quantizelinear" or ins->get_shape().type() != shape::int8_type)
+            continue;
+        auto x = ins->inputs()[0];
+        if(x->name() != "mi355::chain" or x->outputs().size() != 1)
+            continue;
+        const auto& args = ins->inputs(); // x, scale, [zero point], out
+        bool per_tensor  = args[1]->get_shape().type() == shape::float_type;
+        for(std::size_t i = 1; i + 1 < args.size() and per_tensor; i++)
+        {
+            int64_t sr = 0, sc = 0;
+            per_tensor = collapse_2d(args[i]->get_shape(), sr, sc) and sr == 0 and sc == 0;
+        }
+        if(not per_tensor)
+            continue;
+        chain_q8 op;
+        op.steps          = any_cast<chain>(x->get_operator()).steps;
+        op.has_zero_point = args.size() == 4;
+        std::vector<instruction_ref> fused(x->inputs().begin(), x->inputs().end() - 1);
+        fused.insert(fused.end(), args.begin() + 1, args.end());
+        m.replace_instruction(ins, operation{op}, fused);
+    }
+}
+
 // ---- quant_dot(a, b, scale_a, scale_b): block-scaled operands ----------------------------------
 //
 // The four-input form simplify_qdq leaves for the MX formats (src/simplify_qdq.cpp:290-357) goes
@@ -1491,6 +1522,11 @@ void lowering::apply(module& m) const
     for(auto ins : all_instructions(m))
         lower_instruction(m, ins);
     dead_code_elimination{}.apply(m);
+    if(fuse_pointwise)
+    {
+        fuse_chain_quantize(m);
+        dead_code_elimination{}.apply(m);
+    }
     if(prepack_quant_dot_enabled())
     {
         prepack_quant_dot(m);

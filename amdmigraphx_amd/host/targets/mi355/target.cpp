@@ -1426,6 +1426,79 @@ argument chain::compute(migraphx::context& ctx, const shape& out, const std::vec
     return args[n];
 }
 
+shape chain_q8::compute_shape(const std::vector<shape>& inputs) const
+{
+    const std::size_t extra = has_zero_point ? 3 : 2; // scale, [zero point], out
+    if(inputs.size() < extra + 1 or inputs.size() > MI355_CHAIN_MAX_INPUTS + extra)
+        MIGRAPHX_THROW("mi355::chain_q8: between 1 and " + std::to_string(MI355_CHAIN_MAX_INPUTS) +
+                       " inputs, the scale, the zero point if any and the output buffer expected");
+    if(steps.empty() or steps.size() % 4 != 0 or steps.size() / 4 > MI355_CHAIN_MAX_STEPS)
+        MIGRAPHX_THROW("mi355::chain_q8: malformed step list");
+    const shape& out = inputs.back();
+    if(out.type() != shape::int8_type or not out.standard())
+        MIGRAPHX_THROW("mi355::chain_q8: the output buffer must be a dense int8 tensor");
+    const std::size_t n = inputs.size() - extra;
+    for(std::size_t i = 0; i < n; i++)
+    {
+        int64_t sr = 0;
+        int64_t sc = 0;
+        if(inputs[i].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::chain_q8: float tensors only, got " + inputs[i].type_string());
+        if(inputs[i].lens() != out.lens())
+            MIGRAPHX_THROW("mi355::chain_q8: Dimensions do not match");
+        if(not collapse_2d(inputs[i], sr, sc) or (sc != 0 and sc != 1))
+            MIGRAPHX_THROW("mi355::chain_q8: input strides do not collapse to rows and columns");
+    }
+    if(inputs[n].type() != shape::float_type)
+        MIGRAPHX_THROW("mi355::chain_q8: the scale is a float");
+    if(has_zero_point and inputs[n + 1].type() != shape::int8_type)
+        MIGRAPHX_THROW("mi355::chain_q8: the zero point is an int8");
+    return out;
+}
+
+argument chain_q8::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const std::size_t extra = has_zero_point ? 3 : 2;
+    const std::size_t n     = args.size() - extra;
+    std::vector<mi355_chain_step> st(steps.size() / 4);
+    for(std::size_t i = 0; i < st.size(); i++)
+    {
+        st[i].kind     = static_cast<int32_t>(steps[4 * i]);
+        st[i].op       = static_cast<int32_t>(steps[4 * i + 1]);
+        st[i].src      = static_cast<int32_t>(steps[4 * i + 2]);
+        st[i].reversed = static_cast<int32_t>(steps[4 * i + 3]);
+    }
+    std::vector<const float*> ptrs(n);
+    std::vector<int64_t> sr(n);
+    std::vector<int32_t> sc(n);
+    for(std::size_t i = 0; i < n; i++)
+    {
+        int64_t r = 0;
+        int64_t c = 0;
+        collapse_2d(args[i].get_shape(), r, c);
+        ptrs[i] = reinterpret_cast<const float*>(args[i].data());
+        sr[i]   = r;
+        sc[i]   = static_cast<int32_t>(c);
+    }
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(out, rows, cols);
+    status_check(mi355_chain_f32_q8(st.data(),
+                                    static_cast<int32_t>(st.size()),
+                                    ptrs.data(),
+                                    sr.data(),
+                                    sc.data(),
+                                    static_cast<int32_t>(n),
+                                    reinterpret_cast<const float*>(args[n].data()),
+                                    has_zero_point ? reinterpret_cast<const int8_t*>(args[n + 1].data()) : nullptr,
+                                    reinterpret_cast<int8_t*>(args.back().data()),
+                                    rows,
+                                    cols,
+                                    stream_of(ctx)),
+                 name());
+    return args.back();
+}
+
 shape reduce_mean::compute_shape(const std::vector<shape>& inputs) const
 {
     check_inputs(inputs, 2, name());
@@ -1556,6 +1629,7 @@ std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_opti
 } // namespace mi355
 
 MIGRAPHX_REGISTER_OP(mi355::allocate);
+MIGRAPHX_REGISTER_OP(mi355::chain_q8);
 MIGRAPHX_REGISTER_OP(mi355::arena);
 MIGRAPHX_REGISTER_OP(mi355::load);
 MIGRAPHX_REGISTER_OP(mi355::device_literal);

@@ -594,6 +594,15 @@ typedef struct mi355_chain_step
 int mi355_chain_f32(const mi355_chain_step* steps, int32_t n_steps, const float* const* inputs,
                     const int64_t* row_strides, const int32_t* col_strides, int32_t n_inputs,
                     float* out, int64_t rows, int64_t cols, void* stream);
+/* The same chain with quantizelinear (src/include/migraphx/op/quantizelinear.hpp:71-108) as its last
+ * operation: the chain's final value leaves as int8, nearbyint(value / scale[0]) + zero_point[0]
+ * saturated to [-128, 127], one scale and one zero point (NULL: 0) for the whole tensor, both DEVICE
+ * pointers; the float value itself is not stored.  What the target makes of a float pointwise chain
+ * whose only reader is a per-tensor quantizelinear (the activations in front of a quantized layer). */
+int mi355_chain_f32_q8(const mi355_chain_step* steps, int32_t n_steps, const float* const* inputs,
+                       const int64_t* row_strides, const int32_t* col_strides, int32_t n_inputs,
+                       const float* scale, const int8_t* zero_point, int8_t* out, int64_t rows,
+                       int64_t cols, void* stream);
 
 /* Human-readable text for a status code (static storage). */
 const char* mi355_status_string(int status);

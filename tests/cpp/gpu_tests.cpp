@@ -1444,6 +1444,49 @@ TEST_CASE(intermediate_buffers_share_one_arena)
         EXPECT(same_bytes(t.copy_from(again[i]), got[i]));
 }
 
+TEST_CASE(chain_quantized_for_the_next_layer)
+{
+    // A float chain whose only reader is a per-tensor quantizelinear to int8 (the activations in
+    // front of a quantized layer) is one mi355::chain_q8; a chain that something else reads too
+    // keeps its float result and the quantizelinear stays a kernel of its own.  Both equal the CPU
+    // target byte for byte (IEEE-exact operators in the chain).
+    for(bool second_reader : {false, true})
+        for(bool with_zero_point : {false, true})
+        {
+            const std::size_t r = 70, c = 328;
+            program p;
+            auto* mm = p.get_main_module();
+            shape s{shape::float_type, {r, c}};
+            auto x  = mm->add_parameter("x", s);
+            auto y  = mm->add_parameter("y", s);
+            auto v  = mm->add_literal(literal{shape{shape::float_type, {c}}, uniform_floats(c, 0.5f, 2.0f, 77)});
+            auto vb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", s.lens()}}), v);
+            auto t  = mm->add_instruction(make_op("mul"), mm->add_instruction(make_op("add"), x, y), vb);
+            auto sc = mm->add_literal(literal{shape{shape::float_type}, std::vector<float>{0.0625f}});
+            auto sb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", s.lens()}}), sc);
+            std::vector<instruction_ref> qargs{t, sb};
+            if(with_zero_point)
+            {
+                auto z = mm->add_literal(literal{shape{shape::int8_type}, std::vector<float>{-5.0f}});
+                qargs.push_back(mm->add_instruction(make_op("multibroadcast", {{"out_lens", s.lens()}}), z));
+            }
+            // without a zero point the operator's result type is its out_type attribute
+            auto q = mm->add_instruction(make_op("quantizelinear", {{"out_type", shape::int8_type}}), qargs);
+            if(second_reader)
+                mm->add_return({q, mm->add_instruction(make_op("sub"), t, y)});
+            else
+                mm->add_return({q});
+            program compiled = p;
+            compiled.compile(migraphx::make_target("mi355"));
+            const auto& mod = *compiled.get_main_module();
+            EXPECT(count_ops(mod, "mi355::chain_q8") == (second_reader ? 0u : 1u));
+            EXPECT(count_ops(mod, "mi355::quantizelinear") == (second_reader ? 1u : 0u));
+            argument xa{s, normal_floats(r * c, 3.0f, 78)};
+            argument ya{s, normal_floats(r * c, 3.0f, 79)};
+            expect_same(p, {{"x", xa}, {"y", ya}});
+        }
+}
+
 TEST_CASE(pointwise_chains)
 {
     // Chains of float operators become one mi355::chain each.  With IEEE-exact operators the fused
@@ -1628,7 +1671,10 @@ TEST_CASE(encoder_int8_qdq)
     program compiled = p;
     compiled.compile(migraphx::make_target("mi355"));
     EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 6 * c.layers);
-    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quantizelinear") == 4 * c.layers);
+    // four quantized activations per layer; the GELU's, which nothing else reads, is quantized by the
+    // chain that computes it
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quantizelinear") == 3 * c.layers);
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::chain_q8") == c.layers);
     EXPECT(not has_op(compiled, "mi355::dequantizelinear"));
     // and the quantized model stays close to the float one
     encoder::builder fb{c, w, {}, {}};

@@ -134,3 +134,47 @@ def test_bad_arguments_are_rejected():
     assert run_chain(ok, [x], [(8, 2)], 4, 8)[0] != 0                             # column stride 2
     assert run_chain([(LOAD, 0, 0, 0)] + [(UNARY, NEG, 0, 0)] * 24, [x], [(8, 1)], 4, 8)[0] != 0
     assert run_chain(ok, [x], [(8, 1)], 0, 8)[0] == 0                             # empty: nothing to do
+
+
+@pytest.mark.parametrize("rows,cols", [(33, 200), (7, 203), (1, 4), (300, 1024), (5, 1), (9001, 256), (8195, 203)])
+@pytest.mark.parametrize("zero_point", [None, -7])
+def test_quantizing_chain_equals_chain_then_quantizelinear(rows, cols, zero_point):
+    """mi355_chain_f32_q8 against mi355_chain_f32 followed by mi355_quantizelinear (one scale and one
+    zero point for the tensor), byte for byte; values that saturate both ways, ties and a NaN are in."""
+    rng = np.random.default_rng(rows * 7 + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32) * 40
+    x.flat[0] = 1e9
+    x.flat[-1] = -1e9
+    if x.size > 8:
+        x.flat[3] = np.nan
+        x.flat[5] = 0.75     # (0.75 + 0.75) / 0.5 = 3.0; 0.625 -> 2.5: a tie that goes to even
+        x.flat[6] = 0.625
+    y = np.full((rows, cols), 0.0, np.float32)
+    y.flat[5:7] = x.flat[5:7] if x.size > 8 else 0
+    scale = np.float32([0.5])
+    dx, dy, ds = (torch.from_numpy(a).cuda() for a in (x, y, scale))
+    steps = [(LOAD, 0, 0, 0), (BINARY, ADD, 1, 0)]
+    arr = (Step * len(steps))(*[Step(*s) for s in steps])
+    ptrs = (ctypes.c_void_p * 2)(dx.data_ptr(), dy.data_ptr())
+    sr = (ctypes.c_int64 * 2)(cols, cols)
+    sc = (ctypes.c_int32 * 2)(1, 1)
+    dz = torch.tensor([zero_point], dtype=torch.int8, device="cuda") if zero_point is not None else None
+    zp_ptr = ctypes.c_void_p(dz.data_ptr()) if dz is not None else None
+    got = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    print("chain q8", rows, cols, zero_point, flush=True)
+    st = capi.lib().mi355_chain_f32_q8(ctypes.cast(arr, ctypes.c_void_p), 2, ptrs, sr, sc, 2,
+                                       ctypes.c_void_p(ds.data_ptr()), zp_ptr, ctypes.c_void_p(got.data_ptr()),
+                                       rows, cols, stream)
+    assert st == 0
+    st, mid = run_chain(steps, [dx, dy], [(cols, 1), (cols, 1)], rows, cols)
+    assert st == 0
+    want = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+    st = capi.lib().mi355_quantizelinear(ctypes.c_void_p(mid.data_ptr()), capi.DT.F32, ctypes.c_void_p(ds.data_ptr()),
+                                         0, 0, zp_ptr, 0, 0, ctypes.c_void_p(want.data_ptr()), capi.DT.I8, rows, cols,
+                                         stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    w = want.cpu().numpy()
+    assert w.flat[0] == 127 and w.flat[-1] == -128
