@@ -22,7 +22,22 @@ struct dot_params
     int64_t stride_a, stride_b, stride_c;
     int type;
     const float* scale; // fp32 only: the result is multiplied by scale[0] (a `mul` behind the dot); null = none
+    // batch index z = zo * batch_inner + zi: operand z starts at zo * stride_?_outer + zi * stride_?
+    // (two batch axes with strides of their own, e.g. the [batch, head] axes of a transposed view);
+    // one batch axis: batch_inner = the batch count, outer strides 0
+    int64_t batch_inner     = 1;
+    int64_t stride_a_outer  = 0;
+    int64_t stride_b_outer  = 0;
 };
+
+MI355_DEVINL void batch_offsets(const dot_params& p, int64_t& ao, int64_t& bo)
+{
+    const int64_t z  = blockIdx.z;
+    const int64_t zo = z / p.batch_inner;
+    const int64_t zi = z - zo * p.batch_inner;
+    ao               = zo * p.stride_a_outer + zi * p.stride_a;
+    bo               = zo * p.stride_b_outer + zi * p.stride_b;
+}
 
 MI355_DEVINL float load_f32(const void* p, int type, int64_t i)
 {
@@ -58,8 +73,8 @@ __global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
     const int lk   = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.y * 64;
     const int64_t col0 = (int64_t)blockIdx.x * 64;
-    const int64_t ao   = (int64_t)blockIdx.z * p.stride_a;
-    const int64_t bo   = (int64_t)blockIdx.z * p.stride_b;
+    int64_t ao, bo;
+    batch_offsets(p, ao, bo);
     v4d acc[2][2];
 #pragma unroll
     for(int i = 0; i < 2; i++)
@@ -160,8 +175,10 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
     const int lk   = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.y * 64;
     const int64_t col0 = (int64_t)blockIdx.x * 64;
-    const float* a = static_cast<const float*>(p.a) + (int64_t)blockIdx.z * p.stride_a;
-    const float* b = static_cast<const float*>(p.b) + (int64_t)blockIdx.z * p.stride_b;
+    int64_t ao, bo;
+    batch_offsets(p, ao, bo);
+    const float* a = static_cast<const float*>(p.a) + ao;
+    const float* b = static_cast<const float*>(p.b) + bo;
     // this thread's piece of each tile: `major` indexes the strided dimension, `minor` the
     // contiguous one (4 elements)
     const int a_major = A_KCONT ? tid >> 2 : tid >> 4;        // row       | k
@@ -381,9 +398,14 @@ static int dot_launch(bool fp32acc,
                                 int64_t stride_b,
                                 int64_t stride_c,
                                 const float* scale,
-                                void* stream)
+                                void* stream,
+                                int64_t batch_inner    = 0,
+                                int64_t stride_a_outer = 0,
+                                int64_t stride_b_outer = 0)
 {
     if(type != MI355_F32 && type != MI355_F16 && type != MI355_BF16)
+        return MI355_ERR_BAD_ARG;
+    if(batch_inner < 0 || stride_a_outer < 0 || stride_b_outer < 0 || (batch_inner > 0 && batch % batch_inner != 0))
         return MI355_ERR_BAD_ARG;
     if((scale != nullptr || fp32acc) && type != MI355_F32)
         return MI355_ERR_UNSUPPORTED;
@@ -399,6 +421,9 @@ static int dot_launch(bool fp32acc,
         return MI355_ERR_UNSUPPORTED;
     dot_params p{a, b, c, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc,
                  stride_a, stride_b, stride_c, type, scale};
+    p.batch_inner    = batch_inner > 0 ? batch_inner : batch;
+    p.stride_a_outer = stride_a_outer;
+    p.stride_b_outer = stride_b_outer;
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // fp32 with contiguous rows or columns, everything the 16-byte loads touch aligned
@@ -408,6 +433,7 @@ static int dot_launch(bool fp32acc,
     const bool b_n = b_stride_n == 1 && aligned4(b_stride_k);
     const bool b_k = b_stride_k == 1 && aligned4(b_stride_n);
     if(type == MI355_F32 && k > 0 && (a_k || a_m) && (b_n || b_k) && aligned4(stride_a) && aligned4(stride_b) &&
+       aligned4(stride_a_outer) && aligned4(stride_b_outer) &&
        reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0)
     {
         if(fp32acc)
@@ -558,4 +584,36 @@ extern "C" int mi355_contiguous(const void* in,
     default: hipLaunchKernelGGL(gather_kernel<uint64_t>, grid, dim3(256), 0, s, p); break;
     }
     return mi355_launch_status();
+}
+
+extern "C" int mi355_dot_batch2(const void* a,
+                                const void* b,
+                                void* c,
+                                int32_t type,
+                                int64_t m,
+                                int64_t n,
+                                int64_t k,
+                                int64_t a_stride_m,
+                                int64_t a_stride_k,
+                                int64_t b_stride_k,
+                                int64_t b_stride_n,
+                                int64_t batch_outer,
+                                int64_t batch_inner,
+                                int64_t stride_a_outer,
+                                int64_t stride_a_inner,
+                                int64_t stride_b_outer,
+                                int64_t stride_b_inner,
+                                const float* scale,
+                                int32_t fp32acc,
+                                void* stream)
+{
+    if(batch_outer < 0 || batch_inner < 0)
+        return MI355_ERR_BAD_ARG;
+    if(batch_outer == 0 || batch_inner == 0)
+        return MI355_OK;
+    if(batch_outer > 65535 / batch_inner)
+        return MI355_ERR_UNSUPPORTED;
+    return dot_launch(fp32acc != 0, a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, n,
+                      batch_outer * batch_inner, stride_a_inner, stride_b_inner, m * n, scale, stream, batch_inner,
+                      stride_a_outer, stride_b_outer);
 }

@@ -808,9 +808,9 @@ bool fuse_dot_scale(module& m, instruction_ref mul)
             continue;
         auto a = d->inputs()[0];
         auto b = d->inputs()[1];
-        if(not batch_collapses(a->get_shape()))
+        if(not batch_collapses(a->get_shape()) and a->get_shape().ndim() != 4)
             a = make_standard(m, mul, a);
-        if(not batch_collapses(b->get_shape()))
+        if(not batch_collapses(b->get_shape()) and b->get_shape().ndim() != 4)
             b = make_standard(m, mul, b);
         dot op;
         op.scaled  = true;
@@ -1041,6 +1041,27 @@ void fuse_chains(module& m)
     }
 }
 
+// contiguous(x) read only by float dots that take x as it lies (a 4-D view: two batch axes with a
+// stride each): the dots read x, the copy goes (what src/eliminate_contiguous.cpp does when the
+// reader's compute_shape accepts the view).  Runs before the dots are lowered.
+void skip_copies_in_front_of_dots(module& m)
+{
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "contiguous" or ins->outputs().empty())
+            continue;
+        auto x = ins->inputs()[0];
+        if(x->get_shape().ndim() != 4 or x->get_shape().type() != shape::float_type or
+           x->get_shape().broadcasted())
+            continue;
+        auto users = ins->outputs();
+        if(not std::all_of(users.begin(), users.end(), [](instruction_ref u) { return u->name() == "dot"; }))
+            continue;
+        for(auto u : users)
+            instruction::replace_argument(u, ins, x);
+    }
+}
+
 // A chain whose only reader is a quantizelinear to int8 with one scale (and one zero point) for the
 // whole tensor -- the activations in front of a quantized layer, e.g. the GELU of a feed-forward
 // block -- becomes one mi355::chain_q8: the float tensor is neither written nor read back.  Runs
@@ -1264,9 +1285,10 @@ void lower_instruction(module& m, instruction_ref ins)
     {
         auto a = ins->inputs()[0];
         auto b = ins->inputs()[1];
-        if(not batch_collapses(a->get_shape()))
+        // two batch axes keep a stride each (the head split of attention: no copy of q, k and v)
+        if(not batch_collapses(a->get_shape()) and a->get_shape().ndim() != 4)
             a = make_standard(m, ins, a);
-        if(not batch_collapses(b->get_shape()))
+        if(not batch_collapses(b->get_shape()) and b->get_shape().ndim() != 4)
             b = make_standard(m, ins, b);
         dot op;
         op.fp32acc = fp32_dot_requested() and ins->get_shape().type() == shape::float_type;
@@ -1498,6 +1520,9 @@ void lowering::apply(module& m) const
 {
     if(ctx == nullptr)
         MIGRAPHX_THROW("mi355::lowering: no context");
+    // 0. explicit copies that the float dots behind them do not need
+    skip_copies_in_front_of_dots(m);
+    dead_code_elimination{}.apply(m);
     // 1. fused patterns; what they absorb dies
     for(auto ins : all_instructions(m))
     {

@@ -807,10 +807,11 @@ shape dot::compute_shape(const std::vector<shape>& inputs) const
         MIGRAPHX_THROW("mi355::dot: the scale is one float and needs a float dot");
     if(s.type() != shape::float_type and s.type() != shape::half_type and s.type() != shape::bf16_type)
         MIGRAPHX_THROW("mi355::dot: float, half or bf16 only");
-    // any strides are fine inside a matrix; the batch dimensions must collapse into one stride
+    // any strides are fine inside a matrix; the batch dimensions must collapse into one stride, or
+    // be two (each then keeps its own stride: the head split of an attention layer)
     for(int i = 0; i < 2; i++)
     {
-        if(not batch_collapses(inputs[i]))
+        if(not batch_collapses(inputs[i]) and inputs[i].ndim() != 4)
             MIGRAPHX_THROW("mi355::dot: batch dimensions do not collapse into one stride");
     }
     if(inputs.back() != s)
@@ -839,6 +840,31 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
         return r;
     };
     const bool fast = fp32acc and out.type() == shape::float_type;
+    if(nd == 4 and (not batch_collapses(sa) or not batch_collapses(sb)))
+    {
+        status_check(mi355_dot_batch2(args[0].data(),
+                                      args[1].data(),
+                                      args.back().data(),
+                                      to_mi355_type(out.type()),
+                                      m,
+                                      n,
+                                      k,
+                                      static_cast<int64_t>(sa.strides()[2]),
+                                      static_cast<int64_t>(sa.strides()[3]),
+                                      static_cast<int64_t>(sb.strides()[2]),
+                                      static_cast<int64_t>(sb.strides()[3]),
+                                      static_cast<int64_t>(sa.lens()[0]),
+                                      static_cast<int64_t>(sa.lens()[1]),
+                                      static_cast<int64_t>(sa.strides()[0]),
+                                      static_cast<int64_t>(sa.strides()[1]),
+                                      static_cast<int64_t>(sb.strides()[0]),
+                                      static_cast<int64_t>(sb.strides()[1]),
+                                      scaled ? reinterpret_cast<const float*>(args[2].data()) : nullptr,
+                                      fast ? 1 : 0,
+                                      stream_of(ctx)),
+                     name());
+        return args.back();
+    }
     status_check((fast ? mi355_dot_fp32acc : mi355_dot_scaled)(args[0].data(),
                            args[1].data(),
                            args.back().data(),

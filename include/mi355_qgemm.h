@@ -502,6 +502,20 @@ int mi355_dot_fp32acc(const void* a, const void* b, void* c, int32_t type,
                       int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                       const float* scale, void* stream);
 
+/* mi355_dot_scaled (fp32acc == 0) or mi355_dot_fp32acc over TWO batch axes, each operand with a
+ * stride of its own per axis: batch entry (o, i) of A starts at o * stride_a_outer + i *
+ * stride_a_inner.  C is dense, [batch_outer, batch_inner, m, n].  This is how the target multiplies
+ * [batch, heads, rows, k] views whose batch axes do not collapse into one stride -- the head split
+ * of an attention layer, transpose(0, 2, 1, 3) of [batch, rows, heads, k] -- without copying them
+ * (op::dot::compute_shape, src/include/migraphx/op/dot.hpp:43-99, takes any such view). */
+int mi355_dot_batch2(const void* a, const void* b, void* c, int32_t type,
+                     int64_t m, int64_t n, int64_t k,
+                     int64_t a_stride_m, int64_t a_stride_k, int64_t b_stride_k, int64_t b_stride_n,
+                     int64_t batch_outer, int64_t batch_inner,
+                     int64_t stride_a_outer, int64_t stride_a_inner,
+                     int64_t stride_b_outer, int64_t stride_b_inner,
+                     const float* scale, int32_t fp32acc, void* stream);
+
 /*
  * contiguous: gather a strided view (ndim <= MI355_MAX_DIMS, element strides, zero = broadcast)
  * into a dense row-major tensor.  lens / strides are HOST arrays.

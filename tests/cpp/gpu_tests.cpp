@@ -1186,6 +1186,37 @@ TEST_CASE(float_dot_layouts)
     }
 }
 
+TEST_CASE(float_dot_two_batch_axes)
+{
+    // The head split of an attention layer: q, k and v are [batch, rows, heads, width] tensors seen
+    // as [batch, heads, rows, width] (k also with its last two axes swapped).  The two batch axes do
+    // not collapse into one stride; the dot takes a stride for each instead of copies of the views.
+    // Bit-identical to the CPU target; ragged sizes and a width that is not a multiple of 16.
+    struct dims { std::size_t b, h, r, w; };
+    for(auto d : {dims{2, 3, 40, 16}, dims{3, 2, 70, 20}, dims{1, 4, 64, 64}})
+    {
+        program p;
+        auto* mm = p.get_main_module();
+        shape s{shape::float_type, {d.b, d.r, d.h, d.w}};
+        auto q  = mm->add_parameter("q", s);
+        auto k  = mm->add_parameter("k", s);
+        auto v  = mm->add_parameter("v", s);
+        auto qh = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1, 3}}}), q);
+        auto kt = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 3, 1}}}), k);
+        auto vh = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1, 3}}}), v);
+        auto scores = mm->add_instruction(make_op("dot"), qh, kt);   // [b, h, r, r]
+        auto ctx    = mm->add_instruction(make_op("dot"), scores, vh); // [b, h, r, w]
+        mm->add_return({scores, ctx});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::dot") == 2);
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::contiguous") == 0);
+        expect_same(p, {{"q", argument{s, normal_floats(s.elements(), 1.0f, 61)}},
+                        {"k", argument{s, normal_floats(s.elements(), 1.0f, 62)}},
+                        {"v", argument{s, normal_floats(s.elements(), 1.0f, 63)}}});
+    }
+}
+
 TEST_CASE(dot_scale_epilogue)
 {
     // attention scores: dot(q, k^T) * 1/sqrt(d) -- the multiplication joins the dot's store and the
