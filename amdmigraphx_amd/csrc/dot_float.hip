@@ -232,10 +232,7 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
 
     // x * 1.0f is x for every float, so "no scale" needs no second code path
     const float alpha = p.scale != nullptr ? p.scale[0] : 1.0f;
-    v4f va = load_a(0);
-    v4f vb = load_b(0);
-    for(int64_t k0 = 0; k0 < p.k; k0 += 16)
-    {
+    auto stage = [&](const v4f& va, const v4f& vb) {
 #pragma unroll
         for(int e = 0; e < 4; e++)
         {
@@ -248,12 +245,8 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
             else
                 bs[b_minor + e][b_major] = (stage_t)vb[e];
         }
-        __syncthreads();
-        if(k0 + 16 < p.k)
-        {
-            va = load_a(k0 + 16);
-            vb = load_b(k0 + 16);
-        }
+    };
+    auto multiply = [&] {
 #pragma unroll
         for(int kk0 = 0; kk0 < 16; kk0 += 4)
         {
@@ -275,7 +268,71 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
                         acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
                 }
         }
-        __syncthreads();
+    };
+
+    if(row0 + 64 <= p.m && col0 + 64 <= p.n && p.k % 16 == 0 && p.k >= 96)
+    {
+        // A tile inside the matrices and a K long enough to gain by it: every load is one whole
+        // vector, so the loads carry no branches and three K steps of operands can be in flight (the
+        // sixteen matrix instructions of a step last less than a load from memory does).  The three
+        // register sets take turns; a load past the last step reads the last step again and is not
+        // used.
+        const float* a_at = a + (row0 + (A_KCONT ? a_major : a_minor)) * p.a_sm + (A_KCONT ? a_minor : a_major) * p.a_sk;
+        const float* b_at = b + (col0 + (B_NCONT ? b_minor : b_major)) * p.b_sn + (B_NCONT ? b_major : b_minor) * p.b_sk;
+        const int64_t k_last = p.k - 16;
+        auto fetch_a = [&](int64_t k0) {
+            return *reinterpret_cast<const v4f*>(a_at + (k0 < k_last ? k0 : k_last) * p.a_sk);
+        };
+        auto fetch_b = [&](int64_t k0) {
+            return *reinterpret_cast<const v4f*>(b_at + (k0 < k_last ? k0 : k_last) * p.b_sk);
+        };
+        v4f va0 = fetch_a(0), vb0 = fetch_b(0);
+        v4f va1 = fetch_a(16), vb1 = fetch_b(16);
+        v4f va2 = fetch_a(32), vb2 = fetch_b(32);
+        int64_t k0 = 0;
+        auto step = [&](v4f& va, v4f& vb) {
+            stage(va, vb);
+            __syncthreads();
+            va = fetch_a(k0 + 48);
+            vb = fetch_b(k0 + 48);
+            multiply();
+            __syncthreads();
+            k0 += 16;
+        };
+        auto last_step = [&](const v4f& va, const v4f& vb) {
+            stage(va, vb);
+            __syncthreads();
+            multiply();
+            __syncthreads();
+        };
+        int64_t steps = p.k / 16;
+        for(; steps >= 3; steps -= 3)
+        {
+            step(va0, vb0);
+            step(va1, vb1);
+            step(va2, vb2);
+        }
+        if(steps >= 1)
+            last_step(va0, vb0);
+        if(steps == 2)
+            last_step(va1, vb1);
+    }
+    else
+    {
+        v4f va = load_a(0);
+        v4f vb = load_b(0);
+        for(int64_t k0 = 0; k0 < p.k; k0 += 16)
+        {
+            stage(va, vb);
+            __syncthreads();
+            if(k0 + 16 < p.k)
+            {
+                va = load_a(k0 + 16);
+                vb = load_b(k0 + 16);
+            }
+            multiply();
+            __syncthreads();
+        }
     }
 #pragma unroll
     for(int i = 0; i < 2; i++)

@@ -59,6 +59,29 @@ def test_float_dot_whole_tiles_every_layout(ops, trans_a, trans_b):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("k", [80, 96, 112, 128, 400])
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+def test_float_dot_three_steps_in_flight_every_remainder(ops, k, trans_a, trans_b):
+    """Tiles inside the matrices keep three K steps of operands in flight from K = 96 on, in trips of three steps with
+    the one or two steps left over at the end; the tiles on the matrix edges (here the last 36 rows and 20 columns)
+    and shorter sums take the plain loop.  Every number of left-over steps, every layout, bit for bit."""
+    bt, m, n = 2, 128 + 36, 64 + 20
+    rng = np.random.default_rng(500 + k + 2 * trans_a + trans_b)
+    a = rng.standard_normal((bt, k, m) if trans_a else (bt, m, k)).astype(np.float32)
+    b = rng.standard_normal((bt, n, k) if trans_b else (bt, k, n)).astype(np.float32)
+    av = np.swapaxes(a, 1, 2) if trans_a else a
+    bv = np.swapaxes(b, 1, 2) if trans_b else b
+    want = orc.dot(np.ascontiguousarray(av), np.ascontiguousarray(bv), orc.F32)
+    ta = dev(a).transpose(1, 2) if trans_a else dev(a)
+    tb = dev(b).transpose(1, 2) if trans_b else dev(b)
+    print("float dot trips", k, trans_a, trans_b, flush=True)
+    got = ops.dot(ta, tb).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    fast = ops.dot(ta, tb, fp32acc=True).cpu().numpy()
+    mag = np.abs(av).astype(np.float64) @ np.abs(bv).astype(np.float64)
+    assert (np.abs(fast.astype(np.float64) - want) <= mag * k * 2.0**-24 + 1e-30).all()
+
+
 def test_fp32_accumulation_is_float32_only(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((16, 16), dtype=torch.float16, device="cuda")
