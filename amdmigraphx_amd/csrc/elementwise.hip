@@ -379,6 +379,99 @@ MI355_DEVINL double wave_max_f64(double v)
     return v;
 }
 
+// The chain machine with the whole row in the registers of one wave (lane l holds columns l, l + 64,
+// ...: up to 64 * NV of them) and one more step, MI355_CH_ROW_MEAN: the running value becomes the
+// mean of its row -- reduce_mean over the last axis and the broadcast back in one -- summed as
+// reduce_mean_kernel below sums it (a lane's columns in ascending order in a double, then the fixed
+// pairing across the wave, one rounding to float), so a layer normalisation written as reduce_mean /
+// sub / mul / reduce_mean / add / rsqrt / mul ... gives the bits of its separate operators while x
+// is read once and only the result is written.  Columns past the end hold values nobody reads.
+template <int NV>
+__global__ __launch_bounds__(256) void chain_rows_kernel(chain_params p)
+{
+#pragma clang fp contract(off)
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= p.rows)
+        return;
+    float acc[NV], saved[NV], operand[NV];
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+        acc[i] = saved[i] = 0.0f;
+    auto fetch = [&](int in, float(&dst)[NV]) __attribute__((always_inline)) {
+        const float* base = p.in[in] + row * p.sr[in];
+        if(p.sc[in] == 0)
+        {
+            const float s = base[0];
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                dst[i] = s;
+        }
+        else
+        {
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+            {
+                const int64_t c = lane + 64 * i;
+                dst[i]          = c < p.cols ? base[c] : 0.0f;
+            }
+        }
+    };
+    for(int s = 0; s < p.n_steps; s++)
+    {
+        const mi355_chain_step st = p.steps[s];
+        switch(st.kind)
+        {
+        case MI355_CH_LOAD: fetch(st.src, acc); break;
+        case MI355_CH_BINARY: {
+            if(st.src >= 0)
+                fetch(st.src, operand);
+            else
+            {
+#pragma unroll
+                for(int i = 0; i < NV; i++)
+                    operand[i] = st.src == MI355_CH_SAVED ? saved[i] : acc[i];
+            }
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                acc[i] = st.reversed ? binary_apply(st.op, operand[i], acc[i]) : binary_apply(st.op, acc[i], operand[i]);
+            break;
+        }
+        case MI355_CH_UNARY:
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                acc[i] = unary_apply(st.op, acc[i]);
+            break;
+        case MI355_CH_ROW_MEAN: {
+            double sum = 0.0;
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                if(lane + 64 * i < p.cols)
+                    sum += (double)acc[i];
+            sum              = wave_sum_f64(sum);
+            const float mean = (float)(sum / (double)p.cols);
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                acc[i] = mean;
+            break;
+        }
+        default:
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                saved[i] = acc[i];
+            break;
+        }
+    }
+    float* y = p.out + row * p.cols;
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        const int64_t c = lane + 64 * i;
+        if(c < p.cols)
+            y[c] = acc[i];
+    }
+}
+
 // one wave per row; double accumulation (the order differs from the reference's sequential sum,
 // which moves the float result by at most its last bit)
 __global__ __launch_bounds__(256) void reduce_mean_kernel(const float* in, float* out, int64_t rows, int64_t cols)
@@ -591,7 +684,8 @@ int chain_launch(const mi355_chain_step* steps,
                  const int8_t* qzp,
                  int64_t rows,
                  int64_t cols,
-                 void* stream)
+                 void* stream,
+                 bool whole_rows = false)
 {
     if(steps == nullptr || n_steps < 1 || n_steps > MI355_CHAIN_MAX_STEPS || n_inputs < 1 ||
        n_inputs > MI355_CHAIN_MAX_INPUTS || inputs == nullptr || row_strides == nullptr ||
@@ -618,6 +712,10 @@ int chain_launch(const mi355_chain_step* steps,
                 return MI355_ERR_BAD_ARG;
             break;
         case MI355_CH_SAVE: break;
+        case MI355_CH_ROW_MEAN:
+            if(!whole_rows)
+                return MI355_ERR_BAD_ARG;
+            break;
         default: return MI355_ERR_BAD_ARG;
         }
         p.steps[s] = st;
@@ -646,12 +744,31 @@ int chain_launch(const mi355_chain_step* steps,
     p.rows    = rows;
     p.cols    = cols;
     p.n_steps = n_steps;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    if(whole_rows)
+    {
+        // one wave per row, four rows per workgroup
+        const int64_t blocks = (rows + 3) / 4;
+        if(quant || cols > MI355_CHAIN_ROWS_MAX_COLS || blocks > 0x7fffffff)
+            return MI355_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)blocks);
+        if(cols <= 256)
+            hipLaunchKernelGGL(chain_rows_kernel<4>, grid, dim3(256), 0, hs, p);
+        else if(cols <= 768)
+            hipLaunchKernelGGL(chain_rows_kernel<12>, grid, dim3(256), 0, hs, p);
+        else if(cols <= 1024)
+            hipLaunchKernelGGL(chain_rows_kernel<16>, grid, dim3(256), 0, hs, p);
+        else if(cols <= 2048)
+            hipLaunchKernelGGL(chain_rows_kernel<32>, grid, dim3(256), 0, hs, p);
+        else
+            hipLaunchKernelGGL(chain_rows_kernel<64>, grid, dim3(256), 0, hs, p);
+        return mi355_launch_status();
+    }
     // four rows per pass when there are enough rows to keep every CU busy that way
     const int64_t col_blocks = ((vec ? cols / 4 : cols) + 255) / 256;
     const bool rows4         = rows * col_blocks >= 4 * 2048;
     const int64_t row_groups = rows4 ? (rows + 3) / 4 : rows;
     const dim3 grid((unsigned)col_blocks, (unsigned)(row_groups < 65535 ? row_groups : 65535));
-    hipStream_t hs = static_cast<hipStream_t>(stream);
     if(quant)
     {
         if(vec && rows4)
@@ -688,6 +805,21 @@ extern "C" int mi355_chain_f32(const mi355_chain_step* steps,
 {
     return chain_launch(steps, n_steps, inputs, row_strides, col_strides, n_inputs, out, nullptr, nullptr, nullptr,
                         rows, cols, stream);
+}
+
+extern "C" int mi355_chain_rows_f32(const mi355_chain_step* steps,
+                                    int32_t n_steps,
+                                    const float* const* inputs,
+                                    const int64_t* row_strides,
+                                    const int32_t* col_strides,
+                                    int32_t n_inputs,
+                                    float* out,
+                                    int64_t rows,
+                                    int64_t cols,
+                                    void* stream)
+{
+    return chain_launch(steps, n_steps, inputs, row_strides, col_strides, n_inputs, out, nullptr, nullptr, nullptr,
+                        rows, cols, stream, true);
 }
 
 extern "C" int mi355_chain_f32_q8(const mi355_chain_step* steps,

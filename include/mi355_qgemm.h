@@ -593,11 +593,19 @@ int mi355_gather_rows(const void* table, const void* ids, int32_t ids_are_int64,
  * Input i is addressed as inputs[i][row * row_strides[i] + col * col_strides[i]] with a column
  * stride of 0 (constant along the row) or 1.  The first step must be a LOAD.  All arrays are HOST
  * arrays; at most MI355_CHAIN_MAX_STEPS steps and MI355_CHAIN_MAX_INPUTS inputs. */
-typedef enum mi355_chain_kind { MI355_CH_LOAD = 0, MI355_CH_BINARY = 1, MI355_CH_UNARY = 2, MI355_CH_SAVE = 3 } mi355_chain_kind;
+typedef enum mi355_chain_kind
+{
+    MI355_CH_LOAD     = 0,
+    MI355_CH_BINARY   = 1,
+    MI355_CH_UNARY    = 2,
+    MI355_CH_SAVE     = 3,
+    MI355_CH_ROW_MEAN = 4 /* mi355_chain_rows_f32 only */
+} mi355_chain_kind;
 #define MI355_CH_SAVED (-1)
 #define MI355_CH_SELF (-2)
 #define MI355_CHAIN_MAX_STEPS 24
 #define MI355_CHAIN_MAX_INPUTS 8
+#define MI355_CHAIN_ROWS_MAX_COLS 4096
 typedef struct mi355_chain_step
 {
     int32_t kind;     /* mi355_chain_kind */
@@ -608,6 +616,17 @@ typedef struct mi355_chain_step
 int mi355_chain_f32(const mi355_chain_step* steps, int32_t n_steps, const float* const* inputs,
                     const int64_t* row_strides, const int32_t* col_strides, int32_t n_inputs,
                     float* out, int64_t rows, int64_t cols, void* stream);
+/* The chain with one more kind of step, for operators that reduce over the last axis between the
+ * pointwise ones (layer normalisation: reduce_mean, sub, mul, reduce_mean, add, rsqrt, mul, mul, add):
+ *   MI355_CH_ROW_MEAN  value = the mean of the running value over its row, in every column
+ * which is reduce_mean over the last axis (src/include/migraphx/op/reduce_mean.hpp:34-50) followed by
+ * the broadcast back to the row, with mi355_reduce_mean_f32's summation (double, one rounding to
+ * float), so the result equals the separate operators bit for bit.  A wave holds a whole row in
+ * registers: cols <= MI355_CHAIN_ROWS_MAX_COLS, else MI355_ERR_UNSUPPORTED.  The reference reaches the
+ * same fusion through src/fuse_reduce.cpp:251-340, 448-470 and compiles the fused module. */
+int mi355_chain_rows_f32(const mi355_chain_step* steps, int32_t n_steps, const float* const* inputs,
+                         const int64_t* row_strides, const int32_t* col_strides, int32_t n_inputs,
+                         float* out, int64_t rows, int64_t cols, void* stream);
 /* The same chain with quantizelinear (src/include/migraphx/op/quantizelinear.hpp:71-108) as its last
  * operation: the chain's final value leaves as int8, nearbyint(value / scale[0]) + zero_point[0]
  * saturated to [-128, 127], one scale and one zero point (NULL: 0) for the whole tensor, both DEVICE
