@@ -528,6 +528,24 @@ struct chain_q8
     std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
 };
 
+// The chain with MI355_CH_ROW_MEAN steps (the mean over the last axis, in every column of the row):
+// a layer normalisation in one kernel, a whole row in the registers of one wave.  inputs: tensors of
+// the result's dimensions or with one value per row (last dimension 1), then out (dense float, rows
+// of at most MI355_CHAIN_ROWS_MAX_COLS elements)
+struct chain_rows
+{
+    std::vector<int64_t> steps;
+    template <class Self, class F>
+    static void reflect(Self& self, F f)
+    {
+        f(self.steps, "steps");
+    }
+    std::string name() const { return "mi355::chain_rows"; }
+    shape compute_shape(const std::vector<shape>& inputs) const;
+    argument compute(migraphx::context& ctx, const shape&, const std::vector<argument>& args) const;
+    std::ptrdiff_t output_alias(const std::vector<shape>& s) const { return s.size() - 1; }
+};
+
 // inputs: x (standard), out; over the last axis
 struct reduce_mean
 {

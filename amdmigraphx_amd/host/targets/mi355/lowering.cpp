@@ -1041,6 +1041,203 @@ void fuse_chains(module& m)
     }
 }
 
+// ---- layer normalisation -> one kernel ---------------------------------------------------------
+//
+// mean = reduce_mean(x); d = x - mean; var = reduce_mean(d * d); y = d * rsqrt(var + eps) (or
+// d / sqrt(var + eps)), over the last axis -- the expansion of ONNX LayerNormalization -- with an
+// add / sub / mul / div that produces x for nobody else in front and the pointwise operators that
+// follow y one after the other (the scale and the shift) behind: one mi355::chain_rows whose steps
+// repeat these operators in their order, the two means as row-mean steps.  x is read once and only
+// the last value is written; the reference fuses the same group through src/fuse_reduce.cpp:251-340.
+// Runs in front of fuse_chains, which would otherwise take the pointwise parts.
+
+std::vector<instruction_ref> distinct_users(instruction_ref i)
+{
+    std::vector<instruction_ref> users;
+    for(auto u : i->outputs())
+    {
+        if(std::none_of(users.begin(), users.end(), [&](instruction_ref v) { return &*v == &*u; }))
+            users.push_back(u);
+    }
+    return users;
+}
+
+bool only_user_is(instruction_ref i, instruction_ref u)
+{
+    auto users = distinct_users(i);
+    return users.size() == 1 and &*users[0] == &*u;
+}
+
+bool reduce_mean_last(instruction_ref i)
+{
+    if(i->name() != "reduce_mean")
+        return false;
+    const auto& axes = any_cast<op::reduce_mean>(i->get_operator()).axes;
+    const auto nd    = static_cast<int64_t>(i->inputs()[0]->get_shape().ndim());
+    return axes.size() == 1 and (axes[0] == -1 or axes[0] == nd - 1);
+}
+
+bool fuse_layer_norm(module& m, instruction_ref var)
+{
+    if(not reduce_mean_last(var))
+        return false;
+    auto sq = var->inputs()[0];
+    if(sq->name() != "mul" or &*sq->inputs()[0] != &*sq->inputs()[1] or not only_user_is(sq, var))
+        return false;
+    auto d = sq->inputs()[0];
+    if(d->name() != "sub")
+        return false;
+    auto x  = d->inputs()[0];
+    auto mb = d->inputs()[1];
+    if(mb->name() != "multibroadcast" or not only_user_is(mb, d))
+        return false;
+    auto mean = mb->inputs()[0];
+    if(not reduce_mean_last(mean) or &*mean->inputs()[0] != &*x or not only_user_is(mean, mb))
+        return false;
+    const shape& xs = x->get_shape();
+    if(xs.type() != shape::float_type or xs.ndim() == 0 or xs.lens().back() > MI355_CHAIN_ROWS_MAX_COLS or
+       xs.lens().back() < 2 or d->get_shape().lens() != xs.lens() or mb->get_shape().lens() != xs.lens())
+        return false;
+    // var -> + eps -> rsqrt | sqrt -> broadcast over the row -> y
+    auto var_users = distinct_users(var);
+    if(var_users.size() != 1 or var_users[0]->name() != "add")
+        return false;
+    auto ve  = var_users[0];
+    auto eps = &*ve->inputs()[0] == &*var ? ve->inputs()[1] : ve->inputs()[0];
+    if(&*eps == &*var or eps->get_shape().lens() != var->get_shape().lens() or
+       eps->get_shape().type() != shape::float_type)
+        return false;
+    auto ve_users = distinct_users(ve);
+    if(ve_users.size() != 1 or (ve_users[0]->name() != "rsqrt" and ve_users[0]->name() != "sqrt"))
+        return false;
+    auto root        = ve_users[0];
+    const bool recip = root->name() == "rsqrt";
+    auto root_users  = distinct_users(root);
+    if(root_users.size() != 1 or root_users[0]->name() != "multibroadcast" or
+       root_users[0]->get_shape().lens() != xs.lens())
+        return false;
+    auto rb       = root_users[0];
+    auto rb_users = distinct_users(rb);
+    if(rb_users.size() != 1)
+        return false;
+    auto y = rb_users[0];
+    if(recip ? (y->name() != "mul" or not((&*y->inputs()[0] == &*d and &*y->inputs()[1] == &*rb) or
+                                          (&*y->inputs()[0] == &*rb and &*y->inputs()[1] == &*d)))
+             : (y->name() != "div" or &*y->inputs()[0] != &*d or &*y->inputs()[1] != &*rb))
+        return false;
+    // d feeds the square and y, nothing else
+    auto d_users = distinct_users(d);
+    if(d_users.size() != 2 or not std::all_of(d_users.begin(), d_users.end(), [&](instruction_ref u) {
+           return &*u == &*sq or &*u == &*y;
+       }))
+        return false;
+
+    std::vector<instruction_ref> externals;
+    std::vector<int64_t> steps;
+    bool failed   = false;
+    auto per_row  = var->get_shape().lens();
+    auto external = [&](instruction_ref e) {
+        for(std::size_t i = 0; i < externals.size(); i++)
+        {
+            if(&*externals[i] == &*e)
+                return static_cast<int>(i);
+        }
+        int64_t sr = 0;
+        int64_t sc = 0;
+        const shape& es = e->get_shape();
+        if(externals.size() >= MI355_CHAIN_MAX_INPUTS or es.type() != shape::float_type or
+           (es.lens() != xs.lens() and es.lens() != per_row) or not collapse_2d(es, sr, sc) or (sc != 0 and sc != 1))
+        {
+            failed = true;
+            return 0;
+        }
+        externals.push_back(e);
+        return static_cast<int>(externals.size() - 1);
+    };
+    auto push = [&](int kind, int op, int src, int reversed) {
+        if(steps.size() / 4 >= MI355_CHAIN_MAX_STEPS)
+            failed = true;
+        else
+            steps.insert(steps.end(), {kind, op, src, reversed});
+    };
+    // x itself, or the one operator that makes it when nobody else reads its result
+    const int x_bin    = binary_code(x->name());
+    auto x_users       = distinct_users(x);
+    const bool x_taken = x_bin >= 0 and x_users.size() == 2 and &*x->inputs()[0] != &*x->inputs()[1] and
+                         std::all_of(x_users.begin(), x_users.end(), [&](instruction_ref u) {
+                             return &*u == &*mean or &*u == &*d;
+                         }) and
+                         x->inputs()[0]->get_shape().lens() == xs.lens() and
+                         x->inputs()[1]->get_shape().lens() == xs.lens();
+    if(x_taken)
+    {
+        push(MI355_CH_LOAD, 0, external(x->inputs()[0]), 0);
+        push(MI355_CH_BINARY, x_bin, external(x->inputs()[1]), 0);
+    }
+    else
+        push(MI355_CH_LOAD, 0, external(x), 0);
+    push(MI355_CH_SAVE, 0, 0, 0);
+    push(MI355_CH_ROW_MEAN, 0, 0, 0);
+    push(MI355_CH_BINARY, MI355_BIN_SUB, MI355_CH_SAVED, 1); // x - mean
+    push(MI355_CH_SAVE, 0, 0, 0);
+    push(MI355_CH_BINARY, MI355_BIN_MUL, MI355_CH_SELF, 0);
+    push(MI355_CH_ROW_MEAN, 0, 0, 0);
+    push(MI355_CH_BINARY, MI355_BIN_ADD, external(eps), &*ve->inputs()[0] == &*var ? 0 : 1);
+    push(MI355_CH_UNARY, recip ? MI355_UN_RSQRT : MI355_UN_SQRT, 0, 0);
+    // y = d (op) root: the saved value is the first operand, unless the graph has the product the other way round
+    push(MI355_CH_BINARY, recip ? MI355_BIN_MUL : MI355_BIN_DIV, MI355_CH_SAVED, &*y->inputs()[0] == &*d ? 1 : 0);
+    if(failed)
+        return false;
+    // what follows y one operator at a time
+    auto last = y;
+    while(true)
+    {
+        auto users = distinct_users(last);
+        if(users.size() != 1)
+            break;
+        auto u = users[0];
+        if(u->get_shape().type() != shape::float_type or u->get_shape().lens() != xs.lens())
+            break;
+        const auto saved_steps     = steps;
+        const auto saved_externals = externals;
+        const int un               = unary_code(u->name());
+        const int bin              = binary_code(u->name());
+        if(un >= 0)
+            push(MI355_CH_UNARY, un, 0, 0);
+        else if(bin >= 0 and &*u->inputs()[0] == &*u->inputs()[1])
+            push(MI355_CH_BINARY, bin, MI355_CH_SELF, 0);
+        else if(bin >= 0)
+        {
+            const bool first = &*u->inputs()[0] == &*last;
+            push(MI355_CH_BINARY, bin, external(first ? u->inputs()[1] : u->inputs()[0]), first ? 0 : 1);
+        }
+        else
+            break;
+        if(failed)
+        {
+            steps     = saved_steps;
+            externals = saved_externals;
+            break;
+        }
+        last = u;
+    }
+    auto args = externals;
+    args.push_back(insert_allocation(m, last, shape{shape::float_type, xs.lens()}));
+    chain_rows op;
+    op.steps = steps;
+    m.replace_instruction(last, operation{op}, args);
+    return true;
+}
+
+void fuse_layer_norms(module& m)
+{
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() == "reduce_mean" and not ins->outputs().empty())
+            fuse_layer_norm(m, ins);
+    }
+}
+
 // contiguous(x) read only by float dots that take x as it lies (a 4-D view: two batch axes with a
 // stride each): the dots read x, the copy goes (what src/eliminate_contiguous.cpp does when the
 // reader's compute_shape accepts the view).  Runs before the dots are lowered.
@@ -1540,6 +1737,8 @@ void lowering::apply(module& m) const
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)
     {
+        fuse_layer_norms(m);
+        dead_code_elimination{}.apply(m);
         fuse_chains(m);
         dead_code_elimination{}.apply(m);
     }

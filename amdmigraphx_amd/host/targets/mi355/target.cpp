@@ -1388,6 +1388,38 @@ argument unary::compute(migraphx::context& ctx, const shape& out, const std::vec
     return args[1];
 }
 
+namespace {
+// the host arrays the chain entry points take: steps, and a pointer, a row stride and a column
+// stride for each of the first n arguments
+struct chain_call
+{
+    std::vector<mi355_chain_step> st;
+    std::vector<const float*> ptrs;
+    std::vector<int64_t> sr;
+    std::vector<int32_t> sc;
+    chain_call(const std::vector<int64_t>& steps, const std::vector<argument>& args, std::size_t n)
+        : st(steps.size() / 4), ptrs(n), sr(n), sc(n)
+    {
+        for(std::size_t i = 0; i < st.size(); i++)
+        {
+            st[i].kind     = static_cast<int32_t>(steps[4 * i]);
+            st[i].op       = static_cast<int32_t>(steps[4 * i + 1]);
+            st[i].src      = static_cast<int32_t>(steps[4 * i + 2]);
+            st[i].reversed = static_cast<int32_t>(steps[4 * i + 3]);
+        }
+        for(std::size_t i = 0; i < n; i++)
+        {
+            int64_t r = 0;
+            int64_t c = 0;
+            collapse_2d(args[i].get_shape(), r, c);
+            ptrs[i] = reinterpret_cast<const float*>(args[i].data());
+            sr[i]   = r;
+            sc[i]   = static_cast<int32_t>(c);
+        }
+    }
+};
+} // namespace
+
 shape chain::compute_shape(const std::vector<shape>& inputs) const
 {
     if(inputs.size() < 2 or inputs.size() > MI355_CHAIN_MAX_INPUTS + 1)
@@ -1415,39 +1447,70 @@ shape chain::compute_shape(const std::vector<shape>& inputs) const
 argument chain::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
 {
     const std::size_t n = args.size() - 1;
-    std::vector<mi355_chain_step> st(steps.size() / 4);
-    for(std::size_t i = 0; i < st.size(); i++)
-    {
-        st[i].kind     = static_cast<int32_t>(steps[4 * i]);
-        st[i].op       = static_cast<int32_t>(steps[4 * i + 1]);
-        st[i].src      = static_cast<int32_t>(steps[4 * i + 2]);
-        st[i].reversed = static_cast<int32_t>(steps[4 * i + 3]);
-    }
-    std::vector<const float*> ptrs(n);
-    std::vector<int64_t> sr(n);
-    std::vector<int32_t> sc(n);
-    for(std::size_t i = 0; i < n; i++)
-    {
-        int64_t r = 0;
-        int64_t c = 0;
-        collapse_2d(args[i].get_shape(), r, c);
-        ptrs[i] = reinterpret_cast<const float*>(args[i].data());
-        sr[i]   = r;
-        sc[i]   = static_cast<int32_t>(c);
-    }
+    chain_call c(steps, args, n);
     int64_t rows = 0;
     int64_t cols = 0;
     rows_cols(out, rows, cols);
-    status_check(mi355_chain_f32(st.data(),
-                                 static_cast<int32_t>(st.size()),
-                                 ptrs.data(),
-                                 sr.data(),
-                                 sc.data(),
+    status_check(mi355_chain_f32(c.st.data(),
+                                 static_cast<int32_t>(c.st.size()),
+                                 c.ptrs.data(),
+                                 c.sr.data(),
+                                 c.sc.data(),
                                  static_cast<int32_t>(n),
                                  reinterpret_cast<float*>(args[n].data()),
                                  rows,
                                  cols,
                                  stream_of(ctx)),
+                 name());
+    return args[n];
+}
+
+shape chain_rows::compute_shape(const std::vector<shape>& inputs) const
+{
+    if(inputs.size() < 2 or inputs.size() > MI355_CHAIN_MAX_INPUTS + 1)
+        MIGRAPHX_THROW("mi355::chain_rows: between 1 and " + std::to_string(MI355_CHAIN_MAX_INPUTS) +
+                       " inputs and the output buffer expected");
+    if(steps.empty() or steps.size() % 4 != 0 or steps.size() / 4 > MI355_CHAIN_MAX_STEPS)
+        MIGRAPHX_THROW("mi355::chain_rows: malformed step list");
+    const shape& out = inputs.back();
+    if(out.type() != shape::float_type or not out.standard() or out.ndim() == 0)
+        MIGRAPHX_THROW("mi355::chain_rows: the output buffer must be a dense float tensor");
+    if(out.lens().back() > MI355_CHAIN_ROWS_MAX_COLS)
+        MIGRAPHX_THROW("mi355::chain_rows: rows of at most " + std::to_string(MI355_CHAIN_ROWS_MAX_COLS) + " elements");
+    // an input has the result's dimensions, or one value per row (last dimension 1)
+    auto per_row = out.lens();
+    per_row.back() = 1;
+    for(std::size_t i = 0; i + 1 < inputs.size(); i++)
+    {
+        int64_t sr = 0;
+        int64_t sc = 0;
+        if(inputs[i].type() != shape::float_type)
+            MIGRAPHX_THROW("mi355::chain_rows: float tensors only, got " + inputs[i].type_string());
+        if(inputs[i].lens() != out.lens() and inputs[i].lens() != per_row)
+            MIGRAPHX_THROW("mi355::chain_rows: Dimensions do not match");
+        if(not collapse_2d(inputs[i], sr, sc) or (sc != 0 and sc != 1))
+            MIGRAPHX_THROW("mi355::chain_rows: input strides do not collapse to rows and columns");
+    }
+    return out;
+}
+
+argument chain_rows::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
+{
+    const std::size_t n = args.size() - 1;
+    chain_call c(steps, args, n);
+    int64_t rows = 0;
+    int64_t cols = 0;
+    rows_cols(out, rows, cols);
+    status_check(mi355_chain_rows_f32(c.st.data(),
+                                      static_cast<int32_t>(c.st.size()),
+                                      c.ptrs.data(),
+                                      c.sr.data(),
+                                      c.sc.data(),
+                                      static_cast<int32_t>(n),
+                                      reinterpret_cast<float*>(args[n].data()),
+                                      rows,
+                                      cols,
+                                      stream_of(ctx)),
                  name());
     return args[n];
 }
@@ -1486,34 +1549,15 @@ argument chain_q8::compute(migraphx::context& ctx, const shape& out, const std::
 {
     const std::size_t extra = has_zero_point ? 3 : 2;
     const std::size_t n     = args.size() - extra;
-    std::vector<mi355_chain_step> st(steps.size() / 4);
-    for(std::size_t i = 0; i < st.size(); i++)
-    {
-        st[i].kind     = static_cast<int32_t>(steps[4 * i]);
-        st[i].op       = static_cast<int32_t>(steps[4 * i + 1]);
-        st[i].src      = static_cast<int32_t>(steps[4 * i + 2]);
-        st[i].reversed = static_cast<int32_t>(steps[4 * i + 3]);
-    }
-    std::vector<const float*> ptrs(n);
-    std::vector<int64_t> sr(n);
-    std::vector<int32_t> sc(n);
-    for(std::size_t i = 0; i < n; i++)
-    {
-        int64_t r = 0;
-        int64_t c = 0;
-        collapse_2d(args[i].get_shape(), r, c);
-        ptrs[i] = reinterpret_cast<const float*>(args[i].data());
-        sr[i]   = r;
-        sc[i]   = static_cast<int32_t>(c);
-    }
+    chain_call c(steps, args, n);
     int64_t rows = 0;
     int64_t cols = 0;
     rows_cols(out, rows, cols);
-    status_check(mi355_chain_f32_q8(st.data(),
-                                    static_cast<int32_t>(st.size()),
-                                    ptrs.data(),
-                                    sr.data(),
-                                    sc.data(),
+    status_check(mi355_chain_f32_q8(c.st.data(),
+                                    static_cast<int32_t>(c.st.size()),
+                                    c.ptrs.data(),
+                                    c.sr.data(),
+                                    c.sc.data(),
                                     static_cast<int32_t>(n),
                                     reinterpret_cast<const float*>(args[n].data()),
                                     has_zero_point ? reinterpret_cast<const int8_t*>(args[n + 1].data()) : nullptr,
@@ -1656,6 +1700,7 @@ std::vector<pass> target::get_passes(migraphx::context& gctx, const compile_opti
 
 MIGRAPHX_REGISTER_OP(mi355::allocate);
 MIGRAPHX_REGISTER_OP(mi355::chain_q8);
+MIGRAPHX_REGISTER_OP(mi355::chain_rows);
 MIGRAPHX_REGISTER_OP(mi355::arena);
 MIGRAPHX_REGISTER_OP(mi355::load);
 MIGRAPHX_REGISTER_OP(mi355::device_literal);

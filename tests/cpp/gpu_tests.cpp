@@ -1527,7 +1527,7 @@ TEST_CASE(pointwise_chains)
     using builder = std::function<instruction_ref(module&, instruction_ref, instruction_ref, instruction_ref)>;
     struct counts
     {
-        std::size_t chains, singles;
+        std::size_t chains, singles, row_chains = 0;
     };
     auto run = [&](std::size_t r, std::size_t c, const builder& f, bool exact, counts expected) {
         static int case_no = 0;
@@ -1552,6 +1552,7 @@ TEST_CASE(pointwise_chains)
                       << std::endl;
         EXPECT(chains == expected.chains);
         EXPECT(singles == expected.singles);
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::chain_rows") == expected.row_chains);
         auto got = run_on("mi355", p, params);
         setenv("MIGRAPHX_DISABLE_POINTWISE_FUSION", "1", 1);
         program plain = p;
@@ -1559,6 +1560,7 @@ TEST_CASE(pointwise_chains)
         auto unfused = run_on("mi355", p, params);
         unsetenv("MIGRAPHX_DISABLE_POINTWISE_FUSION");
         EXPECT(not has_op(plain, "mi355::chain"));
+        EXPECT(not has_op(plain, "mi355::chain_rows"));
         EXPECT(same_bytes(got[0], unfused[0]));
         auto want = run_on("oracle", p, params);
         if(exact)
@@ -1639,8 +1641,8 @@ TEST_CASE(pointwise_chains)
         auto e = op(m, "add", op(m, "erf", op(m, "mul", h, constant(0.70710678f))), constant(1.0f));
         return op(m, "mul", op(m, "mul", h, constant(0.5f)), e);
     }, false, {1, 0}); // x + bias has two users: both compute it again, the sum is never stored
-    // layer normalisation: x - mean feeds the variance and the normalised value and is recomputed
-    // in both chains; the two operators on the [rows, 1] statistics stay single
+    // layer normalisation with its scale and shift: one kernel that holds the row (the means are
+    // steps of its chain), equal to the separate operators bit for bit
     run(33, 200, [&](module& m, instruction_ref x, instruction_ref, instruction_ref v) {
         auto mean  = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), x);
         auto xm    = op(m, "sub", x, bcast(m, mean, x));
@@ -1648,7 +1650,37 @@ TEST_CASE(pointwise_chains)
         auto eps   = m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{1e-5f}});
         auto sigma = op(m, "sqrt", op(m, "add", var, bcast(m, eps, var)));
         return op(m, "add", op(m, "mul", op(m, "div", xm, bcast(m, sigma, x)), bcast(m, v, x)), bcast(m, v, x));
-    }, false, {2, 2});
+    }, false, {0, 0, 1});
+    // the form with rsqrt, behind a residual sum that nobody else reads, a tanh behind the shift
+    run(130, 768, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref v) {
+        auto sum  = op(m, "add", x, y);
+        auto mean = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), sum);
+        auto d    = op(m, "sub", sum, bcast(m, mean, sum));
+        auto var  = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), op(m, "mul", d, d));
+        auto eps  = m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{1e-5f}});
+        auto rs   = op(m, "rsqrt", op(m, "add", bcast(m, eps, var), var));
+        auto n    = op(m, "mul", bcast(m, rs, sum), d);
+        return op(m, "tanh", op(m, "add", op(m, "mul", n, bcast(m, v, sum)), y));
+    }, false, {0, 0, 1});
+    // a residual sum that is read again later is stored by its own operator and read by the kernel;
+    // x - mean with a third reader keeps the separate operators
+    run(9, 1000, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
+        auto sum  = op(m, "add", x, y);
+        auto mean = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), sum);
+        auto d    = op(m, "sub", sum, bcast(m, mean, sum));
+        auto var  = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), op(m, "mul", d, d));
+        auto eps  = m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{1e-5f}});
+        auto rs   = op(m, "rsqrt", op(m, "add", var, bcast(m, eps, var)));
+        return op(m, "add", op(m, "mul", d, bcast(m, rs, sum)), sum);
+    }, false, {0, 1, 1});
+    run(9, 64, [&](module& m, instruction_ref x, instruction_ref, instruction_ref) {
+        auto mean = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), x);
+        auto d    = op(m, "sub", x, bcast(m, mean, x));
+        auto var  = m.add_instruction(make_op("reduce_mean", {{"axes", {-1}}}), op(m, "mul", d, d));
+        auto eps  = m.add_literal(literal{shape{shape::float_type, {1}}, std::vector<float>{1e-5f}});
+        auto rs   = op(m, "rsqrt", op(m, "add", var, bcast(m, eps, var)));
+        return op(m, "add", op(m, "mul", d, bcast(m, rs, x)), op(m, "neg", d));
+    }, false, {2, 2, 0});
     // a value with a user that is no pointwise operator is stored once and read by the others
     run(16, 64, [&](module& m, instruction_ref x, instruction_ref y, instruction_ref) {
         auto d  = op(m, "sub", x, y);
@@ -1706,6 +1738,10 @@ TEST_CASE(encoder_int8_qdq)
     // chain that computes it
     EXPECT(count_ops(*compiled.get_main_module(), "mi355::quantizelinear") == 3 * c.layers);
     EXPECT(count_ops(*compiled.get_main_module(), "mi355::chain_q8") == c.layers);
+    // each layer normalisation (one behind the embeddings, two per layer) is one kernel, the residual
+    // sum in front of it included
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::chain_rows") == 2 * c.layers + 1);
+    EXPECT(not has_op(compiled, "mi355::reduce_mean"));
     EXPECT(not has_op(compiled, "mi355::dequantizelinear"));
     // and the quantized model stays close to the float one
     encoder::builder fb{c, w, {}, {}};
