@@ -472,6 +472,106 @@ __global__ __launch_bounds__(256) void chain_rows_kernel(chain_params p)
     }
 }
 
+// The step list of a layer normalisation as the lowering writes it -- [x | a (op) b], save, row mean,
+// saved - mean, save, square, row mean, + eps, rsqrt | sqrt, saved * | / root, then up to two more
+// operators with an input each (the scale and the shift) -- has this kernel of its own: the same
+// operations in the same order as the step machine above performs them (the same bits), written out,
+// so that every input row is requested before the first one is waited for, and the operators on
+// the row's statistics run once per row instead of once per column.
+struct layer_norm_plan
+{
+    int x, pre_src, pre_op; // pre_op < 0: the row is input x itself
+    int eps;
+    int recip; // rsqrt and a product, else sqrt and a quotient
+    int n_tail;
+    int tail_op[2], tail_src[2];
+};
+
+template <int NV>
+__global__ __launch_bounds__(256) void layer_norm_rows_kernel(chain_params p, layer_norm_plan q)
+{
+#pragma clang fp contract(off)
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= p.rows)
+        return;
+    auto fetch = [&](int in, float(&dst)[NV]) __attribute__((always_inline)) {
+        const float* base = p.in[in] + row * p.sr[in];
+        if(p.sc[in] == 0)
+        {
+            const float s = base[0];
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+                dst[i] = s;
+        }
+        else
+        {
+#pragma unroll
+            for(int i = 0; i < NV; i++)
+            {
+                const int64_t c = lane + 64 * i;
+                dst[i]          = c < p.cols ? base[c] : 0.0f;
+            }
+        }
+    };
+    auto row_mean = [&](const float(&v)[NV]) __attribute__((always_inline)) {
+        double sum = 0.0;
+#pragma unroll
+        for(int i = 0; i < NV; i++)
+            if(lane + 64 * i < p.cols)
+                sum += (double)v[i];
+        sum = wave_sum_f64(sum);
+        return (float)(sum / (double)p.cols);
+    };
+    float acc[NV], other[NV], tail0[NV], tail1[NV];
+    fetch(q.x, acc);
+    if(q.pre_op >= 0)
+        fetch(q.pre_src, other);
+    if(q.n_tail > 0)
+        fetch(q.tail_src[0], tail0);
+    if(q.n_tail > 1)
+        fetch(q.tail_src[1], tail1);
+    const float eps = p.in[q.eps][row * p.sr[q.eps]];
+    if(q.pre_op >= 0)
+    {
+#pragma unroll
+        for(int i = 0; i < NV; i++)
+            acc[i] = binary_apply(q.pre_op, acc[i], other[i]);
+    }
+    const float mean = row_mean(acc);
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        acc[i]   = acc[i] - mean;
+        other[i] = acc[i] * acc[i];
+    }
+    const float var  = row_mean(other);
+    const float root = unary_apply(q.recip ? MI355_UN_RSQRT : MI355_UN_SQRT, var + eps);
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+        acc[i] = q.recip ? acc[i] * root : acc[i] / root;
+    if(q.n_tail > 0)
+    {
+#pragma unroll
+        for(int i = 0; i < NV; i++)
+            acc[i] = binary_apply(q.tail_op[0], acc[i], tail0[i]);
+    }
+    if(q.n_tail > 1)
+    {
+#pragma unroll
+        for(int i = 0; i < NV; i++)
+            acc[i] = binary_apply(q.tail_op[1], acc[i], tail1[i]);
+    }
+    float* y = p.out + row * p.cols;
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+    {
+        const int64_t c = lane + 64 * i;
+        if(c < p.cols)
+            y[c] = acc[i];
+    }
+}
+
 // one wave per row; double accumulation (the order differs from the reference's sequential sum,
 // which moves the float result by at most its last bit)
 __global__ __launch_bounds__(256) void reduce_mean_kernel(const float* in, float* out, int64_t rows, int64_t cols)
@@ -672,6 +772,54 @@ extern "C" int mi355_binary_f32(int32_t op,
 }
 
 namespace {
+// Is the (validated) step list the layer normalisation layer_norm_rows_kernel evaluates?
+bool layer_norm_steps(const chain_params& p, layer_norm_plan& q)
+{
+    const mi355_chain_step* st = p.steps;
+    auto kind_at = [&](int at, int kind) { return at < p.n_steps && st[at].kind == kind; };
+    auto binary  = [&](int at, int op, int src, int reversed) {
+        return kind_at(at, MI355_CH_BINARY) && st[at].op == op && st[at].src == src && st[at].reversed == reversed;
+    };
+    auto unary = [&](int at, int op) { return kind_at(at, MI355_CH_UNARY) && st[at].op == op; };
+    // an operator with an input as its second operand
+    auto binary_with_input = [&](int at) {
+        return kind_at(at, MI355_CH_BINARY) && st[at].src >= 0 && st[at].reversed == 0;
+    };
+    q.x      = st[0].src; // the first step is a LOAD
+    q.pre_op = -1;
+    int s    = 1;
+    if(binary_with_input(1))
+    {
+        q.pre_op  = st[1].op;
+        q.pre_src = st[1].src;
+        s         = 2;
+    }
+    if(!(kind_at(s, MI355_CH_SAVE) && kind_at(s + 1, MI355_CH_ROW_MEAN) &&
+         binary(s + 2, MI355_BIN_SUB, MI355_CH_SAVED, 1) && kind_at(s + 3, MI355_CH_SAVE) &&
+         binary(s + 4, MI355_BIN_MUL, MI355_CH_SELF, 0) && kind_at(s + 5, MI355_CH_ROW_MEAN) &&
+         binary_with_input(s + 6) && st[s + 6].op == MI355_BIN_ADD && p.sc[st[s + 6].src] == 0))
+        return false;
+    q.eps = st[s + 6].src;
+    if(unary(s + 7, MI355_UN_RSQRT) && binary(s + 8, MI355_BIN_MUL, MI355_CH_SAVED, 1))
+        q.recip = 1;
+    else if(unary(s + 7, MI355_UN_SQRT) && binary(s + 8, MI355_BIN_DIV, MI355_CH_SAVED, 1))
+        q.recip = 0;
+    else
+        return false;
+    s += 9;
+    q.n_tail = p.n_steps - s;
+    if(q.n_tail < 0 || q.n_tail > 2)
+        return false;
+    for(int t = 0; t < q.n_tail; t++)
+    {
+        if(!binary_with_input(s + t))
+            return false;
+        q.tail_op[t]  = st[s + t].op;
+        q.tail_src[t] = st[s + t].src;
+    }
+    return true;
+}
+
 int chain_launch(const mi355_chain_step* steps,
                  int32_t n_steps,
                  const float* const* inputs,
@@ -752,6 +900,17 @@ int chain_launch(const mi355_chain_step* steps,
         if(quant || cols > MI355_CHAIN_ROWS_MAX_COLS || blocks > 0x7fffffff)
             return MI355_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)blocks);
+        layer_norm_plan plan{};
+        if(cols <= 1024 && layer_norm_steps(p, plan))
+        {
+            if(cols <= 256)
+                hipLaunchKernelGGL(layer_norm_rows_kernel<4>, grid, dim3(256), 0, hs, p, plan);
+            else if(cols <= 768)
+                hipLaunchKernelGGL(layer_norm_rows_kernel<12>, grid, dim3(256), 0, hs, p, plan);
+            else
+                hipLaunchKernelGGL(layer_norm_rows_kernel<16>, grid, dim3(256), 0, hs, p, plan);
+            return mi355_launch_status();
+        }
         if(cols <= 256)
             hipLaunchKernelGGL(chain_rows_kernel<4>, grid, dim3(256), 0, hs, p);
         else if(cols <= 768)
