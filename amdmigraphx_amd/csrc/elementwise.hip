@@ -197,6 +197,69 @@ MI355_DEVINL float unary_apply(int op, float x)
     }
 }
 
+// One operator over the N values a thread holds, the operator chosen once for all of them (the
+// code is the same for every lane, so the choice costs scalar branches and each case is N
+// straight-line operations).  value = value (op) operand, or operand (op) value when reversed.
+template <int N>
+MI355_DEVINL void binary_block(int op, bool reversed, float* value, const float* operand)
+{
+#pragma clang fp contract(off)
+#define MI355_BLOCK_OF(EXPR)                                   \
+    _Pragma("unroll") for(int i = 0; i < N; i++)               \
+    {                                                          \
+        const float x = reversed ? operand[i] : value[i];      \
+        const float y = reversed ? value[i] : operand[i];      \
+        value[i]      = EXPR;                                  \
+    }
+    if(reversed)
+    {
+        switch(op)
+        {
+        case MI355_BIN_ADD: MI355_BLOCK_OF(x + y) break;
+        case MI355_BIN_SUB: MI355_BLOCK_OF(x - y) break;
+        case MI355_BIN_MUL: MI355_BLOCK_OF(x * y) break;
+        case MI355_BIN_MAX: MI355_BLOCK_OF(x < y ? y : x) break;
+        case MI355_BIN_MIN: MI355_BLOCK_OF(y < x ? y : x) break;
+        default: MI355_BLOCK_OF(x / y) break;
+        }
+    }
+    else
+    {
+        switch(op)
+        {
+        case MI355_BIN_ADD: MI355_BLOCK_OF(x + y) break;
+        case MI355_BIN_SUB: MI355_BLOCK_OF(x - y) break;
+        case MI355_BIN_MUL: MI355_BLOCK_OF(x * y) break;
+        case MI355_BIN_MAX: MI355_BLOCK_OF(x < y ? y : x) break;
+        case MI355_BIN_MIN: MI355_BLOCK_OF(y < x ? y : x) break;
+        default: MI355_BLOCK_OF(x / y) break;
+        }
+    }
+#undef MI355_BLOCK_OF
+}
+
+template <int N>
+MI355_DEVINL void unary_block(int op, float* value)
+{
+#define MI355_BLOCK_OF(EXPR)                                   \
+    _Pragma("unroll") for(int i = 0; i < N; i++)               \
+    {                                                          \
+        const float x = value[i];                              \
+        value[i]      = EXPR;                                  \
+    }
+    switch(op)
+    {
+    case MI355_UN_ERF: MI355_BLOCK_OF(erff(x)) break;
+    case MI355_UN_SQRT: MI355_BLOCK_OF(sqrtf(x)) break;
+    case MI355_UN_RSQRT: MI355_BLOCK_OF(1.0f / sqrtf(x)) break;
+    case MI355_UN_EXP: MI355_BLOCK_OF(expf(x)) break;
+    case MI355_UN_TANH: MI355_BLOCK_OF(tanhf(x)) break;
+    case MI355_UN_NEARBYINT: MI355_BLOCK_OF(rintf(x)) break;
+    default: MI355_BLOCK_OF(-x) break;
+    }
+#undef MI355_BLOCK_OF
+}
+
 __global__ __launch_bounds__(256) void unary_kernel(const float* in, float* out, int64_t n, int op)
 {
     const int64_t step = (int64_t)gridDim.x * 256;
@@ -299,30 +362,17 @@ __global__ __launch_bounds__(256) void chain_kernel(chain_params p)
             case MI355_CH_LOAD: fetch(st.src, acc); break;
             case MI355_CH_BINARY: {
                 if(st.src >= 0)
-                    fetch(st.src, operand);
-                else
                 {
-#pragma unroll
-                    for(int i = 0; i < R; i++)
-#pragma unroll
-                        for(int e = 0; e < W; e++)
-                            operand[i][e] = st.src == MI355_CH_SAVED ? saved[i][e] : acc[i][e];
+                    fetch(st.src, operand);
+                    binary_block<R * W>(st.op, st.reversed != 0, &acc[0][0], &operand[0][0]);
                 }
-#pragma unroll
-                for(int i = 0; i < R; i++)
-#pragma unroll
-                    for(int e = 0; e < W; e++)
-                        acc[i][e] = st.reversed ? binary_apply(st.op, operand[i][e], acc[i][e])
-                                                : binary_apply(st.op, acc[i][e], operand[i][e]);
+                else if(st.src == MI355_CH_SAVED)
+                    binary_block<R * W>(st.op, st.reversed != 0, &acc[0][0], &saved[0][0]);
+                else
+                    binary_block<R * W>(st.op, st.reversed != 0, &acc[0][0], &acc[0][0]);
                 break;
             }
-            case MI355_CH_UNARY:
-#pragma unroll
-                for(int i = 0; i < R; i++)
-#pragma unroll
-                    for(int e = 0; e < W; e++)
-                        acc[i][e] = unary_apply(st.op, acc[i][e]);
-                break;
+            case MI355_CH_UNARY: unary_block<R * W>(st.op, &acc[0][0]); break;
             default:
 #pragma unroll
                 for(int i = 0; i < R; i++)
@@ -425,23 +475,17 @@ __global__ __launch_bounds__(256) void chain_rows_kernel(chain_params p)
         case MI355_CH_LOAD: fetch(st.src, acc); break;
         case MI355_CH_BINARY: {
             if(st.src >= 0)
-                fetch(st.src, operand);
-            else
             {
-#pragma unroll
-                for(int i = 0; i < NV; i++)
-                    operand[i] = st.src == MI355_CH_SAVED ? saved[i] : acc[i];
+                fetch(st.src, operand);
+                binary_block<NV>(st.op, st.reversed != 0, acc, operand);
             }
-#pragma unroll
-            for(int i = 0; i < NV; i++)
-                acc[i] = st.reversed ? binary_apply(st.op, operand[i], acc[i]) : binary_apply(st.op, acc[i], operand[i]);
+            else if(st.src == MI355_CH_SAVED)
+                binary_block<NV>(st.op, st.reversed != 0, acc, saved);
+            else
+                binary_block<NV>(st.op, st.reversed != 0, acc, acc);
             break;
         }
-        case MI355_CH_UNARY:
-#pragma unroll
-            for(int i = 0; i < NV; i++)
-                acc[i] = unary_apply(st.op, acc[i]);
-            break;
+        case MI355_CH_UNARY: unary_block<NV>(st.op, acc); break;
         case MI355_CH_ROW_MEAN: {
             double sum = 0.0;
 #pragma unroll
@@ -533,11 +577,7 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(chain_params p, la
         fetch(q.tail_src[1], tail1);
     const float eps = p.in[q.eps][row * p.sr[q.eps]];
     if(q.pre_op >= 0)
-    {
-#pragma unroll
-        for(int i = 0; i < NV; i++)
-            acc[i] = binary_apply(q.pre_op, acc[i], other[i]);
-    }
+        binary_block<NV>(q.pre_op, false, acc, other);
     const float mean = row_mean(acc);
 #pragma unroll
     for(int i = 0; i < NV; i++)
@@ -551,17 +591,9 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(chain_params p, la
     for(int i = 0; i < NV; i++)
         acc[i] = q.recip ? acc[i] * root : acc[i] / root;
     if(q.n_tail > 0)
-    {
-#pragma unroll
-        for(int i = 0; i < NV; i++)
-            acc[i] = binary_apply(q.tail_op[0], acc[i], tail0[i]);
-    }
+        binary_block<NV>(q.tail_op[0], false, acc, tail0);
     if(q.n_tail > 1)
-    {
-#pragma unroll
-        for(int i = 0; i < NV; i++)
-            acc[i] = binary_apply(q.tail_op[1], acc[i], tail1[i]);
-    }
+        binary_block<NV>(q.tail_op[1], false, acc, tail1);
     float* y = p.out + row * p.cols;
 #pragma unroll
     for(int i = 0; i < NV; i++)
