@@ -449,22 +449,15 @@ __global__ __launch_bounds__(256) void chain_rows_kernel(chain_params p)
     for(int i = 0; i < NV; i++)
         acc[i] = saved[i] = 0.0f;
     auto fetch = [&](int in, float(&dst)[NV]) __attribute__((always_inline)) {
+        // one form for both column strides and no branch, so that the loads of several inputs are in
+        // flight together; a column past the end reads the last one
         const float* base = p.in[in] + row * p.sr[in];
-        if(p.sc[in] == 0)
-        {
-            const float s = base[0];
+        const int sc      = p.sc[in];
 #pragma unroll
-            for(int i = 0; i < NV; i++)
-                dst[i] = s;
-        }
-        else
+        for(int i = 0; i < NV; i++)
         {
-#pragma unroll
-            for(int i = 0; i < NV; i++)
-            {
-                const int64_t c = lane + 64 * i;
-                dst[i]          = c < p.cols ? base[c] : 0.0f;
-            }
+            const int64_t c = lane + 64 * i;
+            dst[i]          = base[(c < p.cols ? c : p.cols - 1) * sc];
         }
     };
     for(int s = 0; s < p.n_steps; s++)
@@ -540,22 +533,15 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(chain_params p, la
     if(row >= p.rows)
         return;
     auto fetch = [&](int in, float(&dst)[NV]) __attribute__((always_inline)) {
+        // one form for both column strides and no branch, so that the loads of several inputs are in
+        // flight together; a column past the end reads the last one
         const float* base = p.in[in] + row * p.sr[in];
-        if(p.sc[in] == 0)
-        {
-            const float s = base[0];
+        const int sc      = p.sc[in];
 #pragma unroll
-            for(int i = 0; i < NV; i++)
-                dst[i] = s;
-        }
-        else
+        for(int i = 0; i < NV; i++)
         {
-#pragma unroll
-            for(int i = 0; i < NV; i++)
-            {
-                const int64_t c = lane + 64 * i;
-                dst[i]          = c < p.cols ? base[c] : 0.0f;
-            }
+            const int64_t c = lane + 64 * i;
+            dst[i]          = base[(c < p.cols ? c : p.cols - 1) * sc];
         }
     };
     auto row_mean = [&](const float(&v)[NV]) __attribute__((always_inline)) {
@@ -621,6 +607,59 @@ __global__ __launch_bounds__(256) void reduce_mean_kernel(const float* in, float
         out[row] = (float)(s / (double)cols);
 }
 
+// Is the double q within `units` units in its last place of the midpoint between two neighbouring
+// floats (q in the range of the normal floats)?  A value that is not rounds to the same float as
+// every double that close to it.
+MI355_DEVINL bool near_float_midpoint(double q, int units)
+{
+    const int low = (int)((uint32_t)__double_as_longlong(q) & 0x1fffffffu); // the 29 bits a float drops
+    const int d   = low - 0x10000000;
+    return (d < 0 ? -d : d) <= units;
+}
+
+// float(exp(d)), d <= 0 (softmax: a value minus its row's maximum), the float that the exact
+// exponential rounds to.  Eleven Taylor terms behind the usual reduction to |r| <= ln(2) / 2 are
+// within 2^-46 of it (r^12 / 12! < 2^-47, the rounding of the steps a few times 2^-53), i.e. within 90
+// units in the last place of a double; unless that reaches a midpoint between two floats, the
+// float is settled.  The few values where it might (one in a million), and the arguments whose
+// results are float denormals, take the library's exp as before.
+MI355_DEVINL float exp_to_float(double d)
+{
+    const double n = rint(d * 1.4426950408889634074);
+    double r       = fma(-n, 6.93147180369123816490e-01, d);
+    r              = fma(-n, 1.90821492927058770002e-10, r);
+    double p       = 2.50521083854417187751e-08; // 1 / 11!
+    p              = fma(p, r, 2.75573192239858906526e-07);
+    p              = fma(p, r, 2.75573192239858906526e-06);
+    p              = fma(p, r, 2.48015873015873015873e-05);
+    p              = fma(p, r, 1.98412698412698412698e-04);
+    p              = fma(p, r, 1.38888888888888888889e-03);
+    p              = fma(p, r, 8.33333333333333333333e-03);
+    p              = fma(p, r, 4.16666666666666666667e-02);
+    p              = fma(p, r, 1.66666666666666666667e-01);
+    p              = fma(p, r, 0.5);
+    p              = fma(p, r, 1.0);
+    p              = fma(p, r, 1.0);
+    const double q = ldexp(p, (int)n);
+    float e        = (float)q;
+    // one branch for everything the short way does not settle (its value above is then not used):
+    // arguments below the normal floats' exponentials, -inf, NaN, and the midpoints
+    if(!(d >= -87.0) || near_float_midpoint(q, 256))
+        e = d < -104.0 ? 0.0f : (float)exp(d); // exp(-104) < 2^-150 rounds to 0
+    return e;
+}
+
+// float(double(e) / s) given rs = 1 / s: e * rs is within 3 units in the last place of the quotient's
+// double, so unless it comes that close to a midpoint between two floats (or the result is a float
+// denormal) it rounds to the same float, and the division is left to those rare values.
+MI355_DEVINL float quotient_to_float(float e, double s, double rs)
+{
+    const double q = (double)e * rs;
+    if(q != 0.0 && (!(q >= 2.4e-38) || near_float_midpoint(q, 8)))
+        return (float)((double)e / s);
+    return (float)q;
+}
+
 // ref_softmax (src/targets/ref/lowering.cpp:281-312): e = float(exp(double(x) - max)),
 // sum of e in double, out = float(double(e) / sum)
 __global__ __launch_bounds__(256) void softmax_kernel(const float* in, float* out, int64_t rows, int64_t cols)
@@ -638,20 +677,23 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* in, float* ou
     double s = 0.0;
     for(int64_t c = lane; c < cols; c += 64)
     {
-        const float e = (float)exp((double)x[c] - m);
+        const float e = exp_to_float((double)x[c] - m);
         y[c]          = e;
         s += (double)e;
     }
-    s = wave_sum_f64(s);
+    s               = wave_sum_f64(s);
+    const double rs = 1.0 / s;
     for(int64_t c = lane; c < cols; c += 64)
-        y[c] = (float)((double)y[c] / s);
+        y[c] = quotient_to_float(y[c], s, rs);
 }
 
 // The same arithmetic with the row held in registers (up to 64*NV columns): one read and one write
 // of the tensor instead of three and two.  A lane's elements are summed in the same order as above,
-// so the results are the same bits.
-template <int NV>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* in, float* out, int64_t rows, int64_t cols)
+// so the results are the same bits.  FULL: the row has exactly 64*NV columns.  Otherwise the
+// columns past the end enter as -inf, which leaves the maximum alone and adds an exact zero to the
+// sum, so that no step needs a branch of its own.
+template <int NV, bool FULL>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* in, float* out, int64_t rows, int cols)
 {
     const int lane    = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -660,35 +702,39 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* in, floa
     const float* x = in + row * cols;
     float* y       = out + row * cols;
     float v[NV];
-    double m = -1.7976931348623157e308;
+    // every load before the first use, none behind a branch
 #pragma unroll
     for(int i = 0; i < NV; i++)
     {
-        const int64_t c = lane + 64 * i;
-        if(c < cols)
-        {
-            v[i] = x[c];
-            m    = fmax(m, (double)v[i]);
-        }
+        const int c = lane + 64 * i;
+        v[i]        = x[FULL ? c : min(c, cols - 1)];
     }
+    if constexpr(!FULL)
+    {
+#pragma unroll
+        for(int i = 0; i < NV; i++)
+            v[i] = lane + 64 * i < cols ? v[i] : -__builtin_huge_valf();
+    }
+    double m = -1.7976931348623157e308;
+#pragma unroll
+    for(int i = 0; i < NV; i++)
+        m = fmax(m, (double)v[i]);
     m        = wave_max_f64(m);
     double s = 0.0;
 #pragma unroll
     for(int i = 0; i < NV; i++)
     {
-        if(lane + 64 * i < cols)
-        {
-            v[i] = (float)exp((double)v[i] - m);
-            s += (double)v[i];
-        }
+        v[i] = exp_to_float((double)v[i] - m);
+        s += (double)v[i];
     }
-    s = wave_sum_f64(s);
+    s               = wave_sum_f64(s);
+    const double rs = 1.0 / s;
 #pragma unroll
     for(int i = 0; i < NV; i++)
     {
-        const int64_t c = lane + 64 * i;
-        if(c < cols)
-            y[c] = (float)((double)v[i] / s);
+        const int c = lane + 64 * i;
+        if(FULL || c < cols)
+            y[c] = quotient_to_float(v[i], s, rs);
     }
 }
 
@@ -1193,14 +1239,32 @@ extern "C" int mi355_softmax_f32(const float* in, float* out, int64_t rows, int6
         return MI355_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)((rows + 3) / 4));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // rows of up to 1024 columns stay in registers: 2, 6, 8 or 16 values per lane
+    const int nc = (int)(cols <= 1024 ? cols : 0);
+#define MI355_SOFTMAX_ROWS(NV)                                                                              \
+    if(nc == 64 * NV)                                                                                       \
+        hipLaunchKernelGGL((softmax_rows_kernel<NV, true>), grid, dim3(256), 0, s, in, out, rows, nc);      \
+    else                                                                                                    \
+        hipLaunchKernelGGL((softmax_rows_kernel<NV, false>), grid, dim3(256), 0, s, in, out, rows, nc)
     if(cols <= 64 * 2)
-        hipLaunchKernelGGL(softmax_rows_kernel<2>, grid, dim3(256), 0, s, in, out, rows, cols);
+    {
+        MI355_SOFTMAX_ROWS(2);
+    }
+    else if(cols <= 64 * 6)
+    {
+        MI355_SOFTMAX_ROWS(6);
+    }
     else if(cols <= 64 * 8)
-        hipLaunchKernelGGL(softmax_rows_kernel<8>, grid, dim3(256), 0, s, in, out, rows, cols);
+    {
+        MI355_SOFTMAX_ROWS(8);
+    }
     else if(cols <= 64 * 16)
-        hipLaunchKernelGGL(softmax_rows_kernel<16>, grid, dim3(256), 0, s, in, out, rows, cols);
+    {
+        MI355_SOFTMAX_ROWS(16);
+    }
     else
         hipLaunchKernelGGL(softmax_kernel, grid, dim3(256), 0, s, in, out, rows, cols);
+#undef MI355_SOFTMAX_ROWS
     return mi355_launch_status();
 }
 
