@@ -19,7 +19,7 @@ class DT:
 
 
 class QP:
-    NONE, PER_TENSOR, PER_ROW, PER_COL = range(4)
+    NONE, PER_TENSOR, PER_ROW, PER_COL, PER_COL_BATCH = range(5)
 
 
 class W4ZP:

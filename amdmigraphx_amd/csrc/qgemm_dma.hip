@@ -76,6 +76,8 @@ struct dma_params
     int stream_c;   // C is far larger than the caches: streaming stores
     int vec_cols;   // the per-column arrays in use (scale_b, colsum_b, bias) are 16-byte aligned and
                     // N % 4 == 0: four columns' values come with one load
+    int64_t stride_cols = 0; // MI355_QP_PER_COL_BATCH: scale_b and bias hold one [N] vector per batch entry,
+                             // this many elements apart (the dense int8 kernels only)
     // block-scaled operands (qgemm_dma_kernel<.., MX>): exponent bytes of the scales as
     // [batch][slab][rows rounded up to 256][4] (a slab of 64 operand bytes is 128 fp4 elements = 4
     // blocks of 32, or 64 fp8 elements = 2 blocks in bytes 0 and 1), and a word that, when it holds
@@ -910,6 +912,17 @@ __global__ __launch_bounds__(NTHREADS) void qgemm_dma_i8_kernel(dma_params p)
     static_assert(!VIA_LDS || (VEC_STORE && (!DEQ || OUT == MI355_F32)), "32-bit results in groups of 4");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
+    // one vector of column scales (and of the bias) per batch entry
+    if constexpr(DEQ)
+    {
+        if(p.stride_cols != 0)
+        {
+            const int64_t off = (int64_t)blockIdx.y * p.stride_cols;
+            p.scale_b += off;
+            if(p.bias != nullptr)
+                p.bias += off;
+        }
+    }
     const int tid    = threadIdx.x;
     const int lane   = tid & 63;
     const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1447,6 +1460,17 @@ __global__ __launch_bounds__(W4_THREADS) void qgemm_w4_i8_kernel(dma_params p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
+    // one vector of column scales (and of the bias) per batch entry
+    if constexpr(DEQ)
+    {
+        if(p.stride_cols != 0)
+        {
+            const int64_t off = (int64_t)blockIdx.y * p.stride_cols;
+            p.scale_b += off;
+            if(p.bias != nullptr)
+                p.bias += off;
+        }
+    }
     const int tid    = threadIdx.x;
     const int lane   = tid & 63;
     const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -4516,6 +4540,15 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     p.zp_b         = d->zp_b;
     const bool fp8 = d->in_type == MI355_FP8;
     const bool deq = d->dequant != 0;
+    // column scales and a bias per batch entry: the dense int8 kernels with the epilogue
+    const bool cols_per_batch = d->scale_b_mode == MI355_QP_PER_COL_BATCH;
+    if(cols_per_batch)
+    {
+        if(fp8 || !deq || d->n % 4 != 0)
+            return MI355_ERR_UNSUPPORTED;
+        p.scale_b_mode = MI355_QP_PER_COL;
+        p.stride_cols  = d->n;
+    }
     {
         const size_t esz = deq ? mi355_dtype_size(d->out_type) : 4;
         p.vec_store = d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
@@ -4525,7 +4558,7 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
         // half of the 256 MB last-level cache and more: the result streams past it
         p.stream_c = (double)d->batch * (double)d->m * (double)d->n * (double)esz >= 128.0 * 1048576.0;
         auto aligned16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-        p.vec_cols = d->n % 4 == 0 && (d->scale_b_mode != MI355_QP_PER_COL || aligned16(scale_b)) &&
+        p.vec_cols = d->n % 4 == 0 && (p.scale_b_mode != MI355_QP_PER_COL || aligned16(scale_b)) &&
                      (d->zp_a == 0 || aligned16(colsum_b)) && (bias == nullptr || aligned16(bias));
     }
     p.ksplit = 1;
@@ -4566,7 +4599,7 @@ int mi355_dma_gemm_launch(const mi355_quant_dot_desc* d,
     const size_t osz = deq ? mi355_dtype_size(d->out_type) : 4;
     const bool vec   = d->n % 4 == 0 && d->ldc % 4 == 0 && d->stride_c % 4 == 0 &&
                      reinterpret_cast<uintptr_t>(c) % (4 * osz) == 0;
-    if(workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+    if(workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && !cols_per_batch &&
        (!deq || d->out_type == MI355_F32 || d->out_type == MI355_F16 || d->out_type == MI355_BF16))
     {
         const int s = choose_ksplit_ws(p.tiles_m * p.tiles_n, (int)d->batch, p.k / BK, d->m, d->n, d->k);

@@ -277,7 +277,7 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
            d->scale_a_mode != MI355_QP_PER_ROW)
             return MI355_ERR_BAD_ARG;
         if(d->scale_b_mode != MI355_QP_NONE && d->scale_b_mode != MI355_QP_PER_TENSOR &&
-           d->scale_b_mode != MI355_QP_PER_COL)
+           d->scale_b_mode != MI355_QP_PER_COL && d->scale_b_mode != MI355_QP_PER_COL_BATCH)
             return MI355_ERR_BAD_ARG;
         if(d->scale_a_mode != MI355_QP_NONE && scale_a == nullptr)
             return MI355_ERR_BAD_ARG;
@@ -313,6 +313,9 @@ extern "C" int mi355_quant_dot_ws(const mi355_quant_dot_desc* d,
     const bool dma_has_bias = bias == nullptr || fp8 || d->n % 4 == 0;
     if(!u8 && !bf8 && d->k > 0 && dma_has_bias && mi355_dma_gemm_supported(d, a, b))
         return mi355_dma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, workspace, workspace_bytes, s);
+    // a vector of column scales per batch entry exists in the kernels above only
+    if(d->dequant && d->scale_b_mode == MI355_QP_PER_COL_BATCH)
+        return MI355_ERR_UNSUPPORTED;
     if(!u8 && d->k > 0 && mi355_mfma_gemm_supported(d, a, b, c))
         return mi355_mfma_gemm_launch(d, a, b, c, scale_a, scale_b, colsum_b, rowsum_a, bias, s);
 

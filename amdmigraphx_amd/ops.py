@@ -101,23 +101,28 @@ def quant_dot(a, b, fp8=False, scale_a=None, scale_b=None, zp_a=0, zp_b=0,
         if out.dim() > 3 and not out.flatten(0, -3).is_contiguous():
             raise Mi355Error("quant_dot: batch dimensions of the output must be dense")
         stride_c = out.stride(-3)
+    # one vector of column scales (and one bias) per batch entry: scale_b dense [batch, N]
+    cols_per_batch = (scale_b is not None and nb > 1 and scale_b.dim() >= 2 and scale_b.numel() == nb * n and
+                      scale_b.is_contiguous())
     d = QuantDotDesc(m=m, n=n, k=k, lda=lda, ldb=ldb, ldc=ldc, batch=nb, stride_a=sa, stride_b=sb,
                      stride_c=stride_c, trans_a=ta, trans_b=tb, in_type=in_type,
                      out_type=_TORCH2DT[odt], dequant=int(dequant),
                      scale_a_mode=QP.NONE if scale_a is None else
                      (QP.PER_TENSOR if scale_a.numel() == 1 else QP.PER_ROW),
                      scale_b_mode=QP.NONE if scale_b is None else
-                     (QP.PER_TENSOR if scale_b.numel() == 1 else QP.PER_COL),
+                     (QP.PER_TENSOR if scale_b.numel() == 1 else
+                      QP.PER_COL_BATCH if cols_per_batch else QP.PER_COL),
                      zp_a=int(zp_a), zp_b=int(zp_b))
     if scale_a is not None and scale_a.numel() not in (1, m):
         raise Mi355Error("scale_a must be a scalar or have M elements")
-    if scale_b is not None and scale_b.numel() not in (1, n):
-        raise Mi355Error("scale_b must be a scalar or have N elements")
+    if scale_b is not None and scale_b.numel() not in (1, n) and not cols_per_batch:
+        raise Mi355Error("scale_b must be a scalar, have N elements, or batch x N of them (dense)")
     if bias is not None:
         if not dequant:
             raise Mi355Error("quant_dot: a bias needs the dequantizing epilogue")
-        if bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous():
-            raise Mi355Error("bias must be a dense float32 vector of N elements")
+        if bias.dtype != torch.float32 or bias.numel() != (nb * n if cols_per_batch else n) or \
+                not bias.is_contiguous():
+            raise Mi355Error("bias must be a dense float32 vector of N elements (batch x N with such scales)")
     if isinstance(workspace, str):
         if workspace != "static":
             raise Mi355Error("workspace must be a device tensor or the word 'static'")

@@ -50,7 +50,13 @@ typedef enum mi355_qparam_mode {
     MI355_QP_NONE       = 0, /* absent: scale 1, zero point 0 */
     MI355_QP_PER_TENSOR = 1, /* one element */
     MI355_QP_PER_ROW    = 2, /* [M] */
-    MI355_QP_PER_COL    = 3  /* [N] */
+    MI355_QP_PER_COL    = 3, /* [N] */
+    MI355_QP_PER_COL_BATCH = 4 /* scale_b only: [batch, N], one vector of column scales per batch entry, and
+                                  the bias likewise [batch, N] -- several layers that read the same
+                                  activations (stride_a = 0) as one launch.  int8 with the dequantizing
+                                  epilogue, N % 4 == 0, shapes of the matrix-core path; else
+                                  MI355_ERR_UNSUPPORTED.  No counterpart in the reference's operator, which
+                                  has no fused epilogue. */
 } mi355_qparam_mode;
 
 /*

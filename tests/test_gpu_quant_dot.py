@@ -494,6 +494,51 @@ def test_int8_bias_epilogue_bit_exact(ops, m, n, k, trans_b, out):
         assert np.array_equal(half_bits(got), orc.convert(want, orc.F32, ot))
 
 
+@pytest.mark.parametrize("k", [768, 3072])
+@pytest.mark.parametrize("out,with_bias", [("f32", True), ("bf16", True), ("f32", False)])
+def test_int8_layers_over_shared_activations_in_one_launch(ops, k, out, with_bias):
+    """Three layers that read the same activations (the q / k / v projections of an attention block) as one batched
+    launch: A with a batch stride of 0, the weights stacked, one vector of column scales and one bias per batch entry
+    (MI355_QP_PER_COL_BATCH).  Each batch entry equals the oracle's layer bit for bit, on the eight-wave (K = 768) and
+    the four-wave (K = 3072) kernel."""
+    m, n, nb = 640, 768, 3
+    rng = np.random.default_rng(k + len(out))
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-128, 128, (nb, k, n), dtype=np.int8)
+    sa = np.float32(0.0371)
+    sb = rng.uniform(0.001, 0.01, (nb, n)).astype(np.float32)
+    bias = (rng.standard_normal((nb, n)) * 3).astype(np.float32)
+    td = {"f32": torch.float32, "bf16": torch.bfloat16}[out]
+    da = dev(a)
+    print("int8 shared activations", k, out, with_bias, flush=True)
+    got = ops.quant_dot(da.unsqueeze(0).expand(nb, m, k), dev(b), scale_a=dev(np.float32([sa])), scale_b=dev(sb),
+                        out_dtype=td, bias=dev(bias) if with_bias else None)
+    assert got.shape == (nb, m, n)
+    for i in range(nb):
+        want = orc.qdq_matmul_int8(a, b[i], sa, sb[i], 0, 0, orc.F32)
+        if with_bias:
+            want = want + bias[i][None, :]
+        if out == "f32":
+            assert np.array_equal(got[i].cpu().numpy().view(np.uint32), want.view(np.uint32)), i
+        else:
+            assert np.array_equal(half_bits(got[i]), orc.convert(want, orc.F32, orc.BF16)), i
+
+
+def test_column_scales_per_batch_entry_where_no_kernel_has_them(ops):
+    """fp8 operands, a bare result and N % 4 != 0 have no kernel with per-batch column scales: refused, not computed
+    with the first entry's scales."""
+    from amdmigraphx_amd import Mi355Error
+    nb, m, k = 2, 64, 256
+    sa = dev(np.float32([0.1]))
+    for n, fp8 in ((128, True), (130, False)):
+        dt = torch.uint8 if fp8 else torch.int8
+        a = torch.zeros((nb, m, k), dtype=dt, device="cuda")
+        b = torch.zeros((nb, k, n), dtype=dt, device="cuda")
+        sb = torch.ones((nb, n), dtype=torch.float32, device="cuda")
+        with pytest.raises(Mi355Error):
+            ops.quant_dot(a, b, scale_a=sa, scale_b=sb, fp8=fp8)
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 384, 2048), (200, 264, 320), (77, 130, 192)])
 @pytest.mark.parametrize("out", ["f32", "bf16"])
 def test_fp8_bias_epilogue(ops, m, n, k, out):
