@@ -663,6 +663,118 @@ void fuse_shared_w4a16(module& m)
     }
 }
 
+// ---- quantized layers that share their activations -> one batched launch ----------------------
+//
+// The q / k / v projections of an attention block are three mi355::quant_dot over the same int8
+// activations with constant weights of one shape.  At 12288 x 768 x 768 each is 144 output tiles on
+// a chip of 256 CUs: a launch that leaves CUs idle and lasts one tile's pipeline fill, 12 K slabs and
+// a 256 KB store.  Stacked along a batch axis at compile time -- the activations broadcast with a
+// batch stride of 0, the weights [3, K, N], the column scales and the biases [3, N]
+// (MI355_QP_PER_COL_BATCH) -- they are one launch of 432 tiles, and each layer's result is one
+// dense [M, N] block of the stacked result, so nothing downstream changes.  The sums are the same
+// integers and the epilogue the same operations: the same bits.
+// Taken: dequantizing int8 products without zero points, one scale for the activations (the same
+// instruction), per-column weight scales, weights / scales / biases known at compile time and
+// dense, at least 128 rows, fewer tiles than CUs in one member's launch.
+// MIGRAPHX_MI355_DISABLE_SHARED_QUANT_DOT set (to anything but 0) when a program is compiled keeps
+// the launches separate.
+void fuse_shared_quant_dots(module& m)
+{
+    const char* off = std::getenv("MIGRAPHX_MI355_DISABLE_SHARED_QUANT_DOT");
+    if(off != nullptr and std::string(off) != "0")
+        return;
+    std::vector<instruction_ref> gemms;
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() == "mi355::quant_dot")
+            gemms.push_back(ins);
+    }
+    auto constant = [](instruction_ref x) { return x->can_eval() and x->get_shape().standard(); };
+    // a, b, scale_a, scale_b, [bias], out
+    auto candidate = [&](instruction_ref g, const quant_dot& op) {
+        if(not op.dequant or op.zp_a != 0 or op.zp_b != 0 or op.workspace or
+           op.scale_a_mode != MI355_QP_PER_TENSOR or op.scale_b_mode != MI355_QP_PER_COL)
+            return false;
+        const shape& a = g->inputs()[0]->get_shape();
+        const shape& b = g->inputs()[1]->get_shape();
+        // the column scales arrive as a [N] constant broadcast over the rows
+        if(a.type() != shape::int8_type or a.ndim() != 2 or not a.standard() or b.ndim() != 2 or
+           not constant(g->inputs()[1]) or not constant(skip_broadcasts(g->inputs()[3])) or
+           (op.has_bias and not constant(g->inputs()[4])))
+            return false;
+        const auto rows = a.lens()[0], k = a.lens()[1], n = b.lens()[1];
+        const auto tiles = ((rows + 255) / 256) * ((n + 255) / 256);
+        return rows >= 128 and k % 64 == 0 and n % 16 == 0 and tiles < 256 and
+               skip_broadcasts(g->inputs()[3])->get_shape().elements() == n;
+    };
+    std::unordered_set<const instruction*> taken;
+    for(std::size_t i = 0; i < gemms.size(); i++)
+    {
+        auto first = gemms[i];
+        if(taken.count(&*first) > 0)
+            continue;
+        const auto op = any_cast<quant_dot>(first->get_operator());
+        if(not candidate(first, op))
+            continue;
+        std::vector<instruction_ref> members = {first};
+        for(std::size_t j = i + 1; j < gemms.size(); j++)
+        {
+            auto other = gemms[j];
+            if(taken.count(&*other) > 0 or &*other->inputs()[0] != &*first->inputs()[0] or
+               &*skip_broadcasts(other->inputs()[2]) != &*skip_broadcasts(first->inputs()[2]))
+                continue;
+            const auto oop = any_cast<quant_dot>(other->get_operator());
+            if(not candidate(other, oop) or oop.has_bias != op.has_bias or oop.out_type != op.out_type or
+               other->inputs()[1]->get_shape() != first->inputs()[1]->get_shape())
+                continue;
+            members.push_back(other);
+        }
+        if(members.size() < 2)
+            continue;
+        // the stacked launch goes where the first member is: every member's operands are defined
+        // there already (the shared ones are the first member's, the others are constants, which
+        // become literals of their own below)
+        std::string weights, scales, biases;
+        for(auto g : members)
+        {
+            taken.insert(&*g);
+            const argument w = g->inputs()[1]->eval();
+            const argument sc = skip_broadcasts(g->inputs()[3])->eval();
+            weights.append(w.data(), w.get_shape().bytes());
+            scales.append(sc.data(), sc.get_shape().bytes());
+            if(op.has_bias)
+            {
+                const argument bi = g->inputs()[4]->eval();
+                biases.append(bi.data(), bi.get_shape().bytes());
+            }
+        }
+        auto a           = first->inputs()[0];
+        const auto nb    = members.size();
+        const auto rows  = a->get_shape().lens()[0];
+        const auto k     = a->get_shape().lens()[1];
+        const auto n     = first->inputs()[1]->get_shape().lens()[1];
+        auto ab = m.insert_instruction(first, make_op("multibroadcast", {{"out_lens", {nb, rows, k}}}), a);
+        auto wl = m.add_literal(literal{shape{shape::int8_type, {nb, k, n}}, weights.data()});
+        auto sl = m.add_literal(literal{shape{shape::float_type, {nb, n}}, scales.data()});
+        quant_dot fused    = op;
+        fused.scale_b_mode = MI355_QP_PER_COL_BATCH;
+        std::vector<instruction_ref> args = {ab, wl, first->inputs()[2], sl};
+        if(op.has_bias)
+            args.push_back(m.add_literal(literal{shape{shape::float_type, {nb, n}}, biases.data()}));
+        args.push_back(insert_allocation(m, first, shape{op.out_type, {nb, rows, n}}));
+        auto all = m.insert_instruction(first, operation{fused}, args);
+        for(std::size_t at = 0; at < nb; at++)
+        {
+            auto one = m.insert_instruction(members[at],
+                                            make_op("slice", {{"axes", {0}},
+                                                              {"starts", {static_cast<int64_t>(at)}},
+                                                              {"ends", {static_cast<int64_t>(at + 1)}}}),
+                                            all);
+            m.replace_instruction(members[at], make_op("squeeze", {{"axes", {0}}}), {one});
+        }
+    }
+}
+
 // ---- weight-only products of a few rows over constant weights -> the reordered form -------------
 //
 // With one row of activations (or a few: a small batch) the product is a stream of weights, and constant weights can lie in
@@ -1732,6 +1844,8 @@ void lowering::apply(module& m) const
     }
     dead_code_elimination{}.apply(m);
     fuse_shared_w4a16(m);
+    dead_code_elimination{}.apply(m);
+    fuse_shared_quant_dots(m);
     dead_code_elimination{}.apply(m);
     prepack_w4a16(m);
     dead_code_elimination{}.apply(m);

@@ -302,8 +302,17 @@ shape quant_dot::compute_shape(const std::vector<shape>& inputs) const
         const shape& bias = inputs[inputs.size() - (workspace ? 3 : 2)];
         if(not dequant)
             MIGRAPHX_THROW("mi355::quant_dot: a bias needs the dequantizing epilogue");
-        if(bias.type() != shape::float_type or not bias.standard() or bias.elements() != s.lens().back())
-            MIGRAPHX_THROW("mi355::quant_dot: the bias must be a dense float vector of N elements");
+        const auto per = scale_b_mode == MI355_QP_PER_COL_BATCH ? s.elements() / s.lens()[s.ndim() - 2] : s.lens().back();
+        if(bias.type() != shape::float_type or not bias.standard() or bias.elements() != per)
+            MIGRAPHX_THROW("mi355::quant_dot: the bias must be a dense float vector of N elements (one per batch "
+                           "entry with column scales per batch entry)");
+    }
+    if(scale_b_mode == MI355_QP_PER_COL_BATCH)
+    {
+        // [batch, N]: one vector of column scales per batch entry
+        if(not dequant or not inputs[3].standard() or
+           inputs[3].elements() != s.elements() / s.lens()[s.ndim() - 2])
+            MIGRAPHX_THROW("mi355::quant_dot: column scales per batch entry are a dense [batch, N] tensor");
     }
     shape out{out_type, s.lens()};
     if(inputs.back() != out)

@@ -251,6 +251,60 @@ TEST_CASE(qdq_linear_layer_bias)
     }
 }
 
+TEST_CASE(qdq_linear_layers_share_activations)
+{
+    // Three linear layers of one shape over the same quantized activations (the q / k / v projections
+    // of an attention block) and a fourth of another width: the three become one batched launch --
+    // activations with a batch stride of 0, weights, column scales and biases stacked when the
+    // program is compiled -- and each result is a dense block of the stacked one.  Bit-identical to
+    // the CPU target, which evaluates the layers one by one.
+    for(bool with_bias : {true, false})
+    {
+        const std::size_t m = 384, k = 256, n = 256;
+        program p;
+        auto* mm = p.get_main_module();
+        auto x   = mm->add_parameter("x", shape{shape::float_type, {m, k}});
+        auto sx  = mm->add_literal(1.0f / 32);
+        auto zx  = mm->add_literal(static_cast<std::int8_t>(0));
+        auto q   = add_quantize_op(*mm, "quantizelinear", x, sx, zx);
+        auto dx  = add_quantize_op(*mm, "dequantizelinear", q, sx, zx);
+        std::vector<instruction_ref> results;
+        unsigned seed = 70;
+        for(std::size_t width : {n, n, n, std::size_t{512}})
+        {
+            auto w  = mm->add_literal(literal{shape{shape::int8_type, {k, width}}, uniform_ints<int>(k * width, -127, 127, seed++)});
+            auto sw = mm->add_literal(literal{shape{shape::float_type, {width}}, uniform_floats(width, 0.001f, 0.01f, seed++)});
+            auto zw  = mm->add_literal(literal{shape{shape::int8_type, {width}}, std::vector<int>(width, 0)});
+            auto swb = mm->add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", {k, width}}}), sw);
+            auto zwb = mm->add_instruction(make_op("broadcast", {{"axis", 1}, {"out_lens", {k, width}}}), zw);
+            auto dw  = mm->add_instruction(make_op("dequantizelinear"), w, swb, zwb);
+            instruction_ref y = mm->add_instruction(make_op("dot"), dx, dw);
+            if(with_bias)
+            {
+                auto b  = mm->add_literal(literal{shape{shape::float_type, {width}}, normal_floats(width, 2.0f, seed++)});
+                auto bb = mm->add_instruction(make_op("multibroadcast", {{"out_lens", {m, width}}}), b);
+                y       = mm->add_instruction(make_op("add"), y, bb);
+            }
+            results.push_back(y);
+        }
+        mm->add_return(results);
+        migraphx::run_passes(p, {migraphx::simplify_qdq{}, migraphx::dead_code_elimination{}});
+        argument xa{shape{shape::float_type, {m, k}}, normal_floats(m * k, 1.0f, 69)};
+        expect_same(p, {{"x", xa}});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        if(count_ops(*compiled.get_main_module(), "mi355::quant_dot") != 2)
+            std::cout << compiled << std::endl;
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 2);
+        EXPECT(not has_op(compiled, "mi355::binary") and not has_op(compiled, "mi355::chain"));
+        setenv("MIGRAPHX_MI355_DISABLE_SHARED_QUANT_DOT", "1", 1);
+        program separate = p;
+        separate.compile(migraphx::make_target("mi355"));
+        unsetenv("MIGRAPHX_MI355_DISABLE_SHARED_QUANT_DOT");
+        EXPECT(count_ops(*separate.get_main_module(), "mi355::quant_dot") == 4);
+    }
+}
+
 TEST_CASE(qdq_linear_layer_skinny)
 {
     // A few rows against a large weight matrix (decoding, small batches).  Up to 16 rows against
@@ -1895,7 +1949,9 @@ TEST_CASE(encoder_int8_qdq_full_size_replicated)
     auto p32 = encoder::quantized(c32, w, scales);
     program compiled = p32;
     compiled.compile(migraphx::make_target("mi355"));
-    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 6 * c32.layers);
+    // the q / k / v projections of a layer share their activations: one batched launch, then the
+    // output projection and the two feed-forward products
+    EXPECT(count_ops(*compiled.get_main_module(), "mi355::quant_dot") == 4 * c32.layers);
     auto alone = run_on("mi355", p1, {{"ids", ids1}})[0];
     auto batch = run_on("mi355", p32, {{"ids", ids32}})[0];
     const std::size_t bytes = alone.get_shape().bytes();
