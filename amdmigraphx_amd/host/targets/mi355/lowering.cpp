@@ -1351,10 +1351,22 @@ void fuse_layer_norms(module& m)
 }
 
 // contiguous(x) read only by float dots that take x as it lies (a 4-D view: two batch axes with a
-// stride each): the dots read x, the copy goes (what src/eliminate_contiguous.cpp does when the
+// stride each), directly or through a transpose of the last two axes (the keys of an attention
+// layer): the dots read x, the copy goes (what src/eliminate_contiguous.cpp does when the
 // reader's compute_shape accepts the view).  Runs before the dots are lowered.
 void skip_copies_in_front_of_dots(module& m)
 {
+    auto only_dots = [](instruction_ref i) {
+        auto users = i->outputs();
+        return not users.empty() and
+               std::all_of(users.begin(), users.end(), [](instruction_ref u) { return u->name() == "dot"; });
+    };
+    auto swaps_last_two_of_four = [](instruction_ref t) {
+        if(t->name() != "transpose")
+            return false;
+        const auto perm = any_cast<op::transpose>(t->get_operator()).permutation;
+        return perm == std::vector<int64_t>{0, 1, 3, 2};
+    };
     for(auto ins : all_instructions(m))
     {
         if(ins->name() != "contiguous" or ins->outputs().empty())
@@ -1364,7 +1376,9 @@ void skip_copies_in_front_of_dots(module& m)
            x->get_shape().broadcasted())
             continue;
         auto users = ins->outputs();
-        if(not std::all_of(users.begin(), users.end(), [](instruction_ref u) { return u->name() == "dot"; }))
+        if(not std::all_of(users.begin(), users.end(), [&](instruction_ref u) {
+               return u->name() == "dot" or (swaps_last_two_of_four(u) and only_dots(u));
+           }))
             continue;
         for(auto u : users)
             instruction::replace_argument(u, ins, x);

@@ -1269,6 +1269,33 @@ TEST_CASE(float_dot_two_batch_axes)
                         {"k", argument{s, normal_floats(s.elements(), 1.0f, 62)}},
                         {"v", argument{s, normal_floats(s.elements(), 1.0f, 63)}}});
     }
+    // the same graph as exporters write it: a copy behind each head split, the keys transposed after
+    // theirs.  None of the copies is made: the dots read the views.
+    {
+        const dims d{2, 4, 64, 32};
+        program p;
+        auto* mm = p.get_main_module();
+        shape s{shape::float_type, {d.b, d.r, d.h, d.w}};
+        auto split = [&](const std::string& name) {
+            auto x = mm->add_parameter(name, s);
+            auto t = mm->add_instruction(make_op("transpose", {{"permutation", {0, 2, 1, 3}}}), x);
+            return mm->add_instruction(make_op("contiguous"), t);
+        };
+        auto qh = split("q");
+        auto kh = split("k");
+        auto vh = split("v");
+        auto kt = mm->add_instruction(make_op("transpose", {{"permutation", {0, 1, 3, 2}}}), kh);
+        auto scores = mm->add_instruction(make_op("dot"), qh, kt);
+        auto ctx    = mm->add_instruction(make_op("dot"), scores, vh);
+        mm->add_return({scores, ctx});
+        program compiled = p;
+        compiled.compile(migraphx::make_target("mi355"));
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::dot") == 2);
+        EXPECT(count_ops(*compiled.get_main_module(), "mi355::contiguous") == 0);
+        expect_same(p, {{"q", argument{s, normal_floats(s.elements(), 1.0f, 64)}},
+                        {"k", argument{s, normal_floats(s.elements(), 1.0f, 65)}},
+                        {"v", argument{s, normal_floats(s.elements(), 1.0f, 66)}}});
+    }
 }
 
 TEST_CASE(dot_scale_epilogue)
