@@ -108,6 +108,8 @@ EXPORTS = {
                          [ctypes.c_int64] * 12 + [ctypes.c_void_p, ctypes.c_void_p],
     "mi355_dot_batch2": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32] +
                         [ctypes.c_int64] * 13 + [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p],
+    "mi355_dot_batch2_strided": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32] +
+                                [ctypes.c_int64] * 16 + [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p],
     "mi355_contiguous": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
                          ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
                          ctypes.c_void_p],

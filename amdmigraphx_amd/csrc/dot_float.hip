@@ -28,15 +28,17 @@ struct dot_params
     int64_t batch_inner     = 1;
     int64_t stride_a_outer  = 0;
     int64_t stride_b_outer  = 0;
+    int64_t stride_c_outer  = 0; // C likewise: zo * stride_c_outer + zi * stride_c
 };
 
-MI355_DEVINL void batch_offsets(const dot_params& p, int64_t& ao, int64_t& bo)
+MI355_DEVINL void batch_offsets(const dot_params& p, int64_t& ao, int64_t& bo, int64_t& co)
 {
     const int64_t z  = blockIdx.z;
     const int64_t zo = z / p.batch_inner;
     const int64_t zi = z - zo * p.batch_inner;
     ao               = zo * p.stride_a_outer + zi * p.stride_a;
     bo               = zo * p.stride_b_outer + zi * p.stride_b;
+    co               = zo * p.stride_c_outer + zi * p.stride_c;
 }
 
 MI355_DEVINL float load_f32(const void* p, int type, int64_t i)
@@ -73,8 +75,8 @@ __global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
     const int lk   = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.y * 64;
     const int64_t col0 = (int64_t)blockIdx.x * 64;
-    int64_t ao, bo;
-    batch_offsets(p, ao, bo);
+    int64_t ao, bo, co;
+    batch_offsets(p, ao, bo, co);
     v4d acc[2][2];
 #pragma unroll
     for(int i = 0; i < 2; i++)
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(256) void dot_float_mfma_kernel(dot_params p)
                 const int64_t col = col0 + wn * 32 + j * 16 + l16;
                 if(col >= p.n)
                     continue;
-                const int64_t idx = (int64_t)blockIdx.z * p.stride_c + row * p.ldc + col;
+                const int64_t idx = co + row * p.ldc + col;
                 const float f     = (float)acc[i][j][r];
                 if(p.type == MI355_F32)
                     ((float*)p.c)[idx] = p.scale != nullptr ? f * p.scale[0] : f;
@@ -175,8 +177,8 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
     const int lk   = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.y * 64;
     const int64_t col0 = (int64_t)blockIdx.x * 64;
-    int64_t ao, bo;
-    batch_offsets(p, ao, bo);
+    int64_t ao, bo, co;
+    batch_offsets(p, ao, bo, co);
     const float* a = static_cast<const float*>(p.a) + ao;
     const float* b = static_cast<const float*>(p.b) + bo;
     // this thread's piece of each tile: `major` indexes the strided dimension, `minor` the
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(256) void dot_f32_mfma_kernel(dot_params p)
             {
                 const int64_t col = col0 + wn * 32 + j * 16 + l16;
                 if(col < p.n)
-                    static_cast<float*>(p.c)[(int64_t)blockIdx.z * p.stride_c + row * p.ldc + col] =
+                    static_cast<float*>(p.c)[co + row * p.ldc + col] =
                         (float)acc[i][j][r] * alpha;
             }
         }
@@ -458,7 +460,8 @@ static int dot_launch(bool fp32acc,
                                 void* stream,
                                 int64_t batch_inner    = 0,
                                 int64_t stride_a_outer = 0,
-                                int64_t stride_b_outer = 0)
+                                int64_t stride_b_outer = 0,
+                                int64_t stride_c_outer = -1) // -1: batch_inner dense blocks of stride_c
 {
     if(type != MI355_F32 && type != MI355_F16 && type != MI355_BF16)
         return MI355_ERR_BAD_ARG;
@@ -481,6 +484,7 @@ static int dot_launch(bool fp32acc,
     p.batch_inner    = batch_inner > 0 ? batch_inner : batch;
     p.stride_a_outer = stride_a_outer;
     p.stride_b_outer = stride_b_outer;
+    p.stride_c_outer = stride_c_outer >= 0 ? stride_c_outer : p.batch_inner * stride_c;
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // fp32 with contiguous rows or columns, everything the 16-byte loads touch aligned
@@ -673,4 +677,39 @@ extern "C" int mi355_dot_batch2(const void* a,
     return dot_launch(fp32acc != 0, a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, n,
                       batch_outer * batch_inner, stride_a_inner, stride_b_inner, m * n, scale, stream, batch_inner,
                       stride_a_outer, stride_b_outer);
+}
+
+extern "C" int mi355_dot_batch2_strided(const void* a,
+                                        const void* b,
+                                        void* c,
+                                        int32_t type,
+                                        int64_t m,
+                                        int64_t n,
+                                        int64_t k,
+                                        int64_t a_stride_m,
+                                        int64_t a_stride_k,
+                                        int64_t b_stride_k,
+                                        int64_t b_stride_n,
+                                        int64_t ldc,
+                                        int64_t batch_outer,
+                                        int64_t batch_inner,
+                                        int64_t stride_a_outer,
+                                        int64_t stride_a_inner,
+                                        int64_t stride_b_outer,
+                                        int64_t stride_b_inner,
+                                        int64_t stride_c_outer,
+                                        int64_t stride_c_inner,
+                                        const float* scale,
+                                        int32_t fp32acc,
+                                        void* stream)
+{
+    if(batch_outer < 0 || batch_inner < 0 || stride_c_outer < 0 || stride_c_inner < 0)
+        return MI355_ERR_BAD_ARG;
+    if(batch_outer == 0 || batch_inner == 0)
+        return MI355_OK;
+    if(batch_outer > 65535 / batch_inner)
+        return MI355_ERR_UNSUPPORTED;
+    return dot_launch(fp32acc != 0, a, b, c, type, m, n, k, a_stride_m, a_stride_k, b_stride_k, b_stride_n, ldc,
+                      batch_outer * batch_inner, stride_a_inner, stride_b_inner, stride_c_inner, scale, stream,
+                      batch_inner, stride_a_outer, stride_b_outer, stride_c_outer);
 }

@@ -1385,6 +1385,36 @@ void skip_copies_in_front_of_dots(module& m)
     }
 }
 
+// dot -> transpose(0, 2, 1, 3) -> contiguous, the merge of the heads behind an attention layer's
+// context: the dot writes its [batch, heads, rows, width] result into [batch, rows, heads, width]
+// memory (its output buffer is the transposed view of a dense buffer of that layout), the transpose
+// of that is dense already and the copy goes.  Runs behind the lowering of the single operators.
+void write_dots_head_merged(module& m)
+{
+    for(auto ins : all_instructions(m))
+    {
+        if(ins->name() != "mi355::dot" or ins->get_shape().ndim() != 4 or
+           ins->get_shape().type() != shape::float_type or not ins->get_shape().standard())
+            continue;
+        auto users = distinct_users(ins);
+        if(users.size() != 1 or users[0]->name() != "transpose" or
+           any_cast<op::transpose>(users[0]->get_operator()).permutation != std::vector<int64_t>{0, 2, 1, 3})
+            continue;
+        auto t      = users[0];
+        auto copies = distinct_users(t);
+        if(copies.empty() or not std::all_of(copies.begin(), copies.end(), [](instruction_ref c) {
+               return c->name() == "mi355::contiguous";
+           }))
+            continue;
+        const auto& l = ins->get_shape().lens();
+        auto merged   = insert_allocation(m, ins, shape{shape::float_type, {l[0], l[2], l[1], l[3]}});
+        auto view     = m.insert_instruction(ins, make_op("transpose", {{"permutation", {0, 2, 1, 3}}}), merged);
+        instruction::replace_argument(ins, ins->inputs().back(), view);
+        for(auto c : copies)
+            m.replace_instruction(c, t);
+    }
+}
+
 // A chain whose only reader is a quantizelinear to int8 with one scale (and one zero point) for the
 // whole tensor -- the activations in front of a quantized layer, e.g. the GELU of a feed-forward
 // block -- becomes one mi355::chain_q8: the float tensor is neither written nor read back.  Runs
@@ -1873,6 +1903,8 @@ void lowering::apply(module& m) const
     // 2. everything else, one operator at a time
     for(auto ins : all_instructions(m))
         lower_instruction(m, ins);
+    dead_code_elimination{}.apply(m);
+    write_dots_head_merged(m);
     dead_code_elimination{}.apply(m);
     if(fuse_pointwise)
     {

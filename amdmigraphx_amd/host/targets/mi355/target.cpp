@@ -823,9 +823,15 @@ shape dot::compute_shape(const std::vector<shape>& inputs) const
         if(not batch_collapses(inputs[i]) and inputs[i].ndim() != 4)
             MIGRAPHX_THROW("mi355::dot: batch dimensions do not collapse into one stride");
     }
-    if(inputs.back() != s)
+    // the result is dense, or (two batch axes, float) a view with rows of contiguous elements: the
+    // [batch, heads, rows, width] result written into [batch, rows, heads, width] memory
+    const shape& out = inputs.back();
+    if(out == s)
+        return s;
+    if(out.type() != s.type() or out.lens() != s.lens() or s.ndim() != 4 or s.type() != shape::float_type or
+       out.strides().back() != 1 or out.broadcasted())
         MIGRAPHX_THROW("mi355::dot: output buffer has the wrong shape");
-    return s;
+    return out;
 }
 
 argument dot::compute(migraphx::context& ctx, const shape& out, const std::vector<argument>& args) const
@@ -849,6 +855,34 @@ argument dot::compute(migraphx::context& ctx, const shape& out, const std::vecto
         return r;
     };
     const bool fast = fp32acc and out.type() == shape::float_type;
+    if(nd == 4 and not out.standard())
+    {
+        status_check(mi355_dot_batch2_strided(args[0].data(),
+                                              args[1].data(),
+                                              args.back().data(),
+                                              to_mi355_type(out.type()),
+                                              m,
+                                              n,
+                                              k,
+                                              static_cast<int64_t>(sa.strides()[2]),
+                                              static_cast<int64_t>(sa.strides()[3]),
+                                              static_cast<int64_t>(sb.strides()[2]),
+                                              static_cast<int64_t>(sb.strides()[3]),
+                                              static_cast<int64_t>(out.strides()[2]),
+                                              static_cast<int64_t>(sa.lens()[0]),
+                                              static_cast<int64_t>(sa.lens()[1]),
+                                              static_cast<int64_t>(sa.strides()[0]),
+                                              static_cast<int64_t>(sa.strides()[1]),
+                                              static_cast<int64_t>(sb.strides()[0]),
+                                              static_cast<int64_t>(sb.strides()[1]),
+                                              static_cast<int64_t>(out.strides()[0]),
+                                              static_cast<int64_t>(out.strides()[1]),
+                                              scaled ? reinterpret_cast<const float*>(args[2].data()) : nullptr,
+                                              fast ? 1 : 0,
+                                              stream_of(ctx)),
+                     name());
+        return args.back();
+    }
     if(nd == 4 and (not batch_collapses(sa) or not batch_collapses(sb)))
     {
         status_check(mi355_dot_batch2(args[0].data(),

@@ -521,6 +521,20 @@ int mi355_dot_batch2(const void* a, const void* b, void* c, int32_t type,
                      int64_t stride_a_outer, int64_t stride_a_inner,
                      int64_t stride_b_outer, int64_t stride_b_inner,
                      const float* scale, int32_t fp32acc, void* stream);
+/* The same with C as a strided set of row-major blocks: output (o, i, row, col) lies at
+ * c + o * stride_c_outer + i * stride_c_inner + row * ldc + col (blocks that do not overlap).  This is how
+ * the target writes the context of an attention layer, dot(probabilities, values) over [batch, heads],
+ * straight into the [batch, rows, heads, width] layout the transpose(0, 2, 1, 3) + contiguous behind it
+ * would produce (stride_c_inner = width, ldc = heads * width): the copy is not made
+ * (src/eliminate_contiguous.cpp removes such copies where the reference's kernels take the view). */
+int mi355_dot_batch2_strided(const void* a, const void* b, void* c, int32_t type,
+                             int64_t m, int64_t n, int64_t k,
+                             int64_t a_stride_m, int64_t a_stride_k, int64_t b_stride_k, int64_t b_stride_n,
+                             int64_t ldc, int64_t batch_outer, int64_t batch_inner,
+                             int64_t stride_a_outer, int64_t stride_a_inner,
+                             int64_t stride_b_outer, int64_t stride_b_inner,
+                             int64_t stride_c_outer, int64_t stride_c_inner,
+                             const float* scale, int32_t fp32acc, void* stream);
 
 /*
  * contiguous: gather a strided view (ndim <= MI355_MAX_DIMS, element strides, zero = broadcast)

@@ -82,6 +82,37 @@ def test_float_dot_three_steps_in_flight_every_remainder(ops, k, trans_a, trans_
     assert (np.abs(fast.astype(np.float64) - want) <= mag * k * 2.0**-24 + 1e-30).all()
 
 
+@pytest.mark.parametrize("b,h,rows,width", [(2, 3, 40, 16), (1, 4, 128, 64), (3, 2, 70, 20)])
+def test_float_dot_writes_its_result_head_merged(b, h, rows, width):
+    """mi355_dot_batch2_strided: probabilities [b, h, rows, rows] times values seen as [b, h, rows, width] (a view of
+    [b, rows, h, width] storage), the result written straight into [b, rows, h, width] memory -- what transpose(0, 2, 1, 3)
+    + contiguous of the dense result would give -- bit for bit, and nothing outside it touched."""
+    import ctypes
+    from amdmigraphx_amd import capi
+    rng = np.random.default_rng(b * 100 + rows)
+    probs = rng.standard_normal((b, h, rows, rows)).astype(np.float32)
+    vals = rng.standard_normal((b, rows, h, width)).astype(np.float32)
+    want = orc.dot(probs.reshape(b * h, rows, rows),
+                   np.ascontiguousarray(vals.transpose(0, 2, 1, 3)).reshape(b * h, rows, width), orc.F32)
+    want = want.reshape(b, h, rows, width).transpose(0, 2, 1, 3)
+    dp, dv = dev(probs), dev(vals)
+    out = torch.full((b, rows, h, width), float("nan"), dtype=torch.float32, device="cuda")
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    print("float dot head-merged", b, h, rows, width, flush=True)
+    st = capi.lib().mi355_dot_batch2_strided(
+        vp(dp), vp(dv), vp(out), 3, rows, width, rows,
+        rows, 1, h * width, 1,                 # A rows / k strides, B k / n strides
+        h * width,                             # ldc
+        b, h,
+        h * rows * rows, rows * rows,          # A: batch, head
+        rows * h * width, width,               # B: batch, head (the view)
+        rows * h * width, width,               # C: batch, head
+        None, 0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert st == 0
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), np.ascontiguousarray(want).view(np.uint32))
+
+
 def test_fp32_accumulation_is_float32_only(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((16, 16), dtype=torch.float16, device="cuda")
