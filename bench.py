@@ -108,7 +108,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--only-headline", action="store_true",
                     help="time the headline kernel only (for counter runs under rocprofv3)")
-    ap.add_argument("--only", choices=["headline", "fp8", "gemv", "skinny", "conv", "mx"], default=None,
+    ap.add_argument("--only", choices=["headline", "fp8", "gemv", "skinny", "conv", "mx", "encoder"], default=None,
                     help="run one section only, so that a rocprofv3 run holds that section's kernels alone")
     ap.add_argument("--gemv-shape", default=None, metavar="K,N",
                     help="with --only gemv: one (K, N) shape instead of the three of config 4")
@@ -621,6 +621,30 @@ def main():
             del am, bm, om
     except Exception as e:
         also["mx_quant_dot_error"] = str(e)
+
+    # ---- config 5: the BERT-base-shaped int8 QDQ encoder through the host layer --------------------
+    # 12 layers, hidden 768, 12 heads, FFN 3072, 32 x 384 tokens: calibration, compilation for the mi355
+    # target and 8 timed forwards in the C++ test program (a child process; its checks are the
+    # encoder tests of tests/cpp/gpu_tests.cpp, which compare the program with the CPU target)
+    try:
+        skip("encoder")
+        import re
+        import subprocess
+        prog = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "bin", "gpu_tests")
+        if not os.path.exists(prog):
+            raise RuntimeError(f"{prog} is not built (make -C tests/cpp)")
+        run = subprocess.run([prog, "encoder_bench"], capture_output=True, text=True, timeout=300)
+        if run.returncode != 0:
+            raise RuntimeError(f"encoder_bench exited with {run.returncode}: {run.stdout[-300:]} {run.stderr[-300:]}")
+        ms = re.search(r"layers (\d+): ([0-9.]+) ms per forward", run.stdout)
+        launches = re.search(r"quantized MatMul launches per forward: (\d+)", run.stdout)
+        if ms is None:
+            raise RuntimeError("no timing in the output of encoder_bench")
+        also["encoder_int8_qdq_L12_H768_B32_S384"] = {
+            "ms_per_forward": round(float(ms.group(2)), 3), "layers": int(ms.group(1)),
+            "quantized_launches_per_forward": int(launches.group(1)) if launches else None}
+    except Exception as e:
+        also["encoder_error"] = str(e)
 
     line = {
         "metric": "quant_dot TOPS & % MFMA peak (int8/fp8); int4 W-only GEMV GB/s & % HBM",
