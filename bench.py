@@ -630,6 +630,9 @@ def main():
         skip("encoder")
         import re
         import subprocess
+        # under a profiler the child would start inside the profiler's environment: leave it out there
+        if any(k.startswith(("ROCPROF", "ROCP_")) or "rocprofiler" in v.lower() for k, v in os.environ.items()):
+            raise RuntimeError("skipped under a profiler (run tests/cpp/bin/gpu_tests encoder_bench itself)")
         prog = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "bin", "gpu_tests")
         if not os.path.exists(prog):
             raise RuntimeError(f"{prog} is not built (make -C tests/cpp)")
