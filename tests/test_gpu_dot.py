@@ -113,6 +113,24 @@ def test_float_dot_writes_its_result_head_merged(b, h, rows, width):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), np.ascontiguousarray(want).view(np.uint32))
 
 
+def test_strided_result_bad_arguments_are_rejected():
+    import ctypes
+    from amdmigraphx_amd import capi
+    x = torch.zeros(2 * 2 * 8 * 8, dtype=torch.float32, device="cuda")
+    vp = ctypes.c_void_p(x.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(ldc=8, bo=2, bi=2, sco=128, sci=64):
+        return capi.lib().mi355_dot_batch2_strided(vp, vp, vp, 3, 8, 8, 8, 8, 1, 8, 1, ldc, bo, bi,
+                                                   128, 64, 128, 64, sco, sci, None, 0, st)
+    assert call(ldc=4) != 0                    # rows of C shorter than N
+    assert call(sco=-1) != 0 and call(sci=-1) != 0
+    assert call(bo=-1) != 0
+    assert call(bo=70000, bi=1) != 0           # more batch entries than one launch addresses
+    assert call(bo=0) == 0                     # nothing to do
+    torch.cuda.synchronize()
+
+
 def test_fp32_accumulation_is_float32_only(ops):
     from amdmigraphx_amd import Mi355Error
     a = torch.zeros((16, 16), dtype=torch.float16, device="cuda")
