@@ -1193,10 +1193,72 @@ instruction_ref parse_matmulbnb4(const node_info& info, const std::vector<instru
     return out;
 }
 
+// LayerNormalization (src/onnx/parse_layernorm.cpp:33-254): over the axes [axis, rank)
+//   y = (x - mean) * rsqrt(variance + epsilon) * scale [+ bias], mean = reduce_mean(x),
+//   variance = reduce_mean((x - mean)^2); outputs y, mean and the reciprocal standard deviation.
+// 16-bit inputs are computed in float unless stash_type is 0.  The square of the differences is
+// written as a product of x - mean with itself (the reference's sqdiff computes the same float).
+std::vector<instruction_ref> parse_layernorm(const node_info& info, const std::vector<instruction_ref>& args)
+{
+    module& m          = *info.mod;
+    int64_t axis       = info.has("axis") ? info.attr("axis").i : -1;
+    const float eps_in = info.has("epsilon") ? info.attr("epsilon").f : 1e-5f;
+    const bool stash   = info.has("stash_type") ? info.attr("stash_type").i == 1 : true;
+    if(args.size() < 2 or args.size() > 3)
+        MIGRAPHX_THROW("PARSE_LAYERNORM: invalid input count");
+    auto valid = [](shape::type_t t, const std::string& what) {
+        if(t != shape::float_type and t != shape::half_type and t != shape::bf16_type)
+            MIGRAPHX_THROW("PARSE_LAYERNORM: Invalid type for " + what);
+    };
+    auto x          = args[0];
+    const auto type = x->get_shape().type();
+    const auto rank = static_cast<int64_t>(x->get_shape().ndim());
+    valid(type, "input");
+    if(rank < 2)
+        MIGRAPHX_THROW("PARSE_LAYERNORM: invalid ndims=" + std::to_string(rank) + ", must be at least 2");
+    if(axis < -rank or axis >= rank)
+        MIGRAPHX_THROW("PARSE_LAYERNORM: invalid axis");
+    auto scale = args[1];
+    valid(scale->get_shape().type(), "scale");
+    if(args.size() > 2)
+        valid(args[2]->get_shape().type(), "bias");
+    axis             = axis < 0 ? axis + rank : axis;
+    const auto kdims = rank - axis;
+    std::vector<int64_t> axes(kdims);
+    std::iota(axes.begin(), axes.end(), axis);
+    const bool widen = stash and type != shape::float_type;
+    auto xin         = widen ? m.add_instruction(make_op("convert", {{"target_type", shape::float_type}}), x) : x;
+    auto mean        = m.add_instruction(make_op("reduce_mean", {{"axes", axes}}), xin);
+    auto centred     = common_binary(m, "sub", xin, mean, "LayerNormalization");
+    auto variance    = m.add_instruction(make_op("reduce_mean", {{"axes", axes}}),
+                                      m.add_instruction(make_op("mul"), centred, centred));
+    const float eps  = type == shape::half_type and std::abs(eps_in) < 1e-7f ? 1e-7f : eps_in;
+    // epsilon has the input's type (and its rounding), whatever the arithmetic is done in
+    instruction_ref eps_lit = m.add_literal(literal{shape{type}, std::vector<float>{eps}});
+    if(widen)
+        eps_lit = m.add_instruction(make_op("convert", {{"target_type", shape::float_type}}), eps_lit);
+    auto rs          = m.add_instruction(make_op("rsqrt"), common_binary(m, "add", variance, eps_lit, "LayerNormalization"));
+    auto result      = common_binary(m, "mul", centred, rs, "LayerNormalization");
+    if(widen)
+        result = m.add_instruction(make_op("convert", {{"target_type", type}}), result);
+    // a vector of scales (biases) lies along the first normalised axis
+    const auto skipped = static_cast<std::size_t>(rank - kdims);
+    auto along = [&](instruction_ref v) {
+        if(skipped > 0 and v->get_shape().ndim() == 1)
+            return m.add_instruction(make_op("broadcast", {{"axis", skipped}, {"out_lens", x->get_shape().lens()}}), v);
+        return v;
+    };
+    auto y = common_binary(m, "mul", result, along(scale), "LayerNormalization");
+    if(args.size() > 2)
+        y = common_binary(m, "add", y, along(args[2]), "LayerNormalization");
+    return {y, mean, rs};
+}
+
 const std::unordered_map<std::string, multi_parser>& multi_parsers()
 {
     static const std::unordered_map<std::string, multi_parser> table = {
         {"DynamicQuantizeLinear", parse_dynamicquantizelinear},
+        {"LayerNormalization", parse_layernorm},
     };
     return table;
 }

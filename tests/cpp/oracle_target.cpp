@@ -326,6 +326,23 @@ struct cpu_op
             int64_t cols = 0;
             rows_cols(x.get_shape(), rows, cols);
             if(n == "reduce_mean")
+            {
+                // the trailing axes as one: [rows, cols] with rows = what is left of the tensor (the reduced
+                // axes have length 1 in the result)
+                const auto& xl = x.get_shape().lens();
+                const auto& ol = out.lens();
+                std::size_t first = 0;
+                while(first < xl.size() and ol[first] == xl[first])
+                    first++;
+                for(std::size_t d = first; d < xl.size(); d++)
+                {
+                    if(ol[d] != 1)
+                        MIGRAPHX_THROW("oracle target: reduce_mean over axes that are not the trailing ones");
+                }
+                rows = static_cast<int64_t>(out.elements());
+                cols = rows == 0 ? 0 : static_cast<int64_t>(x.get_shape().elements()) / rows;
+            }
+            if(n == "reduce_mean")
                 orc_reduce_mean_f32(reinterpret_cast<float*>(r.data()),
                                     reinterpret_cast<const float*>(x.data()), rows, cols, 1);
             else

@@ -464,6 +464,23 @@ for stem in ("qlinearadd_test", "qlinearadd_bcast_test", "qlinearmul_test", "qli
         shutil.copyfile(os.path.join(REF, "test/onnx", model), os.path.join(os.path.dirname(OUT), "onnx", model))
 out["onnx_qlinearbinary"] = qlb
 
+# ---- LayerNormalization models (test/onnx/verify/layer_norm_3d*_test.cpp): x = 1, 2, 3, ... (norm_test in
+# test/onnx/include/onnx_verify_utils.hpp:33-60), scale and bias as the test gives them
+lnm = []
+for stem in ("layer_norm_3d_test", "layer_norm_3d_half_test", "layer_norm_3d_bf16_test"):
+    rel = "test/onnx/verify/" + stem + ".cpp"
+    for name, body in test_cases(read(rel)).items():
+        flat = re.sub(r"(?:half|bf16|migraphx::half|migraphx::bf16)\{([^}]*)\}", r"\1", body)
+        call = re.search(r"norm_test<(\w+)>\(\{([^}]*)\},\s*scale,\s*bias,\s*read_onnx\(\"([^\"]+)\"\)", flat)
+        c = {"name": name, "source": rel, "model": call.group(3), "type": call.group(1),
+             "x_lens": num_list(call.group(2)), "scale": vec(flat, "scale"), "bias": vec(flat, "bias"),
+             "gold": vec(flat, "gold")}
+        assert c["gold"] and c["scale"] and c["bias"], name
+        lnm.append(c)
+for f in sorted(glob.glob(os.path.join(REF, "test/onnx", "layer_norm_*.onnx"))):
+    shutil.copyfile(f, os.path.join(os.path.dirname(OUT), "onnx", os.path.basename(f)))
+out["onnx_layernorm"] = lnm
+
 with open(OUT, "w") as f:
     json.dump(out, f, indent=0, separators=(",", ":"))
 print("wrote", OUT, os.path.getsize(OUT), "bytes")

@@ -166,3 +166,32 @@ def test_written_qdq_matmul_model_on_device(tmp_path):
     xq = orc.quantizelinear(x, np.float32(1.0 / 32), np.int8(0), orc.F32, orc.I8)
     want = orc.qdq_matmul_int8(xq, w, np.float32(1.0 / 32), sw) + bias[None, :]
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_layernormalization_models_on_device(golden, tmp_path):
+    """LayerNormalization over the last axis: the parser's reduce_mean / sub / mul / reduce_mean / add / rsqrt / mul /
+    mul / add becomes one mi355::chain_rows, with the bits of the CPU target (the float model; its 16-bit siblings
+    go through converts around the same float arithmetic)."""
+    import os
+    from amdmigraphx_amd import migraphx as mgx
+    from host_util import ONNX_DIR
+    p = mgx.parse_onnx(os.path.join(ONNX_DIR, "layer_norm_4d_test.onnx"))
+    p.compile(mgx.get_target("gpu"))
+    text = repr(p)
+    assert text.count("mi355::chain_rows") == 1 and "mi355::reduce_mean" not in text, text
+    rng = np.random.default_rng(23)
+    for model, lens in (("layer_norm_4d_test.onnx", (3, 3, 3, 3)), ("layer_norm_3d_test.onnx", (1, 4, 2)),
+                        ("layer_norm_2d_axis_minus_one_test.onnx", (3, 4))):
+        inputs = {"x": rng.standard_normal(lens).astype(np.float32).flatten(),
+                  "scale": rng.uniform(0.5, 1.5, lens[-1]).astype(np.float32),
+                  "bias": rng.standard_normal(lens[-1]).astype(np.float32)}
+        print("onnx", model, flush=True)
+        got = run_onnx("mi355", model, inputs, tmp_path)
+        want = run_onnx("oracle", model, inputs, tmp_path)
+        assert got.tolist() == want.tolist(), model
+    for c in golden["onnx_layernorm"]:
+        n = int(np.prod(c["x_lens"]))
+        got = run_onnx("mi355", c["model"], {"x": list(range(1, n + 1)), "scale": c["scale"], "bias": c["bias"]},
+                       tmp_path)
+        tol = 1e-5 if c["type"] == "float" else 8e-3
+        np.testing.assert_allclose(got, np.float64(c["gold"]), rtol=tol, atol=tol, err_msg=c["name"])

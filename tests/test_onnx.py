@@ -446,3 +446,55 @@ def test_qlinearbinary_rejects_mismatched_types(tmp_path):
     path.write_bytes(data)
     rc, text = print_onnx(str(path))
     assert rc == 4 and "QLinearAdd: mismatched input types" in text, text
+
+
+def test_layernormalization_models_reference_known_answers(golden, tmp_path):
+    # test/onnx/verify/layer_norm_3d_test.cpp, layer_norm_3d_half_test.cpp, layer_norm_3d_bf16_test.cpp: x = 1, 2, ...
+    # (compared by RMS there; 16-bit models are computed in float and rounded once at the end)
+    assert len(golden["onnx_layernorm"]) == 3
+    for c in golden["onnx_layernorm"]:
+        n = int(np.prod(c["x_lens"]))
+        got = run_onnx("oracle", c["model"], {"x": list(range(1, n + 1)), "scale": c["scale"], "bias": c["bias"]},
+                       tmp_path)
+        tol = 1e-5 if c["type"] == "float" else 8e-3
+        np.testing.assert_allclose(got, np.float64(c["gold"]), rtol=tol, atol=tol, err_msg=c["name"])
+
+
+def test_layernormalization_definition_on_the_other_models(tmp_path):
+    """The models without known answers in the reference's tests, against the definition in numpy: other axes, four
+    dimensions, no bias (src/onnx/parse_layernorm.cpp:103-176)."""
+    rng = np.random.default_rng(17)
+    for model, lens, axis, with_bias in (("layer_norm_2d_axis_zero_test.onnx", (3, 4), 0, True),
+                                         ("layer_norm_2d_axis_one_test.onnx", (3, 4), 1, True),
+                                         ("layer_norm_2d_axis_minus_one_test.onnx", (3, 4), -1, True),
+                                         ("layer_norm_4d_test.onnx", (3, 3, 3, 3), -1, True),
+                                         ("layer_norm_without_bias_test.onnx", (1, 2), -1, False)):
+        x = rng.standard_normal(lens).astype(np.float32)
+        norm_lens = lens[axis:]
+        scale = rng.uniform(0.5, 1.5, norm_lens[:1] if len(norm_lens) > 1 and False else norm_lens[-1:] if len(norm_lens) == 1 else norm_lens).astype(np.float32)
+        bias = rng.standard_normal(scale.shape).astype(np.float32)
+        inputs = {"x": x.flatten(), "scale": scale.flatten()}
+        if with_bias:
+            inputs["bias"] = bias.flatten()
+        got = run_onnx("oracle", model, inputs, tmp_path)
+        axes = tuple(range(axis % len(lens), len(lens)))
+        x64 = x.astype(np.float64)
+        mean = x64.mean(axis=axes, keepdims=True)
+        var = ((x64 - mean) ** 2).mean(axis=axes, keepdims=True)
+        want = (x64 - mean) / np.sqrt(var + 1e-5) * scale.reshape((1,) * (len(lens) - scale.ndim) + scale.shape)
+        if with_bias:
+            want = want + bias.reshape((1,) * (len(lens) - bias.ndim) + bias.shape)
+        np.testing.assert_allclose(got[:want.size], want.flatten(), rtol=2e-5, atol=2e-5, err_msg=model)
+
+
+def test_layernormalization_error_messages():
+    # test/onnx/parse/layer_norm_invalid_*: src/onnx/parse_layernorm.cpp:70-110, 180-200
+    for model, message in (("layer_norm_invalid_axis_error_test.onnx", "PARSE_LAYERNORM: invalid axis"),
+                           ("layer_norm_invalid_minus_axis_error_test.onnx", "PARSE_LAYERNORM: invalid axis"),
+                           ("layer_norm_invalid_input_count_error_test.onnx", "PARSE_LAYERNORM: invalid input count"),
+                           ("layer_norm_invalid_shape_error_test.onnx", "PARSE_LAYERNORM: invalid ndims=1, must be at least 2"),
+                           ("layer_norm_3d_invalid_int8_test.onnx", "PARSE_LAYERNORM: Invalid type for input"),
+                           ("layer_norm_3d_invalid_scale_test.onnx", "PARSE_LAYERNORM: Invalid type for scale"),
+                           ("layer_norm_3d_invalid_bias_test.onnx", "PARSE_LAYERNORM: Invalid type for bias")):
+        rc, text = print_onnx(model)
+        assert rc == 4 and message in text, (model, text)
